@@ -1,0 +1,207 @@
+/* nxhip.h — C ABI of libnxhip, an MI355X (gfx950) engine for the Nx backend
+   contract (Nx_core.Backend_intf.S of raven-ml/raven).
+
+   Everything here is plain C: pointers, sizes and one POD descriptor. A binding
+   (OCaml foreign stubs, ctypes, ...) unpacks its tensor handle into an
+   nxh_tensor and calls one entry point per primitive, exactly where the
+   reference binding calls caml_nx_c_<op> (packages/nx/lib/backend_c/
+   nx_backend.ml:104-168,242-264,349,395-397,482-483).
+
+   Conventions shared by every compute entry point
+   - "output first": the caller allocates the result storage (nxh_alloc) and
+     passes its descriptor as the first tensor argument, as the reference does
+     (nx_backend.ml:170-183).
+   - strides and offset are in ELEMENTS and may be zero (broadcast) or negative
+     (flip) on inputs; rank <= NXH_MAX_NDIM (nx_c.h:45-61).
+   - dtype tags equal Nx's Dtype.Packed.tag (nx_c.h:130-200).
+   - every call is asynchronous on the context's stream; nxh_memcpy_d2h,
+     nxh_gather and nxh_synchronize wait for it.
+   - return value: NXH_OK, NXH_INVALID_ARGUMENT (the reference raises
+     Invalid_argument) or NXH_FAILURE (the reference raises Failure); the
+     message, prefixed "<op>: " like the reference's, is read with
+     nxh_last_error (nx_c.h:365-395, nx_c_engine.c:1345-1351). */
+
+#ifndef NXHIP_H
+#define NXHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NXH_MAX_NDIM 32
+
+/* Status kinds (nx_c_engine.c:1345-1351: which statuses become
+   Invalid_argument, which Failure). */
+enum { NXH_OK = 0, NXH_INVALID_ARGUMENT = 1, NXH_FAILURE = 2 };
+
+/* dtype tags, Dtype.Packed.tag order (nx_c.h:130-168, 197-200). */
+typedef enum {
+  NXH_F16 = 0,
+  NXH_F32 = 1,
+  NXH_F64 = 2,
+  NXH_BF16 = 3,
+  NXH_F8E4M3 = 4,
+  NXH_F8E5M2 = 5,
+  NXH_I4 = 6,
+  NXH_U4 = 7,
+  NXH_I8 = 8,
+  NXH_U8 = 9,
+  NXH_I16 = 10,
+  NXH_U16 = 11,
+  NXH_I32 = 12,
+  NXH_U32 = 13,
+  NXH_I64 = 14,
+  NXH_U64 = 15,
+  NXH_C32 = 16,
+  NXH_C64 = 17,
+  NXH_BOOL = 18,
+  NXH_DTYPE_COUNT = 19
+} nxh_dtype;
+
+/* Unary ops, Backend_intf.S order (backend_intf.ml:240-323;
+   nx_c_map.c:1184-1204). */
+typedef enum {
+  NXH_NEG = 0, NXH_RECIP, NXH_ABS, NXH_SIGN, NXH_SQRT, NXH_EXP, NXH_LOG,
+  NXH_SIN, NXH_COS, NXH_TAN, NXH_ASIN, NXH_ACOS, NXH_ATAN, NXH_SINH, NXH_COSH,
+  NXH_TANH, NXH_TRUNC, NXH_CEIL, NXH_FLOOR, NXH_ROUND, NXH_ERF,
+  NXH_UNARY_COUNT
+} nxh_unary_op;
+
+/* Binary ops (backend_intf.ml:157-228; nx_c_map.c:1207-1219). */
+typedef enum {
+  NXH_ADD = 0, NXH_SUB, NXH_MUL, NXH_IDIV, NXH_FDIV, NXH_MOD, NXH_POW,
+  NXH_ATAN2, NXH_MAX, NXH_MIN, NXH_XOR, NXH_OR, NXH_AND,
+  NXH_BINARY_COUNT
+} nxh_binary_op;
+
+/* Comparisons, bool output (backend_intf.ml:197-207; nx_c_map.c:1253-1256). */
+typedef enum {
+  NXH_CMPEQ = 0, NXH_CMPNE, NXH_CMPLT, NXH_CMPLE, NXH_COMPARE_COUNT
+} nxh_compare_op;
+
+/* Reductions (backend_intf.ml:341-351; nx_c_fold.c:824-831). */
+typedef enum {
+  NXH_SUM = 0, NXH_PROD, NXH_RMAX, NXH_RMIN, NXH_REDUCE_COUNT
+} nxh_reduce_op;
+
+/* The tensor descriptor: storage pointer + the four ABI slots of the reference
+   handle (nx_c.h:47-61, 406-412). `data` is a DEVICE pointer to storage
+   element 0 (not to the view's first element); the first live element is at
+   data + offset * elem_size. */
+typedef struct {
+  void *data;
+  int32_t dtype; /* nxh_dtype */
+  int32_t ndim;
+  int64_t offset;
+  int64_t shape[NXH_MAX_NDIM];
+  int64_t strides[NXH_MAX_NDIM];
+} nxh_tensor;
+
+typedef struct nxh_context nxh_context;
+
+/* ── Context (nx_backend.mli:32-39 create_context) ───────────────────────── */
+
+/* Creates a context on the device named by the environment variable
+   NX_HIP_DEVICE (default 0): one HIP stream, one caching allocator. Fails with
+   NXH_FAILURE when no usable GPU is present; *ctx is then NULL and the message
+   is available from nxh_last_error(NULL). */
+int nxh_context_create(nxh_context **ctx);
+void nxh_context_destroy(nxh_context *ctx);
+/* Message of the last non-OK status returned on the calling thread. */
+const char *nxh_last_error(nxh_context *ctx);
+/* Device ordinal, name, CU count of the context's GPU. */
+int nxh_device_info(nxh_context *ctx, int *device, char *name, size_t name_len,
+                    int *compute_units);
+
+/* ── Device buffers and transfer (backend_intf.ml:108-145 buffer / from_host /
+   to_host; nx_backend.ml:54-69) ──────────────────────────────────────────── */
+
+/* Bytes of `count` elements of dtype (packed int4/uint4: two per byte,
+   nx_c.h:325-328). Returns -1 for a bad tag. */
+int64_t nxh_dtype_bytes(int dtype, int64_t count);
+/* Uninitialised device block from the context's caching allocator
+   (Backend_intf.buffer). bytes == 0 yields a valid non-NULL pointer. */
+int nxh_alloc(nxh_context *ctx, size_t bytes, void **dptr);
+/* Returns a block to the allocator. Stream-ordered: kernels already queued on
+   the context stream may still use it. */
+int nxh_free(nxh_context *ctx, void *dptr);
+/* from_host: host -> device copy; the host buffer may be reused on return. */
+int nxh_memcpy_h2d(nxh_context *ctx, void *dst_device, const void *src_host,
+                   size_t bytes);
+/* to_host: waits for the stream, then device -> host copy. */
+int nxh_memcpy_d2h(nxh_context *ctx, void *dst_host, const void *src_device,
+                   size_t bytes);
+int nxh_synchronize(nxh_context *ctx);
+/* Allocator counters: bytes handed out, bytes cached in free lists, bytes
+   obtained from the driver, number of driver allocations. */
+int nxh_memory_stats(nxh_context *ctx, uint64_t *in_use, uint64_t *cached,
+                     uint64_t *reserved, uint64_t *driver_allocs);
+/* Returns every cached block to the driver. */
+int nxh_trim(nxh_context *ctx);
+
+/* full (backend_intf.ml:130-136; nx_backend.ml:61-64): every element of `out`
+   (any strides) becomes the element whose storage bytes are at `value`
+   (elem_size bytes, already encoded in the dtype's storage format). */
+int nxh_fill(nxh_context *ctx, const nxh_tensor *out, const void *value);
+
+/* ── map family (nx_c_map.c) ─────────────────────────────────────────────── */
+
+/* caml_nx_c_<unary> (nx_c_map.c:1184-1204): out[i] = op(x[i]), computed in the
+   dtype's compute type and rounded/wrapped once on store. */
+int nxh_unary(nxh_context *ctx, int op, const nxh_tensor *out,
+              const nxh_tensor *x);
+/* caml_nx_c_<binary> (nx_c_map.c:1207-1219). */
+int nxh_binary(nxh_context *ctx, int op, const nxh_tensor *out,
+               const nxh_tensor *x, const nxh_tensor *y);
+/* caml_nx_c_cmp{eq,ne,lt,le} (nx_c_map.c:1231-1256): bool (uint8 0/1) output,
+   dispatched on the input dtype. */
+int nxh_compare(nxh_context *ctx, int op, const nxh_tensor *out,
+                const nxh_tensor *x, const nxh_tensor *y);
+/* caml_nx_c_where (nx_c_map.c:809-839, 1224): storage-typed select. */
+int nxh_where(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *cond,
+              const nxh_tensor *if_true, const nxh_tensor *if_false);
+/* caml_nx_c_cast (nx_c_map.c:182-218, 1261-1280): the src x dst matrix. */
+int nxh_cast(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x);
+
+/* ── fold family (nx_c_fold.c) ───────────────────────────────────────────── */
+
+/* caml_nx_c_reduce_{sum,prod,max,min} (nx_c_fold.c:824-831; driver
+   nx_c_engine.c:1052-1170). `axes` strictly increasing; `out` is either the
+   squeezed result or the keepdims-shaped one (nx_c_engine.c:1392-1420). */
+int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out,
+               const nxh_tensor *x, const int32_t *axes, int n_axes);
+/* caml_nx_c_arg{max,min} (nx_c_fold.c:832-833; nx_c_engine.c:1214-1254):
+   int32 output; is_min = 0 for argmax, 1 for argmin. */
+int nxh_argreduce(nxh_context *ctx, int is_min, const nxh_tensor *out,
+                  const nxh_tensor *x, int axis);
+
+/* ── matmul (nx_c_matmul.c:874-1108, 1271-1277) ──────────────────────────── */
+int nxh_matmul(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *a,
+               const nxh_tensor *b);
+
+/* ── move family (nx_c_move.c) ───────────────────────────────────────────── */
+
+/* caml_nx_c_copy (nx_c_move.c:191-201): copy / contiguous / assign. */
+int nxh_copy(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x);
+/* caml_nx_c_gather (nx_c_move.c:342-458). Waits for the stream so that an
+   out-of-bounds index is reported by this call, as in the reference. */
+int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *data,
+               const nxh_tensor *indices, int axis);
+
+/* ── measurement ─────────────────────────────────────────────────────────── */
+
+/* HIP events recorded on the context stream: start, then stop returns the
+   elapsed milliseconds between them after waiting for the stop event. */
+int nxh_timer_start(nxh_context *ctx);
+int nxh_timer_stop(nxh_context *ctx, float *milliseconds);
+/* Name of the kernel path the last compute call on this thread selected
+   (e.g. "map_contig", "map_tiled", "fold_row"), for tests and profiles. */
+const char *nxh_last_path(nxh_context *ctx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NXHIP_H */

@@ -1,0 +1,255 @@
+"""numpy-facing wrapper of the CPU parity oracle (``libnxoracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the
+``cpu_baseline`` leg of ``bench.py`` — never by the product package.
+
+``OracleBackend`` has the same operation names as ``raven_amd.nx_backend`` (and
+therefore as ``Nx_core.Backend_intf.S``), but tensors are host numpy storage
+plus a ``View``; it restates what the reference binding does around each C call
+(packages/nx/lib/backend_c/nx_backend.ml).
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+from raven_amd import dtype as dt
+from raven_amd._ffi import (BINARY_OPS, COMPARE_OPS, NXH_INVALID_ARGUMENT, REDUCE_OPS,
+                            UNARY_OPS, NxhTensor, make_tensor)
+from raven_amd.view import View, c_contiguous_strides, numel
+
+HERE = Path(__file__).resolve().parent
+LIB = HERE / "libnxoracle.so"
+
+
+def build(force: bool = False) -> Path:
+    src = HERE / "nx_oracle.c"
+    if force or not LIB.exists() or LIB.stat().st_mtime < src.stat().st_mtime:
+        subprocess.run(["make", "-C", str(HERE), "-B" if force else "-s"], check=True,
+                       capture_output=True)
+    return LIB
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(str(LIB))
+        T = C.POINTER(NxhTensor)
+        L.nxo_last_error.restype = C.c_char_p
+        for name, args in {
+            "nxo_unary": [C.c_int, T, T],
+            "nxo_binary": [C.c_int, T, T, T],
+            "nxo_compare": [C.c_int, T, T, T],
+            "nxo_where": [T, T, T, T],
+            "nxo_cast": [T, T],
+            "nxo_copy": [T, T],
+            "nxo_fill": [T, C.c_void_p],
+            "nxo_reduce": [C.c_int, T, T, C.POINTER(C.c_int32), C.c_int],
+            "nxo_argreduce": [C.c_int, T, T, C.c_int],
+            "nxo_matmul": [T, T, T],
+            "nxo_gather": [T, T, T, C.c_int],
+        }.items():
+            getattr(L, name).argtypes = args
+            getattr(L, name).restype = C.c_int
+        L.nxo_f32_to_f16.argtypes = [C.c_float]
+        L.nxo_f32_to_f16.restype = C.c_uint16
+        L.nxo_f32_to_bf16.argtypes = [C.c_float]
+        L.nxo_f32_to_bf16.restype = C.c_uint16
+        L.nxo_f16_to_f32.argtypes = [C.c_uint16]
+        L.nxo_f16_to_f32.restype = C.c_float
+        L.nxo_bf16_to_f32.argtypes = [C.c_uint16]
+        L.nxo_bf16_to_f32.restype = C.c_float
+        for n in ("nxo_f32_to_f8e4m3", "nxo_f32_to_f8e5m2"):
+            getattr(L, n).argtypes = [C.c_float]
+            getattr(L, n).restype = C.c_uint8
+        for n in ("nxo_f8e4m3_to_f32", "nxo_f8e5m2_to_f32"):
+            getattr(L, n).argtypes = [C.c_uint8]
+            getattr(L, n).restype = C.c_float
+        L.nxo_set_threads.argtypes = [C.c_int]
+        L.nxo_last_threads.restype = C.c_int
+        L.nxo_ncores.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+class OTensor:
+    """Host tensor: flat numpy storage + view + dtype."""
+
+    def __init__(self, storage: np.ndarray, view: View, dtype: dt.DType):
+        self.storage = storage
+        self.view = view
+        self.dtype = dtype
+
+    @property
+    def shape(self):
+        return self.view.shape
+
+    def desc(self) -> NxhTensor:
+        return make_tensor(self.storage.ctypes.data, self.dtype.tag, self.view.shape,
+                           self.view.strides, self.view.offset)
+
+
+def _check(rc: int, op: str):
+    if rc == 0:
+        return
+    msg = f"{op}: {lib().nxo_last_error().decode()}"
+    if rc == NXH_INVALID_ARGUMENT:
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+class OracleBackend:
+    """Same surface as raven_amd.nx_backend.Backend, on the host."""
+
+    # creation ------------------------------------------------------------
+    def buffer(self, dtype: dt.DType, shape) -> OTensor:
+        n = numel(shape)
+        storage = np.zeros(dtype.nbytes(n) // max(dtype.np_storage.itemsize, 1)
+                           if not dtype.packed else (n + 1) // 2, dtype=dtype.np_storage)
+        return OTensor(storage, View.create(shape), dtype)
+
+    def from_host(self, array: np.ndarray, dtype: dt.DType) -> OTensor:
+        flat = np.ascontiguousarray(array).reshape(-1).view(dtype.np_storage).copy()
+        n = flat.size * 2 if dtype.packed else flat.size
+        return OTensor(flat, View.create((n,)), dtype)
+
+    def to_host(self, t: OTensor) -> np.ndarray:
+        return t.storage
+
+    def full(self, dtype: dt.DType, shape, value_storage: np.ndarray) -> OTensor:
+        out = self.buffer(dtype, shape)
+        v = np.ascontiguousarray(value_storage, dtype=dtype.np_storage).reshape(1)
+        _check(lib().nxo_fill(out.desc(), v.ctypes.data), "full")
+        return out
+
+    # movement ------------------------------------------------------------
+    def _mv(self, t, v):
+        return OTensor(t.storage, v, t.dtype)
+
+    def expand(self, t, shape):
+        return self._mv(t, t.view.expand(shape))
+
+    def reshape(self, t, shape):
+        return self._mv(t, t.view.reshape(shape))
+
+    def permute(self, t, axes):
+        return self._mv(t, t.view.permute(axes))
+
+    def shrink(self, t, bounds):
+        return self._mv(t, t.view.shrink(bounds))
+
+    def flip(self, t, flags):
+        return self._mv(t, t.view.flip(flags))
+
+    # map family ------------------------------------------------------------
+    def unary(self, op: str, x):
+        out = self.buffer(x.dtype, x.shape)
+        _check(lib().nxo_unary(UNARY_OPS.index(op), out.desc(), x.desc()), op)
+        return out
+
+    def binary(self, op: str, x, y):
+        out = self.buffer(x.dtype, x.shape)
+        _check(lib().nxo_binary(BINARY_OPS.index(op), out.desc(), x.desc(), y.desc()), op)
+        return out
+
+    def compare(self, op: str, x, y):
+        out = self.buffer(dt.bool_, x.shape)
+        _check(lib().nxo_compare(COMPARE_OPS.index(op), out.desc(), x.desc(), y.desc()), op)
+        return out
+
+    def where(self, cond, a, b):
+        out = self.buffer(a.dtype, a.shape)
+        _check(lib().nxo_where(out.desc(), cond.desc(), a.desc(), b.desc()), "where")
+        return out
+
+    def cast(self, x, dtype):
+        out = self.buffer(dtype, x.shape)
+        _check(lib().nxo_cast(out.desc(), x.desc()), "cast")
+        return out
+
+    def copy(self, x):
+        out = self.buffer(x.dtype, x.shape)
+        _check(lib().nxo_copy(out.desc(), x.desc()), "copy")
+        return out
+
+    def contiguous(self, x):
+        if x.view.is_c_contiguous() and x.view.offset == 0:
+            return x
+        return self.copy(x)
+
+    def assign(self, dst, src):
+        _check(lib().nxo_copy(dst.desc(), src.desc()), "copy")
+
+    # fold family -----------------------------------------------------------
+    def reduce(self, op: str, axes, x):
+        axes = sorted(int(a) for a in axes)
+        if op in ("max", "min"):
+            for a in axes:
+                if x.shape[a] == 0:
+                    raise ValueError(
+                        f"reduce_{op}: reduction over an empty axis has no identity")
+        oshape = [s for i, s in enumerate(x.shape) if i not in axes]
+        out = self.buffer(x.dtype, oshape)
+        arr = (C.c_int32 * max(len(axes), 1))(*axes)
+        _check(lib().nxo_reduce(REDUCE_OPS.index(op), out.desc(), x.desc(), arr, len(axes)),
+               f"reduce_{op}")
+        return out
+
+    def _arg(self, is_min, axis, keepdims, x):
+        name = "argmin" if is_min else "argmax"
+        if x.shape[axis] == 0:
+            raise ValueError(f"{name}: argument reduction over an empty axis")
+        oshape = [1 if i == axis else s for i, s in enumerate(x.shape)] if keepdims else \
+            [s for i, s in enumerate(x.shape) if i != axis]
+        out = self.buffer(dt.int32, oshape)
+        _check(lib().nxo_argreduce(int(is_min), out.desc(), x.desc(), axis), name)
+        return out
+
+    def argmax(self, x, axis, keepdims=False):
+        return self._arg(False, axis, keepdims, x)
+
+    def argmin(self, x, axis, keepdims=False):
+        return self._arg(True, axis, keepdims, x)
+
+    # matmul / gather ---------------------------------------------------------
+    def matmul(self, x, y):
+        xs, ys = x.shape, y.shape
+        nd = max(len(xs), len(ys))
+        batch = []
+        for i in range(nd - 2):
+            ai, bi = i - (nd - len(xs)), i - (nd - len(ys))
+            batch.append(max(xs[ai] if ai >= 0 else 1, ys[bi] if bi >= 0 else 1))
+        out = self.buffer(x.dtype, batch + [xs[-2], ys[-1]])
+        _check(lib().nxo_matmul(out.desc(), x.desc(), y.desc()), "matmul")
+        return out
+
+    def gather(self, data, indices, axis):
+        out = self.buffer(data.dtype, indices.shape)
+        _check(lib().nxo_gather(out.desc(), data.desc(), indices.desc(), axis), "gather")
+        return out
+
+
+def logical(t: OTensor) -> np.ndarray:
+    """The tensor's logical contents as a numpy array of its storage dtype."""
+    if t.dtype.packed:
+        raise NotImplementedError
+    es = t.storage.dtype.itemsize
+    v = t.view
+    if v.numel == 0:
+        return np.zeros(v.shape, dtype=t.storage.dtype)
+    return np.lib.stride_tricks.as_strided(
+        t.storage[v.offset:] if all(s >= 0 for s in v.strides) else
+        _neg_base(t.storage, v), shape=v.shape,
+        strides=[s * es for s in v.strides]).copy()
+
+
+def _neg_base(storage, v):
+    return storage[v.offset:]
