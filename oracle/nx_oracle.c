@@ -1026,7 +1026,32 @@ NXO_EXPORT int nxo_where(const nxh_tensor *out, const nxh_tensor *cond,
   if (es[0] == 0) return fail(NXH_FAILURE, ERR_PACKED);
   return map_run(t_where.fn[out->dtype], out->dtype, 3, ops, es, COST_BANDWIDTH);
 }
+static bool dense_off0(const nxh_tensor *a) {
+  if (a->offset != 0) return false;
+  int64_t e = 1;
+  for (int i = a->ndim - 1; i >= 0; i--) {
+    if (a->shape[i] == 1) continue;
+    if (a->strides[i] != e) return false;
+    e *= a->shape[i];
+  }
+  return true;
+}
+/* caml_nx_c_copy (nx_c_move.c:191-201); packed dtypes: whole contiguous
+   offset-0 buffers only, the odd trailing nibble merged (nx_c_move.c:143-189) */
 NXO_EXPORT int nxo_copy(const nxh_tensor *out, const nxh_tensor *x) {
+  if (is_packed(out->dtype)) {
+    int64_t n = 1, nx = 1;
+    for (int i = 0; i < out->ndim; i++) n *= out->shape[i];
+    for (int i = 0; i < x->ndim; i++) nx *= x->shape[i];
+    if (n != nx || !dense_off0(out) || !dense_off0(x)) return fail(NXH_FAILURE, ERR_PACKED);
+    memcpy(out->data, x->data, (size_t)(n / 2));
+    if (n & 1) {
+      uint8_t *d = (uint8_t *)out->data + n / 2;
+      const uint8_t *sp = (const uint8_t *)x->data + n / 2;
+      *d = (uint8_t)((*d & 0xF0) | (*sp & 0x0F));
+    }
+    return NXH_OK;
+  }
   if (!check_same_shape(out, x)) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
   const nxh_tensor *ops[2] = {out, x};
   int64_t es[2] = {nxo_elem_size(out->dtype), nxo_elem_size(x->dtype)};

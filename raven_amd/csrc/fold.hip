@@ -1,0 +1,950 @@
+// fold.hip — reductions (sum, prod, max, min) and argmax/argmin.
+//
+// Semantics restate packages/nx/lib/backend_c/nx_c_fold.c:63-101 (combine
+// rules, NaN propagation, first-index ties) with the reference's accumulator
+// widths (nx_c.h:109-116: f16/bf16/fp8 -> f32, small ints -> int64, u32/u64 ->
+// uint64, wrap on store). The driver (nx_c_engine.c:1052-1254) is replaced by a
+// planner that picks, per call:
+//   fold_row   the reduced extent is one unit-stride run: a wave (short rows) or
+//              a 256-lane block (long rows) per output, 16-byte loads, wave64
+//              shuffle + LDS combine; long rows with few outputs are split into
+//              chunks and finished by a second pass over the partials.
+//   fold_col   a kept dim is the unit-stride one (axis-0 style): each lane owns
+//              up to four adjacent output columns and walks the reduced rows;
+//              rows are split across blocks with a second pass over partials.
+//   fold_any   everything else: one lane per output, odometer over the reduced
+//              dims.
+// Float sums are reassociated (tree order); results agree with the reference
+// within its own tolerance, integer results are exact (modular).
+
+#include <algorithm>
+#include <type_traits>
+
+#include "nxh_common.hpp"
+
+constexpr int FOLD_MAXD = 12;
+constexpr int FOLD_THREADS = 256;
+
+static inline bool aligned_to16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// ── combine rules ───────────────────────────────────────────────────────────
+template <int OP, class C, Cat cat>
+struct Combine {
+  __device__ __forceinline__ static C init() {
+    if constexpr (OP == NXH_SUM) {
+      if constexpr (cat == CAT_COMPLEX) return C{0, 0};
+      else return (C)0;
+    } else if constexpr (OP == NXH_PROD) {
+      if constexpr (cat == CAT_COMPLEX) return C{1, 0};
+      else return (C)1;
+    } else if constexpr (OP == NXH_RMAX) {
+      if constexpr (cat == CAT_FLOAT) return (C)(-__builtin_inff());
+      else if constexpr (cat == CAT_SINT || (cat == CAT_UINT && std::is_signed<C>::value)) return (C)INT64_MIN;
+      else return (C)0;
+    } else {
+      if constexpr (cat == CAT_FLOAT) return (C)__builtin_inff();
+      else if constexpr (cat == CAT_BOOL) return (C)1;
+      else if constexpr (std::is_signed<C>::value) return (C)INT64_MAX;
+      else return (C)UINT64_MAX;
+    }
+  }
+  __device__ __forceinline__ static C apply(C m, C v) {
+    if constexpr (OP == NXH_SUM) {
+      if constexpr (cat == CAT_SINT) return (C)((uint64_t)m + (uint64_t)v);
+      else return m + v;
+    } else if constexpr (OP == NXH_PROD) {
+      if constexpr (cat == CAT_SINT) return (C)((uint64_t)m * (uint64_t)v);
+      else return m * v;
+    } else if constexpr (OP == NXH_RMAX) {
+      if constexpr (cat == CAT_FLOAT) return (v > m) ? v : ((v != v) ? v : m);
+      else if constexpr (cat == CAT_BOOL) return (C)(m | v);
+      else return v > m ? v : m;
+    } else {
+      if constexpr (cat == CAT_FLOAT) return (v < m) ? v : ((v != v) ? v : m);
+      else if constexpr (cat == CAT_BOOL) return (C)(m & v);
+      else return v < m ? v : m;
+    }
+  }
+};
+constexpr bool fold_ok(int op, Cat c) {
+  return (op == NXH_SUM || op == NXH_PROD) ? (c != CAT_BOOL) : (c != CAT_COMPLEX);
+}
+
+// ── lane exchange for any trivially copyable accumulator ───────────────────
+template <class T>
+__device__ __forceinline__ T shfl_down_any(T v, int delta) {
+  constexpr int W = (sizeof(T) + 3) / 4;
+  union {
+    T t;
+    uint32_t w[W];
+  } u;
+  u.w[W - 1] = 0;
+  u.t = v;
+#pragma unroll
+  for (int i = 0; i < W; i++) u.w[i] = __shfl_down(u.w[i], delta, 64);
+  return u.t;
+}
+
+// Reduces `acc` over a group of G lanes (64: one wave; 256: the block). The
+// result is valid in the group's first lane.
+template <class CB, class C, int G>
+__device__ __forceinline__ C group_reduce(C acc, C *lds) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) acc = CB::apply(acc, shfl_down_any(acc, d));
+  if constexpr (G == 256) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) lds[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) acc = CB::apply(CB::apply(lds[0], lds[1]), CB::apply(lds[2], lds[3]));
+  }
+  return acc;
+}
+
+// Input / output adaptors: storage-typed (through the dtype converters) or raw
+// compute-typed partials between the two passes.
+template <int DT>
+struct InS {
+  using T = typename Tr<DT>::S;
+  using C = typename Tr<DT>::C;
+  __device__ __forceinline__ static C ld(T s) { return Tr<DT>::ld(s); }
+};
+template <class C_>
+struct InC {
+  using T = C_;
+  using C = C_;
+  __device__ __forceinline__ static C ld(T s) { return s; }
+};
+template <int DT>
+struct OutS {
+  using T = typename Tr<DT>::S;
+  __device__ __forceinline__ static T st(typename Tr<DT>::C c) { return Tr<DT>::st(c); }
+};
+template <class C_>
+struct OutC {
+  using T = C_;
+  __device__ __forceinline__ static T st(C_ c) { return c; }
+};
+
+template <class T, int N>
+struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) FVec {
+  T v[N];
+};
+
+struct FoldDims {
+  int n;
+  uint32_t shape[FOLD_MAXD];
+  int64_t in_stride[FOLD_MAXD];
+  int64_t out_stride[FOLD_MAXD];
+};
+__device__ __forceinline__ void fold_decode(const FoldDims &d, uint64_t idx, int64_t &in_off,
+                                            int64_t &out_off) {
+  in_off = 0;
+  out_off = 0;
+  for (int i = d.n - 1; i >= 0; i--) {
+    uint64_t q = idx / d.shape[i];
+    uint32_t c = (uint32_t)(idx - q * d.shape[i]);
+    idx = q;
+    in_off += (int64_t)c * d.in_stride[i];
+    out_off += (int64_t)c * d.out_stride[i];
+  }
+}
+
+// ── fold_row ────────────────────────────────────────────────────────────────
+struct RowArgs {
+  const void *in;
+  void *out;
+  FoldDims kept;      // output index -> offsets
+  uint64_t n_out;     // number of outputs
+  int64_t R;          // reduced run length (unit stride)
+  int64_t chunk;      // elements per split (== R when unsplit)
+  int nsplit;         // > 1: out is partial[o * nsplit + c], compute-typed
+};
+
+template <class IN, class CB, class OUT, int G, int V>
+__global__ __launch_bounds__(FOLD_THREADS) void fold_row_kernel(RowArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  __shared__ C lds[4];
+  constexpr int GROUPS = FOLD_THREADS / G;
+  const int lane = threadIdx.x % G;
+  const uint64_t o = (uint64_t)blockIdx.x * GROUPS + threadIdx.x / G;
+  const bool live = o < a.n_out;
+  const int c = blockIdx.y;
+  int64_t in_off = 0, out_off = 0;
+  if (live) fold_decode(a.kept, o, in_off, out_off);
+  const int64_t r0 = (int64_t)c * a.chunk;
+  const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
+  const T *p = (const T *)a.in + in_off;
+  C acc0 = CB::init(), acc1 = CB::init(), acc2 = CB::init(), acc3 = CB::init();
+  const int64_t nv = (r1 - r0) / V;
+  const FVec<T, V> *pv = reinterpret_cast<const FVec<T, V> *>(p + r0);
+  int64_t i = lane;
+  for (; i + 3 * G < nv; i += 4 * G) {
+    FVec<T, V> x0 = pv[i], x1 = pv[i + G], x2 = pv[i + 2 * G], x3 = pv[i + 3 * G];
+#pragma unroll
+    for (int k = 0; k < V; k++) {
+      acc0 = CB::apply(acc0, IN::ld(x0.v[k]));
+      acc1 = CB::apply(acc1, IN::ld(x1.v[k]));
+      acc2 = CB::apply(acc2, IN::ld(x2.v[k]));
+      acc3 = CB::apply(acc3, IN::ld(x3.v[k]));
+    }
+  }
+  for (; i < nv; i += G) {
+    FVec<T, V> x0 = pv[i];
+#pragma unroll
+    for (int k = 0; k < V; k++) acc0 = CB::apply(acc0, IN::ld(x0.v[k]));
+  }
+  for (int64_t e = r0 + nv * V + lane; e < r1; e += G) acc1 = CB::apply(acc1, IN::ld(p[e]));
+  C acc = CB::apply(CB::apply(acc0, acc1), CB::apply(acc2, acc3));
+  acc = group_reduce<CB, C, G>(acc, lds);
+  if (live && lane == 0) {
+    if (a.nsplit > 1) ((C *)a.out)[o * a.nsplit + c] = acc;
+    else ((typename OUT::T *)a.out)[out_off] = OUT::st(acc);
+  }
+}
+
+// ── fold_col ────────────────────────────────────────────────────────────────
+struct ColArgs {
+  const void *in;
+  void *out;
+  FoldDims outer;       // kept dims other than the lane dim
+  uint64_t n_outer;
+  uint32_t L;           // lane extent (unit input stride)
+  uint32_t lane_blocks; // blocks along the lane dim
+  int64_t out_lane_stride;
+  int64_t R, r_stride;  // reduced extent and its input stride
+  int64_t chunk;
+  int nsplit;           // > 1: out is partial[(c * n_outer + ob) * L + l]
+};
+
+template <class IN, class CB, class OUT, int V>
+__global__ __launch_bounds__(FOLD_THREADS) void fold_col_kernel(ColArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  const uint32_t lb = blockIdx.x % a.lane_blocks;
+  const uint64_t ob = blockIdx.x / a.lane_blocks;
+  const int c = blockIdx.y;
+  const uint32_t l = (lb * FOLD_THREADS + threadIdx.x) * V;
+  if (l >= a.L) return;
+  int64_t in_off, out_off;
+  fold_decode(a.outer, ob, in_off, out_off);
+  const int64_t r0 = (int64_t)c * a.chunk;
+  const int64_t r1 = r0 + a.chunk < a.R ? r0 + a.chunk : a.R;
+  const T *p = (const T *)a.in + in_off + l;
+  C acc[V];
+#pragma unroll
+  for (int k = 0; k < V; k++) acc[k] = CB::init();
+  int64_t r = r0;
+  for (; r + 4 <= r1; r += 4) {
+    FVec<T, V> x[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j) * a.r_stride);
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x[j].v[k]));
+  }
+  for (; r < r1; r++) {
+    FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
+#pragma unroll
+    for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x.v[k]));
+  }
+  if (a.nsplit > 1) {
+    C *o = (C *)a.out + ((uint64_t)c * a.n_outer + ob) * a.L + l;
+#pragma unroll
+    for (int k = 0; k < V; k++) o[k] = acc[k];
+  } else {
+    typename OUT::T *o = (typename OUT::T *)a.out + out_off + (int64_t)l * a.out_lane_stride;
+#pragma unroll
+    for (int k = 0; k < V; k++) o[(int64_t)k * a.out_lane_stride] = OUT::st(acc[k]);
+  }
+}
+
+// ── fold_any ────────────────────────────────────────────────────────────────
+struct AnyArgs {
+  const void *in;
+  void *out;
+  FoldDims kept;
+  uint64_t n_out;
+  int nr;
+  uint32_t rshape[FOLD_MAXD];
+  int64_t rstride[FOLD_MAXD];
+  uint64_t R;
+};
+template <class IN, class CB, class OUT>
+__global__ __launch_bounds__(FOLD_THREADS) void fold_any_kernel(AnyArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  const uint64_t o = (uint64_t)blockIdx.x * FOLD_THREADS + threadIdx.x;
+  if (o >= a.n_out) return;
+  int64_t in_off, out_off;
+  fold_decode(a.kept, o, in_off, out_off);
+  const T *p = (const T *)a.in + in_off;
+  uint32_t coord[FOLD_MAXD];
+  for (int d = 0; d < a.nr; d++) coord[d] = 0;
+  C acc = CB::init();
+  int64_t off = 0;
+  for (uint64_t r = 0; r < a.R; r++) {
+    acc = CB::apply(acc, IN::ld(p[off]));
+    for (int d = a.nr - 1; d >= 0; d--) {
+      if (++coord[d] < a.rshape[d]) {
+        off += a.rstride[d];
+        break;
+      }
+      coord[d] = 0;
+      off -= (int64_t)(a.rshape[d] - 1) * a.rstride[d];
+    }
+  }
+  ((typename OUT::T *)a.out)[out_off] = OUT::st(acc);
+}
+
+// ── argmax / argmin (nx_c_fold.c:93-101, 180-198) ──────────────────────────
+// `beats(v, b)`: v displaces the running best b. Strict, and a NaN displaces a
+// non-NaN, so among equal candidates the smaller index is kept explicitly.
+template <bool IS_MIN, class C, Cat cat>
+struct ArgCmp {
+  __device__ __forceinline__ static bool beats(C v, C b) {
+    if constexpr (cat == CAT_FLOAT) {
+      if constexpr (IS_MIN) return (v < b) || ((v != v) && !(b != b));
+      else return (v > b) || ((v != v) && !(b != b));
+    } else {
+      if constexpr (IS_MIN) return v < b;
+      else return v > b;
+    }
+  }
+  // merge two (value, index) candidates; index < 0 means "none yet"
+  __device__ __forceinline__ static void merge(C &bv, int64_t &bi, C v, int64_t i) {
+    if (i < 0) return;
+    if (bi < 0 || beats(v, bv) || (!beats(bv, v) && i < bi)) {
+      bv = v;
+      bi = i;
+    }
+  }
+};
+
+struct ArgArgs {
+  const void *in;         // values (storage-typed first pass, compute-typed second)
+  const int32_t *in_idx;  // second pass only: index carried by each partial
+  void *out_val;          // first pass with nsplit > 1: partial values (compute-typed)
+  int32_t *out_idx;       // int32 result, or partial indices
+  FoldDims kept;          // row form: all kept dims; col form: kept dims other than the lane
+  uint64_t n_out;
+  int64_t R, r_stride;
+  int64_t chunk;
+  int nsplit;
+  uint32_t L, lane_blocks;  // col form
+  int64_t out_lane_stride;
+};
+
+// Row form: a group of G lanes per output, strided lanes over the axis.
+template <class IN, class CMP, int G, bool HAS_IDX>
+__global__ __launch_bounds__(FOLD_THREADS) void arg_row_kernel(ArgArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  __shared__ C lv[4];
+  __shared__ int64_t li[4];
+  constexpr int GROUPS = FOLD_THREADS / G;
+  const int lane = threadIdx.x % G;
+  const uint64_t o = (uint64_t)blockIdx.x * GROUPS + threadIdx.x / G;
+  const bool live = o < a.n_out;
+  const int c = blockIdx.y;
+  int64_t in_off = 0, out_off = 0;
+  if (live) fold_decode(a.kept, o, in_off, out_off);
+  const int64_t r0 = (int64_t)c * a.chunk;
+  const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
+  const T *p = (const T *)a.in + in_off;
+  C bv{};
+  int64_t bi = -1;
+  for (int64_t r = r0 + lane; r < r1; r += G) {
+    C v = IN::ld(p[r * a.r_stride]);
+    int64_t idx = HAS_IDX ? (int64_t)a.in_idx[in_off + r * a.r_stride] : r;
+    CMP::merge(bv, bi, v, idx);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    C ov = shfl_down_any(bv, d);
+    int64_t oi = shfl_down_any(bi, d);
+    CMP::merge(bv, bi, ov, oi);
+  }
+  if constexpr (G == 256) {
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+      lv[wave] = bv;
+      li[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+      for (int w = 1; w < 4; w++) CMP::merge(bv, bi, lv[w], li[w]);
+  }
+  if (live && lane == 0) {
+    if (a.nsplit > 1) {
+      ((C *)a.out_val)[o * a.nsplit + c] = bv;
+      a.out_idx[o * a.nsplit + c] = (int32_t)bi;
+    } else {
+      a.out_idx[out_off] = (int32_t)bi;
+    }
+  }
+}
+
+// Column form: one lane per output column, rows walked in order.
+template <class IN, class CMP, bool HAS_IDX>
+__global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  const uint32_t lb = blockIdx.x % a.lane_blocks;
+  const uint64_t ob = blockIdx.x / a.lane_blocks;
+  const int c = blockIdx.y;
+  const uint32_t l = lb * FOLD_THREADS + threadIdx.x;
+  if (l >= a.L) return;
+  int64_t in_off, out_off;
+  fold_decode(a.kept, ob, in_off, out_off);
+  const int64_t r0 = (int64_t)c * a.chunk;
+  const int64_t r1 = r0 + a.chunk < a.R ? r0 + a.chunk : a.R;
+  const T *p = (const T *)a.in + in_off + l;
+  C bv{};
+  int64_t bi = -1;
+  int64_t r = r0;
+  for (; r + 4 <= r1; r += 4) {
+    T x[4];
+    int32_t xi[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      x[j] = p[(r + j) * a.r_stride];
+      if (HAS_IDX) xi[j] = a.in_idx[in_off + l + (r + j) * a.r_stride];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) CMP::merge(bv, bi, IN::ld(x[j]), HAS_IDX ? (int64_t)xi[j] : r + j);
+  }
+  for (; r < r1; r++)
+    CMP::merge(bv, bi, IN::ld(p[r * a.r_stride]),
+               HAS_IDX ? (int64_t)a.in_idx[in_off + l + r * a.r_stride] : r);
+  if (a.nsplit > 1) {
+    uint64_t po = ((uint64_t)c * a.n_out + ob) * a.L + l;
+    ((C *)a.out_val)[po] = bv;
+    a.out_idx[po] = (int32_t)bi;
+  } else {
+    a.out_idx[out_off + (int64_t)l * a.out_lane_stride] = (int32_t)bi;
+  }
+}
+
+// ── host: geometry ──────────────────────────────────────────────────────────
+struct Geom {
+  int nk = 0, nr = 0;
+  int64_t kshape[NXH_MAX_NDIM], kin[NXH_MAX_NDIM], kout[NXH_MAX_NDIM];
+  int64_t rshape[NXH_MAX_NDIM], rin[NXH_MAX_NDIM];
+  int64_t n_out = 1, R = 1;
+};
+
+// Splits dims into kept / reduced (strides in elements), drops size-1 dims and
+// merges neighbours of the same class that compose.
+static void geom_build(const nxh_tensor *in, const nxh_tensor *out_sq, const bool *reduced, Geom *g) {
+  int oj = 0;
+  int last_class = -1;  // 0 kept, 1 reduced: merging needs ADJACENT dims of one class
+  for (int a = 0; a < in->ndim; a++) {
+    int64_t s = in->shape[a], st = in->strides[a];
+    if (reduced[a]) {
+      g->R *= s;
+      if (s != 1) {
+        if (last_class == 1 && g->rin[g->nr - 1] == st * s) {
+          g->rshape[g->nr - 1] *= s;
+          g->rin[g->nr - 1] = st;
+        } else {
+          g->rshape[g->nr] = s;
+          g->rin[g->nr++] = st;
+        }
+        last_class = 1;
+      }
+    } else {
+      int64_t so = out_sq->strides[oj++];
+      g->n_out *= s;
+      if (s != 1) {
+        if (last_class == 0 && g->kin[g->nk - 1] == st * s && g->kout[g->nk - 1] == so * s) {
+          g->kshape[g->nk - 1] *= s;
+          g->kin[g->nk - 1] = st;
+          g->kout[g->nk - 1] = so;
+        } else {
+          g->kshape[g->nk] = s;
+          g->kin[g->nk] = st;
+          g->kout[g->nk++] = so;
+        }
+        last_class = 0;
+      }
+    }
+  }
+}
+
+static bool dims_fill(FoldDims *d, int n, const int64_t *shape, const int64_t *in_s, const int64_t *out_s,
+                      int skip = -1) {
+  d->n = 0;
+  for (int i = 0; i < n; i++) {
+    if (i == skip) continue;
+    if (d->n >= FOLD_MAXD || shape[i] > 0xffffffffLL) return false;
+    d->shape[d->n] = (uint32_t)shape[i];
+    d->in_stride[d->n] = in_s[i];
+    d->out_stride[d->n] = out_s ? out_s[i] : 0;
+    d->n++;
+  }
+  return true;
+}
+// Contiguous (row-major) input strides over the same kept shape, scaled.
+static void dims_contig_in(FoldDims *d, int64_t inner) {
+  int64_t acc = inner;
+  for (int i = d->n - 1; i >= 0; i--) {
+    d->in_stride[i] = acc;
+    acc *= d->shape[i];
+  }
+}
+
+struct Scratch {
+  nxh_context *ctx;
+  void *p[2] = {nullptr, nullptr};
+  explicit Scratch(nxh_context *c) : ctx(c) {}
+  int get(int i, size_t bytes) { return nxh_alloc_locked(ctx, bytes, &p[i]); }
+  ~Scratch() {  // stream-ordered: queued kernels keep using the blocks safely
+    for (void *q : p)
+      if (q) nxh_free_locked(ctx, q);
+  }
+};
+
+static int pick_split(int64_t blocks, int64_t R, int64_t min_chunk, int cus) {
+  // aim for ~8 blocks per CU when a single pass would leave the chip idle
+  const int64_t target = (int64_t)cus * 8;
+  if (blocks >= target / 2 || R < 2 * min_chunk) return 1;
+  int64_t want = (target + blocks - 1) / blocks;
+  int64_t cap = R / min_chunk;
+  int64_t s = std::min<int64_t>(std::min(want, cap), 1024);
+  return (int)std::max<int64_t>(s, 1);
+}
+
+template <int OP, int DT>
+static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, const nxh_tensor *out,
+                       const Geom &g) {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  using S = typename TR::S;
+  using CB = Combine<OP, C, TR::cat>;
+  constexpr int V = 16 / (int)sizeof(S) > 0 ? 16 / (int)sizeof(S) : 1;
+  constexpr int VC = 16 / (int)sizeof(C) > 0 ? 16 / (int)sizeof(C) : 1;
+  const S *ibase = (const S *)in->data + in->offset;
+  S *obase = (S *)out->data + out->offset;
+  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  Scratch scratch(ctx);
+
+  // ---- fold_row: one unit-stride reduced run ----
+  if (g.nr == 1 && g.rin[0] == 1 && g.R >= 64 && g.n_out <= 0x7fffffffLL * 4) {
+    RowArgs a;
+    if (dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout)) {
+      a.in = ibase;
+      a.n_out = (uint64_t)g.n_out;
+      a.R = g.R;
+      const bool wave_rows = g.R < 1024;
+      const int64_t blocks = wave_rows ? (g.n_out + 3) / 4 : g.n_out;
+      int nsplit = wave_rows ? 1 : pick_split(blocks, g.R, 8192, cus);
+      int64_t chunk = g.R;
+      if (nsplit > 1) {
+        chunk = (g.R + nsplit - 1) / nsplit;
+        chunk = (chunk + 63) / 64 * 64;  // keeps every chunk start 16-byte aligned
+        nsplit = (int)((g.R + chunk - 1) / chunk);
+      }
+      a.chunk = chunk;
+      a.nsplit = nsplit;
+      bool vec = aligned_to16(ibase);
+      for (int i = 0; vec && i < g.nk; i++)
+        if (g.kin[i] % V != 0) vec = false;
+      if (nsplit > 1) {
+        int rc = scratch.get(0, (size_t)g.n_out * nsplit * sizeof(C));
+        if (rc) return rc;
+        a.out = scratch.p[0];
+      } else {
+        a.out = obase;
+      }
+      dim3 grid((unsigned)blocks, (unsigned)nsplit);
+      nxh_set_path(nsplit > 1 ? "fold_row_split" : (wave_rows ? "fold_row_wave" : "fold_row"));
+      if (wave_rows) {
+        if (vec) hipLaunchKernelGGL((fold_row_kernel<InS<DT>, CB, OutS<DT>, 64, V>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((fold_row_kernel<InS<DT>, CB, OutS<DT>, 64, 1>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+      } else {
+        if (vec) hipLaunchKernelGGL((fold_row_kernel<InS<DT>, CB, OutS<DT>, 256, V>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((fold_row_kernel<InS<DT>, CB, OutS<DT>, 256, 1>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+      }
+      NXH_HIP(op, hipGetLastError());
+      if (nsplit > 1) {
+        RowArgs b = a;
+        b.in = scratch.p[0];
+        b.out = obase;
+        dims_contig_in(&b.kept, nsplit);
+        b.R = nsplit;
+        b.chunk = nsplit;
+        b.nsplit = 1;
+        dim3 grid2((unsigned)((g.n_out + 3) / 4), 1);
+        hipLaunchKernelGGL((fold_row_kernel<InC<C>, CB, OutS<DT>, 64, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+        NXH_HIP(op, hipGetLastError());
+      }
+      return NXH_OK;
+    }
+  }
+
+  // ---- fold_col: a kept dim is the unit-stride one ----
+  if (g.nr == 1 && g.nk >= 1) {
+    int lane = -1;
+    for (int j = 0; j < g.nk; j++)
+      if (g.kin[j] == 1 && g.kshape[j] >= 16 && g.kshape[j] <= 0x7fffffffLL) lane = j;
+    ColArgs a;
+    if (lane >= 0 && std::llabs(g.rin[0]) > 1 && dims_fill(&a.outer, g.nk, g.kshape, g.kin, g.kout, lane)) {
+      const int64_t L = g.kshape[lane];
+      const int64_t n_outer = g.n_out / L;
+      bool vec = aligned_to16(ibase) && L % V == 0 && g.rin[0] % V == 0;
+      for (int i = 0; vec && i < g.nk; i++)
+        if (i != lane && g.kin[i] % V != 0) vec = false;
+      const int v = vec ? V : 1;
+      const int64_t lane_blocks = (L + (int64_t)FOLD_THREADS * v - 1) / ((int64_t)FOLD_THREADS * v);
+      const int64_t blocks = lane_blocks * n_outer;
+      if (blocks <= 0x7fffffffLL) {
+        int nsplit = pick_split(blocks, g.R, 16, cus);
+        int64_t chunk = (g.R + nsplit - 1) / nsplit;
+        nsplit = (int)((g.R + chunk - 1) / chunk);
+        a.in = ibase;
+        a.n_outer = (uint64_t)n_outer;
+        a.L = (uint32_t)L;
+        a.lane_blocks = (uint32_t)lane_blocks;
+        a.out_lane_stride = g.kout[lane];
+        a.R = g.R;
+        a.r_stride = g.rin[0];
+        a.chunk = chunk;
+        a.nsplit = nsplit;
+        if (nsplit > 1) {
+          int rc = scratch.get(0, (size_t)nsplit * g.n_out * sizeof(C));
+          if (rc) return rc;
+          a.out = scratch.p[0];
+        } else {
+          a.out = obase;
+        }
+        dim3 grid((unsigned)blocks, (unsigned)nsplit);
+        nxh_set_path(nsplit > 1 ? "fold_col_split" : "fold_col");
+        if (vec) hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, V>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        else hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, 1>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        NXH_HIP(op, hipGetLastError());
+        if (nsplit > 1) {
+          ColArgs b = a;
+          b.in = scratch.p[0];
+          b.out = obase;
+          dims_contig_in(&b.outer, L);
+          b.R = nsplit;
+          b.r_stride = g.n_out;
+          b.chunk = nsplit;
+          b.nsplit = 1;
+          const bool vec2 = L % VC == 0;
+          const int v2 = vec2 ? VC : 1;
+          b.lane_blocks = (uint32_t)((L + (int64_t)FOLD_THREADS * v2 - 1) / ((int64_t)FOLD_THREADS * v2));
+          dim3 grid2((unsigned)(b.lane_blocks * n_outer), 1);
+          if (vec2) hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, VC>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+          else hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+          NXH_HIP(op, hipGetLastError());
+        }
+        return NXH_OK;
+      }
+    }
+  }
+
+  // ---- fold_any ----
+  AnyArgs a;
+  if (!dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout) || g.nr > FOLD_MAXD)
+    return nxh_fail(NXH_FAILURE, op, "view has too many non-mergeable dimensions for one launch");
+  a.in = ibase;
+  a.out = obase;
+  a.n_out = (uint64_t)g.n_out;
+  a.nr = g.nr;
+  a.R = (uint64_t)g.R;
+  // the smallest-|stride| reduced dim runs innermost (nx_c_engine.c:1151-1164)
+  int64_t rs[NXH_MAX_NDIM], rst[NXH_MAX_NDIM];
+  for (int d = 0; d < g.nr; d++) {
+    rs[d] = g.rshape[d];
+    rst[d] = g.rin[d];
+  }
+  if (g.nr > 1) {
+    int best = 0;
+    for (int r = 1; r < g.nr; r++)
+      if (std::llabs(rst[r]) < std::llabs(rst[best])) best = r;
+    std::swap(rs[best], rs[g.nr - 1]);
+    std::swap(rst[best], rst[g.nr - 1]);
+  }
+  for (int d = 0; d < g.nr; d++) {
+    if (rs[d] > 0xffffffffLL) return nxh_fail(NXH_FAILURE, op, "reduced dimension too large");
+    a.rshape[d] = (uint32_t)rs[d];
+    a.rstride[d] = rst[d];
+  }
+  const uint64_t blocks = ((uint64_t)g.n_out + FOLD_THREADS - 1) / FOLD_THREADS;
+  if (blocks > 0x7fffffffULL) return nxh_fail(NXH_FAILURE, op, "too many outputs for one launch");
+  nxh_set_path("fold_any");
+  hipLaunchKernelGGL((fold_any_kernel<InS<DT>, CB, OutS<DT>>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+typedef int (*fold_fn)(nxh_context *, const char *, const nxh_tensor *, const nxh_tensor *, const Geom &);
+template <int OP>
+struct FoldRow {
+  fold_fn fn[NXH_DTYPE_COUNT] = {};
+  template <int DT>
+  void set() {
+    if constexpr (fold_ok(OP, Tr<DT>::cat)) fn[DT] = &fold_launch<OP, DT>;
+  }
+  FoldRow() {
+#define NXH_SET(DT) set<DT>();
+    NXH_FOR_COMPUTE_DTYPES(NXH_SET)
+#undef NXH_SET
+  }
+};
+
+// nx_c_engine.c:1392-1420: accept a squeezed or a keepdims-shaped output.
+static int squeeze_out(const char *op, const nxh_tensor *in, const nxh_tensor *out, const int32_t *axes,
+                       int nred, bool *reduced, nxh_tensor *sq) {
+  if (nred < 0 || nred > in->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXES);
+  for (int a = 0; a < in->ndim; a++) reduced[a] = false;
+  for (int i = 0; i < nred; i++) {
+    int a = axes[i];
+    if (a < 0 || a >= in->ndim || reduced[a]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXES);
+    if (i > 0 && axes[i] <= axes[i - 1]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXES);
+    reduced[a] = true;
+  }
+  const int kept = in->ndim - nred;
+  *sq = *out;
+  if (out->ndim != kept) {
+    if (out->ndim != in->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_RANK);
+    sq->ndim = kept;
+    int j = 0;
+    for (int a = 0; a < in->ndim; a++)
+      if (!reduced[a]) {
+        sq->shape[j] = out->shape[a];
+        sq->strides[j] = out->strides[a];
+        j++;
+      }
+  }
+  int j = 0;
+  for (int a = 0; a < in->ndim; a++)
+    if (!reduced[a]) {
+      if (sq->shape[j] != in->shape[a]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+      j++;
+    }
+  return NXH_OK;
+}
+
+// The value 1 in each dtype's storage format, for prod over an empty extent.
+static void storage_one(int dt, void *buf) {
+  memset(buf, 0, 16);
+  switch (dt) {
+    case NXH_F16: *(uint16_t *)buf = 0x3c00; break;
+    case NXH_BF16: *(uint16_t *)buf = 0x3f80; break;
+    case NXH_F32: *(float *)buf = 1.0f; break;
+    case NXH_F64: *(double *)buf = 1.0; break;
+    case NXH_F8E4M3: *(uint8_t *)buf = 0x38; break;
+    case NXH_F8E5M2: *(uint8_t *)buf = 0x3c; break;
+    case NXH_C32: *(float *)buf = 1.0f; break;
+    case NXH_C64: *(double *)buf = 1.0; break;
+    default: *(uint8_t *)buf = 1; break;  // little-endian integers of any width
+  }
+}
+
+NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
+                          const int32_t *axes, int n_axes) {
+  static const char *const names[NXH_REDUCE_COUNT] = {"reduce_sum", "reduce_prod", "reduce_max", "reduce_min"};
+  if ((unsigned)op >= NXH_REDUCE_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "reduce", "unknown op");
+  const char *name = names[op];
+  if (!ctx || !out || !x || (n_axes > 0 && !axes)) return nxh_fail(NXH_INVALID_ARGUMENT, name, "null argument");
+  int rc = nxh_check_tensor(name, out);
+  if (!rc) rc = nxh_check_tensor(name, x);
+  if (rc) return rc;
+  static const FoldRow<NXH_SUM> row_sum;
+  static const FoldRow<NXH_PROD> row_prod;
+  static const FoldRow<NXH_RMAX> row_max;
+  static const FoldRow<NXH_RMIN> row_min;
+  const fold_fn *rows[NXH_REDUCE_COUNT] = {row_sum.fn, row_prod.fn, row_max.fn, row_min.fn};
+  const int dt = x->dtype;
+  bool reduced[NXH_MAX_NDIM];
+  nxh_tensor sq;
+  rc = squeeze_out(name, x, out, axes, n_axes, reduced, &sq);
+  if (rc) return rc;
+  fold_fn fn = rows[op][dt];
+  if (!fn) return nxh_fail(NXH_FAILURE, name, nxh_is_packed(dt) ? NXH_ERR_PACKED : NXH_ERR_UNSUPPORTED);
+  if (out->dtype != dt) return nxh_fail(NXH_FAILURE, name, NXH_ERR_UNSUPPORTED);
+  Geom g;
+  geom_build(x, &sq, reduced, &g);
+  if (g.n_out == 0) return NXH_OK;
+  for (int j = 0; j < sq.ndim; j++)
+    if (sq.shape[j] > 1 && sq.strides[j] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_OUT_ALIASED);
+  if (g.R == 0) {
+    // max/min have no identity (nx_c_engine.c:1101-1105); sum/prod store 0/1
+    if (op == NXH_RMAX || op == NXH_RMIN) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_EMPTY_REDUCE);
+    unsigned char one[16];
+    if (op == NXH_PROD) storage_one(dt, one);
+    else memset(one, 0, sizeof one);
+    return nxh_fill(ctx, &sq, one);
+  }
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(name, hipSetDevice(ctx->device));
+  return fn(ctx, name, x, &sq, g);
+}
+
+// ── argreduce host ──────────────────────────────────────────────────────────
+template <bool IS_MIN, int DT>
+static int arg_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, const nxh_tensor *out,
+                      const Geom &g) {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  using S = typename TR::S;
+  using CMP = ArgCmp<IS_MIN, C, TR::cat>;
+  const S *ibase = (const S *)in->data + in->offset;
+  int32_t *obase = (int32_t *)out->data + out->offset;
+  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  Scratch scratch(ctx);
+  ArgArgs a;
+  a.in = ibase;
+  a.in_idx = nullptr;
+  a.R = g.R;
+  a.r_stride = g.nr ? g.rin[0] : 0;
+  a.n_out = (uint64_t)g.n_out;
+  a.L = 0;
+  a.lane_blocks = 0;
+  a.out_lane_stride = 0;
+
+  // column form: some kept dim is the unit-stride one and the axis is strided
+  int lane = -1;
+  for (int j = 0; j < g.nk; j++)
+    if (g.kin[j] == 1 && g.kshape[j] >= 16 && g.kshape[j] <= 0x7fffffffLL) lane = j;
+  if (lane >= 0 && std::llabs(a.r_stride) > 1 && dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout, lane)) {
+    const int64_t L = g.kshape[lane], n_outer = g.n_out / L;
+    const int64_t lane_blocks = (L + FOLD_THREADS - 1) / FOLD_THREADS;
+    const int64_t blocks = lane_blocks * n_outer;
+    if (blocks <= 0x7fffffffLL) {
+      int nsplit = pick_split(blocks, g.R, 16, cus);
+      int64_t chunk = (g.R + nsplit - 1) / nsplit;
+      nsplit = (int)((g.R + chunk - 1) / chunk);
+      a.n_out = (uint64_t)n_outer;  // col form: number of outer slices
+      a.L = (uint32_t)L;
+      a.lane_blocks = (uint32_t)lane_blocks;
+      a.out_lane_stride = g.kout[lane];
+      a.chunk = chunk;
+      a.nsplit = nsplit;
+      a.out_idx = obase;
+      a.out_val = nullptr;
+      if (nsplit > 1) {
+        int rc = scratch.get(0, (size_t)nsplit * g.n_out * sizeof(C));
+        if (!rc) rc = scratch.get(1, (size_t)nsplit * g.n_out * sizeof(int32_t));
+        if (rc) return rc;
+        a.out_val = scratch.p[0];
+        a.out_idx = (int32_t *)scratch.p[1];
+      }
+      nxh_set_path(nsplit > 1 ? "arg_col_split" : "arg_col");
+      hipLaunchKernelGGL((arg_col_kernel<InS<DT>, CMP, false>), dim3((unsigned)blocks, (unsigned)nsplit),
+                         dim3(FOLD_THREADS), 0, ctx->stream, a);
+      NXH_HIP(op, hipGetLastError());
+      if (nsplit > 1) {
+        ArgArgs b = a;
+        b.in = scratch.p[0];
+        b.in_idx = (const int32_t *)scratch.p[1];
+        b.out_idx = obase;
+        b.out_val = nullptr;
+        dims_contig_in(&b.kept, L);
+        b.R = nsplit;
+        b.r_stride = g.n_out;
+        b.chunk = nsplit;
+        b.nsplit = 1;
+        hipLaunchKernelGGL((arg_col_kernel<InC<C>, CMP, true>), dim3((unsigned)blocks, 1), dim3(FOLD_THREADS), 0,
+                           ctx->stream, b);
+        NXH_HIP(op, hipGetLastError());
+      }
+      return NXH_OK;
+    }
+  }
+
+  // row form: a group of lanes per output walks the axis at its own stride
+  if (!dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout))
+    return nxh_fail(NXH_FAILURE, op, "view has too many non-mergeable dimensions for one launch");
+  const bool wave_rows = g.R < 1024;
+  const int64_t blocks = wave_rows ? (g.n_out + 3) / 4 : g.n_out;
+  if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many outputs for one launch");
+  int nsplit = wave_rows ? 1 : pick_split(blocks, g.R, 8192, cus);
+  int64_t chunk = (g.R + nsplit - 1) / nsplit;
+  nsplit = (int)((g.R + chunk - 1) / chunk);
+  a.chunk = chunk;
+  a.nsplit = nsplit;
+  a.out_idx = obase;
+  a.out_val = nullptr;
+  if (nsplit > 1) {
+    int rc = scratch.get(0, (size_t)nsplit * g.n_out * sizeof(C));
+    if (!rc) rc = scratch.get(1, (size_t)nsplit * g.n_out * sizeof(int32_t));
+    if (rc) return rc;
+    a.out_val = scratch.p[0];
+    a.out_idx = (int32_t *)scratch.p[1];
+  }
+  dim3 grid((unsigned)blocks, (unsigned)nsplit);
+  nxh_set_path(nsplit > 1 ? "arg_row_split" : (wave_rows ? "arg_row_wave" : "arg_row"));
+  if (wave_rows) hipLaunchKernelGGL((arg_row_kernel<InS<DT>, CMP, 64, false>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((arg_row_kernel<InS<DT>, CMP, 256, false>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+  NXH_HIP(op, hipGetLastError());
+  if (nsplit > 1) {
+    ArgArgs b = a;
+    b.in = scratch.p[0];
+    b.in_idx = (const int32_t *)scratch.p[1];
+    b.out_idx = obase;
+    b.out_val = nullptr;
+    dims_contig_in(&b.kept, nsplit);
+    b.R = nsplit;
+    b.r_stride = 1;
+    b.chunk = nsplit;
+    b.nsplit = 1;
+    hipLaunchKernelGGL((arg_row_kernel<InC<C>, CMP, 64, true>), dim3((unsigned)((g.n_out + 3) / 4), 1),
+                       dim3(FOLD_THREADS), 0, ctx->stream, b);
+    NXH_HIP(op, hipGetLastError());
+  }
+  return NXH_OK;
+}
+
+template <bool IS_MIN>
+struct ArgRow {
+  fold_fn fn[NXH_DTYPE_COUNT] = {};
+  template <int DT>
+  void set() {
+    if constexpr (Tr<DT>::cat != CAT_COMPLEX) fn[DT] = &arg_launch<IS_MIN, DT>;
+  }
+  ArgRow() {
+#define NXH_SET(DT) set<DT>();
+    NXH_FOR_COMPUTE_DTYPES(NXH_SET)
+#undef NXH_SET
+  }
+};
+
+NXH_EXPORT int nxh_argreduce(nxh_context *ctx, int is_min, const nxh_tensor *out, const nxh_tensor *x,
+                             int axis) {
+  const char *name = is_min ? "argmin" : "argmax";
+  if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, name, "null argument");
+  int rc = nxh_check_tensor(name, out);
+  if (!rc) rc = nxh_check_tensor(name, x);
+  if (rc) return rc;
+  static const ArgRow<false> row_max;
+  static const ArgRow<true> row_min;
+  const int dt = x->dtype;
+  fold_fn fn = (is_min ? row_min.fn : row_max.fn)[dt];
+  if (axis < 0 || axis >= x->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_AXIS);
+  bool reduced[NXH_MAX_NDIM];
+  nxh_tensor sq;
+  int32_t ax = axis;
+  rc = squeeze_out(name, x, out, &ax, 1, reduced, &sq);
+  if (rc) return rc;
+  if (!fn) return nxh_fail(NXH_FAILURE, name, nxh_is_packed(dt) ? NXH_ERR_PACKED : NXH_ERR_UNSUPPORTED);
+  if (out->dtype != NXH_I32) return nxh_fail(NXH_FAILURE, name, NXH_ERR_UNSUPPORTED);
+  const int64_t alen = x->shape[axis];
+  if (alen == 0) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_EMPTY_REDUCE);
+  if (alen > INT32_MAX) return nxh_fail(NXH_FAILURE, name, NXH_ERR_ARGCAP);
+  Geom g;
+  geom_build(x, &sq, reduced, &g);
+  if (g.n_out == 0) return NXH_OK;
+  if (g.nr == 0) {  // axis of length 1: every index is 0
+    g.nr = 1;
+    g.rshape[0] = 1;
+    g.rin[0] = 0;
+  }
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(name, hipSetDevice(ctx->device));
+  return fn(ctx, name, x, &sq, g);
+}

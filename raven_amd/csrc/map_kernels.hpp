@@ -1,0 +1,513 @@
+// map_kernels.hpp — the elementwise ("map") kernel family and its planner.
+//
+// Host side: descriptor lowering. K operands sharing one shape are stripped of
+// size-1 dims, reordered so the output's strides descend, and merged wherever
+// adjacent dims compose on EVERY operand (the reference's rule,
+// nx_c_engine.c:542-590). The plan then picks one of three kernels:
+//   map_contig   every operand is one contiguous run or a broadcast scalar:
+//                16-byte vector loads/stores, 4 vectors in flight per lane.
+//   map_tiled    some input's unit-stride dim differs from the output's: 64x64
+//                tiles, that input is read along ITS contiguous dim and turned
+//                through LDS, so both sides of HBM see coalesced 256 B rows.
+//   map_generic  anything else: per-lane index decomposition with precomputed
+//                multiply-shift divisors; vectorised along the inner dim when
+//                every operand is contiguous or broadcast there.
+// Kernels are HBM-bound byte movers: no MFMA, LDS only for the turn.
+#pragma once
+
+#include <algorithm>
+#include <type_traits>
+
+#include "nxh_common.hpp"
+
+constexpr int MAP_MAXOP = 4;
+constexpr int MAP_MAXD = 8;
+constexpr int MAP_THREADS = 256;
+constexpr int MAP_UNROLL = 4;
+
+struct MapPlan {
+  int nop = 0, ndim = 0;
+  int64_t total = 0;
+  int64_t shape[NXH_MAX_NDIM];
+  int64_t stride[MAP_MAXOP][NXH_MAX_NDIM];  // element strides
+  char *base[MAP_MAXOP];                    // byte address of logical element 0
+  int esize[MAP_MAXOP];
+};
+
+// Builds the coalesced plan. Returns NXH_OK or a status (aliased output).
+static inline int map_plan_build(const char *op, const nxh_tensor *const *ops, int nop,
+                                 const int *esize, MapPlan *p) {
+  const int nd_in = ops[0]->ndim;
+  p->nop = nop;
+  p->total = 1;
+  for (int i = 0; i < nd_in; i++) p->total *= ops[0]->shape[i];
+  for (int k = 0; k < nop; k++) {
+    p->esize[k] = esize[k];
+    p->base[k] = (char *)ops[k]->data + ops[k]->offset * (int64_t)esize[k];
+  }
+  int order[NXH_MAX_NDIM], n = 0;
+  for (int i = 0; i < nd_in; i++)
+    if (ops[0]->shape[i] != 1) order[n++] = i;
+  if (p->total != 0) {
+    for (int j = 0; j < n; j++)
+      if (ops[0]->strides[order[j]] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+    // Elementwise work is order-free: walk the output in its own memory order.
+    std::stable_sort(order, order + n, [&](int a, int b) {
+      return std::llabs(ops[0]->strides[a]) > std::llabs(ops[0]->strides[b]);
+    });
+  }
+  int nd = 0;
+  for (int j = 0; j < n; j++) {
+    int i = order[j];
+    int64_t s = ops[0]->shape[i];
+    bool merge = nd > 0;
+    for (int k = 0; merge && k < nop; k++)
+      if (p->stride[k][nd - 1] != ops[k]->strides[i] * s) merge = false;
+    if (merge) {
+      p->shape[nd - 1] *= s;
+      for (int k = 0; k < nop; k++) p->stride[k][nd - 1] = ops[k]->strides[i];
+    } else {
+      p->shape[nd] = s;
+      for (int k = 0; k < nop; k++) p->stride[k][nd] = ops[k]->strides[i];
+      nd++;
+    }
+  }
+  if (nd == 0) {
+    p->shape[0] = 1;
+    for (int k = 0; k < nop; k++) p->stride[k][0] = 0;
+    nd = 1;
+  }
+  p->ndim = nd;
+  return NXH_OK;
+}
+
+// ── device helpers ──────────────────────────────────────────────────────────
+
+template <class T, int N>
+struct alignas(sizeof(T) * N) Vec {
+  T v[N];
+};
+
+struct Unused {};  // placeholder input type
+
+// n / d for n < 2^31 by multiply-high and shift (d >= 1).
+struct FastDiv {
+  uint32_t d, m, s;
+};
+static inline FastDiv fastdiv_make(uint32_t d) {
+  FastDiv f;
+  f.d = d;
+  uint32_t s = 0;
+  while (s < 32 && ((uint64_t)1 << s) < d) s++;
+  f.s = s;
+  f.m = (uint32_t)((((uint64_t)1 << 32) * (((uint64_t)1 << s) - d)) / d + 1);
+  return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) {
+  return (__umulhi(n, f.m) + n) >> f.s;
+}
+
+template <class F>
+struct MapTypes {
+  using Out = typename F::Out;
+  using In0 = typename F::In0;
+  using In1 = typename F::In1;
+  using In2 = typename F::In2;
+  static constexpr int s0 = sizeof(In0);
+  static constexpr int s1 = F::NIN > 1 ? sizeof(In1) : 1;
+  static constexpr int s2 = F::NIN > 2 ? sizeof(In2) : 1;
+  static constexpr int smax = std::max(std::max((int)sizeof(Out), s0), std::max(s1, s2));
+  static constexpr int VEC = 16 / smax > 0 ? 16 / smax : 1;
+};
+
+template <class F>
+__device__ __forceinline__ typename F::Out map_apply(typename F::In0 a, typename F::In1 b,
+                                                     typename F::In2 c) {
+  if constexpr (F::NIN == 1) return F::apply(a);
+  else if constexpr (F::NIN == 2) return F::apply(a, b);
+  else return F::apply(a, b, c);
+}
+
+// Loads V elements of operand type T starting at element index e; `bc` selects a
+// broadcast of the single element at e.
+template <class T, int V>
+__device__ __forceinline__ Vec<T, V> load_vec(const T *p, int64_t e, bool bc) {
+  Vec<T, V> r;
+  if (bc) {
+    T x = p[e];
+#pragma unroll
+    for (int i = 0; i < V; i++) r.v[i] = x;
+  } else {
+    r = *reinterpret_cast<const Vec<T, V> *>(p + e);
+  }
+  return r;
+}
+
+// ── map_contig ──────────────────────────────────────────────────────────────
+template <class F>
+struct ContigArgs {
+  typename F::Out *out;
+  const typename F::In0 *in0;
+  const typename F::In1 *in1;
+  const typename F::In2 *in2;
+  int64_t n;       // elements
+  uint32_t bcast;  // bit k set: input k is a broadcast scalar
+};
+
+template <class F, int V>
+__global__ __launch_bounds__(MAP_THREADS) void map_contig_kernel(ContigArgs<F> a) {
+  using MT = MapTypes<F>;
+  const int64_t nvec = a.n / V;
+  const int64_t base = (int64_t)blockIdx.x * (MAP_THREADS * MAP_UNROLL) + threadIdx.x;
+  const bool b0 = a.bcast & 1u, b1 = a.bcast & 2u, b2 = a.bcast & 4u;
+  Vec<typename MT::In0, V> x0[MAP_UNROLL];
+  Vec<typename MT::In1, V> x1[MAP_UNROLL];
+  Vec<typename MT::In2, V> x2[MAP_UNROLL];
+#pragma unroll
+  for (int j = 0; j < MAP_UNROLL; j++) {
+    int64_t u = base + (int64_t)j * MAP_THREADS;
+    if (u < nvec) {
+      x0[j] = load_vec<typename MT::In0, V>(a.in0, b0 ? 0 : u * V, b0);
+      if constexpr (F::NIN > 1) x1[j] = load_vec<typename MT::In1, V>(a.in1, b1 ? 0 : u * V, b1);
+      if constexpr (F::NIN > 2) x2[j] = load_vec<typename MT::In2, V>(a.in2, b2 ? 0 : u * V, b2);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < MAP_UNROLL; j++) {
+    int64_t u = base + (int64_t)j * MAP_THREADS;
+    if (u < nvec) {
+      Vec<typename MT::Out, V> r;
+#pragma unroll
+      for (int i = 0; i < V; i++) r.v[i] = map_apply<F>(x0[j].v[i], x1[j].v[i], x2[j].v[i]);
+      *reinterpret_cast<Vec<typename MT::Out, V> *>(a.out + u * V) = r;
+    }
+  }
+  // ragged tail: fewer than V elements, one lane each
+  if (blockIdx.x == 0 && threadIdx.x < (unsigned)(a.n - nvec * V)) {
+    int64_t e = nvec * V + threadIdx.x;
+    typename MT::In0 v0 = a.in0[b0 ? 0 : e];
+    typename MT::In1 v1{};
+    typename MT::In2 v2{};
+    if constexpr (F::NIN > 1) v1 = a.in1[b1 ? 0 : e];
+    if constexpr (F::NIN > 2) v2 = a.in2[b2 ? 0 : e];
+    a.out[e] = map_apply<F>(v0, v1, v2);
+  }
+}
+
+// ── map_generic ─────────────────────────────────────────────────────────────
+template <class F>
+struct GenericArgs {
+  char *base[MAP_MAXOP];  // byte pointers: out, in0, in1, in2
+  int ndim;
+  uint32_t units;                 // total / V
+  FastDiv div[MAP_MAXD];          // per dim, in units for the innermost
+  int64_t stride[MAP_MAXOP][MAP_MAXD];  // element strides (innermost: per unit = stride * V)
+  uint32_t inner_bcast;           // bit k: operand k has inner stride 0 (V > 1 only)
+};
+
+template <class F, int V>
+__global__ __launch_bounds__(MAP_THREADS) void map_generic_kernel(GenericArgs<F> a) {
+  using MT = MapTypes<F>;
+  const uint32_t first = blockIdx.x * (MAP_THREADS * MAP_UNROLL) + threadIdx.x;
+  Vec<typename MT::In0, V> x0[MAP_UNROLL];
+  Vec<typename MT::In1, V> x1[MAP_UNROLL];
+  Vec<typename MT::In2, V> x2[MAP_UNROLL];
+  int64_t oo[MAP_UNROLL];
+#pragma unroll
+  for (int j = 0; j < MAP_UNROLL; j++) {
+    uint32_t u = first + j * MAP_THREADS;
+    if (u < a.units) {
+      int64_t off[MAP_MAXOP] = {0, 0, 0, 0};
+      uint32_t rem = u;
+      for (int d = a.ndim - 1; d >= 0; d--) {
+        uint32_t q = fastdiv(rem, a.div[d]);
+        uint32_t c = rem - q * a.div[d].d;
+        rem = q;
+#pragma unroll
+        for (int k = 0; k <= F::NIN; k++) off[k] += (int64_t)c * a.stride[k][d];
+      }
+      oo[j] = off[0];
+      x0[j] = load_vec<typename MT::In0, V>((const typename MT::In0 *)a.base[1], off[1],
+                                            V > 1 && (a.inner_bcast & 2u));
+      if constexpr (F::NIN > 1)
+        x1[j] = load_vec<typename MT::In1, V>((const typename MT::In1 *)a.base[2], off[2],
+                                              V > 1 && (a.inner_bcast & 4u));
+      if constexpr (F::NIN > 2)
+        x2[j] = load_vec<typename MT::In2, V>((const typename MT::In2 *)a.base[3], off[3],
+                                              V > 1 && (a.inner_bcast & 8u));
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < MAP_UNROLL; j++) {
+    uint32_t u = first + j * MAP_THREADS;
+    if (u < a.units) {
+      Vec<typename MT::Out, V> r;
+#pragma unroll
+      for (int i = 0; i < V; i++) r.v[i] = map_apply<F>(x0[j].v[i], x1[j].v[i], x2[j].v[i]);
+      *reinterpret_cast<Vec<typename MT::Out, V> *>((typename MT::Out *)a.base[0] + oo[j]) = r;
+    }
+  }
+}
+
+// ── map_tiled ───────────────────────────────────────────────────────────────
+// Plane (y, x): x is the output's unit-stride dim, y the dim along which the
+// turned inputs are contiguous. All other dims are batch dims decoded per
+// block.
+template <class F>
+struct TiledArgs {
+  char *base[MAP_MAXOP];
+  uint32_t nx, ny, tiles_x, tiles_y;
+  int nbatch_dims;
+  uint32_t bshape[MAP_MAXD];
+  int64_t bstride[MAP_MAXOP][MAP_MAXD];
+  int64_t sx[MAP_MAXOP], sy[MAP_MAXOP];  // element strides along x / y
+  uint32_t turn;                          // bit k: operand k is read along y
+};
+
+template <class T, int TILE>
+__device__ __forceinline__ void tile_load(T (&r)[TILE * TILE / MAP_THREADS], T *lds, const T *p,
+                                          int64_t sx, int64_t sy, uint32_t x0, uint32_t y0,
+                                          uint32_t nx, uint32_t ny, bool turn) {
+  constexpr int PER = TILE * TILE / MAP_THREADS;
+  constexpr int ROWS = MAP_THREADS / TILE;
+  const uint32_t lane = threadIdx.x % TILE, row = threadIdx.x / TILE;
+  if (!turn) {
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      uint32_t x = x0 + lane, y = y0 + row + i * ROWS;
+      if (x < nx && y < ny) r[i] = p[(int64_t)y * sy + (int64_t)x * sx];
+    }
+  } else {
+    // lanes run along y (this operand's contiguous dim); rows step along x
+    T t[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      uint32_t y = y0 + lane, x = x0 + row + i * ROWS;
+      if (x < nx && y < ny) t[i] = p[(int64_t)y * sy + (int64_t)x * sx];
+    }
+    __syncthreads();  // previous use of this LDS tile is complete
+#pragma unroll
+    for (int i = 0; i < PER; i++) lds[(row + i * ROWS) * (TILE + 1) + lane] = t[i];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < PER; i++) r[i] = lds[lane * (TILE + 1) + row + i * ROWS];
+  }
+}
+
+template <class F, int TILE>
+__global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) {
+  using MT = MapTypes<F>;
+  constexpr int PER = TILE * TILE / MAP_THREADS;
+  constexpr int ROWS = MAP_THREADS / TILE;
+  __shared__ typename MT::In0 l0[TILE * (TILE + 1)];
+  __shared__ typename MT::In1 l1[F::NIN > 1 ? TILE * (TILE + 1) : 1];
+  __shared__ typename MT::In2 l2[F::NIN > 2 ? TILE * (TILE + 1) : 1];
+  uint32_t b = blockIdx.x;
+  const uint32_t tx = b % a.tiles_x;
+  b /= a.tiles_x;
+  const uint32_t ty = b % a.tiles_y;
+  b /= a.tiles_y;
+  int64_t off[MAP_MAXOP] = {0, 0, 0, 0};
+  for (int d = a.nbatch_dims - 1; d >= 0; d--) {
+    uint32_t c = b % a.bshape[d];
+    b /= a.bshape[d];
+#pragma unroll
+    for (int k = 0; k <= F::NIN; k++) off[k] += (int64_t)c * a.bstride[k][d];
+  }
+  const uint32_t x0 = tx * TILE, y0 = ty * TILE;
+  typename MT::In0 r0[PER];
+  typename MT::In1 r1[PER];
+  typename MT::In2 r2[PER];
+  tile_load<typename MT::In0, TILE>(r0, l0, (const typename MT::In0 *)a.base[1] + off[1], a.sx[1],
+                                    a.sy[1], x0, y0, a.nx, a.ny, a.turn & 2u);
+  if constexpr (F::NIN > 1)
+    tile_load<typename MT::In1, TILE>(r1, l1, (const typename MT::In1 *)a.base[2] + off[2],
+                                      a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.turn & 4u);
+  if constexpr (F::NIN > 2)
+    tile_load<typename MT::In2, TILE>(r2, l2, (const typename MT::In2 *)a.base[3] + off[3],
+                                      a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.turn & 8u);
+  typename MT::Out *o = (typename MT::Out *)a.base[0] + off[0];
+  const uint32_t lane = threadIdx.x % TILE, row = threadIdx.x / TILE;
+#pragma unroll
+  for (int i = 0; i < PER; i++) {
+    uint32_t x = x0 + lane, y = y0 + row + i * ROWS;
+    if (x < a.nx && y < a.ny)
+      o[(int64_t)y * a.sy[0] + (int64_t)x * a.sx[0]] = map_apply<F>(r0[i], r1[i], r2[i]);
+  }
+}
+
+// ── host launcher ───────────────────────────────────────────────────────────
+
+static inline bool aligned_to(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+template <class F>
+static int map_launch_generic(nxh_context *ctx, const char *op, const MapPlan &p) {
+  using MT = MapTypes<F>;
+  constexpr int V = MT::VEC;
+  const int last = p.ndim - 1;
+  const int esz[MAP_MAXOP] = {(int)sizeof(typename MT::Out), MT::s0, MT::s1, MT::s2};
+  bool vec_ok = V > 1 && p.shape[last] % V == 0 && p.stride[0][last] == 1;
+  uint32_t inner_bcast = 0;
+  for (int k = 0; vec_ok && k < p.nop; k++) {
+    int64_t s = p.stride[k][last];
+    if (s == 0) inner_bcast |= 1u << k;
+    else if (s != 1) vec_ok = false;
+    if (s == 1) {
+      if (!aligned_to(p.base[k], (size_t)esz[k] * V)) vec_ok = false;
+      for (int d = 0; d < last; d++)
+        if (p.stride[k][d] % V != 0) vec_ok = false;
+    }
+  }
+  GenericArgs<F> a;
+  for (int k = 0; k < MAP_MAXOP; k++) a.base[k] = k < p.nop ? p.base[k] : nullptr;
+  a.ndim = p.ndim;
+  const int v = vec_ok ? V : 1;
+  a.units = (uint32_t)(p.total / v);
+  a.inner_bcast = vec_ok ? inner_bcast : 0;
+  for (int d = 0; d < p.ndim; d++) {
+    uint32_t sh = (uint32_t)(d == last ? p.shape[d] / v : p.shape[d]);
+    a.div[d] = fastdiv_make(sh);
+    for (int k = 0; k < MAP_MAXOP; k++)
+      a.stride[k][d] = k < p.nop ? p.stride[k][d] * (d == last ? v : 1) : 0;
+  }
+  const uint32_t per_block = MAP_THREADS * MAP_UNROLL;
+  const uint32_t blocks = (a.units + per_block - 1) / per_block;
+  if (vec_ok) {
+    if constexpr (V > 1) {
+      nxh_set_path("map_generic_vec");
+      hipLaunchKernelGGL((map_generic_kernel<F, V>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+    }
+  } else {
+    nxh_set_path("map_generic");
+    hipLaunchKernelGGL((map_generic_kernel<F, 1>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+  }
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+// One launch over a plan whose total is < 2^31 and whose rank is <= MAP_MAXD.
+template <class F>
+static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
+  using MT = MapTypes<F>;
+  constexpr int V = MT::VEC;
+  const int esz[MAP_MAXOP] = {(int)sizeof(typename MT::Out), MT::s0, MT::s1, MT::s2};
+  // 1. contiguous / scalar-broadcast
+  if (p.ndim == 1 && (p.stride[0][0] == 1 || p.total == 1)) {
+    bool ok = true;
+    uint32_t bc = 0;
+    for (int k = 1; k < p.nop; k++) {
+      int64_t s = p.stride[k][0];
+      if (s == 0 || p.total == 1) bc |= (p.total == 1 ? 0u : 1u << (k - 1));
+      else if (s != 1) ok = false;
+    }
+    for (int k = 0; ok && k < p.nop; k++) {
+      bool is_bc = k > 0 && (bc & (1u << (k - 1)));
+      if (!is_bc && !aligned_to(p.base[k], (size_t)esz[k] * V)) ok = false;
+    }
+    if (ok) {
+      ContigArgs<F> a;
+      a.out = (typename MT::Out *)p.base[0];
+      a.in0 = (const typename MT::In0 *)p.base[1];
+      a.in1 = (const typename MT::In1 *)(p.nop > 2 ? p.base[2] : nullptr);
+      a.in2 = (const typename MT::In2 *)(p.nop > 3 ? p.base[3] : nullptr);
+      a.n = p.total;
+      a.bcast = bc;
+      const int64_t nvec = (p.total + V - 1) / V;
+      const int64_t per_block = MAP_THREADS * MAP_UNROLL;
+      const uint32_t blocks = (uint32_t)((nvec + per_block - 1) / per_block);
+      nxh_set_path("map_contig");
+      hipLaunchKernelGGL((map_contig_kernel<F, V>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+      NXH_HIP(op, hipGetLastError());
+      return NXH_OK;
+    }
+  }
+  // 2. an input whose unit-stride dim is not the output's: turn it through LDS
+  const int last = p.ndim - 1;
+  if (p.ndim >= 2 && p.stride[0][last] == 1 && p.shape[last] >= 16) {
+    int ydim = -1;
+    for (int k = 1; k < p.nop && ydim < 0; k++) {
+      int64_t s = p.stride[k][last];
+      if (s == 0 || s == 1) continue;
+      for (int d = last - 1; d >= 0; d--)
+        if (p.stride[k][d] == 1 && p.shape[d] >= 16) {
+          ydim = d;
+          break;
+        }
+    }
+    if (ydim >= 0) {
+      constexpr int TILE = MT::smax <= 4 ? 64 : 32;
+      TiledArgs<F> a;
+      a.turn = 0;
+      for (int k = 0; k < MAP_MAXOP; k++) {
+        a.base[k] = k < p.nop ? p.base[k] : nullptr;
+        a.sx[k] = k < p.nop ? p.stride[k][last] : 0;
+        a.sy[k] = k < p.nop ? p.stride[k][ydim] : 0;
+        if (k > 0 && k < p.nop && p.stride[k][ydim] == 1 && p.stride[k][last] != 1 &&
+            p.stride[k][last] != 0)
+          a.turn |= 1u << k;
+      }
+      a.nx = (uint32_t)p.shape[last];
+      a.ny = (uint32_t)p.shape[ydim];
+      a.tiles_x = (a.nx + TILE - 1) / TILE;
+      a.tiles_y = (a.ny + TILE - 1) / TILE;
+      a.nbatch_dims = 0;
+      int64_t nb = 1;
+      for (int d = 0; d < last; d++) {
+        if (d == ydim) continue;
+        a.bshape[a.nbatch_dims] = (uint32_t)p.shape[d];
+        for (int k = 0; k < MAP_MAXOP; k++)
+          a.bstride[k][a.nbatch_dims] = k < p.nop ? p.stride[k][d] : 0;
+        a.nbatch_dims++;
+        nb *= p.shape[d];
+      }
+      int64_t blocks = nb * a.tiles_x * a.tiles_y;
+      if (blocks < ((int64_t)1 << 31)) {
+        nxh_set_path("map_tiled");
+        hipLaunchKernelGGL((map_tiled_kernel<F, TILE>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+                           ctx->stream, a);
+        NXH_HIP(op, hipGetLastError());
+        return NXH_OK;
+      }
+    }
+  }
+  return map_launch_generic<F>(ctx, op, p);
+}
+
+// Splits plans that exceed one launch (rank > MAP_MAXD or >= 2^31 elements)
+// along their outer dims.
+template <class F>
+static int map_launch(nxh_context *ctx, const char *op, const MapPlan &p) {
+  if (p.total == 0) return NXH_OK;
+  const int64_t LIM = ((int64_t)1 << 31) - 1;
+  if (p.ndim <= MAP_MAXD && p.total <= LIM) return map_launch_one<F>(ctx, op, p);
+  int64_t rest = p.total / p.shape[0];
+  MapPlan q = p;
+  if (p.ndim > 1 && (p.ndim > MAP_MAXD || rest > LIM)) {
+    // peel dim 0 entirely
+    q.ndim = p.ndim - 1;
+    q.total = rest;
+    for (int d = 0; d < q.ndim; d++) {
+      q.shape[d] = p.shape[d + 1];
+      for (int k = 0; k < p.nop; k++) q.stride[k][d] = p.stride[k][d + 1];
+    }
+    for (int64_t i = 0; i < p.shape[0]; i++) {
+      for (int k = 0; k < p.nop; k++) q.base[k] = p.base[k] + i * p.stride[k][0] * p.esize[k];
+      int rc = map_launch<F>(ctx, op, q);
+      if (rc) return rc;
+    }
+    return NXH_OK;
+  }
+  // chunk dim 0
+  int64_t chunk = std::max<int64_t>(1, LIM / std::max<int64_t>(rest, 1));
+  if (p.ndim == 1) chunk = (int64_t)1 << 30;
+  for (int64_t i = 0; i < p.shape[0]; i += chunk) {
+    q.shape[0] = std::min(chunk, p.shape[0] - i);
+    q.total = q.shape[0] * rest;
+    for (int k = 0; k < p.nop; k++) q.base[k] = p.base[k] + i * p.stride[k][0] * p.esize[k];
+    int rc = map_launch_one<F>(ctx, op, q);
+    if (rc) return rc;
+  }
+  return NXH_OK;
+}
+
+typedef int (*map_launch_fn)(nxh_context *, const char *, const MapPlan &);

@@ -1,0 +1,555 @@
+// matmul.hip — batched matrix multiply.
+//
+// Contract restated from packages/nx/lib/backend_c/nx_c_matmul.c:874-1108:
+// [.., m, k] x [.., k, n] with batch dims broadcast by stride 0, arbitrary
+// element strides on both inputs, products accumulated in the dtype's compute
+// type (f32 for bf16/f16/f32/fp8, f64, int64/uint64 modular, complex) and
+// rounded to storage ONCE per output element (nx_c_matmul.c:347-361, 424-440);
+// k == 0 stores zeros.
+//
+// Kernels
+//   gemm_mfma   bf16 / f16 (v_mfma_f32_32x32x16) and f32 (v_mfma_f32_32x32x2,
+//               true f32, no xf32): 128x128 block tile, four wave64s each
+//               owning 64x64 (2x2 MFMA tiles), K-contiguous LDS tiles with a
+//               16-byte pad per row, global->register prefetch of the next
+//               K-slab while the current one is multiplied. Either operand may
+//               be K-contiguous or M/N-contiguous in memory; the turn happens
+//               on the way into LDS.
+//   gemm_skinny m <= 16 (decode-like GEMV): HBM-bound on B; lanes own adjacent
+//               output columns, K is split across blocks, partials are summed by
+//               a second pass.
+//   gemm_any    every other dtype / layout: one lane per output element.
+// Summation order differs from the reference's k-sequential loop, so float
+// results agree within the reference's GEMM tolerances; integer results are
+// exact (modular arithmetic is order-free).
+
+#include <algorithm>
+
+#include "nxh_common.hpp"
+
+constexpr int MM_MAXB = 8;  // batch dims decoded on the device
+
+struct BatchDims {
+  int n;
+  uint32_t shape[MM_MAXB];
+  int64_t a[MM_MAXB], b[MM_MAXB], c[MM_MAXB];
+};
+__device__ __forceinline__ void batch_decode(const BatchDims &d, uint32_t idx, int64_t &ao, int64_t &bo,
+                                             int64_t &co) {
+  ao = bo = co = 0;
+  for (int i = d.n - 1; i >= 0; i--) {
+    uint32_t q = idx / d.shape[i], c = idx - q * d.shape[i];
+    idx = q;
+    ao += (int64_t)c * d.a[i];
+    bo += (int64_t)c * d.b[i];
+    co += (int64_t)c * d.c[i];
+  }
+}
+
+struct GemmArgs {
+  const void *A, *B;
+  void *C;
+  int64_t M, N, K;
+  int64_t ars, acs, brs, bcs, crs, ccs;  // element strides: row, col
+  BatchDims batch;
+  uint32_t batch0;   // first batch index of this launch
+  int a_vec, b_vec;  // 16-byte loads allowed (alignment + stride multiple)
+};
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+struct alignas(16) U4 {
+  uint32_t x, y, z, w;
+};
+
+// Per-dtype MFMA traits. VL = elements per 16-byte vector; one "k-chunk" is
+// 2*VL values of k: lanes 0-31 multiply the first VL of them, lanes 32-63 the
+// second (any fixed assignment of k to lanes is valid as long as A and B agree).
+struct MMbf16 {
+  static constexpr int DT = NXH_BF16;
+  using S = uint16_t;
+  static constexpr int VL = 8;
+  __device__ __forceinline__ static void mac(f32x16 &acc, const U4 &a, const U4 &b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                  acc, 0, 0, 0);
+  }
+};
+struct MMf16 {
+  static constexpr int DT = NXH_F16;
+  using S = uint16_t;
+  static constexpr int VL = 8;
+  __device__ __forceinline__ static void mac(f32x16 &acc, const U4 &a, const U4 &b) {
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b),
+                                                 acc, 0, 0, 0);
+  }
+};
+struct MMf32 {
+  static constexpr int DT = NXH_F32;
+  using S = float;
+  static constexpr int VL = 4;
+  __device__ __forceinline__ static void mac(f32x16 &acc, const U4 &a, const U4 &b) {
+    f32x4 x = __builtin_bit_cast(f32x4, a), y = __builtin_bit_cast(f32x4, b);
+#pragma unroll
+    for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[s], y[s], acc, 0, 0, 0);
+  }
+};
+
+constexpr int GM = 128, GN = 128;  // block tile
+constexpr int GT = 256;            // threads
+
+// Loads this lane's two 16-byte pieces of one operand's K-slab into registers.
+// ROWS = 128 rows (m or n) by BK k-values. `kc` says the operand is contiguous
+// along k (then a vector runs along k), otherwise along its row index.
+template <class MM, int BK>
+__device__ __forceinline__ void slab_load(U4 (&r)[2], const typename MM::S *p, int64_t rs, int64_t ks,
+                                          int64_t row0, int64_t k0, int64_t nrows, int64_t K, bool kc,
+                                          bool vec) {
+  using S = typename MM::S;
+  constexpr int VL = MM::VL;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int v = threadIdx.x + i * GT;
+    int64_t row, k;
+    if (kc) {
+      row = row0 + v / (BK / VL);
+      k = k0 + (v % (BK / VL)) * VL;
+    } else {
+      k = k0 + v / (GM / VL);
+      row = row0 + (v % (GM / VL)) * VL;
+    }
+    const S *q = p + row * rs + k * ks;
+    const bool full = kc ? (row < nrows && k + VL <= K) : (k < K && row + VL <= nrows);
+    if (vec && full) {
+      r[i] = *reinterpret_cast<const U4 *>(q);
+    } else {
+      S t[VL];
+#pragma unroll
+      for (int j = 0; j < VL; j++) {
+        int64_t rr = kc ? row : row + j, kk = kc ? k + j : k;
+        t[j] = (rr < nrows && kk < K) ? q[kc ? j * ks : j * rs] : (S)0;
+      }
+      r[i] = *reinterpret_cast<const U4 *>(t);
+    }
+  }
+}
+
+// Writes the prefetched pieces into the K-contiguous LDS tile [128][LDP].
+template <class MM, int BK, int LDP>
+__device__ __forceinline__ void slab_store(const U4 (&r)[2], typename MM::S *lds, bool kc) {
+  using S = typename MM::S;
+  constexpr int VL = MM::VL;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int v = threadIdx.x + i * GT;
+    if (kc) {
+      const int row = v / (BK / VL), k = (v % (BK / VL)) * VL;
+      *reinterpret_cast<U4 *>(&lds[row * LDP + k]) = r[i];
+    } else {
+      const int k = v / (GM / VL), row = (v % (GM / VL)) * VL;
+      const S *t = reinterpret_cast<const S *>(&r[i]);
+#pragma unroll
+      for (int j = 0; j < VL; j++) lds[(row + j) * LDP + k] = t[j];
+    }
+  }
+}
+
+template <class MM>
+__global__ __launch_bounds__(GT) void gemm_mfma_kernel(GemmArgs a) {
+  using S = typename MM::S;
+  constexpr int VL = MM::VL;
+  constexpr int BK = 4 * VL;   // two k-chunks per slab
+  constexpr int LDP = BK + VL; // 16-byte pad: rows land on distinct bank groups
+  __shared__ alignas(16) S sA[GM * LDP];
+  __shared__ alignas(16) S sB[GN * LDP];
+
+  int64_t ao, bo, co;
+  batch_decode(a.batch, a.batch0 + blockIdx.z, ao, bo, co);
+  const S *A = (const S *)a.A + ao;
+  const S *B = (const S *)a.B + bo;
+  const int64_t m0 = (int64_t)blockIdx.y * GM, n0 = (int64_t)blockIdx.x * GN;
+  const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int r32 = lane & 31, kg = lane >> 5;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int t = 0; t < 2; t++)
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[t][u][e] = 0.0f;
+
+  U4 ra[2], rb[2];
+  const int64_t nk = (a.K + BK - 1) / BK;
+  if (nk > 0) {
+    slab_load<MM, BK>(ra, A, a.ars, a.acs, m0, 0, a.M, a.K, a_kc, a.a_vec);
+    // B is addressed as rows = n, so its "row stride" is bcs and k stride brs
+    slab_load<MM, BK>(rb, B, a.bcs, a.brs, n0, 0, a.N, a.K, b_kc, a.b_vec);
+  }
+  for (int64_t kt = 0; kt < nk; kt++) {
+    slab_store<MM, BK, LDP>(ra, sA, a_kc);
+    slab_store<MM, BK, LDP>(rb, sB, b_kc);
+    __syncthreads();
+    if (kt + 1 < nk) {
+      slab_load<MM, BK>(ra, A, a.ars, a.acs, m0, (kt + 1) * BK, a.M, a.K, a_kc, a.a_vec);
+      slab_load<MM, BK>(rb, B, a.bcs, a.brs, n0, (kt + 1) * BK, a.N, a.K, b_kc, a.b_vec);
+    }
+#pragma unroll
+    for (int ch = 0; ch < 2; ch++) {
+      U4 fa[2], fb[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+        fa[t] = *reinterpret_cast<const U4 *>(&sA[(wm + t * 32 + r32) * LDP + ch * 2 * VL + kg * VL]);
+        fb[t] = *reinterpret_cast<const U4 *>(&sB[(wn + t * 32 + r32) * LDP + ch * 2 * VL + kg * VL]);
+      }
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int u = 0; u < 2; u++) MM::mac(acc[t][u], fa[t], fb[u]);
+    }
+    __syncthreads();
+  }
+
+  // accumulator element e of lane l is C[(e/4)*8 + (l/32)*4 + e%4][l%32]
+  S *C = (S *)a.C + co;
+#pragma unroll
+  for (int t = 0; t < 2; t++)
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int64_t col = n0 + wn + u * 32 + r32;
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        const int64_t row = m0 + wm + t * 32 + (e >> 2) * 8 + kg * 4 + (e & 3);
+        if (row < a.M && col < a.N) C[row * a.crs + col * a.ccs] = Tr<MM::DT>::st(acc[t][u][e]);
+      }
+    }
+}
+
+// ── gemm_skinny: m <= 16, B streamed once ───────────────────────────────────
+// Lane owns VN adjacent columns; block covers 256*VN columns and one K-chunk.
+// A's chunk [m][kchunk] sits in LDS as f32. Partials [split][m][n] in f32.
+struct SkinnyArgs {
+  const void *A, *B;
+  void *C;       // storage-typed result (nsplit == 1) or f32 partials
+  int64_t M, N, K;
+  int64_t ars, acs, brs, crs, ccs;  // B has bcs == 1
+  int64_t kchunk;
+  int nsplit;
+};
+template <int DT, int MMAX, int VN>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  constexpr int KT = 64;  // k rows staged per step
+  __shared__ float sA[MMAX][KT];
+  const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VN;
+  const int64_t k0 = (int64_t)blockIdx.y * a.kchunk;
+  const int64_t k1 = k0 + a.kchunk < a.K ? k0 + a.kchunk : a.K;
+  float acc[MMAX][VN];
+#pragma unroll
+  for (int i = 0; i < MMAX; i++)
+#pragma unroll
+    for (int j = 0; j < VN; j++) acc[i][j] = 0.0f;
+  const S *A = (const S *)a.A;
+  const S *B = (const S *)a.B;
+  const bool col_ok = n + VN <= a.N;
+  for (int64_t kb = k0; kb < k1; kb += KT) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < MMAX * KT; idx += 256) {
+      int i = idx / KT, kk = idx % KT;
+      sA[i][kk] = (i < a.M && kb + kk < k1) ? TR::ld(A[i * a.ars + (kb + kk) * a.acs]) : 0.0f;
+    }
+    __syncthreads();
+    const int64_t kend = kb + KT < k1 ? kb + KT : k1;
+    if (n < a.N) {
+      for (int64_t k = kb; k < kend; k++) {
+        float bv[VN];
+        const S *bp = B + k * a.brs + n;
+        if (col_ok) {
+          struct alignas(sizeof(S) * VN) BV {
+            S v[VN];
+          } t = *reinterpret_cast<const BV *>(bp);
+#pragma unroll
+          for (int j = 0; j < VN; j++) bv[j] = TR::ld(t.v[j]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < VN; j++) bv[j] = n + j < a.N ? TR::ld(bp[j]) : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < MMAX; i++) {
+          const float av = sA[i][k - kb];
+#pragma unroll
+          for (int j = 0; j < VN; j++) acc[i][j] = __builtin_fmaf(av, bv[j], acc[i][j]);
+        }
+      }
+    }
+  }
+  if (n >= a.N) return;
+  if (a.nsplit > 1) {
+    float *P = (float *)a.C + (int64_t)blockIdx.y * a.M * a.N;
+    for (int i = 0; i < a.M; i++)
+#pragma unroll
+      for (int j = 0; j < VN; j++)
+        if (n + j < a.N) P[i * a.N + n + j] = acc[i][j];
+  } else {
+    S *C = (S *)a.C;
+    for (int i = 0; i < a.M; i++)
+#pragma unroll
+      for (int j = 0; j < VN; j++)
+        if (n + j < a.N) C[i * a.crs + (n + j) * a.ccs] = TR::st(acc[i][j]);
+  }
+}
+template <int DT>
+__global__ void skinny_finish_kernel(const float *P, void *Cv, int64_t M, int64_t N, int nsplit,
+                                     int64_t crs, int64_t ccs) {
+  using TR = Tr<DT>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= M * N) return;
+  float s = 0.0f;
+  for (int c = 0; c < nsplit; c++) s += P[(int64_t)c * M * N + e];
+  ((typename TR::S *)Cv)[(e / N) * crs + (e % N) * ccs] = TR::st(s);
+}
+
+// ── gemm_any: one lane per output, any dtype, any strides ───────────────────
+template <int DT>
+__global__ __launch_bounds__(256) void gemm_any_kernel(GemmArgs a) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  int64_t ao, bo, co;
+  batch_decode(a.batch, a.batch0 + blockIdx.z, ao, bo, co);
+  const int64_t col = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
+  const int64_t row = (int64_t)blockIdx.y * 16 + (threadIdx.x >> 4);
+  if (row >= a.M || col >= a.N) return;
+  const S *A = (const S *)a.A + ao + row * a.ars;
+  const S *B = (const S *)a.B + bo + col * a.bcs;
+  C acc;
+  if constexpr (TR::cat == CAT_COMPLEX) acc = C{0, 0};
+  else acc = (C)0;
+  for (int64_t k = 0; k < a.K; k++) {
+    C x = TR::ld(A[k * a.acs]), y = TR::ld(B[k * a.brs]);
+    if constexpr (TR::cat == CAT_SINT) acc = (C)((uint64_t)acc + (uint64_t)x * (uint64_t)y);
+    else acc = acc + x * y;
+  }
+  ((S *)a.C)[co + row * a.crs + col * a.ccs] = TR::st(acc);
+}
+
+typedef int (*mm_fn)(nxh_context *, GemmArgs &, uint32_t nbatch);
+
+template <int DT>
+static int launch_any(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
+  nxh_set_path("gemm_any");
+  const uint32_t gx = (uint32_t)((a.N + 15) / 16), gy = (uint32_t)((a.M + 15) / 16);
+  if (gy > 65535) return nxh_fail(NXH_FAILURE, "matmul", "m too large for this dtype's kernel");
+  for (uint32_t b0 = 0; b0 < nbatch; b0 += 65535) {
+    a.batch0 = b0;
+    hipLaunchKernelGGL((gemm_any_kernel<DT>), dim3(gx, gy, std::min<uint32_t>(65535, nbatch - b0)), dim3(256), 0,
+                       ctx->stream, a);
+    NXH_HIP("matmul", hipGetLastError());
+  }
+  return NXH_OK;
+}
+
+template <class MM>
+static int launch_mfma(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
+  nxh_set_path("gemm_mfma");
+  const uint32_t gx = (uint32_t)((a.N + GN - 1) / GN), gy = (uint32_t)((a.M + GM - 1) / GM);
+  if (gy > 65535) return launch_any<MM::DT>(ctx, a, nbatch);
+  for (uint32_t b0 = 0; b0 < nbatch; b0 += 65535) {
+    a.batch0 = b0;
+    hipLaunchKernelGGL((gemm_mfma_kernel<MM>), dim3(gx, gy, std::min<uint32_t>(65535, nbatch - b0)), dim3(GT), 0,
+                       ctx->stream, a);
+    NXH_HIP("matmul", hipGetLastError());
+  }
+  return NXH_OK;
+}
+
+template <int DT, int VN>
+static int launch_skinny(nxh_context *ctx, GemmArgs &g) {
+  SkinnyArgs a;
+  a.A = g.A;
+  a.B = g.B;
+  a.M = g.M;
+  a.N = g.N;
+  a.K = g.K;
+  a.ars = g.ars;
+  a.acs = g.acs;
+  a.brs = g.brs;
+  a.crs = g.crs;
+  a.ccs = g.ccs;
+  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  const int64_t col_blocks = (g.N + 256 * VN - 1) / (256 * VN);
+  int64_t want = std::max<int64_t>(1, ((int64_t)cus * 4 + col_blocks - 1) / col_blocks);
+  int64_t nsplit = std::min<int64_t>(want, std::max<int64_t>(1, g.K / 64));
+  int64_t kchunk = (g.K + nsplit - 1) / nsplit;
+  kchunk = (kchunk + 63) / 64 * 64;
+  nsplit = std::max<int64_t>(1, (g.K + kchunk - 1) / kchunk);
+  a.kchunk = kchunk;
+  a.nsplit = (int)nsplit;
+  void *part = nullptr;
+  if (nsplit > 1) {
+    int rc = nxh_alloc_locked(ctx, (size_t)nsplit * g.M * g.N * sizeof(float), &part);
+    if (rc) return rc;
+    a.C = part;
+  } else {
+    a.C = g.C;
+  }
+  nxh_set_path(nsplit > 1 ? "gemm_skinny_split" : "gemm_skinny");
+  dim3 grid((unsigned)col_blocks, (unsigned)nsplit);
+  if (g.M <= 8) hipLaunchKernelGGL((gemm_skinny_kernel<DT, 8, VN>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<DT, 16, VN>), grid, dim3(256), 0, ctx->stream, a);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && nsplit > 1) {
+    const int64_t total = g.M * g.N;
+    hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream,
+                       (const float *)part, g.C, g.M, g.N, (int)nsplit, g.crs, g.ccs);
+    e = hipGetLastError();
+  }
+  if (part) nxh_free_locked(ctx, part);
+  if (e != hipSuccess) return nxh_hip_fail("matmul", e);
+  return NXH_OK;
+}
+
+static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+template <class MM>
+static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool batch_aligned_a,
+                          bool batch_aligned_b) {
+  using S = typename MM::S;
+  constexpr int VL = MM::VL;
+  // decode-like shape: one batch, few rows, B row-major: stream B once
+  if (nbatch == 1 && a.M <= 16 && a.bcs == 1 && a.N >= 1024 && a.K >= 256 && a.batch.n == 0) {
+    constexpr int VN = sizeof(S) == 2 ? 4 : 2;
+    if (a.brs % VN == 0 && ((uintptr_t)a.B % (sizeof(S) * VN)) == 0) return launch_skinny<MM::DT, VN>(ctx, a);
+  }
+  const bool a_ok = a.acs == 1 || a.ars == 1, b_ok = a.brs == 1 || a.bcs == 1;
+  if (!a_ok || !b_ok) return launch_any<MM::DT>(ctx, a, nbatch);
+  // 16-byte loads need an aligned base and every other stride a multiple of VL
+  a.a_vec = al16(a.A) && batch_aligned_a && ((a.acs == 1 ? a.ars : a.acs) % VL == 0);
+  a.b_vec = al16(a.B) && batch_aligned_b && ((a.brs == 1 ? a.bcs : a.brs) % VL == 0);
+  return launch_mfma<MM>(ctx, a, nbatch);
+}
+
+NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tensor *A, const nxh_tensor *B) {
+  const char *op = "matmul";
+  if (!ctx || !C || !A || !B) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, C);
+  if (!rc) rc = nxh_check_tensor(op, A);
+  if (!rc) rc = nxh_check_tensor(op, B);
+  if (rc) return rc;
+  if (A->dtype != B->dtype || A->dtype != C->dtype) return nxh_fail(NXH_FAILURE, op, NXH_ERR_MM_DTYPE);
+  const int dt = A->dtype;
+  if (nxh_is_packed(dt)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  if (dt == NXH_BOOL) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  if (A->ndim < 2 || B->ndim < 2) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  const int nd = std::max(A->ndim, B->ndim);
+  if (C->ndim != nd) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  const int64_t m = A->shape[A->ndim - 2], k = A->shape[A->ndim - 1];
+  const int64_t kk = B->shape[B->ndim - 2], n = B->shape[B->ndim - 1];
+  if (k != kk || C->shape[nd - 2] != m || C->shape[nd - 1] != n)
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+
+  GemmArgs g;
+  // batch broadcast strides (nx_c_matmul.c:895-926), then drop size-1 dims and
+  // merge neighbours that compose on all three operands
+  const int bnd = nd - 2, abo = nd - A->ndim, bbo = nd - B->ndim;
+  int64_t bs[NXH_MAX_NDIM], as_[NXH_MAX_NDIM], bs_[NXH_MAX_NDIM], cs_[NXH_MAX_NDIM];
+  int nb = 0;
+  int64_t nbatch = 1;
+  for (int i = 0; i < bnd; i++) {
+    int64_t sa = 1, sb = 1, sta = 0, stb = 0;
+    if (i >= abo) {
+      sa = A->shape[i - abo];
+      sta = A->strides[i - abo];
+    }
+    if (i >= bbo) {
+      sb = B->shape[i - bbo];
+      stb = B->strides[i - bbo];
+    }
+    if (sa != sb && sa != 1 && sb != 1) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    const int64_t s = std::max(sa, sb);
+    if (C->shape[i] != s) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    if (s > 1 && C->strides[i] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+    nbatch *= s;
+    if (s == 1) continue;
+    const int64_t xa = sa == 1 ? 0 : sta, xb = sb == 1 ? 0 : stb, xc = C->strides[i];
+    if (nb > 0 && as_[nb - 1] == xa * s && bs_[nb - 1] == xb * s && cs_[nb - 1] == xc * s) {
+      bs[nb - 1] *= s;
+      as_[nb - 1] = xa;
+      bs_[nb - 1] = xb;
+      cs_[nb - 1] = xc;
+    } else {
+      bs[nb] = s;
+      as_[nb] = xa;
+      bs_[nb] = xb;
+      cs_[nb] = xc;
+      nb++;
+    }
+  }
+  if (m == 0 || n == 0 || nbatch == 0) return NXH_OK;
+  g.ars = A->strides[A->ndim - 2];
+  g.acs = A->strides[A->ndim - 1];
+  g.brs = B->strides[B->ndim - 2];
+  g.bcs = B->strides[B->ndim - 1];
+  g.crs = C->strides[nd - 2];
+  g.ccs = C->strides[nd - 1];
+  if ((m > 1 && g.crs == 0) || (n > 1 && g.ccs == 0)) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  if (nb > MM_MAXB || nbatch > 0xffffffffLL) return nxh_fail(NXH_FAILURE, op, "too many batch dimensions");
+  // a size-1 matrix dim carries no meaningful stride: pick the value that lets
+  // the operand count as contiguous along its other dim
+  if (m == 1) g.ars = g.acs == 1 ? 0 : 1;
+  if (n == 1) g.bcs = g.brs == 1 ? 0 : 1;
+  if (k == 1) {
+    if (g.ars != 1) g.acs = 1;
+    if (g.bcs != 1) g.brs = 1;
+  }
+  const int64_t es = nxh_elem_size(dt);
+  g.A = (const char *)A->data + A->offset * es;
+  g.B = (const char *)B->data + B->offset * es;
+  g.C = (char *)C->data + C->offset * es;
+  g.M = m;
+  g.N = n;
+  g.K = k;
+  g.batch.n = nb;
+  bool al_a = true, al_b = true;
+  for (int i = 0; i < nb; i++) {
+    if (bs[i] > 0xffffffffLL) return nxh_fail(NXH_FAILURE, op, "batch dimension too large");
+    g.batch.shape[i] = (uint32_t)bs[i];
+    g.batch.a[i] = as_[i];
+    g.batch.b[i] = bs_[i];
+    g.batch.c[i] = cs_[i];
+    if ((as_[i] * es) % 16) al_a = false;
+    if ((bs_[i] * es) % 16) al_b = false;
+  }
+  g.batch0 = 0;
+  g.a_vec = g.b_vec = 0;
+
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  switch (dt) {
+    case NXH_BF16: return run_mfma_dtype<MMbf16>(ctx, g, (uint32_t)nbatch, al_a, al_b);
+    case NXH_F16: return run_mfma_dtype<MMf16>(ctx, g, (uint32_t)nbatch, al_a, al_b);
+    case NXH_F32: return run_mfma_dtype<MMf32>(ctx, g, (uint32_t)nbatch, al_a, al_b);
+#define NXH_CASE(DT) \
+  case DT: return launch_any<DT>(ctx, g, (uint32_t)nbatch);
+      NXH_CASE(NXH_F64)
+      NXH_CASE(NXH_F8E4M3)
+      NXH_CASE(NXH_F8E5M2)
+      NXH_CASE(NXH_I8)
+      NXH_CASE(NXH_U8)
+      NXH_CASE(NXH_I16)
+      NXH_CASE(NXH_U16)
+      NXH_CASE(NXH_I32)
+      NXH_CASE(NXH_U32)
+      NXH_CASE(NXH_I64)
+      NXH_CASE(NXH_U64)
+      NXH_CASE(NXH_C32)
+      NXH_CASE(NXH_C64)
+#undef NXH_CASE
+    default: return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  }
+}

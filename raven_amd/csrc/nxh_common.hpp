@@ -1,0 +1,279 @@
+// nxh_common.hpp — shared host/device definitions of libnxhip (gfx950 only).
+//
+// The dtype table below is the device-side counterpart of the reference's
+// single dtype table (packages/nx/lib/backend_c/nx_c.h:130-168): storage type,
+// compute type, load/store converters and category per dtype. The converters
+// reproduce packages/nx/lib/buffer/nx_buffer_stubs.h:70-302 bit for bit.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/nxhip.h"
+
+#define NXH_EXPORT extern "C" __attribute__((visibility("default")))
+
+// ─────────────────────────── context ────────────────────────────────────────
+
+struct nxh_context {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+  int compute_units = 0;
+  char name[128] = {0};
+  std::mutex mu;  // guards the allocator and launches: one stream per context
+  // caching allocator: size class -> free blocks
+  std::map<size_t, std::vector<void *>> free_lists;
+  std::map<void *, size_t> live;  // every block handed out or cached -> its class size
+  uint64_t in_use = 0, cached = 0, reserved = 0, driver_allocs = 0;
+  // one device word, written by kernels that detect a data fault (gather OOB)
+  int *fault_flag = nullptr;       // device
+  int *fault_flag_host = nullptr;  // pinned host mirror for the readback
+};
+
+// thread-local status text (static strings + op prefix)
+void nxh_set_error(const char *op, const char *msg);
+void nxh_set_path(const char *path);
+int nxh_fail(int kind, const char *op, const char *msg);
+int nxh_hip_fail(const char *op, hipError_t e);
+
+#define NXH_HIP(op, call)                                \
+  do {                                                   \
+    hipError_t e__ = (call);                             \
+    if (e__ != hipSuccess) return nxh_hip_fail(op, e__); \
+  } while (0)
+
+// allocator (runtime.hip)
+int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out);
+void nxh_free_locked(nxh_context *ctx, void *p);
+
+// status strings shared with the reference (nx_c.h:381-388, nx_c_engine.h:38-50)
+#define NXH_ERR_NDIM "ndim exceeds NX_C_MAX_NDIM"
+#define NXH_ERR_BAD_KIND "unsupported bigarray kind"
+#define NXH_ERR_UNSUPPORTED "dtype not supported for this operation"
+#define NXH_ERR_PACKED "packed dtype not supported for this operation"
+#define NXH_ERR_SHAPE "shape mismatch"
+#define NXH_ERR_EMPTY_REDUCE "reduction over empty axis has no identity"
+#define NXH_ERR_ALLOC "out of memory"
+#define NXH_ERR_AXES "reduce axes must be strictly increasing and in range"
+#define NXH_ERR_OUT_RANK "output rank inconsistent with the operation"
+#define NXH_ERR_AXIS "axis out of range"
+#define NXH_ERR_OUT_ALIASED "output has a broadcast (zero) stride"
+#define NXH_ERR_ARGCAP "argreduce axis length exceeds INT32_MAX"
+#define NXH_ERR_INDEX_OOB "index out of bounds for the gathered/scattered axis"
+#define NXH_ERR_MM_DTYPE "matmul operands must share one dtype"
+
+static inline bool nxh_is_packed(int dt) { return dt == NXH_I4 || dt == NXH_U4; }
+static inline int64_t nxh_elem_size(int dt) {
+  static const int64_t s[NXH_DTYPE_COUNT] = {2, 4, 8, 2, 1, 1, 0, 0, 1, 1,
+                                             2, 2, 4, 4, 8, 8, 8, 16, 1};
+  return (unsigned)dt < NXH_DTYPE_COUNT ? s[dt] : 0;
+}
+static inline bool nxh_same_shape(const nxh_tensor *a, const nxh_tensor *b) {
+  if (a->ndim != b->ndim) return false;
+  for (int i = 0; i < a->ndim; i++)
+    if (a->shape[i] != b->shape[i]) return false;
+  return true;
+}
+static inline int nxh_check_tensor(const char *op, const nxh_tensor *t) {
+  if (t->ndim < 0 || t->ndim > NXH_MAX_NDIM) return nxh_fail(NXH_FAILURE, op, NXH_ERR_NDIM);
+  if ((unsigned)t->dtype >= NXH_DTYPE_COUNT) return nxh_fail(NXH_FAILURE, op, NXH_ERR_BAD_KIND);
+  return NXH_OK;
+}
+
+// ─────────────────────────── device scalar types ────────────────────────────
+
+enum Cat { CAT_SINT, CAT_UINT, CAT_FLOAT, CAT_COMPLEX, CAT_BOOL };
+
+template <class R>
+struct cplx {
+  R re, im;
+};
+using c32 = cplx<float>;
+using c64 = cplx<double>;
+
+#define HD __host__ __device__ __forceinline__
+
+template <class R>
+HD cplx<R> operator+(cplx<R> a, cplx<R> b) { return {a.re + b.re, a.im + b.im}; }
+template <class R>
+HD cplx<R> operator-(cplx<R> a, cplx<R> b) { return {a.re - b.re, a.im - b.im}; }
+template <class R>
+HD cplx<R> operator-(cplx<R> a) { return {-a.re, -a.im}; }
+template <class R>
+HD cplx<R> operator*(cplx<R> a, cplx<R> b) {
+  return {a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+// Smith's division: no intermediate overflow for representable quotients.
+template <class R>
+HD cplx<R> operator/(cplx<R> a, cplx<R> b) {
+  if (fabs(b.re) >= fabs(b.im)) {
+    if (b.re == 0 && b.im == 0) return {a.re / b.re, a.im / b.re};
+    R r = b.im / b.re, d = b.re + b.im * r;
+    return {(a.re + a.im * r) / d, (a.im - a.re * r) / d};
+  }
+  R r = b.re / b.im, d = b.re * r + b.im;
+  return {(a.re * r + a.im) / d, (a.im * r - a.re) / d};
+}
+template <class R>
+HD bool operator==(cplx<R> a, cplx<R> b) { return a.re == b.re && a.im == b.im; }
+template <class R>
+HD bool operator!=(cplx<R> a, cplx<R> b) { return !(a == b); }
+
+HD uint32_t f2u(float f) { return __builtin_bit_cast(uint32_t, f); }
+HD float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// f32 -> bf16, nx_buffer_stubs.h:73-86: NaN keeps sign/payload and is quieted,
+// everything else rounds to nearest even on the dropped half.
+HD uint16_t f32_to_bf16(float f) {
+  uint32_t u = f2u(f);
+  uint32_t nan = (u >> 16) | 0x40u;
+  uint32_t rne = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? nan : rne);
+}
+HD float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+// f32 -> f16, nx_buffer_stubs.h:99-148. The hardware convert (round to nearest
+// even, subnormals kept) matches on every non-NaN input; a NaN keeps its top
+// ten payload bits and is bumped to stay a NaN.
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  uint32_t u = f2u(f);
+  _Float16 h = (_Float16)f;
+  uint16_t hw = __builtin_bit_cast(uint16_t, h);
+  uint32_t m = u & 0x7fffffu;
+  uint32_t r = 0x7c00u + (m >> 13);
+  r += (r == 0x7c00u);
+  uint16_t nan = (uint16_t)(((u >> 16) & 0x8000u) + r);
+  return ((u & 0x7fffffffu) > 0x7f800000u) ? nan : hw;
+}
+// f16 -> f32, nx_buffer_stubs.h:150-182: exact; NaN payload shifts up and the
+// quiet bit is forced.
+__device__ __forceinline__ float f16_to_f32(uint16_t h) {
+  _Float16 x = __builtin_bit_cast(_Float16, h);
+  float hw = (float)x;
+  uint32_t nan = (((uint32_t)h & 0x8000u) << 16) | 0x7f800000u | (((uint32_t)h & 0x3ffu) << 13) |
+                 0x400000u;
+  return ((h & 0x7fffu) > 0x7c00u) ? u2f(nan) : hw;
+}
+
+// Shared fp8 encoder body (nx_buffer_stubs.h:189-223, 244-278).
+template <int MBITS, int BIAS>
+HD uint32_t f32_to_fp8_bits(uint32_t u) {
+  int exp = (int)((u >> 23) & 0xffu) - 127;
+  constexpr int EMIN = 1 - BIAS;
+  if (exp >= EMIN) {
+    uint32_t sig = u & 0x7fffffu;
+    constexpr int drop = 23 - MBITS;
+    uint32_t q = sig >> drop, rem = sig & ((1u << drop) - 1u), half = 1u << (drop - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return ((uint32_t)(exp + BIAS) << MBITS) + q;
+  }
+  uint32_t sig = (u & 0x7fffffu) | 0x800000u;
+  int shift = (23 - MBITS) + (EMIN - exp);
+  if (shift > 24) return 0;
+  uint32_t q = sig >> shift, rem = sig & ((1u << shift) - 1u), half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1u))) q++;
+  return q;
+}
+HD uint8_t f32_to_f8e4m3(float f) {
+  uint32_t u = f2u(f);
+  uint32_t a = u & 0x7fffffffu;
+  uint8_t sign = (uint8_t)((u >> 31) << 7);
+  if (a > 0x7f800000u) return 0x7f;           // NaN: sign dropped
+  if (a == 0x7f800000u) return sign | 0x7f;   // inf -> NaN, sign kept
+  uint32_t bits = f32_to_fp8_bits<3, 7>(u);
+  return bits >= 0x7fu ? (uint8_t)(sign | 0x7f) : (uint8_t)(sign | bits);
+}
+HD uint8_t f32_to_f8e5m2(float f) {
+  uint32_t u = f2u(f);
+  uint32_t a = u & 0x7fffffffu;
+  uint8_t sign = (uint8_t)((u >> 31) << 7);
+  if (a > 0x7f800000u) return 0x7f;
+  if (a == 0x7f800000u) return sign | 0x7c;
+  uint32_t bits = f32_to_fp8_bits<2, 15>(u);
+  return bits >= 0x7cu ? (uint8_t)(sign | 0x7c) : (uint8_t)(sign | bits);
+}
+// Decoders (nx_buffer_stubs.h:225-240, 280-302), by exact bit construction:
+// a subnormal m * 2^(emin - mbits) is built as an integer-to-float conversion
+// scaled by a power of two, both exact.
+HD float f8e4m3_to_f32(uint8_t v) {
+  uint32_t e = (v >> 3) & 0xfu, m = v & 7u;
+  if (e == 0xfu && m == 7u) return u2f(0x7fc00000u);  // NAN macro: positive quiet NaN
+  float r = e == 0 ? (float)m * 0.001953125f /* 2^-9 */
+                   : u2f(((e + 120u) << 23) | (m << 20));
+  return (v & 0x80) ? -r : r;
+}
+HD float f8e5m2_to_f32(uint8_t v) {
+  uint32_t e = (v >> 2) & 0x1fu, m = v & 3u;
+  bool neg = (v & 0x80) != 0;
+  if (e == 0x1fu) return m == 0 ? u2f(neg ? 0xff800000u : 0x7f800000u) : u2f(0x7fc00000u);
+  float r = e == 0 ? (float)m * 0.0000152587890625f /* 2^-16 */
+                   : u2f(((e + 112u) << 23) | (m << 21));
+  return neg ? -r : r;
+}
+
+// The dtype table.
+template <int DT>
+struct Tr;
+#define NXH_TR(DT, S_, C_, CAT_, LD_, ST_)                                \
+  template <>                                                             \
+  struct Tr<DT> {                                                         \
+    using S = S_;                                                         \
+    using C = C_;                                                         \
+    static constexpr Cat cat = CAT_;                                      \
+    static constexpr int tag = DT;                                        \
+    __device__ __forceinline__ static C ld(S s) { return (C)(LD_(s)); }   \
+    __device__ __forceinline__ static S st(C c) { return (S)(ST_(c)); }   \
+  };
+#define NXH_ID(x) (x)
+#define NXH_BOOLN(x) ((x) != 0)
+NXH_TR(NXH_F16, uint16_t, float, CAT_FLOAT, f16_to_f32, f32_to_f16)
+NXH_TR(NXH_F32, float, float, CAT_FLOAT, NXH_ID, NXH_ID)
+NXH_TR(NXH_F64, double, double, CAT_FLOAT, NXH_ID, NXH_ID)
+NXH_TR(NXH_BF16, uint16_t, float, CAT_FLOAT, bf16_to_f32, f32_to_bf16)
+NXH_TR(NXH_F8E4M3, uint8_t, float, CAT_FLOAT, f8e4m3_to_f32, f32_to_f8e4m3)
+NXH_TR(NXH_F8E5M2, uint8_t, float, CAT_FLOAT, f8e5m2_to_f32, f32_to_f8e5m2)
+NXH_TR(NXH_I8, int8_t, int64_t, CAT_SINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_U8, uint8_t, int64_t, CAT_UINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_I16, int16_t, int64_t, CAT_SINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_U16, uint16_t, int64_t, CAT_UINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_I32, int32_t, int64_t, CAT_SINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_U32, uint32_t, uint64_t, CAT_UINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_I64, int64_t, int64_t, CAT_SINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_U64, uint64_t, uint64_t, CAT_UINT, NXH_ID, NXH_ID)
+NXH_TR(NXH_C32, c32, c32, CAT_COMPLEX, NXH_ID, NXH_ID)
+NXH_TR(NXH_C64, c64, c64, CAT_COMPLEX, NXH_ID, NXH_ID)
+NXH_TR(NXH_BOOL, uint8_t, uint8_t, CAT_BOOL, NXH_BOOLN, NXH_BOOLN)
+
+// Applies X(DT) to every compute dtype tag (packed int4/uint4 excluded).
+#define NXH_FOR_COMPUTE_DTYPES(X)                                                  \
+  X(NXH_F16) X(NXH_F32) X(NXH_F64) X(NXH_BF16) X(NXH_F8E4M3) X(NXH_F8E5M2) X(NXH_I8) \
+  X(NXH_U8) X(NXH_I16) X(NXH_U16) X(NXH_I32) X(NXH_U32) X(NXH_I64) X(NXH_U64)      \
+  X(NXH_C32) X(NXH_C64) X(NXH_BOOL)
+
+// Saturating double -> integer storage (nx_c.h:234-250): NaN -> 0, clamp.
+template <class S>
+__device__ __forceinline__ S f2i_sat(double v) {
+  constexpr int w = (int)sizeof(S) * 8;
+  if constexpr (std::is_signed<S>::value) {
+    const double lim = (double)((uint64_t)1 << (w - 1));
+    if (v != v) return 0;
+    if (v <= -lim) return (S)((uint64_t)1 << (w - 1));
+    if (v >= lim) return (S)(((uint64_t)1 << (w - 1)) - 1);
+    return (S)(int64_t)v;
+  } else {
+    const double lim = w == 64 ? 18446744073709551616.0 : (double)((uint64_t)1 << (w & 63));
+    if (v != v) return 0;
+    if (v <= 0.0) return 0;
+    if (v >= lim) return (S)(~(uint64_t)0);
+    return (S)(uint64_t)v;
+  }
+}

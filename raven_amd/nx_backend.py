@@ -1,0 +1,328 @@
+"""Host-side mirror of the Nx backend binding, on top of the libnxhip C ABI.
+
+This is what ``nx_backend.ml`` of an ``nx_hip`` library does, written in Python
+because this image has no OCaml toolchain: it allocates each result, unpacks
+tensor handles into ``nxh_tensor`` descriptors and makes one C call per
+primitive. Operation names, argument meaning and error kinds follow
+``Nx_core.Backend_intf.S`` (packages/nx/lib/core/backend_intf.ml:77-721) and
+the reference binding (packages/nx/lib/backend_c/nx_backend.ml):
+
+* a tensor is ``{buffer; shape; strides; offset; dtype; context}``; movement ops
+  only rewrite the view and share the buffer (nx_backend.ml:36-84);
+* compute ops allocate a fresh C-contiguous, offset-0 result
+  (nx_backend.ml:170-183);
+* ``ValueError`` stands for OCaml's ``Invalid_argument``, ``RuntimeError`` for
+  ``Failure`` (nx_c_engine.c:1345-1351).
+
+There is no CPU fallback: constructing a ``Backend`` without a GPU or without
+the built library raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from typing import Sequence
+
+import numpy as np
+
+from . import _ffi
+from . import dtype as dt
+from ._ffi import BINARY_OPS, COMPARE_OPS, REDUCE_OPS, UNARY_OPS, make_tensor
+from .view import View, numel
+
+
+class DeviceBuffer:
+    """One device allocation, shared by every view of a tensor. Returned to the
+    context's caching allocator when the last handle goes away (the OCaml
+    binding does the same from a custom-block finaliser)."""
+
+    __slots__ = ("ctx", "ptr", "nbytes", "__weakref__")
+
+    def __init__(self, ctx: "Backend", nbytes: int):
+        p = C.c_void_p()
+        ctx._check(ctx._lib.nxh_alloc(ctx._h, nbytes, C.byref(p)))
+        self.ctx = ctx
+        self.ptr = p.value
+        self.nbytes = nbytes
+
+    def __del__(self):
+        ctx = getattr(self, "ctx", None)
+        if ctx is not None and ctx._h and self.ptr:
+            ctx._lib.nxh_free(ctx._h, self.ptr)
+            self.ptr = None
+
+
+class Tensor:
+    """The backend's tensor handle (nx_backend.ml:36-43)."""
+
+    __slots__ = ("buffer", "view", "dtype", "context")
+
+    def __init__(self, buffer: DeviceBuffer, view: View, dtype: dt.DType, context: "Backend"):
+        self.buffer = buffer
+        self.view = view
+        self.dtype = dtype
+        self.context = context
+
+    @property
+    def shape(self):
+        return self.view.shape
+
+    @property
+    def strides(self):
+        return self.view.strides
+
+    @property
+    def offset(self):
+        return self.view.offset
+
+    def _desc(self):
+        v = self.view
+        return make_tensor(self.buffer.ptr, self.dtype.tag, v.shape, v.strides, v.offset)
+
+    def __repr__(self):  # pragma: no cover
+        return f"Tensor({self.dtype.name}, shape={self.shape}, strides={self.strides}, offset={self.offset})"
+
+
+def encode_scalar(dtype: dt.DType, value) -> np.ndarray:
+    """Host encoding of a ``full`` value, as ``Nx_buffer.fill`` stores it
+    (packages/nx/lib/buffer/nx_buffer_stubs.h:70-302): one storage element."""
+    if dtype is dt.bfloat16:
+        u = np.asarray(value, dtype=np.float32).reshape(1).view(np.uint32)
+        nan = (u & 0x7FFFFFFF) > 0x7F800000
+        r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+        return np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), r)
+    if dtype in (dt.float8_e4m3, dt.float8_e5m2):
+        raise NotImplementedError("encode fp8 scalars with cast from float32")
+    if dtype.packed:
+        return np.asarray(int(value) & 0xF, dtype=np.uint8).reshape(1)
+    if dtype is dt.bool_:
+        return np.asarray(1 if value else 0, dtype=np.uint8).reshape(1)
+    with np.errstate(all="ignore"):
+        return np.asarray(value).astype(dtype.np_storage).reshape(1)
+
+
+class Backend:
+    """An execution context (``create_context``, nx_backend.mli:32-39) plus the
+    operations of ``Backend_intf.S``."""
+
+    def __init__(self):
+        self._lib = _ffi.load()
+        h = C.c_void_p()
+        rc = self._lib.nxh_context_create(C.byref(h))
+        self._h = h.value
+        if rc != _ffi.NXH_OK:
+            self._h = None
+            raise RuntimeError(self._lib.nxh_last_error(None).decode())
+
+    def close(self):
+        if self._h:
+            self._lib.nxh_context_destroy(self._h)
+            self._h = None
+
+    # ── plumbing ────────────────────────────────────────────────────────────
+    def _check(self, rc: int):
+        if rc == _ffi.NXH_OK:
+            return
+        msg = self._lib.nxh_last_error(self._h).decode()
+        if rc == _ffi.NXH_INVALID_ARGUMENT:
+            raise ValueError(msg)
+        raise RuntimeError(msg)
+
+    def device_info(self):
+        dev, cus = C.c_int(), C.c_int()
+        name = C.create_string_buffer(128)
+        self._check(self._lib.nxh_device_info(self._h, C.byref(dev), name, 128, C.byref(cus)))
+        return {"device": dev.value, "name": name.value.decode(), "compute_units": cus.value}
+
+    def synchronize(self):
+        self._check(self._lib.nxh_synchronize(self._h))
+
+    def last_path(self) -> str:
+        return self._lib.nxh_last_path(self._h).decode()
+
+    def memory_stats(self):
+        v = [C.c_uint64() for _ in range(4)]
+        self._check(self._lib.nxh_memory_stats(self._h, *[C.byref(x) for x in v]))
+        return dict(zip(("in_use", "cached", "reserved", "driver_allocs"), (x.value for x in v)))
+
+    def trim(self):
+        self._check(self._lib.nxh_trim(self._h))
+
+    def timer_start(self):
+        self._check(self._lib.nxh_timer_start(self._h))
+
+    def timer_stop(self) -> float:
+        ms = C.c_float()
+        self._check(self._lib.nxh_timer_stop(self._h, C.byref(ms)))
+        return ms.value
+
+    # ── creation (backend_intf.ml:120-145) ──────────────────────────────────
+    def buffer(self, dtype: dt.DType, shape: Sequence[int]) -> Tensor:
+        """Uninitialised C-contiguous tensor."""
+        shape = tuple(int(s) for s in shape)
+        buf = DeviceBuffer(self, dtype.nbytes(numel(shape)))
+        return Tensor(buf, View.create(shape), dtype, self)
+
+    def full(self, dtype: dt.DType, shape: Sequence[int], value) -> Tensor:
+        """Every element is ``value`` (a Python number, or one already-encoded
+        storage element as a numpy array)."""
+        out = self.buffer(dtype, shape)
+        enc = value if isinstance(value, np.ndarray) else encode_scalar(dtype, value)
+        enc = np.ascontiguousarray(enc.reshape(1))
+        d = out._desc()
+        self._check(self._lib.nxh_fill(self._h, C.byref(d), enc.ctypes.data))
+        return out
+
+    def from_host(self, array: np.ndarray, dtype: dt.DType) -> Tensor:
+        """Copies a flat, C-contiguous host buffer to the device; the result is
+        rank 1 (nx_backend.ml:66-69). The host array may be reused on return."""
+        flat = np.ascontiguousarray(array).reshape(-1)
+        if flat.dtype.itemsize != dtype.np_storage.itemsize:
+            raise ValueError("from_host: host array does not hold this dtype's storage type")
+        n = flat.size * 2 if dtype.packed else flat.size
+        buf = DeviceBuffer(self, flat.nbytes)
+        self._check(self._lib.nxh_memcpy_h2d(self._h, buf.ptr, flat.ctypes.data, flat.nbytes))
+        return Tensor(buf, View.create((n,)), dtype, self)
+
+    def to_host(self, t: Tensor) -> np.ndarray:
+        """The WHOLE backing storage as a flat host array, to be read through
+        the tensor's view (backend_intf.ml:108-116). Waits for the stream."""
+        count = t.buffer.nbytes // t.dtype.np_storage.itemsize
+        host = np.empty(count, dtype=t.dtype.np_storage)
+        self._check(self._lib.nxh_memcpy_d2h(self._h, host.ctypes.data, t.buffer.ptr, host.nbytes))
+        return host
+
+    # ── movement: views only (nx_backend.ml:77-84) ──────────────────────────
+    def _of_view(self, t: Tensor, v: View) -> Tensor:
+        return Tensor(t.buffer, v, t.dtype, self)
+
+    def expand(self, t, shape):
+        return self._of_view(t, t.view.expand(shape))
+
+    def reshape(self, t, shape):
+        return self._of_view(t, t.view.reshape(shape))
+
+    def permute(self, t, axes):
+        return self._of_view(t, t.view.permute(axes))
+
+    def shrink(self, t, bounds):
+        return self._of_view(t, t.view.shrink(bounds))
+
+    def flip(self, t, flags):
+        return self._of_view(t, t.view.flip(flags))
+
+    # ── map family (nx_backend.ml:170-234) ──────────────────────────────────
+    def unary(self, op: str, x: Tensor) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_unary(self._h, UNARY_OPS.index(op), C.byref(o), C.byref(a)))
+        return out
+
+    def binary(self, op: str, x: Tensor, y: Tensor) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a, b = out._desc(), x._desc(), y._desc()
+        self._check(self._lib.nxh_binary(self._h, BINARY_OPS.index(op), C.byref(o), C.byref(a), C.byref(b)))
+        return out
+
+    def compare(self, op: str, x: Tensor, y: Tensor) -> Tensor:
+        out = self.buffer(dt.bool_, x.shape)
+        o, a, b = out._desc(), x._desc(), y._desc()
+        self._check(self._lib.nxh_compare(self._h, COMPARE_OPS.index(op), C.byref(o), C.byref(a), C.byref(b)))
+        return out
+
+    def where(self, cond: Tensor, if_true: Tensor, if_false: Tensor) -> Tensor:
+        out = self.buffer(if_true.dtype, if_true.shape)
+        o, c, a, b = out._desc(), cond._desc(), if_true._desc(), if_false._desc()
+        self._check(self._lib.nxh_where(self._h, C.byref(o), C.byref(c), C.byref(a), C.byref(b)))
+        return out
+
+    def cast(self, x: Tensor, dtype: dt.DType) -> Tensor:
+        out = self.buffer(dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_cast(self._h, C.byref(o), C.byref(a)))
+        return out
+
+    # ── move family (nx_backend.ml:349-357, 399-402) ────────────────────────
+    def copy(self, x: Tensor) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_copy(self._h, C.byref(o), C.byref(a)))
+        return out
+
+    def contiguous(self, x: Tensor) -> Tensor:
+        """``x`` itself iff C-contiguous AND offset 0, else a copy."""
+        if x.view.is_c_contiguous() and x.view.offset == 0:
+            return x
+        return self.copy(x)
+
+    def assign(self, dst: Tensor, src: Tensor) -> None:
+        """Writes ``src`` through ``dst``'s strides (visible through every view
+        sharing dst's buffer)."""
+        o, a = dst._desc(), src._desc()
+        self._check(self._lib.nxh_copy(self._h, C.byref(o), C.byref(a)))
+
+    def gather(self, data: Tensor, indices: Tensor, axis: int) -> Tensor:
+        out = self.buffer(data.dtype, indices.shape)
+        o, d, i = out._desc(), data._desc(), indices._desc()
+        self._check(self._lib.nxh_gather(self._h, C.byref(o), C.byref(d), C.byref(i), axis))
+        return out
+
+    # ── fold family (nx_backend.ml:266-307) ─────────────────────────────────
+    def reduce(self, op: str, axes: Sequence[int], x: Tensor) -> Tensor:
+        axes = sorted(int(a) for a in axes)
+        if op in ("max", "min"):
+            for a in axes:
+                if x.shape[a] == 0:
+                    raise ValueError(f"reduce_{op}: reduction over an empty axis has no identity")
+        oshape = [s for i, s in enumerate(x.shape) if i not in axes]
+        out = self.buffer(x.dtype, oshape)
+        arr = (C.c_int32 * max(len(axes), 1))(*axes)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_reduce(self._h, REDUCE_OPS.index(op), C.byref(o), C.byref(a), arr, len(axes)))
+        return out
+
+    def _argreduce(self, is_min: bool, x: Tensor, axis: int, keepdims: bool) -> Tensor:
+        name = "argmin" if is_min else "argmax"
+        if x.shape[axis] == 0:
+            raise ValueError(f"{name}: argument reduction over an empty axis")
+        if keepdims:
+            oshape = [1 if i == axis else s for i, s in enumerate(x.shape)]
+        else:
+            oshape = [s for i, s in enumerate(x.shape) if i != axis]
+        out = self.buffer(dt.int32, oshape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_argreduce(self._h, int(is_min), C.byref(o), C.byref(a), axis))
+        return out
+
+    def argmax(self, x: Tensor, axis: int, keepdims: bool = False) -> Tensor:
+        return self._argreduce(False, x, axis, keepdims)
+
+    def argmin(self, x: Tensor, axis: int, keepdims: bool = False) -> Tensor:
+        return self._argreduce(True, x, axis, keepdims)
+
+    # ── matmul (nx_backend.ml:485-500) ──────────────────────────────────────
+    def matmul(self, x: Tensor, y: Tensor) -> Tensor:
+        xs, ys = x.shape, y.shape
+        nd = max(len(xs), len(ys))
+        batch = []
+        for i in range(nd - 2):
+            ai, bi = i - (nd - len(xs)), i - (nd - len(ys))
+            batch.append(max(xs[ai] if ai >= 0 else 1, ys[bi] if bi >= 0 else 1))
+        out = self.buffer(x.dtype, batch + [xs[-2], ys[-1]])
+        o, a, b = out._desc(), x._desc(), y._desc()
+        self._check(self._lib.nxh_matmul(self._h, C.byref(o), C.byref(a), C.byref(b)))
+        return out
+
+
+def logical(t: Tensor) -> np.ndarray:
+    """Host copy of the tensor's logical contents (storage dtype), read through
+    its view from the full backing storage."""
+    if t.dtype.packed:
+        raise NotImplementedError("packed tensors have no element-addressable host view")
+    storage = t.context.to_host(t)
+    v = t.view
+    if v.numel == 0:
+        return np.zeros(v.shape, dtype=storage.dtype)
+    es = storage.dtype.itemsize
+    return np.lib.stride_tricks.as_strided(storage[v.offset:], shape=v.shape,
+                                           strides=[s * es for s in v.strides]).copy()

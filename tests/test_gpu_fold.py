@@ -1,0 +1,173 @@
+"""GPU parity of reductions and argmax/argmin against the CPU oracle.
+
+Integer sums/products/extremes and every arg result are bit-exact. Float
+max/min are bit-exact (NaN anywhere -> NaN). Float sums and products are
+reassociated on the GPU, so they are compared with the reference contract's
+rule |err| <= k * a_rel * scale (packages/nx/test/backend_contract.ml:908-913)
+against the oracle, and against exact invariants (sums of ones,
+backend_contract.ml:2611-2644)."""
+
+import numpy as np
+import pytest
+
+from helpers import FLOAT_DTYPES, INT_DTYPES, TOL, close, decode, encode, logical, pair, same_bits
+from raven_amd import dtype as dt
+
+pytestmark = pytest.mark.gpu
+
+# (source shape, view builder, logical rank)
+def fold_layouts():
+    return [
+        ("contig", (6, 40, 70), lambda B, t: t),
+        ("transposed", (6, 70, 40), lambda B, t: B.permute(t, (0, 2, 1))),
+        ("sliced", (8, 41, 73), lambda B, t: B.shrink(t, [(1, 7), (0, 40), (3, 73)])),
+        ("flipped", (6, 40, 70), lambda B, t: B.flip(t, (True, False, True))),
+        ("broadcast", (6, 1, 70), lambda B, t: B.expand(t, (6, 40, 70))),
+    ]
+
+AXES = [[0], [1], [2], [0, 1], [1, 2], [0, 2], [0, 1, 2], []]
+
+
+def check_float_reduce(hip, oracle, d, h, o, what):
+    arith = TOL[d.name][0]
+    for axes in AXES:
+        k = int(np.prod([h.shape[a] for a in axes])) if axes else 1
+        g, w = logical(hip.reduce("sum", axes, h)), logical(oracle.reduce("sum", axes, o))
+        vals = np.abs(decode(logical(oracle.copy(o)), d, oracle))
+        scale = float(np.nanmax(np.where(np.isfinite(vals), vals, 0))) * k
+        close(g, w, d, oracle, arith, arith * max(scale, 1.0), f"sum {axes} {what}")
+        for op in ("max", "min"):
+            g, w = logical(hip.reduce(op, axes, h)), logical(oracle.reduce(op, axes, o))
+            gv, wv = decode(g, d, oracle), decode(w, d, oracle)
+            assert np.array_equal(np.isnan(gv), np.isnan(wv)), (op, axes, what)
+            assert np.array_equal(gv[~np.isnan(gv)], wv[~np.isnan(wv)]), (op, axes, what)
+
+
+@pytest.mark.parametrize("d", FLOAT_DTYPES, ids=lambda d: d.name)
+def test_reduce_float(hip, oracle, d):
+    rng = np.random.default_rng(800 + d.tag)
+    for lname, shape, build in fold_layouts():
+        x = rng.uniform(-2, 2, shape)
+        x.reshape(-1)[rng.integers(0, x.size, 5)] = np.nan
+        h, o = pair(encode(x, d, oracle), d, hip, oracle, build)
+        check_float_reduce(hip, oracle, d, h, o, lname)
+    # products stay near 1 so they neither overflow nor vanish
+    x = encode(rng.uniform(0.9, 1.1, (6, 40, 70)), d, oracle)
+    h, o = pair(x, d, hip, oracle)
+    for axes in ([0], [2], [1, 2]):
+        k = int(np.prod([h.shape[a] for a in axes]))
+        close(logical(hip.reduce("prod", axes, h)), logical(oracle.reduce("prod", axes, o)), d, oracle,
+              TOL[d.name][0] * k, TOL[d.name][0], f"prod {axes}")
+
+
+@pytest.mark.parametrize("d", INT_DTYPES + [dt.bool_], ids=lambda d: d.name)
+def test_reduce_int_exact(hip, oracle, d):
+    rng = np.random.default_rng(900 + d.tag)
+    for lname, shape, build in fold_layouts():
+        if d is dt.bool_:
+            x = (rng.random(shape) < 0.97).astype(np.uint8)
+        else:
+            info = np.iinfo(d.np_storage)
+            x = rng.integers(info.min, info.max, shape, endpoint=True, dtype=d.np_storage)
+        h, o = pair(x, d, hip, oracle, build)
+        for axes in AXES:
+            for op in (["max", "min"] if d is dt.bool_ else ["sum", "prod", "max", "min"]):
+                same_bits(logical(hip.reduce(op, axes, h)), logical(oracle.reduce(op, axes, o)))
+    if d is dt.bool_:
+        with pytest.raises(RuntimeError):
+            hip.reduce("sum", [0], h)
+
+
+@pytest.mark.parametrize("d", [dt.complex64, dt.complex128], ids=lambda d: d.name)
+def test_reduce_complex(hip, oracle, d):
+    rng = np.random.default_rng(950)
+    x = (rng.uniform(-1, 1, (6, 40, 70)) + 1j * rng.uniform(-1, 1, (6, 40, 70))).astype(d.np_storage)
+    h, o = pair(x, d, hip, oracle)
+    for axes in ([0], [2], [0, 1, 2]):
+        k = int(np.prod([h.shape[a] for a in axes]))
+        close(logical(hip.reduce("sum", axes, h)), logical(oracle.reduce("sum", axes, o)), d, oracle,
+              TOL[d.name][0], TOL[d.name][0] * k, "csum")
+    with pytest.raises(RuntimeError):
+        hip.reduce("max", [0], h)
+
+
+@pytest.mark.parametrize("d", FLOAT_DTYPES + INT_DTYPES + [dt.bool_], ids=lambda d: d.name)
+def test_argreduce_exact(hip, oracle, d):
+    rng = np.random.default_rng(1000 + d.tag)
+    for lname, shape, build in fold_layouts():
+        if d.is_float:
+            x = np.round(rng.uniform(-3, 3, shape))  # many ties
+            x.reshape(-1)[rng.integers(0, x.size, 40)] = np.nan
+            x = encode(x, d, oracle)
+        elif d is dt.bool_:
+            x = rng.integers(0, 2, shape).astype(np.uint8)
+        else:
+            info = np.iinfo(d.np_storage)
+            x = rng.integers(max(info.min, -4), min(info.max, 4), shape, endpoint=True).astype(d.np_storage)
+            x.reshape(-1)[:2] = [info.max, info.min]
+        h, o = pair(x, d, hip, oracle, build)
+        for axis in (0, 1, 2):
+            for keep in (False, True):
+                for f in ("argmax", "argmin"):
+                    g = getattr(hip, f)(h, axis, keep)
+                    w = getattr(oracle, f)(o, axis, keep)
+                    assert g.shape == w.shape
+                    same_bits(logical(g), logical(w))
+
+
+def test_long_rows_columns_and_full_reductions(hip, oracle):
+    """Shapes that take the split (two-pass) row and column paths."""
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((3, 200_000)).astype(np.float32)
+    x[1, 150_000] = np.nan
+    h, o = pair(x, dt.float32, hip, oracle)
+    close(logical(hip.reduce("sum", [1], h)), logical(oracle.reduce("sum", [1], o)), dt.float32, oracle, 1e-5, 2.0)
+    assert hip.last_path() == "fold_row_split"
+    g, w = logical(hip.reduce("max", [1], h)), logical(oracle.reduce("max", [1], o))
+    assert np.array_equal(np.isnan(g), np.isnan(w)) and np.array_equal(g[~np.isnan(g)], w[~np.isnan(w)])
+    same_bits(logical(hip.argmax(h, 1)), logical(oracle.argmax(o, 1)))
+    assert hip.last_path() == "arg_row_split"
+    same_bits(logical(hip.argmin(h, 1)), logical(oracle.argmin(o, 1)))
+    y = rng.integers(-1000, 1000, (5000, 300)).astype(np.int32)
+    h, o = pair(y, dt.int32, hip, oracle)
+    same_bits(logical(hip.reduce("sum", [0], h)), logical(oracle.reduce("sum", [0], o)))
+    assert hip.last_path() == "fold_col_split"
+    same_bits(logical(hip.argmax(h, 0)), logical(oracle.argmax(o, 0)))
+    assert hip.last_path() == "arg_col_split"
+    same_bits(logical(hip.reduce("sum", [0, 1], h)), logical(oracle.reduce("sum", [0, 1], o)))
+    z = np.round(rng.uniform(-5, 5, (4097, 513))).astype(np.float32)  # ties across chunk boundaries
+    h, o = pair(z, dt.float32, hip, oracle)
+    for axis in (0, 1):
+        same_bits(logical(hip.argmax(h, axis)), logical(oracle.argmax(o, axis)))
+        same_bits(logical(hip.argmin(h, axis)), logical(oracle.argmin(o, axis)))
+
+
+def test_sum_invariants_and_identities(hip, oracle):
+    # backend_contract.ml:2611-2644: a too-narrow accumulator would stall
+    for d, n in ((dt.float32, 1 << 25), (dt.float16, 4096), (dt.bfloat16, 512), (dt.bfloat16, 1024)):
+        ones = hip.full(d, (n,), encode(np.array([1.0]), d, oracle))
+        got = decode(logical(hip.reshape(hip.reduce("sum", [0], ones), (1,))), d, oracle)[0]
+        assert got == float(n), (d.name, n, got)
+    # int sums wrap
+    x = np.full((3, 1000), 2**31 - 1, np.int32)
+    h, o = pair(x, dt.int32, hip, oracle)
+    same_bits(logical(hip.reduce("sum", [1], h)), logical(oracle.reduce("sum", [1], o)))
+    # empty reduced extent: identities for sum/prod, Invalid_argument for max/min/arg
+    for d in (dt.float32, dt.int16, dt.bfloat16, dt.complex64):
+        e = hip.buffer(d, (0, 5)), oracle.buffer(d, (0, 5))
+        for op in ("sum", "prod"):
+            same_bits(logical(hip.reduce(op, [0], e[0])), logical(oracle.reduce(op, [0], e[1])))
+    for op in ("max", "min"):
+        with pytest.raises(ValueError):
+            hip.reduce(op, [0], hip.buffer(dt.float64, (0, 3)))
+    with pytest.raises(ValueError):
+        hip.argmax(hip.buffer(dt.float64, (0, 3)), 0)
+    # an empty RESULT is a no-op, not an error
+    assert logical(hip.reduce("max", [1], hip.buffer(dt.float32, (0, 3)))).shape == (0,)
+    # reference NaN vectors (backend_contract.ml:2486-2512)
+    t, _ = pair(np.array([1.0, np.nan, 3.0, 2.0]), dt.float64, hip, oracle)
+    assert np.isnan(logical(hip.reduce("max", [0], t))) and np.isnan(logical(hip.reduce("min", [0], t)))
+    t, _ = pair(np.array([np.nan, 1.0, 2.0]), dt.float64, hip, oracle)
+    assert int(logical(hip.argmax(t, 0))) == 0 and int(logical(hip.argmin(t, 0))) == 0
+    t, _ = pair(np.array([5, 0x80000000, 3], np.uint32), dt.uint32, hip, oracle)
+    assert int(logical(hip.argmax(t, 0))) == 1  # backend_contract.ml:2810-2816

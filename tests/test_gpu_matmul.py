@@ -1,0 +1,155 @@
+"""GPU parity of matmul against the CPU oracle and an f64 reference.
+
+Tolerances are the reference GEMM suite's (packages/nx/lib/backend_c/test/
+matmul_test.ml:831-974): f32 1e-3, f64 1e-9, f16 2e-2, bf16 6e-2 (relative to
+the f64 product of the QUANTISED inputs, plus the same absolute term); integer
+products are exact modulo 2^w."""
+
+import numpy as np
+import pytest
+
+from helpers import decode, encode, logical, pair, same_bits
+from raven_amd import dtype as dt
+
+pytestmark = pytest.mark.gpu
+
+MM_TOL = {"float32": 1e-3, "float64": 1e-9, "float16": 2e-2, "bfloat16": 6e-2,
+          "float8_e4m3": 0.3, "float8_e5m2": 0.4, "complex64": 1e-3, "complex128": 1e-9}
+
+
+def ref_f64(a, b, d, oracle):
+    return np.matmul(decode(a, d, oracle), decode(b, d, oracle))
+
+
+def check(hip, oracle, d, ha, hb, a_log, b_log, what):
+    got = decode(logical(hip.matmul(ha, hb)), d, oracle)
+    want = ref_f64(a_log, b_log, d, oracle)
+    tol = MM_TOL[d.name]
+    scale = np.sqrt(a_log.shape[-1])  # typical magnitude of a k-term sum of unit-variance products
+    err = np.abs(got - want)
+    lim = tol * (np.abs(want) + scale)
+    assert got.shape == want.shape, what
+    assert np.all(err <= lim), (what, float(err.max()), float(lim.min()))
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16, dt.float64, dt.float8_e4m3],
+                         ids=lambda d: d.name)
+def test_matmul_layouts(hip, oracle, d):
+    rng = np.random.default_rng(1100 + d.tag)
+    sizes = [(1, 1, 1), (3, 5, 7), (33, 70, 41), (128, 128, 128), (130, 257, 200), (257, 64, 129), (64, 300, 8)]
+    for (m, k, n) in sizes:
+        a = encode(rng.standard_normal((m, k)), d, oracle)
+        b = encode(rng.standard_normal((k, n)), d, oracle)
+        for ta in (False, True):
+            for tb in (False, True):
+                ha, _ = pair(np.ascontiguousarray(a.T) if ta else a, d, hip, oracle,
+                             (lambda B, t: B.permute(t, (1, 0))) if ta else None)
+                hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle,
+                             (lambda B, t: B.permute(t, (1, 0))) if tb else None)
+                check(hip, oracle, d, ha, hb, a, b, f"{m}x{k}x{n} ta={ta} tb={tb}")
+    # offset views and row-strided (every other row / column) operands
+    a = encode(rng.standard_normal((70, 90)), d, oracle)
+    b = encode(rng.standard_normal((100, 80)), d, oracle)
+    ha, _ = pair(a, d, hip, oracle, lambda B, t: B.shrink(t, [(3, 67), (5, 85)]))
+    hb, _ = pair(b, d, hip, oracle, lambda B, t: B.shrink(t, [(7, 87), (1, 78)]))
+    check(hip, oracle, d, ha, hb, a[3:67, 5:85], b[7:87, 1:78], "offset")
+    ha, _ = pair(a, d, hip, oracle,
+                 lambda B, t: B.permute(B.shrink(B.reshape(t, (35, 2, 90)), [(0, 35), (0, 1), (0, 90)]), (0, 2, 1)))
+    ha = hip.reshape(ha, (35, 90))
+    check(hip, oracle, d, ha, hip.shrink(hb, [(0, 80), (0, 77)]) if False else
+          pair(b[:90], d, hip, oracle)[0], a[::2], b[:90], "strided rows")
+
+
+def test_matmul_batched_and_broadcast(hip, oracle):
+    rng = np.random.default_rng(12)
+    for d in (dt.float32, dt.bfloat16):
+        a = encode(rng.standard_normal((2, 3, 40, 50)), d, oracle)
+        b = encode(rng.standard_normal((2, 3, 50, 60)), d, oracle)
+        ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
+        check(hip, oracle, d, ha, hb, a, b, "batched 4-D")
+        # [2,1,m,k] x [3,k,n] -> [2,3,m,n]
+        a1, b1 = a[:, :1], b[0]
+        ha, hb = pair(a1, d, hip, oracle)[0], pair(b1, d, hip, oracle)[0]
+        check(hip, oracle, d, ha, hb, a1, b1, "broadcast")
+        # rank-2 weight broadcast over a rank-3 batch, and a transposed K^T-style view
+        w = encode(rng.standard_normal((50, 30)), d, oracle)
+        x3 = a[0]
+        check(hip, oracle, d, pair(x3, d, hip, oracle)[0], pair(w, d, hip, oracle)[0], x3, w, "x @ W")
+        q = encode(rng.standard_normal((2, 3, 40, 16)), d, oracle)
+        kt = encode(rng.standard_normal((2, 3, 40, 16)), d, oracle)
+        hq = pair(q, d, hip, oracle)[0]
+        hk = pair(kt, d, hip, oracle, lambda B, t: B.permute(t, (0, 1, 3, 2)))[0]
+        check(hip, oracle, d, hq, hk, q, np.swapaxes(kt, -1, -2), "q @ k^T")
+
+
+def test_matmul_vs_oracle_small(hip, oracle):
+    """Same inputs through the oracle's k-ordered f32 accumulation: the two
+    agree to within the tolerance, and exactly on small-integer data where
+    every partial sum is representable (backend_contract.ml:2012-2021)."""
+    rng = np.random.default_rng(13)
+    for d in (dt.float32, dt.bfloat16, dt.float16):
+        a = encode(rng.integers(-4, 5, (65, 96)).astype(np.float64), d, oracle)
+        b = encode(rng.integers(-4, 5, (96, 130)).astype(np.float64), d, oracle)
+        (ha, oa), (hb, ob) = pair(a, d, hip, oracle), pair(b, d, hip, oracle)
+        got, want = logical(hip.matmul(ha, hb)), logical(oracle.matmul(oa, ob))
+        if d is dt.float32:
+            same_bits(got, want)
+        else:
+            assert np.max(np.abs(decode(got, d, oracle) - decode(want, d, oracle))) <= \
+                MM_TOL[d.name] * np.max(np.abs(decode(want, d, oracle)))
+
+
+@pytest.mark.parametrize("d", [dt.int8, dt.uint8, dt.int16, dt.int32, dt.uint32, dt.int64, dt.uint64],
+                         ids=lambda d: d.name)
+def test_matmul_int_exact(hip, oracle, d):
+    rng = np.random.default_rng(1200 + d.tag)
+    info = np.iinfo(d.np_storage)
+    a = rng.integers(info.min, info.max, (19, 37), endpoint=True, dtype=d.np_storage)
+    b = rng.integers(info.min, info.max, (37, 23), endpoint=True, dtype=d.np_storage)
+    (ha, oa), (hb, ob) = pair(a, d, hip, oracle), pair(b, d, hip, oracle)
+    same_bits(logical(hip.matmul(ha, hb)), logical(oracle.matmul(oa, ob)))
+    hat, oat = (B.permute(t, (1, 0)) for B, t in ((hip, pair(a.T.copy(), d, hip, oracle)[0]),
+                                                  (oracle, pair(a.T.copy(), d, hip, oracle)[1])))
+    same_bits(logical(hip.matmul(hat, hb)), logical(oracle.matmul(oat, ob)))
+
+
+def test_matmul_complex_and_edges(hip, oracle):
+    rng = np.random.default_rng(14)
+    for d in (dt.complex64, dt.complex128):
+        a = (rng.standard_normal((9, 21)) + 1j * rng.standard_normal((9, 21))).astype(d.np_storage)
+        b = (rng.standard_normal((21, 13)) + 1j * rng.standard_normal((21, 13))).astype(d.np_storage)
+        got = logical(hip.matmul(pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0])).astype(np.complex128)
+        want = a.astype(np.complex128) @ b.astype(np.complex128)
+        assert np.allclose(got, want, rtol=MM_TOL[d.name], atol=MM_TOL[d.name])
+    # k == 0 stores zeros; m == 0 / n == 0 are no-ops
+    z = logical(hip.matmul(hip.buffer(dt.float32, (3, 0)), hip.buffer(dt.float32, (0, 2))))
+    assert z.tolist() == [[0, 0], [0, 0], [0, 0]]
+    assert logical(hip.matmul(hip.buffer(dt.float32, (0, 4)), hip.buffer(dt.float32, (4, 2)))).shape == (0, 2)
+    with pytest.raises(ValueError):
+        hip.matmul(hip.buffer(dt.float32, (3, 4)), hip.buffer(dt.float32, (5, 2)))
+    with pytest.raises(RuntimeError):
+        hip.matmul(hip.buffer(dt.bool_, (3, 4)), hip.buffer(dt.bool_, (4, 2)))
+
+
+def test_matmul_cancellation_witness(hip, oracle):
+    """matmul_test.ml:182-230: +a on the first k/2 columns, -a on the rest, B all
+    b; the exact product is 0, which only an f32 accumulator rounded once
+    reproduces (|C| <= 0.1 is the reference's bound)."""
+    for d, (m, k, n) in [(dt.float16, (16, 4096, 24)), (dt.bfloat16, (16, 4096, 24)),
+                         (dt.float16, (128, 4096, 128)), (dt.bfloat16, (200, 2304, 130))]:
+        av = np.full((m, k), 1.3)
+        av[:, k // 2:] *= -1
+        a, b = encode(av, d, oracle), encode(np.full((k, n), 1.5), d, oracle)
+        got = decode(logical(hip.matmul(pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0])), d, oracle)
+        assert np.max(np.abs(got)) <= 0.1, (d.name, m, k, n, float(np.max(np.abs(got))))
+
+
+def test_matmul_skinny_decode_shape(hip, oracle):
+    rng = np.random.default_rng(15)
+    for d in (dt.bfloat16, dt.float32):
+        for m in (1, 8, 13):
+            a = encode(rng.standard_normal((m, 1024)) * 0.5, d, oracle)
+            b = encode(rng.standard_normal((1024, 2048)) * 0.5, d, oracle)
+            ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
+            check(hip, oracle, d, ha, hb, a, b, f"skinny m={m}")
+            assert hip.last_path().startswith("gemm_skinny")
