@@ -145,6 +145,10 @@ HD float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
 // even, subnormals kept) matches on every non-NaN input; a NaN keeps its top
 // ten payload bits and is bumped to stay a NaN.
 __device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  // Keep the narrowing a plain v_cvt_f16_f32. Without the barrier the compiler
+  // folds a preceding multiply into v_fma_mixlo_f16(a, b, +0), and (-0) + (+0)
+  // turns a negative-zero product into +0.
+  asm("" : "+v"(f));
   uint32_t u = f2u(f);
   _Float16 h = (_Float16)f;
   uint16_t hw = __builtin_bit_cast(uint16_t, h);

@@ -75,9 +75,9 @@ def layouts(shape3):
     ]
 
 
-def same_bits(got: np.ndarray, want: np.ndarray):
-    assert got.shape == want.shape, (got.shape, want.shape)
-    assert got.dtype == want.dtype, (got.dtype, want.dtype)
+def same_bits(got: np.ndarray, want: np.ndarray, what=""):
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    assert got.dtype == want.dtype, (what, got.dtype, want.dtype)
     g = np.ascontiguousarray(got).view(np.uint8)
     w = np.ascontiguousarray(want).view(np.uint8)
     if not np.array_equal(g, w):
@@ -85,19 +85,19 @@ def same_bits(got: np.ndarray, want: np.ndarray):
                              np.ascontiguousarray(want).reshape(-1).view(f"V{want.dtype.itemsize}"))
         i = int(bad[0])
         raise AssertionError(
-            f"{bad.size} of {got.size} elements differ; first at {i}: "
+            f"{what}: {bad.size} of {got.size} elements differ; first at {i}: "
             f"got {got.reshape(-1)[i]!r} want {want.reshape(-1)[i]!r}")
 
 
-def same_bits_nan_any(got: np.ndarray, want: np.ndarray, d: dt.DType, oracle):
+def same_bits_nan_any(got: np.ndarray, want: np.ndarray, d: dt.DType, oracle, what=""):
     """Bit-exact except that any NaN matches any NaN (payload/sign of a NaN
     produced by arithmetic is not part of the contract)."""
     gv, wv = decode(got, d, oracle), decode(want, d, oracle)
     gn, wn = np.isnan(gv), np.isnan(wv)
-    assert np.array_equal(gn, wn), "NaN positions differ"
+    assert np.array_equal(gn, wn), f"{what}: NaN positions differ"
     g = np.where(gn, np.zeros_like(got), got)
     w = np.where(wn, np.zeros_like(want), want)
-    same_bits(g, w)
+    same_bits(g, w, what)
 
 
 def close(got: np.ndarray, want: np.ndarray, d: dt.DType, oracle, rel: float, abs_: float, what=""):

@@ -48,7 +48,7 @@ def test_unary_float(hip, oracle, d):
         x = encode(float_pool(rng, src_shape, d), d, oracle)
         h, o = pair(x, d, hip, oracle, build)
         for op in EXACT_UNARY:
-            same_bits_nan_any(logical(hip.unary(op, h)), logical(oracle.unary(op, o)), d, oracle)
+            same_bits_nan_any(logical(hip.unary(op, h)), logical(oracle.unary(op, o)), d, oracle, f"{op}/{lname}")
         for op in TRANS_UNARY:
             close(logical(hip.unary(op, h)), logical(oracle.unary(op, o)), d, oracle,
                   TOL[d.name][1], TOL[d.name][1], f"{op}/{lname}")
@@ -76,7 +76,7 @@ def test_unary_int(hip, oracle, d):
     for lname, src_shape, build in layouts(SHAPE):
         h, o = pair(int_pool(rng, src_shape, d), d, hip, oracle, build)
         for op in ["neg", "recip", "abs", "sign", "trunc", "ceil", "floor", "round"]:
-            same_bits(logical(hip.unary(op, h)), logical(oracle.unary(op, o)))
+            same_bits(logical(hip.unary(op, h)), logical(oracle.unary(op, o)), f"{op}/{lname}")
 
 
 def layout_pairs():
@@ -94,7 +94,7 @@ def test_binary_float(hip, oracle, d):
         ha, oa = pair(xa, d, hip, oracle, ba)
         hb, ob = pair(xb, d, hip, oracle, bb)
         for op in ["add", "sub", "mul", "fdiv", "idiv", "max", "min", "mod"]:
-            same_bits_nan_any(logical(hip.binary(op, ha, hb)), logical(oracle.binary(op, oa, ob)), d, oracle)
+            same_bits_nan_any(logical(hip.binary(op, ha, hb)), logical(oracle.binary(op, oa, ob)), d, oracle, f"{op}/{na}/{nb}")
         # pow / atan2: libm, contract tolerance; positive bases keep pow real
         pa = encode(np.abs(decode(xa, d, oracle)) + 0.25, d, oracle)
         hpa, opa = pair(pa, d, hip, oracle, ba)
@@ -120,8 +120,8 @@ def test_binary_int(hip, oracle, d):
             if op == "pow":  # small exponents as well as wild ones
                 e = (xb.astype(np.int64) % 9 - (2 if np.iinfo(d.np_storage).min < 0 else 0)).astype(d.np_storage)
                 he, oe = pair(e, d, hip, oracle, bb)
-                same_bits(logical(hip.binary(op, ha, he)), logical(oracle.binary(op, oa, oe)))
-            same_bits(logical(hip.binary(op, ha, hb)), logical(oracle.binary(op, oa, ob)))
+                same_bits(logical(hip.binary(op, ha, he)), logical(oracle.binary(op, oa, oe)), f"{op}(small exp)/{na}/{nb}")
+            same_bits(logical(hip.binary(op, ha, hb)), logical(oracle.binary(op, oa, ob)), f"{op}/{na}/{nb}")
 
 
 @pytest.mark.parametrize("d", COMPLEX_DTYPES, ids=lambda d: d.name)
@@ -169,7 +169,7 @@ def test_compare_where(hip, oracle, d):
         hb, ob = pair(xb, d, hip, oracle, bb)
         for op in ["cmpeq", "cmpne", "cmplt", "cmple"]:
             hm, om = hip.compare(op, ha, hb), oracle.compare(op, oa, ob)
-            same_bits(logical(hm), logical(om))
+            same_bits(logical(hm), logical(om), f"{op}/{na}/{nb}")
         same_bits(logical(hip.where(hm, ha, hb)), logical(oracle.where(om, oa, ob)))
         # a strided condition as well
         cm = rng.integers(0, 2, sb).astype(np.uint8)
