@@ -1,0 +1,274 @@
+/* nx_hip_stubs.c — OCaml foreign stubs over the libnxhip C ABI
+   (include/nxhip.h). One CAMLprim per reference stub caml_nx_c_<op>
+   (packages/nx/lib/backend_c/nx_backend.ml:104-168,242-264,349,395-397,
+   482-483), same "output first" convention.
+
+   Not compiled in this repository's image (no OCaml toolchain / caml headers);
+   it is the binding a maintainer adds next to nx_backend.ml.
+
+   The OCaml tensor handle is
+     { buffer : dev; shape : int array; strides : int array; offset : int;
+       tag : int; dtype; context }
+   and, as in the reference (nx_c.h:47-61), C reads fixed slots: 0 buffer (a
+   custom block holding the device pointer), 1 shape, 2 strides, 3 offset,
+   4 dtype tag. */
+
+#include <dlfcn.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <caml/alloc.h>
+#include <caml/bigarray.h>
+#include <caml/custom.h>
+#include <caml/fail.h>
+#include <caml/memory.h>
+#include <caml/mlvalues.h>
+#include <caml/threads.h>
+
+#include "nxhip.h"
+
+/* ── libnxhip.so, resolved once ──────────────────────────────────────────── */
+#define NXH_SYMBOLS(X)                                                        \
+  X(context_create) X(context_destroy) X(last_error) X(alloc) X(free)         \
+  X(memcpy_h2d) X(memcpy_d2h) X(synchronize) X(fill) X(unary) X(binary)       \
+  X(compare) X(where) X(cast) X(reduce) X(argreduce) X(matmul) X(copy)        \
+  X(gather) X(dtype_bytes)
+static struct {
+#define X(n) __typeof__(nxh_##n) *n;
+  NXH_SYMBOLS(X)
+#undef X
+} L;
+static void *lib_handle;
+
+static void load_library(void) {
+  if (lib_handle) return;
+  const char *path = getenv("NXHIP_LIBRARY");
+  lib_handle = dlopen(path ? path : "libnxhip.so", RTLD_NOW | RTLD_LOCAL);
+  if (!lib_handle) caml_failwith("create_context: cannot load libnxhip.so");
+#define X(n)                                                       \
+  L.n = (__typeof__(L.n))dlsym(lib_handle, "nxh_" #n);             \
+  if (!L.n) caml_failwith("create_context: libnxhip.so lacks nxh_" #n);
+  NXH_SYMBOLS(X)
+#undef X
+}
+
+/* ── context and device buffers as custom blocks ─────────────────────────── */
+#define Ctx_val(v) (*(nxh_context **)Data_custom_val(v))
+typedef struct {
+  nxh_context *ctx;
+  void *ptr;
+  size_t bytes;
+} dev_block;
+#define Dev_val(v) ((dev_block *)Data_custom_val(v))
+
+static void dev_finalize(value v) {
+  dev_block *d = Dev_val(v);
+  if (d->ptr) L.free(d->ctx, d->ptr); /* stream-ordered inside the library */
+  d->ptr = NULL;
+}
+static struct custom_operations ctx_ops = {"nx_hip.context", custom_finalize_default,
+    custom_compare_default, custom_hash_default, custom_serialize_default,
+    custom_deserialize_default, custom_compare_ext_default, custom_fixed_length_default};
+static struct custom_operations dev_ops = {"nx_hip.buffer", dev_finalize,
+    custom_compare_default, custom_hash_default, custom_serialize_default,
+    custom_deserialize_default, custom_compare_ext_default, custom_fixed_length_default};
+
+/* status -> exception, the reference's split (nx_c_engine.c:1345-1351) */
+static void check(nxh_context *ctx, int rc) {
+  if (rc == NXH_OK) return;
+  const char *msg = L.last_error(ctx);
+  if (rc == NXH_INVALID_ARGUMENT) caml_invalid_argument(msg);
+  caml_failwith(msg);
+}
+
+CAMLprim value caml_nx_hip_create_context(value unit) {
+  CAMLparam1(unit);
+  CAMLlocal1(v);
+  load_library();
+  nxh_context *ctx = NULL;
+  int rc = L.context_create(&ctx);
+  if (rc != NXH_OK) caml_failwith(L.last_error(NULL));
+  v = caml_alloc_custom(&ctx_ops, sizeof(nxh_context *), 0, 1);
+  Ctx_val(v) = ctx;
+  CAMLreturn(v);
+}
+
+CAMLprim value caml_nx_hip_alloc(value vctx, value vbytes) {
+  CAMLparam2(vctx, vbytes);
+  CAMLlocal1(v);
+  size_t bytes = (size_t)Long_val(vbytes);
+  void *p = NULL;
+  check(Ctx_val(vctx), L.alloc(Ctx_val(vctx), bytes, &p));
+  /* caml_alloc_custom_mem lets the GC account for the device bytes */
+  v = caml_alloc_custom_mem(&dev_ops, sizeof(dev_block), bytes);
+  Dev_val(v)->ctx = Ctx_val(vctx);
+  Dev_val(v)->ptr = p;
+  Dev_val(v)->bytes = bytes;
+  CAMLreturn(v);
+}
+
+CAMLprim value caml_nx_hip_bytes(value vdev) { return Val_long((long)Dev_val(vdev)->bytes); }
+
+/* from_host: the bigarray may be mutated or dropped as soon as this returns */
+CAMLprim value caml_nx_hip_from_host(value vdev, value vba) {
+  CAMLparam2(vdev, vba);
+  dev_block *d = Dev_val(vdev);
+  check(d->ctx, L.memcpy_h2d(d->ctx, d->ptr, Caml_ba_data_val(vba), d->bytes));
+  CAMLreturn(Val_unit);
+}
+
+/* to_host: the whole backing storage; waits for the stream with the runtime
+   lock released (the bigarray's data is malloc'd, so it does not move) */
+CAMLprim value caml_nx_hip_to_host(value vba, value vdev) {
+  CAMLparam2(vba, vdev);
+  dev_block *d = Dev_val(vdev);
+  void *dst = Caml_ba_data_val(vba);
+  nxh_context *ctx = d->ctx;
+  void *src = d->ptr;
+  size_t n = d->bytes;
+  caml_enter_blocking_section();
+  int rc = L.memcpy_d2h(ctx, dst, src, n);
+  caml_leave_blocking_section();
+  check(ctx, rc);
+  CAMLreturn(Val_unit);
+}
+
+/* ── operand extraction (nx_c.h:420-434) ─────────────────────────────────── */
+static nxh_context *extract(value v, nxh_tensor *t) {
+  value vs = Field(v, 1), vst = Field(v, 2);
+  int nd = (int)Wosize_val(vs);
+  if (nd > NXH_MAX_NDIM) caml_failwith("ndim exceeds NX_C_MAX_NDIM");
+  if ((int)Wosize_val(vst) != nd) caml_failwith("shape and strides rank disagree");
+  dev_block *d = Dev_val(Field(v, 0));
+  t->data = d->ptr;
+  t->ndim = nd;
+  t->offset = Long_val(Field(v, 3));
+  t->dtype = (int32_t)Long_val(Field(v, 4));
+  for (int i = 0; i < nd; i++) {
+    t->shape[i] = Long_val(Field(vs, i));
+    t->strides[i] = Long_val(Field(vst, i));
+  }
+  return d->ctx;
+}
+
+#define UNARY_STUB(name, OP)                                              \
+  CAMLprim value caml_nx_hip_##name(value vout, value vx) {               \
+    CAMLparam2(vout, vx);                                                 \
+    nxh_tensor o, x;                                                      \
+    nxh_context *c = extract(vout, &o);                                   \
+    extract(vx, &x);                                                      \
+    check(c, L.unary(c, OP, &o, &x));                                     \
+    CAMLreturn(Val_unit);                                                 \
+  }
+#define BINARY_STUB(name, OP)                                             \
+  CAMLprim value caml_nx_hip_##name(value vout, value vx, value vy) {     \
+    CAMLparam3(vout, vx, vy);                                             \
+    nxh_tensor o, x, y;                                                   \
+    nxh_context *c = extract(vout, &o);                                   \
+    extract(vx, &x);                                                      \
+    extract(vy, &y);                                                      \
+    check(c, L.binary(c, OP, &o, &x, &y));                                \
+    CAMLreturn(Val_unit);                                                 \
+  }
+#define COMPARE_STUB(name, OP)                                            \
+  CAMLprim value caml_nx_hip_##name(value vout, value vx, value vy) {     \
+    CAMLparam3(vout, vx, vy);                                             \
+    nxh_tensor o, x, y;                                                   \
+    nxh_context *c = extract(vout, &o);                                   \
+    extract(vx, &x);                                                      \
+    extract(vy, &y);                                                      \
+    check(c, L.compare(c, OP, &o, &x, &y));                               \
+    CAMLreturn(Val_unit);                                                 \
+  }
+UNARY_STUB(neg, NXH_NEG) UNARY_STUB(recip, NXH_RECIP) UNARY_STUB(abs, NXH_ABS)
+UNARY_STUB(sign, NXH_SIGN) UNARY_STUB(sqrt, NXH_SQRT) UNARY_STUB(exp, NXH_EXP)
+UNARY_STUB(log, NXH_LOG) UNARY_STUB(sin, NXH_SIN) UNARY_STUB(cos, NXH_COS)
+UNARY_STUB(tan, NXH_TAN) UNARY_STUB(asin, NXH_ASIN) UNARY_STUB(acos, NXH_ACOS)
+UNARY_STUB(atan, NXH_ATAN) UNARY_STUB(sinh, NXH_SINH) UNARY_STUB(cosh, NXH_COSH)
+UNARY_STUB(tanh, NXH_TANH) UNARY_STUB(trunc, NXH_TRUNC) UNARY_STUB(ceil, NXH_CEIL)
+UNARY_STUB(floor, NXH_FLOOR) UNARY_STUB(round, NXH_ROUND) UNARY_STUB(erf, NXH_ERF)
+BINARY_STUB(add, NXH_ADD) BINARY_STUB(sub, NXH_SUB) BINARY_STUB(mul, NXH_MUL)
+BINARY_STUB(idiv, NXH_IDIV) BINARY_STUB(fdiv, NXH_FDIV) BINARY_STUB(mod, NXH_MOD)
+BINARY_STUB(pow, NXH_POW) BINARY_STUB(atan2, NXH_ATAN2) BINARY_STUB(max, NXH_MAX)
+BINARY_STUB(min, NXH_MIN) BINARY_STUB(xor, NXH_XOR) BINARY_STUB(or, NXH_OR)
+BINARY_STUB(and, NXH_AND)
+COMPARE_STUB(cmpeq, NXH_CMPEQ) COMPARE_STUB(cmpne, NXH_CMPNE)
+COMPARE_STUB(cmplt, NXH_CMPLT) COMPARE_STUB(cmple, NXH_CMPLE)
+
+CAMLprim value caml_nx_hip_where(value vout, value vc, value va, value vb) {
+  CAMLparam4(vout, vc, va, vb);
+  nxh_tensor o, c, a, b;
+  nxh_context *ctx = extract(vout, &o);
+  extract(vc, &c);
+  extract(va, &a);
+  extract(vb, &b);
+  check(ctx, L.where(ctx, &o, &c, &a, &b));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_cast(value vout, value vx) {
+  CAMLparam2(vout, vx);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.cast(c, &o, &x));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_copy(value vout, value vx) {
+  CAMLparam2(vout, vx);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.copy(c, &o, &x));
+  CAMLreturn(Val_unit);
+}
+/* full: the value arrives as a one-element bigarray already encoded by
+   Nx_buffer (so bf16/f16/fp8 use the buffer layer's converters) */
+CAMLprim value caml_nx_hip_fill(value vout, value vba) {
+  CAMLparam2(vout, vba);
+  nxh_tensor o;
+  nxh_context *c = extract(vout, &o);
+  check(c, L.fill(c, &o, Caml_ba_data_val(vba)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_reduce(value vop, value vout, value vx, value vaxes) {
+  CAMLparam4(vop, vout, vx, vaxes);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int n = (int)Wosize_val(vaxes);
+  int32_t axes[NXH_MAX_NDIM];
+  if (n > NXH_MAX_NDIM) caml_failwith("ndim exceeds NX_C_MAX_NDIM");
+  for (int i = 0; i < n; i++) axes[i] = (int32_t)Long_val(Field(vaxes, i));
+  check(c, L.reduce(c, Int_val(vop), &o, &x, axes, n));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_argreduce(value vmin, value vout, value vx, value vaxis) {
+  CAMLparam4(vmin, vout, vx, vaxis);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.argreduce(c, Bool_val(vmin), &o, &x, Int_val(vaxis)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_matmul(value vout, value va, value vb) {
+  CAMLparam3(vout, va, vb);
+  nxh_tensor o, a, b;
+  nxh_context *c = extract(vout, &o);
+  extract(va, &a);
+  extract(vb, &b);
+  check(c, L.matmul(c, &o, &a, &b));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_gather(value vout, value vdata, value vidx, value vaxis) {
+  CAMLparam4(vout, vdata, vidx, vaxis);
+  nxh_tensor o, d, i;
+  nxh_context *c = extract(vout, &o);
+  extract(vdata, &d);
+  extract(vidx, &i);
+  /* waits for the stream to report an out-of-range index from this call */
+  caml_enter_blocking_section();
+  int rc = L.gather(c, &o, &d, &i, Int_val(vaxis));
+  caml_leave_blocking_section();
+  check(c, rc);
+  CAMLreturn(Val_unit);
+}
