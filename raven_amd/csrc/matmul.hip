@@ -25,6 +25,7 @@
 
 #include <algorithm>
 
+#include "gemm_big.hpp"
 #include "nxh_common.hpp"
 
 constexpr int MM_MAXB = 8;  // batch dims decoded on the device
@@ -60,9 +61,8 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
-struct alignas(16) U4 {
-  uint32_t x, y, z, w;
-};
+// A native vector, not a struct: arrays of these stay in registers.
+typedef __attribute__((ext_vector_type(4))) uint32_t U4;
 
 // Per-dtype MFMA traits. VL = elements per 16-byte vector; one "k-chunk" is
 // 2*VL values of k: lanes 0-31 multiply the first VL of them, lanes 32-63 the
@@ -124,13 +124,16 @@ __device__ __forceinline__ void slab_load(U4 (&r)[2], const typename MM::S *p, i
     if (vec && full) {
       r[i] = *reinterpret_cast<const U4 *>(q);
     } else {
-      S t[VL];
+      union {
+        S t[VL];
+        U4 v;
+      } u;
 #pragma unroll
       for (int j = 0; j < VL; j++) {
         int64_t rr = kc ? row : row + j, kk = kc ? k + j : k;
-        t[j] = (rr < nrows && kk < K) ? q[kc ? j * ks : j * rs] : (S)0;
+        u.t[j] = (rr < nrows && kk < K) ? q[kc ? j * ks : j * rs] : (S)0;
       }
-      r[i] = *reinterpret_cast<const U4 *>(t);
+      r[i] = u.v;
     }
   }
 }
@@ -148,9 +151,13 @@ __device__ __forceinline__ void slab_store(const U4 (&r)[2], typename MM::S *lds
       *reinterpret_cast<U4 *>(&lds[row * LDP + k]) = r[i];
     } else {
       const int k = v / (GM / VL), row = (v % (GM / VL)) * VL;
-      const S *t = reinterpret_cast<const S *>(&r[i]);
+      union {
+        U4 v;
+        S t[VL];
+      } u;
+      u.v = r[i];
 #pragma unroll
-      for (int j = 0; j < VL; j++) lds[(row + j) * LDP + k] = t[j];
+      for (int j = 0; j < VL; j++) lds[(row + j) * LDP + k] = u.t[j];
     }
   }
 }
@@ -416,6 +423,51 @@ static int launch_skinny(nxh_context *ctx, GemmArgs &g) {
 
 static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
+// The 256x256x64 kernel: whole tiles only, 16-byte aligned rows, unit-stride C.
+// Returns -1 when the call does not qualify.
+template <bool BF16, bool A_KC, bool B_KC>
+static int launch_big(nxh_context *ctx, const gemm_big::Args &g) {
+  auto kern = gemm_big::kernel<BF16, A_KC, B_KC, 4, 2>;
+  static bool configured = false;  // guarded by the context mutex of the caller
+  if (!configured) {
+    NXH_HIP("matmul", hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)gemm_big::LDS_BYTES));
+    configured = true;
+  }
+  nxh_set_path("gemm_big");
+  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(512), gemm_big::LDS_BYTES, ctx->stream, g);
+  NXH_HIP("matmul", hipGetLastError());
+  return NXH_OK;
+}
+template <bool BF16>
+static int try_big(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b) {
+  if (a.M % gemm_big::BM || a.N % gemm_big::BN || a.K % gemm_big::BK || a.K < gemm_big::BK) return -1;
+  if (a.ccs != 1 || a.batch.n > 4 || !al_a || !al_b) return -1;
+  const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
+  gemm_big::Args g{};
+  g.A = (const uint16_t *)a.A;
+  g.B = (const uint16_t *)a.B;
+  g.C = (uint16_t *)a.C;
+  g.lda = a_kc ? a.ars : a.acs;
+  g.ldb = b_kc ? a.bcs : a.brs;
+  g.ldc = a.crs;
+  if (!al16(g.A) || !al16(g.B) || g.lda % 8 || g.ldb % 8) return -1;
+  g.K = a.K;
+  g.tiles_m = (uint32_t)(a.M / gemm_big::BM);
+  g.tiles_n = (uint32_t)(a.N / gemm_big::BN);
+  g.nbatch = nbatch;
+  if ((uint64_t)g.tiles_m * g.tiles_n * nbatch > 0x7fffffffULL) return -1;
+  g.nbd = a.batch.n;
+  for (int i = 0; i < a.batch.n; i++) {
+    g.bshape[i] = a.batch.shape[i];
+    g.ba[i] = a.batch.a[i];
+    g.bb[i] = a.batch.b[i];
+    g.bc[i] = a.batch.c[i];
+  }
+  if (a_kc) return b_kc ? launch_big<BF16, true, true>(ctx, g) : launch_big<BF16, true, false>(ctx, g);
+  return b_kc ? launch_big<BF16, false, true>(ctx, g) : launch_big<BF16, false, false>(ctx, g);
+}
+
 template <class MM>
 static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool batch_aligned_a,
                           bool batch_aligned_b) {
@@ -428,6 +480,10 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
   }
   const bool a_ok = a.acs == 1 || a.ars == 1, b_ok = a.brs == 1 || a.bcs == 1;
   if (!a_ok || !b_ok) return launch_any<MM::DT>(ctx, a, nbatch);
+  if constexpr (sizeof(S) == 2) {
+    int rc = try_big<MM::DT == NXH_BF16>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
+    if (rc != -1) return rc;
+  }
   // 16-byte loads need an aligned base and every other stride a multiple of VL
   a.a_vec = al16(a.A) && batch_aligned_a && ((a.acs == 1 ? a.ars : a.acs) % VL == 0);
   a.b_vec = al16(a.B) && batch_aligned_b && ((a.brs == 1 ? a.bcs : a.brs) % VL == 0);

@@ -153,3 +153,32 @@ def test_matmul_skinny_decode_shape(hip, oracle):
             ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
             check(hip, oracle, d, ha, hb, a, b, f"skinny m={m}")
             assert hip.last_path().startswith("gemm_skinny")
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_big_tile_kernel(hip, oracle, d):
+    """Whole-256-tile shapes take the large-tile kernel in all four operand
+    orientations, batched and batch-broadcast."""
+    rng = np.random.default_rng(1400 + d.tag)
+    for (m, k, n) in [(256, 64, 256), (512, 192, 768), (768, 320, 256)]:
+        a = encode(rng.standard_normal((m, k)), d, oracle)
+        b = encode(rng.standard_normal((k, n)), d, oracle)
+        for ta in (False, True):
+            for tb in (False, True):
+                ha, _ = pair(np.ascontiguousarray(a.T) if ta else a, d, hip, oracle,
+                             (lambda B, t: B.permute(t, (1, 0))) if ta else None)
+                hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle,
+                             (lambda B, t: B.permute(t, (1, 0))) if tb else None)
+                check(hip, oracle, d, ha, hb, a, b, f"big {m}x{k}x{n} ta={ta} tb={tb}")
+                assert hip.last_path() == "gemm_big"
+    a = encode(rng.standard_normal((3, 2, 256, 128)), d, oracle)
+    b = encode(rng.standard_normal((128, 512)), d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "big batched x broadcast W")
+    assert hip.last_path() == "gemm_big"
+    b4 = encode(rng.standard_normal((3, 1, 128, 256)), d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b4, d, hip, oracle)[0], a, b4, "big batch broadcast")
+    # a sliced (offset, larger row stride) operand still qualifies when rows stay 16-byte aligned
+    wide = encode(rng.standard_normal((256, 256 + 64)), d, oracle)
+    hw, _ = pair(wide, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 256), (32, 288)]))
+    hb2, _ = pair(b4[0, 0][:, :256].copy(), d, hip, oracle)
+    check(hip, oracle, d, hip.shrink(hw, [(0, 256), (0, 128)]), hb2, wide[:, 32:160], b4[0, 0][:, :256], "big sliced A")
