@@ -7,7 +7,12 @@
 //   each wave owns (256/WM) x (256/WN) outputs as 32x32 tiles of
 //   v_mfma_f32_32x32x16 (64 x 128 = 2 x 4 tiles, 128 accumulator registers);
 //   global -> registers -> LDS with the loads for slab t+2 in flight while slab
-//   t is multiplied; one barrier per slab.
+//   t is multiplied; one barrier per slab. Inside a slab the work is software-
+//   pipelined by hand: the LDS fragment reads of k-step s+1, a quarter of the
+//   register -> LDS stores of slab t+1 and a quarter of the global loads of slab
+//   t+2 are issued in front of the 8 MFMAs of k-step s (scheduling barriers keep
+//   the compiler from regrouping them), so memory instructions never queue up
+//   in front of the matrix pipe.
 // An operand that is contiguous along K sits in LDS as [row][k] (+16 B pad) and
 // is fetched with ds_read_b128. An operand that is contiguous along M / N (a
 // row-major B) stays in its memory order, [k][row] (+64 B pad), and the
@@ -21,6 +26,8 @@
 #pragma once
 
 #include "nxh_common.hpp"
+
+#include <type_traits>
 
 namespace gemm_big {
 
@@ -59,26 +66,31 @@ __device__ __forceinline__ void mfma16(f32x16 &acc, const V16 &a, const V16 &b) 
     acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
 }
 
-// Global -> registers: this lane's 8 x 16 bytes of one operand's 256 x 64 slab.
-// KC: rows are 128 B apart in the slab (8 vectors per row); otherwise the slab is
-// 64 k-rows of 512 B (32 vectors per k-row).
+// Global -> registers -> LDS, one 16-byte vector at a time: vector i of this lane
+// (of 2048 / THREADS) of one operand's 256 x 64 slab. KC: rows are 128 B apart in
+// the slab (8 vectors per row); otherwise the slab is 64 k-rows of 512 B (32
+// vectors per k-row).
+template <bool KC, int THREADS>
+__device__ __forceinline__ V16 slab_load1(int i, const uint16_t *p, int64_t ld) {
+  const int v = threadIdx.x + i * THREADS;
+  const uint16_t *q = KC ? p + (int64_t)(v >> 3) * ld + (v & 7) * 8 : p + (int64_t)(v >> 5) * ld + (v & 31) * 8;
+  return *reinterpret_cast<const V16 *>(q);
+}
+template <bool KC, int THREADS>
+__device__ __forceinline__ void slab_store1(int i, const V16 &r, uint16_t *lds) {
+  const int v = threadIdx.x + i * THREADS;
+  uint16_t *q = KC ? lds + (v >> 3) * PK + (v & 7) * 8 : lds + (v >> 5) * PR + (v & 31) * 8;
+  *reinterpret_cast<V16 *>(q) = r;
+}
 template <bool KC, int THREADS>
 __device__ __forceinline__ void slab_load(V16 (&r)[2048 / THREADS], const uint16_t *p, int64_t ld) {
 #pragma unroll
-  for (int i = 0; i < 2048 / THREADS; i++) {
-    const int v = threadIdx.x + i * THREADS;
-    const uint16_t *q = KC ? p + (int64_t)(v >> 3) * ld + (v & 7) * 8 : p + (int64_t)(v >> 5) * ld + (v & 31) * 8;
-    r[i] = *reinterpret_cast<const V16 *>(q);
-  }
+  for (int i = 0; i < 2048 / THREADS; i++) r[i] = slab_load1<KC, THREADS>(i, p, ld);
 }
 template <bool KC, int THREADS>
 __device__ __forceinline__ void slab_store(const V16 (&r)[2048 / THREADS], uint16_t *lds) {
 #pragma unroll
-  for (int i = 0; i < 2048 / THREADS; i++) {
-    const int v = threadIdx.x + i * THREADS;
-    uint16_t *q = KC ? lds + (v >> 3) * PK + (v & 7) * 8 : lds + (v >> 5) * PR + (v & 31) * 8;
-    *reinterpret_cast<V16 *>(q) = r[i];
-  }
+  for (int i = 0; i < 2048 / THREADS; i++) slab_store1<KC, THREADS>(i, r[i], lds);
 }
 
 // One MFMA operand fragment (8 k-values for this lane's row) for k-step `ks`
@@ -170,37 +182,75 @@ __global__ __launch_bounds__(64 * WM * WN) void kernel(Args a) {
   slab_store<A_KC, THREADS>(ra, smem);
   slab_store<B_KC, THREADS>(rb, smem + TILE_ELEMS);
   if (nk > 1) {
-    slab_load<A_KC, THREADS>(ra, gA + stepA, a.lda);
-    slab_load<B_KC, THREADS>(rb, gB + stepB, a.ldb);
+    // same issue order as in the main loop, so its in-order wait counts hold
+#pragma unroll
+    for (int i = 0; i < 2048 / THREADS; i++) {
+      ra[i] = slab_load1<A_KC, THREADS>(i, gA + stepA, a.lda);
+      rb[i] = slab_load1<B_KC, THREADS>(i, gB + stepB, a.ldb);
+    }
   }
   __syncthreads();
 
-  for (int kt = 0; kt < nk; kt++) {
+  constexpr int NV = 2048 / THREADS, KSTEPS = BK / 16, VPS = NV / KSTEPS;  // staged vectors per k-step
+  static_assert(NV % KSTEPS == 0, "staging is spread evenly over the k-steps");
+  // One K-slab: multiply slab kt out of LDS; when STAGE, move slab kt+1 from
+  // registers to the other LDS stage; when FETCH, start the loads of slab kt+2.
+  // Fragments for step ks+1 are fetched while step ks multiplies, and the
+  // staging traffic is spread over the k-steps, a few vectors between each group
+  // of MFMAs, so no wave sits behind a full memory-instruction queue when it
+  // could be issuing MFMAs. The steady state (both true) is free of branches.
+  auto slab = [&](int kt, auto stage_c, auto fetch_c) {
+    constexpr bool STAGE = decltype(stage_c)::value, FETCH = decltype(fetch_c)::value;
     const uint16_t *sA = smem + (kt & 1) * STAGE_ELEMS;
     const uint16_t *sB = sA + TILE_ELEMS;
-    if (kt + 1 < nk) {
-      uint16_t *nA = smem + ((kt + 1) & 1) * STAGE_ELEMS;
-      slab_store<A_KC, THREADS>(ra, nA);
-      slab_store<B_KC, THREADS>(rb, nA + TILE_ELEMS);
-      if (kt + 2 < nk) {
-        slab_load<A_KC, THREADS>(ra, gA + (int64_t)(kt + 2) * stepA, a.lda);
-        slab_load<B_KC, THREADS>(rb, gB + (int64_t)(kt + 2) * stepB, a.ldb);
+    uint16_t *nA = smem + ((kt + 1) & 1) * STAGE_ELEMS;
+    uint16_t *nB = nA + TILE_ELEMS;
+    const uint16_t *pA = gA + (int64_t)(kt + 2) * stepA, *pB = gB + (int64_t)(kt + 2) * stepB;
+    V16 fa[2][TM], fb[2][TN];
+#pragma unroll
+    for (int t = 0; t < TM; t++) fa[0][t] = frag_load<A_KC>(sA, wm + t * 32, 0, lane);
+#pragma unroll
+    for (int u = 0; u < TN; u++) fb[0][u] = frag_load<B_KC>(sB, wn + u * 32, 0, lane);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < KSTEPS) {
+#pragma unroll
+        for (int t = 0; t < TM; t++) fa[nxt][t] = frag_load<A_KC>(sA, wm + t * 32, ks + 1, lane);
+#pragma unroll
+        for (int u = 0; u < TN; u++) fb[nxt][u] = frag_load<B_KC>(sB, wn + u * 32, ks + 1, lane);
       }
-    }
+      if constexpr (STAGE) {
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      V16 fa[TM], fb[TN];
+        for (int j = 0; j < VPS; j++) {
+          slab_store1<A_KC, THREADS>(ks * VPS + j, ra[ks * VPS + j], nA);
+          slab_store1<B_KC, THREADS>(ks * VPS + j, rb[ks * VPS + j], nB);
+        }
+      }
+      if constexpr (FETCH) {
 #pragma unroll
-      for (int t = 0; t < TM; t++) fa[t] = frag_load<A_KC>(sA, wm + t * 32, ks, lane);
-#pragma unroll
-      for (int u = 0; u < TN; u++) fb[u] = frag_load<B_KC>(sB, wn + u * 32, ks, lane);
+        for (int j = 0; j < VPS; j++) {
+          ra[ks * VPS + j] = slab_load1<A_KC, THREADS>(ks * VPS + j, pA, a.lda);
+          rb[ks * VPS + j] = slab_load1<B_KC, THREADS>(ks * VPS + j, pB, a.ldb);
+        }
+      }
+      // keep the order written here (LDS returns in order, so the wait before
+      // the first MFMA only covers the current fragments)
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < TM; t++)
 #pragma unroll
-        for (int u = 0; u < TN; u++) mfma16<BF16>(acc[t][u], fa[t], fb[u]);
+        for (int u = 0; u < TN; u++) mfma16<BF16>(acc[t][u], fa[cur][t], fb[cur][u]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
-  }
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+  int kt = 0;
+  for (; kt + 2 < nk; kt++) slab(kt, yes{}, yes{});
+  if (kt + 1 < nk) slab(kt++, yes{}, no{});
+  slab(kt, no{}, no{});
 
   // accumulator element e of lane l is C[(e/4)*8 + (l/32)*4 + e%4][l%32]
   uint16_t *C = a.C + co;
