@@ -252,7 +252,11 @@ __global__ __launch_bounds__(MAP_THREADS) void map_generic_kernel(GenericArgs<F>
 // ── map_tiled ───────────────────────────────────────────────────────────────
 // Plane (y, x): x is the output's unit-stride dim, y the dim along which the
 // turned inputs are contiguous. All other dims are batch dims decoded per
-// block.
+// block. A block of 256 lanes owns a TILE x TILE patch; every lane moves V
+// consecutive elements per access (16 bytes of the widest operand type), so a
+// wave touches whole 256-byte rows on both sides of the turn.
+enum { TILE_ROW = 0, TILE_TURN = 1, TILE_BX = 2, TILE_ANY = 3 };
+
 template <class F>
 struct TiledArgs {
   char *base[MAP_MAXOP];
@@ -261,47 +265,104 @@ struct TiledArgs {
   uint32_t bshape[MAP_MAXD];
   int64_t bstride[MAP_MAXOP][MAP_MAXD];
   int64_t sx[MAP_MAXOP], sy[MAP_MAXOP];  // element strides along x / y
-  uint32_t turn;                          // bit k: operand k is read along y
+  // per input: TILE_ROW unit stride along x, TILE_TURN unit stride along y (read
+  // along y, turned through LDS), TILE_BX broadcast along x, TILE_ANY strided
+  uint32_t mode[MAP_MAXOP];
+  uint32_t any_turn;
 };
 
-template <class T, int TILE>
-__device__ __forceinline__ void tile_load(T (&r)[TILE * TILE / MAP_THREADS], T *lds, const T *p,
-                                          int64_t sx, int64_t sy, uint32_t x0, uint32_t y0,
-                                          uint32_t nx, uint32_t ny, bool turn) {
-  constexpr int PER = TILE * TILE / MAP_THREADS;
-  constexpr int ROWS = MAP_THREADS / TILE;
-  const uint32_t lane = threadIdx.x % TILE, row = threadIdx.x / TILE;
-  if (!turn) {
+template <int TILE, int V>
+struct TileGeom {
+  static constexpr int G = TILE / V;         // lanes across one row of the patch
+  static constexpr int R = MAP_THREADS / G;  // rows covered by one pass of the block
+  static constexpr int N = TILE / R;         // passes
+  static_assert(G * V == TILE && G * R == MAP_THREADS && N * R == TILE && N >= 1, "tile geometry");
+};
+
+// Issues this lane's global loads of one operand. A turned operand is fetched
+// along y (V consecutive y for N different x); anything else arrives in the
+// output arrangement (V consecutive x for N different y).
+template <class T, int TILE, int V, int NP>
+__device__ __forceinline__ void tile_fetch(Vec<T, V> (&r)[NP], const T *p, int64_t sx,
+                                           int64_t sy, uint32_t x0, uint32_t y0, uint32_t nx,
+                                           uint32_t ny, uint32_t mode) {
+  using TG = TileGeom<TILE, V>;
+  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
+  if (mode == TILE_TURN) {
+    const uint32_t y = y0 + g * V;
+    const T *s = p + (int64_t)y + (int64_t)(x0 + q) * sx;
+    const int64_t step = (int64_t)TG::R * sx;
 #pragma unroll
-    for (int i = 0; i < PER; i++) {
-      uint32_t x = x0 + lane, y = y0 + row + i * ROWS;
-      if (x < nx && y < ny) r[i] = p[(int64_t)y * sy + (int64_t)x * sx];
+    for (int i = 0; i < TG::N; i++) {
+      if (x0 + q + i * TG::R < nx && y < ny) r[i] = *reinterpret_cast<const Vec<T, V> *>(s);
+      s += step;
+    }
+    return;
+  }
+  const uint32_t x = x0 + g * V;
+  const T *s = p + (int64_t)(y0 + q) * sy + (int64_t)x * sx;
+  const int64_t step = (int64_t)TG::R * sy;
+  if (mode == TILE_ROW) {
+#pragma unroll
+    for (int i = 0; i < TG::N; i++) {
+      if (x < nx && y0 + q + i * TG::R < ny) r[i] = *reinterpret_cast<const Vec<T, V> *>(s);
+      s += step;
+    }
+  } else if (mode == TILE_BX) {
+#pragma unroll
+    for (int i = 0; i < TG::N; i++) {
+      if (x < nx && y0 + q + i * TG::R < ny) {
+        const T v = *s;
+#pragma unroll
+        for (int j = 0; j < V; j++) r[i].v[j] = v;
+      }
+      s += step;
     }
   } else {
-    // lanes run along y (this operand's contiguous dim); rows step along x
-    T t[PER];
 #pragma unroll
-    for (int i = 0; i < PER; i++) {
-      uint32_t y = y0 + lane, x = x0 + row + i * ROWS;
-      if (x < nx && y < ny) t[i] = p[(int64_t)y * sy + (int64_t)x * sx];
+    for (int i = 0; i < TG::N; i++) {
+      if (x < nx && y0 + q + i * TG::R < ny) {
+#pragma unroll
+        for (int j = 0; j < V; j++) r[i].v[j] = s[(int64_t)j * sx];
+      }
+      s += step;
     }
-    __syncthreads();  // previous use of this LDS tile is complete
-#pragma unroll
-    for (int i = 0; i < PER; i++) lds[(row + i * ROWS) * (TILE + 1) + lane] = t[i];
-    __syncthreads();
-#pragma unroll
-    for (int i = 0; i < PER; i++) r[i] = lds[lane * (TILE + 1) + row + i * ROWS];
   }
 }
 
-template <class F, int TILE>
+// The turn: lds is [y][x] with a one-element pad, written from the fetch
+// arrangement, read in the output arrangement. Element-wide LDS accesses: the
+// odd pitch keeps both directions free of bank conflicts for 4-byte types.
+template <class T, int TILE, int V, int NP>
+__device__ __forceinline__ void tile_put(const Vec<T, V> (&r)[NP], T *lds) {
+  using TG = TileGeom<TILE, V>;
+  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
+#pragma unroll
+  for (int i = 0; i < TG::N; i++)
+#pragma unroll
+    for (int j = 0; j < V; j++) lds[(g * V + j) * (TILE + 1) + q + i * TG::R] = r[i].v[j];
+}
+template <class T, int TILE, int V, int NP>
+__device__ __forceinline__ void tile_get(Vec<T, V> (&r)[NP], const T *lds) {
+  using TG = TileGeom<TILE, V>;
+  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
+#pragma unroll
+  for (int i = 0; i < TG::N; i++)
+#pragma unroll
+    for (int j = 0; j < V; j++) r[i].v[j] = lds[(q + i * TG::R) * (TILE + 1) + g * V + j];
+}
+
+template <class F, int TILE, int V>
 __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) {
   using MT = MapTypes<F>;
-  constexpr int PER = TILE * TILE / MAP_THREADS;
-  constexpr int ROWS = MAP_THREADS / TILE;
-  __shared__ typename MT::In0 l0[TILE * (TILE + 1)];
-  __shared__ typename MT::In1 l1[F::NIN > 1 ? TILE * (TILE + 1) : 1];
-  __shared__ typename MT::In2 l2[F::NIN > 2 ? TILE * (TILE + 1) : 1];
+  using TG = TileGeom<TILE, V>;
+  using I0 = typename MT::In0;
+  using I1 = typename MT::In1;
+  using I2 = typename MT::In2;
+  using O = typename MT::Out;
+  __shared__ I0 l0[TILE * (TILE + 1)];
+  __shared__ I1 l1[F::NIN > 1 ? TILE * (TILE + 1) : 1];
+  __shared__ I2 l2[F::NIN > 2 ? TILE * (TILE + 1) : 1];
   uint32_t b = blockIdx.x;
   const uint32_t tx = b % a.tiles_x;
   b /= a.tiles_x;
@@ -315,24 +376,40 @@ __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) 
     for (int k = 0; k <= F::NIN; k++) off[k] += (int64_t)c * a.bstride[k][d];
   }
   const uint32_t x0 = tx * TILE, y0 = ty * TILE;
-  typename MT::In0 r0[PER];
-  typename MT::In1 r1[PER];
-  typename MT::In2 r2[PER];
-  tile_load<typename MT::In0, TILE>(r0, l0, (const typename MT::In0 *)a.base[1] + off[1], a.sx[1],
-                                    a.sy[1], x0, y0, a.nx, a.ny, a.turn & 2u);
+  Vec<I0, V> r0[TG::N];
+  Vec<I1, V> r1[TG::N];
+  Vec<I2, V> r2[TG::N];
+  tile_fetch<I0, TILE, V>(r0, (const I0 *)a.base[1] + off[1], a.sx[1], a.sy[1], x0, y0, a.nx, a.ny, a.mode[1]);
   if constexpr (F::NIN > 1)
-    tile_load<typename MT::In1, TILE>(r1, l1, (const typename MT::In1 *)a.base[2] + off[2],
-                                      a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.turn & 4u);
+    tile_fetch<I1, TILE, V>(r1, (const I1 *)a.base[2] + off[2], a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.mode[2]);
   if constexpr (F::NIN > 2)
-    tile_load<typename MT::In2, TILE>(r2, l2, (const typename MT::In2 *)a.base[3] + off[3],
-                                      a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.turn & 8u);
-  typename MT::Out *o = (typename MT::Out *)a.base[0] + off[0];
-  const uint32_t lane = threadIdx.x % TILE, row = threadIdx.x / TILE;
+    tile_fetch<I2, TILE, V>(r2, (const I2 *)a.base[3] + off[3], a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.mode[3]);
+  if (a.any_turn) {
+    if (a.mode[1] == TILE_TURN) tile_put<I0, TILE, V>(r0, l0);
+    if constexpr (F::NIN > 1)
+      if (a.mode[2] == TILE_TURN) tile_put<I1, TILE, V>(r1, l1);
+    if constexpr (F::NIN > 2)
+      if (a.mode[3] == TILE_TURN) tile_put<I2, TILE, V>(r2, l2);
+    __syncthreads();
+    if (a.mode[1] == TILE_TURN) tile_get<I0, TILE, V>(r0, l0);
+    if constexpr (F::NIN > 1)
+      if (a.mode[2] == TILE_TURN) tile_get<I1, TILE, V>(r1, l1);
+    if constexpr (F::NIN > 2)
+      if (a.mode[3] == TILE_TURN) tile_get<I2, TILE, V>(r2, l2);
+  }
+  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
+  const uint32_t x = x0 + g * V;
+  O *o = (O *)a.base[0] + off[0] + (int64_t)(y0 + q) * a.sy[0] + x;
+  const int64_t step = (int64_t)TG::R * a.sy[0];
 #pragma unroll
-  for (int i = 0; i < PER; i++) {
-    uint32_t x = x0 + lane, y = y0 + row + i * ROWS;
-    if (x < a.nx && y < a.ny)
-      o[(int64_t)y * a.sy[0] + (int64_t)x * a.sx[0]] = map_apply<F>(r0[i], r1[i], r2[i]);
+  for (int i = 0; i < TG::N; i++) {
+    if (x < a.nx && y0 + q + i * TG::R < a.ny) {
+      Vec<O, V> v;
+#pragma unroll
+      for (int j = 0; j < V; j++) v.v[j] = map_apply<F>(r0[i].v[j], r1[i].v[j], r2[i].v[j]);
+      *reinterpret_cast<Vec<O, V> *>(o) = v;
+    }
+    o += step;
   }
 }
 
@@ -437,14 +514,23 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
     if (ydim >= 0) {
       constexpr int TILE = MT::smax <= 4 ? 64 : 32;
       TiledArgs<F> a;
-      a.turn = 0;
+      a.any_turn = 0;
+      // 16-byte lanes need every vector of every operand aligned and whole
+      bool vec = V > 1 && p.shape[last] % V == 0 && p.shape[ydim] % V == 0;
       for (int k = 0; k < MAP_MAXOP; k++) {
         a.base[k] = k < p.nop ? p.base[k] : nullptr;
         a.sx[k] = k < p.nop ? p.stride[k][last] : 0;
         a.sy[k] = k < p.nop ? p.stride[k][ydim] : 0;
-        if (k > 0 && k < p.nop && p.stride[k][ydim] == 1 && p.stride[k][last] != 1 &&
-            p.stride[k][last] != 0)
-          a.turn |= 1u << k;
+        a.mode[k] = TILE_ANY;
+        if (k >= p.nop) continue;
+        if (a.sx[k] == 1) a.mode[k] = TILE_ROW;
+        else if (a.sx[k] == 0) a.mode[k] = TILE_BX;
+        else if (a.sy[k] == 1) a.mode[k] = TILE_TURN, a.any_turn = 1;
+        if (a.mode[k] == TILE_ROW || a.mode[k] == TILE_TURN) {
+          if (!aligned_to(p.base[k], (size_t)esz[k] * V)) vec = false;
+          for (int d = 0; d < p.ndim; d++)
+            if (p.stride[k][d] != 1 && p.stride[k][d] % V != 0) vec = false;
+        }
       }
       a.nx = (uint32_t)p.shape[last];
       a.ny = (uint32_t)p.shape[ydim];
@@ -463,8 +549,12 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       int64_t blocks = nb * a.tiles_x * a.tiles_y;
       if (blocks < ((int64_t)1 << 31)) {
         nxh_set_path("map_tiled");
-        hipLaunchKernelGGL((map_tiled_kernel<F, TILE>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
-                           ctx->stream, a);
+        if (vec)
+          hipLaunchKernelGGL((map_tiled_kernel<F, TILE, V>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+                             ctx->stream, a);
+        else
+          hipLaunchKernelGGL((map_tiled_kernel<F, TILE, 1>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+                             ctx->stream, a);
         NXH_HIP(op, hipGetLastError());
         return NXH_OK;
       }
