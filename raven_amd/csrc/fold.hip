@@ -17,15 +17,7 @@
 // Float sums are reassociated (tree order); results agree with the reference
 // within its own tolerance, integer results are exact (modular).
 
-#include <algorithm>
-#include <type_traits>
-
-#include "nxh_common.hpp"
-
-constexpr int FOLD_MAXD = 12;
-constexpr int FOLD_THREADS = 256;
-
-static inline bool aligned_to16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+#include "fold_common.hpp"
 
 // ── combine rules ───────────────────────────────────────────────────────────
 template <int OP, class C, Cat cat>
@@ -70,21 +62,6 @@ constexpr bool fold_ok(int op, Cat c) {
   return (op == NXH_SUM || op == NXH_PROD) ? (c != CAT_BOOL) : (c != CAT_COMPLEX);
 }
 
-// ── lane exchange for any trivially copyable accumulator ───────────────────
-template <class T>
-__device__ __forceinline__ T shfl_down_any(T v, int delta) {
-  constexpr int W = (sizeof(T) + 3) / 4;
-  union {
-    T t;
-    uint32_t w[W];
-  } u;
-  u.w[W - 1] = 0;
-  u.t = v;
-#pragma unroll
-  for (int i = 0; i < W; i++) u.w[i] = __shfl_down(u.w[i], delta, 64);
-  return u.t;
-}
-
 // Reduces `acc` over a group of G lanes (64: one wave; 256: the block). The
 // result is valid in the group's first lane.
 template <class CB, class C, int G>
@@ -98,55 +75,6 @@ __device__ __forceinline__ C group_reduce(C acc, C *lds) {
     if (threadIdx.x == 0) acc = CB::apply(CB::apply(lds[0], lds[1]), CB::apply(lds[2], lds[3]));
   }
   return acc;
-}
-
-// Input / output adaptors: storage-typed (through the dtype converters) or raw
-// compute-typed partials between the two passes.
-template <int DT>
-struct InS {
-  using T = typename Tr<DT>::S;
-  using C = typename Tr<DT>::C;
-  __device__ __forceinline__ static C ld(T s) { return Tr<DT>::ld(s); }
-};
-template <class C_>
-struct InC {
-  using T = C_;
-  using C = C_;
-  __device__ __forceinline__ static C ld(T s) { return s; }
-};
-template <int DT>
-struct OutS {
-  using T = typename Tr<DT>::S;
-  __device__ __forceinline__ static T st(typename Tr<DT>::C c) { return Tr<DT>::st(c); }
-};
-template <class C_>
-struct OutC {
-  using T = C_;
-  __device__ __forceinline__ static T st(C_ c) { return c; }
-};
-
-template <class T, int N>
-struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) FVec {
-  T v[N];
-};
-
-struct FoldDims {
-  int n;
-  uint32_t shape[FOLD_MAXD];
-  int64_t in_stride[FOLD_MAXD];
-  int64_t out_stride[FOLD_MAXD];
-};
-__device__ __forceinline__ void fold_decode(const FoldDims &d, uint64_t idx, int64_t &in_off,
-                                            int64_t &out_off) {
-  in_off = 0;
-  out_off = 0;
-  for (int i = d.n - 1; i >= 0; i--) {
-    uint64_t q = idx / d.shape[i];
-    uint32_t c = (uint32_t)(idx - q * d.shape[i]);
-    idx = q;
-    in_off += (int64_t)c * d.in_stride[i];
-    out_off += (int64_t)c * d.out_stride[i];
-  }
 }
 
 // ── fold_row ────────────────────────────────────────────────────────────────
@@ -217,38 +145,60 @@ struct ColArgs {
   int nsplit;           // > 1: out is partial[(c * n_outer + ob) * L + l]
 };
 
-template <class IN, class CB, class OUT, int V>
+// A block is LANES = 256 / RG column lanes (V adjacent columns each, one
+// 16-byte load per row) by RG row groups: row group g walks rows g, g + RG, ...
+// of the block's chunk with 8 loads in flight, and the RG partial results meet
+// in LDS. RG > 1 keeps the number of partial rows a split leaves for the
+// second pass small while the grid still fills the chip.
+template <class IN, class CB, class OUT, int V, int RG>
 __global__ __launch_bounds__(FOLD_THREADS) void fold_col_kernel(ColArgs a) {
   using T = typename IN::T;
   using C = typename IN::C;
+  constexpr int LANES = FOLD_THREADS / RG;
+  constexpr int U = 8;
+  __shared__ C lds[RG > 1 ? (RG - 1) * LANES * V : 1];
   const uint32_t lb = blockIdx.x % a.lane_blocks;
   const uint64_t ob = blockIdx.x / a.lane_blocks;
   const int c = blockIdx.y;
-  const uint32_t l = (lb * FOLD_THREADS + threadIdx.x) * V;
-  if (l >= a.L) return;
+  const uint32_t ln = threadIdx.x % LANES, rg = threadIdx.x / LANES;
+  const uint32_t l = (lb * LANES + ln) * V;
+  const bool live = l < a.L;
   int64_t in_off, out_off;
   fold_decode(a.outer, ob, in_off, out_off);
   const int64_t r0 = (int64_t)c * a.chunk;
-  const int64_t r1 = r0 + a.chunk < a.R ? r0 + a.chunk : a.R;
+  const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
   const T *p = (const T *)a.in + in_off + l;
   C acc[V];
 #pragma unroll
   for (int k = 0; k < V; k++) acc[k] = CB::init();
-  int64_t r = r0;
-  for (; r + 4 <= r1; r += 4) {
-    FVec<T, V> x[4];
+  int64_t r = r0 + rg;
+  for (; r + (U - 1) * RG < r1; r += U * RG) {
+    FVec<T, V> x[U];
 #pragma unroll
-    for (int j = 0; j < 4; j++) x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j) * a.r_stride);
+    for (int j = 0; j < U; j++) x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j * RG) * a.r_stride);
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < U; j++)
 #pragma unroll
       for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x[j].v[k]));
   }
-  for (; r < r1; r++) {
+  for (; r < r1; r += RG) {
     FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
 #pragma unroll
     for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x.v[k]));
   }
+  if constexpr (RG > 1) {
+    if (rg > 0) {
+#pragma unroll
+      for (int k = 0; k < V; k++) lds[((rg - 1) * V + k) * LANES + ln] = acc[k];
+    }
+    __syncthreads();
+    if (rg > 0) return;
+#pragma unroll
+    for (int g = 1; g < RG; g++)
+#pragma unroll
+      for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], lds[((g - 1) * V + k) * LANES + ln]);
+  }
+  if (!live) return;
   if (a.nsplit > 1) {
     C *o = (C *)a.out + ((uint64_t)c * a.n_outer + ob) * a.L + l;
 #pragma unroll
@@ -296,224 +246,6 @@ __global__ __launch_bounds__(FOLD_THREADS) void fold_any_kernel(AnyArgs a) {
     }
   }
   ((typename OUT::T *)a.out)[out_off] = OUT::st(acc);
-}
-
-// ── argmax / argmin (nx_c_fold.c:93-101, 180-198) ──────────────────────────
-// `beats(v, b)`: v displaces the running best b. Strict, and a NaN displaces a
-// non-NaN, so among equal candidates the smaller index is kept explicitly.
-template <bool IS_MIN, class C, Cat cat>
-struct ArgCmp {
-  __device__ __forceinline__ static bool beats(C v, C b) {
-    if constexpr (cat == CAT_FLOAT) {
-      if constexpr (IS_MIN) return (v < b) || ((v != v) && !(b != b));
-      else return (v > b) || ((v != v) && !(b != b));
-    } else {
-      if constexpr (IS_MIN) return v < b;
-      else return v > b;
-    }
-  }
-  // merge two (value, index) candidates; index < 0 means "none yet"
-  __device__ __forceinline__ static void merge(C &bv, int64_t &bi, C v, int64_t i) {
-    if (i < 0) return;
-    if (bi < 0 || beats(v, bv) || (!beats(bv, v) && i < bi)) {
-      bv = v;
-      bi = i;
-    }
-  }
-};
-
-struct ArgArgs {
-  const void *in;         // values (storage-typed first pass, compute-typed second)
-  const int32_t *in_idx;  // second pass only: index carried by each partial
-  void *out_val;          // first pass with nsplit > 1: partial values (compute-typed)
-  int32_t *out_idx;       // int32 result, or partial indices
-  FoldDims kept;          // row form: all kept dims; col form: kept dims other than the lane
-  uint64_t n_out;
-  int64_t R, r_stride;
-  int64_t chunk;
-  int nsplit;
-  uint32_t L, lane_blocks;  // col form
-  int64_t out_lane_stride;
-};
-
-// Row form: a group of G lanes per output, strided lanes over the axis.
-template <class IN, class CMP, int G, bool HAS_IDX>
-__global__ __launch_bounds__(FOLD_THREADS) void arg_row_kernel(ArgArgs a) {
-  using T = typename IN::T;
-  using C = typename IN::C;
-  __shared__ C lv[4];
-  __shared__ int64_t li[4];
-  constexpr int GROUPS = FOLD_THREADS / G;
-  const int lane = threadIdx.x % G;
-  const uint64_t o = (uint64_t)blockIdx.x * GROUPS + threadIdx.x / G;
-  const bool live = o < a.n_out;
-  const int c = blockIdx.y;
-  int64_t in_off = 0, out_off = 0;
-  if (live) fold_decode(a.kept, o, in_off, out_off);
-  const int64_t r0 = (int64_t)c * a.chunk;
-  const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
-  const T *p = (const T *)a.in + in_off;
-  C bv{};
-  int64_t bi = -1;
-  for (int64_t r = r0 + lane; r < r1; r += G) {
-    C v = IN::ld(p[r * a.r_stride]);
-    int64_t idx = HAS_IDX ? (int64_t)a.in_idx[in_off + r * a.r_stride] : r;
-    CMP::merge(bv, bi, v, idx);
-  }
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) {
-    C ov = shfl_down_any(bv, d);
-    int64_t oi = shfl_down_any(bi, d);
-    CMP::merge(bv, bi, ov, oi);
-  }
-  if constexpr (G == 256) {
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) {
-      lv[wave] = bv;
-      li[wave] = bi;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0)
-      for (int w = 1; w < 4; w++) CMP::merge(bv, bi, lv[w], li[w]);
-  }
-  if (live && lane == 0) {
-    if (a.nsplit > 1) {
-      ((C *)a.out_val)[o * a.nsplit + c] = bv;
-      a.out_idx[o * a.nsplit + c] = (int32_t)bi;
-    } else {
-      a.out_idx[out_off] = (int32_t)bi;
-    }
-  }
-}
-
-// Column form: one lane per output column, rows walked in order.
-template <class IN, class CMP, bool HAS_IDX>
-__global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
-  using T = typename IN::T;
-  using C = typename IN::C;
-  const uint32_t lb = blockIdx.x % a.lane_blocks;
-  const uint64_t ob = blockIdx.x / a.lane_blocks;
-  const int c = blockIdx.y;
-  const uint32_t l = lb * FOLD_THREADS + threadIdx.x;
-  if (l >= a.L) return;
-  int64_t in_off, out_off;
-  fold_decode(a.kept, ob, in_off, out_off);
-  const int64_t r0 = (int64_t)c * a.chunk;
-  const int64_t r1 = r0 + a.chunk < a.R ? r0 + a.chunk : a.R;
-  const T *p = (const T *)a.in + in_off + l;
-  C bv{};
-  int64_t bi = -1;
-  int64_t r = r0;
-  for (; r + 4 <= r1; r += 4) {
-    T x[4];
-    int32_t xi[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      x[j] = p[(r + j) * a.r_stride];
-      if (HAS_IDX) xi[j] = a.in_idx[in_off + l + (r + j) * a.r_stride];
-    }
-#pragma unroll
-    for (int j = 0; j < 4; j++) CMP::merge(bv, bi, IN::ld(x[j]), HAS_IDX ? (int64_t)xi[j] : r + j);
-  }
-  for (; r < r1; r++)
-    CMP::merge(bv, bi, IN::ld(p[r * a.r_stride]),
-               HAS_IDX ? (int64_t)a.in_idx[in_off + l + r * a.r_stride] : r);
-  if (a.nsplit > 1) {
-    uint64_t po = ((uint64_t)c * a.n_out + ob) * a.L + l;
-    ((C *)a.out_val)[po] = bv;
-    a.out_idx[po] = (int32_t)bi;
-  } else {
-    a.out_idx[out_off + (int64_t)l * a.out_lane_stride] = (int32_t)bi;
-  }
-}
-
-// ── host: geometry ──────────────────────────────────────────────────────────
-struct Geom {
-  int nk = 0, nr = 0;
-  int64_t kshape[NXH_MAX_NDIM], kin[NXH_MAX_NDIM], kout[NXH_MAX_NDIM];
-  int64_t rshape[NXH_MAX_NDIM], rin[NXH_MAX_NDIM];
-  int64_t n_out = 1, R = 1;
-};
-
-// Splits dims into kept / reduced (strides in elements), drops size-1 dims and
-// merges neighbours of the same class that compose.
-static void geom_build(const nxh_tensor *in, const nxh_tensor *out_sq, const bool *reduced, Geom *g) {
-  int oj = 0;
-  int last_class = -1;  // 0 kept, 1 reduced: merging needs ADJACENT dims of one class
-  for (int a = 0; a < in->ndim; a++) {
-    int64_t s = in->shape[a], st = in->strides[a];
-    if (reduced[a]) {
-      g->R *= s;
-      if (s != 1) {
-        if (last_class == 1 && g->rin[g->nr - 1] == st * s) {
-          g->rshape[g->nr - 1] *= s;
-          g->rin[g->nr - 1] = st;
-        } else {
-          g->rshape[g->nr] = s;
-          g->rin[g->nr++] = st;
-        }
-        last_class = 1;
-      }
-    } else {
-      int64_t so = out_sq->strides[oj++];
-      g->n_out *= s;
-      if (s != 1) {
-        if (last_class == 0 && g->kin[g->nk - 1] == st * s && g->kout[g->nk - 1] == so * s) {
-          g->kshape[g->nk - 1] *= s;
-          g->kin[g->nk - 1] = st;
-          g->kout[g->nk - 1] = so;
-        } else {
-          g->kshape[g->nk] = s;
-          g->kin[g->nk] = st;
-          g->kout[g->nk++] = so;
-        }
-        last_class = 0;
-      }
-    }
-  }
-}
-
-static bool dims_fill(FoldDims *d, int n, const int64_t *shape, const int64_t *in_s, const int64_t *out_s,
-                      int skip = -1) {
-  d->n = 0;
-  for (int i = 0; i < n; i++) {
-    if (i == skip) continue;
-    if (d->n >= FOLD_MAXD || shape[i] > 0xffffffffLL) return false;
-    d->shape[d->n] = (uint32_t)shape[i];
-    d->in_stride[d->n] = in_s[i];
-    d->out_stride[d->n] = out_s ? out_s[i] : 0;
-    d->n++;
-  }
-  return true;
-}
-// Contiguous (row-major) input strides over the same kept shape, scaled.
-static void dims_contig_in(FoldDims *d, int64_t inner) {
-  int64_t acc = inner;
-  for (int i = d->n - 1; i >= 0; i--) {
-    d->in_stride[i] = acc;
-    acc *= d->shape[i];
-  }
-}
-
-struct Scratch {
-  nxh_context *ctx;
-  void *p[2] = {nullptr, nullptr};
-  explicit Scratch(nxh_context *c) : ctx(c) {}
-  int get(int i, size_t bytes) { return nxh_alloc_locked(ctx, bytes, &p[i]); }
-  ~Scratch() {  // stream-ordered: queued kernels keep using the blocks safely
-    for (void *q : p)
-      if (q) nxh_free_locked(ctx, q);
-  }
-};
-
-static int pick_split(int64_t blocks, int64_t R, int64_t min_chunk, int cus) {
-  // aim for ~8 blocks per CU when a single pass would leave the chip idle
-  const int64_t target = (int64_t)cus * 8;
-  if (blocks >= target / 2 || R < 2 * min_chunk) return 1;
-  int64_t want = (target + blocks - 1) / blocks;
-  int64_t cap = R / min_chunk;
-  int64_t s = std::min<int64_t>(std::min(want, cap), 1024);
-  return (int)std::max<int64_t>(s, 1);
 }
 
 template <int OP, int DT>
@@ -597,10 +329,13 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
       for (int i = 0; vec && i < g.nk; i++)
         if (i != lane && g.kin[i] % V != 0) vec = false;
       const int v = vec ? V : 1;
-      const int64_t lane_blocks = (L + (int64_t)FOLD_THREADS * v - 1) / ((int64_t)FOLD_THREADS * v);
+      // long reduced runs: 4 row groups per block (see fold_col_kernel)
+      const bool rg4 = g.R >= 64;
+      const int64_t lanes = rg4 ? FOLD_THREADS / 4 : FOLD_THREADS;
+      const int64_t lane_blocks = (L + lanes * v - 1) / (lanes * v);
       const int64_t blocks = lane_blocks * n_outer;
       if (blocks <= 0x7fffffffLL) {
-        int nsplit = pick_split(blocks, g.R, 16, cus);
+        int nsplit = pick_split(blocks, g.R, rg4 ? 64 : 16, cus);
         int64_t chunk = (g.R + nsplit - 1) / nsplit;
         nsplit = (int)((g.R + chunk - 1) / chunk);
         a.in = ibase;
@@ -621,10 +356,16 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
         }
         dim3 grid((unsigned)blocks, (unsigned)nsplit);
         nxh_set_path(nsplit > 1 ? "fold_col_split" : "fold_col");
-        if (vec) hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, V>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
-        else hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, 1>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        if (rg4) {
+          if (vec) hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, V, 4>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+          else hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, 1, 4>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        } else {
+          if (vec) hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, V, 1>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+          else hipLaunchKernelGGL((fold_col_kernel<InS<DT>, CB, OutS<DT>, 1, 1>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
+        }
         NXH_HIP(op, hipGetLastError());
         if (nsplit > 1) {
+          // the partial rows [nsplit][n_outer * L] are folded the same way
           ColArgs b = a;
           b.in = scratch.p[0];
           b.out = obase;
@@ -635,10 +376,17 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
           b.nsplit = 1;
           const bool vec2 = L % VC == 0;
           const int v2 = vec2 ? VC : 1;
-          b.lane_blocks = (uint32_t)((L + (int64_t)FOLD_THREADS * v2 - 1) / ((int64_t)FOLD_THREADS * v2));
+          const bool rg4b = nsplit >= 16;
+          const int64_t lanes2 = rg4b ? FOLD_THREADS / 4 : FOLD_THREADS;
+          b.lane_blocks = (uint32_t)((L + lanes2 * v2 - 1) / (lanes2 * v2));
           dim3 grid2((unsigned)(b.lane_blocks * n_outer), 1);
-          if (vec2) hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, VC>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
-          else hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+          if (rg4b) {
+            if (vec2) hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, VC, 4>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+            else hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, 1, 4>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+          } else {
+            if (vec2) hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, VC, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+            else hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, 1, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+          }
           NXH_HIP(op, hipGetLastError());
         }
         return NXH_OK;
@@ -681,7 +429,6 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
   return NXH_OK;
 }
 
-typedef int (*fold_fn)(nxh_context *, const char *, const nxh_tensor *, const nxh_tensor *, const Geom &);
 template <int OP>
 struct FoldRow {
   fold_fn fn[NXH_DTYPE_COUNT] = {};
@@ -695,39 +442,6 @@ struct FoldRow {
 #undef NXH_SET
   }
 };
-
-// nx_c_engine.c:1392-1420: accept a squeezed or a keepdims-shaped output.
-static int squeeze_out(const char *op, const nxh_tensor *in, const nxh_tensor *out, const int32_t *axes,
-                       int nred, bool *reduced, nxh_tensor *sq) {
-  if (nred < 0 || nred > in->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXES);
-  for (int a = 0; a < in->ndim; a++) reduced[a] = false;
-  for (int i = 0; i < nred; i++) {
-    int a = axes[i];
-    if (a < 0 || a >= in->ndim || reduced[a]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXES);
-    if (i > 0 && axes[i] <= axes[i - 1]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXES);
-    reduced[a] = true;
-  }
-  const int kept = in->ndim - nred;
-  *sq = *out;
-  if (out->ndim != kept) {
-    if (out->ndim != in->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_RANK);
-    sq->ndim = kept;
-    int j = 0;
-    for (int a = 0; a < in->ndim; a++)
-      if (!reduced[a]) {
-        sq->shape[j] = out->shape[a];
-        sq->strides[j] = out->strides[a];
-        j++;
-      }
-  }
-  int j = 0;
-  for (int a = 0; a < in->ndim; a++)
-    if (!reduced[a]) {
-      if (sq->shape[j] != in->shape[a]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
-      j++;
-    }
-  return NXH_OK;
-}
 
 // The value 1 in each dtype's storage format, for prod over an empty extent.
 static void storage_one(int dt, void *buf) {
@@ -779,170 +493,6 @@ NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const
     if (op == NXH_PROD) storage_one(dt, one);
     else memset(one, 0, sizeof one);
     return nxh_fill(ctx, &sq, one);
-  }
-  std::lock_guard<std::mutex> guard(ctx->mu);
-  NXH_HIP(name, hipSetDevice(ctx->device));
-  return fn(ctx, name, x, &sq, g);
-}
-
-// ── argreduce host ──────────────────────────────────────────────────────────
-template <bool IS_MIN, int DT>
-static int arg_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, const nxh_tensor *out,
-                      const Geom &g) {
-  using TR = Tr<DT>;
-  using C = typename TR::C;
-  using S = typename TR::S;
-  using CMP = ArgCmp<IS_MIN, C, TR::cat>;
-  const S *ibase = (const S *)in->data + in->offset;
-  int32_t *obase = (int32_t *)out->data + out->offset;
-  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
-  Scratch scratch(ctx);
-  ArgArgs a;
-  a.in = ibase;
-  a.in_idx = nullptr;
-  a.R = g.R;
-  a.r_stride = g.nr ? g.rin[0] : 0;
-  a.n_out = (uint64_t)g.n_out;
-  a.L = 0;
-  a.lane_blocks = 0;
-  a.out_lane_stride = 0;
-
-  // column form: some kept dim is the unit-stride one and the axis is strided
-  int lane = -1;
-  for (int j = 0; j < g.nk; j++)
-    if (g.kin[j] == 1 && g.kshape[j] >= 16 && g.kshape[j] <= 0x7fffffffLL) lane = j;
-  if (lane >= 0 && std::llabs(a.r_stride) > 1 && dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout, lane)) {
-    const int64_t L = g.kshape[lane], n_outer = g.n_out / L;
-    const int64_t lane_blocks = (L + FOLD_THREADS - 1) / FOLD_THREADS;
-    const int64_t blocks = lane_blocks * n_outer;
-    if (blocks <= 0x7fffffffLL) {
-      int nsplit = pick_split(blocks, g.R, 16, cus);
-      int64_t chunk = (g.R + nsplit - 1) / nsplit;
-      nsplit = (int)((g.R + chunk - 1) / chunk);
-      a.n_out = (uint64_t)n_outer;  // col form: number of outer slices
-      a.L = (uint32_t)L;
-      a.lane_blocks = (uint32_t)lane_blocks;
-      a.out_lane_stride = g.kout[lane];
-      a.chunk = chunk;
-      a.nsplit = nsplit;
-      a.out_idx = obase;
-      a.out_val = nullptr;
-      if (nsplit > 1) {
-        int rc = scratch.get(0, (size_t)nsplit * g.n_out * sizeof(C));
-        if (!rc) rc = scratch.get(1, (size_t)nsplit * g.n_out * sizeof(int32_t));
-        if (rc) return rc;
-        a.out_val = scratch.p[0];
-        a.out_idx = (int32_t *)scratch.p[1];
-      }
-      nxh_set_path(nsplit > 1 ? "arg_col_split" : "arg_col");
-      hipLaunchKernelGGL((arg_col_kernel<InS<DT>, CMP, false>), dim3((unsigned)blocks, (unsigned)nsplit),
-                         dim3(FOLD_THREADS), 0, ctx->stream, a);
-      NXH_HIP(op, hipGetLastError());
-      if (nsplit > 1) {
-        ArgArgs b = a;
-        b.in = scratch.p[0];
-        b.in_idx = (const int32_t *)scratch.p[1];
-        b.out_idx = obase;
-        b.out_val = nullptr;
-        dims_contig_in(&b.kept, L);
-        b.R = nsplit;
-        b.r_stride = g.n_out;
-        b.chunk = nsplit;
-        b.nsplit = 1;
-        hipLaunchKernelGGL((arg_col_kernel<InC<C>, CMP, true>), dim3((unsigned)blocks, 1), dim3(FOLD_THREADS), 0,
-                           ctx->stream, b);
-        NXH_HIP(op, hipGetLastError());
-      }
-      return NXH_OK;
-    }
-  }
-
-  // row form: a group of lanes per output walks the axis at its own stride
-  if (!dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout))
-    return nxh_fail(NXH_FAILURE, op, "view has too many non-mergeable dimensions for one launch");
-  const bool wave_rows = g.R < 1024;
-  const int64_t blocks = wave_rows ? (g.n_out + 3) / 4 : g.n_out;
-  if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many outputs for one launch");
-  int nsplit = wave_rows ? 1 : pick_split(blocks, g.R, 8192, cus);
-  int64_t chunk = (g.R + nsplit - 1) / nsplit;
-  nsplit = (int)((g.R + chunk - 1) / chunk);
-  a.chunk = chunk;
-  a.nsplit = nsplit;
-  a.out_idx = obase;
-  a.out_val = nullptr;
-  if (nsplit > 1) {
-    int rc = scratch.get(0, (size_t)nsplit * g.n_out * sizeof(C));
-    if (!rc) rc = scratch.get(1, (size_t)nsplit * g.n_out * sizeof(int32_t));
-    if (rc) return rc;
-    a.out_val = scratch.p[0];
-    a.out_idx = (int32_t *)scratch.p[1];
-  }
-  dim3 grid((unsigned)blocks, (unsigned)nsplit);
-  nxh_set_path(nsplit > 1 ? "arg_row_split" : (wave_rows ? "arg_row_wave" : "arg_row"));
-  if (wave_rows) hipLaunchKernelGGL((arg_row_kernel<InS<DT>, CMP, 64, false>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
-  else hipLaunchKernelGGL((arg_row_kernel<InS<DT>, CMP, 256, false>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a);
-  NXH_HIP(op, hipGetLastError());
-  if (nsplit > 1) {
-    ArgArgs b = a;
-    b.in = scratch.p[0];
-    b.in_idx = (const int32_t *)scratch.p[1];
-    b.out_idx = obase;
-    b.out_val = nullptr;
-    dims_contig_in(&b.kept, nsplit);
-    b.R = nsplit;
-    b.r_stride = 1;
-    b.chunk = nsplit;
-    b.nsplit = 1;
-    hipLaunchKernelGGL((arg_row_kernel<InC<C>, CMP, 64, true>), dim3((unsigned)((g.n_out + 3) / 4), 1),
-                       dim3(FOLD_THREADS), 0, ctx->stream, b);
-    NXH_HIP(op, hipGetLastError());
-  }
-  return NXH_OK;
-}
-
-template <bool IS_MIN>
-struct ArgRow {
-  fold_fn fn[NXH_DTYPE_COUNT] = {};
-  template <int DT>
-  void set() {
-    if constexpr (Tr<DT>::cat != CAT_COMPLEX) fn[DT] = &arg_launch<IS_MIN, DT>;
-  }
-  ArgRow() {
-#define NXH_SET(DT) set<DT>();
-    NXH_FOR_COMPUTE_DTYPES(NXH_SET)
-#undef NXH_SET
-  }
-};
-
-NXH_EXPORT int nxh_argreduce(nxh_context *ctx, int is_min, const nxh_tensor *out, const nxh_tensor *x,
-                             int axis) {
-  const char *name = is_min ? "argmin" : "argmax";
-  if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, name, "null argument");
-  int rc = nxh_check_tensor(name, out);
-  if (!rc) rc = nxh_check_tensor(name, x);
-  if (rc) return rc;
-  static const ArgRow<false> row_max;
-  static const ArgRow<true> row_min;
-  const int dt = x->dtype;
-  fold_fn fn = (is_min ? row_min.fn : row_max.fn)[dt];
-  if (axis < 0 || axis >= x->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_AXIS);
-  bool reduced[NXH_MAX_NDIM];
-  nxh_tensor sq;
-  int32_t ax = axis;
-  rc = squeeze_out(name, x, out, &ax, 1, reduced, &sq);
-  if (rc) return rc;
-  if (!fn) return nxh_fail(NXH_FAILURE, name, nxh_is_packed(dt) ? NXH_ERR_PACKED : NXH_ERR_UNSUPPORTED);
-  if (out->dtype != NXH_I32) return nxh_fail(NXH_FAILURE, name, NXH_ERR_UNSUPPORTED);
-  const int64_t alen = x->shape[axis];
-  if (alen == 0) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_EMPTY_REDUCE);
-  if (alen > INT32_MAX) return nxh_fail(NXH_FAILURE, name, NXH_ERR_ARGCAP);
-  Geom g;
-  geom_build(x, &sq, reduced, &g);
-  if (g.n_out == 0) return NXH_OK;
-  if (g.nr == 0) {  // axis of length 1: every index is 0
-    g.nr = 1;
-    g.rshape[0] = 1;
-    g.rin[0] = 0;
   }
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(name, hipSetDevice(ctx->device));
