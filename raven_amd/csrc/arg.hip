@@ -255,6 +255,7 @@ static int arg_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, co
     if (blocks <= 0x7fffffffLL) {
       int nsplit = pick_split(blocks, g.R, rg4 ? 64 : 16, cus);
       int64_t chunk = (g.R + nsplit - 1) / nsplit;
+      if (nsplit > 1) chunk = chunk_off_channel_stride(chunk, a.r_stride * (int64_t)sizeof(S));
       nsplit = (int)((g.R + chunk - 1) / chunk);
       a.n_out = (uint64_t)n_outer;  // col form: number of outer slices
       a.L = (uint32_t)L;

@@ -337,6 +337,7 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
       if (blocks <= 0x7fffffffLL) {
         int nsplit = pick_split(blocks, g.R, rg4 ? 64 : 16, cus);
         int64_t chunk = (g.R + nsplit - 1) / nsplit;
+        if (nsplit > 1) chunk = chunk_off_channel_stride(chunk, g.rin[0] * (int64_t)sizeof(S));
         nsplit = (int)((g.R + chunk - 1) / chunk);
         a.in = ibase;
         a.n_outer = (uint64_t)n_outer;

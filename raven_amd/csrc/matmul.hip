@@ -15,9 +15,11 @@
 //               K-slab while the current one is multiplied. Either operand may
 //               be K-contiguous or M/N-contiguous in memory; the turn happens
 //               on the way into LDS.
-//   gemm_skinny m <= 16 (decode-like GEMV): HBM-bound on B; lanes own adjacent
-//               output columns, K is split across blocks, partials are summed by
-//               a second pass.
+//   gemm_skinny m <= 16 (decode-like GEMV): HBM-bound on B, which is streamed
+//               once; K is split across blocks only as far as it takes to fill
+//               the chip and the f32 partials are summed by a second pass. f32
+//               runs lane-per-column FMAs, bf16 / f16 run v_mfma_f32_16x16x32
+//               behind a wave-private transposing LDS tile.
 //   gemm_any    every other dtype / layout: one lane per output element.
 // Summation order differs from the reference's k-sequential loop, so float
 // results agree within the reference's GEMM tolerances; integer results are
@@ -237,8 +239,13 @@ __global__ __launch_bounds__(GT) void gemm_mfma_kernel(GemmArgs a) {
 }
 
 // ── gemm_skinny: m <= 16, B streamed once ───────────────────────────────────
-// Lane owns VN adjacent columns; block covers 256*VN columns and one K-chunk.
-// A's chunk [m][kchunk] sits in LDS as f32. Partials [split][m][n] in f32.
+// HBM-bound on B. A block is 64 column lanes (VN adjacent columns each: one
+// 16-byte load per row of B) by 4 row groups; row group g walks rows g, g + 4,
+// ... of the block's K-chunk with SK_U loads in flight, multiplying against the
+// chunk of A held in LDS as f32 [k][m]. The four partial tiles meet in LDS
+// (two folding steps). K is split across blocks only as far as it takes to fill
+// the chip; the [split][m][n] f32 partials are summed by skinny_finish.
+constexpr int SK_LANES = 64, SK_RG = 4, SK_U = 4;
 struct SkinnyArgs {
   const void *A, *B;
   void *C;       // storage-typed result (nsplit == 1) or f32 partials
@@ -248,77 +255,221 @@ struct SkinnyArgs {
   int nsplit;
 };
 template <int DT, int MMAX, int VN>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(SK_LANES *SK_RG) void gemm_skinny_kernel(SkinnyArgs a) {
   using TR = Tr<DT>;
   using S = typename TR::S;
-  constexpr int KT = 64;  // k rows staged per step
-  __shared__ float sA[MMAX][KT];
-  const int64_t n = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VN;
+  struct alignas(sizeof(S) * VN) BV {
+    S v[VN];
+  };
+  extern __shared__ __attribute__((aligned(16))) float sk_lds[];  // A chunk, then the fold buffer
+  const int ln = threadIdx.x % SK_LANES, rg = threadIdx.x / SK_LANES;
+  const int64_t n = ((int64_t)blockIdx.x * SK_LANES + ln) * VN;
   const int64_t k0 = (int64_t)blockIdx.y * a.kchunk;
   const int64_t k1 = k0 + a.kchunk < a.K ? k0 + a.kchunk : a.K;
+  const int kn = (int)(k1 - k0);
+  const S *A = (const S *)a.A;
+  const S *B = (const S *)a.B;
+  for (int idx = threadIdx.x; idx < kn * MMAX; idx += SK_LANES * SK_RG) {
+    const int i = idx / kn, kk = idx - i * kn;  // lanes run along k
+    sk_lds[kk * MMAX + i] = i < a.M ? TR::ld(A[i * a.ars + (k0 + kk) * a.acs]) : 0.0f;
+  }
+  __syncthreads();
   float acc[MMAX][VN];
 #pragma unroll
   for (int i = 0; i < MMAX; i++)
 #pragma unroll
     for (int j = 0; j < VN; j++) acc[i][j] = 0.0f;
-  const S *A = (const S *)a.A;
-  const S *B = (const S *)a.B;
   const bool col_ok = n + VN <= a.N;
-  for (int64_t kb = k0; kb < k1; kb += KT) {
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < MMAX * KT; idx += 256) {
-      int i = idx / KT, kk = idx % KT;
-      sA[i][kk] = (i < a.M && kb + kk < k1) ? TR::ld(A[i * a.ars + (kb + kk) * a.acs]) : 0.0f;
+  auto row_fma = [&](int kk, const BV &t) {
+    float bv[VN];
+#pragma unroll
+    for (int j = 0; j < VN; j++) bv[j] = TR::ld(t.v[j]);
+    const float *ar = sk_lds + kk * MMAX;
+#pragma unroll
+    for (int i = 0; i < MMAX; i++) {
+      const float av = ar[i];
+#pragma unroll
+      for (int j = 0; j < VN; j++) acc[i][j] = __builtin_fmaf(av, bv[j], acc[i][j]);
     }
-    __syncthreads();
-    const int64_t kend = kb + KT < k1 ? kb + KT : k1;
-    if (n < a.N) {
-      for (int64_t k = kb; k < kend; k++) {
-        float bv[VN];
-        const S *bp = B + k * a.brs + n;
-        if (col_ok) {
-          struct alignas(sizeof(S) * VN) BV {
-            S v[VN];
-          } t = *reinterpret_cast<const BV *>(bp);
+  };
+  if (col_ok) {
+    const S *bp = B + k0 * a.brs + n;
+    int kk = rg;
+    for (; kk + (SK_U - 1) * SK_RG < kn; kk += SK_U * SK_RG) {
+      BV t[SK_U];
 #pragma unroll
-          for (int j = 0; j < VN; j++) bv[j] = TR::ld(t.v[j]);
-        } else {
+      for (int u = 0; u < SK_U; u++) t[u] = *reinterpret_cast<const BV *>(bp + (int64_t)(kk + u * SK_RG) * a.brs);
 #pragma unroll
-          for (int j = 0; j < VN; j++) bv[j] = n + j < a.N ? TR::ld(bp[j]) : 0.0f;
-        }
+      for (int u = 0; u < SK_U; u++) row_fma(kk + u * SK_RG, t[u]);
+    }
+    for (; kk < kn; kk += SK_RG) row_fma(kk, *reinterpret_cast<const BV *>(bp + (int64_t)kk * a.brs));
+  } else if (n < a.N) {  // the ragged last lane of a row: element loads
+    for (int kk = rg; kk < kn; kk += SK_RG) {
+      BV t;
 #pragma unroll
-        for (int i = 0; i < MMAX; i++) {
-          const float av = sA[i][k - kb];
-#pragma unroll
-          for (int j = 0; j < VN; j++) acc[i][j] = __builtin_fmaf(av, bv[j], acc[i][j]);
-        }
-      }
+      for (int j = 0; j < VN; j++) t.v[j] = n + j < a.N ? B[(k0 + kk) * a.brs + n + j] : S{};
+      row_fma(kk, t);
     }
   }
-  if (n >= a.N) return;
+  // fold the row groups into group 0, one at a time (the A chunk is dead now)
+#pragma unroll 1
+  for (int g = 1; g < SK_RG; g++) {
+    __syncthreads();
+    float *q = sk_lds + ln;
+    if (rg == g) {
+#pragma unroll
+      for (int i = 0; i < MMAX; i++)
+#pragma unroll
+        for (int j = 0; j < VN; j++) q[(i * VN + j) * SK_LANES] = acc[i][j];
+    }
+    __syncthreads();
+    if (rg == 0) {
+#pragma unroll
+      for (int i = 0; i < MMAX; i++)
+#pragma unroll
+        for (int j = 0; j < VN; j++) acc[i][j] += q[(i * VN + j) * SK_LANES];
+    }
+  }
+  if (rg != 0 || n >= a.N) return;
   if (a.nsplit > 1) {
     float *P = (float *)a.C + (int64_t)blockIdx.y * a.M * a.N;
-    for (int i = 0; i < a.M; i++)
 #pragma unroll
-      for (int j = 0; j < VN; j++)
-        if (n + j < a.N) P[i * a.N + n + j] = acc[i][j];
+    for (int i = 0; i < MMAX; i++)
+      if (i < a.M) {
+#pragma unroll
+        for (int j = 0; j < VN; j++)
+          if (n + j < a.N) P[i * a.N + n + j] = acc[i][j];
+      }
   } else {
     S *C = (S *)a.C;
-    for (int i = 0; i < a.M; i++)
 #pragma unroll
-      for (int j = 0; j < VN; j++)
-        if (n + j < a.N) C[i * a.crs + (n + j) * a.ccs] = TR::st(acc[i][j]);
+    for (int i = 0; i < MMAX; i++)
+      if (i < a.M) {
+#pragma unroll
+        for (int j = 0; j < VN; j++)
+          if (n + j < a.N) C[i * a.crs + (n + j) * a.ccs] = TR::st(acc[i][j]);
+      }
   }
 }
+// ── gemm_skinny_mfma: the same shape for bf16 / f16 on the matrix pipe ──────
+// The lane-per-column kernel above spends 8 FMAs per 2-byte element of B and is
+// VALU-bound for 16-bit types. Here every wave streams its own 64 columns of B:
+// 32 k-rows x 64 columns per step go global -> registers -> a wave-private LDS
+// tile in memory order ([k][n], no block barrier: LDS serves one wave's accesses
+// in order), come back k-contiguous through the transposing LDS read, and feed
+// four v_mfma_f32_16x16x32 against the A chunk held in LDS as [16][k] (rows
+// >= m are zero). Loads for step s+2 are in flight while step s multiplies.
+constexpr int SM_KS = 32, SM_WN = 64, SM_PITCH = SM_WN + 8, SM_TILE = SM_KS * SM_PITCH;
+template <bool BF16>
+__global__ __launch_bounds__(256) void gemm_skinny_mfma_kernel(SkinnyArgs a) {
+  using gemm_big::lds_s16x4;
+  using gemm_big::s16x4;
+  typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+  extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t n0 = ((int64_t)blockIdx.x * 4 + wave) * SM_WN;
+  const int64_t k0 = (int64_t)blockIdx.y * a.kchunk;
+  const int64_t k1 = k0 + a.kchunk < a.K ? k0 + a.kchunk : a.K;
+  const int kn = (int)(k1 - k0), kc = (int)a.kchunk, kpitch = kc + 8;
+  const uint16_t *A = (const uint16_t *)a.A;
+  const uint16_t *B = (const uint16_t *)a.B;
+  uint16_t *sA = sm_lds;
+  uint16_t *sB = sm_lds + 16 * kpitch + wave * (2 * SM_TILE);
+  for (int idx = threadIdx.x; idx < 16 * kc; idx += 256) {
+    const int i = idx / kc, kk = idx - i * kc;
+    sA[i * kpitch + kk] = (i < a.M && kk < kn) ? A[i * a.ars + (k0 + kk) * a.acs] : (uint16_t)0;
+  }
+  __syncthreads();
+  // this lane's four 16-byte vectors of a step: vector v covers row v / 8,
+  // columns (v % 8) * 8 .. + 7 of the wave's tile
+  const int c8 = (lane & 7) * 8, rbase = lane >> 3;
+  const bool col_ok = n0 + c8 < a.N;  // N is a multiple of 8: vectors are whole or absent
+  const uint16_t *bp = B + k0 * a.brs + n0 + c8;
+  U4 rb[4];
+  auto load = [&](int step) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int kk = step * SM_KS + rbase + i * 8;
+      rb[i] = (col_ok && kk < kn) ? *reinterpret_cast<const U4 *>(bp + (int64_t)kk * a.brs) : U4{0, 0, 0, 0};
+    }
+  };
+  auto store = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      *reinterpret_cast<U4 *>(sB + buf * SM_TILE + (rbase + i * 8) * SM_PITCH + c8) = rb[i];
+  };
+  f32x4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  const int nsteps = (kn + SM_KS - 1) / SM_KS;
+  load(0);
+  store(0);
+  if (nsteps > 1) load(1);
+  const int g = lane >> 4, L = lane & 15;
+  for (int s = 0; s < nsteps; s++) {
+    if (s + 1 < nsteps) store((s + 1) & 1);
+    if (s + 2 < nsteps) load(s + 2);
+    const U4 xa = *reinterpret_cast<const U4 *>(sA + L * kpitch + s * SM_KS + g * 8);
+    const uint16_t *tile = sB + (s & 1) * SM_TILE + (g * 8 + (L >> 2)) * SM_PITCH + (L & 3) * 4;
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(tile + t * 16)));
+      const u32x2 hi = __builtin_bit_cast(
+          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(tile + t * 16 + 4 * SM_PITCH)));
+      const U4 yb = U4{lo[0], lo[1], hi[0], hi[1]};
+      if constexpr (BF16)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa), __builtin_bit_cast(bf16x8, yb),
+                                                         acc[t], 0, 0, 0);
+      else
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa), __builtin_bit_cast(f16x8, yb),
+                                                        acc[t], 0, 0, 0);
+    }
+  }
+  // accumulator element e of lane l is C[4 * (l / 16) + e][l % 16] of its tile
+#pragma unroll
+  for (int t = 0; t < 4; t++) {
+    const int64_t n = n0 + t * 16 + L;
+    if (n >= a.N) continue;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const int m = g * 4 + e;
+      if (m >= a.M) continue;
+      if (a.nsplit > 1) ((float *)a.C)[((int64_t)blockIdx.y * a.M + m) * a.N + n] = acc[t][e];
+      else ((uint16_t *)a.C)[m * a.crs + n * a.ccs] = BF16 ? f32_to_bf16(acc[t][e]) : f32_to_f16(acc[t][e]);
+    }
+  }
+}
+
+// Sums the [nsplit][m * n] partials in split order, four outputs per lane.
 template <int DT>
-__global__ void skinny_finish_kernel(const float *P, void *Cv, int64_t M, int64_t N, int nsplit,
-                                     int64_t crs, int64_t ccs) {
+__global__ __launch_bounds__(256) void skinny_finish_kernel(const float *P, void *Cv, int64_t M, int64_t N,
+                                                            int nsplit, int64_t crs, int64_t ccs) {
   using TR = Tr<DT>;
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= M * N) return;
-  float s = 0.0f;
-  for (int c = 0; c < nsplit; c++) s += P[(int64_t)c * M * N + e];
-  ((typename TR::S *)Cv)[(e / N) * crs + (e % N) * ccs] = TR::st(s);
+  typedef __attribute__((ext_vector_type(4))) float f32x4;
+  const int64_t total = M * N;
+  const int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (e >= total) return;
+  typename TR::S *C = (typename TR::S *)Cv;
+  if (e + 4 <= total && (total & 3) == 0) {
+    f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+    int c = 0;
+    for (; c + 8 <= nsplit; c += 8) {
+      f32x4 t[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) t[u] = *reinterpret_cast<const f32x4 *>(P + (int64_t)(c + u) * total + e);
+#pragma unroll
+      for (int u = 0; u < 8; u++) s += t[u];
+    }
+    for (; c < nsplit; c++) s += *reinterpret_cast<const f32x4 *>(P + (int64_t)c * total + e);
+#pragma unroll
+    for (int j = 0; j < 4; j++) C[((e + j) / N) * crs + ((e + j) % N) * ccs] = TR::st(s[j]);
+  } else {
+    for (int64_t x = e; x < total && x < e + 4; x++) {
+      float s = 0.0f;
+      for (int c = 0; c < nsplit; c++) s += P[(int64_t)c * total + x];
+      C[(x / N) * crs + (x % N) * ccs] = TR::st(s);
+    }
+  }
 }
 
 // ── gemm_any: one lane per output, any dtype, any strides ───────────────────
@@ -377,6 +528,7 @@ static int launch_mfma(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
 
 template <int DT, int VN>
 static int launch_skinny(nxh_context *ctx, GemmArgs &g) {
+  using S = typename Tr<DT>::S;
   SkinnyArgs a;
   a.A = g.A;
   a.B = g.B;
@@ -389,14 +541,18 @@ static int launch_skinny(nxh_context *ctx, GemmArgs &g) {
   a.crs = g.crs;
   a.ccs = g.ccs;
   const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
-  const int64_t col_blocks = (g.N + 256 * VN - 1) / (256 * VN);
-  int64_t want = std::max<int64_t>(1, ((int64_t)cus * 4 + col_blocks - 1) / col_blocks);
+  const int mmax = g.M <= 8 ? 8 : 16;
+  const int64_t col_blocks = (g.N + SK_LANES * VN - 1) / (SK_LANES * VN);
+  // two blocks per CU keep enough loads in flight; more splits only add partials
+  int64_t want = std::max<int64_t>(1, ((int64_t)cus * 2 + col_blocks - 1) / col_blocks);
   int64_t nsplit = std::min<int64_t>(want, std::max<int64_t>(1, g.K / 64));
   int64_t kchunk = (g.K + nsplit - 1) / nsplit;
-  kchunk = (kchunk + 63) / 64 * 64;
+  kchunk = std::min<int64_t>((kchunk + 7) / 8 * 8, 1024);  // the A chunk must fit in LDS
+  if (kchunk < g.K) kchunk = chunk_off_channel_stride(kchunk, g.brs * (int64_t)sizeof(S));
   nsplit = std::max<int64_t>(1, (g.K + kchunk - 1) / kchunk);
   a.kchunk = kchunk;
   a.nsplit = (int)nsplit;
+  const size_t lds = sizeof(float) * (size_t)std::max<int64_t>(kchunk * mmax, (int64_t)mmax * VN * SK_LANES);
   void *part = nullptr;
   if (nsplit > 1) {
     int rc = nxh_alloc_locked(ctx, (size_t)nsplit * g.M * g.N * sizeof(float), &part);
@@ -407,12 +563,63 @@ static int launch_skinny(nxh_context *ctx, GemmArgs &g) {
   }
   nxh_set_path(nsplit > 1 ? "gemm_skinny_split" : "gemm_skinny");
   dim3 grid((unsigned)col_blocks, (unsigned)nsplit);
-  if (g.M <= 8) hipLaunchKernelGGL((gemm_skinny_kernel<DT, 8, VN>), grid, dim3(256), 0, ctx->stream, a);
-  else hipLaunchKernelGGL((gemm_skinny_kernel<DT, 16, VN>), grid, dim3(256), 0, ctx->stream, a);
+  if (mmax == 8) hipLaunchKernelGGL((gemm_skinny_kernel<DT, 8, VN>), grid, dim3(SK_LANES * SK_RG), lds, ctx->stream, a);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<DT, 16, VN>), grid, dim3(SK_LANES * SK_RG), lds, ctx->stream, a);
   hipError_t e = hipGetLastError();
   if (e == hipSuccess && nsplit > 1) {
     const int64_t total = g.M * g.N;
-    hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream,
+    hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, ctx->stream,
+                       (const float *)part, g.C, g.M, g.N, (int)nsplit, g.crs, g.ccs);
+    e = hipGetLastError();
+  }
+  if (part) nxh_free_locked(ctx, part);
+  if (e != hipSuccess) return nxh_hip_fail("matmul", e);
+  return NXH_OK;
+}
+
+// bf16 / f16, whole 8-column vectors: the MFMA form of the skinny product.
+template <int DT>
+static int launch_skinny_mfma(nxh_context *ctx, GemmArgs &g) {
+  SkinnyArgs a;
+  a.A = g.A;
+  a.B = g.B;
+  a.M = g.M;
+  a.N = g.N;
+  a.K = g.K;
+  a.ars = g.ars;
+  a.acs = g.acs;
+  a.brs = g.brs;
+  a.crs = g.crs;
+  a.ccs = g.ccs;
+  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  const int64_t col_blocks = (g.N + 4 * SM_WN - 1) / (4 * SM_WN);
+  int64_t want = std::max<int64_t>(1, ((int64_t)cus * 2 + col_blocks - 1) / col_blocks);
+  int64_t nsplit = std::min<int64_t>(want, std::max<int64_t>(1, g.K / 128));
+  int64_t kchunk = (g.K + nsplit - 1) / nsplit;
+  kchunk = std::min<int64_t>((kchunk + SM_KS - 1) / SM_KS * SM_KS, 1024);  // the A chunk must fit in LDS
+  if (kchunk < g.K) {
+    kchunk = chunk_off_channel_stride(kchunk, g.brs * 2);
+    kchunk = (kchunk + SM_KS - 1) / SM_KS * SM_KS;
+  }
+  nsplit = std::max<int64_t>(1, (g.K + kchunk - 1) / kchunk);
+  a.kchunk = kchunk;
+  a.nsplit = (int)nsplit;
+  const size_t lds = sizeof(uint16_t) * (size_t)(16 * (kchunk + 8) + 4 * 2 * SM_TILE);
+  void *part = nullptr;
+  if (nsplit > 1) {
+    int rc = nxh_alloc_locked(ctx, (size_t)nsplit * g.M * g.N * sizeof(float), &part);
+    if (rc) return rc;
+    a.C = part;
+  } else {
+    a.C = g.C;
+  }
+  nxh_set_path(nsplit > 1 ? "gemm_skinny_mfma_split" : "gemm_skinny_mfma");
+  dim3 grid((unsigned)col_blocks, (unsigned)nsplit);
+  hipLaunchKernelGGL((gemm_skinny_mfma_kernel<DT == NXH_BF16>), grid, dim3(256), lds, ctx->stream, a);
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess && nsplit > 1) {
+    const int64_t total = g.M * g.N;
+    hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, ctx->stream,
                        (const float *)part, g.C, g.M, g.N, (int)nsplit, g.crs, g.ccs);
     e = hipGetLastError();
   }
@@ -475,8 +682,12 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
   constexpr int VL = MM::VL;
   // decode-like shape: one batch, few rows, B row-major: stream B once
   if (nbatch == 1 && a.M <= 16 && a.bcs == 1 && a.N >= 1024 && a.K >= 256 && a.batch.n == 0) {
-    constexpr int VN = sizeof(S) == 2 ? 4 : 2;
-    if (a.brs % VN == 0 && ((uintptr_t)a.B % (sizeof(S) * VN)) == 0) return launch_skinny<MM::DT, VN>(ctx, a);
+    constexpr int VN = 16 / (int)sizeof(S);  // one 16-byte load per lane and row of B
+    if (a.brs % VN == 0 && ((uintptr_t)a.B % (sizeof(S) * VN)) == 0) {
+      if constexpr (sizeof(S) == 2)
+        if (a.N % 8 == 0) return launch_skinny_mfma<MM::DT>(ctx, a);
+      return launch_skinny<MM::DT, VN>(ctx, a);
+    }
   }
   const bool a_ok = a.acs == 1 || a.ars == 1, b_ok = a.brs == 1 || a.bcs == 1;
   if (!a_ok || !b_ok) return launch_any<MM::DT>(ctx, a, nbatch);

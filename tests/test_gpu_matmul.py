@@ -153,6 +153,27 @@ def test_matmul_skinny_decode_shape(hip, oracle):
             ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
             check(hip, oracle, d, ha, hb, a, b, f"skinny m={m}")
             assert hip.last_path().startswith("gemm_skinny")
+    # ragged shapes: K not a multiple of the row-group unroll, N ending inside a
+    # lane's 16-byte vector (a column slice of a wider, aligned B), m = 16
+    for d in (dt.float16, dt.float32):
+        a = encode(rng.standard_normal((16, 1003)) * 0.5, d, oracle)
+        bw = encode(rng.standard_normal((1003, 2056)) * 0.5, d, oracle)
+        ha = pair(a, d, hip, oracle)[0]
+        hb = pair(bw, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 1003), (0, 2051)]))[0]
+        check(hip, oracle, d, ha, hb, a, np.ascontiguousarray(bw[:, :2051]), "skinny ragged")
+        assert hip.last_path().startswith("gemm_skinny")
+        # whole 8-column vectors but a ragged K and a column count that ends inside a wave's tile
+        hb = pair(bw, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 1003), (8, 2048)]))[0]
+        check(hip, oracle, d, ha, hb, a, np.ascontiguousarray(bw[:, 8:2048]), "skinny ragged K")
+        assert hip.last_path().startswith("gemm_skinny_mfma" if d is dt.float16 else "gemm_skinny")
+    # an Inf in B next to the K tail must not leak through zero padding
+    a = encode(rng.standard_normal((4, 300)) * 0.5, dt.bfloat16, oracle)
+    b = encode(rng.standard_normal((300, 1024)) * 0.5, dt.bfloat16, oracle)
+    b[299, 5] = 0x7F80  # +inf in bf16 storage
+    ha, hb = pair(a, dt.bfloat16, hip, oracle)[0], pair(b, dt.bfloat16, hip, oracle)[0]
+    got = decode(logical(hip.matmul(ha, hb)), dt.bfloat16, oracle)
+    assert hip.last_path().startswith("gemm_skinny_mfma")
+    assert np.all(np.isinf(got[:, 5]) | np.isnan(got[:, 5])) and np.all(np.isfinite(np.delete(got, 5, axis=1)))
 
 
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
