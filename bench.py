@@ -261,6 +261,70 @@ def cpu_baseline(seconds_budget=20.0):
     }, out
 
 
+class CountingBackend:
+    """Forwards to the backend and counts the calls that launch work."""
+
+    LAUNCHING = ("unary", "binary", "compare", "where", "cast", "copy", "contiguous", "gather", "reduce",
+                 "matmul", "full", "from_host")
+
+    def __init__(self, inner):
+        self._inner, self.calls = inner, {}
+
+    def __getattr__(self, name):
+        attr = getattr(self._inner, name)
+        if name not in self.LAUNCHING:
+            return attr
+
+        def counted(*a, **k):
+            self.calls[name] = self.calls.get(name, 0) + 1
+            return attr(*a, **k)
+
+        return counted
+
+
+def config5(hip, iters=3, warmup=1):
+    """GPT-2-small-shaped eager forward (12 layers, d 768, 12 heads, FFN 3072,
+    vocab 50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s."""
+    from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
+    from raven_amd.nx_frontend import Nx
+
+    cfg = Config.small()
+    batch, seq = 8, 1024
+
+    def enc(a, d):  # f32 -> bf16 storage, round to nearest even
+        u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+        return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+    counter = CountingBackend(hip)
+    nx = Nx(counter)
+    params = upload(nx, host_params(cfg, seed=16), dt.bfloat16, enc)
+    ids = nx.create(dt.int32, (batch, seq),
+                    np.random.default_rng(17).integers(0, cfg.vocab_size, (batch, seq)).astype(np.int32))
+    model = Gpt2(nx, cfg)
+    for _ in range(warmup):
+        out = model.logits(params, ids)
+        del out
+    hip.synchronize()
+    counter.calls.clear()
+    t0 = time.perf_counter()
+    hip.timer_start()
+    for _ in range(iters):
+        out = model.logits(params, ids)
+        del out
+    ev_ms = hip.timer_stop() / iters
+    hip.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / iters
+    calls = {k: v // iters for k, v in counter.calls.items()}
+    flops = 284812800 * batch * seq  # matmul FLOPs per forward
+    rec = {"op": "cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 (eager, one backend call per primitive)",
+           "ms": round(ms, 3), "tokens/s": round(batch * seq / (ms * 1e-3), 1), "hip_event_ms": round(ev_ms, 3),
+           "matmul_TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1), "backend_calls": sum(calls.values()),
+           "calls_by_kind": calls}
+    del params, ids, model
+    hip.trim()
+    return rec
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -268,6 +332,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only-step", action="store_true", help="time the headline step only")
+    ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 forward leg only and print its record")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -275,6 +340,9 @@ def main():
 
     hip = Backend()
     info = hip.device_info()
+    if args.only_gpt2:
+        print(json.dumps(config5(hip)))
+        return
     W = Workloads(hip)
     step_ops = W.config2()
     step_bytes = sum(o.nbytes for o in step_ops)
@@ -332,6 +400,7 @@ def main():
             del ops
             W.keep.clear()
             hip.trim()
+        ops_out.append(config5(hip))
 
     line = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,

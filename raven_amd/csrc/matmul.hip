@@ -358,7 +358,7 @@ __global__ __launch_bounds__(SK_LANES *SK_RG) void gemm_skinny_kernel(SkinnyArgs
 // tile in memory order ([k][n], no block barrier: LDS serves one wave's accesses
 // in order), come back k-contiguous through the transposing LDS read, and feed
 // four v_mfma_f32_16x16x32 against the A chunk held in LDS as [16][k] (rows
-// >= m are zero). Loads for step s+2 are in flight while step s multiplies.
+// >= m are zero). Loads run three steps ahead of the multiply.
 constexpr int SM_KS = 32, SM_WN = 64, SM_PITCH = SM_WN + 8, SM_TILE = SM_KS * SM_PITCH;
 template <bool BF16>
 __global__ __launch_bounds__(256) void gemm_skinny_mfma_kernel(SkinnyArgs a) {
@@ -385,30 +385,32 @@ __global__ __launch_bounds__(256) void gemm_skinny_mfma_kernel(SkinnyArgs a) {
   const int c8 = (lane & 7) * 8, rbase = lane >> 3;
   const bool col_ok = n0 + c8 < a.N;  // N is a multiple of 8: vectors are whole or absent
   const uint16_t *bp = B + k0 * a.brs + n0 + c8;
-  U4 rb[4];
-  auto load = [&](int step) {
+  // three register sets rotate through the steps: while step s multiplies, the
+  // loads of steps s+2 .. s+4 are in flight (12 x 16 bytes per lane)
+  U4 rb[3][4];
+  auto load = [&](U4 (&r)[4], int step) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int kk = step * SM_KS + rbase + i * 8;
-      rb[i] = (col_ok && kk < kn) ? *reinterpret_cast<const U4 *>(bp + (int64_t)kk * a.brs) : U4{0, 0, 0, 0};
+      r[i] = (col_ok && kk < kn) ? *reinterpret_cast<const U4 *>(bp + (int64_t)kk * a.brs) : U4{0, 0, 0, 0};
     }
   };
-  auto store = [&](int buf) {
+  auto store = [&](const U4 (&r)[4], int buf) {
 #pragma unroll
     for (int i = 0; i < 4; i++)
-      *reinterpret_cast<U4 *>(sB + buf * SM_TILE + (rbase + i * 8) * SM_PITCH + c8) = rb[i];
+      *reinterpret_cast<U4 *>(sB + buf * SM_TILE + (rbase + i * 8) * SM_PITCH + c8) = r[i];
   };
   f32x4 acc[4];
 #pragma unroll
   for (int t = 0; t < 4; t++) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   const int nsteps = (kn + SM_KS - 1) / SM_KS;
-  load(0);
-  store(0);
-  if (nsteps > 1) load(1);
   const int g = lane >> 4, L = lane & 15;
-  for (int s = 0; s < nsteps; s++) {
-    if (s + 1 < nsteps) store((s + 1) & 1);
-    if (s + 2 < nsteps) load(s + 2);
+  // step s: its tile is in LDS buffer s & 1; the registers of slot (s + 1) % 3
+  // hold step s + 1 and are refilled with step s + 4 once stored
+  auto step = [&](int s, auto slot_c) {
+    constexpr int SL = decltype(slot_c)::value;
+    if (s + 1 < nsteps) store(rb[SL], (s + 1) & 1);
+    if (s + 4 < nsteps) load(rb[SL], s + 4);
     const U4 xa = *reinterpret_cast<const U4 *>(sA + L * kpitch + s * SM_KS + g * 8);
     const uint16_t *tile = sB + (s & 1) * SM_TILE + (g * 8 + (L >> 2)) * SM_PITCH + (L & 3) * 4;
 #pragma unroll
@@ -424,6 +426,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_mfma_kernel(SkinnyArgs a) {
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa), __builtin_bit_cast(f16x8, yb),
                                                         acc[t], 0, 0, 0);
     }
+  };
+  load(rb[0], 0);
+  if (nsteps > 1) load(rb[1], 1);
+  if (nsteps > 2) load(rb[2], 2);
+  store(rb[0], 0);
+  if (nsteps > 3) load(rb[0], 3);
+  for (int s = 0; s < nsteps; s += 3) {
+    step(s, std::integral_constant<int, 1>{});
+    if (s + 1 < nsteps) step(s + 1, std::integral_constant<int, 2>{});
+    if (s + 2 < nsteps) step(s + 2, std::integral_constant<int, 0>{});
   }
   // accumulator element e of lane l is C[4 * (l / 16) + e][l % 16] of its tile
 #pragma unroll
