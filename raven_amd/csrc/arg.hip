@@ -308,7 +308,8 @@ static int arg_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, co
   // row form: a group of lanes per output walks the axis at its own stride
   if (!dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout))
     return nxh_fail(NXH_FAILURE, op, "view has too many non-mergeable dimensions for one launch");
-  const bool wave_rows = g.R < 1024;
+  // a wave per row while rows are short, or of medium length but plentiful
+  const bool wave_rows = g.R < 1024 || (g.R <= 4096 && g.n_out >= (int64_t)cus * 16);
   const int64_t blocks = wave_rows ? (g.n_out + 3) / 4 : g.n_out;
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many outputs for one launch");
   int nsplit = wave_rows ? 1 : pick_split(blocks, g.R, 8192, cus);

@@ -269,7 +269,8 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
       a.in = ibase;
       a.n_out = (uint64_t)g.n_out;
       a.R = g.R;
-      const bool wave_rows = g.R < 1024;
+      // a wave per row while rows are short, or of medium length but plentiful
+      const bool wave_rows = g.R < 1024 || (g.R <= 4096 && g.n_out >= (int64_t)cus * 16);
       const int64_t blocks = wave_rows ? (g.n_out + 3) / 4 : g.n_out;
       int nsplit = wave_rows ? 1 : pick_split(blocks, g.R, 8192, cus);
       int64_t chunk = g.R;

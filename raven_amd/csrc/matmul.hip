@@ -26,8 +26,9 @@
 // exact (modular arithmetic is order-free).
 
 #include <algorithm>
+#include <cstdlib>
 
-#include "gemm_big.hpp"
+#include "gemm_tile.hpp"
 #include "nxh_common.hpp"
 
 constexpr int MM_MAXB = 8;  // batch dims decoded on the device
@@ -362,8 +363,8 @@ __global__ __launch_bounds__(SK_LANES *SK_RG) void gemm_skinny_kernel(SkinnyArgs
 constexpr int SM_KS = 32, SM_WN = 64, SM_PITCH = SM_WN + 8, SM_TILE = SM_KS * SM_PITCH;
 template <bool BF16>
 __global__ __launch_bounds__(256) void gemm_skinny_mfma_kernel(SkinnyArgs a) {
-  using gemm_big::lds_s16x4;
-  using gemm_big::s16x4;
+  using gemm_tile::lds_s16x4;
+  using gemm_tile::s16x4;
   typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
   extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -642,28 +643,48 @@ static int launch_skinny_mfma(nxh_context *ctx, GemmArgs &g) {
 
 static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-// The 256x256x64 kernel: whole tiles only, 16-byte aligned rows, unit-stride C.
-// Returns -1 when the call does not qualify.
-template <bool BF16, bool A_KC, bool B_KC>
-static int launch_big(nxh_context *ctx, const gemm_big::Args &g) {
-  auto kern = gemm_big::kernel<BF16, A_KC, B_KC, 4, 2>;
+// The LDS-tiled family of gemm_tile.hpp: K a multiple of 64, 16-byte aligned
+// rows, unit-stride C. Returns -1 when the call does not qualify.
+template <bool BF16, bool A_KC, bool B_KC, class SH, bool EDGE>
+static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
+  auto kern = gemm_tile::kernel<BF16, A_KC, B_KC, SH, EDGE>;
   static bool configured = false;  // guarded by the context mutex of the caller
   if (!configured) {
     NXH_HIP("matmul", hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)gemm_big::LDS_BYTES));
+                                          (int)SH::LDS_BYTES));
     configured = true;
   }
-  nxh_set_path("gemm_big");
-  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(512), gemm_big::LDS_BYTES, ctx->stream, g);
+  g.tiles_m = (uint32_t)((g.M + SH::BM - 1) / SH::BM);
+  g.tiles_n = (uint32_t)((g.N + SH::BN - 1) / SH::BN);
+  nxh_set_path(path);
+  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(SH::THREADS), SH::LDS_BYTES, ctx->stream, g);
   NXH_HIP("matmul", hipGetLastError());
   return NXH_OK;
 }
+template <bool BF16, class SH>
+static int launch_tile_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc, const char *path) {
+  const bool edge = g.M % SH::BM != 0 || g.N % SH::BN != 0;
+#define NXH_TILE(AK, BK_)                                                        \
+  (edge ? launch_tile<BF16, AK, BK_, SH, true>(ctx, g, path) : launch_tile<BF16, AK, BK_, SH, false>(ctx, g, path))
+  if (a_kc) return b_kc ? NXH_TILE(true, true) : NXH_TILE(true, false);
+  return b_kc ? NXH_TILE(false, true) : NXH_TILE(false, false);
+#undef NXH_TILE
+}
+// 0: pick by shape; 256 / 128 / 64: force that block shape (tuning aid, read once
+// from NXH_GEMM_TILE)
+static int forced_tile() {
+  static const int v = [] {
+    const char *e = getenv("NXH_GEMM_TILE");
+    return e ? atoi(e) : 0;
+  }();
+  return v;
+}
 template <bool BF16>
-static int try_big(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b) {
-  if (a.M % gemm_big::BM || a.N % gemm_big::BN || a.K % gemm_big::BK || a.K < gemm_big::BK) return -1;
+static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b) {
+  if (a.K % gemm_tile::BK || a.K < gemm_tile::BK || a.M < 8 || a.N < 8) return -1;
   if (a.ccs != 1 || a.batch.n > 4 || !al_a || !al_b) return -1;
   const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
-  gemm_big::Args g{};
+  gemm_tile::Args g{};
   g.A = (const uint16_t *)a.A;
   g.B = (const uint16_t *)a.B;
   g.C = (uint16_t *)a.C;
@@ -671,11 +692,12 @@ static int try_big(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al
   g.ldb = b_kc ? a.bcs : a.brs;
   g.ldc = a.crs;
   if (!al16(g.A) || !al16(g.B) || g.lda % 8 || g.ldb % 8) return -1;
+  // an operand contiguous along M / N is read in whole 8-element vectors
+  if ((!a_kc && a.M % 8) || (!b_kc && a.N % 8)) return -1;
+  g.M = a.M;
+  g.N = a.N;
   g.K = a.K;
-  g.tiles_m = (uint32_t)(a.M / gemm_big::BM);
-  g.tiles_n = (uint32_t)(a.N / gemm_big::BN);
   g.nbatch = nbatch;
-  if ((uint64_t)g.tiles_m * g.tiles_n * nbatch > 0x7fffffffULL) return -1;
   g.nbd = a.batch.n;
   for (int i = 0; i < a.batch.n; i++) {
     g.bshape[i] = a.batch.shape[i];
@@ -683,8 +705,24 @@ static int try_big(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al
     g.bb[i] = a.batch.b[i];
     g.bc[i] = a.batch.c[i];
   }
-  if (a_kc) return b_kc ? launch_big<BF16, true, true>(ctx, g) : launch_big<BF16, true, false>(ctx, g);
-  return b_kc ? launch_big<BF16, false, true>(ctx, g) : launch_big<BF16, false, false>(ctx, g);
+  auto tiles = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * (int64_t)nbatch; };
+  if (tiles(128, 64) > 0x7fffffffLL) return -1;
+  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  // Block shape: rounds of resident blocks x relative cost of one block. One
+  // 256x256 block (8 waves, 144 KiB of LDS) fills a CU; two 128x128 blocks fit,
+  // each a quarter of the work at about 0.8 of the big tile's efficiency.
+  int pick = forced_tile();
+  if (!pick) {
+    if (a.N <= 64) pick = 64;
+    else {
+      const double c256 = (double)((tiles(256, 256) + cus - 1) / cus);
+      const double c128 = (double)((tiles(128, 128) + 2 * cus - 1) / (2 * cus)) * 0.6;
+      pick = c256 <= c128 ? 256 : 128;
+    }
+  }
+  if (pick == 64) return launch_tile_oriented<BF16, gemm_tile::Shape256x64>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
+  if (pick == 128) return launch_tile_oriented<BF16, gemm_tile::Shape128x128>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
+  return launch_tile_oriented<BF16, gemm_tile::Shape256x256>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
 }
 
 template <class MM>
@@ -704,7 +742,7 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
   const bool a_ok = a.acs == 1 || a.ars == 1, b_ok = a.brs == 1 || a.bcs == 1;
   if (!a_ok || !b_ok) return launch_any<MM::DT>(ctx, a, nbatch);
   if constexpr (sizeof(S) == 2) {
-    int rc = try_big<MM::DT == NXH_BF16>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
+    int rc = try_tile<MM::DT == NXH_BF16>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
     if (rc != -1) return rc;
   }
   // 16-byte loads need an aligned base and every other stride a multiple of VL

@@ -127,7 +127,7 @@ def test_config4_bf16_batched(hip, oracle):
         hip.assign(hip.shrink(Afull, [(i, i + 1), (0, n), (0, n)]), hip.shrink(A, [(j, j + 1), (0, n), (0, n)]))
         hip.assign(hip.shrink(Bfull, [(i, i + 1), (0, n), (0, n)]), hip.shrink(Bm, [(1 - j, 2 - j), (0, n), (0, n)]))
     Cf = hip.matmul(Afull, Bfull)
-    assert hip.last_path() == "gemm_big" and Cf.shape == (nb, n, n)
+    assert hip.last_path() == "gemm_tile_256x256" and Cf.shape == (nb, n, n)
     aq, bq = decode(logical(A), dt.bfloat16, oracle), decode(logical(Bm), dt.bfloat16, oracle)
     rows, cols = rng.integers(0, n, 48), rng.integers(0, n, 48)
     for i in (0, 1, 7, 15):

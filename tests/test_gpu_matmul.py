@@ -178,24 +178,43 @@ def test_matmul_skinny_decode_shape(hip, oracle):
 
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
 def test_matmul_big_tile_kernel(hip, oracle, d):
-    """Whole-256-tile shapes take the large-tile kernel in all four operand
-    orientations, batched and batch-broadcast."""
+    """The LDS-tiled kernel family: every block shape, whole and ragged tiles,
+    all four operand orientations, batched and batch-broadcast."""
     rng = np.random.default_rng(1400 + d.tag)
-    for (m, k, n) in [(256, 64, 256), (512, 192, 768), (768, 320, 256)]:
+    cases = [
+        # whole tiles
+        (256, 64, 256, "gemm_tile_128x128"), (512, 192, 768, "gemm_tile_128x128"),
+        (768, 320, 256, "gemm_tile_128x128"), (512, 128, 64, "gemm_tile_256x64"),
+        (4096, 64, 4096, "gemm_tile_256x256"),
+        # ragged in M and N (multiples of 8, so M/N-contiguous operands qualify too)
+        (200, 64, 136, "gemm_tile_128x128"), (264, 128, 40, "gemm_tile_256x64"),
+        (4000, 64, 4088, "gemm_tile_256x256"),
+    ]
+    for (m, k, n, path) in cases:
         a = encode(rng.standard_normal((m, k)), d, oracle)
         b = encode(rng.standard_normal((k, n)), d, oracle)
         for ta in (False, True):
             for tb in (False, True):
+                if m * n > 4_000_000 and (ta, tb) not in ((False, False), (True, True)):
+                    continue  # keep the float64 reference products of the large cases to two
                 ha, _ = pair(np.ascontiguousarray(a.T) if ta else a, d, hip, oracle,
                              (lambda B, t: B.permute(t, (1, 0))) if ta else None)
                 hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle,
                              (lambda B, t: B.permute(t, (1, 0))) if tb else None)
-                check(hip, oracle, d, ha, hb, a, b, f"big {m}x{k}x{n} ta={ta} tb={tb}")
-                assert hip.last_path() == "gemm_big"
+                check(hip, oracle, d, ha, hb, a, b, f"tile {m}x{k}x{n} ta={ta} tb={tb}")
+                assert hip.last_path() == path, (m, k, n, ta, tb, hip.last_path())
+    # odd M and N: only K-contiguous operands (A row-major, B given as its transpose) qualify
+    a = encode(rng.standard_normal((203, 128)), d, oracle)
+    b = encode(rng.standard_normal((128, 157)), d, oracle)
+    hb, _ = pair(np.ascontiguousarray(b.T), d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], hb, a, b, "tile odd edges")
+    assert hip.last_path() == "gemm_tile_128x128"
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "odd N, row-major B")
+    assert hip.last_path() == "gemm_mfma"
     a = encode(rng.standard_normal((3, 2, 256, 128)), d, oracle)
     b = encode(rng.standard_normal((128, 512)), d, oracle)
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "big batched x broadcast W")
-    assert hip.last_path() == "gemm_big"
+    assert hip.last_path().startswith("gemm_tile")
     b4 = encode(rng.standard_normal((3, 1, 128, 256)), d, oracle)
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b4, d, hip, oracle)[0], a, b4, "big batch broadcast")
     # a sliced (offset, larger row stride) operand still qualifies when rows stay 16-byte aligned
