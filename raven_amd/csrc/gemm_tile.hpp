@@ -18,7 +18,7 @@
 // memory instructions never queue up in front of the matrix pipe.
 // An operand that is contiguous along K sits in LDS as [row][k] (+16 B pad) and
 // is fetched with ds_read_b128. An operand that is contiguous along M / N (a
-// row-major B) stays in its memory order, [k][row] (+32 B pad), and the
+// row-major B) stays in its memory order, [k][row] (+32 or 64 B pad), and the
 // k-contiguous fragments MFMA wants are produced by the transposing LDS read
 // ds_read_b64_tr_b16: within each group of 16 lanes, result element j of lane L
 // is element (L & 3) of the 8 bytes addressed by lane 4*j + (L >> 2). No 2-byte
@@ -39,7 +39,9 @@ namespace gemm_tile {
 
 constexpr int BK = 64;
 constexpr int PK = BK + 8;  // pitch (elements) of a [row][k] tile
-constexpr int PADR = 16;    // pad (elements) of a [k][row] tile's pitch
+// pad (elements) of a [k][row] tile's pitch: 64 B for 256-row tiles, 32 B for
+// the smaller ones (two 128x128 blocks then fit one CU's LDS)
+constexpr int padr(int rows) { return rows >= 256 ? 32 : 16; }
 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -52,8 +54,8 @@ template <int WM_, int WN_, int TM_, int TN_>
 struct Shape {
   static constexpr int WM = WM_, WN = WN_, TM = TM_, TN = TN_;
   static constexpr int BM = WM * TM * 32, BN = WN * TN * 32, THREADS = 64 * WM * WN;
-  // LDS elements of one operand tile: [rows][PK] or [BK][rows + PADR]
-  static constexpr int tile_elems(int rows) { return rows * PK > BK * (rows + PADR) ? rows * PK : BK * (rows + PADR); }
+  // LDS elements of one operand tile: [rows][PK] or [BK][rows + pad]
+  static constexpr int tile_elems(int rows) { return rows * PK > BK * (rows + padr(rows)) ? rows * PK : BK * (rows + padr(rows)); }
   static constexpr int A_ELEMS = tile_elems(BM), B_ELEMS = tile_elems(BN);
   static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
   static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * sizeof(uint16_t);
@@ -107,7 +109,7 @@ template <bool KC, int ROWS, int THREADS>
 __device__ __forceinline__ void slab_store1(int i, const V16 &r, uint16_t *lds) {
   const int v = threadIdx.x + i * THREADS;
   constexpr int VPR = ROWS / 8;
-  uint16_t *q = KC ? lds + (v >> 3) * PK + (v & 7) * 8 : lds + (v / VPR) * (ROWS + PADR) + (v % VPR) * 8;
+  uint16_t *q = KC ? lds + (v >> 3) * PK + (v & 7) * 8 : lds + (v / VPR) * (ROWS + padr(ROWS)) + (v % VPR) * 8;
   *reinterpret_cast<V16 *>(q) = r;
 }
 
@@ -119,7 +121,7 @@ __device__ __forceinline__ V16 frag_load(const uint16_t *lds, int row0, int ks, 
     return *reinterpret_cast<const V16 *>(lds + (row0 + (lane & 31)) * PK + ks * 16 + (lane >> 5) * 8);
   } else {
     // source address of this lane for the transposing read (see the header)
-    constexpr int PR = ROWS + PADR;
+    constexpr int PR = ROWS + padr(ROWS);
     const int k = ks * 16 + (lane >> 5) * 8 + ((lane & 15) >> 2);
     const int r = row0 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const uint16_t *q = lds + k * PR + r;

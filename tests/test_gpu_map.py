@@ -255,11 +255,17 @@ def test_cast_int4(hip, oracle):
             x = rng.integers(max(info.min, -40), min(info.max, 40), n, endpoint=True).astype(src.np_storage)
         h, o = pair(x, src, hip, oracle)
         hp, op_ = hip.cast(h, p), oracle.cast(o, p)
-        same_bits(hip.to_host(hp)[:(n + 1) // 2], op_.storage[:(n + 1) // 2])
+
+        def nibbles(storage):  # n is odd: the last byte's high nibble is padding, not data
+            b = np.array(storage[:(n + 1) // 2], dtype=np.uint8)
+            b[-1] &= 0x0F
+            return b
+
+        same_bits(nibbles(hip.to_host(hp)), nibbles(op_.storage))
         for back in (dt.int8, dt.int32, dt.float32, dt.int64):
             same_bits(logical(hip.cast(hp, back)), logical(oracle.cast(op_, back)))
         # packed -> packed and whole-buffer copy keep the nibbles
-        same_bits(hip.to_host(hip.copy(hp))[:(n + 1) // 2], op_.storage[:(n + 1) // 2])
+        same_bits(nibbles(hip.to_host(hip.copy(hp))), nibbles(op_.storage))
     with pytest.raises(RuntimeError):  # compute ops reject packed dtypes
         hip.unary("neg", hp)
 
