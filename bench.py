@@ -45,6 +45,13 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}
 METRIC = "Nx op GB/s (elementwise/reduce) + GEMM TFLOP/s, as % of MI355X roofline"
 
 
+# HBM bytes per launch of the headline step's dominant kernel (map_tiled add, f32,
+# [64,512,512]), from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of
+# `bench.py --only-step --no-cpu --pmc-calibration`: 32 817 KiB fetched x 1.9990 (a plain
+# 64 MiB copy reads 32 784 KiB on the same counter) + 65 536 KiB written x 1.0000.
+DOMINANT_KERNEL_HBM_TRAFFIC = 134285312
+
+
 class Op:
     """One pre-built C-ABI call: name, thunk, algorithmic bytes / flops."""
 
@@ -332,6 +339,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--only-step", action="store_true", help="time the headline step only")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also launch 20 plain 64 MiB copies (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    ap.add_argument("--only-config", type=int, choices=(1, 2, 3, 4), default=0,
+                    help="time the operations of one configuration only and print their records")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 forward leg only and print its record")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -342,6 +353,13 @@ def main():
     info = hip.device_info()
     if args.only_gpt2:
         print(json.dumps(config5(hip)))
+        return
+    if args.only_config:
+        # one configuration's operations, each timed alone (for profiling runs)
+        W = Workloads(hip)
+        group = {1: W.config1, 2: W.config2, 3: W.config3, 4: W.config4}[args.only_config]
+        recs = [op_record(op, time_ops(hip, [op], 10 if "16,4096" in op.name else 50, 3)) for op in group()]
+        print(json.dumps({"config": args.only_config, "ops": recs}))
         return
     W = Workloads(hip)
     step_ops = W.config2()
@@ -380,10 +398,18 @@ def main():
         "kernel": f"{dom_path}_kernel<BinaryF<OpAdd, f32>, 64> ({dom.name})",
         "bound": "hbm", "achieved": round(dom.nbytes / (dom_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
         "unit": "GB/s", "frac": round(dom.nbytes / (dom_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-        "bytes_per_launch": dom.nbytes, "avg_launch_ms": round(dom_ms, 5), "traffic": None,
+        "bytes_per_launch": dom.nbytes, "avg_launch_ms": round(dom_ms, 5), "traffic": DOMINANT_KERNEL_HBM_TRAFFIC,
     }
 
     ops_out = []
+    if args.pmc_calibration:
+        # a plain contiguous copy of known size (64 MiB read, 64 MiB written) in the same process:
+        # hardware-counter readings of the step's kernels are scaled by what the counters show here
+        src, dst = hip.full(dt.float32, (64, 512, 512), 1.0), hip.buffer(dt.float32, (64, 512, 512))
+        cal = W.mk("calibration copy 64 MiB", W.lib.nxh_copy, [dst, src], nbytes=2 * 64 * 512 * 512 * 4)
+        for _ in range(20):
+            cal()
+        hip.synchronize()
     if not args.only_step:
         for op in step_ops:
             ops_out.append(op_record(op, time_ops(hip, [op], 100, 5)))

@@ -363,7 +363,11 @@ __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) 
   __shared__ I0 l0[TILE * (TILE + 1)];
   __shared__ I1 l1[F::NIN > 1 ? TILE * (TILE + 1) : 1];
   __shared__ I2 l2[F::NIN > 2 ? TILE * (TILE + 1) : 1];
+  // Blocks with equal id modulo 8 share an XCD (and its L2): hand each XCD a
+  // contiguous run of tiles, so neighbouring tiles that split a cache line of a
+  // narrow operand fetch it once.
   uint32_t b = blockIdx.x;
+  if ((gridDim.x & 7u) == 0) b = (b & 7u) * (gridDim.x >> 3) + (b >> 3);
   const uint32_t tx = b % a.tiles_x;
   b /= a.tiles_x;
   const uint32_t ty = b % a.tiles_y;
