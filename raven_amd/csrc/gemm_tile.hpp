@@ -1,6 +1,8 @@
-// gemm_tile.hpp — the LDS-tiled MFMA GEMM family for 16-bit inputs (bf16 / f16)
-// with f32 accumulation, behind batched [.., M, K] x [.., K, N] whenever K is a
-// multiple of 64 and the operands are 16-byte aligned.
+// gemm_tile.hpp — the LDS-tiled MFMA GEMM family: bf16 / f16 inputs
+// (v_mfma_f32_32x32x16) and f32 inputs (v_mfma_f32_32x32x2, true f32), f32
+// accumulation, behind batched [.., M, K] x [.., K, N] whenever K is a multiple
+// of one slab (128 bytes of k: 64 / 32 elements) and the operands are 16-byte
+// aligned.
 //
 // One kernel template, three block shapes (BM x BN outputs per block, each of
 // the WM x WN wave64s owning TM x TN tiles of v_mfma_f32_32x32x16):
@@ -22,7 +24,8 @@
 // k-contiguous fragments MFMA wants are produced by the transposing LDS read
 // ds_read_b64_tr_b16: within each group of 16 lanes, result element j of lane L
 // is element (L & 3) of the 8 bytes addressed by lane 4*j + (L >> 2). No 2-byte
-// scatter into LDS, no transposed copy in HBM.
+// scatter into LDS, no transposed copy in HBM. For f32 the [k][row] order is
+// already what the 32x32x2 MFMA wants (one float per lane): four ds_read_b32.
 // Ragged M / N (EDGE): loads of rows past the edge are redirected to the last
 // valid row (or, along a contiguous M / N, to the last whole 8-element vector),
 // which only feeds outputs that are never stored; stores are bounds-checked.
@@ -37,38 +40,69 @@
 
 namespace gemm_tile {
 
-constexpr int BK = 64;
-constexpr int PK = BK + 8;  // pitch (elements) of a [row][k] tile
-// pad (elements) of a [k][row] tile's pitch: 64 B for 256-row tiles, 32 B for
-// the smaller ones (two 128x128 blocks then fit one CU's LDS)
-constexpr int padr(int rows) { return rows >= 256 ? 32 : 16; }
+// Element traits. VE = elements per 16-byte vector; a K-slab is 8 vectors (128
+// bytes of k) per row, a k-step is 2 vectors: lanes 0-31 multiply the first VE
+// k-values of a step, lanes 32-63 the second (any fixed assignment of k to
+// lanes is valid as long as A and B agree).
+struct ElBF16 {
+  using S = uint16_t;
+  static constexpr int VE = 8;
+  static constexpr bool F32 = false, BF16 = true;
+};
+struct ElF16 {
+  using S = uint16_t;
+  static constexpr int VE = 8;
+  static constexpr bool F32 = false, BF16 = false;
+};
+struct ElF32 {
+  using S = float;
+  static constexpr int VE = 4;
+  static constexpr bool F32 = true, BF16 = false;
+};
+constexpr int KSTEPS = 4;
 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t V16;  // one 16-byte register quad
 
+// Tile geometry in elements of EL. PK: pitch of a [row][k] tile (+16 B). The
+// [k][row] pitch adds 64 B for 256-row 16-bit tiles, 32 B otherwise (two 128x128
+// blocks then fit one CU's LDS; for f32 it puts the two k-rows a wave reads at
+// once 32 banks apart).
+template <class EL>
+struct Geo {
+  static constexpr int VE = EL::VE, BK = 8 * VE, PK = BK + VE;
+  static constexpr int padr(int rows) { return (!EL::F32 && rows >= 256) ? 4 * VE : 2 * VE; }
+  static constexpr int tile_elems(int rows) {
+    return rows * PK > BK * (rows + padr(rows)) ? rows * PK : BK * (rows + padr(rows));
+  }
+};
+
 template <int WM_, int WN_, int TM_, int TN_>
 struct Shape {
   static constexpr int WM = WM_, WN = WN_, TM = TM_, TN = TN_;
   static constexpr int BM = WM * TM * 32, BN = WN * TN * 32, THREADS = 64 * WM * WN;
-  // LDS elements of one operand tile: [rows][PK] or [BK][rows + pad]
-  static constexpr int tile_elems(int rows) { return rows * PK > BK * (rows + padr(rows)) ? rows * PK : BK * (rows + padr(rows)); }
-  static constexpr int A_ELEMS = tile_elems(BM), B_ELEMS = tile_elems(BN);
-  static constexpr int STAGE_ELEMS = A_ELEMS + B_ELEMS;
-  static constexpr size_t LDS_BYTES = 2 * (size_t)STAGE_ELEMS * sizeof(uint16_t);
-  static constexpr int NVA = BM * BK / 8 / THREADS, NVB = BN * BK / 8 / THREADS;  // staged vectors per lane
-  static_assert(NVA >= 1 && NVB >= 1 && NVA * THREADS * 8 == BM * BK && NVB * THREADS * 8 == BN * BK, "staging");
+  // staged 16-byte vectors per lane and slab: rows x 8 vectors / THREADS
+  static constexpr int NVA = BM * 8 / THREADS, NVB = BN * 8 / THREADS;
+  static_assert(NVA >= 1 && NVB >= 1 && NVA * THREADS == BM * 8 && NVB * THREADS == BN * 8, "staging");
+  template <class EL>
+  static constexpr int a_elems() { return Geo<EL>::tile_elems(BM); }
+  template <class EL>
+  static constexpr int stage_elems() { return Geo<EL>::tile_elems(BM) + Geo<EL>::tile_elems(BN); }
+  template <class EL>
+  static constexpr size_t lds_bytes() { return 2 * (size_t)stage_elems<EL>() * sizeof(typename EL::S); }
 };
 using Shape256x256 = Shape<4, 2, 2, 4>;
 using Shape128x128 = Shape<2, 2, 2, 2>;
 using Shape256x64 = Shape<4, 1, 2, 2>;
 
 struct Args {
-  const uint16_t *A, *B;
-  uint16_t *C;
+  const void *A, *B;
+  void *C;
   int64_t lda, ldb, ldc;  // the non-unit stride of each matrix (elements)
   int64_t M, N, K;
   uint32_t tiles_m, tiles_n, nbatch;
@@ -78,50 +112,65 @@ struct Args {
   int64_t ba[4], bb[4], bc[4];
 };
 
-template <bool BF16>
-__device__ __forceinline__ void mfma16(f32x16 &acc, const V16 &a, const V16 &b) {
-  if constexpr (BF16)
+// One k-step of one 32x32 tile: a, b hold this lane's VE k-values of its row.
+template <class EL>
+__device__ __forceinline__ void mfma_step(f32x16 &acc, const V16 &a, const V16 &b) {
+  if constexpr (EL::F32) {
+    const f32x4 x = __builtin_bit_cast(f32x4, a), y = __builtin_bit_cast(f32x4, b);
+#pragma unroll
+    for (int s = 0; s < 4; s++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x[s], y[s], acc, 0, 0, 0);
+  } else if constexpr (EL::BF16) {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
-  else
+  } else {
     acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+  }
 }
 
 // Global -> registers -> LDS, one 16-byte vector at a time: vector i of this lane
-// of one operand's ROWS x 64 slab. KC: rows are 128 B apart in the slab (8
-// vectors per row); otherwise the slab is 64 k-rows of ROWS elements (ROWS / 8
+// of one operand's ROWS x BK slab. KC: rows are 128 B apart in the slab (8
+// vectors per row); otherwise the slab is BK k-rows of ROWS elements (ROWS / VE
 // vectors per k-row). `edge` is the number of valid rows from the slab's
 // origin (EDGE only).
-template <bool KC, int ROWS, int THREADS, bool EDGE>
-__device__ __forceinline__ V16 slab_load1(int i, const uint16_t *p, int64_t ld, int edge) {
+template <class EL, bool KC, int ROWS, int THREADS, bool EDGE>
+__device__ __forceinline__ V16 slab_load1(int i, const typename EL::S *p, int64_t ld, int edge) {
+  constexpr int VE = EL::VE;
   const int v = threadIdx.x + i * THREADS;
   if constexpr (KC) {
     int row = v >> 3;
     if constexpr (EDGE) row = row < edge ? row : edge - 1;
-    return *reinterpret_cast<const V16 *>(p + (int64_t)row * ld + (v & 7) * 8);
+    return *reinterpret_cast<const V16 *>(p + (int64_t)row * ld + (v & 7) * VE);
   } else {
-    constexpr int VPR = ROWS / 8;
-    int c = (v % VPR) * 8;
-    if constexpr (EDGE) c = c + 8 <= edge ? c : edge - 8;
+    constexpr int VPR = ROWS / VE;
+    int c = (v % VPR) * VE;
+    if constexpr (EDGE) c = c + VE <= edge ? c : edge - VE;
     return *reinterpret_cast<const V16 *>(p + (int64_t)(v / VPR) * ld + c);
   }
 }
-template <bool KC, int ROWS, int THREADS>
-__device__ __forceinline__ void slab_store1(int i, const V16 &r, uint16_t *lds) {
+template <class EL, bool KC, int ROWS, int THREADS>
+__device__ __forceinline__ void slab_store1(int i, const V16 &r, typename EL::S *lds) {
+  using G = Geo<EL>;
+  constexpr int VE = EL::VE, VPR = ROWS / VE;
   const int v = threadIdx.x + i * THREADS;
-  constexpr int VPR = ROWS / 8;
-  uint16_t *q = KC ? lds + (v >> 3) * PK + (v & 7) * 8 : lds + (v / VPR) * (ROWS + padr(ROWS)) + (v % VPR) * 8;
+  typename EL::S *q = KC ? lds + (v >> 3) * G::PK + (v & 7) * VE : lds + (v / VPR) * (ROWS + G::padr(ROWS)) + (v % VPR) * VE;
   *reinterpret_cast<V16 *>(q) = r;
 }
 
-// One MFMA operand fragment (8 k-values for this lane's row) for k-step `ks`
-// (16 k-values per step) and the 32-row group starting at `row0`.
-template <bool KC, int ROWS>
-__device__ __forceinline__ V16 frag_load(const uint16_t *lds, int row0, int ks, int lane) {
+// One MFMA operand fragment (VE k-values for this lane's row) for k-step `ks`
+// (2 * VE k-values per step) and the 32-row group starting at `row0`.
+template <class EL, bool KC, int ROWS>
+__device__ __forceinline__ V16 frag_load(const typename EL::S *lds, int row0, int ks, int lane) {
+  using G = Geo<EL>;
+  constexpr int VE = EL::VE;
   if constexpr (KC) {
-    return *reinterpret_cast<const V16 *>(lds + (row0 + (lane & 31)) * PK + ks * 16 + (lane >> 5) * 8);
+    return *reinterpret_cast<const V16 *>(lds + (row0 + (lane & 31)) * G::PK + ks * 2 * VE + (lane >> 5) * VE);
+  } else if constexpr (EL::F32) {
+    constexpr int PR = ROWS + G::padr(ROWS);
+    const float *q = lds + (ks * 2 * VE + (lane >> 5) * VE) * PR + row0 + (lane & 31);
+    const f32x4 x = {q[0], q[PR], q[2 * PR], q[3 * PR]};
+    return __builtin_bit_cast(V16, x);
   } else {
     // source address of this lane for the transposing read (see the header)
-    constexpr int PR = ROWS + padr(ROWS);
+    constexpr int PR = ROWS + G::padr(ROWS);
     const int k = ks * 16 + (lane >> 5) * 8 + ((lane & 15) >> 2);
     const int r = row0 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
     const uint16_t *q = lds + k * PR + r;
@@ -156,11 +205,14 @@ __device__ __forceinline__ void tile_of_block(const Args &a, uint32_t bid, uint3
   tn = in_strip / gsz;
 }
 
-template <bool BF16, bool A_KC, bool B_KC, class SH, bool EDGE>
+template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE>
 __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   constexpr int THREADS = SH::THREADS, BM = SH::BM, BN = SH::BN, TM = SH::TM, TN = SH::TN;
-  constexpr int NVA = SH::NVA, NVB = SH::NVB, KSTEPS = BK / 16;
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  constexpr int NVA = SH::NVA, NVB = SH::NVB, BK = Geo<EL>::BK;
+  constexpr int A_ELEMS = SH::template a_elems<EL>(), STAGE_ELEMS = SH::template stage_elems<EL>();
+  using S = typename EL::S;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  S *smem = reinterpret_cast<S *>(smem_raw);
   uint32_t batch, tm, tn;
   tile_of_block(a, blockIdx.x, batch, tm, tn);
   int64_t ao = 0, bo = 0, co = 0;
@@ -181,8 +233,8 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   const int edge_m = EDGE ? (int)(a.M - m0 < BM ? a.M - m0 : BM) : BM;
   const int edge_n = EDGE ? (int)(a.N - n0 < BN ? a.N - n0 : BN) : BN;
   // slab origin and per-slab advance of each operand
-  const uint16_t *gA = a.A + ao + (A_KC ? m0 * a.lda : m0);
-  const uint16_t *gB = a.B + bo + (B_KC ? n0 * a.ldb : n0);
+  const S *gA = (const S *)a.A + ao + (A_KC ? m0 * a.lda : m0);
+  const S *gB = (const S *)a.B + bo + (B_KC ? n0 * a.ldb : n0);
   const int64_t stepA = A_KC ? BK : (int64_t)BK * a.lda;
   const int64_t stepB = B_KC ? BK : (int64_t)BK * a.ldb;
 
@@ -201,26 +253,26 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   const int nk = (int)(a.K / BK);
   // Staged vector i of an operand moves at k-step i % KSTEPS; the prologue uses
   // the same issue order, so the loop's in-order wait counts hold from the start.
-  auto fetch_step = [&](int ks, const uint16_t *pA, const uint16_t *pB) {
+  auto fetch_step = [&](int ks, const S *pA, const S *pB) {
 #pragma unroll
     for (int i = 0; i < (NVA > NVB ? NVA : NVB); i++) {
       if (i % KSTEPS != ks) continue;
-      if (i < NVA) ra[i] = slab_load1<A_KC, BM, THREADS, EDGE>(i, pA, a.lda, edge_m);
-      if (i < NVB) rb[i] = slab_load1<B_KC, BN, THREADS, EDGE>(i, pB, a.ldb, edge_n);
+      if (i < NVA) ra[i] = slab_load1<EL, A_KC, BM, THREADS, EDGE>(i, pA, a.lda, edge_m);
+      if (i < NVB) rb[i] = slab_load1<EL, B_KC, BN, THREADS, EDGE>(i, pB, a.ldb, edge_n);
     }
   };
-  auto stage_step = [&](int ks, uint16_t *nA, uint16_t *nB) {
+  auto stage_step = [&](int ks, S *nA, S *nB) {
 #pragma unroll
     for (int i = 0; i < (NVA > NVB ? NVA : NVB); i++) {
       if (i % KSTEPS != ks) continue;
-      if (i < NVA) slab_store1<A_KC, BM, THREADS>(i, ra[i], nA);
-      if (i < NVB) slab_store1<B_KC, BN, THREADS>(i, rb[i], nB);
+      if (i < NVA) slab_store1<EL, A_KC, BM, THREADS>(i, ra[i], nA);
+      if (i < NVB) slab_store1<EL, B_KC, BN, THREADS>(i, rb[i], nB);
     }
   };
 #pragma unroll
   for (int ks = 0; ks < KSTEPS; ks++) fetch_step(ks, gA, gB);
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ks++) stage_step(ks, smem, smem + SH::A_ELEMS);
+  for (int ks = 0; ks < KSTEPS; ks++) stage_step(ks, smem, smem + A_ELEMS);
   if (nk > 1) {
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) fetch_step(ks, gA + stepA, gB + stepB);
@@ -232,24 +284,24 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   // The steady state (both true) is free of branches.
   auto slab = [&](int kt, auto stage_c, auto fetch_c) {
     constexpr bool STAGE = decltype(stage_c)::value, FETCH = decltype(fetch_c)::value;
-    const uint16_t *sA = smem + (kt & 1) * SH::STAGE_ELEMS;
-    const uint16_t *sB = sA + SH::A_ELEMS;
-    uint16_t *nA = smem + ((kt + 1) & 1) * SH::STAGE_ELEMS;
-    uint16_t *nB = nA + SH::A_ELEMS;
-    const uint16_t *pA = gA + (int64_t)(kt + 2) * stepA, *pB = gB + (int64_t)(kt + 2) * stepB;
+    const S *sA = smem + (kt & 1) * STAGE_ELEMS;
+    const S *sB = sA + A_ELEMS;
+    S *nA = smem + ((kt + 1) & 1) * STAGE_ELEMS;
+    S *nB = nA + A_ELEMS;
+    const S *pA = gA + (int64_t)(kt + 2) * stepA, *pB = gB + (int64_t)(kt + 2) * stepB;
     V16 fa[2][TM], fb[2][TN];
 #pragma unroll
-    for (int t = 0; t < TM; t++) fa[0][t] = frag_load<A_KC, BM>(sA, wm + t * 32, 0, lane);
+    for (int t = 0; t < TM; t++) fa[0][t] = frag_load<EL, A_KC, BM>(sA, wm + t * 32, 0, lane);
 #pragma unroll
-    for (int u = 0; u < TN; u++) fb[0][u] = frag_load<B_KC, BN>(sB, wn + u * 32, 0, lane);
+    for (int u = 0; u < TN; u++) fb[0][u] = frag_load<EL, B_KC, BN>(sB, wn + u * 32, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
       const int cur = ks & 1, nxt = cur ^ 1;
       if (ks + 1 < KSTEPS) {
 #pragma unroll
-        for (int t = 0; t < TM; t++) fa[nxt][t] = frag_load<A_KC, BM>(sA, wm + t * 32, ks + 1, lane);
+        for (int t = 0; t < TM; t++) fa[nxt][t] = frag_load<EL, A_KC, BM>(sA, wm + t * 32, ks + 1, lane);
 #pragma unroll
-        for (int u = 0; u < TN; u++) fb[nxt][u] = frag_load<B_KC, BN>(sB, wn + u * 32, ks + 1, lane);
+        for (int u = 0; u < TN; u++) fb[nxt][u] = frag_load<EL, B_KC, BN>(sB, wn + u * 32, ks + 1, lane);
       }
       if constexpr (STAGE) stage_step(ks, nA, nB);
       if constexpr (FETCH) fetch_step(ks, pA, pB);
@@ -259,7 +311,7 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
 #pragma unroll
       for (int t = 0; t < TM; t++)
 #pragma unroll
-        for (int u = 0; u < TN; u++) mfma16<BF16>(acc[t][u], fa[cur][t], fb[cur][u]);
+        for (int u = 0; u < TN; u++) mfma_step<EL>(acc[t][u], fa[cur][t], fb[cur][u]);
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
@@ -272,7 +324,7 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   slab(kt, no{}, no{});
 
   // accumulator element e of lane l is C[(e/4)*8 + (l/32)*4 + e%4][l%32]
-  uint16_t *C = a.C + co;
+  S *C = (S *)a.C + co;
   const int r32 = lane & 31, kg = lane >> 5;
 #pragma unroll
   for (int t = 0; t < TM; t++)
@@ -284,7 +336,9 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
       for (int e = 0; e < 16; e++) {
         const int rl = wm + t * 32 + (e >> 2) * 8 + kg * 4 + (e & 3);
         if (EDGE && rl >= edge_m) continue;
-        C[(m0 + rl) * a.ldc + n0 + cl] = BF16 ? f32_to_bf16(acc[t][u][e]) : f32_to_f16(acc[t][u][e]);
+        S *c = C + (m0 + rl) * a.ldc + n0 + cl;
+        if constexpr (EL::F32) *c = acc[t][u][e];
+        else *c = EL::BF16 ? f32_to_bf16(acc[t][u][e]) : f32_to_f16(acc[t][u][e]);
       }
     }
 }

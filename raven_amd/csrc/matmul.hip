@@ -643,29 +643,29 @@ static int launch_skinny_mfma(nxh_context *ctx, GemmArgs &g) {
 
 static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-// The LDS-tiled family of gemm_tile.hpp: K a multiple of 64, 16-byte aligned
-// rows, unit-stride C. Returns -1 when the call does not qualify.
-template <bool BF16, bool A_KC, bool B_KC, class SH, bool EDGE>
+// The LDS-tiled family of gemm_tile.hpp: K a multiple of one slab (64 two-byte or
+// 32 four-byte elements), 16-byte aligned rows, unit-stride C. Returns -1 when the call does not qualify.
+template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE>
 static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
-  auto kern = gemm_tile::kernel<BF16, A_KC, B_KC, SH, EDGE>;
+  auto kern = gemm_tile::kernel<EL, A_KC, B_KC, SH, EDGE>;
+  constexpr size_t LDS = SH::template lds_bytes<EL>();
   static bool configured = false;  // guarded by the context mutex of the caller
   if (!configured) {
-    NXH_HIP("matmul", hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                          (int)SH::LDS_BYTES));
+    NXH_HIP("matmul", hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
     configured = true;
   }
   g.tiles_m = (uint32_t)((g.M + SH::BM - 1) / SH::BM);
   g.tiles_n = (uint32_t)((g.N + SH::BN - 1) / SH::BN);
   nxh_set_path(path);
-  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(SH::THREADS), SH::LDS_BYTES, ctx->stream, g);
+  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(SH::THREADS), LDS, ctx->stream, g);
   NXH_HIP("matmul", hipGetLastError());
   return NXH_OK;
 }
-template <bool BF16, class SH>
+template <class EL, class SH>
 static int launch_tile_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc, const char *path) {
   const bool edge = g.M % SH::BM != 0 || g.N % SH::BN != 0;
 #define NXH_TILE(AK, BK_)                                                        \
-  (edge ? launch_tile<BF16, AK, BK_, SH, true>(ctx, g, path) : launch_tile<BF16, AK, BK_, SH, false>(ctx, g, path))
+  (edge ? launch_tile<EL, AK, BK_, SH, true>(ctx, g, path) : launch_tile<EL, AK, BK_, SH, false>(ctx, g, path))
   if (a_kc) return b_kc ? NXH_TILE(true, true) : NXH_TILE(true, false);
   return b_kc ? NXH_TILE(false, true) : NXH_TILE(false, false);
 #undef NXH_TILE
@@ -679,21 +679,22 @@ static int forced_tile() {
   }();
   return v;
 }
-template <bool BF16>
+template <class EL>
 static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b) {
-  if (a.K % gemm_tile::BK || a.K < gemm_tile::BK || a.M < 8 || a.N < 8) return -1;
+  constexpr int VE = EL::VE, BK = gemm_tile::Geo<EL>::BK;
+  if (a.K % BK || a.K < BK || a.M < VE || a.N < VE) return -1;
   if (a.ccs != 1 || a.batch.n > 4 || !al_a || !al_b) return -1;
   const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
   gemm_tile::Args g{};
-  g.A = (const uint16_t *)a.A;
-  g.B = (const uint16_t *)a.B;
-  g.C = (uint16_t *)a.C;
+  g.A = a.A;
+  g.B = a.B;
+  g.C = a.C;
   g.lda = a_kc ? a.ars : a.acs;
   g.ldb = b_kc ? a.bcs : a.brs;
   g.ldc = a.crs;
-  if (!al16(g.A) || !al16(g.B) || g.lda % 8 || g.ldb % 8) return -1;
-  // an operand contiguous along M / N is read in whole 8-element vectors
-  if ((!a_kc && a.M % 8) || (!b_kc && a.N % 8)) return -1;
+  if (!al16(g.A) || !al16(g.B) || g.lda % VE || g.ldb % VE) return -1;
+  // an operand contiguous along M / N is read in whole 16-byte vectors
+  if ((!a_kc && a.M % VE) || (!b_kc && a.N % VE)) return -1;
   g.M = a.M;
   g.N = a.N;
   g.K = a.K;
@@ -720,9 +721,9 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       pick = c256 <= c128 ? 256 : 128;
     }
   }
-  if (pick == 64) return launch_tile_oriented<BF16, gemm_tile::Shape256x64>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
-  if (pick == 128) return launch_tile_oriented<BF16, gemm_tile::Shape128x128>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
-  return launch_tile_oriented<BF16, gemm_tile::Shape256x256>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
+  if (pick == 64) return launch_tile_oriented<EL, gemm_tile::Shape256x64>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
+  if (pick == 128) return launch_tile_oriented<EL, gemm_tile::Shape128x128>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
+  return launch_tile_oriented<EL, gemm_tile::Shape256x256>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
 }
 
 template <class MM>
@@ -741,8 +742,10 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
   }
   const bool a_ok = a.acs == 1 || a.ars == 1, b_ok = a.brs == 1 || a.bcs == 1;
   if (!a_ok || !b_ok) return launch_any<MM::DT>(ctx, a, nbatch);
-  if constexpr (sizeof(S) == 2) {
-    int rc = try_tile<MM::DT == NXH_BF16>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
+  {
+    using EL = std::conditional_t<MM::DT == NXH_F32, gemm_tile::ElF32,
+                                  std::conditional_t<MM::DT == NXH_BF16, gemm_tile::ElBF16, gemm_tile::ElF16>>;
+    int rc = try_tile<EL>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
     if (rc != -1) return rc;
   }
   // 16-byte loads need an aligned base and every other stride a multiple of VL

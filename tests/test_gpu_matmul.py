@@ -176,7 +176,7 @@ def test_matmul_skinny_decode_shape(hip, oracle):
     assert np.all(np.isinf(got[:, 5]) | np.isnan(got[:, 5])) and np.all(np.isfinite(np.delete(got, 5, axis=1)))
 
 
-@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16, dt.float32], ids=lambda d: d.name)
 def test_matmul_big_tile_kernel(hip, oracle, d):
     """The LDS-tiled kernel family: every block shape, whole and ragged tiles,
     all four operand orientations, batched and batch-broadcast."""
