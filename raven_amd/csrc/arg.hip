@@ -71,9 +71,11 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_row_kernel(ArgArgs a) {
   __shared__ int64_t li[4];
   constexpr int GROUPS = FOLD_THREADS / G;
   const int lane = threadIdx.x % G;
-  const uint64_t o = (uint64_t)blockIdx.x * GROUPS + threadIdx.x / G;
+  // blocks walk the input from its end: the tail of a tensor that was just
+  // written front to back is still in the memory-side cache
+  const uint64_t o = (uint64_t)(gridDim.x - 1 - blockIdx.x) * GROUPS + threadIdx.x / G;
   const bool live = o < a.n_out;
-  const int c = blockIdx.y;
+  const int c = gridDim.y - 1 - blockIdx.y;
   int64_t in_off = 0, out_off = 0;
   if (live) fold_decode(a.kept, o, in_off, out_off);
   const int64_t r0 = (int64_t)c * a.chunk;
@@ -144,9 +146,10 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
   constexpr int U = 4;
   __shared__ C lv[RG > 1 ? (RG - 1) * LANES * V : 1];
   __shared__ int32_t li[RG > 1 ? (RG - 1) * LANES * V : 1];
-  const uint32_t lb = blockIdx.x % a.lane_blocks;
-  const uint64_t ob = blockIdx.x / a.lane_blocks;
-  const int c = blockIdx.y;
+  const uint32_t bx = gridDim.x - 1 - blockIdx.x;  // from the end, as in arg_row_kernel
+  const uint32_t lb = bx % a.lane_blocks;
+  const uint64_t ob = bx / a.lane_blocks;
+  const int c = gridDim.y - 1 - blockIdx.y;
   const uint32_t ln = threadIdx.x % LANES, rg = threadIdx.x / LANES;
   const uint32_t l = (lb * LANES + ln) * V;
   const bool live = l < a.L;

@@ -95,45 +95,43 @@ __global__ __launch_bounds__(FOLD_THREADS) void fold_row_kernel(RowArgs a) {
   __shared__ C lds[4];
   constexpr int GROUPS = FOLD_THREADS / G;
   const int lane = threadIdx.x % G;
-  const int c = blockIdx.y;
-  // One output per group and pass. Wave-sized groups (no block barrier inside)
-  // walk the outputs with a grid stride, so a capped grid amortises the launch
-  // of a wave over several short rows.
-  for (uint64_t o = (uint64_t)blockIdx.x * GROUPS + threadIdx.x / G;; o += (uint64_t)gridDim.x * GROUPS) {
-    const bool live = o < a.n_out;
-    if (G == 64 && !live) break;
-    int64_t in_off = 0, out_off = 0;
-    if (live) fold_decode(a.kept, o, in_off, out_off);
-    const int64_t r0 = (int64_t)c * a.chunk;
-    const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
-    const T *p = (const T *)a.in + in_off;
-    C acc0 = CB::init(), acc1 = CB::init(), acc2 = CB::init(), acc3 = CB::init();
-    const int64_t nv = (r1 - r0) / V;
-    const FVec<T, V> *pv = reinterpret_cast<const FVec<T, V> *>(p + r0);
-    int64_t i = lane;
-    for (; i + 3 * G < nv; i += 4 * G) {
-      FVec<T, V> x0 = pv[i], x1 = pv[i + G], x2 = pv[i + 2 * G], x3 = pv[i + 3 * G];
+  // Blocks walk the input from its end: a tensor that the previous kernel has
+  // just written front to back still has its tail in the memory-side cache, and
+  // a reader that starts there finds it (measured on a 402 MB row max right
+  // after its producer: 77 us against 105 us front to back).
+  const uint64_t o = (uint64_t)(gridDim.x - 1 - blockIdx.x) * GROUPS + threadIdx.x / G;
+  const bool live = o < a.n_out;
+  const int c = gridDim.y - 1 - blockIdx.y;
+  int64_t in_off = 0, out_off = 0;
+  if (live) fold_decode(a.kept, o, in_off, out_off);
+  const int64_t r0 = (int64_t)c * a.chunk;
+  const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
+  const T *p = (const T *)a.in + in_off;
+  C acc0 = CB::init(), acc1 = CB::init(), acc2 = CB::init(), acc3 = CB::init();
+  const int64_t nv = (r1 - r0) / V;
+  const FVec<T, V> *pv = reinterpret_cast<const FVec<T, V> *>(p + r0);
+  int64_t i = lane;
+  for (; i + 3 * G < nv; i += 4 * G) {
+    FVec<T, V> x0 = pv[i], x1 = pv[i + G], x2 = pv[i + 2 * G], x3 = pv[i + 3 * G];
 #pragma unroll
-      for (int k = 0; k < V; k++) {
-        acc0 = CB::apply(acc0, IN::ld(x0.v[k]));
-        acc1 = CB::apply(acc1, IN::ld(x1.v[k]));
-        acc2 = CB::apply(acc2, IN::ld(x2.v[k]));
-        acc3 = CB::apply(acc3, IN::ld(x3.v[k]));
-      }
+    for (int k = 0; k < V; k++) {
+      acc0 = CB::apply(acc0, IN::ld(x0.v[k]));
+      acc1 = CB::apply(acc1, IN::ld(x1.v[k]));
+      acc2 = CB::apply(acc2, IN::ld(x2.v[k]));
+      acc3 = CB::apply(acc3, IN::ld(x3.v[k]));
     }
-    for (; i < nv; i += G) {
-      FVec<T, V> x0 = pv[i];
+  }
+  for (; i < nv; i += G) {
+    FVec<T, V> x0 = pv[i];
 #pragma unroll
-      for (int k = 0; k < V; k++) acc0 = CB::apply(acc0, IN::ld(x0.v[k]));
-    }
-    for (int64_t e = r0 + nv * V + lane; e < r1; e += G) acc1 = CB::apply(acc1, IN::ld(p[e]));
-    C acc = CB::apply(CB::apply(acc0, acc1), CB::apply(acc2, acc3));
-    acc = group_reduce<CB, C, G>(acc, lds);
-    if (live && lane == 0) {
-      if (a.nsplit > 1) ((C *)a.out)[o * a.nsplit + c] = acc;
-      else ((typename OUT::T *)a.out)[out_off] = OUT::st(acc);
-    }
-    if (G != 64) break;
+    for (int k = 0; k < V; k++) acc0 = CB::apply(acc0, IN::ld(x0.v[k]));
+  }
+  for (int64_t e = r0 + nv * V + lane; e < r1; e += G) acc1 = CB::apply(acc1, IN::ld(p[e]));
+  C acc = CB::apply(CB::apply(acc0, acc1), CB::apply(acc2, acc3));
+  acc = group_reduce<CB, C, G>(acc, lds);
+  if (live && lane == 0) {
+    if (a.nsplit > 1) ((C *)a.out)[o * a.nsplit + c] = acc;
+    else ((typename OUT::T *)a.out)[out_off] = OUT::st(acc);
   }
 }
 
@@ -163,9 +161,11 @@ __global__ __launch_bounds__(FOLD_THREADS) void fold_col_kernel(ColArgs a) {
   constexpr int LANES = FOLD_THREADS / RG;
   constexpr int U = 8;
   __shared__ C lds[RG > 1 ? (RG - 1) * LANES * V : 1];
-  const uint32_t lb = blockIdx.x % a.lane_blocks;
-  const uint64_t ob = blockIdx.x / a.lane_blocks;
-  const int c = blockIdx.y;
+  // blocks walk the input from its end (see fold_row_kernel)
+  const uint32_t bx = gridDim.x - 1 - blockIdx.x;
+  const uint32_t lb = bx % a.lane_blocks;
+  const uint64_t ob = bx / a.lane_blocks;
+  const int c = gridDim.y - 1 - blockIdx.y;
   const uint32_t ln = threadIdx.x % LANES, rg = threadIdx.x / LANES;
   const uint32_t l = (lb * LANES + ln) * V;
   const bool live = l < a.L;
@@ -277,7 +277,7 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
       a.R = g.R;
       // a wave per row while rows are short, or of medium length but plentiful
       const bool wave_rows = g.R < 1024 || (g.R <= 4096 && g.n_out >= (int64_t)cus * 16);
-      const int64_t blocks = wave_rows ? std::min<int64_t>((g.n_out + 3) / 4, (int64_t)cus * 16) : g.n_out;
+      const int64_t blocks = wave_rows ? (g.n_out + 3) / 4 : g.n_out;
       int nsplit = wave_rows ? 1 : pick_split(blocks, g.R, 8192, cus);
       int64_t chunk = g.R;
       if (nsplit > 1) {

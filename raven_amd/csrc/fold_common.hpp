@@ -70,6 +70,16 @@ __device__ __forceinline__ void fold_decode(const FoldDims &d, uint64_t idx, int
                                             int64_t &out_off) {
   in_off = 0;
   out_off = 0;
+  if (idx <= 0xffffffffull) {  // the common case: 32-bit divisions are an order cheaper
+    uint32_t x = (uint32_t)idx;
+    for (int i = d.n - 1; i >= 0; i--) {
+      const uint32_t q = x / d.shape[i], c = x - q * d.shape[i];
+      x = q;
+      in_off += (int64_t)c * d.in_stride[i];
+      out_off += (int64_t)c * d.out_stride[i];
+    }
+    return;
+  }
   for (int i = d.n - 1; i >= 0; i--) {
     uint64_t q = idx / d.shape[i];
     uint32_t c = (uint32_t)(idx - q * d.shape[i]);

@@ -214,7 +214,9 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   S *smem = reinterpret_cast<S *>(smem_raw);
   uint32_t batch, tm, tn;
-  tile_of_block(a, blockIdx.x, batch, tm, tn);
+  // tiles are walked from the end: an operand the previous kernel has just written
+  // front to back still has its tail in the memory-side cache
+  tile_of_block(a, gridDim.x - 1 - blockIdx.x, batch, tm, tn);
   int64_t ao = 0, bo = 0, co = 0;
   {
     uint32_t idx = batch;
