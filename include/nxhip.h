@@ -15,7 +15,7 @@
      (flip) on inputs; rank <= NXH_MAX_NDIM (nx_c.h:45-61).
    - dtype tags equal Nx's Dtype.Packed.tag (nx_c.h:130-200).
    - every call is asynchronous on the context's stream; nxh_memcpy_d2h,
-     nxh_gather and nxh_synchronize wait for it.
+     nxh_gather, nxh_scatter and nxh_synchronize wait for it.
    - return value: NXH_OK, NXH_INVALID_ARGUMENT (the reference raises
      Invalid_argument) or NXH_FAILURE (the reference raises Failure); the
      message, prefixed "<op>: " like the reference's, is read with
@@ -190,6 +190,36 @@ int nxh_copy(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x);
    out-of-bounds index is reported by this call, as in the reference. */
 int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *data,
                const nxh_tensor *indices, int axis);
+
+/* caml_nx_c_scatter (nx_c_move.c:460-586): `out` already holds the template (the
+   binding copies it first, nx_backend.ml:412-416). mode 0 = Set (the last update
+   in row-major order of the index space wins), 1 = Add (accumulates in that
+   order, in the dtype's compute type). Deterministic. Waits for the stream so
+   that an out-of-bounds index is reported by this call. */
+int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *indices,
+                const nxh_tensor *updates, int axis, int mode);
+/* caml_nx_c_pad (nx_c_move.c:203-276): out = x widened by pad_before[d] elements
+   in front of every axis d (the rest of out's extent behind it), the border
+   holding *fill_value (one storage element of the dtype, host memory; the
+   reference passes it as a scalar tensor filled by the binding). */
+int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+            const void *fill_value, const int64_t *pad_before);
+/* caml_nx_c_cat (nx_c_move.c:278-312): the members, in order, along `axis`. */
+int nxh_cat(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *const *inputs,
+            int n_inputs, int axis);
+
+/* ── scan (nx_c_fold.c:161-176, 741-837; driver nx_c_engine.c:1257-1331) ───── */
+
+/* caml_nx_c_cumsum / cumprod / cummax / cummin: inclusive prefix scan along
+   `axis`; `op` is an nxh_reduce_op. out has x's shape and dtype. */
+int nxh_scan(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x, int axis);
+
+/* ── random (nx_c_random.c) ──────────────────────────────────────────────── */
+
+/* caml_nx_c_threefry (nx_c_random.c:36-133): Threefry-2x32, 20 rounds, on int32
+   tensors of equal shape whose last axis (extent 2) holds the word pair. */
+int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *key,
+                 const nxh_tensor *counter);
 
 /* ── measurement ─────────────────────────────────────────────────────────── */
 

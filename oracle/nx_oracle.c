@@ -1850,3 +1850,208 @@ NXO_EXPORT int nxo_gather(const nxh_tensor *out, const nxh_tensor *data,
     return fail(NXH_FAILURE, "index out of bounds for the gathered/scattered axis");
   return NXH_OK;
 }
+
+/* ── pad (nx_c_move.c:203-276) ───────────────────────────────────────────────
+   Border slabs filled by broadcasting the fill scalar through copy, then the
+   interior copied; every output element is written once. `fill` is one
+   storage element of out's dtype. */
+static int pad_fill(const nxh_tensor *slab, const void *fill) {
+  for (int d = 0; d < slab->ndim; d++)
+    if (slab->shape[d] == 0) return NXH_OK;
+  return nxo_fill(slab, fill);
+}
+NXO_EXPORT int nxo_pad(const nxh_tensor *out, const nxh_tensor *in, const void *fill,
+                       const int64_t *pad_before) {
+  if ((unsigned)out->dtype >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (out->ndim != in->ndim) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+  if (is_packed(out->dtype)) return fail(NXH_FAILURE, ERR_PACKED);
+  nxh_tensor slab = *out;
+  for (int d = 0; d < out->ndim; d++) {
+    int64_t before = pad_before[d];
+    int64_t after = out->shape[d] - in->shape[d] - before;
+    if (before < 0 || after < 0) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+    if (before > 0) {
+      slab.shape[d] = before;
+      int rc = pad_fill(&slab, fill);
+      if (rc) return rc;
+    }
+    if (after > 0) {
+      slab.shape[d] = after;
+      slab.offset += (before + in->shape[d]) * out->strides[d];
+      int rc = pad_fill(&slab, fill);
+      if (rc) return rc;
+      slab.offset -= (before + in->shape[d]) * out->strides[d];
+    }
+    slab.shape[d] = in->shape[d];
+    slab.offset += before * out->strides[d];
+  }
+  return nxo_copy(&slab, in);
+}
+
+/* ── cat (nx_c_move.c:278-312) ───────────────────────────────────────────────
+   One strided copy per member into successive slices of the output. */
+NXO_EXPORT int nxo_cat(const nxh_tensor *out, const nxh_tensor *const *inputs, int n,
+                       int axis) {
+  if ((unsigned)out->dtype >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (axis < 0 || axis >= out->ndim) return fail(NXH_INVALID_ARGUMENT, ERR_AXIS);
+  int64_t pos = 0;
+  for (int m = 0; m < n; m++) {
+    const nxh_tensor *in = inputs[m];
+    if (in->ndim != out->ndim) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+    nxh_tensor slice = *out;
+    slice.offset = out->offset + pos * out->strides[axis];
+    for (int d = 0; d < out->ndim; d++) slice.shape[d] = in->shape[d];
+    int rc = nxo_copy(&slice, in);
+    if (rc) return rc;
+    pos += in->shape[axis];
+  }
+  return NXH_OK;
+}
+
+/* ── inclusive scan (nx_c_fold.c:161-176, driver nx_c_engine.c:1257-1331) ────
+   Sequential within a slice: the running value lives in the compute type and a
+   rounded copy is stored per element. One element at a time through the fold
+   step is exactly the reference's CMB(s, v); st(out, s). */
+NXO_EXPORT int nxo_scan(int op, const nxh_tensor *out, const nxh_tensor *in, int axis) {
+  if ((unsigned)op >= NXH_REDUCE_COUNT) return fail(NXH_INVALID_ARGUMENT, "unknown op");
+  const fold_table *t = fold_tables[op];
+  int dt = in->dtype;
+  if ((unsigned)dt >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (!t->init[dt] || !t->step[dt])
+    return fail(NXH_FAILURE, is_packed(dt) ? ERR_PACKED : ERR_UNSUPPORTED);
+  if (axis < 0 || axis >= in->ndim) return fail(NXH_INVALID_ARGUMENT, ERR_AXIS);
+  if (out->ndim != in->ndim) return fail(NXH_INVALID_ARGUMENT, "output rank mismatch");
+  int64_t es = nxo_elem_size(dt), oes = nxo_elem_size(out->dtype);
+  int64_t slices = 1, alen = in->shape[axis];
+  for (int a = 0; a < in->ndim; a++)
+    if (a != axis) slices *= in->shape[a];
+  if (slices == 0 || alen == 0) return NXH_OK;
+  for (int64_t it = 0; it < slices; it++) {
+    int64_t rem = it, io = in->offset, oo = out->offset;
+    for (int a = in->ndim - 1; a >= 0; a--) {
+      if (a == axis) continue;
+      int64_t c = rem % in->shape[a];
+      rem /= in->shape[a];
+      io += c * in->strides[a];
+      oo += c * out->strides[a];
+    }
+    acc_t acc;
+    t->init[dt](&acc);
+    for (int64_t k = 0; k < alen; k++) {
+      t->step[dt](&acc, (const char *)in->data + (io + k * in->strides[axis]) * es, es, 1);
+      t->fini[dt]((char *)out->data + (oo + k * out->strides[axis]) * oes, &acc);
+    }
+  }
+  return NXH_OK;
+}
+
+/* ── threefry2x32-20 (nx_c_random.c:36-133) ──────────────────────────────── */
+static inline uint32_t rotl32(uint32_t x, int r) { return (uint32_t)((x << r) | (x >> (32 - r))); }
+static void threefry2x32(uint32_t k0, uint32_t k1, uint32_t c0, uint32_t c1, uint32_t *o0,
+                         uint32_t *o1) {
+  static const int rots[8] = {13, 15, 26, 6, 17, 29, 16, 24};
+  uint32_t ks[3] = {k0, k1, (uint32_t)0x1BD11BDA ^ k0 ^ k1};
+  uint32_t x0 = c0 + k0, x1 = c1 + k1;
+  for (int r = 0; r < 20; r++) {
+    x0 += x1;
+    x1 = rotl32(x1, rots[r % 8]);
+    x1 ^= x0;
+    if ((r + 1) % 4 == 0) {
+      int s = (r + 1) / 4;
+      x0 += ks[s % 3];
+      x1 += ks[(s + 1) % 3] + (uint32_t)s;
+    }
+  }
+  *o0 = x0;
+  *o1 = x1;
+}
+NXO_EXPORT int nxo_threefry(const nxh_tensor *out, const nxh_tensor *key, const nxh_tensor *ctr) {
+  if (out->dtype != NXH_I32 || key->dtype != NXH_I32 || ctr->dtype != NXH_I32)
+    return fail(NXH_FAILURE, ERR_UNSUPPORTED);
+  const char *bad = "threefry: last axis must have extent 2";
+  if (key->ndim < 1 || key->ndim != ctr->ndim || key->ndim != out->ndim)
+    return fail(NXH_INVALID_ARGUMENT, bad);
+  int last = key->ndim - 1;
+  for (int d = 0; d < key->ndim; d++)
+    if (key->shape[d] != ctr->shape[d] || key->shape[d] != out->shape[d])
+      return fail(NXH_INVALID_ARGUMENT, bad);
+  if (key->shape[last] != 2) return fail(NXH_INVALID_ARGUMENT, bad);
+  int64_t vectors = 1;
+  for (int d = 0; d < last; d++) vectors *= key->shape[d];
+  const int32_t *kd = key->data, *cd = ctr->data;
+  int32_t *od = out->data;
+  for (int64_t it = 0; it < vectors; it++) {
+    int64_t rem = it, kb = key->offset, cb = ctr->offset, ob = out->offset;
+    for (int d = last - 1; d >= 0; d--) {
+      int64_t c = rem % key->shape[d];
+      rem /= key->shape[d];
+      kb += c * key->strides[d];
+      cb += c * ctr->strides[d];
+      ob += c * out->strides[d];
+    }
+    uint32_t o0, o1;
+    threefry2x32((uint32_t)kd[kb], (uint32_t)kd[kb + key->strides[last]], (uint32_t)cd[cb],
+                 (uint32_t)cd[cb + ctr->strides[last]], &o0, &o1);
+    od[ob] = (int32_t)o0;
+    od[ob + out->strides[last]] = (int32_t)o1;
+  }
+  return NXH_OK;
+}
+
+/* ── scatter (nx_c_move.c:460-586) ───────────────────────────────────────────
+   out already holds the template. A serial row-major walk over the index space:
+   Set keeps the last write, Add accumulates in the compute type in that order. */
+#define MOVE_ADD_SINT(a, b) ((int64_t)((uint64_t)(a) + (uint64_t)(b)))
+#define MOVE_ADD_UINT(a, b) ((a) + (b))
+#define MOVE_ADD_FLOAT(a, b) ((a) + (b))
+#define MOVE_ADD_COMPLEX(a, b) ((a) + (b))
+#define MOVE_ADD_BOOL(a, b) ((a) + (b))
+typedef void scatter_add_fn(char *out, const char *upd);
+#define SCATTER_ADD(tag, sfx, S, C, LD, ST, cat) \
+  static void scatter_add_##sfx(char *out, const char *upd) { \
+    st_##sfx(out, (C)MOVE_ADD_##cat(ld_##sfx(out), ld_##sfx(upd))); \
+  }
+NXO_TABLE(SCATTER_ADD)
+#define SCATTER_ADD_ROW(tag, sfx, S, C, LD, ST, cat) [tag] = scatter_add_##sfx,
+static scatter_add_fn *const scatter_add_tbl[NXH_DTYPE_COUNT] = {NXO_TABLE(SCATTER_ADD_ROW)};
+
+NXO_EXPORT int nxo_scatter(const nxh_tensor *out, const nxh_tensor *indices,
+                           const nxh_tensor *updates, int axis, int mode) {
+  int dt = out->dtype;
+  if ((unsigned)dt >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (is_packed(dt)) return fail(NXH_FAILURE, ERR_PACKED);
+  if (axis < 0 || axis >= out->ndim) return fail(NXH_INVALID_ARGUMENT, ERR_AXIS);
+  if (out->ndim != indices->ndim || out->ndim != updates->ndim)
+    return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+  for (int d = 0; d < out->ndim; d++) {
+    if (indices->shape[d] != updates->shape[d]) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+    if (d != axis && indices->shape[d] != out->shape[d]) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+  }
+  scatter_add_fn *add = mode == 1 ? scatter_add_tbl[dt] : NULL;
+  if (mode == 1 && !add) return fail(NXH_FAILURE, ERR_UNSUPPORTED);
+  int nd = indices->ndim;
+  int64_t total = 1, es = nxo_elem_size(dt), alen = out->shape[axis];
+  for (int d = 0; d < nd; d++) total *= indices->shape[d];
+  for (int64_t it = 0; it < total; it++) {
+    int64_t coord[NXH_MAX_NDIM], rem = it;
+    for (int d = nd - 1; d >= 0; d--) {
+      coord[d] = rem % indices->shape[d];
+      rem /= indices->shape[d];
+    }
+    int64_t io = indices->offset, uo = updates->offset, oo = out->offset;
+    for (int d = 0; d < nd; d++) {
+      io += coord[d] * indices->strides[d];
+      uo += coord[d] * updates->strides[d];
+    }
+    int64_t index = ((const int32_t *)indices->data)[io];
+    if (index < 0) index += alen;
+    if (index < 0 || index >= alen)
+      return fail(NXH_FAILURE, "index out of bounds for the gathered/scattered axis");
+    for (int d = 0; d < nd; d++) oo += (d == axis ? index : coord[d]) * out->strides[d];
+    char *op = (char *)out->data + oo * es;
+    const char *up = (const char *)updates->data + uo * es;
+    if (add) add(op, up);
+    else memcpy(op, up, (size_t)es);
+  }
+  return NXH_OK;
+}

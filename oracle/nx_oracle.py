@@ -56,6 +56,11 @@ def lib() -> C.CDLL:
             "nxo_argreduce": [C.c_int, T, T, C.c_int],
             "nxo_matmul": [T, T, T],
             "nxo_gather": [T, T, T, C.c_int],
+            "nxo_pad": [T, T, C.c_void_p, C.POINTER(C.c_int64)],
+            "nxo_cat": [T, C.POINTER(T), C.c_int, C.c_int],
+            "nxo_scan": [C.c_int, T, T, C.c_int],
+            "nxo_threefry": [T, T, T],
+            "nxo_scatter": [T, T, T, C.c_int, C.c_int],
         }.items():
             getattr(L, name).argtypes = args
             getattr(L, name).restype = C.c_int
@@ -234,6 +239,46 @@ class OracleBackend:
     def gather(self, data, indices, axis):
         out = self.buffer(data.dtype, indices.shape)
         _check(lib().nxo_gather(out.desc(), data.desc(), indices.desc(), axis), "gather")
+        return out
+
+    # materialising movement, scan, random, scatter -------------------------
+    def pad(self, x, padding, fill_storage: np.ndarray):
+        out = self.buffer(x.dtype, [s + b + a for s, (b, a) in zip(x.shape, padding)])
+        fill = np.ascontiguousarray(fill_storage, dtype=x.dtype.np_storage).reshape(1)
+        before = (C.c_int64 * max(len(padding), 1))(*[b for b, _ in padding])
+        _check(lib().nxo_pad(out.desc(), x.desc(), fill.ctypes.data, before), "pad")
+        return out
+
+    def cat(self, tensors, axis):
+        if not tensors:
+            raise ValueError("cat: empty tensor list")
+        first = tensors[0]
+        axis = axis + len(first.shape) if axis < 0 else axis
+        if not 0 <= axis < len(first.shape):
+            raise ValueError("cat: axis out of range")
+        shape = list(first.shape)
+        shape[axis] = sum(t.shape[axis] for t in tensors)
+        out = self.buffer(first.dtype, shape)
+        descs = [t.desc() for t in tensors]
+        arr = (C.POINTER(NxhTensor) * len(descs))(*[C.pointer(d) for d in descs])
+        _check(lib().nxo_cat(out.desc(), arr, len(descs), axis), "cat")
+        return out
+
+    def associative_scan(self, axis, op: str, x):
+        out = self.buffer(x.dtype, x.shape)
+        _check(lib().nxo_scan(REDUCE_OPS.index(op), out.desc(), x.desc(), axis),
+               {"sum": "cumsum", "prod": "cumprod", "max": "cummax", "min": "cummin"}[op])
+        return out
+
+    def threefry(self, key, counter):
+        out = self.buffer(dt.int32, counter.shape)
+        _check(lib().nxo_threefry(out.desc(), key.desc(), counter.desc()), "threefry")
+        return out
+
+    def scatter(self, mode: str, unique_indices: bool, template, indices, updates, axis):
+        out = self.copy(template)
+        _check(lib().nxo_scatter(out.desc(), indices.desc(), updates.desc(), axis,
+                                 {"set": 0, "add": 1}[mode]), "scatter")
         return out
 
 

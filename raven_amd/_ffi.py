@@ -84,6 +84,11 @@ SIGNATURES = {
     "nxh_argreduce": (C.c_int, [_CTX, C.c_int, _T, _T, C.c_int]),
     "nxh_matmul": (C.c_int, [_CTX, _T, _T, _T]),
     "nxh_copy": (C.c_int, [_CTX, _T, _T]),
+    "nxh_scatter": (C.c_int, [_CTX, _T, _T, _T, C.c_int, C.c_int]),
+    "nxh_pad": (C.c_int, [_CTX, _T, _T, C.c_void_p, C.POINTER(C.c_int64)]),
+    "nxh_cat": (C.c_int, [_CTX, _T, C.POINTER(_T), C.c_int, C.c_int]),
+    "nxh_scan": (C.c_int, [_CTX, C.c_int, _T, _T, C.c_int]),
+    "nxh_threefry": (C.c_int, [_CTX, _T, _T, _T]),
     "nxh_gather": (C.c_int, [_CTX, _T, _T, _T, C.c_int]),
     "nxh_timer_start": (C.c_int, [_CTX]),
     "nxh_timer_stop": (C.c_int, [_CTX, _P(C.c_float)]),

@@ -1,7 +1,7 @@
-// fold_common.hpp — what the reduction (fold.hip) and argmax/argmin (arg.hip)
-// translation units share: storage/compute adapters, lane exchange, index
-// decoding on the device; reduction geometry, output squeezing, scratch blocks
-// and split sizing on the host.
+// fold_common.hpp — what the reduction (fold.hip), argmax/argmin (arg.hip) and
+// scan (scan.hip) translation units share: combine rules, storage/compute
+// adapters, lane exchange and index decoding on the device; reduction
+// geometry, output squeezing, scratch blocks and split sizing on the host.
 #pragma once
 
 #include <algorithm>
@@ -13,6 +13,49 @@ constexpr int FOLD_MAXD = 12;
 constexpr int FOLD_THREADS = 256;
 
 static inline bool aligned_to16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// ── combine rules ───────────────────────────────────────────────────────────
+template <int OP, class C, Cat cat>
+struct Combine {
+  __device__ __forceinline__ static C init() {
+    if constexpr (OP == NXH_SUM) {
+      if constexpr (cat == CAT_COMPLEX) return C{0, 0};
+      else return (C)0;
+    } else if constexpr (OP == NXH_PROD) {
+      if constexpr (cat == CAT_COMPLEX) return C{1, 0};
+      else return (C)1;
+    } else if constexpr (OP == NXH_RMAX) {
+      if constexpr (cat == CAT_FLOAT) return (C)(-__builtin_inff());
+      else if constexpr (cat == CAT_SINT || (cat == CAT_UINT && std::is_signed<C>::value)) return (C)INT64_MIN;
+      else return (C)0;
+    } else {
+      if constexpr (cat == CAT_FLOAT) return (C)__builtin_inff();
+      else if constexpr (cat == CAT_BOOL) return (C)1;
+      else if constexpr (std::is_signed<C>::value) return (C)INT64_MAX;
+      else return (C)UINT64_MAX;
+    }
+  }
+  __device__ __forceinline__ static C apply(C m, C v) {
+    if constexpr (OP == NXH_SUM) {
+      if constexpr (cat == CAT_SINT) return (C)((uint64_t)m + (uint64_t)v);
+      else return m + v;
+    } else if constexpr (OP == NXH_PROD) {
+      if constexpr (cat == CAT_SINT) return (C)((uint64_t)m * (uint64_t)v);
+      else return m * v;
+    } else if constexpr (OP == NXH_RMAX) {
+      if constexpr (cat == CAT_FLOAT) return (v > m) ? v : ((v != v) ? v : m);
+      else if constexpr (cat == CAT_BOOL) return (C)(m | v);
+      else return v > m ? v : m;
+    } else {
+      if constexpr (cat == CAT_FLOAT) return (v < m) ? v : ((v != v) ? v : m);
+      else if constexpr (cat == CAT_BOOL) return (C)(m & v);
+      else return v < m ? v : m;
+    }
+  }
+};
+constexpr bool fold_ok(int op, Cat c) {
+  return (op == NXH_SUM || op == NXH_PROD) ? (c != CAT_BOOL) : (c != CAT_COMPLEX);
+}
 
 // ── lane exchange for any trivially copyable accumulator ───────────────────
 template <class T>

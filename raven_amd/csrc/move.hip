@@ -1,5 +1,7 @@
-// move.hip — gather (packages/nx/lib/backend_c/nx_c_move.c:342-458).
+// move.hip — gather, scatter, pad, cat (packages/nx/lib/backend_c/nx_c_move.c)
+// and threefry (nx_c_random.c).
 //
+// gather (nx_c_move.c:342-458):
 // out[c] = data[c with c[axis] <- indices[c]]; int32 indices, one negative wrap,
 // then a bounds check whose failure is reported by the gather call itself, as
 // in the reference: kernels raise a device flag and skip the access, the host
@@ -8,6 +10,21 @@
 //                embedding lookup): one wave64 copies one row with 16-byte
 //                loads.
 //   gather_any   one lane per output element, per-lane unravel.
+//
+// scatter (nx_c_move.c:460-586): the reference walks the index space serially in
+// row-major order, so `Set keeps the last write and `Add accumulates in that
+// order. All updates that can meet in one output element share their
+// coordinates off the scatter axis and are visited in ascending axis order, so
+// one lane per off-axis coordinate ("column") walking the axis in order
+// reproduces the serial result exactly, with no atomics and no race: different
+// columns touch disjoint outputs.
+//
+// pad / cat (nx_c_move.c:203-312) are, as in the reference, compositions of the
+// copy and fill kernels over sub-views of the output: every output element is
+// written once.
+//
+// threefry (nx_c_random.c:36-133): Threefry-2x32, 20 rounds, one lane per
+// (key, counter) vector; normative bit for bit.
 
 #include "nxh_common.hpp"
 
@@ -181,5 +198,289 @@ NXH_EXPORT int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
     NXH_HIP(op, hipStreamSynchronize(ctx->stream));
     return nxh_fail(NXH_FAILURE, op, NXH_ERR_INDEX_OOB);
   }
+  return NXH_OK;
+}
+
+// ── scatter ─────────────────────────────────────────────────────────────────
+struct ScatterArgs {
+  char *out;
+  const int32_t *idx;
+  const char *upd;
+  int ncol_dims;  // off-axis dims
+  int64_t columns, n_idx, axis_len;
+  int64_t cshape[NXH_MAX_NDIM];
+  int64_t c_ostride[NXH_MAX_NDIM], c_istride[NXH_MAX_NDIM], c_ustride[NXH_MAX_NDIM];
+  int64_t a_ostride, a_istride, a_ustride;  // along the scatter axis
+  int *fault;
+};
+// ADD: accumulate in the dtype's compute type; otherwise a byte-exact store.
+template <int DT, bool ADD>
+__global__ __launch_bounds__(256) void scatter_kernel(ScatterArgs a) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= a.columns) return;
+  int64_t rem = col, oo = 0, io = 0, uo = 0;
+  for (int d = a.ncol_dims - 1; d >= 0; d--) {
+    const int64_t c = rem % a.cshape[d];
+    rem /= a.cshape[d];
+    oo += c * a.c_ostride[d];
+    io += c * a.c_istride[d];
+    uo += c * a.c_ustride[d];
+  }
+  S *out = reinterpret_cast<S *>(a.out) + oo;
+  const int32_t *idx = a.idx + io;
+  const S *upd = reinterpret_cast<const S *>(a.upd) + uo;
+  for (int64_t i = 0; i < a.n_idx; i++) {
+    int64_t index = idx[i * a.a_istride];
+    if (index < 0) index += a.axis_len;
+    if (index < 0 || index >= a.axis_len) {
+      atomicOr(a.fault, 1);
+      return;
+    }
+    S *o = out + index * a.a_ostride;
+    const S u = upd[i * a.a_ustride];
+    if constexpr (ADD) {
+      const C x = TR::ld(*o), y = TR::ld(u);
+      if constexpr (TR::cat == CAT_SINT) *o = TR::st((C)((uint64_t)x + (uint64_t)y));
+      else *o = TR::st((C)(x + y));
+    } else {
+      *o = u;
+    }
+  }
+}
+typedef void (*scatter_launch_fn)(nxh_context *, const ScatterArgs &, bool);
+template <int DT>
+static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add) {
+  const dim3 grid((unsigned)((a.columns + 255) / 256));
+  if (add) hipLaunchKernelGGL((scatter_kernel<DT, true>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((scatter_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, a);
+}
+
+// Reads the out-of-bounds flag back after the launch: the failure is reported by
+// the call that caused it (nx_c_move.c:448-458, 571-586).
+static int collect_index_fault(nxh_context *ctx, const char *op) {
+  NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag_host, ctx->fault_flag, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+  NXH_HIP(op, hipStreamSynchronize(ctx->stream));
+  if (*ctx->fault_flag_host != 0) {
+    *ctx->fault_flag_host = 0;
+    NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag, ctx->fault_flag_host, sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+    NXH_HIP(op, hipStreamSynchronize(ctx->stream));
+    return nxh_fail(NXH_FAILURE, op, NXH_ERR_INDEX_OOB);
+  }
+  return NXH_OK;
+}
+
+NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *indices,
+                           const nxh_tensor *updates, int axis, int mode) {
+  const char *op = "scatter";
+  if (!ctx || !out || !indices || !updates) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, indices);
+  if (!rc) rc = nxh_check_tensor(op, updates);
+  if (rc) return rc;
+  const int dt = out->dtype;
+  if (nxh_is_packed(dt)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  if (updates->dtype != dt || indices->dtype != NXH_I32) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  if (mode != 0 && mode != 1) return nxh_fail(NXH_INVALID_ARGUMENT, op, "mode must be 0 (set) or 1 (add)");
+  if (axis < 0 || axis >= out->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXIS);
+  if (out->ndim != indices->ndim || out->ndim != updates->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  for (int d = 0; d < out->ndim; d++) {
+    if (indices->shape[d] != updates->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    if (d != axis && indices->shape[d] != out->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  }
+  for (int d = 0; d < out->ndim; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  ScatterArgs a;
+  a.columns = 1;
+  a.ncol_dims = 0;
+  for (int d = 0; d < out->ndim; d++) {
+    if (d == axis) continue;
+    a.cshape[a.ncol_dims] = indices->shape[d];
+    a.c_ostride[a.ncol_dims] = out->strides[d];
+    a.c_istride[a.ncol_dims] = indices->strides[d];
+    a.c_ustride[a.ncol_dims] = updates->strides[d];
+    a.columns *= indices->shape[d];
+    a.ncol_dims++;
+  }
+  a.n_idx = indices->shape[axis];
+  if (a.columns == 0 || a.n_idx == 0) return NXH_OK;
+  if (a.columns > 0x7fffffffLL * 256) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  const int64_t es = nxh_elem_size(dt);
+  a.out = (char *)out->data + out->offset * es;
+  a.idx = (const int32_t *)indices->data + indices->offset;
+  a.upd = (const char *)updates->data + updates->offset * es;
+  a.axis_len = out->shape[axis];
+  a.a_ostride = out->strides[axis];
+  a.a_istride = indices->strides[axis];
+  a.a_ustride = updates->strides[axis];
+  a.fault = ctx->fault_flag;
+  static const scatter_launch_fn table[NXH_DTYPE_COUNT] = {
+#define NXH_SC(DT) [DT] = &scatter_launch<DT>,
+      NXH_FOR_COMPUTE_DTYPES(NXH_SC)
+#undef NXH_SC
+  };
+  if (!table[dt]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("scatter_columns");
+  table[dt](ctx, a, mode == 1);
+  NXH_HIP(op, hipGetLastError());
+  return collect_index_fault(ctx, op);
+}
+
+// ── threefry2x32-20 ─────────────────────────────────────────────────────────
+struct ThreefryArgs {
+  const int32_t *key, *ctr;
+  int32_t *out;
+  int prefix_ndim;
+  int64_t vectors;
+  int64_t shape[NXH_MAX_NDIM];
+  int64_t kstride[NXH_MAX_NDIM], cstride[NXH_MAX_NDIM], ostride[NXH_MAX_NDIM];
+  int64_t key_last, ctr_last, out_last;  // stride of the 2-word axis
+};
+__device__ __forceinline__ uint32_t rotl32(uint32_t x, int r) { return (x << r) | (x >> (32 - r)); }
+__global__ __launch_bounds__(256) void threefry_kernel(ThreefryArgs a) {
+  const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (it >= a.vectors) return;
+  int64_t rem = it, kb = 0, cb = 0, ob = 0;
+  for (int d = a.prefix_ndim - 1; d >= 0; d--) {
+    const int64_t c = rem % a.shape[d];
+    rem /= a.shape[d];
+    kb += c * a.kstride[d];
+    cb += c * a.cstride[d];
+    ob += c * a.ostride[d];
+  }
+  const uint32_t k0 = (uint32_t)a.key[kb], k1 = (uint32_t)a.key[kb + a.key_last];
+  const uint32_t ks[3] = {k0, k1, 0x1BD11BDAu ^ k0 ^ k1};
+  uint32_t x0 = (uint32_t)a.ctr[cb] + k0, x1 = (uint32_t)a.ctr[cb + a.ctr_last] + k1;
+  constexpr int rots[8] = {13, 15, 26, 6, 17, 29, 16, 24};
+#pragma unroll
+  for (int r = 0; r < 20; r++) {
+    x0 += x1;
+    x1 = rotl32(x1, rots[r % 8]);
+    x1 ^= x0;
+    if ((r + 1) % 4 == 0) {
+      const int s = (r + 1) / 4;
+      x0 += ks[s % 3];
+      x1 += ks[(s + 1) % 3] + (uint32_t)s;
+    }
+  }
+  a.out[ob] = (int32_t)x0;
+  a.out[ob + a.out_last] = (int32_t)x1;
+}
+
+NXH_EXPORT int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *key,
+                            const nxh_tensor *counter) {
+  const char *op = "threefry";
+  if (!ctx || !out || !key || !counter) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, key);
+  if (!rc) rc = nxh_check_tensor(op, counter);
+  if (rc) return rc;
+  if (out->dtype != NXH_I32 || key->dtype != NXH_I32 || counter->dtype != NXH_I32)
+    return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  const char *bad = "threefry: last axis must have extent 2";
+  if (key->ndim < 1 || key->ndim != counter->ndim || key->ndim != out->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, bad);
+  const int last = key->ndim - 1;
+  for (int d = 0; d < key->ndim; d++)
+    if (key->shape[d] != counter->shape[d] || key->shape[d] != out->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, bad);
+  if (key->shape[last] != 2) return nxh_fail(NXH_INVALID_ARGUMENT, op, bad);
+  ThreefryArgs a;
+  a.vectors = 1;
+  a.prefix_ndim = last;
+  for (int d = 0; d < last; d++) {
+    a.shape[d] = key->shape[d];
+    a.kstride[d] = key->strides[d];
+    a.cstride[d] = counter->strides[d];
+    a.ostride[d] = out->strides[d];
+    a.vectors *= key->shape[d];
+  }
+  if (a.vectors == 0) return NXH_OK;
+  if (a.vectors > 0x7fffffffLL * 256) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  a.key = (const int32_t *)key->data + key->offset;
+  a.ctr = (const int32_t *)counter->data + counter->offset;
+  a.out = (int32_t *)out->data + out->offset;
+  a.key_last = key->strides[last];
+  a.ctr_last = counter->strides[last];
+  a.out_last = out->strides[last];
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("threefry");
+  hipLaunchKernelGGL(threefry_kernel, dim3((unsigned)((a.vectors + 255) / 256)), dim3(256), 0, ctx->stream, a);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+// ── pad / cat: compositions of fill and copy over sub-views of the output ──
+static bool has_zero_extent(const nxh_tensor *t) {
+  for (int d = 0; d < t->ndim; d++)
+    if (t->shape[d] == 0) return true;
+  return false;
+}
+
+NXH_EXPORT int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *fill_value,
+                       const int64_t *pad_before) {
+  const char *op = "pad";
+  if (!ctx || !out || !x || !fill_value || (out->ndim > 0 && !pad_before))
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (rc) return rc;
+  if (out->ndim != x->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  if (nxh_is_packed(out->dtype)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  if (out->dtype != x->dtype) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  for (int d = 0; d < out->ndim; d++)
+    if (pad_before[d] < 0 || out->shape[d] - x->shape[d] - pad_before[d] < 0)
+      return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  // `slab` narrows toward the interior: entering step d, axes < d carry the
+  // interior extent and offset, axes >= d are still full (nx_c_move.c:246-268)
+  nxh_tensor slab = *out;
+  for (int d = 0; d < out->ndim; d++) {
+    const int64_t before = pad_before[d];
+    const int64_t after = out->shape[d] - x->shape[d] - before;
+    if (before > 0) {
+      slab.shape[d] = before;
+      if (!has_zero_extent(&slab) && (rc = nxh_fill(ctx, &slab, fill_value))) return rc;
+    }
+    if (after > 0) {
+      slab.shape[d] = after;
+      slab.offset += (before + x->shape[d]) * out->strides[d];
+      if (!has_zero_extent(&slab) && (rc = nxh_fill(ctx, &slab, fill_value))) return rc;
+      slab.offset -= (before + x->shape[d]) * out->strides[d];
+    }
+    slab.shape[d] = x->shape[d];
+    slab.offset += before * out->strides[d];
+  }
+  rc = nxh_copy(ctx, &slab, x);
+  nxh_set_path("pad_slabs");
+  return rc;
+}
+
+NXH_EXPORT int nxh_cat(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *const *inputs, int n_inputs,
+                       int axis) {
+  const char *op = "cat";
+  if (!ctx || !out || (n_inputs > 0 && !inputs)) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (rc) return rc;
+  if (axis < 0 || axis >= out->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXIS);
+  int64_t pos = 0;
+  for (int m = 0; m < n_inputs; m++) {
+    const nxh_tensor *in = inputs[m];
+    if (!in) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+    if ((rc = nxh_check_tensor(op, in))) return rc;
+    if (in->ndim != out->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    if (in->dtype != out->dtype) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+    for (int d = 0; d < out->ndim; d++)
+      if (d != axis && in->shape[d] != out->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    if (pos + in->shape[axis] > out->shape[axis]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    nxh_tensor slice = *out;
+    slice.offset = out->offset + pos * out->strides[axis];
+    for (int d = 0; d < out->ndim; d++) slice.shape[d] = in->shape[d];
+    if (!has_zero_extent(&slice) && (rc = nxh_copy(ctx, &slice, in))) return rc;
+    pos += in->shape[axis];
+  }
+  nxh_set_path("cat_slices");
   return NXH_OK;
 }

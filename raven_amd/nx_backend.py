@@ -27,7 +27,7 @@ import numpy as np
 
 from . import _ffi
 from . import dtype as dt
-from ._ffi import BINARY_OPS, COMPARE_OPS, REDUCE_OPS, UNARY_OPS, make_tensor
+from ._ffi import BINARY_OPS, COMPARE_OPS, REDUCE_OPS, UNARY_OPS, NxhTensor, make_tensor
 from .view import View, numel
 
 
@@ -265,6 +265,54 @@ class Backend:
         out = self.buffer(data.dtype, indices.shape)
         o, d, i = out._desc(), data._desc(), indices._desc()
         self._check(self._lib.nxh_gather(self._h, C.byref(o), C.byref(d), C.byref(i), axis))
+        return out
+
+    # ── scatter / pad / cat / scan / threefry (nx_backend.ml:309-319, 362-416, 474-477)
+    def scatter(self, mode: str, unique_indices: bool, template: Tensor, indices: Tensor, updates: Tensor,
+                axis: int) -> Tensor:
+        """``mode`` is "set" or "add"; ``unique_indices`` is accepted and ignored,
+        as in the reference binding. The result starts as a copy of ``template``."""
+        out = self.copy(template)
+        o, i, u = out._desc(), indices._desc(), updates._desc()
+        self._check(self._lib.nxh_scatter(self._h, C.byref(o), C.byref(i), C.byref(u), axis,
+                                          {"set": 0, "add": 1}[mode]))
+        return out
+
+    def pad(self, x: Tensor, padding: Sequence[Sequence[int]], fill_value) -> Tensor:
+        out = self.buffer(x.dtype, [s + int(b) + int(a) for s, (b, a) in zip(x.shape, padding)])
+        enc = fill_value if isinstance(fill_value, np.ndarray) else encode_scalar(x.dtype, fill_value)
+        enc = np.ascontiguousarray(enc.reshape(1))
+        before = (C.c_int64 * max(len(padding), 1))(*[int(b) for b, _ in padding])
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_pad(self._h, C.byref(o), C.byref(a), enc.ctypes.data, before))
+        return out
+
+    def cat(self, tensors: Sequence[Tensor], axis: int) -> Tensor:
+        if not tensors:
+            raise ValueError("cat: empty tensor list")
+        first = tensors[0]
+        axis = axis + len(first.shape) if axis < 0 else axis
+        if not 0 <= axis < len(first.shape):
+            raise ValueError("cat: axis out of range")
+        shape = list(first.shape)
+        shape[axis] = sum(t.shape[axis] for t in tensors)
+        out = self.buffer(first.dtype, shape)
+        descs = [t._desc() for t in tensors]
+        arr = (C.POINTER(NxhTensor) * len(descs))(*[C.pointer(d) for d in descs])
+        o = out._desc()
+        self._check(self._lib.nxh_cat(self._h, C.byref(o), arr, len(descs), axis))
+        return out
+
+    def associative_scan(self, axis: int, op: str, x: Tensor) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_scan(self._h, REDUCE_OPS.index(op), C.byref(o), C.byref(a), axis))
+        return out
+
+    def threefry(self, key: Tensor, counter: Tensor) -> Tensor:
+        out = self.buffer(dt.int32, counter.shape)
+        o, k, c = out._desc(), key._desc(), counter._desc()
+        self._check(self._lib.nxh_threefry(self._h, C.byref(o), C.byref(k), C.byref(c)))
         return out
 
     # ── fold family (nx_backend.ml:266-307) ─────────────────────────────────

@@ -558,3 +558,136 @@ def test_layouts_copy_and_errors():
         B.unary("round", T(np.ones(2, np.complex64), dt.complex64))
     with pytest.raises(RuntimeError):
         B.compare("cmplt", T(np.ones(2, np.complex64), dt.complex64), T(np.ones(2, np.complex64), dt.complex64))
+
+
+# ── pad, cat, scan, threefry, scatter ────────────────────────────────────────
+
+def _mk(B, a, d):
+    a = np.ascontiguousarray(a)
+    return B.reshape(B.from_host(a, d), a.shape)
+
+
+def _threefry_py(k0, k1, c0, c1):
+    """Threefry-2x32-20 from its published definition, in Python integers."""
+    m = 0xFFFFFFFF
+    rots = (13, 15, 26, 6, 17, 29, 16, 24)
+    ks = (k0, k1, 0x1BD11BDA ^ k0 ^ k1)
+    x0, x1 = (c0 + k0) & m, (c1 + k1) & m
+    for r in range(20):
+        x0 = (x0 + x1) & m
+        x1 = ((x1 << rots[r % 8]) | (x1 >> (32 - rots[r % 8]))) & m
+        x1 ^= x0
+        if (r + 1) % 4 == 0:
+            s = (r + 1) // 4
+            x0 = (x0 + ks[s % 3]) & m
+            x1 = (x1 + ks[(s + 1) % 3] + s) & m
+    return x0, x1
+
+
+def test_threefry_known_answers_and_independent_port():
+    B = OracleBackend()
+    for case in GOLD["threefry_kat"]["cases"]:
+        k = _mk(B, np.array(case["key"], np.int32), dt.int32)
+        c = _mk(B, np.array(case["counter"], np.int32), dt.int32)
+        assert logical(B.threefry(k, c)).tolist() == case["out"]
+    rng = np.random.default_rng(5)
+    key = rng.integers(-2**31, 2**31, (3, 7, 2)).astype(np.int32)
+    ctr = rng.integers(-2**31, 2**31, (3, 7, 2)).astype(np.int32)
+    want = np.empty_like(key)
+    for i in np.ndindex(3, 7):
+        a, b = _threefry_py(*(int(v) & 0xFFFFFFFF for v in (*key[i], *ctr[i])))
+        want[i] = np.array([a, b], np.uint32).view(np.int32)
+    assert np.array_equal(logical(B.threefry(_mk(B, key, dt.int32), _mk(B, ctr, dt.int32))), want)
+    # strided operands: the word pair is read along the last axis' own stride
+    kt = B.permute(_mk(B, np.ascontiguousarray(key.transpose(2, 0, 1)), dt.int32), (1, 2, 0))
+    assert np.array_equal(logical(B.threefry(kt, _mk(B, ctr, dt.int32))), want)
+    with pytest.raises(ValueError):
+        B.threefry(_mk(B, key[..., :1], dt.int32), _mk(B, ctr[..., :1], dt.int32))
+
+
+def test_pad_cat_reference_vectors_and_numpy():
+    B = OracleBackend()
+    g = GOLD["pad_cat"]
+    pc = g["pad_constant"]
+    got = B.pad(_mk(B, np.array(pc["x"]), dt.float64), pc["padding"], np.array([pc["fill"]]))
+    assert logical(got).tolist() == pc["out"]
+    c0 = g["cat_axis0"]
+    assert logical(B.cat([_mk(B, np.array(c0["a"]), dt.float64), _mk(B, np.array(c0["b"]), dt.float64)], 0)).tolist() == c0["out"]
+    c1 = g["cat_axis1_strided"]
+    a = B.permute(_mk(B, np.array(c1["a_storage"]), dt.float64), c1["a_permute"])
+    assert logical(B.cat([a, _mk(B, np.array(c1["b"]), dt.float64)], 1)).tolist() == c1["out"]
+    rng = np.random.default_rng(9)
+    x = rng.integers(-100, 100, (3, 4, 5)).astype(np.int16)
+    t = B.flip(B.permute(_mk(B, x, dt.int16), (2, 0, 1)), (False, True, False))
+    xl = x.transpose(2, 0, 1)[:, ::-1, :]
+    padding = [(2, 0), (0, 3), (1, 1)]
+    assert np.array_equal(logical(B.pad(t, padding, np.array([7], np.int16))), np.pad(xl, padding, constant_values=7))
+    assert np.array_equal(logical(B.pad(t, [(0, 0)] * 3, np.array([7], np.int16))), xl)
+    parts = [xl, xl[:, :1, :], np.zeros((5, 0, 4), np.int16), xl[:, 1:, :]]
+    tens = [t, B.shrink(t, [(0, 5), (0, 1), (0, 4)]), _mk(B, parts[2], dt.int16), B.shrink(t, [(0, 5), (1, 3), (0, 4)])]
+    assert np.array_equal(logical(B.cat(tens, 1)), np.concatenate(parts, 1))
+    assert np.array_equal(logical(B.cat(tens, -2)), np.concatenate(parts, 1))
+
+
+def test_scan_vs_numpy_and_reference_vector():
+    B = OracleBackend()
+    g = GOLD["cumprod_int32"]
+    assert logical(B.associative_scan(g["axis"], "prod", _mk(B, np.array(g["x"], np.int32), dt.int32))).tolist() == g["out"]
+    rng = np.random.default_rng(21)
+    # integers: exact with wrap-around in the storage width
+    x = rng.integers(-120, 120, (4, 9, 6)).astype(np.int8)
+    t = B.permute(_mk(B, x, dt.int8), (1, 0, 2))
+    xl = x.transpose(1, 0, 2)
+    for axis in (0, 1, 2):
+        assert np.array_equal(logical(B.associative_scan(axis, "sum", t)), np.cumsum(xl.astype(np.int64), axis).astype(np.int8))
+        # |x| <= 120 and at most 9 factors: the int64 running product never overflows, so the
+        # reference's modular product is the exact product truncated to 8 bits
+        assert np.array_equal(logical(B.associative_scan(axis, "prod", t)),
+                              np.cumprod(xl.astype(np.int64), axis).astype(np.int8))
+        assert np.array_equal(logical(B.associative_scan(axis, "max", t)), np.maximum.accumulate(xl, axis))
+        assert np.array_equal(logical(B.associative_scan(axis, "min", t)), np.minimum.accumulate(xl, axis))
+    # floats: f64 is the sequential IEEE sum exactly; NaN sticks from its position on
+    y = rng.standard_normal((5, 33))
+    y[2, 7] = np.nan
+    ty = _mk(B, y, dt.float64)
+    assert np.array_equal(logical(B.associative_scan(1, "sum", ty)), np.cumsum(y, 1), equal_nan=True)
+    got = logical(B.associative_scan(1, "max", ty))
+    assert np.all(np.isnan(got[2, 7:])) and not np.any(np.isnan(got[2, :7]))
+    assert np.array_equal(np.delete(got, 2, 0), np.maximum.accumulate(np.delete(y, 2, 0), 1))
+    # narrow floats carry the running value in f32 and store rounded copies
+    h = (rng.standard_normal(200) * 4).astype(np.float16)
+    run, want = np.float32(0), []
+    for v in h:
+        run = np.float32(run + np.float32(v))
+        want.append(np.float16(run))
+    assert np.array_equal(logical(B.associative_scan(0, "sum", _mk(B, h, dt.float16))), np.array(want, np.float16))
+    with pytest.raises(RuntimeError):
+        B.associative_scan(0, "sum", _mk(B, np.array([1, 0], np.uint8), dt.bool_))
+
+
+def test_scatter_reference_vectors_and_brute_force():
+    B = OracleBackend()
+    for c in GOLD["scatter"]["cases"]:
+        got = B.scatter(c["mode"], False, _mk(B, np.array(c["template"]), dt.float64),
+                        _mk(B, np.array(c["indices"], np.int32), dt.int32),
+                        _mk(B, np.array(c["updates"]), dt.float64), c["axis"])
+        assert logical(got).tolist() == c["out"], c["name"]
+    rng = np.random.default_rng(33)
+    tmpl = rng.integers(-50, 50, (4, 6, 5)).astype(np.int32)
+    for axis in (0, 1, 2):
+        ishape = list(tmpl.shape)
+        ishape[axis] = 9
+        idx = rng.integers(-tmpl.shape[axis], tmpl.shape[axis], ishape).astype(np.int32)  # negatives wrap once
+        upd = rng.integers(-50, 50, ishape).astype(np.int32)
+        for mode in ("set", "add"):
+            want = tmpl.copy()
+            for c in np.ndindex(*ishape):  # row-major serial walk
+                o = list(c)
+                o[axis] = int(idx[c]) % tmpl.shape[axis]
+                want[tuple(o)] = upd[c] if mode == "set" else want[tuple(o)] + upd[c]
+            got = B.scatter(mode, False, _mk(B, tmpl, dt.int32), _mk(B, idx, dt.int32), _mk(B, upd, dt.int32), axis)
+            assert np.array_equal(logical(got), want), (axis, mode)
+    bad = np.array([[9]], np.int32)
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        B.scatter("set", False, _mk(B, np.zeros((1, 4)), dt.float64), _mk(B, bad, dt.int32),
+                  _mk(B, np.ones((1, 1)), dt.float64), 1)
