@@ -194,6 +194,50 @@ class Workloads:
         return ops
 
 
+def next_ops(hip, W):
+    """The operations beside the named hot path (pad, cat, scan, threefry,
+    scatter), timed through the Python mirror with HIP events."""
+    rng = np.random.default_rng(20)
+    out = []
+
+    def timed(name, fn, nbytes, iters=20):
+        for _ in range(3):
+            r = fn()
+            del r
+        hip.synchronize()
+        hip.timer_start()
+        for _ in range(iters):
+            r = fn()
+            del r
+        ms = hip.timer_stop() / iters
+        out.append({"op": name, "ms": round(ms, 5), "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                    "frac_hbm": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "bound": "hbm"})
+
+    x = W.dev(rng.standard_normal((2048, 4100)).astype(np.float32), dt.float32)
+    timed("pad [2048,4100] f32 by ((3,5),(7,1))", lambda: hip.pad(x, [(3, 5), (7, 1)], -2.5),
+          2048 * 4100 * 4 + 2056 * 4108 * 4)
+    parts = [W.dev(rng.standard_normal((1024, 4096)).astype(np.float32), dt.float32) for _ in range(4)]
+    timed("cat 4 x [1024,4096] f32 along axis 0", lambda: hip.cat(parts, 0), 2 * 4 * 1024 * 4096 * 4)
+    timed("cat 4 x [1024,4096] f32 along axis 1", lambda: hip.cat(parts, 1), 2 * 4 * 1024 * 4096 * 4)
+    y = W.dev(rng.standard_normal((4096, 8192)).astype(np.float32), dt.float32)
+    timed("cumsum [4096,8192] f32 axis 1 (scan_rows)", lambda: hip.associative_scan(1, "sum", y), 2 * 4096 * 8192 * 4)
+    timed("cumsum [4096,8192] f32 axis 0 (scan_chunks: 3 passes over the data)", lambda: hip.associative_scan(0, "sum", y), 2 * 4096 * 8192 * 4)
+    n = 1 << 24
+    ctr = W.dev(np.arange(2 * n, dtype=np.int64).astype(np.int32).reshape(n, 2), dt.int32)
+    key = hip.expand(W.dev(np.array([[1234, -99]], np.int32), dt.int32), (n, 2))
+    timed("threefry 2^24 vectors (one key)", lambda: hip.threefry(key, ctr), 2 * n * 8)
+    vocab, dim, ntok = 50257, 768, 8192
+    ids = W.dev(rng.integers(0, vocab, (ntok, 1)).astype(np.int32), dt.int32)
+    idx = hip.expand(ids, (ntok, dim))
+    upd = W.dev(rng.standard_normal((ntok, dim)).astype(np.float32), dt.float32)
+    table = hip.full(dt.float32, (vocab, dim), 0.0)
+    # template copy (read + write of the table) + indices + updates + read-modify-write of the touched rows
+    timed("scatter-add [8192,768] f32 rows into [50257,768] (embedding gradient)",
+          lambda: hip.scatter("add", False, table, idx, upd, 0),
+          2 * vocab * dim * 4 + ntok * 4 + 3 * ntok * dim * 4, iters=5)
+    return out
+
+
 def time_ops(hip, ops, iters, warmup):
     """Average milliseconds per pass of `ops`, HIP events on the context stream."""
     for _ in range(warmup):
@@ -343,6 +387,7 @@ def main():
                     help="also launch 20 plain 64 MiB copies (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--only-config", type=int, choices=(1, 2, 3, 4), default=0,
                     help="time the operations of one configuration only and print their records")
+    ap.add_argument("--only-next", action="store_true", help="time pad/cat/scan/threefry/scatter only")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 forward leg only and print its record")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -353,6 +398,9 @@ def main():
     info = hip.device_info()
     if args.only_gpt2:
         print(json.dumps(config5(hip)))
+        return
+    if args.only_next:
+        print(json.dumps({"ops": next_ops(hip, Workloads(hip))}))
         return
     if args.only_config:
         # one configuration's operations, each timed alone (for profiling runs)
@@ -427,6 +475,7 @@ def main():
             W.keep.clear()
             hip.trim()
         ops_out.append(config5(hip))
+        ops_out.extend(next_ops(hip, W))
 
     line = {
         "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,

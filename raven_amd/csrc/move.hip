@@ -232,15 +232,7 @@ __global__ __launch_bounds__(256) void scatter_kernel(ScatterArgs a) {
   S *out = reinterpret_cast<S *>(a.out) + oo;
   const int32_t *idx = a.idx + io;
   const S *upd = reinterpret_cast<const S *>(a.upd) + uo;
-  for (int64_t i = 0; i < a.n_idx; i++) {
-    int64_t index = idx[i * a.a_istride];
-    if (index < 0) index += a.axis_len;
-    if (index < 0 || index >= a.axis_len) {
-      atomicOr(a.fault, 1);
-      return;
-    }
-    S *o = out + index * a.a_ostride;
-    const S u = upd[i * a.a_ustride];
+  auto apply = [&](S *o, S u) {
     if constexpr (ADD) {
       const C x = TR::ld(*o), y = TR::ld(u);
       if constexpr (TR::cat == CAT_SINT) *o = TR::st((C)((uint64_t)x + (uint64_t)y));
@@ -248,6 +240,61 @@ __global__ __launch_bounds__(256) void scatter_kernel(ScatterArgs a) {
     } else {
       *o = u;
     }
+  };
+  // Steps are taken eight at a time. When their targets are pairwise distinct
+  // (the common case) the eight read-modify-writes are independent and their
+  // memory round trips overlap; otherwise the batch is applied one by one, in
+  // order, so duplicates still see each other.
+  constexpr int B = 8;
+  int64_t i = 0;
+  for (; i + B <= a.n_idx; i += B) {
+    int64_t t[B];
+    S u[B];
+    bool ok = true;
+#pragma unroll
+    for (int j = 0; j < B; j++) {
+      int64_t index = idx[(i + j) * a.a_istride];
+      if (index < 0) index += a.axis_len;
+      ok &= index >= 0 && index < a.axis_len;
+      t[j] = index;
+      u[j] = upd[(i + j) * a.a_ustride];
+    }
+    if (!ok) {
+      atomicOr(a.fault, 1);
+      return;
+    }
+    bool distinct = true;
+#pragma unroll
+    for (int j = 1; j < B; j++)
+#pragma unroll
+      for (int k = 0; k < j; k++) distinct &= t[j] != t[k];
+    if (distinct) {
+      if constexpr (ADD) {
+        S cur[B];
+#pragma unroll
+        for (int j = 0; j < B; j++) cur[j] = out[t[j] * a.a_ostride];
+#pragma unroll
+        for (int j = 0; j < B; j++) {
+          const C x = TR::ld(cur[j]), y = TR::ld(u[j]);
+          if constexpr (TR::cat == CAT_SINT) out[t[j] * a.a_ostride] = TR::st((C)((uint64_t)x + (uint64_t)y));
+          else out[t[j] * a.a_ostride] = TR::st((C)(x + y));
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < B; j++) out[t[j] * a.a_ostride] = u[j];
+      }
+    } else {
+      for (int j = 0; j < B; j++) apply(out + t[j] * a.a_ostride, u[j]);
+    }
+  }
+  for (; i < a.n_idx; i++) {
+    int64_t index = idx[i * a.a_istride];
+    if (index < 0) index += a.axis_len;
+    if (index < 0 || index >= a.axis_len) {
+      atomicOr(a.fault, 1);
+      return;
+    }
+    apply(out + index * a.a_ostride, upd[i * a.a_ustride]);
   }
 }
 typedef void (*scatter_launch_fn)(nxh_context *, const ScatterArgs &, bool);

@@ -13,7 +13,10 @@
 //   scan_lines  anything else (the unit-stride dim is a kept one, or strided
 //               views): one lane per line walks the axis in order, 4 loads in
 //               flight; adjacent lanes own adjacent lines, so accesses coalesce
-//               whenever a kept dim is contiguous.
+//               whenever a kept dim is contiguous. When there are too few lines
+//               to fill the chip the axis is cut into chunks (scan_chunks):
+//               chunk totals, an exclusive scan of the totals per line, then
+//               every chunk is scanned from its carry-in.
 // Float sums and products are reassociated by scan_rows (tolerance-level
 // differences, inside the reference contract's 6x arithmetic tolerance for
 // scans); integer results are exact.
@@ -58,6 +61,53 @@ __global__ __launch_bounds__(FOLD_THREADS) void scan_lines_kernel(ScanArgs a) {
   }
 }
 
+// The chunked form: blockIdx.y is the chunk, `carry` is C[chunks][lines].
+// PHASE 0 writes each chunk's total, PHASE 2 scans each chunk from its carry-in.
+template <int DT, class CB, int PHASE>
+__global__ __launch_bounds__(FOLD_THREADS) void scan_chunks_kernel(ScanArgs a, int64_t chunk, void *carry_v) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  const uint64_t line = (uint64_t)blockIdx.x * FOLD_THREADS + threadIdx.x;
+  if (line >= a.n_lines) return;
+  int64_t in_off, out_off;
+  fold_decode(a.lines, line, in_off, out_off);
+  const int64_t k0 = (int64_t)blockIdx.y * chunk;
+  const int64_t k1 = k0 + chunk < a.len ? k0 + chunk : a.len;
+  const S *p = (const S *)a.in + in_off;
+  S *q = (S *)a.out + out_off;
+  C *carry = (C *)carry_v + (uint64_t)blockIdx.y * a.n_lines + line;
+  C s = PHASE == 0 ? CB::init() : *carry;
+  int64_t k = k0;
+  for (; k + 4 <= k1; k += 4) {
+    S x[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) x[j] = p[(k + j) * a.in_step];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      s = CB::apply(s, TR::ld(x[j]));
+      if (PHASE == 2) q[(k + j) * a.out_step] = TR::st(s);
+    }
+  }
+  for (; k < k1; k++) {
+    s = CB::apply(s, TR::ld(p[k * a.in_step]));
+    if (PHASE == 2) q[k * a.out_step] = TR::st(s);
+  }
+  if (PHASE == 0) *carry = s;
+}
+// Turns the chunk totals of each line into carry-ins (an exclusive scan).
+template <class C, class CB>
+__global__ __launch_bounds__(FOLD_THREADS) void scan_carry_kernel(C *carry, uint64_t n_lines, int chunks) {
+  const uint64_t line = (uint64_t)blockIdx.x * FOLD_THREADS + threadIdx.x;
+  if (line >= n_lines) return;
+  C run = CB::init();
+  for (int c = 0; c < chunks; c++) {
+    const C t = carry[(uint64_t)c * n_lines + line];
+    carry[(uint64_t)c * n_lines + line] = run;
+    run = CB::apply(run, t);
+  }
+}
+
 template <class T>
 __device__ __forceinline__ T shfl_up_any(T v, int delta) {
   constexpr int W = (sizeof(T) + 3) / 4;
@@ -85,9 +135,11 @@ __device__ __forceinline__ T shfl_any(T v, int src) {
   return u.t;
 }
 
-// One wave per line; VEC: lines and chunks are 16-byte aligned.
-template <int DT, class CB, int V, bool VEC>
-__global__ __launch_bounds__(FOLD_THREADS) void scan_rows_kernel(ScanArgs a) {
+// One wave per line (PHASE 1), or per chunk of a line (blockIdx.y; PHASE 0
+// writes the chunk's total to `carry`, PHASE 2 scans the chunk from its
+// carry-in). VEC: lines and chunks are 16-byte aligned.
+template <int DT, class CB, int V, bool VEC, int PHASE>
+__global__ __launch_bounds__(FOLD_THREADS) void scan_rows_kernel(ScanArgs a, int64_t chunk, void *carry_v) {
   using TR = Tr<DT>;
   using S = typename TR::S;
   using C = typename TR::C;
@@ -98,10 +150,13 @@ __global__ __launch_bounds__(FOLD_THREADS) void scan_rows_kernel(ScanArgs a) {
   fold_decode(a.lines, line, in_off, out_off);
   const S *p = (const S *)a.in + in_off;
   S *q = (S *)a.out + out_off;
-  C carry = CB::init();
-  for (int64_t base = 0; base < a.len; base += 64 * V) {
+  const int64_t k0 = PHASE == 1 ? 0 : (int64_t)blockIdx.y * chunk;
+  const int64_t k1 = PHASE == 1 ? a.len : (k0 + chunk < a.len ? k0 + chunk : a.len);
+  C *slot = PHASE == 1 ? nullptr : (C *)carry_v + (uint64_t)blockIdx.y * a.n_lines + line;
+  C carry = PHASE == 2 ? *slot : CB::init();
+  for (int64_t base = k0; base < k1; base += 64 * V) {
     const int64_t e0 = base + (int64_t)lane * V;
-    const int n = (int)(a.len - e0 < V ? (a.len - e0 < 0 ? 0 : a.len - e0) : V);  // this lane's live elements
+    const int n = (int)(k1 - e0 < V ? (k1 - e0 < 0 ? 0 : k1 - e0) : V);  // this lane's live elements
     FVec<S, V> x;
     if (VEC && n == V) {
       x = *reinterpret_cast<const FVec<S, V> *>(p + e0);
@@ -124,20 +179,23 @@ __global__ __launch_bounds__(FOLD_THREADS) void scan_rows_kernel(ScanArgs a) {
       const C up = shfl_up_any(incl, d);
       if (lane >= d) incl = CB::apply(up, incl);
     }
-    C excl = shfl_up_any(incl, 1);
-    excl = lane == 0 ? carry : CB::apply(carry, excl);
-    FVec<S, V> y;
+    if constexpr (PHASE != 0) {
+      C excl = shfl_up_any(incl, 1);
+      excl = lane == 0 ? carry : CB::apply(carry, excl);
+      FVec<S, V> y;
 #pragma unroll
-    for (int j = 0; j < V; j++) y.v[j] = TR::st(CB::apply(excl, r[j]));
-    if (VEC && n == V) {
-      *reinterpret_cast<FVec<S, V> *>(q + e0) = y;
-    } else {
+      for (int j = 0; j < V; j++) y.v[j] = TR::st(CB::apply(excl, r[j]));
+      if (VEC && n == V) {
+        *reinterpret_cast<FVec<S, V> *>(q + e0) = y;
+      } else {
 #pragma unroll
-      for (int j = 0; j < V; j++)
-        if (j < n) q[e0 + j] = y.v[j];
+        for (int j = 0; j < V; j++)
+          if (j < n) q[e0 + j] = y.v[j];
+      }
     }
     carry = CB::apply(carry, shfl_any(incl, 63));
   }
+  if (PHASE == 0 && lane == 0) *slot = carry;
 }
 
 template <int OP, int DT>
@@ -162,14 +220,54 @@ static int scan_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
     bool vec = V > 1 && aligned_to16(a.in) && aligned_to16(a.out);
     for (int i = 0; vec && i < g.nk; i++)
       if (g.kin[i] % V != 0 || g.kout[i] % V != 0) vec = false;
-    nxh_set_path("scan_rows");
-    if (vec) hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, true>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a);
-    else hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, false>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a);
+    const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    // few long lines: a wave per chunk of 64 * V * k elements instead of per line
+    int64_t chunks = std::min<int64_t>(((int64_t)cus * 16 + g.n_out - 1) / g.n_out, a.len / (64 * V * 4));
+    if (chunks >= 2 && chunks <= 65535) {
+      using C = typename TR::C;
+      int64_t chunk = (a.len + chunks - 1) / chunks;
+      chunk = (chunk + 64 * V - 1) / (64 * V) * (64 * V);  // whole wave steps: chunk starts stay aligned
+      chunks = (a.len + chunk - 1) / chunk;
+      Scratch scratch(ctx);
+      int rc = scratch.get(0, (size_t)chunks * g.n_out * sizeof(C));
+      if (rc) return rc;
+      const dim3 grid((unsigned)blocks, (unsigned)chunks);
+      nxh_set_path("scan_rows_chunks");
+      if (vec) hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, true, 0>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
+      else hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, false, 0>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
+      hipLaunchKernelGGL((scan_carry_kernel<C, CB>), dim3((unsigned)((g.n_out + FOLD_THREADS - 1) / FOLD_THREADS)),
+                         dim3(FOLD_THREADS), 0, ctx->stream, (C *)scratch.p[0], (uint64_t)g.n_out, (int)chunks);
+      if (vec) hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, true, 2>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
+      else hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, false, 2>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
+    } else {
+      nxh_set_path("scan_rows");
+      if (vec) hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, true, 1>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a, (int64_t)0, nullptr);
+      else hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, false, 1>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a, (int64_t)0, nullptr);
+    }
   } else {
     const int64_t blocks = (g.n_out + FOLD_THREADS - 1) / FOLD_THREADS;
     if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many lines for one launch");
-    nxh_set_path("scan_lines");
-    hipLaunchKernelGGL((scan_lines_kernel<DT, CB>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a);
+    const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    // too few lines for one lane each to fill the chip: cut the axis into chunks
+    int64_t chunks = std::min<int64_t>(((int64_t)cus * 1024 + g.n_out - 1) / g.n_out, a.len / 16);
+    if (chunks >= 2 && chunks <= 65535) {
+      using C = typename TR::C;
+      int64_t chunk = (a.len + chunks - 1) / chunks;
+      chunk = chunk_off_channel_stride(chunk, a.in_step * (int64_t)sizeof(S));
+      chunks = (a.len + chunk - 1) / chunk;
+      Scratch scratch(ctx);
+      int rc = scratch.get(0, (size_t)chunks * g.n_out * sizeof(C));
+      if (rc) return rc;
+      const dim3 grid((unsigned)blocks, (unsigned)chunks);
+      nxh_set_path("scan_chunks");
+      hipLaunchKernelGGL((scan_chunks_kernel<DT, CB, 0>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
+      hipLaunchKernelGGL((scan_carry_kernel<C, CB>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream,
+                         (C *)scratch.p[0], (uint64_t)g.n_out, (int)chunks);
+      hipLaunchKernelGGL((scan_chunks_kernel<DT, CB, 2>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
+    } else {
+      nxh_set_path("scan_lines");
+      hipLaunchKernelGGL((scan_lines_kernel<DT, CB>), dim3((unsigned)blocks), dim3(FOLD_THREADS), 0, ctx->stream, a);
+    }
   }
   NXH_HIP(op, hipGetLastError());
   return NXH_OK;

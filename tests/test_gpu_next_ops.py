@@ -153,7 +153,7 @@ def test_scan_matches_oracle(hip, oracle, d):
                         assert np.allclose(g, w, rtol=1e-4, atol=1e-4), what
                     else:
                         same_bits(g, w, what)
-    assert hip.last_path() in ("scan_rows", "scan_lines")
+    assert hip.last_path() in ("scan_rows", "scan_lines", "scan_chunks", "scan_rows_chunks")
 
 
 def test_scan_paths_nan_and_reference_vector(hip, oracle):
@@ -177,6 +177,20 @@ def test_scan_paths_nan_and_reference_vector(hip, oracle):
     z = rng.integers(-5, 5, (7, 333)).astype(np.int16)
     hz, oz = pair(z, dt.int16, hip, oracle, lambda B, t: B.shrink(t, [(1, 6), (3, 330)]))
     same_bits(logical(hip.associative_scan(1, "sum", hz)), logical(oracle.associative_scan(1, "sum", oz)))
+    # few long lines: the axis is cut into chunks with carried totals (both forms)
+    w = rng.integers(-9, 9, (3, 70001)).astype(np.int32)
+    hw, ow = pair(w, dt.int32, hip, oracle)
+    same_bits(logical(hip.associative_scan(1, "sum", hw)), logical(oracle.associative_scan(1, "sum", ow)))
+    assert hip.last_path() == "scan_rows_chunks"
+    hw, ow = pair(np.ascontiguousarray(w.T), dt.int32, hip, oracle)
+    same_bits(logical(hip.associative_scan(0, "max", hw)), logical(oracle.associative_scan(0, "max", ow)))
+    assert hip.last_path() == "scan_chunks"
+    f = rng.standard_normal((2, 50000)).astype(np.float32)
+    f[1, 12345] = np.nan
+    hf, of = pair(f, dt.float32, hip, oracle)
+    same_bits(logical(hip.associative_scan(1, "min", hf)), logical(oracle.associative_scan(1, "min", of)))
+    close(logical(hip.associative_scan(1, "sum", hf)), logical(oracle.associative_scan(1, "sum", of)), dt.float32, oracle,
+          6e-5, 6e-5 * 50000, "chunked float cumsum")
     with pytest.raises(RuntimeError):
         hip.associative_scan(0, "sum", mk(hip, np.array([1, 0], np.uint8), dt.bool_))
     with pytest.raises(ValueError):
