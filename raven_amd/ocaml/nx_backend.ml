@@ -97,6 +97,12 @@ external caml_reduce : int -> ('a, 'b) t -> ('a, 'b) t -> int array -> unit = "c
 external caml_argreduce : bool -> (int32, Dtype.int32_elt) t -> ('a, 'b) t -> int -> unit = "caml_nx_hip_argreduce"
 external caml_matmul : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_matmul"
 external caml_gather : ('a, 'b) t -> ('a, 'b) t -> (int32, Dtype.int32_elt) t -> int -> unit = "caml_nx_hip_gather"
+external caml_scatter : ('a, 'b) t -> (int32, Dtype.int32_elt) t -> ('a, 'b) t -> int -> int -> unit = "caml_nx_hip_scatter"
+external caml_pad : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) Nx_buffer.t -> int array -> unit = "caml_nx_hip_pad"
+external caml_cat : ('a, 'b) t -> ('a, 'b) t array -> int -> unit = "caml_nx_hip_cat"
+external caml_scan : int -> ('a, 'b) t -> ('a, 'b) t -> int -> unit = "caml_nx_hip_scan"
+external caml_threefry :
+  (int32, Dtype.int32_elt) t -> (int32, Dtype.int32_elt) t -> (int32, Dtype.int32_elt) t -> unit = "caml_nx_hip_threefry"
 (* ... one external per remaining unary / binary / compare stub, same shapes ... *)
 
 let unary op x = let out = create_tensor x.context x.dtype x.shape in op out x; out
@@ -153,3 +159,41 @@ let matmul x y =
       Int.max (if ai >= 0 then xs.(ai) else 1) (if bi >= 0 then ys.(bi) else 1)) in
   let out = create_tensor x.context x.dtype (Array.append batch [| xs.(xnd - 2); ys.(ynd - 1) |]) in
   caml_matmul out x y; out
+
+(* nx_backend.ml:309-319 of the C backend *)
+let associative_scan ~axis ~op x =
+  let code = match op with `Sum -> 0 | `Prod -> 1 | `Max -> 2 | `Min -> 3 in
+  let out = create_tensor x.context x.dtype x.shape in
+  caml_scan code out x axis; out
+
+(* nx_backend.ml:362-373: the fill value is stored into a 1-element host buffer
+   with the typed Nx_buffer setter (so narrow floats use the buffer layer's
+   converters) and handed to the stub as bytes *)
+let pad x padding fill_value =
+  let out_shape = Array.mapi (fun i d -> let b, a = padding.(i) in d + b + a) x.shape in
+  let out = create_tensor x.context x.dtype out_shape in
+  let fill = Nx_buffer.create x.dtype 1 in
+  Nx_buffer.set fill 0 fill_value;
+  caml_pad out x fill (Array.map fst padding); out
+
+(* nx_backend.ml:379-393 *)
+let cat tensors ~axis =
+  match tensors with
+  | [] -> invalid_arg "cat: empty tensor list"
+  | first :: _ ->
+    let ndim = Array.length first.shape in
+    let axis = if axis < 0 then axis + ndim else axis in
+    let total = List.fold_left (fun acc t -> acc + t.shape.(axis)) 0 tensors in
+    let out = create_tensor first.context first.dtype
+        (Array.mapi (fun i d -> if i = axis then total else d) first.shape) in
+    caml_cat out (Array.of_list tensors) axis; out
+
+(* nx_backend.ml:412-416 *)
+let scatter ~mode ~unique_indices:_ template ~indices ~updates ~axis =
+  let out = copy template in
+  caml_scatter out indices updates axis (match mode with `Set -> 0 | `Add -> 1); out
+
+(* nx_backend.ml:474-477 *)
+let threefry key counter =
+  let out = create_tensor counter.context Dtype.Int32 counter.shape in
+  caml_threefry out key counter; out

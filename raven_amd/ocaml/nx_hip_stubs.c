@@ -32,7 +32,7 @@
   X(context_create) X(context_destroy) X(last_error) X(alloc) X(free)         \
   X(memcpy_h2d) X(memcpy_d2h) X(synchronize) X(fill) X(unary) X(binary)       \
   X(compare) X(where) X(cast) X(reduce) X(argreduce) X(matmul) X(copy)        \
-  X(gather) X(dtype_bytes)
+  X(gather) X(scatter) X(pad) X(cat) X(scan) X(threefry) X(dtype_bytes)
 static struct {
 #define X(n) __typeof__(nxh_##n) *n;
   NXH_SYMBOLS(X)
@@ -270,5 +270,66 @@ CAMLprim value caml_nx_hip_gather(value vout, value vdata, value vidx, value vax
   int rc = L.gather(c, &o, &d, &i, Int_val(vaxis));
   caml_leave_blocking_section();
   check(c, rc);
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_scatter(value vout, value vidx, value vupd, value vaxis, value vmode) {
+  CAMLparam5(vout, vidx, vupd, vaxis, vmode);
+  nxh_tensor o, i, u;
+  nxh_context *c = extract(vout, &o);
+  extract(vidx, &i);
+  extract(vupd, &u);
+  /* waits for the stream to report an out-of-range index from this call */
+  caml_enter_blocking_section();
+  int rc = L.scatter(c, &o, &i, &u, Int_val(vaxis), Int_val(vmode));
+  caml_leave_blocking_section();
+  check(c, rc);
+  CAMLreturn(Val_unit);
+}
+/* the fill value arrives as a 1-element host Nx_buffer, like caml_nx_hip_fill */
+CAMLprim value caml_nx_hip_pad(value vout, value vx, value vfill, value vbefore) {
+  CAMLparam4(vout, vx, vfill, vbefore);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int n = (int)Wosize_val(vbefore);
+  int64_t before[NXH_MAX_NDIM];
+  if (n > NXH_MAX_NDIM) caml_failwith("ndim exceeds NX_C_MAX_NDIM");
+  for (int d = 0; d < n; d++) before[d] = Long_val(Field(vbefore, d));
+  if (n != o.ndim) caml_invalid_argument("pad: shape mismatch");
+  check(c, L.pad(c, &o, &x, Caml_ba_data_val(vfill), before));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_cat(value vout, value vinputs, value vaxis) {
+  CAMLparam3(vout, vinputs, vaxis);
+  nxh_tensor o;
+  nxh_context *c = extract(vout, &o);
+  int n = (int)Wosize_val(vinputs);
+  nxh_tensor *members = (nxh_tensor *)caml_stat_alloc(sizeof(nxh_tensor) * (size_t)(n > 0 ? n : 1));
+  const nxh_tensor **ptrs = (const nxh_tensor **)caml_stat_alloc(sizeof(nxh_tensor *) * (size_t)(n > 0 ? n : 1));
+  for (int m = 0; m < n; m++) {
+    extract(Field(vinputs, m), &members[m]);
+    ptrs[m] = &members[m];
+  }
+  int rc = L.cat(c, &o, ptrs, n, Int_val(vaxis));
+  caml_stat_free(ptrs);
+  caml_stat_free(members);
+  check(c, rc);
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_scan(value vop, value vout, value vx, value vaxis) {
+  CAMLparam4(vop, vout, vx, vaxis);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.scan(c, Int_val(vop), &o, &x, Int_val(vaxis)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_threefry(value vout, value vkey, value vctr) {
+  CAMLparam3(vout, vkey, vctr);
+  nxh_tensor o, k, t;
+  nxh_context *c = extract(vout, &o);
+  extract(vkey, &k);
+  extract(vctr, &t);
+  check(c, L.threefry(c, &o, &k, &t));
   CAMLreturn(Val_unit);
 }

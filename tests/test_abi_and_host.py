@@ -26,7 +26,7 @@ def declared_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _ffi.load()
     names = declared_symbols()
-    assert len(names) >= 26
+    assert len(names) >= 31
     for n in names:
         assert hasattr(lib, n), n
     assert set(names) == set(_ffi.SIGNATURES), set(names) ^ set(_ffi.SIGNATURES)
