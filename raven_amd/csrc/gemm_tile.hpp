@@ -13,7 +13,8 @@
 //                                    by streaming A
 // Common structure: K-slab 64, LDS double-buffered, global -> registers -> LDS
 // with the loads for slab t+2 in flight while slab t is multiplied, one barrier
-// per slab. Inside a slab the work is software-pipelined by hand: the LDS
+// per slab, placed so that the next slab's first fragment reads overlap the
+// current slab's last MFMAs. Inside a slab the work is software-pipelined by hand: the LDS
 // fragment reads of k-step s+1, a share of the register -> LDS stores of slab
 // t+1 and of the global loads of slab t+2 are issued in front of the MFMAs of
 // k-step s (scheduling barriers keep the compiler from regrouping them), so
@@ -283,7 +284,17 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
 
   // One K-slab: multiply slab kt out of LDS; when STAGE, move slab kt+1 from
   // registers to the other LDS stage; when FETCH, start the loads of slab kt+2.
-  // The steady state (both true) is free of branches.
+  // The steady state (both true) is free of branches. The block's one barrier per
+  // slab sits in the LAST k-step, after this wave's share of slab kt+1 has been
+  // written: by then every wave has also issued (and waited for) its last
+  // fragment reads of slab kt, so the next slab's first fragments can be fetched
+  // right behind the barrier, under the MFMAs of the last k-step, and no LDS
+  // latency is exposed at the slab boundary.
+  V16 fa[2][TM], fb[2][TN];
+#pragma unroll
+  for (int t = 0; t < TM; t++) fa[0][t] = frag_load<EL, A_KC, BM>(smem, wm + t * 32, 0, lane);
+#pragma unroll
+  for (int u = 0; u < TN; u++) fb[0][u] = frag_load<EL, B_KC, BN>(smem + A_ELEMS, wn + u * 32, 0, lane);
   auto slab = [&](int kt, auto stage_c, auto fetch_c) {
     constexpr bool STAGE = decltype(stage_c)::value, FETCH = decltype(fetch_c)::value;
     const S *sA = smem + (kt & 1) * STAGE_ELEMS;
@@ -291,22 +302,23 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
     S *nA = smem + ((kt + 1) & 1) * STAGE_ELEMS;
     S *nB = nA + A_ELEMS;
     const S *pA = gA + (int64_t)(kt + 2) * stepA, *pB = gB + (int64_t)(kt + 2) * stepB;
-    V16 fa[2][TM], fb[2][TN];
-#pragma unroll
-    for (int t = 0; t < TM; t++) fa[0][t] = frag_load<EL, A_KC, BM>(sA, wm + t * 32, 0, lane);
-#pragma unroll
-    for (int u = 0; u < TN; u++) fb[0][u] = frag_load<EL, B_KC, BN>(sB, wn + u * 32, 0, lane);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
       const int cur = ks & 1, nxt = cur ^ 1;
+      if constexpr (STAGE) stage_step(ks, nA, nB);
+      if constexpr (FETCH) fetch_step(ks, pA, pB);
       if (ks + 1 < KSTEPS) {
 #pragma unroll
         for (int t = 0; t < TM; t++) fa[nxt][t] = frag_load<EL, A_KC, BM>(sA, wm + t * 32, ks + 1, lane);
 #pragma unroll
         for (int u = 0; u < TN; u++) fb[nxt][u] = frag_load<EL, B_KC, BN>(sB, wn + u * 32, ks + 1, lane);
+      } else if constexpr (STAGE) {
+        __syncthreads();  // slab kt+1 is complete in LDS; nobody reads slab kt's buffer any more
+#pragma unroll
+        for (int t = 0; t < TM; t++) fa[nxt][t] = frag_load<EL, A_KC, BM>(nA, wm + t * 32, 0, lane);
+#pragma unroll
+        for (int u = 0; u < TN; u++) fb[nxt][u] = frag_load<EL, B_KC, BN>(nB, wn + u * 32, 0, lane);
       }
-      if constexpr (STAGE) stage_step(ks, nA, nB);
-      if constexpr (FETCH) fetch_step(ks, pA, pB);
       // keep the order written here (LDS returns in order, so the wait before
       // the first MFMA only covers the current fragments)
       __builtin_amdgcn_sched_barrier(0);
@@ -316,7 +328,6 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
         for (int u = 0; u < TN; u++) mfma_step<EL>(acc[t][u], fa[cur][t], fb[cur][u]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();
   };
   using yes = std::integral_constant<bool, true>;
   using no = std::integral_constant<bool, false>;
