@@ -649,11 +649,13 @@ template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE>
 static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
   auto kern = gemm_tile::kernel<EL, A_KC, B_KC, SH, EDGE>;
   constexpr size_t LDS = SH::template lds_bytes<EL>();
-  static bool configured = false;  // guarded by the context mutex of the caller
-  if (!configured) {
-    NXH_HIP("matmul", hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS));
-    configured = true;
-  }
+  // once per process and kernel (contexts have separate mutexes): allow > 64 KiB of dynamic LDS
+  static std::once_flag once;
+  static hipError_t attr_status = hipSuccess;
+  std::call_once(once, [&] {
+    attr_status = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+  });
+  NXH_HIP("matmul", attr_status);
   g.tiles_m = (uint32_t)((g.M + SH::BM - 1) / SH::BM);
   g.tiles_n = (uint32_t)((g.N + SH::BN - 1) / SH::BN);
   nxh_set_path(path);

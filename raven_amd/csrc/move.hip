@@ -21,7 +21,9 @@
 //
 // pad / cat (nx_c_move.c:203-312) are, as in the reference, compositions of the
 // copy and fill kernels over sub-views of the output: every output element is
-// written once.
+// written once. With a contiguous output row, pad and cat of up to 8 members
+// run as ONE kernel instead (each lane decides where its 16 bytes of output
+// come from).
 //
 // threefry (nx_c_random.c:36-133): Threefry-2x32, 20 rounds, one lane per
 // (key, counter) vector; normative bit for bit.
@@ -363,11 +365,16 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
   a.a_istride = indices->strides[axis];
   a.a_ustride = updates->strides[axis];
   a.fault = ctx->fault_flag;
-  static const scatter_launch_fn table[NXH_DTYPE_COUNT] = {
-#define NXH_SC(DT) [DT] = &scatter_launch<DT>,
+  struct Table {
+    scatter_launch_fn fn[NXH_DTYPE_COUNT] = {};
+    Table() {
+#define NXH_SC(DT) fn[DT] = &scatter_launch<DT>;
       NXH_FOR_COMPUTE_DTYPES(NXH_SC)
 #undef NXH_SC
+    }
   };
+  static const Table table_;
+  const scatter_launch_fn *table = table_.fn;
   if (!table[dt]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
@@ -467,6 +474,115 @@ static bool has_zero_extent(const nxh_tensor *t) {
   return false;
 }
 
+// The fused form: one lane per VP consecutive outputs of a row; each output is
+// either the fill value or the input element `before` positions earlier. Used
+// when rows are contiguous on both sides; the slab composition below covers the
+// rest.
+constexpr int PAD_MAXD = 8;
+struct PadArgs {
+  char *out;
+  const char *in;
+  int ndim;
+  int64_t units;                 // lanes: outputs / VP
+  uint32_t oshape[PAD_MAXD];     // out extents; the last one in units of VP elements
+  int64_t ostride[PAD_MAXD], istride[PAD_MAXD];  // elements (outer dims)
+  int64_t before[PAD_MAXD], ishape[PAD_MAXD];
+  unsigned char fill[16];
+};
+template <class E, int VP>
+__global__ __launch_bounds__(256) void pad_kernel(PadArgs a) {
+  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (u >= a.units) return;
+  int64_t rem = u, oo = 0, io = 0;
+  bool inside = true;
+  int64_t x0 = 0;
+  for (int d = a.ndim - 1; d >= 0; d--) {
+    const int64_t c = rem % a.oshape[d];
+    rem /= a.oshape[d];
+    if (d == a.ndim - 1) {
+      x0 = c * VP;
+      oo += x0;
+    } else {
+      oo += c * a.ostride[d];
+      const int64_t ci = c - a.before[d];
+      inside &= ci >= 0 && ci < a.ishape[d];
+      io += ci * a.istride[d];
+    }
+  }
+  const int last = a.ndim - 1;
+  E fill;
+  __builtin_memcpy(&fill, a.fill, sizeof(E));
+  E v[VP];
+  const int64_t xi = x0 - a.before[last];
+  const E *src = reinterpret_cast<const E *>(a.in) + io + xi;
+  if (inside && xi >= 0 && xi + VP <= a.ishape[last]) {
+    // element-aligned only: the interior is shifted against the input by `before`
+#pragma unroll
+    for (int j = 0; j < VP; j++) v[j] = src[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < VP; j++) v[j] = (inside && xi + j >= 0 && xi + j < a.ishape[last]) ? src[j] : fill;
+  }
+  struct alignas(sizeof(E) * VP >= 16 ? 16 : sizeof(E) * VP) Pack {
+    E v[VP];
+  } pk;
+#pragma unroll
+  for (int j = 0; j < VP; j++) pk.v[j] = v[j];
+  *reinterpret_cast<Pack *>(reinterpret_cast<E *>(a.out) + oo) = pk;
+}
+template <class E>
+static void pad_launch(nxh_context *ctx, const PadArgs &a, int vp) {
+  const dim3 grid((unsigned)((a.units + 255) / 256));
+  constexpr int VMAX = 16 / (int)sizeof(E) > 0 ? 16 / (int)sizeof(E) : 1;
+  if (vp == VMAX && VMAX > 1) hipLaunchKernelGGL((pad_kernel<E, VMAX>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((pad_kernel<E, 1>), grid, dim3(256), 0, ctx->stream, a);
+}
+// Returns -1 when the call does not qualify for the fused kernel.
+static int pad_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *fill_value,
+                     const int64_t *pad_before) {
+  const int nd = out->ndim;
+  if (nd < 1 || nd > PAD_MAXD) return -1;
+  if (out->strides[nd - 1] != 1 || (x->strides[nd - 1] != 1 && x->shape[nd - 1] > 1)) return -1;
+  const int es = (int)nxh_elem_size(out->dtype);
+  int64_t total = 1;
+  for (int d = 0; d < nd; d++) total *= out->shape[d];
+  if (total == 0) return NXH_OK;
+  for (int d = 0; d < nd; d++)
+    if (out->shape[d] > 0xffffffffLL || (d < nd - 1 && out->strides[d] <= 0)) return -1;
+  PadArgs a;
+  a.out = (char *)out->data + out->offset * es;
+  a.in = (const char *)x->data + x->offset * es;
+  a.ndim = nd;
+  const int vmax = 16 / es > 0 ? 16 / es : 1;
+  bool vec = vmax > 1 && out->shape[nd - 1] % vmax == 0 && ((uintptr_t)a.out % 16) == 0;
+  for (int d = 0; d < nd - 1 && vec; d++)
+    if (out->shape[d] > 1 && out->strides[d] % vmax != 0) vec = false;
+  const int vp = vec ? vmax : 1;
+  for (int d = 0; d < nd; d++) {
+    a.oshape[d] = (uint32_t)(d == nd - 1 ? out->shape[d] / vp : out->shape[d]);
+    a.ostride[d] = out->strides[d];
+    a.istride[d] = x->strides[d];
+    a.before[d] = pad_before[d];
+    a.ishape[d] = x->shape[d];
+  }
+  a.units = total / vp;
+  if (a.units > 0x7fffffffLL * 256) return -1;
+  memset(a.fill, 0, sizeof a.fill);
+  memcpy(a.fill, fill_value, (size_t)es);
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP("pad", hipSetDevice(ctx->device));
+  nxh_set_path("pad_fused");
+  switch (es) {
+    case 1: pad_launch<uint8_t>(ctx, a, vp); break;
+    case 2: pad_launch<uint16_t>(ctx, a, vp); break;
+    case 4: pad_launch<uint32_t>(ctx, a, vp); break;
+    case 8: pad_launch<uint64_t>(ctx, a, vp); break;
+    default: pad_launch<G16>(ctx, a, vp); break;
+  }
+  NXH_HIP("pad", hipGetLastError());
+  return NXH_OK;
+}
+
 NXH_EXPORT int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *fill_value,
                        const int64_t *pad_before) {
   const char *op = "pad";
@@ -481,6 +597,10 @@ NXH_EXPORT int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor
   for (int d = 0; d < out->ndim; d++)
     if (pad_before[d] < 0 || out->shape[d] - x->shape[d] - pad_before[d] < 0)
       return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  for (int d = 0; d < out->ndim; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  rc = pad_fused(ctx, out, x, fill_value, pad_before);
+  if (rc != -1) return rc;
   // `slab` narrows toward the interior: entering step d, axes < d carry the
   // interior extent and offset, axes >= d are still full (nx_c_move.c:246-268)
   nxh_tensor slab = *out;
@@ -505,6 +625,128 @@ NXH_EXPORT int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor
   return rc;
 }
 
+// The fused form of cat: one kernel for up to CAT_MAXM members; a lane owns VP
+// consecutive outputs of a row, finds the member its axis coordinate falls in
+// and reads that member through its own strides.
+constexpr int CAT_MAXM = 8;
+struct CatArgs {
+  char *out;
+  const char *in[CAT_MAXM];
+  int ndim, axis, n;
+  uint32_t whole;  // bit m: a lane's VP outputs inside member m are one aligned vector of it
+  int64_t units;
+  uint32_t oshape[PAD_MAXD];  // out extents; the last one in units of VP elements
+  int64_t ostride[PAD_MAXD];
+  int64_t istride[CAT_MAXM][PAD_MAXD];
+  int64_t start[CAT_MAXM + 1];  // first axis coordinate of each member, and the end
+};
+template <class E, int VP>
+__global__ __launch_bounds__(256) void cat_kernel(CatArgs a) {
+  const int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (u >= a.units) return;
+  int64_t coord[PAD_MAXD], rem = u, oo = 0;
+  const int last = a.ndim - 1;
+  for (int d = last; d >= 0; d--) {
+    const int64_t c = rem % a.oshape[d];
+    rem /= a.oshape[d];
+    coord[d] = d == last ? c * VP : c;
+    oo += coord[d] * (d == last ? 1 : a.ostride[d]);
+  }
+  struct alignas(sizeof(E) * VP >= 16 ? 16 : sizeof(E) * VP) Pack {
+    E v[VP];
+  } pk;
+  int m0 = 0;
+  while (m0 + 1 < a.n && coord[a.axis] >= a.start[m0 + 1]) m0++;
+  if (VP == 1 || (a.whole >> m0 & 1)) {
+    // all VP outputs come from VP consecutive, aligned elements of member m0
+    int64_t io = 0;
+    for (int d = 0; d < a.ndim; d++) io += (coord[d] - (d == a.axis ? a.start[m0] : 0)) * a.istride[m0][d];
+    pk = *reinterpret_cast<const Pack *>(reinterpret_cast<const E *>(a.in[m0]) + io);
+  } else {
+#pragma unroll
+    for (int j = 0; j < VP; j++) {
+      const int64_t ax = coord[a.axis] + (a.axis == last ? j : 0);
+      int m = m0;
+      while (m + 1 < a.n && ax >= a.start[m + 1]) m++;
+      int64_t io = 0;
+      for (int d = 0; d < a.ndim; d++) {
+        int64_t c = coord[d] + (d == last ? j : 0);
+        if (d == a.axis) c -= a.start[m];
+        io += c * a.istride[m][d];
+      }
+      pk.v[j] = reinterpret_cast<const E *>(a.in[m])[io];
+    }
+  }
+  *reinterpret_cast<Pack *>(reinterpret_cast<E *>(a.out) + oo) = pk;
+}
+template <class E>
+static void cat_launch(nxh_context *ctx, const CatArgs &a, int vp) {
+  const dim3 grid((unsigned)((a.units + 255) / 256));
+  constexpr int VMAX = 16 / (int)sizeof(E) > 0 ? 16 / (int)sizeof(E) : 1;
+  if (vp == VMAX && VMAX > 1) hipLaunchKernelGGL((cat_kernel<E, VMAX>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((cat_kernel<E, 1>), grid, dim3(256), 0, ctx->stream, a);
+}
+// Returns -1 when the call does not qualify (then the per-member copies run).
+static int cat_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *const *inputs, int n, int axis) {
+  const int nd = out->ndim;
+  if (n < 2 || n > CAT_MAXM || nd < 1 || nd > PAD_MAXD || out->strides[nd - 1] != 1) return -1;
+  const int es = (int)nxh_elem_size(out->dtype);
+  if (es == 0) return -1;
+  int64_t total = 1;
+  for (int d = 0; d < nd; d++) {
+    if (out->shape[d] > 0xffffffffLL || (d < nd - 1 && out->shape[d] > 1 && out->strides[d] <= 0)) return -1;
+    total *= out->shape[d];
+  }
+  if (total == 0) return NXH_OK;
+  CatArgs a;
+  a.out = (char *)out->data + out->offset * es;
+  a.ndim = nd;
+  a.axis = axis;
+  a.n = n;
+  int64_t pos = 0;
+  for (int m = 0; m < n; m++) {
+    a.in[m] = (const char *)inputs[m]->data + inputs[m]->offset * es;
+    a.start[m] = pos;
+    pos += inputs[m]->shape[axis];
+    for (int d = 0; d < nd; d++) a.istride[m][d] = inputs[m]->strides[d];
+  }
+  a.start[n] = pos;
+  if (pos != out->shape[axis]) return -1;
+  const int vmax = 16 / es > 0 ? 16 / es : 1;
+  bool vec = vmax > 1 && out->shape[nd - 1] % vmax == 0 && ((uintptr_t)a.out % 16) == 0;
+  for (int d = 0; d < nd - 1 && vec; d++)
+    if (out->shape[d] > 1 && out->strides[d] % vmax != 0) vec = false;
+  const int vp = vec ? vmax : 1;
+  for (int d = 0; d < nd; d++) {
+    a.oshape[d] = (uint32_t)(d == nd - 1 ? out->shape[d] / vp : out->shape[d]);
+    a.ostride[d] = out->strides[d];
+  }
+  a.units = total / vp;
+  if (a.units > 0x7fffffffLL * 256) return -1;
+  a.whole = 0;
+  for (int m = 0; m < n && vp > 1; m++) {
+    const nxh_tensor *in = inputs[m];
+    bool ok = in->strides[nd - 1] == 1 && ((uintptr_t)a.in[m] % 16) == 0;
+    for (int d = 0; d < nd - 1 && ok; d++)
+      if (in->shape[d] > 1 && in->strides[d] % vp != 0) ok = false;
+    // along the last axis a vector must not straddle two members
+    if (axis == nd - 1 && (a.start[m] % vp != 0 || in->shape[axis] % vp != 0)) ok = false;
+    if (ok) a.whole |= 1u << m;
+  }
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP("cat", hipSetDevice(ctx->device));
+  nxh_set_path("cat_fused");
+  switch (es) {
+    case 1: cat_launch<uint8_t>(ctx, a, vp); break;
+    case 2: cat_launch<uint16_t>(ctx, a, vp); break;
+    case 4: cat_launch<uint32_t>(ctx, a, vp); break;
+    case 8: cat_launch<uint64_t>(ctx, a, vp); break;
+    default: cat_launch<G16>(ctx, a, vp); break;
+  }
+  NXH_HIP("cat", hipGetLastError());
+  return NXH_OK;
+}
+
 NXH_EXPORT int nxh_cat(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *const *inputs, int n_inputs,
                        int axis) {
   const char *op = "cat";
@@ -521,7 +763,17 @@ NXH_EXPORT int nxh_cat(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor
     if (in->dtype != out->dtype) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
     for (int d = 0; d < out->ndim; d++)
       if (d != axis && in->shape[d] != out->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
-    if (pos + in->shape[axis] > out->shape[axis]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    pos += in->shape[axis];
+    if (pos > out->shape[axis]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  }
+  if (nxh_is_packed(out->dtype)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  for (int d = 0; d < out->ndim; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  rc = cat_fused(ctx, out, inputs, n_inputs, axis);
+  if (rc != -1) return rc;
+  pos = 0;
+  for (int m = 0; m < n_inputs; m++) {
+    const nxh_tensor *in = inputs[m];
     nxh_tensor slice = *out;
     slice.offset = out->offset + pos * out->strides[axis];
     for (int d = 0; d < out->ndim; d++) slice.shape[d] = in->shape[d];

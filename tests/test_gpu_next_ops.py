@@ -70,7 +70,7 @@ def test_pad_and_cat_match_oracle(hip, oracle, d):
         fill = np.frombuffer(bytes([1] * d.itemsize), dtype=d.np_storage)[:1] if d is not dt.bool_ else np.array([1], np.uint8)
         for padding in ([(0, 0)] * 3, [(2, 0), (0, 3), (1, 1)], [(0, 1), (4, 4), (0, 0)]):
             same_bits(logical(hip.pad(h, padding, fill)), logical(oracle.pad(o, padding, fill)), f"pad {lname} {padding}")
-        assert hip.last_path() == "pad_slabs"
+        assert hip.last_path() in ("pad_slabs", "pad_fused")
         for axis in (0, 1, 2, -1):
             ax = axis % 3
             lo = [(0, s) for s in SHAPE]
@@ -78,7 +78,7 @@ def test_pad_and_cat_match_oracle(hip, oracle, d):
             members = lambda B, t: [t, B.shrink(t, lo), t]
             same_bits(logical(hip.cat(members(hip, h), axis)), logical(oracle.cat(members(oracle, o), axis)),
                       f"cat {lname} axis {axis}")
-        assert hip.last_path() == "cat_slices"
+        assert hip.last_path() in ("cat_slices", "cat_fused")
     # an empty member contributes nothing; a single member is a copy
     e = np.zeros((5, 0, 14), d.np_storage)
     he, oe = pair(e, d, hip, oracle)
