@@ -17,7 +17,9 @@
 // coordinates off the scatter axis and are visited in ascending axis order, so
 // one lane per off-axis coordinate ("column") walking the axis in order
 // reproduces the serial result exactly, with no atomics and no race: different
-// columns touch disjoint outputs.
+// columns touch disjoint outputs. When the index is the same for every column
+// (indices broadcast off the axis) and the columns alone would not fill the
+// chip, the targets are split over blocks as well (scatter_rows).
 //
 // pad / cat (nx_c_move.c:203-312) are, as in the reference, compositions of the
 // copy and fill kernels over sub-views of the output: every output element is
@@ -299,10 +301,134 @@ __global__ __launch_bounds__(256) void scatter_kernel(ScatterArgs a) {
     apply(out + index * a.a_ostride, upd[i * a.a_ustride]);
   }
 }
-typedef void (*scatter_launch_fn)(nxh_context *, const ScatterArgs &, bool);
+// The index depends on the axis position only (every stride of `indices` off
+// the axis is 0: the embedding-gradient shape). One lane per column leaves most
+// of the chip idle there, so the targets are cut into ranges of `range_rows`
+// output rows as well: block (x, y) owns 256 columns and target range y. The
+// block reads the index list SPAN positions at a time, each lane SCAN of them,
+// and compacts the positions whose target falls in its range into an ordered
+// list in LDS (ballots and popcounts keep the ascending position order). Every
+// lane then applies the listed updates to its own column in that order, eight
+// at a time when their targets are pairwise distinct. Outputs of different
+// blocks are disjoint and each lane sees its column's updates in the serial
+// order, so the result is the reference's.
+template <int DT, bool ADD>
+__global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterArgs a, int64_t range_rows) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  constexpr int SCAN = 8, SPAN = 256 * SCAN, B = 8;
+  __shared__ int s_cnt[4 * SCAN];
+  __shared__ int s_pos[SPAN], s_tgt[SPAN];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const bool live = col < a.columns;
+  if (!live) col = a.columns - 1;  // idle lanes still take part in ballots and barriers
+  int64_t rem = col, oo = 0, uo = 0;
+  for (int d = a.ncol_dims - 1; d >= 0; d--) {
+    const int64_t c = rem % a.cshape[d];
+    rem /= a.cshape[d];
+    oo += c * a.c_ostride[d];
+    uo += c * a.c_ustride[d];
+  }
+  S *out = reinterpret_cast<S *>(a.out) + oo;
+  const S *upd = reinterpret_cast<const S *>(a.upd) + uo;
+  const int64_t lo = (int64_t)blockIdx.y * range_rows, hi = lo + range_rows;
+  auto combine = [](S cur, S u) -> S {
+    if constexpr (ADD) {
+      const C x = TR::ld(cur), y = TR::ld(u);
+      if constexpr (TR::cat == CAT_SINT) return TR::st((C)((uint64_t)x + (uint64_t)y));
+      else return TR::st((C)(x + y));
+    } else {
+      return u;
+    }
+  };
+  for (int64_t base = 0; base < a.n_idx; base += SPAN) {
+    int t[SCAN];  // targets index an axis of the output checked to fit 31 bits
+    bool bad = false;
+#pragma unroll
+    for (int k = 0; k < SCAN; k++) {
+      const int64_t i = base + (wave * SCAN + k) * 64 + lane;
+      int64_t index = i < a.n_idx ? (int64_t)a.idx[i * a.a_istride] : 0;
+      if (index < 0) index += a.axis_len;
+      bad |= index < 0 || index >= a.axis_len;
+      t[k] = (int)index;
+    }
+    // also separates this round's LDS writes from the last round's reads
+    if (__syncthreads_or(bad)) {
+      if (threadIdx.x == 0) atomicOr(a.fault, 1);
+      return;
+    }
+    uint64_t hits[SCAN];
+#pragma unroll
+    for (int k = 0; k < SCAN; k++) {
+      const int64_t i = base + (wave * SCAN + k) * 64 + lane;
+      hits[k] = __ballot(t[k] >= lo && t[k] < hi && i < a.n_idx);
+      if (lane == 0) s_cnt[wave * SCAN + k] = __popcll(hits[k]);
+    }
+    __syncthreads();
+    int off = 0;
+    for (int q = 0; q < wave * SCAN; q++) off += s_cnt[q];
+#pragma unroll
+    for (int k = 0; k < SCAN; k++) {
+      if (hits[k] >> lane & 1) {
+        const int r = off + __popcll(hits[k] & ((1ull << lane) - 1));
+        s_pos[r] = (wave * SCAN + k) * 64 + lane;
+        s_tgt[r] = t[k];
+      }
+      off += __popcll(hits[k]);
+    }
+    __syncthreads();
+    int total = 0;
+    for (int q = 0; q < 4 * SCAN; q++) total += s_cnt[q];
+    if (!live) continue;  // barriers are reached at the top of the next round
+    int m = 0;
+    for (; m + B <= total; m += B) {
+      int tg[B];
+      S u[B];
+#pragma unroll
+      for (int j = 0; j < B; j++) {
+        tg[j] = s_tgt[m + j];
+        u[j] = upd[(base + s_pos[m + j]) * a.a_ustride];
+      }
+      bool distinct = true;
+#pragma unroll
+      for (int j = 1; j < B; j++)
+#pragma unroll
+        for (int k = 0; k < j; k++) distinct &= tg[j] != tg[k];
+      if (distinct) {
+        S cur[B];
+        if constexpr (ADD) {
+#pragma unroll
+          for (int j = 0; j < B; j++) cur[j] = out[(int64_t)tg[j] * a.a_ostride];
+        }
+#pragma unroll
+        for (int j = 0; j < B; j++) out[(int64_t)tg[j] * a.a_ostride] = combine(cur[j], u[j]);
+      } else {
+        for (int j = 0; j < B; j++) {
+          S *o = out + (int64_t)tg[j] * a.a_ostride;
+          *o = combine(*o, u[j]);
+        }
+      }
+    }
+    for (; m < total; m++) {
+      S *o = out + (int64_t)s_tgt[m] * a.a_ostride;
+      *o = combine(*o, upd[(base + s_pos[m]) * a.a_ustride]);
+    }
+  }
+}
+typedef void (*scatter_launch_fn)(nxh_context *, const ScatterArgs &, bool, int64_t);
+// range_rows > 0 selects the kernel that also splits the targets into ranges.
 template <int DT>
-static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add) {
-  const dim3 grid((unsigned)((a.columns + 255) / 256));
+static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add, int64_t range_rows) {
+  const unsigned col_blocks = (unsigned)((a.columns + 255) / 256);
+  if (range_rows > 0) {
+    const dim3 grid(col_blocks, (unsigned)((a.axis_len + range_rows - 1) / range_rows));
+    if (add) hipLaunchKernelGGL((scatter_rows_kernel<DT, true>), grid, dim3(256), 0, ctx->stream, a, range_rows);
+    else hipLaunchKernelGGL((scatter_rows_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, a, range_rows);
+    return;
+  }
+  const dim3 grid(col_blocks);
   if (add) hipLaunchKernelGGL((scatter_kernel<DT, true>), grid, dim3(256), 0, ctx->stream, a);
   else hipLaunchKernelGGL((scatter_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, a);
 }
@@ -378,8 +504,23 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
   if (!table[dt]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
-  nxh_set_path("scatter_columns");
-  table[dt](ctx, a, mode == 1);
+  // Too few columns to fill the chip and one index per axis position: split the
+  // targets over blocks too. The index list is read once per block, so this
+  // pays only while the list is short next to the rows it spreads over.
+  bool uniform_index = a.axis_len <= 0x7fffffffLL;
+  for (int d = 0; d < a.ncol_dims; d++)
+    if (a.cshape[d] > 1 && a.c_istride[d] != 0) uniform_index = false;
+  int64_t range_rows = 0;
+  const int64_t col_blocks = (a.columns + 255) / 256;
+  const int64_t want_blocks = (int64_t)ctx->compute_units * 3;  // measured best on the embedding-gradient shape
+  if (uniform_index && a.n_idx >= 256 && col_blocks * 4 <= want_blocks) {
+    int64_t ranges = want_blocks / col_blocks;
+    if (ranges > a.axis_len) ranges = a.axis_len;
+    if (ranges > 65535) ranges = 65535;
+    if (ranges >= 2) range_rows = (a.axis_len + ranges - 1) / ranges;
+  }
+  nxh_set_path(range_rows > 0 ? "scatter_rows" : "scatter_columns");
+  table[dt](ctx, a, mode == 1, range_rows);
   NXH_HIP(op, hipGetLastError());
   return collect_index_fault(ctx, op);
 }

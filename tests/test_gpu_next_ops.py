@@ -274,6 +274,39 @@ def test_scatter_reference_vectors_and_errors(hip):
         hip.scatter("set", False, t, mk(hip, np.zeros((2, 1), np.int64), dt.int64), mk(hip, np.ones((2, 1)), dt.float64), 1)
 
 
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.int16], ids=lambda d: d.name)
+def test_scatter_one_index_per_position_matches_oracle(hip, oracle, d):
+    """Indices broadcast across the off-axis dims (the embedding-gradient form)
+    take the kernel that also splits the targets over blocks; sums of inexact
+    floats with heavy duplication pin the order of accumulation."""
+    rng = np.random.default_rng(90 + d.tag)
+    for axis, tshape, n in ((0, (301, 70), 2000), (1, (33, 517), 1111), (0, (9, 5), 700)):
+        ishape = list(tshape)
+        ishape[axis] = n
+        ids = rng.integers(-tshape[axis], tshape[axis], n).astype(np.int32)
+        if d.is_float:
+            t = encode(rng.standard_normal(tshape), d, oracle)
+            upd = encode(rng.standard_normal(ishape) * 3, d, oracle)
+        else:
+            t = rng.integers(-30000, 30000, tshape).astype(d.np_storage)
+            upd = rng.integers(-30000, 30000, ishape).astype(d.np_storage)
+        ht, ot = pair(t, d, hip, oracle)
+        hu, ou = pair(upd, d, hip, oracle)
+        line = [1, 1]
+        line[axis] = n
+        hi, oi = (B.expand(B.reshape(B.from_host(ids, dt.int32), tuple(line)), tuple(ishape)) for B in (hip, oracle))
+        for mode in ("set", "add"):
+            same_bits(logical(hip.scatter(mode, False, ht, hi, hu, axis)),
+                      logical(oracle.scatter(mode, False, ot, oi, ou, axis)), f"{mode} axis {axis} {tshape}")
+            assert hip.last_path() == "scatter_rows"
+    bad = ids.copy()
+    bad[n // 2] = tshape[axis]
+    hb = hip.expand(hip.reshape(hip.from_host(bad, dt.int32), tuple(line)), tuple(ishape))
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        hip.scatter("add", False, ht, hb, hu, axis)
+    same_bits(logical(hip.scatter("set", False, ht, hi, hu, axis)), logical(oracle.scatter("set", False, ot, oi, ou, axis)))
+
+
 def test_scatter_add_large_is_a_histogram(hip):
     """The embedding-gradient shape: 65 536 rows of ones scattered by row index
     into a [50257, 64] table equals the histogram of the indices in every column."""
