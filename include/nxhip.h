@@ -221,6 +221,35 @@ int nxh_scan(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *
 int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *key,
                  const nxh_tensor *counter);
 
+/* ── fused sequences of primitives ───────────────────────────────────────── */
+
+/* Each call below equals a fixed sequence of the primitives above, as the
+   reference's frontend and layers issue them, done in one pass over the data
+   with every intermediate rounded to the dtype its primitive would have stored.
+   They have no binding of their own in the reference: a caller that sees the
+   sequence (a deferred-evaluation window in the binding) substitutes the call.
+   Floating dtypes f16/bf16/f32/f64; rows (the last axis) contiguous and at most
+   8192 long, otherwise Failure and the caller issues the primitives. */
+
+/* frontend.ml:4242-4252 softmax over the last axis: max, sub, exp, sum, div.
+   With `scale` (one storage element of x's dtype, host memory) x is first
+   multiplied by it; with `mask` (bool, x's shape, stride-0 broadcast allowed)
+   elements whose mask is 0 are replaced by *masked_value, as the mul and where
+   of kaun/lib/attention.ml:67-110. out may be x's dtype or, for f32 input,
+   f16/bf16 (the cast that follows in attention.ml:105-108). */
+int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+                     const void *scale, const nxh_tensor *mask, const void *masked_value);
+/* kaun/lib/layer_norm.ml:43-68: (x - mean) / sqrt(var + eps) over the last axis
+   (biased variance of the centred values; statistics in float32 for 16-bit
+   dtypes), then * gamma and + beta when given (rank 1, the row length). */
+int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+                        const nxh_tensor *gamma, const nxh_tensor *beta, double eps);
+/* kaun/lib/fn.ml:31-38: ((x * (tanh((x + x*(x*x) * c0) * c1) + c2)) * c3);
+   `constants` = c0..c3 as four storage elements of x's dtype (host memory),
+   the scalars the sequence would have been given. C-contiguous operands. */
+int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+                  const void *constants);
+
 /* ── measurement ─────────────────────────────────────────────────────────── */
 
 /* HIP events recorded on the context stream: start, then stop returns the

@@ -90,6 +90,9 @@ SIGNATURES = {
     "nxh_scan": (C.c_int, [_CTX, C.c_int, _T, _T, C.c_int]),
     "nxh_threefry": (C.c_int, [_CTX, _T, _T, _T]),
     "nxh_gather": (C.c_int, [_CTX, _T, _T, _T, C.c_int]),
+    "nxh_softmax_rows": (C.c_int, [_CTX, _T, _T, C.c_void_p, _T, C.c_void_p]),
+    "nxh_layer_norm_rows": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_double]),
+    "nxh_gelu_tanh": (C.c_int, [_CTX, _T, _T, C.c_void_p]),
     "nxh_timer_start": (C.c_int, [_CTX]),
     "nxh_timer_stop": (C.c_int, [_CTX, _P(C.c_float)]),
     "nxh_last_path": (C.c_char_p, [_CTX]),

@@ -31,7 +31,7 @@ struct ArgCmp {
   // (hipcc 7.2, gfx950, several candidates per lane) to code that never took
   // the update for float candidates.
   __device__ __forceinline__ static void merge(C &bv, int64_t &bi, C v, int64_t i) {
-    const bool take = (i >= 0) & ((bi < 0) | beats(v, bv) | (!beats(bv, v) & (i < bi)));
+    const bool take = (int)(i >= 0) & ((int)(bi < 0) | (int)beats(v, bv) | ((int)!beats(bv, v) & (int)(i < bi)));
     bv = take ? v : bv;
     bi = take ? i : bi;
   }

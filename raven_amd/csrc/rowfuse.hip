@@ -1,0 +1,516 @@
+// rowfuse.hip — three sequences of backend operations that the frontend and
+// Kaun issue one primitive at a time, each as ONE kernel that reads its input
+// once and writes its result once:
+//
+//   nxh_softmax_rows     frontend.ml:4242-4252 (max, sub, exp, sum, div over the
+//                        last axis), optionally behind the scale and mask of
+//                        kaun/lib/attention.ml:67-110 (mul by a scalar, where
+//                        against a scalar) and in front of a cast;
+//   nxh_layer_norm_rows  kaun/lib/layer_norm.ml:43-68 (mean, centre, biased
+//                        variance, divide by sqrt(var + eps); statistics in
+//                        float32 for 16-bit inputs; then * gamma + beta);
+//   nxh_gelu_tanh        kaun/lib/fn.ml:31-38.
+//
+// Every elementwise step is the expression of the corresponding primitive
+// (map_ops.hpp) and is rounded to the dtype that primitive would have stored,
+// so a fused result differs from the op-by-op one only through the order in
+// which a row's sum is added up.
+//
+// Rows live in registers: one wave64 per row up to 2048 elements, one block of
+// four waves up to 8192; longer rows are rejected (the caller then issues the
+// primitives).
+
+#include <cmath>
+
+#include "fold_common.hpp"
+#include "map_ops.hpp"
+
+namespace {
+
+constexpr int ROW_MAXD = 8;
+constexpr int EPL = 32;  // elements per lane at most
+
+struct RowGeom {
+  int64_t rows;
+  int n, nouter;
+  uint32_t oshape[ROW_MAXD];
+};
+struct RowOperand {
+  const char *base;
+  int64_t stride[ROW_MAXD];  // per outer dim, elements
+};
+
+template <int DT>
+__device__ __forceinline__ typename Tr<DT>::C rnd(typename Tr<DT>::C v) {
+  return Tr<DT>::ld(Tr<DT>::st(v));
+}
+
+template <class S, int V>
+struct alignas(sizeof(S) * V) Pk {
+  S v[V];
+};
+
+// Sum / max of one value per lane over the row's lanes; every lane gets the
+// result (the butterfly adds the same two operands on both sides of a pair).
+template <int OP, class C, int RW>
+__device__ __forceinline__ C row_combine(C v, C *lds) {
+  using CB = Combine<OP, C, CAT_FLOAT>;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    C o;
+    if constexpr (sizeof(C) == 8) {
+      const uint64_t u = __builtin_bit_cast(uint64_t, v);
+      const uint32_t lo = __shfl_xor((uint32_t)u, d, 64), hi = __shfl_xor((uint32_t)(u >> 32), d, 64);
+      o = __builtin_bit_cast(C, ((uint64_t)hi << 32) | lo);
+    } else {
+      o = __builtin_bit_cast(C, __shfl_xor(__builtin_bit_cast(uint32_t, v), d, 64));
+    }
+    // operands in lane order on both sides, so a pair computes identical bits
+    const bool low = (threadIdx.x & d) == 0;
+    v = low ? CB::apply(v, o) : CB::apply(o, v);
+  }
+  if constexpr (RW > 1) {
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) lds[w] = v;
+    __syncthreads();
+    v = lds[0];
+#pragma unroll
+    for (int i = 1; i < RW; i++) v = CB::apply(v, lds[i]);
+  }
+  return v;
+}
+
+__device__ __forceinline__ int64_t row_offsets(const RowGeom &g, int64_t row, const RowOperand &a,
+                                               const RowOperand &b, const RowOperand &c, int64_t &ob,
+                                               int64_t &oc) {
+  int64_t oa = 0;
+  ob = 0;
+  oc = 0;
+  for (int d = g.nouter - 1; d >= 0; d--) {
+    const int64_t i = row % g.oshape[d];
+    row /= g.oshape[d];
+    oa += i * a.stride[d];
+    ob += i * b.stride[d];
+    oc += i * c.stride[d];
+  }
+  return oa;
+}
+
+// ── softmax ─────────────────────────────────────────────────────────────────
+struct SoftmaxArgs {
+  RowGeom g;
+  RowOperand x, out, mask;
+  int has_scale, has_mask;
+  int64_t mask_last;  // 0 or 1
+  double scale, masked;  // exact images of the encoded scalars
+};
+template <int DTX, int DTO, int V, int RW>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
+  using TX = Tr<DTX>;
+  using TO = Tr<DTO>;
+  using C = typename TX::C;
+  using SX = typename TX::S;
+  using SO = typename TO::S;
+  constexpr int NV = EPL / V, T = 64 * RW;
+  __shared__ C lds[4];
+  const int tid = RW == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  const int64_t row = RW == 1 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
+  if (row >= a.g.rows) return;  // whole waves (RW == 1) or whole blocks leave together
+  int64_t oo, mo;
+  const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.mask, oo, mo);
+  const SX *x = reinterpret_cast<const SX *>(a.x.base) + xo;
+  SO *out = reinterpret_cast<SO *>(const_cast<char *>(a.out.base)) + oo;
+  const uint8_t *mask = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
+  const int nvec = a.g.n / V;
+  C t[NV][V];
+  Pk<SX, V> raw[NV];
+  Pk<uint8_t, V> mk[NV];
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    const int c = v * T + tid;
+    if (c < nvec) {
+      raw[v] = *reinterpret_cast<const Pk<SX, V> *>(x + (int64_t)c * V);
+      if (a.has_mask) {
+        if (a.mask_last) mk[v] = *reinterpret_cast<const Pk<uint8_t, V> *>(mask + (int64_t)c * V);
+        else
+#pragma unroll
+          for (int j = 0; j < V; j++) mk[v].v[j] = mask[0];
+      }
+    }
+  }
+  const C scale = (C)a.scale, masked = (C)a.masked;
+  C m = Combine<NXH_RMAX, C, CAT_FLOAT>::init();
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    if (v * T + tid < nvec) {
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        C e = TX::ld(raw[v].v[j]);
+        if (a.has_scale) e = rnd<DTX>(OpMul::eval<CAT_FLOAT, C>(e, scale));
+        if (a.has_mask) e = mk[v].v[j] != 0 ? e : masked;
+        t[v][j] = e;
+        m = Combine<NXH_RMAX, C, CAT_FLOAT>::apply(m, e);
+      }
+    }
+  }
+  m = row_combine<NXH_RMAX, C, RW>(m, lds);
+  C s = 0;
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    if (v * T + tid < nvec) {
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        const C d = rnd<DTX>(OpSub::eval<CAT_FLOAT, C>(t[v][j], m));
+        const C e = rnd<DTX>(OpExp::eval<CAT_FLOAT, C>(d));
+        t[v][j] = e;
+        s = s + e;
+      }
+    }
+  }
+  s = rnd<DTX>(row_combine<NXH_SUM, C, RW>(s, lds));
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    const int c = v * T + tid;
+    if (c < nvec) {
+      Pk<SO, V> o;
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        const C y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t[v][j], s));
+        o.v[j] = TO::st((typename TO::C)y);
+      }
+      *reinterpret_cast<Pk<SO, V> *>(out + (int64_t)c * V) = o;
+    }
+  }
+}
+
+// ── layer norm ──────────────────────────────────────────────────────────────
+struct LayerNormArgs {
+  RowGeom g;
+  RowOperand x, out, unused;
+  const char *gamma, *beta;  // null: that step is left out
+  double eps, count;         // exact images of the float scalars the chain would have filled
+};
+template <int DT, int V, int RW>
+__global__ __launch_bounds__(256) void layer_norm_rows_kernel(LayerNormArgs a) {
+  using TX = Tr<DT>;
+  using C = typename TX::C;  // float for the 16-bit dtypes: their float32 island
+  using S = typename TX::S;
+  constexpr int NV = EPL / V, T = 64 * RW;
+  __shared__ C lds[4];
+  const int tid = RW == 1 ? (threadIdx.x & 63) : threadIdx.x;
+  const int64_t row = RW == 1 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
+  if (row >= a.g.rows) return;
+  int64_t oo, uo;
+  const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.unused, oo, uo);
+  const S *x = reinterpret_cast<const S *>(a.x.base) + xo;
+  S *out = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
+  const S *gamma = reinterpret_cast<const S *>(a.gamma), *beta = reinterpret_cast<const S *>(a.beta);
+  const int nvec = a.g.n / V;
+  C t[NV][V];
+  Pk<S, V> raw[NV];
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    const int c = v * T + tid;
+    if (c < nvec) raw[v] = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+  }
+  const C count = (C)a.count, eps = (C)a.eps;
+  C s = 0;
+#pragma unroll
+  for (int v = 0; v < NV; v++)
+    if (v * T + tid < nvec)
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        t[v][j] = TX::ld(raw[v].v[j]);
+        s = s + t[v][j];
+      }
+  const C mu = row_combine<NXH_SUM, C, RW>(s, lds) / count;
+  s = 0;
+#pragma unroll
+  for (int v = 0; v < NV; v++)
+    if (v * T + tid < nvec)
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        t[v][j] = t[v][j] - mu;
+        s = s + t[v][j] * t[v][j];
+      }
+  const C var = row_combine<NXH_SUM, C, RW>(s, lds) / count;
+  const C r = m_sqrt(var + eps);
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    const int c = v * T + tid;
+    if (c < nvec) {
+      Pk<S, V> o, gv, bv;
+      if (gamma) gv = *reinterpret_cast<const Pk<S, V> *>(gamma + (int64_t)c * V);
+      if (beta) bv = *reinterpret_cast<const Pk<S, V> *>(beta + (int64_t)c * V);
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        C y = rnd<DT>(t[v][j] / r);  // leaves the float32 island here
+        if (gamma) y = rnd<DT>(y * TX::ld(gv.v[j]));
+        if (beta) y = rnd<DT>(y + TX::ld(bv.v[j]));
+        o.v[j] = TX::st(y);
+      }
+      *reinterpret_cast<Pk<S, V> *>(out + (int64_t)c * V) = o;
+    }
+  }
+}
+
+// ── gelu (tanh form) ────────────────────────────────────────────────────────
+struct GeluArgs {
+  const char *x;
+  char *out;
+  int64_t n;
+  double c[4];
+};
+template <int DT, int V>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(GeluArgs a) {
+  using TX = Tr<DT>;
+  using C = typename TX::C;
+  using S = typename TX::S;
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+  if (i >= a.n) return;
+  const S *x = reinterpret_cast<const S *>(a.x);
+  S *out = reinterpret_cast<S *>(a.out);
+  Pk<S, V> in, o;
+  if (V > 1 && i + V <= a.n) in = *reinterpret_cast<const Pk<S, V> *>(x + i);
+  else
+#pragma unroll
+    for (int j = 0; j < V; j++) in.v[j] = i + j < a.n ? x[i + j] : S{};
+  const C c0 = (C)a.c[0], c1 = (C)a.c[1], c2 = (C)a.c[2], c3 = (C)a.c[3];
+#pragma unroll
+  for (int j = 0; j < V; j++) {
+    const C v = TX::ld(in.v[j]);
+    const C x2 = rnd<DT>(v * v);
+    const C x3 = rnd<DT>(v * x2);
+    const C p = rnd<DT>(x3 * c0);
+    const C q = rnd<DT>(v + p);
+    const C inner = rnd<DT>(q * c1);
+    const C th = rnd<DT>(m_tanh(inner));
+    const C u = rnd<DT>(th + c2);
+    const C w = rnd<DT>(v * u);
+    o.v[j] = TX::st(w * c3);
+  }
+  if (V > 1 && i + V <= a.n) *reinterpret_cast<Pk<S, V> *>(out + i) = o;
+  else
+#pragma unroll
+    for (int j = 0; j < V; j++)
+      if (i + j < a.n) out[i + j] = o.v[j];
+}
+
+// ── host side ───────────────────────────────────────────────────────────────
+bool float_dtype_ok(int dt) { return dt == NXH_F32 || dt == NXH_F64 || dt == NXH_BF16 || dt == NXH_F16; }
+
+double decode_scalar(int dt, const void *p) {
+  switch (dt) {
+    case NXH_F32: return (double)*(const float *)p;
+    case NXH_F64: return *(const double *)p;
+    case NXH_BF16: return (double)bf16_to_f32(*(const uint16_t *)p);
+    default: {  // NXH_F16, exact by construction
+      const uint16_t h = *(const uint16_t *)p;
+      const int e = (h >> 10) & 31, m = h & 1023;
+      double v = e == 0 ? std::ldexp((double)m, -24)
+                        : (e == 31 ? (m ? std::nan("") : HUGE_VAL) : std::ldexp((double)(m | 1024), e - 25));
+      return (h & 0x8000) ? -v : v;
+    }
+  }
+}
+
+// Fills the row geometry from `x` (rows = product of the outer extents).
+int row_geometry(const char *op, const nxh_tensor *x, RowGeom &g) {
+  if (x->ndim < 1) return nxh_fail(NXH_INVALID_ARGUMENT, op, "input must not be a scalar");
+  if (x->ndim - 1 > ROW_MAXD) return nxh_fail(NXH_FAILURE, op, "more than 8 outer dimensions");
+  if (x->shape[x->ndim - 1] > 64 * 4 * EPL) return nxh_fail(NXH_FAILURE, op, "rows longer than 8192 elements");
+  g.n = (int)x->shape[x->ndim - 1];
+  g.nouter = x->ndim - 1;
+  g.rows = 1;
+  for (int d = 0; d < g.nouter; d++) {
+    if (x->shape[d] > 0xffffffffLL) return nxh_fail(NXH_FAILURE, op, "extent exceeds 32 bits");
+    g.oshape[d] = (uint32_t)x->shape[d];
+    g.rows *= x->shape[d];
+  }
+  return NXH_OK;
+}
+void row_operand(const nxh_tensor *t, RowOperand &o) {
+  o.base = t ? (const char *)t->data + t->offset * (int64_t)nxh_elem_size(t->dtype) : nullptr;
+  for (int d = 0; d < ROW_MAXD; d++) o.stride[d] = (t && d < t->ndim - 1) ? t->strides[d] : 0;
+}
+// A row operand can be moved V elements at a time when its rows are contiguous
+// and every row starts on a V-element boundary.
+bool rows_vector_ok(const nxh_tensor *t, int v) {
+  const int es = (int)nxh_elem_size(t->dtype);
+  if ((((uintptr_t)t->data + t->offset * es) % (uintptr_t)(es * v)) != 0) return false;
+  for (int d = 0; d < t->ndim - 1; d++)
+    if (t->shape[d] > 1 && t->strides[d] % v != 0) return false;
+  return true;
+}
+int same_shape(const char *op, const nxh_tensor *a, const nxh_tensor *b) {
+  if (a->ndim != b->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  for (int d = 0; d < a->ndim; d++)
+    if (a->shape[d] != b->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  return NXH_OK;
+}
+int out_rows_ok(const char *op, const nxh_tensor *out) {
+  for (int d = 0; d < out->ndim; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  return NXH_OK;
+}
+
+template <int DTX, int DTO>
+void softmax_launch(nxh_context *ctx, const SoftmaxArgs &a, bool vec) {
+  const bool wave = a.g.n <= 64 * EPL;
+  const dim3 grid((unsigned)(wave ? (a.g.rows + 3) / 4 : a.g.rows));
+  if (wave && vec) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 1>), grid, dim3(256), 0, ctx->stream, a);
+  else if (wave) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 1, 1>), grid, dim3(256), 0, ctx->stream, a);
+  else if (vec) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 4>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
+}
+template <int DT>
+void layer_norm_launch(nxh_context *ctx, const LayerNormArgs &a, bool vec) {
+  const bool wave = a.g.n <= 64 * EPL;
+  const dim3 grid((unsigned)(wave ? (a.g.rows + 3) / 4 : a.g.rows));
+  if (wave && vec) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 1>), grid, dim3(256), 0, ctx->stream, a);
+  else if (wave) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 1, 1>), grid, dim3(256), 0, ctx->stream, a);
+  else if (vec) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 4>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
+}
+template <int DT>
+void gelu_launch(nxh_context *ctx, const GeluArgs &a, bool vec) {
+  constexpr int V = 16 / (int)sizeof(typename Tr<DT>::S);
+  if (vec) hipLaunchKernelGGL((gelu_tanh_kernel<DT, V>), dim3((unsigned)(((a.n + V - 1) / V + 255) / 256)), dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((gelu_tanh_kernel<DT, 1>), dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, ctx->stream, a);
+}
+
+}  // namespace
+
+NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *scale,
+                                const nxh_tensor *mask, const void *masked_value) {
+  const char *op = "softmax_rows";
+  if (!ctx || !out || !x || (mask && !masked_value)) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (!rc && mask) rc = nxh_check_tensor(op, mask);
+  if (!rc) rc = same_shape(op, out, x);
+  if (!rc && mask) rc = same_shape(op, mask, x);
+  if (!rc) rc = out_rows_ok(op, out);
+  if (rc) return rc;
+  const int dx = x->dtype, dout = out->dtype;
+  if (!float_dtype_ok(dx) || (mask && mask->dtype != NXH_BOOL) ||
+      !(dout == dx || (dx == NXH_F32 && (dout == NXH_BF16 || dout == NXH_F16))))
+    return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  SoftmaxArgs a;
+  if ((rc = row_geometry(op, x, a.g))) return rc;
+  if (a.g.rows == 0) return NXH_OK;
+  if (a.g.n == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_EMPTY_REDUCE);
+  const int nd = x->ndim;
+  if (x->strides[nd - 1] != 1 || out->strides[nd - 1] != 1 ||
+      (mask && mask->strides[nd - 1] != 1 && mask->strides[nd - 1] != 0))
+    return nxh_fail(NXH_FAILURE, op, "rows must be contiguous");
+  if (a.g.rows > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many rows for one launch");
+  row_operand(x, a.x);
+  row_operand(out, a.out);
+  row_operand(mask, a.mask);
+  a.has_scale = scale != nullptr;
+  a.has_mask = mask != nullptr;
+  a.mask_last = mask ? mask->strides[nd - 1] : 0;
+  a.scale = scale ? decode_scalar(dx, scale) : 1.0;
+  a.masked = mask ? decode_scalar(dx, masked_value) : 0.0;
+  const bool vec = a.g.n % 4 == 0 && rows_vector_ok(x, 4) && rows_vector_ok(out, 4) &&
+                   (!mask || a.mask_last == 0 || rows_vector_ok(mask, 4));
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("softmax_rows");
+  if (dx == NXH_F32 && dout == NXH_F32) softmax_launch<NXH_F32, NXH_F32>(ctx, a, vec);
+  else if (dx == NXH_F32 && dout == NXH_BF16) softmax_launch<NXH_F32, NXH_BF16>(ctx, a, vec);
+  else if (dx == NXH_F32) softmax_launch<NXH_F32, NXH_F16>(ctx, a, vec);
+  else if (dx == NXH_BF16) softmax_launch<NXH_BF16, NXH_BF16>(ctx, a, vec);
+  else if (dx == NXH_F16) softmax_launch<NXH_F16, NXH_F16>(ctx, a, vec);
+  else softmax_launch<NXH_F64, NXH_F64>(ctx, a, vec);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+                                   const nxh_tensor *gamma, const nxh_tensor *beta, double eps) {
+  const char *op = "layer_norm_rows";
+  if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (!rc && gamma) rc = nxh_check_tensor(op, gamma);
+  if (!rc && beta) rc = nxh_check_tensor(op, beta);
+  if (!rc) rc = same_shape(op, out, x);
+  if (!rc) rc = out_rows_ok(op, out);
+  if (rc) return rc;
+  if (!(eps >= 0.0)) return nxh_fail(NXH_INVALID_ARGUMENT, op, "eps must be >= 0");
+  const int dx = x->dtype;
+  if (!float_dtype_ok(dx) || out->dtype != dx || (gamma && gamma->dtype != dx) || (beta && beta->dtype != dx))
+    return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  LayerNormArgs a;
+  if ((rc = row_geometry(op, x, a.g))) return rc;
+  for (const nxh_tensor *p : {gamma, beta})
+    if (p && (p->ndim != 1 || p->shape[0] != a.g.n)) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  if (a.g.rows == 0) return NXH_OK;
+  if (a.g.n == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_EMPTY_REDUCE);
+  const int nd = x->ndim;
+  if (x->strides[nd - 1] != 1 || out->strides[nd - 1] != 1 || (gamma && a.g.n > 1 && gamma->strides[0] != 1) ||
+      (beta && a.g.n > 1 && beta->strides[0] != 1))
+    return nxh_fail(NXH_FAILURE, op, "rows must be contiguous");
+  if (a.g.rows > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many rows for one launch");
+  row_operand(x, a.x);
+  row_operand(out, a.out);
+  row_operand(nullptr, a.unused);
+  const int es = (int)nxh_elem_size(dx);
+  a.gamma = gamma ? (const char *)gamma->data + gamma->offset * es : nullptr;
+  a.beta = beta ? (const char *)beta->data + beta->offset * es : nullptr;
+  // the scalars the primitives would have been given: eps and the row length
+  // filled into the statistics dtype (float32 for 16-bit inputs)
+  a.eps = dx == NXH_F64 ? eps : (double)(float)eps;
+  a.count = dx == NXH_F64 ? (double)a.g.n : (double)(float)a.g.n;
+  const bool vec = a.g.n % 4 == 0 && rows_vector_ok(x, 4) && rows_vector_ok(out, 4) &&
+                   (!gamma || ((uintptr_t)a.gamma % (es * 4)) == 0) && (!beta || ((uintptr_t)a.beta % (es * 4)) == 0);
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("layer_norm_rows");
+  if (dx == NXH_F32) layer_norm_launch<NXH_F32>(ctx, a, vec);
+  else if (dx == NXH_BF16) layer_norm_launch<NXH_BF16>(ctx, a, vec);
+  else if (dx == NXH_F16) layer_norm_launch<NXH_F16>(ctx, a, vec);
+  else layer_norm_launch<NXH_F64>(ctx, a, vec);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+NXH_EXPORT int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *constants) {
+  const char *op = "gelu_tanh";
+  if (!ctx || !out || !x || !constants) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (!rc) rc = same_shape(op, out, x);
+  if (rc) return rc;
+  const int dx = x->dtype;
+  if (!float_dtype_ok(dx) || out->dtype != dx) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  int64_t n = 1, expect = 1;
+  bool dense = x->offset >= 0;
+  for (int d = x->ndim - 1; d >= 0; d--) {
+    if (x->shape[d] > 1 && (x->strides[d] != expect || out->strides[d] != expect)) dense = false;
+    expect *= x->shape[d];
+    n *= x->shape[d];
+  }
+  if (!dense) return nxh_fail(NXH_FAILURE, op, "operands must be C-contiguous");
+  if (n == 0) return NXH_OK;
+  const int es = (int)nxh_elem_size(dx);
+  GeluArgs a;
+  a.x = (const char *)x->data + x->offset * es;
+  a.out = (char *)out->data + out->offset * es;
+  a.n = n;
+  for (int i = 0; i < 4; i++) a.c[i] = decode_scalar(dx, (const char *)constants + i * es);
+  if (n / 256 > 0x7ffffff0LL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  const bool vec = ((uintptr_t)a.x % 16) == 0 && ((uintptr_t)a.out % 16) == 0;
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("gelu_tanh");
+  if (dx == NXH_F32) gelu_launch<NXH_F32>(ctx, a, vec);
+  else if (dx == NXH_BF16) gelu_launch<NXH_BF16>(ctx, a, vec);
+  else if (dx == NXH_F16) gelu_launch<NXH_F16>(ctx, a, vec);
+  else gelu_launch<NXH_F64>(ctx, a, vec);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}

@@ -315,6 +315,51 @@ class Backend:
         self._check(self._lib.nxh_threefry(self._h, C.byref(o), C.byref(k), C.byref(c)))
         return out
 
+    # ── fused sequences of primitives (no counterpart in Backend_intf.S) ────
+    def _scalar_arg(self, dtype: dt.DType, value):
+        if value is None:
+            return None, None
+        enc = value if isinstance(value, np.ndarray) else encode_scalar(dtype, value)
+        enc = np.ascontiguousarray(enc.reshape(-1))
+        return enc, enc.ctypes.data
+
+    def softmax_rows(self, x: Tensor, scale=None, mask: Tensor | None = None, masked_value=None,
+                     out_dtype: dt.DType | None = None) -> Tensor:
+        """softmax over the last axis of ``x * scale`` with masked-out elements
+        replaced by ``masked_value`` first, optionally cast: the sequence mul,
+        where, max, sub, exp, sum, div, cast in one kernel. Scalars are Python
+        numbers or already-encoded storage elements."""
+        out = self.buffer(out_dtype or x.dtype, x.shape)
+        keep_s, ps = self._scalar_arg(x.dtype, scale)
+        keep_m, pm = self._scalar_arg(x.dtype, masked_value)
+        o, a = out._desc(), x._desc()
+        m = mask._desc() if mask is not None else None
+        self._check(self._lib.nxh_softmax_rows(self._h, C.byref(o), C.byref(a), ps,
+                                               C.byref(m) if m is not None else None, pm))
+        return out
+
+    def layer_norm_rows(self, x: Tensor, gamma: Tensor | None, beta: Tensor | None, eps: float) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        g = gamma._desc() if gamma is not None else None
+        b = beta._desc() if beta is not None else None
+        self._check(self._lib.nxh_layer_norm_rows(self._h, C.byref(o), C.byref(a),
+                                                  C.byref(g) if g is not None else None,
+                                                  C.byref(b) if b is not None else None, float(eps)))
+        return out
+
+    def gelu_tanh(self, x: Tensor, constants=(0.044715, 0.7978845608028654, 1.0, 0.5)) -> Tensor:
+        """``constants`` are four Python numbers or one array of four encoded
+        storage elements."""
+        out = self.buffer(x.dtype, x.shape)
+        if isinstance(constants, np.ndarray):
+            enc = np.ascontiguousarray(constants.reshape(4))
+        else:
+            enc = np.concatenate([encode_scalar(x.dtype, c) for c in constants])
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_gelu_tanh(self._h, C.byref(o), C.byref(a), enc.ctypes.data))
+        return out
+
     # ── fold family (nx_backend.ml:266-307) ─────────────────────────────────
     def reduce(self, op: str, axes: Sequence[int], x: Tensor) -> Tensor:
         axes = sorted(int(a) for a in axes)

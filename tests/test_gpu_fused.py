@@ -1,0 +1,174 @@
+"""The fused row kernels (softmax_rows, layer_norm_rows, gelu_tanh) through the
+C ABI against the op-by-op sequences they stand for.
+
+Two references per case: the sequence of primitives on the CPU oracle (the
+reference's lowering, frontend.ml:4242-4252, kaun/lib/{layer_norm,fn,attention}.ml)
+and the same sequence on the GPU backend. Elementwise steps are the same
+expressions with the same rounding points, so against the GPU sequence only the
+order of a row's sum can differ: a few ulp of the result dtype. gelu has no sum
+and must equal the GPU sequence bit for bit."""
+
+import numpy as np
+import pytest
+
+from helpers import TOL, close, decode, encode, logical, pair, same_bits
+from raven_amd import dtype as dt
+from raven_amd.kaun_gpt2 import Config, Gpt2, LayerNorm
+from raven_amd.nx_frontend import Nx
+
+pytestmark = pytest.mark.gpu
+
+ULP = {"float64": 2.0 ** -52, "float32": 2.0 ** -23, "float16": 2.0 ** -10, "bfloat16": 2.0 ** -7}
+FLOATS = [dt.float32, dt.bfloat16, dt.float16, dt.float64]
+
+
+def within_ulps(got, want, d, oracle, n, what=""):
+    """|got - want| <= n ulp of dtype d at the magnitude of want (+ the smallest
+    normal as absolute slack for results that round to zero)."""
+    close(got, want, d, oracle, n * ULP[d.name], 1e-37 if d is not dt.float16 else 1e-7, what)
+
+
+def softmax_sequence(B, x, scale, mask, out_dtype):
+    """attention.ml:93-108: scale, mask against -inf, softmax, cast."""
+    nx = Nx(B)
+    t = x
+    if scale is not None:
+        t = nx.mul_s(t, scale)
+    if mask is not None:
+        t = nx.where(mask, t, nx.scalar_like(t, float("-inf")))
+    t = nx.softmax(t)
+    return nx.cast(out_dtype, t) if out_dtype is not None else t
+
+
+@pytest.mark.parametrize("d", FLOATS, ids=lambda d: d.name)
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (5, 770), (3, 2050), (2, 4100), (1, 8192), (4, 1)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_softmax_rows_matches_the_sequence(hip, oracle, d, shape):
+    rng = np.random.default_rng(sum(shape) + d.tag)
+    x = encode(rng.standard_normal(shape) * 4, d, oracle)
+    hx, ox = pair(x, d, hip, oracle)
+    for scale, masked, cast in ((None, False, None), (0.125, True, None),
+                                (0.125, True, dt.bfloat16 if d is dt.float32 else None),
+                                (None, False, dt.float16 if d is dt.float32 else None)):
+        hm = om = None
+        if masked:
+            n = shape[-1]
+            tri = np.tril(np.ones((shape[-2], n), np.uint8), k=max(0, n - shape[-2]))
+            hm, om = (B.expand(B.reshape(B.from_host(tri, dt.bool_), (1,) * (len(shape) - 2) + tri.shape), shape)
+                      for B in (hip, oracle))
+        got = hip.softmax_rows(hx, scale, hm, float("-inf") if masked else None, cast)
+        assert hip.last_path() == "softmax_rows"
+        od = cast or d
+        want_cpu = logical(softmax_sequence(oracle, ox, scale, om, cast))
+        want_gpu = logical(softmax_sequence(hip, hx, scale, hm, cast))
+        what = f"{d.name} {shape} scale={scale} mask={masked} cast={cast and cast.name}"
+        within_ulps(logical(got), want_gpu, od, oracle, 4 if od.itemsize == 2 else 16, what + " vs GPU sequence")
+        close(logical(got), want_cpu, od, oracle, TOL[od.name][1], 1e-30, what + " vs oracle sequence")
+        rows = decode(logical(got), od, oracle).sum(-1)
+        assert np.all(np.abs(rows - 1) <= 8 * shape[-1] ** 0.5 * ULP[od.name] + 1e-6)
+
+
+def test_softmax_rows_special_values_and_errors(hip, oracle):
+    x = np.zeros((6, 8), np.float32)
+    x[0] = np.arange(8)
+    x[1, 3] = np.nan              # a NaN poisons its row (max keeps NaN)
+    x[2] = -np.inf                # exp(-inf - -inf) = NaN
+    x[3, 2] = np.inf              # inf - inf = NaN at that element, 0 elsewhere
+    x[4] = 1e30
+    mask = np.ones((6, 8), np.uint8)
+    mask[5] = 0                   # fully masked row: -inf everywhere
+    hx, ox = pair(x, dt.float32, hip, oracle)
+    hm, om = pair(mask, dt.bool_, hip, oracle)
+    got = logical(hip.softmax_rows(hx, None, hm, float("-inf")))
+    want = logical(softmax_sequence(oracle, ox, None, om, None))
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.allclose(got[~np.isnan(got)], want[~np.isnan(want)], rtol=1e-6)
+    assert np.isnan(got[1]).all() and np.isnan(got[2]).all() and np.isnan(got[5]).all()
+    # a masked value other than -inf, taken as given
+    got = logical(hip.softmax_rows(hx, 2.0, hm, -1e4))
+    nx = Nx(oracle)
+    want = logical(nx.softmax(nx.where(om, nx.mul_s(ox, 2.0), nx.scalar_like(ox, -1e4))))
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.allclose(got[~np.isnan(got)], want[~np.isnan(want)], rtol=1e-6)
+    with pytest.raises(RuntimeError, match="8192"):
+        hip.softmax_rows(hip.full(dt.float32, (2, 8200), 0.0))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hip.softmax_rows(hip.permute(hx, (1, 0)))
+    with pytest.raises(RuntimeError):
+        hip.softmax_rows(hip.full(dt.int32, (2, 8), 1))
+    with pytest.raises(ValueError):
+        hip.softmax_rows(hx, None, hip.full(dt.bool_, (6, 4), 1), 0.0)
+    # strided rows (a column slice of a wider tensor) and an empty tensor
+    wide = np.random.default_rng(5).standard_normal((9, 40)).astype(np.float32)
+    hw, ow = pair(wide, dt.float32, hip, oracle, lambda B, t: B.shrink(t, [(0, 9), (3, 35)]))
+    within_ulps(logical(hip.softmax_rows(hw)), logical(Nx(oracle).softmax(ow)), dt.float32, oracle, 16)
+    assert logical(hip.softmax_rows(hip.full(dt.float32, (0, 8), 0.0))).shape == (0, 8)
+
+
+@pytest.mark.parametrize("d", FLOATS, ids=lambda d: d.name)
+@pytest.mark.parametrize("shape", [(4, 33, 768), (7, 770), (3, 4100), (5, 1)], ids=lambda s: "x".join(map(str, s)))
+def test_layer_norm_rows_matches_the_sequence(hip, oracle, d, shape):
+    rng = np.random.default_rng(sum(shape) + 7 * d.tag)
+    n = shape[-1]
+    x = encode(rng.standard_normal(shape) * 2 + 3, d, oracle)
+    gamma = encode(rng.standard_normal(n) * 0.5 + 1, d, oracle)
+    beta = encode(rng.standard_normal(n) * 0.1, d, oracle)
+    hx, ox = pair(x, d, hip, oracle)
+    hg, og = pair(gamma, d, hip, oracle)
+    hb, ob = pair(beta, d, hip, oracle)
+    eps = 1e-5
+    got = hip.layer_norm_rows(hx, hg, hb, eps)
+    assert hip.last_path() == "layer_norm_rows"
+    cfg = Config()
+    want_cpu = logical(Gpt2(Nx(oracle), cfg).layer_norm(LayerNorm(og, ob), ox, eps))
+    want_gpu = logical(Gpt2(Nx(hip), cfg).layer_norm(LayerNorm(hg, hb), hx, eps))
+    what = f"{d.name} {shape}"
+    # the mean and variance carry the sum-order difference into every element:
+    # a few ulp of float32 in the statistics, at most one rounding step of d
+    close(logical(got), want_gpu, d, oracle, 2 * ULP[d.name] + 1e-5, 1e-5, what + " vs GPU sequence")
+    close(logical(got), want_cpu, d, oracle, TOL[d.name][0], TOL[d.name][0], what + " vs oracle sequence")
+    if d in (dt.bfloat16, dt.float16) and n > 1:
+        frac = np.mean(logical(got) == want_gpu)
+        assert frac > 0.98, (what, frac)
+    # without the affine step: the normalisation alone (layer_norm.ml:43-49)
+    got = logical(hip.layer_norm_rows(hx, None, None, eps))
+    ones, zeros = (encode(np.full(n, v), d, oracle) for v in (1.0, 0.0))
+    og1, ob0 = pair(ones, d, oracle, oracle)[0], pair(zeros, d, oracle, oracle)[0]
+    want = logical(Gpt2(Nx(oracle), cfg).layer_norm(LayerNorm(og1, ob0), ox, eps))
+    close(got, want, d, oracle, TOL[d.name][0], TOL[d.name][0], what + " plain")
+
+
+def test_layer_norm_rows_errors(hip):
+    x = hip.full(dt.float32, (4, 8), 1.0)
+    with pytest.raises(ValueError):
+        hip.layer_norm_rows(x, hip.full(dt.float32, (7,), 1.0), None, 1e-5)
+    with pytest.raises(ValueError, match="eps"):
+        hip.layer_norm_rows(x, None, None, -1.0)
+    with pytest.raises(RuntimeError):
+        hip.layer_norm_rows(x, hip.full(dt.float64, (8,), 1.0), None, 1e-5)
+    with pytest.raises(RuntimeError, match="8192"):
+        hip.layer_norm_rows(hip.full(dt.float32, (1, 9000), 1.0), None, None, 1e-5)
+    # a constant row has zero variance: 0 / sqrt(eps) = 0
+    assert np.array_equal(logical(hip.layer_norm_rows(x, None, None, 1e-5)), np.zeros((4, 8), np.float32))
+
+
+@pytest.mark.parametrize("d", FLOATS, ids=lambda d: d.name)
+def test_gelu_tanh_equals_the_sequence(hip, oracle, d):
+    rng = np.random.default_rng(300 + d.tag)
+    for shape in ((8, 3072), (1001,), (3, 5, 7)):
+        v = rng.standard_normal(shape) * 3
+        v.reshape(-1)[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, 60.0]
+        x = encode(v, d, oracle)
+        hx, ox = pair(x, d, hip, oracle)
+        got = logical(hip.gelu_tanh(hx))
+        assert hip.last_path() == "gelu_tanh"
+        cfg = Config()
+        want_gpu = logical(Gpt2(Nx(hip), cfg).gelu_approx(hx))
+        nan = np.isnan(decode(want_gpu, d, oracle))
+        assert np.array_equal(np.isnan(decode(got, d, oracle)), nan)
+        same_bits(np.where(nan, np.zeros_like(got), got), np.where(nan, np.zeros_like(got), want_gpu),
+                  f"{d.name} {shape}")
+        want_cpu = logical(Gpt2(Nx(oracle), cfg).gelu_approx(ox))
+        close(got, want_cpu, d, oracle, TOL[d.name][1], TOL[d.name][1], f"{d.name} {shape} vs oracle sequence")
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hip.gelu_tanh(hip.permute(hip.full(d, (3, 4), 1.0), (1, 0)))
