@@ -316,7 +316,7 @@ class CountingBackend:
     """Forwards to the backend and counts the calls that launch work."""
 
     LAUNCHING = ("unary", "binary", "compare", "where", "cast", "copy", "contiguous", "gather", "reduce",
-                 "matmul", "full", "from_host")
+                 "matmul", "full", "from_host", "softmax_rows", "layer_norm_rows", "gelu_tanh")
 
     def __init__(self, inner):
         self._inner, self.calls = inner, {}
@@ -333,11 +333,15 @@ class CountingBackend:
         return counted
 
 
-def config5(hip, iters=3, warmup=1):
-    """GPT-2-small-shaped eager forward (12 layers, d 768, 12 heads, FFN 3072,
-    vocab 50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s."""
+def config5(hip, iters=3, warmup=1, window=False):
+    """GPT-2-small-shaped forward (12 layers, d 768, 12 heads, FFN 3072, vocab
+    50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s. Eager: one
+    backend call per primitive. With ``window``: the same frontend calls go
+    through the deferred-evaluation window, which replaces the softmax, layer
+    norm and GELU sequences by the fused row kernels."""
     from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
     from raven_amd.nx_frontend import Nx
+    from raven_amd.nx_window import Window
 
     cfg = Config.small()
     batch, seq = 8, 1024
@@ -347,7 +351,8 @@ def config5(hip, iters=3, warmup=1):
         return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
     counter = CountingBackend(hip)
-    nx = Nx(counter)
+    front = Window(counter) if window else counter
+    nx = Nx(front)
     params = upload(nx, host_params(cfg, seed=16), dt.bfloat16, enc)
     ids = nx.create(dt.int32, (batch, seq),
                     np.random.default_rng(17).integers(0, cfg.vocab_size, (batch, seq)).astype(np.int32))
@@ -355,23 +360,25 @@ def config5(hip, iters=3, warmup=1):
     for _ in range(warmup):
         out = model.logits(params, ids)
         del out
-    hip.synchronize()
+    front.synchronize()
     counter.calls.clear()
     t0 = time.perf_counter()
-    hip.timer_start()
+    front.timer_start()
     for _ in range(iters):
         out = model.logits(params, ids)
         del out
-    ev_ms = hip.timer_stop() / iters
-    hip.synchronize()
+    ev_ms = front.timer_stop() / iters
+    front.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / iters
     calls = {k: v // iters for k, v in counter.calls.items()}
     flops = 284812800 * batch * seq  # matmul FLOPs per forward
-    rec = {"op": "cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 (eager, one backend call per primitive)",
+    how = ("deferred-evaluation window: softmax / layer norm / GELU sequences as fused row kernels" if window
+           else "eager, one backend call per primitive")
+    rec = {"op": f"cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 ({how})",
            "ms": round(ms, 3), "tokens/s": round(batch * seq / (ms * 1e-3), 1), "hip_event_ms": round(ev_ms, 3),
            "matmul_TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1), "backend_calls": sum(calls.values()),
            "calls_by_kind": calls}
-    del params, ids, model
+    del params, ids, model, nx, front
     hip.trim()
     return rec
 
@@ -398,6 +405,7 @@ def main():
     info = hip.device_info()
     if args.only_gpt2:
         print(json.dumps(config5(hip)))
+        print(json.dumps(config5(hip, window=True)))
         return
     if args.only_next:
         print(json.dumps({"ops": next_ops(hip, Workloads(hip))}))
@@ -475,6 +483,7 @@ def main():
             W.keep.clear()
             hip.trim()
         ops_out.append(config5(hip))
+        ops_out.append(config5(hip, window=True))
         ops_out.extend(next_ops(hip, W))
 
     line = {

@@ -139,6 +139,9 @@ class OracleBackend:
     def _mv(self, t, v):
         return OTensor(t.storage, v, t.dtype)
 
+    def with_view(self, t, v):
+        return OTensor(t.storage, v, t.dtype)
+
     def expand(self, t, shape):
         return self._mv(t, t.view.expand(shape))
 

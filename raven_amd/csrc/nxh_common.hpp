@@ -39,6 +39,15 @@ struct nxh_context {
   // one device word, written by kernels that detect a data fault (gather OOB)
   int *fault_flag = nullptr;       // device
   int *fault_flag_host = nullptr;  // pinned host mirror for the readback
+  // pinned staging slots for small host-to-device uploads: the caller's bytes
+  // are copied into a slot and the transfer is queued on the stream, so an
+  // upload does not wait for the work already queued
+  static constexpr int STAGE_SLOTS = 16;
+  static constexpr size_t STAGE_BYTES = (size_t)256 << 10;
+  char *stage = nullptr;  // STAGE_SLOTS * STAGE_BYTES
+  hipEvent_t stage_done[STAGE_SLOTS] = {};
+  bool stage_used[STAGE_SLOTS] = {};
+  int stage_next = 0;
 };
 
 // thread-local status text (static strings + op prefix)

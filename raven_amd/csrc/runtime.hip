@@ -63,6 +63,10 @@ NXH_EXPORT int nxh_context_create(nxh_context **out) {
   if (e == hipSuccess) e = hipEventCreate(&ctx->ev_stop);
   if (e == hipSuccess) e = hipMalloc((void **)&ctx->fault_flag, 256);
   if (e == hipSuccess) e = hipHostMalloc((void **)&ctx->fault_flag_host, 256, hipHostMallocDefault);
+  if (e == hipSuccess)
+    e = hipHostMalloc((void **)&ctx->stage, nxh_context::STAGE_SLOTS * nxh_context::STAGE_BYTES, hipHostMallocDefault);
+  for (int i = 0; i < nxh_context::STAGE_SLOTS && e == hipSuccess; i++)
+    e = hipEventCreateWithFlags(&ctx->stage_done[i], hipEventDisableTiming);
   if (e == hipSuccess) e = hipMemsetAsync(ctx->fault_flag, 0, 256, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
   if (e != hipSuccess) {
@@ -80,6 +84,9 @@ NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   for (auto &kv : ctx->live) (void)hipFree(kv.first);
   if (ctx->fault_flag) (void)hipFree(ctx->fault_flag);
   if (ctx->fault_flag_host) (void)hipHostFree(ctx->fault_flag_host);
+  if (ctx->stage) (void)hipHostFree(ctx->stage);
+  for (hipEvent_t ev : ctx->stage_done)
+    if (ev) (void)hipEventDestroy(ev);
   if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
   if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
   if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -209,14 +216,28 @@ NXH_EXPORT int nxh_memory_stats(nxh_context *ctx, uint64_t *in_use, uint64_t *ca
 
 // ── transfer ───────────────────────────────────────────────────────────────
 // from_host must not return before the caller's buffer has been read: the
-// frontend fills a temporary and drops it (frontend.ml:347-351). hipMemcpyAsync
-// from pageable memory stages the data before returning; the explicit wait
-// makes that hold for pinned sources too.
+// frontend fills a temporary and drops it (frontend.ml:347-351). Uploads of up
+// to 256 KiB (index vectors, aranges, scalars) are copied into a pinned slot
+// of the context and queued, so they do not drain the stream; larger ones are
+// queued from the caller's buffer and waited for.
 NXH_EXPORT int nxh_memcpy_h2d(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "from_host", "null context");
   if (bytes == 0) return NXH_OK;
   std::lock_guard<std::mutex> g(ctx->mu);
   NXH_HIP("from_host", hipSetDevice(ctx->device));
+  if (bytes <= nxh_context::STAGE_BYTES) {
+    // small upload: through a pinned slot, in stream order, without waiting
+    // for the stream. A slot is reused only after its last transfer finished.
+    const int slot = ctx->stage_next;
+    ctx->stage_next = (slot + 1) % nxh_context::STAGE_SLOTS;
+    if (ctx->stage_used[slot]) NXH_HIP("from_host", hipEventSynchronize(ctx->stage_done[slot]));
+    char *staged = ctx->stage + (size_t)slot * nxh_context::STAGE_BYTES;
+    memcpy(staged, src, bytes);
+    NXH_HIP("from_host", hipMemcpyAsync(dst, staged, bytes, hipMemcpyHostToDevice, ctx->stream));
+    NXH_HIP("from_host", hipEventRecord(ctx->stage_done[slot], ctx->stream));
+    ctx->stage_used[slot] = true;
+    return NXH_OK;
+  }
   NXH_HIP("from_host", hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
   NXH_HIP("from_host", hipStreamSynchronize(ctx->stream));
   return NXH_OK;

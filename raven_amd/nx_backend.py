@@ -196,6 +196,10 @@ class Backend:
     def _of_view(self, t: Tensor, v: View) -> Tensor:
         return Tensor(t.buffer, v, t.dtype, self)
 
+    def with_view(self, t: Tensor, v: View) -> Tensor:
+        """``t``'s storage seen through ``v`` (any view the storage can hold)."""
+        return Tensor(t.buffer, v, t.dtype, self)
+
     def expand(self, t, shape):
         return self._of_view(t, t.view.expand(shape))
 

@@ -8,7 +8,6 @@ counterpart of OCaml's ``Invalid_argument``.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
 from typing import Sequence, Tuple
 
 
@@ -29,24 +28,48 @@ def numel(shape: Sequence[int]) -> int:
     return n
 
 
-@dataclass(frozen=True)
+_CONTIGUOUS: dict = {}  # shape -> its C-contiguous, offset-0 view (views are immutable)
+
+
 class View:
-    shape: Tuple[int, ...]
-    strides: Tuple[int, ...]
-    offset: int = 0
+    """Immutable by convention: every operation returns a new view."""
+
+    __slots__ = ("shape", "strides", "offset")
+
+    def __init__(self, shape: Tuple[int, ...], strides: Tuple[int, ...], offset: int = 0):
+        self.shape = shape
+        self.strides = strides
+        self.offset = offset
+
+    def __eq__(self, other):
+        return (isinstance(other, View) and self.shape == other.shape and self.strides == other.strides
+                and self.offset == other.offset)
+
+    def __hash__(self):
+        return hash((self.shape, self.strides, self.offset))
+
+    def __repr__(self):  # pragma: no cover
+        return f"View(shape={self.shape}, strides={self.strides}, offset={self.offset})"
 
     # -- construction (view.ml:43-78) -------------------------------------
     @staticmethod
     def create(shape, strides=None, offset=0) -> "View":
-        shape = tuple(int(s) for s in shape)
+        shape = tuple([int(s) for s in shape])
         if strides is None:
+            if offset == 0 or 0 in shape:
+                v = _CONTIGUOUS.get(shape)
+                if v is None:
+                    v = View(shape, c_contiguous_strides(shape), 0)
+                    if len(_CONTIGUOUS) < 4096:
+                        _CONTIGUOUS[shape] = v
+                return v
             strides = c_contiguous_strides(shape)
         else:
-            strides = tuple(int(s) for s in strides)
+            strides = tuple([int(s) for s in strides])
             if len(strides) != len(shape):
                 raise ValueError(
                     f"create: strides length {len(strides)} != shape length {len(shape)}")
-        if any(s == 0 for s in shape):
+        if 0 in shape:
             offset = 0
         return View(shape, strides, int(offset))
 

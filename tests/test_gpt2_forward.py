@@ -99,3 +99,31 @@ def test_gpt2_forward_bf16_matches_oracle(hip, oracle):
     # bf16 transcendental tolerance of the reference contract: rel = abs = 6e-2
     assert np.all(np.abs(got - want) <= 6e-2 + 6e-2 * np.abs(want))
     assert np.mean(got.argmax(-1) == want.argmax(-1)) >= 0.97
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16], ids=lambda d: d.name)
+def test_gpt2_forward_through_the_window_on_the_gpu(hip, oracle, d):
+    """The same frontend calls through the deferred-evaluation window: every
+    softmax, layer norm and GELU runs as its fused kernel, and the logits agree
+    with the eager GPU forward (a row sum's order is the only difference) and
+    with the oracle."""
+    from raven_amd.nx_window import Window
+
+    hp = host_params(SMALL, seed=16, stddev=0.05)
+    ids = np.random.default_rng(17).integers(0, SMALL.vocab_size, (2, 96))
+    win = Window(hip)
+    got = decode(logical(win.force(run(win, oracle, SMALL, hp, ids, d))), d, oracle)
+    L = SMALL.n_layer
+    assert (win.stats["softmax_rows"], win.stats["layer_norm_rows"], win.stats["gelu_tanh"]) == (L, 2 * L + 1, L)
+    assert win.stats["fallbacks"] == 0
+    eager = decode(logical(run(hip, oracle, SMALL, hp, ids, d)), d, oracle)
+    want = decode(logical(run(oracle, oracle, SMALL, hp, ids, d)), d, oracle)
+    if d is dt.float32:
+        assert np.max(np.abs(got - eager)) <= 2e-5 * max(1.0, np.max(np.abs(eager)))
+        assert np.max(np.abs(got - want)) <= 1e-4 * max(1.0, np.max(np.abs(want)))
+        assert np.mean(got.argmax(-1) == want.argmax(-1)) >= 0.999
+    else:
+        assert np.all(np.abs(got - want) <= 6e-2 + 6e-2 * np.abs(want))
+        assert np.all(np.abs(got - eager) <= 6e-2 + 6e-2 * np.abs(eager))
+        assert np.mean(got.argmax(-1) == want.argmax(-1)) >= 0.97
