@@ -196,7 +196,7 @@ class Workloads:
 
 def next_ops(hip, W):
     """The operations beside the named hot path (pad, cat, scan, threefry,
-    scatter), timed through the Python mirror with HIP events."""
+    scatter, sort, unfold, fold), timed through the Python mirror with HIP events."""
     rng = np.random.default_rng(20)
     out = []
 
@@ -235,6 +235,25 @@ def next_ops(hip, W):
     timed("scatter-add [8192,768] f32 rows into [50257,768] (embedding gradient)",
           lambda: hip.scatter("add", False, table, idx, upd, 0),
           2 * vocab * dim * 4 + ntok * 4 + 3 * ntok * dim * 4, iters=5)
+    del table, upd, idx, ctr, key, y, parts, x
+    # sort moves each element once in and once out; the network in between is
+    # compare-exchange work, so the rate is quoted in keys per second too
+    rows = W.dev(rng.standard_normal((16384, 1024)).astype(np.float32), dt.float32)
+    timed("sort [16384,1024] f32 axis 1 (sort_lds)", lambda: hip.sort(rows, 1, False), 2 * 16384 * 1024 * 4)
+    out[-1]["Mkeys/s"] = round(16384 * 1024 / out[-1]["ms"] / 1e3, 1)
+    timed("argsort [16384,1024] f32 axis 1, descending (sort_lds)", lambda: hip.argsort(rows, 1, True),
+          2 * 16384 * 1024 * 4)
+    out[-1]["Mkeys/s"] = round(16384 * 1024 / out[-1]["ms"] / 1e3, 1)
+    one = W.dev(rng.standard_normal(1 << 24).astype(np.float32), dt.float32)
+    timed("sort 2^24 f32, one slice (sort_global)", lambda: hip.sort(one, 0, False), 2 * (1 << 24) * 4, iters=5)
+    out[-1]["Mkeys/s"] = round((1 << 24) / out[-1]["ms"] / 1e3, 1)
+    del rows, one
+    img = W.dev(rng.standard_normal((8, 64, 128, 128)).astype(np.float32), dt.float32)
+    geo = ([3, 3], [1, 1], [1, 1], [(1, 1), (1, 1)])
+    nin, ncols = 8 * 64 * 128 * 128 * 4, 9 * 8 * 64 * 128 * 128 * 4
+    timed("unfold [8,64,128,128] f32, 3x3 same (im2col)", lambda: hip.unfold(img, *geo), nin + ncols)
+    cols = hip.unfold(img, *geo)
+    timed("fold back to [8,64,128,128] (col2im, 9 taps per output)", lambda: hip.fold(cols, [128, 128], *geo), nin + ncols)
     return out
 
 

@@ -221,6 +221,37 @@ int nxh_scan(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *
 int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *key,
                  const nxh_tensor *counter);
 
+/* ── sort (nx_c_sort.c) ──────────────────────────────────────────────────── */
+
+/* caml_nx_c_sort (nx_c_sort.c:262-292, driver :366-470): out = x sorted along
+   `axis` in the dtype's compute type; NaN-class elements last in both
+   directions; complex is lexicographic. Elements that compare equal but differ
+   in bits (IEEE +-0) come out in ascending original index, reversed for
+   descending — one of the orders the reference's unstable sort may give. */
+int nxh_sort(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int axis,
+             int descending);
+/* caml_nx_c_argsort (nx_c_sort.c:294-312): int32 indices that sort x along
+   `axis`; ties keep the first index first in both directions, NaN-class
+   elements last in index order. */
+int nxh_argsort(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int axis,
+                int descending);
+
+/* ── windows (nx_c_move.c:588-870) ───────────────────────────────────────── */
+
+/* caml_nx_c_unfold (nx_c_move.c:655-690, 789-822): x (leading..., spatial...)
+   -> out (leading..., prod(kernel_size), L), the last n_window_dims dims of x
+   being the windowed ones; taps that fall into the padding read as zero.
+   `padding` is flat: before0, after0, before1, ... */
+int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+               int n_window_dims, const int64_t *kernel_size, const int64_t *stride,
+               const int64_t *dilation, const int64_t *padding);
+/* caml_nx_c_fold (nx_c_move.c:745-787, 829-866): x (leading..., prod(kernel),
+   L) -> out (leading..., output_size...); taps landing on one output element
+   are summed in ascending tap order in the compute type. */
+int nxh_fold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+             int n_window_dims, const int64_t *output_size, const int64_t *kernel_size,
+             const int64_t *stride, const int64_t *dilation, const int64_t *padding);
+
 /* ── fused sequences of primitives ───────────────────────────────────────── */
 
 /* Each call below equals a fixed sequence of the primitives above, as the

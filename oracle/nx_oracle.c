@@ -2055,3 +2055,241 @@ NXO_EXPORT int nxo_scatter(const nxh_tensor *out, const nxh_tensor *indices,
   }
   return NXH_OK;
 }
+
+/* ── sort / argsort (nx_c_sort.c:46-112, 262-330; driver :366-470) ────────────
+   Each slice along `axis` is gathered into the compute type, NaN-class elements
+   go to the tail in both directions, and the rest is ordered by the dtype's
+   total order (complex: real, then imaginary). argsort breaks ties by the
+   original index in both directions (nx_c_sort.c:96-104). The value sort of the
+   reference is unstable and its descending result is the reverse of the
+   ascending finite prefix (:283-289): elements that compare equal are
+   indistinguishable except IEEE +-0, whose order the reference leaves
+   unspecified; here that order is fixed as "ascending by original index, then
+   reversed for descending", i.e. what a stable ascending sort followed by the
+   reference's reversal gives. NaN-class elements keep their original order.
+   A stable merge sort stands in for the reference's introsort: the result is
+   determined by the order relation alone. */
+#define SORT_LT_SINT(a, b) ((a) < (b))
+#define SORT_LT_UINT(a, b) ((a) < (b))
+#define SORT_LT_BOOL(a, b) ((a) < (b))
+#define SORT_LT_FLOAT(a, b) ((a) < (b))
+#define SORT_LT_COMPLEX(a, b) \
+  (__real__(a) < __real__(b) || (__real__(a) == __real__(b) && __imag__(a) < __imag__(b)))
+#define SORT_NAN_SINT(x) (0)
+#define SORT_NAN_UINT(x) (0)
+#define SORT_NAN_BOOL(x) (0)
+#define SORT_NAN_FLOAT(x) (isnan(x))
+#define SORT_NAN_COMPLEX(x) (isnan(__real__(x)) || isnan(__imag__(x)))
+
+typedef void sort_slice_fn(char *o, int64_t os, const char *in, int64_t is, int64_t n, int desc,
+                           int is_arg);
+#define SORT_SLICE(tag, sfx, S, C, LD, ST, cat)                                              \
+  /* a sorts strictly before b under the ascending value order, ties by index */             \
+  static int sort_before_##sfx(const C *keys, int32_t i, int32_t j, int desc) {              \
+    C x = keys[i], y = keys[j];                                                              \
+    if (SORT_LT_##cat(x, y)) return !desc;                                                   \
+    if (SORT_LT_##cat(y, x)) return desc;                                                    \
+    return i < j;                                                                            \
+  }                                                                                          \
+  static void sort_merge_##sfx(const C *keys, int32_t *a, int32_t *tmp, int64_t n, int desc) { \
+    if (n < 2) return;                                                                       \
+    int64_t h = n / 2;                                                                       \
+    sort_merge_##sfx(keys, a, tmp, h, desc);                                                 \
+    sort_merge_##sfx(keys, a + h, tmp, n - h, desc);                                         \
+    int64_t i = 0, j = h, k = 0;                                                             \
+    while (i < h && j < n) tmp[k++] = sort_before_##sfx(keys, a[j], a[i], desc) ? a[j++] : a[i++]; \
+    while (i < h) tmp[k++] = a[i++];                                                         \
+    while (j < n) tmp[k++] = a[j++];                                                         \
+    memcpy(a, tmp, (size_t)n * sizeof(int32_t));                                             \
+  }                                                                                          \
+  static void sort_slice_##sfx(char *o, int64_t os, const char *in, int64_t is, int64_t n,   \
+                               int desc, int is_arg) {                                       \
+    C *keys = malloc((size_t)n * sizeof(C));                                                 \
+    int32_t *idx = malloc((size_t)n * sizeof(int32_t)), *tmp = malloc((size_t)n * sizeof(int32_t)); \
+    for (int64_t k = 0; k < n; k++) keys[k] = ld_##sfx(in + k * is);                         \
+    int64_t f = 0;                                                                           \
+    for (int64_t k = 0; k < n; k++)                                                          \
+      if (!(SORT_NAN_##cat(keys[k]))) idx[f++] = (int32_t)k;                                 \
+    int64_t tail = f;                                                                        \
+    for (int64_t k = 0; k < n; k++)                                                          \
+      if (SORT_NAN_##cat(keys[k])) idx[tail++] = (int32_t)k;                                 \
+    if (is_arg) {                                                                            \
+      sort_merge_##sfx(keys, idx, tmp, f, desc);                                             \
+      for (int64_t k = 0; k < n; k++) *(int32_t *)(o + k * os) = idx[k];                     \
+    } else {                                                                                 \
+      sort_merge_##sfx(keys, idx, tmp, f, 0);                                                \
+      if (desc)                                                                              \
+        for (int64_t i = 0, j = f - 1; i < j; i++, j--) {                                    \
+          int32_t t = idx[i];                                                                \
+          idx[i] = idx[j];                                                                   \
+          idx[j] = t;                                                                        \
+        }                                                                                    \
+      for (int64_t k = 0; k < n; k++) st_##sfx(o + k * os, keys[idx[k]]);                    \
+    }                                                                                        \
+    free(keys);                                                                              \
+    free(idx);                                                                               \
+    free(tmp);                                                                               \
+  }
+NXO_TABLE(SORT_SLICE)
+#define SORT_ROW(tag, sfx, S, C, LD, ST, cat) [tag] = sort_slice_##sfx,
+static sort_slice_fn *const sort_tbl[NXH_DTYPE_COUNT] = {NXO_TABLE(SORT_ROW)};
+
+static int sort_drive(const nxh_tensor *out, const nxh_tensor *in, int axis, int desc, int is_arg) {
+  int dt = in->dtype;
+  if ((unsigned)dt >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (is_packed(dt)) return fail(NXH_FAILURE, ERR_PACKED);
+  if (axis < 0 || axis >= in->ndim) return fail(NXH_INVALID_ARGUMENT, ERR_AXIS);
+  if (out->ndim != in->ndim) return fail(NXH_INVALID_ARGUMENT, "output rank inconsistent with the operation");
+  int64_t n = in->shape[axis];
+  if (is_arg && n > INT32_MAX) return fail(NXH_FAILURE, "argsort axis length exceeds INT32_MAX");
+  int64_t ies = nxo_elem_size(dt), oes = is_arg ? 4 : ies, nslices = 1;
+  for (int d = 0; d < in->ndim; d++)
+    if (d != axis) nslices *= in->shape[d];
+  if (nslices == 0 || n == 0) return NXH_OK;
+  for (int64_t s = 0; s < nslices; s++) {
+    int64_t rem = s, io = in->offset, oo = out->offset;
+    for (int d = in->ndim - 1; d >= 0; d--) {
+      if (d == axis) continue;
+      int64_t c = rem % in->shape[d];
+      rem /= in->shape[d];
+      io += c * in->strides[d];
+      oo += c * out->strides[d];
+    }
+    sort_tbl[dt]((char *)out->data + oo * oes, out->strides[axis] * oes, (const char *)in->data + io * ies,
+                 in->strides[axis] * ies, n, desc, is_arg);
+  }
+  return NXH_OK;
+}
+NXO_EXPORT int nxo_sort(const nxh_tensor *out, const nxh_tensor *in, int axis, int descending) {
+  return sort_drive(out, in, axis, descending, 0);
+}
+NXO_EXPORT int nxo_argsort(const nxh_tensor *out, const nxh_tensor *in, int axis, int descending) {
+  return sort_drive(out, in, axis, descending, 1);
+}
+
+/* ── unfold / fold (nx_c_move.c:588-870) ──────────────────────────────────────
+   unfold: (leading..., spatial...) -> (leading..., prod(kernel), L); element
+   (lead, tap kf, window w) reads x[lead, w*stride + k*dilation - pad_before] per
+   spatial dim, or zero outside the input (:655-690). fold: the inverse, summing
+   the taps that land on each output element in ascending tap order, in the
+   compute type (:745-787). padding is flat [before0, after0, ...]. */
+typedef struct {
+  int K, ld;
+  int64_t kernel[NXH_MAX_NDIM], stride[NXH_MAX_NDIM], dilation[NXH_MAX_NDIM], before[NXH_MAX_NDIM];
+  int64_t win[NXH_MAX_NDIM], win_cp[NXH_MAX_NDIM], ker_cp[NXH_MAX_NDIM], kernel_prod, L;
+} window_t;
+static void window_counts(window_t *w, const int64_t *extent, const int64_t *padding) {
+  for (int d = 0; d < w->K; d++) {
+    int64_t eff = w->dilation[d] * (w->kernel[d] - 1) + 1;
+    int64_t padded = extent[d] + padding[2 * d] + padding[2 * d + 1];
+    int64_t win = (padded - eff) / w->stride[d] + 1;
+    w->win[d] = win < 1 ? 1 : win;
+    w->before[d] = padding[2 * d];
+  }
+  w->win_cp[w->K - 1] = 1;
+  w->ker_cp[w->K - 1] = 1;
+  for (int d = w->K - 2; d >= 0; d--) {
+    w->win_cp[d] = w->win_cp[d + 1] * w->win[d + 1];
+    w->ker_cp[d] = w->ker_cp[d + 1] * w->kernel[d + 1];
+  }
+}
+NXO_EXPORT int nxo_unfold(const nxh_tensor *out, const nxh_tensor *in, int K, const int64_t *kernel,
+                          const int64_t *stride, const int64_t *dilation, const int64_t *padding) {
+  int dt = out->dtype;
+  if ((unsigned)dt >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (is_packed(dt)) return fail(NXH_FAILURE, ERR_PACKED);
+  if (K < 1 || K > NXH_MAX_NDIM || in->ndim < K) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+  window_t w;
+  w.K = K;
+  w.ld = in->ndim - K;
+  for (int d = 0; d < K; d++) w.kernel[d] = kernel[d], w.stride[d] = stride[d], w.dilation[d] = dilation[d];
+  w.kernel_prod = out->shape[w.ld];
+  w.L = out->shape[w.ld + 1];
+  window_counts(&w, &in->shape[w.ld], padding);
+  int64_t lead = 1, es = nxo_elem_size(dt);
+  for (int d = 0; d < w.ld; d++) lead *= in->shape[d];
+  int64_t total = lead * w.kernel_prod * w.L;
+  for (int64_t it = 0; it < total; it++) {
+    int64_t wf = it % w.L, rem = it / w.L, kf = rem % w.kernel_prod, l = rem / w.kernel_prod;
+    int64_t oo = out->offset + kf * out->strides[w.ld] + wf * out->strides[w.ld + 1], io = in->offset;
+    for (int d = w.ld - 1; d >= 0; d--) {
+      int64_t c = l % in->shape[d];
+      l /= in->shape[d];
+      oo += c * out->strides[d];
+      io += c * in->strides[d];
+    }
+    bool valid = true;
+    for (int d = 0; d < K && valid; d++) {
+      int64_t wc = (wf / w.win_cp[d]) % w.win[d], kc = (kf / w.ker_cp[d]) % w.kernel[d];
+      int64_t sp = wc * w.stride[d] + kc * w.dilation[d] - w.before[d];
+      if (sp < 0 || sp >= in->shape[w.ld + d]) valid = false;
+      else io += sp * in->strides[w.ld + d];
+    }
+    char *dst = (char *)out->data + oo * es;
+    if (valid) memcpy(dst, (const char *)in->data + io * es, (size_t)es);
+    else memset(dst, 0, (size_t)es);
+  }
+  return NXH_OK;
+}
+
+typedef void fold_sum_fn(char *out, const char *const *taps, int ntaps);
+#define FOLD_SUM(tag, sfx, S, C, LD, ST, cat)                                   \
+  static void fold_sum_##sfx(char *out, const char *const *taps, int ntaps) {   \
+    C acc = (C)0;                                                               \
+    for (int i = 0; i < ntaps; i++) acc = (C)MOVE_ADD_##cat(acc, ld_##sfx(taps[i])); \
+    st_##sfx(out, acc);                                                         \
+  }
+NXO_TABLE(FOLD_SUM)
+#define FOLD_SUM_ROW(tag, sfx, S, C, LD, ST, cat) [tag] = fold_sum_##sfx,
+static fold_sum_fn *const fold_sum_tbl[NXH_DTYPE_COUNT] = {NXO_TABLE(FOLD_SUM_ROW)};
+
+NXO_EXPORT int nxo_fold(const nxh_tensor *out, const nxh_tensor *in, int K, const int64_t *output_size,
+                        const int64_t *kernel, const int64_t *stride, const int64_t *dilation,
+                        const int64_t *padding) {
+  int dt = out->dtype;
+  if ((unsigned)dt >= NXH_DTYPE_COUNT) return fail(NXH_FAILURE, "unsupported bigarray kind");
+  if (is_packed(dt)) return fail(NXH_FAILURE, ERR_PACKED);
+  if (K < 1 || K > NXH_MAX_NDIM || in->ndim < 2) return fail(NXH_INVALID_ARGUMENT, ERR_SHAPE);
+  window_t w;
+  w.K = K;
+  w.ld = in->ndim - 2;
+  for (int d = 0; d < K; d++) w.kernel[d] = kernel[d], w.stride[d] = stride[d], w.dilation[d] = dilation[d];
+  w.kernel_prod = in->shape[w.ld];
+  w.L = in->shape[w.ld + 1];
+  window_counts(&w, output_size, padding);
+  int64_t lead = 1, spatial = 1, es = nxo_elem_size(dt);
+  for (int d = 0; d < w.ld; d++) lead *= in->shape[d];
+  for (int d = 0; d < K; d++) spatial *= output_size[d];
+  const char **taps = malloc((size_t)(w.kernel_prod > 0 ? w.kernel_prod : 1) * sizeof(char *));
+  for (int64_t it = 0; it < lead * spatial; it++) {
+    int64_t ol = it % spatial, l = it / spatial, oc[NXH_MAX_NDIM];
+    for (int d = K - 1; d >= 0; d--) {
+      oc[d] = ol % output_size[d];
+      ol /= output_size[d];
+    }
+    int64_t oo = out->offset, il = in->offset;
+    for (int d = w.ld - 1; d >= 0; d--) {
+      int64_t c = l % out->shape[d];
+      l /= out->shape[d];
+      oo += c * out->strides[d];
+      il += c * in->strides[d];
+    }
+    for (int d = 0; d < K; d++) oo += oc[d] * out->strides[w.ld + d];
+    int ntaps = 0;
+    for (int64_t kf = 0; kf < w.kernel_prod; kf++) {
+      bool valid = true;
+      int64_t wf = 0;
+      for (int d = 0; d < K && valid; d++) {
+        int64_t kc = (kf / w.ker_cp[d]) % w.kernel[d];
+        int64_t num = oc[d] + w.before[d] - kc * w.dilation[d];
+        if (num < 0 || num % w.stride[d] != 0 || num / w.stride[d] >= w.win[d]) valid = false;
+        else wf += (num / w.stride[d]) * w.win_cp[d];
+      }
+      if (valid)
+        taps[ntaps++] = (const char *)in->data + (il + kf * in->strides[w.ld] + wf * in->strides[w.ld + 1]) * es;
+    }
+    fold_sum_tbl[dt]((char *)out->data + oo * es, taps, ntaps);
+  }
+  free(taps);
+  return NXH_OK;
+}

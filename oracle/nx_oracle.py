@@ -61,6 +61,10 @@ def lib() -> C.CDLL:
             "nxo_scan": [C.c_int, T, T, C.c_int],
             "nxo_threefry": [T, T, T],
             "nxo_scatter": [T, T, T, C.c_int, C.c_int],
+            "nxo_sort": [T, T, C.c_int, C.c_int],
+            "nxo_argsort": [T, T, C.c_int, C.c_int],
+            "nxo_unfold": [T, T, C.c_int] + [C.POINTER(C.c_int64)] * 4,
+            "nxo_fold": [T, T, C.c_int] + [C.POINTER(C.c_int64)] * 5,
         }.items():
             getattr(L, name).argtypes = args
             getattr(L, name).restype = C.c_int
@@ -283,6 +287,50 @@ class OracleBackend:
         _check(lib().nxo_scatter(out.desc(), indices.desc(), updates.desc(), axis,
                                  {"set": 0, "add": 1}[mode]), "scatter")
         return out
+
+    # sort, windows -----------------------------------------------------------
+    def sort(self, x, axis: int, descending: bool):
+        out = self.buffer(x.dtype, x.shape)
+        _check(lib().nxo_sort(out.desc(), x.desc(), axis, int(descending)), "sort")
+        return out
+
+    def argsort(self, x, axis: int, descending: bool):
+        out = self.buffer(dt.int32, x.shape)
+        _check(lib().nxo_argsort(out.desc(), x.desc(), axis, int(descending)), "argsort")
+        return out
+
+    def unfold(self, x, kernel_size, stride, dilation, padding):
+        shape, params = window_shapes(x.shape, kernel_size, stride, dilation, padding)
+        out = self.buffer(x.dtype, shape)
+        _check(lib().nxo_unfold(out.desc(), x.desc(), len(kernel_size), *params), "unfold")
+        return out
+
+    def fold(self, x, output_size, kernel_size, stride, dilation, padding):
+        _, params = window_shapes(tuple(x.shape[:-2]) + tuple(output_size), kernel_size, stride, dilation, padding)
+        out = self.buffer(x.dtype, tuple(x.shape[:-2]) + tuple(int(s) for s in output_size))
+        osz = (C.c_int64 * len(output_size))(*[int(s) for s in output_size])
+        _check(lib().nxo_fold(out.desc(), x.desc(), len(kernel_size), osz, *params), "fold")
+        return out
+
+
+def window_shapes(in_shape, kernel_size, stride, dilation, padding):
+    """Result shape of unfold (nx_backend.ml:427-445) and the K-long parameter
+    arrays as C int64 arrays (padding flattened to [before0, after0, ...])."""
+    k = len(kernel_size)
+    if not (len(stride) == len(dilation) == len(padding) == k) or k < 1 or len(in_shape) < k:
+        raise ValueError("unfold: shape mismatch")
+    lead, spatial = tuple(in_shape[:len(in_shape) - k]), in_shape[len(in_shape) - k:]
+    windows = 1
+    for i in range(k):
+        padded = spatial[i] + padding[i][0] + padding[i][1]
+        extent = dilation[i] * (kernel_size[i] - 1) + 1
+        windows *= (padded - extent) // stride[i] + 1
+    kp = 1
+    for s in kernel_size:
+        kp *= s
+    arr = lambda v: (C.c_int64 * len(v))(*[int(a) for a in v])
+    flat = [int(v) for pair in padding for v in pair]
+    return lead + (kp, windows), (arr(kernel_size), arr(stride), arr(dilation), arr(flat))
 
 
 def logical(t: OTensor) -> np.ndarray:

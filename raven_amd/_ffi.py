@@ -90,6 +90,10 @@ SIGNATURES = {
     "nxh_scan": (C.c_int, [_CTX, C.c_int, _T, _T, C.c_int]),
     "nxh_threefry": (C.c_int, [_CTX, _T, _T, _T]),
     "nxh_gather": (C.c_int, [_CTX, _T, _T, _T, C.c_int]),
+    "nxh_sort": (C.c_int, [_CTX, _T, _T, C.c_int, C.c_int]),
+    "nxh_argsort": (C.c_int, [_CTX, _T, _T, C.c_int, C.c_int]),
+    "nxh_unfold": (C.c_int, [_CTX, _T, _T, C.c_int] + [_P(C.c_int64)] * 4),
+    "nxh_fold": (C.c_int, [_CTX, _T, _T, C.c_int] + [_P(C.c_int64)] * 5),
     "nxh_softmax_rows": (C.c_int, [_CTX, _T, _T, C.c_void_p, _T, C.c_void_p]),
     "nxh_layer_norm_rows": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_double]),
     "nxh_gelu_tanh": (C.c_int, [_CTX, _T, _T, C.c_void_p]),

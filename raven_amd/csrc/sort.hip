@@ -1,0 +1,363 @@
+// sort.hip — sort and argsort along one axis (packages/nx/lib/backend_c/
+// nx_c_sort.c).
+//
+// Order (nx_c_sort.c:46-112): each slice is compared in the dtype's compute
+// type; NaN-class elements (either part of a complex) go last in both
+// directions; complex is lexicographic (real, then imaginary). argsort breaks
+// ties by the original index in both directions, so it is stable. The value
+// sort of the reference is an unstable introsort whose descending result is the
+// ascending finite prefix reversed (:283-289); elements that compare equal are
+// indistinguishable except IEEE +-0, whose order it leaves open. Here every
+// comparison is a TOTAL order on (class, value, index) — ties by ascending
+// index, by descending index for the descending value sort (what reversing a
+// stable ascending sort gives), NaN-class elements in index order — so the
+// result is unique and a sorting network reproduces it whatever its exchange
+// pattern.
+//
+// Algorithm: bitonic sorting network on (key, index) pairs, the slice padded to
+// a power of two with elements that sort last.
+//   sort_lds     slices of up to 4096 elements (2048 for 16-byte keys): whole
+//                network in LDS, several short slices per block;
+//   sort_global  longer slices: pairs staged in scratch memory; chunks are
+//                sorted in LDS, then each merge level runs its long-distance
+//                exchanges as passes over global memory and finishes the
+//                short-distance ones in LDS.
+
+#include "fold_common.hpp"
+
+namespace {
+
+constexpr int SORT_MAXD = 12;
+constexpr int32_t PAD_INDEX = 0x7fffffff;
+
+enum SortMode { VALUE_ASC = 0, VALUE_DESC = 1, ARG_ASC = 2, ARG_DESC = 3 };
+
+template <int DT>
+struct Key {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  __device__ __forceinline__ static bool is_nan(C x) {
+    if constexpr (TR::cat == CAT_FLOAT) return x != x;
+    else if constexpr (TR::cat == CAT_COMPLEX) return x.re != x.re || x.im != x.im;
+    else return false;
+  }
+  __device__ __forceinline__ static bool lt(C a, C b) {
+    if constexpr (TR::cat == CAT_COMPLEX) return a.re < b.re || (a.re == b.re && a.im < b.im);
+    else return a < b;
+  }
+  // (ka, ia) sorts strictly before (kb, ib)
+  template <int MODE>
+  __device__ __forceinline__ static bool before(C ka, int32_t ia, C kb, int32_t ib) {
+    const int ca = ia == PAD_INDEX ? 2 : (is_nan(ka) ? 1 : 0);
+    const int cb = ib == PAD_INDEX ? 2 : (is_nan(kb) ? 1 : 0);
+    if (ca != cb) return ca < cb;
+    if (ca == 2) return false;
+    if (ca == 1) return ia < ib;
+    const bool l = lt(ka, kb), g = lt(kb, ka);
+    constexpr bool desc = MODE == VALUE_DESC || MODE == ARG_DESC;
+    if (l != g) return desc ? g : l;
+    return MODE == VALUE_DESC ? ia > ib : ia < ib;
+  }
+};
+
+struct SortArgs {
+  const char *in;
+  char *out;
+  void *keys;      // scratch (sort_global): slices * n_pad keys
+  int32_t *index;  // scratch (sort_global): slices * n_pad indices
+  int64_t slices, n, n_pad;
+  int64_t in_axis, out_axis;  // strides along the sorted axis, elements
+  int nk;
+  int64_t kshape[SORT_MAXD], k_in[SORT_MAXD], k_out[SORT_MAXD];
+};
+
+__device__ __forceinline__ void slice_offsets(const SortArgs &a, int64_t s, int64_t &io, int64_t &oo) {
+  io = 0;
+  oo = 0;
+  for (int d = a.nk - 1; d >= 0; d--) {
+    const int64_t c = s % a.kshape[d];
+    s /= a.kshape[d];
+    io += c * a.k_in[d];
+    oo += c * a.k_out[d];
+  }
+}
+
+template <int DT>
+constexpr int lds_elems() {
+  return sizeof(typename Tr<DT>::C) > 8 ? 2048 : 4096;
+}
+
+// One compare-exchange step of distance j inside LDS over `count` elements;
+// `up` tells the direction of element i's subsequence. `base` is added to a
+// local position to get the position inside its slice (direction bits).
+template <int DT, int MODE>
+__device__ __forceinline__ void lds_step(typename Tr<DT>::C *k, int32_t *ix, int count, int j, int64_t kk,
+                                         int64_t base, int64_t mask) {
+  using K = Key<DT>;
+  for (int p = threadIdx.x; p < count / 2; p += 256) {
+    const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));
+    const int l = i | j;
+    const bool up = (((base + i) & mask) & kk) == 0;
+    const auto ka = k[i], kb = k[l];
+    const int32_t ia = ix[i], ib = ix[l];
+    const bool swap = up ? K::template before<MODE>(kb, ib, ka, ia) : K::template before<MODE>(ka, ia, kb, ib);
+    if (swap) {
+      k[i] = kb;
+      k[l] = ka;
+      ix[i] = ib;
+      ix[l] = ia;
+    }
+  }
+  __syncthreads();
+}
+
+// Whole slices in LDS: a block holds `spb` slices of n_pad elements each.
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void sort_lds_kernel(SortArgs a, int spb) {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  using S = typename TR::S;
+  constexpr int NL = lds_elems<DT>();
+  __shared__ C k[NL];
+  __shared__ int32_t ix[NL];
+  const int np = (int)a.n_pad, count = spb * np;
+  const int64_t first = (int64_t)blockIdx.x * spb;
+  for (int e = threadIdx.x; e < count; e += 256) {
+    const int64_t s = first + e / np;
+    const int i = e % np;
+    C key{};
+    int32_t id = PAD_INDEX;
+    if (s < a.slices && i < a.n) {
+      int64_t io, oo;
+      slice_offsets(a, s, io, oo);
+      key = TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]);
+      id = i;
+    }
+    k[e] = key;
+    ix[e] = id;
+  }
+  __syncthreads();
+  for (int kk = 2; kk <= np; kk <<= 1)
+    for (int j = kk >> 1; j >= 1; j >>= 1) lds_step<DT, MODE>(k, ix, count, j, kk, 0, np - 1);
+  for (int e = threadIdx.x; e < count; e += 256) {
+    const int64_t s = first + e / np;
+    const int i = e % np;
+    if (s < a.slices && i < a.n) {
+      int64_t io, oo;
+      slice_offsets(a, s, io, oo);
+      if constexpr (MODE >= ARG_ASC) reinterpret_cast<int32_t *>(a.out)[oo + i * a.out_axis] = ix[e];
+      else reinterpret_cast<S *>(a.out)[oo + i * a.out_axis] = TR::st(k[e]);
+    }
+  }
+}
+
+// sort_global, phase 0: gather the slices into scratch and sort each chunk of
+// NL elements (all levels kk <= NL).
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void sort_chunks_kernel(SortArgs a) {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  using S = typename TR::S;
+  constexpr int NL = lds_elems<DT>();
+  __shared__ C k[NL];
+  __shared__ int32_t ix[NL];
+  const int64_t chunks = a.n_pad / NL;
+  const int64_t s = blockIdx.x / chunks, base = (blockIdx.x % chunks) * NL;
+  int64_t io, oo;
+  slice_offsets(a, s, io, oo);
+  for (int e = threadIdx.x; e < NL; e += 256) {
+    const int64_t i = base + e;
+    C key{};
+    int32_t id = PAD_INDEX;
+    if (i < a.n) {
+      key = TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]);
+      id = (int32_t)i;
+    }
+    k[e] = key;
+    ix[e] = id;
+  }
+  __syncthreads();
+  for (int kk = 2; kk <= NL; kk <<= 1)
+    for (int j = kk >> 1; j >= 1; j >>= 1) lds_step<DT, MODE>(k, ix, NL, j, kk, base, a.n_pad - 1);
+  C *gk = reinterpret_cast<C *>(a.keys) + s * a.n_pad + base;
+  int32_t *gi = a.index + s * a.n_pad + base;
+  for (int e = threadIdx.x; e < NL; e += 256) {
+    gk[e] = k[e];
+    gi[e] = ix[e];
+  }
+}
+
+// One long-distance exchange pass of level kk, distance j >= NL, over scratch.
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void sort_exchange_kernel(SortArgs a, int64_t kk, int64_t j) {
+  using C = typename Tr<DT>::C;
+  using K = Key<DT>;
+  const int64_t half = a.n_pad / 2;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= a.slices * half) return;
+  const int64_t s = t / half, p = t % half;
+  const int64_t i = ((p & ~(j - 1)) << 1) | (p & (j - 1)), l = i | j;
+  C *gk = reinterpret_cast<C *>(a.keys) + s * a.n_pad;
+  int32_t *gi = a.index + s * a.n_pad;
+  const bool up = (i & kk) == 0;
+  const C ka = gk[i], kb = gk[l];
+  const int32_t ia = gi[i], ib = gi[l];
+  const bool swap = up ? K::template before<MODE>(kb, ib, ka, ia) : K::template before<MODE>(ka, ia, kb, ib);
+  if (swap) {
+    gk[i] = kb;
+    gk[l] = ka;
+    gi[i] = ib;
+    gi[l] = ia;
+  }
+}
+
+// The short-distance steps (j < NL) of level kk, chunk by chunk in LDS. After
+// the last level (`final`), the chunk goes to the output instead of scratch.
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void sort_merge_kernel(SortArgs a, int64_t kk, int final) {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  using S = typename TR::S;
+  constexpr int NL = lds_elems<DT>();
+  __shared__ C k[NL];
+  __shared__ int32_t ix[NL];
+  const int64_t chunks = a.n_pad / NL;
+  const int64_t s = blockIdx.x / chunks, base = (blockIdx.x % chunks) * NL;
+  C *gk = reinterpret_cast<C *>(a.keys) + s * a.n_pad + base;
+  int32_t *gi = a.index + s * a.n_pad + base;
+  for (int e = threadIdx.x; e < NL; e += 256) {
+    k[e] = gk[e];
+    ix[e] = gi[e];
+  }
+  __syncthreads();
+  for (int j = NL >> 1; j >= 1; j >>= 1) lds_step<DT, MODE>(k, ix, NL, j, kk, base, a.n_pad - 1);
+  if (!final) {
+    for (int e = threadIdx.x; e < NL; e += 256) {
+      gk[e] = k[e];
+      gi[e] = ix[e];
+    }
+    return;
+  }
+  int64_t io, oo;
+  slice_offsets(a, s, io, oo);
+  for (int e = threadIdx.x; e < NL; e += 256) {
+    const int64_t i = base + e;
+    if (i < a.n) {
+      if constexpr (MODE >= ARG_ASC) reinterpret_cast<int32_t *>(a.out)[oo + i * a.out_axis] = ix[e];
+      else reinterpret_cast<S *>(a.out)[oo + i * a.out_axis] = TR::st(k[e]);
+    }
+  }
+}
+
+template <int DT, int MODE>
+int sort_run(nxh_context *ctx, const char *op, SortArgs &a) {
+  using C = typename Tr<DT>::C;
+  constexpr int NL = lds_elems<DT>();
+  if (a.n_pad <= NL) {
+    // several short slices per block, at least 1024 elements of work
+    int spb = (int)std::max<int64_t>(1, std::min<int64_t>(NL, 1024) / a.n_pad);
+    if (spb > a.slices) spb = (int)a.slices;
+    const int64_t blocks = (a.slices + spb - 1) / spb;
+    if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many slices for one launch");
+    nxh_set_path("sort_lds");
+    hipLaunchKernelGGL((sort_lds_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a, spb);
+    NXH_HIP(op, hipGetLastError());
+    return NXH_OK;
+  }
+  const int64_t chunks = a.n_pad / NL, blocks = a.slices * chunks;
+  const int64_t pairs = a.slices * (a.n_pad / 2);
+  if (blocks > 0x7fffffffLL || (pairs + 255) / 256 > 0x7fffffffLL)
+    return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  Scratch scratch(ctx);
+  int rc = scratch.get(0, (size_t)(a.slices * a.n_pad) * sizeof(C));
+  if (!rc) rc = scratch.get(1, (size_t)(a.slices * a.n_pad) * sizeof(int32_t));
+  if (rc) return nxh_fail(NXH_FAILURE, op, NXH_ERR_ALLOC);
+  a.keys = scratch.p[0];
+  a.index = (int32_t *)scratch.p[1];
+  nxh_set_path("sort_global");
+  hipLaunchKernelGGL((sort_chunks_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
+  for (int64_t kk = 2 * (int64_t)NL; kk <= a.n_pad; kk <<= 1) {
+    for (int64_t j = kk >> 1; j >= NL; j >>= 1)
+      hipLaunchKernelGGL((sort_exchange_kernel<DT, MODE>), dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0,
+                         ctx->stream, a, kk, j);
+    hipLaunchKernelGGL((sort_merge_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a, kk,
+                       kk == a.n_pad ? 1 : 0);
+  }
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+typedef int (*sort_fn)(nxh_context *, const char *, SortArgs &);
+struct SortTable {
+  sort_fn fn[NXH_DTYPE_COUNT][4] = {};
+  template <int DT>
+  void set() {
+    fn[DT][VALUE_ASC] = &sort_run<DT, VALUE_ASC>;
+    fn[DT][VALUE_DESC] = &sort_run<DT, VALUE_DESC>;
+    fn[DT][ARG_ASC] = &sort_run<DT, ARG_ASC>;
+    fn[DT][ARG_DESC] = &sort_run<DT, ARG_DESC>;
+  }
+  SortTable() {
+#define NXH_ST(DT) set<DT>();
+    NXH_FOR_COMPUTE_DTYPES(NXH_ST)
+#undef NXH_ST
+  }
+};
+
+int sort_entry(nxh_context *ctx, const char *op, const nxh_tensor *out, const nxh_tensor *x, int axis,
+               int descending, bool is_arg) {
+  if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (rc) return rc;
+  const int dt = x->dtype;
+  if (nxh_is_packed(dt)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  if (out->dtype != (is_arg ? NXH_I32 : dt)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  if (axis < 0 || axis >= x->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_AXIS);
+  if (out->ndim != x->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_RANK);
+  for (int d = 0; d < x->ndim; d++)
+    if (out->shape[d] != x->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  SortArgs a;
+  a.n = x->shape[axis];
+  // indices are int32 (nx_c_sort.c:41-43); the value sort carries them too
+  if (a.n > ((int64_t)1 << 30))
+    return nxh_fail(NXH_FAILURE, op, is_arg ? "argsort axis length exceeds INT32_MAX" : "sort axis longer than 2^30 elements");
+  a.slices = 1;
+  a.nk = 0;
+  for (int d = 0; d < x->ndim; d++) {
+    if (d == axis) continue;
+    a.slices *= x->shape[d];
+    if (x->shape[d] == 1) continue;
+    if (a.nk == SORT_MAXD) return nxh_fail(NXH_FAILURE, op, "more than 12 dimensions beside the sorted axis");
+    a.kshape[a.nk] = x->shape[d];
+    a.k_in[a.nk] = x->strides[d];
+    a.k_out[a.nk] = out->strides[d];
+    a.nk++;
+  }
+  if (a.slices == 0 || a.n == 0) return NXH_OK;
+  for (int d = 0; d < x->ndim; d++)
+    if (x->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  a.n_pad = 2;
+  while (a.n_pad < a.n) a.n_pad <<= 1;
+  a.in_axis = x->strides[axis];
+  a.out_axis = out->strides[axis];
+  a.in = (const char *)x->data + x->offset * (int64_t)nxh_elem_size(dt);
+  a.out = (char *)out->data + out->offset * (int64_t)nxh_elem_size(out->dtype);
+  a.keys = nullptr;
+  a.index = nullptr;
+  static const SortTable table;
+  const int mode = (is_arg ? 2 : 0) + (descending ? 1 : 0);
+  if (!table.fn[dt][mode]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  return table.fn[dt][mode](ctx, op, a);
+}
+
+}  // namespace
+
+NXH_EXPORT int nxh_sort(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int axis, int descending) {
+  return sort_entry(ctx, "sort", out, x, axis, descending, false);
+}
+NXH_EXPORT int nxh_argsort(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int axis, int descending) {
+  return sort_entry(ctx, "argsort", out, x, axis, descending, true);
+}

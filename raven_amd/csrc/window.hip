@@ -1,0 +1,392 @@
+// window.hip — unfold (im2col) and fold (col2im), packages/nx/lib/backend_c/
+// nx_c_move.c:588-870.
+//
+// unfold: (leading..., spatial...) -> (leading..., prod(kernel), L). Output
+// element (lead, tap kf, window w) is one input element, or zero when the tap
+// falls into the padding; every output is written once. A block owns one
+// (leading index, tap) row of the output and a run of its windows (the
+// contiguous axis), each lane eight of them 256 apart: the row is decoded once
+// per lane, the window coordinates once, and from then on they advance by an
+// odometer step, so no division is left in the per-element work.
+//
+// fold: (leading..., prod(kernel), L) -> (leading..., output...). One lane per
+// OUTPUT element sums the taps that land on it, in ascending tap order and in
+// the dtype's compute type, as nx_c_move.c:745-787 does: no atomics, no zeroing
+// pass, and float results equal the reference's bit for bit.
+//
+// Limits: at most 6 window dims and 8 leading dims (the reference allows 32 in
+// total); beyond that the call fails with Failure.
+
+#include "nxh_common.hpp"
+
+namespace {
+
+constexpr int WIN_MAXK = 6;
+constexpr int WIN_MAXLEAD = 8;
+constexpr int WINDOWS_PER_LANE = 8;
+
+// Window dims are right-aligned in arrays of the kernel's compile-time rank KT
+// (1, 2, 3 or 6); unused leading slots hold a neutral dim (extent, kernel,
+// window count, stride, dilation 1; padding 0; tensor stride 0).
+struct WindowArgs {
+  const char *in;
+  char *out;
+  int ld;
+  int64_t total, rows;  // elements launched over; (leading, tap) rows of the windowed tensor
+  int64_t kernel_prod, L;
+  int64_t lshape[WIN_MAXLEAD], l_in[WIN_MAXLEAD], l_out[WIN_MAXLEAD];
+  int64_t kernel[WIN_MAXK], stride[WIN_MAXK], dilation[WIN_MAXK], before[WIN_MAXK];
+  int64_t win[WIN_MAXK], win_cp[WIN_MAXK];
+  int64_t step[WIN_MAXK];       // 256 written in the mixed radix of win[]
+  int64_t extent[WIN_MAXK];     // spatial extents of the un-windowed tensor
+  int64_t sp_stride[WIN_MAXK];  // its strides along those dims
+  int64_t tap_stride, win_stride;  // strides of the windowed tensor's last two dims
+};
+
+// I is the type the index arithmetic runs in: int32_t whenever every extent,
+// element count and window coordinate fits (64-bit division is an order of
+// magnitude slower on this machine), int64_t otherwise. Memory offsets are
+// always 64-bit. `rows_per_block` > 1 packs several short rows into one block,
+// one window per lane.
+template <class E, class I, int KT>
+__global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, int rows_per_block) {
+  const I L = (I)a.L;
+  I row, w0;
+  int reps = WINDOWS_PER_LANE;
+  if (rows_per_block > 1) {
+    const I lanes_per_row = 256 / rows_per_block;
+    row = (I)blockIdx.x * rows_per_block + (I)threadIdx.x / lanes_per_row;
+    w0 = (I)threadIdx.x % lanes_per_row;
+    reps = 1;
+    if (w0 >= L) return;
+  } else {
+    row = (I)(blockIdx.x / (unsigned)wblocks);
+    w0 = (I)(blockIdx.x % (unsigned)wblocks) * (256 * WINDOWS_PER_LANE) + (I)threadIdx.x;
+  }
+  if (row >= (I)a.rows) return;
+  I kf = row % (I)a.kernel_prod;
+  I lead = row / (I)a.kernel_prod;
+  int64_t oo = (int64_t)kf * a.tap_stride, io = 0;
+  for (int d = a.ld - 1; d >= 0; d--) {
+    const I c = lead % (I)a.lshape[d];
+    lead /= (I)a.lshape[d];
+    oo += (int64_t)c * a.l_out[d];
+    io += (int64_t)c * a.l_in[d];
+  }
+  I tap[KT], wc[KT];  // tap: kc * dilation - pad_before; wc: window coordinate
+  I rest = w0;
+#pragma unroll
+  for (int d = KT - 1; d >= 0; d--) {
+    tap[d] = kf % (I)a.kernel[d] * (I)a.dilation[d] - (I)a.before[d];
+    kf /= (I)a.kernel[d];
+    wc[d] = rest % (I)a.win[d];
+    rest /= (I)a.win[d];
+  }
+  const E *in = reinterpret_cast<const E *>(a.in);
+  E *out = reinterpret_cast<E *>(a.out);
+#pragma unroll
+  for (int u = 0; u < WINDOWS_PER_LANE; u++) {
+    const I wf = w0 + (I)u * 256;
+    if (u >= reps || wf >= L) break;
+    bool valid = true;
+    int64_t off = io;
+#pragma unroll
+    for (int d = 0; d < KT; d++) {
+      const I sp = wc[d] * (I)a.stride[d] + tap[d];
+      valid = valid && sp >= 0 && sp < (I)a.extent[d];
+      off += (int64_t)sp * a.sp_stride[d];
+    }
+    E v = E{};
+    if (valid) v = in[off];
+    out[oo + (int64_t)wf * a.win_stride] = v;
+    // 256 windows further: add the digits of 256, carrying towards the front
+    I carry = 0;
+#pragma unroll
+    for (int d = KT - 1; d >= 0; d--) {
+      const I t = wc[d] + (I)a.step[d] + carry;
+      carry = t >= (I)a.win[d] ? 1 : 0;
+      wc[d] = carry ? t - (I)a.win[d] : t;
+    }
+  }
+}
+
+template <int DT, class I, int KT>
+__global__ __launch_bounds__(256) void fold_kernel(WindowArgs a) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  const int64_t it64 = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (it64 >= a.total) return;
+  I ol = (I)it64;
+  I oc[KT];  // position in the padded frame
+  int64_t oo = 0, il = 0;
+#pragma unroll
+  for (int d = KT - 1; d >= 0; d--) {
+    const I c = ol % (I)a.extent[d];
+    ol /= (I)a.extent[d];
+    oc[d] = c + (I)a.before[d];
+    oo += (int64_t)c * a.sp_stride[d];
+  }
+  for (int d = a.ld - 1; d >= 0; d--) {
+    const I c = ol % (I)a.lshape[d];
+    ol /= (I)a.lshape[d];
+    oo += (int64_t)c * a.l_out[d];
+    il += (int64_t)c * a.l_in[d];
+  }
+  const S *in = reinterpret_cast<const S *>(a.in);
+  C acc;
+  if constexpr (TR::cat == CAT_COMPLEX) acc = C{0, 0};
+  else acc = (C)0;
+  // taps in ascending flat order kf; kc[] is kf's odometer over the kernel dims
+  I kc[KT];
+#pragma unroll
+  for (int d = 0; d < KT; d++) kc[d] = 0;
+  const I taps = (I)a.kernel_prod;
+  for (I kf = 0; kf < taps; kf++) {
+    bool valid = true;
+    int64_t wf = 0;
+#pragma unroll
+    for (int d = 0; d < KT; d++) {
+      const I num = oc[d] - kc[d] * (I)a.dilation[d];
+      const I st = (I)a.stride[d];
+      const I wc = st == 1 ? num : num / st;
+      valid = valid && num >= 0 && (st == 1 || num % st == 0) && wc < (I)a.win[d];
+      wf += (int64_t)wc * a.win_cp[d];
+    }
+    if (valid) {
+      const C v = TR::ld(in[il + (int64_t)kf * a.tap_stride + wf * a.win_stride]);
+      if constexpr (TR::cat == CAT_SINT) acc = (C)((uint64_t)acc + (uint64_t)v);
+      else acc = (C)(acc + v);
+    }
+    bool carry = true;
+#pragma unroll
+    for (int d = KT - 1; d >= 0; d--) {
+      if (carry) {
+        kc[d]++;
+        carry = kc[d] >= (I)a.kernel[d];
+        if (carry) kc[d] = 0;
+      }
+    }
+  }
+  reinterpret_cast<S *>(a.out)[oo] = TR::st(acc);
+}
+
+struct G16w {
+  uint64_t lo, hi;
+};
+
+// 32-bit index arithmetic is exact when every quantity that is divided, and
+// every coordinate built from the quotients, stays below 2^31.
+bool fits_int32(const WindowArgs &a) {
+  const int64_t lim = (int64_t)1 << 31;
+  if (a.total >= lim || a.rows >= lim || a.L + 256 * WINDOWS_PER_LANE >= lim || a.kernel_prod >= lim) return false;
+  for (int d = 0; d < WIN_MAXK; d++) {
+    const int64_t reach = (a.win[d] + 256) * a.stride[d] + a.kernel[d] * a.dilation[d] + a.before[d] + a.extent[d];
+    if (reach >= lim) return false;
+  }
+  return true;
+}
+int rank_class(int K) { return K <= 3 ? K : WIN_MAXK; }
+
+typedef void (*fold_launch_fn)(nxh_context *, const WindowArgs &, int);
+template <int DT>
+void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt) {
+  const dim3 grid((unsigned)((a.total + 255) / 256)), block(256);
+  const bool narrow = fits_int32(a);
+#define NXH_FOLD_CASE(KT)                                                                                  \
+  case KT:                                                                                                 \
+    if (narrow) hipLaunchKernelGGL((fold_kernel<DT, int32_t, KT>), grid, block, 0, ctx->stream, a);        \
+    else hipLaunchKernelGGL((fold_kernel<DT, int64_t, KT>), grid, block, 0, ctx->stream, a);               \
+    break;
+  switch (kt) {
+    NXH_FOLD_CASE(1)
+    NXH_FOLD_CASE(2)
+    NXH_FOLD_CASE(3)
+    NXH_FOLD_CASE(WIN_MAXK)
+  }
+#undef NXH_FOLD_CASE
+}
+
+template <class E>
+int unfold_launch(nxh_context *ctx, const char *op, const WindowArgs &a, int kt) {
+  int rows_per_block = 1;
+  int64_t wblocks = (a.L + 256 * WINDOWS_PER_LANE - 1) / (256 * WINDOWS_PER_LANE), blocks = a.rows * wblocks;
+  if (a.L <= 128) {  // short rows: a power-of-two share of the block per row
+    int lanes = 1;
+    while (lanes < a.L) lanes <<= 1;
+    rows_per_block = 256 / lanes;
+    blocks = (a.rows + rows_per_block - 1) / rows_per_block;
+  }
+  if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  const dim3 grid((unsigned)blocks), block(256);
+  const bool narrow = fits_int32(a);
+#define NXH_UNFOLD_CASE(KT)                                                                                 \
+  case KT:                                                                                                  \
+    if (narrow)                                                                                             \
+      hipLaunchKernelGGL((unfold_kernel<E, int32_t, KT>), grid, block, 0, ctx->stream, a, (int32_t)wblocks, \
+                         rows_per_block);                                                                   \
+    else                                                                                                    \
+      hipLaunchKernelGGL((unfold_kernel<E, int64_t, KT>), grid, block, 0, ctx->stream, a, wblocks,          \
+                         rows_per_block);                                                                   \
+    break;
+  switch (kt) {
+    NXH_UNFOLD_CASE(1)
+    NXH_UNFOLD_CASE(2)
+    NXH_UNFOLD_CASE(3)
+    NXH_UNFOLD_CASE(WIN_MAXK)
+  }
+#undef NXH_UNFOLD_CASE
+  return NXH_OK;
+}
+
+// Parameters common to both directions. `plain` is the un-windowed tensor
+// (unfold's input, fold's output), `cols` the windowed one. Returns the
+// kernels' compile-time rank in *kt.
+int window_setup(const char *op, const nxh_tensor *plain, const nxh_tensor *cols, int K, const int64_t *spatial,
+                 const int64_t *kernel, const int64_t *stride, const int64_t *dilation, const int64_t *padding,
+                 WindowArgs &a, int *kt) {
+  if (K < 1 || plain->ndim < K || cols->ndim < 2) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  const int ld = plain->ndim - K;
+  if (cols->ndim != ld + 2) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  if (K > WIN_MAXK || ld > WIN_MAXLEAD) return nxh_fail(NXH_FAILURE, op, "more than 6 window or 8 leading dimensions");
+  a.ld = ld;
+  for (int d = 0; d < ld; d++) {
+    if (plain->shape[d] != cols->shape[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    a.lshape[d] = plain->shape[d];
+  }
+  const int KT = rank_class(K), shift = KT - K;
+  *kt = KT;
+  for (int d = 0; d < WIN_MAXK; d++) {
+    a.kernel[d] = a.stride[d] = a.dilation[d] = a.win[d] = a.extent[d] = 1;
+    a.before[d] = a.step[d] = a.sp_stride[d] = a.win_cp[d] = 0;
+  }
+  int64_t kp = 1, L = 1;
+  for (int d = 0; d < K; d++) {
+    if (kernel[d] < 1 || stride[d] < 1 || dilation[d] < 1 || padding[2 * d] < 0 || padding[2 * d + 1] < 0)
+      return nxh_fail(NXH_INVALID_ARGUMENT, op, "kernel, stride and dilation must be positive, padding non-negative");
+    const int s = d + shift;
+    a.kernel[s] = kernel[d];
+    a.stride[s] = stride[d];
+    a.dilation[s] = dilation[d];
+    a.before[s] = padding[2 * d];
+    a.extent[s] = spatial[d];
+    if (plain->shape[ld + d] != spatial[d]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    a.sp_stride[s] = plain->strides[ld + d];
+    const int64_t eff = dilation[d] * (kernel[d] - 1) + 1;
+    const int64_t padded = spatial[d] + padding[2 * d] + padding[2 * d + 1];
+    const int64_t win = (padded - eff) / stride[d] + 1;
+    a.win[s] = win < 1 ? 1 : win;  // nx_c_move.c:640
+    kp *= kernel[d];
+    L *= a.win[s];
+  }
+  int64_t cp = 1, rest = 256;
+  for (int s = KT - 1; s >= 0; s--) {
+    a.win_cp[s] = cp;
+    cp *= a.win[s];
+    a.step[s] = rest % a.win[s];
+    rest /= a.win[s];
+  }
+  a.kernel_prod = cols->shape[ld];
+  a.L = cols->shape[ld + 1];
+  // the windowed tensor must hold exactly the taps and windows of this geometry
+  if (a.kernel_prod != kp || a.L != L) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  a.tap_stride = cols->strides[ld];
+  a.win_stride = cols->strides[ld + 1];
+  return NXH_OK;
+}
+
+}  // namespace
+
+NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int n_window_dims,
+                          const int64_t *kernel_size, const int64_t *stride, const int64_t *dilation,
+                          const int64_t *padding) {
+  const char *op = "unfold";
+  if (!ctx || !out || !x || !kernel_size || !stride || !dilation || !padding)
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (rc) return rc;
+  if (nxh_is_packed(out->dtype)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  if (x->dtype != out->dtype) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  WindowArgs a;
+  int kt = 0;
+  const int K = n_window_dims;
+  if (K < 1 || x->ndim < K) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  if ((rc = window_setup(op, x, out, K, &x->shape[x->ndim - K], kernel_size, stride, dilation, padding, a, &kt))) return rc;
+  for (int d = 0; d < out->ndim; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  const int es = (int)nxh_elem_size(out->dtype);
+  for (int d = 0; d < a.ld; d++) {
+    a.l_in[d] = x->strides[d];
+    a.l_out[d] = out->strides[d];
+  }
+  a.rows = a.kernel_prod;
+  for (int d = 0; d < a.ld; d++) a.rows *= a.lshape[d];
+  a.total = a.rows * a.L;
+  if (a.total == 0) return NXH_OK;
+  if (a.total > 0x7fffffffLL * 256) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  a.in = (const char *)x->data + x->offset * es;
+  a.out = (char *)out->data + out->offset * es;
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("unfold");
+  switch (es) {
+    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt); break;
+    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt); break;
+    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt); break;
+    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt); break;
+    default: rc = unfold_launch<G16w>(ctx, op, a, kt); break;
+  }
+  if (rc) return rc;
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+NXH_EXPORT int nxh_fold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int n_window_dims,
+                        const int64_t *output_size, const int64_t *kernel_size, const int64_t *stride,
+                        const int64_t *dilation, const int64_t *padding) {
+  const char *op = "fold";
+  if (!ctx || !out || !x || !output_size || !kernel_size || !stride || !dilation || !padding)
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  int rc = nxh_check_tensor(op, out);
+  if (!rc) rc = nxh_check_tensor(op, x);
+  if (rc) return rc;
+  const int dt = out->dtype;
+  if (nxh_is_packed(dt)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
+  if (x->dtype != dt) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  WindowArgs a;
+  int kt = 0;
+  const int K = n_window_dims;
+  if ((rc = window_setup(op, out, x, K, output_size, kernel_size, stride, dilation, padding, a, &kt))) return rc;
+  for (int d = 0; d < out->ndim; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  const int es = (int)nxh_elem_size(dt);
+  for (int d = 0; d < a.ld; d++) {
+    a.l_in[d] = x->strides[d];
+    a.l_out[d] = out->strides[d];
+  }
+  a.total = 1;
+  for (int d = 0; d < a.ld; d++) a.total *= a.lshape[d];
+  a.rows = a.total * a.kernel_prod;
+  for (int d = 0; d < K; d++) a.total *= output_size[d];
+  if (a.total == 0) return NXH_OK;
+  if (a.total > 0x7fffffffLL * 256) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  a.in = (const char *)x->data + x->offset * es;
+  a.out = (char *)out->data + out->offset * es;
+  struct Table {
+    fold_launch_fn fn[NXH_DTYPE_COUNT] = {};
+    Table() {
+#define NXH_FD(DT) fn[DT] = &fold_launch<DT>;
+      NXH_FOR_COMPUTE_DTYPES(NXH_FD)
+#undef NXH_FD
+    }
+  };
+  static const Table table;
+  if (!table.fn[dt]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("fold");
+  table.fn[dt](ctx, a, kt);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}

@@ -319,6 +319,54 @@ class Backend:
         self._check(self._lib.nxh_threefry(self._h, C.byref(o), C.byref(k), C.byref(c)))
         return out
 
+    # ── sort (nx_backend.ml:330-338) ─────────────────────────────────────────
+    def sort(self, x: Tensor, axis: int, descending: bool) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_sort(self._h, C.byref(o), C.byref(a), axis, int(descending)))
+        return out
+
+    def argsort(self, x: Tensor, axis: int, descending: bool) -> Tensor:
+        out = self.buffer(dt.int32, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_argsort(self._h, C.byref(o), C.byref(a), axis, int(descending)))
+        return out
+
+    # ── windows (nx_backend.ml:427-464) ──────────────────────────────────────
+    @staticmethod
+    def _window_params(op, in_shape, kernel_size, stride, dilation, padding):
+        k = len(kernel_size)
+        if not (len(stride) == len(dilation) == len(padding) == k) or k < 1 or len(in_shape) < k:
+            raise ValueError(f"{op}: shape mismatch")
+        spatial = in_shape[len(in_shape) - k:]
+        windows, taps = 1, 1
+        for i in range(k):
+            padded = spatial[i] + padding[i][0] + padding[i][1]
+            extent = dilation[i] * (kernel_size[i] - 1) + 1
+            windows *= (padded - extent) // stride[i] + 1
+            taps *= kernel_size[i]
+        arr = lambda v: (C.c_int64 * len(v))(*[int(a) for a in v])
+        flat = [int(v) for pair in padding for v in pair]
+        return taps, windows, (arr(kernel_size), arr(stride), arr(dilation), arr(flat))
+
+    def unfold(self, x: Tensor, kernel_size, stride, dilation, padding) -> Tensor:
+        taps, windows, params = self._window_params("unfold", x.shape, kernel_size, stride, dilation, padding)
+        out = self.buffer(x.dtype, tuple(x.shape[:len(x.shape) - len(kernel_size)]) + (taps, windows))
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_unfold(self._h, C.byref(o), C.byref(a), len(kernel_size), *params))
+        return out
+
+    def fold(self, x: Tensor, output_size, kernel_size, stride, dilation, padding) -> Tensor:
+        if len(x.shape) < 2:
+            raise ValueError("fold: shape mismatch")
+        oshape = tuple(x.shape[:-2]) + tuple(int(s) for s in output_size)
+        _, _, params = self._window_params("fold", oshape, kernel_size, stride, dilation, padding)
+        out = self.buffer(x.dtype, oshape)
+        osz = (C.c_int64 * len(output_size))(*[int(s) for s in output_size])
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_fold(self._h, C.byref(o), C.byref(a), len(kernel_size), osz, *params))
+        return out
+
     # ── fused sequences of primitives (no counterpart in Backend_intf.S) ────
     def _scalar_arg(self, dtype: dt.DType, value):
         if value is None:

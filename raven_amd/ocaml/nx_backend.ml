@@ -6,12 +6,10 @@
    OCaml toolchain); raven_amd/nx_backend.py is its executable twin and is what
    the parity tests drive.
 
-   Only the operations of the eager hot path are wired to the GPU. The
-   remaining members of Backend_intf.S (sort, scan, pad, cat, scatter, unfold,
-   fold, threefry, fft, linalg) must exist for the module to satisfy the
-   signature; until they have device kernels they are answered by copying to the
-   host, calling the C backend's routine and copying back, and are omitted from
-   this excerpt. *)
+   Every member of Backend_intf.S except the fft and linalg families is wired to
+   the GPU. Those two must exist for the module to satisfy the signature; until
+   they have device kernels they are answered by copying to the host, calling
+   the C backend's routine and copying back, and are omitted from this excerpt. *)
 
 open Nx_core
 
@@ -103,6 +101,13 @@ external caml_cat : ('a, 'b) t -> ('a, 'b) t array -> int -> unit = "caml_nx_hip
 external caml_scan : int -> ('a, 'b) t -> ('a, 'b) t -> int -> unit = "caml_nx_hip_scan"
 external caml_threefry :
   (int32, Dtype.int32_elt) t -> (int32, Dtype.int32_elt) t -> (int32, Dtype.int32_elt) t -> unit = "caml_nx_hip_threefry"
+external caml_sort : ('a, 'b) t -> ('a, 'b) t -> int -> bool -> unit = "caml_nx_hip_sort"
+external caml_argsort : (int32, Dtype.int32_elt) t -> ('a, 'b) t -> int -> bool -> unit = "caml_nx_hip_argsort"
+external caml_unfold : ('a, 'b) t -> ('a, 'b) t -> int array -> int array -> int array -> int array -> unit
+  = "caml_nx_hip_unfold_bc" "caml_nx_hip_unfold"
+external caml_fold_window :
+  ('a, 'b) t -> ('a, 'b) t -> int array -> int array -> int array -> int array -> int array -> unit
+  = "caml_nx_hip_fold_bc" "caml_nx_hip_fold"
 (* ... one external per remaining unary / binary / compare stub, same shapes ... *)
 
 let unary op x = let out = create_tensor x.context x.dtype x.shape in op out x; out
@@ -197,3 +202,35 @@ let scatter ~mode ~unique_indices:_ template ~indices ~updates ~axis =
 let threefry key counter =
   let out = create_tensor counter.context Dtype.Int32 counter.shape in
   caml_threefry out key counter; out
+
+(* nx_backend.ml:330-338 *)
+let sort ~axis ~descending x =
+  let out = create_tensor x.context x.dtype x.shape in
+  caml_sort out x axis descending; out
+
+let argsort ~axis ~descending x =
+  let out = create_tensor x.context Dtype.Int32 x.shape in
+  caml_argsort out x axis descending; out
+
+(* nx_backend.ml:427-464 *)
+let flatten_pairs p = Array.concat (Array.to_list (Array.map (fun (a, b) -> [| a; b |]) p))
+
+let unfold x ~kernel_size ~stride ~dilation ~padding =
+  let k = Array.length kernel_size in
+  let leading_ndim = Array.length x.shape - k in
+  let windows = ref 1 in
+  for i = 0 to k - 1 do
+    let before, after = padding.(i) in
+    let padded = x.shape.(leading_ndim + i) + before + after in
+    let extent = (dilation.(i) * (kernel_size.(i) - 1)) + 1 in
+    windows := !windows * (((padded - extent) / stride.(i)) + 1)
+  done;
+  let taps = Array.fold_left ( * ) 1 kernel_size in
+  let out = create_tensor x.context x.dtype
+      (Array.append (Array.sub x.shape 0 leading_ndim) [| taps; !windows |]) in
+  caml_unfold out x kernel_size stride dilation (flatten_pairs padding); out
+
+let fold x ~output_size ~kernel_size ~stride ~dilation ~padding =
+  let leading = Array.sub x.shape 0 (Array.length x.shape - 2) in
+  let out = create_tensor x.context x.dtype (Array.append leading output_size) in
+  caml_fold_window out x output_size kernel_size stride dilation (flatten_pairs padding); out

@@ -32,7 +32,8 @@
   X(context_create) X(context_destroy) X(last_error) X(alloc) X(free)         \
   X(memcpy_h2d) X(memcpy_d2h) X(synchronize) X(fill) X(unary) X(binary)       \
   X(compare) X(where) X(cast) X(reduce) X(argreduce) X(matmul) X(copy)        \
-  X(gather) X(scatter) X(pad) X(cat) X(scan) X(threefry) X(dtype_bytes)
+  X(gather) X(scatter) X(pad) X(cat) X(scan) X(threefry) X(dtype_bytes)       \
+  X(sort) X(argsort) X(unfold) X(fold)
 static struct {
 #define X(n) __typeof__(nxh_##n) *n;
   NXH_SYMBOLS(X)
@@ -332,4 +333,71 @@ CAMLprim value caml_nx_hip_threefry(value vout, value vkey, value vctr) {
   extract(vctr, &t);
   check(c, L.threefry(c, &o, &k, &t));
   CAMLreturn(Val_unit);
+}
+
+/* sort / argsort: same shape as caml_nx_c_sort / caml_nx_c_argsort (nx_c_sort.c:472-514) */
+CAMLprim value caml_nx_hip_sort(value vout, value vx, value vaxis, value vdesc) {
+  CAMLparam4(vout, vx, vaxis, vdesc);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.sort(c, &o, &x, Int_val(vaxis), Bool_val(vdesc)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_argsort(value vout, value vx, value vaxis, value vdesc) {
+  CAMLparam4(vout, vx, vaxis, vdesc);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.argsort(c, &o, &x, Int_val(vaxis), Bool_val(vdesc)));
+  CAMLreturn(Val_unit);
+}
+
+/* int array -> int64_t[], at most `cap` entries; returns the length */
+static int long_array(value v, int64_t *dst, int cap) {
+  int n = (int)Wosize_val(v);
+  if (n > cap) caml_failwith("ndim exceeds NX_C_MAX_NDIM");
+  for (int i = 0; i < n; i++) dst[i] = Long_val(Field(v, i));
+  return n;
+}
+/* windows: arguments as caml_nx_c_unfold / caml_nx_c_fold (nx_c_move.c:789-870),
+   padding already flattened to [before0; after0; ...] by the OCaml side */
+CAMLprim value caml_nx_hip_unfold(value vout, value vx, value vkernel, value vstride, value vdilation,
+                                  value vpadding) {
+  CAMLparam5(vout, vx, vkernel, vstride, vdilation);
+  CAMLxparam1(vpadding);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int64_t kernel[NXH_MAX_NDIM], stride[NXH_MAX_NDIM], dilation[NXH_MAX_NDIM], padding[2 * NXH_MAX_NDIM];
+  int k = long_array(vkernel, kernel, NXH_MAX_NDIM);
+  if (long_array(vstride, stride, NXH_MAX_NDIM) != k || long_array(vdilation, dilation, NXH_MAX_NDIM) != k ||
+      long_array(vpadding, padding, 2 * NXH_MAX_NDIM) != 2 * k)
+    caml_invalid_argument("unfold: shape mismatch");
+  check(c, L.unfold(c, &o, &x, k, kernel, stride, dilation, padding));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_unfold_bc(value *argv, int argn) {
+  (void)argn;
+  return caml_nx_hip_unfold(argv[0], argv[1], argv[2], argv[3], argv[4], argv[5]);
+}
+CAMLprim value caml_nx_hip_fold(value vout, value vx, value vosize, value vkernel, value vstride,
+                                value vdilation, value vpadding) {
+  CAMLparam5(vout, vx, vosize, vkernel, vstride);
+  CAMLxparam2(vdilation, vpadding);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int64_t osize[NXH_MAX_NDIM], kernel[NXH_MAX_NDIM], stride[NXH_MAX_NDIM], dilation[NXH_MAX_NDIM],
+      padding[2 * NXH_MAX_NDIM];
+  int k = long_array(vkernel, kernel, NXH_MAX_NDIM);
+  if (long_array(vosize, osize, NXH_MAX_NDIM) != k || long_array(vstride, stride, NXH_MAX_NDIM) != k ||
+      long_array(vdilation, dilation, NXH_MAX_NDIM) != k || long_array(vpadding, padding, 2 * NXH_MAX_NDIM) != 2 * k)
+    caml_invalid_argument("fold: shape mismatch");
+  check(c, L.fold(c, &o, &x, k, osize, kernel, stride, dilation, padding));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_fold_bc(value *argv, int argn) {
+  (void)argn;
+  return caml_nx_hip_fold(argv[0], argv[1], argv[2], argv[3], argv[4], argv[5], argv[6]);
 }

@@ -691,3 +691,106 @@ def test_scatter_reference_vectors_and_brute_force():
     with pytest.raises(RuntimeError, match="out of bounds"):
         B.scatter("set", False, _mk(B, np.zeros((1, 4)), dt.float64), _mk(B, bad, dt.int32),
                   _mk(B, np.ones((1, 1)), dt.float64), 1)
+
+
+def _nanlist(v):
+    return np.array([[float(c) for c in e] if isinstance(e, list) else float(e) for e in v])
+
+
+def _sort_case_arrays(c):
+    d = getattr(dt, c["dtype"])
+    x, want = _nanlist(c["x"]), _nanlist(c["out"])
+    if d.is_complex:
+        x, want = (x[:, 0] + 1j * x[:, 1]).astype(np.complex64), (want[:, 0] + 1j * want[:, 1]).astype(np.complex64)
+    return d, x, want
+
+
+def test_sort_reference_vectors_and_numpy():
+    B = OracleBackend()
+    for c in GOLD["sort"]["cases"]:
+        d, x, want = _sort_case_arrays(c)
+        got = logical(B.sort(_mk(B, x, d), 0, c["descending"]))
+        assert np.array_equal(got, want, equal_nan=True), c["name"]
+    t = GOLD["sort"]["complex_ties_nan"]
+    x = _nanlist(t["x"])
+    got = logical(B.sort(_mk(B, (x[:, 0] + 1j * x[:, 1]).astype(np.complex64), dt.complex64), 0, False))
+    pre = _nanlist(t["finite_prefix"])
+    assert np.array_equal(got[:len(pre)], (pre[:, 0] + 1j * pre[:, 1]).astype(np.complex64))
+    assert np.all(np.isnan(got[len(pre):].real) | np.isnan(got[len(pre):].imag))
+    a = GOLD["sort"]["argsort_int32"]
+    idx = logical(B.argsort(_mk(B, np.array(a["x"], np.int32), dt.int32), 0, False))
+    assert [a["x"][i] for i in idx] == a["gathered"]
+    # against numpy on every axis: values, stable indices, both directions,
+    # NaNs last both ways, unsigned high bits, bool
+    rng = np.random.default_rng(60)
+    for d, arr in ((dt.int32, rng.integers(-5, 5, (4, 7, 3)).astype(np.int32)),
+                   (dt.uint32, rng.integers(0, 2**32, (4, 7, 3), dtype=np.uint64).astype(np.uint32)),
+                   (dt.uint8, rng.integers(0, 4, (4, 7, 3)).astype(np.uint8)),
+                   (dt.bool_, rng.integers(0, 2, (4, 7, 3)).astype(np.uint8))):
+        for ax in range(3):
+            neg = arr.astype(np.int64) * -1
+            assert np.array_equal(logical(B.sort(_mk(B, arr, d), ax, False)), np.sort(arr, axis=ax))
+            assert np.array_equal(logical(B.sort(_mk(B, arr, d), ax, True)), np.flip(np.sort(arr, axis=ax), ax))
+            assert np.array_equal(logical(B.argsort(_mk(B, arr, d), ax, False)), np.argsort(arr, axis=ax, kind="stable"))
+            assert np.array_equal(logical(B.argsort(_mk(B, arr, d), ax, True)), np.argsort(neg, axis=ax, kind="stable"))
+    f = rng.standard_normal((6, 40)).astype(np.float32)
+    f[rng.random(f.shape) < 0.2] = np.nan
+    f[0, :5] = [0.0, -0.0, 0.0, np.inf, -np.inf]
+    got = logical(B.sort(_mk(B, f, dt.float32), 1, False))
+    assert np.array_equal(got, np.sort(f, axis=1), equal_nan=True)  # numpy also puts NaN last
+    got = logical(B.sort(_mk(B, f, dt.float32), 1, True))
+    for r in range(6):
+        fin = f[r][~np.isnan(f[r])]
+        assert np.array_equal(got[r][:fin.size], np.sort(fin)[::-1]) and np.all(np.isnan(got[r][fin.size:]))
+    ia = logical(B.argsort(_mk(B, f, dt.float32), 1, True))
+    for r in range(6):
+        key = np.where(np.isnan(f[r]), np.inf, -f[r].astype(np.float64))  # NaN last, descending otherwise
+        assert np.array_equal(ia[r], np.argsort(key, kind="stable"))
+    with pytest.raises(ValueError):
+        B.sort(_mk(B, f, dt.float32), 2, False)
+
+
+def test_window_reference_vectors_and_brute_force():
+    B = OracleBackend()
+    W = GOLD["window"]
+    for c in W["cases"]:
+        got = B.unfold(_mk(B, np.array(c["x"]), dt.float64), c["kernel"], c["stride"], c["dilation"],
+                       [tuple(p) for p in c["padding"]])
+        assert logical(got).tolist() == c["out"], c["name"]
+    c = W["fold_inverts_unfold"]
+    x = np.array(c["x"])
+    u = B.unfold(_mk(B, x, dt.float64), c["kernel"], c["stride"], [1], [(0, 0)])
+    assert np.array_equal(logical(B.fold(u, [x.shape[1]], c["kernel"], c["stride"], [1], [(0, 0)])), x)
+    # fold(unfold(x))[i] = coverage[i] * x[i] (backend_contract.ml:1861-1890)
+    for leading, length, k, s in W["fold_overlap"]:
+        x = ((np.arange(leading * length) % 13) + 1).astype(np.float64).reshape(leading, length)
+        u = B.unfold(_mk(B, x, dt.float64), [k], [s], [1], [(0, 0)])
+        f = logical(B.fold(u, [length], [k], [s], [1], [(0, 0)]))
+        nwin = (length - k) // s + 1
+        cover = np.array([sum(1 for w in range(nwin) if w * s <= j < w * s + k) for j in range(length)])
+        assert np.array_equal(f, x * cover)
+    # two window dims with stride, dilation and asymmetric padding, against a direct numpy im2col
+    rng = np.random.default_rng(61)
+    x = rng.standard_normal((2, 3, 7, 9))
+    ks, st, dl, pd = [3, 2], [2, 1], [1, 2], [(1, 0), (2, 1)]
+    u = logical(B.unfold(_mk(B, x, dt.float64), ks, st, dl, pd))
+    xp = np.pad(x, ((0, 0), (0, 0), pd[0], pd[1]))
+    oh = (xp.shape[2] - (dl[0] * (ks[0] - 1) + 1)) // st[0] + 1
+    ow = (xp.shape[3] - (dl[1] * (ks[1] - 1) + 1)) // st[1] + 1
+    want = np.zeros((2, 3, ks[0] * ks[1], oh * ow))
+    for a in range(ks[0]):
+        for b in range(ks[1]):
+            for i in range(oh):
+                for j in range(ow):
+                    want[:, :, a * ks[1] + b, i * ow + j] = xp[:, :, i * st[0] + a * dl[0], j * st[1] + b * dl[1]]
+    assert u.shape == want.shape and np.array_equal(u, want)
+    # fold is the adjoint of unfold: <unfold(x), y> = <x, fold(y)>, and on integers exactly col2im
+    y = rng.integers(-9, 9, want.shape).astype(np.int32)
+    f = logical(B.fold(_mk(B, y, dt.int32), [7, 9], ks, st, dl, pd))
+    acc = np.zeros(xp.shape, np.int64)
+    for a in range(ks[0]):
+        for b in range(ks[1]):
+            for i in range(oh):
+                for j in range(ow):
+                    acc[:, :, i * st[0] + a * dl[0], j * st[1] + b * dl[1]] += y[:, :, a * ks[1] + b, i * ow + j]
+    assert np.array_equal(f, acc[:, :, pd[0][0]:pd[0][0] + 7, pd[1][0]:pd[1][0] + 9].astype(np.int32))
