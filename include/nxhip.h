@@ -281,6 +281,21 @@ int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tenso
 int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
                   const void *constants);
 
+/* kaun/lib/attention.ml:67-110 for f16 / bf16 operands, as one kernel that never
+   writes the score tensor:
+     out = matmul (cast dtype (softmax (where mask (matmul (cast f32 q)
+           (transpose (cast f32 k)) * scale) masked_value))) v
+   q, out: [batch..., Sq, D]; k, v: [batch..., Sk, D]; D in {32, 64, 128}; rows
+   contiguous and 16-byte aligned, any other strides (head-split views are fine).
+   `scale` and `masked_value` are float32 elements in host memory (the scalars
+   of the float32 island), scale may be NULL. Either `mask` (bool,
+   [batch..., Sq, Sk], stride-0 broadcast allowed) or `causal` != 0 (mask[i][j]
+   = j <= i, generated; needs Sq == Sk; key tiles above the diagonal are
+   skipped), or neither. */
+int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q,
+                  const nxh_tensor *k, const nxh_tensor *v, const void *scale,
+                  const nxh_tensor *mask, const void *masked_value, int causal);
+
 /* ── measurement ─────────────────────────────────────────────────────────── */
 
 /* HIP events recorded on the context stream: start, then stop returns the

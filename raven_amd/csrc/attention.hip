@@ -1,0 +1,330 @@
+// attention.hip — scaled dot-product attention for 16-bit operands as ONE
+// kernel that never writes the S x S score tensor.
+//
+// It stands for the sequence kaun/lib/attention.ml:67-110 issues for f16 / bf16
+// inputs, primitive by primitive:
+//   scores = matmul (cast f32 q) (transpose (cast f32 k))      -- f32
+//   scores = scores * scale                                     -- f32
+//   scores = where mask scores masked_value                     -- f32
+//   probs  = cast dtype (softmax scores)                        -- frontend.ml:4242-4252
+//   out    = matmul probs v                                     -- dtype, f32 accumulation
+// with the same rounding points: products of 16-bit values are exact in the
+// f32 accumulator of v_mfma_f32_32x32x16, the scale is one f32 multiply, the
+// exponentials are the primitive's expf of (t - rowmax), each probability is
+// e / rowsum rounded to the 16-bit dtype BEFORE it meets v, and the output is
+// rounded once from the f32 accumulator. What differs from the op-by-op result
+// is the order of the f32 sums (scores, row sum, probs x v) and that the row sum
+// is accumulated tile by tile against a running maximum.
+//
+// Layout of the work: a block of four wave64s owns 128 queries of one
+// (batch, head); each wave 32 of them. Keys are visited 64 at a time through
+// LDS (K as [key][d], V as [key][d] too and read back with the transposing LDS
+// load, so no operand is ever transposed in memory). The wave computes the
+// TRANSPOSED score tile S^T = K Q^T, so that a lane holds 16 scores of ONE
+// query (accumulator column = lane % 32): row maxima and sums are 16 in-lane
+// steps plus one exchange with lane ^ 32. Pass 1 walks the keys for the row
+// maximum and sum; pass 2 walks them again, forms the rounded probabilities in
+// registers, exchanges halves with lane ^ 32 to lay them out as the B operand
+// of O^T = V^T P^T, and accumulates the output. Recomputing Q K^T is cheap
+// next to the 2 x S x S x 4 bytes it saves. With `causal` the mask is generated from
+// indices and key tiles above the diagonal are skipped.
+
+#include "fold_common.hpp"
+#include "gemm_tile.hpp"
+#include "map_ops.hpp"
+
+namespace {
+
+using gemm_tile::f32x16;
+using gemm_tile::lds_s16x4;
+using gemm_tile::s16x4;
+using gemm_tile::V16;
+
+constexpr int ATT_MAXB = 4;   // outer (batch) dims
+constexpr int QUERIES = 128;  // per block
+constexpr int KEYS = 64;      // per LDS tile
+
+struct AttOperand {
+  const char *base;
+  int64_t outer[ATT_MAXB];  // strides of the outer dims, elements
+  int64_t row;              // stride of the sequence dim
+};
+struct AttArgs {
+  AttOperand q, k, v, out, mask;
+  int64_t mask_col;  // stride of the mask along keys
+  int nouter;
+  uint32_t oshape[ATT_MAXB];
+  int64_t batches;
+  int sq, sk, qtiles;
+  int causal, has_mask, has_scale;
+  float scale, masked;
+};
+
+template <class EL>
+__device__ __forceinline__ uint16_t narrow(float x) {
+  return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x);
+}
+
+__device__ __forceinline__ float xor32(float v) {
+  return __builtin_bit_cast(float, __shfl_xor(__builtin_bit_cast(int, v), 32, 64));
+}
+
+template <class EL, int DHEAD>
+__global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
+  using S = uint16_t;
+  using MX = Combine<NXH_RMAX, float, CAT_FLOAT>;
+  constexpr int KSTEPS = DHEAD / 16;  // k-steps of Q K^T
+  constexpr int OT = DHEAD / 32;      // 32-row tiles of O^T
+  constexpr int PK = DHEAD + 8;       // pitch of K in LDS ([key][d], read along d)
+  constexpr int PV = DHEAD + 16;      // pitch of V in LDS ([key][d], read transposed)
+  constexpr int VPR = DHEAD / 8;      // 16-byte vectors per row
+  __shared__ __attribute__((aligned(16))) S Ks[KEYS * PK];
+  __shared__ __attribute__((aligned(16))) S Vs[KEYS * PV];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c32 = lane & 31, g = lane >> 5;
+  // heavy (late) query tiles first: with a causal mask they have the most keys
+  const int64_t bid = (int64_t)gridDim.x - 1 - blockIdx.x;
+  const int qt = (int)(bid % a.qtiles);
+  int64_t batch = bid / a.qtiles;
+  int64_t qo = 0, ko = 0, vo = 0, oo = 0, mo = 0;
+  for (int d = a.nouter - 1; d >= 0; d--) {
+    const int64_t c = batch % a.oshape[d];
+    batch /= a.oshape[d];
+    qo += c * a.q.outer[d];
+    ko += c * a.k.outer[d];
+    vo += c * a.v.outer[d];
+    oo += c * a.out.outer[d];
+    mo += c * a.mask.outer[d];
+  }
+  const S *Q = reinterpret_cast<const S *>(a.q.base) + qo;
+  const S *K = reinterpret_cast<const S *>(a.k.base) + ko;
+  const S *V = reinterpret_cast<const S *>(a.v.base) + vo;
+  S *O = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
+  const uint8_t *M = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
+
+  const int q0 = qt * QUERIES, qw = q0 + wave * 32;  // first query of the block / wave
+  const int qi = qw + c32;                           // this lane's query
+  const int qrow = qi < a.sq ? qi : a.sq - 1;        // clamp: rows past the end are never stored
+  // Q fragments: B operand of S^T = K Q^T, this lane's 8 d-values per k-step
+  V16 qf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; s++)
+    qf[s] = *reinterpret_cast<const V16 *>(Q + (int64_t)qrow * a.q.row + s * 16 + g * 8);
+
+  // keys this block needs: all, or up to its last query under a causal mask
+  const int klimit = a.causal ? (q0 + QUERIES < a.sk ? q0 + QUERIES : a.sk) : a.sk;
+  const int ktiles = (klimit + KEYS - 1) / KEYS;
+
+  float m_run = MX::init(), l_run = 0.0f;
+  f32x16 oacc[OT];
+#pragma unroll
+  for (int t = 0; t < OT; t++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) oacc[t][e] = 0.0f;
+
+  // One 32-key sub-tile of scores for this wave: t[e] is the masked, scaled
+  // score of key j0 + (e/4)*8 + g*4 + e%4 against query qi.
+  auto scores = [&](int j0, float (&t)[16]) {
+    f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    const S *kr = Ks + (j0 % KEYS + c32) * PK + g * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++) {
+      const V16 kf = *reinterpret_cast<const V16 *>(kr + s * 16);
+      gemm_tile::mfma_step<EL>(acc, kf, qf[s]);
+    }
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const int j = j0 + (e >> 2) * 8 + g * 4 + (e & 3);
+      float x = acc[e];
+      if (a.has_scale) x = x * a.scale;
+      bool keep = true;
+      if (a.causal) keep = j <= qi;
+      else if (a.has_mask) keep = M[(int64_t)qrow * a.mask.row + (int64_t)(j < a.sk ? j : a.sk - 1) * a.mask_col] != 0;
+      x = keep ? x : a.masked;
+      t[e] = j < a.sk ? x : -__builtin_inff();  // keys past the end do not exist
+    }
+  };
+
+  for (int pass = 0; pass < 2; pass++) {
+    float l_total = 0.0f;
+    if (pass == 1) l_total = l_run + xor32(l_run);
+    for (int kt = 0; kt < ktiles; kt++) {
+      __syncthreads();  // the previous tile has been consumed
+      for (int v = threadIdx.x; v < KEYS * VPR; v += 256) {
+        const int r = v / VPR, c = (v % VPR) * 8;
+        int key = kt * KEYS + r;
+        key = key < a.sk ? key : a.sk - 1;
+        *reinterpret_cast<V16 *>(Ks + r * PK + c) = *reinterpret_cast<const V16 *>(K + (int64_t)key * a.k.row + c);
+        if (pass == 1)
+          *reinterpret_cast<V16 *>(Vs + r * PV + c) = *reinterpret_cast<const V16 *>(V + (int64_t)key * a.v.row + c);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int sub = 0; sub < KEYS / 32; sub++) {
+        const int j0 = kt * KEYS + sub * 32;
+        // nothing of this sub-tile is visible to the wave's queries
+        if (j0 >= a.sk || (a.causal && j0 > qw + 31)) continue;
+        float t[16];
+        scores(j0, t);
+        if (pass == 0) {
+          float tm = t[0];
+#pragma unroll
+          for (int e = 1; e < 16; e++) tm = MX::apply(tm, t[e]);
+          float m_new = MX::apply(m_run, tm);
+          m_new = MX::apply(m_new, xor32(m_new));  // both halves of a query agree on the maximum
+          if (m_new != -__builtin_inff()) {
+            float s = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; e++) s = s + OpExp::eval<CAT_FLOAT, float>(t[e] - m_new);
+            l_run = l_run * OpExp::eval<CAT_FLOAT, float>(m_run - m_new) + s;
+          }
+          m_run = m_new;
+        } else {
+          // rounded probabilities, two per register, in accumulator order
+          uint32_t pk[8];
+#pragma unroll
+          for (int e = 0; e < 16; e += 2) {
+            const float p0 = OpExp::eval<CAT_FLOAT, float>(t[e] - m_run) / l_total;
+            const float p1 = OpExp::eval<CAT_FLOAT, float>(t[e + 1] - m_run) / l_total;
+            pk[e >> 1] = (uint32_t)narrow<EL>(p0) | ((uint32_t)narrow<EL>(p1) << 16);
+          }
+          // B operand of O^T = V^T P^T for k-step ks: this lane's query, keys
+          // ks*16 + g*8 + 0..7. The accumulator gave keys ks*16 + g*4 + 0..3 and
+          // ks*16 + 8 + g*4 + 0..3: swap one half with lane ^ 32.
+#pragma unroll
+          for (int ks = 0; ks < 2; ks++) {
+            const uint32_t a0 = pk[ks * 4 + 0], a1 = pk[ks * 4 + 1];  // keys g*4 + 0..3
+            const uint32_t b0 = pk[ks * 4 + 2], b1 = pk[ks * 4 + 3];  // keys 8 + g*4 + 0..3
+            const uint32_t s0 = g == 0 ? b0 : a0, s1 = g == 0 ? b1 : a1;
+            const uint32_t r0 = (uint32_t)__shfl_xor((int)s0, 32, 64), r1 = (uint32_t)__shfl_xor((int)s1, 32, 64);
+            const V16 pf = g == 0 ? V16{a0, a1, r0, r1} : V16{r0, r1, b0, b1};
+#pragma unroll
+            for (int ot = 0; ot < OT; ot++) {
+              // A operand: V^T rows d = ot*32 + lane%32, keys as above, by transposing LDS reads
+              const int kk = sub * 32 + ks * 16 + g * 8 + ((lane & 15) >> 2);
+              const int rr = ot * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+              const S *src = Vs + kk * PV + rr;
+              const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)src);
+              const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src + 4 * PV));
+              typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+              const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+              gemm_tile::mfma_step<EL>(oacc[ot], V16{l2[0], l2[1], h2[0], h2[1]}, pf);
+            }
+          }
+        }
+      }
+    }
+  }
+  // O^T element e of tile ot: d = ot*32 + (e/4)*8 + g*4 + e%4, query qi
+  if (qi < a.sq) {
+    S *orow = O + (int64_t)qi * a.out.row;
+#pragma unroll
+    for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+      for (int e = 0; e < 16; e += 4) {
+        const int d = ot * 32 + (e >> 2) * 8 + g * 4;
+        uint2 w;
+        w.x = (uint32_t)narrow<EL>(oacc[ot][e]) | ((uint32_t)narrow<EL>(oacc[ot][e + 1]) << 16);
+        w.y = (uint32_t)narrow<EL>(oacc[ot][e + 2]) | ((uint32_t)narrow<EL>(oacc[ot][e + 3]) << 16);
+        *reinterpret_cast<uint2 *>(orow + d) = w;
+      }
+  }
+}
+
+template <class EL>
+int attention_launch(nxh_context *ctx, const char *op, const AttArgs &a, int hd) {
+  const int64_t blocks = a.batches * a.qtiles;
+  if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  const dim3 grid((unsigned)blocks), block(256);
+  switch (hd) {
+    case 32: hipLaunchKernelGGL((attention_kernel<EL, 32>), grid, block, 0, ctx->stream, a); break;
+    case 64: hipLaunchKernelGGL((attention_kernel<EL, 64>), grid, block, 0, ctx->stream, a); break;
+    case 128: hipLaunchKernelGGL((attention_kernel<EL, 128>), grid, block, 0, ctx->stream, a); break;
+    default: return nxh_fail(NXH_FAILURE, op, "head dimension must be 32, 64 or 128");
+  }
+  return NXH_OK;
+}
+
+// Rows of `t` must be contiguous and 16-byte aligned (8-byte for the output).
+bool rows_aligned(const nxh_tensor *t, int bytes) {
+  const int nd = t->ndim;
+  if (t->shape[nd - 1] > 1 && t->strides[nd - 1] != 1) return false;
+  if ((((uintptr_t)t->data + t->offset * 2) % (uintptr_t)bytes) != 0) return false;
+  for (int d = 0; d < nd - 1; d++)
+    if (t->shape[d] > 1 && (t->strides[d] * 2) % bytes != 0) return false;
+  return true;
+}
+
+}  // namespace
+
+NXH_EXPORT int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q, const nxh_tensor *k,
+                             const nxh_tensor *v, const void *scale, const nxh_tensor *mask,
+                             const void *masked_value, int causal) {
+  const char *op = "attention";
+  if (!ctx || !out || !q || !k || !v || (mask && !masked_value) || (causal && !masked_value))
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
+  if (causal && mask) return nxh_fail(NXH_INVALID_ARGUMENT, op, "give either a mask or causal, not both");
+  int rc = NXH_OK;
+  for (const nxh_tensor *t : {out, q, k, v, mask})
+    if (t && !rc) rc = nxh_check_tensor(op, t);
+  if (rc) return rc;
+  const int dt = q->dtype, nd = q->ndim;
+  if ((dt != NXH_BF16 && dt != NXH_F16) || k->dtype != dt || v->dtype != dt || out->dtype != dt ||
+      (mask && mask->dtype != NXH_BOOL))
+    return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  if (nd < 2 || k->ndim != nd || v->ndim != nd || out->ndim != nd || (mask && mask->ndim != nd))
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  if (nd - 2 > ATT_MAXB) return nxh_fail(NXH_FAILURE, op, "more than 4 batch dimensions");
+  AttArgs a;
+  const int64_t sq = q->shape[nd - 2], sk = k->shape[nd - 2], hd = q->shape[nd - 1];
+  if (k->shape[nd - 1] != hd || v->shape[nd - 1] != hd || v->shape[nd - 2] != sk || out->shape[nd - 2] != sq ||
+      out->shape[nd - 1] != hd || (mask && (mask->shape[nd - 2] != sq || mask->shape[nd - 1] != sk)))
+    return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  a.batches = 1;
+  a.nouter = nd - 2;
+  for (int d = 0; d < nd - 2; d++) {
+    const int64_t e = q->shape[d];
+    if (k->shape[d] != e || v->shape[d] != e || out->shape[d] != e || (mask && mask->shape[d] != e))
+      return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    if (e > 0xffffffffLL) return nxh_fail(NXH_FAILURE, op, "extent exceeds 32 bits");
+    a.oshape[d] = (uint32_t)e;
+    a.batches *= e;
+  }
+  if (causal && sq != sk) return nxh_fail(NXH_INVALID_ARGUMENT, op, "causal needs as many queries as keys");
+  if (a.batches == 0 || sq == 0) return NXH_OK;
+  if (sk == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_EMPTY_REDUCE);
+  if (sq > 0x3fffffff || sk > 0x3fffffff) return nxh_fail(NXH_FAILURE, op, "sequence longer than 2^30");
+  for (int d = 0; d < nd; d++)
+    if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
+  if (!rows_aligned(q, 16) || !rows_aligned(k, 16) || !rows_aligned(v, 16) || !rows_aligned(out, 8))
+    return nxh_fail(NXH_FAILURE, op, "rows must be contiguous and 16-byte aligned");
+  auto operand = [&](const nxh_tensor *t, AttOperand &o, int es) {
+    o.base = t ? (const char *)t->data + t->offset * es : nullptr;
+    for (int d = 0; d < ATT_MAXB; d++) o.outer[d] = (t && d < nd - 2) ? t->strides[d] : 0;
+    o.row = t ? t->strides[nd - 2] : 0;
+  };
+  operand(q, a.q, 2);
+  operand(k, a.k, 2);
+  operand(v, a.v, 2);
+  operand(out, a.out, 2);
+  operand(mask, a.mask, 1);
+  a.mask_col = mask ? mask->strides[nd - 1] : 0;
+  a.sq = (int)sq;
+  a.sk = (int)sk;
+  a.qtiles = (int)((sq + QUERIES - 1) / QUERIES);
+  a.causal = causal ? 1 : 0;
+  a.has_mask = mask ? 1 : 0;
+  a.has_scale = scale ? 1 : 0;
+  a.scale = scale ? *(const float *)scale : 1.0f;
+  a.masked = masked_value ? *(const float *)masked_value : 0.0f;
+  std::lock_guard<std::mutex> guard(ctx->mu);
+  NXH_HIP(op, hipSetDevice(ctx->device));
+  nxh_set_path("attention_fused");
+  rc = dt == NXH_BF16 ? attention_launch<gemm_tile::ElBF16>(ctx, op, a, (int)hd)
+                      : attention_launch<gemm_tile::ElF16>(ctx, op, a, (int)hd);
+  if (rc) return rc;
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}

@@ -412,6 +412,20 @@ class Backend:
         self._check(self._lib.nxh_gelu_tanh(self._h, C.byref(o), C.byref(a), enc.ctypes.data))
         return out
 
+    def attention(self, q: Tensor, k: Tensor, v: Tensor, scale=None, mask: Tensor | None = None,
+                  masked_value=None, causal: bool = False) -> Tensor:
+        """Scaled dot-product attention of f16 / bf16 operands in one kernel
+        (the sequence of kaun/lib/attention.ml:67-110). ``scale`` and
+        ``masked_value`` are float32 scalars."""
+        out = self.buffer(q.dtype, q.shape)
+        keep_s, ps = self._scalar_arg(dt.float32, scale)
+        keep_m, pm = self._scalar_arg(dt.float32, masked_value)
+        o, a, b, c = out._desc(), q._desc(), k._desc(), v._desc()
+        m = mask._desc() if mask is not None else None
+        self._check(self._lib.nxh_attention(self._h, C.byref(o), C.byref(a), C.byref(b), C.byref(c), ps,
+                                            C.byref(m) if m is not None else None, pm, int(causal)))
+        return out
+
     # ── fold family (nx_backend.ml:266-307) ─────────────────────────────────
     def reduce(self, op: str, axes: Sequence[int], x: Tensor) -> Tensor:
         axes = sorted(int(a) for a in axes)

@@ -1,0 +1,116 @@
+"""The fused attention kernel through the C ABI against the sequence it stands
+for (kaun/lib/attention.ml:67-110: cast to float32, Q K^T, scale, mask, softmax,
+cast back, probs x V), run primitive by primitive on the CPU oracle and on the
+GPU backend. The rounding points are the same; only the order of the float32
+sums differs, so the results agree to about one unit of the 16-bit output."""
+
+import math
+
+import numpy as np
+import pytest
+
+from helpers import TOL, close, decode, encode, logical, pair
+from raven_amd import dtype as dt
+from raven_amd.kaun_gpt2 import Config, Gpt2
+from raven_amd.nx_frontend import Nx
+
+pytestmark = pytest.mark.gpu
+ULP = {"float16": 2.0 ** -10, "bfloat16": 2.0 ** -7}
+
+
+def sequence(B, q, k, v, mask):
+    return Gpt2(Nx(B), Config()).scaled_dot_product_attention(q, k, v, mask)
+
+
+def bool_mask(B, m, shape):
+    t = B.reshape(B.from_host(np.ascontiguousarray(m), dt.bool_), (1,) * (len(shape) - m.ndim) + m.shape)
+    return B.expand(t, shape)
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+@pytest.mark.parametrize("shape", [(2, 3, 100, 64), (1, 2, 256, 64), (2, 2, 130, 32), (1, 1, 64, 128), (3, 40, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_attention_matches_the_sequence(hip, oracle, d, shape):
+    rng = np.random.default_rng(sum(shape) + d.tag)
+    s, hd = shape[-2], shape[-1]
+    q, k, v = (encode(rng.standard_normal(shape), d, oracle) for _ in range(3))
+    (hq, oq), (hk, ok), (hv, ov) = (pair(x, d, hip, oracle) for x in (q, k, v))
+    scale = 1.0 / math.sqrt(hd)
+    tri = np.tril(np.ones((s, s), np.uint8))
+    rnd = (rng.random((s, s)) < 0.7).astype(np.uint8)
+    rnd[:, 0] = 1  # no row is masked out completely
+    sshape = tuple(shape[:-1]) + (s,)
+    for name, m, kwargs in (("causal", tri, {"causal": True, "masked_value": float("-inf")}),
+                            ("mask", rnd, None), ("none", None, {})):
+        hm = bool_mask(hip, m, sshape) if m is not None else None
+        om = bool_mask(oracle, m, sshape) if m is not None else None
+        if kwargs is None:
+            kwargs = {"mask": hm, "masked_value": float("-inf")}
+        got = logical(hip.attention(hq, hk, hv, scale, **kwargs))
+        assert hip.last_path() == "attention_fused"
+        want_gpu = logical(sequence(hip, hq, hk, hv, hm))
+        want_cpu = logical(sequence(oracle, oq, ok, ov, om))
+        what = f"{d.name} {shape} {name}"
+        close(got, want_gpu, d, oracle, 2 * ULP[d.name], 2e-3, what + " vs GPU sequence")
+        close(got, want_cpu, d, oracle, TOL[d.name][0], TOL[d.name][0], what + " vs oracle sequence")
+        same = np.mean(got == want_gpu)
+        assert same > 0.9, (what, same)
+    # causality: the output at position i does not see keys behind it
+    k2, v2 = k.copy(), v.copy()
+    k2[..., s // 2:, :] = encode(rng.standard_normal(k2[..., s // 2:, :].shape), d, oracle)
+    v2[..., s // 2:, :] = encode(rng.standard_normal(v2[..., s // 2:, :].shape), d, oracle)
+    a = logical(hip.attention(hq, hk, hv, scale, causal=True, masked_value=float("-inf")))
+    b = logical(hip.attention(hq, pair(k2, d, hip, oracle)[0], pair(v2, d, hip, oracle)[0], scale, causal=True,
+                              masked_value=float("-inf")))
+    assert np.array_equal(a[..., :s // 2, :], b[..., :s // 2, :])
+
+
+def test_attention_on_head_split_views_and_special_rows(hip, oracle):
+    """q, k, v as the strided views Kaun builds (reshape to heads, swap axes), a
+    fully masked row (NaN, as the sequence gives), and a finite masked value."""
+    rng = np.random.default_rng(5)
+    b, s, h, hd = 2, 96, 4, 64
+    d = dt.bfloat16
+    x = [encode(rng.standard_normal((b, s, h * hd)), d, oracle) for _ in range(3)]
+
+    def split(B, t):
+        return B.permute(B.reshape(t, (b, s, h, hd)), (0, 2, 1, 3))
+
+    hq, hk, hv = (split(hip, pair(a, d, hip, oracle)[0]) for a in x)
+    oq, ok, ov = (split(oracle, pair(a, d, hip, oracle)[1]) for a in x)
+    m = np.tril(np.ones((s, s), np.uint8))
+    m[7] = 0
+    hm, om = bool_mask(hip, m, (b, h, s, s)), bool_mask(oracle, m, (b, h, s, s))
+    scale = 0.125
+    got = logical(hip.attention(hq, hk, hv, scale, mask=hm, masked_value=float("-inf")))
+    want = logical(sequence(oracle, oq, ok, ov, om))
+    gv, wv = decode(got, d, oracle), decode(want, d, oracle)
+    assert np.isnan(gv[:, :, 7]).all() and np.isnan(wv[:, :, 7]).all()
+    close(got, want, d, oracle, TOL[d.name][0], TOL[d.name][0], "split views")
+    # a finite masked value takes part in the softmax
+    got = decode(logical(hip.attention(hq, hk, hv, scale, mask=hm, masked_value=-2.0)), d, oracle)
+    nx = Nx(oracle)
+    sc = nx.mul_s(nx.matmul(nx.cast(dt.float32, oq), nx.swapaxes(2, 3, nx.cast(dt.float32, ok))), scale)
+    pr = nx.cast(d, nx.softmax(nx.where(om, sc, nx.scalar_like(sc, -2.0))))
+    want = decode(logical(nx.matmul(pr, ov)), d, oracle)
+    assert np.all(np.abs(got - want) <= TOL[d.name][0] * (1 + np.abs(want)))
+
+
+def test_attention_errors(hip):
+    q = hip.full(dt.bfloat16, (2, 16, 64), 1.0)
+    with pytest.raises(RuntimeError):
+        hip.attention(hip.full(dt.float32, (2, 16, 64), 1.0), hip.full(dt.float32, (2, 16, 64), 1.0),
+                      hip.full(dt.float32, (2, 16, 64), 1.0))
+    with pytest.raises(ValueError):
+        hip.attention(q, hip.full(dt.bfloat16, (2, 16, 32), 1.0), q)
+    with pytest.raises(RuntimeError, match="head dimension"):
+        hip.attention(hip.full(dt.bfloat16, (2, 16, 48), 1.0), hip.full(dt.bfloat16, (2, 16, 48), 1.0),
+                      hip.full(dt.bfloat16, (2, 16, 48), 1.0))
+    with pytest.raises(ValueError, match="causal"):
+        hip.attention(q, hip.full(dt.bfloat16, (2, 8, 64), 1.0), hip.full(dt.bfloat16, (2, 8, 64), 1.0),
+                      causal=True, masked_value=float("-inf"))
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hip.attention(hip.permute(hip.full(dt.bfloat16, (2, 64, 16), 1.0), (0, 2, 1)), q, q)
+    # uniform values: every key gets the same weight, the output is v's mean (here v itself)
+    out = logical(hip.attention(q, q, q))
+    assert np.array_equal(out, logical(q))
