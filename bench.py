@@ -254,6 +254,26 @@ def next_ops(hip, W):
     timed("unfold [8,64,128,128] f32, 3x3 same (im2col)", lambda: hip.unfold(img, *geo), nin + ncols)
     cols = hip.unfold(img, *geo)
     timed("fold back to [8,64,128,128] (col2im, 9 taps per output)", lambda: hip.fold(cols, [128, 128], *geo), nin + ncols)
+    del img, cols
+    # fused attention and the row kernels at GPT-2-small's shapes (bf16, batch 8, seq 1024)
+    bf = lambda shape: W.dev((rng.standard_normal(shape).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16),
+                             dt.bfloat16)
+    b, h, sq, hd = 8, 12, 1024, 64
+    q, k, v = (hip.permute(hip.reshape(bf((b, sq, h * hd)), (b, sq, h, hd)), (0, 2, 1, 3)) for _ in range(3))
+    timed("attention [8,12,1024,64] bf16, causal, head-split views (attention_fused)",
+          lambda: hip.attention(q, k, v, 0.125, causal=True, masked_value=float("-inf")), 4 * b * sq * h * hd * 2)
+    useful = 4 * b * h * sq * (sq + 1) // 2 * hd  # Q K^T and probs x V over the visible half
+    out[-1].update({"bound": "mfma", "TFLOP/s": round(useful / (out[-1]["ms"] * 1e-3) / 1e12, 1),
+                    "frac_mfma_bf16": round(useful / (out[-1]["ms"] * 1e-3) / 1e12 / 2500.0, 4)})
+    scores = W.dev(rng.standard_normal((b * h * sq, sq)).astype(np.float32), dt.float32)
+    timed("softmax_rows [98304,1024] f32 -> bf16 with scale (fused)",
+          lambda: hip.softmax_rows(scores, 0.125, None, None, dt.bfloat16), b * h * sq * sq * 6)
+    del scores
+    x = bf((b * sq, 768))
+    gam, bet = bf((768,)), bf((768,))
+    timed("layer_norm_rows [8192,768] bf16 (fused)", lambda: hip.layer_norm_rows(x, gam, bet, 1e-5), 2 * b * sq * 768 * 2)
+    y = bf((b * sq, 3072))
+    timed("gelu_tanh [8192,3072] bf16 (fused)", lambda: hip.gelu_tanh(y), 2 * b * sq * 3072 * 2)
     return out
 
 
@@ -335,7 +355,7 @@ class CountingBackend:
     """Forwards to the backend and counts the calls that launch work."""
 
     LAUNCHING = ("unary", "binary", "compare", "where", "cast", "copy", "contiguous", "gather", "reduce",
-                 "matmul", "full", "from_host", "softmax_rows", "layer_norm_rows", "gelu_tanh")
+                 "matmul", "full", "from_host", "softmax_rows", "layer_norm_rows", "gelu_tanh", "attention")
 
     def __init__(self, inner):
         self._inner, self.calls = inner, {}
@@ -391,7 +411,7 @@ def config5(hip, iters=3, warmup=1, window=False):
     ms = (time.perf_counter() - t0) * 1e3 / iters
     calls = {k: v // iters for k, v in counter.calls.items()}
     flops = 284812800 * batch * seq  # matmul FLOPs per forward
-    how = ("deferred-evaluation window: softmax / layer norm / GELU sequences as fused row kernels" if window
+    how = ("deferred-evaluation window: attention, layer norm and GELU sequences as fused kernels" if window
            else "eager, one backend call per primitive")
     rec = {"op": f"cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 ({how})",
            "ms": round(ms, 3), "tokens/s": round(batch * seq / (ms * 1e-3), 1), "hip_event_ms": round(ev_ms, 3),

@@ -16,8 +16,9 @@
 // is the order of the f32 sums (scores, row sum, probs x v) and that the row sum
 // is accumulated tile by tile against a running maximum.
 //
-// Layout of the work: a block of four wave64s owns 128 queries of one
-// (batch, head); each wave 32 of them. Keys are visited 64 at a time through
+// Layout of the work: a block of four wave64s owns two 64-query tiles of one
+// (batch, head), tile t and tile T-1-t, so that every block meets the same
+// number of keys under a causal mask; each wave 32 queries. Keys are visited 64 at a time through
 // LDS (K as [key][d], V as [key][d] too and read back with the transposing LDS
 // load, so no operand is ever transposed in memory). The wave computes the
 // TRANSPOSED score tile S^T = K Q^T, so that a lane holds 16 scores of ONE
@@ -41,7 +42,6 @@ using gemm_tile::s16x4;
 using gemm_tile::V16;
 
 constexpr int ATT_MAXB = 4;   // outer (batch) dims
-constexpr int QUERIES = 128;  // per block
 constexpr int KEYS = 64;      // per LDS tile
 
 struct AttOperand {
@@ -83,8 +83,8 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c32 = lane & 31, g = lane >> 5;
   // heavy (late) query tiles first: with a causal mask they have the most keys
-  const int64_t bid = (int64_t)gridDim.x - 1 - blockIdx.x;
-  const int qt = (int)(bid % a.qtiles);
+  const int64_t bid = blockIdx.x;
+  const int pair = (int)(bid % a.qtiles);
   int64_t batch = bid / a.qtiles;
   int64_t qo = 0, ko = 0, vo = 0, oo = 0, mo = 0;
   for (int d = a.nouter - 1; d >= 0; d--) {
@@ -102,9 +102,16 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
   S *O = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
   const uint8_t *M = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
 
-  const int q0 = qt * QUERIES, qw = q0 + wave * 32;  // first query of the block / wave
-  const int qi = qw + c32;                           // this lane's query
-  const int qrow = qi < a.sq ? qi : a.sq - 1;        // clamp: rows past the end are never stored
+  // Waves 0-1 take the pair's low 64-query tile, waves 2-3 its high one (tile
+  // t pairs with tile T-1-t): under a causal mask every block then sees the
+  // same number of keys in total. The middle tile of an odd count pairs with
+  // itself: its upper waves have nothing to do.
+  const int t64 = (a.sq + 63) / 64, hi_tile = t64 - 1 - pair;
+  const bool upper = wave >= 2;
+  const bool idle = upper && hi_tile == pair;
+  const int qw = (upper ? hi_tile : pair) * 64 + (wave & 1) * 32;  // first query of the wave
+  const int qi = idle ? a.sq : qw + c32;                           // this lane's query
+  const int qrow = qi < a.sq ? qi : a.sq - 1;  // clamp: rows past the end are never stored
   // Q fragments: B operand of S^T = K Q^T, this lane's 8 d-values per k-step
   V16 qf[KSTEPS];
 #pragma unroll
@@ -112,7 +119,8 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
     qf[s] = *reinterpret_cast<const V16 *>(Q + (int64_t)qrow * a.q.row + s * 16 + g * 8);
 
   // keys this block needs: all, or up to its last query under a causal mask
-  const int klimit = a.causal ? (q0 + QUERIES < a.sk ? q0 + QUERIES : a.sk) : a.sk;
+  const int qend = (hi_tile + 1) * 64;  // one past the block's last query
+  const int klimit = a.causal ? (qend < a.sk ? qend : a.sk) : a.sk;
   const int ktiles = (klimit + KEYS - 1) / KEYS;
 
   float m_run = MX::init(), l_run = 0.0f;
@@ -123,8 +131,10 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
     for (int e = 0; e < 16; e++) oacc[t][e] = 0.0f;
 
   // One 32-key sub-tile of scores for this wave: t[e] is the masked, scaled
-  // score of key j0 + (e/4)*8 + g*4 + e%4 against query qi.
-  auto scores = [&](int j0, float (&t)[16]) {
+  // score of key j0 + (e/4)*8 + g*4 + e%4 against query qi. `inner` sub-tiles
+  // lie wholly inside the keys every query of the wave may see: no mask, no
+  // bounds to test.
+  auto scores = [&](int j0, float (&t)[16], bool inner) {
     f32x16 acc;
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[e] = 0.0f;
@@ -133,6 +143,11 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
     for (int s = 0; s < KSTEPS; s++) {
       const V16 kf = *reinterpret_cast<const V16 *>(kr + s * 16);
       gemm_tile::mfma_step<EL>(acc, kf, qf[s]);
+    }
+    if (inner) {
+#pragma unroll
+      for (int e = 0; e < 16; e++) t[e] = a.has_scale ? acc[e] * a.scale : acc[e];
+      return;
     }
 #pragma unroll
     for (int e = 0; e < 16; e++) {
@@ -147,27 +162,45 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
     }
   };
 
+  // Global -> registers for one key tile (K, and V when the tile is for pass
+  // 1), issued a tile ahead so that the loads fly during the previous tile's
+  // arithmetic; registers -> LDS between the two barriers.
+  constexpr int NV = KEYS * VPR / 256;
+  V16 kpre[NV], vpre[NV];
+  auto prefetch = [&](int pass, int kt) {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int v = threadIdx.x + i * 256;
+      const int r = v / VPR, c = (v % VPR) * 8;
+      int key = kt * KEYS + r;
+      key = key < a.sk ? key : a.sk - 1;
+      kpre[i] = *reinterpret_cast<const V16 *>(K + (int64_t)key * a.k.row + c);
+      if (pass == 1) vpre[i] = *reinterpret_cast<const V16 *>(V + (int64_t)key * a.v.row + c);
+    }
+  };
+  prefetch(0, 0);
   for (int pass = 0; pass < 2; pass++) {
     float l_total = 0.0f;
     if (pass == 1) l_total = l_run + xor32(l_run);
     for (int kt = 0; kt < ktiles; kt++) {
       __syncthreads();  // the previous tile has been consumed
-      for (int v = threadIdx.x; v < KEYS * VPR; v += 256) {
+#pragma unroll
+      for (int i = 0; i < NV; i++) {
+        const int v = threadIdx.x + i * 256;
         const int r = v / VPR, c = (v % VPR) * 8;
-        int key = kt * KEYS + r;
-        key = key < a.sk ? key : a.sk - 1;
-        *reinterpret_cast<V16 *>(Ks + r * PK + c) = *reinterpret_cast<const V16 *>(K + (int64_t)key * a.k.row + c);
-        if (pass == 1)
-          *reinterpret_cast<V16 *>(Vs + r * PV + c) = *reinterpret_cast<const V16 *>(V + (int64_t)key * a.v.row + c);
+        *reinterpret_cast<V16 *>(Ks + r * PK + c) = kpre[i];
+        if (pass == 1) *reinterpret_cast<V16 *>(Vs + r * PV + c) = vpre[i];
       }
       __syncthreads();
+      if (kt + 1 < ktiles) prefetch(pass, kt + 1);
+      else if (pass == 0) prefetch(1, 0);
 #pragma unroll
       for (int sub = 0; sub < KEYS / 32; sub++) {
         const int j0 = kt * KEYS + sub * 32;
         // nothing of this sub-tile is visible to the wave's queries
-        if (j0 >= a.sk || (a.causal && j0 > qw + 31)) continue;
+        if (idle || j0 >= a.sk || (a.causal && j0 > qw + 31)) continue;
         float t[16];
-        scores(j0, t);
+        scores(j0, t, j0 + 32 <= a.sk && !a.has_mask && (!a.causal || j0 + 31 <= qw));
         if (pass == 0) {
           float tm = t[0];
 #pragma unroll
@@ -313,7 +346,7 @@ NXH_EXPORT int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_
   a.mask_col = mask ? mask->strides[nd - 1] : 0;
   a.sq = (int)sq;
   a.sk = (int)sk;
-  a.qtiles = (int)((sq + QUERIES - 1) / QUERIES);
+  a.qtiles = (int)(((sq + 63) / 64 + 1) / 2);  // pairs of 64-query tiles
   a.causal = causal ? 1 : 0;
   a.has_mask = mask ? 1 : 0;
   a.has_scale = scale ? 1 : 0;

@@ -45,7 +45,7 @@ class Entry:
     """One recorded primitive."""
 
     __slots__ = ("kind", "op", "ins", "shape", "dtype", "axes", "cell", "alive", "result", "readers", "fused_into",
-                 "value", "__weakref__")
+                 "value", "tag", "__weakref__")
 
     def __init__(self, kind, op, ins, shape, dtype, axes=None):
         self.kind, self.op, self.ins = kind, op, ins
@@ -56,25 +56,31 @@ class Entry:
         self.readers = []      # entries of the window that read this one
         self.fused_into = None
         self.value = None      # kind "full": the encoded element
+        self.tag = None        # what is known about the result's contents (("causal", n))
 
 
 class Operand:
     """An input of an entry: a pending entry or a backend tensor, seen through a view."""
 
-    __slots__ = ("entry", "root", "view", "scalar")
+    __slots__ = ("entry", "root", "view", "scalar", "tag")
 
-    def __init__(self, entry, root, view, scalar):
-        self.entry, self.root, self.view, self.scalar = entry, root, view, scalar
+    def __init__(self, entry, root, view, scalar, tag=None):
+        self.entry, self.root, self.view, self.scalar, self.tag = entry, root, view, scalar, tag
 
     def same(self, other: "Operand") -> bool:
         return self.entry is other.entry and self.root is other.root and self.view == other.view
 
 
 class Cell:
-    __slots__ = ("root", "entry", "scalar", "__weakref__")
+    """Storage shared by the views of one tensor: the backend's tensor (`root`)
+    or the entry that will produce it, plus what the window knows about the
+    contents: `scalar` (the encoded element of a one-element full), `host` (a
+    small int32 array uploaded with from_host), `tag` (see Entry.tag)."""
 
-    def __init__(self, root=None, entry=None, scalar=None):
-        self.root, self.entry, self.scalar = root, entry, scalar
+    __slots__ = ("root", "entry", "scalar", "host", "tag", "__weakref__")
+
+    def __init__(self, root=None, entry=None, scalar=None, host=None):
+        self.root, self.entry, self.scalar, self.host, self.tag = root, entry, scalar, host, None
 
     def __del__(self):
         e = self.entry
@@ -135,10 +141,26 @@ def _vector_broadcast(view: View, shape) -> bool:
             and all(s == 1 or st == 0 for s, st in zip(shape[:-1], view.strides[:-1])))
 
 
+def _causal_length(op, x: "WTensor", y: "WTensor"):
+    """n if ``compare op x y`` is the n x n causal mask of attention.ml:236-243:
+    cmple of arange(n) along the columns against arange(n) down the rows, so
+    that element [i][j] is (j <= i)."""
+    if op != "cmple" or len(x.shape) != 2 or x.shape[0] != x.shape[1]:
+        return None
+    n = x.shape[0]
+    hx, hy = x.cell.host, y.cell.host
+    if hx is None or hy is None or hx.size != n or hy.size != n:
+        return None
+    if (x.view.offset, y.view.offset) != (0, 0) or x.view.strides != (0, 1) or y.view.strides != (1, 0):
+        return None
+    ar = np.arange(n)
+    return n if np.array_equal(hx, ar) and np.array_equal(hy, ar) else None
+
+
 class Window:
     """``Window(backend)``: same operations, deferred as described above."""
 
-    DEFERRED = ("unary", "binary", "where", "cast", "reduce")
+    DEFERRED = ("unary", "binary", "where", "cast", "reduce", "compare", "matmul")
 
     def __init__(self, backend, limit: int = 512, fuse: bool = True):
         self.B = backend
@@ -146,7 +168,7 @@ class Window:
         self.fuse = fuse
         self.entries: List[Entry] = []
         self.stats = {"recorded": 0, "issued": 0, "softmax_rows": 0, "layer_norm_rows": 0, "gelu_tanh": 0,
-                      "flushes": 0, "fallbacks": 0}
+                      "attention": 0, "flushes": 0, "fallbacks": 0}
 
     # ── handles ─────────────────────────────────────────────────────────────
     def _wrap(self, t, scalar=None) -> WTensor:
@@ -164,8 +186,8 @@ class Window:
     def _operand(self, t: WTensor) -> Operand:
         c = t.cell
         if c.root is None:
-            return Operand(c.entry, None, t.view, c.scalar)
-        return Operand(None, c.root, t.view, c.scalar)
+            return Operand(c.entry, None, t.view, c.scalar, c.entry.tag)
+        return Operand(None, c.root, t.view, c.scalar, c.tag)
 
     def _record(self, kind, op, ins: Sequence[WTensor], shape, dtype, axes=None) -> WTensor:
         e = Entry(kind, op, [self._operand(t) for t in ins], shape, dtype, axes)
@@ -201,6 +223,32 @@ class Window:
 
     def cast(self, x, dtype):
         return self._record("cast", None, [x], x.shape, dtype)
+
+    def compare(self, op, x, y):
+        self._same_shape(op, x, y)
+        out = self._record("compare", op, [x, y], x.shape, dt.bool_)
+        n = _causal_length(op, x, y)
+        if n is not None and out.cell.entry is not None:
+            out.cell.entry.tag = ("causal", n)
+        elif n is not None:
+            out.cell.tag = ("causal", n)
+        return out
+
+    def matmul(self, x, y):
+        xs, ys = tuple(x.shape), tuple(y.shape)
+        if len(xs) < 2 or len(ys) < 2 or xs[-1] != ys[-2] or x.dtype is not y.dtype:
+            self.flush()  # let the backend phrase the error
+            return self._lift(self.B.matmul(self.force(x), self.force(y)))
+        nd = max(len(xs), len(ys))
+        batch = []
+        for i in range(nd - 2):
+            ai, bi = i - (nd - len(xs)), i - (nd - len(ys))
+            a, b = (xs[ai] if ai >= 0 else 1), (ys[bi] if bi >= 0 else 1)
+            if a != b and a != 1 and b != 1:
+                self.flush()
+                return self._lift(self.B.matmul(self.force(x), self.force(y)))
+            batch.append(max(a, b) if min(a, b) != 0 else 0)
+        return self._record("matmul", None, [x, y], tuple(batch) + (xs[-2], ys[-1]), x.dtype)
 
     def reduce(self, op, axes, x):
         axes = sorted(int(a) for a in axes)
@@ -255,7 +303,11 @@ class Window:
         return self._wrap(self.B.buffer(dtype, shape))
 
     def from_host(self, array, dtype):
-        return self._wrap(self.B.from_host(array, dtype))
+        t = self._wrap(self.B.from_host(array, dtype))
+        a = np.asarray(array)
+        if dtype.name == "int32" and a.nbytes <= 65536:
+            t.cell.host = a.reshape(-1).copy()  # lets a compare of two aranges be recognised as a causal mask
+        return t
 
     # ── everything else: execute the record, then call through ──────────────
     def __getattr__(self, name):
@@ -305,6 +357,10 @@ class Window:
             r = self.B.where(ins[0], ins[1], ins[2])
         elif e.kind == "cast":
             r = self.B.cast(ins[0], e.dtype)
+        elif e.kind == "compare":
+            r = self.B.compare(e.op, ins[0], ins[1])
+        elif e.kind == "matmul":
+            r = self.B.matmul(ins[0], ins[1])
         else:
             r = self.B.reduce(e.op, e.axes, ins[0])
         self.stats["issued"] += 1
@@ -317,6 +373,7 @@ class Window:
         if cell is not None:
             cell.root = r
             cell.entry = None
+            cell.tag = e.tag
 
     def flush(self):
         entries, self.entries = self.entries, []
@@ -414,20 +471,22 @@ def _rows_ok(o: Operand, shape) -> bool:
 
 
 def _match(w: Window, e: Entry) -> Optional[Plan]:
-    for m in (_match_softmax, _match_layer_norm, _match_gelu):
+    for m in (_match_attention, _match_softmax, _match_layer_norm, _match_gelu):
         p = m(w, e)
         if p is not None:
             return p
     return None
 
 
-def _match_softmax(w: Window, anchor: Entry) -> Optional[Plan]:
+def _softmax_parts(anchor: Entry):
+    """The softmax run ending in `anchor` (the final division, or the cast behind
+    it): (interior, x, scale, mask, masked_value, shape), or None. `x` is the
+    operand the run starts from, behind the optional scale and mask."""
     interior = []
-    out_dtype = anchor.dtype
     d = anchor
     if anchor.kind == "cast":
         d = _producer(anchor.ins[0], "binary", "fdiv")
-        if d is None or d.dtype.name != "float32" or out_dtype.name not in ("float16", "bfloat16"):
+        if d is None or d.dtype.name != "float32" or anchor.dtype.name not in ("float16", "bfloat16"):
             return None
         interior.append(d)
     if d.kind != "binary" or d.op != "fdiv" or d.dtype.name not in FUSED_FLOATS or not d.shape:
@@ -463,14 +522,80 @@ def _match_softmax(w: Window, anchor: Entry) -> Optional[Plan]:
         if sc is not None:
             interior.append(mul)
             scale, x = sc, mul.ins[0]
-    if not _hidden(interior, anchor) or not _rows_ok(x, shape):
+    if not _hidden(interior, anchor):
         return None
+    return interior, x, scale, mask, masked, shape
+
+
+def _match_softmax(w: Window, anchor: Entry) -> Optional[Plan]:
+    parts = _softmax_parts(anchor)
+    if parts is None:
+        return None
+    interior, x, scale, mask, masked, shape = parts
+    if not _rows_ok(x, shape):
+        return None
+    out_dtype = anchor.dtype
 
     def run(win: Window):
         return win.B.softmax_rows(win._tensor_of(x), scale, win._tensor_of(mask) if mask is not None else None,
                                   masked, out_dtype)
 
     return Plan("softmax_rows", interior, run)
+
+
+def _match_attention(w: Window, anchor: Entry) -> Optional[Plan]:
+    """kaun/lib/attention.ml:67-110 for 16-bit operands: cast q and k to float32,
+    Q K^T, [scale], [mask], softmax, cast back, probs x V."""
+    if anchor.kind != "matmul" or anchor.dtype.name not in ISLAND or len(anchor.shape) < 2:
+        return None
+    dtype = anchor.dtype
+    probs = _producer(anchor.ins[0], "cast")
+    if probs is None or probs.dtype is not dtype:
+        return None
+    parts = _softmax_parts(probs)
+    if parts is None:
+        return None
+    interior, x, scale, mask, masked, sshape = parts
+    scores = _producer(x, "matmul")
+    if scores is None or scores.dtype.name != "float32":
+        return None
+    cq = _producer(scores.ins[0], "cast")
+    kt = scores.ins[1]
+    ck = kt.entry
+    if cq is None or ck is None or ck.kind != "cast" or ck.fused_into is not None or len(ck.shape) < 2:
+        return None
+    r = len(ck.shape)
+    axes = list(range(r))
+    axes[-1], axes[-2] = axes[-2], axes[-1]
+    if kt.view != View.create(ck.shape).permute(axes):
+        return None
+    q, k, v = cq.ins[0], ck.ins[0], anchor.ins[1]
+    dt_of = lambda o: o.entry.dtype if o.entry is not None else o.root.dtype
+    if dt_of(q) is not dtype or dt_of(k) is not dtype or dt_of(v) is not dtype:
+        return None
+    qs, ks, vs = q.view.shape, k.view.shape, v.view.shape
+    if (len(qs) != r or len(vs) != r or qs[:-2] != ks[:-2] or qs[:-2] != vs[:-2] or ks != vs or qs[-1] != ks[-1]
+            or qs[-1] not in (32, 64, 128) or tuple(anchor.shape) != qs or len(qs) > 6
+            or any(o.view.strides[-1] != 1 for o in (q, k, v))):
+        return None
+    interior = interior + [probs, scores, cq, ck]
+    if not _hidden(interior, anchor):
+        return None
+    causal = False
+    if mask is not None:
+        n = qs[-2]
+        flat = tuple(0 if s_ != 1 else st for s_, st in zip(sshape[:-2], mask.view.strides[:-2]))
+        if (mask.tag == ("causal", n) and ks[-2] == n and mask.view.offset == 0 and mask.view.strides[-2:] == (n, 1)
+                and all(st == 0 or s_ == 1 for s_, st in zip(sshape[:-2], mask.view.strides[:-2]))):
+            causal, mask = True, None
+        del flat
+    as_f32 = lambda a: None if a is None else np.asarray(a, dtype=np.float32).reshape(1)
+
+    def run(win: Window):
+        return win.B.attention(win._tensor_of(q), win._tensor_of(k), win._tensor_of(v), as_f32(scale),
+                               win._tensor_of(mask) if mask is not None else None, as_f32(masked), causal)
+
+    return Plan("attention", interior, run)
 
 
 def _match_layer_norm(w: Window, anchor: Entry) -> Optional[Plan]:

@@ -115,7 +115,9 @@ def test_gpt2_forward_through_the_window_on_the_gpu(hip, oracle, d):
     win = Window(hip)
     got = decode(logical(win.force(run(win, oracle, SMALL, hp, ids, d))), d, oracle)
     L = SMALL.n_layer
-    assert (win.stats["softmax_rows"], win.stats["layer_norm_rows"], win.stats["gelu_tanh"]) == (L, 2 * L + 1, L)
+    assert (win.stats["layer_norm_rows"], win.stats["gelu_tanh"]) == (2 * L + 1, L)
+    # head dim 64: bfloat16 runs the whole attention core as one kernel, float32 its softmax
+    assert (win.stats["attention"], win.stats["softmax_rows"]) == ((L, 0) if d is dt.bfloat16 else (0, L))
     assert win.stats["fallbacks"] == 0
     eager = decode(logical(run(hip, oracle, SMALL, hp, ids, d)), d, oracle)
     want = decode(logical(run(oracle, oracle, SMALL, hp, ids, d)), d, oracle)

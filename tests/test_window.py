@@ -19,7 +19,7 @@ from raven_amd.kaun_gpt2 import Config, Gpt2, LayerNorm, host_params, upload
 from raven_amd.nx_frontend import Nx
 from raven_amd.nx_window import Window
 
-TINY = Config(vocab_size=97, n_positions=16, n_embd=32, n_layer=2, n_head=4, n_inner=64)
+TINY = Config(vocab_size=97, n_positions=16, n_embd=128, n_layer=2, n_head=4, n_inner=256)  # head dim 32
 
 
 class SequencedOracle(OracleBackend):
@@ -42,6 +42,21 @@ class SequencedOracle(OracleBackend):
     def layer_norm_rows(self, x, gamma, beta, eps):
         self.calls.append("layer_norm_rows")
         return Gpt2(Nx(self), TINY).layer_norm(LayerNorm(gamma, beta), x, eps)
+
+    def attention(self, q, k, v, scale=None, mask=None, masked_value=None, causal=False):
+        self.calls.append("attention_causal" if causal else "attention")
+        nx = Nx(self)
+        r = len(q.shape)
+        sc = nx.matmul(nx.cast(dt.float32, q), nx.swapaxes(r - 2, r - 1, nx.cast(dt.float32, k)))
+        if scale is not None:
+            sc = nx.mul(sc, self.full(dt.float32, (), scale))
+        if causal:
+            n = q.shape[-2]
+            idx = nx.arange(dt.int32, 0, n, 1)
+            mask = nx.less_equal(nx.reshape((1, n), idx), nx.reshape((n, 1), idx))
+        if mask is not None:
+            sc = nx.where(mask, sc, self.full(dt.float32, (), masked_value))
+        return nx.matmul(nx.cast(q.dtype, nx.softmax(sc)), v)
 
     def gelu_tanh(self, x, constants):
         self.calls.append("gelu_tanh")
@@ -78,14 +93,21 @@ def test_gpt2_forward_through_the_window_fuses_every_sequence(oracle, d):
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
     L = TINY.n_layer
     assert w.stats["layer_norm_rows"] == 2 * L + 1
-    assert w.stats["softmax_rows"] == L
     assert w.stats["gelu_tanh"] == L
     assert w.stats["fallbacks"] == 0
-    assert base.calls.count("softmax_rows") == L
-    # what is left op by op: bias adds, residual adds, embedding add, and for
-    # bfloat16 the casts of q and k into the float32 island
-    per_block = 6 + 2 + (2 if d is dt.bfloat16 else 0)
-    assert w.stats["issued"] == L * per_block + 1
+    if d is dt.bfloat16:
+        # the whole attention core is one call, recognised as causal from the aranges of its mask
+        assert (w.stats["attention"], w.stats["softmax_rows"]) == (L, 0)
+        assert base.calls.count("attention_causal") == L
+    else:
+        # float32 has no float32 island: the softmax alone is fused
+        assert (w.stats["attention"], w.stats["softmax_rows"]) == (0, L)
+        assert base.calls.count("softmax_rows") == L
+    # what is left op by op per block: 6 linears (matmul + bias add), 2 residual
+    # adds, the mask compare, and for float32 the two attention matmuls;
+    # outside the blocks the embedding add and the head matmul
+    per_block = 12 + 2 + 1 + (0 if d is dt.bfloat16 else 2)
+    assert w.stats["issued"] == L * per_block + 2
     # with fusion switched off the window only defers
     w2 = Window(SequencedOracle(), fuse=False)
     got2 = value(w2, forward(w2, hp, ids, d, oracle))
@@ -152,6 +174,49 @@ def test_scale_mask_and_cast_join_the_softmax(win, oracle):
     assert np.array_equal(got, ological(weights(oracle)))
     assert win.stats["softmax_rows"] == 1 and win.stats["issued"] == 0
     assert win.B.calls == ["softmax_rows"]
+
+
+def test_attention_run_and_what_blocks_it(oracle):
+    rng = np.random.default_rng(8)
+    b, h, s, hd = 2, 3, 16, 32
+    d = dt.bfloat16
+    q, k, v = (encode(rng.standard_normal((b, h, s, hd)), d, oracle) for _ in range(3))
+    rnd = (rng.random((s, s)) < 0.6).astype(np.uint8)
+    rnd[:, 0] = 1
+
+    def run(B, mask_kind, keep=None):
+        nx = Nx(B)
+        tq, tk, tv = (nx.create(d, a.shape, a) for a in (q, k, v))
+        if mask_kind == "causal":
+            idx = nx.arange(dt.int32, 0, s, 1)
+            mask = nx.less_equal(nx.reshape((1, s), idx), nx.reshape((s, 1), idx))
+        elif mask_kind == "random":
+            mask = nx.create(dt.bool_, (s, s), rnd)
+        else:
+            mask = None
+        model = Gpt2(nx, TINY)
+        if keep is None:
+            return model.scaled_dot_product_attention(tq, tk, tv, mask)
+        # the same calls with the probabilities kept alive
+        sc = nx.mul_s(nx.matmul(nx.cast(dt.float32, tq), nx.swapaxes(2, 3, nx.cast(dt.float32, tk))), 0.25)
+        sc = nx.where(mask, sc, nx.scalar_like(sc, float("-inf")))
+        keep.append(nx.cast(d, nx.softmax(sc)))
+        return nx.matmul(keep[-1], tv)
+
+    for kind, expect in (("causal", "attention_causal"), ("random", "attention"), (None, "attention")):
+        base = SequencedOracle()
+        w = Window(base)
+        got = value(w, run(w, kind))
+        assert np.array_equal(got, ological(run(oracle, kind))), kind
+        assert base.calls == [expect] and w.stats["attention"] == 1, (kind, base.calls)
+    base = SequencedOracle()
+    w = Window(base)
+    kept = []
+    got = value(w, run(w, "causal", kept))
+    okept = []
+    want = ological(run(oracle, "causal", okept))
+    assert np.array_equal(got, want) and np.array_equal(value(w, kept[0]), ological(okept[0]))
+    assert w.stats["attention"] == 0 and base.calls == ["softmax_rows"]   # the softmax alone still fuses
 
 
 def test_gelu_and_layer_norm_alone(win, oracle):
