@@ -154,17 +154,17 @@ struct ContigArgs {
   uint32_t bcast;  // bit k set: input k is a broadcast scalar
 };
 
-template <class F, int V>
+template <class F, int V, int UNR>
 __global__ __launch_bounds__(MAP_THREADS) void map_contig_kernel(ContigArgs<F> a) {
   using MT = MapTypes<F>;
   const int64_t nvec = a.n / V;
-  const int64_t base = (int64_t)blockIdx.x * (MAP_THREADS * MAP_UNROLL) + threadIdx.x;
+  const int64_t base = (int64_t)blockIdx.x * (MAP_THREADS * UNR) + threadIdx.x;
   const bool b0 = a.bcast & 1u, b1 = a.bcast & 2u, b2 = a.bcast & 4u;
-  Vec<typename MT::In0, V> x0[MAP_UNROLL];
-  Vec<typename MT::In1, V> x1[MAP_UNROLL];
-  Vec<typename MT::In2, V> x2[MAP_UNROLL];
+  Vec<typename MT::In0, V> x0[UNR];
+  Vec<typename MT::In1, V> x1[UNR];
+  Vec<typename MT::In2, V> x2[UNR];
 #pragma unroll
-  for (int j = 0; j < MAP_UNROLL; j++) {
+  for (int j = 0; j < UNR; j++) {
     int64_t u = base + (int64_t)j * MAP_THREADS;
     if (u < nvec) {
       x0[j] = load_vec<typename MT::In0, V>(a.in0, b0 ? 0 : u * V, b0);
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(MAP_THREADS) void map_contig_kernel(ContigArgs<F> a
     }
   }
 #pragma unroll
-  for (int j = 0; j < MAP_UNROLL; j++) {
+  for (int j = 0; j < UNR; j++) {
     int64_t u = base + (int64_t)j * MAP_THREADS;
     if (u < nvec) {
       Vec<typename MT::Out, V> r;
@@ -481,9 +481,18 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       if (s == 0 || p.total == 1) bc |= (p.total == 1 ? 0u : 1u << (k - 1));
       else if (s != 1) ok = false;
     }
+    // A narrow output (compare, narrowing casts) widens the lane's vector until
+    // it stores 16 bytes, with fewer vectors per lane so that the bytes in
+    // flight stay the same; operands must then be aligned to the wider vector.
+    constexpr int VW = (int)sizeof(typename MT::Out) < MT::smax
+                           ? std::min(16 / (int)sizeof(typename MT::Out), V * MAP_UNROLL) : V;
+    constexpr int UW = V * MAP_UNROLL / VW;
+    bool wide = VW > V;
     for (int k = 0; ok && k < p.nop; k++) {
       bool is_bc = k > 0 && (bc & (1u << (k - 1)));
-      if (!is_bc && !aligned_to(p.base[k], (size_t)esz[k] * V)) ok = false;
+      if (is_bc) continue;
+      if (!aligned_to(p.base[k], (size_t)esz[k] * V)) ok = false;
+      if (!aligned_to(p.base[k], (size_t)esz[k] * VW)) wide = false;
     }
     if (ok) {
       ContigArgs<F> a;
@@ -493,11 +502,16 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       a.in2 = (const typename MT::In2 *)(p.nop > 3 ? p.base[3] : nullptr);
       a.n = p.total;
       a.bcast = bc;
-      const int64_t nvec = (p.total + V - 1) / V;
-      const int64_t per_block = MAP_THREADS * MAP_UNROLL;
-      const uint32_t blocks = (uint32_t)((nvec + per_block - 1) / per_block);
       nxh_set_path("map_contig");
-      hipLaunchKernelGGL((map_contig_kernel<F, V>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+      if (wide) {
+        const int64_t nvec = (p.total + VW - 1) / VW, per_block = MAP_THREADS * UW;
+        const uint32_t blocks = (uint32_t)((nvec + per_block - 1) / per_block);
+        hipLaunchKernelGGL((map_contig_kernel<F, VW, UW>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+      } else {
+        const int64_t nvec = (p.total + V - 1) / V, per_block = MAP_THREADS * MAP_UNROLL;
+        const uint32_t blocks = (uint32_t)((nvec + per_block - 1) / per_block);
+        hipLaunchKernelGGL((map_contig_kernel<F, V, MAP_UNROLL>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+      }
       NXH_HIP(op, hipGetLastError());
       return NXH_OK;
     }
