@@ -1,0 +1,211 @@
+"""Randomised views against the CPU oracle: every case draws a rank, extents
+(zeros and ones included), a chain of view operations per operand (permute,
+flip, shrink, broadcast from a singleton) and an operation, and compares the
+GPU result with the oracle bit for bit. Integer dtypes and IEEE-exact float
+operations only, so that any difference is an indexing or planning fault, not
+rounding. Seeds are fixed: a failure names the case that reproduces it."""
+
+import numpy as np
+import pytest
+
+from helpers import logical, same_bits, same_bits_nan_any
+from raven_amd import dtype as dt
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [dt.int32, dt.uint8, dt.int64, dt.float32, dt.bfloat16, dt.int16, dt.float64, dt.bool_]
+EXACT_BINARY = {"int": ["add", "sub", "mul", "idiv", "mod", "max", "min", "xor", "or", "and"],
+                "float": ["add", "sub", "mul", "fdiv", "max", "min"], "bool": ["xor", "or", "and", "max", "min"]}
+EXACT_UNARY = {"int": ["neg", "abs", "sign"], "float": ["neg", "abs", "sign", "sqrt", "floor", "round"], "bool": []}
+
+
+def kind(d):
+    return "bool" if d is dt.bool_ else ("float" if d.is_float else "int")
+
+
+def values(rng, shape, d):
+    n = int(np.prod(shape, dtype=np.int64))
+    if d is dt.bool_:
+        return rng.integers(0, 2, n).astype(np.uint8).reshape(shape)
+    if d is dt.bfloat16:  # small integers and halves are exact in bfloat16
+        f = (rng.integers(-16, 16, n) / 2).astype(np.float32)
+        return (f.view(np.uint32) >> 16).astype(np.uint16).reshape(shape)
+    if d.is_float:
+        return (rng.integers(-64, 64, n) / 4).astype(d.np_storage).reshape(shape)
+    info = np.iinfo(d.np_storage)
+    return rng.integers(max(info.min, -50), min(info.max, 50), n, endpoint=True).astype(d.np_storage).reshape(shape)
+
+
+def build_operand(rng, hip, oracle, d, target):
+    """Same random storage and the same random view chain on both backends,
+    ending in logical shape `target`."""
+    r = len(target)
+    perm = rng.permutation(r) if r else np.array([], int)
+    bcast = [bool(rng.random() < 0.2) and target[i] > 1 for i in range(r)]
+    pad_lo = [int(rng.integers(0, 3)) for _ in range(r)]
+    pad_hi = [int(rng.integers(0, 3)) for _ in range(r)]
+    flip = [bool(rng.random() < 0.3) for _ in range(r)]
+    if 0 in target:  # an empty tensor has nothing to slice: plain layout
+        bcast, pad_lo, pad_hi = [False] * r, [0] * r, [0] * r
+    # source extents in logical order, then stored permuted
+    src = [1 if bcast[i] else target[i] + pad_lo[i] + pad_hi[i] for i in range(r)]
+    stored = [src[p] for p in perm]
+    x = values(rng, stored, d)
+    inv = np.argsort(perm) if r else perm
+
+    def view(B):
+        t = B.reshape(B.from_host(np.ascontiguousarray(x), d), tuple(stored))
+        if r == 0:
+            return t
+        t = B.permute(t, [int(i) for i in inv])  # back to logical order
+        bounds = [(0, 1) if bcast[i] else (pad_lo[i], pad_lo[i] + target[i]) for i in range(r)]
+        if 0 not in target:
+            t = B.shrink(t, bounds)
+        t = B.flip(t, flip)
+        return B.expand(t, tuple(target))
+
+    return view(hip), view(oracle)
+
+
+CASES = list(range(480))
+
+
+@pytest.mark.parametrize("seed", CASES)
+def test_random_views(hip, oracle, seed):
+    rng = np.random.default_rng(7000 + seed)
+    d = DTYPES[seed % len(DTYPES)]
+    k = kind(d)
+    r = int(rng.integers(0, 6))
+    target = [int(rng.choice([0, 1, 2, 3, 5, 8, 17, 33], p=[0.04, 0.12, 0.16, 0.16, 0.16, 0.16, 0.1, 0.1]))
+              for _ in range(r)]
+    if int(np.prod(target, dtype=np.int64)) > 200000:
+        target = [min(t, 8) for t in target]
+    ops = ["binary", "unary", "compare", "where", "cast", "copy", "reduce", "argmax", "scan", "sort", "pad", "cat"]
+    op = ops[int(rng.integers(0, len(ops)))]
+    what = f"seed {seed}: {op} {d.name} {target}"
+
+    def eq(g, w, dd=d):
+        g, w = logical(g), logical(w)
+        if dd.is_float:
+            same_bits_nan_any(g, w, dd, oracle, what)
+        else:
+            same_bits(g, w, what)
+
+    ha, oa = build_operand(rng, hip, oracle, d, target)
+    if op == "binary":
+        hb, ob = build_operand(rng, hip, oracle, d, target)
+        for name in EXACT_BINARY[k]:
+            eq(hip.binary(name, ha, hb), oracle.binary(name, oa, ob))
+    elif op == "unary":
+        for name in EXACT_UNARY[k]:
+            eq(hip.unary(name, ha), oracle.unary(name, oa))
+    elif op == "compare":
+        hb, ob = build_operand(rng, hip, oracle, d, target)
+        for name in ("cmpeq", "cmpne", "cmplt", "cmple"):
+            eq(hip.compare(name, ha, hb), oracle.compare(name, oa, ob), dt.bool_)
+    elif op == "where":
+        hb, ob = build_operand(rng, hip, oracle, d, target)
+        hc, oc = build_operand(rng, hip, oracle, dt.bool_, target)
+        eq(hip.where(hc, ha, hb), oracle.where(oc, oa, ob))
+    elif op == "cast":
+        for to in (dt.int32, dt.float32, dt.uint8, dt.bool_, dt.int64):
+            eq(hip.cast(ha, to), oracle.cast(oa, to), to)
+    elif op == "copy":
+        eq(hip.copy(ha), oracle.copy(oa))
+        eq(hip.contiguous(ha), oracle.contiguous(oa))
+    elif op == "reduce":
+        if r == 0:
+            return
+        axes = sorted(int(a) for a in rng.choice(r, size=int(rng.integers(1, r + 1)), replace=False))
+        names = ["sum", "max", "min"] if k != "bool" else ["max", "min"]
+        if k == "int":
+            names.append("prod")
+        for name in names:
+            if name in ("max", "min") and any(target[a] == 0 for a in axes):
+                continue
+            eq(hip.reduce(name, axes, ha), oracle.reduce(name, axes, oa))
+    elif op == "argmax":
+        if r == 0 or k == "bool":
+            return
+        axis = int(rng.integers(0, r))
+        if target[axis] == 0:
+            return
+        eq(hip.argmax(ha, axis), oracle.argmax(oa, axis), dt.int32)
+        eq(hip.argmin(ha, axis, True), oracle.argmin(oa, axis, True), dt.int32)
+    elif op == "scan":
+        if r == 0:
+            return
+        axis = int(rng.integers(0, r))
+        for name in (["sum", "max", "min"] if k != "bool" else ["max", "min"]):
+            eq(hip.associative_scan(axis, name, ha), oracle.associative_scan(axis, name, oa))
+    elif op == "sort":
+        if r == 0:
+            return
+        axis = int(rng.integers(0, r))
+        desc = bool(rng.integers(0, 2))
+        eq(hip.sort(ha, axis, desc), oracle.sort(oa, axis, desc))
+        eq(hip.argsort(ha, axis, desc), oracle.argsort(oa, axis, desc), dt.int32)
+    elif op == "pad":
+        padding = [(int(rng.integers(0, 3)), int(rng.integers(0, 3))) for _ in range(r)]
+        fill = values(rng, (1,), d)
+        eq(hip.pad(ha, padding, fill), oracle.pad(oa, padding, fill))
+    elif op == "cat":
+        if r == 0:
+            return
+        axis = int(rng.integers(0, r))
+        other = list(target)
+        other[axis] = int(rng.integers(0, 4))
+        hb, ob = build_operand(rng, hip, oracle, d, other)
+        eq(hip.cat([ha, hb, ha], axis), oracle.cat([oa, ob, oa], axis))
+
+
+@pytest.mark.parametrize("seed", list(range(96)))
+def test_random_views_at_fast_path_sizes(hip, oracle, seed):
+    """The same game with two or three dims of 60-400: these sizes reach the
+    tiled-transpose, vectorised and split-reduction paths the small cases miss."""
+    rng = np.random.default_rng(9000 + seed)
+    d = [dt.float32, dt.int32, dt.bfloat16, dt.uint8, dt.int64, dt.float64][seed % 6]
+    k = kind(d)
+    r = int(rng.integers(2, 4))
+    target = [int(rng.choice([60, 64, 97, 128, 200, 256, 257, 400])) for _ in range(r)]
+    if r == 3:
+        target[int(rng.integers(0, 3))] = int(rng.choice([1, 3, 8]))
+    op = ["binary", "where", "cast", "copy", "reduce", "argmax", "scan", "compare"][int(rng.integers(0, 8))]
+    what = f"seed {seed}: {op} {d.name} {target}"
+
+    def eq(g, w, dd=d):
+        g, w = logical(g), logical(w)
+        if dd.is_float:
+            same_bits_nan_any(g, w, dd, oracle, what)
+        else:
+            same_bits(g, w, what)
+
+    ha, oa = build_operand(rng, hip, oracle, d, target)
+    if op == "binary":
+        hb, ob = build_operand(rng, hip, oracle, d, target)
+        for name in ("add", "mul", "max"):
+            eq(hip.binary(name, ha, hb), oracle.binary(name, oa, ob))
+    elif op == "compare":
+        hb, ob = build_operand(rng, hip, oracle, d, target)
+        eq(hip.compare("cmplt", ha, hb), oracle.compare("cmplt", oa, ob), dt.bool_)
+    elif op == "where":
+        hb, ob = build_operand(rng, hip, oracle, d, target)
+        hc, oc = build_operand(rng, hip, oracle, dt.bool_, target)
+        eq(hip.where(hc, ha, hb), oracle.where(oc, oa, ob))
+    elif op == "cast":
+        for to in (dt.float16, dt.int32, dt.uint8):
+            eq(hip.cast(ha, to), oracle.cast(oa, to), to)
+    elif op == "copy":
+        eq(hip.copy(ha), oracle.copy(oa))
+    elif op == "reduce":
+        axes = sorted(int(a) for a in rng.choice(r, size=int(rng.integers(1, r + 1)), replace=False))
+        for name in ("sum", "max", "min"):  # quarter-integers: float sums are exact in any order
+            eq(hip.reduce(name, axes, ha), oracle.reduce(name, axes, oa))
+    elif op == "argmax":
+        axis = int(rng.integers(0, r))
+        eq(hip.argmax(ha, axis), oracle.argmax(oa, axis), dt.int32)
+        eq(hip.argmin(ha, axis), oracle.argmin(oa, axis), dt.int32)
+    elif op == "scan":
+        axis = int(rng.integers(0, r))
+        for name in ("sum", "max"):
+            eq(hip.associative_scan(axis, name, ha), oracle.associative_scan(axis, name, oa))
