@@ -372,6 +372,74 @@ class CountingBackend:
         return counted
 
 
+def cpu_configs():
+    """The CPU oracle on bounded samples of the other configurations, on this
+    host's cores with the reference's thread policy: the CPU path beside each
+    GPU figure. Every sample is named in its record."""
+    from oracle.nx_oracle import OracleBackend, lib
+
+    B = OracleBackend()
+    out = []
+    mk = lambda arr, d: B.reshape(B.from_host(arr, d), arr.shape)  # noqa: E731
+
+    def timed(name, fn, nbytes=0, flops=0, budget=4.0):
+        fn()
+        t0, reps = time.perf_counter(), 0
+        while reps < 2 or (time.perf_counter() - t0 < budget and reps < 20):
+            fn()
+            reps += 1
+        sec = (time.perf_counter() - t0) / reps
+        rec = {"op": name, "ms": round(sec * 1e3, 3), "threads": lib().nxo_last_threads()}
+        if nbytes:
+            rec["GB/s"] = round(nbytes / sec / 1e9, 2)
+        if flops:
+            rec["GFLOP/s"] = round(flops / sec / 1e9, 1)
+        out.append(rec)
+
+    n = 4096
+    a, b, c = (mk(np.random.default_rng(s).uniform(-1, 1, (n, n)).astype(np.float32), dt.float32) for s in (1, 2, 3))
+    e = n * n * 4
+    timed("cfg1 f32 mul [4096,4096]", lambda: B.binary("mul", a, b), 3 * e)
+    timed("cfg1 f32 sin [4096,4096]", lambda: B.unary("sin", c), 2 * e)
+    timed("cfg1 f32 reduce_sum axis 1 [4096,4096]", lambda: B.reduce("sum", [1], a), e)
+    del a, b, c
+    n = 8192
+    x = mk(np.random.default_rng(8).standard_normal((n, n)).astype(np.float32), dt.float32)
+    e = n * n * 4
+    for axis in (1, 0):
+        timed(f"cfg3 f32 sum axis {axis} [8192,8192]", lambda: B.reduce("sum", [axis], x), e)
+        timed(f"cfg3 f32 argmax axis {axis} [8192,8192]", lambda: B.argmax(x, axis), e)
+    del x
+    m = 2048
+    fa, fb = (mk((np.random.default_rng(s).standard_normal((m, m)) * 0.02).astype(np.float32), dt.float32) for s in (10, 11))
+    timed("cfg4 f32 matmul 2048^3", lambda: B.matmul(fa, fb), flops=2 * m ** 3, budget=8.0)
+    ba, bb = B.cast(B.reshape(fa, (1, m, m)), dt.bfloat16), B.cast(B.reshape(fb, (1, m, m)), dt.bfloat16)
+    timed("cfg4 bf16 matmul, sample [1,2048,2048]^2 of [16,4096,4096]^2", lambda: B.matmul(ba, bb), flops=2 * m ** 3,
+          budget=8.0)
+    sa = mk((np.random.default_rng(14).standard_normal((8, 4096)) * 0.02).astype(np.float32), dt.float32)
+    sb = mk((np.random.default_rng(15).standard_normal((4096, 16384)) * 0.02).astype(np.float32), dt.float32)
+    timed("cfg4 f32 skinny [8,4096]x[4096,16384]", lambda: B.matmul(sa, sb), nbytes=(8 * 4096 + 4096 * 16384 + 8 * 16384) * 4,
+          flops=2 * 8 * 4096 * 16384)
+    del fa, fb, ba, bb, sa, sb
+    # config 5: the eager GPT-2-small forward at batch 1 x seq 128 (1/64 of the tokens of the GPU run)
+    from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
+    from raven_amd.nx_frontend import Nx
+
+    cfg = Config.small()
+    enc = lambda v, d: ((np.ascontiguousarray(v, np.float32).view(np.uint32) + 0x7FFF  # noqa: E731
+                         + ((np.ascontiguousarray(v, np.float32).view(np.uint32) >> 16) & 1)) >> 16).astype(np.uint16)
+    nx = Nx(B)
+    params = upload(nx, host_params(cfg, seed=16), dt.bfloat16, enc)
+    ids = nx.create(dt.int32, (1, 128), np.random.default_rng(17).integers(0, cfg.vocab_size, (1, 128)).astype(np.int32))
+    model = Gpt2(nx, cfg)
+    t0 = time.perf_counter()
+    model.logits(params, ids)
+    sec = time.perf_counter() - t0
+    out.append({"op": "cfg5 GPT-2 small forward, bf16, sample batch 1 x seq 128 (one pass)", "ms": round(sec * 1e3, 1),
+                "tokens/s": round(128 / sec, 1)})
+    return {"host_cores": lib().nxo_ncores(), "ops": out}
+
+
 def config5(hip, iters=3, warmup=1, window=False):
     """GPT-2-small-shaped forward (12 layers, d 768, 12 heads, FFN 3072, vocab
     50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s. Eager: one
@@ -435,11 +503,16 @@ def main():
                     help="time the operations of one configuration only and print their records")
     ap.add_argument("--only-next", action="store_true", help="time pad/cat/scan/threefry/scatter only")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 forward leg only and print its record")
+    ap.add_argument("--cpu-configs", action="store_true",
+                    help="time the CPU oracle on bounded samples of configurations 1, 3, 4, 5 and print the records")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
 
+    if args.cpu_configs:
+        print(json.dumps({"cpu_configs": cpu_configs()}))
+        return
     hip = Backend()
     info = hip.device_info()
     if args.only_gpt2:
