@@ -14,8 +14,9 @@
 // result is unique and a sorting network reproduces it whatever its exchange
 // pattern.
 //
-// Algorithm: bitonic sorting network on (key, index) pairs, the slice padded to
-// a power of two with elements that sort last.
+// Algorithm: bitonic sorting network, the slice padded to a power of two with
+// elements that sort last. Elements are (key, index) pairs for 64-bit and
+// complex keys and one packed 64-bit word otherwise (see "packed keys").
 //   sort_lds     slices of up to 4096 elements (2048 for 16-byte keys): whole
 //                network in LDS, several short slices per block;
 //   sort_global  longer slices: pairs staged in scratch memory; chunks are
@@ -249,10 +250,266 @@ __global__ __launch_bounds__(256) void sort_merge_kernel(SortArgs a, int64_t kk,
   }
 }
 
+// ── packed keys ─────────────────────────────────────────────────────────────
+// Dtypes whose compute-type value fits 32 bits (every float but f64, every
+// integer up to 32 bits, bool) are sorted as ONE 64-bit word per element:
+//   high half  the value mapped to an unsigned that ascends in sort order
+//              (floats: sign-flipped bits with -0 folded onto +0; ints offset by
+//              2^31; the whole half inverted for descending); 0xFFFFFFFE for a
+//              NaN; 0xFFFFFFFF for padding;
+//   low half   the original index (2^31 - 1 - index for the descending value
+//              sort, whose ties go by descending index; NaNs always keep index
+//              order). Indices stay below 2^30, so no element equals the padding.
+// Unsigned order of the words is then exactly the total order above, one
+// compare-exchange is a 64-bit min / max, and both halves of a pair are always
+// written, so the network has no data-dependent branch.
+template <int DT>
+struct Packed {
+  using TR = Tr<DT>;
+  using C = typename TR::C;
+  static constexpr bool ok = DT == NXH_F16 || DT == NXH_F32 || DT == NXH_BF16 || DT == NXH_F8E4M3 ||
+                             DT == NXH_F8E5M2 || DT == NXH_I8 || DT == NXH_U8 || DT == NXH_I16 || DT == NXH_U16 ||
+                             DT == NXH_I32 || DT == NXH_U32 || DT == NXH_BOOL;
+  static constexpr uint32_t K_NAN = 0xFFFFFFFEu;
+  template <int MODE>
+  __device__ __forceinline__ static uint64_t pack(C x, uint32_t index) {
+    constexpr bool desc = MODE == VALUE_DESC || MODE == ARG_DESC;
+    uint32_t m;
+    if constexpr (TR::cat == CAT_FLOAT) {
+      if (x != x) return ((uint64_t)K_NAN << 32) | index;
+      uint32_t u = __builtin_bit_cast(uint32_t, (float)x);
+      if ((u << 1) == 0) u = 0;  // -0 and +0 compare equal
+      m = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+    } else if constexpr (TR::cat == CAT_SINT) {
+      m = (uint32_t)(int32_t)x ^ 0x80000000u;
+    } else {
+      m = (uint32_t)x;
+    }
+    if (desc) m = ~m;
+    return ((uint64_t)m << 32) | (MODE == VALUE_DESC ? 0x7FFFFFFFu - index : index);
+  }
+  template <int MODE>
+  __device__ __forceinline__ static uint32_t index_of(uint64_t w) {
+    const uint32_t lo = (uint32_t)w;
+    if constexpr (MODE == VALUE_DESC) {
+      if (TR::cat != CAT_FLOAT || (uint32_t)(w >> 32) != K_NAN) return 0x7FFFFFFFu - lo;
+    }
+    return lo;
+  }
+};
+constexpr uint64_t PACKED_PAD = ~(uint64_t)0;
+constexpr int PNL = 4096;  // packed elements per LDS chunk (32 KB)
+
+__device__ __forceinline__ void packed_step(uint64_t *w, int count, int j, int64_t kk, int64_t base, int64_t mask) {
+  for (int p = threadIdx.x; p < count / 2; p += 256) {
+    const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));
+    const int l = i | j;
+    const bool up = (((base + i) & mask) & kk) == 0;
+    const uint64_t x = w[i], y = w[l];
+    const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
+    w[i] = up ? lo : hi;
+    w[l] = up ? hi : lo;
+  }
+  __syncthreads();
+}
+
+// The last log2(4) steps of every merge level stay inside aligned groups of
+// four elements: one lane takes a group through both of them in registers.
+__device__ __forceinline__ void packed_tail4(uint64_t *w, int count, int64_t kk, int64_t base, int64_t mask) {
+  for (int q = threadIdx.x; q < count / 4; q += 256) {
+    const int i = q * 4;
+    const bool up = (((base + i) & mask) & kk) == 0;
+    uint64_t e0 = w[i], e1 = w[i + 1], e2 = w[i + 2], e3 = w[i + 3];
+    auto cx = [&](uint64_t &x, uint64_t &y) {
+      const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
+      x = up ? lo : hi;
+      y = up ? hi : lo;
+    };
+    cx(e0, e2);
+    cx(e1, e3);
+    cx(e0, e1);
+    cx(e2, e3);
+    w[i] = e0;
+    w[i + 1] = e1;
+    w[i + 2] = e2;
+    w[i + 3] = e3;
+  }
+  __syncthreads();
+}
+
+// All steps j of level kk from `jtop` down to 1 inside LDS.
+__device__ __forceinline__ void packed_level(uint64_t *w, int count, int64_t kk, int jtop, int64_t base, int64_t mask) {
+  int j = jtop;
+  for (; j >= 4; j >>= 1) packed_step(w, count, j, kk, base, mask);
+  if (jtop >= 2 && count >= 4) packed_tail4(w, count, kk, base, mask);
+  else
+    for (; j >= 1; j >>= 1) packed_step(w, count, j, kk, base, mask);
+}
+
+template <int DT, int MODE>
+__device__ __forceinline__ void packed_store(const SortArgs &a, int64_t oo, int64_t io, int64_t i, uint64_t word) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  const uint32_t src = Packed<DT>::template index_of<MODE>(word);
+  if constexpr (MODE >= ARG_ASC) reinterpret_cast<int32_t *>(a.out)[oo + i * a.out_axis] = (int32_t)src;
+  else  // through the compute type, as the reference's gather-sort-scatter does (nx_c_sort.c:270-291)
+    reinterpret_cast<S *>(a.out)[oo + i * a.out_axis] =
+        TR::st(TR::ld(reinterpret_cast<const S *>(a.in)[io + (int64_t)src * a.in_axis]));
+}
+
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void psort_lds_kernel(SortArgs a, int spb) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  __shared__ uint64_t w[PNL];
+  const int np = (int)a.n_pad, count = spb * np;
+  const int64_t first = (int64_t)blockIdx.x * spb;
+  for (int e = threadIdx.x; e < count; e += 256) {
+    const int64_t s = first + e / np;
+    const int i = e % np;
+    uint64_t word = PACKED_PAD;
+    if (s < a.slices && i < a.n) {
+      int64_t io, oo;
+      slice_offsets(a, s, io, oo);
+      word = Packed<DT>::template pack<MODE>(TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]), (uint32_t)i);
+    }
+    w[e] = word;
+  }
+  __syncthreads();
+  for (int kk = 2; kk <= np; kk <<= 1) packed_level(w, count, kk, kk >> 1, 0, np - 1);
+  for (int e = threadIdx.x; e < count; e += 256) {
+    const int64_t s = first + e / np;
+    const int i = e % np;
+    if (s < a.slices && i < a.n) {
+      int64_t io, oo;
+      slice_offsets(a, s, io, oo);
+      packed_store<DT, MODE>(a, oo, io, i, w[e]);
+    }
+  }
+}
+
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void psort_chunks_kernel(SortArgs a) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  __shared__ uint64_t w[PNL];
+  const int64_t chunks = a.n_pad / PNL;
+  const int64_t s = blockIdx.x / chunks, base = (blockIdx.x % chunks) * PNL;
+  int64_t io, oo;
+  slice_offsets(a, s, io, oo);
+  for (int e = threadIdx.x; e < PNL; e += 256) {
+    const int64_t i = base + e;
+    w[e] = i < a.n ? Packed<DT>::template pack<MODE>(TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]), (uint32_t)i)
+                   : PACKED_PAD;
+  }
+  __syncthreads();
+  for (int kk = 2; kk <= PNL; kk <<= 1) packed_level(w, PNL, kk, kk >> 1, base, a.n_pad - 1);
+  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad + base;
+  for (int e = threadIdx.x; e < PNL; e += 256) gw[e] = w[e];
+}
+
+// Two exchange distances (j and j/2) of level kk in one pass over scratch: a
+// lane owns the four words i, i + j/2, i + j, i + 3j/2 that these two steps
+// keep among themselves. j/2 >= PNL.
+__global__ __launch_bounds__(256) void psort_exchange2_kernel(SortArgs a, int64_t kk, int64_t j) {
+  const int64_t quarter = a.n_pad / 4, h = j >> 1;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= a.slices * quarter) return;
+  const int64_t s = t / quarter, p = t % quarter;
+  // insert zero bits at positions log2(h) and log2(j)
+  int64_t i = ((p & ~(h - 1)) << 1) | (p & (h - 1));
+  i = ((i & ~(j - 1)) << 1) | (i & (j - 1));
+  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad;
+  const bool up = (i & kk) == 0;
+  uint64_t e0 = gw[i], e1 = gw[i + h], e2 = gw[i + j], e3 = gw[i + j + h];
+  auto cx = [&](uint64_t &x, uint64_t &y) {
+    const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
+    x = up ? lo : hi;
+    y = up ? hi : lo;
+  };
+  cx(e0, e2);
+  cx(e1, e3);
+  cx(e0, e1);
+  cx(e2, e3);
+  gw[i] = e0;
+  gw[i + h] = e1;
+  gw[i + j] = e2;
+  gw[i + j + h] = e3;
+}
+__global__ __launch_bounds__(256) void psort_exchange_kernel(SortArgs a, int64_t kk, int64_t j) {
+  const int64_t half = a.n_pad / 2;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= a.slices * half) return;
+  const int64_t s = t / half, p = t % half;
+  const int64_t i = ((p & ~(j - 1)) << 1) | (p & (j - 1)), l = i | j;
+  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad;
+  const bool up = (i & kk) == 0;
+  const uint64_t x = gw[i], y = gw[l];
+  const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
+  gw[i] = up ? lo : hi;
+  gw[l] = up ? hi : lo;
+}
+
+template <int DT, int MODE>
+__global__ __launch_bounds__(256) void psort_merge_kernel(SortArgs a, int64_t kk, int final) {
+  __shared__ uint64_t w[PNL];
+  const int64_t chunks = a.n_pad / PNL;
+  const int64_t s = blockIdx.x / chunks, base = (blockIdx.x % chunks) * PNL;
+  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad + base;
+  for (int e = threadIdx.x; e < PNL; e += 256) w[e] = gw[e];
+  __syncthreads();
+  packed_level(w, PNL, kk, PNL >> 1, base, a.n_pad - 1);
+  if (!final) {
+    for (int e = threadIdx.x; e < PNL; e += 256) gw[e] = w[e];
+    return;
+  }
+  int64_t io, oo;
+  slice_offsets(a, s, io, oo);
+  for (int e = threadIdx.x; e < PNL; e += 256) {
+    const int64_t i = base + e;
+    if (i < a.n) packed_store<DT, MODE>(a, oo, io, i, w[e]);
+  }
+}
+
+template <int DT, int MODE>
+int psort_run(nxh_context *ctx, const char *op, SortArgs &a) {
+  if (a.n_pad <= PNL) {
+    int spb = (int)std::max<int64_t>(1, 1024 / a.n_pad);
+    if (spb > a.slices) spb = (int)a.slices;
+    const int64_t blocks = (a.slices + spb - 1) / spb;
+    if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many slices for one launch");
+    nxh_set_path("sort_lds");
+    hipLaunchKernelGGL((psort_lds_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a, spb);
+    NXH_HIP(op, hipGetLastError());
+    return NXH_OK;
+  }
+  const int64_t chunks = a.n_pad / PNL, blocks = a.slices * chunks;
+  const int64_t pairs = a.slices * (a.n_pad / 2), quads = pairs / 2;
+  if (blocks > 0x7fffffffLL || (pairs + 255) / 256 > 0x7fffffffLL)
+    return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  Scratch scratch(ctx);
+  if (scratch.get(0, (size_t)(a.slices * a.n_pad) * sizeof(uint64_t))) return nxh_fail(NXH_FAILURE, op, NXH_ERR_ALLOC);
+  a.keys = scratch.p[0];
+  nxh_set_path("sort_global");
+  hipLaunchKernelGGL((psort_chunks_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
+  for (int64_t kk = 2 * (int64_t)PNL; kk <= a.n_pad; kk <<= 1) {
+    int64_t j = kk >> 1;
+    for (; (j >> 1) >= PNL; j >>= 2)
+      hipLaunchKernelGGL(psort_exchange2_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, ctx->stream, a, kk, j);
+    for (; j >= PNL; j >>= 1)
+      hipLaunchKernelGGL(psort_exchange_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, ctx->stream, a, kk, j);
+    hipLaunchKernelGGL((psort_merge_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a, kk,
+                       kk == a.n_pad ? 1 : 0);
+  }
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
 template <int DT, int MODE>
 int sort_run(nxh_context *ctx, const char *op, SortArgs &a) {
   using C = typename Tr<DT>::C;
   constexpr int NL = lds_elems<DT>();
+  if constexpr (Packed<DT>::ok) return psort_run<DT, MODE>(ctx, op, a);
   if (a.n_pad <= NL) {
     // several short slices per block, at least 1024 elements of work
     int spb = (int)std::max<int64_t>(1, std::min<int64_t>(NL, 1024) / a.n_pad);
