@@ -48,8 +48,10 @@ struct WindowArgs {
 // magnitude slower on this machine), int64_t otherwise. Memory offsets are
 // always 64-bit. `rows_per_block` > 1 packs several short rows into one block,
 // one window per lane.
-template <class E, class I, int KT>
+template <class E, class I, int KT, int VW>
 __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, int rows_per_block) {
+  // With VW > 1 a "window" below is a unit of VW consecutive windows of the last
+  // window dim (a.L and a.win[KT-1] count units); the unit is stored as one vector.
   const I L = (I)a.L;
   I row, w0;
   int reps = WINDOWS_PER_LANE;
@@ -84,6 +86,9 @@ __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, in
   }
   const E *in = reinterpret_cast<const E *>(a.in);
   E *out = reinterpret_cast<E *>(a.out);
+  struct alignas(sizeof(E) * VW) Pack {
+    E v[VW];
+  };
 #pragma unroll
   for (int u = 0; u < WINDOWS_PER_LANE; u++) {
     const I wf = w0 + (I)u * 256;
@@ -91,14 +96,21 @@ __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, in
     bool valid = true;
     int64_t off = io;
 #pragma unroll
-    for (int d = 0; d < KT; d++) {
+    for (int d = 0; d < KT - 1; d++) {
       const I sp = wc[d] * (I)a.stride[d] + tap[d];
       valid = valid && sp >= 0 && sp < (I)a.extent[d];
       off += (int64_t)sp * a.sp_stride[d];
     }
-    E v = E{};
-    if (valid) v = in[off];
-    out[oo + (int64_t)wf * a.win_stride] = v;
+    Pack pk;
+#pragma unroll
+    for (int v = 0; v < VW; v++) {
+      const I sp = (wc[KT - 1] * VW + v) * (I)a.stride[KT - 1] + tap[KT - 1];
+      const bool ok = valid && sp >= 0 && sp < (I)a.extent[KT - 1];
+      pk.v[v] = E{};
+      if (ok) pk.v[v] = in[off + (int64_t)sp * a.sp_stride[KT - 1]];
+    }
+    if constexpr (VW == 1) out[oo + (int64_t)wf * a.win_stride] = pk.v[0];
+    else *reinterpret_cast<Pack *>(out + oo + (int64_t)wf * VW) = pk;
     // 256 windows further: add the digits of 256, carrying towards the front
     I carry = 0;
 #pragma unroll
@@ -207,8 +219,8 @@ void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt) {
 #undef NXH_FOLD_CASE
 }
 
-template <class E>
-int unfold_launch(nxh_context *ctx, const char *op, const WindowArgs &a, int kt) {
+template <class E, int VW>
+int unfold_launch_v(nxh_context *ctx, const char *op, const WindowArgs &a, int kt) {
   int rows_per_block = 1;
   int64_t wblocks = (a.L + 256 * WINDOWS_PER_LANE - 1) / (256 * WINDOWS_PER_LANE), blocks = a.rows * wblocks;
   if (a.L <= 128) {  // short rows: a power-of-two share of the block per row
@@ -220,14 +232,14 @@ int unfold_launch(nxh_context *ctx, const char *op, const WindowArgs &a, int kt)
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
   const dim3 grid((unsigned)blocks), block(256);
   const bool narrow = fits_int32(a);
-#define NXH_UNFOLD_CASE(KT)                                                                                 \
-  case KT:                                                                                                  \
-    if (narrow)                                                                                             \
-      hipLaunchKernelGGL((unfold_kernel<E, int32_t, KT>), grid, block, 0, ctx->stream, a, (int32_t)wblocks, \
-                         rows_per_block);                                                                   \
-    else                                                                                                    \
-      hipLaunchKernelGGL((unfold_kernel<E, int64_t, KT>), grid, block, 0, ctx->stream, a, wblocks,          \
-                         rows_per_block);                                                                   \
+#define NXH_UNFOLD_CASE(KT)                                                                                     \
+  case KT:                                                                                                      \
+    if (narrow)                                                                                                 \
+      hipLaunchKernelGGL((unfold_kernel<E, int32_t, KT, VW>), grid, block, 0, ctx->stream, a, (int32_t)wblocks, \
+                         rows_per_block);                                                                       \
+    else                                                                                                        \
+      hipLaunchKernelGGL((unfold_kernel<E, int64_t, KT, VW>), grid, block, 0, ctx->stream, a, wblocks,          \
+                         rows_per_block);                                                                       \
     break;
   switch (kt) {
     NXH_UNFOLD_CASE(1)
@@ -237,6 +249,25 @@ int unfold_launch(nxh_context *ctx, const char *op, const WindowArgs &a, int kt)
   }
 #undef NXH_UNFOLD_CASE
   return NXH_OK;
+}
+
+// Four consecutive windows of the last window dim become one store when the
+// output allows it: that dim's window count a multiple of 4, windows
+// contiguous, every row of the output starting on a 4-element boundary.
+template <class E>
+int unfold_launch(nxh_context *ctx, const char *op, WindowArgs &a, int kt, bool vector_ok) {
+  constexpr int VW = sizeof(E) <= 4 ? 4 : 1;
+  if (VW > 1 && vector_ok && a.win[kt - 1] % VW == 0) {
+    a.L /= VW;
+    a.win[kt - 1] /= VW;
+    int64_t rest = 256;
+    for (int s = kt - 1; s >= 0; s--) {  // 256 units further, in the new radix
+      a.step[s] = rest % a.win[s];
+      rest /= a.win[s];
+    }
+    return unfold_launch_v<E, VW>(ctx, op, a, kt);
+  }
+  return unfold_launch_v<E, 1>(ctx, op, a, kt);
 }
 
 // Parameters common to both directions. `plain` is the un-windowed tensor
@@ -327,15 +358,18 @@ NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
   if (a.total > 0x7fffffffLL * 256) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
   a.in = (const char *)x->data + x->offset * es;
   a.out = (char *)out->data + out->offset * es;
+  bool vector_ok = a.win_stride == 1 && a.tap_stride % 4 == 0 && ((uintptr_t)a.out % (uintptr_t)(4 * es)) == 0;
+  for (int d = 0; d < a.ld; d++)
+    if (a.lshape[d] > 1 && a.l_out[d] % 4 != 0) vector_ok = false;
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path("unfold");
   switch (es) {
-    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt); break;
-    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt); break;
-    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt); break;
-    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt); break;
-    default: rc = unfold_launch<G16w>(ctx, op, a, kt); break;
+    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt, vector_ok); break;
+    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt, vector_ok); break;
+    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt, vector_ok); break;
+    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt, vector_ok); break;
+    default: rc = unfold_launch<G16w>(ctx, op, a, kt, vector_ok); break;
   }
   if (rc) return rc;
   NXH_HIP(op, hipGetLastError());
