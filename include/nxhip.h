@@ -296,6 +296,18 @@ int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q,
                   const nxh_tensor *k, const nxh_tensor *v, const void *scale,
                   const nxh_tensor *mask, const void *masked_value, int causal);
 
+/* kaun/lib/linear.ml:50-52 (matmul, then the bias add) followed by the residual
+   add of kaun/examples/04-gpt2/gpt2.ml:165-176, inside the GEMM's epilogue:
+     out = (matmul x w + bias) + residual
+   each of the three results rounded to the dtype as its primitive would store
+   it, so the value equals the op-by-op one of this library bit for bit. bias:
+   rank 1 of out's last extent, or NULL; residual: out's shape, or NULL (both
+   NULL is nxh_matmul). f16 / bf16 / f32 operands that take the tiled MFMA GEMM
+   (K a multiple of 128 bytes of k, 16-byte aligned rows, unit-stride output
+   columns); otherwise Failure and the caller issues the primitives. */
+int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+               const nxh_tensor *w, const nxh_tensor *bias, const nxh_tensor *residual);
+
 /* ── measurement ─────────────────────────────────────────────────────────── */
 
 /* HIP events recorded on the context stream: start, then stop returns the

@@ -97,6 +97,7 @@ SIGNATURES = {
     "nxh_softmax_rows": (C.c_int, [_CTX, _T, _T, C.c_void_p, _T, C.c_void_p]),
     "nxh_layer_norm_rows": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_double]),
     "nxh_gelu_tanh": (C.c_int, [_CTX, _T, _T, C.c_void_p]),
+    "nxh_linear": (C.c_int, [_CTX, _T, _T, _T, _T, _T]),
     "nxh_attention": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_void_p, _T, C.c_void_p, C.c_int]),
     "nxh_timer_start": (C.c_int, [_CTX]),
     "nxh_timer_stop": (C.c_int, [_CTX, _P(C.c_float)]),

@@ -111,6 +111,10 @@ struct Args {
   int nbd;
   uint32_t bshape[4];
   int64_t ba[4], bb[4], bc[4];
+  // EPI kernels only: out = round(round(round(A B) + bias[col]) + R), each step
+  // skipped when its pointer is null. R has C's shape, unit column stride.
+  const void *bias, *R;
+  int64_t ldr, br[4];
 };
 
 // One k-step of one 32x32 tile: a, b hold this lane's VE k-values of its row.
@@ -206,7 +210,7 @@ __device__ __forceinline__ void tile_of_block(const Args &a, uint32_t bid, uint3
   tn = in_strip / gsz;
 }
 
-template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE>
+template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI = false>
 __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   constexpr int THREADS = SH::THREADS, BM = SH::BM, BN = SH::BN, TM = SH::TM, TN = SH::TN;
   constexpr int NVA = SH::NVA, NVB = SH::NVB, BK = Geo<EL>::BK;
@@ -218,7 +222,7 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   // tiles are walked from the end: an operand the previous kernel has just written
   // front to back still has its tail in the memory-side cache
   tile_of_block(a, gridDim.x - 1 - blockIdx.x, batch, tm, tn);
-  int64_t ao = 0, bo = 0, co = 0;
+  int64_t ao = 0, bo = 0, co = 0, ro = 0;
   {
     uint32_t idx = batch;
 #pragma unroll
@@ -229,6 +233,7 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
         ao += (int64_t)c * a.ba[i];
         bo += (int64_t)c * a.bb[i];
         co += (int64_t)c * a.bc[i];
+        if constexpr (EPI) ro += (int64_t)c * a.br[i];
       }
     }
   }
@@ -339,19 +344,35 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   // accumulator element e of lane l is C[(e/4)*8 + (l/32)*4 + e%4][l%32]
   S *C = (S *)a.C + co;
   const int r32 = lane & 31, kg = lane >> 5;
+  auto narrow = [](float x) -> S {
+    if constexpr (EL::F32) return x;
+    else return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x);
+  };
+  auto widen = [](S x) -> float {
+    if constexpr (EL::F32) return x;
+    else return EL::BF16 ? bf16_to_f32(x) : f16_to_f32(x);
+  };
 #pragma unroll
   for (int t = 0; t < TM; t++)
 #pragma unroll
     for (int u = 0; u < TN; u++) {
       const int cl = wn + u * 32 + r32;
       if (EDGE && cl >= edge_n) continue;
+      float bias = 0.0f;
+      if constexpr (EPI)
+        if (a.bias) bias = widen(((const S *)a.bias)[n0 + cl]);
 #pragma unroll
       for (int e = 0; e < 16; e++) {
         const int rl = wm + t * 32 + (e >> 2) * 8 + kg * 4 + (e & 3);
         if (EDGE && rl >= edge_m) continue;
         S *c = C + (m0 + rl) * a.ldc + n0 + cl;
-        if constexpr (EL::F32) *c = acc[t][u][e];
-        else *c = EL::BF16 ? f32_to_bf16(acc[t][u][e]) : f32_to_f16(acc[t][u][e]);
+        S v = narrow(acc[t][u][e]);
+        if constexpr (EPI) {
+          // the bias add and the residual add of the op-by-op sequence, each rounded to the dtype
+          if (a.bias) v = narrow(widen(v) + bias);
+          if (a.R) v = narrow(widen(v) + widen(((const S *)a.R)[ro + (m0 + rl) * a.ldr + n0 + cl]));
+        }
+        *c = v;
       }
     }
 }

@@ -645,9 +645,9 @@ static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // The LDS-tiled family of gemm_tile.hpp: K a multiple of one slab (64 two-byte or
 // 32 four-byte elements), 16-byte aligned rows, unit-stride C. Returns -1 when the call does not qualify.
-template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE>
+template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI>
 static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
-  auto kern = gemm_tile::kernel<EL, A_KC, B_KC, SH, EDGE>;
+  auto kern = gemm_tile::kernel<EL, A_KC, B_KC, SH, EDGE, EPI>;
   constexpr size_t LDS = SH::template lds_bytes<EL>();
   // once per process and kernel (contexts have separate mutexes): allow > 64 KiB of dynamic LDS
   static std::once_flag once;
@@ -663,11 +663,11 @@ static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
   NXH_HIP("matmul", hipGetLastError());
   return NXH_OK;
 }
-template <class EL, class SH>
+template <class EL, class SH, bool EPI>
 static int launch_tile_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc, const char *path) {
   const bool edge = g.M % SH::BM != 0 || g.N % SH::BN != 0;
-#define NXH_TILE(AK, BK_)                                                        \
-  (edge ? launch_tile<EL, AK, BK_, SH, true>(ctx, g, path) : launch_tile<EL, AK, BK_, SH, false>(ctx, g, path))
+#define NXH_TILE(AK, BK_)                                                                  \
+  (edge ? launch_tile<EL, AK, BK_, SH, true, EPI>(ctx, g, path) : launch_tile<EL, AK, BK_, SH, false, EPI>(ctx, g, path))
   if (a_kc) return b_kc ? NXH_TILE(true, true) : NXH_TILE(true, false);
   return b_kc ? NXH_TILE(false, true) : NXH_TILE(false, false);
 #undef NXH_TILE
@@ -681,8 +681,14 @@ static int forced_tile() {
   }();
   return v;
 }
-template <class EL>
-static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b) {
+// The epilogue operands of nxh_linear (null members: that step is left out).
+struct Epilogue {
+  const void *bias = nullptr, *R = nullptr;
+  int64_t ldr = 0, br[MM_MAXB] = {};
+};
+template <class EL, bool EPI = false>
+static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b,
+                    const Epilogue *epi = nullptr) {
   constexpr int VE = EL::VE, BK = gemm_tile::Geo<EL>::BK;
   if (a.K % BK || a.K < BK || a.M < VE || a.N < VE) return -1;
   if (a.ccs != 1 || a.batch.n > 4 || !al_a || !al_b) return -1;
@@ -707,6 +713,12 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
     g.ba[i] = a.batch.a[i];
     g.bb[i] = a.batch.b[i];
     g.bc[i] = a.batch.c[i];
+    if (EPI) g.br[i] = epi->br[i];
+  }
+  if (EPI) {
+    g.bias = epi->bias;
+    g.R = epi->R;
+    g.ldr = epi->ldr;
   }
   auto tiles = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * (int64_t)nbatch; };
   if (tiles(128, 64) > 0x7fffffffLL) return -1;
@@ -723,9 +735,20 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       pick = c256 <= c128 ? 256 : 128;
     }
   }
-  if (pick == 64) return launch_tile_oriented<EL, gemm_tile::Shape256x64>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
-  if (pick == 128) return launch_tile_oriented<EL, gemm_tile::Shape128x128>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
-  return launch_tile_oriented<EL, gemm_tile::Shape256x256>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
+  if constexpr (EPI) {
+    // Two block shapes are enough for the epilogue family; f16 keeps to the small one (its
+    // conversions make the 256x256 epilogue too large to stay in registers).
+    constexpr bool big_ok = EL::F32 || EL::BF16;
+    if (pick == 64 || !big_ok) pick = 128;
+    if (pick == 128)
+      return launch_tile_oriented<EL, gemm_tile::Shape128x128, true>(ctx, g, a_kc, b_kc, "linear_tile_128x128");
+    if constexpr (big_ok)
+      return launch_tile_oriented<EL, gemm_tile::Shape256x256, true>(ctx, g, a_kc, b_kc, "linear_tile_256x256");
+  }
+  if (pick == 64) return launch_tile_oriented<EL, gemm_tile::Shape256x64, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
+  if (pick == 128)
+    return launch_tile_oriented<EL, gemm_tile::Shape128x128, false>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
+  return launch_tile_oriented<EL, gemm_tile::Shape256x256, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
 }
 
 template <class MM>
@@ -756,12 +779,16 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
   return launch_mfma<MM>(ctx, a, nbatch);
 }
 
-NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tensor *A, const nxh_tensor *B) {
-  const char *op = "matmul";
+// matmul, and with `bias` / `R` the fused linear: C = A B, then + bias[col], then
+// + R, each rounded to the dtype (tiled MFMA path only).
+static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, const nxh_tensor *A,
+                        const nxh_tensor *B, const nxh_tensor *bias, const nxh_tensor *R) {
   if (!ctx || !C || !A || !B) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, C);
   if (!rc) rc = nxh_check_tensor(op, A);
   if (!rc) rc = nxh_check_tensor(op, B);
+  if (!rc && bias) rc = nxh_check_tensor(op, bias);
+  if (!rc && R) rc = nxh_check_tensor(op, R);
   if (rc) return rc;
   if (A->dtype != B->dtype || A->dtype != C->dtype) return nxh_fail(NXH_FAILURE, op, NXH_ERR_MM_DTYPE);
   const int dt = A->dtype;
@@ -774,12 +801,24 @@ NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tenso
   const int64_t kk = B->shape[B->ndim - 2], n = B->shape[B->ndim - 1];
   if (k != kk || C->shape[nd - 2] != m || C->shape[nd - 1] != n)
     return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  const bool fused = bias || R;
+  if (bias && (bias->dtype != dt || bias->ndim != 1 || bias->shape[0] != n))
+    return nxh_fail(bias->dtype != dt ? NXH_FAILURE : NXH_INVALID_ARGUMENT, op, bias->dtype != dt ? NXH_ERR_MM_DTYPE : NXH_ERR_SHAPE);
+  if (R) {
+    if (R->dtype != dt) return nxh_fail(NXH_FAILURE, op, NXH_ERR_MM_DTYPE);
+    if (R->ndim != nd) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+    for (int i = 0; i < nd; i++)
+      if (R->shape[i] != C->shape[i]) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
+  }
+  if (fused && dt != NXH_BF16 && dt != NXH_F16 && dt != NXH_F32) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  if (fused && ((bias && n > 1 && bias->strides[0] != 1) || (R && n > 1 && R->strides[nd - 1] != 1)))
+    return nxh_fail(NXH_FAILURE, op, "bias and residual must be contiguous along the columns");
 
   GemmArgs g;
   // batch broadcast strides (nx_c_matmul.c:895-926), then drop size-1 dims and
   // merge neighbours that compose on all three operands
   const int bnd = nd - 2, abo = nd - A->ndim, bbo = nd - B->ndim;
-  int64_t bs[NXH_MAX_NDIM], as_[NXH_MAX_NDIM], bs_[NXH_MAX_NDIM], cs_[NXH_MAX_NDIM];
+  int64_t bs[NXH_MAX_NDIM], as_[NXH_MAX_NDIM], bs_[NXH_MAX_NDIM], cs_[NXH_MAX_NDIM], rs_[NXH_MAX_NDIM];
   int nb = 0;
   int64_t nbatch = 1;
   for (int i = 0; i < bnd; i++) {
@@ -799,16 +838,20 @@ NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tenso
     nbatch *= s;
     if (s == 1) continue;
     const int64_t xa = sa == 1 ? 0 : sta, xb = sb == 1 ? 0 : stb, xc = C->strides[i];
-    if (nb > 0 && as_[nb - 1] == xa * s && bs_[nb - 1] == xb * s && cs_[nb - 1] == xc * s) {
+    const int64_t xr = R ? R->strides[i] : 0;
+    if (nb > 0 && as_[nb - 1] == xa * s && bs_[nb - 1] == xb * s && cs_[nb - 1] == xc * s &&
+        rs_[nb - 1] == xr * s) {
       bs[nb - 1] *= s;
       as_[nb - 1] = xa;
       bs_[nb - 1] = xb;
       cs_[nb - 1] = xc;
+      rs_[nb - 1] = xr;
     } else {
       bs[nb] = s;
       as_[nb] = xa;
       bs_[nb] = xb;
       cs_[nb] = xc;
+      rs_[nb] = xr;
       nb++;
     }
   }
@@ -852,6 +895,22 @@ NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tenso
 
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
+  if (fused) {
+    Epilogue epi;
+    epi.bias = bias ? (const char *)bias->data + bias->offset * es : nullptr;
+    epi.R = R ? (const char *)R->data + R->offset * es : nullptr;
+    epi.ldr = R ? R->strides[nd - 2] : 0;
+    for (int i = 0; i < nb && i < MM_MAXB; i++) epi.br[i] = rs_[i];
+    const bool a_ok = g.acs == 1 || g.ars == 1, b_ok = g.brs == 1 || g.bcs == 1;
+    rc = -1;
+    if (a_ok && b_ok) {
+      if (dt == NXH_BF16) rc = try_tile<gemm_tile::ElBF16, true>(ctx, g, (uint32_t)nbatch, al_a, al_b, &epi);
+      else if (dt == NXH_F16) rc = try_tile<gemm_tile::ElF16, true>(ctx, g, (uint32_t)nbatch, al_a, al_b, &epi);
+      else rc = try_tile<gemm_tile::ElF32, true>(ctx, g, (uint32_t)nbatch, al_a, al_b, &epi);
+    }
+    if (rc == -1) return nxh_fail(NXH_FAILURE, op, "operands do not fit the tiled GEMM (K a multiple of 64 bytes-of-k slabs, aligned rows)");
+    return rc;
+  }
   switch (dt) {
     case NXH_BF16: return run_mfma_dtype<MMbf16>(ctx, g, (uint32_t)nbatch, al_a, al_b);
     case NXH_F16: return run_mfma_dtype<MMf16>(ctx, g, (uint32_t)nbatch, al_a, al_b);
@@ -874,4 +933,14 @@ NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tenso
 #undef NXH_CASE
     default: return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
   }
+}
+
+NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tensor *A, const nxh_tensor *B) {
+  return matmul_entry(ctx, "matmul", C, A, B, nullptr, nullptr);
+}
+
+NXH_EXPORT int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const nxh_tensor *w,
+                          const nxh_tensor *bias, const nxh_tensor *residual) {
+  if (!bias && !residual) return matmul_entry(ctx, "matmul", out, x, w, nullptr, nullptr);
+  return matmul_entry(ctx, "linear", out, x, w, bias, residual);
 }

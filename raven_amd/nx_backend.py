@@ -412,6 +412,24 @@ class Backend:
         self._check(self._lib.nxh_gelu_tanh(self._h, C.byref(o), C.byref(a), enc.ctypes.data))
         return out
 
+    def linear(self, x: Tensor, w: Tensor, bias: Tensor | None = None, residual: Tensor | None = None) -> Tensor:
+        """``(matmul x w + bias) + residual`` in the GEMM's epilogue, every step
+        rounded to the dtype as the primitives would (kaun/lib/linear.ml:50-52)."""
+        xs, ws = x.shape, w.shape
+        nd = max(len(xs), len(ws))
+        batch = []
+        for i in range(nd - 2):
+            ai, bi = i - (nd - len(xs)), i - (nd - len(ws))
+            batch.append(max(xs[ai] if ai >= 0 else 1, ws[bi] if bi >= 0 else 1))
+        out = self.buffer(x.dtype, batch + [xs[-2], ws[-1]])
+        o, a, b = out._desc(), x._desc(), w._desc()
+        bd = bias._desc() if bias is not None else None
+        rd = residual._desc() if residual is not None else None
+        self._check(self._lib.nxh_linear(self._h, C.byref(o), C.byref(a), C.byref(b),
+                                         C.byref(bd) if bd is not None else None,
+                                         C.byref(rd) if rd is not None else None))
+        return out
+
     def attention(self, q: Tensor, k: Tensor, v: Tensor, scale=None, mask: Tensor | None = None,
                   masked_value=None, causal: bool = False) -> Tensor:
         """Scaled dot-product attention of f16 / bf16 operands in one kernel
