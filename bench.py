@@ -357,7 +357,7 @@ class CountingBackend:
     """Forwards to the backend and counts the calls that launch work."""
 
     LAUNCHING = ("unary", "binary", "compare", "where", "cast", "copy", "contiguous", "gather", "reduce",
-                 "matmul", "full", "from_host", "softmax_rows", "layer_norm_rows", "gelu_tanh", "attention")
+                 "matmul", "full", "from_host", "softmax_rows", "layer_norm_rows", "gelu_tanh", "attention", "linear")
 
     def __init__(self, inner):
         self._inner, self.calls = inner, {}
@@ -481,7 +481,7 @@ def config5(hip, iters=3, warmup=1, window=False):
     ms = (time.perf_counter() - t0) * 1e3 / iters
     calls = {k: v // iters for k, v in counter.calls.items()}
     flops = 284812800 * batch * seq  # matmul FLOPs per forward
-    how = ("deferred-evaluation window: attention, layer norm and GELU sequences as fused kernels" if window
+    how = ("deferred-evaluation window: attention, layer norm, GELU and linear sequences as fused kernels" if window
            else "eager, one backend call per primitive")
     rec = {"op": f"cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 ({how})",
            "ms": round(ms, 3), "tokens/s": round(batch * seq / (ms * 1e-3), 1), "hip_event_ms": round(ev_ms, 3),

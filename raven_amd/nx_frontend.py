@@ -32,6 +32,9 @@ def _broadcast_shapes(a: Sequence[int], b: Sequence[int]) -> tuple:
     return tuple(out)
 
 
+_ENCODED: dict = {}  # (dtype name, Python value) -> its encoded storage element
+
+
 class Nx:
     """Frontend functions bound to one backend."""
 
@@ -45,7 +48,14 @@ class Nx:
 
     def scalar(self, dtype: dt.DType, value):
         """frontend.ml:360: ``B.full ctx dt [||] value``."""
-        return self.B.full(dtype, (), encode_scalar(dtype, value))
+        key = (dtype.name, value)
+        enc = _ENCODED.get(key)
+        if enc is None:
+            enc = encode_scalar(dtype, value)
+            enc.setflags(write=False)
+            if len(_ENCODED) < 1024 and value == value:  # a NaN never equals its own key
+                _ENCODED[key] = enc
+        return self.B.full(dtype, (), enc)
 
     def scalar_like(self, x, value):
         return self.scalar(x.dtype, value)
@@ -64,7 +74,7 @@ class Nx:
         if tuple(x.shape) == shape:
             return x
         pad = len(shape) - len(x.shape)
-        if pad > 0:
+        if pad > 0 and len(x.shape) > 0:  # a rank-0 view expands to any rank directly (view.ml expand)
             x = self.B.reshape(x, (1,) * pad + tuple(x.shape))
         return self.B.expand(x, shape)
 

@@ -168,7 +168,7 @@ class Window:
         self.fuse = fuse
         self.entries: List[Entry] = []
         self.stats = {"recorded": 0, "issued": 0, "softmax_rows": 0, "layer_norm_rows": 0, "gelu_tanh": 0,
-                      "attention": 0, "flushes": 0, "fallbacks": 0}
+                      "attention": 0, "linear": 0, "flushes": 0, "fallbacks": 0}
 
     # ── handles ─────────────────────────────────────────────────────────────
     def _wrap(self, t, scalar=None) -> WTensor:
@@ -471,7 +471,23 @@ def _rows_ok(o: Operand, shape) -> bool:
 
 
 def _match(w: Window, e: Entry) -> Optional[Plan]:
-    for m in (_match_attention, _match_softmax, _match_layer_norm, _match_gelu):
+    """Tries the runs that can END in an entry of e's kind."""
+    if e.kind == "matmul":
+        matchers = (_match_attention,)
+    elif e.kind == "cast":
+        matchers = (_match_softmax,)
+    elif e.kind == "binary":
+        if e.op == "add":
+            matchers = (_match_linear, _match_layer_norm)
+        elif e.op == "mul":
+            matchers = (_match_gelu,)
+        elif e.op == "fdiv":
+            matchers = (_match_softmax,)
+        else:
+            return None
+    else:
+        return None
+    for m in matchers:
         p = m(w, e)
         if p is not None:
             return p
@@ -596,6 +612,62 @@ def _match_attention(w: Window, anchor: Entry) -> Optional[Plan]:
                                win._tensor_of(mask) if mask is not None else None, as_f32(masked), causal)
 
     return Plan("attention", interior, run)
+
+
+def _match_linear(w: Window, anchor: Entry) -> Optional[Plan]:
+    """kaun/lib/linear.ml:50-52 and the residual add around it (gpt2.ml:165-176):
+    add(matmul(x, w), bias), optionally inside add(residual, .), as one GEMM with
+    the adds in its epilogue."""
+    if anchor.kind != "binary" or anchor.op != "add" or anchor.dtype.name not in ("float16", "bfloat16", "float32"):
+        return None
+    shape = anchor.shape
+    if len(shape) < 2:
+        return None
+
+    def biased(o: Operand):
+        """(matmul entry, bias operand) if `o` is add(matmul, broadcast vector)."""
+        e = _producer(o, "binary", "add")
+        if e is None:
+            return None
+        mm = _producer(e.ins[0], "matmul")
+        b = e.ins[1]
+        if mm is None or b.entry is not None or not _vector_broadcast(b.view, shape):
+            return None
+        return e, mm, b
+
+    interior, bias, residual, mm = None, None, None, None
+    # residual + (matmul + bias), either operand order; then matmul + bias; then residual + matmul
+    for inner, other in ((anchor.ins[1], anchor.ins[0]), (anchor.ins[0], anchor.ins[1])):
+        hit = biased(inner)
+        if hit is not None and _hidden([hit[0], hit[1]], anchor) and other.view.shape == tuple(shape):
+            interior, mm, bias, residual = [hit[0], hit[1]], hit[1], hit[2], other
+            break
+    if interior is None:
+        m0 = _producer(anchor.ins[0], "matmul")
+        if m0 is not None and anchor.ins[1].entry is None and _vector_broadcast(anchor.ins[1].view, shape) \
+                and _hidden([m0], anchor):
+            interior, mm, bias = [m0], m0, anchor.ins[1]
+    if interior is None:
+        for inner, other in ((anchor.ins[1], anchor.ins[0]), (anchor.ins[0], anchor.ins[1])):
+            m0 = _producer(inner, "matmul")
+            if m0 is not None and _hidden([m0], anchor) and other.view.shape == tuple(shape):
+                interior, mm, residual = [m0], m0, other
+                break
+    if interior is None or tuple(mm.shape) != tuple(shape):
+        return None
+    if residual is not None and shape[-1] > 1 and residual.view.strides[-1] != 1:
+        return None
+    x, wt = mm.ins
+
+    def vector(win: Window, o: Operand):
+        t = win._tensor_of(o)
+        return win.B.with_view(t, View.create((shape[-1],), (o.view.strides[-1] if shape[-1] > 1 else 1,), o.view.offset))
+
+    def run(win: Window):
+        return win.B.linear(win._tensor_of(x), win._tensor_of(wt), vector(win, bias) if bias is not None else None,
+                            win._tensor_of(residual) if residual is not None else None)
+
+    return Plan("linear", interior, run)
 
 
 def _match_layer_norm(w: Window, anchor: Entry) -> Optional[Plan]:

@@ -118,6 +118,7 @@ def test_gpt2_forward_through_the_window_on_the_gpu(hip, oracle, d):
     assert (win.stats["layer_norm_rows"], win.stats["gelu_tanh"]) == (2 * L + 1, L)
     # head dim 64: bfloat16 runs the whole attention core as one kernel, float32 its softmax
     assert (win.stats["attention"], win.stats["softmax_rows"]) == ((L, 0) if d is dt.bfloat16 else (0, L))
+    assert win.stats["linear"] == 6 * L   # every bias add, and the two residual adds, ride their GEMM
     assert win.stats["fallbacks"] == 0
     eager = decode(logical(run(hip, oracle, SMALL, hp, ids, d)), d, oracle)
     want = decode(logical(run(oracle, oracle, SMALL, hp, ids, d)), d, oracle)

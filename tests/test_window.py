@@ -58,6 +58,14 @@ class SequencedOracle(OracleBackend):
             sc = nx.where(mask, sc, self.full(dt.float32, (), masked_value))
         return nx.matmul(nx.cast(q.dtype, nx.softmax(sc)), v)
 
+    def linear(self, x, w, bias=None, residual=None):
+        self.calls.append("linear")
+        nx = Nx(self)
+        y = nx.matmul(x, w)
+        if bias is not None:
+            y = nx.add(y, bias)
+        return nx.add(residual, y) if residual is not None else y
+
     def gelu_tanh(self, x, constants):
         self.calls.append("gelu_tanh")
         nx = Nx(self)
@@ -103,10 +111,12 @@ def test_gpt2_forward_through_the_window_fuses_every_sequence(oracle, d):
         # float32 has no float32 island: the softmax alone is fused
         assert (w.stats["attention"], w.stats["softmax_rows"]) == (0, L)
         assert base.calls.count("softmax_rows") == L
-    # what is left op by op per block: 6 linears (matmul + bias add), 2 residual
-    # adds, the mask compare, and for float32 the two attention matmuls;
-    # outside the blocks the embedding add and the head matmul
-    per_block = 12 + 2 + 1 + (0 if d is dt.bfloat16 else 2)
+    # the six linears of a block take their bias add, and two of them the residual
+    # add, into the GEMM; what is left op by op per block is the mask compare and,
+    # for float32, the two attention matmuls; outside the blocks the embedding
+    # add and the head matmul
+    assert w.stats["linear"] == 6 * L and base.calls.count("linear") == 6 * L
+    per_block = 1 + (0 if d is dt.bfloat16 else 2)
     assert w.stats["issued"] == L * per_block + 2
     # with fusion switched off the window only defers
     w2 = Window(SequencedOracle(), fuse=False)
@@ -273,3 +283,40 @@ def test_errors_and_limits(oracle):
     y = nx.softmax(wide)
     assert np.allclose(value(win, y), 1 / 9000)
     assert win.stats["softmax_rows"] == 0
+
+
+def test_linear_runs(oracle):
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((2, 6, 16)).astype(np.float32)
+    wt = rng.standard_normal((16, 8)).astype(np.float32)
+    b = rng.standard_normal(8).astype(np.float32)
+    r = rng.standard_normal((2, 6, 8)).astype(np.float32)
+
+    def run(B, form, keep=None):
+        nx = Nx(B)
+        tx, tw, tb, tr = (nx.create(dt.float32, a.shape, a) for a in (x, wt, b, r))
+        y = nx.matmul(tx, tw)
+        if form in ("bias", "both", "both-flipped"):
+            y = nx.add(y, tb)
+        if keep is not None:
+            keep.append(y)
+        if form == "both":
+            y = nx.add(tr, y)
+        elif form in ("both-flipped", "residual"):
+            y = nx.add(y, tr)
+        return y
+
+    for form, calls in (("bias", 1), ("both", 1), ("both-flipped", 1), ("residual", 1), ("plain", 0)):
+        base = SequencedOracle()
+        w = Window(base)
+        got = value(w, run(w, form))
+        assert np.array_equal(got, ological(run(oracle, form))), form
+        assert base.calls.count("linear") == calls and w.stats["linear"] == calls, (form, base.calls)
+    # the biased product kept alive: only the bias add joins the GEMM, the residual add is issued
+    base = SequencedOracle()
+    w = Window(base)
+    kept, okept = [], []
+    got = value(w, run(w, "both", kept))
+    want = ological(run(oracle, "both", okept))
+    assert np.array_equal(got, want) and np.array_equal(value(w, kept[0]), ological(okept[0]))
+    assert w.stats["linear"] == 1 and w.stats["issued"] == 1
