@@ -352,6 +352,70 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
     if constexpr (EL::F32) return x;
     else return EL::BF16 ? bf16_to_f32(x) : f16_to_f32(x);
   };
+  if constexpr (!EL::F32) {
+    // 16-bit outputs go through LDS: in accumulator order a lane would store
+    // (and, with a residual, load) two bytes at a time. Each wave parks its
+    // rounded TM*32 x TN*32 patch in a private piece of the (now idle) stage
+    // buffers and sends it out as whole 16-byte row segments.
+    constexpr int WC = TN * 32, WP = WC + 8;  // patch width and its LDS pitch (elements)
+    static_assert((size_t)SH::WM * SH::WN * TM * 32 * WP * sizeof(S) <= SH::template lds_bytes<EL>(), "epilogue patch");
+    const bool wide = ((uintptr_t)C % 16) == 0 && a.ldc % 8 == 0 &&
+                      (!EPI || ((!a.bias || (uintptr_t)a.bias % 16 == 0) &&
+                                (!a.R || (((uintptr_t)((const S *)a.R + ro)) % 16 == 0 && a.ldr % 8 == 0))));
+    if (wide) {
+      __syncthreads();  // every wave has read its last fragments
+      S *patch = smem + wave * (TM * 32 * WP);
+#pragma unroll
+      for (int t = 0; t < TM; t++)
+#pragma unroll
+        for (int u = 0; u < TN; u++)
+#pragma unroll
+          for (int e = 0; e < 16; e++)
+            patch[(t * 32 + (e >> 2) * 8 + kg * 4 + (e & 3)) * WP + u * 32 + r32] = narrow(acc[t][u][e]);
+      // the patch is read back by other lanes of the same wave only: LDS serves a wave in order
+      constexpr int CPR = WC / 8;  // 16-byte chunks per patch row
+#pragma unroll
+      for (int i = 0; i < TM * 32 * CPR / 64; i++) {
+        const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
+        const int rl = wm + row, cl = wn + col;
+        if (EDGE && (rl >= edge_m || cl >= edge_n)) continue;
+        union {
+          V16 q;
+          S s[8];
+        } v, bb, rr;
+        v.q = *reinterpret_cast<const V16 *>(patch + row * WP + col);
+        S *c = C + (m0 + rl) * a.ldc + n0 + cl;
+        const bool whole = !EDGE || cl + 8 <= edge_n;
+        if constexpr (EPI) {
+          const S *bp = (const S *)a.bias + n0 + cl;
+          const S *rp = (const S *)a.R + ro + (m0 + rl) * a.ldr + n0 + cl;
+          if (whole) {
+            if (a.bias) bb.q = *reinterpret_cast<const V16 *>(bp);
+            if (a.R) rr.q = *reinterpret_cast<const V16 *>(rp);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              if (cl + j < edge_n) {
+                if (a.bias) bb.s[j] = bp[j];
+                if (a.R) rr.s[j] = rp[j];
+              }
+          }
+#pragma unroll
+          for (int j = 0; j < 8; j++) {
+            // the bias add and the residual add of the op-by-op sequence, each rounded to the dtype
+            if (a.bias) v.s[j] = narrow(widen(v.s[j]) + widen(bb.s[j]));
+            if (a.R) v.s[j] = narrow(widen(v.s[j]) + widen(rr.s[j]));
+          }
+        }
+        if (whole) *reinterpret_cast<V16 *>(c) = v.q;
+        else
+#pragma unroll
+          for (int j = 0; j < 8; j++)
+            if (cl + j < edge_n) c[j] = v.s[j];
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int t = 0; t < TM; t++)
 #pragma unroll
