@@ -26,9 +26,16 @@
    - matmul: f64 triple loop on the quantised inputs with the reference's
      tolerances (backend_c/test/matmul_test.ml:831-974) and its cancellation
      witness (matmul_test.ml:182-230).
+   - pad / cat / scan / threefry / scatter / sort / argsort / unfold / fold: the
+     reference tests' vectors (backend_contract.ml:1431-1457, 1661-1666,
+     1727-1925, 2504-2580, 2782-2810; Random123's known answers for threefry)
+     and numpy or brute-force statements of each (pad, concatenate, cumsum,
+     stable sorts, a serial scatter walk, a direct im2col / col2im).
    Parity unpinned bit-for-bit (tolerance only, by the reference's own
    contract): the exact rounding of float sums, transcendental results and GEMM
-   last bits. */
+   last bits. The value sort fixes the order of IEEE +0 / -0, which the
+   reference leaves unspecified (nx_c_sort.c:262-292), to ascending original
+   index. */
 
 #include <complex.h>
 #include <math.h>
