@@ -442,12 +442,13 @@ def cpu_configs():
     return {"host_cores": lib().nxo_ncores(), "ops": out}
 
 
-def config5(hip, iters=3, warmup=1, window=False):
+def config5(hip, iters=3, warmup=1, window=False, graph=False):
     """GPT-2-small-shaped forward (12 layers, d 768, 12 heads, FFN 3072, vocab
     50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s. Eager: one
     backend call per primitive. With ``window``: the same frontend calls go
     through the deferred-evaluation window, which replaces the softmax, layer
-    norm and GELU sequences by the fused row kernels."""
+    norm and GELU sequences by the fused row kernels. With ``graph`` too: the
+    windowed forward is recorded once and each timed step is one replay."""
     from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
     from raven_amd.nx_frontend import Nx
     from raven_amd.nx_window import Window
@@ -470,18 +471,32 @@ def config5(hip, iters=3, warmup=1, window=False):
         out = model.logits(params, ids)
         del out
     front.synchronize()
+    recorded = None
+    if graph:
+        front.capture_begin()
+        try:
+            out = front.force(model.logits(params, ids))
+        finally:
+            recorded = front.capture_end()
     counter.calls.clear()
     t0 = time.perf_counter()
     front.timer_start()
     for _ in range(iters):
-        out = model.logits(params, ids)
-        del out
+        if recorded is not None:
+            recorded.launch()
+        else:
+            out = model.logits(params, ids)
+            del out
     ev_ms = front.timer_stop() / iters
     front.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / iters
     calls = {k: v // iters for k, v in counter.calls.items()}
+    if recorded is not None:
+        del out
+        recorded.destroy()
     flops = 284812800 * batch * seq  # matmul FLOPs per forward
-    how = ("deferred-evaluation window: attention, layer norm, GELU and linear sequences as fused kernels" if window
+    how = ("the windowed forward recorded once, each step one graph replay" if graph else
+           "deferred-evaluation window: attention, layer norm, GELU and linear sequences as fused kernels" if window
            else "eager, one backend call per primitive")
     rec = {"op": f"cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 ({how})",
            "ms": round(ms, 3), "tokens/s": round(batch * seq / (ms * 1e-3), 1), "hip_event_ms": round(ev_ms, 3),
@@ -520,6 +535,7 @@ def main():
     if args.only_gpt2:
         print(json.dumps(config5(hip)))
         print(json.dumps(config5(hip, window=True)))
+        print(json.dumps(config5(hip, window=True, graph=True, iters=10)))
         return
     if args.only_next:
         print(json.dumps({"ops": next_ops(hip, Workloads(hip))}))
@@ -598,6 +614,7 @@ def main():
             hip.trim()
         ops_out.append(config5(hip))
         ops_out.append(config5(hip, window=True))
+        ops_out.append(config5(hip, window=True, graph=True, iters=10))
         ops_out.extend(next_ops(hip, W))
 
     line = {

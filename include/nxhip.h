@@ -308,6 +308,37 @@ int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q,
 int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
                const nxh_tensor *w, const nxh_tensor *bias, const nxh_tensor *residual);
 
+/* ── recorded sequences ──────────────────────────────────────────────────── */
+
+/* The reference backend has no counterpart: its eager calls cost a C stub
+   each (nx_c_stubs.c), where a GPU call costs a launch of several
+   microseconds, which a forward pass of small kernels (Kaun's GPT-2,
+   kaun/examples/gpt2 via rune/lib/autodiff.ml's eager path) is bound by.
+   Between nxh_capture_begin and nxh_capture_end every entry point above
+   records its launches into a HIP graph instead of running them;
+   nxh_graph_launch then replays them all with one call, in stream order with
+   whatever else is issued on the context.
+   - Storage allocated during the capture is the graph's: a tensor that lives on
+     (the result) is overwritten by every replay, and its block returns to the
+     allocator only after both nxh_free and nxh_graph_destroy. Storage that
+     existed before (weights, inputs) is read at replay time as it then is:
+     write new inputs into the same buffers (nxh_assign / nxh_memcpy_h2d)
+     before a replay.
+   - nxh_memcpy_h2d of up to 256 KiB is recorded with a private copy of the
+     bytes. nxh_memcpy_d2h, nxh_synchronize, nxh_trim and the timer fail while
+     capturing (Failure), and so does an allocation the driver refuses.
+   - nxh_gather / nxh_scatter cannot report an index out of bounds from inside a
+     capture: the out-of-range lanes are skipped as always, and the first
+     nxh_synchronize after a replay that met one fails with Failure.
+   - shapes, strides and scalars are frozen at capture; warm every entry point
+     once eagerly before capturing it. */
+typedef struct nxh_graph nxh_graph;
+int nxh_capture_begin(nxh_context *ctx);
+int nxh_capture_end(nxh_context *ctx, nxh_graph **graph);
+int nxh_graph_launch(nxh_context *ctx, nxh_graph *graph);
+/* Waits for the stream, then releases the graph and its idle storage. */
+int nxh_graph_destroy(nxh_context *ctx, nxh_graph *graph);
+
 /* ── measurement ─────────────────────────────────────────────────────────── */
 
 /* HIP events recorded on the context stream: start, then stop returns the

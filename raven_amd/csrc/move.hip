@@ -194,15 +194,7 @@ NXH_EXPORT int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
   }
   NXH_HIP(op, hipGetLastError());
   // Data faults surface from this call (nx_c_move.c:448-458): read the flag back.
-  NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag_host, ctx->fault_flag, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
-  NXH_HIP(op, hipStreamSynchronize(ctx->stream));
-  if (*ctx->fault_flag_host != 0) {
-    *ctx->fault_flag_host = 0;
-    NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag, ctx->fault_flag_host, sizeof(int), hipMemcpyHostToDevice, ctx->stream));
-    NXH_HIP(op, hipStreamSynchronize(ctx->stream));
-    return nxh_fail(NXH_FAILURE, op, NXH_ERR_INDEX_OOB);
-  }
-  return NXH_OK;
+  return nxh_collect_index_fault(ctx, op);
 }
 
 // ── scatter ─────────────────────────────────────────────────────────────────
@@ -433,20 +425,6 @@ static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add, int
   else hipLaunchKernelGGL((scatter_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, a);
 }
 
-// Reads the out-of-bounds flag back after the launch: the failure is reported by
-// the call that caused it (nx_c_move.c:448-458, 571-586).
-static int collect_index_fault(nxh_context *ctx, const char *op) {
-  NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag_host, ctx->fault_flag, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
-  NXH_HIP(op, hipStreamSynchronize(ctx->stream));
-  if (*ctx->fault_flag_host != 0) {
-    *ctx->fault_flag_host = 0;
-    NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag, ctx->fault_flag_host, sizeof(int), hipMemcpyHostToDevice, ctx->stream));
-    NXH_HIP(op, hipStreamSynchronize(ctx->stream));
-    return nxh_fail(NXH_FAILURE, op, NXH_ERR_INDEX_OOB);
-  }
-  return NXH_OK;
-}
-
 NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *indices,
                            const nxh_tensor *updates, int axis, int mode) {
   const char *op = "scatter";
@@ -522,7 +500,7 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
   nxh_set_path(range_rows > 0 ? "scatter_rows" : "scatter_columns");
   table[dt](ctx, a, mode == 1, range_rows);
   NXH_HIP(op, hipGetLastError());
-  return collect_index_fault(ctx, op);
+  return nxh_collect_index_fault(ctx, op);
 }
 
 // ── threefry2x32-20 ─────────────────────────────────────────────────────────

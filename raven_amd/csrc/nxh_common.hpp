@@ -48,6 +48,20 @@ struct nxh_context {
   hipEvent_t stage_done[STAGE_SLOTS] = {};
   bool stage_used[STAGE_SLOTS] = {};
   int stage_next = 0;
+  // stream capture: while `capture` is set, launches are recorded into its graph
+  // and allocations come from (and go back to) the graph's own blocks
+  struct nxh_graph *capture = nullptr;
+  std::map<void *, struct nxh_graph *> graph_blocks;  // block -> the graph that holds it
+  int deferred_faults = 0;  // live graphs whose gathers / scatters report at the next synchronize
+};
+
+// A captured sequence of launches (runtime.hip).
+struct nxh_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::map<size_t, std::vector<void *>> free_lists;  // its blocks not in use by a tensor
+  std::vector<void *> pinned;                        // host staging of captured uploads
+  bool has_index_checks = false;
 };
 
 // thread-local status text (static strings + op prefix)
@@ -65,6 +79,8 @@ int nxh_hip_fail(const char *op, hipError_t e);
 // allocator (runtime.hip)
 int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out);
 void nxh_free_locked(nxh_context *ctx, void *p);
+// the out-of-bounds flag of gather / scatter, read back (or left for the replay) (runtime.hip)
+int nxh_collect_index_fault(nxh_context *ctx, const char *op);
 
 // status strings shared with the reference (nx_c.h:381-388, nx_c_engine.h:38-50)
 #define NXH_ERR_NDIM "ndim exceeds NX_C_MAX_NDIM"

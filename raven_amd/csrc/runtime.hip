@@ -80,6 +80,12 @@ NXH_EXPORT int nxh_context_create(nxh_context **out) {
 NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   if (!ctx) return;
   (void)hipSetDevice(ctx->device);
+  if (ctx->capture) {  // abandoned capture: close it so the stream can be destroyed
+    hipGraph_t dropped = nullptr;
+    (void)hipStreamEndCapture(ctx->stream, &dropped);
+    if (dropped) (void)hipGraphDestroy(dropped);
+    (void)hipGetLastError();
+  }
   (void)hipStreamSynchronize(ctx->stream);
   for (auto &kv : ctx->live) (void)hipFree(kv.first);
   if (ctx->fault_flag) (void)hipFree(ctx->fault_flag);
@@ -114,6 +120,11 @@ NXH_EXPORT int64_t nxh_dtype_bytes(int dtype, int64_t count) {
 // thousand per GPT-2 forward), so hipMalloc/hipFree never sit on that path once
 // the working set has been seen. Every block is 256-byte aligned, exact-size
 // from the caller's point of view, and never a sub-range of another block.
+static int refuse_while_capturing(nxh_context *ctx, const char *op) {
+  if (ctx->capture) return nxh_fail(NXH_FAILURE, op, "not allowed while a graph is being captured");
+  return NXH_OK;
+}
+
 static size_t size_class(size_t bytes) {
   if (bytes == 0) bytes = 1;
   if (bytes <= ((size_t)1 << 20)) return (bytes + 511) & ~(size_t)511;
@@ -124,17 +135,28 @@ static size_t size_class(size_t bytes) {
 
 int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out) {
   size_t cls = size_class(bytes);
+  nxh_graph *cap = ctx->capture;
+  if (cap) {  // a block the graph already holds, before anything else
+    auto git = cap->free_lists.find(cls);
+    if (git != cap->free_lists.end() && !git->second.empty()) {
+      *out = git->second.back();
+      git->second.pop_back();
+      ctx->in_use += cls;
+      return NXH_OK;
+    }
+  }
   auto it = ctx->free_lists.find(cls);
   if (it != ctx->free_lists.end() && !it->second.empty()) {
     *out = it->second.back();
     it->second.pop_back();
     ctx->cached -= cls;
     ctx->in_use += cls;
+    if (cap) ctx->graph_blocks[*out] = cap;  // from now on the graph's
     return NXH_OK;
   }
   void *p = nullptr;
   hipError_t e = hipMalloc(&p, cls);
-  if (e != hipSuccess) {
+  if (e != hipSuccess && !cap) {
     // give cached blocks back to the driver and retry once
     (void)hipGetLastError();
     (void)hipStreamSynchronize(ctx->stream);
@@ -148,15 +170,16 @@ int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out) {
       kv.second.clear();
     }
     e = hipMalloc(&p, cls);
-    if (e != hipSuccess) {
-      (void)hipGetLastError();
-      return nxh_fail(NXH_FAILURE, "buffer", NXH_ERR_ALLOC);
-    }
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return nxh_fail(NXH_FAILURE, "buffer", NXH_ERR_ALLOC);
   }
   ctx->live[p] = cls;
   ctx->reserved += cls;
   ctx->in_use += cls;
   ctx->driver_allocs++;
+  if (cap) ctx->graph_blocks[p] = cap;
   *out = p;
   return NXH_OK;
 }
@@ -164,8 +187,15 @@ int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out) {
 void nxh_free_locked(nxh_context *ctx, void *p) {
   auto it = ctx->live.find(p);
   if (it == ctx->live.end()) return;
-  ctx->free_lists[it->second].push_back(p);
   ctx->in_use -= it->second;
+  // a block a graph holds stays with that graph (its replays write there): it is
+  // reused only by later allocations of the same capture
+  auto g = ctx->graph_blocks.find(p);
+  if (g != ctx->graph_blocks.end()) {
+    g->second->free_lists[it->second].push_back(p);
+    return;
+  }
+  ctx->free_lists[it->second].push_back(p);
   ctx->cached += it->second;
 }
 
@@ -189,6 +219,7 @@ NXH_EXPORT int nxh_free(nxh_context *ctx, void *dptr) {
 NXH_EXPORT int nxh_trim(nxh_context *ctx) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "trim", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "trim")) return rc;
   NXH_HIP("trim", hipSetDevice(ctx->device));
   NXH_HIP("trim", hipStreamSynchronize(ctx->stream));
   for (auto &kv : ctx->free_lists) {
@@ -225,6 +256,17 @@ NXH_EXPORT int nxh_memcpy_h2d(nxh_context *ctx, void *dst, const void *src, size
   if (bytes == 0) return NXH_OK;
   std::lock_guard<std::mutex> g(ctx->mu);
   NXH_HIP("from_host", hipSetDevice(ctx->device));
+  if (ctx->capture) {
+    // recorded as a copy from pinned memory the graph keeps: every replay uploads these bytes again
+    if (bytes > nxh_context::STAGE_BYTES)
+      return nxh_fail(NXH_FAILURE, "from_host", "uploads over 256 KiB are not recorded into a graph");
+    void *pin = nullptr;
+    NXH_HIP("from_host", hipHostMalloc(&pin, bytes, hipHostMallocDefault));
+    ctx->capture->pinned.push_back(pin);
+    memcpy(pin, src, bytes);
+    NXH_HIP("from_host", hipMemcpyAsync(dst, pin, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return NXH_OK;
+  }
   if (bytes <= nxh_context::STAGE_BYTES) {
     // small upload: through a pinned slot, in stream order, without waiting
     // for the stream. A slot is reused only after its last transfer finished.
@@ -243,9 +285,37 @@ NXH_EXPORT int nxh_memcpy_h2d(nxh_context *ctx, void *dst, const void *src, size
   return NXH_OK;
 }
 
+// Reads the out-of-bounds flag back after a gather or scatter launch: the failure
+// is reported by the call that caused it (nx_c_move.c:448-458, 571-586). A stream
+// that is being recorded cannot be waited for: there the flag stays on the device
+// and the next synchronize after a replay reports it.
+static int read_fault_flag(nxh_context *ctx, const char *op, const char *message) {
+  NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag_host, ctx->fault_flag, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+  NXH_HIP(op, hipStreamSynchronize(ctx->stream));
+  if (*ctx->fault_flag_host == 0) return NXH_OK;
+  *ctx->fault_flag_host = 0;
+  NXH_HIP(op, hipMemcpyAsync(ctx->fault_flag, ctx->fault_flag_host, sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+  NXH_HIP(op, hipStreamSynchronize(ctx->stream));
+  return nxh_fail(NXH_FAILURE, op, message);
+}
+
+int nxh_collect_index_fault(nxh_context *ctx, const char *op) {
+  if (ctx->capture) {
+    ctx->capture->has_index_checks = true;
+    return NXH_OK;
+  }
+  return read_fault_flag(ctx, op, NXH_ERR_INDEX_OOB);
+}
+
+static int report_deferred_faults(nxh_context *ctx, const char *op) {
+  if (!ctx->deferred_faults) return NXH_OK;
+  return read_fault_flag(ctx, op, "index out of bounds in a replayed gather or scatter");
+}
+
 NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "to_host", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "to_host")) return rc;
   NXH_HIP("to_host", hipSetDevice(ctx->device));
   if (bytes)
     NXH_HIP("to_host", hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
@@ -256,21 +326,106 @@ NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size
 NXH_EXPORT int nxh_synchronize(nxh_context *ctx) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "synchronize", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "synchronize")) return rc;
   NXH_HIP("synchronize", hipSetDevice(ctx->device));
   NXH_HIP("synchronize", hipStreamSynchronize(ctx->stream));
+  return report_deferred_faults(ctx, "synchronize");
+}
+
+// ── graphs ─────────────────────────────────────────────────────────────────
+// Everything launched between capture_begin and capture_end is recorded instead
+// of run. Blocks allocated in between belong to the graph until it is destroyed
+// (its replays write there), including those whose tensors die during the
+// capture: these are recycled inside the capture exactly as the eager allocator
+// would recycle them, so a replay walks the same addresses in the same order.
+// Callers hold ctx->mu and have drained the stream.
+static void graph_release(nxh_context *ctx, nxh_graph *gr) {
+  if (gr->exec && gr->has_index_checks) ctx->deferred_faults--;
+  if (gr->exec) (void)hipGraphExecDestroy(gr->exec);
+  if (gr->graph) (void)hipGraphDestroy(gr->graph);
+  for (void *p : gr->pinned) (void)hipHostFree(p);
+  // its idle blocks go back to the context's free lists; blocks still inside a
+  // tensor become ordinary blocks
+  for (auto &kv : gr->free_lists)
+    for (void *p : kv.second) {
+      ctx->free_lists[kv.first].push_back(p);
+      ctx->cached += kv.first;
+    }
+  for (auto it = ctx->graph_blocks.begin(); it != ctx->graph_blocks.end();)
+    it = it->second == gr ? ctx->graph_blocks.erase(it) : std::next(it);
+  delete gr;
+}
+
+NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
+  if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "capture_begin", "null context");
+  std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "capture_begin")) return rc;
+  NXH_HIP("capture_begin", hipSetDevice(ctx->device));
+  NXH_HIP("capture_begin", hipStreamSynchronize(ctx->stream));
+  nxh_graph *gr = new nxh_graph();
+  hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) {
+    delete gr;
+    return nxh_hip_fail("capture_begin", e);
+  }
+  ctx->capture = gr;
   return NXH_OK;
+}
+
+NXH_EXPORT int nxh_capture_end(nxh_context *ctx, nxh_graph **out) {
+  if (!ctx || !out) return nxh_fail(NXH_INVALID_ARGUMENT, "capture_end", "null argument");
+  std::lock_guard<std::mutex> g(ctx->mu);
+  *out = nullptr;
+  nxh_graph *gr = ctx->capture;
+  if (!gr) return nxh_fail(NXH_FAILURE, "capture_end", "no capture in progress");
+  ctx->capture = nullptr;
+  hipError_t e = hipStreamEndCapture(ctx->stream, &gr->graph);
+  if (e == hipSuccess) e = hipGraphInstantiate(&gr->exec, gr->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(ctx->stream);
+    graph_release(ctx, gr);
+    return nxh_hip_fail("capture_end", e);
+  }
+  if (gr->has_index_checks) ctx->deferred_faults++;
+  *out = gr;
+  return NXH_OK;
+}
+
+NXH_EXPORT int nxh_graph_launch(nxh_context *ctx, nxh_graph *gr) {
+  if (!ctx || !gr || !gr->exec) return nxh_fail(NXH_INVALID_ARGUMENT, "graph_launch", "null argument");
+  std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "graph_launch")) return rc;
+  NXH_HIP("graph_launch", hipSetDevice(ctx->device));
+  NXH_HIP("graph_launch", hipGraphLaunch(gr->exec, ctx->stream));
+  return NXH_OK;
+}
+
+NXH_EXPORT int nxh_graph_destroy(nxh_context *ctx, nxh_graph *gr) {
+  if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "graph_destroy", "null context");
+  if (!gr) return NXH_OK;
+  std::lock_guard<std::mutex> g(ctx->mu);
+  if (ctx->capture == gr) return nxh_fail(NXH_FAILURE, "graph_destroy", "this graph is still being captured");
+  (void)hipSetDevice(ctx->device);
+  (void)hipStreamSynchronize(ctx->stream);
+  // a fault of its last replays is not lost with it
+  const int rc = gr->exec && gr->has_index_checks ? report_deferred_faults(ctx, "graph_destroy") : NXH_OK;
+  graph_release(ctx, gr);
+  return rc;
 }
 
 // ── timing ─────────────────────────────────────────────────────────────────
 NXH_EXPORT int nxh_timer_start(nxh_context *ctx) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "timer", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "timer")) return rc;
   NXH_HIP("timer", hipEventRecord(ctx->ev_start, ctx->stream));
   return NXH_OK;
 }
 NXH_EXPORT int nxh_timer_stop(nxh_context *ctx, float *ms) {
   if (!ctx || !ms) return nxh_fail(NXH_INVALID_ARGUMENT, "timer", "null argument");
   std::lock_guard<std::mutex> g(ctx->mu);
+  if (int rc = refuse_while_capturing(ctx, "timer")) return rc;
   NXH_HIP("timer", hipEventRecord(ctx->ev_stop, ctx->stream));
   NXH_HIP("timer", hipEventSynchronize(ctx->ev_stop));
   NXH_HIP("timer", hipEventElapsedTime(ms, ctx->ev_start, ctx->ev_stop));

@@ -101,6 +101,25 @@ def encode_scalar(dtype: dt.DType, value) -> np.ndarray:
         return np.asarray(value).astype(dtype.np_storage).reshape(1)
 
 
+class Graph:
+    """Launches recorded between Backend.capture_begin and capture_end. Tensors
+    created in between keep their storage: `launch` recomputes them in place
+    from what the older tensors they were computed from hold at that time."""
+
+    def __init__(self, backend, handle):
+        self._backend, self._h = backend, handle
+
+    def launch(self):
+        b = self._backend
+        b._check(b._lib.nxh_graph_launch(b._h, self._h))
+
+    def destroy(self):
+        if self._h:
+            b = self._backend
+            b._check(b._lib.nxh_graph_destroy(b._h, self._h))
+            self._h = None
+
+
 class Backend:
     """An execution context (``create_context``, nx_backend.mli:32-39) plus the
     operations of ``Backend_intf.S``."""
@@ -139,6 +158,17 @@ class Backend:
 
     def last_path(self) -> str:
         return self._lib.nxh_last_path(self._h).decode()
+
+    # -- recorded sequences: no counterpart in Backend_intf.S, whose calls run as they are made --
+    def capture_begin(self):
+        """From here to capture_end every call records its launches instead of
+        running them; to_host / synchronize raise until then."""
+        self._check(self._lib.nxh_capture_begin(self._h))
+
+    def capture_end(self) -> "Graph":
+        g = C.c_void_p()
+        self._check(self._lib.nxh_capture_end(self._h, C.byref(g)))
+        return Graph(self, g)
 
     def memory_stats(self):
         v = [C.c_uint64() for _ in range(4)]

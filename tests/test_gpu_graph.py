@@ -1,0 +1,156 @@
+"""Recorded sequences (nxh_capture_begin / nxh_capture_end / nxh_graph_launch):
+a replay must give what the same calls give eagerly, bit for bit, on every
+replay, with other work of the same context between the replays, and after its
+inputs were rewritten in place."""
+
+import numpy as np
+import pytest
+
+from helpers import decode, encode, logical, same_bits
+from raven_amd import dtype as dt
+
+pytestmark = pytest.mark.gpu
+
+
+class capture:
+    """Closes the capture even when the recorded calls raise, so that a failing
+    test leaves the shared context usable."""
+
+    def __init__(self, backend):
+        self.B, self.graph = backend, None
+
+    def __enter__(self):
+        self.B.capture_begin()
+        return self
+
+    def __exit__(self, *exc):
+        self.graph = self.B.capture_end()
+        return False
+
+
+def chain(B, a, b, idx):
+    """Map, strided view, reduction with a scratch buffer, scan, sort, GEMM and a
+    gather: one launch of most kernel families, with temporaries that die."""
+    c = B.binary("add", a, b)
+    d = B.binary("mul", c, B.permute(c, (1, 0)))
+    s = B.reduce("sum", [0], d)
+    m = B.matmul(d, c)
+    k = B.associative_scan(1, "max", m)
+    o = B.sort(B.binary("sub", k, B.expand(B.reshape(s, (1, 192)), (192, 192))), 1, True)
+    return B.gather(o, idx, 0)
+
+
+def inputs(seed):
+    rng = np.random.default_rng(seed)
+    a = (rng.integers(-8, 8, (192, 192)) / 4).astype(np.float32)  # quarter-integers: sums are exact in any order
+    b = (rng.integers(-8, 8, (192, 192)) / 4).astype(np.float32)
+    idx = rng.integers(0, 192, (64, 192)).astype(np.int32)
+    return a, b, idx
+
+
+def test_replays_match_eager_results_between_other_work(hip, oracle):
+    a0, b0, i0 = inputs(1)
+    ta, tb = (hip.reshape(hip.from_host(x, dt.float32), x.shape) for x in (a0, b0))
+    ti = hip.reshape(hip.from_host(i0, dt.int32), i0.shape)
+    chain(hip, ta, tb, ti)  # warm every entry point once
+    before = hip.memory_stats()["in_use"]
+    with capture(hip) as cap:
+        out = chain(hip, ta, tb, ti)
+    g = cap.graph
+    try:
+        for seed in (1, 2, 3, 4):
+            a, b, i = inputs(seed)
+            # rewrite the inputs in place, then run unrelated eager work that allocates and frees
+            for t, x, d in ((ta, a, dt.float32), (tb, b, dt.float32), (ti, i, dt.int32)):
+                hip.assign(t, hip.reshape(hip.from_host(x, d), x.shape))
+            junk = hip.binary("mul", hip.full(dt.float32, (257, 129), 3.0), hip.full(dt.float32, (257, 129), 2.0))
+            assert float(logical(hip.reduce("max", [0, 1], junk))) == 6.0
+            g.launch()
+            eager = chain(hip, ta, tb, ti)
+            oa, ob = (oracle.reshape(oracle.from_host(x, dt.float32), x.shape) for x in (a, b))
+            want = chain(oracle, oa, ob, oracle.reshape(oracle.from_host(i, dt.int32), i.shape))
+            same_bits(logical(out), logical(eager), f"replay {seed} against eager")
+            same_bits(logical(out), logical(want), f"replay {seed} against the oracle")
+    finally:
+        g.destroy()
+    del out, eager, junk
+    assert hip.memory_stats()["in_use"] == before
+
+
+def test_uploads_are_replayed_and_host_reads_are_refused(hip):
+    x = hip.from_host(np.arange(1000, dtype=np.int32), dt.int32)
+    with capture(hip) as cap:
+        y = hip.from_host(np.full(1000, 5, np.int32), dt.int32)  # recorded with its own copy of the bytes
+        z = hip.binary("add", x, y)
+        with pytest.raises(RuntimeError, match="while a graph is being captured"):
+            hip.to_host(z)
+        with pytest.raises(RuntimeError, match="while a graph is being captured"):
+            hip.synchronize()
+        with pytest.raises(RuntimeError, match="256 KiB"):
+            hip.from_host(np.zeros(1 << 20, np.uint8), dt.uint8)
+    g = cap.graph
+    try:
+        for k in range(3):
+            hip.assign(x, hip.from_host(np.arange(1000, dtype=np.int32) * k, dt.int32))
+            hip.assign(y, hip.from_host(np.zeros(1000, np.int32), dt.int32))  # the replay uploads the fives again
+            g.launch()
+            same_bits(logical(z), np.arange(1000, dtype=np.int32) * k + 5, f"replay {k}")
+    finally:
+        g.destroy()
+    with pytest.raises(RuntimeError, match="no capture in progress"):
+        hip.capture_end()
+
+
+def test_index_fault_of_a_replay_surfaces_at_synchronize(hip):
+    data = hip.reshape(hip.from_host(np.arange(64, dtype=np.float32), dt.float32), (8, 8))
+    idx = hip.reshape(hip.from_host(np.zeros(8, np.int32), dt.int32), (1, 8))
+    hip.gather(data, idx, 0)
+    with capture(hip) as cap:
+        out = hip.gather(data, idx, 0)
+    g = cap.graph
+    try:
+        g.launch()
+        hip.synchronize()
+        same_bits(logical(out), np.arange(8, dtype=np.float32).reshape(1, 8))
+        hip.assign(idx, hip.reshape(hip.from_host(np.full(8, 8, np.int32), dt.int32), (1, 8)))
+        g.launch()
+        with pytest.raises(RuntimeError, match="index out of bounds"):
+            hip.synchronize()
+        hip.synchronize()  # reported once
+        hip.assign(idx, hip.reshape(hip.from_host(np.full(8, 7, np.int32), dt.int32), (1, 8)))
+        g.launch()
+        same_bits(logical(out), np.arange(56, 64, dtype=np.float32).reshape(1, 8))
+    finally:
+        g.destroy()
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16], ids=lambda d: d.name)
+def test_captured_gpt2_forward_replays_the_windowed_forward(hip, oracle, d):
+    """The whole windowed forward as one graph: new token ids are written into
+    the captured input tensor and each replay equals the eager windowed result."""
+    from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
+    from raven_amd.nx_frontend import Nx
+    from raven_amd.nx_window import Window
+
+    cfg = Config(vocab_size=1031, n_positions=128, n_embd=256, n_layer=2, n_head=4, n_inner=1024)
+    hp = host_params(cfg, seed=16, stddev=0.05)
+    win = Window(hip)
+    nx = Nx(win)
+    params = upload(nx, hp, d, lambda a, dd: encode(a, dd, oracle))
+    model = Gpt2(nx, cfg)
+    ids = [np.random.default_rng(40 + k).integers(0, cfg.vocab_size, (2, 96)).astype(np.int32) for k in range(3)]
+    t_ids = nx.create(dt.int32, ids[0].shape, ids[0])
+    eager = [logical(win.force(model.logits(params, nx.create(dt.int32, i.shape, i)))) for i in ids]
+    with capture(win) as cap:
+        out = win.force(model.logits(params, t_ids))
+    g = cap.graph
+    try:
+        for k in (0, 1, 2, 1):
+            hip.assign(win.force(t_ids), hip.reshape(hip.from_host(ids[k], dt.int32), ids[k].shape))
+            g.launch()
+            same_bits(logical(out), eager[k], f"replay with ids {k}")
+            # eager work of the same context between replays
+            assert logical(win.force(model.logits(params, nx.create(dt.int32, ids[k].shape, ids[k])))).shape == eager[k].shape
+    finally:
+        g.destroy()
+    assert np.all(np.isfinite(decode(eager[0], d, oracle)))
