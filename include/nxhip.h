@@ -308,6 +308,31 @@ int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q,
 int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
                const nxh_tensor *w, const nxh_tensor *bias, const nxh_tensor *residual);
 
+/* ── Fourier transforms ──────────────────────────────────────────────────── */
+
+/* fft / ifft (backend_intf.ml:594-598; nx_backend.ml:507-528; nx_c_fft.c:940-956,
+   1173-1182): complex64 / complex128, out has x's shape and dtype. UNNORMALISED
+   (nx_c_fft.c:30-32): fft is the -sign DFT, ifft the +sign DFT without 1/n.
+   One 1-D pass per entry of `axes`, in that order, the first reading x, the
+   later ones transforming out in place; arithmetic in double, one rounding per
+   pass on store. Any length up to 2^26 (2^25 when it is not a power of two). */
+int nxh_fft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+            const int32_t *axes, int n_axes, int inverse);
+/* rfft (backend_intf.ml:600-608; nx_backend.ml:530-536; nx_c_fft.c:958-982):
+   x f32 / f64, out complex64 / complex128 with n/2+1 bins along the LAST listed
+   axis, which is transformed first (from the real lines); the other listed axes
+   follow as complex passes on out. */
+int nxh_rfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+             const int32_t *axes, int n_axes);
+/* irfft (backend_intf.ml:610-623; nx_backend.ml:538-548; nx_c_fft.c:997-1144):
+   x complex, out f32 / f64 of length s along the last listed axis, s = s_last
+   when positive, else 2 (bins - 1). The other listed axes are transformed first
+   (+sign, in complex128); then each line's spectrum of length s is rebuilt from
+   min(bins, s/2+1) bins by conjugate symmetry (missing bins are zero) and the
+   real part of its +sign transform is stored. */
+int nxh_irfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+              const int32_t *axes, int n_axes, int64_t s_last);
+
 /* ── recorded sequences ──────────────────────────────────────────────────── */
 
 /* The reference backend has no counterpart: its eager calls cost a C stub

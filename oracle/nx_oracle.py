@@ -312,6 +312,54 @@ class OracleBackend:
         _check(lib().nxo_fold(out.desc(), x.desc(), len(kernel_size), osz, *params), "fold")
         return out
 
+    # Fourier transforms ------------------------------------------------------
+    # nx_c_fft.c computes every 1-D pass in double precision from the DFT's
+    # definition (unnormalised; -sign forward, +sign inverse) and rounds to the
+    # output dtype once per pass (nx_c_fft.c:30-32, 869-894). numpy's transform is
+    # double precision too; its 1/n on the inverse is multiplied back out.
+    def _from_array(self, a: np.ndarray, d: dt.DType):
+        return self.reshape(self.from_host(np.ascontiguousarray(a.astype(d.np_storage)), d), a.shape)
+
+    def fft(self, x, axes, inverse: bool = False):
+        cur = logical(x)
+        for ax in axes:  # nx_c_fft.c:940-956: one pass per listed axis, rounded to the dtype in between
+            wide = cur.astype(np.complex128)
+            y = np.fft.ifft(wide, axis=ax) * wide.shape[ax] if inverse else np.fft.fft(wide, axis=ax)
+            cur = y.astype(x.dtype.np_storage)
+        return self._from_array(cur, x.dtype)
+
+    def ifft(self, x, axes):
+        return self.fft(x, axes, inverse=True)
+
+    def rfft(self, x, dtype, axes):
+        axes = [int(a) for a in axes]
+        last = axes[-1]
+        a = logical(x).astype(np.float64)
+        n = a.shape[last]
+        full = np.fft.fft(a.astype(np.complex128), axis=last)  # nx_c_fft.c:968-972: full transform, keep n/2+1 bins
+        cur = np.take(full, range(n // 2 + 1), axis=last).astype(dtype.np_storage)
+        for ax in axes[:-1]:
+            cur = np.fft.fft(cur.astype(np.complex128), axis=ax).astype(dtype.np_storage)
+        return self._from_array(cur, dtype)
+
+    def irfft(self, x, dtype, axes, s=None):
+        axes = [int(a) for a in axes]
+        last = axes[-1]
+        tmp = logical(x).astype(np.complex128)
+        for ax in axes[:-1]:  # nx_c_fft.c:1101-1114, complex128 throughout
+            tmp = np.fft.ifft(tmp, axis=ax) * tmp.shape[ax]
+        in_half = tmp.shape[last]
+        size = int(s[len(axes) - 1]) if s is not None else 2 * (in_half - 1)
+        half = min(in_half, size // 2 + 1)
+        g = np.moveaxis(tmp, last, -1)
+        f = np.zeros(g.shape[:-1] + (size,), np.complex128)
+        f[..., :half] = g[..., :half]
+        for k in range(1, half):  # nx_c_fft.c:1013-1023
+            if size - k != k:
+                f[..., size - k] = np.conj(g[..., k])
+        y = (np.fft.ifft(f, axis=-1) * size).real if size else np.zeros(f.shape)
+        return self._from_array(np.moveaxis(y, -1, last), dtype)
+
 
 def window_shapes(in_shape, kernel_size, stride, dilation, padding):
     """Result shape of unfold (nx_backend.ml:427-445) and the K-long parameter

@@ -94,6 +94,9 @@ SIGNATURES = {
     "nxh_argsort": (C.c_int, [_CTX, _T, _T, C.c_int, C.c_int]),
     "nxh_unfold": (C.c_int, [_CTX, _T, _T, C.c_int] + [_P(C.c_int64)] * 4),
     "nxh_fold": (C.c_int, [_CTX, _T, _T, C.c_int] + [_P(C.c_int64)] * 5),
+    "nxh_fft": (C.c_int, [_CTX, _T, _T, _P(C.c_int32), C.c_int, C.c_int]),
+    "nxh_rfft": (C.c_int, [_CTX, _T, _T, _P(C.c_int32), C.c_int]),
+    "nxh_irfft": (C.c_int, [_CTX, _T, _T, _P(C.c_int32), C.c_int, C.c_int64]),
     "nxh_softmax_rows": (C.c_int, [_CTX, _T, _T, C.c_void_p, _T, C.c_void_p]),
     "nxh_layer_norm_rows": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_double]),
     "nxh_gelu_tanh": (C.c_int, [_CTX, _T, _T, C.c_void_p]),

@@ -52,6 +52,8 @@ struct nxh_context {
   // and allocations come from (and go back to) the graph's own blocks
   struct nxh_graph *capture = nullptr;
   std::map<void *, struct nxh_graph *> graph_blocks;  // block -> the graph that holds it
+  // twiddle and chirp tables of the transforms, by (kind, sign, length); freed with the context
+  std::map<uint64_t, void *> device_tables;
   int deferred_faults = 0;  // live graphs whose gathers / scatters report at the next synchronize
 };
 

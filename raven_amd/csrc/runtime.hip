@@ -88,6 +88,7 @@ NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   }
   (void)hipStreamSynchronize(ctx->stream);
   for (auto &kv : ctx->live) (void)hipFree(kv.first);
+  for (auto &kv : ctx->device_tables) (void)hipFree(kv.second);
   if (ctx->fault_flag) (void)hipFree(ctx->fault_flag);
   if (ctx->fault_flag_host) (void)hipHostFree(ctx->fault_flag_host);
   if (ctx->stage) (void)hipHostFree(ctx->stage);

@@ -397,6 +397,45 @@ class Backend:
         self._check(self._lib.nxh_fold(self._h, C.byref(o), C.byref(a), len(kernel_size), osz, *params))
         return out
 
+    # ── Fourier transforms (nx_backend.ml:502-548): unnormalised, the frontend owns 1/n ──
+    @staticmethod
+    def _axes_arg(axes):
+        axes = [int(a) for a in axes]
+        return (C.c_int32 * max(len(axes), 1))(*axes), len(axes)
+
+    def fft(self, x: Tensor, axes, inverse: bool = False) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        ax, n = self._axes_arg(axes)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_fft(self._h, C.byref(o), C.byref(a), ax, n, int(inverse)))
+        return out
+
+    def ifft(self, x: Tensor, axes) -> Tensor:
+        return self.fft(x, axes, inverse=True)
+
+    def rfft(self, x: Tensor, dtype: dt.DType, axes) -> Tensor:
+        ax, n = self._axes_arg(axes)
+        if n < 1 or not 0 <= ax[n - 1] < len(x.shape):
+            raise ValueError("rfft: axis out of range")
+        shape = list(x.shape)
+        shape[ax[n - 1]] = shape[ax[n - 1]] // 2 + 1
+        out = self.buffer(dtype, shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_rfft(self._h, C.byref(o), C.byref(a), ax, n))
+        return out
+
+    def irfft(self, x: Tensor, dtype: dt.DType, axes, s=None) -> Tensor:
+        ax, n = self._axes_arg(axes)
+        if n < 1 or not 0 <= ax[n - 1] < len(x.shape):
+            raise ValueError("irfft: axis out of range")
+        size = int(s[n - 1]) if s is not None else (x.shape[ax[n - 1]] - 1) * 2
+        shape = list(x.shape)
+        shape[ax[n - 1]] = size
+        out = self.buffer(dtype, shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_irfft(self._h, C.byref(o), C.byref(a), ax, n, size if s is not None else 0))
+        return out
+
     # ── fused sequences of primitives (no counterpart in Backend_intf.S) ────
     def _scalar_arg(self, dtype: dt.DType, value):
         if value is None:

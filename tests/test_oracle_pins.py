@@ -794,3 +794,72 @@ def test_window_reference_vectors_and_brute_force():
                 for j in range(ow):
                     acc[:, :, i * st[0] + a * dl[0], j * st[1] + b * dl[1]] += y[:, :, a * ks[1] + b, i * ow + j]
     assert np.array_equal(f, acc[:, :, pd[0][0]:pd[0][0] + 7, pd[1][0]:pd[1][0] + 9].astype(np.int32))
+
+
+def _dft(a, inverse=False):
+    """The O(n^2) transform straight from the definition, as backend_contract.ml:2831-2844 states it."""
+    n = len(a)
+    k = np.arange(n)
+    ang = (1.0 if inverse else -1.0) * 2.0 * np.pi * ((k[:, None] * k[None, :]) % n) / n
+    return (np.cos(ang) + 1j * np.sin(ang)) @ np.asarray(a, np.complex128)
+
+
+def test_fft_reference_cases_and_the_definition():
+    B = OracleBackend()
+    F = GOLD["fft"]
+    cdata = lambda n: np.array([((i % 5) - 2) + 1j * ((i % 3) - 1) for i in range(n)], np.complex128)
+    tol = F["tolerance"]["complex128"]
+    near = lambda got, want, t=tol: np.all(np.abs(np.asarray(got) - np.asarray(want)) <= t * (1 + np.abs(want)))
+    for n in F["dft_lengths"]:  # powers of two, radix 7, mixed radix, odd prime products, a Bluestein prime
+        x = cdata(n)
+        assert near(logical(B.fft(_mk(B, x, dt.complex128), [0])), _dft(x)), n
+        assert near(logical(B.ifft(_mk(B, x, dt.complex128), [0])), _dft(x, inverse=True)), n
+        assert near(logical(B.ifft(B.fft(_mk(B, x, dt.complex128), [0]), [0])), n * x), n
+    n = F["complex64_length"]
+    got = logical(B.fft(_mk(B, cdata(n).astype(np.complex64), dt.complex64), [0]))
+    assert got.dtype == np.complex64 and near(got, _dft(cdata(n)), F["tolerance"]["complex64"])
+    # a strided axis: the signal interleaved with filler, then sliced out (backend_contract.ml:2877-2887)
+    n = F["strided"]["n"]
+    inter = np.empty((n, 2), np.complex128)
+    inter[:, 0] = complex(*F["strided"]["filler"])
+    inter[:, 1] = cdata(n)
+    view = B.shrink(_mk(B, inter, dt.complex128), [(0, n), (1, 2)])
+    assert near(logical(B.fft(view, [0]))[:, 0], _dft(cdata(n)))
+    rt = F["roundtrip_2d"]
+    x = cdata(12).reshape(rt["shape"])
+    assert near(logical(B.ifft(B.fft(_mk(B, x, dt.complex128), [0, 1]), [0, 1])), rt["scale"] * x)
+    # two axes are the two 1-D definitions composed, first listed axis first
+    got = logical(B.fft(_mk(B, x, dt.complex128), [0, 1]))
+    want = np.array([_dft(r) for r in np.array([_dft(c) for c in x.T]).T])
+    assert near(got, want)
+    for key in ("rfft_even", "rfft_odd"):
+        x = np.array(F[key]["x"])
+        n = F[key]["n"]
+        spec = B.rfft(_mk(B, x, dt.float64), dt.complex128, [0])
+        assert logical(spec).shape == (n // 2 + 1,) and near(logical(spec), _dft(x)[:n // 2 + 1])
+        assert near(logical(B.irfft(spec, dt.float64, [0], [n])), n * x), key
+    c = F["irfft_truncates"]
+    ones = _mk(B, np.ones(c["bins"], np.complex128), dt.complex128)
+    assert near(logical(B.irfft(ones, dt.float64, [0], [c["s"]])), np.array(c["out"], float))
+    c = F["irfft_pads"]
+    ones = _mk(B, np.ones(c["bins"], np.complex128), dt.complex128)
+    want = np.array([a + b * math.sqrt(2.0) for a, b in c["out_sqrt2_form"]])
+    assert near(logical(B.irfft(ones, dt.float64, [0], [c["s"]])), want)
+    # irfft = real part of the +sign definition on the conjugate-symmetric extension; bins' imaginary
+    # parts at 0 and at the Nyquist index contribute nothing
+    rng = np.random.default_rng(71)
+    for bins, s in ((5, 8), (5, 9), (4, 9), (7, 6)):
+        g = rng.standard_normal(bins) + 1j * rng.standard_normal(bins)
+        half = min(bins, s // 2 + 1)
+        full = np.zeros(s, np.complex128)
+        full[:half] = g[:half]
+        for k in range(1, half):
+            if s - k != k:
+                full[s - k] = np.conj(g[k])
+        assert near(logical(B.irfft(_mk(B, g, dt.complex128), dt.float64, [0], [s])), _dft(full, inverse=True).real)
+    k = F["known"]
+    assert near(logical(B.fft(_mk(B, np.ones(4, np.complex128), dt.complex128), [0])), np.array(k["ones4"], complex))
+    assert near(logical(B.fft(_mk(B, np.array([1, 0, 0, 0], np.complex128), dt.complex128), [0])), np.array(k["delta4"], complex))
+    x = cdata(F["parseval"]["n"])
+    e = lambda a: float(np.sum(np.abs(a) ** 2))
+    assert abs(e(logical(B.fft(_mk(B, x, dt.complex128), [0]))) - len(x) * e(x)) <= F["parseval"]["rel"] * len(x) * e(x)
