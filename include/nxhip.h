@@ -333,6 +333,44 @@ int nxh_rfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
 int nxh_irfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
               const int32_t *axes, int n_axes, int64_t s_last);
 
+/* ── linear algebra ──────────────────────────────────────────────────────── */
+
+/* The last two dims are the matrix, earlier dims the batch (backend_intf.ml:625-
+   638). Storage dtypes f16 / bf16 / f32 / f64 / fp8 / complex64 / complex128;
+   arithmetic in double. Numeric failures are Failure with the reference's status
+   text as the message's tail (nx_c_linalg.h:29-36; nx_backend.ml:573-591 lifts
+   them to Linalg_error by that suffix): "matrix is not positive definite",
+   "triangular matrix is singular", "eigenvalue iteration did not converge".
+   Every call waits for the stream (the failure belongs to the call). */
+
+/* cholesky (backend_intf.ml:640-646; nx_c_tri.c:303-400): reads the lower
+   triangle; out = L (upper == 0) or U = L^H, the other triangle zero. */
+int nxh_cholesky(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int upper);
+/* triangular_solve (backend_intf.ml:703-720; nx_c_tri.c:88-118, 459-562): b and
+   out are [..., n, nrhs] (a vector right-hand side is passed as one column,
+   nx_backend.ml:598-611). flags: bit 0 upper, bit 1 transpose (the conjugate
+   transpose for complex), bit 2 unit diagonal. An exactly zero pivot fails. */
+int nxh_triangular_solve(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *a,
+                         const nxh_tensor *b, int flags);
+/* qr (backend_intf.ml:648-653; nx_c_qr.c:24-80; nx_backend.ml:613-626): q is
+   [..., m, k] and r [..., k, n] when reduced (k = min(m, n)), else [..., m, m]
+   and [..., m, n]. LAPACK's reflector convention, so R's diagonal is real. */
+int nxh_qr(nxh_context *ctx, const nxh_tensor *q, const nxh_tensor *r, const nxh_tensor *x, int reduced);
+/* eigh / eigvalsh (backend_intf.ml:685-701; nx_c_eigh.c:14-21; nx_backend.ml:628-
+   649): reads the lower triangle; w [..., n] float64 ascending; v (may be null:
+   values only) [..., n, n] of x's dtype, column k the unit eigenvector of w[k].
+   n <= 4096. */
+int nxh_eigh(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nxh_tensor *x);
+/* svd (backend_intf.ml:655-664; nx_backend.ml:651-677): s [..., k] float64
+   descending; u [..., m, k] and vt [..., k, n] (thin) or [..., m, m] and
+   [..., n, n] (full), told apart by their shapes as in the reference. k <= 4096. */
+int nxh_svd(nxh_context *ctx, const nxh_tensor *u, const nxh_tensor *s, const nxh_tensor *vt, const nxh_tensor *x);
+/* eig / eigvals (backend_intf.ml:666-683; nx_c_eig.c:43-62; nx_backend.ml:679-
+   707): w [..., n] and v [..., n, n] complex128 whatever x's dtype; v may be
+   null (values only); eigenvectors have unit 2-norm, eigenvalues come in the
+   order of the Schur factor's diagonal. n <= 2048. */
+int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nxh_tensor *x);
+
 /* ── recorded sequences ──────────────────────────────────────────────────── */
 
 /* The reference backend has no counterpart: its eager calls cost a C stub

@@ -360,6 +360,124 @@ class OracleBackend:
         y = (np.fft.ifft(f, axis=-1) * size).real if size else np.zeros(f.shape)
         return self._from_array(np.moveaxis(y, -1, last), dtype)
 
+    # linear algebra ------------------------------------------------------------
+    # The reference factors with its own LAPACK-style kernels in the storage's
+    # compute type (nx_c_tri.c, nx_c_qr.c, nx_c_eigh.c, nx_c_svd.c, nx_c_eig.c);
+    # its tests accept any factorisation that reconstructs the matrix
+    # (backend_contract.ml:2075-2311). Here numpy / LAPACK in double precision
+    # stands for it: same conventions (lower triangle read, real R diagonal,
+    # ascending / descending order, unit-norm vectors), results rounded to the
+    # result dtype by the oracle's own cast.
+    def _wide(self, x):
+        return logical(self.cast(x, dt.complex128 if x.dtype.is_complex else dt.float64))
+
+    def _narrow(self, a, d):
+        wide = dt.complex128 if np.iscomplexobj(a) else dt.float64
+        t = self._from_array(np.asarray(a), wide)
+        return t if d is wide else self.cast(t, d)
+
+    @staticmethod
+    def _check_float(op, x):
+        if not (x.dtype.is_float or x.dtype.is_complex):
+            raise RuntimeError(f"{op}: linalg requires a float or complex dtype")
+
+    def cholesky(self, x, upper: bool = False):
+        self._check_float("cholesky", x)
+        a = self._wide(x)
+        low = np.tril(a)
+        herm = low + np.swapaxes(np.tril(a, -1), -1, -2).conj()  # nx_c_tri.c:11-16: only the lower triangle is read
+        try:
+            if not np.all(np.isfinite(herm)):
+                raise np.linalg.LinAlgError
+            l = np.linalg.cholesky(herm)
+        except np.linalg.LinAlgError:
+            raise RuntimeError("cholesky: matrix is not positive definite") from None
+        return self._narrow(np.swapaxes(l, -1, -2).conj() if upper else l, x.dtype)
+
+    def triangular_solve(self, a, b, upper: bool, transpose: bool, unit_diag: bool):
+        import scipy.linalg
+
+        self._check_float("triangular_solve", a)
+        A, Bm = self._wide(a), self._wide(b)
+        vector = Bm.ndim == A.ndim - 1
+        if vector:
+            Bm = Bm[..., None]
+        out = np.empty(Bm.shape, np.result_type(A, Bm))
+        n = A.shape[-1]
+        for idx in np.ndindex(*A.shape[:-2]):
+            if not unit_diag and np.any(np.diagonal(A[idx]) == 0):  # nx_c_tri.c:113-118: exact zero only
+                raise RuntimeError("triangular_solve: triangular matrix is singular")
+            out[idx] = (scipy.linalg.solve_triangular(A[idx], Bm[idx], lower=not upper, trans="C" if transpose else "N",
+                                                      unit_diagonal=unit_diag, check_finite=False)
+                        if n else Bm[idx])
+        return self._narrow(out[..., 0] if vector else out, b.dtype)
+
+    @staticmethod
+    def _householder_qr(a, reduced):
+        """nx_c_qr.c:44-110 restated: LAPACK's reflectors (real beta = -sign(re alpha) |x|,
+        tau = ((beta - re alpha) / beta, -im alpha / beta), H_j^H applied while factoring,
+        Q = H_0 H_1 ...), except that a column with nothing below the diagonal takes no
+        reflector even when its diagonal element is complex (LAPACK would rotate it real)."""
+        m, n = a.shape
+        k = min(m, n)
+        A = a.copy()
+        tau = np.zeros(k, A.dtype)
+        for j in range(k):
+            x = A[j + 1:, j]
+            xnorm2 = float(np.sum(x.real ** 2 + x.imag ** 2))
+            alpha = A[j, j]
+            if xnorm2 == 0.0:
+                continue
+            anorm = np.sqrt(alpha.real ** 2 + alpha.imag ** 2 + xnorm2)
+            beta = -anorm if alpha.real >= 0 else anorm
+            tau[j] = complex((beta - alpha.real) / beta, -alpha.imag / beta) if np.iscomplexobj(A) else (beta - alpha) / beta
+            A[j + 1:, j] = x / (alpha - beta)
+            A[j, j] = beta
+            v = np.concatenate([[1.0], A[j + 1:, j]])
+            w = np.conj(tau[j]) * (v.conj() @ A[j:, j + 1:])
+            A[j:, j + 1:] -= np.outer(v, w)
+        nq = k if reduced else m
+        Q = np.eye(m, nq, dtype=A.dtype)
+        for j in range(k - 1, -1, -1):
+            v = np.concatenate([[1.0], A[j + 1:, j]])
+            w = tau[j] * (v.conj() @ Q[j:, j:])
+            Q[j:, j:] -= np.outer(v, w)
+        return Q, np.triu(A[:(k if reduced else m), :])
+
+    def qr(self, x, reduced: bool = True):
+        self._check_float("qr", x)
+        a = self._wide(x)
+        m, n = a.shape[-2:]
+        k = min(m, n)
+        q = np.empty(a.shape[:-2] + (m, k if reduced else m), a.dtype)
+        r = np.empty(a.shape[:-2] + (k if reduced else m, n), a.dtype)
+        for idx in np.ndindex(*a.shape[:-2]):
+            q[idx], r[idx] = self._householder_qr(a[idx], reduced)
+        return self._narrow(q, x.dtype), self._narrow(r, x.dtype)
+
+    def eigh(self, x):
+        self._check_float("eigh", x)
+        w, v = np.linalg.eigh(self._wide(x), UPLO="L")  # nx_c_eigh.c:14-21: lower triangle, ascending
+        return self._narrow(w, dt.float64), self._narrow(v, x.dtype)
+
+    def eigvalsh(self, x):
+        self._check_float("eigvalsh", x)
+        return self._narrow(np.linalg.eigvalsh(self._wide(x), UPLO="L"), dt.float64)
+
+    def svd(self, x, full_matrices: bool = False):
+        self._check_float("svd", x)
+        u, s, vt = np.linalg.svd(self._wide(x), full_matrices=full_matrices)
+        return self._narrow(u, x.dtype), self._narrow(s, dt.float64), self._narrow(vt, x.dtype)
+
+    def eig(self, x):
+        self._check_float("eig", x)
+        w, v = np.linalg.eig(self._wide(x))  # unit 2-norm columns, as nx_c_eig.c:56
+        return self._narrow(w.astype(np.complex128), dt.complex128), self._narrow(v.astype(np.complex128), dt.complex128)
+
+    def eigvals(self, x):
+        self._check_float("eigvals", x)
+        return self._narrow(np.linalg.eigvals(self._wide(x)).astype(np.complex128), dt.complex128)
+
 
 def window_shapes(in_shape, kernel_size, stride, dilation, padding):
     """Result shape of unfold (nx_backend.ml:427-445) and the K-long parameter

@@ -97,6 +97,12 @@ SIGNATURES = {
     "nxh_fft": (C.c_int, [_CTX, _T, _T, _P(C.c_int32), C.c_int, C.c_int]),
     "nxh_rfft": (C.c_int, [_CTX, _T, _T, _P(C.c_int32), C.c_int]),
     "nxh_irfft": (C.c_int, [_CTX, _T, _T, _P(C.c_int32), C.c_int, C.c_int64]),
+    "nxh_cholesky": (C.c_int, [_CTX, _T, _T, C.c_int]),
+    "nxh_triangular_solve": (C.c_int, [_CTX, _T, _T, _T, C.c_int]),
+    "nxh_qr": (C.c_int, [_CTX, _T, _T, _T, C.c_int]),
+    "nxh_eigh": (C.c_int, [_CTX, _T, _T, _T]),
+    "nxh_svd": (C.c_int, [_CTX, _T, _T, _T, _T]),
+    "nxh_eig": (C.c_int, [_CTX, _T, _T, _T]),
     "nxh_softmax_rows": (C.c_int, [_CTX, _T, _T, C.c_void_p, _T, C.c_void_p]),
     "nxh_layer_norm_rows": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_double]),
     "nxh_gelu_tanh": (C.c_int, [_CTX, _T, _T, C.c_void_p]),

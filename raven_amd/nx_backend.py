@@ -436,6 +436,77 @@ class Backend:
         self._check(self._lib.nxh_irfft(self._h, C.byref(o), C.byref(a), ax, n, size if s is not None else 0))
         return out
 
+    # ── linear algebra (nx_backend.ml:550-707): the binding allocates every result ──
+    def cholesky(self, x: Tensor, upper: bool = False) -> Tensor:
+        out = self.buffer(x.dtype, x.shape)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_cholesky(self._h, C.byref(o), C.byref(a), int(upper)))
+        return out
+
+    def triangular_solve(self, a: Tensor, b: Tensor, upper: bool, transpose: bool, unit_diag: bool) -> Tensor:
+        vector = len(b.shape) == len(a.shape) - 1
+        bm = self.reshape(b, tuple(b.shape) + (1,)) if vector else b
+        out = self.buffer(b.dtype, bm.shape)
+        flags = int(upper) | (int(transpose) << 1) | (int(unit_diag) << 2)
+        o, da, db = out._desc(), a._desc(), bm._desc()
+        self._check(self._lib.nxh_triangular_solve(self._h, C.byref(o), C.byref(da), C.byref(db), flags))
+        return self.reshape(out, b.shape) if vector else out
+
+    def qr(self, x: Tensor, reduced: bool = True):
+        if len(x.shape) < 2:
+            raise ValueError("qr: shape mismatch")
+        *batch, m, n = x.shape
+        k = min(m, n)
+        q = self.buffer(x.dtype, (*batch, m, k if reduced else m))
+        r = self.buffer(x.dtype, (*batch, k if reduced else m, n))
+        dq, dr, a = q._desc(), r._desc(), x._desc()
+        self._check(self._lib.nxh_qr(self._h, C.byref(dq), C.byref(dr), C.byref(a), int(reduced)))
+        return q, r
+
+    def _eigh(self, x: Tensor, vectors: bool):
+        if len(x.shape) < 2:
+            raise ValueError("eigh: shape mismatch")
+        w = self.buffer(dt.float64, tuple(x.shape[:-2]) + (x.shape[-1],))
+        v = self.buffer(x.dtype, x.shape) if vectors else None
+        dw, a = w._desc(), x._desc()
+        dv = v._desc() if vectors else None
+        self._check(self._lib.nxh_eigh(self._h, C.byref(dw), C.byref(dv) if vectors else None, C.byref(a)))
+        return w, v
+
+    def eigh(self, x: Tensor):
+        return self._eigh(x, True)
+
+    def eigvalsh(self, x: Tensor) -> Tensor:
+        return self._eigh(x, False)[0]
+
+    def svd(self, x: Tensor, full_matrices: bool = False):
+        if len(x.shape) < 2:
+            raise ValueError("svd: shape mismatch")
+        *batch, m, n = x.shape
+        k = min(m, n)
+        u = self.buffer(x.dtype, (*batch, m, m if full_matrices else k))
+        s = self.buffer(dt.float64, (*batch, k))
+        vt = self.buffer(x.dtype, (*batch, n if full_matrices else k, n))
+        du, ds, dv, a = u._desc(), s._desc(), vt._desc(), x._desc()
+        self._check(self._lib.nxh_svd(self._h, C.byref(du), C.byref(ds), C.byref(dv), C.byref(a)))
+        return u, s, vt
+
+    def _eig(self, x: Tensor, vectors: bool):
+        if len(x.shape) < 2:
+            raise ValueError("eig: shape mismatch")
+        w = self.buffer(dt.complex128, tuple(x.shape[:-2]) + (x.shape[-1],))
+        v = self.buffer(dt.complex128, x.shape) if vectors else None
+        dw, a = w._desc(), x._desc()
+        dv = v._desc() if vectors else None
+        self._check(self._lib.nxh_eig(self._h, C.byref(dw), C.byref(dv) if vectors else None, C.byref(a)))
+        return w, v
+
+    def eig(self, x: Tensor):
+        return self._eig(x, True)
+
+    def eigvals(self, x: Tensor) -> Tensor:
+        return self._eig(x, False)[0]
+
     # ── fused sequences of primitives (no counterpart in Backend_intf.S) ────
     def _scalar_arg(self, dtype: dt.DType, value):
         if value is None:

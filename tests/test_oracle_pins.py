@@ -863,3 +863,79 @@ def test_fft_reference_cases_and_the_definition():
     x = cdata(F["parseval"]["n"])
     e = lambda a: float(np.sum(np.abs(a) ** 2))
     assert abs(e(logical(B.fft(_mk(B, x, dt.complex128), [0]))) - len(x) * e(x)) <= F["parseval"]["rel"] * len(x) * e(x)
+
+
+def test_linalg_reference_cases():
+    """The reference's own linalg cases, checked the way it checks them: residuals
+    relative to the matrix norm (backend_contract.ml:2075-2311), exact values where it has them."""
+    B = OracleBackend()
+    L = GOLD["linalg"]
+    tol = L["tolerance"]
+    f = lambda a: _mk(B, np.array(a, np.float64), dt.float64)
+    rr = lambda ref, x: np.max(np.abs(np.asarray(ref) - np.asarray(x))) / max(1e-30, np.sqrt(np.sum(np.abs(ref) ** 2)))
+    Hm = lambda a: np.swapaxes(a, -1, -2).conj()
+    m4x3, sq4 = np.array(L["m4x3"], float), np.array(L["sq4"], float)
+    spd4 = sq4 @ sq4.T + 4 * np.eye(4)
+    low = logical(B.cholesky(f(spd4), False))
+    assert np.all(np.triu(low, 1) == 0) and rr(spd4, low @ low.T) <= tol
+    up = logical(B.cholesky(f(spd4), True))
+    assert np.all(np.tril(up, -1) == 0) and rr(spd4, up.T @ up) <= tol
+    for reduced, qs, rs in ((True, (4, 3), (3, 3)), (False, (4, 4), (4, 3))):
+        q, r = (logical(t) for t in B.qr(f(m4x3), reduced))
+        assert q.shape == qs and r.shape == rs and rr(m4x3, q @ r) <= tol
+        assert rr(np.eye(qs[1]), q.T @ q) <= tol and np.all(np.abs(np.tril(r, -1)) <= tol)
+    for full, us, vs in ((False, (4, 3), (3, 3)), (True, (4, 4), (3, 3))):
+        u, s, vt = (logical(t) for t in B.svd(f(m4x3), full))
+        assert u.shape == us and s.shape == (3,) and vt.shape == vs and s.dtype == np.float64
+        assert np.all(s >= -tol) and np.all(np.diff(s) <= tol)
+        sigma = np.zeros((us[1], 3))
+        sigma[:3, :3] = np.diag(s)
+        assert rr(m4x3, u @ sigma @ vt) <= tol
+    w, v = (logical(t) for t in B.eigh(f(spd4)))
+    assert rr(spd4 @ v, v @ np.diag(w)) <= tol and rr(np.eye(4), v.T @ v) <= tol
+    assert rr(w, logical(B.eigvalsh(f(spd4)))) <= tol
+    tri = np.array(L["tri3"], float)
+    x = logical(B.triangular_solve(f(tri), f(L["tri3_rhs"]), False, False, False))
+    assert rr(np.array(L["tri3_rhs"], float), tri @ x) <= tol
+    c = L["tri3_vector"]
+    x = logical(B.triangular_solve(f(tri), f(c["b"]), False, False, False))
+    assert x.shape == (3,) and np.max(np.abs(x - c["x"])) <= c["tol"]
+    c = L["tri_batched"]
+    x = logical(B.triangular_solve(f(c["a"]), f(c["b"]), False, False, False))
+    assert x.shape == (2, 2) and np.max(np.abs(x - np.array(c["x"]))) <= c["tol"]
+    a = np.array(L["eig3"], float)
+    w, v = (logical(t) for t in B.eig(f(a)))
+    assert w.dtype == np.complex128 and rr(a @ v, v @ np.diag(w)) <= tol
+    assert rr(w, logical(B.eigvals(f(a)))) <= tol
+    ab = np.array(L["eigh_batched"], float)
+    w, v = (logical(t) for t in B.eigh(f(ab)))
+    assert w.shape == (2, 3)
+    for i in range(2):
+        assert rr(ab[i] @ v[i], v[i] @ np.diag(w[i])) <= tol
+    ca = np.array([[complex(*e) for e in row] for row in L["chol_complex"]])
+    l = logical(B.cholesky(_mk(B, ca, dt.complex128), False))
+    assert rr(ca, l @ Hm(l)) <= tol
+    # beyond the reference's cases: every substitution variant against numpy's general solver,
+    # the failures, and complex Householder factors
+    rng = np.random.default_rng(81)
+    A = rng.standard_normal((5, 5)) + 1j * rng.standard_normal((5, 5)) + 6 * np.eye(5)
+    Bm = rng.standard_normal((5, 3)) + 1j * rng.standard_normal((5, 3))
+    for upper in (False, True):
+        for transpose in (False, True):
+            for unit in (False, True):
+                M = np.triu(A) if upper else np.tril(A)
+                if unit:
+                    M = M - np.diag(np.diag(M)) + np.eye(5)
+                want = np.linalg.solve(Hm(M) if transpose else M, Bm)
+                got = logical(B.triangular_solve(_mk(B, A, dt.complex128), _mk(B, Bm, dt.complex128), upper, transpose, unit))
+                assert np.max(np.abs(got - want)) <= 1e-12, (upper, transpose, unit)
+    with pytest.raises(RuntimeError, match="not positive definite"):
+        B.cholesky(f(np.diag([1.0, -1.0])), False)
+    with pytest.raises(RuntimeError, match="singular"):
+        B.triangular_solve(f(np.diag([1.0, 0.0])), f([1.0, 1.0]), False, False, False)
+    for m, n in ((6, 4), (4, 6), (5, 5)):
+        a = rng.standard_normal((m, n)) + 1j * rng.standard_normal((m, n))
+        q, r = (logical(t) for t in B.qr(_mk(B, a, dt.complex128), True))
+        assert rr(a, q @ r) <= 1e-13 and rr(np.eye(q.shape[1]), Hm(q) @ q) <= 1e-13
+        k = min(m, n)
+        assert np.max(np.abs(np.diagonal(r)[:k - 1].imag)) <= 1e-15  # reflected columns have a real diagonal
