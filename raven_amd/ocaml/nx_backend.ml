@@ -6,10 +6,8 @@
    OCaml toolchain); raven_amd/nx_backend.py is its executable twin and is what
    the parity tests drive.
 
-   Every member of Backend_intf.S except the fft and linalg families is wired to
-   the GPU. Those two must exist for the module to satisfy the signature; until
-   they have device kernels they are answered by copying to the host, calling
-   the C backend's routine and copying back, and are omitted from this excerpt. *)
+   Every member of Backend_intf.S is wired to the GPU, the fft and linalg
+   families included. *)
 
 open Nx_core
 
@@ -234,3 +232,110 @@ let fold x ~output_size ~kernel_size ~stride ~dilation ~padding =
   let leading = Array.sub x.shape 0 (Array.length x.shape - 2) in
   let out = create_tensor x.context x.dtype (Array.append leading output_size) in
   caml_fold_window out x output_size kernel_size stride dilation (flatten_pairs padding); out
+
+(* Fourier transforms, nx_backend.ml:502-548: unnormalised; the binding owns shape and dtype *)
+external caml_fft : (Complex.t, 'b) t -> (Complex.t, 'b) t -> int array -> unit = "caml_nx_hip_fft"
+external caml_ifft : (Complex.t, 'b) t -> (Complex.t, 'b) t -> int array -> unit = "caml_nx_hip_ifft"
+external caml_rfft : (Complex.t, 'b) t -> (float, 'a) t -> int array -> unit = "caml_nx_hip_rfft"
+external caml_irfft : (float, 'b) t -> (Complex.t, 'a) t -> int array -> int array -> unit = "caml_nx_hip_irfft"
+
+let fft x ~axes =
+  let out = create_tensor x.context x.dtype x.shape in
+  caml_fft out x axes; out
+
+let ifft x ~axes =
+  let out = create_tensor x.context x.dtype x.shape in
+  caml_ifft out x axes; out
+
+let rfft x ~dtype ~axes =
+  let last = axes.(Array.length axes - 1) in
+  let shape = Array.copy x.shape in
+  shape.(last) <- (x.shape.(last) / 2) + 1;
+  let out = create_tensor x.context dtype shape in
+  caml_rfft out x axes; out
+
+let irfft ?s x ~dtype ~axes =
+  let li = Array.length axes - 1 in
+  let last = axes.(li) in
+  let size = match s with Some sizes -> sizes.(li) | None -> (x.shape.(last) - 1) * 2 in
+  let shape = Array.copy x.shape in
+  shape.(last) <- size;
+  let out = create_tensor x.context dtype shape in
+  caml_irfft out x axes (match s with Some sizes -> sizes | None -> [||]); out
+
+(* linear algebra, nx_backend.ml:550-707. Numeric failures arrive as Failure with the
+   reference's status text as suffix and are lifted to Linalg_error the same way. *)
+external caml_cholesky : ('a, 'b) t -> ('a, 'b) t -> bool -> unit = "caml_nx_hip_cholesky"
+external caml_triangular_solve : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> int -> unit = "caml_nx_hip_triangular_solve"
+external caml_qr : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> bool -> unit = "caml_nx_hip_qr"
+external caml_eigh : (float, Dtype.float64_elt) t -> ('a, 'b) t -> ('a, 'b) t -> bool -> unit = "caml_nx_hip_eigh"
+external caml_svd : ('a, 'b) t -> (float, Dtype.float64_elt) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_svd"
+external caml_eig :
+  (Complex.t, Dtype.complex64_elt) t -> (Complex.t, Dtype.complex64_elt) t -> ('a, 'b) t -> bool -> unit
+  = "caml_nx_hip_eig"
+
+let reraise_linalg ~op f =
+  try f ()
+  with Failure msg as e ->
+    let ends suffix = String.ends_with ~suffix msg in
+    if ends "matrix is not positive definite" then raise (Backend_intf.Linalg_error { op; kind = `Not_positive_definite })
+    else if ends "triangular matrix is singular" then raise (Backend_intf.Linalg_error { op; kind = `Singular })
+    else if ends "eigenvalue iteration did not converge" then raise (Backend_intf.Linalg_error { op; kind = `No_convergence })
+    else raise e
+
+let cholesky ~upper x =
+  let out = create_tensor x.context x.dtype x.shape in
+  reraise_linalg ~op:"cholesky" (fun () -> caml_cholesky out x upper); out
+
+let triangular_solve ~upper ~transpose ~unit_diag a b =
+  let vector_rhs = Array.length b.shape = Array.length a.shape - 1 in
+  let bm = if vector_rhs then reshape b (Array.append b.shape [| 1 |]) else b in
+  let out = create_tensor b.context b.dtype bm.shape in
+  let flags = (if upper then 1 else 0) lor (if transpose then 2 else 0) lor (if unit_diag then 4 else 0) in
+  reraise_linalg ~op:"triangular_solve" (fun () -> caml_triangular_solve out a bm flags);
+  if vector_rhs then reshape out b.shape else out
+
+let matrix_dims x =
+  let nd = Array.length x.shape in
+  (Array.sub x.shape 0 (nd - 2), x.shape.(nd - 2), x.shape.(nd - 1))
+
+let qr ~reduced x =
+  let batch, m, n = matrix_dims x in
+  let k = Int.min m n in
+  let q = create_tensor x.context x.dtype (Array.append batch [| m; (if reduced then k else m) |]) in
+  let r = create_tensor x.context x.dtype (Array.append batch [| (if reduced then k else m); n |]) in
+  reraise_linalg ~op:"qr" (fun () -> caml_qr q r x reduced); (q, r)
+
+let eigh_values x =
+  let batch, _, n = matrix_dims x in
+  create_tensor x.context Dtype.Float64 (Array.append batch [| n |])
+
+let eigvalsh x =
+  let w = eigh_values x in
+  reraise_linalg ~op:"eigvalsh" (fun () -> caml_eigh w x x false); w
+
+let eigh x =
+  let w = eigh_values x in
+  let v = create_tensor x.context x.dtype x.shape in
+  reraise_linalg ~op:"eigh" (fun () -> caml_eigh w v x true); (w, v)
+
+let svd ~full_matrices x =
+  let batch, m, n = matrix_dims x in
+  let k = Int.min m n in
+  let u = create_tensor x.context x.dtype (Array.append batch (if full_matrices then [| m; m |] else [| m; k |])) in
+  let s = create_tensor x.context Dtype.Float64 (Array.append batch [| k |]) in
+  let vt = create_tensor x.context x.dtype (Array.append batch (if full_matrices then [| n; n |] else [| k; n |])) in
+  reraise_linalg ~op:"svd" (fun () -> caml_svd u s vt x); (u, s, vt)
+
+let eig_values x =
+  let batch, _, n = matrix_dims x in
+  create_tensor x.context Dtype.Complex128 (Array.append batch [| n |])
+
+let eigvals x =
+  let w = eig_values x in
+  reraise_linalg ~op:"eigvals" (fun () -> caml_eig w w x false); w
+
+let eig x =
+  let w = eig_values x in
+  let v = create_tensor x.context Dtype.Complex128 x.shape in
+  reraise_linalg ~op:"eig" (fun () -> caml_eig w v x true); (w, v)

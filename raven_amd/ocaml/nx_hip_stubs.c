@@ -33,7 +33,8 @@
   X(memcpy_h2d) X(memcpy_d2h) X(synchronize) X(fill) X(unary) X(binary)       \
   X(compare) X(where) X(cast) X(reduce) X(argreduce) X(matmul) X(copy)        \
   X(gather) X(scatter) X(pad) X(cat) X(scan) X(threefry) X(dtype_bytes)       \
-  X(sort) X(argsort) X(unfold) X(fold)
+  X(sort) X(argsort) X(unfold) X(fold) X(fft) X(rfft) X(irfft) X(cholesky)    \
+  X(triangular_solve) X(qr) X(eigh) X(svd) X(eig)
 static struct {
 #define X(n) __typeof__(nxh_##n) *n;
   NXH_SYMBOLS(X)
@@ -400,4 +401,122 @@ CAMLprim value caml_nx_hip_fold(value vout, value vx, value vosize, value vkerne
 CAMLprim value caml_nx_hip_fold_bc(value *argv, int argn) {
   (void)argn;
   return caml_nx_hip_fold(argv[0], argv[1], argv[2], argv[3], argv[4], argv[5], argv[6]);
+}
+
+/* ── Fourier transforms: arguments as caml_nx_c_fft / _ifft / _rfft / _irfft
+   (nx_c_fft.c:1159-1230); axes is an OCaml int array, s the optional sizes
+   (empty = inferred), of which only the last entry is read ─────────────── */
+static int axes_array(value v, int32_t *dst) {
+  int n = (int)Wosize_val(v);
+  if (n > NXH_MAX_NDIM) caml_failwith("ndim exceeds NX_C_MAX_NDIM");
+  for (int i = 0; i < n; i++) dst[i] = (int32_t)Long_val(Field(v, i));
+  return n;
+}
+static value fft_common(value vout, value vx, value vaxes, int inverse) {
+  CAMLparam3(vout, vx, vaxes);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int32_t axes[NXH_MAX_NDIM];
+  int n = axes_array(vaxes, axes);
+  check(c, L.fft(c, &o, &x, axes, n, inverse));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_fft(value vout, value vx, value vaxes) { return fft_common(vout, vx, vaxes, 0); }
+CAMLprim value caml_nx_hip_ifft(value vout, value vx, value vaxes) { return fft_common(vout, vx, vaxes, 1); }
+CAMLprim value caml_nx_hip_rfft(value vout, value vx, value vaxes) {
+  CAMLparam3(vout, vx, vaxes);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int32_t axes[NXH_MAX_NDIM];
+  int n = axes_array(vaxes, axes);
+  check(c, L.rfft(c, &o, &x, axes, n));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_irfft(value vout, value vx, value vaxes, value vs) {
+  CAMLparam4(vout, vx, vaxes, vs);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int32_t axes[NXH_MAX_NDIM];
+  int n = axes_array(vaxes, axes);
+  int ns = (int)Wosize_val(vs);
+  int64_t s_last = ns > 0 ? (int64_t)Long_val(Field(vs, ns - 1)) : 0;
+  check(c, L.irfft(c, &o, &x, axes, n, s_last));
+  CAMLreturn(Val_unit);
+}
+
+/* ── linear algebra: arguments as the reference's stubs (nx_c_tri.c:564-600,
+   nx_c_qr.c, nx_c_eigh.c:1765-, nx_c_svd.c, nx_c_eig.c:1324-). These calls wait
+   for the stream (a numeric failure belongs to the call), so the runtime lock is
+   released around them ───────────────────────────────────────────────────── */
+#define BLOCKING(call)                \
+  do {                                \
+    caml_release_runtime_system();    \
+    int rc__ = (call);                \
+    caml_acquire_runtime_system();    \
+    check(c, rc__);                   \
+  } while (0)
+
+CAMLprim value caml_nx_hip_cholesky(value vout, value vx, value vupper) {
+  CAMLparam3(vout, vx, vupper);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int upper = Bool_val(vupper);
+  BLOCKING(L.cholesky(c, &o, &x, upper));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_triangular_solve(value vout, value va, value vb, value vflags) {
+  CAMLparam4(vout, va, vb, vflags);
+  nxh_tensor o, a, b;
+  nxh_context *c = extract(vout, &o);
+  extract(va, &a);
+  extract(vb, &b);
+  int flags = Int_val(vflags);
+  BLOCKING(L.triangular_solve(c, &o, &a, &b, flags));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_qr(value vq, value vr, value vx, value vreduced) {
+  CAMLparam4(vq, vr, vx, vreduced);
+  nxh_tensor q, r, x;
+  nxh_context *c = extract(vq, &q);
+  extract(vr, &r);
+  extract(vx, &x);
+  int reduced = Bool_val(vreduced);
+  BLOCKING(L.qr(c, &q, &r, &x, reduced));
+  CAMLreturn(Val_unit);
+}
+/* vectors = false: the eigenvector slot holds the input again and is not read
+   (nx_backend.ml:566-571, 679-689) */
+CAMLprim value caml_nx_hip_eigh(value vw, value vv, value vx, value vvectors) {
+  CAMLparam4(vw, vv, vx, vvectors);
+  nxh_tensor w, v, x;
+  nxh_context *c = extract(vw, &w);
+  extract(vv, &v);
+  extract(vx, &x);
+  int vectors = Bool_val(vvectors);
+  BLOCKING(L.eigh(c, &w, vectors ? &v : NULL, &x));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_svd(value vu, value vs, value vvt, value vx) {
+  CAMLparam4(vu, vs, vvt, vx);
+  nxh_tensor u, s, vt, x;
+  nxh_context *c = extract(vu, &u);
+  extract(vs, &s);
+  extract(vvt, &vt);
+  extract(vx, &x);
+  BLOCKING(L.svd(c, &u, &s, &vt, &x));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_eig(value vw, value vv, value vx, value vvectors) {
+  CAMLparam4(vw, vv, vx, vvectors);
+  nxh_tensor w, v, x;
+  nxh_context *c = extract(vw, &w);
+  extract(vv, &v);
+  extract(vx, &x);
+  int vectors = Bool_val(vvectors);
+  BLOCKING(L.eig(c, &w, vectors ? &v : NULL, &x));
+  CAMLreturn(Val_unit);
 }
