@@ -276,6 +276,45 @@ def next_ops(hip, W):
     timed("layer_norm_rows [8192,768] bf16 (fused)", lambda: hip.layer_norm_rows(x, gam, bet, 1e-5), 2 * b * sq * 768 * 2)
     y = bf((b * sq, 3072))
     timed("gelu_tanh [8192,3072] bf16 (fused)", lambda: hip.gelu_tanh(y), 2 * b * sq * 3072 * 2)
+    del x, y, gam, bet, q, k, v
+    # Fourier transforms: one pass reads and writes the tensor once; the butterflies run in LDS
+    cplx = lambda shape: W.dev((rng.standard_normal(shape) + 1j * rng.standard_normal(shape)).astype(np.complex64),
+                               dt.complex64)
+    z = cplx((16384, 1024))
+    timed("fft [16384,1024] complex64 axis 1 (fft_lines, radix-2 in LDS)", lambda: hip.fft(z, [1]), 2 * 16384 * 1024 * 8)
+    out[-1]["GFLOP/s"] = round(5 * 16384 * 1024 * 10 / out[-1]["ms"] / 1e6, 1)
+    z2 = cplx((4096, 4096))
+    timed("fft [4096,4096] complex64 axis 0 (strided lines)", lambda: hip.fft(z2, [0]), 2 * 4096 * 4096 * 8)
+    z3 = cplx((8192, 1000))
+    timed("fft [8192,1000] complex64 axis 1 (Bluestein in LDS, M = 2048)", lambda: hip.fft(z3, [1]), 2 * 8192 * 1000 * 8)
+    r = W.dev(rng.standard_normal((16384, 2048)).astype(np.float32), dt.float32)
+    timed("rfft [16384,2048] f32 -> complex64 axis 1", lambda: hip.rfft(r, dt.complex64, [1]),
+          16384 * 2048 * 4 + 16384 * 1025 * 8)
+    big = cplx((4, 1 << 20))
+    timed("fft [4,2^20] complex64 axis 1 (four-step through a workspace)", lambda: hip.fft(big, [1]),
+          2 * 4 * (1 << 20) * 8, iters=5)
+    for rec in out[-5:]:
+        rec["bound"] = "lds"
+    del z, z2, z3, r, big
+    # linear algebra: one workgroup per matrix, correctness first; times only
+    def la(name, fn, iters=3):
+        timed(name, fn, 0, iters=iters)
+        for key in ("GB/s", "frac_hbm"):
+            out[-1].pop(key)
+        out[-1]["bound"] = "latency"
+
+    g = rng.standard_normal((256, 64, 64)).astype(np.float32)
+    spd = W.dev(g @ g.transpose(0, 2, 1) + 64 * np.eye(64, dtype=np.float32), dt.float32)
+    gen = W.dev(g, dt.float32)
+    la("cholesky [256,64,64] f32", lambda: hip.cholesky(spd))
+    la("qr [256,64,64] f32, reduced", lambda: hip.qr(gen))
+    la("eigh [256,64,64] f32 (Jacobi)", lambda: hip.eigh(spd))
+    la("svd [256,64,64] f32 (one-sided Jacobi)", lambda: hip.svd(gen))
+    la("eig [256,64,64] f32 (Hessenberg + shifted QR)", lambda: hip.eig(gen))
+    one = rng.standard_normal((1, 512, 512)).astype(np.float32)
+    big_spd = W.dev(one @ one.transpose(0, 2, 1) + 512 * np.eye(512, dtype=np.float32), dt.float32)
+    la("cholesky [1,512,512] f32", lambda: hip.cholesky(big_spd))
+    la("eigh [1,512,512] f32 (Jacobi)", lambda: hip.eigh(big_spd), iters=1)
     return out
 
 

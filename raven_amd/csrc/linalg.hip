@@ -278,6 +278,24 @@ __device__ __forceinline__ void jacobi_rotation(double app, double aqq, T g, dou
   *sp = S::scale(g, t * cc / ga);
 }
 
+// Ascending order, ties by position (nx_c_eigh.c:21): eigenvalue k goes to its
+// rank, its eigenvector column with it.
+template <class T>
+__device__ void eigh_sort_block(const T *A, const T *V, T *Vs, double *w, int n, int wantv) {
+  using S = Sc<T>;
+  for (int k = threadIdx.x; k < n; k += blockDim.x) {
+    const double wk = S::re(A[(size_t)k * n + k]);
+    int rank = 0;
+    for (int j = 0; j < n; j++) {
+      const double wj = S::re(A[(size_t)j * n + j]);
+      rank += (wj < wk) || (wj == wk && j < k);
+    }
+    w[rank] = wk;
+    if (wantv)
+      for (int i = 0; i < n; i++) Vs[(size_t)i * n + rank] = V[(size_t)i * n + k];
+  }
+}
+
 // ── eigh: two-sided Jacobi ──────────────────────────────────────────────────
 // A (row-major, overwritten), V (row-major; the eigenvectors when wantv), sorted
 // results to w (n doubles) and Vs (row-major, column k = eigenvector of w[k]).
@@ -369,17 +387,27 @@ __global__ __launch_bounds__(LA_THREADS) void eigh_kernel(T *a_all, T *v_all, T 
     if (threadIdx.x == 0) raise(status, LA_NO_CONVERGE);
     return;
   }
-  // ascending order, ties by position (nx_c_eigh.c:21)
-  for (int k = threadIdx.x; k < n; k += blockDim.x) {
-    const double wk = S::re(A[(size_t)k * n + k]);
+  eigh_sort_block(A, V, Vs, w, n, wantv);
+}
+
+// Columns by descending norm (ties by position) into Gs / Vs; `norms` holds nn doubles.
+template <class T>
+__device__ void svd_sort_block(const T *G, const T *V, T *Gs, T *Vs, int mm, int nn, double *norms) {
+  using S = Sc<T>;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  for (int c = wave; c < nn; c += waves) {
+    double a = 0.0;
+    for (int i = lane; i < mm; i += 64) a += S::abs2(G[(size_t)c * mm + i]);
+    a = wave_sum(a);
+    if (lane == 0) norms[c] = a;
+  }
+  __syncthreads();
+  for (int c = wave; c < nn; c += waves) {
+    const double a = norms[c];
     int rank = 0;
-    for (int j = 0; j < n; j++) {
-      const double wj = S::re(A[(size_t)j * n + j]);
-      rank += (wj < wk) || (wj == wk && j < k);
-    }
-    w[rank] = wk;
-    if (wantv)
-      for (int i = 0; i < n; i++) Vs[(size_t)i * n + rank] = V[(size_t)i * n + k];
+    for (int j = 0; j < nn; j++) rank += (norms[j] > a) || (norms[j] == a && j < c);
+    for (int i = lane; i < mm; i += 64) Gs[(size_t)rank * mm + i] = G[(size_t)c * mm + i];
+    for (int i = lane; i < nn; i += 64) Vs[(size_t)rank * nn + i] = V[(size_t)c * nn + i];
   }
 }
 
@@ -452,20 +480,7 @@ __global__ __launch_bounds__(LA_THREADS) void svd_jacobi_kernel(T *g_all, T *v_a
     if (threadIdx.x == 0) raise(status, LA_NO_CONVERGE);
     return;
   }
-  for (int c = wave; c < nn; c += waves) {
-    double a = 0.0;
-    for (int i = lane; i < mm; i += 64) a += S::abs2(G[(size_t)c * mm + i]);
-    a = wave_sum(a);
-    if (lane == 0) norms[c] = a;
-  }
-  __syncthreads();
-  for (int c = wave; c < nn; c += waves) {
-    const double a = norms[c];
-    int rank = 0;
-    for (int j = 0; j < nn; j++) rank += (norms[j] > a) || (norms[j] == a && j < c);
-    for (int i = lane; i < mm; i += 64) Gs[(size_t)rank * mm + i] = G[(size_t)c * mm + i];
-    for (int i = lane; i < nn; i += 64) Vs[(size_t)rank * nn + i] = V[(size_t)c * nn + i];
-  }
+  svd_sort_block(G, V, Gs, Vs, mm, nn, norms);
 }
 
 // After the QR of the sorted, orthogonal columns: R's diagonal carries the
@@ -486,6 +501,300 @@ __global__ __launch_bounds__(LA_THREADS) void svd_finish_kernel(const T *rt_all,
       for (int i = lane; i < mm; i += 64) Qt[(size_t)j * mm + i] = Qt[(size_t)j * mm + i] * phase;
     }
   }
+}
+
+// ── the same Jacobi iterations over the whole device ────────────────────────
+// One workgroup per matrix leaves 255 of 256 compute units idle when the batch is
+// small and the matrix is not: above 64 rows each phase of a round is a launch of
+// its own over every (matrix, pair, row) item, the host reads one convergence
+// counter per sweep, and a matrix that has converged is skipped by later rounds.
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void eigh_wide_prepare(T *a_all, T *v_all, int n, int wantv, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int64_t nn2 = (int64_t)n * n;
+  T *A = a_all + (e / nn2) * nn2;
+  const int i = (int)((e % nn2) / n), j = (int)(e % n);
+  if (i < j) A[(size_t)i * n + j] = S::conj(A[(size_t)j * n + i]);  // the lower triangle is never written here
+  else if (i == j) A[(size_t)i * n + i] = S::make(S::re(A[(size_t)i * n + i]), 0.0);
+  if (wantv) v_all[e] = i == j ? S::make(1.0, 0.0) : S::make(0.0, 0.0);
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void eigh_wide_check(const T *a_all, int n, int *done, int *remaining, int *status) {
+  using S = Sc<T>;
+  __shared__ double scratch[LA_THREADS / 64];
+  if (done[blockIdx.x]) return;
+  const T *A = a_all + (size_t)blockIdx.x * n * n;
+  double off = 0.0, all = 0.0;
+  for (int64_t e = threadIdx.x; e < (int64_t)n * n; e += blockDim.x) {
+    const double a2 = S::abs2(A[e]);
+    all += a2;
+    if (e / n != e % n) off += a2;
+  }
+  off = block_sum(off, scratch);
+  all = block_sum(all, scratch);
+  if (threadIdx.x != 0) return;
+  if (!(all == all) || !(off == off)) {
+    raise(status, LA_NO_CONVERGE);
+    done[blockIdx.x] = 1;
+  } else if (off <= all * 1e-29 * n) {
+    done[blockIdx.x] = 1;
+  } else {
+    atomicAdd(remaining, 1);
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void eigh_wide_params(const T *a_all, double *rc_all, T *rs_all, const int *done, int n,
+                                                              int N, int r, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int P = N / 2, t = (int)(e % P);
+  const int64_t b = e / P;
+  if (done[b]) return;
+  const T *A = a_all + (size_t)b * n * n;
+  int p, q;
+  round_robin(N, r, t, &p, &q);
+  double c = 1.0;
+  T sp = S::make(0.0, 0.0);
+  if (q < n) jacobi_rotation(S::re(A[(size_t)p * n + p]), S::re(A[(size_t)q * n + q]), A[(size_t)p * n + q], &c, &sp);
+  rc_all[e] = c;
+  rs_all[e] = sp;
+}
+
+// ROWS = false: X <- X J on the columns of A and V; ROWS = true: A <- J^H A.
+template <class T, bool ROWS>
+__global__ __launch_bounds__(LA_THREADS) void eigh_wide_rotate(T *a_all, T *v_all, const double *rc_all, const T *rs_all,
+                                                              const int *done, int n, int N, int r, int wantv, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int P = N / 2;
+  const int i = (int)(e % n), t = (int)((e / n) % P);
+  const int64_t b = e / ((int64_t)n * P);
+  if (done[b]) return;
+  int p, q;
+  round_robin(N, r, t, &p, &q);
+  if (q >= n) return;
+  const double c = rc_all[b * P + t];
+  const T sp = rs_all[b * P + t];
+  if (c == 1.0 && sp == S::make(0.0, 0.0)) return;
+  T *A = a_all + (size_t)b * n * n;
+  if (ROWS) {
+    const T x = A[(size_t)p * n + i], y = A[(size_t)q * n + i];
+    A[(size_t)p * n + i] = S::scale(x, c) - sp * y;
+    A[(size_t)q * n + i] = S::conj(sp) * x + S::scale(y, c);
+  } else {
+    T x = A[(size_t)i * n + p], y = A[(size_t)i * n + q];
+    A[(size_t)i * n + p] = S::scale(x, c) - S::conj(sp) * y;
+    A[(size_t)i * n + q] = sp * x + S::scale(y, c);
+    if (wantv) {
+      T *V = v_all + (size_t)b * n * n;
+      x = V[(size_t)i * n + p];
+      y = V[(size_t)i * n + q];
+      V[(size_t)i * n + p] = S::scale(x, c) - S::conj(sp) * y;
+      V[(size_t)i * n + q] = sp * x + S::scale(y, c);
+    }
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void eigh_wide_sort(const T *a_all, const T *v_all, T *vs_all, double *w_all, int n,
+                                                            int wantv) {
+  const size_t m = (size_t)blockIdx.x * n * n;
+  eigh_sort_block(a_all + m, v_all + m, vs_all + m, w_all + (size_t)blockIdx.x * n, n, wantv);
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void svd_wide_init(T *v_all, int nn, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int64_t w = e % ((int64_t)nn * nn);
+  v_all[e] = (w / nn) == (w % nn) ? S::make(1.0, 0.0) : S::make(0.0, 0.0);
+}
+
+// One round: a wave per (matrix, pair).
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void svd_wide_round(T *g_all, T *v_all, int mm, int nn, int N, int r, int64_t pairs,
+                                                            int *rotated) {
+  using S = Sc<T>;
+  const int lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= pairs) return;
+  const int P = N / 2, t = (int)(item % P);
+  const int64_t b = item / P;
+  int p, q;
+  round_robin(N, r, t, &p, &q);
+  if (q >= nn) return;
+  T *gp = g_all + ((size_t)b * nn + p) * mm, *gq = g_all + ((size_t)b * nn + q) * mm;
+  double a = 0.0, bb = 0.0;
+  T g = S::make(0.0, 0.0);
+  for (int i = lane; i < mm; i += 64) {
+    const T x = gp[i], y = gq[i];
+    a += S::abs2(x);
+    bb += S::abs2(y);
+    g = g + S::conj(x) * y;
+  }
+  a = wave_sum(a);
+  bb = wave_sum(bb);
+  g = wave_sum(g);
+  const double tol = fmax(1e-15, 8.0 * 2.220446049250313e-16 * sqrt((double)mm)), g2 = S::abs2(g);
+  if (!(g2 > tol * tol * a * bb) || !(g2 > 1e-300)) return;
+  double c;
+  T sp;
+  jacobi_rotation(a, bb, g, &c, &sp);
+  if (lane == 0) atomicAdd(rotated, 1);
+  for (int i = lane; i < mm; i += 64) {
+    const T x = gp[i], y = gq[i];
+    gp[i] = S::scale(x, c) - S::conj(sp) * y;
+    gq[i] = sp * x + S::scale(y, c);
+  }
+  T *vp = v_all + ((size_t)b * nn + p) * nn, *vq = v_all + ((size_t)b * nn + q) * nn;
+  for (int i = lane; i < nn; i += 64) {
+    const T x = vp[i], y = vq[i];
+    vp[i] = S::scale(x, c) - S::conj(sp) * y;
+    vq[i] = sp * x + S::scale(y, c);
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void svd_wide_sort(const T *g_all, const T *v_all, T *gs_all, T *vs_all, int mm, int nn) {
+  extern __shared__ double norms[];
+  const size_t g = (size_t)blockIdx.x * mm * nn, v = (size_t)blockIdx.x * nn * nn;
+  svd_sort_block(g_all + g, v_all + v, gs_all + g, vs_all + v, mm, nn, norms);
+}
+
+__global__ void la_fill_int(int *p, int count, int value) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) p[i] = value;
+}
+
+// ── cholesky and qr over the whole device ───────────────────────────────────
+// Column j of every matrix in one launch, a wave per (matrix, row >= j): the
+// lanes split the dot product along the finished columns (contiguous in the
+// row-major matrix). Every wave recomputes row j's own dot product for the pivot
+// instead of waiting for it.
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void cholesky_wide_column(T *all, double *diag_all, int n, int j, int64_t waves_total,
+                                                                  int *status) {
+  using S = Sc<T>;
+  const int lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= waves_total) return;
+  const int rows = n - j, i = j + (int)(item % rows);
+  T *A = all + (size_t)(item / rows) * n * n;
+  const T *ri = A + (size_t)i * n, *rj = A + (size_t)j * n;
+  T s = S::make(0.0, 0.0);
+  double dj = 0.0;
+  for (int k = lane; k < j; k += 64) {
+    const T ljk = rj[k];
+    s = s + ri[k] * S::conj(ljk);
+    dj += S::abs2(ljk);
+  }
+  s = wave_sum(s);
+  const double d = S::re(rj[j]) - wave_sum(dj);
+  if (!(d > 0.0)) {
+    if (i == j && lane == 0) raise(status, LA_NOT_PD);
+    return;  // later columns see an unfinished factor; the call fails as a whole
+  }
+  const double l = sqrt(d);
+  if (lane != 0) return;
+  // the pivot is kept aside until the end: the other waves of this launch still read A[j][j]
+  if (i == j) diag_all[(item / rows) * n + j] = l;
+  else A[(size_t)i * n + j] = S::scale(A[(size_t)i * n + j] - s, 1.0 / l);
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void cholesky_wide_finish(T *all, const double *diag_all, int n, int upper,
+                                                                  int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int64_t nn2 = (int64_t)n * n;
+  T *A = all + (e / nn2) * nn2;
+  const int i = (int)((e % nn2) / n), k = (int)(e % n);
+  if (i == k) A[(size_t)i * n + i] = S::make(diag_all[(e / nn2) * n + i], 0.0);
+  if (i <= k) return;
+  if (upper) {
+    A[(size_t)k * n + i] = S::conj(A[(size_t)i * n + k]);
+    A[(size_t)i * n + k] = S::make(0.0, 0.0);
+  } else {
+    A[(size_t)k * n + i] = S::make(0.0, 0.0);
+  }
+}
+
+// Reflector of column j (one workgroup per matrix), then its application to the
+// trailing columns (a wave per (matrix, column)).
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void qr_wide_reflect(T *at_all, T *tau_all, int m, int n, int k, int j) {
+  using S = Sc<T>;
+  __shared__ double scratch[LA_THREADS / 64];
+  T *col = at_all + ((size_t)blockIdx.x * n + j) * m;
+  T *tau = tau_all + (size_t)blockIdx.x * k;
+  double part = 0.0;
+  for (int i = j + 1 + threadIdx.x; i < m; i += blockDim.x) part += S::abs2(col[i]);
+  const double xnorm2 = block_sum(part, scratch);
+  const T alpha = col[j];
+  __syncthreads();
+  if (xnorm2 == 0.0) {
+    if (threadIdx.x == 0) tau[j] = S::make(0.0, 0.0);
+    return;
+  }
+  const double alphr = S::re(alpha), anorm = sqrt(S::abs2(alpha) + xnorm2);
+  const double beta = alphr >= 0.0 ? -anorm : anorm;
+  const T scal = alpha - S::make(beta, 0.0);
+  for (int i = j + 1 + threadIdx.x; i < m; i += blockDim.x) col[i] = col[i] / scal;
+  if (threadIdx.x == 0) {
+    col[j] = S::make(beta, 0.0);
+    tau[j] = S::make((beta - alphr) / beta, -S::im(alpha) / beta);
+  }
+}
+
+// X (column-major, `cols` columns of m rows per matrix) <- (I - t v v^H) X on the
+// columns from `first` on, v the reflector stored below the diagonal of column j
+// of At; t = conj(tau_j) while factoring, tau_j while forming Q.
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void qr_wide_apply(const T *at_all, const T *tau_all, T *x_all, int m, int n, int k, int j,
+                                                           int cols, int first, int conj_tau, int64_t waves_total) {
+  using S = Sc<T>;
+  const int lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= waves_total) return;
+  const int span = cols - first, c = first + (int)(item % span);
+  const int64_t b = item / span;
+  T t = tau_all[(size_t)b * k + j];
+  if (t == S::make(0.0, 0.0)) return;
+  if (conj_tau) t = S::conj(t);
+  const T *v = at_all + ((size_t)b * n + j) * m;
+  T *xc = x_all + ((size_t)b * cols + c) * m;
+  T w = lane == 0 ? xc[j] : S::make(0.0, 0.0);
+  for (int i = j + 1 + lane; i < m; i += 64) w = w + S::conj(v[i]) * xc[i];
+  w = t * wave_sum(w);
+  if (lane == 0) xc[j] = xc[j] - w;
+  for (int i = j + 1 + lane; i < m; i += 64) xc[i] = xc[i] - v[i] * w;
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void qr_wide_identity(T *qt_all, int m, int nq, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int64_t w = e % ((int64_t)m * nq);
+  qt_all[e] = (w / m) == (w % m) ? S::make(1.0, 0.0) : S::make(0.0, 0.0);
+}
+
+// R's zeros: below the diagonal of every matrix (where the reflectors were).
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void qr_wide_clear(T *at_all, int m, int n, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int i = (int)(e % m), c = (int)((e / m) % n);
+  if (i > c) at_all[e] = S::make(0.0, 0.0);
 }
 
 // conj in place (V^H from a column-major V; U'^H likewise)
@@ -827,6 +1136,148 @@ static int la_collect(nxh_context *ctx, const char *op) {
   return nxh_fail(NXH_FAILURE, op, LA_MESSAGES[code <= LA_NO_CONVERGE ? code : LA_NO_CONVERGE]);
 }
 
+// One int of device memory as it is once the queued work has run (a stream wait).
+static int la_read_int(nxh_context *ctx, const char *op, const int *dev, int *out) {
+  std::lock_guard<std::mutex> g(ctx->mu);
+  int *host = ctx->fault_flag_host + 2;
+  NXH_HIP(op, hipMemcpyAsync(host, dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+  NXH_HIP(op, hipStreamSynchronize(ctx->stream));
+  *out = *host;
+  return NXH_OK;
+}
+
+static inline unsigned la_blocks(int64_t items, int per_block = LA_THREADS) { return (unsigned)((items + per_block - 1) / per_block); }
+constexpr int LA_WIDE_FROM = 65;  // rows from which the Jacobi iterations run as device-wide launches
+
+template <class T>
+static int eigh_wide(nxh_context *ctx, const char *op, Work &work, int64_t batch, int n, int wantv, T *A, T *V, T *Vs, double *W) {
+  const int N = (n + 1) & ~1, P = N / 2;
+  const int64_t elems = batch * n * n, rots = batch * P, items = rots * n;
+  if (items / LA_THREADS > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  void *flags, *rc, *rs;
+  int rcode;
+  if ((rcode = work.get((size_t)(batch + 1) * sizeof(int), &flags)) || (rcode = work.get((size_t)rots * sizeof(double), &rc)) ||
+      (rcode = work.get((size_t)rots * sizeof(T), &rs)))
+    return rcode;
+  int *counter = (int *)flags, *done = counter + 1;
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    hipLaunchKernelGGL(la_fill_int, dim3(la_blocks(batch + 1)), dim3(LA_THREADS), 0, ctx->stream, counter, (int)(batch + 1), 0);
+    hipLaunchKernelGGL(eigh_wide_prepare<T>, dim3(la_blocks(elems)), dim3(LA_THREADS), 0, ctx->stream, A, V, n, wantv, elems);
+  }
+  bool converged = false;
+  for (int sweep = 0; sweep < 60 && !converged; sweep++) {
+    {
+      std::lock_guard<std::mutex> g(ctx->mu);
+      hipLaunchKernelGGL(la_fill_int, dim3(1), dim3(64), 0, ctx->stream, counter, 1, 0);
+      hipLaunchKernelGGL(eigh_wide_check<T>, dim3((unsigned)batch), dim3(LA_THREADS), 0, ctx->stream, (const T *)A, n, done, counter,
+                         la_status(ctx));
+    }
+    int remaining = 0;
+    if ((rcode = la_read_int(ctx, op, counter, &remaining))) return rcode;
+    if (remaining == 0) {
+      converged = true;
+      break;
+    }
+    std::lock_guard<std::mutex> g(ctx->mu);
+    for (int r = 0; r < N - 1; r++) {
+      hipLaunchKernelGGL(eigh_wide_params<T>, dim3(la_blocks(rots)), dim3(LA_THREADS), 0, ctx->stream, (const T *)A, (double *)rc,
+                         (T *)rs, (const int *)done, n, N, r, rots);
+      hipLaunchKernelGGL((eigh_wide_rotate<T, false>), dim3(la_blocks(items)), dim3(LA_THREADS), 0, ctx->stream, A, V,
+                         (const double *)rc, (const T *)rs, (const int *)done, n, N, r, wantv, items);
+      hipLaunchKernelGGL((eigh_wide_rotate<T, true>), dim3(la_blocks(items)), dim3(LA_THREADS), 0, ctx->stream, A, V,
+                         (const double *)rc, (const T *)rs, (const int *)done, n, N, r, wantv, items);
+    }
+    NXH_HIP(op, hipGetLastError());
+  }
+  if (!converged) return nxh_fail(NXH_FAILURE, op, LA_MESSAGES[LA_NO_CONVERGE]);
+  std::lock_guard<std::mutex> g(ctx->mu);
+  hipLaunchKernelGGL(eigh_wide_sort<T>, dim3((unsigned)batch), dim3(LA_THREADS), 0, ctx->stream, (const T *)A, (const T *)V, Vs, W, n,
+                     wantv);
+  return NXH_OK;
+}
+
+template <class T>
+static int svd_wide(nxh_context *ctx, const char *op, Work &work, int64_t batch, int mm, int nn, T *G, T *V, T *Gs, T *Vs) {
+  const int N = (nn + 1) & ~1, P = N / 2;
+  const int64_t pairs = batch * P, vcount = batch * nn * nn;
+  void *flags;
+  int rcode;
+  if ((rcode = work.get(sizeof(int), &flags))) return rcode;
+  int *counter = (int *)flags;
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    hipLaunchKernelGGL(svd_wide_init<T>, dim3(la_blocks(vcount)), dim3(LA_THREADS), 0, ctx->stream, V, nn, vcount);
+  }
+  bool converged = false;
+  for (int sweep = 0; sweep < 60 && !converged; sweep++) {
+    {
+      std::lock_guard<std::mutex> g(ctx->mu);
+      hipLaunchKernelGGL(la_fill_int, dim3(1), dim3(64), 0, ctx->stream, counter, 1, 0);
+      for (int r = 0; r < N - 1; r++)
+        hipLaunchKernelGGL(svd_wide_round<T>, dim3(la_blocks(pairs, LA_THREADS / 64)), dim3(LA_THREADS), 0, ctx->stream, G, V, mm, nn,
+                           N, r, pairs, counter);
+      NXH_HIP(op, hipGetLastError());
+    }
+    int rotated = 0;
+    if ((rcode = la_read_int(ctx, op, counter, &rotated))) return rcode;
+    converged = rotated == 0;
+  }
+  if (!converged) return nxh_fail(NXH_FAILURE, op, LA_MESSAGES[LA_NO_CONVERGE]);
+  std::lock_guard<std::mutex> g(ctx->mu);
+  hipLaunchKernelGGL(svd_wide_sort<T>, dim3((unsigned)batch), dim3(LA_THREADS), (size_t)nn * 8, ctx->stream, (const T *)G, (const T *)V,
+                     Gs, Vs, mm, nn);
+  return NXH_OK;
+}
+
+template <class T>
+static int cholesky_wide(nxh_context *ctx, const char *op, Work &work, int64_t batch, int n, int upper, T *A) {
+  void *diag;
+  if (int rc = work.get((size_t)(batch * n) * sizeof(double), &diag)) return rc;
+  std::lock_guard<std::mutex> g(ctx->mu);
+  for (int j = 0; j < n; j++) {
+    const int64_t waves = batch * (n - j);
+    hipLaunchKernelGGL(cholesky_wide_column<T>, dim3(la_blocks(waves, LA_THREADS / 64)), dim3(LA_THREADS), 0, ctx->stream, A,
+                       (double *)diag, n, j, waves, la_status(ctx));
+  }
+  const int64_t total = batch * n * n;
+  hipLaunchKernelGGL(cholesky_wide_finish<T>, dim3(la_blocks(total)), dim3(LA_THREADS), 0, ctx->stream, A, (const double *)diag, n,
+                     upper, total);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+// Householder QR of `batch` column-major m x n matrices At, Q's first nq columns to Qt.
+template <class T>
+static int run_qr(nxh_context *ctx, const char *op, int64_t batch, int m, int n, int nq, T *At, T *Qt, T *tau) {
+  std::lock_guard<std::mutex> g(ctx->mu);
+  if (std::max(m, n) < LA_WIDE_FROM) {
+    hipLaunchKernelGGL(qr_kernel<T>, dim3((unsigned)batch), dim3(LA_THREADS), 0, ctx->stream, At, Qt, tau, m, n, nq);
+    NXH_HIP(op, hipGetLastError());
+    return NXH_OK;
+  }
+  const int k = std::min(m, n), per = LA_THREADS / 64;
+  for (int j = 0; j < k; j++) {
+    hipLaunchKernelGGL(qr_wide_reflect<T>, dim3((unsigned)batch), dim3(LA_THREADS), 0, ctx->stream, At, tau, m, n, k, j);
+    const int64_t waves = batch * (n - j - 1);
+    if (waves > 0)
+      hipLaunchKernelGGL(qr_wide_apply<T>, dim3(la_blocks(waves, per)), dim3(LA_THREADS), 0, ctx->stream, (const T *)At, (const T *)tau,
+                         At, m, n, k, j, n, j + 1, 1, waves);
+  }
+  const int64_t qcount = batch * m * nq;
+  if (qcount > 0) hipLaunchKernelGGL(qr_wide_identity<T>, dim3(la_blocks(qcount)), dim3(LA_THREADS), 0, ctx->stream, Qt, m, nq, qcount);
+  for (int j = k - 1; j >= 0; j--) {
+    const int64_t waves = batch * (nq - j);
+    if (waves > 0)
+      hipLaunchKernelGGL(qr_wide_apply<T>, dim3(la_blocks(waves, per)), dim3(LA_THREADS), 0, ctx->stream, (const T *)At, (const T *)tau,
+                         Qt, m, n, k, j, nq, j, 0, waves);
+  }
+  const int64_t acount = batch * m * n;
+  if (acount > 0) hipLaunchKernelGGL(qr_wide_clear<T>, dim3(la_blocks(acount)), dim3(LA_THREADS), 0, ctx->stream, At, m, n, acount);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
 struct Problem {
   int64_t batch, rows, cols;
   bool cx;
@@ -858,6 +1309,13 @@ static int same_dims(const char *op, const nxh_tensor *t, const nxh_tensor *like
   return NXH_OK;
 }
 
+// The casts that carry operands in and results out report their own paths: the
+// factorisation's is set last.
+struct PathAtExit {
+  const char *name;
+  ~PathAtExit() { nxh_set_path(name); }
+};
+
 #define LA_LAUNCH(ctx, kernel, blocks, lds, ...)                                                        \
   do {                                                                                                  \
     std::lock_guard<std::mutex> g_((ctx)->mu);                                                          \
@@ -884,9 +1342,16 @@ NXH_EXPORT int nxh_cholesky(nxh_context *ctx, const nxh_tensor *out, const nxh_t
   if ((rc = work.get((size_t)(p.batch * n * n) * p.esize, &A))) return rc;
   nxh_tensor wa = workspace_tensor(x, A, p.wdt, n, n, false);
   if ((rc = nxh_cast(ctx, &wa, x))) return rc;
-  nxh_set_path("cholesky_columns");
-  if (p.cx) LA_LAUNCH(ctx, cholesky_kernel<c64>, p.batch, 0, (c64 *)A, (int)n, upper, la_status(ctx));
-  else LA_LAUNCH(ctx, cholesky_kernel<double>, p.batch, 0, (double *)A, (int)n, upper, la_status(ctx));
+  PathAtExit path{n >= LA_WIDE_FROM ? "cholesky_columns_wide" : "cholesky_columns"};
+  if (n >= LA_WIDE_FROM) {
+    rc = p.cx ? cholesky_wide<c64>(ctx, op, work, p.batch, (int)n, upper, (c64 *)A)
+              : cholesky_wide<double>(ctx, op, work, p.batch, (int)n, upper, (double *)A);
+    if (rc) return rc;
+  } else if (p.cx) {
+    LA_LAUNCH(ctx, cholesky_kernel<c64>, p.batch, 0, (c64 *)A, (int)n, upper, la_status(ctx));
+  } else {
+    LA_LAUNCH(ctx, cholesky_kernel<double>, p.batch, 0, (double *)A, (int)n, upper, la_status(ctx));
+  }
   if ((rc = la_collect(ctx, op))) return rc;
   return nxh_cast(ctx, out, &wa);
 }
@@ -916,7 +1381,7 @@ NXH_EXPORT int nxh_triangular_solve(nxh_context *ctx, const nxh_tensor *out, con
   nxh_tensor wa = workspace_tensor(a, A, p.wdt, n, n, false);
   nxh_tensor wx = workspace_tensor(b, X, p.wdt, n, nrhs, false);
   if ((rc = nxh_cast(ctx, &wa, a)) || (rc = nxh_cast(ctx, &wx, b))) return rc;
-  nxh_set_path("triangular_substitution");
+  PathAtExit path{"triangular_substitution"};
   const int up = flags & 1, tr = (flags >> 1) & 1, unit = (flags >> 2) & 1;
   if (p.cx) LA_LAUNCH(ctx, trsm_kernel<c64>, p.batch, 0, (const c64 *)A, (c64 *)X, (int)n, (int)nrhs, up, tr, unit, la_status(ctx));
   else LA_LAUNCH(ctx, trsm_kernel<double>, p.batch, 0, (const double *)A, (double *)X, (int)n, (int)nrhs, up, tr, unit, la_status(ctx));
@@ -950,9 +1415,10 @@ NXH_EXPORT int nxh_qr(nxh_context *ctx, const nxh_tensor *q, const nxh_tensor *r
   if ((rc = work.get((size_t)(p.batch * k) * p.esize, &tau))) return rc;
   nxh_tensor wa = workspace_tensor(x, At, p.wdt, m, n, true);
   if (n > 0 && (rc = nxh_cast(ctx, &wa, x))) return rc;
-  nxh_set_path("qr_householder");
-  if (p.cx) LA_LAUNCH(ctx, qr_kernel<c64>, p.batch, 0, (c64 *)At, (c64 *)Qt, (c64 *)tau, (int)m, (int)n, (int)nq);
-  else LA_LAUNCH(ctx, qr_kernel<double>, p.batch, 0, (double *)At, (double *)Qt, (double *)tau, (int)m, (int)n, (int)nq);
+  PathAtExit path{std::max(m, n) >= LA_WIDE_FROM ? "qr_householder_wide" : "qr_householder"};
+  rc = p.cx ? run_qr<c64>(ctx, op, p.batch, (int)m, (int)n, (int)nq, (c64 *)At, (c64 *)Qt, (c64 *)tau)
+            : run_qr<double>(ctx, op, p.batch, (int)m, (int)n, (int)nq, (double *)At, (double *)Qt, (double *)tau);
+  if (rc) return rc;
   nxh_tensor wq = workspace_tensor(x, Qt, p.wdt, m, nq, true);
   if ((rc = nxh_cast(ctx, q, &wq))) return rc;
   if (n == 0 || rr == 0) return NXH_OK;
@@ -987,10 +1453,17 @@ NXH_EXPORT int nxh_eigh(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor 
   if (v && ((rc = work.get(mat, &V)) || (rc = work.get(mat, &Vs)))) return rc;
   nxh_tensor wa = workspace_tensor(x, A, p.wdt, n, n, false);
   if ((rc = nxh_cast(ctx, &wa, x))) return rc;
-  nxh_set_path("eigh_jacobi");
+  PathAtExit path{n >= LA_WIDE_FROM ? "eigh_jacobi_wide" : "eigh_jacobi"};
   const size_t lds = (size_t)((n + 1) / 2) * (8 + p.esize);
-  if (p.cx) LA_LAUNCH(ctx, eigh_kernel<c64>, p.batch, lds, (c64 *)A, (c64 *)V, (c64 *)Vs, (double *)W, (int)n, v ? 1 : 0, la_status(ctx));
-  else LA_LAUNCH(ctx, eigh_kernel<double>, p.batch, lds, (double *)A, (double *)V, (double *)Vs, (double *)W, (int)n, v ? 1 : 0, la_status(ctx));
+  if (n >= LA_WIDE_FROM) {
+    rc = p.cx ? eigh_wide<c64>(ctx, op, work, p.batch, (int)n, v ? 1 : 0, (c64 *)A, (c64 *)V, (c64 *)Vs, (double *)W)
+              : eigh_wide<double>(ctx, op, work, p.batch, (int)n, v ? 1 : 0, (double *)A, (double *)V, (double *)Vs, (double *)W);
+    if (rc) return rc;
+  } else if (p.cx) {
+    LA_LAUNCH(ctx, eigh_kernel<c64>, p.batch, lds, (c64 *)A, (c64 *)V, (c64 *)Vs, (double *)W, (int)n, v ? 1 : 0, la_status(ctx));
+  } else {
+    LA_LAUNCH(ctx, eigh_kernel<double>, p.batch, lds, (double *)A, (double *)V, (double *)Vs, (double *)W, (int)n, v ? 1 : 0, la_status(ctx));
+  }
   if ((rc = la_collect(ctx, op))) return rc;
   nxh_tensor ww = workspace_tensor(x, W, NXH_F64, n, 0, false, 1);
   if ((rc = nxh_cast(ctx, w, &ww))) return rc;
@@ -1039,20 +1512,27 @@ NXH_EXPORT int nxh_svd(nxh_context *ctx, const nxh_tensor *u, const nxh_tensor *
   // column-major G of x is x's row-major transpose; of x^H it is conj(x) laid out row-major
   nxh_tensor wg = flip ? workspace_tensor(x, G, p.wdt, m, n, false) : workspace_tensor(x, G, p.wdt, m, n, true);
   if ((rc = nxh_cast(ctx, &wg, x))) return rc;
-  nxh_set_path("svd_jacobi");
+  PathAtExit path{std::min(m, n) >= LA_WIDE_FROM ? "svd_jacobi_wide" : "svd_jacobi"};
   const int64_t gcount = p.batch * mm * nn;
   if (flip && p.cx) {
     std::lock_guard<std::mutex> g_(ctx->mu);
     hipLaunchKernelGGL(conj_kernel<c64>, dim3((unsigned)((gcount + 255) / 256)), dim3(256), 0, ctx->stream, (c64 *)G, gcount);
   }
   const size_t lds = (size_t)nn * 8;
+  if (nn >= LA_WIDE_FROM) {
+    rc = p.cx ? svd_wide<c64>(ctx, op, work, p.batch, (int)mm, (int)nn, (c64 *)G, (c64 *)V, (c64 *)Gs, (c64 *)Vs)
+              : svd_wide<double>(ctx, op, work, p.batch, (int)mm, (int)nn, (double *)G, (double *)V, (double *)Gs, (double *)Vs);
+    if (rc) return rc;
+  }
   if (p.cx) {
-    LA_LAUNCH(ctx, svd_jacobi_kernel<c64>, p.batch, lds, (c64 *)G, (c64 *)V, (c64 *)Gs, (c64 *)Vs, (int)mm, (int)nn, la_status(ctx));
-    LA_LAUNCH(ctx, qr_kernel<c64>, p.batch, 0, (c64 *)Gs, (c64 *)Qt, (c64 *)tau, (int)mm, (int)nn, (int)nq);
+    if (nn < LA_WIDE_FROM)
+      LA_LAUNCH(ctx, svd_jacobi_kernel<c64>, p.batch, lds, (c64 *)G, (c64 *)V, (c64 *)Gs, (c64 *)Vs, (int)mm, (int)nn, la_status(ctx));
+    if ((rc = run_qr<c64>(ctx, op, p.batch, (int)mm, (int)nn, (int)nq, (c64 *)Gs, (c64 *)Qt, (c64 *)tau))) return rc;
     LA_LAUNCH(ctx, svd_finish_kernel<c64>, p.batch, 0, (const c64 *)Gs, (c64 *)Qt, (double *)S, (int)mm, (int)nn, (int)nq);
   } else {
-    LA_LAUNCH(ctx, svd_jacobi_kernel<double>, p.batch, lds, (double *)G, (double *)V, (double *)Gs, (double *)Vs, (int)mm, (int)nn, la_status(ctx));
-    LA_LAUNCH(ctx, qr_kernel<double>, p.batch, 0, (double *)Gs, (double *)Qt, (double *)tau, (int)mm, (int)nn, (int)nq);
+    if (nn < LA_WIDE_FROM)
+      LA_LAUNCH(ctx, svd_jacobi_kernel<double>, p.batch, lds, (double *)G, (double *)V, (double *)Gs, (double *)Vs, (int)mm, (int)nn, la_status(ctx));
+    if ((rc = run_qr<double>(ctx, op, p.batch, (int)mm, (int)nn, (int)nq, (double *)Gs, (double *)Qt, (double *)tau))) return rc;
     LA_LAUNCH(ctx, svd_finish_kernel<double>, p.batch, 0, (const double *)Gs, (double *)Qt, (double *)S, (int)mm, (int)nn, (int)nq);
   }
   if ((rc = la_collect(ctx, op))) return rc;
@@ -1106,7 +1586,7 @@ NXH_EXPORT int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *
   if (v && ((rc = work.get(mat, &Q)) || (rc = work.get(mat, &Y)) || (rc = work.get(mat, &V)))) return rc;
   nxh_tensor wh = workspace_tensor(x, H, NXH_C64, n, n, false);
   if ((rc = nxh_cast(ctx, &wh, x))) return rc;
-  nxh_set_path("eig_hessenberg_qr");
+  PathAtExit path{"eig_hessenberg_qr"};
   LA_LAUNCH(ctx, eig_kernel, p.batch, (size_t)n * 24, (c64 *)H, (c64 *)Q, (c64 *)Y, (c64 *)W, (c64 *)V, (int)n, v ? 1 : 0, la_status(ctx));
   if ((rc = la_collect(ctx, op))) return rc;
   nxh_tensor ww = workspace_tensor(x, W, NXH_C64, n, 0, false, 1);

@@ -129,12 +129,13 @@ def test_qr(hip, oracle, name):
 def test_eigh_and_eigvalsh(hip, oracle, name):
     d, tol = DTYPES[name], TOL[name] * 20
     rng = np.random.default_rng(4)
-    for batch, n in (((), 1), ((), 2), ((), 3), ((2,), 4), ((3,), 17), ((), 64), ((), 129)):
+    for batch, n in (((), 1), ((), 2), ((), 3), ((2,), 4), ((3,), 17), ((), 64), ((), 129), ((3,), 70)):
         g = matrix(rng, batch + (n, n), d)
         a = (g + H(g)).astype(d.np_storage)
         a[..., 0, n - 1] = 55 if n > 1 else a[..., 0, 0]  # the upper triangle is not read (nx_c_eigh.c:14)
         h, o = both(hip, oracle, a, d)
         w, v = hip.eigh(h)
+        assert hip.last_path() == ("eigh_jacobi_wide" if n > 64 else "eigh_jacobi")
         ow, _ = oracle.eigh(o)
         w, v, ow = logical(w), arr(v), logical(ow)
         assert w.dtype == np.float64 and w.shape == batch + (n,)
@@ -154,7 +155,8 @@ def test_eigh_and_eigvalsh(hip, oracle, name):
 def test_svd(hip, oracle, name):
     d, tol = DTYPES[name], TOL[name] * 20
     rng = np.random.default_rng(5)
-    cases = [((), 4, 3), ((), 3, 4), ((2,), 16, 16), ((3,), 40, 7), ((), 9, 70), ((), 1, 1), ((), 100, 100)]
+    cases = [((), 4, 3), ((), 3, 4), ((2,), 16, 16), ((3,), 40, 7), ((), 9, 70), ((), 1, 1), ((), 100, 100),
+             ((2,), 90, 75), ((2,), 67, 130)]
     for batch, m, n in cases:
         a = matrix(rng, batch + (m, n), d)
         if m == 16:
