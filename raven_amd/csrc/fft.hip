@@ -13,7 +13,7 @@
 //
 // How it runs here: one axis pass = one launch in which a workgroup owns one
 // line (or several short ones), loads it strided into LDS as double2, does all
-// radix-2 stages there and stores it strided, so a pass reads and writes the
+// radix-2 stages there (two at a time, four elements per lane in registers) and stores it strided, so a pass reads and writes the
 // tensor exactly once. Lengths that are not a power of two go through Bluestein's
 // identity inside the same kernel: chirp on load, a power-of-two convolution of
 // length M >= 2n-1 (forward DIF, multiply by the transformed chirp filter in
@@ -117,8 +117,11 @@ __device__ __forceinline__ double2 fetch(const FftArgs &a, int64_t off, int j) {
 // One radix-2 butterfly stage over the G lines of the workgroup. `s` is the
 // stage (sub-transform length 2^s). DIT: input bit-reversed, output natural.
 // DIF: input natural, output bit-reversed.
+// The twiddle table stays in global memory (it is small and cache-resident): the
+// stages are bound by LDS bandwidth, and a copy of the table in LDS measured slower.
 template <bool DIF>
 __device__ __forceinline__ void stage(double2 *lds, const FftArgs &a, int s, int sign) {
+  const double2 *tw = a.tw;
   const int half = 1 << (s - 1);
   const int per_line = a.M >> 1;
   const int total = a.G * per_line;
@@ -128,7 +131,7 @@ __device__ __forceinline__ void stage(double2 *lds, const FftArgs &a, int s, int
     const int pos = r & (half - 1);
     const int i = (g << a.logM) + ((r >> (s - 1)) << s) + pos;
     const int j = i + half;
-    double2 w = a.tw[pos << (a.logM - s)];
+    double2 w = tw[pos << (a.logM - s)];
     if (sign > 0) w.y = -w.y;
     const double2 u = lds[i], v = lds[j];
     if (DIF) {
@@ -141,6 +144,82 @@ __device__ __forceinline__ void stage(double2 *lds, const FftArgs &a, int s, int
     }
   }
   __syncthreads();
+}
+
+// Stages s and s + 1 in one pass: a lane holds the four elements h = 2^(s-1)
+// apart in registers and does both butterflies of each, so the lines go through
+// LDS once for two stages. The arithmetic per element is that of two calls of
+// `stage`, in the same order.
+template <bool DIF>
+__device__ __forceinline__ void stage_pair(double2 *lds, const FftArgs &a, int s, int sign) {
+  const double2 *tw = a.tw;
+  const int h = 1 << (s - 1);
+  const int per_line = a.M >> 2;
+  const int total = a.G * per_line;
+  auto add = [](double2 u, double2 v) { return make_double2(u.x + v.x, u.y + v.y); };
+  auto sub = [](double2 u, double2 v) { return make_double2(u.x - v.x, u.y - v.y); };
+  for (int b = threadIdx.x; b < total; b += blockDim.x) {
+    const int g = b >> (a.logM - 2);
+    const int r = b & (per_line - 1);
+    const int pos = r & (h - 1);
+    const int i0 = (g << a.logM) + ((r >> (s - 1)) << (s + 1)) + pos;
+    const int i1 = i0 + h, i2 = i0 + 2 * h, i3 = i0 + 3 * h;
+    double2 w1 = tw[pos << (a.logM - s)], w2 = tw[pos << (a.logM - s - 1)], w3 = tw[(pos + h) << (a.logM - s - 1)];
+    if (sign > 0) {
+      w1.y = -w1.y;
+      w2.y = -w2.y;
+      w3.y = -w3.y;
+    }
+    double2 x0 = lds[i0], x1 = lds[i1], x2 = lds[i2], x3 = lds[i3];
+    if (DIF) {
+      double2 u = x0, v = x2;
+      x0 = add(u, v);
+      x2 = cmul(sub(u, v), w2);
+      u = x1, v = x3;
+      x1 = add(u, v);
+      x3 = cmul(sub(u, v), w3);
+      u = x0, v = x1;
+      x0 = add(u, v);
+      x1 = cmul(sub(u, v), w1);
+      u = x2, v = x3;
+      x2 = add(u, v);
+      x3 = cmul(sub(u, v), w1);
+    } else {
+      double2 t = cmul(w1, x1), u = x0;
+      x0 = add(u, t);
+      x1 = sub(u, t);
+      t = cmul(w1, x3), u = x2;
+      x2 = add(u, t);
+      x3 = sub(u, t);
+      t = cmul(w2, x2), u = x0;
+      x0 = add(u, t);
+      x2 = sub(u, t);
+      t = cmul(w3, x3), u = x1;
+      x1 = add(u, t);
+      x3 = sub(u, t);
+    }
+    lds[i0] = x0;
+    lds[i1] = x1;
+    lds[i2] = x2;
+    lds[i3] = x3;
+  }
+  __syncthreads();
+}
+
+// All stages of the lines in LDS. DIT runs the stages upwards (bit-reversed in,
+// natural out), DIF downwards (natural in, bit-reversed out); an odd count starts
+// with one single stage.
+template <bool DIF>
+__device__ __forceinline__ void all_stages(double2 *lds, const FftArgs &a, int sign) {
+  if (DIF) {
+    int s = a.logM;
+    if (s & 1) stage<true>(lds, a, s--, sign);
+    for (; s >= 2; s -= 2) stage_pair<true>(lds, a, s - 1, sign);
+  } else {
+    int s = 1;
+    if (a.logM & 1) stage<false>(lds, a, s++, sign);
+    for (; s + 1 <= a.logM; s += 2) stage_pair<false>(lds, a, s, sign);
+  }
 }
 
 template <bool BLUE>
@@ -173,16 +252,16 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
   }
   __syncthreads();
   if (BLUE) {
-    for (int s = a.logM; s >= 1; s--) stage<true>(lds, a, s, -1);
+    all_stages<true>(lds, a, -1);
     for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
       const int p = idx & (a.M - 1);
       const int k = a.logM == 0 ? 0 : (int)(__brev((unsigned)p) >> shift);
       lds[idx] = cmul(lds[idx], a.bf[k]);
     }
     __syncthreads();
-    for (int s = 1; s <= a.logM; s++) stage<false>(lds, a, s, +1);
+    all_stages<false>(lds, a, +1);
   } else {
-    for (int s = 1; s <= a.logM; s++) stage<false>(lds, a, s, a.sign);
+    all_stages<false>(lds, a, a.sign);
   }
   const double inv_m = 1.0 / (double)a.M;
   const int stores = a.G * a.n_store;
