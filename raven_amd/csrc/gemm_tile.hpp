@@ -90,6 +90,10 @@ struct Shape {
   // staged 16-byte vectors per lane and slab: rows x 8 vectors / THREADS
   static constexpr int NVA = BM * 8 / THREADS, NVB = BN * 8 / THREADS;
   static_assert(NVA >= 1 && NVB >= 1 && NVA * THREADS == BM * 8 && NVB * THREADS == BN * 8, "staging");
+  // Two blocks of a four-wave shape fit a compute unit's LDS; they also fit its register
+  // file when a wave stays within 256 registers (accumulators included), which the
+  // kernel asks the compiler for: the second block hides the first one's load latency.
+  static constexpr int WAVES_PER_SIMD = THREADS <= 256 ? 2 : 1;
   template <class EL>
   static constexpr int a_elems() { return Geo<EL>::tile_elems(BM); }
   template <class EL>
@@ -211,7 +215,7 @@ __device__ __forceinline__ void tile_of_block(const Args &a, uint32_t bid, uint3
 }
 
 template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI = false>
-__global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
+__global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH::WAVES_PER_SIMD))) void kernel(Args a) {
   constexpr int THREADS = SH::THREADS, BM = SH::BM, BN = SH::BN, TM = SH::TM, TN = SH::TN;
   constexpr int NVA = SH::NVA, NVB = SH::NVB, BK = Geo<EL>::BK;
   constexpr int A_ELEMS = SH::template a_elems<EL>(), STAGE_ELEMS = SH::template stage_elems<EL>();

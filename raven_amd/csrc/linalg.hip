@@ -673,6 +673,42 @@ __global__ void la_fill_int(int *p, int count, int value) {
   if (i < count) p[i] = value;
 }
 
+// ── triangular solve over the whole device ──────────────────────────────────
+// Row i of the solution (one launch), then its elimination from the rows not yet
+// solved (another), for every matrix and right-hand side at once.
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void trsm_wide_scale(const T *a_all, T *x_all, int n, int nrhs, int i, int transpose,
+                                                             int64_t total, int *status) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int64_t b = e / nrhs;
+  const int j = (int)(e % nrhs);
+  T diag = a_all[(size_t)b * n * n + (size_t)i * n + i];
+  if (transpose) diag = S::conj(diag);
+  if (diag == S::make(0.0, 0.0)) {
+    if (j == 0) raise(status, LA_SINGULAR);
+    return;
+  }
+  T *x = x_all + (size_t)b * n * nrhs + (size_t)i * nrhs + j;
+  *x = *x / diag;
+}
+
+template <class T>
+__global__ __launch_bounds__(LA_THREADS) void trsm_wide_eliminate(const T *a_all, T *x_all, int n, int nrhs, int i, int rest,
+                                                                 int forward, int transpose, int64_t total) {
+  using S = Sc<T>;
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const int j = (int)(e % nrhs), rr = (int)((e / nrhs) % rest);
+  const int64_t b = e / ((int64_t)nrhs * rest);
+  const int r = forward ? i + 1 + rr : i - 1 - rr;
+  const T *A = a_all + (size_t)b * n * n;
+  T *X = x_all + (size_t)b * n * nrhs;
+  const T m = transpose ? S::conj(A[(size_t)i * n + r]) : A[(size_t)r * n + i];
+  X[(size_t)r * nrhs + j] = X[(size_t)r * nrhs + j] - m * X[(size_t)i * nrhs + j];
+}
+
 // ── cholesky and qr over the whole device ───────────────────────────────────
 // Column j of every matrix in one launch, a wave per (matrix, row >= j): the
 // lanes split the dot product along the finished columns (contiguous in the
@@ -1231,6 +1267,25 @@ static int svd_wide(nxh_context *ctx, const char *op, Work &work, int64_t batch,
 }
 
 template <class T>
+static int trsm_wide(nxh_context *ctx, const char *op, int64_t batch, int n, int nrhs, int upper, int transpose, int unit, const T *A,
+                     T *X) {
+  const int forward = (upper != 0) == (transpose != 0);
+  std::lock_guard<std::mutex> g(ctx->mu);
+  for (int ii = 0; ii < n; ii++) {
+    const int i = forward ? ii : n - 1 - ii, rest = n - 1 - ii;
+    if (!unit)
+      hipLaunchKernelGGL(trsm_wide_scale<T>, dim3(la_blocks(batch * nrhs)), dim3(LA_THREADS), 0, ctx->stream, A, X, n, nrhs, i,
+                         transpose, batch * nrhs, la_status(ctx));
+    const int64_t items = batch * rest * nrhs;
+    if (items > 0)
+      hipLaunchKernelGGL(trsm_wide_eliminate<T>, dim3(la_blocks(items)), dim3(LA_THREADS), 0, ctx->stream, A, X, n, nrhs, i, rest,
+                         forward, transpose, items);
+  }
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
+template <class T>
 static int cholesky_wide(nxh_context *ctx, const char *op, Work &work, int64_t batch, int n, int upper, T *A) {
   void *diag;
   if (int rc = work.get((size_t)(batch * n) * sizeof(double), &diag)) return rc;
@@ -1381,9 +1436,14 @@ NXH_EXPORT int nxh_triangular_solve(nxh_context *ctx, const nxh_tensor *out, con
   nxh_tensor wa = workspace_tensor(a, A, p.wdt, n, n, false);
   nxh_tensor wx = workspace_tensor(b, X, p.wdt, n, nrhs, false);
   if ((rc = nxh_cast(ctx, &wa, a)) || (rc = nxh_cast(ctx, &wx, b))) return rc;
-  PathAtExit path{"triangular_substitution"};
+  PathAtExit path{n >= LA_WIDE_FROM ? "triangular_substitution_wide" : "triangular_substitution"};
   const int up = flags & 1, tr = (flags >> 1) & 1, unit = (flags >> 2) & 1;
-  if (p.cx) LA_LAUNCH(ctx, trsm_kernel<c64>, p.batch, 0, (const c64 *)A, (c64 *)X, (int)n, (int)nrhs, up, tr, unit, la_status(ctx));
+  if (n >= LA_WIDE_FROM) {
+    if (p.batch * n * nrhs / LA_THREADS > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+    rc = p.cx ? trsm_wide<c64>(ctx, op, p.batch, (int)n, (int)nrhs, up, tr, unit, (const c64 *)A, (c64 *)X)
+              : trsm_wide<double>(ctx, op, p.batch, (int)n, (int)nrhs, up, tr, unit, (const double *)A, (double *)X);
+    if (rc) return rc;
+  } else if (p.cx) LA_LAUNCH(ctx, trsm_kernel<c64>, p.batch, 0, (const c64 *)A, (c64 *)X, (int)n, (int)nrhs, up, tr, unit, la_status(ctx));
   else LA_LAUNCH(ctx, trsm_kernel<double>, p.batch, 0, (const double *)A, (double *)X, (int)n, (int)nrhs, up, tr, unit, la_status(ctx));
   if ((rc = la_collect(ctx, op))) return rc;
   return nxh_cast(ctx, out, &wx);
