@@ -209,3 +209,91 @@ def test_random_views_at_fast_path_sizes(hip, oracle, seed):
         axis = int(rng.integers(0, r))
         for name in ("sum", "max"):
             eq(hip.associative_scan(axis, name, ha), oracle.associative_scan(axis, name, oa))
+
+
+def build_float_operand(rng, hip, oracle, d, target):
+    """build_operand for the float and complex dtypes of the transforms and factorisations."""
+    r = len(target)
+    perm = rng.permutation(r)
+    pad_lo = [int(rng.integers(0, 3)) for _ in range(r)]
+    pad_hi = [int(rng.integers(0, 3)) for _ in range(r)]
+    flip = [bool(rng.random() < 0.3) for _ in range(r)]
+    src = [target[i] + pad_lo[i] + pad_hi[i] for i in range(r)]
+    stored = [src[p] for p in perm]
+    x = rng.standard_normal(stored)
+    if d.is_complex:
+        x = x + 1j * rng.standard_normal(stored)
+    x = x.astype(d.np_storage)
+    inv = np.argsort(perm)
+
+    def view(B):
+        t = B.reshape(B.from_host(np.ascontiguousarray(x), d), tuple(stored))
+        t = B.permute(t, [int(i) for i in inv])
+        t = B.shrink(t, [(pad_lo[i], pad_lo[i] + target[i]) for i in range(r)])
+        return B.flip(t, flip)
+
+    return view(hip), view(oracle)
+
+
+@pytest.mark.parametrize("seed", list(range(120)))
+def test_random_views_transforms_and_factorisations(hip, oracle, seed):
+    """fft family and the unique parts of the factorisations on permuted, sliced
+    and flipped operands: a wrong stride or offset in how lines and matrices are
+    addressed shows as an error far above rounding."""
+    rng = np.random.default_rng(11000 + seed)
+    op = ["fft", "ifft", "rfft", "irfft", "qr", "eigvalsh", "svd", "cholesky", "solve"][seed % 9]
+    single = bool(rng.integers(0, 2))
+    cd, rd = (dt.complex64, dt.float32) if single else (dt.complex128, dt.float64)
+    tol = 2e-4 if single else 1e-9
+    r = int(rng.integers(2, 5))
+    target = [int(rng.choice([1, 2, 3, 5, 8, 12, 16, 17, 33])) for _ in range(r)]
+    what = f"seed {seed}: {op} {'single' if single else 'double'} {target}"
+
+    def close(g, w):
+        g, w = logical(g).astype(np.complex128), logical(w).astype(np.complex128)
+        assert g.shape == w.shape, what
+        assert np.max(np.abs(g - w), initial=0.0) <= tol * max(1.0, np.max(np.abs(w), initial=0.0)) * max(target), what
+
+    if op in ("fft", "ifft"):
+        h, o = build_float_operand(rng, hip, oracle, cd, target)
+        axes = [int(a) for a in rng.choice(r, size=int(rng.integers(1, r + 1)), replace=False)]
+        close(hip.fft(h, axes, op == "ifft"), oracle.fft(o, axes, op == "ifft"))
+    elif op == "rfft":
+        h, o = build_float_operand(rng, hip, oracle, rd, target)
+        axes = [int(a) for a in rng.choice(r, size=int(rng.integers(1, 3)), replace=False)]
+        close(hip.rfft(h, cd, axes), oracle.rfft(o, cd, axes))
+    elif op == "irfft":
+        h, o = build_float_operand(rng, hip, oracle, cd, target)
+        axes = [int(a) for a in rng.choice(r, size=int(rng.integers(1, 3)), replace=False)]
+        sizes = [target[a] for a in axes]
+        sizes[-1] = int(rng.integers(1, 2 * target[axes[-1]] + 2))
+        close(hip.irfft(h, rd, axes, sizes), oracle.irfft(o, rd, axes, sizes))
+    else:
+        d = cd if rng.integers(0, 2) else rd
+        if op in ("eigvalsh", "cholesky", "solve"):
+            target[-1] = target[-2]
+        h, o = build_float_operand(rng, hip, oracle, d, target)
+        if op == "qr":
+            reduced = bool(rng.integers(0, 2))
+            for g, w in zip(hip.qr(h, reduced), oracle.qr(o, reduced)):
+                k = min(target[-2:])
+                close(hip.shrink(g, [(0, s) for s in g.shape[:-1]] + [(0, min(k, g.shape[-1]))]) if g.shape[-1] > k else g,
+                      oracle.shrink(w, [(0, s) for s in w.shape[:-1]] + [(0, min(k, w.shape[-1]))]) if w.shape[-1] > k else w)
+        elif op == "eigvalsh":
+            close(hip.eigvalsh(h), oracle.eigvalsh(o))
+        elif op == "svd":
+            close(hip.svd(h)[1], oracle.svd(o)[1])
+        else:
+            # a diagonally dominant matrix from the same view: add n * I on both sides
+            n = target[-1]
+            eye = np.broadcast_to(np.eye(n) * (4.0 * n), tuple(target)).astype(d.np_storage)
+            he = hip.reshape(hip.from_host(np.ascontiguousarray(eye), d), tuple(target))
+            oe = oracle.reshape(oracle.from_host(np.ascontiguousarray(eye), d), tuple(target))
+            if op == "cholesky":
+                # Hermitian part of the lower triangle is what is read; make it dominant
+                close(hip.cholesky(hip.binary("add", h, he)), oracle.cholesky(oracle.binary("add", o, oe)))
+            else:
+                hb, ob = build_float_operand(rng, hip, oracle, d, target[:-1] + [int(rng.integers(1, 6))])
+                flags = [bool(rng.integers(0, 2)) for _ in range(3)]
+                close(hip.triangular_solve(hip.binary("add", h, he), hb, *flags),
+                      oracle.triangular_solve(oracle.binary("add", o, oe), ob, *flags))
