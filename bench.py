@@ -606,6 +606,23 @@ def main():
     ms_per_step = wall_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    # the same step recorded once and replayed: what the launch gaps between the seven calls cost
+    hip.capture_begin()
+    try:
+        for op in step_ops:
+            op()
+    finally:
+        recorded = hip.capture_end()
+    for _ in range(args.warmup):
+        recorded.launch()
+    hip.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        recorded.launch()
+    hip.synchronize()
+    replay_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    recorded.destroy()
+
     # parity of what was just timed, against the oracle on the same seeded inputs
     cpu, parity = None, None
     if not args.no_cpu:
@@ -664,7 +681,11 @@ def main():
                                "mul scalar, cast f16) and int32 (add, mul, cmplt, where); 7 backend calls per step",
                    "algorithmic_bytes_per_step": step_bytes, "device": info["name"].strip(),
                    "compute_units": info["compute_units"], "hip_event_ms_per_step": round(ev_ms / args.steps, 5),
-                   "frac_of_hbm_peak": round(value / PEAK_HBM_GBS, 4), "parity_vs_oracle": parity},
+                   "frac_of_hbm_peak": round(value / PEAK_HBM_GBS, 4), "parity_vs_oracle": parity,
+                   "graph_replay": {"ms_per_step": round(replay_ms, 5),
+                                    "GB/s": round(step_bytes / (replay_ms * 1e-3) / 1e9, 1),
+                                    "note": "the step recorded with nxh_capture_begin/_end and replayed with "
+                                            "nxh_graph_launch; not the headline value"}},
         "roofline": roofline, "cpu_baseline": cpu, "ops": ops_out,
     }
     print(json.dumps(line))

@@ -573,7 +573,10 @@ __global__ __launch_bounds__(LA_THREADS) void eigh_wide_rotate(T *a_all, T *v_al
   const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (e >= total) return;
   const int P = N / 2;
-  const int i = (int)(e % n), t = (int)((e / n) % P);
+  // rows: neighbouring lanes take neighbouring columns i of the row pair. Columns:
+  // neighbouring lanes take the pairs of one row i, which together cover that row
+  // exactly once (a lane per row would stride the whole matrix)
+  const int i = ROWS ? (int)(e % n) : (int)((e / P) % n), t = ROWS ? (int)((e / n) % P) : (int)(e % P);
   const int64_t b = e / ((int64_t)n * P);
   if (done[b]) return;
   int p, q;
