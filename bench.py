@@ -194,7 +194,7 @@ class Workloads:
         return ops
 
 
-def next_ops(hip, W):
+def next_ops(hip, W, linalg=False):
     """The operations beside the named hot path (pad, cat, scan, threefry,
     scatter, sort, unfold, fold), timed through the Python mirror with HIP events."""
     rng = np.random.default_rng(20)
@@ -296,7 +296,11 @@ def next_ops(hip, W):
     for rec in out[-5:]:
         rec["bound"] = "lds"
     del z, z2, z3, r, big
-    # linear algebra: one workgroup per matrix, correctness first; times only
+    if not linalg:
+        return out
+
+    # linear algebra (only with --only-next: thousands of short launches that would drown a
+    # kernel-time profile of the hot path): correctness first, times only
     def la(name, fn, iters=3):
         timed(name, fn, 0, iters=iters)
         for key in ("GB/s", "frac_hbm"):
@@ -557,7 +561,8 @@ def main():
                     help="also launch 20 plain 64 MiB copies (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--only-config", type=int, choices=(1, 2, 3, 4), default=0,
                     help="time the operations of one configuration only and print their records")
-    ap.add_argument("--only-next", action="store_true", help="time pad/cat/scan/threefry/scatter only")
+    ap.add_argument("--only-next", action="store_true",
+                    help="time the operations beside the hot path only (pad ... fft), the linear-algebra family included")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 forward leg only and print its record")
     ap.add_argument("--cpu-configs", action="store_true",
                     help="time the CPU oracle on bounded samples of configurations 1, 3, 4, 5 and print the records")
@@ -577,7 +582,7 @@ def main():
         print(json.dumps(config5(hip, window=True, graph=True, iters=10)))
         return
     if args.only_next:
-        print(json.dumps({"ops": next_ops(hip, Workloads(hip))}))
+        print(json.dumps({"ops": next_ops(hip, Workloads(hip), linalg=True)}))
         return
     if args.only_config:
         # one configuration's operations, each timed alone (for profiling runs)
