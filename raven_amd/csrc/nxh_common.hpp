@@ -163,10 +163,22 @@ HD float u2f(uint32_t u) { return __builtin_bit_cast(float, u); }
 // f32 -> bf16, nx_buffer_stubs.h:73-86: NaN keeps sign/payload and is quieted,
 // everything else rounds to nearest even on the dropped half.
 HD uint16_t f32_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  // One v_cvt_pk_bf16_f32. It returns what the rule below returns for every one of
+  // the 2^32 float bit patterns, NaNs included (compared exhaustively on an MI355X);
+  // the rule itself costs eight integer instructions per element, which made the
+  // narrowing epilogues and the fused row kernels VALU-bound.
+  // The barrier keeps the conversion a scalar one: without it the compiler pairs it
+  // with neighbouring float operations into two-element vector nodes that the
+  // backend cannot select when packed f32 operations are switched off.
+  asm("" : "+v"(f));
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+#else
   uint32_t u = f2u(f);
   uint32_t nan = (u >> 16) | 0x40u;
   uint32_t rne = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
   return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? nan : rne);
+#endif
 }
 HD float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
 
