@@ -45,7 +45,7 @@ class Entry:
     """One recorded primitive."""
 
     __slots__ = ("kind", "op", "ins", "shape", "dtype", "axes", "cell", "alive", "result", "readers", "fused_into",
-                 "value", "tag", "__weakref__")
+                 "value", "tag", "wanted", "__weakref__")
 
     def __init__(self, kind, op, ins, shape, dtype, axes=None):
         self.kind, self.op, self.ins = kind, op, ins
@@ -57,6 +57,7 @@ class Entry:
         self.fused_into = None
         self.value = None      # kind "full": the encoded element
         self.tag = None        # what is known about the result's contents (("causal", n))
+        self.wanted = False    # a caller asked for the result itself (force)
 
 
 class Operand:
@@ -180,6 +181,7 @@ class Window:
     def force(self, t: WTensor):
         """The backend's tensor for ``t`` (executes the record if ``t`` is pending)."""
         if t.cell.root is None:
+            t.cell.entry.wanted = True
             self.flush()
         return self.B.with_view(t.cell.root, t.view)
 
@@ -303,11 +305,20 @@ class Window:
         return self._wrap(self.B.buffer(dtype, shape))
 
     def from_host(self, array, dtype):
-        t = self._wrap(self.B.from_host(array, dtype))
+        """Small int32 uploads (index vectors: the aranges of a causal mask, token
+        ids) are kept on the host until something reads them: a compare of two
+        aranges is then recognised as a causal mask, and when the attention kernel
+        takes that mask as a flag neither the compare nor the uploads happen."""
         a = np.asarray(array)
-        if dtype.name == "int32" and a.nbytes <= 65536:
-            t.cell.host = a.reshape(-1).copy()  # lets a compare of two aranges be recognised as a causal mask
-        return t
+        if dtype.name != "int32" or a.nbytes > 65536 or a.size == 0:
+            return self._wrap(self.B.from_host(array, dtype))
+        host = np.ascontiguousarray(a).reshape(-1).copy()
+        e = Entry("upload", None, [], (host.size,), dtype)
+        e.value = host
+        cell = Cell(entry=e, host=host)
+        e.cell = weakref.ref(cell)
+        self.entries.append(e)
+        return WTensor(cell, View.create((host.size,)), dtype, self)
 
     # ── everything else: execute the record, then call through ──────────────
     def __getattr__(self, name):
@@ -339,14 +350,17 @@ class Window:
     # ── executing the record ────────────────────────────────────────────────
     def _tensor_of(self, o: Operand):
         e = o.entry
-        if e is not None and e.result is None and e.kind == "full":
-            self._issue(e)  # a scalar that something still reads
+        if e is not None and e.result is None and e.kind in ("full", "upload"):
+            self._issue(e)  # a scalar or an upload that something still reads
         root = e.result if e is not None else o.root
         return self.B.with_view(root, o.view)
 
     def _issue(self, e: Entry):
         if e.kind == "full":
             self._deliver(e, self.B.full(e.dtype, e.shape, e.value))
+            return
+        if e.kind == "upload":
+            self._deliver(e, self.B.from_host(e.value, e.dtype))
             return
         ins = [self._tensor_of(o) for o in e.ins]
         if e.kind == "unary":
@@ -390,9 +404,28 @@ class Window:
                     plans[id(e)] = plan
                     for inner in plan.interior:
                         inner.fused_into = e
+        carried = []
         try:
             for e in entries:
                 if e.fused_into is not None:
+                    continue
+                if e.kind == "compare" and e.tag is not None and e.result is None and not e.wanted:
+                    # A causal mask whose readers all went into fused runs that take it as a
+                    # flag: nobody has needed its elements yet. It stays recorded (with the
+                    # uploads it reads) until a reader outside a fused run or a caller wants
+                    # it, and is dropped once its last handle is gone.
+                    if all(r.fused_into is not None and _takes_flag(plans, r) for r in e.readers):
+                        if e.alive:
+                            carried += [o.entry for o in e.ins if o.entry is not None and o.entry.result is None]
+                            carried.append(e)
+                        continue
+                if e.kind == "upload":
+                    # uploaded when a reader is issued or a caller wants it; kept while a handle is left
+                    if e.result is None:
+                        if e.wanted:
+                            self._issue(e)
+                        elif e.alive:
+                            carried.append(e)
                     continue
                 if e.kind == "full":
                     # filled only if a handle is left or, later, when a reader is issued
@@ -415,8 +448,14 @@ class Window:
                 self.stats[plan.name] += 1
                 self._deliver(e, r)
         finally:
+            keep = set(map(id, carried))
             for e in entries:  # drop the graph: results stay alive through their cells only
-                e.ins, e.readers, e.result = [], [], None
+                if id(e) in keep:
+                    e.readers = []
+                else:
+                    e.ins, e.readers, e.result = [], [], None
+            seen = set()
+            self.entries = [e for e in carried if not (id(e) in seen or seen.add(id(e)))] + self.entries
 
     def synchronize(self):
         self.flush()
@@ -445,6 +484,12 @@ def _producer(o: Operand, kind, op=None, identity=True) -> Optional[Entry]:
     if identity and not _identity(o.view, e.shape):
         return None
     return e
+
+
+def _takes_flag(plans, reader: Entry) -> bool:
+    """The fused run `reader` went into replaces its mask operand by a flag."""
+    plan = plans.get(id(reader.fused_into))
+    return plan is not None and plan.name == "attention" and getattr(plan, "causal", False)
 
 
 def _hidden(interior: Sequence[Entry], anchor: Entry) -> bool:
@@ -603,7 +648,7 @@ def _match_attention(w: Window, anchor: Entry) -> Optional[Plan]:
         flat = tuple(0 if s_ != 1 else st for s_, st in zip(sshape[:-2], mask.view.strides[:-2]))
         if (mask.tag == ("causal", n) and ks[-2] == n and mask.view.offset == 0 and mask.view.strides[-2:] == (n, 1)
                 and all(st == 0 or s_ == 1 for s_, st in zip(sshape[:-2], mask.view.strides[:-2]))):
-            causal, mask = True, None
+            causal, mask = True, None  # the kernel takes the mask as a flag (see Window.flush for the compare)
         del flat
     as_f32 = lambda a: None if a is None else np.asarray(a, dtype=np.float32).reshape(1)
 
@@ -611,7 +656,9 @@ def _match_attention(w: Window, anchor: Entry) -> Optional[Plan]:
         return win.B.attention(win._tensor_of(q), win._tensor_of(k), win._tensor_of(v), as_f32(scale),
                                win._tensor_of(mask) if mask is not None else None, as_f32(masked), causal)
 
-    return Plan("attention", interior, run)
+    plan = Plan("attention", interior, run)
+    plan.causal = causal
+    return plan
 
 
 def _match_linear(w: Window, anchor: Entry) -> Optional[Plan]:

@@ -140,6 +140,7 @@ def test_captured_gpt2_forward_replays_the_windowed_forward(hip, oracle, d):
     model = Gpt2(nx, cfg)
     ids = [np.random.default_rng(40 + k).integers(0, cfg.vocab_size, (2, 96)).astype(np.int32) for k in range(3)]
     t_ids = nx.create(dt.int32, ids[0].shape, ids[0])
+    win.force(t_ids)  # the window uploads small index tensors on first use: the input must exist before the capture
     eager = [logical(win.force(model.logits(params, nx.create(dt.int32, i.shape, i)))) for i in ids]
     with capture(win) as cap:
         out = win.force(model.logits(params, t_ids))

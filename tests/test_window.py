@@ -28,6 +28,7 @@ class SequencedOracle(OracleBackend):
     def __init__(self):
         self.calls = []
 
+
     def softmax_rows(self, x, scale=None, mask=None, masked_value=None, out_dtype=None):
         self.calls.append("softmax_rows")
         nx = Nx(self)
@@ -84,6 +85,25 @@ def win():
     return Window(SequencedOracle())
 
 
+class Counting:
+    """Counts what the window asks of the backend (not what the backend's own
+    sequences call internally)."""
+
+    def __init__(self, inner):
+        self._inner, self.asked = inner, {}
+
+    def __getattr__(self, name):
+        attr = getattr(self._inner, name)
+        if not callable(attr):
+            return attr
+
+        def counted(*a, **k):
+            self.asked[name] = self.asked.get(name, 0) + 1
+            return attr(*a, **k)
+
+        return counted
+
+
 def forward(backend, hp, ids, d, oracle):
     nx = Nx(backend)
     params = upload(nx, hp, d, lambda a, dd: encode(a, dd, oracle))
@@ -96,7 +116,8 @@ def test_gpt2_forward_through_the_window_fuses_every_sequence(oracle, d):
     ids = np.random.default_rng(12).integers(0, TINY.vocab_size, (2, 8))
     want = ological(forward(oracle, hp, ids, d, oracle))
     base = SequencedOracle()
-    w = Window(base)
+    asked = Counting(base)
+    w = Window(asked)
     got = value(w, forward(w, hp, ids, d, oracle))
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
     L = TINY.n_layer
@@ -112,12 +133,17 @@ def test_gpt2_forward_through_the_window_fuses_every_sequence(oracle, d):
         assert (w.stats["attention"], w.stats["softmax_rows"]) == (0, L)
         assert base.calls.count("softmax_rows") == L
     # the six linears of a block take their bias add, and two of them the residual
-    # add, into the GEMM; what is left op by op per block is the mask compare and,
-    # for float32, the two attention matmuls; outside the blocks the embedding
-    # add and the head matmul
+    # add, into the GEMM; what is left op by op per block is, for float32, the mask
+    # compare and the two attention matmuls (the causal attention kernel takes the
+    # mask as a flag: neither its compare nor the two aranges it reads are ever
+    # issued); outside the blocks the embedding add and the head matmul
     assert w.stats["linear"] == 6 * L and base.calls.count("linear") == 6 * L
-    per_block = 1 + (0 if d is dt.bfloat16 else 2)
+    per_block = 0 if d is dt.bfloat16 else 3
     assert w.stats["issued"] == L * per_block + 2
+    assert asked.asked.get("compare", 0) == (0 if d is dt.bfloat16 else L)
+    n_params = 4 + 16 * L  # wte, wpe, ln_f (2) and 16 leaves per block
+    # ids and positions, and for float32 the arange of each mask
+    assert asked.asked["from_host"] - n_params == (2 if d is dt.bfloat16 else 2 + L)
     # with fusion switched off the window only defers
     w2 = Window(SequencedOracle(), fuse=False)
     got2 = value(w2, forward(w2, hp, ids, d, oracle))
