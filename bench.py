@@ -281,7 +281,7 @@ def next_ops(hip, W, linalg=False):
     cplx = lambda shape: W.dev((rng.standard_normal(shape) + 1j * rng.standard_normal(shape)).astype(np.complex64),
                                dt.complex64)
     z = cplx((16384, 1024))
-    timed("fft [16384,1024] complex64 axis 1 (fft_lines, radix-2 in LDS)", lambda: hip.fft(z, [1]), 2 * 16384 * 1024 * 8)
+    timed("fft [16384,1024] complex64 axis 1 (fft_lines, four radix-2 stages per LDS pass)", lambda: hip.fft(z, [1]), 2 * 16384 * 1024 * 8)
     out[-1]["GFLOP/s"] = round(5 * 16384 * 1024 * 10 / out[-1]["ms"] / 1e6, 1)
     z2 = cplx((4096, 4096))
     timed("fft [4096,4096] complex64 axis 0 (strided lines)", lambda: hip.fft(z2, [0]), 2 * 4096 * 4096 * 8)

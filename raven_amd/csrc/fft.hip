@@ -13,7 +13,7 @@
 //
 // How it runs here: one axis pass = one launch in which a workgroup owns one
 // line (or several short ones), loads it strided into LDS as double2, does all
-// radix-2 stages there (two at a time, four elements per lane in registers) and stores it strided, so a pass reads and writes the
+// radix-2 stages there (four at a time, sixteen elements per lane in registers) and stores it strided, so a pass reads and writes the
 // tensor exactly once. Lengths that are not a power of two go through Bluestein's
 // identity inside the same kernel: chirp on load, a power-of-two convolution of
 // length M >= 2n-1 (forward DIF, multiply by the transformed chirp filter in
@@ -65,6 +65,11 @@ struct FftArgs {
   int64_t tw_total;      // four-step: multiply bin k of a line by exp(sign 2 pi i inner k / tw_total)
 };
 
+// Element i of the lines lives at LDS index i + i / 16: one pad element per 16
+// (per 256 bytes, the width of the banks) turns the power-of-two strides of the
+// butterflies and of the bit-reversed scatter into conflict-free ones.
+__device__ __forceinline__ int pad(int i) { return i + (i >> 4); }
+
 __device__ __forceinline__ double2 cmul(double2 a, double2 b) {
   return make_double2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x);
 }
@@ -114,118 +119,81 @@ __device__ __forceinline__ double2 fetch(const FftArgs &a, int64_t off, int j) {
   return load_elem(a.in.base, a.in.kind, off + j * a.in.estride);
 }
 
-// One radix-2 butterfly stage over the G lines of the workgroup. `s` is the
-// stage (sub-transform length 2^s). DIT: input bit-reversed, output natural.
-// DIF: input natural, output bit-reversed.
-// The twiddle table stays in global memory (it is small and cache-resident): the
-// stages are bound by LDS bandwidth, and a copy of the table in LDS measured slower.
-template <bool DIF>
-__device__ __forceinline__ void stage(double2 *lds, const FftArgs &a, int s, int sign) {
-  const double2 *tw = a.tw;
-  const int half = 1 << (s - 1);
-  const int per_line = a.M >> 1;
-  const int total = a.G * per_line;
-  for (int b = threadIdx.x; b < total; b += blockDim.x) {
-    const int g = b >> (a.logM - 1);
-    const int r = b & (per_line - 1);
-    const int pos = r & (half - 1);
-    const int i = (g << a.logM) + ((r >> (s - 1)) << s) + pos;
-    const int j = i + half;
-    double2 w = tw[pos << (a.logM - s)];
-    if (sign > 0) w.y = -w.y;
-    const double2 u = lds[i], v = lds[j];
-    if (DIF) {
-      lds[i] = make_double2(u.x + v.x, u.y + v.y);
-      lds[j] = cmul(make_double2(u.x - v.x, u.y - v.y), w);
-    } else {
-      const double2 t = cmul(w, v);
-      lds[i] = make_double2(u.x + t.x, u.y + t.y);
-      lds[j] = make_double2(u.x - t.x, u.y - t.y);
-    }
-  }
-  __syncthreads();
-}
-
-// Stages s and s + 1 in one pass: a lane holds the four elements h = 2^(s-1)
-// apart in registers and does both butterflies of each, so the lines go through
-// LDS once for two stages. The arithmetic per element is that of two calls of
-// `stage`, in the same order.
-template <bool DIF>
-__device__ __forceinline__ void stage_pair(double2 *lds, const FftArgs &a, int s, int sign) {
+// R consecutive radix-2 stages, s .. s + R - 1 (stage s has sub-transform length
+// 2^s), in one pass over the G lines of the workgroup: a lane holds the 2^R
+// elements h = 2^(s-1) apart in registers and does every butterfly among them,
+// so the lines go through LDS once per R stages (the stages are bound by LDS
+// bandwidth: 32 bytes per element and pass). The arithmetic per element is that
+// of R single stages in the same order. DIT (stages upwards): input bit-reversed,
+// output natural. DIF (stages downwards): input natural, output bit-reversed.
+// The twiddle table stays in global memory (small and cache-resident; a copy in
+// LDS measured slower).
+template <bool DIF, int R>
+__device__ __forceinline__ void stages(double2 *lds, const FftArgs &a, int s, int sign) {
+  constexpr int N = 1 << R;
   const double2 *tw = a.tw;
   const int h = 1 << (s - 1);
-  const int per_line = a.M >> 2;
+  const int per_line = a.M >> R;
   const int total = a.G * per_line;
-  auto add = [](double2 u, double2 v) { return make_double2(u.x + v.x, u.y + v.y); };
-  auto sub = [](double2 u, double2 v) { return make_double2(u.x - v.x, u.y - v.y); };
   for (int b = threadIdx.x; b < total; b += blockDim.x) {
-    const int g = b >> (a.logM - 2);
+    const int g = b >> (a.logM - R);
     const int r = b & (per_line - 1);
     const int pos = r & (h - 1);
-    const int i0 = (g << a.logM) + ((r >> (s - 1)) << (s + 1)) + pos;
-    const int i1 = i0 + h, i2 = i0 + 2 * h, i3 = i0 + 3 * h;
-    double2 w1 = tw[pos << (a.logM - s)], w2 = tw[pos << (a.logM - s - 1)], w3 = tw[(pos + h) << (a.logM - s - 1)];
-    if (sign > 0) {
-      w1.y = -w1.y;
-      w2.y = -w2.y;
-      w3.y = -w3.y;
+    const int i0 = (g << a.logM) + ((r >> (s - 1)) << (s - 1 + R)) + pos;
+    double2 x[N];
+#pragma unroll
+    for (int k = 0; k < N; k++) x[k] = lds[pad(i0 + k * h)];
+#pragma unroll
+    for (int qq = 0; qq < R; qq++) {
+      const int q = DIF ? R - 1 - qq : qq, span = 1 << q;
+#pragma unroll
+      for (int k = 0; k < N; k++) {
+        if (k & span) continue;
+        // the pair's position inside its sub-transform of length 2^(s+q)
+        double2 w = tw[(pos + (k & (span - 1)) * h) << (a.logM - s - q)];
+        if (sign > 0) w.y = -w.y;
+        const double2 u = x[k], v = x[k + span];
+        if (DIF) {
+          x[k] = make_double2(u.x + v.x, u.y + v.y);
+          x[k + span] = cmul(make_double2(u.x - v.x, u.y - v.y), w);
+        } else {
+          const double2 t = cmul(w, v);
+          x[k] = make_double2(u.x + t.x, u.y + t.y);
+          x[k + span] = make_double2(u.x - t.x, u.y - t.y);
+        }
+      }
     }
-    double2 x0 = lds[i0], x1 = lds[i1], x2 = lds[i2], x3 = lds[i3];
-    if (DIF) {
-      double2 u = x0, v = x2;
-      x0 = add(u, v);
-      x2 = cmul(sub(u, v), w2);
-      u = x1, v = x3;
-      x1 = add(u, v);
-      x3 = cmul(sub(u, v), w3);
-      u = x0, v = x1;
-      x0 = add(u, v);
-      x1 = cmul(sub(u, v), w1);
-      u = x2, v = x3;
-      x2 = add(u, v);
-      x3 = cmul(sub(u, v), w1);
-    } else {
-      double2 t = cmul(w1, x1), u = x0;
-      x0 = add(u, t);
-      x1 = sub(u, t);
-      t = cmul(w1, x3), u = x2;
-      x2 = add(u, t);
-      x3 = sub(u, t);
-      t = cmul(w2, x2), u = x0;
-      x0 = add(u, t);
-      x2 = sub(u, t);
-      t = cmul(w3, x3), u = x1;
-      x1 = add(u, t);
-      x3 = sub(u, t);
-    }
-    lds[i0] = x0;
-    lds[i1] = x1;
-    lds[i2] = x2;
-    lds[i3] = x3;
+#pragma unroll
+    for (int k = 0; k < N; k++) lds[pad(i0 + k * h)] = x[k];
   }
   __syncthreads();
 }
 
-// All stages of the lines in LDS. DIT runs the stages upwards (bit-reversed in,
-// natural out), DIF downwards (natural in, bit-reversed out); an odd count starts
-// with one single stage.
+// All stages of the lines in LDS, FFT_RADIX_LOG2 at a time; the stages left over
+// (fewer than that) go first in DIT order, last in DIF order.
+constexpr int FFT_RADIX_LOG2 = 4;
 template <bool DIF>
 __device__ __forceinline__ void all_stages(double2 *lds, const FftArgs &a, int sign) {
+  constexpr int R = FFT_RADIX_LOG2;
+  const int rem = a.logM % R;
+  auto odd = [&](int s) {
+    if (rem == 1) stages<DIF, 1>(lds, a, s, sign);
+    else if (rem == 2) stages<DIF, 2>(lds, a, s, sign);
+    else if (rem == 3) stages<DIF, 3>(lds, a, s, sign);
+  };
   if (DIF) {
-    int s = a.logM;
-    if (s & 1) stage<true>(lds, a, s--, sign);
-    for (; s >= 2; s -= 2) stage_pair<true>(lds, a, s - 1, sign);
+    for (int s = a.logM - R + 1; s >= rem + 1; s -= R) stages<true, R>(lds, a, s, sign);
+    odd(1);
   } else {
-    int s = 1;
-    if (a.logM & 1) stage<false>(lds, a, s++, sign);
-    for (; s + 1 <= a.logM; s += 2) stage_pair<false>(lds, a, s, sign);
+    odd(1);
+    for (int s = rem + 1; s + R - 1 <= a.logM; s += R) stages<false, R>(lds, a, s, sign);
   }
 }
 
 template <bool BLUE>
 __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
   extern __shared__ double2 lds[];
-  int64_t *off_in = (int64_t *)(lds + ((size_t)a.G << a.logM));
+  int64_t *off_in = (int64_t *)(lds + pad(a.G << a.logM) + 1);
   int64_t *off_out = off_in + a.G;
   int *inner = (int *)(off_out + a.G);
   const int64_t first = (int64_t)blockIdx.x * a.G;
@@ -248,7 +216,7 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
     }
     // the plain transform is decimation in time: it wants its input bit-reversed
     const int p = BLUE || a.logM == 0 ? j : (int)(__brev((unsigned)j) >> shift);
-    lds[(g << a.logM) + p] = v;
+    lds[pad((g << a.logM) + p)] = v;
   }
   __syncthreads();
   if (BLUE) {
@@ -256,7 +224,7 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
     for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
       const int p = idx & (a.M - 1);
       const int k = a.logM == 0 ? 0 : (int)(__brev((unsigned)p) >> shift);
-      lds[idx] = cmul(lds[idx], a.bf[k]);
+      lds[pad(idx)] = cmul(lds[pad(idx)], a.bf[k]);
     }
     __syncthreads();
     all_stages<false>(lds, a, +1);
@@ -266,9 +234,10 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
   const double inv_m = 1.0 / (double)a.M;
   const int stores = a.G * a.n_store;
   for (int idx = threadIdx.x; idx < stores; idx += blockDim.x) {
-    const int g = idx / a.n_store, k = idx - g * a.n_store;
+    // whole power-of-two lines (the common case) are decoded without a division
+    const int g = a.n_store == a.M ? idx >> a.logM : idx / a.n_store, k = idx - g * a.n_store;
     if (first + g >= a.lines) break;
-    double2 v = lds[(g << a.logM) + k];
+    double2 v = lds[pad((g << a.logM) + k)];
     if (BLUE) {
       const double2 c = a.chirp[k];
       v = cmul(v, make_double2(c.x * inv_m, c.y * inv_m));
@@ -416,13 +385,13 @@ static int launch_lines(nxh_context *ctx, FftArgs &a, bool blue) {
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, "fft", "too many lines for one launch");
   const int64_t elems = (int64_t)a.G * a.M;
   const int threads = elems >= 8192 ? 1024 : elems >= 4096 ? 512 : 256;
-  const size_t lds = (size_t)elems * sizeof(double2) + (size_t)a.G * (2 * sizeof(int64_t) + sizeof(int));
+  const size_t lds = (size_t)(elems + elems / 16 + 1) * sizeof(double2) + (size_t)a.G * (2 * sizeof(int64_t) + sizeof(int));
   auto kern = blue ? fft_lines_kernel<true> : fft_lines_kernel<false>;
   static std::once_flag once[2];
   static hipError_t attr_status[2] = {hipSuccess, hipSuccess};
   std::call_once(once[blue], [&] {
     attr_status[blue] = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                            (int)(FFT_LDS_MAX * sizeof(double2) + 4096));
+                                            (int)((FFT_LDS_MAX + FFT_LDS_MAX / 16) * sizeof(double2) + 4096));
   });
   NXH_HIP("fft", attr_status[blue]);
   hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(threads), lds, ctx->stream, a);
