@@ -392,14 +392,18 @@ __global__ __launch_bounds__(LA_THREADS) void eigh_kernel(T *a_all, T *v_all, T 
 
 // Columns by descending norm (ties by position) into Gs / Vs; `norms` holds nn doubles.
 template <class T>
-__device__ void svd_sort_block(const T *G, const T *V, T *Gs, T *Vs, int mm, int nn, double *norms) {
+__device__ void svd_sort_block(const T *G, const T *V, T *Gs, T *Vs, int mm, int nn, double *norms, int *status) {
   using S = Sc<T>;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
   for (int c = wave; c < nn; c += waves) {
     double a = 0.0;
     for (int i = lane; i < mm; i += 64) a += S::abs2(G[(size_t)c * mm + i]);
     a = wave_sum(a);
-    if (lane == 0) norms[c] = a;
+    if (lane == 0) {
+      norms[c] = a;
+      // a NaN or infinity in the matrix stops no rotation and orders nowhere: the iteration has not converged
+      if (!(a - a == 0.0)) raise(status, LA_NO_CONVERGE);
+    }
   }
   __syncthreads();
   for (int c = wave; c < nn; c += waves) {
@@ -480,7 +484,7 @@ __global__ __launch_bounds__(LA_THREADS) void svd_jacobi_kernel(T *g_all, T *v_a
     if (threadIdx.x == 0) raise(status, LA_NO_CONVERGE);
     return;
   }
-  svd_sort_block(G, V, Gs, Vs, mm, nn, norms);
+  svd_sort_block(G, V, Gs, Vs, mm, nn, norms, status);
 }
 
 // After the QR of the sorted, orthogonal columns: R's diagonal carries the
@@ -665,10 +669,11 @@ __global__ __launch_bounds__(LA_THREADS) void svd_wide_round(T *g_all, T *v_all,
 }
 
 template <class T>
-__global__ __launch_bounds__(LA_THREADS) void svd_wide_sort(const T *g_all, const T *v_all, T *gs_all, T *vs_all, int mm, int nn) {
+__global__ __launch_bounds__(LA_THREADS) void svd_wide_sort(const T *g_all, const T *v_all, T *gs_all, T *vs_all, int mm, int nn,
+                                                           int *status) {
   extern __shared__ double norms[];
   const size_t g = (size_t)blockIdx.x * mm * nn, v = (size_t)blockIdx.x * nn * nn;
-  svd_sort_block(g_all + g, v_all + v, gs_all + g, vs_all + v, mm, nn, norms);
+  svd_sort_block(g_all + g, v_all + v, gs_all + g, vs_all + v, mm, nn, norms, status);
 }
 
 __global__ void la_fill_int(int *p, int count, int value) {
@@ -1265,7 +1270,7 @@ static int svd_wide(nxh_context *ctx, const char *op, Work &work, int64_t batch,
   if (!converged) return nxh_fail(NXH_FAILURE, op, LA_MESSAGES[LA_NO_CONVERGE]);
   std::lock_guard<std::mutex> g(ctx->mu);
   hipLaunchKernelGGL(svd_wide_sort<T>, dim3((unsigned)batch), dim3(LA_THREADS), (size_t)nn * 8, ctx->stream, (const T *)G, (const T *)V,
-                     Gs, Vs, mm, nn);
+                     Gs, Vs, mm, nn, la_status(ctx));
   return NXH_OK;
 }
 

@@ -147,8 +147,9 @@ def test_eigh_and_eigvalsh(hip, oracle, name):
         assert np.max(np.abs(full @ v - v * w[..., None, :])) <= tol * scale * n
         assert rel(H(v) @ v, np.broadcast_to(np.eye(n), batch + (n, n))) <= tol * n
     nan = np.full((3, 3), np.nan).astype(d.np_storage)
-    with pytest.raises(RuntimeError, match="did not converge"):
-        hip.eigh(hip.reshape(hip.from_host(nan, d), (3, 3)))
+    for call in (hip.eigh, hip.svd, hip.eig):
+        with pytest.raises(RuntimeError, match="did not converge"):
+            call(hip.reshape(hip.from_host(nan, d), (3, 3)))
 
 
 @pytest.mark.parametrize("name", list(DTYPES))
@@ -223,3 +224,37 @@ def test_half_precision_storage_and_rejections(hip, oracle):
             call(rect)
     empty = hip.reshape(hip.from_host(np.zeros(0, np.float32), dt.float32), (0, 3, 3))
     assert logical(hip.cholesky(empty)).shape == (0, 3, 3)
+
+
+def test_failures_of_the_device_wide_forms(hip):
+    """From 65 rows on the factorisations run as many launches: the numeric
+    failures must come out of those too, and must not stick to the next call."""
+    d, n = dt.float64, 100
+    rng = np.random.default_rng(8)
+    g = rng.standard_normal((n, n))
+    a = g @ g.T + n * np.eye(n)
+    mk = lambda x: hip.reshape(hip.from_host(np.ascontiguousarray(x), d), x.shape)
+    bad = a.copy()
+    bad[60, 60] = -1e6
+    with pytest.raises(RuntimeError, match="not positive definite"):
+        hip.cholesky(mk(bad))
+    assert hip.last_path() == "cholesky_columns_wide"
+    low = arr(hip.cholesky(mk(a)))
+    assert rel(low @ low.T, a) <= 1e-12
+    tri = np.tril(a)
+    tri[77, 77] = 0.0
+    with pytest.raises(RuntimeError, match="singular"):
+        hip.triangular_solve(mk(tri), mk(np.ones((n, 3))), False, False, False)
+    x = arr(hip.triangular_solve(mk(np.tril(a)), mk(np.ones((n, 3))), False, False, False))
+    assert rel(np.tril(a) @ x, np.ones((n, 3))) <= 1e-10
+    nan = a.copy()
+    nan[5, 3] = np.nan
+    for call in (hip.eigh, hip.svd):
+        with pytest.raises(RuntimeError, match="did not converge"):
+            call(mk(nan))
+    w, _ = hip.eigh(mk(a))
+    assert np.max(np.abs(logical(w) - np.linalg.eigvalsh(a))) <= 1e-9 * np.max(np.abs(a))
+    # two matrices, one of which fails: the call fails as a whole
+    pair = np.stack([a, bad])
+    with pytest.raises(RuntimeError, match="not positive definite"):
+        hip.cholesky(mk(pair))
