@@ -65,5 +65,19 @@ def build_all(force: bool = True, jobs: int | None = None) -> Path:
     return LIB
 
 
+ABI_CHECK_SRC = CSRC.parent.parent / "tests" / "abi_c" / "nxh_abi_check.c"
+ABI_CHECK_BIN = ABI_CHECK_SRC.with_suffix("")
+
+
+def build_abi_check() -> Path:
+    """The plain-C user of the ABI (tests/abi_c): gcc, no HIP, no Python at run time."""
+    cmd = ["gcc", "-std=gnu11", "-O1", "-Wall", "-Wextra", "-I", str(CSRC.parent.parent / "include"),
+           "-o", str(ABI_CHECK_BIN), str(ABI_CHECK_SRC), "-ldl", "-lm"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0 or r.stderr.strip():
+        raise RuntimeError(f"gcc failed on {ABI_CHECK_SRC.name}:\n{r.stderr}")
+    return ABI_CHECK_BIN
+
+
 if __name__ == "__main__":
     print(build_all(force="--force" in sys.argv))

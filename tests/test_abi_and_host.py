@@ -97,3 +97,18 @@ def test_scalar_encoding_matches_oracle_converters():
         assert int(encode_scalar(dt.bfloat16, v)[0]) == L.nxo_f32_to_bf16(np.float32(v))
         with np.errstate(all="ignore"):
             assert int(encode_scalar(dt.float16, v).view(np.uint16)[0]) == L.nxo_f32_to_f16(np.float32(v))
+
+
+@pytest.mark.gpu
+def test_the_abi_from_plain_c():
+    """tests/abi_c/nxh_abi_check.c drives the library the way the OCaml stubs do
+    (dlopen, descriptors, statuses), with no Python or torch in the process, and
+    checks every result against the same arithmetic on the host."""
+    import subprocess
+
+    from raven_amd import _ffi, build
+
+    assert build.ABI_CHECK_BIN.exists(), "run __graft_entry__.build() first"
+    r = subprocess.run([str(build.ABI_CHECK_BIN), str(_ffi.LIB_PATH)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and r.stdout.strip().endswith("all ok"), r.stdout + r.stderr
+    assert "FAIL" not in r.stdout
