@@ -16,9 +16,11 @@
 // is the order of the f32 sums (scores, row sum, probs x v) and that the row sum
 // is accumulated tile by tile against a running maximum.
 //
-// Layout of the work: a block of four wave64s owns two 64-query tiles of one
-// (batch, head), tile t and tile T-1-t, so that every block meets the same
-// number of keys under a causal mask; each wave 32 queries. Keys are visited 64 at a time through
+// Layout of the work: a block of two wave64s owns two 64-query tiles of one
+// (batch, head), tile t and then tile T-1-t, so that every block meets the same
+// number of keys under a causal mask and both waves of a block always walk the
+// same keys (four waves on the two tiles at once left the waves of the short tile
+// idle at the barriers of the long one); each wave 32 queries. Keys are visited 64 at a time through
 // LDS (K as [key][d], V as [key][d] too and read back with the transposing LDS
 // load, so no operand is ever transposed in memory). The wave computes the
 // TRANSPOSED score tile S^T = K Q^T, so that a lane holds 16 scores of ONE
@@ -70,7 +72,7 @@ __device__ __forceinline__ float xor32(float v) {
 }
 
 template <class EL, int DHEAD>
-__global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
+__global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
   using S = uint16_t;
   using MX = Combine<NXH_RMAX, float, CAT_FLOAT>;
   constexpr int KSTEPS = DHEAD / 16;  // k-steps of Q K^T
@@ -102,15 +104,18 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
   S *O = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
   const uint8_t *M = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
 
-  // Waves 0-1 take the pair's low 64-query tile, waves 2-3 its high one (tile
-  // t pairs with tile T-1-t): under a causal mask every block then sees the
-  // same number of keys in total. The middle tile of an odd count pairs with
-  // itself: its upper waves have nothing to do.
+  // A block is two waves on one 64-query tile at a time: first tile `pair`, then
+  // tile T-1-pair. Under a causal mask every block then sees the same number of
+  // keys in total, and its two waves always have (almost) the same key range, so
+  // no wave idles at the tile barriers while the other works. The middle tile of
+  // an odd count pairs with itself and is done once.
   const int t64 = (a.sq + 63) / 64, hi_tile = t64 - 1 - pair;
-  const bool upper = wave >= 2;
-  const bool idle = upper && hi_tile == pair;
-  const int qw = (upper ? hi_tile : pair) * 64 + (wave & 1) * 32;  // first query of the wave
-  const int qi = idle ? a.sq : qw + c32;                           // this lane's query
+  for (int phase = 0; phase < 2; phase++) {
+  if (phase == 1 && hi_tile == pair) break;
+  const int tile = phase ? hi_tile : pair;
+  const bool idle = false;
+  const int qw = tile * 64 + wave * 32;        // first query of the wave
+  const int qi = qw + c32;                     // this lane's query
   const int qrow = qi < a.sq ? qi : a.sq - 1;  // clamp: rows past the end are never stored
   // Q fragments: B operand of S^T = K Q^T, this lane's 8 d-values per k-step
   V16 qf[KSTEPS];
@@ -119,7 +124,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
     qf[s] = *reinterpret_cast<const V16 *>(Q + (int64_t)qrow * a.q.row + s * 16 + g * 8);
 
   // keys this block needs: all, or up to its last query under a causal mask
-  const int qend = (hi_tile + 1) * 64;  // one past the block's last query
+  const int qend = (tile + 1) * 64;  // one past the tile's last query
   const int klimit = a.causal ? (qend < a.sk ? qend : a.sk) : a.sk;
   const int ktiles = (klimit + KEYS - 1) / KEYS;
 
@@ -165,12 +170,12 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
   // Global -> registers for one key tile (K, and V when the tile is for pass
   // 1), issued a tile ahead so that the loads fly during the previous tile's
   // arithmetic; registers -> LDS between the two barriers.
-  constexpr int NV = KEYS * VPR / 256;
+  constexpr int NV = KEYS * VPR / 128;
   V16 kpre[NV], vpre[NV];
   auto prefetch = [&](int pass, int kt) {
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-      const int v = threadIdx.x + i * 256;
+      const int v = threadIdx.x + i * 128;
       const int r = v / VPR, c = (v % VPR) * 8;
       int key = kt * KEYS + r;
       key = key < a.sk ? key : a.sk - 1;
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
       __syncthreads();  // the previous tile has been consumed
 #pragma unroll
       for (int i = 0; i < NV; i++) {
-        const int v = threadIdx.x + i * 256;
+        const int v = threadIdx.x + i * 128;
         const int r = v / VPR, c = (v % VPR) * 8;
         *reinterpret_cast<V16 *>(Ks + r * PK + c) = kpre[i];
         if (pass == 1) *reinterpret_cast<V16 *>(Vs + r * PV + c) = vpre[i];
@@ -264,13 +269,15 @@ __global__ __launch_bounds__(256) void attention_kernel(AttArgs a) {
         *reinterpret_cast<uint2 *>(orow + d) = w;
       }
   }
+  __syncthreads();  // the next phase refills the key tiles
+  }
 }
 
 template <class EL>
 int attention_launch(nxh_context *ctx, const char *op, const AttArgs &a, int hd) {
   const int64_t blocks = a.batches * a.qtiles;
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
-  const dim3 grid((unsigned)blocks), block(256);
+  const dim3 grid((unsigned)blocks), block(128);
   switch (hd) {
     case 32: hipLaunchKernelGGL((attention_kernel<EL, 32>), grid, block, 0, ctx->stream, a); break;
     case 64: hipLaunchKernelGGL((attention_kernel<EL, 64>), grid, block, 0, ctx->stream, a); break;
