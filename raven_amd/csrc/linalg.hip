@@ -858,21 +858,35 @@ __device__ __forceinline__ c64 csqrt_principal(c64 z) {
   return {fabs(z.im) / (2.0 * t), copysign(t, z.im)};
 }
 
-// G = [[c, s], [-conj(s), c]] with G [a; b] = [r; 0]
+// G = [[c, s], [-conj(s), c]] with G [a; b] = [r; 0]. Every lane of the workgroup
+// computes it at every step of a QR sweep, on the chain from one rotation to the
+// next: the moduli come from one square root each after a common power-of-two
+// scaling (exact, and safe against overflow of the squares) instead of three
+// calls of hypot.
 __device__ __forceinline__ void givens(c64 a, c64 b, double *c, c64 *s) {
-  const double na = cabs2(a), nb = cabs2(b);
-  if (nb == 0.0) {
+  const double m = fmax(fmax(fabs(a.re), fabs(a.im)), fmax(fabs(b.re), fabs(b.im)));
+  if (!(m > 0.0) || !(m < __builtin_inf())) {  // all zero, or not finite: no rotation (NaNs surface in the convergence test)
     *c = 1.0;
     *s = {0.0, 0.0};
-  } else if (na == 0.0) {
+    return;
+  }
+  const int e = -ilogb(m);
+  a = {ldexp(a.re, e), ldexp(a.im, e)};
+  b = {ldexp(b.re, e), ldexp(b.im, e)};
+  const double a2 = a.re * a.re + a.im * a.im, b2 = b.re * b.re + b.im * b.im;
+  if (b2 == 0.0) {
+    *c = 1.0;
+    *s = {0.0, 0.0};
+  } else if (a2 == 0.0) {
+    const double nb = sqrt(b2);
     *c = 0.0;
     *s = {b.re / nb, -b.im / nb};
   } else {
-    const double norm = hypot(na, nb);
-    *c = na / norm;
+    const double na = sqrt(a2), inv = 1.0 / sqrt(a2 + b2);
+    *c = na * inv;
     const c64 ph = {a.re / na, a.im / na};
-    *s = ph * c64{b.re, -b.im};
-    *s = {s->re / norm, s->im / norm};
+    const c64 t = ph * c64{b.re, -b.im};
+    *s = {t.re * inv, t.im * inv};
   }
 }
 
@@ -883,7 +897,9 @@ __global__ __launch_bounds__(LA_THREADS) void eig_kernel(c64 *h_all, c64 *q_all,
                                                         int wantv, int *status) {
   extern __shared__ double lds_raw[];
   c64 *vec = (c64 *)lds_raw;     // n: a reflector, then the sines of one QR sweep
-  double *cs = (double *)(vec + n);  // n cosines
+  c64 *sub = vec + n;            // n: the subdiagonal as a QR sweep found it
+  double *cs = (double *)(sub + n);  // n cosines
+  __shared__ c64 s_pivot[2];
   __shared__ c64 scratch[LA_THREADS / 64];
   __shared__ int s_lo, s_hi, s_its, s_total, s_state;
   __shared__ c64 s_mu;
@@ -1012,45 +1028,79 @@ __global__ __launch_bounds__(LA_THREADS) void eig_kernel(c64 *h_all, c64 *q_all,
     const int col_end = wantv ? n : hi + 1, row_begin = wantv ? 0 : lo;
     for (int i = lo + threadIdx.x; i <= hi; i += blockDim.x) H[(size_t)i * n + i] = H[(size_t)i * n + i] - mu;
     __syncthreads();
-    for (int k = lo; k < hi; k++) {
-      double c;
-      c64 s;
-      givens(H[(size_t)k * n + k], H[(size_t)(k + 1) * n + k], &c, &s);
-      __syncthreads();  // every lane has read the pivot pair before it changes
-      if (threadIdx.x == 0) {
-        cs[k] = c;
-        vec[k] = s;
+    // G_k ... G_lo (H - mu): rotation k needs the pivot H[k][k] as the rotations before it
+    // left it, and nothing else that changes: the subdiagonal is still the sweep's
+    // original (kept in LDS), and a lane that owns column j carries row k's element
+    // of its column from step to step in a register, so the only memory on the
+    // chain from one rotation to the next is a two-slot mailbox in LDS for the
+    // pivot. Row k + 1 of a column is read one step ahead of its use.
+    {
+      constexpr int CPT = LA_MAX_N / 2 / LA_THREADS;  // columns per lane
+      c64 carry[CPT], ynext[CPT];
+      for (int k = lo + threadIdx.x; k < hi; k += blockDim.x) sub[k] = H[(size_t)(k + 1) * n + k];
+#pragma unroll
+      for (int m = 0; m < CPT; m++) {
+        const int j = threadIdx.x + m * LA_THREADS;
+        carry[m] = ynext[m] = zero;
+        if (j >= lo && j < col_end) {
+          carry[m] = H[(size_t)lo * n + j];
+          ynext[m] = H[(size_t)(lo + 1) * n + j];
+        }
       }
-      for (int j = k + threadIdx.x; j < col_end; j += blockDim.x) {
-        const c64 x = H[(size_t)k * n + j], y = H[(size_t)(k + 1) * n + j];
-        H[(size_t)k * n + j] = c64{x.re * c, x.im * c} + s * y;
-        H[(size_t)(k + 1) * n + j] = c64{y.re * c, y.im * c} - c64{s.re, -s.im} * x;
+      if (threadIdx.x == 0) s_pivot[lo & 1] = H[(size_t)lo * n + lo];
+      for (int k = lo; k < hi; k++) {
+        __syncthreads();
+        double c;
+        c64 s;
+        givens(s_pivot[k & 1], sub[k], &c, &s);
+        if (threadIdx.x == 0) {
+          cs[k] = c;
+          vec[k] = s;
+        }
+#pragma unroll
+        for (int m = 0; m < CPT; m++) {
+          const int j = threadIdx.x + m * LA_THREADS;
+          if (j < k || j >= col_end) continue;
+          const c64 x = carry[m], y = ynext[m];
+          if (k + 2 <= hi && j >= k + 1) ynext[m] = H[(size_t)(k + 2) * n + j];
+          H[(size_t)k * n + j] = c64{x.re * c, x.im * c} + s * y;
+          const c64 low = c64{y.re * c, y.im * c} - c64{s.re, -s.im} * x;
+          carry[m] = low;
+          if (j == k) H[(size_t)(k + 1) * n + k] = low;
+          if (j == k + 1) s_pivot[(k + 1) & 1] = low;
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < CPT; m++) {
+        const int j = threadIdx.x + m * LA_THREADS;
+        if (j >= hi && j < col_end) H[(size_t)hi * n + j] = carry[m];
       }
       __syncthreads();
     }
-    // R G_lo^H G_{lo+1}^H ...: row i takes the rotations in order, no lane depends on another
-    for (int i = row_begin + threadIdx.x; i <= hi; i += blockDim.x) {
-      c64 *row = H + (size_t)i * n;
-      for (int k = (i - 1 > lo ? i - 1 : lo); k < hi; k++) {
-        const double c = cs[k];
-        const c64 s = vec[k];
-        const c64 x = row[k], y = row[k + 1];
-        row[k] = c64{x.re * c, x.im * c} + y * c64{s.re, -s.im};
-        row[k + 1] = c64{y.re * c, y.im * c} - x * s;
-      }
-    }
-    if (wantv) {
-      for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        c64 *row = Q + (size_t)i * n;
-        for (int k = lo; k < hi; k++) {
-          const double c = cs[k];
-          const c64 s = vec[k];
-          const c64 x = row[k], y = row[k + 1];
-          row[k] = c64{x.re * c, x.im * c} + y * c64{s.re, -s.im};
-          row[k + 1] = c64{y.re * c, y.im * c} - x * s;
+    // R G_lo^H G_{lo+1}^H ...: row i takes the rotations in order, no lane depends on
+    // another. The element that moves along the row stays in a register and the
+    // row is read eight elements ahead, so that no rotation waits for memory.
+    auto rotate_row = [&](c64 *row, int kstart) {
+      c64 x = row[kstart];
+      for (int k = kstart; k < hi; k += 8) {
+        c64 yb[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+          if (k + u < hi) yb[u] = row[k + 1 + u];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          if (k + u >= hi) break;
+          const double c = cs[k + u];
+          const c64 s = vec[k + u];
+          row[k + u] = c64{x.re * c, x.im * c} + yb[u] * c64{s.re, -s.im};
+          x = c64{yb[u].re * c, yb[u].im * c} - x * s;
         }
       }
-    }
+      row[hi] = x;
+    };
+    for (int i = row_begin + threadIdx.x; i <= hi; i += blockDim.x) rotate_row(H + (size_t)i * n, i - 1 > lo ? i - 1 : lo);
+    if (wantv)
+      for (int i = threadIdx.x; i < n; i += blockDim.x) rotate_row(Q + (size_t)i * n, lo);
     __syncthreads();
     for (int i = lo + threadIdx.x; i <= hi; i += blockDim.x) H[(size_t)i * n + i] = H[(size_t)i * n + i] + mu;
     __syncthreads();
@@ -1655,7 +1705,15 @@ NXH_EXPORT int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *
   nxh_tensor wh = workspace_tensor(x, H, NXH_C64, n, n, false);
   if ((rc = nxh_cast(ctx, &wh, x))) return rc;
   PathAtExit path{"eig_hessenberg_qr"};
-  LA_LAUNCH(ctx, eig_kernel, p.batch, (size_t)n * 24, (c64 *)H, (c64 *)Q, (c64 *)Y, (c64 *)W, (c64 *)V, (int)n, v ? 1 : 0, la_status(ctx));
+  {
+    static std::once_flag once;
+    static hipError_t attr = hipSuccess;
+    std::call_once(once, [&] {
+      attr = hipFuncSetAttribute((const void *)eig_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LA_MAX_N / 2 * 40);
+    });
+    NXH_HIP(op, attr);
+  }
+  LA_LAUNCH(ctx, eig_kernel, p.batch, (size_t)n * 40, (c64 *)H, (c64 *)Q, (c64 *)Y, (c64 *)W, (c64 *)V, (int)n, v ? 1 : 0, la_status(ctx));
   if ((rc = la_collect(ctx, op))) return rc;
   nxh_tensor ww = workspace_tensor(x, W, NXH_C64, n, 0, false, 1);
   if ((rc = nxh_cast(ctx, w, &ww))) return rc;
