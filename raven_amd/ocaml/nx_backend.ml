@@ -106,7 +106,40 @@ external caml_unfold : ('a, 'b) t -> ('a, 'b) t -> int array -> int array -> int
 external caml_fold_window :
   ('a, 'b) t -> ('a, 'b) t -> int array -> int array -> int array -> int array -> int array -> unit
   = "caml_nx_hip_fold_bc" "caml_nx_hip_fold"
-(* ... one external per remaining unary / binary / compare stub, same shapes ... *)
+external caml_sub : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_sub"
+external caml_fdiv : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_fdiv"
+external caml_idiv : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_idiv"
+external caml_mod : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_mod"
+external caml_pow : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_pow"
+external caml_atan2 : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_atan2"
+external caml_max : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_max"
+external caml_min : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_min"
+external caml_xor : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_xor"
+external caml_or : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_or"
+external caml_and : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_and"
+external caml_neg : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_neg"
+external caml_recip : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_recip"
+external caml_abs : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_abs"
+external caml_sqrt : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_sqrt"
+external caml_sign : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_sign"
+external caml_exp : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_exp"
+external caml_log : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_log"
+external caml_cos : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_cos"
+external caml_tan : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_tan"
+external caml_asin : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_asin"
+external caml_acos : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_acos"
+external caml_atan : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_atan"
+external caml_sinh : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_sinh"
+external caml_cosh : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_cosh"
+external caml_tanh : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_tanh"
+external caml_trunc : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_trunc"
+external caml_ceil : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_ceil"
+external caml_floor : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_floor"
+external caml_round : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_round"
+external caml_erf : ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_erf"
+external caml_cmpeq : (bool, Dtype.bool_elt) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_cmpeq"
+external caml_cmpne : (bool, Dtype.bool_elt) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_cmpne"
+external caml_cmple : (bool, Dtype.bool_elt) t -> ('a, 'b) t -> ('a, 'b) t -> unit = "caml_nx_hip_cmple"
 
 let unary op x = let out = create_tensor x.context x.dtype x.shape in op out x; out
 let binary op x y = let out = create_tensor x.context x.dtype x.shape in op out x y; out
@@ -116,6 +149,40 @@ let add x y = binary caml_add x y
 let mul x y = binary caml_mul x y
 let sin x = unary caml_sin x
 let cmplt x y = comparison caml_cmplt x y
+let sub x y = binary caml_sub x y
+let fdiv x y = binary caml_fdiv x y
+let idiv x y = binary caml_idiv x y
+let mod_ x y = binary caml_mod x y
+let pow x y = binary caml_pow x y
+let atan2 x y = binary caml_atan2 x y
+let max x y = binary caml_max x y
+let min x y = binary caml_min x y
+let xor x y = binary caml_xor x y
+let or_ x y = binary caml_or x y
+let and_ x y = binary caml_and x y
+let neg x = unary caml_neg x
+let recip x = unary caml_recip x
+let abs x = unary caml_abs x
+let sqrt x = unary caml_sqrt x
+let sign x = unary caml_sign x
+let exp x = unary caml_exp x
+let log x = unary caml_log x
+let cos x = unary caml_cos x
+let tan x = unary caml_tan x
+let asin x = unary caml_asin x
+let acos x = unary caml_acos x
+let atan x = unary caml_atan x
+let sinh x = unary caml_sinh x
+let cosh x = unary caml_cosh x
+let tanh x = unary caml_tanh x
+let trunc x = unary caml_trunc x
+let ceil x = unary caml_ceil x
+let floor x = unary caml_floor x
+let round x = unary caml_round x
+let erf x = unary caml_erf x
+let cmpeq x y = comparison caml_cmpeq x y
+let cmpne x y = comparison caml_cmpne x y
+let cmple x y = comparison caml_cmple x y
 
 let where cond a b =
   let out = create_tensor a.context a.dtype a.shape in
