@@ -9,12 +9,15 @@
 //   probs  = cast dtype (softmax scores)                        -- frontend.ml:4242-4252
 //   out    = matmul probs v                                     -- dtype, f32 accumulation
 // with the same rounding points: products of 16-bit values are exact in the
-// f32 accumulator of v_mfma_f32_32x32x16, the scale is one f32 multiply, the
-// exponentials are the primitive's expf of (t - rowmax), each probability is
-// e / rowsum rounded to the 16-bit dtype BEFORE it meets v, and the output is
-// rounded once from the f32 accumulator. What differs from the op-by-op result
-// is the order of the f32 sums (scores, row sum, probs x v) and that the row sum
-// is accumulated tile by tile against a running maximum.
+// f32 accumulator of v_mfma_f32_32x32x16, the scale is one f32 multiply, each
+// probability is exp(t - rowmax) / rowsum rounded to the 16-bit dtype BEFORE it
+// meets v, and the output is rounded once from the f32 accumulator. What
+// differs from the op-by-op result: the order of the f32 sums (scores, row sum,
+// probs x v); the row sum is accumulated tile by tile against a running maximum;
+// the exponential is this file's six-instruction form (within 2 ulp, the
+// primitive's within 1) and the quotient one Newton step on e x (1 / rowsum),
+// which is the correctly rounded quotient in all but rare cases. Both sit far
+// below the 16-bit rounding that follows them.
 //
 // Layout of the work: a block of two wave64s owns two 64-query tiles of one
 // (batch, head), tile t and then tile T-1-t, so that every block meets the same
@@ -66,9 +69,40 @@ template <class EL>
 __device__ __forceinline__ uint16_t narrow(float x) {
   return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x);
 }
+template <class EL>
+__device__ __forceinline__ uint32_t narrow2(float lo, float hi) {
+  if constexpr (EL::BF16) return f32x2_to_bf16x2(lo, hi);
+  else return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
+}
 
 __device__ __forceinline__ float xor32(float v) {
   return __builtin_bit_cast(float, __shfl_xor(__builtin_bit_cast(int, v), 32, 64));
+}
+
+// e^x for the softmax of this kernel (x <= 0, -inf or NaN). The library's expf
+// costs about thirteen instructions a score, twice per score here, and bounded
+// the kernel. Six do: 2^(x log2 e) by the hardware exponential on the rounded
+// product p, times e^d for what the rounding of p dropped, d = x - p ln 2 in two
+// fused steps, e^d = 1 + d to 2^-39. Within 2 ulp of the exact value (the
+// primitive's expf is within 1), far inside the reference's tolerance for f32
+// transcendentals (rel 1e-4, backend_contract.ml:179-188). x = -inf has p = -inf,
+// r = 0 and d = inf - inf = NaN: the maximum drops that NaN (a true d is tiny),
+// so the result is 0; a NaN x gives NaN through r. Results below 2^-126 are
+// flushed to zero.
+__device__ __forceinline__ float exp_att(float x) {
+  const float p = x * 0x1.715476p+0f;
+  const float r = __builtin_amdgcn_exp2f(p);
+  float d = __builtin_fmaf(p, -0x1.62e400p-1f, x);  // ln 2 in two parts (0.693145751953125 + 1.4286068e-6)
+  d = __builtin_fmaf(p, -0x1.7f7d1cp-20f, d);
+  return __builtin_fmaf(r, __builtin_fmaxf(d, -1.0f), r);
+}
+
+// e / l with 1 / l at hand: one Newton step on the quotient (Markstein), which is
+// the correctly rounded e / l whenever rl is the correctly rounded reciprocal and
+// the quotient is a normal number; three instructions against the ten of a division.
+__device__ __forceinline__ float div_att(float e, float l, float rl) {
+  const float q = e * rl;
+  return __builtin_fmaf(__builtin_fmaf(-q, l, e), rl, q);
 }
 
 template <class EL, int DHEAD>
@@ -185,8 +219,11 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
   };
   prefetch(0, 0);
   for (int pass = 0; pass < 2; pass++) {
-    float l_total = 0.0f;
-    if (pass == 1) l_total = l_run + xor32(l_run);
+    float l_total = 0.0f, l_recip = 0.0f;
+    if (pass == 1) {
+      l_total = l_run + xor32(l_run);
+      l_recip = 1.0f / l_total;
+    }
     for (int kt = 0; kt < ktiles; kt++) {
       __syncthreads();  // the previous tile has been consumed
 #pragma unroll
@@ -207,16 +244,25 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
         float t[16];
         scores(j0, t, j0 + 32 <= a.sk && !a.has_mask && (!a.causal || j0 + 31 <= qw));
         if (pass == 0) {
+          // The hardware maximum skips NaNs; a NaN score reaches the row through the
+          // sum of exponentials instead (every probability of the row is then NaN, as
+          // after the primitive's NaN-keeping max), or through the scan below while
+          // nothing of the row has been visible yet.
           float tm = t[0];
 #pragma unroll
-          for (int e = 1; e < 16; e++) tm = MX::apply(tm, t[e]);
-          float m_new = MX::apply(m_run, tm);
-          m_new = MX::apply(m_new, xor32(m_new));  // both halves of a query agree on the maximum
+          for (int e = 1; e < 16; e++) tm = __builtin_fmaxf(tm, t[e]);
+          float m_new = __builtin_fmaxf(m_run, tm);
+          m_new = __builtin_fmaxf(m_new, xor32(m_new));  // both halves of a query agree on the maximum
           if (m_new != -__builtin_inff()) {
             float s = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 16; e++) s = s + OpExp::eval<CAT_FLOAT, float>(t[e] - m_new);
-            l_run = l_run * OpExp::eval<CAT_FLOAT, float>(m_run - m_new) + s;
+            for (int e = 0; e < 16; e++) s = s + exp_att(t[e] - m_new);
+            l_run = l_run * exp_att(m_run - m_new) + s;
+          } else {
+            bool nan = false;
+#pragma unroll
+            for (int e = 0; e < 16; e++) nan = nan || t[e] != t[e];
+            if (nan) l_run = __builtin_nanf("");
           }
           m_run = m_new;
         } else {
@@ -224,9 +270,9 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
           uint32_t pk[8];
 #pragma unroll
           for (int e = 0; e < 16; e += 2) {
-            const float p0 = OpExp::eval<CAT_FLOAT, float>(t[e] - m_run) / l_total;
-            const float p1 = OpExp::eval<CAT_FLOAT, float>(t[e + 1] - m_run) / l_total;
-            pk[e >> 1] = (uint32_t)narrow<EL>(p0) | ((uint32_t)narrow<EL>(p1) << 16);
+            const float p0 = div_att(exp_att(t[e] - m_run), l_total, l_recip);
+            const float p1 = div_att(exp_att(t[e + 1] - m_run), l_total, l_recip);
+            pk[e >> 1] = narrow2<EL>(p0, p1);
           }
           // B operand of O^T = V^T P^T for k-step ks: this lane's query, keys
           // ks*16 + g*8 + 0..7. The accumulator gave keys ks*16 + g*4 + 0..3 and
@@ -264,8 +310,8 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
       for (int e = 0; e < 16; e += 4) {
         const int d = ot * 32 + (e >> 2) * 8 + g * 4;
         uint2 w;
-        w.x = (uint32_t)narrow<EL>(oacc[ot][e]) | ((uint32_t)narrow<EL>(oacc[ot][e + 1]) << 16);
-        w.y = (uint32_t)narrow<EL>(oacc[ot][e + 2]) | ((uint32_t)narrow<EL>(oacc[ot][e + 3]) << 16);
+        w.x = narrow2<EL>(oacc[ot][e], oacc[ot][e + 1]);
+        w.y = narrow2<EL>(oacc[ot][e + 2], oacc[ot][e + 3]);
         *reinterpret_cast<uint2 *>(orow + d) = w;
       }
   }

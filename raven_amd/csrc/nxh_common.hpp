@@ -181,6 +181,17 @@ HD uint16_t f32_to_bf16(float f) {
 #endif
 }
 HD float bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+// Two neighbours narrowed by ONE v_cvt_pk_bf16_f32: `lo` in the low half.
+HD uint32_t f32x2_to_bf16x2(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  asm("" : "+v"(lo), "+v"(hi));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+#else
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+#endif
+}
 
 // f32 -> f16, nx_buffer_stubs.h:99-148. The hardware convert (round to nearest
 // even, subnormals kept) matches on every non-NaN input; a NaN keeps its top

@@ -96,6 +96,36 @@ def test_attention_on_head_split_views_and_special_rows(hip, oracle):
     assert np.all(np.abs(got - want) <= TOL[d.name][0] * (1 + np.abs(want)))
 
 
+def test_nan_scores_poison_exactly_the_rows_the_sequence_poisons(hip, oracle):
+    """A NaN in a key reaches every query that may see that key, a NaN in a query
+    its own row only, also when the NaN sits in the first keys of a row whose other
+    early keys are all masked (the running maximum is still -inf there)."""
+    rng = np.random.default_rng(11)
+    d, shape = dt.bfloat16, (1, 2, 160, 64)
+    s = shape[-2]
+    q, k, v = (rng.standard_normal(shape).astype(np.float32) for _ in range(3))
+    k[0, 0, 70, 3] = np.nan   # head 0: queries 70.. under the causal mask
+    q[0, 1, 5, 0] = np.nan    # head 1: query 5 only
+    k[0, 1, 2, 9] = np.nan    # head 1: key 2, visible from query 2 on causally; masked below for most rows
+    q, k, v = (encode(x, d, oracle) for x in (q, k, v))
+    (hq, oq), (hk, ok), (hv, ov) = (pair(x, d, hip, oracle) for x in (q, k, v))
+    m = np.tril(np.ones((s, s), np.uint8))
+    m[40:, :33] = 0           # rows 40.. see nothing of the first 33 keys: the NaN key 2 is masked for them
+    m[100, :] = 0
+    m[100, 2] = 1             # row 100 sees only the NaN key
+    sshape = shape[:-1] + (s,)
+    hm, om = bool_mask(hip, m, sshape), bool_mask(oracle, m, sshape)
+    for name, kw_h, o_mask in (("causal", {"causal": True, "masked_value": float("-inf")}, bool_mask(oracle, np.tril(np.ones((s, s), np.uint8)), sshape)),
+                               ("mask", {"mask": hm, "masked_value": float("-inf")}, om)):
+        got = logical(hip.attention(hq, hk, hv, 0.125, **kw_h))
+        assert hip.last_path() == "attention_fused"
+        want = logical(sequence(oracle, oq, ok, ov, o_mask))
+        gv, wv = decode(got, d, oracle), decode(want, d, oracle)
+        assert np.array_equal(np.isnan(gv), np.isnan(wv)), name
+        assert np.isnan(wv).any() and not np.isnan(wv).all()
+        close(got, want, d, oracle, TOL[d.name][0], TOL[d.name][0], "NaN scores, " + name)
+
+
 def test_attention_errors(hip):
     q = hip.full(dt.bfloat16, (2, 16, 64), 1.0)
     with pytest.raises(RuntimeError):
