@@ -96,6 +96,27 @@ def test_attention_on_head_split_views_and_special_rows(hip, oracle):
     assert np.all(np.abs(got - want) <= TOL[d.name][0] * (1 + np.abs(want)))
 
 
+@pytest.mark.parametrize("sq,sk,hd", [(70, 200, 64), (1, 333, 32), (129, 31, 128)])
+def test_more_or_fewer_keys_than_queries(hip, oracle, sq, sk, hd):
+    """Cross attention: the key count differs from the query count (no causal form there)."""
+    rng = np.random.default_rng(sq + sk)
+    d = dt.float16
+    q = encode(rng.standard_normal((2, 2, sq, hd)), d, oracle)
+    k, v = (encode(rng.standard_normal((2, 2, sk, hd)), d, oracle) for _ in range(2))
+    (hq, oq), (hk, ok), (hv, ov) = (pair(x, d, hip, oracle) for x in (q, k, v))
+    m = (rng.random((sq, sk)) < 0.6).astype(np.uint8)
+    m[:, sk // 2] = 1
+    hm, om = bool_mask(hip, m, (2, 2, sq, sk)), bool_mask(oracle, m, (2, 2, sq, sk))
+    scale = 1.0 / math.sqrt(hd)
+    for name, kw, o_mask in (("mask", {"mask": hm, "masked_value": float("-inf")}, om), ("none", {}, None)):
+        got = logical(hip.attention(hq, hk, hv, scale, **kw))
+        assert hip.last_path() == "attention_fused"
+        want = logical(sequence(oracle, oq, ok, ov, o_mask))
+        close(got, want, d, oracle, TOL[d.name][0], TOL[d.name][0], f"{sq}x{sk}x{hd} {name}")
+        want_gpu = logical(sequence(hip, hq, hk, hv, hm if o_mask is not None else None))
+        close(got, want_gpu, d, oracle, 2 * ULP[d.name], 2e-3, f"{sq}x{sk}x{hd} {name} vs GPU sequence")
+
+
 def test_nan_scores_poison_exactly_the_rows_the_sequence_poisons(hip, oracle):
     """A NaN in a key reaches every query that may see that key, a NaN in a query
     its own row only, also when the NaN sits in the first keys of a row whose other
