@@ -108,12 +108,9 @@ def to_device(context, t):
     as it is; one of another context of this GPU is copied by a kernel of the
     target context, through its view, after the source context's stream has
     drained, and the target's stream is drained before returning so that the
-    source may be released at once. A deferred tensor is filled into ``context``."""
-    if isinstance(t, Deferred):
-        if t.forced is None and t.context is not context:
-            d = Deferred(context, t.dtype, t._view.shape, t._fill)
-            return force(d)
-        t = force(t)
+    source may be released at once. A deferred tensor is forced first (its fill
+    runs at most once, whoever asks)."""
+    t = unwrap(t)
     if t.context is context:
         return t
     t.context.synchronize()

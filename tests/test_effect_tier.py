@@ -62,9 +62,10 @@ def test_const_scalar_to_device_and_deferred_on_the_gpu(hip):
 
         d = E.deferred(hip, dt.int32, x.shape, fill)
         assert E.view(d).shape == x.shape and not calls
-        moved = E.to_device(other, d)  # filled straight into the target context
+        moved = E.to_device(other, d)  # forced in its own context, then copied
         assert moved.context is other and calls == [1]
         same_bits(logical(moved), x)
+        assert E.unwrap(d).context is hip and calls == [1]  # the fill ran once, whoever asked
         same_bits(E.to_host(E.deferred(hip, dt.int32, x.shape, fill)).reshape(x.shape), x)
     finally:
         del u, v, moved
