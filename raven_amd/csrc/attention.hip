@@ -36,6 +36,7 @@
 // indices and key tiles above the diagonal are skipped.
 
 #include "fold_common.hpp"
+#include "softmax_math.hpp"
 #include "gemm_tile.hpp"
 #include "map_ops.hpp"
 
@@ -77,32 +78,6 @@ __device__ __forceinline__ uint32_t narrow2(float lo, float hi) {
 
 __device__ __forceinline__ float xor32(float v) {
   return __builtin_bit_cast(float, __shfl_xor(__builtin_bit_cast(int, v), 32, 64));
-}
-
-// e^x for the softmax of this kernel (x <= 0, -inf or NaN). The library's expf
-// costs about thirteen instructions a score, twice per score here, and bounded
-// the kernel. Six do: 2^(x log2 e) by the hardware exponential on the rounded
-// product p, times e^d for what the rounding of p dropped, d = x - p ln 2 in two
-// fused steps, e^d = 1 + d to 2^-39. Within 2 ulp of the exact value (the
-// primitive's expf is within 1), far inside the reference's tolerance for f32
-// transcendentals (rel 1e-4, backend_contract.ml:179-188). x = -inf has p = -inf,
-// r = 0 and d = inf - inf = NaN: the maximum drops that NaN (a true d is tiny),
-// so the result is 0; a NaN x gives NaN through r. Results below 2^-126 are
-// flushed to zero.
-__device__ __forceinline__ float exp_att(float x) {
-  const float p = x * 0x1.715476p+0f;
-  const float r = __builtin_amdgcn_exp2f(p);
-  float d = __builtin_fmaf(p, -0x1.62e400p-1f, x);  // ln 2 in two parts (0.693145751953125 + 1.4286068e-6)
-  d = __builtin_fmaf(p, -0x1.7f7d1cp-20f, d);
-  return __builtin_fmaf(r, __builtin_fmaxf(d, -1.0f), r);
-}
-
-// e / l with 1 / l at hand: one Newton step on the quotient (Markstein), which is
-// the correctly rounded e / l whenever rl is the correctly rounded reciprocal and
-// the quotient is a normal number; three instructions against the ten of a division.
-__device__ __forceinline__ float div_att(float e, float l, float rl) {
-  const float q = e * rl;
-  return __builtin_fmaf(__builtin_fmaf(-q, l, e), rl, q);
 }
 
 template <class EL, int DHEAD>
@@ -247,8 +222,8 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
           if (m_new != -__builtin_inff()) {
             float s = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 16; e++) s = s + exp_att(t[e] - m_new);
-            l_run = l_run * exp_att(m_run - m_new) + s;
+            for (int e = 0; e < 16; e++) s = s + exp_nonpositive(t[e] - m_new);
+            l_run = l_run * exp_nonpositive(m_run - m_new) + s;
           } else {
             bool nan = false;
 #pragma unroll
@@ -261,8 +236,8 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
           uint32_t pk[8];
 #pragma unroll
           for (int e = 0; e < 16; e += 2) {
-            const float p0 = div_att(exp_att(t[e] - m_run), l_total, l_recip);
-            const float p1 = div_att(exp_att(t[e + 1] - m_run), l_total, l_recip);
+            const float p0 = div_by_reciprocal(exp_nonpositive(t[e] - m_run), l_total, l_recip);
+            const float p1 = div_by_reciprocal(exp_nonpositive(t[e + 1] - m_run), l_total, l_recip);
             pk[e >> 1] = narrow2<EL>(p0, p1);
           }
           // B operand of O^T = V^T P^T for k-step ks: this lane's query, keys

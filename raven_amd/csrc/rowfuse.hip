@@ -23,6 +23,7 @@
 #include <cmath>
 
 #include "fold_common.hpp"
+#include "softmax_math.hpp"
 #include "map_ops.hpp"
 
 namespace {
@@ -140,6 +141,12 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
     }
   }
   const C scale = (C)a.scale, masked = (C)a.masked;
+  // float32 scores narrowed to 16 bits on the way out (the probabilities of an
+  // attention): the exponential, the quotient and the maximum take the short forms
+  // of softmax_math.hpp, whose differences from the primitives' disappear under
+  // the narrowing in all but rare elements. The hardware maximum skips NaNs; a
+  // NaN element still turns the whole row into NaNs through the sum.
+  constexpr bool SHORT = DTX == NXH_F32 && (DTO == NXH_BF16 || DTO == NXH_F16);
   C m = Combine<NXH_RMAX, C, CAT_FLOAT>::init();
 #pragma unroll
   for (int v = 0; v < NV; v++) {
@@ -150,7 +157,8 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
         if (a.has_scale) e = rnd<DTX>(OpMul::eval<CAT_FLOAT, C>(e, scale));
         if (a.has_mask) e = mk[v].v[j] != 0 ? e : masked;
         t[v][j] = e;
-        m = Combine<NXH_RMAX, C, CAT_FLOAT>::apply(m, e);
+        if constexpr (SHORT) m = __builtin_fmaxf(m, e);
+        else m = Combine<NXH_RMAX, C, CAT_FLOAT>::apply(m, e);
       }
     }
   }
@@ -162,13 +170,17 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
 #pragma unroll
       for (int j = 0; j < V; j++) {
         const C d = rnd<DTX>(OpSub::eval<CAT_FLOAT, C>(t[v][j], m));
-        const C e = rnd<DTX>(OpExp::eval<CAT_FLOAT, C>(d));
+        C e;
+        if constexpr (SHORT) e = exp_nonpositive(d);
+        else e = rnd<DTX>(OpExp::eval<CAT_FLOAT, C>(d));
         t[v][j] = e;
         s = s + e;
       }
     }
   }
   s = rnd<DTX>(row_combine<NXH_SUM, C, RW>(s, lds));
+  C s_recip = 0;
+  if constexpr (SHORT) s_recip = 1.0f / s;
 #pragma unroll
   for (int v = 0; v < NV; v++) {
     const int c = v * T + tid;
@@ -176,7 +188,9 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
       Pk<SO, V> o;
 #pragma unroll
       for (int j = 0; j < V; j++) {
-        const C y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t[v][j], s));
+        C y;
+        if constexpr (SHORT) y = div_by_reciprocal(t[v][j], s, s_recip);
+        else y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t[v][j], s));
         o.v[j] = TO::st((typename TO::C)y);
       }
       *reinterpret_cast<Pk<SO, V> *>(out + (int64_t)c * V) = o;
