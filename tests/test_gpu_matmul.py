@@ -211,6 +211,15 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
     assert hip.last_path() == "gemm_tile_128x128"
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "odd N, row-major B")
     assert hip.last_path() == "gemm_mfma"
+    # odd N on every block shape: the rows of C start at every 2-byte alignment, and 16-bit
+    # results leave as 16-byte stores at the aligned addresses plus single elements at the ends
+    for (m, k, n, path) in [(4000, 64, 4087, "gemm_tile_256x256"), (264, 128, 57, "gemm_tile_256x64"),
+                            (203, 192, 1031, "gemm_tile_128x128"), (131, 64, 9, "gemm_tile_256x64")]:
+        a = encode(rng.standard_normal((m, k)), d, oracle)
+        b = encode(rng.standard_normal((k, n)), d, oracle)
+        hb, _ = pair(np.ascontiguousarray(b.T), d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))
+        check(hip, oracle, d, pair(a, d, hip, oracle)[0], hb, a, b, f"odd N {m}x{k}x{n}")
+        assert hip.last_path() == path, (m, k, n, hip.last_path())
     a = encode(rng.standard_normal((3, 2, 256, 128)), d, oracle)
     b = encode(rng.standard_normal((128, 512)), d, oracle)
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "big batched x broadcast W")
