@@ -71,13 +71,16 @@ typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t V16;  // one 16-byte register quad
 
 // Tile geometry in elements of EL. PK: pitch of a [row][k] tile (+16 B). The
-// [k][row] pitch adds 64 B for 256-row 16-bit tiles, 32 B otherwise (two 128x128
-// blocks then fit one CU's LDS; for f32 it puts the two k-rows a wave reads at
-// once 32 banks apart).
+// [k][row] pitch adds 64 B for 16-bit tiles: the four k-rows a half-wave's
+// transposing read touches then start 16 banks apart and its 32 lanes cover all 64
+// banks once (with 32 B a 128-row tile's k-rows were 8 banks apart and met the
+// lanes 16 rows further on: a fifth of its LDS cycles were bank conflicts); two
+// 128x128 blocks still fit one CU's LDS. For f32 it adds 32 B, which puts the two
+// k-rows a wave reads at once 32 banks apart.
 template <class EL>
 struct Geo {
   static constexpr int VE = EL::VE, BK = 8 * VE, PK = BK + VE;
-  static constexpr int padr(int rows) { return (!EL::F32 && rows >= 256) ? 4 * VE : 2 * VE; }
+  static constexpr int padr(int) { return EL::F32 ? 2 * VE : 4 * VE; }
   static constexpr int tile_elems(int rows) {
     return rows * PK > BK * (rows + padr(rows)) ? rows * PK : BK * (rows + padr(rows));
   }
