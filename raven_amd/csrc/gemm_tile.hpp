@@ -381,7 +381,7 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
             patch[(t * 32 + (e >> 2) * 8 + kg * 4 + (e & 3)) * WP + u * 32 + r32] = narrow(acc[t][u][e]);
       // the patch is read back by other lanes of the same wave only: LDS serves a wave in order
       constexpr int CPR = WC / 8;  // 16-byte chunks per patch row
-      if constexpr (EPI && !EDGE && EL::BF16) {
+      if constexpr (EPI && !EDGE) {
         // Whole tiles of the fused linear: a lane keeps one column chunk for all its rows,
         // so the bias is read once, and every residual chunk is requested before the
         // first one is used. (Written as one loop with the loads where they are
@@ -390,10 +390,17 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
         static_assert(64 % CPR == 0, "a lane's chunk column is the same in every pass");
         constexpr int NIT = TM * 32 * CPR / 64, RSTEP = 64 / CPR;
         const int col = (lane % CPR) * 8, row0 = lane / CPR;
-        auto add2 = [](uint32_t x, uint32_t y) {
-          const float lo = __builtin_bit_cast(float, x << 16) + __builtin_bit_cast(float, y << 16);
-          const float hi = __builtin_bit_cast(float, x & 0xffff0000u) + __builtin_bit_cast(float, y & 0xffff0000u);
-          return f32x2_to_bf16x2(lo, hi);
+        // two neighbours per register: bf16 is widened by a shift and a mask and narrowed by one conversion
+        auto add2 = [&](uint32_t x, uint32_t y) -> uint32_t {
+          if constexpr (EL::BF16) {
+            const float lo = __builtin_bit_cast(float, x << 16) + __builtin_bit_cast(float, y << 16);
+            const float hi = __builtin_bit_cast(float, x & 0xffff0000u) + __builtin_bit_cast(float, y & 0xffff0000u);
+            return f32x2_to_bf16x2(lo, hi);
+          } else {
+            const S lo = narrow(widen((S)(x & 0xffffu)) + widen((S)(y & 0xffffu)));
+            const S hi = narrow(widen((S)(x >> 16)) + widen((S)(y >> 16)));
+            return (uint32_t)lo | ((uint32_t)hi << 16);
+          }
         };
         S *c = C + (m0 + wm + row0) * a.ldc + n0 + wn + col;
         const S *p = patch + row0 * WP + col;
