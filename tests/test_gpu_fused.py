@@ -84,6 +84,12 @@ def test_softmax_rows_special_values_and_errors(hip, oracle):
     assert np.array_equal(np.isnan(got), np.isnan(want))
     assert np.allclose(got[~np.isnan(got)], want[~np.isnan(want)], rtol=1e-6)
     assert np.isnan(got[1]).all() and np.isnan(got[2]).all() and np.isnan(got[5]).all()
+    # the 16-bit outputs take the short exponential, quotient and hardware maximum: same NaN rows
+    for od in (dt.bfloat16, dt.float16):
+        got16 = decode(logical(hip.softmax_rows(hx, None, hm, float("-inf"), od)), od, oracle)
+        want16 = decode(logical(softmax_sequence(oracle, ox, None, om, od)), od, oracle)
+        assert np.array_equal(np.isnan(got16), np.isnan(want16)), od.name
+        assert np.allclose(got16[~np.isnan(got16)], want16[~np.isnan(want16)], rtol=2 * ULP[od.name], atol=1e-30)
     # a masked value other than -inf, taken as given
     got = logical(hip.softmax_rows(hx, 2.0, hm, -1e4))
     nx = Nx(oracle)
