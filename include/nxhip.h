@@ -173,6 +173,21 @@ int nxh_cast(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x);
    squeezed result or the keepdims-shaped one (nx_c_engine.c:1392-1420). */
 int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out,
                const nxh_tensor *x, const int32_t *axes, int n_axes);
+/* No counterpart in the reference. nxh_reduce for callers that cannot allocate
+   (code under HIP graph capture by the caller's own stream machinery, tight
+   serving loops, harnesses that forbid hipMalloc): the same kernels, the same
+   split, bit-identical results, but the partial results of a split reduction
+   live in a static device array of NXH_STATIC_WORKSPACE_BYTES that every GPU
+   the library runs on holds until the process ends, so the call allocates and
+   frees nothing. A reduction whose partials would not fit is refused with
+   Failure before anything is launched (it needs at most
+   splits * outputs * sizeof(accumulator) bytes; e.g. float32 [8192,8192] over
+   axis 0 takes 2 MiB). All calls on one GPU share that array: calls on one
+   context are ordered by its stream, calls that overlap on one GPU from
+   different contexts race. */
+#define NXH_STATIC_WORKSPACE_BYTES (8u << 20)
+int nxh_reduce_noalloc(nxh_context *ctx, int op, const nxh_tensor *out,
+                       const nxh_tensor *x, const int32_t *axes, int n_axes);
 /* caml_nx_c_arg{max,min} (nx_c_fold.c:832-833; nx_c_engine.c:1214-1254):
    int32 output; is_min = 0 for argmax, 1 for argmin. */
 int nxh_argreduce(nxh_context *ctx, int is_min, const nxh_tensor *out,
@@ -385,7 +400,7 @@ int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nx
      (the result) is overwritten by every replay, and its block returns to the
      allocator only after both nxh_free and nxh_graph_destroy. Storage that
      existed before (weights, inputs) is read at replay time as it then is:
-     write new inputs into the same buffers (nxh_assign / nxh_memcpy_h2d)
+     write new inputs into the same buffers (nxh_copy / nxh_memcpy_h2d)
      before a replay.
    - nxh_memcpy_h2d of up to 256 KiB is recorded with a private copy of the
      bytes. nxh_memcpy_d2h, nxh_synchronize, nxh_trim and the timer fail while

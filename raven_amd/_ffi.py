@@ -81,6 +81,7 @@ SIGNATURES = {
     "nxh_where": (C.c_int, [_CTX, _T, _T, _T, _T]),
     "nxh_cast": (C.c_int, [_CTX, _T, _T]),
     "nxh_reduce": (C.c_int, [_CTX, C.c_int, _T, _T, _P(C.c_int32), C.c_int]),
+    "nxh_reduce_noalloc": (C.c_int, [_CTX, C.c_int, _T, _T, _P(C.c_int32), C.c_int]),
     "nxh_argreduce": (C.c_int, [_CTX, C.c_int, _T, _T, C.c_int]),
     "nxh_matmul": (C.c_int, [_CTX, _T, _T, _T]),
     "nxh_copy": (C.c_int, [_CTX, _T, _T]),

@@ -223,7 +223,7 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
   const S *ibase = (const S *)in->data + in->offset;
   S *obase = (S *)out->data + out->offset;
   const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
-  Scratch scratch(ctx);
+  Scratch scratch(ctx, g.fixed_scratch);
 
   // ---- fold_row: one unit-stride reduced run ----
   if (g.nr == 1 && g.rin[0] == 1 && g.R >= 64 && g.n_out <= 0x7fffffffLL * 4) {
@@ -424,8 +424,8 @@ static void storage_one(int dt, void *buf) {
   }
 }
 
-NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
-                          const int32_t *axes, int n_axes) {
+static int reduce_entry(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
+                        const int32_t *axes, int n_axes, bool fixed_scratch) {
   static const char *const names[NXH_REDUCE_COUNT] = {"reduce_sum", "reduce_prod", "reduce_max", "reduce_min"};
   if ((unsigned)op >= NXH_REDUCE_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "reduce", "unknown op");
   const char *name = names[op];
@@ -448,6 +448,7 @@ NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const
   if (out->dtype != dt) return nxh_fail(NXH_FAILURE, name, NXH_ERR_UNSUPPORTED);
   Geom g;
   geom_build(x, &sq, reduced, &g);
+  g.fixed_scratch = fixed_scratch;
   if (g.n_out == 0) return NXH_OK;
   for (int j = 0; j < sq.ndim; j++)
     if (sq.shape[j] > 1 && sq.strides[j] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, name, NXH_ERR_OUT_ALIASED);
@@ -462,4 +463,18 @@ NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(name, hipSetDevice(ctx->device));
   return fn(ctx, name, x, &sq, g);
+}
+
+NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
+                          const int32_t *axes, int n_axes) {
+  return reduce_entry(ctx, op, out, x, axes, n_axes, false);
+}
+
+// The same reduction with the partial results of its split forms in the device's
+// static workspace: no allocation, no free, the same kernels and the same split,
+// so the result equals nxh_reduce's bit for bit. A split whose partials exceed
+// the workspace is refused before anything is launched.
+NXH_EXPORT int nxh_reduce_noalloc(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
+                                  const int32_t *axes, int n_axes) {
+  return reduce_entry(ctx, op, out, x, axes, n_axes, true);
 }

@@ -138,6 +138,7 @@ struct Geom {
   int64_t kshape[NXH_MAX_NDIM], kin[NXH_MAX_NDIM], kout[NXH_MAX_NDIM];
   int64_t rshape[NXH_MAX_NDIM], rin[NXH_MAX_NDIM];
   int64_t n_out = 1, R = 1;
+  bool fixed_scratch = false;  // partial results go to the static workspace (no allocation)
 };
 
 // Splits dims into kept / reduced (strides in elements), drops size-1 dims and
@@ -200,12 +201,25 @@ static void dims_contig_in(FoldDims *d, int64_t inner) {
   }
 }
 
+// Scratch blocks of one call. Normally they come from the context's allocator.
+// With `fixed` the single block is the device's static workspace instead:
+// nothing is allocated or freed, and a request beyond its size fails.
 struct Scratch {
   nxh_context *ctx;
+  bool fixed;
   void *p[2] = {nullptr, nullptr};
-  explicit Scratch(nxh_context *c) : ctx(c) {}
-  int get(int i, size_t bytes) { return nxh_alloc_locked(ctx, bytes, &p[i]); }
+  explicit Scratch(nxh_context *c, bool fixed_ = false) : ctx(c), fixed(fixed_) {}
+  int get(int i, size_t bytes) {
+    if (!fixed) return nxh_alloc_locked(ctx, bytes, &p[i]);
+    if (i != 0 || bytes > NXH_STATIC_WS_BYTES || !ctx->static_ws)
+      return nxh_fail(NXH_FAILURE, "reduce_noalloc",
+                      "the partial results of this reduction exceed the static workspace "
+                      "(NXH_STATIC_WORKSPACE_BYTES); use nxh_reduce");
+    p[0] = ctx->static_ws;
+    return NXH_OK;
+  }
   ~Scratch() {  // stream-ordered: queued kernels keep using the blocks safely
+    if (fixed) return;
     for (void *q : p)
       if (q) nxh_free_locked(ctx, q);
   }

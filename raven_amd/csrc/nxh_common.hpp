@@ -55,7 +55,13 @@ struct nxh_context {
   // twiddle and chirp tables of the transforms, by (kind, sign, length); freed with the context
   std::map<uint64_t, void *> device_tables;
   int deferred_faults = 0;  // live graphs whose gathers / scatters report at the next synchronize
+  // this device's copy of the library's static workspace (runtime.hip), for the
+  // entry point that may not allocate; shared by every context of the device
+  unsigned char *static_ws = nullptr;
 };
+
+// Size of the static per-device workspace behind nxh_reduce_noalloc.
+constexpr size_t NXH_STATIC_WS_BYTES = (size_t)NXH_STATIC_WORKSPACE_BYTES;
 
 // A captured sequence of launches (runtime.hip).
 struct nxh_graph {

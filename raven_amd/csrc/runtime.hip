@@ -32,6 +32,30 @@ int nxh_hip_fail(const char *op, hipError_t e) {
   return nxh_fail(NXH_FAILURE, op, buf);
 }
 
+// ── static workspace ───────────────────────────────────────────────────────
+// Device memory that exists from the moment the code object is loaded, one copy
+// per GPU, for the entry point that must not allocate (nxh_reduce_noalloc keeps
+// the partial results of a split reduction here). In host code the array's name
+// is only a handle for hipGetSymbolAddress: the device address is looked up once
+// per device, with that device current, and every launch is given that address.
+static __device__ __align__(256) unsigned char scratch[NXH_STATIC_WS_BYTES];
+
+static std::mutex scratch_mu;
+static unsigned char *scratch_ptr[64] = {};
+
+static hipError_t static_workspace(int device, unsigned char **out) {
+  std::lock_guard<std::mutex> g(scratch_mu);
+  if ((unsigned)device >= 64) return hipErrorInvalidDevice;
+  if (!scratch_ptr[device]) {
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    scratch_ptr[device] = (unsigned char *)p;
+  }
+  *out = scratch_ptr[device];
+  return hipSuccess;
+}
+
 NXH_EXPORT const char *nxh_last_error(nxh_context *) { return tls_error; }
 NXH_EXPORT const char *nxh_last_path(nxh_context *) { return tls_path; }
 
@@ -69,6 +93,7 @@ NXH_EXPORT int nxh_context_create(nxh_context **out) {
     e = hipEventCreateWithFlags(&ctx->stage_done[i], hipEventDisableTiming);
   if (e == hipSuccess) e = hipMemsetAsync(ctx->fault_flag, 0, 256, ctx->stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+  if (e == hipSuccess) e = static_workspace(dev, &ctx->static_ws);  // device `dev` is current
   if (e != hipSuccess) {
     delete ctx;
     return nxh_hip_fail("create_context", e);

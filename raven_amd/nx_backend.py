@@ -598,6 +598,16 @@ class Backend:
         self._check(self._lib.nxh_reduce(self._h, REDUCE_OPS.index(op), C.byref(o), C.byref(a), arr, len(axes)))
         return out
 
+    def reduce_noalloc(self, op: str, axes: Sequence[int], x: Tensor, out: Tensor) -> Tensor:
+        """`reduce` into a result the caller allocated beforehand, through the entry
+        point that neither allocates nor frees device memory (its split partials
+        live in the library's static per-device workspace)."""
+        axes = sorted(int(a) for a in axes)
+        arr = (C.c_int32 * max(len(axes), 1))(*axes)
+        o, a = out._desc(), x._desc()
+        self._check(self._lib.nxh_reduce_noalloc(self._h, REDUCE_OPS.index(op), C.byref(o), C.byref(a), arr, len(axes)))
+        return out
+
     def _argreduce(self, is_min: bool, x: Tensor, axis: int, keepdims: bool) -> Tensor:
         name = "argmin" if is_min else "argmax"
         if x.shape[axis] == 0:
