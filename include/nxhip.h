@@ -305,8 +305,9 @@ int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
    `scale` and `masked_value` are float32 elements in host memory (the scalars
    of the float32 island), scale may be NULL. Either `mask` (bool,
    [batch..., Sq, Sk], stride-0 broadcast allowed) or `causal` != 0 (mask[i][j]
-   = j <= i, generated; needs Sq == Sk; key tiles above the diagonal are
-   skipped), or neither. */
+   = j <= i, generated; needs Sq == Sk and *masked_value == -inf, since key
+   tiles above the diagonal are skipped; any other fill is Failure and the
+   caller passes the mask tensor), or neither. */
 int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q,
                   const nxh_tensor *k, const nxh_tensor *v, const void *scale,
                   const nxh_tensor *mask, const void *masked_value, int causal);

@@ -343,6 +343,12 @@ NXH_EXPORT int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_
     a.batches *= e;
   }
   if (causal && sq != sk) return nxh_fail(NXH_INVALID_ARGUMENT, op, "causal needs as many queries as keys");
+  // The causal form skips the key tiles above the diagonal, which equals the
+  // `where mask scores masked_value` of the sequence only when the masked scores
+  // vanish from the softmax, i.e. for -inf (what attention.ml fills in). Any other
+  // fill gives the hidden keys a weight: the caller passes the mask tensor then.
+  if (causal && !(*(const float *)masked_value == -__builtin_inff()))
+    return nxh_fail(NXH_FAILURE, op, "the causal form needs masked_value = -inf; pass the mask tensor for any other fill");
   if (a.batches == 0 || sq == 0) return NXH_OK;
   if (sk == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_EMPTY_REDUCE);
   if (sq > 0x3fffffff || sk > 0x3fffffff) return nxh_fail(NXH_FAILURE, op, "sequence longer than 2^30");

@@ -343,6 +343,13 @@ static int table_lookup(nxh_context *ctx, uint64_t key, size_t bytes, double2 **
     *fresh = false;
     return NXH_OK;
   }
+  // A table is filled by a kernel on the context's stream. While that stream is being
+  // recorded the fill would only be recorded too: the table would count as present with
+  // nothing in it, for every eager transform until the first replay, and every replay
+  // would rewrite a table that other work reads. So a length is never first used there.
+  if (ctx->capture)
+    return nxh_fail(NXH_FAILURE, "fft",
+                    "first use of this transform length while a graph is being captured: run it once eagerly first");
   void *p = nullptr;
   if (hipMalloc(&p, bytes ? bytes : 16) != hipSuccess) {
     (void)hipGetLastError();
@@ -354,11 +361,26 @@ static int table_lookup(nxh_context *ctx, uint64_t key, size_t bytes, double2 **
   return NXH_OK;
 }
 
+// Takes a table whose fill could not be queued out of the registry again.
+static void table_drop(nxh_context *ctx, uint64_t key) {
+  auto it = ctx->device_tables.find(key);
+  if (it == ctx->device_tables.end()) return;
+  (void)hipStreamSynchronize(ctx->stream);  // a fill kernel already queued may still write it
+  (void)hipFree(it->second);
+  ctx->device_tables.erase(it);
+}
+
 static int twiddles(nxh_context *ctx, int M, const double2 **out) {
   double2 *t;
   bool fresh;
   if (int rc = table_lookup(ctx, table_key(T_TWIDDLE, M, -1), (size_t)(M / 2) * sizeof(double2), &t, &fresh)) return rc;
-  if (fresh && M >= 2) hipLaunchKernelGGL(twiddle_kernel, dim3((M / 2 + 255) / 256), dim3(256), 0, ctx->stream, t, M);
+  if (fresh && M >= 2) {
+    hipLaunchKernelGGL(twiddle_kernel, dim3((M / 2 + 255) / 256), dim3(256), 0, ctx->stream, t, M);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) {
+      table_drop(ctx, table_key(T_TWIDDLE, M, -1));
+      return nxh_hip_fail("fft", e);
+    }
+  }
   *out = t;
   return NXH_OK;
 }
@@ -449,14 +471,28 @@ static int bluestein_tables(nxh_context *ctx, int64_t n, int64_t M, int sign, co
   double2 *c, *f;
   bool fresh_c, fresh_f;
   if (int rc = table_lookup(ctx, table_key(T_CHIRP, n, sign), (size_t)n * sizeof(double2), &c, &fresh_c)) return rc;
-  if (fresh_c) hipLaunchKernelGGL(chirp_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, c, n, sign);
+  if (fresh_c) {
+    hipLaunchKernelGGL(chirp_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, c, n, sign);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) {
+      table_drop(ctx, table_key(T_CHIRP, n, sign));
+      return nxh_hip_fail("fft", e);
+    }
+  }
   if (int rc = table_lookup(ctx, table_key(T_FILTER, n, sign), (size_t)M * sizeof(double2), &f, &fresh_f)) return rc;
   if (fresh_f) {
+    // the filter counts as present only once every launch that fills it has been queued
     Scratch tmp{ctx};
-    if (int rc = nxh_alloc_locked(ctx, (size_t)M * sizeof(double2), &tmp.p[0])) return rc;
-    hipLaunchKernelGGL(chirp_filter_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, ctx->stream,
-                       (double2 *)tmp.p[0], c, n, M);
-    if (int rc = pow2_workspace(ctx, (double2 *)tmp.p[0], f, 1, M, -1)) return rc;
+    int rc = nxh_alloc_locked(ctx, (size_t)M * sizeof(double2), &tmp.p[0]);
+    if (!rc) {
+      hipLaunchKernelGGL(chirp_filter_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, ctx->stream,
+                         (double2 *)tmp.p[0], c, n, M);
+      if (hipError_t e = hipGetLastError(); e != hipSuccess) rc = nxh_hip_fail("fft", e);
+    }
+    if (!rc) rc = pow2_workspace(ctx, (double2 *)tmp.p[0], f, 1, M, -1);
+    if (rc) {
+      table_drop(ctx, table_key(T_FILTER, n, sign));
+      return rc;
+    }
   }
   *chirp = c;
   *bf = f;

@@ -1449,6 +1449,8 @@ NXH_EXPORT int nxh_cholesky(nxh_context *ctx, const nxh_tensor *out, const nxh_t
   if (rc) return rc;
   const int64_t n = p.rows;
   if (p.batch == 0 || n == 0) return NXH_OK;
+  // one factorisation at a time per context: they share the status word and its host slot
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
   if ((rc = la_begin(ctx, op))) return rc;
   Work work(ctx);
   void *A;
@@ -1486,6 +1488,8 @@ NXH_EXPORT int nxh_triangular_solve(nxh_context *ctx, const nxh_tensor *out, con
   const int64_t n = p.rows, nrhs = b->shape[b->ndim - 1];
   if ((rc = same_dims(op, b, a, n, nrhs)) || (rc = same_dims(op, out, a, n, nrhs))) return rc;
   if (p.batch == 0 || n == 0 || nrhs == 0) return NXH_OK;
+  // one factorisation at a time per context: they share the status word and its host slot
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
   if ((rc = la_begin(ctx, op))) return rc;
   Work work(ctx);
   void *A, *X;
@@ -1525,6 +1529,8 @@ NXH_EXPORT int nxh_qr(nxh_context *ctx, const nxh_tensor *q, const nxh_tensor *r
   if (m == 0 || n == 0) {  // nothing to factor: Q is the identity (if it has elements), R is empty
     if (m == 0 || nq == 0) return NXH_OK;
   }
+  // one factorisation at a time per context: they share the status word and its host slot
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
   if ((rc = la_begin(ctx, op))) return rc;
   Work work(ctx);
   void *At, *Qt, *tau;
@@ -1563,6 +1569,8 @@ NXH_EXPORT int nxh_eigh(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor 
   if (v && (rc = same_dims(op, v, x, n, n))) return rc;
   if (n > LA_MAX_N) return nxh_fail(NXH_FAILURE, op, "matrix too large (the limit is 4096)");
   if (p.batch == 0 || n == 0) return NXH_OK;
+  // one factorisation at a time per context: they share the status word and its host slot
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
   if ((rc = la_begin(ctx, op))) return rc;
   Work work(ctx);
   void *A, *V = nullptr, *Vs = nullptr, *W;
@@ -1615,6 +1623,8 @@ NXH_EXPORT int nxh_svd(nxh_context *ctx, const nxh_tensor *u, const nxh_tensor *
   if (k > LA_MAX_N) return nxh_fail(NXH_FAILURE, op, "matrix too large (the limit is 4096 on the shorter side)");
   if (p.batch == 0) return NXH_OK;
   if (k == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, "empty matrix");
+  // one factorisation at a time per context: they share the status word and its host slot
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
   if ((rc = la_begin(ctx, op))) return rc;
   // G = x (m >= n) or x^H (m < n): mm rows >= nn columns, column-major
   const bool flip = m < n;
@@ -1696,6 +1706,8 @@ NXH_EXPORT int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *
   if (v && (rc = same_dims(op, v, x, n, n))) return rc;
   if (n > LA_MAX_N / 2) return nxh_fail(NXH_FAILURE, op, "matrix too large (the limit is 2048)");
   if (p.batch == 0 || n == 0) return NXH_OK;
+  // one factorisation at a time per context: they share the status word and its host slot
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
   if ((rc = la_begin(ctx, op))) return rc;
   Work work(ctx);
   void *H, *Q = nullptr, *Y = nullptr, *W, *V = nullptr;

@@ -136,6 +136,7 @@ NXH_EXPORT int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
 
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
+  if (int frc = nxh_settle_replay_faults(ctx, op)) return frc;
   const char *dbase = (const char *)data->data + data->offset * es;
   char *obase = (char *)out->data + out->offset * es;
   const int32_t *ibase = (const int32_t *)indices->data + indices->offset;
@@ -482,6 +483,7 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
   if (!table[dt]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
+  if (int frc = nxh_settle_replay_faults(ctx, op)) return frc;
   // Too few columns to fill the chip and one index per axis position: split the
   // targets over blocks too. The index list is read once per block, so this
   // pays only while the list is short next to the rows it spreads over.

@@ -32,6 +32,9 @@ struct nxh_context {
   int compute_units = 0;
   char name[128] = {0};
   std::mutex mu;  // guards the allocator and launches: one stream per context
+  // held for the whole of a call made of several locked steps (the factorisations) and by
+  // capture_begin, so that no capture starts in the middle of one; taken before `mu`
+  std::mutex call_mu;
   // caching allocator: size class -> free blocks
   std::map<size_t, std::vector<void *>> free_lists;
   std::map<void *, size_t> live;  // every block handed out or cached -> its class size
@@ -89,6 +92,9 @@ int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out);
 void nxh_free_locked(nxh_context *ctx, void *p);
 // the out-of-bounds flag of gather / scatter, read back (or left for the replay) (runtime.hip)
 int nxh_collect_index_fault(nxh_context *ctx, const char *op);
+// Before an eager gather / scatter is launched: a fault that a replayed graph left in
+// the flag is reported now, as the replay's, so that this call answers only for itself.
+int nxh_settle_replay_faults(nxh_context *ctx, const char *op);
 
 // status strings shared with the reference (nx_c.h:381-388, nx_c_engine.h:38-50)
 #define NXH_ERR_NDIM "ndim exceeds NX_C_MAX_NDIM"

@@ -338,6 +338,11 @@ static int report_deferred_faults(nxh_context *ctx, const char *op) {
   return read_fault_flag(ctx, op, "index out of bounds in a replayed gather or scatter");
 }
 
+int nxh_settle_replay_faults(nxh_context *ctx, const char *op) {
+  if (ctx->capture) return NXH_OK;
+  return report_deferred_faults(ctx, op);
+}
+
 NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "to_host", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
@@ -384,6 +389,7 @@ static void graph_release(nxh_context *ctx, nxh_graph *gr) {
 
 NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "capture_begin", "null context");
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);  // not in the middle of a factorisation
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "capture_begin")) return rc;
   NXH_HIP("capture_begin", hipSetDevice(ctx->device));

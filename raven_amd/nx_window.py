@@ -646,7 +646,8 @@ def _match_attention(w: Window, anchor: Entry) -> Optional[Plan]:
     if mask is not None:
         n = qs[-2]
         flat = tuple(0 if s_ != 1 else st for s_, st in zip(sshape[:-2], mask.view.strides[:-2]))
-        if (mask.tag == ("causal", n) and ks[-2] == n and mask.view.offset == 0 and mask.view.strides[-2:] == (n, 1)
+        neg_inf = masked is not None and float(np.asarray(masked, dtype=np.float32).reshape(-1)[0]) == float("-inf")
+        if (neg_inf and mask.tag == ("causal", n) and ks[-2] == n and mask.view.offset == 0 and mask.view.strides[-2:] == (n, 1)
                 and all(st == 0 or s_ == 1 for s_, st in zip(sshape[:-2], mask.view.strides[:-2]))):
             causal, mask = True, None  # the kernel takes the mask as a flag (see Window.flush for the compare)
         del flat

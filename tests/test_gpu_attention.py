@@ -160,6 +160,8 @@ def test_attention_errors(hip):
     with pytest.raises(ValueError, match="causal"):
         hip.attention(q, hip.full(dt.bfloat16, (2, 8, 64), 1.0), hip.full(dt.bfloat16, (2, 8, 64), 1.0),
                       causal=True, masked_value=float("-inf"))
+    with pytest.raises(RuntimeError, match="-inf"):  # the causal form skips keys: only -inf may fill them
+        hip.attention(q, q, q, causal=True, masked_value=-1.0e4)
     with pytest.raises(RuntimeError, match="contiguous"):
         hip.attention(hip.permute(hip.full(dt.bfloat16, (2, 64, 16), 1.0), (0, 2, 1)), q, q)
     # uniform values: every key gets the same weight, the output is v's mean (here v itself)

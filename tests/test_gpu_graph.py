@@ -117,6 +117,14 @@ def test_index_fault_of_a_replay_surfaces_at_synchronize(hip):
         with pytest.raises(RuntimeError, match="index out of bounds"):
             hip.synchronize()
         hip.synchronize()  # reported once
+        # an eager gather issued behind a faulting replay reports the replay's fault as the
+        # replay's (before its own launch) and then answers for itself only
+        g.launch()
+        good = hip.reshape(hip.from_host(np.full(8, 3, np.int32), dt.int32), (1, 8))
+        with pytest.raises(RuntimeError, match="replayed gather or scatter"):
+            hip.gather(data, good, 0)
+        same_bits(logical(hip.gather(data, good, 0)), np.arange(24, 32, dtype=np.float32).reshape(1, 8))
+        hip.synchronize()
         hip.assign(idx, hip.reshape(hip.from_host(np.full(8, 7, np.int32), dt.int32), (1, 8)))
         g.launch()
         same_bits(logical(out), np.arange(56, 64, dtype=np.float32).reshape(1, 8))
@@ -155,3 +163,28 @@ def test_captured_gpt2_forward_replays_the_windowed_forward(hip, oracle, d):
     finally:
         g.destroy()
     assert np.all(np.isfinite(decode(eager[0], d, oracle)))
+
+
+def test_a_transform_length_is_never_first_used_inside_a_capture(hip, oracle):
+    """The twiddle / chirp tables of a transform are filled by kernels on the
+    context's stream. Inside a capture such a fill would only be recorded, and the
+    table would count as present while still empty: the first use of a length is
+    refused there, and the same length then works eagerly and in a later capture."""
+    rng = np.random.default_rng(77)
+    for n in (1536, 2 * 3 * 5 * 7 * 11):  # lengths no other test uses: a power-of-two-free one takes the chirp tables too
+        a = (rng.standard_normal((4, n)) + 1j * rng.standard_normal((4, n))).astype(np.complex64)
+        x = hip.reshape(hip.from_host(a, dt.complex64), a.shape)
+        ox = oracle.reshape(oracle.from_host(a, dt.complex64), a.shape)
+        with pytest.raises(RuntimeError, match="run it once eagerly"):
+            with capture(hip):
+                hip.fft(x, [1])
+        want = logical(oracle.fft(ox, [1]))
+        eager = logical(hip.fft(x, [1]))
+        assert np.all(np.abs(eager - want) <= 1e-4 * (1 + np.abs(want))), n
+        with capture(hip) as c:
+            out = hip.fft(x, [1])
+        for _ in range(2):
+            c.graph.launch()
+            hip.synchronize()
+            same_bits(logical(out), eager, f"replayed fft {n}")
+        c.graph.destroy()

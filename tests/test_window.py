@@ -245,6 +245,22 @@ def test_attention_run_and_what_blocks_it(oracle):
         got = value(w, run(w, kind))
         assert np.array_equal(got, ological(run(oracle, kind))), kind
         assert base.calls == [expect] and w.stats["attention"] == 1, (kind, base.calls)
+    # a finite fill gives the hidden keys a weight: the run still fuses, but with the mask
+    # tensor, never with the flag that lets the kernel skip the keys above the diagonal
+    def finite(B):
+        nx = Nx(B)
+        tq, tk, tv = (nx.create(d, a.shape, a) for a in (q, k, v))
+        idx = nx.arange(dt.int32, 0, s, 1)
+        mask = nx.less_equal(nx.reshape((1, s), idx), nx.reshape((s, 1), idx))
+        sc = nx.mul_s(nx.matmul(nx.cast(dt.float32, tq), nx.swapaxes(2, 3, nx.cast(dt.float32, tk))), 0.25)
+        sc = nx.where(mask, sc, nx.scalar_like(sc, -1.5))
+        return nx.matmul(nx.cast(d, nx.softmax(sc)), tv)
+
+    base = SequencedOracle()
+    w = Window(base)
+    got = value(w, finite(w))
+    assert np.array_equal(got, ological(finite(oracle)))
+    assert base.calls == ["attention"] and w.stats["attention"] == 1, base.calls
     base = SequencedOracle()
     w = Window(base)
     kept = []
