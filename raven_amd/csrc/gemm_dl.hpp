@@ -1,0 +1,228 @@
+// gemm_dl.hpp — the large-product form of the 16-bit tiled GEMM: 256 x 256 outputs per
+// block, operands fetched from global memory straight into LDS, v_mfma_f32_16x16x32.
+//
+// Same contract as gemm_tile.hpp (f32 accumulation, one rounding per output element,
+// batched with broadcastable batch dims), for whole tiles only: M and N multiples of
+// 256, K a multiple of 64. What differs from gemm_tile's 256 x 256 shape:
+//   * No register staging. A slab (64 k-values of 256 rows per operand, 64 KiB) is
+//     requested with global_load_lds_dwordx4: each of the 64 lanes of a load delivers
+//     16 bytes to consecutive LDS addresses, so 40 vector registers and every
+//     ds_write of the staged form disappear. LDS holds a ring of two slabs; the loads
+//     of slab t + 2 are issued as soon as every wave has read its last fragments of
+//     slab t, behind the block's one barrier per slab.
+//   * No padding. A load writes 1 KiB without gaps, so bank conflicts are avoided by
+//     choosing WHICH 16 bytes each lane fetches: the 16-byte units of a k-contiguous
+//     row are XOR-ed with bits of the row number, those of a row-contiguous k-row with
+//     bits of k. Fragment reads apply the same XOR and touch every bank once per
+//     half-wave (ds_read_b128 for k-contiguous tiles, ds_read_b64_tr_b16 otherwise).
+//   * v_mfma_f32_16x16x32 instead of 32x32x16: the same LDS bytes and MFMA cycles per
+//     flop, but a quarter of the accumulator registers rewritten per instruction.
+//     Under the board's power limit (random N(0, 0.02) operands pull this chip from
+//     2.4 to about 1.8 GHz inside a GEMM) that is worth 4-7 % of throughput; on
+//     all-zero operands, where the clock holds, the two forms time the same.
+// The loads are written as assembly on purpose: the compiler then sees no LDS
+// writes, so it places no vmcnt(0) in front of the fragment reads (it cannot tell
+// the two slabs of the ring apart) and the waits are the explicit ones below.
+#pragma once
+
+#include "gemm_tile.hpp"
+
+namespace gemm_dl {
+using namespace gemm_tile;
+
+constexpr int BM = 256, BN = 256, BK = 64, NS = 2, THREADS = 512;
+constexpr int UPR = BK / 8;                       // 16-byte units per row of a k-contiguous tile
+constexpr int UNITS = 256 * UPR;                  // units per operand and slab
+constexpr int LOADS = UNITS / 64 / 8;             // load instructions per wave, operand and slab
+constexpr int OP_BYTES = UNITS * 16, STAGE_BYTES = 2 * OP_BYTES;
+constexpr int PATCH_PITCH = 128 + 8;              // epilogue: a wave's 64 x 128 patch, padded rows (elements)
+constexpr size_t LDS_BYTES = (size_t)8 * 64 * PATCH_PITCH * 2 > (size_t)NS * STAGE_BYTES ? (size_t)8 * 64 * PATCH_PITCH * 2
+                                                                                           : (size_t)NS * STAGE_BYTES;
+
+template <int N>
+__device__ __forceinline__ void wait_loads_and_meet() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// LDS position (16-byte unit) <-> which data it holds.
+// k-contiguous tile [row][unit kv]: physical unit = kv ^ ((row >> 1) & 7): sixteen consecutive
+// rows reading the same logical unit cover the sixteen 16-byte bank groups once.
+// row-contiguous tile [k][unit nv]: physical unit = nv ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1)):
+// the eight k-rows x two units a half-wave's transposing read touches are all distinct.
+__device__ __forceinline__ int swz_kc(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int swz_rc(int k) { return ((k & 3) << 2) | (((k >> 3) & 1) << 1); }
+
+template <class EL, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(THREADS) void kernel(Args a) {
+  using S = typename EL::S;
+  static_assert(!EL::F32, "16-bit operands only");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  uint32_t batch, tm, tn;
+  tile_of_block(a, gridDim.x - 1 - blockIdx.x, batch, tm, tn);
+  int64_t ao = 0, bo = 0, co = 0;
+  {
+    uint32_t idx = batch;
+#pragma unroll
+    for (int i = 3; i >= 0; i--) {
+      if (i < a.nbd) {
+        uint32_t q = idx / a.bshape[i], c = idx - q * a.bshape[i];
+        idx = q;
+        ao += (int64_t)c * a.ba[i];
+        bo += (int64_t)c * a.bb[i];
+        co += (int64_t)c * a.bc[i];
+      }
+    }
+  }
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+  const S *gA = (const S *)a.A + ao + (A_KC ? m0 * a.lda : m0);
+  const S *gB = (const S *)a.B + bo + (B_KC ? n0 * a.ldb : n0);
+  const int64_t stepA = A_KC ? BK : (int64_t)BK * a.lda;
+  const int64_t stepB = B_KC ? BK : (int64_t)BK * a.ldb;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;  // 4 x 2 waves of 64 x 128 outputs
+
+  // Byte offset, from the slab's origin in global memory, of the 16 bytes this lane
+  // fetches with its i-th load: that load fills units [64 j, 64 j + 64), j = wave * LOADS + i.
+  uint32_t offA[LOADS], offB[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; i++) {
+    const int j = wave * LOADS + i;
+    auto kc = [&](int64_t ld) -> uint32_t {
+      const int row = j * (64 / UPR) + lane / UPR, kp = lane % UPR;
+      return (uint32_t)((row * ld + (kp ^ swz_kc(row)) * 8) * 2);
+    };
+    auto rc = [&](int64_t ld) -> uint32_t {
+      const int k = 2 * j + (lane >> 5), np = lane & 31;
+      return (uint32_t)((k * ld + (np ^ swz_rc(k)) * 8) * 2);
+    };
+    offA[i] = A_KC ? kc(a.lda) : rc(a.lda);
+    offB[i] = B_KC ? kc(a.ldb) : rc(a.ldb);
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
+  // m0 carries the LDS address of lane 0's 16 bytes. It is not declared as clobbered: the
+  // compiler treats it as reserved and writes it itself right in front of each of its own uses.
+  auto load1 = [&](const S *base, uint32_t off_bytes, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(off_bytes), "s"(base)
+                 : "memory");
+  };
+  auto issue = [&](int t, int buf) {
+    const uint32_t sb = lds0 + buf * STAGE_BYTES + wave * (LOADS * 1024);
+    const S *pa = gA + (int64_t)t * stepA, *pb = gB + (int64_t)t * stepB;
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) load1(pa, offA[i], sb + i * 1024);
+#pragma unroll
+    for (int i = 0; i < LOADS; i++) load1(pb, offB[i], sb + OP_BYTES + i * 1024);
+  };
+
+  // Fragments of v_mfma_f32_16x16x32: lane 16 g + q holds row (column) q and k = 8 g .. 8 g + 7 of the 32.
+  const int q16 = lane & 15, g16 = lane >> 4;
+  const int kc_sw = (lane >> 1) & 7;  // swz_kc(row0 + q16): row0 is a multiple of 16
+  const int kc_row = q16 * (UPR * 16);
+  const int rc_k = g16 * 8 + (q16 >> 2);
+  const int rc_sw = (((lane >> 2) & 3) << 2) | ((g16 & 1) << 1);  // swz_rc(32 k32 + rc_k (+4))
+  auto frag = [&](const unsigned char *tile, bool kcont, int row0, int k32) -> V16 {
+    if (kcont) return *reinterpret_cast<const V16 *>(tile + row0 * (UPR * 16) + kc_row + (((k32 * 4 + g16) ^ kc_sw) << 4));
+    // transposing read (gemm_tile.hpp): lane q of a 16-lane group addresses the 8 bytes at
+    // k-row (q >> 2), rows 4 (q & 3) .. + 3; the second read takes the k-rows four further on
+    const int r = row0 + (q16 & 3) * 4;
+    const unsigned char *p = tile + (k32 * 32 + rc_k) * 512 + (((r >> 3) ^ rc_sw) << 4) + (r & 7) * 2;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * 512));
+    typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    return V16{l2[0], l2[1], h2[0], h2[1]};
+  };
+
+  f32x4 acc[4][8];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
+
+  const int nt = (int)(a.K / BK);
+#pragma unroll
+  for (int s = 0; s < NS; s++)
+    if (s < nt) issue(s, s);
+  if (nt >= NS) wait_loads_and_meet<(NS - 1) * 2 * LOADS>();
+  else wait_loads_and_meet<0>();
+
+  // A step is 16 MFMAs: the four 16-row fragments of A against four 16-column fragments of B
+  // (one half of the wave's 128 columns) over 32 k-values; a slab is four steps. The reads of
+  // step s + 1 are issued in front of the MFMAs of step s.
+  V16 fa[2][4], fb[2][4];
+  auto load_step = [&](int buf, int st) {
+    const unsigned char *sa = smem_raw + buf * STAGE_BYTES, *sb = sa + OP_BYTES;
+    const int k32 = st >> 1, half = st & 1;
+    if (half == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) fa[k32 & 1][i] = frag(sa, A_KC, wm + i * 16, k32);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) fb[st & 1][j] = frag(sb, B_KC, wn + (half * 4 + j) * 16, k32);
+  };
+  load_step(0, 0);
+  int buf = 0;
+  // In a slab's last step: wait for this wave's share of the next slab, meet the other waves
+  // (now the next slab is complete and nobody reads this one any more), request slab t + NS
+  // into this slab's buffer, fetch the next slab's first fragments, then issue the last MFMAs.
+  auto slab = [&](int t, auto fetch_c, auto last_c) {
+    constexpr bool FETCH = decltype(fetch_c)::value, LAST = decltype(last_c)::value;
+    const int nbuf = buf + 1 == NS ? 0 : buf + 1;
+#pragma unroll
+    for (int st = 0; st < 4; st++) {
+      if (st + 1 < 4) {
+        load_step(buf, st + 1);
+      } else if constexpr (!LAST) {
+        if constexpr (FETCH) wait_loads_and_meet<(NS - 2) * 2 * LOADS>();
+        else wait_loads_and_meet<0>();
+        if constexpr (FETCH) issue(t + NS, buf);
+        load_step(nbuf, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int k32 = st >> 1, half = st & 1;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          f32x4 &c = acc[i][half * 4 + j];
+          if constexpr (EL::BF16)
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fa[k32 & 1][i]), __builtin_bit_cast(bf16x8, fb[st & 1][j]), c, 0, 0, 0);
+          else
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fa[k32 & 1][i]), __builtin_bit_cast(f16x8, fb[st & 1][j]), c, 0, 0, 0);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    buf = nbuf;
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+  int t = 0;
+  for (; t + NS < nt; t++) slab(t, yes{}, no{});
+  for (; t + 1 < nt; t++) slab(t, no{}, no{});
+  slab(t, no{}, yes{});
+
+  // Epilogue: element e of accumulator (i, j) is C[16 i + 4 g + e][16 j + q]. Each wave parks its
+  // rounded 64 x 128 patch in LDS and sends it out as whole 16-byte row segments.
+  S *C = (S *)a.C + co;
+  auto narrow = [](float x) -> S { return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x); };
+  wait_loads_and_meet<0>();  // every wave has read its last fragments; no load is in flight
+  S *patch = reinterpret_cast<S *>(smem_raw) + wave * (64 * PATCH_PITCH);
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) patch[(i * 16 + g16 * 4 + e) * PATCH_PITCH + j * 16 + q16] = narrow(acc[i][j][e]);
+  // the patch is read back by lanes of the same wave only: LDS serves a wave in order
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const int ch = i * 64 + lane, row = ch >> 4, col = (ch & 15) * 8;
+    const V16 v = *reinterpret_cast<const V16 *>(patch + row * PATCH_PITCH + col);
+    *reinterpret_cast<V16 *>(C + (m0 + wm + row) * a.ldc + n0 + wn + col) = v;
+  }
+}
+
+}  // namespace gemm_dl

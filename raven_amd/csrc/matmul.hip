@@ -29,6 +29,7 @@
 #include <cstdlib>
 
 #include "gemm_tile.hpp"
+#include "gemm_dl.hpp"
 #include "nxh_common.hpp"
 
 constexpr int MM_MAXB = 8;  // batch dims decoded on the device
@@ -672,8 +673,34 @@ static int launch_tile_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc,
   return b_kc ? NXH_TILE(false, true) : NXH_TILE(false, false);
 #undef NXH_TILE
 }
-// 0: pick by shape; 256 / 128 / 64: force that block shape (tuning aid, read once
-// from NXH_GEMM_TILE)
+// The direct-to-LDS form of the 256 x 256 shape (gemm_dl.hpp): whole tiles of 16-bit operands.
+template <class EL, bool A_KC, bool B_KC>
+static int launch_dl(nxh_context *ctx, gemm_tile::Args &g) {
+  auto kern = gemm_dl::kernel<EL, A_KC, B_KC>;
+  static std::once_flag once;
+  static hipError_t attr_status = hipSuccess;
+  std::call_once(once, [&] {
+    attr_status = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_dl::LDS_BYTES);
+  });
+  NXH_HIP("matmul", attr_status);
+  g.tiles_m = (uint32_t)(g.M / gemm_dl::BM);
+  g.tiles_n = (uint32_t)(g.N / gemm_dl::BN);
+  nxh_set_path("gemm_dl_256x256");
+  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(gemm_dl::THREADS), gemm_dl::LDS_BYTES, ctx->stream, g);
+  NXH_HIP("matmul", hipGetLastError());
+  return NXH_OK;
+}
+template <class EL>
+static int launch_dl_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc) {
+  if constexpr (EL::F32) {
+    return -1;
+  } else {
+    if (a_kc) return b_kc ? launch_dl<EL, true, true>(ctx, g) : launch_dl<EL, true, false>(ctx, g);
+    return b_kc ? launch_dl<EL, false, true>(ctx, g) : launch_dl<EL, false, false>(ctx, g);
+  }
+}
+// 0: pick by shape; 256 / 128 / 64: force that block shape; 257: the 256 shape in its
+// register-staged form (tuning aid, read once from NXH_GEMM_TILE)
 static int forced_tile() {
   static const int v = [] {
     const char *e = getenv("NXH_GEMM_TILE");
@@ -748,6 +775,11 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   if (pick == 64) return launch_tile_oriented<EL, gemm_tile::Shape256x64, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
   if (pick == 128)
     return launch_tile_oriented<EL, gemm_tile::Shape128x128, false>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
+  // whole 256 x 256 tiles of 16-bit operands: straight into LDS (load offsets are 32-bit:
+  // 256 rows of a k-contiguous operand must stay below 4 GiB)
+  if (!EL::F32 && pick == 256 && a.M % gemm_dl::BM == 0 && a.N % gemm_dl::BN == 0 && al16(g.C) && g.ldc % 8 == 0 &&
+      g.lda < ((int64_t)1 << 22) && g.ldb < ((int64_t)1 << 22))
+    return launch_dl_oriented<EL>(ctx, g, a_kc, b_kc);
   return launch_tile_oriented<EL, gemm_tile::Shape256x256, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
 }
 

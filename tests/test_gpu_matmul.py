@@ -202,7 +202,9 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
                 hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle,
                              (lambda B, t: B.permute(t, (1, 0))) if tb else None)
                 check(hip, oracle, d, ha, hb, a, b, f"tile {m}x{k}x{n} ta={ta} tb={tb}")
-                assert hip.last_path() == path, (m, k, n, ta, tb, hip.last_path())
+                # whole 256-tiles of 16-bit operands take the direct-to-LDS form
+                want_path = "gemm_dl_256x256" if (path, m % 256, n % 256) == ("gemm_tile_256x256", 0, 0) and d is not dt.float32 else path
+                assert hip.last_path() == want_path, (m, k, n, ta, tb, hip.last_path())
     # odd M and N: only K-contiguous operands (A row-major, B given as its transpose) qualify
     a = encode(rng.standard_normal((203, 128)), d, oracle)
     b = encode(rng.standard_normal((128, 157)), d, oracle)
@@ -231,6 +233,47 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
     hw, _ = pair(wide, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 256), (32, 288)]))
     hb2, _ = pair(b4[0, 0][:, :256].copy(), d, hip, oracle)
     check(hip, oracle, d, hip.shrink(hw, [(0, 256), (0, 128)]), hb2, wide[:, 32:160], b4[0, 0][:, :256], "big sliced A")
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_direct_to_lds_kernel(hip, oracle, d):
+    """The large-product form (operands straight from global memory into swizzled LDS
+    tiles, 16x16x32 MFMA): every operand orientation, one to seven K-slabs, batches
+    with a broadcast operand, a sliced operand with a larger row stride."""
+    rng = np.random.default_rng(1500 + d.tag)
+    T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
+    for k in (64, 128, 192, 448):
+        a = encode(rng.standard_normal((4096, k)), d, oracle)
+        b = encode(rng.standard_normal((k, 4096)), d, oracle)
+        want = ref_f64(a, b, d, oracle)
+        for ta in (False, True):
+            for tb in (False, True):
+                if k != 192 and ta != tb:
+                    continue
+                ha, _ = pair(np.ascontiguousarray(a.T) if ta else a, d, hip, oracle, T if ta else None)
+                hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle, T if tb else None)
+                got = decode(logical(hip.matmul(ha, hb)), d, oracle)
+                assert hip.last_path() == "gemm_dl_256x256", (k, ta, tb, hip.last_path())
+                lim = MM_TOL[d.name] * (np.abs(want) + np.sqrt(k))
+                assert np.all(np.abs(got - want) <= lim), (k, ta, tb, float(np.abs(got - want).max()))
+                # a 16-bit result is the f32 sum rounded once: within one unit of the f64 product rounded
+                ulp = 2.0 ** (-8 if d is dt.bfloat16 else -11)
+                assert np.all(np.abs(got - want) <= ulp * 2 * np.abs(want) + np.sqrt(k) * 2e-6), (k, ta, tb)
+    # batches: [4, 2048, 128] x [128, 2048] (one B for all), [4,1,..] x [1,2,..] (both broadcast)
+    a = encode(rng.standard_normal((4, 2048, 128)), d, oracle)
+    b = encode(rng.standard_normal((128, 2048)), d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "dl batched x one B")
+    assert hip.last_path() == "gemm_dl_256x256"
+    a4 = encode(rng.standard_normal((4, 1, 1024, 64)), d, oracle)
+    b4 = encode(rng.standard_normal((1, 4, 64, 1024)), d, oracle)
+    check(hip, oracle, d, pair(a4, d, hip, oracle)[0], pair(b4, d, hip, oracle)[0], a4, b4, "dl both batch-broadcast")
+    assert hip.last_path() == "gemm_dl_256x256"
+    # a column slice of a wider matrix (row stride 4096 + 64, offset 32 elements: still 16-byte aligned)
+    wide = encode(rng.standard_normal((4096, 128 + 64)), d, oracle)
+    hw, _ = pair(wide, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 4096), (32, 160)]))
+    b = encode(rng.standard_normal((128, 4096)), d, oracle)
+    check(hip, oracle, d, hw, pair(b, d, hip, oracle)[0], wide[:, 32:160], b, "dl sliced A")
+    assert hip.last_path() == "gemm_dl_256x256"
 
 
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16, dt.float32], ids=lambda d: d.name)
