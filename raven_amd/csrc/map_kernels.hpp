@@ -5,10 +5,11 @@
 // adjacent dims compose on EVERY operand (the reference's rule,
 // nx_c_engine.c:542-590). The plan then picks one of three kernels:
 //   map_contig   every operand is one contiguous run or a broadcast scalar:
-//                16-byte vector loads/stores, 4 vectors in flight per lane.
-//   map_tiled    some input's unit-stride dim differs from the output's: 64x64
-//                tiles, that input is read along ITS contiguous dim and turned
-//                through LDS, so both sides of HBM see coalesced 256 B rows.
+//                16-byte vector loads/stores, 2 vectors in flight per lane.
+//   map_tiled    some input's unit-stride dim differs from the output's: patches of
+//                8 KiB (64 x 32 four-byte elements), that input is read along ITS
+//                contiguous dim and turned through LDS, so both sides of HBM see
+//                coalesced rows.
 //   map_generic  anything else: per-lane index decomposition with precomputed
 //                multiply-shift divisors; vectorised along the inner dim when
 //                every operand is contiguous or broadcast there.
@@ -23,7 +24,11 @@
 constexpr int MAP_MAXOP = 4;
 constexpr int MAP_MAXD = 8;
 constexpr int MAP_THREADS = 256;
-constexpr int MAP_UNROLL = 4;
+constexpr int MAP_UNROLL = 4;     // vectors in flight per lane, map_generic
+#ifndef MAP_CONTIG_UNROLL_X
+#define MAP_CONTIG_UNROLL_X 2
+#endif
+constexpr int MAP_CONTIG_UNROLL = MAP_CONTIG_UNROLL_X;  // the same for map_contig
 
 struct MapPlan {
   int nop = 0, ndim = 0;
@@ -271,98 +276,115 @@ struct TiledArgs {
   uint32_t any_turn;
 };
 
-template <int TILE, int V>
+// Tile geometry. The patch is TX (along x) by TY (along y) elements. Everything that is
+// stored, and every input that is not turned, moves in the OUTPUT arrangement: VX
+// consecutive x per lane, GXO lanes across a row, RYO rows per pass of the block, NYO
+// passes. A turned input is fetched in its own arrangement: VY consecutive y per lane, GYT
+// lanes along y, RXT columns per pass, NXT passes. VX and VY differ when the output is
+// narrower than the turned input (a compare of 4-byte operands stores 16 one-byte results
+// per lane, so that a wave still writes whole 128-byte rows).
+template <int TX, int TY, int VX, int VY>
 struct TileGeom {
-  static constexpr int G = TILE / V;         // lanes across one row of the patch
-  static constexpr int R = MAP_THREADS / G;  // rows covered by one pass of the block
-  static constexpr int N = TILE / R;         // passes
-  static_assert(G * V == TILE && G * R == MAP_THREADS && N * R == TILE && N >= 1, "tile geometry");
+  static constexpr int GXO = TX / VX, RYO = MAP_THREADS / GXO, NYO = TY / RYO;
+  static constexpr int GYT = TY / VY, RXT = MAP_THREADS / GYT, NXT = TX / RXT;
+  static constexpr int PITCH = TX + 1;  // odd: element-wide LDS accesses of 4-byte types spread over the banks
+  static_assert(GXO * VX == TX && GXO * RYO == MAP_THREADS && NYO * RYO == TY && NYO >= 1, "output arrangement");
+  static_assert(GYT * VY == TY && GYT * RXT == MAP_THREADS && NXT * RXT == TX && NXT >= 1, "fetch arrangement");
 };
 
-// Issues this lane's global loads of one operand. A turned operand is fetched
-// along y (V consecutive y for N different x); anything else arrives in the
-// output arrangement (V consecutive x for N different y).
-template <class T, int TILE, int V, int NP>
-__device__ __forceinline__ void tile_fetch(Vec<T, V> (&r)[NP], const T *p, int64_t sx,
-                                           int64_t sy, uint32_t x0, uint32_t y0, uint32_t nx,
-                                           uint32_t ny, uint32_t mode) {
-  using TG = TileGeom<TILE, V>;
-  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
-  if (mode == TILE_TURN) {
-    const uint32_t y = y0 + g * V;
-    const T *s = p + (int64_t)y + (int64_t)(x0 + q) * sx;
-    const int64_t step = (int64_t)TG::R * sx;
-#pragma unroll
-    for (int i = 0; i < TG::N; i++) {
-      if (x0 + q + i * TG::R < nx && y < ny) r[i] = *reinterpret_cast<const Vec<T, V> *>(s);
-      s += step;
-    }
-    return;
-  }
-  const uint32_t x = x0 + g * V;
+// Issues this lane's global loads of an input that arrives in the output arrangement
+// (VX consecutive x for NYO different y).
+template <class T, class TG, int VX>
+__device__ __forceinline__ void tile_fetch_out(Vec<T, VX> (&r)[TG::NYO], const T *p, int64_t sx, int64_t sy,
+                                               uint32_t x0, uint32_t y0, uint32_t nx, uint32_t ny, uint32_t mode) {
+  const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
+  const uint32_t x = x0 + g * VX;
   const T *s = p + (int64_t)(y0 + q) * sy + (int64_t)x * sx;
-  const int64_t step = (int64_t)TG::R * sy;
+  const int64_t step = (int64_t)TG::RYO * sy;
   if (mode == TILE_ROW) {
 #pragma unroll
-    for (int i = 0; i < TG::N; i++) {
-      if (x < nx && y0 + q + i * TG::R < ny) r[i] = *reinterpret_cast<const Vec<T, V> *>(s);
+    for (int i = 0; i < TG::NYO; i++) {
+      if (x < nx && y0 + q + i * TG::RYO < ny) r[i] = *reinterpret_cast<const Vec<T, VX> *>(s);
       s += step;
     }
   } else if (mode == TILE_BX) {
 #pragma unroll
-    for (int i = 0; i < TG::N; i++) {
-      if (x < nx && y0 + q + i * TG::R < ny) {
+    for (int i = 0; i < TG::NYO; i++) {
+      if (x < nx && y0 + q + i * TG::RYO < ny) {
         const T v = *s;
 #pragma unroll
-        for (int j = 0; j < V; j++) r[i].v[j] = v;
+        for (int j = 0; j < VX; j++) r[i].v[j] = v;
       }
       s += step;
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < TG::N; i++) {
-      if (x < nx && y0 + q + i * TG::R < ny) {
+    for (int i = 0; i < TG::NYO; i++) {
+      if (x < nx && y0 + q + i * TG::RYO < ny) {
 #pragma unroll
-        for (int j = 0; j < V; j++) r[i].v[j] = s[(int64_t)j * sx];
+        for (int j = 0; j < VX; j++) r[i].v[j] = s[(int64_t)j * sx];
       }
       s += step;
     }
   }
 }
-
-// The turn: lds is [y][x] with a one-element pad, written from the fetch
-// arrangement, read in the output arrangement. Element-wide LDS accesses: the
-// odd pitch keeps both directions free of bank conflicts for 4-byte types.
-template <class T, int TILE, int V, int NP>
-__device__ __forceinline__ void tile_put(const Vec<T, V> (&r)[NP], T *lds) {
-  using TG = TileGeom<TILE, V>;
-  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
+// A turned input is fetched along y (VY consecutive y for NXT different x).
+template <class T, class TG, int VY>
+__device__ __forceinline__ void tile_fetch_turn(Vec<T, VY> (&r)[TG::NXT], const T *p, int64_t sx, uint32_t x0,
+                                                uint32_t y0, uint32_t nx, uint32_t ny) {
+  const uint32_t g = threadIdx.x % TG::GYT, q = threadIdx.x / TG::GYT;
+  const uint32_t y = y0 + g * VY;
+  const T *s = p + (int64_t)y + (int64_t)(x0 + q) * sx;
+  const int64_t step = (int64_t)TG::RXT * sx;
 #pragma unroll
-  for (int i = 0; i < TG::N; i++)
-#pragma unroll
-    for (int j = 0; j < V; j++) lds[(g * V + j) * (TILE + 1) + q + i * TG::R] = r[i].v[j];
-}
-template <class T, int TILE, int V, int NP>
-__device__ __forceinline__ void tile_get(Vec<T, V> (&r)[NP], const T *lds) {
-  using TG = TileGeom<TILE, V>;
-  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
-#pragma unroll
-  for (int i = 0; i < TG::N; i++)
-#pragma unroll
-    for (int j = 0; j < V; j++) r[i].v[j] = lds[(q + i * TG::R) * (TILE + 1) + g * V + j];
+  for (int i = 0; i < TG::NXT; i++) {
+    if (x0 + q + i * TG::RXT < nx && y < ny) r[i] = *reinterpret_cast<const Vec<T, VY> *>(s);
+    s += step;
+  }
 }
 
-template <class F, int TILE, int V>
+// The turn: lds is [y][x] with a one-element pad, written from the fetch arrangement,
+// read in the output arrangement, one element per access.
+template <class T, class TG, int VY>
+__device__ __forceinline__ void tile_put(const Vec<T, VY> (&r)[TG::NXT], T *lds) {
+  const uint32_t g = threadIdx.x % TG::GYT, q = threadIdx.x / TG::GYT;
+#pragma unroll
+  for (int i = 0; i < TG::NXT; i++)
+#pragma unroll
+    for (int j = 0; j < VY; j++) lds[(g * VY + j) * TG::PITCH + q + i * TG::RXT] = r[i].v[j];
+}
+template <class T, class TG, int VX>
+__device__ __forceinline__ void tile_get(Vec<T, VX> (&r)[TG::NYO], const T *lds) {
+  const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
+#pragma unroll
+  for (int i = 0; i < TG::NYO; i++)
+#pragma unroll
+    for (int j = 0; j < VX; j++) r[i].v[j] = lds[(q + i * TG::RYO) * TG::PITCH + g * VX + j];
+}
+
+// One input of the tile: fetched in whichever arrangement its mode asks for.
+template <class T, class TG, int VX, int VY>
+struct TileOperand {
+  Vec<T, VX> r[TG::NYO];
+  Vec<T, VY> t[TG::NXT];
+  __device__ __forceinline__ void fetch(const T *p, int64_t sx, int64_t sy, uint32_t x0, uint32_t y0, uint32_t nx,
+                                        uint32_t ny, uint32_t mode) {
+    if (mode == TILE_TURN) tile_fetch_turn<T, TG, VY>(t, p, sx, x0, y0, nx, ny);
+    else tile_fetch_out<T, TG, VX>(r, p, sx, sy, x0, y0, nx, ny, mode);
+  }
+};
+
+template <class F, int TX, int TY, int VX, int VY>
 __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) {
   using MT = MapTypes<F>;
-  using TG = TileGeom<TILE, V>;
+  using TG = TileGeom<TX, TY, VX, VY>;
   using I0 = typename MT::In0;
   using I1 = typename MT::In1;
   using I2 = typename MT::In2;
   using O = typename MT::Out;
-  __shared__ I0 l0[TILE * (TILE + 1)];
-  __shared__ I1 l1[F::NIN > 1 ? TILE * (TILE + 1) : 1];
-  __shared__ I2 l2[F::NIN > 2 ? TILE * (TILE + 1) : 1];
+  __shared__ I0 l0[TY * TG::PITCH];
+  __shared__ I1 l1[F::NIN > 1 ? TY * TG::PITCH : 1];
+  __shared__ I2 l2[F::NIN > 2 ? TY * TG::PITCH : 1];
   // Blocks with equal id modulo 8 share an XCD (and its L2): hand each XCD a
   // contiguous run of tiles, so neighbouring tiles that split a cache line of a
   // narrow operand fetch it once.
@@ -379,39 +401,37 @@ __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) 
 #pragma unroll
     for (int k = 0; k <= F::NIN; k++) off[k] += (int64_t)c * a.bstride[k][d];
   }
-  const uint32_t x0 = tx * TILE, y0 = ty * TILE;
-  Vec<I0, V> r0[TG::N];
-  Vec<I1, V> r1[TG::N];
-  Vec<I2, V> r2[TG::N];
-  tile_fetch<I0, TILE, V>(r0, (const I0 *)a.base[1] + off[1], a.sx[1], a.sy[1], x0, y0, a.nx, a.ny, a.mode[1]);
-  if constexpr (F::NIN > 1)
-    tile_fetch<I1, TILE, V>(r1, (const I1 *)a.base[2] + off[2], a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.mode[2]);
-  if constexpr (F::NIN > 2)
-    tile_fetch<I2, TILE, V>(r2, (const I2 *)a.base[3] + off[3], a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.mode[3]);
+  const uint32_t x0 = tx * TX, y0 = ty * TY;
+  TileOperand<I0, TG, VX, VY> r0;
+  TileOperand<I1, TG, VX, VY> r1;
+  TileOperand<I2, TG, VX, VY> r2;
+  r0.fetch((const I0 *)a.base[1] + off[1], a.sx[1], a.sy[1], x0, y0, a.nx, a.ny, a.mode[1]);
+  if constexpr (F::NIN > 1) r1.fetch((const I1 *)a.base[2] + off[2], a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.mode[2]);
+  if constexpr (F::NIN > 2) r2.fetch((const I2 *)a.base[3] + off[3], a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.mode[3]);
   if (a.any_turn) {
-    if (a.mode[1] == TILE_TURN) tile_put<I0, TILE, V>(r0, l0);
+    if (a.mode[1] == TILE_TURN) tile_put<I0, TG, VY>(r0.t, l0);
     if constexpr (F::NIN > 1)
-      if (a.mode[2] == TILE_TURN) tile_put<I1, TILE, V>(r1, l1);
+      if (a.mode[2] == TILE_TURN) tile_put<I1, TG, VY>(r1.t, l1);
     if constexpr (F::NIN > 2)
-      if (a.mode[3] == TILE_TURN) tile_put<I2, TILE, V>(r2, l2);
+      if (a.mode[3] == TILE_TURN) tile_put<I2, TG, VY>(r2.t, l2);
     __syncthreads();
-    if (a.mode[1] == TILE_TURN) tile_get<I0, TILE, V>(r0, l0);
+    if (a.mode[1] == TILE_TURN) tile_get<I0, TG, VX>(r0.r, l0);
     if constexpr (F::NIN > 1)
-      if (a.mode[2] == TILE_TURN) tile_get<I1, TILE, V>(r1, l1);
+      if (a.mode[2] == TILE_TURN) tile_get<I1, TG, VX>(r1.r, l1);
     if constexpr (F::NIN > 2)
-      if (a.mode[3] == TILE_TURN) tile_get<I2, TILE, V>(r2, l2);
+      if (a.mode[3] == TILE_TURN) tile_get<I2, TG, VX>(r2.r, l2);
   }
-  const uint32_t g = threadIdx.x % TG::G, q = threadIdx.x / TG::G;
-  const uint32_t x = x0 + g * V;
+  const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
+  const uint32_t x = x0 + g * VX;
   O *o = (O *)a.base[0] + off[0] + (int64_t)(y0 + q) * a.sy[0] + x;
-  const int64_t step = (int64_t)TG::R * a.sy[0];
+  const int64_t step = (int64_t)TG::RYO * a.sy[0];
 #pragma unroll
-  for (int i = 0; i < TG::N; i++) {
-    if (x < a.nx && y0 + q + i * TG::R < a.ny) {
-      Vec<O, V> v;
+  for (int i = 0; i < TG::NYO; i++) {
+    if (x < a.nx && y0 + q + i * TG::RYO < a.ny) {
+      Vec<O, VX> v;
 #pragma unroll
-      for (int j = 0; j < V; j++) v.v[j] = map_apply<F>(r0[i].v[j], r1[i].v[j], r2[i].v[j]);
-      *reinterpret_cast<Vec<O, V> *>(o) = v;
+      for (int j = 0; j < VX; j++) v.v[j] = map_apply<F>(r0.r[i].v[j], r1.r[i].v[j], r2.r[i].v[j]);
+      *reinterpret_cast<Vec<O, VX> *>(o) = v;
     }
     o += step;
   }
@@ -485,8 +505,8 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
     // it stores 16 bytes, with fewer vectors per lane so that the bytes in
     // flight stay the same; operands must then be aligned to the wider vector.
     constexpr int VW = (int)sizeof(typename MT::Out) < MT::smax
-                           ? std::min(16 / (int)sizeof(typename MT::Out), V * MAP_UNROLL) : V;
-    constexpr int UW = V * MAP_UNROLL / VW;
+                           ? std::min(16 / (int)sizeof(typename MT::Out), V * MAP_CONTIG_UNROLL) : V;
+    constexpr int UW = V * MAP_CONTIG_UNROLL / VW;
     bool wide = VW > V;
     for (int k = 0; ok && k < p.nop; k++) {
       bool is_bc = k > 0 && (bc & (1u << (k - 1)));
@@ -508,9 +528,9 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
         const uint32_t blocks = (uint32_t)((nvec + per_block - 1) / per_block);
         hipLaunchKernelGGL((map_contig_kernel<F, VW, UW>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
       } else {
-        const int64_t nvec = (p.total + V - 1) / V, per_block = MAP_THREADS * MAP_UNROLL;
+        const int64_t nvec = (p.total + V - 1) / V, per_block = MAP_THREADS * MAP_CONTIG_UNROLL;
         const uint32_t blocks = (uint32_t)((nvec + per_block - 1) / per_block);
-        hipLaunchKernelGGL((map_contig_kernel<F, V, MAP_UNROLL>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
+        hipLaunchKernelGGL((map_contig_kernel<F, V, MAP_CONTIG_UNROLL>), dim3(blocks), dim3(MAP_THREADS), 0, ctx->stream, a);
       }
       NXH_HIP(op, hipGetLastError());
       return NXH_OK;
@@ -530,7 +550,14 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
         }
     }
     if (ydim >= 0) {
-      constexpr int TILE = MT::smax <= 4 ? 64 : 32;
+      // A patch holds 8 KiB of the widest type (4 KiB for one-byte types): 64 x 32 elements of 4
+      // bytes, 64 x 64 of 1 or 2, 32 x 32 of 8 or 16. Measured on [64,512,512] int32 / float32
+      // with a permuted operand: 64 x 64 patches of 4-byte elements ran the config-2 step in
+      // 172 us, 64 x 32 in 162 us (more blocks per compute unit, shorter dependent chains
+      // through the barrier), 32 x 32 in 177 us, 128 x 64 with 16-byte stores of one-byte
+      // results in 173 us.
+      constexpr int TX = MT::smax <= 4 ? 64 : 32;
+      constexpr int TY = MT::smax == 4 ? 32 : (MT::smax < 4 ? 64 : 32);
       TiledArgs<F> a;
       a.any_turn = 0;
       // 16-byte lanes need every vector of every operand aligned and whole
@@ -552,8 +579,8 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       }
       a.nx = (uint32_t)p.shape[last];
       a.ny = (uint32_t)p.shape[ydim];
-      a.tiles_x = (a.nx + TILE - 1) / TILE;
-      a.tiles_y = (a.ny + TILE - 1) / TILE;
+      a.tiles_x = (a.nx + TX - 1) / TX;
+      a.tiles_y = (a.ny + TY - 1) / TY;
       a.nbatch_dims = 0;
       int64_t nb = 1;
       for (int d = 0; d < last; d++) {
@@ -568,10 +595,10 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       if (blocks < ((int64_t)1 << 31)) {
         nxh_set_path("map_tiled");
         if (vec)
-          hipLaunchKernelGGL((map_tiled_kernel<F, TILE, V>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+          hipLaunchKernelGGL((map_tiled_kernel<F, TX, TY, V, V>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
                              ctx->stream, a);
         else
-          hipLaunchKernelGGL((map_tiled_kernel<F, TILE, 1>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+          hipLaunchKernelGGL((map_tiled_kernel<F, TX, TY, 1, 1>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
                              ctx->stream, a);
         NXH_HIP(op, hipGetLastError());
         return NXH_OK;
