@@ -387,6 +387,39 @@ int nxh_svd(nxh_context *ctx, const nxh_tensor *u, const nxh_tensor *s, const nx
    order of the Schur factor's diagonal. n <= 2048. */
 int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nxh_tensor *x);
 
+/* ── deferred evaluation ─────────────────────────────────────────────────── */
+
+/* No counterpart in the reference, whose frontend lowers softmax, layer norm, GELU,
+   attention and a linear layer to runs of primitives (frontend.ml:4242-4252,
+   kaun/lib/layer_norm.ml:43-68, fn.ml:31-38, attention.ml:67-110, linear.ml:50-52)
+   and whose backend runs each primitive as it is called. With the mode on,
+   nxh_unary / nxh_binary / nxh_compare / nxh_where / nxh_cast / nxh_reduce /
+   nxh_matmul and a one-element nxh_fill only record their call. The record is
+   executed, in issue order, by the next call of any other entry point (a host
+   read and nxh_synchronize included) or when it reaches 512 entries; a run that
+   spells one of those sequences, and whose intermediate results were given back
+   with nxh_free while still recorded and are read only inside the run, is replaced
+   by the fused entry point below. Observable results are the eager ones, except
+   that an error of a recorded primitive is returned by the call that executes the
+   record, and that a fused row sum may be added in another order. nxh_free of a
+   block the record still uses takes effect once the record has run. Switching
+   the mode (either way) executes the record first. */
+int nxh_set_deferred(nxh_context *ctx, int on);
+/* Counters since the context was created, in this order. */
+enum {
+  NXH_DEFER_RECORDED = 0,   /* primitives recorded */
+  NXH_DEFER_ISSUED,         /* primitives issued as recorded */
+  NXH_DEFER_FLUSHES,        /* executions of a non-empty record */
+  NXH_DEFER_FALLBACKS,      /* fused calls that were declined (the run was issued as recorded) */
+  NXH_DEFER_SOFTMAX,        /* runs replaced by nxh_softmax_rows */
+  NXH_DEFER_LAYER_NORM,     /* ... nxh_layer_norm_rows */
+  NXH_DEFER_GELU,           /* ... nxh_gelu_tanh */
+  NXH_DEFER_ATTENTION,      /* ... nxh_attention */
+  NXH_DEFER_LINEAR,         /* ... nxh_linear */
+  NXH_DEFER_STAT_COUNT
+};
+int nxh_deferred_stats(nxh_context *ctx, uint64_t *stats, int count);
+
 /* ── recorded sequences ──────────────────────────────────────────────────── */
 
 /* The reference backend has no counterpart: its eager calls cost a C stub

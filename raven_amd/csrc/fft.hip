@@ -624,6 +624,7 @@ static inline int length_as_int(const char *op, int64_t n) {
 // nx_c_fft.c:940-956
 NXH_EXPORT int nxh_fft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const int32_t *axes, int n_axes,
                        int inverse) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = inverse ? "ifft" : "fft";
   if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -653,6 +654,7 @@ NXH_EXPORT int nxh_fft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor
 
 // nx_c_fft.c:958-982
 NXH_EXPORT int nxh_rfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const int32_t *axes, int n_axes) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = "rfft";
   if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -689,6 +691,7 @@ NXH_EXPORT int nxh_rfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tenso
 // nx_c_fft.c:1029-1144
 NXH_EXPORT int nxh_irfft(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const int32_t *axes, int n_axes,
                          int64_t s_last) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = "irfft";
   if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);

@@ -467,6 +467,7 @@ static int reduce_entry(nxh_context *ctx, int op, const nxh_tensor *out, const n
 
 NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
                           const int32_t *axes, int n_axes) {
+  NXH_DEFER_RECORD(ctx, NXH_D_REDUCE, op, out, 1, axes, n_axes, nullptr, x);
   return reduce_entry(ctx, op, out, x, axes, n_axes, false);
 }
 
@@ -476,5 +477,6 @@ NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const
 // the workspace is refused before anything is launched.
 NXH_EXPORT int nxh_reduce_noalloc(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
                                   const int32_t *axes, int n_axes) {
+  NXH_DEFER_BARRIER(ctx, out);
   return reduce_entry(ctx, op, out, x, axes, n_axes, true);
 }

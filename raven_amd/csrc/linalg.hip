@@ -1439,6 +1439,7 @@ struct PathAtExit {
 
 // nx_c_tri.c:303-400, 564-578
 NXH_EXPORT int nxh_cholesky(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int upper) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = "cholesky";
   if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   Problem p;
@@ -1476,6 +1477,7 @@ NXH_EXPORT int nxh_cholesky(nxh_context *ctx, const nxh_tensor *out, const nxh_t
 // flags: bit 0 upper, bit 1 transpose (conjugate transpose for complex), bit 2 unit diagonal.
 NXH_EXPORT int nxh_triangular_solve(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *a, const nxh_tensor *b,
                                     int flags) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = "triangular_solve";
   if (!ctx || !out || !a || !b) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   Problem p;
@@ -1514,6 +1516,7 @@ NXH_EXPORT int nxh_triangular_solve(nxh_context *ctx, const nxh_tensor *out, con
 // nx_c_qr.c; nx_backend.ml:613-626. q is [..., m, k] (reduced) or [..., m, m]; r is
 // [..., k, n] or [..., m, n], k = min(m, n).
 NXH_EXPORT int nxh_qr(nxh_context *ctx, const nxh_tensor *q, const nxh_tensor *r, const nxh_tensor *x, int reduced) {
+  NXH_DEFER_BARRIER(ctx, q, r);
   const char *op = "qr";
   if (!ctx || !q || !r || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   Problem p;
@@ -1554,6 +1557,7 @@ NXH_EXPORT int nxh_qr(nxh_context *ctx, const nxh_tensor *q, const nxh_tensor *r
 
 // nx_c_eigh.c:1492-1500, 1765-; nx_backend.ml:628-649. v may be null (eigvalsh).
 NXH_EXPORT int nxh_eigh(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nxh_tensor *x) {
+  NXH_DEFER_BARRIER(ctx, w, v);
   const char *op = v ? "eigh" : "eigvalsh";
   if (!ctx || !w || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   Problem p;
@@ -1601,6 +1605,7 @@ NXH_EXPORT int nxh_eigh(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor 
 // nx_c_svd.c; nx_backend.ml:651-677. u is [..., m, k] or [..., m, m], s [..., k]
 // float64 descending, vt [..., k, n] or [..., n, n]; k = min(m, n).
 NXH_EXPORT int nxh_svd(nxh_context *ctx, const nxh_tensor *u, const nxh_tensor *s, const nxh_tensor *vt, const nxh_tensor *x) {
+  NXH_DEFER_BARRIER(ctx, u, s, vt);
   const char *op = "svd";
   if (!ctx || !u || !s || !vt || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   Problem p;
@@ -1691,6 +1696,7 @@ NXH_EXPORT int nxh_svd(nxh_context *ctx, const nxh_tensor *u, const nxh_tensor *
 // nx_c_eig.c; nx_backend.ml:679-707. w [..., n] and v [..., n, n] are complex128;
 // v may be null (eigvals).
 NXH_EXPORT int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nxh_tensor *x) {
+  NXH_DEFER_BARRIER(ctx, w, v);
   const char *op = v ? "eig" : "eigvals";
   if (!ctx || !w || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   Problem p;

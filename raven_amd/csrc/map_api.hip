@@ -59,6 +59,7 @@ NXH_EXPORT int nxh_unary(nxh_context *ctx, int op, const nxh_tensor *out, const 
   if ((unsigned)op >= NXH_UNARY_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "unary", "unknown op");
   const char *name = unary_names[op];
   NXH_CHECK_ARGS(name, out, x);
+  NXH_DEFER_RECORD(ctx, NXH_D_UNARY, op, out, 1, nullptr, 0, nullptr, x);
   const int dt = out->dtype;
   if (nxh_is_packed(dt) || nxh_is_packed(x->dtype)) return nxh_fail(NXH_FAILURE, name, NXH_ERR_PACKED);
   if (x->dtype != dt) return nxh_fail(NXH_FAILURE, name, NXH_ERR_UNSUPPORTED);
@@ -76,6 +77,7 @@ NXH_EXPORT int nxh_binary(nxh_context *ctx, int op, const nxh_tensor *out, const
   if ((unsigned)op >= NXH_BINARY_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "binary", "unknown op");
   const char *name = binary_names[op];
   NXH_CHECK_ARGS(name, out, x, y);
+  NXH_DEFER_RECORD(ctx, NXH_D_BINARY, op, out, 2, nullptr, 0, nullptr, x, y);
   const int dt = out->dtype;
   if (nxh_is_packed(dt) || nxh_is_packed(x->dtype) || nxh_is_packed(y->dtype))
     return nxh_fail(NXH_FAILURE, name, NXH_ERR_PACKED);
@@ -94,6 +96,7 @@ NXH_EXPORT int nxh_compare(nxh_context *ctx, int op, const nxh_tensor *out, cons
   if ((unsigned)op >= NXH_COMPARE_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "compare", "unknown op");
   const char *name = compare_names[op];
   NXH_CHECK_ARGS(name, out, x, y);
+  NXH_DEFER_RECORD(ctx, NXH_D_COMPARE, op, out, 2, nullptr, 0, nullptr, x, y);
   const int dt = x->dtype;
   if (nxh_is_packed(dt) || nxh_is_packed(y->dtype)) return nxh_fail(NXH_FAILURE, name, NXH_ERR_PACKED);
   if (y->dtype != dt || nxh_elem_size(out->dtype) != 1)
@@ -108,6 +111,7 @@ NXH_EXPORT int nxh_compare(nxh_context *ctx, int op, const nxh_tensor *out, cons
 NXH_EXPORT int nxh_where(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *cond,
                          const nxh_tensor *a, const nxh_tensor *b) {
   NXH_CHECK_ARGS("where", out, cond, a, b);
+  NXH_DEFER_RECORD(ctx, NXH_D_WHERE, 0, out, 3, nullptr, 0, nullptr, cond, a, b);
   const int dt = out->dtype;
   if (nxh_is_packed(dt)) return nxh_fail(NXH_FAILURE, "where", NXH_ERR_PACKED);
   if (a->dtype != dt || b->dtype != dt || nxh_elem_size(cond->dtype) != 1)
@@ -124,6 +128,7 @@ struct alignas(16) B16x {
 static int copy_impl(nxh_context *ctx, const char *op, const nxh_tensor *out, const nxh_tensor *x);
 
 NXH_EXPORT int nxh_copy(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x) {
+  NXH_DEFER_BARRIER(ctx, out);
   NXH_CHECK_ARGS("copy", out, x);
   return copy_impl(ctx, "copy", out, x);
 }
@@ -251,7 +256,11 @@ NXH_EXPORT int nxh_cast(nxh_context *ctx, const nxh_tensor *out, const nxh_tenso
   NXH_CHECK_ARGS("cast", out, x);
   if (!nxh_same_shape(out, x)) return nxh_fail(NXH_INVALID_ARGUMENT, "cast", NXH_ERR_SHAPE);
   const int src = x->dtype, dst = out->dtype;
-  if (nxh_is_packed(src) || nxh_is_packed(dst)) return cast_packed(ctx, out, x);
+  if (nxh_is_packed(src) || nxh_is_packed(dst)) {
+    NXH_DEFER_BARRIER(ctx, out);
+    return cast_packed(ctx, out, x);
+  }
+  NXH_DEFER_RECORD(ctx, NXH_D_CAST, 0, out, 1, nullptr, 0, nullptr, x);
   map_launch_fn fn = nxh_lookup_cast_a(src, dst);
   if (!fn) fn = nxh_lookup_cast_b(src, dst);
   if (!fn) fn = nxh_lookup_cast_c(src, dst);
@@ -322,6 +331,12 @@ __global__ __launch_bounds__(256) void fill_contig_kernel(uint8_t *out, int64_t 
 NXH_EXPORT int nxh_fill(nxh_context *ctx, const nxh_tensor *out, const void *value) {
   NXH_CHECK_ARGS("full", out);
   if (!value) return nxh_fail(NXH_INVALID_ARGUMENT, "full", "null value");
+  if (nxh_defer_active(ctx)) {
+    // a one-element fill is recorded (the scalars of a fused run are then never filled on the
+    // device); any other fill runs the record first
+    const int drc = nxh_defer_record(ctx, NXH_D_FULL, 0, out, nullptr, 0, nullptr, 0, value);
+    if (drc != -1) return drc;
+  }
   const int dt = out->dtype;
   int64_t n = 1;
   for (int i = 0; i < out->ndim; i++) n *= out->shape[i];

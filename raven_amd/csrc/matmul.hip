@@ -968,11 +968,13 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
 }
 
 NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tensor *A, const nxh_tensor *B) {
+  NXH_DEFER_RECORD(ctx, NXH_D_MATMUL, 0, C, 2, nullptr, 0, nullptr, A, B);
   return matmul_entry(ctx, "matmul", C, A, B, nullptr, nullptr);
 }
 
 NXH_EXPORT int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const nxh_tensor *w,
                           const nxh_tensor *bias, const nxh_tensor *residual) {
+  NXH_DEFER_BARRIER(ctx, out);
   if (!bias && !residual) return matmul_entry(ctx, "matmul", out, x, w, nullptr, nullptr);
   return matmul_entry(ctx, "linear", out, x, w, bias, residual);
 }

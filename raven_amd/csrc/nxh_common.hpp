@@ -96,6 +96,33 @@ int nxh_collect_index_fault(nxh_context *ctx, const char *op);
 // the flag is reported now, as the replay's, so that this call answers only for itself.
 int nxh_settle_replay_faults(nxh_context *ctx, const char *op);
 
+// the deferred-evaluation window (defer.hip)
+bool nxh_defer_active(nxh_context *ctx);
+int nxh_defer_flush(nxh_context *ctx);
+int nxh_defer_barrier(nxh_context *ctx, const nxh_tensor *out0 = nullptr, const nxh_tensor *out1 = nullptr,
+                      const nxh_tensor *out2 = nullptr);
+int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, const nxh_tensor *const *ins, int nin,
+                     const int32_t *axes, int n_axes, const void *value);
+bool nxh_defer_free(nxh_context *ctx, void *p);
+int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes);
+void nxh_defer_context_gone(nxh_context *ctx);
+enum { NXH_D_UNARY, NXH_D_BINARY, NXH_D_COMPARE, NXH_D_WHERE, NXH_D_CAST, NXH_D_REDUCE, NXH_D_MATMUL, NXH_D_FULL };
+// Entry points that are not recorded run the record first.
+#define NXH_DEFER_BARRIER(ctx, ...)                              \
+  do {                                                           \
+    if ((ctx) && nxh_defer_active(ctx))                          \
+      if (int drc__ = nxh_defer_barrier(ctx, ##__VA_ARGS__)) return drc__; \
+  } while (0)
+// Recorded entry points: NXH_OK means recorded; -1 means run now.
+#define NXH_DEFER_RECORD(ctx, kind, op, out, nin, axes, n_axes, value, ...)                             \
+  do {                                                                                                  \
+    if ((ctx) && nxh_defer_active(ctx)) {                                                               \
+      const nxh_tensor *dins__[] = {__VA_ARGS__};                                                       \
+      const int drc__ = nxh_defer_record(ctx, kind, op, out, dins__, nin, axes, n_axes, value);         \
+      if (drc__ != -1) return drc__;                                                                    \
+    }                                                                                                   \
+  } while (0)
+
 // status strings shared with the reference (nx_c.h:381-388, nx_c_engine.h:38-50)
 #define NXH_ERR_NDIM "ndim exceeds NX_C_MAX_NDIM"
 #define NXH_ERR_BAD_KIND "unsupported bigarray kind"

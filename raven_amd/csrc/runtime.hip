@@ -104,6 +104,7 @@ NXH_EXPORT int nxh_context_create(nxh_context **out) {
 
 NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   if (!ctx) return;
+  nxh_defer_context_gone(ctx);
   (void)hipSetDevice(ctx->device);
   if (ctx->capture) {  // abandoned capture: close it so the stream can be destroyed
     hipGraph_t dropped = nullptr;
@@ -235,6 +236,7 @@ NXH_EXPORT int nxh_alloc(nxh_context *ctx, size_t bytes, void **dptr) {
 NXH_EXPORT int nxh_free(nxh_context *ctx, void *dptr) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "free", "null context");
   if (!dptr) return NXH_OK;
+  if (nxh_defer_free(ctx, dptr)) return NXH_OK;  // recorded entries still use the block: freed once they have run
   std::lock_guard<std::mutex> g(ctx->mu);
   if (ctx->live.find(dptr) == ctx->live.end())
     return nxh_fail(NXH_INVALID_ARGUMENT, "free", "pointer not owned by this context");
@@ -243,6 +245,7 @@ NXH_EXPORT int nxh_free(nxh_context *ctx, void *dptr) {
 }
 
 NXH_EXPORT int nxh_trim(nxh_context *ctx) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "trim", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "trim")) return rc;
@@ -280,6 +283,7 @@ NXH_EXPORT int nxh_memory_stats(nxh_context *ctx, uint64_t *in_use, uint64_t *ca
 NXH_EXPORT int nxh_memcpy_h2d(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "from_host", "null context");
   if (bytes == 0) return NXH_OK;
+  if (int drc = nxh_defer_uploaded(ctx, dst, src, bytes)) return drc;
   std::lock_guard<std::mutex> g(ctx->mu);
   NXH_HIP("from_host", hipSetDevice(ctx->device));
   if (ctx->capture) {
@@ -344,6 +348,7 @@ int nxh_settle_replay_faults(nxh_context *ctx, const char *op) {
 }
 
 NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "to_host", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "to_host")) return rc;
@@ -355,6 +360,7 @@ NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size
 }
 
 NXH_EXPORT int nxh_synchronize(nxh_context *ctx) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "synchronize", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "synchronize")) return rc;
@@ -388,6 +394,7 @@ static void graph_release(nxh_context *ctx, nxh_graph *gr) {
 }
 
 NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "capture_begin", "null context");
   std::lock_guard<std::mutex> whole_call(ctx->call_mu);  // not in the middle of a factorisation
   std::lock_guard<std::mutex> g(ctx->mu);
@@ -405,6 +412,7 @@ NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
 }
 
 NXH_EXPORT int nxh_capture_end(nxh_context *ctx, nxh_graph **out) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx || !out) return nxh_fail(NXH_INVALID_ARGUMENT, "capture_end", "null argument");
   std::lock_guard<std::mutex> g(ctx->mu);
   *out = nullptr;
@@ -425,6 +433,7 @@ NXH_EXPORT int nxh_capture_end(nxh_context *ctx, nxh_graph **out) {
 }
 
 NXH_EXPORT int nxh_graph_launch(nxh_context *ctx, nxh_graph *gr) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx || !gr || !gr->exec) return nxh_fail(NXH_INVALID_ARGUMENT, "graph_launch", "null argument");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "graph_launch")) return rc;
@@ -434,6 +443,7 @@ NXH_EXPORT int nxh_graph_launch(nxh_context *ctx, nxh_graph *gr) {
 }
 
 NXH_EXPORT int nxh_graph_destroy(nxh_context *ctx, nxh_graph *gr) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "graph_destroy", "null context");
   if (!gr) return NXH_OK;
   std::lock_guard<std::mutex> g(ctx->mu);
@@ -448,6 +458,7 @@ NXH_EXPORT int nxh_graph_destroy(nxh_context *ctx, nxh_graph *gr) {
 
 // ── timing ─────────────────────────────────────────────────────────────────
 NXH_EXPORT int nxh_timer_start(nxh_context *ctx) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "timer", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "timer")) return rc;
@@ -455,6 +466,7 @@ NXH_EXPORT int nxh_timer_start(nxh_context *ctx) {
   return NXH_OK;
 }
 NXH_EXPORT int nxh_timer_stop(nxh_context *ctx, float *ms) {
+  NXH_DEFER_BARRIER(ctx);
   if (!ctx || !ms) return nxh_fail(NXH_INVALID_ARGUMENT, "timer", "null argument");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "timer")) return rc;

@@ -289,6 +289,7 @@ struct ScanRow {
 };
 
 NXH_EXPORT int nxh_scan(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x, int axis) {
+  NXH_DEFER_BARRIER(ctx, out);
   static const char *const names[NXH_REDUCE_COUNT] = {"cumsum", "cumprod", "cummax", "cummin"};
   if ((unsigned)op >= NXH_REDUCE_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "scan", "unknown op");
   const char *name = names[op];

@@ -613,8 +613,10 @@ int sort_entry(nxh_context *ctx, const char *op, const nxh_tensor *out, const nx
 }  // namespace
 
 NXH_EXPORT int nxh_sort(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int axis, int descending) {
+  NXH_DEFER_BARRIER(ctx, out);
   return sort_entry(ctx, "sort", out, x, axis, descending, false);
 }
 NXH_EXPORT int nxh_argsort(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int axis, int descending) {
+  NXH_DEFER_BARRIER(ctx, out);
   return sort_entry(ctx, "argsort", out, x, axis, descending, true);
 }

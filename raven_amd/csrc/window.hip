@@ -331,6 +331,7 @@ int window_setup(const char *op, const nxh_tensor *plain, const nxh_tensor *cols
 NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int n_window_dims,
                           const int64_t *kernel_size, const int64_t *stride, const int64_t *dilation,
                           const int64_t *padding) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = "unfold";
   if (!ctx || !out || !x || !kernel_size || !stride || !dilation || !padding)
     return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
@@ -379,6 +380,7 @@ NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
 NXH_EXPORT int nxh_fold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, int n_window_dims,
                         const int64_t *output_size, const int64_t *kernel_size, const int64_t *stride,
                         const int64_t *dilation, const int64_t *padding) {
+  NXH_DEFER_BARRIER(ctx, out);
   const char *op = "fold";
   if (!ctx || !out || !x || !output_size || !kernel_size || !stride || !dilation || !padding)
     return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");

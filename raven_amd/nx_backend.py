@@ -170,6 +170,22 @@ class Backend:
         self._check(self._lib.nxh_capture_end(self._h, C.byref(g)))
         return Graph(self, g)
 
+    # -- deferred evaluation: primitives are recorded and fused below the C ABI --
+    DEFER_STATS = ("recorded", "issued", "flushes", "fallbacks", "softmax_rows", "layer_norm_rows", "gelu_tanh",
+                   "attention", "linear")
+
+    def set_deferred(self, on: bool):
+        """With the mode on, unary / binary / compare / where / cast / reduce / matmul and
+        one-element fills are recorded by the library and executed (fused where a run spells
+        softmax, layer norm, GELU, attention or a linear layer whose intermediates have died)
+        by the next call of anything else, a host read included."""
+        self._check(self._lib.nxh_set_deferred(self._h, int(bool(on))))
+
+    def deferred_stats(self):
+        v = (C.c_uint64 * len(self.DEFER_STATS))()
+        self._check(self._lib.nxh_deferred_stats(self._h, v, len(self.DEFER_STATS)))
+        return dict(zip(self.DEFER_STATS, (int(x) for x in v)))
+
     def memory_stats(self):
         v = [C.c_uint64() for _ in range(4)]
         self._check(self._lib.nxh_memory_stats(self._h, *[C.byref(x) for x in v]))

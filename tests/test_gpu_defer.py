@@ -1,0 +1,214 @@
+"""The deferred-evaluation window below the C ABI (nxh_set_deferred): the frontend
+issues its primitives one by one through the plain backend, the library records
+them and replaces the runs that spell softmax (frontend.ml:4242-4252), layer
+norm (kaun/lib/layer_norm.ml:43-68), GELU (fn.ml:31-38), the attention core
+(attention.ml:67-110) and linear + residual (linear.ml:50-52, gpt2.ml:165-176)
+by the fused entry points.
+
+What is checked: the fused call really ran (the library's counters), its result
+is bit for bit what the fused entry point gives when called directly, it agrees
+with the eager op-by-op result as closely as the fused tests promise, an
+intermediate that is still alive is written exactly as the eager path writes it,
+and nothing the record touches is handed out again before the record has run."""
+
+import math
+
+import numpy as np
+import pytest
+
+from helpers import TOL, close, decode, encode, logical, pair, same_bits
+from raven_amd import dtype as dt
+from raven_amd.kaun_gpt2 import Config, Gpt2, LayerNorm, Linear, host_params, upload
+from raven_amd.nx_frontend import Nx
+
+pytestmark = pytest.mark.gpu
+
+
+class deferred:
+    """The mode is switched off again even when the body raises (the context is shared)."""
+
+    def __init__(self, hip):
+        self.hip = hip
+
+    def __enter__(self):
+        self.hip.set_deferred(True)
+        self.before = self.hip.deferred_stats()
+        return self
+
+    def delta(self):
+        now = self.hip.deferred_stats()
+        return {k: now[k] - self.before[k] for k in now}
+
+    def __exit__(self, *exc):
+        try:
+            self.hip.set_deferred(False)
+        except Exception:
+            if exc[0] is None:
+                raise
+        return False
+
+
+def tensor(hip, a, d):
+    return hip.reshape(hip.from_host(np.ascontiguousarray(a), d), a.shape)
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_softmax_layer_norm_and_gelu_runs_fuse(hip, oracle, d):
+    rng = np.random.default_rng(300 + d.tag)
+    nx = Nx(hip)
+    model = Gpt2(nx, Config())
+    x = tensor(hip, encode(rng.standard_normal((6, 40, 96)) * 2, d, oracle), d)
+    gamma = tensor(hip, encode(1 + 0.1 * rng.standard_normal(96), d, oracle), d)
+    beta = tensor(hip, encode(0.1 * rng.standard_normal(96), d, oracle), d)
+    eager = [logical(nx.softmax(x)), logical(model.layer_norm(LayerNorm(gamma, beta), x, 1e-5)), logical(model.gelu_approx(x))]
+    direct = [logical(hip.softmax_rows(x)), logical(hip.layer_norm_rows(x, gamma, beta, 1e-5)), logical(hip.gelu_tanh(x))]
+    with deferred(hip) as win:
+        got = [nx.softmax(x), model.layer_norm(LayerNorm(gamma, beta), x, 1e-5), model.gelu_approx(x)]
+        got = [logical(t) for t in got]
+        s = win.delta()
+    assert (s["softmax_rows"], s["layer_norm_rows"], s["gelu_tanh"], s["fallbacks"]) == (1, 1, 1, 0), s
+    assert s["issued"] == 0 and s["recorded"] >= 5 + 14 + 9
+    for g, dr, e, name in zip(got, direct, eager, ("softmax", "layer_norm", "gelu")):
+        same_bits(g, dr, f"{name}: the recorded run against the fused entry point")
+        close(g, e, d, oracle, 4 * TOL[d.name][0] if d is not dt.float32 else 2e-6, 2e-6, f"{name}: against the eager sequence")
+    same_bits(got[2], eager[2], "gelu has no sum: equal to the eager sequence bit for bit")
+
+
+def test_an_intermediate_that_is_still_held_is_written_as_recorded(hip, oracle):
+    rng = np.random.default_rng(31)
+    nx = Nx(hip)
+    x = tensor(hip, rng.standard_normal((33, 70)).astype(np.float32), dt.float32)
+    want_e = logical(nx.exp(nx.sub(x, nx.max(x, [-1], keepdims=True))))
+    want = logical(nx.softmax(x))
+    with deferred(hip) as win:
+        # the same five primitives, with the exponentials kept by the caller
+        mx = nx.max(x, [-1], keepdims=True)
+        e = nx.exp(nx.sub(x, mx))
+        out = nx.div(e, nx.sum(e, [-1], keepdims=True))
+        del mx
+        got, got_e = logical(out), logical(e)
+        s = win.delta()
+    assert s["softmax_rows"] == 0 and s["issued"] == s["recorded"] == 5, s
+    same_bits(got, want, "softmax with an observed intermediate")
+    same_bits(got_e, want_e, "the observed intermediate")
+
+
+def test_blocks_of_recorded_entries_are_not_handed_out_again(hip):
+    """An output is freed while its entry is recorded and a new, equally large output is
+    allocated right behind it: the free is held back, so the two never share a block."""
+    nx = Nx(hip)
+    a = hip.full(dt.float32, (256, 256), 3.0)
+    b = hip.full(dt.float32, (256, 256), 4.0)
+    with deferred(hip):
+        t = nx.add(a, b)          # recorded: 7
+        u = nx.mul(t, t)          # recorded: 49, reads t
+        del t                     # t's block may not be reused before the record has run
+        v = nx.sub(nx.add(a, a), b)  # fresh outputs of the same size: 2
+        w = nx.add(u, v)          # 51
+        got = logical(w)
+    assert np.all(got == 51.0)
+    stats = hip.memory_stats()
+    hip.synchronize()
+    assert hip.memory_stats()["in_use"] <= stats["in_use"]
+
+
+def test_linear_with_bias_and_residual_fuses(hip, oracle):
+    rng = np.random.default_rng(32)
+    d = dt.bfloat16
+    nx = Nx(hip)
+    model = Gpt2(nx, Config())
+    x = tensor(hip, encode(rng.standard_normal((4, 128, 256)), d, oracle), d)
+    w = tensor(hip, encode(rng.standard_normal((256, 512)) * 0.05, d, oracle), d)
+    b = tensor(hip, encode(rng.standard_normal(512), d, oracle), d)
+    r = tensor(hip, encode(rng.standard_normal((4, 128, 512)), d, oracle), d)
+    eager = logical(nx.add(r, model.linear(Linear(w, b), x)))
+    with deferred(hip) as win:
+        got = logical(nx.add(r, model.linear(Linear(w, b), x)))
+        s = win.delta()
+    assert (s["linear"], s["issued"], s["fallbacks"]) == (1, 0, 0), s
+    same_bits(got, eager, "linear + bias + residual: the epilogue rounds where the three calls round")
+
+
+@pytest.mark.parametrize("kind", ["causal", "mask", "none"])
+def test_attention_core_fuses(hip, oracle, kind):
+    rng = np.random.default_rng(33)
+    d = dt.bfloat16
+    b, h, s, hd = 2, 3, 96, 64
+    nx = Nx(hip)
+    model = Gpt2(nx, Config())
+    q, k, v = (tensor(hip, encode(rng.standard_normal((b, h, s, hd)), d, oracle), d) for _ in range(3))
+
+    def mask_of():
+        if kind == "causal":
+            idx = nx.arange(dt.int32, 0, s, 1)
+            return nx.less_equal(nx.reshape((1, s), idx), nx.reshape((s, 1), idx))
+        if kind == "mask":
+            m = (np.random.default_rng(34).random((s, s)) < 0.7).astype(np.uint8)
+            m[:, 0] = 1
+            return tensor(hip, m, dt.bool_)
+        return None
+
+    eager = logical(model.scaled_dot_product_attention(q, k, v, mask_of()))
+    with deferred(hip) as win:
+        got = logical(model.scaled_dot_product_attention(q, k, v, mask_of()))
+        st = win.delta()
+    assert (st["attention"], st["fallbacks"], st["softmax_rows"]) == (1, 0, 0), st
+    # the causal mask is recognised from its aranges and never computed; a given mask is only read
+    assert st["issued"] == 0, st
+    direct = logical(hip.attention(q, k, v, 1.0 / math.sqrt(hd),
+                                   mask=None if kind != "mask" else hip.expand(hip.reshape(mask_of(), (1, 1, s, s)), (b, h, s, s)),
+                                   masked_value=None if kind == "none" else float("-inf"), causal=kind == "causal"))
+    same_bits(got, direct, "the recorded run against nxh_attention")
+    close(got, eager, d, oracle, 2 * 2.0 ** -7, 2e-3, "against the eager sequence")
+
+
+def test_errors_of_recorded_primitives_surface_when_the_record_runs(hip):
+    a = hip.full(dt.float32, (4, 5), 1.0)
+    bad = hip.full(dt.float32, (4, 6), 1.0)
+    with deferred(hip):
+        out = hip.buffer(dt.float32, (4, 5))
+        import ctypes as C
+
+        o, x, y = out._desc(), a._desc(), bad._desc()
+        rc = hip._lib.nxh_binary(hip._h, 0, C.byref(o), C.byref(x), C.byref(y))
+        assert rc == 0  # recorded, not checked yet
+        with pytest.raises(ValueError, match="shape mismatch"):
+            hip.synchronize()
+        hip.synchronize()  # the record is gone
+        ok = Nx(hip).add(a, a)
+        assert np.all(logical(ok) == 2.0)
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16], ids=lambda d: d.name)
+def test_gpt2_forward_with_the_library_window(hip, oracle, d):
+    """The frontend's calls straight through the plain backend, recorded and fused below the ABI:
+    every sequence is found, and the logits are bit for bit those of the Python window (which
+    issues the same fused calls on the same operands)."""
+    from raven_amd.nx_window import Window
+
+    cfg = Config(vocab_size=1031, n_positions=128, n_embd=256, n_layer=2, n_head=4, n_inner=1024)
+    hp = host_params(cfg, seed=16, stddev=0.05)
+    ids = np.random.default_rng(17).integers(0, cfg.vocab_size, (2, 96)).astype(np.int32)
+    enc = lambda a, dd: encode(a, dd, oracle)  # noqa: E731
+
+    def run(front):
+        nx = Nx(front)
+        params = upload(nx, hp, d, enc)
+        t_ids = nx.create(dt.int32, ids.shape, ids)
+        return Gpt2(nx, cfg).logits(params, t_ids)
+
+    eager = decode(logical(run(hip)), d, oracle)
+    win = Window(hip)
+    py = logical(win.force(run(win)))
+    with deferred(hip) as lib:
+        got = logical(run(hip))
+        s = lib.delta()
+    L = cfg.n_layer
+    assert (s["layer_norm_rows"], s["gelu_tanh"], s["linear"], s["fallbacks"]) == (2 * L + 1, L, 6 * L, 0), s
+    assert (s["attention"], s["softmax_rows"]) == ((L, 0) if d is dt.bfloat16 else (0, L)), s
+    same_bits(got, py, "library window against the Python window")
+    gv = decode(got, d, oracle)
+    if d is dt.float32:
+        assert np.max(np.abs(gv - eager)) <= 2e-5 * max(1.0, np.max(np.abs(eager)))
+    else:
+        assert np.all(np.abs(gv - eager) <= 6e-2 + 6e-2 * np.abs(eager))
