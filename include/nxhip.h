@@ -396,14 +396,21 @@ int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nx
    nxh_unary / nxh_binary / nxh_compare / nxh_where / nxh_cast / nxh_reduce /
    nxh_matmul and a one-element nxh_fill only record their call. The record is
    executed, in issue order, by the next call of any other entry point (a host
-   read and nxh_synchronize included) or when it reaches 512 entries; a run that
-   spells one of those sequences, and whose intermediate results were given back
-   with nxh_free while still recorded and are read only inside the run, is replaced
-   by the fused entry point below. Observable results are the eager ones, except
-   that an error of a recorded primitive is returned by the call that executes the
-   record, and that a fused row sum may be added in another order. nxh_free of a
-   block the record still uses takes effect once the record has run. Switching
-   the mode (either way) executes the record first. */
+   read and nxh_synchronize included) or when it reaches 512 entries. A run that
+   spells one of those sequences, and whose intermediate results are read only
+   inside the run, is replaced by the fused entry point below. An intermediate
+   whose block was given back with nxh_free while recorded is never written; one
+   whose block is still held when the record executes is postponed: it is
+   written, as recorded, just before the first call that reads it (or that
+   writes something it was computed from), and never if nxh_free comes first.
+   So handles that are released late (finalisers) fuse like handles released at
+   once. Observable results are the eager ones, except that an error of a
+   recorded primitive is returned by the call that executes it, and that a
+   fused row sum may be added in another order. nxh_free of a block that
+   recorded or postponed work still uses takes effect once that work has run or
+   been dropped. Switching the mode (either way) executes the record first, and
+   switching it off writes everything postponed. Nothing is postponed while a
+   graph is being captured. */
 int nxh_set_deferred(nxh_context *ctx, int on);
 /* Counters since the context was created, in this order. */
 enum {
@@ -416,6 +423,8 @@ enum {
   NXH_DEFER_GELU,           /* ... nxh_gelu_tanh */
   NXH_DEFER_ATTENTION,      /* ... nxh_attention */
   NXH_DEFER_LINEAR,         /* ... nxh_linear */
+  NXH_DEFER_POSTPONED,      /* entries of fused runs left unexecuted because their result was still held */
+  NXH_DEFER_MATERIALISED,   /* of those, issued later because something read the result */
   NXH_DEFER_STAT_COUNT
 };
 int nxh_deferred_stats(nxh_context *ctx, uint64_t *stats, int count);

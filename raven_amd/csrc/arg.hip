@@ -380,7 +380,7 @@ struct ArgRow {
 
 NXH_EXPORT int nxh_argreduce(nxh_context *ctx, int is_min, const nxh_tensor *out, const nxh_tensor *x,
                              int axis) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x);
   const char *name = is_min ? "argmin" : "argmax";
   if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, name, "null argument");
   int rc = nxh_check_tensor(name, out);

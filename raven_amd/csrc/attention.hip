@@ -312,7 +312,7 @@ bool rows_aligned(const nxh_tensor *t, int bytes) {
 NXH_EXPORT int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q, const nxh_tensor *k,
                              const nxh_tensor *v, const void *scale, const nxh_tensor *mask,
                              const void *masked_value, int causal) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, q, k, v, mask);
   const char *op = "attention";
   if (!ctx || !out || !q || !k || !v || (mask && !masked_value) || (causal && !masked_value))
     return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");

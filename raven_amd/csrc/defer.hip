@@ -12,19 +12,26 @@
 // reaches 512 entries. At that moment a run of entries that spells one of the
 // five sequences is replaced by the fused call (nxh_softmax_rows,
 // nxh_layer_norm_rows, nxh_gelu_tanh, nxh_attention, nxh_linear), provided that
-// nobody can observe its intermediate results: their storage was given back with
-// nxh_free while the entry was still recorded, and all their readers are inside
-// the run. Everything else is issued as recorded, so what a caller can observe is
-// the eager result, with two differences: an error of a recorded primitive
-// surfaces from the call that executes the record, and a fused float result may
-// differ from the op-by-op one by the order in which a row's sum is added.
+// every recorded reader of its intermediate results is inside the run. An
+// intermediate whose storage was given back with nxh_free while recorded is never
+// written. One whose handle is still held is POSTPONED: its entry (and the rest
+// of the run, with the blocks it reads kept from reuse) stays behind, unexecuted,
+// and is issued as recorded the moment anything reads that block (an operand of a
+// later call, a host read) or writes a block the run reads; when nxh_free arrives
+// first, it is dropped. So a host whose handles die late (a garbage collector's
+// finalisers) gets the same fused kernels as one that frees at once. Everything
+// else is issued as recorded: what a caller can observe is the eager result, with
+// two differences: an error of a recorded primitive surfaces from the call that
+// executes it, and a fused float result may differ from the op-by-op one by the
+// order in which a row's sum is added.
 //
 // Any binding gets this by switching the mode on: the caller keeps allocating
 // outputs (nxh_alloc) and freeing dead handles (nxh_free) exactly as before. A
-// free that arrives while recorded entries still use the block is held back until
-// they have run, so the allocator never hands out memory the record will touch.
-// A host whose handles die late (a garbage collector's finalisers) fuses less,
-// never wrongly: an intermediate that is still alive is written as recorded.
+// free that arrives while recorded or postponed entries still use the block is
+// held back until they have run or been dropped, so the allocator never hands out
+// memory they will touch. While a graph is being captured nothing is postponed
+// (a later materialisation would fall outside the graph): there an intermediate
+// that is still held blocks the fusion and is written as recorded.
 
 #include <array>
 #include <memory>
@@ -61,10 +68,20 @@ struct Known {  // what the window knows about the contents of a block
   int64_t causal = 0;
 };
 
+// The unexecuted rest of a fused run: interior entries, and the scalar fills and causal
+// mask that only the run read, in issue order. `alive` counts members whose handle is held.
+struct Postponed {
+  std::vector<std::unique_ptr<DEntry>> members;
+  int alive = 0;
+};
+
 struct Window {
   std::mutex mu;
   bool on = false;
+  bool may_postpone = true;  // false while the executing flush is being captured
   std::vector<std::unique_ptr<DEntry>> entries;
+  std::vector<std::unique_ptr<Postponed>> postponed;
+  std::unordered_map<void *, Postponed *> postponed_out;  // block -> the run one of whose members writes it
   std::unordered_map<void *, DEntry *> producer;  // block -> its recorded writer
   std::unordered_map<void *, int> pinned;         // block -> recorded entries that read or write it
   std::vector<void *> held_frees;
@@ -164,10 +181,12 @@ bool rows_ok(const Opnd &o, const nxh_tensor &shape) {
   if (!same_shape(*o.t, shape)) return false;
   return shape.shape[shape.ndim - 1] == 1 || o.t->strides[shape.ndim - 1] == 1;
 }
-// No handle to an interior result is left and all its readers are inside the run.
+// All recorded readers of the interior results are inside the run (and, where nothing may be
+// postponed, no handle to one is left).
+thread_local bool tls_may_postpone = true;
 bool hidden(const std::vector<DEntry *> &interior, const DEntry *anchor) {
   for (DEntry *e : interior) {
-    if (e->alive) return false;
+    if (e->alive && !tls_may_postpone) return false;
     for (DEntry *r : e->readers) {
       bool inside = r == anchor;
       for (DEntry *i : interior) inside = inside || i == r;
@@ -609,6 +628,92 @@ void unpin(Window *w, void *block) {
   auto it = w->pinned.find(block);
   if (it != w->pinned.end() && --it->second <= 0) w->pinned.erase(it);
 }
+void unpin_entry(Window *w, const DEntry *e) {
+  unpin(w, e->out.data);
+  for (int i = 0; i < e->nin; i++) unpin(w, e->in[i].data);
+}
+// What the window now knows about a result that was written and is still held.
+void remember(Window *w, const DEntry *e) {
+  if (!e->alive || (e->kind != D_FULL && !e->causal)) return;
+  Known &k = w->known[e->out.data];
+  k = Known{};
+  k.dtype = e->out.dtype;
+  if (e->kind == D_FULL) memcpy(k.scalar, e->value, 16), k.has_scalar = true;
+  k.causal = e->causal;
+}
+// Frees that were held back for blocks nothing recorded or postponed uses any more.
+void release_held(nxh_context *ctx, Window *w) {
+  std::vector<void *> frees;
+  frees.swap(w->held_frees);
+  for (void *p : frees) {
+    if (w->pinned.count(p)) {
+      w->held_frees.push_back(p);
+      continue;
+    }
+    w->known.erase(p);
+    std::lock_guard<std::mutex> g(ctx->mu);
+    nxh_free_locked(ctx, p);
+  }
+}
+
+// Ends a postponed run: with `write`, its members are issued as recorded first (somebody is
+// about to look); without, they are forgotten (every handle is gone).
+int retire(nxh_context *ctx, Window *w, Postponed *run, bool write) {
+  int rc = NXH_OK;
+  const bool outer = tls_in_flush;
+  tls_in_flush = true;
+  for (auto &m : run->members) {
+    if (write && !rc && !m->done) {
+      rc = issue(ctx, m.get());
+      w->stats[NXH_DEFER_ISSUED]++;
+      w->stats[NXH_DEFER_MATERIALISED]++;
+      if (!rc) remember(w, m.get());
+    }
+    w->postponed_out.erase(m->out.data);
+    unpin_entry(w, m.get());
+  }
+  tls_in_flush = outer;
+  for (size_t i = 0; i < w->postponed.size(); i++)
+    if (w->postponed[i].get() == run) {
+      w->postponed.erase(w->postponed.begin() + (long)i);
+      break;
+    }
+  release_held(ctx, w);
+  return rc;
+}
+int retire_all(nxh_context *ctx, Window *w, bool write) {
+  int rc = NXH_OK;
+  while (!w->postponed.empty()) {
+    const int r = retire(ctx, w, w->postponed.front().get(), write);
+    if (!rc) rc = r;
+  }
+  return rc;
+}
+// Before `block` is read: the postponed run that would have written it runs now. A scalar fill
+// or a causal mask that rode along with a run depends on nothing in it and is written alone.
+int settle_read(nxh_context *ctx, Window *w, const void *block) {
+  if (w->postponed.empty()) return NXH_OK;
+  auto it = w->postponed_out.find(const_cast<void *>(block));
+  if (it == w->postponed_out.end()) return NXH_OK;
+  for (auto &m : it->second->members) {
+    if (m->out.data != block || (m->kind != D_FULL && !(m->kind == D_COMPARE && m->causal))) continue;
+    if (m->done) return NXH_OK;
+    const bool outer = tls_in_flush;
+    tls_in_flush = true;
+    const int rc = issue(ctx, m.get());
+    tls_in_flush = outer;
+    w->stats[NXH_DEFER_ISSUED]++;
+    w->stats[NXH_DEFER_MATERIALISED]++;
+    if (!rc) remember(w, m.get());
+    return rc;
+  }
+  return retire(ctx, w, it->second, true);
+}
+// Before `block` is written by anything but the record: a postponed run may read it, or write it later.
+int settle_write(nxh_context *ctx, Window *w, const void *block) {
+  if (w->postponed.empty() || !w->pinned.count(const_cast<void *>(block))) return NXH_OK;
+  return retire_all(ctx, w, true);
+}
 
 // Executes the record. Called with w->mu held.
 int flush_locked(nxh_context *ctx, Window *w) {
@@ -617,6 +722,11 @@ int flush_locked(nxh_context *ctx, Window *w) {
   entries.swap(w->entries);
   w->producer.clear();
   w->stats[NXH_DEFER_FLUSHES]++;
+  {
+    std::lock_guard<std::mutex> g(ctx->mu);
+    w->may_postpone = ctx->capture == nullptr;
+  }
+  tls_may_postpone = w->may_postpone;
   std::unordered_map<DEntry *, Plan> plans;
   for (size_t i = entries.size(); i-- > 0;) {
     DEntry *e = entries[i].get();
@@ -627,14 +737,41 @@ int flush_locked(nxh_context *ctx, Window *w) {
       plans.emplace(e, std::move(p));
     }
   }
+  // A scalar fill, or a causal mask taken as a flag, that only one fused run reads belongs to that
+  // run: it is written only if the run is (when it is declined, or postponed and looked at later).
+  std::unordered_map<DEntry *, DEntry *> home;  // entry -> the anchor of its run
+  for (auto &up : entries) {
+    DEntry *e = up.get();
+    if ((e->kind != D_FULL && !(e->kind == D_COMPARE && e->causal)) || e->readers.empty()) continue;
+    if (e->alive && !w->may_postpone) continue;
+    DEntry *anchor = nullptr;
+    bool single = true;
+    for (DEntry *r : e->readers) {
+      DEntry *a = r->fused_into ? r->fused_into : (plans.count(r) ? r : nullptr);
+      single = single && a && (!anchor || anchor == a);
+      anchor = a;
+    }
+    if (!single) continue;
+    const Plan &pl = plans.at(anchor);
+    if (e->kind == D_COMPARE && !(pl.stat == NXH_DEFER_ATTENTION && pl.causal_flag)) continue;
+    home[e] = anchor;
+  }
+  auto members_of = [&](DEntry *anchor) {
+    std::vector<DEntry *> run = plans.at(anchor).interior;
+    for (auto &h : home)
+      if (h.second == anchor) run.push_back(h.first);
+    std::sort(run.begin(), run.end(), [](DEntry *a, DEntry *b) { return a->id < b->id; });
+    return run;
+  };
+  std::vector<DEntry *> fused;  // anchors whose fused call ran
   int rc = NXH_OK;
   tls_in_flush = true;
   for (auto &up : entries) {
     DEntry *e = up.get();
     if (rc) break;
-    if (e->fused_into || e->done) continue;
-    if (e->kind == D_COMPARE && e->causal && !e->alive) {
-      // a causal mask nobody holds any more, whose readers all took it as a flag: never computed
+    if (e->fused_into || e->done || home.count(e)) continue;
+    if (e->kind == D_COMPARE && e->causal && !e->alive && !e->readers.empty()) {
+      // a causal mask nobody holds any more, whose readers (several runs) all took it as a flag
       bool flagged = true;
       for (DEntry *r : e->readers) {
         auto it = r->fused_into ? plans.find(r->fused_into) : plans.end();
@@ -646,7 +783,7 @@ int flush_locked(nxh_context *ctx, Window *w) {
       }
     }
     if (e->kind == D_FULL) {
-      // filled only if a handle is left (or, above, when a reader outside a fused run is issued)
+      // filled only if a handle is left (or, in issue(), when a reader outside a fused run is issued)
       if (e->alive) rc = issue(ctx, e);
       continue;
     }
@@ -661,44 +798,50 @@ int flush_locked(nxh_context *ctx, Window *w) {
     if (rc == NXH_FAILURE) {
       // the fused form was declined: the run as recorded, in its own order
       w->stats[NXH_DEFER_FALLBACKS]++;
-      std::vector<DEntry *> run = it->second.interior;
-      std::sort(run.begin(), run.end(), [](DEntry *a, DEntry *b) { return a->id < b->id; });
       rc = NXH_OK;
-      for (DEntry *inner : run) {
+      for (DEntry *inner : members_of(e)) {
         inner->fused_into = nullptr;
-        if (!rc) rc = issue(ctx, inner);
+        home.erase(inner);
+        if (!rc) rc = issue(ctx, inner), w->stats[NXH_DEFER_ISSUED]++;
       }
       e->done = false;
-      if (!rc) rc = issue(ctx, e);
+      if (!rc) rc = issue(ctx, e), w->stats[NXH_DEFER_ISSUED]++;
     } else if (!rc) {
       w->stats[it->second.stat]++;
+      fused.push_back(e);
     }
   }
   tls_in_flush = false;
-  // what is known about results that were written, and the blocks the record held
+  // The members of a fused run that somebody still holds stay behind with the rest of their run.
+  std::unordered_map<DEntry *, Postponed *> kept;
+  if (!rc && w->may_postpone)
+    for (DEntry *anchor : fused) {
+      std::vector<DEntry *> run = members_of(anchor);
+      int alive = 0;
+      for (DEntry *m : run) alive += m->alive ? 1 : 0;
+      if (!alive) continue;
+      auto pr = std::make_unique<Postponed>();
+      pr->alive = alive;
+      for (DEntry *m : run) kept[m] = pr.get();
+      w->postponed.push_back(std::move(pr));
+    }
   for (auto &up : entries) {
     DEntry *e = up.get();
-    if (e->alive && e->done && !rc && (e->kind == D_FULL || e->causal)) {
-      Known &k = w->known[e->out.data];
-      k = Known{};
-      k.dtype = e->out.dtype;
-      if (e->kind == D_FULL) memcpy(k.scalar, e->value, 16), k.has_scalar = true;
-      k.causal = e->causal;
-    }
-    unpin(w, e->out.data);
-    for (int i = 0; i < e->nin; i++) unpin(w, e->in[i].data);
-  }
-  std::vector<void *> frees;
-  frees.swap(w->held_frees);
-  for (void *p : frees) {
-    if (w->pinned.count(p)) {
-      w->held_frees.push_back(p);
+    auto k = kept.find(e);
+    if (k == kept.end()) {
+      if (e->done && !rc) remember(w, e);
+      unpin_entry(w, e);
       continue;
     }
-    w->known.erase(p);
-    std::lock_guard<std::mutex> g(ctx->mu);
-    nxh_free_locked(ctx, p);
+    // cut loose from entries that are about to go away; its operands' blocks stay pinned
+    for (int i = 0; i < 3; i++) e->prod[i] = nullptr;
+    e->readers.clear();
+    e->fused_into = nullptr;
+    w->postponed_out[e->out.data] = k->second;
+    w->stats[NXH_DEFER_POSTPONED]++;
+    k->second->members.push_back(std::move(up));  // `entries` is in issue order, so the run is too
   }
+  release_held(ctx, w);
   return rc;
 }
 
@@ -736,17 +879,70 @@ int nxh_defer_flush(nxh_context *ctx) {
   return flush_locked(ctx, w);
 }
 
-// Before an entry point that is not recorded: the record runs first, and whatever the
-// window knew about the blocks this call writes is forgotten.
+// Before an entry point that is not recorded and does not say what it reads: the record runs
+// first, everything postponed is written, and whatever the window knew about the blocks this
+// call writes is forgotten.
 int nxh_defer_barrier(nxh_context *ctx, const nxh_tensor *out0, const nxh_tensor *out1, const nxh_tensor *out2) {
   if (!ctx || tls_in_flush) return NXH_OK;
   Window *w = window_of(ctx, false);
   if (!w) return NXH_OK;
   std::lock_guard<std::mutex> g(w->mu);
-  const int rc = flush_locked(ctx, w);
+  int rc = flush_locked(ctx, w);
+  if (!rc) rc = retire_all(ctx, w, true);
   for (const nxh_tensor *t : {out0, out1, out2})
     if (t) w->known.erase(t->data);
   return rc;
+}
+
+// The same for an entry point that names its operands: the first n_out are written, the
+// others read. Only the postponed runs those blocks belong to are written.
+int nxh_defer_touch(nxh_context *ctx, const nxh_tensor *const *tensors, int n, int n_out) {
+  if (!ctx || tls_in_flush) return NXH_OK;
+  Window *w = window_of(ctx, false);
+  if (!w) return NXH_OK;
+  std::lock_guard<std::mutex> g(w->mu);
+  int rc = flush_locked(ctx, w);
+  for (int i = 0; i < n; i++) {
+    const nxh_tensor *t = tensors[i];
+    if (!t) continue;
+    if (i < n_out) {
+      if (!rc) rc = settle_write(ctx, w, t->data);
+      w->known.erase(t->data);
+    } else if (!rc) {
+      rc = settle_read(ctx, w, t->data);
+    }
+  }
+  return rc;
+}
+
+// An entry point that touches no tensor (a synchronisation, a timer): the record runs, what is
+// postponed stays so.
+int nxh_defer_quiet(nxh_context *ctx) {
+  if (!ctx || tls_in_flush) return NXH_OK;
+  Window *w = window_of(ctx, false);
+  if (!w) return NXH_OK;
+  std::lock_guard<std::mutex> g(w->mu);
+  return flush_locked(ctx, w);
+}
+
+// A host read of device bytes at `src` (any address inside a block).
+int nxh_defer_host_read(nxh_context *ctx, const void *src) {
+  if (!ctx || tls_in_flush) return NXH_OK;
+  Window *w = window_of(ctx, false);
+  if (!w) return NXH_OK;
+  std::lock_guard<std::mutex> g(w->mu);
+  int rc = flush_locked(ctx, w);
+  if (rc || w->postponed.empty()) return rc;
+  const void *block = nullptr;
+  {
+    std::lock_guard<std::mutex> a(ctx->mu);
+    for (auto &po : w->postponed_out) {
+      auto live = ctx->live.find(po.first);
+      const char *base = (const char *)po.first;
+      if (live != ctx->live.end() && (const char *)src >= base && (const char *)src < base + std::max<size_t>(live->second, 1)) block = po.first;
+    }
+  }
+  return block ? settle_read(ctx, w, block) : NXH_OK;
 }
 
 // Records one primitive. Returns NXH_OK when recorded, -1 when the call has to run now (the
@@ -758,6 +954,10 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
   std::lock_guard<std::mutex> g(w->mu);
   bool ok = out && out->ndim >= 0 && out->ndim <= NXH_MAX_NDIM && n_axes <= NXH_MAX_NDIM;
   for (int k = 0; ok && k < nin; k++) ok = ins[k] && ins[k]->ndim >= 0 && ins[k]->ndim <= NXH_MAX_NDIM;
+  // an operand that a postponed run would have written is written now, ahead of the record
+  // (nothing recorded writes what that run reads: recorded outputs are fresh blocks)
+  for (int k = 0; ok && k < nin; k++)
+    if (int rc = settle_read(ctx, w, ins[k]->data)) return rc;
   // The output must be a whole block of this context that no recorded entry touches yet:
   // results are fresh allocations (backend_intf.ml:61-67); anything else runs now.
   if (ok) {
@@ -767,8 +967,11 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
   ok = ok && out->offset == 0 && c_contiguous(*out) && !w->pinned.count(out->data);
   if (ok && kind == D_FULL) ok = numel(*out) == 1 && !nxh_is_packed(out->dtype);
   if (!ok) {
-    const int rc = flush_locked(ctx, w);
-    if (out) w->known.erase(out->data);
+    int rc = flush_locked(ctx, w);
+    if (out) {
+      if (!rc) rc = settle_write(ctx, w, out->data);
+      w->known.erase(out->data);
+    }
     return rc ? rc : -1;
   }
   auto e = std::make_unique<DEntry>();
@@ -795,7 +998,8 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
   return NXH_OK;
 }
 
-// nxh_free: true when the window took the free over (the block is used by the record).
+// nxh_free: true when the window took the free over (the block is used by the record, or by a
+// postponed run that other handles keep).
 bool nxh_defer_free(nxh_context *ctx, void *p) {
   if (tls_in_flush) return false;
   Window *w = window_of(ctx, false);
@@ -803,6 +1007,13 @@ bool nxh_defer_free(nxh_context *ctx, void *p) {
   std::lock_guard<std::mutex> g(w->mu);
   auto it = w->producer.find(p);
   if (it != w->producer.end()) it->second->alive = false;
+  auto po = w->postponed_out.find(p);
+  if (po != w->postponed_out.end()) {
+    Postponed *run = po->second;
+    for (auto &m : run->members)
+      if (m->out.data == p && m->alive) m->alive = false, run->alive--;
+    if (run->alive <= 0) retire(ctx, w, run, false);  // nobody can look any more
+  }
   if (w->pinned.count(p)) {
     w->held_frees.push_back(p);
     return true;
@@ -811,15 +1022,18 @@ bool nxh_defer_free(nxh_context *ctx, void *p) {
   return false;
 }
 
-// nxh_memcpy_h2d: the record runs first if it touches the block; a small upload is remembered
-// (the aranges of a causal mask are recognised from it).
+// nxh_memcpy_h2d: the record runs first if it touches the block, and so does whatever is
+// postponed; a small upload is remembered (the aranges of a causal mask are recognised from it).
 int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
   if (tls_in_flush) return NXH_OK;
   Window *w = window_of(ctx, false);
   if (!w) return NXH_OK;
   std::lock_guard<std::mutex> g(w->mu);
   int rc = NXH_OK;
-  if (w->pinned.count(dst)) rc = flush_locked(ctx, w);
+  if (w->pinned.count(dst)) {
+    rc = flush_locked(ctx, w);
+    if (!rc) rc = settle_write(ctx, w, dst);
+  }
   w->known.erase(dst);
   if (w->on && bytes > 0 && bytes <= 65536 && bytes % 4 == 0) {
     Known &k = w->known[dst];
@@ -839,9 +1053,14 @@ NXH_EXPORT int nxh_set_deferred(nxh_context *ctx, int on) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "set_deferred", "null context");
   Window *w = window_of(ctx, true);
   std::lock_guard<std::mutex> g(w->mu);
-  const int rc = flush_locked(ctx, w);
+  int rc = flush_locked(ctx, w);
   w->on = on != 0;
-  if (!w->on) w->known.clear();
+  if (!w->on) {
+    // with the mode off no call announces what it reads: nothing may stay unwritten
+    const int r = retire_all(ctx, w, true);
+    if (!rc) rc = r;
+    w->known.clear();
+  }
   return rc;
 }
 

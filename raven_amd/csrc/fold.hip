@@ -477,6 +477,6 @@ NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const
 // the workspace is refused before anything is launched.
 NXH_EXPORT int nxh_reduce_noalloc(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
                                   const int32_t *axes, int n_axes) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x);
   return reduce_entry(ctx, op, out, x, axes, n_axes, true);
 }

@@ -128,7 +128,7 @@ struct alignas(16) B16x {
 static int copy_impl(nxh_context *ctx, const char *op, const nxh_tensor *out, const nxh_tensor *x);
 
 NXH_EXPORT int nxh_copy(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x);
   NXH_CHECK_ARGS("copy", out, x);
   return copy_impl(ctx, "copy", out, x);
 }
@@ -257,7 +257,7 @@ NXH_EXPORT int nxh_cast(nxh_context *ctx, const nxh_tensor *out, const nxh_tenso
   if (!nxh_same_shape(out, x)) return nxh_fail(NXH_INVALID_ARGUMENT, "cast", NXH_ERR_SHAPE);
   const int src = x->dtype, dst = out->dtype;
   if (nxh_is_packed(src) || nxh_is_packed(dst)) {
-    NXH_DEFER_BARRIER(ctx, out);
+    NXH_DEFER_TOUCH(ctx, 1, out, x);
     return cast_packed(ctx, out, x);
   }
   NXH_DEFER_RECORD(ctx, NXH_D_CAST, 0, out, 1, nullptr, 0, nullptr, x);

@@ -974,7 +974,7 @@ NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tenso
 
 NXH_EXPORT int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const nxh_tensor *w,
                           const nxh_tensor *bias, const nxh_tensor *residual) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x, w, bias, residual);
   if (!bias && !residual) return matmul_entry(ctx, "matmul", out, x, w, nullptr, nullptr);
   return matmul_entry(ctx, "linear", out, x, w, bias, residual);
 }

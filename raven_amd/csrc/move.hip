@@ -111,7 +111,7 @@ static void launch_any_e(nxh_context *ctx, const GatherAnyArgs &a) {
 
 NXH_EXPORT int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *data,
                           const nxh_tensor *indices, int axis) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, data, indices);
   const char *op = "gather";
   if (!ctx || !out || !data || !indices) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -429,7 +429,7 @@ static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add, int
 
 NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *indices,
                            const nxh_tensor *updates, int axis, int mode) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, indices, updates);
   const char *op = "scatter";
   if (!ctx || !out || !indices || !updates) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -550,7 +550,7 @@ __global__ __launch_bounds__(256) void threefry_kernel(ThreefryArgs a) {
 
 NXH_EXPORT int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *key,
                             const nxh_tensor *counter) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, key, counter);
   const char *op = "threefry";
   if (!ctx || !out || !key || !counter) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -709,7 +709,7 @@ static int pad_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *
 
 NXH_EXPORT int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *fill_value,
                        const int64_t *pad_before) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x);
   const char *op = "pad";
   if (!ctx || !out || !x || !fill_value || (out->ndim > 0 && !pad_before))
     return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");

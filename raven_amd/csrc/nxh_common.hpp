@@ -101,17 +101,34 @@ bool nxh_defer_active(nxh_context *ctx);
 int nxh_defer_flush(nxh_context *ctx);
 int nxh_defer_barrier(nxh_context *ctx, const nxh_tensor *out0 = nullptr, const nxh_tensor *out1 = nullptr,
                       const nxh_tensor *out2 = nullptr);
+int nxh_defer_touch(nxh_context *ctx, const nxh_tensor *const *tensors, int n, int n_out);
+int nxh_defer_quiet(nxh_context *ctx);
+int nxh_defer_host_read(nxh_context *ctx, const void *src);
 int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, const nxh_tensor *const *ins, int nin,
                      const int32_t *axes, int n_axes, const void *value);
 bool nxh_defer_free(nxh_context *ctx, void *p);
 int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes);
 void nxh_defer_context_gone(nxh_context *ctx);
 enum { NXH_D_UNARY, NXH_D_BINARY, NXH_D_COMPARE, NXH_D_WHERE, NXH_D_CAST, NXH_D_REDUCE, NXH_D_MATMUL, NXH_D_FULL };
-// Entry points that are not recorded run the record first.
+// Entry points that are not recorded run the record first. BARRIER also writes everything
+// that was postponed; TOUCH (the first n_out tensors are written, the others read; NULL entries
+// are skipped) only what those blocks need; QUIET nothing.
 #define NXH_DEFER_BARRIER(ctx, ...)                              \
   do {                                                           \
     if ((ctx) && nxh_defer_active(ctx))                          \
       if (int drc__ = nxh_defer_barrier(ctx, ##__VA_ARGS__)) return drc__; \
+  } while (0)
+#define NXH_DEFER_TOUCH(ctx, n_out, ...)                                                                      \
+  do {                                                                                                        \
+    if ((ctx) && nxh_defer_active(ctx)) {                                                                     \
+      const nxh_tensor *dts__[] = {__VA_ARGS__};                                                              \
+      if (int drc__ = nxh_defer_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out)) return drc__;  \
+    }                                                                                                         \
+  } while (0)
+#define NXH_DEFER_QUIET(ctx)                                     \
+  do {                                                           \
+    if ((ctx) && nxh_defer_active(ctx))                          \
+      if (int drc__ = nxh_defer_quiet(ctx)) return drc__;        \
   } while (0)
 // Recorded entry points: NXH_OK means recorded; -1 means run now.
 #define NXH_DEFER_RECORD(ctx, kind, op, out, nin, axes, n_axes, value, ...)                             \

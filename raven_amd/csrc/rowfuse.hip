@@ -398,7 +398,7 @@ void gelu_launch(nxh_context *ctx, const GeluArgs &a, bool vec) {
 
 NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *scale,
                                 const nxh_tensor *mask, const void *masked_value) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x, mask);
   const char *op = "softmax_rows";
   if (!ctx || !out || !x || (mask && !masked_value)) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -446,7 +446,7 @@ NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const n
 
 NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
                                    const nxh_tensor *gamma, const nxh_tensor *beta, double eps) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x, gamma, beta);
   const char *op = "layer_norm_rows";
   if (!ctx || !out || !x) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -495,7 +495,7 @@ NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, cons
 }
 
 NXH_EXPORT int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *constants) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_TOUCH(ctx, 1, out, x);
   const char *op = "gelu_tanh";
   if (!ctx || !out || !x || !constants) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);

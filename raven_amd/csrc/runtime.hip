@@ -245,7 +245,7 @@ NXH_EXPORT int nxh_free(nxh_context *ctx, void *dptr) {
 }
 
 NXH_EXPORT int nxh_trim(nxh_context *ctx) {
-  NXH_DEFER_BARRIER(ctx);
+  NXH_DEFER_QUIET(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "trim", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "trim")) return rc;
@@ -348,7 +348,8 @@ int nxh_settle_replay_faults(nxh_context *ctx, const char *op) {
 }
 
 NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
-  NXH_DEFER_BARRIER(ctx);
+  if (ctx && nxh_defer_active(ctx))
+    if (int drc = nxh_defer_host_read(ctx, src)) return drc;
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "to_host", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "to_host")) return rc;
@@ -360,7 +361,7 @@ NXH_EXPORT int nxh_memcpy_d2h(nxh_context *ctx, void *dst, const void *src, size
 }
 
 NXH_EXPORT int nxh_synchronize(nxh_context *ctx) {
-  NXH_DEFER_BARRIER(ctx);
+  NXH_DEFER_QUIET(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "synchronize", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "synchronize")) return rc;
@@ -412,7 +413,7 @@ NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
 }
 
 NXH_EXPORT int nxh_capture_end(nxh_context *ctx, nxh_graph **out) {
-  NXH_DEFER_BARRIER(ctx);
+  NXH_DEFER_QUIET(ctx);
   if (!ctx || !out) return nxh_fail(NXH_INVALID_ARGUMENT, "capture_end", "null argument");
   std::lock_guard<std::mutex> g(ctx->mu);
   *out = nullptr;
@@ -443,7 +444,7 @@ NXH_EXPORT int nxh_graph_launch(nxh_context *ctx, nxh_graph *gr) {
 }
 
 NXH_EXPORT int nxh_graph_destroy(nxh_context *ctx, nxh_graph *gr) {
-  NXH_DEFER_BARRIER(ctx);
+  NXH_DEFER_QUIET(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "graph_destroy", "null context");
   if (!gr) return NXH_OK;
   std::lock_guard<std::mutex> g(ctx->mu);
@@ -458,7 +459,7 @@ NXH_EXPORT int nxh_graph_destroy(nxh_context *ctx, nxh_graph *gr) {
 
 // ── timing ─────────────────────────────────────────────────────────────────
 NXH_EXPORT int nxh_timer_start(nxh_context *ctx) {
-  NXH_DEFER_BARRIER(ctx);
+  NXH_DEFER_QUIET(ctx);
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "timer", "null context");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "timer")) return rc;
@@ -466,7 +467,7 @@ NXH_EXPORT int nxh_timer_start(nxh_context *ctx) {
   return NXH_OK;
 }
 NXH_EXPORT int nxh_timer_stop(nxh_context *ctx, float *ms) {
-  NXH_DEFER_BARRIER(ctx);
+  NXH_DEFER_QUIET(ctx);
   if (!ctx || !ms) return nxh_fail(NXH_INVALID_ARGUMENT, "timer", "null argument");
   std::lock_guard<std::mutex> g(ctx->mu);
   if (int rc = refuse_while_capturing(ctx, "timer")) return rc;

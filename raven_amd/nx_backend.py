@@ -172,7 +172,7 @@ class Backend:
 
     # -- deferred evaluation: primitives are recorded and fused below the C ABI --
     DEFER_STATS = ("recorded", "issued", "flushes", "fallbacks", "softmax_rows", "layer_norm_rows", "gelu_tanh",
-                   "attention", "linear")
+                   "attention", "linear", "postponed", "materialised")
 
     def set_deferred(self, on: bool):
         """With the mode on, unary / binary / compare / where / cast / reduce / matmul and

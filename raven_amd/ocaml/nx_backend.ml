@@ -17,6 +17,7 @@ type dev (* device allocation; finalised through the allocator of its context *)
 external create_context : unit -> context = "caml_nx_hip_create_context"
 external dev_alloc : context -> int -> dev = "caml_nx_hip_alloc"
 external dev_bytes : dev -> int = "caml_nx_hip_bytes"
+external dtype_bytes : int -> int -> int = "caml_nx_hip_dtype_bytes" (* tag, count: the library's own count *)
 
 (* FIELD ORDER IS ABI (nx_hip_stubs.c reads slots 0-4). *)
 type ('a, 'b) t = {
@@ -406,3 +407,126 @@ let eig x =
   let w = eig_values x in
   let v = create_tensor x.context Dtype.Complex128 x.shape in
   reraise_linalg ~op:"eig" (fun () -> caml_eig w v x true); (w, v)
+
+(* ── beyond Backend_intf.S ────────────────────────────────────────────────────
+   Nothing below has a counterpart in the C backend. The frontend needs none of
+   it to reach the fused kernels: [set_deferred ctx true] makes the primitive
+   stubs above record their calls, and the library replaces the runs that spell
+   softmax (frontend.ml:4242-4252), layer norm (kaun/lib/layer_norm.ml:43-68),
+   GELU (fn.ml:31-38), the attention core (attention.ml:67-110) and linear +
+   residual (linear.ml:50-52) by one kernel each when the next host read,
+   [synchronize] or non-recordable operation executes the record. Intermediates
+   are dropped from the record when their buffers are finalised before that, so
+   a caller that wants the fusion to happen regardless of the collector's timing
+   calls the operation by name through [Fused]. *)
+
+external synchronize : context -> unit = "caml_nx_hip_synchronize"
+external trim : context -> unit = "caml_nx_hip_trim"
+external device_info : context -> int * string * int = "caml_nx_hip_device_info"
+external memory_stats : context -> int array = "caml_nx_hip_memory_stats"
+external last_path : context -> string = "caml_nx_hip_last_path"
+external timer_start : context -> unit = "caml_nx_hip_timer_start"
+external timer_stop : context -> float = "caml_nx_hip_timer_stop"
+external set_deferred : context -> bool -> unit = "caml_nx_hip_set_deferred"
+
+(* recorded, issued as recorded, flushes, fallbacks, then the runs replaced by
+   softmax_rows, layer_norm_rows, gelu_tanh, attention and linear *)
+external deferred_stats : context -> int array = "caml_nx_hip_deferred_stats"
+
+(* nx_effect.ml:376 returns its argument: the reference has one memory. Here a
+   tensor of another context of the same GPU is copied by the target context's
+   stream once the source stream has drained, and the target is drained before
+   the source may be released. *)
+let to_device ctx t =
+  if t.context == ctx then t
+  else begin
+    synchronize t.context;
+    let out = create_tensor ctx t.dtype t.shape in
+    caml_copy out t;
+    synchronize ctx;
+    out
+  end
+
+(* reduce for callers that may not allocate: the split partials live in a static
+   device array, the output is the caller's *)
+external caml_reduce_noalloc : int -> ('a, 'b) t -> ('a, 'b) t -> int array -> unit = "caml_nx_hip_reduce_noalloc"
+
+let reduce_into ~op ~axes ~out x =
+  let code = match op with `Sum -> 0 | `Prod -> 1 | `Max -> 2 | `Min -> 3 in
+  let axes = let a = Array.copy axes in Array.sort compare a; a in
+  caml_reduce_noalloc code out x axes
+
+module Fused = struct
+  external caml_softmax_rows :
+    ('c, 'd) t -> ('a, 'b) t -> ('a, 'b) Nx_buffer.t option -> (bool, Dtype.bool_elt) t option ->
+    ('a, 'b) Nx_buffer.t option -> unit = "caml_nx_hip_softmax_rows"
+  external caml_layer_norm_rows :
+    ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t option -> ('a, 'b) t option -> float -> unit = "caml_nx_hip_layer_norm_rows"
+  external caml_gelu_tanh : ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) Nx_buffer.t -> unit = "caml_nx_hip_gelu_tanh"
+  external caml_attention :
+    ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> (float, Dtype.float32_elt) Nx_buffer.t option ->
+    (bool, Dtype.bool_elt) t option -> (float, Dtype.float32_elt) Nx_buffer.t option -> bool -> unit
+    = "caml_nx_hip_attention_bc" "caml_nx_hip_attention"
+  external caml_linear :
+    ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t option -> ('a, 'b) t option -> unit = "caml_nx_hip_linear"
+
+  let host_scalar dtype v =
+    let b = Nx_buffer.create dtype 1 in
+    Nx_buffer.set b 0 v; b
+
+  (* softmax over the last axis of [x * scale], masked positions replaced by [fill] first *)
+  let softmax ?scale ?mask x =
+    let out = create_tensor x.context x.dtype x.shape in
+    let mask, fill = match mask with
+      | Some (m, fill) -> (Some (expand m x.shape), Some (host_scalar x.dtype fill))
+      | None -> (None, None) in
+    caml_softmax_rows out x (Option.map (host_scalar x.dtype) scale) mask fill; out
+
+  let layer_norm ?gamma ?beta ~eps x =
+    let out = create_tensor x.context x.dtype x.shape in
+    caml_layer_norm_rows out x gamma beta eps; out
+
+  let gelu_approx x =
+    let out = create_tensor x.context x.dtype x.shape in
+    let c = Nx_buffer.create x.dtype 4 in
+    List.iteri (Nx_buffer.set c) [ 0.044715; Float.sqrt (2. /. Float.pi); 1.0; 0.5 ];
+    caml_gelu_tanh out (contiguous x) c; out
+
+  (* attention.ml:67-110 for float16 / bfloat16 operands of [batch..., seq, head_dim] *)
+  let attention ?mask ?(causal = false) ~scale q k v =
+    let out = create_tensor q.context q.dtype q.shape in
+    let masked = if causal || mask <> None then Some (host_scalar Dtype.Float32 Float.neg_infinity) else None in
+    let mask = Option.map (fun m ->
+        let nd = Array.length q.shape in
+        let target = Array.copy q.shape in
+        target.(nd - 1) <- k.shape.(nd - 2);
+        expand m target) mask in
+    caml_attention out q k v (Some (host_scalar Dtype.Float32 scale)) mask masked causal; out
+
+  (* linear.ml:50-52 and the residual add of gpt2.ml:165-176 in the GEMM's epilogue *)
+  let linear ?bias ?residual x w =
+    let nd = Array.length x.shape in
+    let shape = Array.copy x.shape in
+    shape.(nd - 1) <- w.shape.(Array.length w.shape - 1);
+    let out = create_tensor x.context x.dtype shape in
+    caml_linear out x w bias residual; out
+end
+
+(* Recorded sequences: every operation between [capture_begin] and [capture_end]
+   is recorded instead of run; [Graph.launch] replays the whole sequence with
+   one call, reading the inputs' current contents and writing the same outputs.
+   Host reads, [synchronize], [trim] and the timer fail during a capture. *)
+module Graph = struct
+  type graph
+
+  external capture_begin : context -> unit = "caml_nx_hip_capture_begin"
+  external capture_end : context -> graph = "caml_nx_hip_capture_end"
+  external launch : graph -> unit = "caml_nx_hip_graph_launch"
+  external destroy : graph -> unit = "caml_nx_hip_graph_destroy"
+
+  let record ctx f =
+    capture_begin ctx;
+    match f () with
+    | result -> (capture_end ctx, result)
+    | exception e -> (try destroy (capture_end ctx) with _ -> ()); raise e
+end

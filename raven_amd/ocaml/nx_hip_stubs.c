@@ -15,6 +15,7 @@
 
 #include <dlfcn.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <caml/alloc.h>
@@ -34,7 +35,11 @@
   X(compare) X(where) X(cast) X(reduce) X(argreduce) X(matmul) X(copy)        \
   X(gather) X(scatter) X(pad) X(cat) X(scan) X(threefry) X(dtype_bytes)       \
   X(sort) X(argsort) X(unfold) X(fold) X(fft) X(rfft) X(irfft) X(cholesky)    \
-  X(triangular_solve) X(qr) X(eigh) X(svd) X(eig)
+  X(triangular_solve) X(qr) X(eigh) X(svd) X(eig) X(device_info)              \
+  X(memory_stats) X(trim) X(reduce_noalloc) X(softmax_rows) X(layer_norm_rows) \
+  X(gelu_tanh) X(attention) X(linear) X(set_deferred) X(deferred_stats)        \
+  X(capture_begin) X(capture_end) X(graph_launch) X(graph_destroy)             \
+  X(timer_start) X(timer_stop) X(last_path)
 static struct {
 #define X(n) __typeof__(nxh_##n) *n;
   NXH_SYMBOLS(X)
@@ -54,24 +59,59 @@ static void load_library(void) {
 #undef X
 }
 
-/* ── context and device buffers as custom blocks ─────────────────────────── */
-#define Ctx_val(v) (*(nxh_context **)Data_custom_val(v))
+/* ── context, device buffers and graphs as custom blocks ─────────────────────
+   The collector finalises blocks in no particular order, so the context is
+   counted: its own block, every buffer and every graph hold one reference, and
+   whichever is finalised last destroys it (a buffer finalised after the
+   context block still finds its allocator). */
 typedef struct {
   nxh_context *ctx;
+  long refs;
+} ctx_box;
+#define Box_val(v) (*(ctx_box **)Data_custom_val(v))
+#define Ctx_val(v) (Box_val(v)->ctx)
+typedef struct {
+  ctx_box *box;
   void *ptr;
   size_t bytes;
 } dev_block;
 #define Dev_val(v) ((dev_block *)Data_custom_val(v))
+typedef struct {
+  ctx_box *box;
+  nxh_graph *graph;
+} graph_block;
+#define Graph_val(v) ((graph_block *)Data_custom_val(v))
 
+static ctx_box *box_retain(ctx_box *b) {
+  __atomic_add_fetch(&b->refs, 1, __ATOMIC_RELAXED);
+  return b;
+}
+static void box_release(ctx_box *b) {
+  if (__atomic_sub_fetch(&b->refs, 1, __ATOMIC_ACQ_REL) == 0) {
+    L.context_destroy(b->ctx); /* waits for the stream, returns every block to the driver */
+    free(b);
+  }
+}
+static void ctx_finalize(value v) { box_release(Box_val(v)); }
 static void dev_finalize(value v) {
   dev_block *d = Dev_val(v);
-  if (d->ptr) L.free(d->ctx, d->ptr); /* stream-ordered inside the library */
+  if (d->ptr) L.free(d->box->ctx, d->ptr); /* stream-ordered inside the library */
   d->ptr = NULL;
+  box_release(d->box);
 }
-static struct custom_operations ctx_ops = {"nx_hip.context", custom_finalize_default,
+static void graph_finalize(value v) {
+  graph_block *g = Graph_val(v);
+  if (g->graph) L.graph_destroy(g->box->ctx, g->graph);
+  g->graph = NULL;
+  box_release(g->box);
+}
+static struct custom_operations ctx_ops = {"nx_hip.context", ctx_finalize,
     custom_compare_default, custom_hash_default, custom_serialize_default,
     custom_deserialize_default, custom_compare_ext_default, custom_fixed_length_default};
 static struct custom_operations dev_ops = {"nx_hip.buffer", dev_finalize,
+    custom_compare_default, custom_hash_default, custom_serialize_default,
+    custom_deserialize_default, custom_compare_ext_default, custom_fixed_length_default};
+static struct custom_operations graph_ops = {"nx_hip.graph", graph_finalize,
     custom_compare_default, custom_hash_default, custom_serialize_default,
     custom_deserialize_default, custom_compare_ext_default, custom_fixed_length_default};
 
@@ -90,8 +130,15 @@ CAMLprim value caml_nx_hip_create_context(value unit) {
   nxh_context *ctx = NULL;
   int rc = L.context_create(&ctx);
   if (rc != NXH_OK) caml_failwith(L.last_error(NULL));
-  v = caml_alloc_custom(&ctx_ops, sizeof(nxh_context *), 0, 1);
-  Ctx_val(v) = ctx;
+  ctx_box *box = (ctx_box *)malloc(sizeof *box);
+  if (!box) {
+    L.context_destroy(ctx);
+    caml_raise_out_of_memory();
+  }
+  box->ctx = ctx;
+  box->refs = 1;
+  v = caml_alloc_custom(&ctx_ops, sizeof(ctx_box *), 0, 1);
+  Box_val(v) = box;
   CAMLreturn(v);
 }
 
@@ -103,19 +150,24 @@ CAMLprim value caml_nx_hip_alloc(value vctx, value vbytes) {
   check(Ctx_val(vctx), L.alloc(Ctx_val(vctx), bytes, &p));
   /* caml_alloc_custom_mem lets the GC account for the device bytes */
   v = caml_alloc_custom_mem(&dev_ops, sizeof(dev_block), bytes);
-  Dev_val(v)->ctx = Ctx_val(vctx);
+  Dev_val(v)->box = box_retain(Box_val(vctx));
   Dev_val(v)->ptr = p;
   Dev_val(v)->bytes = bytes;
   CAMLreturn(v);
 }
 
+/* storage bytes of `count` elements of the dtype with this tag, as the library counts them */
+CAMLprim value caml_nx_hip_dtype_bytes(value vtag, value vcount) {
+  load_library();
+  return Val_long((long)L.dtype_bytes(Int_val(vtag), (int64_t)Long_val(vcount)));
+}
 CAMLprim value caml_nx_hip_bytes(value vdev) { return Val_long((long)Dev_val(vdev)->bytes); }
 
 /* from_host: the bigarray may be mutated or dropped as soon as this returns */
 CAMLprim value caml_nx_hip_from_host(value vdev, value vba) {
   CAMLparam2(vdev, vba);
   dev_block *d = Dev_val(vdev);
-  check(d->ctx, L.memcpy_h2d(d->ctx, d->ptr, Caml_ba_data_val(vba), d->bytes));
+  check(d->box->ctx, L.memcpy_h2d(d->box->ctx, d->ptr, Caml_ba_data_val(vba), d->bytes));
   CAMLreturn(Val_unit);
 }
 
@@ -125,7 +177,7 @@ CAMLprim value caml_nx_hip_to_host(value vba, value vdev) {
   CAMLparam2(vba, vdev);
   dev_block *d = Dev_val(vdev);
   void *dst = Caml_ba_data_val(vba);
-  nxh_context *ctx = d->ctx;
+  nxh_context *ctx = d->box->ctx;
   void *src = d->ptr;
   size_t n = d->bytes;
   caml_enter_blocking_section();
@@ -150,7 +202,7 @@ static nxh_context *extract(value v, nxh_tensor *t) {
     t->shape[i] = Long_val(Field(vs, i));
     t->strides[i] = Long_val(Field(vst, i));
   }
-  return d->ctx;
+  return d->box->ctx;
 }
 
 #define UNARY_STUB(name, OP)                                              \
@@ -518,5 +570,189 @@ CAMLprim value caml_nx_hip_eig(value vw, value vv, value vx, value vvectors) {
   extract(vx, &x);
   int vectors = Bool_val(vvectors);
   BLOCKING(L.eig(c, &w, vectors ? &v : NULL, &x));
+  CAMLreturn(Val_unit);
+}
+
+/* ── what the reference backend has no stub for ─────────────────────────────
+   Context services, the call that allocates nothing, the fused entry points,
+   deferred evaluation and recorded sequences. The frontend reaches the fused
+   kernels without any of the five fused stubs: with set_deferred on, the
+   primitive stubs above record, and the library replaces the runs it recognises.
+   The fused stubs are for callers that name the operation themselves. */
+
+CAMLprim value caml_nx_hip_synchronize(value vctx) {
+  CAMLparam1(vctx);
+  nxh_context *c = Ctx_val(vctx);
+  BLOCKING(L.synchronize(c));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_trim(value vctx) {
+  CAMLparam1(vctx);
+  nxh_context *c = Ctx_val(vctx);
+  BLOCKING(L.trim(c));
+  CAMLreturn(Val_unit);
+}
+/* (device ordinal, device name, compute units) */
+CAMLprim value caml_nx_hip_device_info(value vctx) {
+  CAMLparam1(vctx);
+  CAMLlocal2(v, vname);
+  int device = 0, units = 0;
+  char name[256];
+  check(Ctx_val(vctx), L.device_info(Ctx_val(vctx), &device, name, sizeof name, &units));
+  vname = caml_copy_string(name);
+  v = caml_alloc_tuple(3);
+  Store_field(v, 0, Val_int(device));
+  Store_field(v, 1, vname);
+  Store_field(v, 2, Val_int(units));
+  CAMLreturn(v);
+}
+/* [| in_use; cached; reserved; driver_allocs |] */
+CAMLprim value caml_nx_hip_memory_stats(value vctx) {
+  CAMLparam1(vctx);
+  CAMLlocal1(v);
+  uint64_t s[4] = {0, 0, 0, 0};
+  check(Ctx_val(vctx), L.memory_stats(Ctx_val(vctx), &s[0], &s[1], &s[2], &s[3]));
+  v = caml_alloc_tuple(4);
+  for (int i = 0; i < 4; i++) Store_field(v, i, Val_long((long)s[i]));
+  CAMLreturn(v);
+}
+CAMLprim value caml_nx_hip_last_path(value vctx) {
+  CAMLparam1(vctx);
+  const char *p = L.last_path(Ctx_val(vctx));
+  CAMLreturn(caml_copy_string(p ? p : ""));
+}
+CAMLprim value caml_nx_hip_timer_start(value vctx) {
+  CAMLparam1(vctx);
+  check(Ctx_val(vctx), L.timer_start(Ctx_val(vctx)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_timer_stop(value vctx) {
+  CAMLparam1(vctx);
+  nxh_context *c = Ctx_val(vctx);
+  float ms = 0.0f;
+  BLOCKING(L.timer_stop(c, &ms));
+  CAMLreturn(caml_copy_double((double)ms));
+}
+
+CAMLprim value caml_nx_hip_reduce_noalloc(value vop, value vout, value vx, value vaxes) {
+  CAMLparam4(vop, vout, vx, vaxes);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  int32_t axes[NXH_MAX_NDIM];
+  int n = axes_array(vaxes, axes);
+  check(c, L.reduce_noalloc(c, Int_val(vop), &o, &x, axes, n));
+  CAMLreturn(Val_unit);
+}
+
+/* an OCaml `'a t option` as a descriptor pointer or NULL; a `buffer option`
+   (a one-element host Nx_buffer holding an encoded scalar) as its bytes or NULL */
+static const nxh_tensor *optional(value v, nxh_tensor *slot) {
+  if (!Is_block(v)) return NULL;
+  extract(Field(v, 0), slot);
+  return slot;
+}
+static const void *optional_bytes(value v) { return Is_block(v) ? Caml_ba_data_val(Field(v, 0)) : NULL; }
+
+CAMLprim value caml_nx_hip_softmax_rows(value vout, value vx, value vscale, value vmask, value vfill) {
+  CAMLparam5(vout, vx, vscale, vmask, vfill);
+  nxh_tensor o, x, m;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.softmax_rows(c, &o, &x, optional_bytes(vscale), optional(vmask, &m), optional_bytes(vfill)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_layer_norm_rows(value vout, value vx, value vgamma, value vbeta, value veps) {
+  CAMLparam5(vout, vx, vgamma, vbeta, veps);
+  nxh_tensor o, x, g, b;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.layer_norm_rows(c, &o, &x, optional(vgamma, &g), optional(vbeta, &b), Double_val(veps)));
+  CAMLreturn(Val_unit);
+}
+/* constants: a four-element host Nx_buffer of x's dtype (c0..c3 of fn.ml:31-38) */
+CAMLprim value caml_nx_hip_gelu_tanh(value vout, value vx, value vconstants) {
+  CAMLparam3(vout, vx, vconstants);
+  nxh_tensor o, x;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  check(c, L.gelu_tanh(c, &o, &x, Caml_ba_data_val(vconstants)));
+  CAMLreturn(Val_unit);
+}
+/* scale, fill: one-element float32 host buffers */
+CAMLprim value caml_nx_hip_attention(value vout, value vq, value vk, value vv, value vscale, value vmask,
+                                     value vfill, value vcausal) {
+  CAMLparam5(vout, vq, vk, vv, vscale);
+  CAMLxparam3(vmask, vfill, vcausal);
+  nxh_tensor o, q, k, v, m;
+  nxh_context *c = extract(vout, &o);
+  extract(vq, &q);
+  extract(vk, &k);
+  extract(vv, &v);
+  check(c, L.attention(c, &o, &q, &k, &v, optional_bytes(vscale), optional(vmask, &m), optional_bytes(vfill),
+                       Bool_val(vcausal)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_attention_bc(value *argv, int argn) {
+  (void)argn;
+  return caml_nx_hip_attention(argv[0], argv[1], argv[2], argv[3], argv[4], argv[5], argv[6], argv[7]);
+}
+CAMLprim value caml_nx_hip_linear(value vout, value vx, value vw, value vbias, value vresidual) {
+  CAMLparam5(vout, vx, vw, vbias, vresidual);
+  nxh_tensor o, x, w, b, r;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  extract(vw, &w);
+  check(c, L.linear(c, &o, &x, &w, optional(vbias, &b), optional(vresidual, &r)));
+  CAMLreturn(Val_unit);
+}
+
+CAMLprim value caml_nx_hip_set_deferred(value vctx, value von) {
+  CAMLparam2(vctx, von);
+  check(Ctx_val(vctx), L.set_deferred(Ctx_val(vctx), Bool_val(von)));
+  CAMLreturn(Val_unit);
+}
+/* the counters of nxhip.h, in its order */
+CAMLprim value caml_nx_hip_deferred_stats(value vctx) {
+  CAMLparam1(vctx);
+  CAMLlocal1(v);
+  uint64_t s[NXH_DEFER_STAT_COUNT];
+  check(Ctx_val(vctx), L.deferred_stats(Ctx_val(vctx), s, NXH_DEFER_STAT_COUNT));
+  v = caml_alloc_tuple(NXH_DEFER_STAT_COUNT);
+  for (int i = 0; i < NXH_DEFER_STAT_COUNT; i++) Store_field(v, i, Val_long((long)s[i]));
+  CAMLreturn(v);
+}
+
+CAMLprim value caml_nx_hip_capture_begin(value vctx) {
+  CAMLparam1(vctx);
+  check(Ctx_val(vctx), L.capture_begin(Ctx_val(vctx)));
+  CAMLreturn(Val_unit);
+}
+CAMLprim value caml_nx_hip_capture_end(value vctx) {
+  CAMLparam1(vctx);
+  CAMLlocal1(v);
+  nxh_graph *g = NULL;
+  check(Ctx_val(vctx), L.capture_end(Ctx_val(vctx), &g));
+  v = caml_alloc_custom(&graph_ops, sizeof(graph_block), 0, 1);
+  Graph_val(v)->box = box_retain(Box_val(vctx));
+  Graph_val(v)->graph = g;
+  CAMLreturn(v);
+}
+CAMLprim value caml_nx_hip_graph_launch(value vgraph) {
+  CAMLparam1(vgraph);
+  graph_block *g = Graph_val(vgraph);
+  if (!g->graph) caml_invalid_argument("graph_launch: the graph was destroyed");
+  check(g->box->ctx, L.graph_launch(g->box->ctx, g->graph));
+  CAMLreturn(Val_unit);
+}
+/* releases the recorded launches and the storage they pinned now rather than at collection */
+CAMLprim value caml_nx_hip_graph_destroy(value vgraph) {
+  CAMLparam1(vgraph);
+  graph_block *g = Graph_val(vgraph);
+  if (g->graph) {
+    nxh_graph *graph = g->graph;
+    g->graph = NULL;
+    check(g->box->ctx, L.graph_destroy(g->box->ctx, graph));
+  }
   CAMLreturn(Val_unit);
 }

@@ -2,8 +2,9 @@
 three layers are cross-checked as text: every `external` of nx_backend.ml names
 a CAMLprim of nx_hip_stubs.c with the same number of arguments, every library
 call of the stubs matches its declaration in include/nxhip.h, the module defines
-every operation of Backend_intf.S (packages/nx/lib/core/backend_intf.ml), and
-the dlsym table covers what the stubs call."""
+every operation of Backend_intf.S (packages/nx/lib/core/backend_intf.ml), the
+dlsym table covers what the stubs call, and every export of the header is
+resolved by that table, called by a stub, and reachable from an `external`."""
 
 import re
 from pathlib import Path
@@ -108,7 +109,8 @@ def test_every_external_names_a_primitive_of_the_same_arity():
             assert len(targets) == 1
 
 
-def test_library_calls_of_the_stubs_match_the_header():
+def header_exports():
+    """name -> number of parameters, for every function nxhip.h declares."""
     h = strip_comments(HEADER, "/*", "*/")
     h = re.sub(r"//[^\n]*", "", h)
     declared = {}
@@ -116,8 +118,17 @@ def test_library_calls_of_the_stubs_match_the_header():
         before = h[:m.start()].rstrip()
         if re.search(r"(int|int64_t|void|\*)\s*$", before):
             declared[m.group(1)] = len(top_level_split(balanced(h, m.end() - 1), ","))
+    return declared
+
+
+def symbol_table(c):
+    return set(re.findall(r"X\((\w+)\)", c.split("#define NXH_SYMBOLS(X)")[1].split("static struct")[0]))
+
+
+def test_library_calls_of_the_stubs_match_the_header():
+    declared = header_exports()
     c = strip_comments(STUBS, "/*", "*/")
-    table = set(re.findall(r"X\((\w+)\)", c.split("#define NXH_SYMBOLS(X)")[1].split("static struct")[0]))
+    table = symbol_table(c)
     calls = list(re.finditer(r"\bL\.(\w+)\(", c))
     assert len(calls) >= 30
     for m in calls:
@@ -139,3 +150,35 @@ def test_the_module_defines_every_operation_of_the_backend_signature():
     assert not missing, f"nx_backend.ml lacks {missing}"
     for op in ("NXH_NEG", "NXH_ERF", "NXH_ADD", "NXH_AND", "NXH_CMPEQ", "NXH_CMPLE"):
         assert op in HEADER and op in STUBS
+
+
+def test_every_export_of_the_header_is_bound():
+    """No entry point of the library is out of the binding's reach: each one is resolved
+    at load time, called by at least one stub, and every stub is named by an `external`
+    (or is the bytecode twin of one)."""
+    declared = header_exports()
+    assert len(declared) >= 56
+    c = strip_comments(STUBS, "/*", "*/")
+    table = symbol_table(c)
+    unresolved = sorted(n for n in declared if n[4:] not in table)
+    assert not unresolved, f"nx_hip_stubs.c does not resolve {unresolved}"
+    called = set(re.findall(r"\bL\.(\w+)\(", c))
+    idle = sorted(n for n in table if n not in called)
+    assert not idle, f"resolved but never called: {idle}"
+    ml = strip_comments(ML, "(*", "*)")
+    named = set(re.findall(r"\"(caml_nx_hip_\w+)\"", ml))
+    orphans = sorted(p for p in c_primitives() if p not in named)
+    assert not orphans, f"CAMLprims that no external names: {orphans}"
+
+
+def test_the_context_is_destroyed_by_its_last_holder():
+    """The context block, every buffer and every graph hold one reference each; the
+    finaliser that drops the last one calls nxh_context_destroy."""
+    c = strip_comments(STUBS, "/*", "*/")
+    assert "custom_finalize_default" not in c
+    release = c.split("static void box_release")[1].split("}\n}")[0]
+    assert "L.context_destroy" in release
+    for fin in ("ctx_finalize", "dev_finalize", "graph_finalize"):
+        body = c.split(f"static void {fin}(value v)")[1].split("\n}")[0]
+        assert "box_release" in body, fin
+    assert c.count("box_retain(Box_val(vctx))") == 2  # buffers and graphs
