@@ -528,6 +528,28 @@ class Gpt2Workload:
         self.ids = np.random.default_rng(17).integers(0, self.cfg.vocab_size, (self.batch, self.seq)).astype(np.int32)
 
 
+def compiled_host_config5(iters=3):
+    """Config 5 issued by the compiled host (raven_amd/host_c/kaun_gpt2_host.c): the same call sequence
+    through the C ABI with no interpreter between the calls, in a process of its own. Wall time per
+    forward, eagerly and with the library's deferred mode (no graph), and the replayed graph's GPU time."""
+    import subprocess
+
+    from raven_amd import _ffi, build
+
+    if not build.GPT2_HOST_BIN.exists():
+        return {"cfg5_c_host": "not built"}
+    r = subprocess.run([str(build.GPT2_HOST_BIN), str(_ffi.LIB_PATH), "--iters", str(iters)], capture_output=True, text=True,
+                       timeout=300)
+    if r.returncode != 0:
+        return {"cfg5_c_host": ("failed: " + r.stderr.strip())[:100]}
+    t = json.loads(r.stdout.strip().splitlines()[-1])
+    tokens = t["batch"] * t["seq"]
+    return {"cfg5_c_host_eager_ms": t["eager_wall_ms"], "cfg5_c_host_deferred_ms": t["deferred_wall_ms"],
+            "cfg5_c_host_deferred_late_free_ms": t["late_free_wall_ms"], "cfg5_c_host_replay_gpu_ms": t["replay_gpu_ms"],
+            "cfg5_c_host_deferred_tokens_per_s": round(tokens / (t["deferred_wall_ms"] * 1e-3), 1),
+            "cfg5_c_host_deferred_wall_over_replay_gpu": t["deferred_wall_over_replay_gpu"]}
+
+
 def config5(hip, work, iters=3, warmup=1, window=False, graph=False, keep_positions=64):
     """GPT-2-small-shaped forward (12 layers, d 768, 12 heads, FFN 3072, vocab
     50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s. Eager: one
@@ -879,6 +901,7 @@ def main():
             parity[5], cpu_figs = check_config5(work, heads)
             flat.update(cpu_figs)
         del work, heads
+        flat.update(compiled_host_config5())
         ops_out.extend(next_ops(hip, W))
 
     config = {"workload": "config 2: [64,512,512] f32 add(permuted, broadcast) / mul scalar / cast f16 + int32 add / mul / "

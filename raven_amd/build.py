@@ -79,5 +79,19 @@ def build_abi_check() -> Path:
     return ABI_CHECK_BIN
 
 
+GPT2_HOST_SRC = CSRC.parent / "host_c" / "kaun_gpt2_host.c"
+GPT2_HOST_BIN = GPT2_HOST_SRC.with_suffix("")
+
+
+def build_gpt2_host() -> Path:
+    """The compiled host of Kaun's GPT-2 forward over the C ABI (raven_amd/host_c): gcc only."""
+    cmd = ["gcc", "-std=gnu11", "-O2", "-Wall", "-Wextra", "-I", str(CSRC.parent.parent / "include"),
+           "-o", str(GPT2_HOST_BIN), str(GPT2_HOST_SRC), "-ldl", "-lm"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0 or r.stderr.strip():
+        raise RuntimeError(f"gcc failed on {GPT2_HOST_SRC.name}:\n{r.stderr}")
+    return GPT2_HOST_BIN
+
+
 if __name__ == "__main__":
     print(build_all(force="--force" in sys.argv))
