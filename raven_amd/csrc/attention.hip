@@ -80,7 +80,7 @@ __device__ __forceinline__ float xor32(float v) {
   return __builtin_bit_cast(float, __shfl_xor(__builtin_bit_cast(int, v), 32, 64));
 }
 
-template <class EL, int DHEAD>
+template <class EL, int DHEAD, bool ONLINE>
 __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
   using S = uint16_t;
   using MX = Combine<NXH_RMAX, float, CAT_FLOAT>;
@@ -183,10 +183,10 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
       if (pass == 1) vpre[i] = *reinterpret_cast<const V16 *>(V + (int64_t)key * a.v.row + c);
     }
   };
-  prefetch(0, 0);
-  for (int pass = 0; pass < 2; pass++) {
+  prefetch(ONLINE ? 1 : 0, 0);
+  for (int pass = ONLINE ? 1 : 0; pass < 2; pass++) {
     float l_total = 0.0f, l_recip = 0.0f;
-    if (pass == 1) {
+    if (!ONLINE && pass == 1) {
       l_total = l_run + xor32(l_run);
       l_recip = 1.0f / l_total;
     }
@@ -234,11 +234,42 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
         } else {
           // rounded probabilities, two per register, in accumulator order
           uint32_t pk[8];
+          if constexpr (ONLINE) {
+            // One walk over the keys: the exponentials are taken against the maximum seen so
+            // far, rounded, and multiplied into the output at once; when a later tile raises
+            // the maximum, what has been accumulated (output and row sum, all of it this
+            // lane's own query) is scaled down by e^(old - new). The division by the row sum
+            // is left for the end.
+            float tm = t[0];
 #pragma unroll
-          for (int e = 0; e < 16; e += 2) {
-            const float p0 = div_by_reciprocal(exp_nonpositive(t[e] - m_run), l_total, l_recip);
-            const float p1 = div_by_reciprocal(exp_nonpositive(t[e + 1] - m_run), l_total, l_recip);
-            pk[e >> 1] = narrow2<EL>(p0, p1);
+            for (int e = 1; e < 16; e++) tm = __builtin_fmaxf(tm, t[e]);
+            float m_new = __builtin_fmaxf(m_run, tm);
+            m_new = __builtin_fmaxf(m_new, xor32(m_new));
+            // nothing visible yet: exponentials of -inf against 0 are 0, not NaN
+            const float m_ref = m_new == -__builtin_inff() ? 0.0f : m_new;
+            const float alpha = exp_nonpositive(m_run - m_ref);
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+              const float p0 = exp_nonpositive(t[e] - m_ref), p1 = exp_nonpositive(t[e + 1] - m_ref);
+              sum = sum + p0 + p1;
+              pk[e >> 1] = narrow2<EL>(p0, p1);
+            }
+            l_run = __builtin_fmaf(l_run, alpha, sum);
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+              for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) oacc[ot][e] = oacc[ot][e] * alpha;
+            }
+            m_run = m_new;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+              const float p0 = div_by_reciprocal(exp_nonpositive(t[e] - m_run), l_total, l_recip);
+              const float p1 = div_by_reciprocal(exp_nonpositive(t[e + 1] - m_run), l_total, l_recip);
+              pk[e >> 1] = narrow2<EL>(p0, p1);
+            }
           }
           // B operand of O^T = V^T P^T for k-step ks: this lane's query, keys
           // ks*16 + g*8 + 0..7. The accumulator gave keys ks*16 + g*4 + 0..3 and
@@ -267,6 +298,13 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
       }
     }
   }
+  if constexpr (ONLINE) {
+    const float l_total = l_run + xor32(l_run);
+#pragma unroll
+    for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) oacc[ot][e] = oacc[ot][e] / l_total;
+  }
   // O^T element e of tile ot: d = ot*32 + (e/4)*8 + g*4 + e%4, query qi
   if (qi < a.sq) {
     S *orow = O + (int64_t)qi * a.out.row;
@@ -283,15 +321,22 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
   }
 }
 
-template <class EL>
+// NXH_ATTENTION=twopass selects the form that rounds each probability after the division by
+// the full row sum, as the primitive sequence does; the default walks the keys once.
+bool two_pass_wanted() {
+  const char *e = getenv("NXH_ATTENTION");  // read per call: a test switches it inside one process
+  return e && strcmp(e, "twopass") == 0;
+}
+
+template <class EL, bool ONLINE>
 int attention_launch(nxh_context *ctx, const char *op, const AttArgs &a, int hd) {
   const int64_t blocks = a.batches * a.qtiles;
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
   const dim3 grid((unsigned)blocks), block(128);
   switch (hd) {
-    case 32: hipLaunchKernelGGL((attention_kernel<EL, 32>), grid, block, 0, ctx->stream, a); break;
-    case 64: hipLaunchKernelGGL((attention_kernel<EL, 64>), grid, block, 0, ctx->stream, a); break;
-    case 128: hipLaunchKernelGGL((attention_kernel<EL, 128>), grid, block, 0, ctx->stream, a); break;
+    case 32: hipLaunchKernelGGL((attention_kernel<EL, 32, ONLINE>), grid, block, 0, ctx->stream, a); break;
+    case 64: hipLaunchKernelGGL((attention_kernel<EL, 64, ONLINE>), grid, block, 0, ctx->stream, a); break;
+    case 128: hipLaunchKernelGGL((attention_kernel<EL, 128, ONLINE>), grid, block, 0, ctx->stream, a); break;
     default: return nxh_fail(NXH_FAILURE, op, "head dimension must be 32, 64 or 128");
   }
   return NXH_OK;
@@ -379,8 +424,12 @@ NXH_EXPORT int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path("attention_fused");
-  rc = dt == NXH_BF16 ? attention_launch<gemm_tile::ElBF16>(ctx, op, a, (int)hd)
-                      : attention_launch<gemm_tile::ElF16>(ctx, op, a, (int)hd);
+  if (two_pass_wanted())
+    rc = dt == NXH_BF16 ? attention_launch<gemm_tile::ElBF16, false>(ctx, op, a, (int)hd)
+                        : attention_launch<gemm_tile::ElF16, false>(ctx, op, a, (int)hd);
+  else
+    rc = dt == NXH_BF16 ? attention_launch<gemm_tile::ElBF16, true>(ctx, op, a, (int)hd)
+                        : attention_launch<gemm_tile::ElF16, true>(ctx, op, a, (int)hd);
   if (rc) return rc;
   NXH_HIP(op, hipGetLastError());
   return NXH_OK;

@@ -16,6 +16,7 @@
    Usage:
      kaun_gpt2_host LIB [--vocab V --positions P --embd D --layers L --heads H --inner I]
                         [--batch B --seq S] [--dtype bf16|f32] [--iters N]
+                        [--time eager,deferred,late,replay]
                         [--params FILE --ids FILE --logits FILE --mode eager|deferred|late]
    Without --params the weights are seeded noise of standard deviation 0.02 generated here;
    with it, FILE holds every leaf's storage bytes in the order of `leaves` below, --ids the
@@ -335,7 +336,7 @@ int main(int argc, char **argv) {
     fprintf(stderr, "usage: %s libnxhip.so [options]\n", argv[0]);
     return 2;
   }
-  const char *params_path = NULL, *ids_path = NULL, *logits_path = NULL, *mode = "deferred";
+  const char *params_path = NULL, *ids_path = NULL, *logits_path = NULL, *mode = "deferred", *which = "eager,deferred,late,replay";
   int iters = 5;
   for (int i = 2; i + 1 < argc; i += 2) {
     const char *k = argv[i], *v = argv[i + 1];
@@ -353,6 +354,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(k, "--ids")) ids_path = v;
     else if (!strcmp(k, "--logits")) logits_path = v;
     else if (!strcmp(k, "--mode")) mode = v;
+    else if (!strcmp(k, "--time")) which = v;
     else {
       fprintf(stderr, "unknown option %s\n", k);
       return 2;
@@ -424,10 +426,11 @@ int main(int argc, char **argv) {
     return 0;
   }
 
-  const timing eager = time_forwards(&p, ids.t, 0, 0, iters);
-  const timing deferred = time_forwards(&p, ids.t, 1, 0, iters);
-  const timing late = time_forwards(&p, ids.t, 1, 1, iters);
-  const timing replay = time_replays(&p, ids.t, iters);
+  const timing none = {0, 0};
+  const timing eager = strstr(which, "eager") ? time_forwards(&p, ids.t, 0, 0, iters) : none;
+  const timing deferred = strstr(which, "deferred") ? time_forwards(&p, ids.t, 1, 0, iters) : none;
+  const timing late = strstr(which, "late") ? time_forwards(&p, ids.t, 1, 1, iters) : none;
+  const timing replay = strstr(which, "replay") ? time_replays(&p, ids.t, iters) : none;
   const double tokens = (double)(cfg.batch * cfg.seq);
   printf("{\"host\": \"c\", \"dtype\": \"%s\", \"batch\": %lld, \"seq\": %lld, \"layers\": %lld, \"embd\": %lld, \"iters\": %d, "
          "\"eager_wall_ms\": %.3f, \"eager_gpu_ms\": %.3f, \"deferred_wall_ms\": %.3f, \"deferred_gpu_ms\": %.3f, "
@@ -435,7 +438,8 @@ int main(int argc, char **argv) {
          "\"deferred_wall_over_replay_gpu\": %.3f, \"deferred_tokens_per_s\": %.0f}\n",
          cfg.dtype == NXH_F32 ? "f32" : "bf16", (long long)cfg.batch, (long long)cfg.seq, (long long)cfg.layers,
          (long long)cfg.embd, iters, eager.wall_ms, eager.gpu_ms, deferred.wall_ms, deferred.gpu_ms, late.wall_ms, late.gpu_ms,
-         replay.wall_ms, replay.gpu_ms, deferred.wall_ms / replay.gpu_ms, tokens / (deferred.wall_ms * 1e-3));
+         replay.wall_ms, replay.gpu_ms, replay.gpu_ms > 0 ? deferred.wall_ms / replay.gpu_ms : 0.0,
+         deferred.wall_ms > 0 ? tokens / (deferred.wall_ms * 1e-3) : 0.0);
   L.context_destroy(ctx);
   return 0;
 }

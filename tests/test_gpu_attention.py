@@ -1,8 +1,17 @@
 """The fused attention kernel through the C ABI against the sequence it stands
 for (kaun/lib/attention.ml:67-110: cast to float32, Q K^T, scale, mask, softmax,
 cast back, probs x V), run primitive by primitive on the CPU oracle and on the
-GPU backend. The rounding points are the same; only the order of the float32
-sums differs, so the results agree to about one unit of the 16-bit output."""
+GPU backend, in both of its forms. The two-pass form (NXH_ATTENTION=twopass) has
+the sequence's rounding points, only the order of the float32 sums differs, and
+agrees with it to about one unit of the 16-bit output. The one-pass form (the
+default) rounds each exponential BEFORE the division by the row sum instead of
+the quotient after it: the same relative error per probability (2^-9 for
+bfloat16, 2^-12 for float16), made at another point, so it is held to the
+reference's own tolerance for arithmetic in these dtypes against the oracle
+(bf16 3e-2, f16 5e-3: backend_contract.ml:171-188) and to a few units of the
+output against the GPU sequence."""
+
+import os
 
 import math
 
@@ -18,6 +27,25 @@ pytestmark = pytest.mark.gpu
 ULP = {"float16": 2.0 ** -10, "bfloat16": 2.0 ** -7}
 
 
+@pytest.fixture(params=["onepass", "twopass"], autouse=True)
+def form(request):
+    """Both forms of the kernel run every test of this file."""
+    old = os.environ.get("NXH_ATTENTION")
+    os.environ["NXH_ATTENTION"] = request.param
+    yield request.param
+    if old is None:
+        del os.environ["NXH_ATTENTION"]
+    else:
+        os.environ["NXH_ATTENTION"] = old
+
+
+def near_the_gpu_sequence(form, got, want_gpu, d, oracle, what):
+    if form == "twopass":
+        close(got, want_gpu, d, oracle, 2 * ULP[d.name], 2e-3, what + " vs GPU sequence")
+    else:
+        close(got, want_gpu, d, oracle, 4 * ULP[d.name], 4 * ULP[d.name], what + " vs GPU sequence")
+
+
 def sequence(B, q, k, v, mask):
     return Gpt2(Nx(B), Config()).scaled_dot_product_attention(q, k, v, mask)
 
@@ -30,7 +58,7 @@ def bool_mask(B, m, shape):
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
 @pytest.mark.parametrize("shape", [(2, 3, 100, 64), (1, 2, 256, 64), (2, 2, 130, 32), (1, 1, 64, 128), (3, 40, 64)],
                          ids=lambda s: "x".join(map(str, s)))
-def test_attention_matches_the_sequence(hip, oracle, d, shape):
+def test_attention_matches_the_sequence(hip, oracle, d, shape, form):
     rng = np.random.default_rng(sum(shape) + d.tag)
     s, hd = shape[-2], shape[-1]
     q, k, v = (encode(rng.standard_normal(shape), d, oracle) for _ in range(3))
@@ -51,10 +79,10 @@ def test_attention_matches_the_sequence(hip, oracle, d, shape):
         want_gpu = logical(sequence(hip, hq, hk, hv, hm))
         want_cpu = logical(sequence(oracle, oq, ok, ov, om))
         what = f"{d.name} {shape} {name}"
-        close(got, want_gpu, d, oracle, 2 * ULP[d.name], 2e-3, what + " vs GPU sequence")
+        near_the_gpu_sequence(form, got, want_gpu, d, oracle, what)
         close(got, want_cpu, d, oracle, TOL[d.name][0], TOL[d.name][0], what + " vs oracle sequence")
         same = np.mean(got == want_gpu)
-        assert same > 0.9, (what, same)
+        assert same > (0.9 if form == "twopass" else 0.4), (what, same)
     # causality: the output at position i does not see keys behind it
     k2, v2 = k.copy(), v.copy()
     k2[..., s // 2:, :] = encode(rng.standard_normal(k2[..., s // 2:, :].shape), d, oracle)
@@ -97,7 +125,7 @@ def test_attention_on_head_split_views_and_special_rows(hip, oracle):
 
 
 @pytest.mark.parametrize("sq,sk,hd", [(70, 200, 64), (1, 333, 32), (129, 31, 128)])
-def test_more_or_fewer_keys_than_queries(hip, oracle, sq, sk, hd):
+def test_more_or_fewer_keys_than_queries(hip, oracle, sq, sk, hd, form):
     """Cross attention: the key count differs from the query count (no causal form there)."""
     rng = np.random.default_rng(sq + sk)
     d = dt.float16
@@ -114,7 +142,7 @@ def test_more_or_fewer_keys_than_queries(hip, oracle, sq, sk, hd):
         want = logical(sequence(oracle, oq, ok, ov, o_mask))
         close(got, want, d, oracle, TOL[d.name][0], TOL[d.name][0], f"{sq}x{sk}x{hd} {name}")
         want_gpu = logical(sequence(hip, hq, hk, hv, hm if o_mask is not None else None))
-        close(got, want_gpu, d, oracle, 2 * ULP[d.name], 2e-3, f"{sq}x{sk}x{hd} {name} vs GPU sequence")
+        near_the_gpu_sequence(form, got, want_gpu, d, oracle, f"{sq}x{sk}x{hd} {name}")
 
 
 def test_nan_scores_poison_exactly_the_rows_the_sequence_poisons(hip, oracle):

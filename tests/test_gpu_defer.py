@@ -257,7 +257,8 @@ def test_attention_core_fuses(hip, oracle, kind):
                                    mask=None if kind != "mask" else hip.expand(hip.reshape(mask_of(), (1, 1, s, s)), (b, h, s, s)),
                                    masked_value=None if kind == "none" else float("-inf"), causal=kind == "causal"))
     same_bits(got, direct, "the recorded run against nxh_attention")
-    close(got, eager, d, oracle, 2 * 2.0 ** -7, 2e-3, "against the eager sequence")
+    # the one-pass kernel rounds the exponentials, the sequence the quotients: a few units of bfloat16 apart
+    close(got, eager, d, oracle, 2 * 2.0 ** -7, 8e-3, "against the eager sequence")
 
 
 def test_errors_of_recorded_primitives_surface_when_the_record_runs(hip):
