@@ -324,6 +324,17 @@ int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *q,
 int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
                const nxh_tensor *w, const nxh_tensor *bias, const nxh_tensor *residual);
 
+/* nxh_linear without a residual followed by nxh_gelu_tanh (the first half of the MLP of
+   kaun/examples/04-gpt2/gpt2.ml:165-176: Fn.gelu_approx (Linear.apply fc x)), the GELU
+   applied in the GEMM's epilogue:
+     out = gelu_tanh (matmul x w + bias)
+   with every rounding of the eleven primitives it stands for, so the value equals the
+   two calls' bit for bit. bfloat16 / float16 operands whose product is made of whole
+   128 x 128 tiles with 16-byte aligned rows; anything else is Failure and the caller
+   issues the two calls. `constants` as for nxh_gelu_tanh. */
+int nxh_linear_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
+                         const nxh_tensor *w, const nxh_tensor *bias, const void *constants);
+
 /* ── Fourier transforms ──────────────────────────────────────────────────── */
 
 /* fft / ifft (backend_intf.ml:594-598; nx_backend.ml:507-528; nx_c_fft.c:940-956,
@@ -425,6 +436,8 @@ enum {
   NXH_DEFER_LINEAR,         /* ... nxh_linear */
   NXH_DEFER_POSTPONED,      /* entries of fused runs left unexecuted because their result was still held */
   NXH_DEFER_MATERIALISED,   /* of those, issued later because something read the result */
+  NXH_DEFER_LINEAR_GELU,    /* runs replaced by nxh_linear_gelu_tanh (counted here only) */
+  NXH_DEFER_GROUPED,        /* of the nxh_linear runs, those launched together with others that read the same x */
   NXH_DEFER_STAT_COUNT
 };
 int nxh_deferred_stats(nxh_context *ctx, uint64_t *stats, int count);

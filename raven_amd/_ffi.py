@@ -108,6 +108,7 @@ SIGNATURES = {
     "nxh_layer_norm_rows": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_double]),
     "nxh_gelu_tanh": (C.c_int, [_CTX, _T, _T, C.c_void_p]),
     "nxh_linear": (C.c_int, [_CTX, _T, _T, _T, _T, _T]),
+    "nxh_linear_gelu_tanh": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_void_p]),
     "nxh_attention": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_void_p, _T, C.c_void_p, C.c_int]),
     "nxh_set_deferred": (C.c_int, [_CTX, C.c_int]),
     "nxh_deferred_stats": (C.c_int, [_CTX, _P(C.c_uint64), C.c_int]),

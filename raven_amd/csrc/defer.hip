@@ -233,6 +233,7 @@ struct Plan {
   int stat = 0;
   std::vector<DEntry *> interior;
   bool causal_flag = false;
+  DEntry *linear_out = nullptr;  // LINEAR_GELU: the bias add whose result the GELU read
   // operands of the fused call
   Opnd x, a, b, c;
   unsigned char s0[16] = {}, s1[16] = {}, consts[64] = {};
@@ -548,6 +549,25 @@ bool match_gelu(Window *w, DEntry *anchor, Plan *p) {
   p->stat = NXH_DEFER_GELU;
   p->interior = interior;
   p->x = x;
+  // gelu (matmul x w + bias), the first half of the MLP (gpt2.ml:165-176): one GEMM whose
+  // epilogue applies the GELU, when nothing else reads the linear layer's result
+  if (is_island(d) && x.t->offset == 0) {
+    DEntry *add = producer_of(x, D_BINARY, NXH_ADD);
+    DEntry *mm = add ? producer_of(in_of(add, 0), D_MATMUL) : nullptr;
+    if (mm && !add->prod[1] && add->out.ndim >= 2 && vector_broadcast(add->in[1], add->out) && same_shape(mm->out, add->out)) {
+      std::vector<DEntry *> with = interior;
+      with.push_back(add);
+      with.push_back(mm);
+      if (hidden(with, anchor)) {
+        p->stat = NXH_DEFER_LINEAR_GELU;
+        p->interior = with;
+        p->linear_out = add;
+        p->x = in_of(mm, 0);
+        p->a = in_of(mm, 1);
+        p->b = in_of(add, 1);
+      }
+    }
+  }
   return true;
 }
 
@@ -619,6 +639,15 @@ int run_plan(nxh_context *ctx, DEntry *anchor, const Plan &p) {
     case NXH_DEFER_LAYER_NORM: {
       nxh_tensor gamma = vector_of(*p.a.t), beta = vector_of(*p.b.t);
       return nxh_layer_norm_rows(ctx, &anchor->out, p.x.t, &gamma, &beta, p.eps);
+    }
+    case NXH_DEFER_LINEAR_GELU: {
+      nxh_tensor bias = vector_of(*p.b.t);
+      const int rc = nxh_linear_gelu_tanh(ctx, &anchor->out, p.x.t, p.a.t, &bias, p.consts);
+      if (rc != NXH_FAILURE) return rc;
+      // the epilogue does not take this shape: the fused linear into the block the bias add
+      // was given (held back while the record uses it), then the GELU from there
+      if (const int r2 = nxh_linear(ctx, &p.linear_out->out, p.x.t, p.a.t, &bias, nullptr)) return r2;
+      return nxh_gelu_tanh(ctx, &anchor->out, &p.linear_out->out, p.consts);
     }
     default: return nxh_gelu_tanh(ctx, &anchor->out, p.x.t, p.consts);
   }
@@ -763,9 +792,75 @@ int flush_locked(nxh_context *ctx, Window *w) {
     std::sort(run.begin(), run.end(), [](DEntry *a, DEntry *b) { return a->id < b->id; });
     return run;
   };
+  // Linear layers (bias, no residual) that read one x through equal views, with weights, biases
+  // and outputs of one shape and layout, run as ONE launch at the place of the last of them:
+  // the q / k / v projections of attention.ml:218-265. Nothing recorded before that place
+  // may read an earlier member's result.
+  std::unordered_map<DEntry *, std::vector<DEntry *>> group_at;  // last member -> all members, in order
+  std::unordered_map<DEntry *, DEntry *> grouped;                 // member -> last member
+  {
+    auto same_layout = [](const nxh_tensor &a, const nxh_tensor &b) {
+      if (a.dtype != b.dtype || a.offset != b.offset || !same_shape(a, b)) return false;
+      for (int i = 0; i < a.ndim; i++)
+        if (a.shape[i] != 1 && a.strides[i] != b.strides[i]) return false;
+      return true;
+    };
+    std::vector<std::vector<DEntry *>> open;
+    for (auto &up : entries) {
+      DEntry *e = up.get();
+      auto it = plans.find(e);
+      if (it == plans.end() || it->second.stat != NXH_DEFER_LINEAR || !it->second.b || it->second.c) continue;
+      const Plan &pe = it->second;
+      bool placed = false;
+      for (auto &g : open) {
+        const Plan &p0 = plans.at(g.front());
+        if (g.size() >= 3 || !same_operand(pe.x, p0.x) || !same_layout(*pe.a.t, *p0.a.t) || !same_layout(*pe.b.t, *p0.b.t) ||
+            !same_layout(e->out, g.front()->out))
+          continue;
+        bool safe = true;
+        for (DEntry *m : g) {
+          for (DEntry *r : m->readers) safe = safe && r->id > e->id;
+          // a member whose own run holds entries of another run's operands stays alone
+          for (DEntry *inner : plans.at(m).interior)
+            for (DEntry *r : inner->readers) safe = safe && (r->fused_into == m || r == m);
+        }
+        if (!safe) continue;
+        g.push_back(e);
+        placed = true;
+        break;
+      }
+      if (!placed) open.push_back({e});
+    }
+    for (auto &g : open)
+      if (g.size() >= 2) {
+        for (DEntry *m : g) grouped[m] = g.back();
+        group_at[g.back()] = g;
+      }
+  }
   std::vector<DEntry *> fused;  // anchors whose fused call ran
   int rc = NXH_OK;
   tls_in_flush = true;
+  // One fused run at its anchor: the fused call, or (declined) the run as recorded.
+  auto run_anchor = [&](DEntry *e) {
+    Plan &pl = plans.at(e);
+    e->done = true;
+    rc = run_plan(ctx, e, pl);
+    if (rc == NXH_FAILURE) {
+      // the fused form was declined: the run as recorded, in its own order
+      w->stats[NXH_DEFER_FALLBACKS]++;
+      rc = NXH_OK;
+      for (DEntry *inner : members_of(e)) {
+        inner->fused_into = nullptr;
+        home.erase(inner);
+        if (!rc) rc = issue(ctx, inner), w->stats[NXH_DEFER_ISSUED]++;
+      }
+      e->done = false;
+      if (!rc) rc = issue(ctx, e), w->stats[NXH_DEFER_ISSUED]++;
+    } else if (!rc) {
+      w->stats[pl.stat]++;
+      fused.push_back(e);
+    }
+  };
   for (auto &up : entries) {
     DEntry *e = up.get();
     if (rc) break;
@@ -793,22 +888,35 @@ int flush_locked(nxh_context *ctx, Window *w) {
       w->stats[NXH_DEFER_ISSUED]++;
       continue;
     }
-    e->done = true;
-    rc = run_plan(ctx, e, it->second);
-    if (rc == NXH_FAILURE) {
-      // the fused form was declined: the run as recorded, in its own order
-      w->stats[NXH_DEFER_FALLBACKS]++;
-      rc = NXH_OK;
-      for (DEntry *inner : members_of(e)) {
-        inner->fused_into = nullptr;
-        home.erase(inner);
-        if (!rc) rc = issue(ctx, inner), w->stats[NXH_DEFER_ISSUED]++;
+    auto gr = grouped.find(e);
+    if (gr == grouped.end()) {
+      run_anchor(e);
+      continue;
+    }
+    if (gr->second != e) continue;  // runs with the last member of its group
+    const std::vector<DEntry *> &members = group_at.at(e);
+    const nxh_tensor *outs[3], *ws[3], *biases[3];
+    nxh_tensor bias_v[3];
+    for (size_t i = 0; i < members.size(); i++) {
+      const Plan &pm = plans.at(members[i]);
+      outs[i] = &members[i]->out;
+      ws[i] = pm.a.t;
+      bias_v[i] = vector_of(*pm.b.t);
+      biases[i] = &bias_v[i];
+    }
+    const int grc = nxh_linear_group(ctx, (int)members.size(), outs, plans.at(members[0]).x.t, ws, biases);
+    if (grc == NXH_OK) {
+      for (DEntry *m : members) {
+        m->done = true;
+        w->stats[NXH_DEFER_LINEAR]++;
+        fused.push_back(m);
       }
-      e->done = false;
-      if (!rc) rc = issue(ctx, e), w->stats[NXH_DEFER_ISSUED]++;
-    } else if (!rc) {
-      w->stats[it->second.stat]++;
-      fused.push_back(e);
+      w->stats[NXH_DEFER_GROUPED] += members.size();
+    } else if (grc == NXH_FAILURE) {
+      for (DEntry *m : members)
+        if (!rc) run_anchor(m);  // one by one, each with its own fallback
+    } else {
+      rc = grc;
     }
   }
   tls_in_flush = false;

@@ -122,6 +122,16 @@ struct Args {
   // skipped when its pointer is null. R has C's shape, unit column stride.
   const void *bias, *R;
   int64_t ldr, br[4];
+  // EPI kernels, 16-bit dtypes, whole tiles, no R: then the tanh GELU of kaun/lib/fn.ml:31-38 on
+  // the biased product, step by step with the roundings of its nine primitives
+  // (c0..c3 = 0.044715, sqrt(2/pi), 1, 0.5 as the dtype holds them).
+  int gelu;
+  float gc[4];
+  // EPI kernels: up to three products that share A and differ in (B, bias, C) of one shape and
+  // layout, as one launch (the q / k / v linears of an attention layer): tile column tn of
+  // the launch belongs to member tn / gtn. Offsets of members 1 and 2 from member 0, in elements.
+  uint32_t ngroup, gtn;
+  int64_t goff_b[2], goff_c[2], goff_bias[2];
 };
 
 // One k-step of one 32x32 tile: a, b hold this lane's VE k-values of its row.
@@ -230,6 +240,17 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
   // front to back still has its tail in the memory-side cache
   tile_of_block(a, gridDim.x - 1 - blockIdx.x, batch, tm, tn);
   int64_t ao = 0, bo = 0, co = 0, ro = 0;
+  if constexpr (EPI) {
+    if (a.ngroup > 1) {
+      const uint32_t member = tn / a.gtn;
+      tn -= member * a.gtn;
+      if (member) {
+        bo = member == 1 ? a.goff_b[0] : a.goff_b[1];
+        co = member == 1 ? a.goff_c[0] : a.goff_c[1];
+        if (a.bias) a.bias = (const S *)a.bias + (member == 1 ? a.goff_bias[0] : a.goff_bias[1]);
+      }
+    }
+  }
   {
     uint32_t idx = batch;
 #pragma unroll
@@ -402,6 +423,46 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
             return (uint32_t)lo | ((uint32_t)hi << 16);
           }
         };
+        // both neighbours rounded to the dtype, as a primitive's store and the next one's load would
+        auto rnd2 = [&](float &lo, float &hi) {
+          if constexpr (EL::BF16) {
+            const uint32_t u = f32x2_to_bf16x2(lo, hi);
+            lo = __builtin_bit_cast(float, u << 16);
+            hi = __builtin_bit_cast(float, u & 0xffff0000u);
+          } else {
+            lo = widen(narrow(lo));
+            hi = widen(narrow(hi));
+          }
+        };
+        auto gelu2 = [&](uint32_t x) -> uint32_t {
+          float v0, v1;
+          if constexpr (EL::BF16) {
+            v0 = __builtin_bit_cast(float, x << 16);
+            v1 = __builtin_bit_cast(float, x & 0xffff0000u);
+          } else {
+            v0 = widen((S)(x & 0xffffu));
+            v1 = widen((S)(x >> 16));
+          }
+          float a0 = v0 * v0, a1 = v1 * v1;  // x * x
+          rnd2(a0, a1);
+          a0 = v0 * a0, a1 = v1 * a1;        // x * (x * x)
+          rnd2(a0, a1);
+          a0 = a0 * a.gc[0], a1 = a1 * a.gc[0];
+          rnd2(a0, a1);
+          a0 = v0 + a0, a1 = v1 + a1;
+          rnd2(a0, a1);
+          a0 = a0 * a.gc[1], a1 = a1 * a.gc[1];
+          rnd2(a0, a1);
+          a0 = tanh_for_16bit(a0), a1 = tanh_for_16bit(a1);
+          rnd2(a0, a1);
+          a0 = a0 + a.gc[2], a1 = a1 + a.gc[2];
+          rnd2(a0, a1);
+          a0 = v0 * a0, a1 = v1 * a1;
+          rnd2(a0, a1);
+          a0 = a0 * a.gc[3], a1 = a1 * a.gc[3];
+          if constexpr (EL::BF16) return f32x2_to_bf16x2(a0, a1);
+          else return (uint32_t)narrow(a0) | ((uint32_t)narrow(a1) << 16);
+        };
         S *c = C + (m0 + wm + row0) * a.ldc + n0 + wn + col;
         const S *p = patch + row0 * WP + col;
         V16 bq = {0, 0, 0, 0};
@@ -428,6 +489,10 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
             if (a.bias) {
 #pragma unroll
               for (int w = 0; w < 4; w++) q[w] = add2(q[w], bq[w]);
+            }
+            if (a.gelu) {
+#pragma unroll
+              for (int w = 0; w < 4; w++) q[w] = gelu2(q[w]);
             }
             *reinterpret_cast<V16 *>(c + (int64_t)i * RSTEP * a.ldc) = q;
           }

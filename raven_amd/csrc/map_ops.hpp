@@ -6,6 +6,7 @@
 // packages/nx/lib/backend_c/nx_c_map.c:300-803; unsupported pairs are holes in
 // the dispatch tables and are rejected, never identity.
 #pragma once
+#include <type_traits>
 
 #include "map_kernels.hpp"
 
@@ -316,7 +317,8 @@ struct UnaryF {
   using In1 = Unused;
   using In2 = Unused;
   __device__ __forceinline__ static Out apply(In0 a) {
-    return T::st(OP::template eval<T::cat, typename T::C>(T::ld(a)));
+    if constexpr (std::is_same<OP, OpTanh>::value && (DT == NXH_BF16 || DT == NXH_F16)) return T::st(tanh_for_16bit(T::ld(a)));
+    else return T::st(OP::template eval<T::cat, typename T::C>(T::ld(a)));
   }
 };
 template <class OP, int DT>

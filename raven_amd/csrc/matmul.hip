@@ -659,6 +659,10 @@ static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
   NXH_HIP("matmul", attr_status);
   g.tiles_m = (uint32_t)((g.M + SH::BM - 1) / SH::BM);
   g.tiles_n = (uint32_t)((g.N + SH::BN - 1) / SH::BN);
+  if (EPI && g.ngroup > 1) {
+    g.gtn = g.tiles_n;
+    g.tiles_n *= g.ngroup;  // the members side by side, as one product of ngroup x N columns would be walked
+  }
   nxh_set_path(path);
   hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(SH::THREADS), LDS, ctx->stream, g);
   NXH_HIP("matmul", hipGetLastError());
@@ -712,6 +716,10 @@ static int forced_tile() {
 struct Epilogue {
   const void *bias = nullptr, *R = nullptr;
   int64_t ldr = 0, br[MM_MAXB] = {};
+  const double *gelu = nullptr;  // c0..c3 of the tanh GELU, applied to the biased product
+  // further members of a grouped launch: byte distances of their B, C and bias from the first's
+  int ngroup = 1;
+  int64_t goff_b[2] = {}, goff_c[2] = {}, goff_bias[2] = {};
 };
 template <class EL, bool EPI = false>
 static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool al_a, bool al_b,
@@ -746,8 +754,28 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
     g.bias = epi->bias;
     g.R = epi->R;
     g.ldr = epi->ldr;
+    if (epi->ngroup > 1) {
+      constexpr int64_t es = (int64_t)sizeof(typename EL::S);
+      g.ngroup = (uint32_t)epi->ngroup;
+      for (int i = 0; i + 1 < epi->ngroup; i++) {
+        // the members' rows must be as aligned as the first's: whole 16-byte steps apart
+        if (epi->goff_b[i] % 16 || epi->goff_c[i] % 16 || epi->goff_bias[i] % 16) return -1;
+        g.goff_b[i] = epi->goff_b[i] / es;
+        g.goff_c[i] = epi->goff_c[i] / es;
+        g.goff_bias[i] = epi->goff_bias[i] / es;
+      }
+    }
+    if (epi->gelu) {
+      // only the path that sends whole 16-byte row segments of whole 128 x 128 tiles applies it
+      if (EL::F32 || epi->R || a.M % 128 || a.N % 128 || !al16(g.C) || g.ldc % 8 || (g.bias && !al16(g.bias))) return -1;
+      for (int i = 0; i < a.batch.n; i++)
+        if (g.bc[i] % 8) return -1;
+      g.gelu = 1;
+      for (int i = 0; i < 4; i++) g.gc[i] = (float)epi->gelu[i];
+    }
   }
-  auto tiles = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * (int64_t)nbatch; };
+  const int members = EPI && epi ? epi->ngroup : 1;
+  auto tiles = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * (int64_t)nbatch * members; };
   if (tiles(128, 64) > 0x7fffffffLL) return -1;
   const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
   // Block shape: rounds of resident blocks x relative cost of one block. One
@@ -766,7 +794,7 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
     // Two block shapes are enough for the epilogue family; f16 keeps to the small one (its
     // conversions make the 256x256 epilogue too large to stay in registers).
     constexpr bool big_ok = EL::F32 || EL::BF16;
-    if (pick == 64 || !big_ok) pick = 128;
+    if (pick == 64 || !big_ok || (g.gelu && (a.M % 256 || a.N % 256))) pick = 128;
     if (pick == 128)
       return launch_tile_oriented<EL, gemm_tile::Shape128x128, true>(ctx, g, a_kc, b_kc, "linear_tile_128x128");
     if constexpr (big_ok)
@@ -813,8 +841,13 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
 
 // matmul, and with `bias` / `R` the fused linear: C = A B, then + bias[col], then
 // + R, each rounded to the dtype (tiled MFMA path only).
+struct GroupRest {  // members 1.. of a grouped linear, checked against member 0 by the caller
+  int n = 0;
+  const nxh_tensor *B[2] = {}, *bias[2] = {}, *C[2] = {};
+};
 static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, const nxh_tensor *A,
-                        const nxh_tensor *B, const nxh_tensor *bias, const nxh_tensor *R) {
+                        const nxh_tensor *B, const nxh_tensor *bias, const nxh_tensor *R, const double *gelu = nullptr,
+                        const GroupRest *rest = nullptr) {
   if (!ctx || !C || !A || !B) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, C);
   if (!rc) rc = nxh_check_tensor(op, A);
@@ -833,7 +866,7 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
   const int64_t kk = B->shape[B->ndim - 2], n = B->shape[B->ndim - 1];
   if (k != kk || C->shape[nd - 2] != m || C->shape[nd - 1] != n)
     return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
-  const bool fused = bias || R;
+  const bool fused = bias || R || gelu;
   if (bias && (bias->dtype != dt || bias->ndim != 1 || bias->shape[0] != n))
     return nxh_fail(bias->dtype != dt ? NXH_FAILURE : NXH_INVALID_ARGUMENT, op, bias->dtype != dt ? NXH_ERR_MM_DTYPE : NXH_ERR_SHAPE);
   if (R) {
@@ -932,6 +965,15 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
     epi.bias = bias ? (const char *)bias->data + bias->offset * es : nullptr;
     epi.R = R ? (const char *)R->data + R->offset * es : nullptr;
     epi.ldr = R ? R->strides[nd - 2] : 0;
+    epi.gelu = gelu;
+    if (rest && rest->n > 0) {
+      epi.ngroup = 1 + rest->n;
+      for (int i = 0; i < rest->n; i++) {
+        epi.goff_b[i] = ((const char *)rest->B[i]->data + rest->B[i]->offset * es) - (const char *)g.B;
+        epi.goff_c[i] = ((const char *)rest->C[i]->data + rest->C[i]->offset * es) - (const char *)g.C;
+        epi.goff_bias[i] = ((const char *)rest->bias[i]->data + rest->bias[i]->offset * es) - (const char *)epi.bias;
+      }
+    }
     for (int i = 0; i < nb && i < MM_MAXB; i++) epi.br[i] = rs_[i];
     const bool a_ok = g.acs == 1 || g.ars == 1, b_ok = g.brs == 1 || g.bcs == 1;
     rc = -1;
@@ -977,4 +1019,52 @@ NXH_EXPORT int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
   NXH_DEFER_TOUCH(ctx, 1, out, x, w, bias, residual);
   if (!bias && !residual) return matmul_entry(ctx, "matmul", out, x, w, nullptr, nullptr);
   return matmul_entry(ctx, "linear", out, x, w, bias, residual);
+}
+
+// linear.ml:50-52 followed by the tanh GELU of fn.ml:31-38 (the first half of gpt2.ml's MLP) in
+// the GEMM's epilogue; anything the epilogue cannot take is Failure and runs as two calls.
+NXH_EXPORT int nxh_linear_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const nxh_tensor *w,
+                                    const nxh_tensor *bias, const void *constants) {
+  NXH_DEFER_TOUCH(ctx, 1, out, x, w, bias);
+  if (!constants) return nxh_fail(NXH_INVALID_ARGUMENT, "linear_gelu", "null argument");
+  if (!out || (out->dtype != NXH_BF16 && out->dtype != NXH_F16))
+    return nxh_fail(NXH_FAILURE, "linear_gelu", "the fused form takes bfloat16 / float16 operands");
+  double c[4];
+  for (int i = 0; i < 4; i++) {
+    const uint16_t h = ((const uint16_t *)constants)[i];
+    if (out->dtype == NXH_BF16) {
+      c[i] = (double)bf16_to_f32(h);
+    } else {  // float16, exact
+      const int e = (h >> 10) & 31, m = h & 1023;
+      const double v = e == 0 ? std::ldexp((double)m, -24) : (e == 31 ? (m ? std::nan("") : HUGE_VAL) : std::ldexp((double)(m | 1024), e - 25));
+      c[i] = (h & 0x8000) ? -v : v;
+    }
+  }
+  return matmul_entry(ctx, "linear_gelu", out, x, w, bias, nullptr, c);
+}
+
+// out[i] = matmul x w[i] + bias[i] for two or three (w, bias, out) of one dtype, shape and layout
+// as ONE launch (the q / k / v projections of attention.ml:218-265 all read the same x). Failure
+// when the members differ in anything but their addresses, or the tiled GEMM does not take them;
+// the caller then runs them one by one.
+int nxh_linear_group(nxh_context *ctx, int n, const nxh_tensor *const *outs, const nxh_tensor *x,
+                     const nxh_tensor *const *ws, const nxh_tensor *const *biases) {
+  if (n < 2 || n > 3) return nxh_fail(NXH_FAILURE, "linear", "a group has two or three members");
+  auto same_layout = [](const nxh_tensor *a, const nxh_tensor *b) {
+    if (!a || !b || a->dtype != b->dtype || a->ndim != b->ndim) return false;
+    for (int d = 0; d < a->ndim; d++)
+      if (a->shape[d] != b->shape[d] || (a->shape[d] > 1 && a->strides[d] != b->strides[d])) return false;
+    return true;
+  };
+  GroupRest rest;
+  for (int i = 1; i < n; i++) {
+    if (!same_layout(outs[0], outs[i]) || !same_layout(ws[0], ws[i]) || !same_layout(biases[0], biases[i]))
+      return nxh_fail(NXH_FAILURE, "linear", "the members of a group differ in shape or layout");
+    if (int rc = nxh_check_tensor("linear", outs[i])) return rc;
+    if (int rc = nxh_check_tensor("linear", ws[i])) return rc;
+    if (int rc = nxh_check_tensor("linear", biases[i])) return rc;
+    rest.B[i - 1] = ws[i], rest.bias[i - 1] = biases[i], rest.C[i - 1] = outs[i];
+  }
+  rest.n = n - 1;
+  return matmul_entry(ctx, "linear", outs[0], x, ws[0], biases[0], nullptr, nullptr, &rest);
 }

@@ -96,6 +96,9 @@ int nxh_collect_index_fault(nxh_context *ctx, const char *op);
 // the flag is reported now, as the replay's, so that this call answers only for itself.
 int nxh_settle_replay_faults(nxh_context *ctx, const char *op);
 
+// several linear layers over one x as one launch (matmul.hip); used by the deferred window
+int nxh_linear_group(nxh_context *ctx, int n, const nxh_tensor *const *outs, const nxh_tensor *x,
+                     const nxh_tensor *const *ws, const nxh_tensor *const *biases);
 // the deferred-evaluation window (defer.hip)
 bool nxh_defer_active(nxh_context *ctx);
 int nxh_defer_flush(nxh_context *ctx);
@@ -249,6 +252,21 @@ HD uint32_t f32x2_to_bf16x2(float lo, float hi) {
 #endif
 }
 
+// tanh for a result that is rounded to a 16-bit float right behind it (bfloat16 / float16
+// tensors compute in float): (1 - t) / (1 + t) with t = e^(-2|x|) from the hardware
+// exponential and reciprocal, the odd polynomial x - x^3/3 + 2x^5/15 - 17x^7/315 below 1/8
+// where that quotient cancels. Within 4e-7 relative of tanh, against the 2^-12 of a float16
+// rounding; the library's tanhf costs about four times as many instructions and made the
+// fused GELU and the tanh primitive of those dtypes bound by the vector unit. NaN stays NaN,
+// the sign of zero is kept, +-inf gives +-1.
+__device__ __forceinline__ float tanh_for_16bit(float x) {
+  const float ax = __builtin_fabsf(x);
+  const float t = __builtin_amdgcn_exp2f(ax * -0x1.715476p+1f);  // e^(-2|x|)
+  const float big = (1.0f - t) * __builtin_amdgcn_rcpf(1.0f + t);
+  const float x2 = x * x;
+  const float small = ax * __builtin_fmaf(x2, __builtin_fmaf(x2, __builtin_fmaf(x2, -0x1.ba1ba2p-5f, 0x1.111112p-3f), -0x1.555556p-2f), 1.0f);
+  return __builtin_copysignf(ax < 0.125f ? small : big, x);
+}
 // f32 -> f16, nx_buffer_stubs.h:99-148. The hardware convert (round to nearest
 // even, subnormals kept) matches on every non-NaN input; a NaN keeps its top
 // ten payload bits and is bumped to stay a NaN.

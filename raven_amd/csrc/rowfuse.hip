@@ -299,7 +299,9 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(GeluArgs a) {
     const C p = rnd<DT>(x3 * c0);
     const C q = rnd<DT>(v + p);
     const C inner = rnd<DT>(q * c1);
-    const C th = rnd<DT>(m_tanh(inner));
+    C th;
+    if constexpr (DT == NXH_BF16 || DT == NXH_F16) th = rnd<DT>(tanh_for_16bit(inner));  // as the tanh primitive of these dtypes
+    else th = rnd<DT>(m_tanh(inner));
     const C u = rnd<DT>(th + c2);
     const C w = rnd<DT>(v * u);
     o.v[j] = TX::st(w * c3);

@@ -410,7 +410,7 @@ int main(int argc, char **argv) {
     fclose(f);
     free(host);
     printf("{\"mode\": \"%s\", \"recorded\": %llu, \"issued\": %llu, \"fallbacks\": %llu, \"softmax_rows\": %llu, "
-           "\"layer_norm_rows\": %llu, \"gelu_tanh\": %llu, \"attention\": %llu, \"linear\": %llu, \"postponed\": %llu, "
+           "\"layer_norm_rows\": %llu, \"gelu_tanh\": %llu, \"attention\": %llu, \"linear\": %llu, \"linear_gelu\": %llu, \"postponed\": %llu, "
            "\"materialised\": %llu}\n",
            mode, (unsigned long long)(s1[NXH_DEFER_RECORDED] - s0[NXH_DEFER_RECORDED]),
            (unsigned long long)(s1[NXH_DEFER_ISSUED] - s0[NXH_DEFER_ISSUED]),
@@ -420,6 +420,7 @@ int main(int argc, char **argv) {
            (unsigned long long)(s1[NXH_DEFER_GELU] - s0[NXH_DEFER_GELU]),
            (unsigned long long)(s1[NXH_DEFER_ATTENTION] - s0[NXH_DEFER_ATTENTION]),
            (unsigned long long)(s1[NXH_DEFER_LINEAR] - s0[NXH_DEFER_LINEAR]),
+           (unsigned long long)(s1[NXH_DEFER_LINEAR_GELU] - s0[NXH_DEFER_LINEAR_GELU]),
            (unsigned long long)(s1[NXH_DEFER_POSTPONED] - s0[NXH_DEFER_POSTPONED]),
            (unsigned long long)(s2[NXH_DEFER_MATERIALISED] - s0[NXH_DEFER_MATERIALISED]));
     L.context_destroy(ctx);

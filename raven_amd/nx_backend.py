@@ -172,7 +172,7 @@ class Backend:
 
     # -- deferred evaluation: primitives are recorded and fused below the C ABI --
     DEFER_STATS = ("recorded", "issued", "flushes", "fallbacks", "softmax_rows", "layer_norm_rows", "gelu_tanh",
-                   "attention", "linear", "postponed", "materialised")
+                   "attention", "linear", "postponed", "materialised", "linear_gelu", "grouped")
 
     def set_deferred(self, on: bool):
         """With the mode on, unary / binary / compare / where / cast / reduce / matmul and
@@ -584,6 +584,22 @@ class Backend:
         self._check(self._lib.nxh_linear(self._h, C.byref(o), C.byref(a), C.byref(b),
                                          C.byref(bd) if bd is not None else None,
                                          C.byref(rd) if rd is not None else None))
+        return out
+
+    def linear_gelu_tanh(self, x: Tensor, w: Tensor, bias: Tensor | None = None,
+                         constants=(0.044715, 0.7978845608028654, 1.0, 0.5)) -> Tensor:
+        """``gelu_tanh(matmul x w + bias)`` with the GELU in the GEMM's epilogue: the bits of
+        ``linear`` followed by ``gelu_tanh``. Raises for anything but bfloat16 / float16 products made
+        of whole 128 x 128 tiles (the caller then issues the two calls)."""
+        out = self.buffer(x.dtype, list(x.shape[:-1]) + [w.shape[-1]])
+        if isinstance(constants, np.ndarray):
+            enc = np.ascontiguousarray(constants.reshape(4))
+        else:
+            enc = np.concatenate([encode_scalar(x.dtype, c) for c in constants])
+        o, a, b = out._desc(), x._desc(), w._desc()
+        bd = bias._desc() if bias is not None else None
+        self._check(self._lib.nxh_linear_gelu_tanh(self._h, C.byref(o), C.byref(a), C.byref(b),
+                                                   C.byref(bd) if bd is not None else None, enc.ctypes.data))
         return out
 
     def attention(self, q: Tensor, k: Tensor, v: Tensor, scale=None, mask: Tensor | None = None,

@@ -470,6 +470,10 @@ module Fused = struct
   external caml_linear :
     ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t option -> ('a, 'b) t option -> unit = "caml_nx_hip_linear"
 
+  external caml_linear_gelu_tanh :
+    ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t -> ('a, 'b) t option -> ('a, 'b) Nx_buffer.t -> unit
+    = "caml_nx_hip_linear_gelu_tanh"
+
   let host_scalar dtype v =
     let b = Nx_buffer.create dtype 1 in
     Nx_buffer.set b 0 v; b
@@ -491,6 +495,19 @@ module Fused = struct
     let c = Nx_buffer.create x.dtype 4 in
     List.iteri (Nx_buffer.set c) [ 0.044715; Float.sqrt (2. /. Float.pi); 1.0; 0.5 ];
     caml_gelu_tanh out (contiguous x) c; out
+
+  let gelu_constants dtype =
+    let c = Nx_buffer.create dtype 4 in
+    List.iteri (Nx_buffer.set c) [ 0.044715; Float.sqrt (2. /. Float.pi); 1.0; 0.5 ];
+    c
+
+  (* gelu_approx (linear x w + bias) in the GEMM's epilogue; Failure for shapes it does not take *)
+  let linear_gelu ?bias x w =
+    let nd = Array.length x.shape in
+    let shape = Array.copy x.shape in
+    shape.(nd - 1) <- w.shape.(Array.length w.shape - 1);
+    let out = create_tensor x.context x.dtype shape in
+    caml_linear_gelu_tanh out x w bias (gelu_constants x.dtype); out
 
   (* attention.ml:67-110 for float16 / bfloat16 operands of [batch..., seq, head_dim] *)
   let attention ?mask ?(causal = false) ~scale q k v =

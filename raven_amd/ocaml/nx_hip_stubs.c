@@ -37,7 +37,7 @@
   X(sort) X(argsort) X(unfold) X(fold) X(fft) X(rfft) X(irfft) X(cholesky)    \
   X(triangular_solve) X(qr) X(eigh) X(svd) X(eig) X(device_info)              \
   X(memory_stats) X(trim) X(reduce_noalloc) X(softmax_rows) X(layer_norm_rows) \
-  X(gelu_tanh) X(attention) X(linear) X(set_deferred) X(deferred_stats)        \
+  X(gelu_tanh) X(attention) X(linear) X(linear_gelu_tanh) X(set_deferred) X(deferred_stats)        \
   X(capture_begin) X(capture_end) X(graph_launch) X(graph_destroy)             \
   X(timer_start) X(timer_stop) X(last_path)
 static struct {
@@ -704,6 +704,17 @@ CAMLprim value caml_nx_hip_linear(value vout, value vx, value vw, value vbias, v
   extract(vx, &x);
   extract(vw, &w);
   check(c, L.linear(c, &o, &x, &w, optional(vbias, &b), optional(vresidual, &r)));
+  CAMLreturn(Val_unit);
+}
+
+/* constants: as for caml_nx_hip_gelu_tanh */
+CAMLprim value caml_nx_hip_linear_gelu_tanh(value vout, value vx, value vw, value vbias, value vconstants) {
+  CAMLparam5(vout, vx, vw, vbias, vconstants);
+  nxh_tensor o, x, w, b;
+  nxh_context *c = extract(vout, &o);
+  extract(vx, &x);
+  extract(vw, &w);
+  check(c, L.linear_gelu_tanh(c, &o, &x, &w, optional(vbias, &b), Caml_ba_data_val(vconstants)));
   CAMLreturn(Val_unit);
 }
 

@@ -46,7 +46,7 @@ def test_the_compiled_host_matches_the_python_mirror(hip, oracle, tmp_path, d):
             f.write(np.ascontiguousarray(enc(a, d)).tobytes())
     ids.tofile(tmp_path / "ids.bin")
 
-    counted = ("recorded", "issued", "fallbacks", "softmax_rows", "layer_norm_rows", "gelu_tanh", "attention", "linear")
+    counted = ("recorded", "issued", "fallbacks", "softmax_rows", "layer_norm_rows", "gelu_tanh", "attention", "linear", "linear_gelu")
 
     def python_logits(deferred):
         nx = Nx(hip)
@@ -81,7 +81,8 @@ def test_the_compiled_host_matches_the_python_mirror(hip, oracle, tmp_path, d):
             continue
         # the same record, the same runs found, the same few primitives issued as recorded
         assert {k: s[k] for k in counted} == mirror_stats, (s, mirror_stats)
-        assert (s["layer_norm_rows"], s["gelu_tanh"], s["linear"], s["fallbacks"]) == (2 * L + 1, L, 6 * L, 0), s
+        mlp = L if d is dt.bfloat16 else 0  # linear + GELU as one GEMM (16-bit dtypes)
+        assert (s["layer_norm_rows"], s["gelu_tanh"], s["linear"], s["linear_gelu"], s["fallbacks"]) == (2 * L + 1, L - mlp, 6 * L - mlp, mlp, 0), s
         if d is dt.bfloat16:  # the sum of the two embeddings and the tied head's matmul, nothing else
             assert s["issued"] == 2, s
         assert (s["attention"], s["softmax_rows"]) == ((L, 0) if d is dt.bfloat16 else (0, L)), s

@@ -303,8 +303,11 @@ def test_gpt2_forward_with_the_library_window(hip, oracle, d):
         got = logical(run(hip))
         s = lib.delta()
     L = cfg.n_layer
-    assert (s["layer_norm_rows"], s["gelu_tanh"], s["linear"], s["fallbacks"]) == (2 * L + 1, L, 6 * L, 0), s
+    # 16-bit dtypes: the MLP's first linear layer and its GELU are one GEMM with the GELU in its epilogue
+    mlp = L if d is dt.bfloat16 else 0
+    assert (s["layer_norm_rows"], s["gelu_tanh"], s["linear"], s["linear_gelu"], s["fallbacks"]) == (2 * L + 1, L - mlp, 6 * L - mlp, mlp, 0), s
     assert (s["attention"], s["softmax_rows"]) == ((L, 0) if d is dt.bfloat16 else (0, L)), s
+    assert s["grouped"] == 3 * L, s  # the q, k and v projections of a layer share one launch
     # (the causal mask is still a local of the attention layer when its head merge executes the
     # record: it waits, with its run, and is dropped unwritten when the layer returns)
     assert s["materialised"] == 0
@@ -317,7 +320,7 @@ def test_gpt2_forward_with_the_library_window(hip, oracle, d):
         held.release()
         hip.synchronize()
         s3 = lib.delta()
-    for k in ("layer_norm_rows", "gelu_tanh", "linear", "attention", "softmax_rows", "fallbacks", "issued"):
+    for k in ("layer_norm_rows", "gelu_tanh", "linear", "linear_gelu", "attention", "softmax_rows", "fallbacks", "issued"):
         assert s2[k] == s[k], (k, s2, s)
     assert s2["postponed"] > 0 and s3["materialised"] == 0, (s2, s3)
     same_bits(late, got, "handles that die late against handles that die at once")
@@ -326,3 +329,63 @@ def test_gpt2_forward_with_the_library_window(hip, oracle, d):
         assert np.max(np.abs(gv - eager)) <= 2e-5 * max(1.0, np.max(np.abs(eager)))
     else:
         assert np.all(np.abs(gv - eager) <= 6e-2 + 6e-2 * np.abs(eager))
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+@pytest.mark.parametrize("rows,inputs,outputs", [(256, 128, 384), (200, 128, 384)], ids=["whole_tiles", "ragged_rows"])
+def test_linear_then_gelu_is_one_gemm(hip, oracle, d, rows, inputs, outputs):
+    """gelu_approx (linear x): with whole 128 x 128 tiles the GELU runs in the GEMM's epilogue,
+    otherwise as the fused linear followed by the fused GELU; either way the bits of the eleven
+    primitives."""
+    rng = np.random.default_rng(38)
+    nx = Nx(hip)
+    model = Gpt2(nx, Config())
+    x = tensor(hip, encode(rng.standard_normal((2, rows, inputs)), d, oracle), d)
+    w = tensor(hip, encode(rng.standard_normal((inputs, outputs)) * 0.2, d, oracle), d)
+    b = tensor(hip, encode(rng.standard_normal(outputs), d, oracle), d)
+    eager = logical(model.gelu_approx(model.linear(Linear(w, b), x)))
+    with deferred(hip) as win:
+        got = logical(model.gelu_approx(model.linear(Linear(w, b), x)))
+        s = win.delta()
+    assert (s["linear_gelu"], s["linear"], s["gelu_tanh"], s["issued"], s["fallbacks"]) == (1, 0, 0, 0, 0), s
+    same_bits(got, eager, "linear + gelu in one run against the primitives")
+    if rows % 128 == 0:
+        assert hip.last_path() == "linear_tile_128x128"
+        direct = logical(hip.linear_gelu_tanh(x, w, b))
+        same_bits(got, direct, "against nxh_linear_gelu_tanh called by name")
+    else:
+        with pytest.raises(RuntimeError):
+            hip.linear_gelu_tanh(x, w, b)
+
+
+def test_linear_layers_over_one_input_share_a_launch(hip, oracle):
+    """q, k and v of an attention layer: three linear layers over the same x. Recorded one after the
+    other, launched as one GEMM over the three weight matrices, each result the bits of its own call."""
+    rng = np.random.default_rng(39)
+    d = dt.bfloat16
+    nx = Nx(hip)
+    model = Gpt2(nx, Config())
+    x = tensor(hip, encode(rng.standard_normal((2, 192, 256)), d, oracle), d)
+    ws = [tensor(hip, encode(rng.standard_normal((256, 256)) * 0.1, d, oracle), d) for _ in range(3)]
+    bs = [tensor(hip, encode(rng.standard_normal(256), d, oracle), d) for _ in range(3)]
+    other_w = tensor(hip, encode(rng.standard_normal((256, 128)) * 0.1, d, oracle), d)
+    other_b = tensor(hip, encode(rng.standard_normal(128), d, oracle), d)
+    eager = [logical(model.linear(Linear(w, b), x)) for w, b in zip(ws, bs)] + [logical(model.linear(Linear(other_w, other_b), x))]
+    with deferred(hip) as win:
+        outs = [model.linear(Linear(w, b), x) for w, b in zip(ws, bs)]
+        outs.append(model.linear(Linear(other_w, other_b), x))  # another shape: on its own
+        got = [logical(t) for t in outs]
+        s = win.delta()
+    assert (s["linear"], s["grouped"], s["issued"], s["fallbacks"]) == (4, 3, 0, 0), s
+    for i, (g, e) in enumerate(zip(got, eager)):
+        same_bits(g, e, f"member {i} of the grouped launch against its own call")
+    # a member whose result is read before the last member was recorded stays out of the group
+    with deferred(hip) as win:
+        a = model.linear(Linear(ws[0], bs[0]), x)
+        a2 = nx.add(a, a)
+        b = model.linear(Linear(ws[1], bs[1]), x)
+        got = [logical(t) for t in (a, a2, b)]
+        s = win.delta()
+    assert s["grouped"] == 0 and s["linear"] == 2, s
+    same_bits(got[0], eager[0], "ungrouped member")
+    same_bits(got[2], eager[1], "ungrouped member")

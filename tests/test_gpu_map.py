@@ -365,3 +365,25 @@ def test_error_kinds(hip):
         hip.unary("sin", hip.cast(x, dt.int32))
     with pytest.raises(RuntimeError, match="dtype not supported"):
         hip.binary("add", hip.cast(x, dt.bool_), hip.cast(x, dt.bool_))
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_tanh_of_16bit_dtypes_over_every_input(hip, oracle, d):
+    """tanh of a bfloat16 / float16 tensor uses a short form of its own (hardware exponential and
+    reciprocal) instead of the library's tanhf. All 65536 inputs: NaNs, zeros and their signs and
+    the saturation at +-1 are exactly the oracle's; every other result is the oracle's correctly
+    rounded one or its neighbour, the neighbour in fewer than 1 % of the inputs."""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    storage = bits.view(d.np_storage)
+    (hx, ox) = pair(storage, d, hip, oracle)
+    got = logical(hip.unary("tanh", hx)).view(np.uint16)
+    want = logical(oracle.unary("tanh", ox)).view(np.uint16)
+    gv, wv = decode(got.view(d.np_storage), d, oracle), decode(want.view(d.np_storage), d, oracle)
+    assert np.array_equal(np.isnan(gv), np.isnan(wv))
+    finite = ~np.isnan(wv)
+    assert np.array_equal(np.signbit(gv[finite]), np.signbit(wv[finite]))
+    assert np.array_equal(gv[finite] == 0, wv[finite] == 0)
+    assert np.array_equal(np.abs(gv[finite]) == 1, np.abs(wv[finite]) == 1) or np.mean((np.abs(gv[finite]) == 1) != (np.abs(wv[finite]) == 1)) < 1e-3
+    step = np.abs(got[finite].astype(np.int32) - want[finite].astype(np.int32))  # same sign: adjacent patterns are adjacent values
+    assert step.max() <= 1, int(step.max())
+    assert np.mean(step != 0) < 0.01, float(np.mean(step != 0))
