@@ -553,19 +553,29 @@ def compiled_host_config5(iters=3):
 def config5(hip, work, iters=3, warmup=1, window=False, graph=False, keep_positions=64):
     """GPT-2-small-shaped forward (12 layers, d 768, 12 heads, FFN 3072, vocab
     50257, batch 8 x seq 1024, bf16 random-init weights): tokens/s. Eager: one
-    backend call per primitive. With ``window``: the same frontend calls go
-    through the deferred-evaluation window, which replaces the softmax, layer
-    norm and GELU sequences by the fused row kernels. With ``graph`` too: the
-    windowed forward is recorded once and each timed step is one replay.
+    backend call per primitive. With ``window``: the same calls with the library's
+    deferred mode on (nxh_set_deferred): it records the primitives and replaces the
+    attention, softmax, layer-norm, GELU and linear sequences by fused kernels. With
+    ``graph`` too: that forward is recorded once and each timed step is one replay.
     Returns the record and logits[0, :keep_positions, :] of the last timed step."""
     from raven_amd.kaun_gpt2 import Gpt2, upload
     from raven_amd.nx_frontend import Nx
-    from raven_amd.nx_window import Window
 
     cfg, batch, seq = work.cfg, work.batch, work.seq
     counter = CountingBackend(hip)
-    front = Window(counter) if window else counter
+    front = counter
     nx = Nx(front)
+    hip.set_deferred(bool(window))
+    try:
+        return _config5_timed(hip, work, counter, front, nx, iters, warmup, window, graph, keep_positions)
+    finally:
+        hip.set_deferred(False)
+
+
+def _config5_timed(hip, work, counter, front, nx, iters, warmup, window, graph, keep_positions):
+    from raven_amd.kaun_gpt2 import Gpt2, upload
+
+    cfg, batch, seq = work.cfg, work.batch, work.seq
     params = upload(nx, work.hp, dt.bfloat16, lambda a, d: bf16_bits(a))
     ids = nx.create(dt.int32, (batch, seq), work.ids)
     model = Gpt2(nx, cfg)
@@ -577,10 +587,11 @@ def config5(hip, work, iters=3, warmup=1, window=False, graph=False, keep_positi
     if graph:
         front.capture_begin()
         try:
-            out = front.force(model.logits(params, ids))
+            out = model.logits(params, ids)
         finally:
             recorded = front.capture_end()
     counter.calls.clear()
+    stats0 = hip.deferred_stats()
     t0 = time.perf_counter()
     front.timer_start()
     for i in range(iters):
@@ -594,19 +605,23 @@ def config5(hip, work, iters=3, warmup=1, window=False, graph=False, keep_positi
     front.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / iters
     calls = {k: v // iters for k, v in counter.calls.items()}
-    final = out if recorded is not None or not window else front.force(out)
+    stats1 = hip.deferred_stats()
+    fused = {k: (stats1[k] - stats0[k]) // iters for k in stats1 if stats1[k] != stats0[k]}
+    final = out
     head = logical(hip.contiguous(hip.shrink(final, [(0, 1), (0, keep_positions), (0, cfg.vocab_size)])))
     del out, final
     if recorded is not None:
         recorded.destroy()
     flops = 284812800 * batch * seq  # matmul FLOPs per forward
     how = ("the windowed forward recorded once, each step one graph replay" if graph else
-           "deferred-evaluation window: attention, layer norm, GELU and linear sequences as fused kernels" if window
+           "the library's deferred mode: attention, layer norm, GELU and linear sequences as fused kernels" if window
            else "eager, one backend call per primitive")
     rec = {"op": f"cfg5 GPT-2 small forward, bf16, batch 8 x seq 1024 ({how})",
            "ms": round(ms, 3), "tokens/s": round(batch * seq / (ms * 1e-3), 1), "hip_event_ms": round(ev_ms, 3),
            "matmul_TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1), "backend_calls": sum(calls.values()),
            "calls_by_kind": calls}
+    if window and recorded is None:
+        rec["library_counters_per_forward"] = fused  # primitives recorded, issued as recorded, runs fused
     del params, ids, model, nx, front
     hip.trim()
     return rec, head
