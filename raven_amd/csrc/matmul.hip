@@ -454,6 +454,109 @@ __global__ __launch_bounds__(256) void gemm_skinny_mfma_kernel(SkinnyArgs a) {
   }
 }
 
+// ── gemm_skinny_mfma_k8: the same stream when N alone fills the chip ────────
+// One block of eight waves owns 64 columns; the waves split K eight ways and fold their
+// accumulators through LDS in wave order at the end, so there are no f32 partials in memory
+// and no second launch. A (at most 16 x K, a few dozen KiB, resident in L2) is not staged:
+// each lane reads its 16-byte fragment of the step straight from memory, three steps ahead
+// like the B vectors, so a block starts streaming with its first instruction.
+constexpr int SM8_WAVES = 8;
+template <bool BF16>
+__global__ __launch_bounds__(64 * SM8_WAVES) void gemm_skinny_mfma_k8_kernel(SkinnyArgs a) {
+  using gemm_tile::lds_s16x4;
+  using gemm_tile::s16x4;
+  typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+  extern __shared__ __attribute__((aligned(16))) uint16_t sm_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t n0 = (int64_t)blockIdx.x * SM_WN;
+  const int64_t k0 = (int64_t)wave * a.kchunk;
+  const int64_t k1 = k0 + a.kchunk < a.K ? k0 + a.kchunk : a.K;
+  const int kn = k1 > k0 ? (int)(k1 - k0) : 0;  // a multiple of 8 (K is)
+  const uint16_t *A = (const uint16_t *)a.A;
+  const uint16_t *B = (const uint16_t *)a.B;
+  uint16_t *sB = sm_lds + wave * (2 * SM_TILE);
+  const int c8 = (lane & 7) * 8, rbase = lane >> 3;
+  const bool col_ok = n0 + c8 < a.N;
+  const uint16_t *bp = B + k0 * a.brs + n0 + c8;
+  const int g = lane >> 4, L = lane & 15;
+  const uint16_t *ap = A + (int64_t)L * a.ars + k0 + g * 8;  // rows >= M read as zero
+  const bool row_ok = L < a.M;
+  U4 rb[3][4], ra[3];
+  auto load = [&](U4 (&r)[4], U4 &x, int step) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int kk = step * SM_KS + rbase + i * 8;
+      r[i] = (col_ok && kk < kn) ? *reinterpret_cast<const U4 *>(bp + (int64_t)kk * a.brs) : U4{0, 0, 0, 0};
+    }
+    const int ka = step * SM_KS + g * 8;
+    x = (row_ok && ka < kn) ? *reinterpret_cast<const U4 *>(ap + step * SM_KS) : U4{0, 0, 0, 0};
+  };
+  auto store = [&](const U4 (&r)[4], int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      *reinterpret_cast<U4 *>(sB + buf * SM_TILE + (rbase + i * 8) * SM_PITCH + c8) = r[i];
+  };
+  f32x4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; t++) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  const int nsteps = (kn + SM_KS - 1) / SM_KS;
+  // step s multiplies the tile in LDS buffer s & 1 by the A fragment of slot s % 3; slot (s + 1) % 3
+  // is stored for step s + 1 and refilled with step s + 4
+  auto step = [&](int s, auto slot_c) {
+    constexpr int SL = decltype(slot_c)::value;       // slot of step s + 1
+    constexpr int CUR = (SL + 2) % 3;                 // slot of step s
+    const U4 xa = ra[CUR];
+    if (s + 1 < nsteps) store(rb[SL], (s + 1) & 1);
+    const uint16_t *tile = sB + (s & 1) * SM_TILE + (g * 8 + (L >> 2)) * SM_PITCH + (L & 3) * 4;
+    U4 yb[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(tile + t * 16)));
+      const u32x2 hi = __builtin_bit_cast(
+          u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(tile + t * 16 + 4 * SM_PITCH)));
+      yb[t] = U4{lo[0], lo[1], hi[0], hi[1]};
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      if constexpr (BF16)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa), __builtin_bit_cast(bf16x8, yb[t]),
+                                                         acc[t], 0, 0, 0);
+      else
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, xa), __builtin_bit_cast(f16x8, yb[t]),
+                                                        acc[t], 0, 0, 0);
+    }
+    // the slot of step s is free once its fragment has been multiplied: refill it with step s + 3
+    if (s + 3 < nsteps) load(rb[CUR], ra[CUR], s + 3);
+  };
+  // slots: step s lives in slot s % 3
+  if (nsteps > 0) load(rb[0], ra[0], 0);
+  if (nsteps > 1) load(rb[1], ra[1], 1);
+  if (nsteps > 2) load(rb[2], ra[2], 2);
+  if (nsteps > 0) store(rb[0], 0);
+  for (int s = 0; s < nsteps; s += 3) {
+    step(s, std::integral_constant<int, 1>{});
+    if (s + 1 < nsteps) step(s + 1, std::integral_constant<int, 2>{});
+    if (s + 2 < nsteps) step(s + 2, std::integral_constant<int, 0>{});
+  }
+  // fold the eight waves' [16][64] tiles in wave order
+  __syncthreads();  // every wave is done with its tiles: the buffer becomes [wave][16][64] floats
+  float *red = reinterpret_cast<float *>(sm_lds);
+#pragma unroll
+  for (int t = 0; t < 4; t++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) red[(wave * 16 + g * 4 + e) * SM_WN + t * 16 + L] = acc[t][e];
+  __syncthreads();
+  for (int o = threadIdx.x; o < 16 * SM_WN; o += 64 * SM8_WAVES) {
+    const int m = o / SM_WN, c = o - m * SM_WN;
+    const int64_t n = n0 + c;
+    if (m >= a.M || n >= a.N) continue;
+    float sum = red[o];
+#pragma unroll
+    for (int w = 1; w < SM8_WAVES; w++) sum += red[w * 16 * SM_WN + o];
+    ((uint16_t *)a.C)[m * a.crs + n * a.ccs] = BF16 ? f32_to_bf16(sum) : f32_to_f16(sum);
+  }
+}
+
 // Sums the [nsplit][m * n] partials in split order, four outputs per lane.
 template <int DT>
 __global__ __launch_bounds__(256) void skinny_finish_kernel(const float *P, void *Cv, int64_t M, int64_t N,
@@ -606,6 +709,27 @@ static int launch_skinny_mfma(nxh_context *ctx, GemmArgs &g) {
   a.crs = g.crs;
   a.ccs = g.ccs;
   const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  // N alone fills the chip with 64-column blocks: K is split inside the block, one launch
+  const int64_t strips = (g.N + SM_WN - 1) / SM_WN;
+  if (strips >= cus && g.K % 8 == 0 && g.K >= SM8_WAVES * 2 * SM_KS && (g.M == 1 || (g.acs == 1 && g.ars % 8 == 0)) &&
+      (g.M > 1 || g.acs == 1) && ((uintptr_t)g.A % 16) == 0 && strips <= 0x7fffffffLL) {
+    auto kern = gemm_skinny_mfma_k8_kernel<DT == NXH_BF16>;
+    constexpr size_t LDS = sizeof(uint16_t) * (size_t)(SM8_WAVES * 2 * SM_TILE);
+    static_assert(LDS >= sizeof(float) * SM8_WAVES * 16 * SM_WN, "the fold buffer reuses the tiles");
+    static std::once_flag once;
+    static hipError_t attr_status = hipSuccess;
+    std::call_once(once, [&] {
+      attr_status = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+    });
+    NXH_HIP("matmul", attr_status);
+    a.kchunk = ((g.K + SM8_WAVES - 1) / SM8_WAVES + SM_KS - 1) / SM_KS * SM_KS;
+    a.nsplit = 1;
+    a.C = g.C;
+    nxh_set_path("gemm_skinny_mfma_k8");
+    hipLaunchKernelGGL(kern, dim3((unsigned)strips), dim3(64 * SM8_WAVES), LDS, ctx->stream, a);
+    NXH_HIP("matmul", hipGetLastError());
+    return NXH_OK;
+  }
   const int64_t col_blocks = (g.N + 4 * SM_WN - 1) / (4 * SM_WN);
   int64_t want = std::max<int64_t>(1, ((int64_t)cus * 2 + col_blocks - 1) / col_blocks);
   int64_t nsplit = std::min<int64_t>(want, std::max<int64_t>(1, g.K / 128));

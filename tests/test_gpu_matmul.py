@@ -176,6 +176,23 @@ def test_matmul_skinny_decode_shape(hip, oracle):
     assert np.all(np.isinf(got[:, 5]) | np.isnan(got[:, 5])) and np.all(np.isfinite(np.delete(got, 5, axis=1)))
 
 
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+@pytest.mark.parametrize("m,k,n", [(8, 1024, 16384), (1, 520, 16392), (16, 4096, 16384), (13, 768, 17000)],
+                         ids=lambda v: str(v))
+def test_matmul_skinny_wide_output(hip, oracle, d, m, k, n):
+    """Decode-like products whose N alone fills the chip: K is split over the eight waves of a block
+    and folded in LDS (one launch, no partials in memory). Ragged K (a multiple of 8, not of the
+    waves' 32-row steps), N ending inside a block's 64 columns, m = 1 and m = 16."""
+    rng = np.random.default_rng(m + k + n + d.tag)
+    a = encode(rng.standard_normal((m, k)) * 0.5, d, oracle)
+    b = encode(rng.standard_normal((k, n)) * 0.5, d, oracle)
+    ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
+    check(hip, oracle, d, ha, hb, a, b, f"skinny wide m={m} k={k} n={n}")
+    assert hip.last_path() == "gemm_skinny_mfma_k8"
+    # the same product twice: the fold order is fixed, so the bits repeat
+    assert np.array_equal(logical(hip.matmul(ha, hb)), logical(hip.matmul(ha, hb)))
+
+
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16, dt.float32], ids=lambda d: d.name)
 def test_matmul_big_tile_kernel(hip, oracle, d):
     """The LDS-tiled kernel family: every block shape, whole and ragged tiles,
