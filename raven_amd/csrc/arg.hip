@@ -30,7 +30,8 @@ struct ArgCmp {
   // selects on one predicate: an if-statement form of this function compiled
   // (hipcc 7.2, gfx950, several candidates per lane) to code that never took
   // the update for float candidates.
-  __device__ __forceinline__ static void merge(C &bv, int64_t &bi, C v, int64_t i) {
+  template <class I>
+  __device__ __forceinline__ static void merge(C &bv, I &bi, C v, I i) {
     const bool take = (int)(i >= 0) & ((int)(bi < 0) | (int)beats(v, bv) | ((int)!beats(bv, v) & (int)(i < bi)));
     bv = take ? v : bv;
     bi = take ? i : bi;
@@ -53,8 +54,8 @@ struct ArgArgs {
 
 // A lane meets its candidates in ascending index order, so only a strictly
 // better one (or the first) replaces its running best.
-template <class CMP, class C>
-__device__ __forceinline__ void arg_take(C &bv, int64_t &bi, C v, int64_t i) {
+template <class CMP, class C, class I>
+__device__ __forceinline__ void arg_take(C &bv, I &bi, C v, I i) {
   const bool take = (bi < 0) | CMP::beats(v, bv);
   bv = take ? v : bv;
   bi = take ? i : bi;
@@ -143,7 +144,8 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
   using C = typename IN::C;
   static_assert(V == 1 || !HAS_IDX, "carried indices are read one at a time");
   constexpr int LANES = FOLD_THREADS / RG;
-  constexpr int U = 4;
+  constexpr int U = HAS_IDX ? 4 : 8;  // loads in flight per lane
+  using I = int32_t;               // row indices fit the int32 result
   __shared__ C lv[RG > 1 ? (RG - 1) * LANES * V : 1];
   __shared__ int32_t li[RG > 1 ? (RG - 1) * LANES * V : 1];
   const uint32_t bx = gridDim.x - 1 - blockIdx.x;  // from the end, as in arg_row_kernel
@@ -159,7 +161,7 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
   const int64_t r1 = live ? (r0 + a.chunk < a.R ? r0 + a.chunk : a.R) : r0;
   const T *p = (const T *)a.in + in_off + l;
   C bv[V];
-  int64_t bi[V];
+  I bi[V];
 #pragma unroll
   for (int k = 0; k < V; k++) bv[k] = C{}, bi[k] = -1;
   int64_t r = r0 + rg;
@@ -175,16 +177,16 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
     for (int j = 0; j < U; j++)
 #pragma unroll
       for (int k = 0; k < V; k++) {
-        if (HAS_IDX) CMP::merge(bv[k], bi[k], IN::ld(x[j].v[k]), (int64_t)xi[j]);
-        else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x[j].v[k]), r + j * RG);
+        if (HAS_IDX) CMP::merge(bv[k], bi[k], IN::ld(x[j].v[k]), (I)xi[j]);
+        else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x[j].v[k]), (I)(r + j * RG));
       }
   }
   for (; r < r1; r += RG) {
     FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
 #pragma unroll
     for (int k = 0; k < V; k++) {
-      if (HAS_IDX) CMP::merge(bv[k], bi[k], IN::ld(x.v[k]), (int64_t)a.in_idx[in_off + l + r * a.r_stride]);
-      else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x.v[k]), r);
+      if (HAS_IDX) CMP::merge(bv[k], bi[k], IN::ld(x.v[k]), (I)a.in_idx[in_off + l + r * a.r_stride]);
+      else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x.v[k]), (I)r);
     }
   }
   if constexpr (RG > 1) {
@@ -201,7 +203,7 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
     for (int g = 1; g < RG; g++)
 #pragma unroll
       for (int k = 0; k < V; k++)
-        CMP::merge(bv[k], bi[k], lv[((g - 1) * V + k) * LANES + ln], (int64_t)li[((g - 1) * V + k) * LANES + ln]);
+        CMP::merge(bv[k], bi[k], lv[((g - 1) * V + k) * LANES + ln], (I)li[((g - 1) * V + k) * LANES + ln]);
   }
   if (!live) return;
   if (a.nsplit > 1) {
