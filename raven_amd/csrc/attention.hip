@@ -64,6 +64,10 @@ struct AttArgs {
   int sq, sk, qtiles;
   int causal, has_mask, has_scale;
   float scale, masked;
+  // one-pass form with a positive scale and a -inf fill: the scores stay unscaled and the scale
+  // goes into the exponent, e^(scale (s - m)) = 2^(s c - m c) with c = scale log2(e)
+  int raw;
+  float c2;
 };
 
 template <class EL>
@@ -149,16 +153,17 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
       const V16 kf = *reinterpret_cast<const V16 *>(kr + s * 16);
       gemm_tile::mfma_step<EL>(acc, kf, qf[s]);
     }
+    const bool scaled = a.has_scale && !(ONLINE && a.raw);
     if (inner) {
 #pragma unroll
-      for (int e = 0; e < 16; e++) t[e] = a.has_scale ? acc[e] * a.scale : acc[e];
+      for (int e = 0; e < 16; e++) t[e] = scaled ? acc[e] * a.scale : acc[e];
       return;
     }
 #pragma unroll
     for (int e = 0; e < 16; e++) {
       const int j = j0 + (e >> 2) * 8 + g * 4 + (e & 3);
       float x = acc[e];
-      if (a.has_scale) x = x * a.scale;
+      if (scaled) x = x * a.scale;
       bool keep = true;
       if (a.causal) keep = j <= qi;
       else if (a.has_mask) keep = M[(int64_t)qrow * a.mask.row + (int64_t)(j < a.sk ? j : a.sk - 1) * a.mask_col] != 0;
@@ -247,13 +252,29 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
             m_new = __builtin_fmaxf(m_new, xor32(m_new));
             // nothing visible yet: exponentials of -inf against 0 are 0, not NaN
             const float m_ref = m_new == -__builtin_inff() ? 0.0f : m_new;
-            const float alpha = exp_nonpositive(m_run - m_ref);
-            float sum = 0.0f;
+            float alpha, sum = 0.0f;
+            if (a.raw) {
+              // The exponential is the bare hardware 2^x of one fused multiply-add: about 1e-6
+              // relative, three orders below the 16-bit rounding that follows (the six-instruction
+              // form of the two-pass kernel is kept where the quotient is rounded instead).
+              const float mc = -m_ref * a.c2;
+              // (an unchanged maximum must give exactly 1: the product in the fused form is not rounded as mc was)
+              alpha = m_run == m_ref ? 1.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(m_run, a.c2, mc));
 #pragma unroll
-            for (int e = 0; e < 16; e += 2) {
-              const float p0 = exp_nonpositive(t[e] - m_ref), p1 = exp_nonpositive(t[e + 1] - m_ref);
-              sum = sum + p0 + p1;
-              pk[e >> 1] = narrow2<EL>(p0, p1);
+              for (int e = 0; e < 16; e += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(t[e], a.c2, mc));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(t[e + 1], a.c2, mc));
+                sum = sum + p0 + p1;
+                pk[e >> 1] = narrow2<EL>(p0, p1);
+              }
+            } else {
+              alpha = exp_nonpositive(m_run - m_ref);
+#pragma unroll
+              for (int e = 0; e < 16; e += 2) {
+                const float p0 = exp_nonpositive(t[e] - m_ref), p1 = exp_nonpositive(t[e + 1] - m_ref);
+                sum = sum + p0 + p1;
+                pk[e >> 1] = narrow2<EL>(p0, p1);
+              }
             }
             l_run = __builtin_fmaf(l_run, alpha, sum);
             if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -421,6 +442,8 @@ NXH_EXPORT int nxh_attention(nxh_context *ctx, const nxh_tensor *out, const nxh_
   a.has_scale = scale ? 1 : 0;
   a.scale = scale ? *(const float *)scale : 1.0f;
   a.masked = masked_value ? *(const float *)masked_value : 0.0f;
+  a.raw = a.scale > 0.0f && a.scale < __builtin_inff() && (!(mask || causal) || a.masked == -__builtin_inff());
+  a.c2 = a.scale * 0x1.715476p+0f;
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path("attention_fused");
