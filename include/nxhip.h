@@ -405,9 +405,12 @@ int nxh_eig(nxh_context *ctx, const nxh_tensor *w, const nxh_tensor *v, const nx
    kaun/lib/layer_norm.ml:43-68, fn.ml:31-38, attention.ml:67-110, linear.ml:50-52)
    and whose backend runs each primitive as it is called. With the mode on,
    nxh_unary / nxh_binary / nxh_compare / nxh_where / nxh_cast / nxh_reduce /
-   nxh_matmul and a one-element nxh_fill only record their call. The record is
+   nxh_matmul / nxh_copy, a one-element nxh_fill and an nxh_memcpy_h2d of at most
+   64 KiB (whose bytes are kept) only record their call. The record is
    executed, in issue order, by the next call of any other entry point (a host
-   read and nxh_synchronize included) or when it reaches 512 entries. A run that
+   read and nxh_synchronize included), at a recorded copy once it holds 48
+   entries (so that the device works while the host records on), or when it
+   reaches 2048 entries. A run that
    spells one of those sequences, and whose intermediate results are read only
    inside the run, is replaced by the fused entry point below. An intermediate
    whose block was given back with nxh_free while recorded is never written; one

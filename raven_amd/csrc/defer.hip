@@ -42,16 +42,22 @@
 namespace {
 
 enum { D_UNARY = NXH_D_UNARY, D_BINARY = NXH_D_BINARY, D_COMPARE = NXH_D_COMPARE, D_WHERE = NXH_D_WHERE, D_CAST = NXH_D_CAST,
-       D_REDUCE = NXH_D_REDUCE, D_MATMUL = NXH_D_MATMUL, D_FULL = NXH_D_FULL };
-constexpr size_t LIMIT = 512;
+       D_REDUCE = NXH_D_REDUCE, D_MATMUL = NXH_D_MATMUL, D_FULL = NXH_D_FULL, D_COPY = NXH_D_COPY, D_UPLOAD = NXH_D_UPLOAD };
+constexpr size_t LIMIT = 2048;
+// A recorded copy (the frontend's `contiguous`) ends whatever run led up to it; once the record holds
+// this many entries it is executed there, so that the device works while the host records on.
+constexpr size_t COPY_FLUSH = 48;
+constexpr size_t UPLOAD_LIMIT = 65536;  // bytes of a host upload that may wait in the record
 constexpr int64_t MAX_ROW = 8192;
 
 struct DEntry {
   int kind = 0, op = 0, nin = 0, n_axes = 0;
   nxh_tensor out{}, in[3] = {};
   DEntry *prod[3] = {nullptr, nullptr, nullptr};  // recorded producer of each input, if any
+  DEntry *upl[3] = {nullptr, nullptr, nullptr};   // or the recorded upload that fills it (an operand like any stored tensor)
   int32_t axes[NXH_MAX_NDIM] = {};
   unsigned char value[16] = {};  // D_FULL: the element
+  std::vector<unsigned char> payload;  // D_UPLOAD: the host bytes
   bool alive = true;             // the output block has not been freed
   bool done = false;             // issued, or inside a fused run that was issued
   DEntry *fused_into = nullptr;
@@ -165,9 +171,10 @@ bool is_island(int dt) { return dt == NXH_F16 || dt == NXH_BF16; }
 struct Opnd {
   const nxh_tensor *t = nullptr;
   DEntry *prod = nullptr;
+  DEntry *upl = nullptr;
   explicit operator bool() const { return t != nullptr; }
 };
-Opnd in_of(DEntry *e, int k) { return Opnd{&e->in[k], e->prod[k]}; }
+Opnd in_of(DEntry *e, int k) { return Opnd{&e->in[k], e->prod[k], e->upl[k]}; }
 bool same_operand(const Opnd &a, const Opnd &b) { return a.prod == b.prod && same_view(*a.t, *b.t); }
 
 DEntry *producer_of(const Opnd &o, int kind, int op = -1, bool identity = true) {
@@ -233,6 +240,8 @@ struct Plan {
   int stat = 0;
   std::vector<DEntry *> interior;
   bool causal_flag = false;
+  bool has_out_view = false;  // ATTENTION: the result goes straight into a following transposing copy's output
+  nxh_tensor out_view{};
   DEntry *linear_out = nullptr;  // LINEAR_GELU: the bias add whose result the GELU read
   // operands of the fused call
   Opnd x, a, b, c;
@@ -590,6 +599,10 @@ int issue_inputs(nxh_context *ctx, DEntry *e) {
   for (int k = 0; k < e->nin; k++)
     if (e->prod[k] && !e->prod[k]->done && e->prod[k]->kind == D_FULL)
       if (int rc = issue(ctx, e->prod[k])) return rc;
+  // and an upload that nobody holds any more happens now
+  for (int k = 0; k < e->nin; k++)
+    if (e->upl[k] && !e->upl[k]->done)
+      if (int rc = issue(ctx, e->upl[k])) return rc;
   return NXH_OK;
 }
 
@@ -605,6 +618,8 @@ int issue(nxh_context *ctx, DEntry *e) {
     case D_CAST: return nxh_cast(ctx, &e->out, &e->in[0]);
     case D_REDUCE: return nxh_reduce(ctx, e->op, &e->out, &e->in[0], e->axes, e->n_axes);
     case D_MATMUL: return nxh_matmul(ctx, &e->out, &e->in[0], &e->in[1]);
+    case D_COPY: return nxh_copy(ctx, &e->out, &e->in[0]);
+    case D_UPLOAD: return nxh_memcpy_h2d(ctx, e->out.data, e->payload.data(), e->payload.size());
     default: return nxh_fill(ctx, &e->out, e->value);
   }
 }
@@ -622,14 +637,17 @@ nxh_tensor vector_of(const nxh_tensor &v) {
 int run_plan(nxh_context *ctx, DEntry *anchor, const Plan &p) {
   // inputs of the fused call that are recorded scalars never reach it as tensors; the
   // tensors it reads are results of entries issued before the run or existing storage
-  for (const Opnd *o : {&p.x, &p.a, &p.b, &p.c})
+  for (const Opnd *o : {&p.x, &p.a, &p.b, &p.c}) {
     if (*o && o->prod && !o->prod->done && o->prod->kind == D_FULL)
       if (int rc = issue(ctx, o->prod)) return rc;
+    if (*o && o->upl && !o->upl->done)
+      if (int rc = issue(ctx, o->upl)) return rc;
+  }
   switch (p.stat) {
     case NXH_DEFER_SOFTMAX:
       return nxh_softmax_rows(ctx, &anchor->out, p.x.t, p.has_s0 ? p.s0 : nullptr, p.a ? p.a.t : nullptr, p.has_s1 ? p.s1 : nullptr);
     case NXH_DEFER_ATTENTION:
-      return nxh_attention(ctx, &anchor->out, p.x.t, p.a.t, p.b.t, p.has_s0 ? p.s0 : nullptr, p.c ? p.c.t : nullptr,
+      return nxh_attention(ctx, p.has_out_view ? &p.out_view : &anchor->out, p.x.t, p.a.t, p.b.t, p.has_s0 ? p.s0 : nullptr, p.c ? p.c.t : nullptr,
                            p.has_s1 ? p.s1 : nullptr, p.causal_flag ? 1 : 0);
     case NXH_DEFER_LINEAR: {
       nxh_tensor bias;
@@ -725,11 +743,20 @@ int settle_read(nxh_context *ctx, Window *w, const void *block) {
   auto it = w->postponed_out.find(const_cast<void *>(block));
   if (it == w->postponed_out.end()) return NXH_OK;
   for (auto &m : it->second->members) {
-    if (m->out.data != block || (m->kind != D_FULL && !(m->kind == D_COMPARE && m->causal))) continue;
+    if (m->out.data != block || (m->kind != D_FULL && m->kind != D_UPLOAD && !(m->kind == D_COMPARE && m->causal))) continue;
     if (m->done) return NXH_OK;
     const bool outer = tls_in_flush;
     tls_in_flush = true;
-    const int rc = issue(ctx, m.get());
+    int rc = NXH_OK;
+    // a causal mask is computed from uploads that may be waiting beside it
+    if (m->kind == D_COMPARE)
+      for (auto &u : it->second->members)
+        if (!rc && u->kind == D_UPLOAD && !u->done && (u->out.data == m->in[0].data || u->out.data == m->in[1].data)) {
+          rc = issue(ctx, u.get());
+          w->stats[NXH_DEFER_ISSUED]++;
+          w->stats[NXH_DEFER_MATERIALISED]++;
+        }
+    if (!rc) rc = issue(ctx, m.get());
     tls_in_flush = outer;
     w->stats[NXH_DEFER_ISSUED]++;
     w->stats[NXH_DEFER_MATERIALISED]++;
@@ -766,6 +793,50 @@ int flush_locked(nxh_context *ctx, Window *w) {
       plans.emplace(e, std::move(p));
     }
   }
+  // attention.ml:218-265 merges the heads by `contiguous (swapaxes ...)` of the attention result:
+  // when that copy is the result's only reader, the kernel writes through the copy's output with
+  // the permuted strides, and the copy becomes the run's last entry.
+  {
+    std::vector<std::pair<DEntry *, DEntry *>> moves;  // (attention anchor, copy)
+    for (auto &pl : plans) {
+      DEntry *e = pl.first;
+      if (pl.second.stat != NXH_DEFER_ATTENTION || e->readers.size() != 1) continue;
+      DEntry *r = e->readers[0];
+      if (r->kind != D_COPY || r->prod[0] != e || r->fused_into || plans.count(r) || (e->alive && !w->may_postpone)) continue;
+      const nxh_tensor &v = r->in[0], &o = e->out, &ro = r->out;
+      const int nd = o.ndim;
+      if (v.ndim != nd || ro.ndim != nd || v.offset != 0 || ro.dtype != o.dtype || !same_shape(v, ro) || !c_contiguous(ro) ||
+          ro.offset != 0)
+        continue;
+      // v is a permutation of the result's axes: axis j of v is axis perm[j] of the result
+      int64_t cs[NXH_MAX_NDIM], acc = 1;
+      for (int i = nd - 1; i >= 0; i--) cs[i] = acc, acc *= o.shape[i];
+      int perm[NXH_MAX_NDIM];
+      bool used[NXH_MAX_NDIM] = {}, ok = true;
+      for (int j = 0; j < nd && ok; j++) {
+        int hit = -1;
+        for (int i = 0; i < nd && hit < 0; i++)
+          if (!used[i] && o.shape[i] == v.shape[j] && (o.shape[i] == 1 || cs[i] == v.strides[j])) hit = i;
+        if (hit < 0) ok = false;
+        else used[hit] = true, perm[j] = hit;
+      }
+      if (!ok || perm[nd - 1] != nd - 1) continue;  // rows stay contiguous
+      nxh_tensor view = o;                           // the result's shape, laid over the copy's output
+      view.data = ro.data;
+      view.offset = 0;
+      for (int j = 0; j < nd; j++) view.strides[perm[j]] = ro.strides[j];
+      pl.second.has_out_view = true;
+      pl.second.out_view = view;
+      moves.push_back({e, r});
+    }
+    for (auto &mv : moves) {
+      Plan p = std::move(plans.at(mv.first));
+      plans.erase(mv.first);
+      p.interior.push_back(mv.first);
+      for (DEntry *inner : p.interior) inner->fused_into = mv.second;
+      plans.emplace(mv.second, std::move(p));
+    }
+  }
   // A scalar fill, or a causal mask taken as a flag, that only one fused run reads belongs to that
   // run: it is written only if the run is (when it is declined, or postponed and looked at later).
   std::unordered_map<DEntry *, DEntry *> home;  // entry -> the anchor of its run
@@ -784,6 +855,19 @@ int flush_locked(nxh_context *ctx, Window *w) {
     const Plan &pl = plans.at(anchor);
     if (e->kind == D_COMPARE && !(pl.stat == NXH_DEFER_ATTENTION && pl.causal_flag)) continue;
     home[e] = anchor;
+  }
+  // an upload that only such entries read (the aranges of a causal mask) goes with them
+  for (size_t i = entries.size(); i-- > 0;) {
+    DEntry *e = entries[i].get();
+    if (e->kind != D_UPLOAD || e->readers.empty() || (e->alive && !w->may_postpone)) continue;
+    DEntry *anchor = nullptr;
+    bool single = true;
+    for (DEntry *r : e->readers) {
+      auto h = home.find(r);
+      single = single && h != home.end() && (!anchor || anchor == h->second);
+      if (h != home.end()) anchor = h->second;
+    }
+    if (single && anchor) home[e] = anchor;
   }
   auto members_of = [&](DEntry *anchor) {
     std::vector<DEntry *> run = plans.at(anchor).interior;
@@ -877,8 +961,8 @@ int flush_locked(nxh_context *ctx, Window *w) {
         continue;
       }
     }
-    if (e->kind == D_FULL) {
-      // filled only if a handle is left (or, in issue(), when a reader outside a fused run is issued)
+    if (e->kind == D_FULL || e->kind == D_UPLOAD) {
+      // filled / sent only if a handle is left (or, in issue(), when a reader outside a fused run is issued)
       if (e->alive) rc = issue(ctx, e);
       continue;
     }
@@ -942,7 +1026,7 @@ int flush_locked(nxh_context *ctx, Window *w) {
       continue;
     }
     // cut loose from entries that are about to go away; its operands' blocks stay pinned
-    for (int i = 0; i < 3; i++) e->prod[i] = nullptr;
+    for (int i = 0; i < 3; i++) e->prod[i] = e->upl[i] = nullptr;
     e->readers.clear();
     e->fused_into = nullptr;
     w->postponed_out[e->out.data] = k->second;
@@ -1091,7 +1175,7 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
     e->in[k] = *ins[k];
     auto it = w->producer.find(ins[k]->data);
     if (it != w->producer.end()) {
-      e->prod[k] = it->second;
+      (it->second->kind == D_UPLOAD ? e->upl[k] : e->prod[k]) = it->second;
       it->second->readers.push_back(e.get());
     }
     w->pinned[ins[k]->data]++;
@@ -1102,7 +1186,7 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
   w->producer[out->data] = e.get();
   w->entries.push_back(std::move(e));
   w->stats[NXH_DEFER_RECORDED]++;
-  if (w->entries.size() >= LIMIT) return flush_locked(ctx, w);
+  if (w->entries.size() >= LIMIT || (kind == D_COPY && w->entries.size() >= COPY_FLUSH)) return flush_locked(ctx, w);
   return NXH_OK;
 }
 
@@ -1130,26 +1214,54 @@ bool nxh_defer_free(nxh_context *ctx, void *p) {
   return false;
 }
 
-// nxh_memcpy_h2d: the record runs first if it touches the block, and so does whatever is
-// postponed; a small upload is remembered (the aranges of a causal mask are recognised from it).
-int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
+// nxh_memcpy_h2d. With the mode on, a small upload into a whole block that nothing recorded touches
+// waits in the record with its bytes (*recorded = true: the caller copies nothing): the aranges
+// behind a causal mask that is taken as a flag are then never sent at all. Otherwise the record
+// runs first if it touches the block, and so does whatever is postponed. What a small upload
+// holds is remembered either way (the aranges of a causal mask are recognised from it).
+int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes, bool *recorded) {
+  *recorded = false;
   if (tls_in_flush) return NXH_OK;
   Window *w = window_of(ctx, false);
   if (!w) return NXH_OK;
   std::lock_guard<std::mutex> g(w->mu);
   int rc = NXH_OK;
-  if (w->pinned.count(dst)) {
+  const bool pinned = w->pinned.count(dst) != 0;
+  if (pinned) {
     rc = flush_locked(ctx, w);
     if (!rc) rc = settle_write(ctx, w, dst);
   }
   w->known.erase(dst);
-  if (w->on && bytes > 0 && bytes <= 65536 && bytes % 4 == 0) {
+  if (rc || !w->on || bytes == 0 || bytes > UPLOAD_LIMIT) return rc;
+  if (bytes % 4 == 0) {
     Known &k = w->known[dst];
     k.dtype = NXH_I32;
     k.host_i32.resize(bytes / 4);
     memcpy(k.host_i32.data(), src, bytes);
   }
-  return rc;
+  bool whole = false;
+  {
+    std::lock_guard<std::mutex> a(ctx->mu);
+    auto live = ctx->live.find(dst);
+    whole = live != ctx->live.end() && live->second >= bytes;
+  }
+  if (!whole || w->pinned.count(dst)) return NXH_OK;
+  auto e = std::make_unique<DEntry>();
+  e->kind = D_UPLOAD;
+  e->id = w->entries.size();
+  e->out.data = dst;
+  e->out.dtype = NXH_U8;
+  e->out.ndim = 1;
+  e->out.shape[0] = (int64_t)bytes;
+  e->out.strides[0] = 1;
+  e->payload.assign((const unsigned char *)src, (const unsigned char *)src + bytes);
+  w->pinned[dst]++;
+  w->producer[dst] = e.get();
+  w->entries.push_back(std::move(e));
+  w->stats[NXH_DEFER_RECORDED]++;
+  *recorded = true;
+  if (w->entries.size() >= LIMIT) return flush_locked(ctx, w);
+  return NXH_OK;
 }
 
 void nxh_defer_context_gone(nxh_context *ctx) {

@@ -128,7 +128,11 @@ struct alignas(16) B16x {
 static int copy_impl(nxh_context *ctx, const char *op, const nxh_tensor *out, const nxh_tensor *x);
 
 NXH_EXPORT int nxh_copy(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x) {
-  NXH_DEFER_TOUCH(ctx, 1, out, x);
+  if (out && x && !nxh_is_packed(out->dtype) && !nxh_is_packed(x->dtype)) {
+    NXH_DEFER_RECORD(ctx, NXH_D_COPY, 0, out, 1, nullptr, 0, nullptr, x);
+  } else {
+    NXH_DEFER_TOUCH(ctx, 1, out, x);
+  }
   NXH_CHECK_ARGS("copy", out, x);
   return copy_impl(ctx, "copy", out, x);
 }

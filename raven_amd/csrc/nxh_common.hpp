@@ -110,9 +110,9 @@ int nxh_defer_host_read(nxh_context *ctx, const void *src);
 int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, const nxh_tensor *const *ins, int nin,
                      const int32_t *axes, int n_axes, const void *value);
 bool nxh_defer_free(nxh_context *ctx, void *p);
-int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes);
+int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t bytes, bool *recorded);
 void nxh_defer_context_gone(nxh_context *ctx);
-enum { NXH_D_UNARY, NXH_D_BINARY, NXH_D_COMPARE, NXH_D_WHERE, NXH_D_CAST, NXH_D_REDUCE, NXH_D_MATMUL, NXH_D_FULL };
+enum { NXH_D_UNARY, NXH_D_BINARY, NXH_D_COMPARE, NXH_D_WHERE, NXH_D_CAST, NXH_D_REDUCE, NXH_D_MATMUL, NXH_D_FULL, NXH_D_COPY, NXH_D_UPLOAD };
 // Entry points that are not recorded run the record first. BARRIER also writes everything
 // that was postponed; TOUCH (the first n_out tensors are written, the others read; NULL entries
 // are skipped) only what those blocks need; QUIET nothing.

@@ -283,7 +283,9 @@ NXH_EXPORT int nxh_memory_stats(nxh_context *ctx, uint64_t *in_use, uint64_t *ca
 NXH_EXPORT int nxh_memcpy_h2d(nxh_context *ctx, void *dst, const void *src, size_t bytes) {
   if (!ctx) return nxh_fail(NXH_INVALID_ARGUMENT, "from_host", "null context");
   if (bytes == 0) return NXH_OK;
-  if (int drc = nxh_defer_uploaded(ctx, dst, src, bytes)) return drc;
+  bool recorded = false;  // deferred mode: a small upload waits in the record with its bytes
+  if (int drc = nxh_defer_uploaded(ctx, dst, src, bytes, &recorded)) return drc;
+  if (recorded) return NXH_OK;
   std::lock_guard<std::mutex> g(ctx->mu);
   NXH_HIP("from_host", hipSetDevice(ctx->device));
   if (ctx->capture) {

@@ -389,3 +389,52 @@ def test_linear_layers_over_one_input_share_a_launch(hip, oracle):
     assert s["grouped"] == 0 and s["linear"] == 2, s
     same_bits(got[0], eager[0], "ungrouped member")
     same_bits(got[2], eager[1], "ungrouped member")
+
+
+def test_small_uploads_wait_in_the_record(hip, oracle):
+    """A host upload of up to 64 KiB is recorded with its bytes. It is sent when something needs
+    it (a recorded reader, an entry point that reads the block, a host read) and in issue order with
+    the other writes of its block; the host array may change right after the call."""
+    nx = Nx(hip)
+    a = np.arange(24, dtype=np.float32).reshape(4, 6)
+    with deferred(hip) as win:
+        t = hip.reshape(hip.from_host(a.reshape(-1), dt.float32), a.shape)
+        src = a.copy()
+        a[:] = -1.0  # the caller's buffer is free again
+        doubled = nx.add(t, t)            # a recorded reader
+        gathered = hip.gather(t, hip.reshape(hip.from_host(np.array([3, 0], np.int32), dt.int32), (2, 1)), 0)  # an entry point
+        s = win.delta()
+        assert s["recorded"] >= 3
+        assert np.array_equal(logical(doubled), 2 * src)
+        assert np.array_equal(logical(gathered)[:, 0], src[[3, 0], 0])
+        assert np.array_equal(logical(t), src)
+        # a second upload into the same block comes after the first
+        hip._check(hip._lib.nxh_memcpy_h2d(hip._h, t.buffer.ptr, (src + 100).ctypes.data, src.nbytes))
+        assert np.array_equal(logical(t), src + 100)
+
+
+def test_attention_writes_the_merged_heads_directly(hip, oracle):
+    """attention.ml:218-265: contiguous (swapaxes 1 2 (attention ...)). The copy is recorded; as the
+    attention result's only reader it becomes the end of the run, and the kernel writes through the
+    copy's output with permuted strides: no copy kernel, same bits."""
+    rng = np.random.default_rng(40)
+    d = dt.bfloat16
+    b, h, s, hd = 2, 3, 80, 64
+    nx = Nx(hip)
+    model = Gpt2(nx, Config())
+    q, k, v = (tensor(hip, encode(rng.standard_normal((b, h, s, hd)), d, oracle), d) for _ in range(3))
+
+    def merged():
+        idx = nx.arange(dt.int32, 0, s, 1)
+        mask = nx.less_equal(nx.reshape((1, s), idx), nx.reshape((s, 1), idx))
+        a = model.scaled_dot_product_attention(q, k, v, mask)
+        return nx.reshape((b, s, h * hd), nx.contiguous(nx.swapaxes(1, 2, a)))
+
+    direct = logical(hip.contiguous(hip.permute(hip.attention(q, k, v, 1.0 / math.sqrt(hd), masked_value=float("-inf"), causal=True),
+                                                (0, 2, 1, 3)))).reshape(b, s, h * hd)
+    with deferred(hip) as win:
+        got = logical(merged())
+        st = win.delta()
+    assert (st["attention"], st["issued"], st["fallbacks"]) == (1, 0, 0), st   # the copy was not issued
+    assert hip.last_path() == "attention_fused"
+    same_bits(got, direct, "attention into the merged layout against attention followed by the copy")
