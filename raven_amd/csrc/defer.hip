@@ -1152,9 +1152,11 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
     if (int rc = settle_read(ctx, w, ins[k]->data)) return rc;
   // The output must be a whole block of this context that no recorded entry touches yet:
   // results are fresh allocations (backend_intf.ml:61-67); anything else runs now.
+  bool capturing = false;
   if (ok) {
     std::lock_guard<std::mutex> a(ctx->mu);
     ok = ctx->live.count(out->data) != 0;
+    capturing = ctx->capture != nullptr;
   }
   ok = ok && out->offset == 0 && c_contiguous(*out) && !w->pinned.count(out->data);
   if (ok && kind == D_FULL) ok = numel(*out) == 1 && !nxh_is_packed(out->dtype);
@@ -1186,7 +1188,8 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
   w->producer[out->data] = e.get();
   w->entries.push_back(std::move(e));
   w->stats[NXH_DEFER_RECORDED]++;
-  if (w->entries.size() >= LIMIT || (kind == D_COPY && w->entries.size() >= COPY_FLUSH)) return flush_locked(ctx, w);
+  // (while a graph is captured nothing executes anyway: the record stays whole)
+  if (w->entries.size() >= LIMIT || (kind == D_COPY && !capturing && w->entries.size() >= COPY_FLUSH)) return flush_locked(ctx, w);
   return NXH_OK;
 }
 

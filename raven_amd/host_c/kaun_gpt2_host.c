@@ -311,9 +311,17 @@ static timing time_forwards(const params *p, nxh_tensor ids, int deferred, int l
 static timing time_replays(const params *p, nxh_tensor ids, int iters) {
   must(L.set_deferred(ctx, 1), "set_deferred");
   nxh_graph *graph = NULL;
+  uint64_t s0[NXH_DEFER_STAT_COUNT], s1[NXH_DEFER_STAT_COUNT];
+  must(L.deferred_stats(ctx, s0, NXH_DEFER_STAT_COUNT), "deferred_stats");
   must(L.capture_begin(ctx), "capture_begin");
   val out = logits(p, ids);
   must(L.capture_end(ctx, &graph), "capture_end");
+  must(L.deferred_stats(ctx, s1, NXH_DEFER_STAT_COUNT), "deferred_stats");
+  if (getenv("NXHOST_VERBOSE")) {
+    fprintf(stderr, "captured:");
+    for (int i = 0; i < NXH_DEFER_STAT_COUNT; i++) fprintf(stderr, " %llu", (unsigned long long)(s1[i] - s0[i]));
+    fprintf(stderr, "\n");
+  }
   timing t = {0, 0};
   for (int i = -2; i < iters; i++) {
     must(L.synchronize(ctx), "synchronize");
