@@ -557,6 +557,64 @@ __global__ __launch_bounds__(64 * SM8_WAVES) void gemm_skinny_mfma_k8_kernel(Ski
   }
 }
 
+// ── gemm_skinny_f32_k8: float32, N alone fills the chip ──────────────────────
+// The matrix pipe straight from registers, no LDS on the way: a lane loads 16 bytes of one row
+// of B (k = k0 + lane / 16, columns 4 (lane % 16) .. + 3) and feeds the four values to four
+// v_mfma_f32_16x16x4_f32 (true float32), whose B operand wants exactly one value of row
+// lane / 16 per lane; that MFMA j then holds columns 4 l + j instead of l is undone at the
+// store. The A operand of the same instructions is A[lane % 16][k], one 4-byte load from L2
+// (rows >= M read as zero). A wave so covers 64 columns by 4 k-rows per load instruction,
+// 256 contiguous bytes per row; the eight waves of a block split K and fold through LDS.
+constexpr int SF_U = 8;  // steps (of 4 k-rows) in flight per wave
+__global__ __launch_bounds__(64 * SM8_WAVES) void gemm_skinny_f32_k8_kernel(SkinnyArgs a) {
+  typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+  __shared__ float red[SM8_WAVES * 16 * 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kg = lane >> 4, l = lane & 15;
+  const int64_t n0 = (int64_t)blockIdx.x * 64;
+  const int64_t k0 = (int64_t)wave * a.kchunk;
+  const int64_t k1 = k0 + a.kchunk < a.K ? k0 + a.kchunk : a.K;
+  const float *A = (const float *)a.A;
+  const float *B = (const float *)a.B;
+  const bool col_ok = n0 + 4 * l < a.N;  // N is a multiple of 4: vectors are whole or absent
+  const bool row_ok = l < a.M;
+  const float *bp = B + n0 + 4 * l;
+  const float *ap = A + (int64_t)l * a.ars;
+  f32x4_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) acc[j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int64_t kb = k0; kb < k1; kb += 4 * SF_U) {
+    f32x4_t b[SF_U];
+    float av[SF_U];
+#pragma unroll
+    for (int u = 0; u < SF_U; u++) {
+      const int64_t k = kb + 4 * u + kg;
+      const bool in = k < k1;
+      b[u] = (in && col_ok) ? *reinterpret_cast<const f32x4_t *>(bp + k * a.brs) : f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+      av[u] = (in && row_ok) ? ap[k * a.acs] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < SF_U; u++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u], b[u][j], acc[j], 0, 0, 0);
+  }
+  // accumulator element e of MFMA j is C[4 kg + e][column 4 l + j] of the wave's partial tile
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int e = 0; e < 4; e++) red[(wave * 16 + 4 * kg + e) * 64 + 4 * l + j] = acc[j][e];
+  __syncthreads();
+  for (int o = threadIdx.x; o < 16 * 64; o += 64 * SM8_WAVES) {
+    const int m = o >> 6, c = o & 63;
+    const int64_t n = n0 + c;
+    if (m >= a.M || n >= a.N) continue;
+    float sum = red[o];
+#pragma unroll
+    for (int w = 1; w < SM8_WAVES; w++) sum += red[w * 16 * 64 + o];  // wave order: the bits repeat
+    ((float *)a.C)[m * a.crs + n * a.ccs] = sum;
+  }
+}
+
 // Sums the [nsplit][m * n] partials in split order, four outputs per lane.
 template <int DT>
 __global__ __launch_bounds__(256) void skinny_finish_kernel(const float *P, void *Cv, int64_t M, int64_t N,
@@ -658,6 +716,20 @@ static int launch_skinny(nxh_context *ctx, GemmArgs &g) {
   a.crs = g.crs;
   a.ccs = g.ccs;
   const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  if constexpr (DT == NXH_F32) {
+    // N alone fills the chip with 64-column blocks: K is split inside the block, one launch
+    const int64_t strips = (g.N + 63) / 64;
+    if (strips >= cus && strips <= 0x7fffffffLL && g.N % 4 == 0 && g.brs % 4 == 0 && ((uintptr_t)g.B % 16) == 0 &&
+        g.K >= 4 * SF_U * SM8_WAVES) {
+      a.kchunk = ((g.K + SM8_WAVES - 1) / SM8_WAVES + 3) / 4 * 4;
+      a.nsplit = 1;
+      a.C = g.C;
+      nxh_set_path("gemm_skinny_f32_k8");
+      hipLaunchKernelGGL(gemm_skinny_f32_k8_kernel, dim3((unsigned)strips), dim3(64 * SM8_WAVES), 0, ctx->stream, a);
+      NXH_HIP("matmul", hipGetLastError());
+      return NXH_OK;
+    }
+  }
   const int mmax = g.M <= 8 ? 8 : 16;
   const int64_t col_blocks = (g.N + SK_LANES * VN - 1) / (SK_LANES * VN);
   // two blocks per CU keep enough loads in flight; more splits only add partials

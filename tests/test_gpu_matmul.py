@@ -193,6 +193,27 @@ def test_matmul_skinny_wide_output(hip, oracle, d, m, k, n):
     assert np.array_equal(logical(hip.matmul(ha, hb)), logical(hip.matmul(ha, hb)))
 
 
+@pytest.mark.parametrize("m,k,n", [(8, 1024, 16384), (1, 515, 16388), (16, 4096, 16384), (13, 770, 17000)],
+                         ids=lambda v: str(v))
+def test_matmul_skinny_wide_output_f32(hip, oracle, m, k, n):
+    """The float32 form: B rows go from registers straight into v_mfma_f32_16x16x4_f32, the eight
+    waves of a block split K. Ragged K (not a multiple of the 4-row steps), N ending inside a
+    block's 64 columns, a transposed A (its elements are read one by one)."""
+    rng = np.random.default_rng(m + k + n)
+    d = dt.float32
+    a = encode(rng.standard_normal((m, k)) * 0.5, d, oracle)
+    b = encode(rng.standard_normal((k, n)) * 0.5, d, oracle)
+    ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
+    check(hip, oracle, d, ha, hb, a, b, f"skinny wide f32 m={m} k={k} n={n}")
+    assert hip.last_path() == "gemm_skinny_f32_k8"
+    assert np.array_equal(logical(hip.matmul(ha, hb)), logical(hip.matmul(ha, hb)))
+    at = np.ascontiguousarray(a.T)
+    hat = pair(at, d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))[0]
+    same = logical(hip.matmul(hat, hb))
+    assert hip.last_path() == "gemm_skinny_f32_k8"
+    assert np.array_equal(same, logical(hip.matmul(ha, hb)))
+
+
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16, dt.float32], ids=lambda d: d.name)
 def test_matmul_big_tile_kernel(hip, oracle, d):
     """The LDS-tiled kernel family: every block shape, whole and ragged tiles,
