@@ -88,12 +88,19 @@ __device__ __forceinline__ int64_t row_offsets(const RowGeom &g, int64_t row, co
   int64_t oa = 0;
   ob = 0;
   oc = 0;
+  // rows fit 32 bits (checked on the host) and the host has merged the outer dims that compose, so
+  // the usual case is one dim and no division; the rest are 32-bit divisions, not 64-bit ones
+  uint32_t r = (uint32_t)row;
   for (int d = g.nouter - 1; d >= 0; d--) {
-    const int64_t i = row % g.oshape[d];
-    row /= g.oshape[d];
-    oa += i * a.stride[d];
-    ob += i * b.stride[d];
-    oc += i * c.stride[d];
+    uint32_t i = r;
+    if (d > 0) {
+      const uint32_t q = r / g.oshape[d];
+      i = r - q * g.oshape[d];
+      r = q;
+    }
+    oa += (int64_t)i * a.stride[d];
+    ob += (int64_t)i * b.stride[d];
+    oc += (int64_t)i * c.stride[d];
   }
   return oa;
 }
@@ -350,6 +357,24 @@ void row_operand(const nxh_tensor *t, RowOperand &o) {
   o.base = t ? (const char *)t->data + t->offset * (int64_t)nxh_elem_size(t->dtype) : nullptr;
   for (int d = 0; d < ROW_MAXD; d++) o.stride[d] = (t && d < t->ndim - 1) ? t->strides[d] : 0;
 }
+// Outer dims that compose on every operand (stride[d - 1] == stride[d] * extent[d], a broadcast
+// with both strides 0 included) become one: contiguous rows end up with a single outer dim.
+void merge_outer_dims(RowGeom &g, std::initializer_list<RowOperand *> ops) {
+  int n = g.nouter;
+  for (int d = n - 1; d > 0; d--) {
+    bool composes = true;
+    for (RowOperand *o : ops) composes = composes && o->stride[d - 1] == o->stride[d] * (int64_t)g.oshape[d];
+    if (!composes || (uint64_t)g.oshape[d - 1] * g.oshape[d] > 0xffffffffULL) continue;
+    g.oshape[d - 1] *= g.oshape[d];
+    for (RowOperand *o : ops) o->stride[d - 1] = o->stride[d];
+    for (int e = d; e + 1 < n; e++) {
+      g.oshape[e] = g.oshape[e + 1];
+      for (RowOperand *o : ops) o->stride[e] = o->stride[e + 1];
+    }
+    n--;
+  }
+  g.nouter = n;
+}
 // A row operand can be moved V elements at a time when its rows are contiguous
 // and every row starts on a V-element boundary.
 bool rows_vector_ok(const nxh_tensor *t, int v) {
@@ -426,6 +451,7 @@ NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const n
   row_operand(x, a.x);
   row_operand(out, a.out);
   row_operand(mask, a.mask);
+  merge_outer_dims(a.g, {&a.x, &a.out, &a.mask});
   a.has_scale = scale != nullptr;
   a.has_mask = mask != nullptr;
   a.mask_last = mask ? mask->strides[nd - 1] : 0;
@@ -476,6 +502,7 @@ NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, cons
   row_operand(x, a.x);
   row_operand(out, a.out);
   row_operand(nullptr, a.unused);
+  merge_outer_dims(a.g, {&a.x, &a.out, &a.unused});
   const int es = (int)nxh_elem_size(dx);
   a.gamma = gamma ? (const char *)gamma->data + gamma->offset * es : nullptr;
   a.beta = beta ? (const char *)beta->data + beta->offset * es : nullptr;
