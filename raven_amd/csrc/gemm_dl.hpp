@@ -15,6 +15,9 @@
 //     row are XOR-ed with bits of the row number, those of a row-contiguous k-row with
 //     bits of k. Fragment reads apply the same XOR and touch every bank once per
 //     half-wave (ds_read_b128 for k-contiguous tiles, ds_read_b64_tr_b16 otherwise).
+//   * Eight waves as 2 x 4, each 128 x 64 outputs: the wide side is A, whose k-contiguous
+//     fragments come with ds_read_b128 (about 180 B/clk/CU measured), the narrow side B,
+//     whose row-contiguous tile needs the slower transposing read (about 111 B/clk).
 //   * v_mfma_f32_16x16x32 instead of 32x32x16: the same LDS bytes and MFMA cycles per
 //     flop, but a quarter of the accumulator registers rewritten per instruction.
 //     Under the board's power limit (random N(0, 0.02) operands pull this chip from
@@ -35,9 +38,11 @@ constexpr int UPR = BK / 8;                       // 16-byte units per row of a 
 constexpr int UNITS = 256 * UPR;                  // units per operand and slab
 constexpr int LOADS = UNITS / 64 / 8;             // load instructions per wave, operand and slab
 constexpr int OP_BYTES = UNITS * 16, STAGE_BYTES = 2 * OP_BYTES;
-constexpr int PATCH_PITCH = 128 + 8;              // epilogue: a wave's 64 x 128 patch, padded rows (elements)
-constexpr size_t LDS_BYTES = (size_t)8 * 64 * PATCH_PITCH * 2 > (size_t)NS * STAGE_BYTES ? (size_t)8 * 64 * PATCH_PITCH * 2
-                                                                                           : (size_t)NS * STAGE_BYTES;
+constexpr int WM = 128, WN = 64;                   // a wave's outputs: 2 x 4 waves
+constexpr int FA = WM / 16, FB = WN / 16;          // 16-row fragments of A, 16-column fragments of B per wave
+constexpr int PATCH_PITCH = WN + 8;                // epilogue: a wave's 128 x 64 patch, padded rows (elements)
+constexpr size_t PATCH_BYTES = (size_t)8 * WM * PATCH_PITCH * 2;
+constexpr size_t LDS_BYTES = PATCH_BYTES > (size_t)NS * STAGE_BYTES ? PATCH_BYTES : (size_t)NS * STAGE_BYTES;
 
 template <int N>
 __device__ __forceinline__ void wait_loads_and_meet() {
@@ -80,7 +85,7 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
   const int64_t stepB = B_KC ? BK : (int64_t)BK * a.ldb;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 128;  // 4 x 2 waves of 64 x 128 outputs
+  const int wm = (wave >> 2) * WM, wn = (wave & 3) * WN;  // 2 x 4 waves of 128 x 64 outputs
 
   // Byte offset, from the slab's origin in global memory, of the 16 bytes this lane
   // fetches with its i-th load: that load fills units [64 j, 64 j + 64), j = wave * LOADS + i.
@@ -134,11 +139,11 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
     return V16{l2[0], l2[1], h2[0], h2[1]};
   };
 
-  f32x4 acc[4][8];
+  f32x4 acc[FA][FB];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < FA; i++)
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (int j = 0; j < FB; j++)
 #pragma unroll
       for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
 
@@ -149,50 +154,51 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
   if (nt >= NS) wait_loads_and_meet<(NS - 1) * 2 * LOADS>();
   else wait_loads_and_meet<0>();
 
-  // A step is 16 MFMAs: the four 16-row fragments of A against four 16-column fragments of B
-  // (one half of the wave's 128 columns) over 32 k-values; a slab is four steps. The reads of
-  // step s + 1 are issued in front of the MFMAs of step s.
-  V16 fa[2][4], fb[2][4];
-  auto load_step = [&](int buf, int st) {
+  // A step is 32 MFMAs: the eight 16-row fragments of A against the four 16-column fragments
+  // of B over 32 k-values; a slab is two steps. The reads of step s + 1 are issued among the
+  // MFMAs of step s, one behind each MFMA (scheduling groups below): a wave then never queues
+  // its sixteen LDS reads in one burst in front of a cold MFMA pipe, which is worth 3-5 % here.
+  V16 fa[2][FA], fb[2][FB];
+  auto load_step = [&](int buf, int k32) {
     const unsigned char *sa = smem_raw + buf * STAGE_BYTES, *sb = sa + OP_BYTES;
-    const int k32 = st >> 1, half = st & 1;
-    if (half == 0) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) fa[k32 & 1][i] = frag(sa, A_KC, wm + i * 16, k32);
-    }
+    for (int i = 0; i < FA; i++) fa[k32][i] = frag(sa, A_KC, wm + i * 16, k32);
 #pragma unroll
-    for (int j = 0; j < 4; j++) fb[st & 1][j] = frag(sb, B_KC, wn + (half * 4 + j) * 16, k32);
+    for (int j = 0; j < FB; j++) fb[k32][j] = frag(sb, B_KC, wn + j * 16, k32);
   };
   load_step(0, 0);
   int buf = 0;
   // In a slab's last step: wait for this wave's share of the next slab, meet the other waves
   // (now the next slab is complete and nobody reads this one any more), request slab t + NS
-  // into this slab's buffer, fetch the next slab's first fragments, then issue the last MFMAs.
+  // into this slab's buffer, fetch the next slab's first fragments among the last MFMAs.
   auto slab = [&](int t, auto fetch_c, auto last_c) {
     constexpr bool FETCH = decltype(fetch_c)::value, LAST = decltype(last_c)::value;
     const int nbuf = buf + 1 == NS ? 0 : buf + 1;
 #pragma unroll
-    for (int st = 0; st < 4; st++) {
-      if (st + 1 < 4) {
-        load_step(buf, st + 1);
+    for (int k32 = 0; k32 < 2; k32++) {
+      if (k32 == 0) {
+        load_step(buf, 1);
       } else if constexpr (!LAST) {
         if constexpr (FETCH) wait_loads_and_meet<(NS - 2) * 2 * LOADS>();
         else wait_loads_and_meet<0>();
         if constexpr (FETCH) issue(t + NS, buf);
         load_step(nbuf, 0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      const int k32 = st >> 1, half = st & 1;
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+      for (int i = 0; i < FA; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-          f32x4 &c = acc[i][half * 4 + j];
+        for (int j = 0; j < FB; j++) {
+          f32x4 &c = acc[i][j];
           if constexpr (EL::BF16)
-            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fa[k32 & 1][i]), __builtin_bit_cast(bf16x8, fb[st & 1][j]), c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, fa[k32][i]), __builtin_bit_cast(bf16x8, fb[k32][j]), c, 0, 0, 0);
           else
-            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fa[k32 & 1][i]), __builtin_bit_cast(f16x8, fb[st & 1][j]), c, 0, 0, 0);
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, fa[k32][i]), __builtin_bit_cast(f16x8, fb[k32][j]), c, 0, 0, 0);
         }
+#pragma unroll
+      for (int x = 0; x < FA * FB; x++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     buf = nbuf;
@@ -205,21 +211,22 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
   slab(t, no{}, yes{});
 
   // Epilogue: element e of accumulator (i, j) is C[16 i + 4 g + e][16 j + q]. Each wave parks its
-  // rounded 64 x 128 patch in LDS and sends it out as whole 16-byte row segments.
+  // rounded 128 x 64 patch in LDS and sends it out as whole 16-byte row segments.
   S *C = (S *)a.C + co;
   auto narrow = [](float x) -> S { return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x); };
   wait_loads_and_meet<0>();  // every wave has read its last fragments; no load is in flight
-  S *patch = reinterpret_cast<S *>(smem_raw) + wave * (64 * PATCH_PITCH);
+  S *patch = reinterpret_cast<S *>(smem_raw) + wave * (WM * PATCH_PITCH);
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < FA; i++)
 #pragma unroll
-    for (int j = 0; j < 8; j++)
+    for (int j = 0; j < FB; j++)
 #pragma unroll
       for (int e = 0; e < 4; e++) patch[(i * 16 + g16 * 4 + e) * PATCH_PITCH + j * 16 + q16] = narrow(acc[i][j][e]);
   // the patch is read back by lanes of the same wave only: LDS serves a wave in order
+  constexpr int CPR = WN / 8;  // 16-byte pieces per patch row
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const int ch = i * 64 + lane, row = ch >> 4, col = (ch & 15) * 8;
+  for (int i = 0; i < WM * CPR / 64; i++) {
+    const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
     const V16 v = *reinterpret_cast<const V16 *>(patch + row * PATCH_PITCH + col);
     *reinterpret_cast<V16 *>(C + (m0 + wm + row) * a.ldc + n0 + wn + col) = v;
   }
