@@ -1,12 +1,17 @@
-// gemm_dl.hpp — the large-product form of the 16-bit tiled GEMM: 256 x 256 outputs per
-// block, operands fetched from global memory straight into LDS, v_mfma_f32_16x16x32.
-//
+// gemm_dl.hpp — the 16-bit tiled GEMM with operands fetched from global memory straight
+// into LDS, v_mfma_f32_16x16x32, eight waves per block. Two block shapes:
+//   256 x 256  2 x 4 waves of 128 x 64   large products
+//   128 x 192  2 x 4 waves of  64 x 48   products of a few hundred 128-row tiles: with
+//                                        N = 768 (GPT-2's linears) [8192, 768] is exactly
+//                                        256 blocks, one per compute unit, and N = 2304 or
+//                                        3072 whole multiples of that
 // Same contract as gemm_tile.hpp (f32 accumulation, one rounding per output element,
-// batched with broadcastable batch dims), for whole tiles only: M and N multiples of
-// 256, K a multiple of 64. What differs from gemm_tile's 256 x 256 shape:
-//   * No register staging. A slab (64 k-values of 256 rows per operand, 64 KiB) is
+// batched with broadcastable batch dims, the fused linear's epilogue and grouped launch),
+// for whole tiles only: M and N multiples of the block, K a multiple of 64. What differs
+// from gemm_tile:
+//   * No register staging. A slab (64 k-values of every row of both operands) is
 //     requested with global_load_lds_dwordx4: each of the 64 lanes of a load delivers
-//     16 bytes to consecutive LDS addresses, so 40 vector registers and every
+//     16 bytes to consecutive LDS addresses, so the staging registers and every
 //     ds_write of the staged form disappear. LDS holds a ring of two slabs; the loads
 //     of slab t + 2 are issued as soon as every wave has read its last fragments of
 //     slab t, behind the block's one barrier per slab.
@@ -15,9 +20,9 @@
 //     row are XOR-ed with bits of the row number, those of a row-contiguous k-row with
 //     bits of k. Fragment reads apply the same XOR and touch every bank once per
 //     half-wave (ds_read_b128 for k-contiguous tiles, ds_read_b64_tr_b16 otherwise).
-//   * Eight waves as 2 x 4, each 128 x 64 outputs: the wide side is A, whose k-contiguous
-//     fragments come with ds_read_b128 (about 180 B/clk/CU measured), the narrow side B,
-//     whose row-contiguous tile needs the slower transposing read (about 111 B/clk).
+//   * The wide side of a wave's outputs is A, whose k-contiguous fragments come with
+//     ds_read_b128 (about 180 B/clk/CU measured), the narrow side B, whose
+//     row-contiguous tile needs the slower transposing read (about 111 B/clk).
 //   * v_mfma_f32_16x16x32 instead of 32x32x16: the same LDS bytes and MFMA cycles per
 //     flop, but a quarter of the accumulator registers rewritten per instruction.
 //     Under the board's power limit (random N(0, 0.02) operands pull this chip from
@@ -33,16 +38,23 @@
 namespace gemm_dl {
 using namespace gemm_tile;
 
-constexpr int BM = 256, BN = 256, BK = 64, NS = 2, THREADS = 512;
-constexpr int UPR = BK / 8;                       // 16-byte units per row of a k-contiguous tile
-constexpr int UNITS = 256 * UPR;                  // units per operand and slab
-constexpr int LOADS = UNITS / 64 / 8;             // load instructions per wave, operand and slab
-constexpr int OP_BYTES = UNITS * 16, STAGE_BYTES = 2 * OP_BYTES;
-constexpr int WM = 128, WN = 64;                   // a wave's outputs: 2 x 4 waves
-constexpr int FA = WM / 16, FB = WN / 16;          // 16-row fragments of A, 16-column fragments of B per wave
-constexpr int PATCH_PITCH = WN + 8;                // epilogue: a wave's 128 x 64 patch, padded rows (elements)
-constexpr size_t PATCH_BYTES = (size_t)8 * WM * PATCH_PITCH * 2;
-constexpr size_t LDS_BYTES = PATCH_BYTES > (size_t)NS * STAGE_BYTES ? PATCH_BYTES : (size_t)NS * STAGE_BYTES;
+constexpr int BK = 64, NS = 2;
+constexpr int UPR = BK / 8;  // 16-byte units per row of a k-contiguous tile
+
+template <int BM_, int BN_>
+struct Shape {
+  static constexpr int BM = BM_, BN = BN_, WVM = 2, WVN = 4, WAVES = WVM * WVN, THREADS = 64 * WAVES;
+  static constexpr int WM = BM / WVM, WN = BN / WVN;   // a wave's outputs
+  static constexpr int FA = WM / 16, FB = WN / 16;     // 16-row fragments of A, 16-column fragments of B per wave
+  static constexpr int LA = BM / 8 / WAVES, LB = BN / 8 / WAVES, LPW = LA + LB;  // load instructions per wave and slab
+  static_assert(LA * 8 * WAVES == BM && LB * 8 * WAVES == BN && FA * 16 * WVM == BM && FB * 16 * WVN == BN, "shape");
+  static constexpr int A_BYTES = BM * BK * 2, STAGE_BYTES = (BM + BN) * BK * 2;
+  static constexpr int PATCH_PITCH = WN + 8;           // epilogue: a wave's WM x WN patch, padded rows (elements)
+  static constexpr size_t PATCH_BYTES = (size_t)WAVES * WM * PATCH_PITCH * 2;
+  static constexpr size_t LDS_BYTES = PATCH_BYTES > (size_t)NS * STAGE_BYTES ? PATCH_BYTES : (size_t)NS * STAGE_BYTES;
+};
+using Shape256x256 = Shape<256, 256>;
+using Shape128x192 = Shape<128, 192>;
 
 template <int N>
 __device__ __forceinline__ void wait_loads_and_meet() {
@@ -52,19 +64,42 @@ __device__ __forceinline__ void wait_loads_and_meet() {
 // LDS position (16-byte unit) <-> which data it holds.
 // k-contiguous tile [row][unit kv]: physical unit = kv ^ ((row >> 1) & 7): sixteen consecutive
 // rows reading the same logical unit cover the sixteen 16-byte bank groups once.
-// row-contiguous tile [k][unit nv]: physical unit = nv ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1)):
-// the eight k-rows x two units a half-wave's transposing read touches are all distinct.
+// row-contiguous tile [k][UPK units nv]: physical unit = nv ^ swz_rc(k). A half-wave's
+// transposing read touches two neighbouring units in each of the eight k-rows
+// {0..3, 8..11} (+ 4, + 16): the XOR must send those to eight different 32-byte bank pairs.
+// With a pitch of 256 or 512 bytes every k-row starts at bank 0 and three bits are needed;
+// with 384 bytes (192 columns) odd k-rows already sit 128 bytes further on and two bits,
+// which stay inside the row's groups of eight units, are enough.
 __device__ __forceinline__ int swz_kc(int row) { return (row >> 1) & 7; }
-__device__ __forceinline__ int swz_rc(int k) { return ((k & 3) << 2) | (((k >> 3) & 1) << 1); }
+template <int UPK>
+__device__ __forceinline__ int swz_rc(int k) {
+  if constexpr (UPK % 16 == 0) return ((k & 3) << 2) | (((k >> 3) & 1) << 1);
+  else return (((k >> 1) & 1) | (((k >> 3) & 1) << 1)) << 1;
+}
 
-template <class EL, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(THREADS) void kernel(Args a) {
+template <class EL, bool A_KC, bool B_KC, class SH, bool EPI>
+__global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   using S = typename EL::S;
   static_assert(!EL::F32, "16-bit operands only");
+  constexpr int BM = SH::BM, BN = SH::BN, FA = SH::FA, FB = SH::FB, LA = SH::LA, LB = SH::LB, LPW = SH::LPW;
+  constexpr int STAGE_BYTES = SH::STAGE_BYTES, A_BYTES = SH::A_BYTES;
+  constexpr int UPK_A = BM / 8, UPK_B = BN / 8;  // units per k-row of a row-contiguous tile
+  static_assert(UPK_A % 8 == 0 && UPK_B % 8 == 0, "swizzle groups");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   uint32_t batch, tm, tn;
   tile_of_block(a, gridDim.x - 1 - blockIdx.x, batch, tm, tn);
-  int64_t ao = 0, bo = 0, co = 0;
+  int64_t ao = 0, bo = 0, co = 0, ro = 0;
+  if constexpr (EPI) {
+    if (a.ngroup > 1) {
+      const uint32_t member = tn / a.gtn;
+      tn -= member * a.gtn;
+      if (member) {
+        bo = member == 1 ? a.goff_b[0] : a.goff_b[1];
+        co = member == 1 ? a.goff_c[0] : a.goff_c[1];
+        if (a.bias) a.bias = (const S *)a.bias + (member == 1 ? a.goff_bias[0] : a.goff_bias[1]);
+      }
+    }
+  }
   {
     uint32_t idx = batch;
 #pragma unroll
@@ -75,6 +110,7 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
         ao += (int64_t)c * a.ba[i];
         bo += (int64_t)c * a.bb[i];
         co += (int64_t)c * a.bc[i];
+        if constexpr (EPI) ro += (int64_t)c * a.br[i];
       }
     }
   }
@@ -85,25 +121,26 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
   const int64_t stepB = B_KC ? BK : (int64_t)BK * a.ldb;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = (wave >> 2) * WM, wn = (wave & 3) * WN;  // 2 x 4 waves of 128 x 64 outputs
+  const int wm = (wave / SH::WVN) * SH::WM, wn = (wave % SH::WVN) * SH::WN;
 
   // Byte offset, from the slab's origin in global memory, of the 16 bytes this lane
-  // fetches with its i-th load: that load fills units [64 j, 64 j + 64), j = wave * LOADS + i.
-  uint32_t offA[LOADS], offB[LOADS];
+  // fetches with load j of an operand: that load fills units [64 j, 64 j + 64) of its tile.
+  auto off_kc = [&](int j, int64_t ld) -> uint32_t {
+    const int row = j * (64 / UPR) + lane / UPR, kp = lane % UPR;
+    return (uint32_t)((row * ld + (kp ^ swz_kc(row)) * 8) * 2);
+  };
+  auto off_rc = [&](int j, int64_t ld, auto upk_c) -> uint32_t {
+    constexpr int UPK = decltype(upk_c)::value;
+    const int u = j * 64 + lane, k = u / UPK, p = u % UPK;
+    return (uint32_t)((k * ld + (p ^ swz_rc<UPK>(k)) * 8) * 2);
+  };
+  using upk_a = std::integral_constant<int, UPK_A>;
+  using upk_b = std::integral_constant<int, UPK_B>;
+  uint32_t offA[LA], offB[LB];
 #pragma unroll
-  for (int i = 0; i < LOADS; i++) {
-    const int j = wave * LOADS + i;
-    auto kc = [&](int64_t ld) -> uint32_t {
-      const int row = j * (64 / UPR) + lane / UPR, kp = lane % UPR;
-      return (uint32_t)((row * ld + (kp ^ swz_kc(row)) * 8) * 2);
-    };
-    auto rc = [&](int64_t ld) -> uint32_t {
-      const int k = 2 * j + (lane >> 5), np = lane & 31;
-      return (uint32_t)((k * ld + (np ^ swz_rc(k)) * 8) * 2);
-    };
-    offA[i] = A_KC ? kc(a.lda) : rc(a.lda);
-    offB[i] = B_KC ? kc(a.ldb) : rc(a.ldb);
-  }
+  for (int i = 0; i < LA; i++) offA[i] = A_KC ? off_kc(wave * LA + i, a.lda) : off_rc(wave * LA + i, a.lda, upk_a{});
+#pragma unroll
+  for (int i = 0; i < LB; i++) offB[i] = B_KC ? off_kc(wave * LB + i, a.ldb) : off_rc(wave * LB + i, a.ldb, upk_b{});
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;
   // m0 carries the LDS address of lane 0's 16 bytes. It is not declared as clobbered: the
   // compiler treats it as reserved and writes it itself right in front of each of its own uses.
@@ -112,12 +149,12 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
                  : "memory");
   };
   auto issue = [&](int t, int buf) {
-    const uint32_t sb = lds0 + buf * STAGE_BYTES + wave * (LOADS * 1024);
+    const uint32_t sb = lds0 + buf * STAGE_BYTES;
     const S *pa = gA + (int64_t)t * stepA, *pb = gB + (int64_t)t * stepB;
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) load1(pa, offA[i], sb + i * 1024);
+    for (int i = 0; i < LA; i++) load1(pa, offA[i], sb + (wave * LA + i) * 1024);
 #pragma unroll
-    for (int i = 0; i < LOADS; i++) load1(pb, offB[i], sb + OP_BYTES + i * 1024);
+    for (int i = 0; i < LB; i++) load1(pb, offB[i], sb + A_BYTES + (wave * LB + i) * 1024);
   };
 
   // Fragments of v_mfma_f32_16x16x32: lane 16 g + q holds row (column) q and k = 8 g .. 8 g + 7 of the 32.
@@ -125,15 +162,17 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
   const int kc_sw = (lane >> 1) & 7;  // swz_kc(row0 + q16): row0 is a multiple of 16
   const int kc_row = q16 * (UPR * 16);
   const int rc_k = g16 * 8 + (q16 >> 2);
-  const int rc_sw = (((lane >> 2) & 3) << 2) | ((g16 & 1) << 1);  // swz_rc(32 k32 + rc_k (+4))
-  auto frag = [&](const unsigned char *tile, bool kcont, int row0, int k32) -> V16 {
+  auto frag = [&](const unsigned char *tile, bool kcont, auto upk_c, int row0, int k32) -> V16 {
+    constexpr int UPK = decltype(upk_c)::value;
     if (kcont) return *reinterpret_cast<const V16 *>(tile + row0 * (UPR * 16) + kc_row + (((k32 * 4 + g16) ^ kc_sw) << 4));
     // transposing read (gemm_tile.hpp): lane q of a 16-lane group addresses the 8 bytes at
     // k-row (q >> 2), rows 4 (q & 3) .. + 3; the second read takes the k-rows four further on
+    // (the XOR leaves out bit 2 of k and everything above bit 3: the same for both reads)
+    const int rc_sw = swz_rc<UPK>(rc_k);
     const int r = row0 + (q16 & 3) * 4;
-    const unsigned char *p = tile + (k32 * 32 + rc_k) * 512 + (((r >> 3) ^ rc_sw) << 4) + (r & 7) * 2;
+    const unsigned char *p = tile + (k32 * 32 + rc_k) * (UPK * 16) + (((r >> 3) ^ rc_sw) << 4) + (r & 7) * 2;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * 512));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * (UPK * 16)));
     typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
     const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
     return V16{l2[0], l2[1], h2[0], h2[1]};
@@ -151,20 +190,20 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
 #pragma unroll
   for (int s = 0; s < NS; s++)
     if (s < nt) issue(s, s);
-  if (nt >= NS) wait_loads_and_meet<(NS - 1) * 2 * LOADS>();
+  if (nt >= NS) wait_loads_and_meet<(NS - 1) * LPW>();
   else wait_loads_and_meet<0>();
 
-  // A step is 32 MFMAs: the eight 16-row fragments of A against the four 16-column fragments
+  // A step is FA x FB MFMAs: the wave's 16-row fragments of A against its 16-column fragments
   // of B over 32 k-values; a slab is two steps. The reads of step s + 1 are issued among the
   // MFMAs of step s, one behind each MFMA (scheduling groups below): a wave then never queues
-  // its sixteen LDS reads in one burst in front of a cold MFMA pipe, which is worth 3-5 % here.
+  // all its LDS reads in one burst in front of a cold MFMA pipe, which is worth 3-5 % here.
   V16 fa[2][FA], fb[2][FB];
   auto load_step = [&](int buf, int k32) {
-    const unsigned char *sa = smem_raw + buf * STAGE_BYTES, *sb = sa + OP_BYTES;
+    const unsigned char *sa = smem_raw + buf * STAGE_BYTES, *sb = sa + A_BYTES;
 #pragma unroll
-    for (int i = 0; i < FA; i++) fa[k32][i] = frag(sa, A_KC, wm + i * 16, k32);
+    for (int i = 0; i < FA; i++) fa[k32][i] = frag(sa, A_KC, upk_a{}, wm + i * 16, k32);
 #pragma unroll
-    for (int j = 0; j < FB; j++) fb[k32][j] = frag(sb, B_KC, wn + j * 16, k32);
+    for (int j = 0; j < FB; j++) fb[k32][j] = frag(sb, B_KC, upk_b{}, wn + j * 16, k32);
   };
   load_step(0, 0);
   int buf = 0;
@@ -179,7 +218,7 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
       if (k32 == 0) {
         load_step(buf, 1);
       } else if constexpr (!LAST) {
-        if constexpr (FETCH) wait_loads_and_meet<(NS - 2) * 2 * LOADS>();
+        if constexpr (FETCH) wait_loads_and_meet<(NS - 2) * LPW>();
         else wait_loads_and_meet<0>();
         if constexpr (FETCH) issue(t + NS, buf);
         load_step(nbuf, 0);
@@ -211,24 +250,60 @@ __global__ __launch_bounds__(THREADS) void kernel(Args a) {
   slab(t, no{}, yes{});
 
   // Epilogue: element e of accumulator (i, j) is C[16 i + 4 g + e][16 j + q]. Each wave parks its
-  // rounded 128 x 64 patch in LDS and sends it out as whole 16-byte row segments.
+  // rounded WM x WN patch in LDS and sends it out as whole 16-byte row segments; the fused
+  // linear's bias, residual and GELU are applied to those segments on the way
+  // (gemm_tile.hpp: each step rounded to the dtype).
   S *C = (S *)a.C + co;
   auto narrow = [](float x) -> S { return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x); };
   wait_loads_and_meet<0>();  // every wave has read its last fragments; no load is in flight
-  S *patch = reinterpret_cast<S *>(smem_raw) + wave * (WM * PATCH_PITCH);
+  constexpr int PITCH = SH::PATCH_PITCH;
+  S *patch = reinterpret_cast<S *>(smem_raw) + wave * (SH::WM * PITCH);
 #pragma unroll
   for (int i = 0; i < FA; i++)
 #pragma unroll
     for (int j = 0; j < FB; j++)
 #pragma unroll
-      for (int e = 0; e < 4; e++) patch[(i * 16 + g16 * 4 + e) * PATCH_PITCH + j * 16 + q16] = narrow(acc[i][j][e]);
+      for (int e = 0; e < 4; e++) patch[(i * 16 + g16 * 4 + e) * PITCH + j * 16 + q16] = narrow(acc[i][j][e]);
   // the patch is read back by lanes of the same wave only: LDS serves a wave in order
-  constexpr int CPR = WN / 8;  // 16-byte pieces per patch row
+  constexpr int CPR = SH::WN / 8;             // 16-byte pieces per patch row
+  constexpr int NIT = SH::WM * CPR / 64;      // pieces per lane
+  static_assert(NIT * 64 == SH::WM * CPR, "whole passes");
+  S *ctile = C + (m0 + wm) * a.ldc + n0 + wn;
+  if constexpr (EPI) {
+    // the bias and residual pieces of a group are requested before the first one is used
+    const S *btile = a.bias ? (const S *)a.bias + n0 + wn : nullptr;
+    const S *rtile = a.R ? (const S *)a.R + ro + (m0 + wm) * a.ldr + n0 + wn : nullptr;
+    constexpr int G = NIT <= 8 ? NIT : 4;  // pieces in flight per lane
+    static_assert(NIT % G == 0, "whole groups");
 #pragma unroll
-  for (int i = 0; i < WM * CPR / 64; i++) {
-    const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
-    const V16 v = *reinterpret_cast<const V16 *>(patch + row * PATCH_PITCH + col);
-    *reinterpret_cast<V16 *>(C + (m0 + wm + row) * a.ldc + n0 + wn + col) = v;
+    for (int i0 = 0; i0 < NIT; i0 += G) {
+      V16 bq[G], rq[G];
+#pragma unroll
+      for (int i = 0; i < G; i++) {
+        const int ch = (i0 + i) * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
+        if (btile) bq[i] = *reinterpret_cast<const V16 *>(btile + col);
+        if (rtile) rq[i] = *reinterpret_cast<const V16 *>(rtile + (int64_t)row * a.ldr + col);
+      }
+#pragma unroll
+      for (int i = 0; i < G; i++) {
+        const int ch = (i0 + i) * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
+        V16 q = *reinterpret_cast<const V16 *>(patch + row * PITCH + col);
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+          if (btile) q[w] = epi_add2<EL>(q[w], bq[i][w]);
+          if (rtile) q[w] = epi_add2<EL>(q[w], rq[i][w]);
+          else if (a.gelu) q[w] = epi_gelu2<EL>(q[w], a.gc[0], a.gc[1], a.gc[2], a.gc[3]);
+        }
+        *reinterpret_cast<V16 *>(ctile + (int64_t)row * a.ldc + col) = q;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+      const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
+      const V16 v = *reinterpret_cast<const V16 *>(patch + row * PITCH + col);
+      *reinterpret_cast<V16 *>(ctile + (int64_t)row * a.ldc + col) = v;
+    }
   }
 }
 

@@ -134,6 +134,62 @@ struct Args {
   int64_t goff_b[2], goff_c[2], goff_bias[2];
 };
 
+// The arithmetic of the fused linear's epilogue on 16-bit results, two neighbours per
+// register (low half first): every step is rounded to the dtype, as a primitive's store
+// and the next primitive's load would. bf16 is widened by a shift and a mask and
+// narrowed by one conversion of the pair.
+template <class EL>
+__device__ __forceinline__ void epi_widen2(uint32_t x, float &lo, float &hi) {
+  if constexpr (EL::BF16) {
+    lo = __builtin_bit_cast(float, x << 16);
+    hi = __builtin_bit_cast(float, x & 0xffff0000u);
+  } else {
+    lo = f16_to_f32((uint16_t)(x & 0xffffu));
+    hi = f16_to_f32((uint16_t)(x >> 16));
+  }
+}
+template <class EL>
+__device__ __forceinline__ uint32_t epi_narrow2(float lo, float hi) {
+  if constexpr (EL::BF16) return f32x2_to_bf16x2(lo, hi);
+  else return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
+}
+template <class EL>
+__device__ __forceinline__ void epi_rnd2(float &lo, float &hi) {
+  epi_widen2<EL>(epi_narrow2<EL>(lo, hi), lo, hi);
+}
+template <class EL>
+__device__ __forceinline__ uint32_t epi_add2(uint32_t x, uint32_t y) {
+  float x0, x1, y0, y1;
+  epi_widen2<EL>(x, x0, x1);
+  epi_widen2<EL>(y, y0, y1);
+  return epi_narrow2<EL>(x0 + y0, x1 + y1);
+}
+// The tanh GELU of kaun/lib/fn.ml:31-38, primitive by primitive; c0..c3 = 0.044715,
+// sqrt(2/pi), 1, 0.5 as the dtype holds them.
+template <class EL>
+__device__ __forceinline__ uint32_t epi_gelu2(uint32_t x, float c0, float c1, float c2, float c3) {
+  float v0, v1;
+  epi_widen2<EL>(x, v0, v1);
+  float a0 = v0 * v0, a1 = v1 * v1;  // x * x
+  epi_rnd2<EL>(a0, a1);
+  a0 = v0 * a0, a1 = v1 * a1;        // x * (x * x)
+  epi_rnd2<EL>(a0, a1);
+  a0 = a0 * c0, a1 = a1 * c0;
+  epi_rnd2<EL>(a0, a1);
+  a0 = v0 + a0, a1 = v1 + a1;
+  epi_rnd2<EL>(a0, a1);
+  a0 = a0 * c1, a1 = a1 * c1;
+  epi_rnd2<EL>(a0, a1);
+  a0 = tanh_for_16bit(a0), a1 = tanh_for_16bit(a1);
+  epi_rnd2<EL>(a0, a1);
+  a0 = a0 + c2, a1 = a1 + c2;
+  epi_rnd2<EL>(a0, a1);
+  a0 = v0 * a0, a1 = v1 * a1;
+  epi_rnd2<EL>(a0, a1);
+  a0 = a0 * c3, a1 = a1 * c3;
+  return epi_narrow2<EL>(a0, a1);
+}
+
 // One k-step of one 32x32 tile: a, b hold this lane's VE k-values of its row.
 template <class EL>
 __device__ __forceinline__ void mfma_step(f32x16 &acc, const V16 &a, const V16 &b) {
@@ -411,58 +467,8 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
         static_assert(64 % CPR == 0, "a lane's chunk column is the same in every pass");
         constexpr int NIT = TM * 32 * CPR / 64, RSTEP = 64 / CPR;
         const int col = (lane % CPR) * 8, row0 = lane / CPR;
-        // two neighbours per register: bf16 is widened by a shift and a mask and narrowed by one conversion
-        auto add2 = [&](uint32_t x, uint32_t y) -> uint32_t {
-          if constexpr (EL::BF16) {
-            const float lo = __builtin_bit_cast(float, x << 16) + __builtin_bit_cast(float, y << 16);
-            const float hi = __builtin_bit_cast(float, x & 0xffff0000u) + __builtin_bit_cast(float, y & 0xffff0000u);
-            return f32x2_to_bf16x2(lo, hi);
-          } else {
-            const S lo = narrow(widen((S)(x & 0xffffu)) + widen((S)(y & 0xffffu)));
-            const S hi = narrow(widen((S)(x >> 16)) + widen((S)(y >> 16)));
-            return (uint32_t)lo | ((uint32_t)hi << 16);
-          }
-        };
-        // both neighbours rounded to the dtype, as a primitive's store and the next one's load would
-        auto rnd2 = [&](float &lo, float &hi) {
-          if constexpr (EL::BF16) {
-            const uint32_t u = f32x2_to_bf16x2(lo, hi);
-            lo = __builtin_bit_cast(float, u << 16);
-            hi = __builtin_bit_cast(float, u & 0xffff0000u);
-          } else {
-            lo = widen(narrow(lo));
-            hi = widen(narrow(hi));
-          }
-        };
-        auto gelu2 = [&](uint32_t x) -> uint32_t {
-          float v0, v1;
-          if constexpr (EL::BF16) {
-            v0 = __builtin_bit_cast(float, x << 16);
-            v1 = __builtin_bit_cast(float, x & 0xffff0000u);
-          } else {
-            v0 = widen((S)(x & 0xffffu));
-            v1 = widen((S)(x >> 16));
-          }
-          float a0 = v0 * v0, a1 = v1 * v1;  // x * x
-          rnd2(a0, a1);
-          a0 = v0 * a0, a1 = v1 * a1;        // x * (x * x)
-          rnd2(a0, a1);
-          a0 = a0 * a.gc[0], a1 = a1 * a.gc[0];
-          rnd2(a0, a1);
-          a0 = v0 + a0, a1 = v1 + a1;
-          rnd2(a0, a1);
-          a0 = a0 * a.gc[1], a1 = a1 * a.gc[1];
-          rnd2(a0, a1);
-          a0 = tanh_for_16bit(a0), a1 = tanh_for_16bit(a1);
-          rnd2(a0, a1);
-          a0 = a0 + a.gc[2], a1 = a1 + a.gc[2];
-          rnd2(a0, a1);
-          a0 = v0 * a0, a1 = v1 * a1;
-          rnd2(a0, a1);
-          a0 = a0 * a.gc[3], a1 = a1 * a.gc[3];
-          if constexpr (EL::BF16) return f32x2_to_bf16x2(a0, a1);
-          else return (uint32_t)narrow(a0) | ((uint32_t)narrow(a1) << 16);
-        };
+        auto add2 = [](uint32_t x, uint32_t y) -> uint32_t { return epi_add2<EL>(x, y); };
+        auto gelu2 = [&](uint32_t x) -> uint32_t { return epi_gelu2<EL>(x, a.gc[0], a.gc[1], a.gc[2], a.gc[3]); };
         S *c = C + (m0 + wm + row0) * a.ldc + n0 + wn + col;
         const S *p = patch + row0 * WP + col;
         V16 bq = {0, 0, 0, 0};

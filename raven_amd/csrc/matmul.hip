@@ -873,33 +873,42 @@ static int launch_tile_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc,
   return b_kc ? NXH_TILE(false, true) : NXH_TILE(false, false);
 #undef NXH_TILE
 }
-// The direct-to-LDS form of the 256 x 256 shape (gemm_dl.hpp): whole tiles of 16-bit operands.
-template <class EL, bool A_KC, bool B_KC>
-static int launch_dl(nxh_context *ctx, gemm_tile::Args &g) {
-  auto kern = gemm_dl::kernel<EL, A_KC, B_KC>;
+// The direct-to-LDS kernels (gemm_dl.hpp): whole tiles of 16-bit operands.
+template <class EL, bool A_KC, bool B_KC, class SH, bool EPI>
+static int launch_dl(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
+  auto kern = gemm_dl::kernel<EL, A_KC, B_KC, SH, EPI>;
   static std::once_flag once;
   static hipError_t attr_status = hipSuccess;
   std::call_once(once, [&] {
-    attr_status = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_dl::LDS_BYTES);
+    attr_status = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SH::LDS_BYTES);
   });
   NXH_HIP("matmul", attr_status);
-  g.tiles_m = (uint32_t)(g.M / gemm_dl::BM);
-  g.tiles_n = (uint32_t)(g.N / gemm_dl::BN);
-  nxh_set_path("gemm_dl_256x256");
-  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(gemm_dl::THREADS), gemm_dl::LDS_BYTES, ctx->stream, g);
+  g.tiles_m = (uint32_t)(g.M / SH::BM);
+  g.tiles_n = (uint32_t)(g.N / SH::BN);
+  if (EPI && g.ngroup > 1) {
+    g.gtn = g.tiles_n;
+    g.tiles_n *= g.ngroup;  // the members side by side, as in launch_tile
+  }
+  nxh_set_path(path);
+  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * g.nbatch), dim3(SH::THREADS), SH::LDS_BYTES, ctx->stream, g);
   NXH_HIP("matmul", hipGetLastError());
   return NXH_OK;
 }
-template <class EL>
-static int launch_dl_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc) {
+// Returns -1 for an orientation that has no instance: a transposed A (contiguous along M)
+// is only built for the plain 256 x 256 product.
+template <class EL, class SH, bool EPI>
+static int launch_dl_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc, const char *path) {
   if constexpr (EL::F32) {
     return -1;
   } else {
-    if (a_kc) return b_kc ? launch_dl<EL, true, true>(ctx, g) : launch_dl<EL, true, false>(ctx, g);
-    return b_kc ? launch_dl<EL, false, true>(ctx, g) : launch_dl<EL, false, false>(ctx, g);
+    if (a_kc) return b_kc ? launch_dl<EL, true, true, SH, EPI>(ctx, g, path) : launch_dl<EL, true, false, SH, EPI>(ctx, g, path);
+    if constexpr (!EPI && SH::BM == 256)
+      return b_kc ? launch_dl<EL, false, true, SH, EPI>(ctx, g, path) : launch_dl<EL, false, false, SH, EPI>(ctx, g, path);
+    return -1;
   }
 }
-// 0: pick by shape; 256 / 128 / 64: force that block shape; 257: the 256 shape in its
+// 0: pick by shape; 256 / 192 / 128 / 64: force that block shape (192: 128 x 192, direct to
+// LDS; 128: the register-staged 128 x 128); 257: the 256 shape in its
 // register-staged form (tuning aid, read once from NXH_GEMM_TILE)
 static int forced_tile() {
   static const int v = [] {
@@ -962,17 +971,20 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       }
     }
     if (epi->gelu) {
-      // only the path that sends whole 16-byte row segments of whole 128 x 128 tiles applies it
-      if (EL::F32 || epi->R || a.M % 128 || a.N % 128 || !al16(g.C) || g.ldc % 8 || (g.bias && !al16(g.bias))) return -1;
+      // only the paths that send whole 16-byte row segments of whole tiles apply it
+      const bool whole = (a.M % 128 == 0 && a.N % 128 == 0) || (a_kc && a.M % 128 == 0 && a.N % 192 == 0);
+      if (EL::F32 || epi->R || !whole || !al16(g.C) || g.ldc % 8 || (g.bias && !al16(g.bias))) return -1;
       for (int i = 0; i < a.batch.n; i++)
         if (g.bc[i] % 8) return -1;
       g.gelu = 1;
       for (int i = 0; i < 4; i++) g.gc[i] = (float)epi->gelu[i];
     }
   }
+  // tiles of one member: a grouped launch picks the block shape its members would pick alone,
+  // so that each member's bits are those of its own call
   const int members = EPI && epi ? epi->ngroup : 1;
-  auto tiles = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * (int64_t)nbatch * members; };
-  if (tiles(128, 64) > 0x7fffffffLL) return -1;
+  auto tiles = [&](int bm, int bn) { return ((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn) * (int64_t)nbatch; };
+  if (tiles(128, 64) * members > 0x7fffffffLL) return -1;
   const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
   // Block shape: rounds of resident blocks x relative cost of one block. One
   // 256x256 block (8 waves, 144 KiB of LDS) fills a CU; two 128x128 blocks fit,
@@ -986,6 +998,36 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       pick = c256 <= c128 ? 256 : 128;
     }
   }
+  // Whole tiles of 16-bit operands go straight into LDS (gemm_dl.hpp; load offsets are 32-bit:
+  // 256 rows of a k-contiguous operand must stay below 4 GiB, and every row segment the
+  // epilogue touches must be 16-byte aligned).
+  if constexpr (!EL::F32) {
+    const int forced = forced_tile();
+    bool dl_ok = (pick == 256 || pick == 128 || pick == 192) && forced != 257 && forced != 128 && al16(g.C) &&
+                 g.ldc % 8 == 0 && g.lda < ((int64_t)1 << 22) && g.ldb < ((int64_t)1 << 22);
+    for (int i = 0; i < a.batch.n; i++)
+      if (g.bc[i] % 8 || (EPI && g.R && g.br[i] % 8)) dl_ok = false;
+    if (EPI && ((g.bias && !al16(g.bias)) || (g.R && (!al16(g.R) || g.ldr % 8)))) dl_ok = false;
+    if (dl_ok) {
+      // (the f16 conversions make the large shape's epilogue spill: f16 linears keep to the others)
+      const bool can256 = a.M % 256 == 0 && a.N % 256 == 0 && forced != 192 && !(EPI && !EL::BF16);
+      const bool can192 = a_kc && a.M % 128 == 0 && a.N % 192 == 0 && forced != 256;
+      // rounds of one block per compute unit x the block's share of a 256 x 256 tile's work,
+      // the smaller shape at about 0.8 of the large one's rate
+      const double d256 = (double)((tiles(256, 256) + cus - 1) / cus);
+      const double d192 = (double)((tiles(128, 192) + cus - 1) / cus) * (128.0 * 192.0 / 65536.0 / 0.8);
+      int rc = -1;
+      if (can192 && (!can256 || pick != 256 || d192 < d256))
+        rc = launch_dl_oriented<EL, gemm_dl::Shape128x192, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_dl_128x192" : "gemm_dl_128x192");
+      else if (can256 && pick == 256) {
+        if constexpr (!EPI || EL::BF16)
+          rc = launch_dl_oriented<EL, gemm_dl::Shape256x256, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_dl_256x256" : "gemm_dl_256x256");
+      }
+      if (rc != -1) return rc;
+    }
+  }
+  if (g.gelu && (a.M % 128 || a.N % 128)) return -1;
+  if (pick == 192) pick = 128;
   if constexpr (EPI) {
     // Two block shapes are enough for the epilogue family; f16 keeps to the small one (its
     // conversions make the 256x256 epilogue too large to stay in registers).
@@ -999,11 +1041,6 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   if (pick == 64) return launch_tile_oriented<EL, gemm_tile::Shape256x64, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
   if (pick == 128)
     return launch_tile_oriented<EL, gemm_tile::Shape128x128, false>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");
-  // whole 256 x 256 tiles of 16-bit operands: straight into LDS (load offsets are 32-bit:
-  // 256 rows of a k-contiguous operand must stay below 4 GiB)
-  if (!EL::F32 && pick == 256 && a.M % gemm_dl::BM == 0 && a.N % gemm_dl::BN == 0 && al16(g.C) && g.ldc % 8 == 0 &&
-      g.lda < ((int64_t)1 << 22) && g.ldb < ((int64_t)1 << 22))
-    return launch_dl_oriented<EL>(ctx, g, a_kc, b_kc);
   return launch_tile_oriented<EL, gemm_tile::Shape256x256, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
 }
 

@@ -350,7 +350,7 @@ def test_linear_then_gelu_is_one_gemm(hip, oracle, d, rows, inputs, outputs):
     assert (s["linear_gelu"], s["linear"], s["gelu_tanh"], s["issued"], s["fallbacks"]) == (1, 0, 0, 0, 0), s
     same_bits(got, eager, "linear + gelu in one run against the primitives")
     if rows % 128 == 0:
-        assert hip.last_path() == "linear_tile_128x128"
+        assert hip.last_path() == "linear_dl_128x192"  # 384 outputs: two 192-column blocks
         direct = logical(hip.linear_gelu_tanh(x, w, b))
         same_bits(got, direct, "against nxh_linear_gelu_tanh called by name")
     else:
@@ -358,16 +358,18 @@ def test_linear_then_gelu_is_one_gemm(hip, oracle, d, rows, inputs, outputs):
             hip.linear_gelu_tanh(x, w, b)
 
 
-def test_linear_layers_over_one_input_share_a_launch(hip, oracle):
+@pytest.mark.parametrize("rows,width,path", [(192, 256, "linear_tile_128x128"), (256, 384, "linear_dl_128x192")],
+                         ids=["staged_tiles", "direct_to_lds"])
+def test_linear_layers_over_one_input_share_a_launch(hip, oracle, rows, width, path):
     """q, k and v of an attention layer: three linear layers over the same x. Recorded one after the
     other, launched as one GEMM over the three weight matrices, each result the bits of its own call."""
     rng = np.random.default_rng(39)
     d = dt.bfloat16
     nx = Nx(hip)
     model = Gpt2(nx, Config())
-    x = tensor(hip, encode(rng.standard_normal((2, 192, 256)), d, oracle), d)
-    ws = [tensor(hip, encode(rng.standard_normal((256, 256)) * 0.1, d, oracle), d) for _ in range(3)]
-    bs = [tensor(hip, encode(rng.standard_normal(256), d, oracle), d) for _ in range(3)]
+    x = tensor(hip, encode(rng.standard_normal((2, rows, 256)), d, oracle), d)
+    ws = [tensor(hip, encode(rng.standard_normal((256, width)) * 0.1, d, oracle), d) for _ in range(3)]
+    bs = [tensor(hip, encode(rng.standard_normal(width), d, oracle), d) for _ in range(3)]
     other_w = tensor(hip, encode(rng.standard_normal((256, 128)) * 0.1, d, oracle), d)
     other_b = tensor(hip, encode(rng.standard_normal(128), d, oracle), d)
     eager = [logical(model.linear(Linear(w, b), x)) for w, b in zip(ws, bs)] + [logical(model.linear(Linear(other_w, other_b), x))]
@@ -379,6 +381,11 @@ def test_linear_layers_over_one_input_share_a_launch(hip, oracle):
     assert (s["linear"], s["grouped"], s["issued"], s["fallbacks"]) == (4, 3, 0, 0), s
     for i, (g, e) in enumerate(zip(got, eager)):
         same_bits(g, e, f"member {i} of the grouped launch against its own call")
+    with deferred(hip) as win:  # the members alone: which kernel the grouped launch took
+        outs = [model.linear(Linear(w, b), x) for w, b in zip(ws, bs)]
+        same_bits(logical(outs[2]), eager[2], "last member")
+        assert hip.last_path() == path, hip.last_path()
+        assert win.delta()["grouped"] == 3
     # a member whose result is read before the last member was recorded stays out of the group
     with deferred(hip) as win:
         a = model.linear(Linear(ws[0], bs[0]), x)

@@ -242,6 +242,9 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
                 check(hip, oracle, d, ha, hb, a, b, f"tile {m}x{k}x{n} ta={ta} tb={tb}")
                 # whole 256-tiles of 16-bit operands take the direct-to-LDS form
                 want_path = "gemm_dl_256x256" if (path, m % 256, n % 256) == ("gemm_tile_256x256", 0, 0) and d is not dt.float32 else path
+                # and 128 x 192 blocks where they fit and A is k-contiguous
+                if d is not dt.float32 and not ta and want_path == "gemm_tile_128x128" and (m % 128, n % 192) == (0, 0):
+                    want_path = "gemm_dl_128x192"
                 assert hip.last_path() == want_path, (m, k, n, ta, tb, hip.last_path())
     # odd M and N: only K-contiguous operands (A row-major, B given as its transpose) qualify
     a = encode(rng.standard_normal((203, 128)), d, oracle)
@@ -314,6 +317,64 @@ def test_matmul_direct_to_lds_kernel(hip, oracle, d):
     assert hip.last_path() == "gemm_dl_256x256"
 
 
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_and_linear_on_128x192_blocks(hip, oracle, d):
+    """The 128 x 192 direct-to-LDS shape (N = 768-like widths): both orientations of B, one to
+    fifty K-slabs, batches; then the fused linear on it (bias, residual, both, tanh GELU), bit for
+    bit the sequence of primitives, whose matmul takes the same kernel."""
+    rng = np.random.default_rng(1700 + d.tag)
+    T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
+    for m, k, n in ((1024, 64, 768), (1024, 192, 768), (384, 448, 192), (1024, 3200, 384)):
+        a = encode(rng.standard_normal((m, k)) * 0.5, d, oracle)
+        b = encode(rng.standard_normal((k, n)) * 0.5, d, oracle)
+        want = ref_f64(a, b, d, oracle)
+        ha, _ = pair(a, d, hip, oracle)
+        for tb in (False, True):
+            hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle, T if tb else None)
+            got = decode(logical(hip.matmul(ha, hb)), d, oracle)
+            assert hip.last_path() == "gemm_dl_128x192", (m, k, n, tb, hip.last_path())
+            ulp = 2.0 ** (-8 if d is dt.bfloat16 else -11)
+            assert np.all(np.abs(got - want) <= ulp * 2 * np.abs(want) + np.sqrt(k) * 2e-6), (m, k, n, tb, float(np.abs(got - want).max()))
+    a = encode(rng.standard_normal((3, 256, 128)), d, oracle)
+    b = encode(rng.standard_normal((128, 576)), d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "128x192 batched x one B")
+    assert hip.last_path() == "gemm_dl_128x192"
+    a4 = encode(rng.standard_normal((2, 1, 128, 64)), d, oracle)
+    b4 = encode(rng.standard_normal((1, 3, 64, 192)), d, oracle)
+    check(hip, oracle, d, pair(a4, d, hip, oracle)[0], pair(b4, d, hip, oracle)[0], a4, b4, "128x192 both batch-broadcast")
+    assert hip.last_path() == "gemm_dl_128x192"
+    # the fused linear
+    for xs, ws in (((4, 128, 256), (256, 768)), ((640, 1024), (1024, 192))):
+        x = encode(rng.standard_normal(xs) * 0.5, d, oracle)
+        w = encode(rng.standard_normal(ws) * 0.1, d, oracle)
+        bias = encode(rng.standard_normal(ws[-1]), d, oracle)
+        r = encode(rng.standard_normal(xs[:-1] + (ws[-1],)), d, oracle)
+        hx, hw, hb, hr = (pair(v, d, hip, oracle)[0] for v in (x, w, bias, r))
+        bshape = (1,) * (len(xs) - 1) + (ws[-1],)
+        for use_b, use_r in ((True, True), (True, False), (False, True)):
+            got = logical(hip.linear(hx, hw, hb if use_b else None, hr if use_r else None))
+            assert hip.last_path() == "linear_dl_128x192", hip.last_path()
+            y = hip.matmul(hx, hw)
+            assert hip.last_path() == "gemm_dl_128x192"
+            if use_b:
+                y = hip.binary("add", y, hip.expand(hip.reshape(hb, bshape), y.shape))
+            if use_r:
+                y = hip.binary("add", hr, y)
+            same_bits(got, logical(y), f"{d.name} {xs}x{ws} bias={use_b} residual={use_r}")
+        # a residual that is a column slice of a wider tensor, the weight given transposed
+        wide = encode(rng.standard_normal(xs[:-1] + (ws[-1] + 8,)), d, oracle)
+        hwide = hip.shrink(pair(wide, d, hip, oracle)[0], [(0, s) for s in xs[:-1]] + [(8, ws[-1] + 8)])
+        hwt = hip.permute(pair(np.ascontiguousarray(np.swapaxes(w, 0, 1)), d, hip, oracle)[0], (1, 0))
+        got = logical(hip.linear(hx, hwt, hb, hwide))
+        assert hip.last_path() == "linear_dl_128x192", hip.last_path()
+        y = hip.binary("add", hip.matmul(hx, hwt), hip.expand(hip.reshape(hb, bshape), got.shape))
+        same_bits(got, logical(hip.binary("add", hwide, y)), f"{d.name} strided residual, transposed weight")
+        # the tanh GELU in the epilogue against the fused linear followed by the GELU kernel
+        got = logical(hip.linear_gelu_tanh(hx, hw, hb))
+        assert hip.last_path() == "linear_dl_128x192", hip.last_path()
+        same_bits(got, logical(hip.gelu_tanh(hip.linear(hx, hw, hb))), f"{d.name} linear + gelu")
+
+
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16, dt.float32], ids=lambda d: d.name)
 def test_linear_epilogue_equals_the_sequence(hip, oracle, d):
     """nxh_linear = matmul, + bias, + residual with the primitives' rounding
@@ -339,7 +400,7 @@ def test_linear_epilogue_equals_the_sequence(hip, oracle, d):
 
         for use_b, use_r in ((True, True), (True, False), (False, True)):
             got = logical(hip.linear(hx, hw, hb if use_b else None, hr if use_r else None))
-            assert hip.last_path().startswith("linear_tile"), hip.last_path()
+            assert hip.last_path().startswith(("linear_tile", "linear_dl")), hip.last_path()
             want_gpu = logical(sequence(hip, hx, hw, hb if use_b else None, hr if use_r else None))
             same_bits(got, want_gpu, f"{d.name} {xs}x{ws} bias={use_b} residual={use_r}")
             want_cpu = logical(sequence(oracle, ox, ow, ob if use_b else None, orr if use_r else None))
