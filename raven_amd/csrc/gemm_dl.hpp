@@ -38,12 +38,17 @@
 namespace gemm_dl {
 using namespace gemm_tile;
 
-constexpr int BK = 64, NS = 2;
+constexpr int BK = 64;
 constexpr int UPR = BK / 8;  // 16-byte units per row of a k-contiguous tile
 
-template <int BM_, int BN_>
+// NS: slabs in the LDS ring. Two leave room for a second 128 x 192 block on the compute unit
+// (2 x 80 KiB), which is what hides a block's barriers and epilogue when a launch is several
+// rounds of blocks; a launch of at most one block per compute unit takes a deeper ring
+// instead: its operands come from memory, not from L2, and one slab of lookahead (about
+// 0.8 us) does not cover that latency. The order of additions does not depend on NS.
+template <int BM_, int BN_, int NS_>
 struct Shape {
-  static constexpr int BM = BM_, BN = BN_, WVM = 2, WVN = 4, WAVES = WVM * WVN, THREADS = 64 * WAVES;
+  static constexpr int BM = BM_, BN = BN_, NS = NS_, WVM = 2, WVN = 4, WAVES = WVM * WVN, THREADS = 64 * WAVES;
   static constexpr int WM = BM / WVM, WN = BN / WVN;   // a wave's outputs
   static constexpr int FA = WM / 16, FB = WN / 16;     // 16-row fragments of A, 16-column fragments of B per wave
   static constexpr int LA = BM / 8 / WAVES, LB = BN / 8 / WAVES, LPW = LA + LB;  // load instructions per wave and slab
@@ -53,8 +58,10 @@ struct Shape {
   static constexpr size_t PATCH_BYTES = (size_t)WAVES * WM * PATCH_PITCH * 2;
   static constexpr size_t LDS_BYTES = PATCH_BYTES > (size_t)NS * STAGE_BYTES ? PATCH_BYTES : (size_t)NS * STAGE_BYTES;
 };
-using Shape256x256 = Shape<256, 256>;
-using Shape128x192 = Shape<128, 192>;
+using Shape256x256 = Shape<256, 256, 2>;
+using Shape128x192 = Shape<128, 192, 2>;
+using Shape128x192Deep = Shape<128, 192, 4>;
+static_assert(Shape128x192Deep::LDS_BYTES <= 160 * 1024 && Shape256x256::LDS_BYTES <= 160 * 1024, "LDS");
 
 template <int N>
 __device__ __forceinline__ void wait_loads_and_meet() {
@@ -81,7 +88,7 @@ template <class EL, bool A_KC, bool B_KC, class SH, bool EPI>
 __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   using S = typename EL::S;
   static_assert(!EL::F32, "16-bit operands only");
-  constexpr int BM = SH::BM, BN = SH::BN, FA = SH::FA, FB = SH::FB, LA = SH::LA, LB = SH::LB, LPW = SH::LPW;
+  constexpr int BM = SH::BM, BN = SH::BN, NS = SH::NS, FA = SH::FA, FB = SH::FB, LA = SH::LA, LB = SH::LB, LPW = SH::LPW;
   constexpr int STAGE_BYTES = SH::STAGE_BYTES, A_BYTES = SH::A_BYTES;
   constexpr int UPK_A = BM / 8, UPK_B = BN / 8;  // units per k-row of a row-contiguous tile
   static_assert(UPK_A % 8 == 0 && UPK_B % 8 == 0, "swizzle groups");

@@ -1017,8 +1017,13 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       const double d256 = (double)((tiles(256, 256) + cus - 1) / cus);
       const double d192 = (double)((tiles(128, 192) + cus - 1) / cus) * (128.0 * 192.0 / 65536.0 / 0.8);
       int rc = -1;
-      if (can192 && (!can256 || pick != 256 || d192 < d256))
-        rc = launch_dl_oriented<EL, gemm_dl::Shape128x192, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_dl_128x192" : "gemm_dl_128x192");
+      if (can192 && (!can256 || pick != 256 || d192 < d256)) {
+        // one block per compute unit at most: nothing shares the unit, so the ring goes deeper
+        if (tiles(128, 192) * members <= cus)
+          rc = launch_dl_oriented<EL, gemm_dl::Shape128x192Deep, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_dl_128x192" : "gemm_dl_128x192");
+        else
+          rc = launch_dl_oriented<EL, gemm_dl::Shape128x192, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_dl_128x192" : "gemm_dl_128x192");
+      }
       else if (can256 && pick == 256) {
         if constexpr (!EPI || EL::BF16)
           rc = launch_dl_oriented<EL, gemm_dl::Shape256x256, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_dl_256x256" : "gemm_dl_256x256");
