@@ -48,7 +48,14 @@ struct WindowArgs {
 // magnitude slower on this machine), int64_t otherwise. Memory offsets are
 // always 64-bit. `rows_per_block` > 1 packs several short rows into one block,
 // one window per lane.
-template <class E, class I, int KT, int VW>
+// AL > 0 (VW = 4 only): the last window dim has stride AL (1 or 2) over a unit-stride
+// input dim whose rows are whole, aligned 4-element vectors. The 3 AL + 1 input elements
+// behind a unit of four windows then lie in two or three aligned vectors, which are
+// fetched whole (a vector is inside the row or in the padding as a whole) and picked
+// apart in registers: the position of the first element inside its vector is the tap
+// offset modulo 4, the same for the whole row. Four separate element loads per lane,
+// 16 or 32 bytes apart from lane to lane, made the address path the bound.
+template <class E, class I, int KT, int VW, int AL = 0>
 __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, int rows_per_block) {
   // With VW > 1 a "window" below is a unit of VW consecutive windows of the last
   // window dim (a.L and a.win[KT-1] count units); the unit is stored as one vector.
@@ -68,12 +75,12 @@ __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, in
   if (row >= (I)a.rows) return;
   I kf = row % (I)a.kernel_prod;
   I lead = row / (I)a.kernel_prod;
-  int64_t oo = (int64_t)kf * a.tap_stride, io = 0;
+  I oo = kf * (I)a.tap_stride, io = 0;  // element offsets: I is 32 bits wide only when both spans fit
   for (int d = a.ld - 1; d >= 0; d--) {
     const I c = lead % (I)a.lshape[d];
     lead /= (I)a.lshape[d];
-    oo += (int64_t)c * a.l_out[d];
-    io += (int64_t)c * a.l_in[d];
+    oo += c * (I)a.l_out[d];
+    io += c * (I)a.l_in[d];
   }
   I tap[KT], wc[KT];  // tap: kc * dilation - pad_before; wc: window coordinate
   I rest = w0;
@@ -89,40 +96,73 @@ __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, in
   struct alignas(sizeof(E) * VW) Pack {
     E v[VW];
   };
+  auto units = [&](auto r_c) {
+    constexpr int R = decltype(r_c)::value;  // AL > 0: first element's place in its aligned vector
 #pragma unroll
-  for (int u = 0; u < WINDOWS_PER_LANE; u++) {
-    const I wf = w0 + (I)u * 256;
-    if (u >= reps || wf >= L) break;
-    bool valid = true;
-    int64_t off = io;
+    for (int u = 0; u < WINDOWS_PER_LANE; u++) {
+      const I wf = w0 + (I)u * 256;
+      if (u >= reps || wf >= L) break;
+      bool valid = true;
+      I off = io;
 #pragma unroll
-    for (int d = 0; d < KT - 1; d++) {
-      const I sp = wc[d] * (I)a.stride[d] + tap[d];
-      valid = valid && sp >= 0 && sp < (I)a.extent[d];
-      off += (int64_t)sp * a.sp_stride[d];
+      for (int d = 0; d < KT - 1; d++) {
+        const I sp = wc[d] * (I)a.stride[d] + tap[d];
+        valid = valid && sp >= 0 && sp < (I)a.extent[d];
+        off += sp * (I)a.sp_stride[d];
+      }
+      Pack pk;
+      if constexpr (AL > 0) {
+        static_assert(AL == 0 || VW == 4, "aligned rows come in units of four windows");
+        constexpr int NV = (R + 3 * AL + 1 + 3) / 4;
+        const I q = wc[KT - 1] * (VW * AL) + tap[KT - 1] - R;  // a multiple of 4, possibly negative
+        E e[NV * 4];
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+          const I at = q + 4 * j;
+          Pack got;
+#pragma unroll
+          for (int v = 0; v < 4; v++) got.v[v] = E{};
+          if (valid && at >= 0 && at < (I)a.extent[KT - 1]) got = *reinterpret_cast<const Pack *>(in + (off + at));
+#pragma unroll
+          for (int v = 0; v < 4; v++) e[4 * j + v] = got.v[v];
+        }
+#pragma unroll
+        for (int v = 0; v < VW; v++) pk.v[v] = e[R + v * AL];
+      } else {
+#pragma unroll
+        for (int v = 0; v < VW; v++) {
+          const I sp = (wc[KT - 1] * VW + v) * (I)a.stride[KT - 1] + tap[KT - 1];
+          const bool ok = valid && sp >= 0 && sp < (I)a.extent[KT - 1];
+          pk.v[v] = E{};
+          if (ok) pk.v[v] = in[off + sp * (I)a.sp_stride[KT - 1]];
+        }
+      }
+      if constexpr (VW == 1) out[oo + wf * (I)a.win_stride] = pk.v[0];
+      else *reinterpret_cast<Pack *>(out + (oo + wf * VW)) = pk;
+      // 256 windows further: add the digits of 256, carrying towards the front
+      I carry = 0;
+#pragma unroll
+      for (int d = KT - 1; d >= 0; d--) {
+        const I t = wc[d] + (I)a.step[d] + carry;
+        carry = t >= (I)a.win[d] ? 1 : 0;
+        wc[d] = carry ? t - (I)a.win[d] : t;
+      }
     }
-    Pack pk;
-#pragma unroll
-    for (int v = 0; v < VW; v++) {
-      const I sp = (wc[KT - 1] * VW + v) * (I)a.stride[KT - 1] + tap[KT - 1];
-      const bool ok = valid && sp >= 0 && sp < (I)a.extent[KT - 1];
-      pk.v[v] = E{};
-      if (ok) pk.v[v] = in[off + (int64_t)sp * a.sp_stride[KT - 1]];
+  };
+  if constexpr (AL > 0) {
+    switch ((int)(tap[KT - 1] & 3)) {  // two's complement: also right for negative offsets
+      case 0: units(std::integral_constant<int, 0>{}); break;
+      case 1: units(std::integral_constant<int, 1>{}); break;
+      case 2: units(std::integral_constant<int, 2>{}); break;
+      default: units(std::integral_constant<int, 3>{}); break;
     }
-    if constexpr (VW == 1) out[oo + (int64_t)wf * a.win_stride] = pk.v[0];
-    else *reinterpret_cast<Pack *>(out + oo + (int64_t)wf * VW) = pk;
-    // 256 windows further: add the digits of 256, carrying towards the front
-    I carry = 0;
-#pragma unroll
-    for (int d = KT - 1; d >= 0; d--) {
-      const I t = wc[d] + (I)a.step[d] + carry;
-      carry = t >= (I)a.win[d] ? 1 : 0;
-      wc[d] = carry ? t - (I)a.win[d] : t;
-    }
+  } else {
+    units(std::integral_constant<int, 0>{});
   }
 }
 
-template <int DT, class I, int KT>
+// UNIT: every window stride is 1, so no tap needs a division to find its window.
+template <int DT, class I, int KT, bool UNIT>
 __global__ __launch_bounds__(256) void fold_kernel(WindowArgs a) {
   using TR = Tr<DT>;
   using S = typename TR::S;
@@ -131,53 +171,74 @@ __global__ __launch_bounds__(256) void fold_kernel(WindowArgs a) {
   if (it64 >= a.total) return;
   I ol = (I)it64;
   I oc[KT];  // position in the padded frame
-  int64_t oo = 0, il = 0;
+  I oo = 0, il = 0;  // element offsets: I is 32 bits wide only when both tensors' spans fit
 #pragma unroll
   for (int d = KT - 1; d >= 0; d--) {
     const I c = ol % (I)a.extent[d];
     ol /= (I)a.extent[d];
     oc[d] = c + (I)a.before[d];
-    oo += (int64_t)c * a.sp_stride[d];
+    oo += c * (I)a.sp_stride[d];
   }
   for (int d = a.ld - 1; d >= 0; d--) {
     const I c = ol % (I)a.lshape[d];
     ol /= (I)a.lshape[d];
-    oo += (int64_t)c * a.l_out[d];
-    il += (int64_t)c * a.l_in[d];
+    oo += c * (I)a.l_out[d];
+    il += c * (I)a.l_in[d];
   }
   const S *in = reinterpret_cast<const S *>(a.in);
   C acc;
   if constexpr (TR::cat == CAT_COMPLEX) acc = C{0, 0};
   else acc = (C)0;
-  // taps in ascending flat order kf; kc[] is kf's odometer over the kernel dims
+  // Taps in ascending flat order kf; kc[] is kf's odometer over the kernel dims. They are
+  // taken TB at a time: the addresses of a batch first (a tap that misses reads element 0
+  // of this leading index instead and is not added), then all its loads, then the sums in
+  // order. One load per loop turn left every wave waiting out a memory latency per tap.
+  constexpr int TB = 9;
   I kc[KT];
 #pragma unroll
   for (int d = 0; d < KT; d++) kc[d] = 0;
   const I taps = (I)a.kernel_prod;
-  for (I kf = 0; kf < taps; kf++) {
-    bool valid = true;
-    int64_t wf = 0;
+  for (I kf0 = 0; kf0 < taps; kf0 += TB) {
+    bool ok[TB];
+    I at[TB];
 #pragma unroll
-    for (int d = 0; d < KT; d++) {
-      const I num = oc[d] - kc[d] * (I)a.dilation[d];
-      const I st = (I)a.stride[d];
-      const I wc = st == 1 ? num : num / st;
-      valid = valid && num >= 0 && (st == 1 || num % st == 0) && wc < (I)a.win[d];
-      wf += (int64_t)wc * a.win_cp[d];
-    }
-    if (valid) {
-      const C v = TR::ld(in[il + (int64_t)kf * a.tap_stride + wf * a.win_stride]);
-      if constexpr (TR::cat == CAT_SINT) acc = (C)((uint64_t)acc + (uint64_t)v);
-      else acc = (C)(acc + v);
-    }
-    bool carry = true;
+    for (int j = 0; j < TB; j++) {
+      bool valid = kf0 + j < taps;
+      I wf = 0;
 #pragma unroll
-    for (int d = KT - 1; d >= 0; d--) {
-      if (carry) {
-        kc[d]++;
-        carry = kc[d] >= (I)a.kernel[d];
-        if (carry) kc[d] = 0;
+      for (int d = 0; d < KT; d++) {
+        const I num = oc[d] - kc[d] * (I)a.dilation[d];
+        I wc = num;
+        if constexpr (!UNIT) {
+          const I st = (I)a.stride[d];
+          wc = num / st;
+          valid = valid && num % st == 0;
+        }
+        valid = valid && num >= 0 && wc < (I)a.win[d];
+        wf += wc * (I)a.win_cp[d];
       }
+      ok[j] = valid;
+      at[j] = valid ? il + (kf0 + j) * (I)a.tap_stride + wf * (I)a.win_stride : il;
+      bool carry = true;
+#pragma unroll
+      for (int d = KT - 1; d >= 0; d--) {
+        if (carry) {
+          kc[d]++;
+          carry = kc[d] >= (I)a.kernel[d];
+          if (carry) kc[d] = 0;
+        }
+      }
+    }
+    S raw[TB];
+#pragma unroll
+    for (int j = 0; j < TB; j++) raw[j] = in[at[j]];
+#pragma unroll
+    for (int j = 0; j < TB; j++) {
+      const C v = TR::ld(raw[j]);
+      C sum;
+      if constexpr (TR::cat == CAT_SINT) sum = (C)((uint64_t)acc + (uint64_t)v);
+      else sum = (C)(acc + v);
+      acc = ok[j] ? sum : acc;
     }
   }
   reinterpret_cast<S *>(a.out)[oo] = TR::st(acc);
@@ -198,17 +259,33 @@ bool fits_int32(const WindowArgs &a) {
   }
   return true;
 }
+// Element offsets fit 32 bits too: the spans of the windowed tensor (`windows` along its last
+// dim) and of the plain one.
+bool spans_fit_int32(const WindowArgs &a, int64_t windows) {
+  int64_t cols_span = (a.kernel_prod - 1) * std::llabs(a.tap_stride) + (windows - 1) * std::llabs(a.win_stride), plain_span = 0;
+  for (int d = 0; d < a.ld; d++) {
+    // l_in / l_out: which of the two is the windowed tensor depends on the direction; bound both by the larger
+    const int64_t m = std::max(std::llabs(a.l_in[d]), std::llabs(a.l_out[d]));
+    cols_span += (a.lshape[d] - 1) * m;
+    plain_span += (a.lshape[d] - 1) * m;
+  }
+  for (int d = 0; d < WIN_MAXK; d++) plain_span += (a.extent[d] - 1) * std::llabs(a.sp_stride[d]);
+  return cols_span < ((int64_t)1 << 31) && plain_span < ((int64_t)1 << 31);
+}
 int rank_class(int K) { return K <= 3 ? K : WIN_MAXK; }
 
 typedef void (*fold_launch_fn)(nxh_context *, const WindowArgs &, int);
 template <int DT>
 void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt) {
   const dim3 grid((unsigned)((a.total + 255) / 256)), block(256);
-  const bool narrow = fits_int32(a);
-#define NXH_FOLD_CASE(KT)                                                                                  \
-  case KT:                                                                                                 \
-    if (narrow) hipLaunchKernelGGL((fold_kernel<DT, int32_t, KT>), grid, block, 0, ctx->stream, a);        \
-    else hipLaunchKernelGGL((fold_kernel<DT, int64_t, KT>), grid, block, 0, ctx->stream, a);               \
+  const bool narrow = fits_int32(a) && spans_fit_int32(a, a.L);  // 32-bit index arithmetic, offsets included
+  bool unit = true;
+  for (int d = 0; d < WIN_MAXK; d++) unit = unit && a.stride[d] == 1;
+#define NXH_FOLD_CASE(KT)                                                                                        \
+  case KT:                                                                                                       \
+    if (narrow && unit) hipLaunchKernelGGL((fold_kernel<DT, int32_t, KT, true>), grid, block, 0, ctx->stream, a); \
+    else if (narrow) hipLaunchKernelGGL((fold_kernel<DT, int32_t, KT, false>), grid, block, 0, ctx->stream, a);  \
+    else hipLaunchKernelGGL((fold_kernel<DT, int64_t, KT, false>), grid, block, 0, ctx->stream, a);              \
     break;
   switch (kt) {
     NXH_FOLD_CASE(1)
@@ -219,7 +296,7 @@ void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt) {
 #undef NXH_FOLD_CASE
 }
 
-template <class E, int VW>
+template <class E, int VW, int AL = 0>
 int unfold_launch_v(nxh_context *ctx, const char *op, const WindowArgs &a, int kt) {
   int rows_per_block = 1;
   int64_t wblocks = (a.L + 256 * WINDOWS_PER_LANE - 1) / (256 * WINDOWS_PER_LANE), blocks = a.rows * wblocks;
@@ -231,14 +308,14 @@ int unfold_launch_v(nxh_context *ctx, const char *op, const WindowArgs &a, int k
   }
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
   const dim3 grid((unsigned)blocks), block(256);
-  const bool narrow = fits_int32(a);
+  const bool narrow = fits_int32(a) && spans_fit_int32(a, a.L * VW);
 #define NXH_UNFOLD_CASE(KT)                                                                                     \
   case KT:                                                                                                      \
     if (narrow)                                                                                                 \
-      hipLaunchKernelGGL((unfold_kernel<E, int32_t, KT, VW>), grid, block, 0, ctx->stream, a, (int32_t)wblocks, \
-                         rows_per_block);                                                                       \
+      hipLaunchKernelGGL((unfold_kernel<E, int32_t, KT, VW, AL>), grid, block, 0, ctx->stream, a,               \
+                         (int32_t)wblocks, rows_per_block);                                                     \
     else                                                                                                        \
-      hipLaunchKernelGGL((unfold_kernel<E, int64_t, KT, VW>), grid, block, 0, ctx->stream, a, wblocks,          \
+      hipLaunchKernelGGL((unfold_kernel<E, int64_t, KT, VW, AL>), grid, block, 0, ctx->stream, a, wblocks,      \
                          rows_per_block);                                                                       \
     break;
   switch (kt) {
@@ -254,18 +331,29 @@ int unfold_launch_v(nxh_context *ctx, const char *op, const WindowArgs &a, int k
 // Four consecutive windows of the last window dim become one store when the
 // output allows it: that dim's window count a multiple of 4, windows
 // contiguous, every row of the output starting on a 4-element boundary.
+// `aligned_rows`: the input side of the aligned form (see unfold_kernel) holds.
 template <class E>
-int unfold_launch(nxh_context *ctx, const char *op, WindowArgs &a, int kt, bool vector_ok) {
+int unfold_launch(nxh_context *ctx, const char *op, WindowArgs &a, int kt, bool vector_ok, bool aligned_rows) {
   constexpr int VW = sizeof(E) <= 4 ? 4 : 1;
-  if (VW > 1 && vector_ok && a.win[kt - 1] % VW == 0) {
-    a.L /= VW;
-    a.win[kt - 1] /= VW;
-    int64_t rest = 256;
-    for (int s = kt - 1; s >= 0; s--) {  // 256 units further, in the new radix
-      a.step[s] = rest % a.win[s];
-      rest /= a.win[s];
+  if constexpr (VW > 1) {
+    if (vector_ok && a.win[kt - 1] % VW == 0) {
+      a.L /= VW;
+      a.win[kt - 1] /= VW;
+      int64_t rest = 256;
+      for (int s = kt - 1; s >= 0; s--) {  // 256 units further, in the new radix
+        a.step[s] = rest % a.win[s];
+        rest /= a.win[s];
+      }
+      if (aligned_rows && a.stride[kt - 1] == 1) {
+        nxh_set_path("unfold_aligned");
+        return unfold_launch_v<E, VW, 1>(ctx, op, a, kt);
+      }
+      if (aligned_rows && a.stride[kt - 1] == 2) {
+        nxh_set_path("unfold_aligned");
+        return unfold_launch_v<E, VW, 2>(ctx, op, a, kt);
+      }
+      return unfold_launch_v<E, VW>(ctx, op, a, kt);
     }
-    return unfold_launch_v<E, VW>(ctx, op, a, kt);
   }
   return unfold_launch_v<E, 1>(ctx, op, a, kt);
 }
@@ -362,15 +450,22 @@ NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
   bool vector_ok = a.win_stride == 1 && a.tap_stride % 4 == 0 && ((uintptr_t)a.out % (uintptr_t)(4 * es)) == 0;
   for (int d = 0; d < a.ld; d++)
     if (a.lshape[d] > 1 && a.l_out[d] % 4 != 0) vector_ok = false;
+  // the input side of the aligned form: unit stride along the last window dim, whose rows
+  // are whole 4-element vectors, every other step of the input a multiple of 4 elements
+  bool aligned_rows = a.sp_stride[kt - 1] == 1 && a.extent[kt - 1] % 4 == 0 && ((uintptr_t)a.in % (uintptr_t)(4 * es)) == 0;
+  for (int d = 0; d < kt - 1; d++)
+    if (a.extent[d] > 1 && a.sp_stride[d] % 4 != 0) aligned_rows = false;
+  for (int d = 0; d < a.ld; d++)
+    if (a.lshape[d] > 1 && a.l_in[d] % 4 != 0) aligned_rows = false;
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path("unfold");
   switch (es) {
-    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt, vector_ok); break;
-    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt, vector_ok); break;
-    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt, vector_ok); break;
-    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt, vector_ok); break;
-    default: rc = unfold_launch<G16w>(ctx, op, a, kt, vector_ok); break;
+    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
+    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
+    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
+    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
+    default: rc = unfold_launch<G16w>(ctx, op, a, kt, vector_ok, false); break;
   }
   if (rc) return rc;
   NXH_HIP(op, hipGetLastError());

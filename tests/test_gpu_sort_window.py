@@ -164,7 +164,15 @@ GEOMETRIES = [
     ((2, 5, 6, 4), [2, 3, 2], [1, 2, 1], [2, 1, 1], [(1, 1), (0, 2), (0, 0)]),
     ((3, 8, 8), [8, 8], [1, 1], [1, 1], [(0, 0), (0, 0)]),          # one window
     ((1, 2, 16, 16), [3, 3], [1, 1], [1, 1], [(1, 1), (1, 1)]),     # "same" convolution
+    # rows of whole 4-element vectors, window counts that are multiples of 4: the aligned-load form
+    # of unfold, with tap offsets of every residue modulo 4, strides 1 and 2, a dilation
+    ((2, 3, 12, 16), [2, 5], [1, 1], [1, 1], [(0, 1), (2, 2)]),
+    ((2, 2, 9, 32), [3, 7], [2, 2], [1, 1], [(1, 1), (3, 3)]),
+    ((3, 24), [3], [1], [2], [(2, 2)]),
+    ((5, 40), [4], [2], [3], [(1, 7)]),
+    ((2, 4, 4, 8), [2, 2, 3], [1, 2, 1], [1, 1, 1], [(0, 0), (0, 0), (1, 1)]),
 ]
+ALIGNED_FROM = 5  # index of the first geometry above that takes the aligned form (1-, 2- and 4-byte elements)
 
 
 @pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.int16, dt.uint8, dt.complex64, dt.bool_],
@@ -182,6 +190,8 @@ def test_unfold_and_fold_match_oracle(hip, oracle, d):
             x = rng.integers(0, 100, shape).astype(d.np_storage)
         h, o = pair(x, d, hip, oracle)
         hu, ou = hip.unfold(h, ks, st, dl, pd), oracle.unfold(o, ks, st, dl, pd)
+        if d.itemsize <= 4 and GEOMETRIES.index((shape, ks, st, dl, pd)) >= ALIGNED_FROM - 1:
+            assert hip.last_path() == "unfold_aligned", (shape, hip.last_path())
         same_bits(logical(hu), logical(ou), f"unfold {d.name} {shape}")
         k = len(ks)
         # fold sums taps in the reference's order: equal bits, floats included
@@ -222,6 +232,7 @@ def test_window_large_and_errors(hip):
     x = rng.integers(-4, 4, (8, 16, 128, 128)).astype(np.float32)
     t = mk(hip, x, dt.float32)
     u = hip.unfold(t, [3, 3], [1, 1], [1, 1], [(1, 1), (1, 1)])
+    assert hip.last_path() == "unfold_aligned"
     assert tuple(u.shape) == (8, 16, 9, 128 * 128)
     centre = logical(hip.shrink(u, [(0, 8), (0, 16), (4, 5), (0, 128 * 128)])).reshape(x.shape)
     assert np.array_equal(centre, x)
