@@ -59,6 +59,11 @@ struct FftArgs {
   int n_store;
   int sign;              // -1 forward, +1 inverse
   int G;                 // lines per workgroup
+  // The workgroup's G lines are neighbours in memory while a line's own elements are strided
+  // (a transform down the columns of a row-major tensor): consecutive lanes then take the
+  // same element of consecutive lines, so that a wave's accesses are contiguous runs of G
+  // elements instead of 64 separate ones. Separately for the load and the store side.
+  int in_lines_fast, out_lines_fast;
   const double2 *tw;     // exp(-2 pi i k / M), k < M/2
   const double2 *chirp;  // Bluestein: exp(sign pi i j^2 / n), j < n
   const double2 *bf;     // Bluestein: forward transform (length M) of the wrapped conjugate chirp
@@ -196,7 +201,11 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
   int64_t *off_in = (int64_t *)(lds + pad(a.G << a.logM) + 1);
   int64_t *off_out = off_in + a.G;
   int *inner = (int *)(off_out + a.G);
-  const int64_t first = (int64_t)blockIdx.x * a.G;
+  // blocks that share an XCD (ids equal modulo 8) take neighbouring groups of lines: with
+  // strided lines a 128-byte line of memory serves several workgroups, which then meet in one L2
+  uint32_t bx = blockIdx.x;
+  if ((gridDim.x & 7u) == 0) bx = (bx & 7u) * (gridDim.x >> 3) + (bx >> 3);
+  const int64_t first = (int64_t)bx * a.G;
   for (int g = threadIdx.x; g < a.G; g += blockDim.x) {
     const int64_t l = first + g;
     int in_c = 0, out_c = 0;
@@ -208,7 +217,8 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
   const int total = a.G << a.logM;
   const int shift = 32 - a.logM;
   for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
-    const int g = idx >> a.logM, j = idx & (a.M - 1);
+    int g = idx >> a.logM, j = idx & (a.M - 1);
+    if (a.in_lines_fast) j = idx / a.G, g = idx - j * a.G;
     double2 v = make_double2(0.0, 0.0);
     if (first + g < a.lines && j < a.n) {
       v = fetch(a, off_in[g], j);
@@ -235,8 +245,13 @@ __global__ __launch_bounds__(1024) void fft_lines_kernel(FftArgs a) {
   const int stores = a.G * a.n_store;
   for (int idx = threadIdx.x; idx < stores; idx += blockDim.x) {
     // whole power-of-two lines (the common case) are decoded without a division
-    const int g = a.n_store == a.M ? idx >> a.logM : idx / a.n_store, k = idx - g * a.n_store;
-    if (first + g >= a.lines) break;
+    int g = a.n_store == a.M ? idx >> a.logM : idx / a.n_store, k = idx - g * a.n_store;
+    if (a.out_lines_fast) {
+      k = idx / a.G, g = idx - k * a.G;
+      if (first + g >= a.lines) continue;
+    } else if (first + g >= a.lines) {
+      break;
+    }
     double2 v = lds[pad((g << a.logM) + k)];
     if (BLUE) {
       const double2 c = a.chirp[k];
@@ -402,7 +417,14 @@ static Lines workspace_lines(double2 *w, int64_t outer, int64_t outer_stride, in
 static int launch_lines(nxh_context *ctx, FftArgs &a, bool blue) {
   // short lines share a workgroup of FFT_LDS_MIN elements; long ones get one each
   a.G = a.M >= FFT_LDS_MIN ? 1 : FFT_LDS_MIN / a.M;
+  // strided lines whose neighbours are adjacent in memory: as many lines per workgroup as make
+  // runs of 128 bytes, or as the LDS holds
+  auto neighbours = [](const Lines &v) { return v.estride != 1 && v.nd >= 1 && v.strides[v.nd - 1] == 1 && v.dims[v.nd - 1] > 1; };
+  a.in_lines_fast = neighbours(a.in);
+  a.out_lines_fast = neighbours(a.out);
+  if (a.in_lines_fast || a.out_lines_fast) a.G = std::max(1, std::min(FFT_LDS_MAX / a.M, std::max(16, FFT_LDS_MIN / a.M)));
   if ((int64_t)a.G > a.lines) a.G = (int)a.lines;
+  if (a.G == 1) a.in_lines_fast = a.out_lines_fast = 0;
   const int64_t blocks = (a.lines + a.G - 1) / a.G;
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, "fft", "too many lines for one launch");
   const int64_t elems = (int64_t)a.G * a.M;
