@@ -330,8 +330,8 @@ int nxh_linear(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
      out = gelu_tanh (matmul x w + bias)
    with every rounding of the eleven primitives it stands for, so the value equals the
    two calls' bit for bit. bfloat16 / float16 operands whose product is made of whole
-   128 x 128 tiles with 16-byte aligned rows; anything else is Failure and the caller
-   issues the two calls. `constants` as for nxh_gelu_tanh. */
+   128 x 128 tiles (or, with a row-major x, 128 x 192 ones) with 16-byte aligned rows;
+   anything else is Failure and the caller issues the two calls. `constants` as for nxh_gelu_tanh. */
 int nxh_linear_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
                          const nxh_tensor *w, const nxh_tensor *bias, const void *constants);
 

@@ -590,7 +590,7 @@ class Backend:
                          constants=(0.044715, 0.7978845608028654, 1.0, 0.5)) -> Tensor:
         """``gelu_tanh(matmul x w + bias)`` with the GELU in the GEMM's epilogue: the bits of
         ``linear`` followed by ``gelu_tanh``. Raises for anything but bfloat16 / float16 products made
-        of whole 128 x 128 tiles (the caller then issues the two calls)."""
+        of whole 128 x 128 (or 128 x 192) tiles (the caller then issues the two calls)."""
         out = self.buffer(x.dtype, list(x.shape[:-1]) + [w.shape[-1]])
         if isinstance(constants, np.ndarray):
             enc = np.ascontiguousarray(constants.reshape(4))
