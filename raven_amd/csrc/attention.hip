@@ -177,7 +177,28 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
   // arithmetic; registers -> LDS between the two barriers.
   constexpr int NV = KEYS * VPR / 128;
   V16 kpre[NV], vpre[NV];
+  // this lane's vectors inside a key tile, as element offsets from the tile's first row (a whole
+  // tile then costs no address arithmetic per load: one uniform base per operand and tile)
+  uint32_t koff[NV], voff[NV];
+  const bool short_offsets = (int64_t)KEYS * a.k.row < ((int64_t)1 << 31) && (int64_t)KEYS * a.v.row < ((int64_t)1 << 31) &&
+                             a.k.row >= 0 && a.v.row >= 0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int v = threadIdx.x + i * 128;
+    const int r = v / VPR, c = (v % VPR) * 8;
+    koff[i] = (uint32_t)(r * a.k.row + c);
+    voff[i] = (uint32_t)(r * a.v.row + c);
+  }
   auto prefetch = [&](int pass, int kt) {
+    if (short_offsets && (kt + 1) * KEYS <= a.sk) {  // uniform: every key of the tile exists
+      const S *kb = K + (int64_t)kt * KEYS * a.k.row, *vb = V + (int64_t)kt * KEYS * a.v.row;
+#pragma unroll
+      for (int i = 0; i < NV; i++) {
+        kpre[i] = *reinterpret_cast<const V16 *>(kb + koff[i]);
+        if (pass == 1) vpre[i] = *reinterpret_cast<const V16 *>(vb + voff[i]);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int v = threadIdx.x + i * 128;
@@ -207,6 +228,100 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
       __syncthreads();
       if (kt + 1 < ktiles) prefetch(pass, kt + 1);
       else if (pass == 0) prefetch(1, 0);
+      // B operand of O^T = V^T P^T for k-step ks of sub-tile `sub`: this lane's query, keys
+      // ks*16 + g*8 + 0..7. The accumulator gave keys ks*16 + g*4 + 0..3 and
+      // ks*16 + 8 + g*4 + 0..3: swap one half with lane ^ 32. Then the products with V^T.
+      auto times_v = [&](int sub, const uint32_t (&pk)[8]) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+          const uint32_t a0 = pk[ks * 4 + 0], a1 = pk[ks * 4 + 1];  // keys g*4 + 0..3
+          const uint32_t b0 = pk[ks * 4 + 2], b1 = pk[ks * 4 + 3];  // keys 8 + g*4 + 0..3
+          const uint32_t s0 = g == 0 ? b0 : a0, s1 = g == 0 ? b1 : a1;
+          const uint32_t r0 = (uint32_t)__shfl_xor((int)s0, 32, 64), r1 = (uint32_t)__shfl_xor((int)s1, 32, 64);
+          const V16 pf = g == 0 ? V16{a0, a1, r0, r1} : V16{r0, r1, b0, b1};
+#pragma unroll
+          for (int ot = 0; ot < OT; ot++) {
+            // A operand: V^T rows d = ot*32 + lane%32, keys as above, by transposing LDS reads
+            const int kk = sub * 32 + ks * 16 + g * 8 + ((lane & 15) >> 2);
+            const int rr = ot * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+            const S *src = Vs + kk * PV + rr;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)src);
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src + 4 * PV));
+            typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            gemm_tile::mfma_step<EL>(oacc[ot], V16{l2[0], l2[1], h2[0], h2[1]}, pf);
+          }
+        }
+      };
+      if constexpr (ONLINE) {
+        if (a.raw) {
+          // Both 32-key sub-tiles of the tile in one step: one maximum, one decision about the
+          // reference and 32 independent exponentials per lane instead of two dependent rounds
+          // of 16. The first sub-tile is visible whenever the tile is visited (its first key is
+          // at or before the wave's first query and inside the keys); the second may lie wholly
+          // above the diagonal or past the last key: then only the first is worked on.
+          const int j0 = kt * KEYS;
+          const bool two = !(j0 + 32 >= a.sk || (a.causal && j0 + 32 > qw + 31));
+          float t0[16], t1[16];
+          scores(j0, t0, j0 + 32 <= a.sk && !a.has_mask && (!a.causal || j0 + 31 <= qw));
+          if (two) {
+            scores(j0 + 32, t1, j0 + 64 <= a.sk && !a.has_mask && (!a.causal || j0 + 63 <= qw));
+          } else {
+#pragma unroll
+            for (int e = 0; e < 16; e++) t1[e] = -__builtin_inff();
+          }
+          float tm = t0[0];
+#pragma unroll
+          for (int e = 1; e < 16; e++) tm = __builtin_fmaxf(tm, t0[e]);
+#pragma unroll
+          for (int e = 0; e < 16; e++) tm = __builtin_fmaxf(tm, t1[e]);
+          tm = __builtin_fmaxf(tm, xor32(tm));  // this query's maximum over the tile, both halves agree
+          // The reference of the exponentials follows the maximum lazily: it moves only when a
+          // tile's maximum lies more than 2^8 above it (or when it is the first thing the query
+          // sees). In between the exponentials are taken against the older, smaller reference and
+          // may reach 256: harmless in f32 and in the 16-bit rounding, which is relative, and the
+          // row sum carries the same reference. Following every new maximum exactly rescaled the
+          // 32 output accumulators of every lane in most steps (with 32 queries per wave one of
+          // them often sees a new maximum). The exponential is the bare hardware 2^x of one fused
+          // multiply-add: about 1e-6 relative, three orders below the 16-bit rounding that follows
+          // (the six-instruction form is kept where the quotient is rounded instead).
+          const bool first = m_run == -__builtin_inff();
+          const bool grow = tm > m_run && (first || __builtin_fmaf(tm, a.c2, -m_run * a.c2) > 8.0f);
+          const float m_new = grow ? tm : m_run;
+          const float m_ref = m_new == -__builtin_inff() ? 0.0f : m_new;
+          const float mc = -m_ref * a.c2;
+          const float alpha = grow ? __builtin_amdgcn_exp2f(__builtin_fmaf(m_run, a.c2, mc)) : 1.0f;
+          if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+            for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+              for (int e = 0; e < 16; e++) oacc[ot][e] = oacc[ot][e] * alpha;
+          }
+          uint32_t pk0[8], pk1[8];
+          float sum0 = 0.0f, sum1 = 0.0f;
+#pragma unroll
+          for (int e = 0; e < 16; e += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(t0[e], a.c2, mc));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(t0[e + 1], a.c2, mc));
+            sum0 = sum0 + p0 + p1;
+            pk0[e >> 1] = narrow2<EL>(p0, p1);
+          }
+          times_v(0, pk0);
+          if (two) {
+#pragma unroll
+            for (int e = 0; e < 16; e += 2) {
+              const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[e], a.c2, mc));
+              const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(t1[e + 1], a.c2, mc));
+              sum1 = sum1 + p0 + p1;
+              pk1[e >> 1] = narrow2<EL>(p0, p1);
+            }
+            times_v(1, pk1);
+          }
+          l_run = __builtin_fmaf(l_run, alpha, sum0 + sum1);
+          m_run = m_new;
+          continue;
+        }
+      }
 #pragma unroll
       for (int sub = 0; sub < KEYS / 32; sub++) {
         const int j0 = kt * KEYS + sub * 32;
@@ -248,33 +363,18 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
             float tm = t[0];
 #pragma unroll
             for (int e = 1; e < 16; e++) tm = __builtin_fmaxf(tm, t[e]);
-            float m_new = __builtin_fmaxf(m_run, tm);
-            m_new = __builtin_fmaxf(m_new, xor32(m_new));
+            tm = __builtin_fmaxf(tm, xor32(tm));  // this query's maximum over the sub-tile, both halves agree
+            // (the raw form took the merged step above; here the scores are scaled and masked)
+            float sum = 0.0f;
+            const float m_new = __builtin_fmaxf(m_run, tm);
             // nothing visible yet: exponentials of -inf against 0 are 0, not NaN
             const float m_ref = m_new == -__builtin_inff() ? 0.0f : m_new;
-            float alpha, sum = 0.0f;
-            if (a.raw) {
-              // The exponential is the bare hardware 2^x of one fused multiply-add: about 1e-6
-              // relative, three orders below the 16-bit rounding that follows (the six-instruction
-              // form of the two-pass kernel is kept where the quotient is rounded instead).
-              const float mc = -m_ref * a.c2;
-              // (an unchanged maximum must give exactly 1: the product in the fused form is not rounded as mc was)
-              alpha = m_run == m_ref ? 1.0f : __builtin_amdgcn_exp2f(__builtin_fmaf(m_run, a.c2, mc));
+            const float alpha = exp_nonpositive(m_run - m_ref);
 #pragma unroll
-              for (int e = 0; e < 16; e += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(t[e], a.c2, mc));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(t[e + 1], a.c2, mc));
-                sum = sum + p0 + p1;
-                pk[e >> 1] = narrow2<EL>(p0, p1);
-              }
-            } else {
-              alpha = exp_nonpositive(m_run - m_ref);
-#pragma unroll
-              for (int e = 0; e < 16; e += 2) {
-                const float p0 = exp_nonpositive(t[e] - m_ref), p1 = exp_nonpositive(t[e + 1] - m_ref);
-                sum = sum + p0 + p1;
-                pk[e >> 1] = narrow2<EL>(p0, p1);
-              }
+            for (int e = 0; e < 16; e += 2) {
+              const float p0 = exp_nonpositive(t[e] - m_ref), p1 = exp_nonpositive(t[e + 1] - m_ref);
+              sum = sum + p0 + p1;
+              pk[e >> 1] = narrow2<EL>(p0, p1);
             }
             l_run = __builtin_fmaf(l_run, alpha, sum);
             if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -292,29 +392,7 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
               pk[e >> 1] = narrow2<EL>(p0, p1);
             }
           }
-          // B operand of O^T = V^T P^T for k-step ks: this lane's query, keys
-          // ks*16 + g*8 + 0..7. The accumulator gave keys ks*16 + g*4 + 0..3 and
-          // ks*16 + 8 + g*4 + 0..3: swap one half with lane ^ 32.
-#pragma unroll
-          for (int ks = 0; ks < 2; ks++) {
-            const uint32_t a0 = pk[ks * 4 + 0], a1 = pk[ks * 4 + 1];  // keys g*4 + 0..3
-            const uint32_t b0 = pk[ks * 4 + 2], b1 = pk[ks * 4 + 3];  // keys 8 + g*4 + 0..3
-            const uint32_t s0 = g == 0 ? b0 : a0, s1 = g == 0 ? b1 : a1;
-            const uint32_t r0 = (uint32_t)__shfl_xor((int)s0, 32, 64), r1 = (uint32_t)__shfl_xor((int)s1, 32, 64);
-            const V16 pf = g == 0 ? V16{a0, a1, r0, r1} : V16{r0, r1, b0, b1};
-#pragma unroll
-            for (int ot = 0; ot < OT; ot++) {
-              // A operand: V^T rows d = ot*32 + lane%32, keys as above, by transposing LDS reads
-              const int kk = sub * 32 + ks * 16 + g * 8 + ((lane & 15) >> 2);
-              const int rr = ot * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
-              const S *src = Vs + kk * PV + rr;
-              const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)src);
-              const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src + 4 * PV));
-              typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-              const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-              gemm_tile::mfma_step<EL>(oacc[ot], V16{l2[0], l2[1], h2[0], h2[1]}, pf);
-            }
-          }
+          times_v(sub, pk);
         }
       }
     }
