@@ -408,13 +408,21 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
 #pragma unroll
         for (int u = 0; u < TN; u++) fb[nxt][u] = frag_load<EL, B_KC, BN>(nB, wn + u * 32, 0, lane);
       }
-      // keep the order written here (LDS returns in order, so the wait before
-      // the first MFMA only covers the current fragments)
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int t = 0; t < TM; t++)
 #pragma unroll
         for (int u = 0; u < TN; u++) mfma_step<EL>(acc[t][u], fa[cur][t], fb[cur][u]);
+      // The memory instructions of this k-step are issued among its MFMAs, one LDS read, one
+      // LDS write and one global load behind each (LDS returns in order, so the wait before the
+      // first MFMA only covers the current fragments): queueing them all in front of the step
+      // left the matrix pipe cold while they issued.
+#pragma unroll
+      for (int x = 0; x < TM * TN * (EL::F32 ? 4 : 1); x++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS reads
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // LDS write
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global load
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
