@@ -471,6 +471,295 @@ __global__ __launch_bounds__(256) void psort_merge_kernel(SortArgs a, int64_t kk
   }
 }
 
+// ── long slices of packed words: a radix sort ──────────────────────────────
+// The network above costs log^2 n passes over a long slice; from RX_MIN_N elements on the
+// packed words are sorted least significant digit first instead, eight bits at a time, over
+// the HIGH half only: the low half (the index) ascends with the position the words start at
+// and every pass is stable, so words with equal high halves stay in index order. The
+// descending value sort wants its ties in descending index order and its NaNs in ascending:
+// it sorts ascending and writes the non-NaN prefix out reversed, which is how the reference
+// defines it (nx_c_sort.c:283-289).
+// One pass is four launches: a histogram of the digit per 4096-word tile, laid out bin by
+// bin ([256][tiles], so that its exclusive scan is a tile's first output position for each
+// digit), the scan in two levels (segments of 4096 entries, then the segment totals), and the
+// scatter, in which every tile ranks its words stably: a wave owns 1024 consecutive words,
+// takes them 64 at a time in order, finds for each lane the lanes with the same digit by
+// eight ballots, and keeps a running count per digit; the waves' counts are then offset
+// against each other. No inter-block waiting anywhere.
+// Digits that cannot change the order are skipped: the low bits of a widened 16- or 8-bit
+// float, and the sign-extension bytes of a narrow integer, are functions of higher bits.
+constexpr int RX_TILE = 4096;
+constexpr int RX_ROWS = RX_TILE / 256;
+constexpr int RX_SEG = 4096;
+constexpr int64_t RX_MIN_N = 16384;
+
+template <int DT>
+constexpr int rx_pass_mask() {  // bit p: the pass over bits 8p .. 8p+7 of the mapped value is needed
+  switch (DT) {
+    case NXH_BF16: case NXH_F8E4M3: case NXH_F8E5M2: return 0b1100;
+    case NXH_F16: return 0b1110;
+    case NXH_U8: case NXH_BOOL: return 0b0001;
+    case NXH_I8: return 0b1001;
+    case NXH_U16: return 0b0011;
+    case NXH_I16: return 0b1011;
+    default: return 0b1111;
+  }
+}
+
+struct RadixArgs {
+  const uint64_t *src;
+  uint64_t *dst;
+  uint32_t *hist;  // [slices][256 * nblk], bin-major; after the scans: exclusive inside its segment
+  uint32_t *seg;   // [slices][nseg]: segment totals, then their exclusive scan
+  int64_t slices, n;
+  int nblk, nseg, shift;
+};
+
+__global__ __launch_bounds__(256) void rx_zero_kernel(uint32_t *p, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < count) p[i] = 0;
+}
+
+// Packs the slices into words (position = index); counts the NaN words of each slice.
+template <int DT, int PM, bool COUNT_NAN>
+__global__ __launch_bounds__(256) void rx_pack_kernel(SortArgs a, uint64_t *w, uint32_t *nan_count, int nblk) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  const int64_t s = blockIdx.x / nblk, base = (int64_t)(blockIdx.x % nblk) * RX_TILE;
+  int64_t io, oo;
+  slice_offsets(a, s, io, oo);
+  uint32_t nans = 0;
+  for (int e = threadIdx.x; e < RX_TILE; e += 256) {
+    const int64_t i = base + e;
+    if (i >= a.n) break;
+    const uint64_t word = Packed<DT>::template pack<PM>(TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]), (uint32_t)i);
+    w[s * a.n + i] = word;
+    nans += (uint32_t)(word >> 32) == Packed<DT>::K_NAN && TR::cat == CAT_FLOAT;
+  }
+  if constexpr (COUNT_NAN) {
+    if (TR::cat == CAT_FLOAT && nans) atomicAdd(nan_count + s, nans);
+  }
+}
+
+__global__ __launch_bounds__(256) void rx_hist_kernel(RadixArgs r) {
+  __shared__ uint32_t h[256];
+  const int64_t s = blockIdx.x / r.nblk;
+  const int blk = (int)(blockIdx.x % r.nblk);
+  h[threadIdx.x] = 0;
+  __syncthreads();
+  const uint64_t *src = r.src + s * r.n;
+  for (int e = threadIdx.x; e < RX_TILE; e += 256) {
+    const int64_t i = (int64_t)blk * RX_TILE + e;
+    if (i < r.n) atomicAdd(&h[(uint32_t)(src[i] >> r.shift) & 255u], 1u);
+  }
+  __syncthreads();
+  r.hist[s * 256 * r.nblk + (int64_t)threadIdx.x * r.nblk + blk] = h[threadIdx.x];
+}
+
+// Exclusive scan of 256 per-thread values across the block; returns this thread's offset and
+// the block total. `tmp` holds 4 words.
+__device__ __forceinline__ uint32_t rx_block_scan(uint32_t v, uint32_t *tmp, uint32_t &total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t inc = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t o = (uint32_t)__shfl_up((int)inc, d, 64);
+    if (lane >= d) inc += o;
+  }
+  if (lane == 63) tmp[wave] = inc;
+  __syncthreads();
+  uint32_t before = 0;
+  for (int w = 0; w < wave; w++) before += tmp[w];
+  total = tmp[0] + tmp[1] + tmp[2] + tmp[3];
+  __syncthreads();
+  return before + inc - v;
+}
+
+// Level one of the scan: every segment of RX_SEG histogram entries in place, its total to `seg`.
+__global__ __launch_bounds__(256) void rx_scan_segments_kernel(RadixArgs r) {
+  __shared__ uint32_t tmp[4];
+  const int64_t s = blockIdx.x / r.nseg;
+  const int g = (int)(blockIdx.x % r.nseg);
+  const int64_t len = (int64_t)256 * r.nblk;
+  uint32_t *h = r.hist + s * len;
+  constexpr int PER = RX_SEG / 256;
+  const int64_t first = (int64_t)g * RX_SEG + (int64_t)threadIdx.x * PER;
+  uint32_t v[PER], sum = 0;
+#pragma unroll
+  for (int k = 0; k < PER; k++) {
+    v[k] = first + k < len ? h[first + k] : 0;
+    sum += v[k];
+  }
+  uint32_t total;
+  uint32_t run = rx_block_scan(sum, tmp, total);
+#pragma unroll
+  for (int k = 0; k < PER; k++) {
+    if (first + k < len) h[first + k] = run;
+    run += v[k];
+  }
+  if (threadIdx.x == 0) r.seg[s * r.nseg + g] = total;
+}
+
+// Level two: the segment totals of a slice, one block per slice.
+__global__ __launch_bounds__(256) void rx_scan_totals_kernel(RadixArgs r) {
+  __shared__ uint32_t tmp[4];
+  uint32_t *t = r.seg + (int64_t)blockIdx.x * r.nseg;
+  uint32_t carry = 0;
+  for (int base = 0; base < r.nseg; base += 256) {
+    const int i = base + threadIdx.x;
+    const uint32_t v = i < r.nseg ? t[i] : 0;
+    uint32_t total;
+    const uint32_t off = rx_block_scan(v, tmp, total);
+    if (i < r.nseg) t[i] = carry + off;
+    carry += total;
+  }
+}
+
+__global__ __launch_bounds__(256) void rx_scatter_kernel(RadixArgs r) {
+  __shared__ uint32_t cnt[4][256];
+  __shared__ uint32_t base[256];
+  const int64_t s = blockIdx.x / r.nblk;
+  const int blk = (int)(blockIdx.x % r.nblk);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int w = 0; w < 4; w++) cnt[w][threadIdx.x] = 0;
+  {
+    const int64_t at = (int64_t)threadIdx.x * r.nblk + blk;  // this tile's entry for digit threadIdx.x
+    base[threadIdx.x] = r.hist[s * 256 * r.nblk + at] + r.seg[s * r.nseg + at / RX_SEG];
+  }
+  __syncthreads();
+  const uint64_t *src = r.src + s * r.n;
+  uint64_t *dst = r.dst + s * r.n;
+  const int64_t i0 = (int64_t)blk * RX_TILE + wave * (RX_ROWS * 64) + lane;
+  uint64_t w[RX_ROWS];
+  uint32_t rk[RX_ROWS];
+#pragma unroll
+  for (int q = 0; q < RX_ROWS; q++) {
+    const int64_t i = i0 + q * 64;
+    w[q] = i < r.n ? src[i] : ~(uint64_t)0;
+  }
+  const uint64_t lower = ((uint64_t)1 << lane) - 1;
+#pragma unroll
+  for (int q = 0; q < RX_ROWS; q++) {
+    const bool valid = i0 + q * 64 < r.n;
+    const uint32_t d = (uint32_t)(w[q] >> r.shift) & 255u;
+    uint64_t same = __builtin_amdgcn_ballot_w64(valid);
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+      const bool bit = (d >> b) & 1u;
+      const uint64_t bal = __builtin_amdgcn_ballot_w64(bit);
+      same &= bit ? bal : ~bal;
+    }
+    const uint32_t below = (uint32_t)__builtin_popcountll(same & lower);
+    const uint32_t prev = cnt[wave][d];
+    rk[q] = prev + below;
+    // the first lane of each group of equal digits moves the wave's count on (LDS serves a wave in order)
+    if (valid && below == 0) cnt[wave][d] = prev + (uint32_t)__builtin_popcountll(same);
+  }
+  __syncthreads();
+  {
+    const uint32_t c0 = cnt[0][threadIdx.x], c1 = cnt[1][threadIdx.x], c2 = cnt[2][threadIdx.x];
+    cnt[0][threadIdx.x] = 0;
+    cnt[1][threadIdx.x] = c0;
+    cnt[2][threadIdx.x] = c0 + c1;
+    cnt[3][threadIdx.x] = c0 + c1 + c2;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < RX_ROWS; q++) {
+    if (i0 + q * 64 < r.n) {
+      const uint32_t d = (uint32_t)(w[q] >> r.shift) & 255u;
+      dst[base[d] + cnt[wave][d] + rk[q]] = w[q];
+    }
+  }
+}
+
+// Writes the sorted words out: indices, or the values they point at. DESC_VALUES: the
+// non-NaN prefix reversed.
+template <int DT, int PM, bool DESC_VALUES>
+__global__ __launch_bounds__(256) void rx_unpack_kernel(SortArgs a, const uint64_t *w, const uint32_t *nan_count, int nblk) {
+  const int64_t s = blockIdx.x / nblk, base = (int64_t)(blockIdx.x % nblk) * RX_TILE;
+  int64_t io, oo;
+  slice_offsets(a, s, io, oo);
+  const int64_t reals = DESC_VALUES ? a.n - (int64_t)nan_count[s] : 0;
+  for (int e = threadIdx.x; e < RX_TILE; e += 256) {
+    const int64_t i = base + e;
+    if (i >= a.n) break;
+    const int64_t from = DESC_VALUES && i < reals ? reals - 1 - i : i;
+    const uint64_t word = w[s * a.n + from];
+    if constexpr (PM == VALUE_ASC) {
+      // The value is the mapped key read backwards; only a zero (both signs share a key) and a
+      // NaN (its payload is not in the key) are fetched from the input through the index. A
+      // gather for every element cost a third of the whole sort.
+      using TR = Tr<DT>;
+      using C = typename TR::C;
+      using S = typename TR::S;
+      const uint32_t m = (uint32_t)(word >> 32);
+      bool direct = true;
+      C x;
+      if constexpr (TR::cat == CAT_FLOAT) {
+        direct = m != Packed<DT>::K_NAN && m != 0x80000000u;
+        const uint32_t u = (m & 0x80000000u) ? m ^ 0x80000000u : ~m;
+        x = (C)__builtin_bit_cast(float, u);
+      } else if constexpr (TR::cat == CAT_SINT) {
+        x = (C)(int32_t)(m ^ 0x80000000u);
+      } else {
+        x = (C)m;
+      }
+      if (direct) {
+        reinterpret_cast<S *>(a.out)[oo + i * a.out_axis] = TR::st(x);
+        continue;
+      }
+    }
+    packed_store<DT, PM>(a, oo, io, i, word);
+  }
+}
+
+template <int DT, int MODE>
+int radix_run(nxh_context *ctx, const char *op, SortArgs &a) {
+  constexpr int PM = MODE == VALUE_DESC ? VALUE_ASC : MODE;
+  constexpr bool DESC_VALUES = MODE == VALUE_DESC;
+  const int64_t nblk = (a.n + RX_TILE - 1) / RX_TILE, len = 256 * nblk, nseg = (len + RX_SEG - 1) / RX_SEG;
+  if (a.slices * nblk > 0x7fffffffLL || a.slices * nseg > 0x7fffffffLL || nblk > 0x7fffffffLL / 256)
+    return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
+  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+  const size_t words = up((size_t)(a.slices * a.n) * sizeof(uint64_t));
+  const size_t hist = up((size_t)(a.slices * len) * sizeof(uint32_t)), seg = up((size_t)(a.slices * nseg) * sizeof(uint32_t));
+  const size_t nans = up((size_t)a.slices * sizeof(uint32_t));
+  Scratch scratch(ctx);
+  if (scratch.get(0, 2 * words + hist + seg + nans)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_ALLOC);
+  char *p = (char *)scratch.p[0];
+  uint64_t *w0 = (uint64_t *)p, *w1 = (uint64_t *)(p + words);
+  RadixArgs r{};
+  r.hist = (uint32_t *)(p + 2 * words);
+  r.seg = (uint32_t *)(p + 2 * words + hist);
+  uint32_t *nan_count = (uint32_t *)(p + 2 * words + hist + seg);
+  r.slices = a.slices;
+  r.n = a.n;
+  r.nblk = (int)nblk;
+  r.nseg = (int)nseg;
+  const dim3 tiles((unsigned)(a.slices * nblk)), block(256);
+  nxh_set_path("sort_radix");
+  if (DESC_VALUES)
+    hipLaunchKernelGGL(rx_zero_kernel, dim3((unsigned)((a.slices + 255) / 256)), block, 0, ctx->stream, nan_count, a.slices);
+  hipLaunchKernelGGL((rx_pack_kernel<DT, PM, DESC_VALUES>), tiles, block, 0, ctx->stream, a, w0, nan_count, (int)nblk);
+  uint64_t *src = w0, *dst = w1;
+  for (int pass = 0; pass < 4; pass++) {
+    if (!(rx_pass_mask<DT>() >> pass & 1)) continue;
+    r.src = src;
+    r.dst = dst;
+    r.shift = 32 + 8 * pass;
+    hipLaunchKernelGGL(rx_hist_kernel, tiles, block, 0, ctx->stream, r);
+    hipLaunchKernelGGL(rx_scan_segments_kernel, dim3((unsigned)(a.slices * nseg)), block, 0, ctx->stream, r);
+    hipLaunchKernelGGL(rx_scan_totals_kernel, dim3((unsigned)a.slices), block, 0, ctx->stream, r);
+    hipLaunchKernelGGL(rx_scatter_kernel, tiles, block, 0, ctx->stream, r);
+    std::swap(src, dst);
+  }
+  hipLaunchKernelGGL((rx_unpack_kernel<DT, PM, DESC_VALUES>), tiles, block, 0, ctx->stream, a, src, nan_count, (int)nblk);
+  NXH_HIP(op, hipGetLastError());
+  return NXH_OK;
+}
+
 template <int DT, int MODE>
 int psort_run(nxh_context *ctx, const char *op, SortArgs &a) {
   if (a.n_pad <= PNL) {
@@ -483,6 +772,7 @@ int psort_run(nxh_context *ctx, const char *op, SortArgs &a) {
     NXH_HIP(op, hipGetLastError());
     return NXH_OK;
   }
+  if (a.n >= RX_MIN_N) return radix_run<DT, MODE>(ctx, op, a);
   const int64_t chunks = a.n_pad / PNL, blocks = a.slices * chunks;
   const int64_t pairs = a.slices * (a.n_pad / 2), quads = pairs / 2;
   if (blocks > 0x7fffffffLL || (pairs + 255) / 256 > 0x7fffffffLL)

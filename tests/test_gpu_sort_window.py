@@ -86,7 +86,11 @@ def test_sort_and_argsort_match_oracle(hip, oracle, d):
     assert hip.last_path() == "sort_lds"
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 1000, 4096, 4097, 20000, 70001])
+def path_for(n):
+    return "sort_lds" if n <= 4096 else ("sort_global" if n < 16384 else "sort_radix")
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 1000, 4096, 4097, 12000, 16383, 16384, 16385, 20000, 70001])
 def test_sort_lengths_across_both_paths(hip, oracle, n):
     rng = np.random.default_rng(n)
     x = rng.integers(-1000, 1000, (3, n)).astype(np.float32)
@@ -95,7 +99,7 @@ def test_sort_lengths_across_both_paths(hip, oracle, n):
     for desc in (False, True):
         same_bits_nan_any(logical(hip.sort(h, 1, desc)), logical(oracle.sort(o, 1, desc)), dt.float32, oracle, f"n={n}")
         same_bits(logical(hip.argsort(h, 1, desc)), logical(oracle.argsort(o, 1, desc)), f"argsort n={n}")
-    assert hip.last_path() == ("sort_lds" if n <= 4096 else "sort_global")
+    assert hip.last_path() == path_for(n)
     # along a strided axis (columns of the transposed tensor)
     ht, ot = pair(np.ascontiguousarray(x.T), dt.float32, hip, oracle)
     same_bits(logical(hip.argsort(ht, 0, False)), logical(oracle.argsort(ot, 0, False)), f"axis 0 n={n}")
@@ -103,6 +107,45 @@ def test_sort_lengths_across_both_paths(hip, oracle, n):
     z = (rng.integers(-50, 50, n) + 1j * rng.integers(-50, 50, n)).astype(np.complex128)
     hz, oz = pair(z, dt.complex128, hip, oracle)
     same_bits(logical(hip.sort(hz, 0, True)), logical(oracle.sort(oz, 0, True)), f"complex128 n={n}")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16, dt.float8_e4m3, dt.float8_e5m2, dt.int8, dt.uint8,
+                               dt.int16, dt.uint16, dt.int32, dt.uint32, dt.bool_], ids=lambda d: d.name)
+def test_radix_sort_matches_oracle(hip, oracle, d):
+    """Long slices of every packed dtype (some of their digit passes are skipped): values with many
+    ties, both zeros, NaNs and the extremes, both directions, sort and argsort, two slices of a
+    length that is no multiple of the tile, and a strided axis."""
+    rng = np.random.default_rng(600 + d.tag)
+    n = 16384 + 4096 + 37
+    x = values_for(d, (2, n), rng, oracle)
+    h, o = pair(x, d, hip, oracle)
+    for desc in (False, True):
+        got, want = logical(hip.sort(h, 1, desc)), logical(oracle.sort(o, 1, desc))
+        assert hip.last_path() == "sort_radix"
+        if d.is_float:
+            same_bits_nan_any(got, want, d, oracle, f"radix sort {d.name} desc {desc}")
+        else:
+            same_bits(got, want, f"radix sort {d.name} desc {desc}")
+        same_bits(logical(hip.argsort(h, 1, desc)), logical(oracle.argsort(o, 1, desc)), f"radix argsort {d.name} desc {desc}")
+    ht, ot = pair(np.ascontiguousarray(x.T), d, hip, oracle)
+    same_bits(logical(hip.argsort(ht, 0, True)), logical(oracle.argsort(ot, 0, True)), f"radix argsort {d.name} strided axis")
+    assert hip.last_path() == "sort_radix"
+    if d in (dt.float32, dt.int32, dt.uint32):  # every bit of the key in use
+        if d is dt.float32:
+            wide = (rng.standard_normal(50_000) * 10.0 ** rng.integers(-30, 30, 50_000)).astype(np.float32)
+            wide[::97] = np.nan
+            wide[1::101] = -wide[2::101][:wide[1::101].size]
+        else:
+            info = np.iinfo(d.np_storage)
+            wide = rng.integers(info.min, info.max, 50_000, endpoint=True).astype(d.np_storage)
+        hw, ow = pair(wide, d, hip, oracle)
+        for desc in (False, True):
+            got, want = logical(hip.sort(hw, 0, desc)), logical(oracle.sort(ow, 0, desc))
+            if d.is_float:
+                same_bits_nan_any(got, want, d, oracle, f"radix sort wide {d.name} desc {desc}")
+            else:
+                same_bits(got, want, f"radix sort wide {d.name} desc {desc}")
+            same_bits(logical(hip.argsort(hw, 0, desc)), logical(oracle.argsort(ow, 0, desc)), f"radix argsort wide {d.name} desc {desc}")
 
 
 def test_sort_large_properties(hip):
