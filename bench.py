@@ -266,7 +266,7 @@ def next_ops(hip, W, linalg=False):
           2 * 16384 * 1024 * 4)
     out[-1]["Mkeys/s"] = round(16384 * 1024 / out[-1]["ms"] / 1e3, 1)
     one = W.dev(rng.standard_normal(1 << 24).astype(np.float32), dt.float32)
-    timed("sort 2^24 f32, one slice (sort_global)", lambda: hip.sort(one, 0, False), 2 * (1 << 24) * 4, iters=5)
+    timed("sort 2^24 f32, one slice (sort_radix)", lambda: hip.sort(one, 0, False), 2 * (1 << 24) * 4, iters=5)
     out[-1]["Mkeys/s"] = round((1 << 24) / out[-1]["ms"] / 1e3, 1)
     for rec in out[-3:]:
         rec["bound"] = "lds"  # compare-exchange steps through LDS, not bytes, set the time
