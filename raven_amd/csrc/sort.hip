@@ -19,10 +19,12 @@
 // complex keys and one packed 64-bit word otherwise (see "packed keys").
 //   sort_lds     slices of up to 4096 elements (2048 for 16-byte keys): whole
 //                network in LDS, several short slices per block;
-//   sort_global  longer slices: pairs staged in scratch memory; chunks are
-//                sorted in LDS, then each merge level runs its long-distance
-//                exchanges as passes over global memory and finishes the
-//                short-distance ones in LDS.
+//   sort_global  longer slices of (key, index) pairs: staged in scratch memory;
+//                chunks are sorted in LDS, then each merge level runs its
+//                long-distance exchanges as passes over global memory and
+//                finishes the short-distance ones in LDS;
+//   sort_radix   longer slices of packed words: a stable radix sort over the key
+//                half (see "a radix sort" below).
 
 #include "fold_common.hpp"
 
@@ -388,92 +390,9 @@ __global__ __launch_bounds__(256) void psort_lds_kernel(SortArgs a, int spb) {
   }
 }
 
-template <int DT, int MODE>
-__global__ __launch_bounds__(256) void psort_chunks_kernel(SortArgs a) {
-  using TR = Tr<DT>;
-  using S = typename TR::S;
-  __shared__ uint64_t w[PNL];
-  const int64_t chunks = a.n_pad / PNL;
-  const int64_t s = blockIdx.x / chunks, base = (blockIdx.x % chunks) * PNL;
-  int64_t io, oo;
-  slice_offsets(a, s, io, oo);
-  for (int e = threadIdx.x; e < PNL; e += 256) {
-    const int64_t i = base + e;
-    w[e] = i < a.n ? Packed<DT>::template pack<MODE>(TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]), (uint32_t)i)
-                   : PACKED_PAD;
-  }
-  __syncthreads();
-  for (int kk = 2; kk <= PNL; kk <<= 1) packed_level(w, PNL, kk, kk >> 1, base, a.n_pad - 1);
-  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad + base;
-  for (int e = threadIdx.x; e < PNL; e += 256) gw[e] = w[e];
-}
-
-// Two exchange distances (j and j/2) of level kk in one pass over scratch: a
-// lane owns the four words i, i + j/2, i + j, i + 3j/2 that these two steps
-// keep among themselves. j/2 >= PNL.
-__global__ __launch_bounds__(256) void psort_exchange2_kernel(SortArgs a, int64_t kk, int64_t j) {
-  const int64_t quarter = a.n_pad / 4, h = j >> 1;
-  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (t >= a.slices * quarter) return;
-  const int64_t s = t / quarter, p = t % quarter;
-  // insert zero bits at positions log2(h) and log2(j)
-  int64_t i = ((p & ~(h - 1)) << 1) | (p & (h - 1));
-  i = ((i & ~(j - 1)) << 1) | (i & (j - 1));
-  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad;
-  const bool up = (i & kk) == 0;
-  uint64_t e0 = gw[i], e1 = gw[i + h], e2 = gw[i + j], e3 = gw[i + j + h];
-  auto cx = [&](uint64_t &x, uint64_t &y) {
-    const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
-    x = up ? lo : hi;
-    y = up ? hi : lo;
-  };
-  cx(e0, e2);
-  cx(e1, e3);
-  cx(e0, e1);
-  cx(e2, e3);
-  gw[i] = e0;
-  gw[i + h] = e1;
-  gw[i + j] = e2;
-  gw[i + j + h] = e3;
-}
-__global__ __launch_bounds__(256) void psort_exchange_kernel(SortArgs a, int64_t kk, int64_t j) {
-  const int64_t half = a.n_pad / 2;
-  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (t >= a.slices * half) return;
-  const int64_t s = t / half, p = t % half;
-  const int64_t i = ((p & ~(j - 1)) << 1) | (p & (j - 1)), l = i | j;
-  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad;
-  const bool up = (i & kk) == 0;
-  const uint64_t x = gw[i], y = gw[l];
-  const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
-  gw[i] = up ? lo : hi;
-  gw[l] = up ? hi : lo;
-}
-
-template <int DT, int MODE>
-__global__ __launch_bounds__(256) void psort_merge_kernel(SortArgs a, int64_t kk, int final) {
-  __shared__ uint64_t w[PNL];
-  const int64_t chunks = a.n_pad / PNL;
-  const int64_t s = blockIdx.x / chunks, base = (blockIdx.x % chunks) * PNL;
-  uint64_t *gw = reinterpret_cast<uint64_t *>(a.keys) + s * a.n_pad + base;
-  for (int e = threadIdx.x; e < PNL; e += 256) w[e] = gw[e];
-  __syncthreads();
-  packed_level(w, PNL, kk, PNL >> 1, base, a.n_pad - 1);
-  if (!final) {
-    for (int e = threadIdx.x; e < PNL; e += 256) gw[e] = w[e];
-    return;
-  }
-  int64_t io, oo;
-  slice_offsets(a, s, io, oo);
-  for (int e = threadIdx.x; e < PNL; e += 256) {
-    const int64_t i = base + e;
-    if (i < a.n) packed_store<DT, MODE>(a, oo, io, i, w[e]);
-  }
-}
-
 // ── long slices of packed words: a radix sort ──────────────────────────────
-// The network above costs log^2 n passes over a long slice; from RX_MIN_N elements on the
-// packed words are sorted least significant digit first instead, eight bits at a time, over
+// The network costs log^2 n passes over a slice that does not fit LDS; the packed words of
+// such a slice are sorted least significant digit first instead, eight bits at a time, over
 // the HIGH half only: the low half (the index) ascends with the position the words start at
 // and every pass is stable, so words with equal high halves stay in index order. The
 // descending value sort wants its ties in descending index order and its NaNs in ascending:
@@ -491,7 +410,6 @@ __global__ __launch_bounds__(256) void psort_merge_kernel(SortArgs a, int64_t kk
 constexpr int RX_TILE = 4096;
 constexpr int RX_ROWS = RX_TILE / 256;
 constexpr int RX_SEG = 4096;
-constexpr int64_t RX_MIN_N = 16384;
 
 template <int DT>
 constexpr int rx_pass_mask() {  // bit p: the pass over bits 8p .. 8p+7 of the mapped value is needed
@@ -616,8 +534,11 @@ __global__ __launch_bounds__(256) void rx_scan_totals_kernel(RadixArgs r) {
 }
 
 __global__ __launch_bounds__(256) void rx_scatter_kernel(RadixArgs r) {
+  __shared__ uint64_t sorted[RX_TILE];  // the tile in digit order, so that lanes next to each other write next to each other
   __shared__ uint32_t cnt[4][256];
-  __shared__ uint32_t base[256];
+  __shared__ uint32_t base[256];   // first output position of this tile's words with digit d
+  __shared__ uint32_t first[256];  // first position inside the tile of those words
+  __shared__ uint32_t tmp[4];
   const int64_t s = blockIdx.x / r.nblk;
   const int blk = (int)(blockIdx.x % r.nblk);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -630,7 +551,8 @@ __global__ __launch_bounds__(256) void rx_scatter_kernel(RadixArgs r) {
   __syncthreads();
   const uint64_t *src = r.src + s * r.n;
   uint64_t *dst = r.dst + s * r.n;
-  const int64_t i0 = (int64_t)blk * RX_TILE + wave * (RX_ROWS * 64) + lane;
+  const int64_t tile0 = (int64_t)blk * RX_TILE;
+  const int64_t i0 = tile0 + wave * (RX_ROWS * 64) + lane;
   uint64_t w[RX_ROWS];
   uint32_t rk[RX_ROWS];
 #pragma unroll
@@ -657,19 +579,34 @@ __global__ __launch_bounds__(256) void rx_scatter_kernel(RadixArgs r) {
     if (valid && below == 0) cnt[wave][d] = prev + (uint32_t)__builtin_popcountll(same);
   }
   __syncthreads();
+  uint32_t mine;
   {
-    const uint32_t c0 = cnt[0][threadIdx.x], c1 = cnt[1][threadIdx.x], c2 = cnt[2][threadIdx.x];
+    const uint32_t c0 = cnt[0][threadIdx.x], c1 = cnt[1][threadIdx.x], c2 = cnt[2][threadIdx.x], c3 = cnt[3][threadIdx.x];
     cnt[0][threadIdx.x] = 0;
     cnt[1][threadIdx.x] = c0;
     cnt[2][threadIdx.x] = c0 + c1;
     cnt[3][threadIdx.x] = c0 + c1 + c2;
+    mine = c0 + c1 + c2 + c3;
   }
+  uint32_t total;
+  first[threadIdx.x] = rx_block_scan(mine, tmp, total);  // (its barriers also publish cnt)
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < RX_ROWS; q++) {
     if (i0 + q * 64 < r.n) {
       const uint32_t d = (uint32_t)(w[q] >> r.shift) & 255u;
-      dst[base[d] + cnt[wave][d] + rk[q]] = w[q];
+      sorted[first[d] + cnt[wave][d] + rk[q]] = w[q];
+    }
+  }
+  __syncthreads();
+  const int count = (int)(r.n - tile0 < RX_TILE ? r.n - tile0 : RX_TILE);
+#pragma unroll
+  for (int q = 0; q < RX_ROWS; q++) {
+    const int p = q * 256 + threadIdx.x;
+    if (p < count) {
+      const uint64_t word = sorted[p];
+      const uint32_t d = (uint32_t)(word >> r.shift) & 255u;
+      dst[base[d] + ((uint32_t)p - first[d])] = word;
     }
   }
 }
@@ -772,27 +709,7 @@ int psort_run(nxh_context *ctx, const char *op, SortArgs &a) {
     NXH_HIP(op, hipGetLastError());
     return NXH_OK;
   }
-  if (a.n >= RX_MIN_N) return radix_run<DT, MODE>(ctx, op, a);
-  const int64_t chunks = a.n_pad / PNL, blocks = a.slices * chunks;
-  const int64_t pairs = a.slices * (a.n_pad / 2), quads = pairs / 2;
-  if (blocks > 0x7fffffffLL || (pairs + 255) / 256 > 0x7fffffffLL)
-    return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
-  Scratch scratch(ctx);
-  if (scratch.get(0, (size_t)(a.slices * a.n_pad) * sizeof(uint64_t))) return nxh_fail(NXH_FAILURE, op, NXH_ERR_ALLOC);
-  a.keys = scratch.p[0];
-  nxh_set_path("sort_global");
-  hipLaunchKernelGGL((psort_chunks_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a);
-  for (int64_t kk = 2 * (int64_t)PNL; kk <= a.n_pad; kk <<= 1) {
-    int64_t j = kk >> 1;
-    for (; (j >> 1) >= PNL; j >>= 2)
-      hipLaunchKernelGGL(psort_exchange2_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, ctx->stream, a, kk, j);
-    for (; j >= PNL; j >>= 1)
-      hipLaunchKernelGGL(psort_exchange_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, ctx->stream, a, kk, j);
-    hipLaunchKernelGGL((psort_merge_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a, kk,
-                       kk == a.n_pad ? 1 : 0);
-  }
-  NXH_HIP(op, hipGetLastError());
-  return NXH_OK;
+  return radix_run<DT, MODE>(ctx, op, a);
 }
 
 template <int DT, int MODE>

@@ -87,7 +87,7 @@ def test_sort_and_argsort_match_oracle(hip, oracle, d):
 
 
 def path_for(n):
-    return "sort_lds" if n <= 4096 else ("sort_global" if n < 16384 else "sort_radix")
+    return "sort_lds" if n <= 4096 else "sort_radix"  # packed dtypes; (key, index) pairs take sort_global
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 1000, 4096, 4097, 12000, 16383, 16384, 16385, 20000, 70001])
