@@ -4,10 +4,11 @@
 // unfold: (leading..., spatial...) -> (leading..., prod(kernel), L). Output
 // element (lead, tap kf, window w) is one input element, or zero when the tap
 // falls into the padding; every output is written once. A block owns one
-// (leading index, tap) row of the output and a run of its windows (the
-// contiguous axis), each lane eight of them 256 apart: the row is decoded once
-// per lane, the window coordinates once, and from then on they advance by an
-// odometer step, so no division is left in the per-element work.
+// leading index (several, when the rows are short) and a run of windows (the
+// contiguous axis), each lane eight of them 256 apart, and walks all taps of
+// them: the leading index and the window coordinates are decoded once per
+// lane, and from then on windows advance by an odometer step and taps by
+// another, so no division is left in the per-element work.
 //
 // fold: (leading..., prod(kernel), L) -> (leading..., output...). One lane per
 // OUTPUT element sums the taps that land on it, in ascending tap order and in
@@ -46,8 +47,8 @@ struct WindowArgs {
 // I is the type the index arithmetic runs in: int32_t whenever every extent,
 // element count and window coordinate fits (64-bit division is an order of
 // magnitude slower on this machine), int64_t otherwise. Memory offsets are
-// always 64-bit. `rows_per_block` > 1 packs several short rows into one block,
-// one window per lane.
+// always 64-bit. `leads_per_block` > 1 packs several leading indices with short
+// rows into one block, one window per lane.
 // AL > 0 (VW = 4 only): the last window dim has stride AL (1 or 2) over a unit-stride
 // input dim whose rows are whole, aligned 4-element vectors. The 3 AL + 1 input elements
 // behind a unit of four windows then lie in two or three aligned vectors, which are
@@ -56,39 +57,45 @@ struct WindowArgs {
 // offset modulo 4, the same for the whole row. Four separate element loads per lane,
 // 16 or 32 bytes apart from lane to lane, made the address path the bound.
 template <class E, class I, int KT, int VW, int AL = 0>
-__global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, int rows_per_block) {
+__global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, int leads_per_block, int taps_per_block) {
   // With VW > 1 a "window" below is a unit of VW consecutive windows of the last
   // window dim (a.L and a.win[KT-1] count units); the unit is stored as one vector.
+  // A block owns one leading index (several when the rows are short) and a run of windows, and
+  // walks ALL taps of them: the leading index and the window coordinates are decoded once per
+  // lane for kernel_prod x up to eight stores (one (leading, tap) row per block left 14 x 14
+  // images with one store per decode and a block per 196 outputs), and the taps of a window
+  // read neighbouring input elements, which the first tap leaves in the L1. When that leaves
+  // too few blocks to fill the chip, the taps are shared out over blockIdx.y.
   const I L = (I)a.L;
-  I row, w0;
+  I lead, w0;
   int reps = WINDOWS_PER_LANE;
-  if (rows_per_block > 1) {
-    const I lanes_per_row = 256 / rows_per_block;
-    row = (I)blockIdx.x * rows_per_block + (I)threadIdx.x / lanes_per_row;
-    w0 = (I)threadIdx.x % lanes_per_row;
+  if (leads_per_block > 1) {
+    const I lanes_per_lead = 256 / leads_per_block;
+    lead = (I)blockIdx.x * leads_per_block + (I)threadIdx.x / lanes_per_lead;
+    w0 = (I)threadIdx.x % lanes_per_lead;
     reps = 1;
     if (w0 >= L) return;
   } else {
-    row = (I)(blockIdx.x / (unsigned)wblocks);
+    lead = (I)(blockIdx.x / (unsigned)wblocks);
     w0 = (I)(blockIdx.x % (unsigned)wblocks) * (256 * WINDOWS_PER_LANE) + (I)threadIdx.x;
   }
-  if (row >= (I)a.rows) return;
-  I kf = row % (I)a.kernel_prod;
-  I lead = row / (I)a.kernel_prod;
-  I oo = kf * (I)a.tap_stride, io = 0;  // element offsets: I is 32 bits wide only when both spans fit
+  if (lead >= (I)(a.rows / a.kernel_prod)) return;
+  I oo_lead = 0, io = 0;  // element offsets: I is 32 bits wide only when both spans fit
   for (int d = a.ld - 1; d >= 0; d--) {
     const I c = lead % (I)a.lshape[d];
     lead /= (I)a.lshape[d];
-    oo += c * (I)a.l_out[d];
+    oo_lead += c * (I)a.l_out[d];
     io += c * (I)a.l_in[d];
   }
-  I tap[KT], wc[KT];  // tap: kc * dilation - pad_before; wc: window coordinate
+  I tap[KT], wc0[KT], wc[KT], kc[KT];  // tap: kc * dilation - pad_before; wc: window coordinate
   I rest = w0;
+  const I kf0 = (I)blockIdx.y * taps_per_block;
+  I kfr = kf0;
 #pragma unroll
   for (int d = KT - 1; d >= 0; d--) {
-    tap[d] = kf % (I)a.kernel[d] * (I)a.dilation[d] - (I)a.before[d];
-    kf /= (I)a.kernel[d];
-    wc[d] = rest % (I)a.win[d];
+    kc[d] = kfr % (I)a.kernel[d];
+    kfr /= (I)a.kernel[d];
+    wc0[d] = rest % (I)a.win[d];
     rest /= (I)a.win[d];
   }
   const E *in = reinterpret_cast<const E *>(a.in);
@@ -96,6 +103,7 @@ __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, in
   struct alignas(sizeof(E) * VW) Pack {
     E v[VW];
   };
+  I oo = 0;
   auto units = [&](auto r_c) {
     constexpr int R = decltype(r_c)::value;  // AL > 0: first element's place in its aligned vector
 #pragma unroll
@@ -149,15 +157,34 @@ __global__ __launch_bounds__(256) void unfold_kernel(WindowArgs a, I wblocks, in
       }
     }
   };
-  if constexpr (AL > 0) {
-    switch ((int)(tap[KT - 1] & 3)) {  // two's complement: also right for negative offsets
-      case 0: units(std::integral_constant<int, 0>{}); break;
-      case 1: units(std::integral_constant<int, 1>{}); break;
-      case 2: units(std::integral_constant<int, 2>{}); break;
-      default: units(std::integral_constant<int, 3>{}); break;
+  const I taps = kf0 + taps_per_block < (I)a.kernel_prod ? kf0 + taps_per_block : (I)a.kernel_prod;
+  for (I kf = kf0; kf < taps; kf++) {
+    oo = oo_lead + kf * (I)a.tap_stride;
+#pragma unroll
+    for (int d = 0; d < KT; d++) {
+      tap[d] = kc[d] * (I)a.dilation[d] - (I)a.before[d];
+      wc[d] = wc0[d];
     }
-  } else {
-    units(std::integral_constant<int, 0>{});
+    if constexpr (AL > 0) {
+      switch ((int)(tap[KT - 1] & 3)) {  // two's complement: also right for negative offsets
+        case 0: units(std::integral_constant<int, 0>{}); break;
+        case 1: units(std::integral_constant<int, 1>{}); break;
+        case 2: units(std::integral_constant<int, 2>{}); break;
+        default: units(std::integral_constant<int, 3>{}); break;
+      }
+    } else {
+      units(std::integral_constant<int, 0>{});
+    }
+    // next tap: the odometer over the kernel dims
+    bool carry = true;
+#pragma unroll
+    for (int d = KT - 1; d >= 0; d--) {
+      if (carry) {
+        kc[d]++;
+        carry = kc[d] >= (I)a.kernel[d];
+        if (carry) kc[d] = 0;
+      }
+    }
   }
 }
 
@@ -298,25 +325,30 @@ void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt) {
 
 template <class E, int VW, int AL = 0>
 int unfold_launch_v(nxh_context *ctx, const char *op, const WindowArgs &a, int kt) {
-  int rows_per_block = 1;
-  int64_t wblocks = (a.L + 256 * WINDOWS_PER_LANE - 1) / (256 * WINDOWS_PER_LANE), blocks = a.rows * wblocks;
-  if (a.L <= 128) {  // short rows: a power-of-two share of the block per row
+  const int64_t leads = a.rows / a.kernel_prod;
+  int leads_per_block = 1;
+  int64_t wblocks = (a.L + 256 * WINDOWS_PER_LANE - 1) / (256 * WINDOWS_PER_LANE), blocks = leads * wblocks;
+  if (a.L <= 256) {  // short rows: a power-of-two share of the block per leading index, one unit per lane
     int lanes = 1;
     while (lanes < a.L) lanes <<= 1;
-    rows_per_block = 256 / lanes;
-    blocks = (a.rows + rows_per_block - 1) / rows_per_block;
+    leads_per_block = 256 / lanes;
+    blocks = (leads + leads_per_block - 1) / leads_per_block;
   }
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
-  const dim3 grid((unsigned)blocks), block(256);
+  // all taps in one block unless that leaves the chip short of blocks (about 16 per compute unit)
+  const int64_t want = ((int64_t)(ctx->compute_units > 0 ? ctx->compute_units : 256) * 16 + blocks - 1) / blocks;
+  const int64_t groups = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, a.kernel_prod), 65535));
+  const int taps_per_block = (int)((a.kernel_prod + groups - 1) / groups);
+  const dim3 grid((unsigned)blocks, (unsigned)((a.kernel_prod + taps_per_block - 1) / taps_per_block)), block(256);
   const bool narrow = fits_int32(a) && spans_fit_int32(a, a.L * VW);
 #define NXH_UNFOLD_CASE(KT)                                                                                     \
   case KT:                                                                                                      \
     if (narrow)                                                                                                 \
       hipLaunchKernelGGL((unfold_kernel<E, int32_t, KT, VW, AL>), grid, block, 0, ctx->stream, a,               \
-                         (int32_t)wblocks, rows_per_block);                                                     \
+                         (int32_t)wblocks, leads_per_block, taps_per_block);                                    \
     else                                                                                                        \
       hipLaunchKernelGGL((unfold_kernel<E, int64_t, KT, VW, AL>), grid, block, 0, ctx->stream, a, wblocks,      \
-                         rows_per_block);                                                                       \
+                         leads_per_block, taps_per_block);                                                      \
     break;
   switch (kt) {
     NXH_UNFOLD_CASE(1)
