@@ -113,6 +113,9 @@ struct Args {
   void *C;
   int64_t lda, ldb, ldc;  // the non-unit stride of each matrix (elements)
   int64_t M, N, K;
+  // Extents that may be LOADED along M / N (>= M / N, whole 16-byte vectors): an operand
+  // contiguous along that dim may be padded past the logical edge.
+  int64_t Mld, Nld;
   uint32_t tiles_m, tiles_n, nbatch;
   // batch offsets: up to 4 broadcastable batch dims
   int nbd;
@@ -324,6 +327,10 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
   const int edge_m = EDGE ? (int)(a.M - m0 < BM ? a.M - m0 : BM) : BM;
   const int edge_n = EDGE ? (int)(a.N - n0 < BN ? a.N - n0 : BN) : BN;
+  // a k-contiguous operand clamps its rows to the logical edge; one contiguous along M / N
+  // clamps its vectors to the loadable extent
+  const int ledge_m = EDGE && !A_KC ? (int)(a.Mld - m0 < BM ? a.Mld - m0 : BM) : edge_m;
+  const int ledge_n = EDGE && !B_KC ? (int)(a.Nld - n0 < BN ? a.Nld - n0 : BN) : edge_n;
   // slab origin and per-slab advance of each operand
   const S *gA = (const S *)a.A + ao + (A_KC ? m0 * a.lda : m0);
   const S *gB = (const S *)a.B + bo + (B_KC ? n0 * a.ldb : n0);
@@ -349,8 +356,8 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
 #pragma unroll
     for (int i = 0; i < (NVA > NVB ? NVA : NVB); i++) {
       if (i % KSTEPS != ks) continue;
-      if (i < NVA) ra[i] = slab_load1<EL, A_KC, BM, THREADS, EDGE>(i, pA, a.lda, edge_m);
-      if (i < NVB) rb[i] = slab_load1<EL, B_KC, BN, THREADS, EDGE>(i, pB, a.ldb, edge_n);
+      if (i < NVA) ra[i] = slab_load1<EL, A_KC, BM, THREADS, EDGE>(i, pA, a.lda, ledge_m);
+      if (i < NVB) rb[i] = slab_load1<EL, B_KC, BN, THREADS, EDGE>(i, pB, a.ldb, ledge_n);
     }
   };
   auto stage_step = [&](int ks, S *nA, S *nB) {

@@ -59,6 +59,8 @@ struct GemmArgs {
   BatchDims batch;
   uint32_t batch0;   // first batch index of this launch
   int a_vec, b_vec;  // 16-byte loads allowed (alignment + stride multiple)
+  // tiled kernels only: extents that may be loaded along M / N (a padded copy's row length)
+  int64_t m_ld, n_ld;
 };
 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
@@ -942,10 +944,12 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   g.ldc = a.crs;
   if (!al16(g.A) || !al16(g.B) || g.lda % VE || g.ldb % VE) return -1;
   // an operand contiguous along M / N is read in whole 16-byte vectors
-  if ((!a_kc && a.M % VE) || (!b_kc && a.N % VE)) return -1;
+  if ((!a_kc && a.m_ld % VE) || (!b_kc && a.n_ld % VE)) return -1;
   g.M = a.M;
   g.N = a.N;
   g.K = a.K;
+  g.Mld = a.m_ld;
+  g.Nld = a.n_ld;
   g.nbatch = nbatch;
   g.nbd = a.batch.n;
   for (int i = 0; i < a.batch.n; i++) {
@@ -1049,6 +1053,137 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   return launch_tile_oriented<EL, gemm_tile::Shape256x256, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x256");
 }
 
+// ── padded copies for the tiled kernels ─────────────────────────────────────
+// The tiled kernels read whole 16-byte vectors of whole K-slabs. An operand whose rows are not
+// that (a [.., K, 196] matrix of unfolded 14 x 14 windows, a K of 196) is copied once into a
+// buffer whose contiguous dim is rounded up to whole vectors and whose K is rounded up to
+// whole slabs, the new positions filled with zeros (0 x 0 adds nothing to any sum; both operands
+// are padded along K). A broadcast batch dim stays a zero stride of the copy.
+struct RepackArgs {
+  const void *src;
+  void *dst;
+  int64_t rows, cols;    // logical extents: `cols` is the dim that becomes contiguous
+  int64_t prows, pcols;  // padded extents (pcols a multiple of the vector)
+  int64_t srs, scs;      // source strides of (row, col), elements
+  int nbd;
+  uint32_t bshape[MM_MAXB];
+  int64_t bsrc[MM_MAXB];  // source strides of the batch dims that are not broadcast
+  int64_t total;          // vectors to write
+};
+template <class S>
+__global__ __launch_bounds__(256) void gemm_repack_kernel(RepackArgs a) {
+  constexpr int VE = 16 / (int)sizeof(S);
+  const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (v >= a.total) return;
+  const int64_t vpr = a.pcols / VE;
+  const int64_t t = v / vpr, c0 = (v - t * vpr) * VE;
+  int64_t bidx = t / a.prows;
+  const int64_t r = t - bidx * a.prows;
+  int64_t so = 0;
+  for (int i = a.nbd - 1; i >= 0; i--) {
+    const int64_t q = bidx / a.bshape[i];
+    so += (bidx - q * a.bshape[i]) * a.bsrc[i];
+    bidx = q;
+  }
+  const S *src = (const S *)a.src + so + r * a.srs;
+  union {
+    U4 v4;
+    S s[VE];
+  } o;
+  o.v4 = U4{0, 0, 0, 0};
+  if (r < a.rows) {
+#pragma unroll
+    for (int j = 0; j < VE; j++)
+      if (c0 + j < a.cols) o.s[j] = src[(c0 + j) * a.scs];
+  }
+  ((U4 *)a.dst)[v] = o.v4;
+}
+
+// Copies one operand (kc: contiguous along K in the copy, else along its M / N dim) and
+// rewrites its strides in place. `bstr` are the operand's batch strides.
+template <class S>
+static int repack_operand(nxh_context *ctx, const GemmArgs &g, const void *src, bool kc, int64_t rows_mn, int64_t Kp,
+                          int64_t &stride_mn, int64_t &stride_k, int64_t *bstr, int64_t &ld_mn, void **block) {
+  constexpr int VE = 16 / (int)sizeof(S);
+  RepackArgs r{};
+  r.src = src;
+  if (kc) {
+    r.rows = r.prows = rows_mn;
+    r.cols = g.K;
+    r.pcols = Kp;
+    r.srs = stride_mn;
+    r.scs = stride_k;
+  } else {
+    r.rows = g.K;
+    r.prows = Kp;
+    r.cols = rows_mn;
+    r.pcols = (rows_mn + VE - 1) / VE * VE;
+    r.srs = stride_k;
+    r.scs = stride_mn;
+  }
+  // the copy's batch layout: dense over the dims the operand really has
+  int64_t run = r.prows * r.pcols, nstr[MM_MAXB] = {};
+  for (int i = g.batch.n - 1; i >= 0; i--) {
+    if (bstr[i] == 0) continue;
+    nstr[i] = run;
+    run *= g.batch.shape[i];
+  }
+  for (int i = 0; i < g.batch.n; i++) {
+    if (bstr[i] == 0) continue;
+    r.bshape[r.nbd] = g.batch.shape[i];
+    r.bsrc[r.nbd] = bstr[i];
+    r.nbd++;
+  }
+  if (run > ((int64_t)1 << 32)) return -1;  // more than the fast path is worth
+  int rc = nxh_alloc_locked(ctx, (size_t)run * sizeof(S), block);
+  if (rc) return rc;
+  r.dst = *block;
+  r.total = run / VE;
+  hipLaunchKernelGGL((gemm_repack_kernel<S>), dim3((unsigned)((r.total + 255) / 256)), dim3(256), 0, ctx->stream, r);
+  NXH_HIP("matmul", hipGetLastError());
+  if (kc) {
+    stride_mn = Kp;
+    stride_k = 1;
+  } else {
+    stride_mn = 1;
+    stride_k = r.pcols;
+    ld_mn = r.pcols;
+  }
+  for (int i = 0; i < g.batch.n; i++) bstr[i] = nstr[i];
+  return NXH_OK;
+}
+
+// The tiled path over padded copies of the operands that do not fit it as they are. -1: not
+// worth it or not possible (the caller falls back to the general kernel).
+template <class EL>
+static int try_tile_repacked(nxh_context *ctx, const GemmArgs &a0, uint32_t nbatch, bool al_a, bool al_b) {
+  using S = typename EL::S;
+  constexpr int VE = EL::VE, BK = gemm_tile::Geo<EL>::BK;
+  if (a0.ccs != 1 || a0.batch.n > 4 || a0.M < 32 || a0.N < 32 || a0.K < 32) return -1;
+  // two more launches and a pass over the copied operand: only for products that outweigh them
+  if ((double)a0.M * (double)a0.N * (double)a0.K * (double)nbatch < (double)(1 << 27)) return -1;
+  GemmArgs a = a0;
+  const int64_t Kp = (a.K + BK - 1) / BK * BK;
+  const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
+  const bool fit_a = Kp == a.K && al_a && al16(a.A) && (a_kc ? a.ars % VE == 0 : (a.acs % VE == 0 && a.M % VE == 0));
+  const bool fit_b = Kp == a.K && al_b && al16(a.B) && (b_kc ? a.bcs % VE == 0 : (a.brs % VE == 0 && a.N % VE == 0));
+  if (fit_a && fit_b) return -1;  // the tiled path refused for another reason
+  void *blk_a = nullptr, *blk_b = nullptr;
+  int rc = NXH_OK;
+  if (!fit_a) rc = repack_operand<S>(ctx, a, a.A, a_kc, a.M, Kp, a.ars, a.acs, a.batch.a, a.m_ld, &blk_a);
+  if (rc == NXH_OK && !fit_b) rc = repack_operand<S>(ctx, a, a.B, b_kc, a.N, Kp, a.bcs, a.brs, a.batch.b, a.n_ld, &blk_b);
+  if (rc == NXH_OK) {
+    if (blk_a) a.A = blk_a;
+    if (blk_b) a.B = blk_b;
+    a.K = Kp;
+    rc = try_tile<EL>(ctx, a, nbatch, true, true);
+    if (rc == NXH_OK) nxh_set_path("gemm_tile_padded");
+  }
+  if (blk_a) nxh_free_locked(ctx, blk_a);
+  if (blk_b) nxh_free_locked(ctx, blk_b);
+  return rc;
+}
+
 template <class MM>
 static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool batch_aligned_a,
                           bool batch_aligned_b) {
@@ -1069,6 +1204,7 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
     using EL = std::conditional_t<MM::DT == NXH_F32, gemm_tile::ElF32,
                                   std::conditional_t<MM::DT == NXH_BF16, gemm_tile::ElBF16, gemm_tile::ElF16>>;
     int rc = try_tile<EL>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
+    if (rc == -1) rc = try_tile_repacked<EL>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
     if (rc != -1) return rc;
   }
   // 16-byte loads need an aligned base and every other stride a multiple of VL
@@ -1179,8 +1315,8 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
   g.A = (const char *)A->data + A->offset * es;
   g.B = (const char *)B->data + B->offset * es;
   g.C = (char *)C->data + C->offset * es;
-  g.M = m;
-  g.N = n;
+  g.M = g.m_ld = m;
+  g.N = g.n_ld = n;
   g.K = k;
   g.batch.n = nb;
   bool al_a = true, al_b = true;

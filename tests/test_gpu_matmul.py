@@ -276,6 +276,56 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
     check(hip, oracle, d, hip.shrink(hw, [(0, 256), (0, 128)]), hb2, wide[:, 32:160], b4[0, 0][:, :256], "big sliced A")
 
 
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_padded_copies(hip, oracle, d):
+    """Large products whose operands are not whole 16-byte vectors of whole K-slabs (the
+    [C k k, 14 x 14] matrices of unfolded windows, their transposes, a ragged K) run the
+    tiled kernels over zero-padded copies; the inputs are left as they were."""
+    rng = np.random.default_rng(1450 + d.tag)
+    # weights broadcast over a batch of window matrices: [co, ckk] x [n, ckk, L]
+    for (n, co, ckk, L) in [(8, 256, 576, 196), (32, 128, 1152, 49)]:
+        w = encode(rng.standard_normal((1, co, ckk)), d, oracle)
+        cols = encode(rng.standard_normal((n, ckk, L)), d, oracle)
+        hw, _ = pair(w, d, hip, oracle, lambda B, t: B.expand(t, (n, co, ckk)))
+        hc, oc = pair(cols, d, hip, oracle)
+        check(hip, oracle, d, hw, hc, np.broadcast_to(w, (n, co, ckk)), cols, f"conv {co}x{ckk}x{L}")
+        # (rows of 196 floats are whole vectors already)
+        vec_rows = d is dt.float32 and L % 4 == 0
+        assert hip.last_path() == ("gemm_tile_128x128" if vec_rows else "gemm_tile_padded"), hip.last_path()
+        same_bits(logical(hc), cols, "input untouched")
+        # the weight gradient's shape: K is the ragged dim of both operands
+        dy = encode(rng.standard_normal((n, co, L)), d, oracle)
+        hd = pair(dy, d, hip, oracle)[0]
+        hct = pair(cols, d, hip, oracle, lambda B, t: B.permute(t, (0, 2, 1)))[0]
+        check(hip, oracle, d, hd, hct, dy, np.swapaxes(cols, 1, 2), f"ragged K {co}x{L}x{ckk}")
+        assert hip.last_path() == "gemm_tile_padded", hip.last_path()
+        # the input gradient's shape: A is the transposed weight (contiguous along M)
+        hwt = pair(w[0], d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))[0]
+        check(hip, oracle, d, hwt, hd, w[0].T, dy, f"transposed A {ckk}x{co}x{L}")
+        assert hip.last_path() == ("gemm_tile_128x128" if vec_rows else "gemm_tile_padded"), hip.last_path()
+    # an odd row pitch of a k-contiguous A and an odd M of an M-contiguous A
+    a = encode(rng.standard_normal((515, 517)), d, oracle)
+    b = encode(rng.standard_normal((512, 519)), d, oracle)
+    ha = pair(a, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 515), (1, 513)]))[0]
+    check(hip, oracle, d, ha, pair(b, d, hip, oracle)[0], a[:, 1:513], b, "odd pitches")
+    assert hip.last_path() == "gemm_tile_padded", hip.last_path()
+    at = np.ascontiguousarray(a[:, 1:513].T)
+    hat = pair(at, d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))[0]
+    check(hip, oracle, d, hat, pair(b, d, hip, oracle)[0], a[:, 1:513], b, "odd M, M-contiguous A")
+    assert hip.last_path() == "gemm_tile_padded", hip.last_path()
+    # a NaN or an infinity next to the padding stays where it is and reaches no other element
+    a = encode(rng.standard_normal((256, 196)), d, oracle)
+    b = encode(rng.standard_normal((196, 3000)), d, oracle)
+    af, bf_ = decode(a, d, oracle).copy(), decode(b, d, oracle).copy()
+    af[7, 195] = np.inf
+    bf_[195, 2999] = np.nan
+    a, b = encode(af, d, oracle), encode(bf_, d, oracle)
+    got = decode(logical(hip.matmul(pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0])), d, oracle)
+    assert hip.last_path() == "gemm_tile_padded", hip.last_path()
+    want = ref_f64(a, b, d, oracle)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+
+
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
 def test_matmul_direct_to_lds_kernel(hip, oracle, d):
     """The large-product form (operands straight from global memory into swizzled LDS
