@@ -107,6 +107,8 @@ struct Shape {
 using Shape256x256 = Shape<4, 2, 2, 4>;
 using Shape128x128 = Shape<2, 2, 2, 2>;
 using Shape256x64 = Shape<4, 1, 2, 2>;
+using Shape128x64 = Shape<2, 2, 2, 1>;
+using Shape64x64 = Shape<2, 2, 1, 1>;
 
 struct Args {
   const void *A, *B;

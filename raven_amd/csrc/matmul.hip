@@ -909,8 +909,8 @@ static int launch_dl_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, b
     return -1;
   }
 }
-// 0: pick by shape; 256 / 192 / 128 / 64: force that block shape (192: 128 x 192, direct to
-// LDS; 128: the register-staged 128 x 128); 257: the 256 shape in its
+// 0: pick by shape; 256 / 192 / 128 / 64 / 1264 / 6464: force that block shape (192: 128 x 192, direct to
+// LDS; 128: the register-staged 128 x 128; 1264: 128 x 64; 6464: 64 x 64, f32); 257: the 256 shape in its
 // register-staged form (tuning aid, read once from NXH_GEMM_TILE)
 static int forced_tile() {
   static const int v = [] {
@@ -1001,6 +1001,14 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       const double c128 = (double)((tiles(128, 128) + 2 * cus - 1) / (2 * cus)) * 0.6;
       pick = c256 <= c128 ? 256 : 128;
     }
+    // Fewer blocks than half the compute units: half blocks (128 x 64, four waves of 64 x 32)
+    // put twice as many of them to work (f32 1024^3: 64 blocks 68 us, 128 half blocks 40 us).
+    if (pick != 256 && !(EPI && epi->gelu) && (pick == 64 ? tiles(256, 64) : tiles(128, 128)) * members <= cus / 2)
+      pick = 1264;
+    // f32 (a compute unit's f32 matrix rate is a sixteenth of its 16-bit rate, so a block's
+    // time is all arithmetic): quarter blocks, while they still leave units idle
+    if constexpr (EL::F32)
+      if (pick == 1264 && tiles(128, 64) * members <= cus / 2) pick = 6464;
   }
   // Whole tiles of 16-bit operands go straight into LDS (gemm_dl.hpp; load offsets are 32-bit:
   // 256 rows of a k-contiguous operand must stay below 4 GiB, and every row segment the
@@ -1037,16 +1045,61 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   }
   if (g.gelu && (a.M % 128 || a.N % 128)) return -1;
   if (pick == 192) pick = 128;
+  if constexpr (EL::F32 && !EPI) {
+    // One f32 product whose blocks leave three quarters of the units idle and whose K is long (a
+    // weight gradient: [768, 8192] x [8192, 768]): K is cut into `split` equal runs of whole slabs,
+    // walked as a batch dim that writes [split][M][N] partial sums, which a second kernel adds in
+    // run order (a fixed order: the same bits on every call).
+    if (nbatch == 1 && a.batch.n == 0 && (pick == 1264 || pick == 6464)) {
+      const int64_t blocks = pick == 6464 ? tiles(64, 64) : tiles(128, 64);
+      const int64_t slabs = a.K / BK;
+      int64_t split = std::min<int64_t>(cus / blocks, slabs / 4);
+      while (split > 1 && slabs % split) split--;
+      if (split >= 2 && blocks * 4 <= cus && a.M * a.N % 4 == 0) {
+        void *part = nullptr;
+        int rc = nxh_alloc_locked(ctx, (size_t)split * a.M * a.N * sizeof(float), &part);
+        if (rc) return rc;
+        gemm_tile::Args gs = g;
+        gs.K = a.K / split;
+        gs.nbatch = (uint32_t)split;
+        gs.nbd = 1;
+        gs.bshape[0] = (uint32_t)split;
+        gs.ba[0] = gs.K * (a_kc ? 1 : g.lda);
+        gs.bb[0] = gs.K * (b_kc ? 1 : g.ldb);
+        gs.bc[0] = a.M * a.N;
+        gs.C = part;
+        gs.ldc = a.N;
+        rc = pick == 6464 ? launch_tile_oriented<EL, gemm_tile::Shape64x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_64x64_splitk")
+                          : launch_tile_oriented<EL, gemm_tile::Shape128x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
+        if (rc == NXH_OK) {
+          const int64_t total = a.M * a.N;
+          hipLaunchKernelGGL((skinny_finish_kernel<NXH_F32>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0,
+                             ctx->stream, (const float *)part, g.C, a.M, a.N, (int)split, g.ldc, (int64_t)1);
+          hipError_t e = hipGetLastError();
+          if (e != hipSuccess) rc = nxh_hip_fail("matmul", e);
+        }
+        nxh_free_locked(ctx, part);
+        return rc;
+      }
+    }
+  }
+  if constexpr (EL::F32) {
+    if (pick == 6464)
+      return launch_tile_oriented<EL, gemm_tile::Shape64x64, EPI>(ctx, g, a_kc, b_kc, EPI ? "linear_tile_64x64" : "gemm_tile_64x64");
+  }
   if constexpr (EPI) {
     // Two block shapes are enough for the epilogue family; f16 keeps to the small one (its
     // conversions make the 256x256 epilogue too large to stay in registers).
     constexpr bool big_ok = EL::F32 || EL::BF16;
+    if (pick == 1264)
+      return launch_tile_oriented<EL, gemm_tile::Shape128x64, true>(ctx, g, a_kc, b_kc, "linear_tile_128x64");
     if (pick == 64 || !big_ok || (g.gelu && (a.M % 256 || a.N % 256))) pick = 128;
     if (pick == 128)
       return launch_tile_oriented<EL, gemm_tile::Shape128x128, true>(ctx, g, a_kc, b_kc, "linear_tile_128x128");
     if constexpr (big_ok)
       return launch_tile_oriented<EL, gemm_tile::Shape256x256, true>(ctx, g, a_kc, b_kc, "linear_tile_256x256");
   }
+  if (pick == 1264) return launch_tile_oriented<EL, gemm_tile::Shape128x64, false>(ctx, g, a_kc, b_kc, "gemm_tile_128x64");
   if (pick == 64) return launch_tile_oriented<EL, gemm_tile::Shape256x64, false>(ctx, g, a_kc, b_kc, "gemm_tile_256x64");
   if (pick == 128)
     return launch_tile_oriented<EL, gemm_tile::Shape128x128, false>(ctx, g, a_kc, b_kc, "gemm_tile_128x128");

@@ -358,8 +358,9 @@ def test_linear_then_gelu_is_one_gemm(hip, oracle, d, rows, inputs, outputs):
             hip.linear_gelu_tanh(x, w, b)
 
 
-@pytest.mark.parametrize("rows,width,path", [(192, 256, "linear_tile_128x128"), (256, 384, "linear_dl_128x192")],
-                         ids=["staged_tiles", "direct_to_lds"])
+@pytest.mark.parametrize("rows,width,path", [(192, 256, "linear_tile_128x64"), (1408, 256, "linear_tile_128x128"),
+                                             (1024, 384, "linear_dl_128x192")],
+                         ids=["half_blocks", "staged_tiles", "direct_to_lds"])
 def test_linear_layers_over_one_input_share_a_launch(hip, oracle, rows, width, path):
     """q, k and v of an attention layer: three linear layers over the same x. Recorded one after the
     other, launched as one GEMM over the three weight matrices, each result the bits of its own call."""

@@ -219,13 +219,18 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
     """The LDS-tiled kernel family: every block shape, whole and ragged tiles,
     all four operand orientations, batched and batch-broadcast."""
     rng = np.random.default_rng(1400 + d.tag)
+    # (blocks of 128 x 128 up to half the compute units become 128 x 64, and for f32 64 x 64; one
+    # f32 product with a long K is cut along K on top of that)
+    small = "gemm_tile_64x64" if d is dt.float32 else "gemm_tile_128x64"
     cases = [
         # whole tiles
-        (256, 64, 256, "gemm_tile_128x128"), (512, 192, 768, "gemm_tile_128x128"),
-        (768, 320, 256, "gemm_tile_128x128"), (512, 128, 64, "gemm_tile_256x64"),
+        (256, 64, 256, small), (512, 192, 768, small),
+        (768, 320, 256, small), (512, 128, 64, small),
+        (1536, 64, 1664, "gemm_tile_128x128"), (33024, 64, 64, "gemm_tile_256x64"),
         (4096, 64, 4096, "gemm_tile_256x256"),
         # ragged in M and N (multiples of 8, so M/N-contiguous operands qualify too)
-        (200, 64, 136, "gemm_tile_128x128"), (264, 128, 40, "gemm_tile_256x64"),
+        (200, 64, 136, small), (264, 128, 40, small),
+        (1528, 64, 1672, "gemm_tile_128x128"), (33000, 128, 40, "gemm_tile_256x64"),
         (4000, 64, 4088, "gemm_tile_256x256"),
     ]
     for (m, k, n, path) in cases:
@@ -242,22 +247,22 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
                 check(hip, oracle, d, ha, hb, a, b, f"tile {m}x{k}x{n} ta={ta} tb={tb}")
                 # whole 256-tiles of 16-bit operands take the direct-to-LDS form
                 want_path = "gemm_dl_256x256" if (path, m % 256, n % 256) == ("gemm_tile_256x256", 0, 0) and d is not dt.float32 else path
-                # and 128 x 192 blocks where they fit and A is k-contiguous
-                if d is not dt.float32 and not ta and want_path == "gemm_tile_128x128" and (m % 128, n % 192) == (0, 0):
-                    want_path = "gemm_dl_128x192"
+                if d is dt.float32 and k >= 256 and want_path == small:
+                    want_path += "_splitk"
                 assert hip.last_path() == want_path, (m, k, n, ta, tb, hip.last_path())
     # odd M and N: only K-contiguous operands (A row-major, B given as its transpose) qualify
     a = encode(rng.standard_normal((203, 128)), d, oracle)
     b = encode(rng.standard_normal((128, 157)), d, oracle)
     hb, _ = pair(np.ascontiguousarray(b.T), d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], hb, a, b, "tile odd edges")
-    assert hip.last_path() == "gemm_tile_128x128"
+    assert hip.last_path() == small
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "odd N, row-major B")
     assert hip.last_path() == "gemm_mfma"
     # odd N on every block shape: the rows of C start at every 2-byte alignment, and 16-bit
     # results leave as 16-byte stores at the aligned addresses plus single elements at the ends
-    for (m, k, n, path) in [(4000, 64, 4087, "gemm_tile_256x256"), (264, 128, 57, "gemm_tile_256x64"),
-                            (203, 192, 1031, "gemm_tile_128x128"), (131, 64, 9, "gemm_tile_256x64")]:
+    for (m, k, n, path) in [(4000, 64, 4087, "gemm_tile_256x256"), (264, 128, 57, small),
+                            (203, 192, 1031, small), (131, 64, 9, small),
+                            (1531, 64, 1671, "gemm_tile_128x128"), (33001, 64, 57, "gemm_tile_256x64")]:
         a = encode(rng.standard_normal((m, k)), d, oracle)
         b = encode(rng.standard_normal((k, n)), d, oracle)
         hb, _ = pair(np.ascontiguousarray(b.T), d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))
@@ -291,7 +296,7 @@ def test_matmul_padded_copies(hip, oracle, d):
         check(hip, oracle, d, hw, hc, np.broadcast_to(w, (n, co, ckk)), cols, f"conv {co}x{ckk}x{L}")
         # (rows of 196 floats are whole vectors already)
         vec_rows = d is dt.float32 and L % 4 == 0
-        assert hip.last_path() == ("gemm_tile_128x128" if vec_rows else "gemm_tile_padded"), hip.last_path()
+        assert hip.last_path() == ("gemm_tile_64x64" if vec_rows else "gemm_tile_padded"), hip.last_path()
         same_bits(logical(hc), cols, "input untouched")
         # the weight gradient's shape: K is the ragged dim of both operands
         dy = encode(rng.standard_normal((n, co, L)), d, oracle)
@@ -302,7 +307,7 @@ def test_matmul_padded_copies(hip, oracle, d):
         # the input gradient's shape: A is the transposed weight (contiguous along M)
         hwt = pair(w[0], d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))[0]
         check(hip, oracle, d, hwt, hd, w[0].T, dy, f"transposed A {ckk}x{co}x{L}")
-        assert hip.last_path() == ("gemm_tile_128x128" if vec_rows else "gemm_tile_padded"), hip.last_path()
+        assert hip.last_path() == ("gemm_tile_128x64" if vec_rows else "gemm_tile_padded"), hip.last_path()
     # an odd row pitch of a k-contiguous A and an odd M of an M-contiguous A
     a = encode(rng.standard_normal((515, 517)), d, oracle)
     b = encode(rng.standard_normal((512, 519)), d, oracle)
@@ -324,6 +329,40 @@ def test_matmul_padded_copies(hip, oracle, d):
     assert hip.last_path() == "gemm_tile_padded", hip.last_path()
     want = ref_f64(a, b, d, oracle)
     assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+
+
+def test_matmul_f32_few_blocks_cut_along_k(hip, oracle):
+    """One f32 product with few output blocks and a long K (a weight gradient) is cut along K; the
+    partial sums are added in a fixed order: within the matmul tolerance, and the same bits every call."""
+    d = dt.float32
+    rng = np.random.default_rng(1460)
+    T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
+    for (m, k, n, path) in [(128, 4096, 64, "gemm_tile_64x64_splitk"), (256, 2048, 256, "gemm_tile_64x64_splitk"),
+                            (200, 1024, 72, "gemm_tile_64x64_splitk"), (768, 8192, 768, "gemm_tile_64x64"),
+                            (64, 96, 64, "gemm_tile_64x64")]:
+        a = encode(rng.standard_normal((m, k)), d, oracle)
+        b = encode(rng.standard_normal((k, n)), d, oracle)
+        for ta in (False, True):
+            for tb in (False, True):
+                ha, _ = pair(np.ascontiguousarray(a.T) if ta else a, d, hip, oracle, T if ta else None)
+                hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle, T if tb else None)
+                check(hip, oracle, d, ha, hb, a, b, f"{m}x{k}x{n} ta={ta} tb={tb}")
+                assert hip.last_path() == path, (m, k, n, ta, tb, hip.last_path())
+                first = logical(hip.matmul(ha, hb))
+                same_bits(logical(hip.matmul(ha, hb)), first, "same bits on every call")
+    # into a strided output: a column slice of a wider result
+    a = encode(rng.standard_normal((128, 2048)), d, oracle)
+    b = encode(rng.standard_normal((2048, 64)), d, oracle)
+    ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
+    dense = logical(hip.matmul(ha, hb))
+    wide = hip.reshape(hip.from_host(np.zeros(128 * 80, np.float32), d), (128, 80))
+    import ctypes as C
+    view = hip.shrink(wide, [(0, 128), (8, 72)])
+    hip._check(hip._lib.nxh_matmul(hip._h, C.byref(view._desc()), C.byref(ha._desc()), C.byref(hb._desc())))
+    assert hip.last_path() == "gemm_tile_64x64_splitk"
+    w = logical(wide)
+    same_bits(np.ascontiguousarray(w[:, 8:72]), dense, "strided output")
+    assert not w[:, :8].any() and not w[:, 72:].any()
 
 
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
@@ -374,7 +413,7 @@ def test_matmul_and_linear_on_128x192_blocks(hip, oracle, d):
     bit the sequence of primitives, whose matmul takes the same kernel."""
     rng = np.random.default_rng(1700 + d.tag)
     T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
-    for m, k, n in ((1024, 64, 768), (1024, 192, 768), (384, 448, 192), (1024, 3200, 384)):
+    for m, k, n in ((3072, 64, 768), (3072, 192, 768), (8448, 448, 192), (5632, 3200, 384)):
         a = encode(rng.standard_normal((m, k)) * 0.5, d, oracle)
         b = encode(rng.standard_normal((k, n)) * 0.5, d, oracle)
         want = ref_f64(a, b, d, oracle)
@@ -385,16 +424,16 @@ def test_matmul_and_linear_on_128x192_blocks(hip, oracle, d):
             assert hip.last_path() == "gemm_dl_128x192", (m, k, n, tb, hip.last_path())
             ulp = 2.0 ** (-8 if d is dt.bfloat16 else -11)
             assert np.all(np.abs(got - want) <= ulp * 2 * np.abs(want) + np.sqrt(k) * 2e-6), (m, k, n, tb, float(np.abs(got - want).max()))
-    a = encode(rng.standard_normal((3, 256, 128)), d, oracle)
+    a = encode(rng.standard_normal((3, 2304, 128)), d, oracle)
     b = encode(rng.standard_normal((128, 576)), d, oracle)
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "128x192 batched x one B")
     assert hip.last_path() == "gemm_dl_128x192"
-    a4 = encode(rng.standard_normal((2, 1, 128, 64)), d, oracle)
-    b4 = encode(rng.standard_normal((1, 3, 64, 192)), d, oracle)
+    a4 = encode(rng.standard_normal((2, 1, 1536, 64)), d, oracle)
+    b4 = encode(rng.standard_normal((1, 3, 64, 768)), d, oracle)
     check(hip, oracle, d, pair(a4, d, hip, oracle)[0], pair(b4, d, hip, oracle)[0], a4, b4, "128x192 both batch-broadcast")
     assert hip.last_path() == "gemm_dl_128x192"
     # the fused linear
-    for xs, ws in (((4, 128, 256), (256, 768)), ((640, 1024), (1024, 192))):
+    for xs, ws in (((4, 1152, 256), (256, 768)), ((8448, 1024), (1024, 192))):
         x = encode(rng.standard_normal(xs) * 0.5, d, oracle)
         w = encode(rng.standard_normal(ws) * 0.1, d, oracle)
         bias = encode(rng.standard_normal(ws[-1]), d, oracle)
