@@ -994,7 +994,29 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   // 256x256 block (8 waves, 144 KiB of LDS) fills a CU; two 128x128 blocks fit,
   // each a quarter of the work at about 0.8 of the big tile's efficiency.
   int pick = forced_tile();
-  if (!pick) {
+  if (!pick && EL::F32) {
+    // f32: a compute unit's f32 matrix rate is a sixteenth of its 16-bit rate, so a block's time
+    // is all arithmetic and the shapes differ only in what they leave idle: rounds of one block
+    // per unit x the block's area (ragged edges count as whole blocks) x the shape's measured cost
+    // per flop against the 256 x 256 block (4096^3: 138 TFLOP/s there, 123 with half blocks;
+    // 1024^3 on quarter blocks about 100 inside the K loop).
+    struct Cand {
+      int pick, bm, bn;
+      double pen;
+    };
+    const Cand cands[] = {{256, 256, 256, 1.0}, {128, 128, 128, 1.12}, {64, 256, 64, 1.12},
+                          {1264, 128, 64, 1.15}, {6464, 64, 64, 1.3}};
+    double best = 0.0;
+    for (const Cand &c : cands) {
+      if (c.pick == 64 && a.N > 64) continue;
+      if (EPI && epi->gelu && c.pick != 256 && c.pick != 128) continue;
+      const double cost = (double)((tiles(c.bm, c.bn) * members + cus - 1) / cus) * c.bm * c.bn * c.pen;
+      if (!pick || cost < best) {
+        pick = c.pick;
+        best = cost;
+      }
+    }
+  } else if (!pick) {
     if (a.N <= 64) pick = 64;
     else {
       const double c256 = (double)((tiles(256, 256) + cus - 1) / cus);
@@ -1002,13 +1024,9 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       pick = c256 <= c128 ? 256 : 128;
     }
     // Fewer blocks than half the compute units: half blocks (128 x 64, four waves of 64 x 32)
-    // put twice as many of them to work (f32 1024^3: 64 blocks 68 us, 128 half blocks 40 us).
+    // put twice as many of them to work (bf16 [1024,768] x [768,768]: 9.5 -> 7.9 us).
     if (pick != 256 && !(EPI && epi->gelu) && (pick == 64 ? tiles(256, 64) : tiles(128, 128)) * members <= cus / 2)
       pick = 1264;
-    // f32 (a compute unit's f32 matrix rate is a sixteenth of its 16-bit rate, so a block's
-    // time is all arithmetic): quarter blocks, while they still leave units idle
-    if constexpr (EL::F32)
-      if (pick == 1264 && tiles(128, 64) * members <= cus / 2) pick = 6464;
   }
   // Whole tiles of 16-bit operands go straight into LDS (gemm_dl.hpp; load offsets are 32-bit:
   // 256 rows of a k-contiguous operand must stay below 4 GiB, and every row segment the
@@ -1046,7 +1064,7 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   if (g.gelu && (a.M % 128 || a.N % 128)) return -1;
   if (pick == 192) pick = 128;
   if constexpr (EL::F32 && !EPI) {
-    // One f32 product whose blocks leave three quarters of the units idle and whose K is long (a
+    // One f32 product whose blocks leave half of the units idle and whose K is long (a
     // weight gradient: [768, 8192] x [8192, 768]): K is cut into `split` equal runs of whole slabs,
     // walked as a batch dim that writes [split][M][N] partial sums, which a second kernel adds in
     // run order (a fixed order: the same bits on every call).
@@ -1055,7 +1073,7 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
       const int64_t slabs = a.K / BK;
       int64_t split = std::min<int64_t>(cus / blocks, slabs / 4);
       while (split > 1 && slabs % split) split--;
-      if (split >= 2 && blocks * 4 <= cus && a.M * a.N % 4 == 0) {
+      if (split >= 2) {
         void *part = nullptr;
         int rc = nxh_alloc_locked(ctx, (size_t)split * a.M * a.N * sizeof(float), &part);
         if (rc) return rc;

@@ -226,11 +226,11 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
         # whole tiles
         (256, 64, 256, small), (512, 192, 768, small),
         (768, 320, 256, small), (512, 128, 64, small),
-        (1536, 64, 1664, "gemm_tile_128x128"), (33024, 64, 64, "gemm_tile_256x64"),
+        (2048, 64, 2048, "gemm_tile_128x128"), (65536, 64, 64, "gemm_tile_256x64"),
         (4096, 64, 4096, "gemm_tile_256x256"),
         # ragged in M and N (multiples of 8, so M/N-contiguous operands qualify too)
         (200, 64, 136, small), (264, 128, 40, small),
-        (1528, 64, 1672, "gemm_tile_128x128"), (33000, 128, 40, "gemm_tile_256x64"),
+        (2040, 64, 2040, "gemm_tile_128x128"), (65528, 128, 40, "gemm_tile_256x64"),
         (4000, 64, 4088, "gemm_tile_256x256"),
     ]
     for (m, k, n, path) in cases:
@@ -262,7 +262,7 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
     # results leave as 16-byte stores at the aligned addresses plus single elements at the ends
     for (m, k, n, path) in [(4000, 64, 4087, "gemm_tile_256x256"), (264, 128, 57, small),
                             (203, 192, 1031, small), (131, 64, 9, small),
-                            (1531, 64, 1671, "gemm_tile_128x128"), (33001, 64, 57, "gemm_tile_256x64")]:
+                            (2041, 64, 2039, "gemm_tile_128x128"), (65529, 64, 57, "gemm_tile_256x64")]:
         a = encode(rng.standard_normal((m, k)), d, oracle)
         b = encode(rng.standard_normal((k, n)), d, oracle)
         hb, _ = pair(np.ascontiguousarray(b.T), d, hip, oracle, lambda B, t: B.permute(t, (1, 0)))
