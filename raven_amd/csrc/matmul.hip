@@ -689,6 +689,166 @@ static int launch_any(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
   return NXH_OK;
 }
 
+// ── gemm_f64: float64 on the f64 matrix instruction ─────────────────────────
+// v_mfma_f64_16x16x4: lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16]; register v of
+// lane l of the result is D[4 v + l / 16][l % 16]. A block is 32T x 32T outputs (T = 4, 2 or 1),
+// four waves as 2 x 2, T x T result tiles per wave, K-slabs of BK: global -> registers (the
+// next slab, while this one is multiplied) -> K-contiguous LDS tiles [row][BK + 2] (the pad puts
+// the 16 rows and 2 k-columns a half-wave reads on distinct banks). Operands are read
+// element by element with bounds checks (zeros outside), lanes running along whichever of the
+// operand's two dims is contiguous: any strides (negative too), any edge, no alignment condition. One
+// instruction is 64 cycles on this chip, so a k-step's T^2 instructions hide its 2 T LDS
+// reads with room to spare; several blocks per unit hide the slab barrier.
+typedef __attribute__((ext_vector_type(4))) double f64x4;
+__device__ double gemm_f64_zero[2] = {0.0, 0.0};  // (not const: a load through it stays a global load)
+template <int T, int BK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f64_kernel(GemmArgs a) {
+  constexpr int BMN = 32 * T, LDP = BK + 2, NL = BMN * BK / 256;
+  __shared__ double sA[BMN * LDP];
+  __shared__ double sB[BMN * LDP];
+  int64_t ao, bo, co;
+  batch_decode(a.batch, a.batch0 + blockIdx.z, ao, bo, co);
+  const double *A = (const double *)a.A + ao;
+  const double *B = (const double *)a.B + bo;
+  const int64_t m0 = (int64_t)blockIdx.y * BMN, n0 = (int64_t)blockIdx.x * BMN;
+  const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = (wave >> 1) * (16 * T), wn = (wave & 1) * (16 * T);
+  const int r16 = lane & 15, kq = lane >> 4;
+
+  // Element e = thread + 256 i of an operand's slab: lanes run along k (kc) or along the row
+  // index; element e + 256 then lies a fixed number of rows or k-values further on, one uniform
+  // pointer step. No branch around a load and nothing to do to its result (the wait counters
+  // stay exact, so a slab's stores wait only for their own loads): an element outside the
+  // operand is read from a zero in memory instead.
+  struct Lane {
+    const double *p;  // this lane's element of slab 0
+    int64_t step;     // to element e + 256
+    int row, k, drow, dk;
+  };
+  auto lane_of = [&](const double *P, bool kc, int64_t rs, int64_t ks) {
+    Lane l;
+    l.row = kc ? threadIdx.x / BK : threadIdx.x % BMN;
+    l.k = kc ? threadIdx.x % BK : threadIdx.x / BMN;
+    l.drow = kc ? 256 / BK : 0;
+    l.dk = kc ? 0 : 256 / BMN;
+    l.p = P + l.row * rs + l.k * ks;
+    l.step = l.drow * rs + l.dk * ks;
+    return l;
+  };
+  const Lane la = lane_of(A + m0 * a.ars, a_kc, a.ars, a.acs);
+  const Lane lb = lane_of(B + n0 * a.bcs, b_kc, a.bcs, a.brs);  // B by rows = n
+  const int64_t a_left = a.M - m0, b_left = a.N - n0;
+  auto load = [&](double(&r)[NL], const Lane &l, int64_t ks, int64_t rows_left, int64_t k0) {
+    const double *p = l.p + k0 * ks;
+    if (rows_left >= BMN && k0 + BK <= a.K) {  // (uniform) a whole slab: nothing to check
+#pragma unroll
+      for (int i = 0; i < NL; i++) r[i] = p[i * l.step];
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      const bool ok = l.row + i * l.drow < rows_left && k0 + l.k + i * l.dk < a.K;
+      r[i] = *(ok ? p : gemm_f64_zero);
+      p += l.step;
+    }
+  };
+  auto store = [&](const double(&r)[NL], const Lane &l, double *s) {
+#pragma unroll
+    for (int i = 0; i < NL; i++) s[(l.row + i * l.drow) * LDP + l.k + i * l.dk] = r[i];
+  };
+
+  f64x4 acc[T][T];
+#pragma unroll
+  for (int t = 0; t < T; t++)
+#pragma unroll
+    for (int u = 0; u < T; u++) acc[t][u] = f64x4{0.0, 0.0, 0.0, 0.0};
+  const int64_t nk = (a.K + BK - 1) / BK;
+  // one slab: registers -> LDS, the loads of slab kt + 1 into the registers just freed, multiply
+  auto slab = [&](int64_t kt, double(&ra)[NL], double(&rb)[NL]) {
+    store(ra, la, sA);
+    store(rb, lb, sB);
+    __syncthreads();
+    load(ra, la, a.acs, a_left, (kt + 1) * BK);  // (past K: zeros nobody uses)
+    load(rb, lb, a.brs, b_left, (kt + 1) * BK);
+    // the fragments of k-step ks + 1 are read behind the first instructions of k-step ks
+    double fa[2][T], fb[2][T];
+    auto frags = [&](int ks, double(&fa_)[T], double(&fb_)[T]) {
+#pragma unroll
+      for (int t = 0; t < T; t++) {
+        fa_[t] = sA[(wm + t * 16 + r16) * LDP + ks * 4 + kq];
+        fb_[t] = sB[(wn + t * 16 + r16) * LDP + ks * 4 + kq];
+      }
+    };
+    frags(0, fa[0], fb[0]);
+#pragma unroll
+    for (int ks = 0; ks < BK / 4; ks++) {
+      const int cur = ks & 1;
+      if (ks + 1 < BK / 4) frags(ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
+#pragma unroll
+      for (int t = 0; t < T; t++)
+#pragma unroll
+        for (int u = 0; u < T; u++)
+          acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[cur][t], fb[cur][u], acc[t][u], 0, 0, 0);
+      // behind each matrix instruction (64 cycles): an LDS read, and the address arithmetic and
+      // issue of one or two of the next slab's loads
+#pragma unroll
+      for (int x = 0; x < T * T; x++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // matrix instruction
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
+        __builtin_amdgcn_sched_group_barrier(0x020, T == 4 ? 1 : 2, 0);  // global loads
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();
+  };
+  double ra0[NL], rb0[NL];
+  if (nk > 0) {
+    load(ra0, la, a.acs, a_left, 0);
+    load(rb0, lb, a.brs, b_left, 0);
+  }
+  for (int64_t kt = 0; kt < nk; kt++) slab(kt, ra0, rb0);
+  double *C = (double *)a.C + co;
+#pragma unroll
+  for (int t = 0; t < T; t++)
+#pragma unroll
+    for (int u = 0; u < T; u++) {
+      const int64_t col = n0 + wn + u * 16 + r16;
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        const int64_t row = m0 + wm + t * 16 + 4 * v + kq;
+        if (row < a.M && col < a.N) C[row * a.crs + col * a.ccs] = acc[t][u][v];
+      }
+    }
+}
+static int launch_f64(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
+  // Block shape: rounds of one block per unit x block area x the shape's measured cost per flop
+  // against the 128 x 128 block (4096^3: 57-63 TFLOP/s there; one wave per SIMD leaves about
+  // half of a small block's time to its loads and barriers).
+  const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+  auto cost = [&](int b, double pen) {
+    const int64_t tiles = ((a.M + b - 1) / b) * ((a.N + b - 1) / b) * (int64_t)nbatch;
+    return (double)((tiles + cus - 1) / cus) * b * b * pen;
+  };
+  int bmn = 128;
+  double best = cost(128, 1.0);
+  if (cost(64, 1.3) < best) bmn = 64, best = cost(64, 1.3);
+  if (cost(32, 1.6) < best) bmn = 32;
+  const uint32_t gx = (uint32_t)((a.N + bmn - 1) / bmn), gy = (uint32_t)((a.M + bmn - 1) / bmn);
+  if (gy > 65535) return launch_any<NXH_F64>(ctx, a, nbatch);
+  nxh_set_path(bmn == 128 ? "gemm_f64_128x128" : bmn == 64 ? "gemm_f64_64x64" : "gemm_f64_32x32");
+  for (uint32_t b0 = 0; b0 < nbatch; b0 += 65535) {
+    a.batch0 = b0;
+    const dim3 grid(gx, gy, std::min<uint32_t>(65535, nbatch - b0));
+    if (bmn == 128) hipLaunchKernelGGL((gemm_f64_kernel<4, 16>), grid, dim3(256), 0, ctx->stream, a);
+    else if (bmn == 64) hipLaunchKernelGGL((gemm_f64_kernel<2, 32>), grid, dim3(256), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((gemm_f64_kernel<1, 32>), grid, dim3(256), 0, ctx->stream, a);
+    NXH_HIP("matmul", hipGetLastError());
+  }
+  return NXH_OK;
+}
+
 template <class MM>
 static int launch_mfma(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
   nxh_set_path("gemm_mfma");
@@ -1436,7 +1596,7 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
     case NXH_F32: return run_mfma_dtype<MMf32>(ctx, g, (uint32_t)nbatch, al_a, al_b);
 #define NXH_CASE(DT) \
   case DT: return launch_any<DT>(ctx, g, (uint32_t)nbatch);
-      NXH_CASE(NXH_F64)
+    case NXH_F64: return launch_f64(ctx, g, (uint32_t)nbatch);
       NXH_CASE(NXH_F8E4M3)
       NXH_CASE(NXH_F8E5M2)
       NXH_CASE(NXH_I8)

@@ -331,6 +331,55 @@ def test_matmul_padded_copies(hip, oracle, d):
     assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
 
 
+def test_matmul_f64_matrix_kernel(hip, oracle):
+    """float64 on the f64 matrix instruction: the three block shapes, every orientation, ragged M / N / K,
+    batches with a broadcast operand, operands with no unit stride; products of doubles summed in
+    double, so 1e-9 of the float64 reference is loose by orders of magnitude."""
+    d = dt.float64
+    rng = np.random.default_rng(1470)
+    T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
+    for (m, k, n, path) in [(512, 300, 700, "gemm_f64_32x32"), (1024, 40, 1024, "gemm_f64_64x64"),
+                            (1000, 100, 1001, "gemm_f64_64x64"), (2048, 64, 2048, "gemm_f64_128x128"),
+                            (2041, 37, 2039, "gemm_f64_128x128"), (1, 5, 1, "gemm_f64_32x32"), (130, 1, 3, "gemm_f64_32x32")]:
+        a = rng.standard_normal((m, k))
+        b = rng.standard_normal((k, n))
+        for ta in (False, True):
+            for tb in (False, True):
+                ha, _ = pair(np.ascontiguousarray(a.T) if ta else a, d, hip, oracle, T if ta else None)
+                hb, _ = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle, T if tb else None)
+                got = logical(hip.matmul(ha, hb))
+                assert hip.last_path() == path, (m, k, n, hip.last_path())
+                want = a @ b
+                assert np.all(np.abs(got - want) <= 1e-12 * (np.abs(want) + np.sqrt(k))), (m, k, n, ta, tb)
+    a = rng.standard_normal((3, 1, 70, 50))
+    b = rng.standard_normal((1, 4, 50, 90))
+    got = logical(hip.matmul(pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]))
+    assert hip.last_path() == "gemm_f64_32x32" and np.allclose(got, a @ b, rtol=1e-12, atol=1e-12)
+    # every other row and column of both operands: no unit stride anywhere
+    a = rng.standard_normal((200, 160))
+    b = rng.standard_normal((160, 120))
+    every_other = lambda B, t: B.shrink(B.reshape(t, (t.shape[0] // 2, 2, t.shape[1] // 2, 2)),  # noqa: E731
+                                        [(0, t.shape[0] // 2), (0, 1), (0, t.shape[1] // 2), (0, 1)])
+    ha = pair(a, d, hip, oracle, every_other)[0]
+    hb = pair(b, d, hip, oracle, every_other)[0]
+    ha, hb = hip.reshape(ha, (100, 80)), hip.reshape(hb, (80, 60))
+    got = logical(hip.matmul(ha, hb))
+    assert hip.last_path() == "gemm_f64_32x32" and np.allclose(got, a[::2, ::2] @ b[::2, ::2], rtol=1e-12, atol=1e-12)
+    # flipped operands (negative strides)
+    fl = lambda B, t: B.flip(t, (True, True))  # noqa: E731
+    got = logical(hip.matmul(pair(a, d, hip, oracle, fl)[0], pair(b, d, hip, oracle, fl)[0]))
+    assert hip.last_path() == "gemm_f64_32x32" and np.allclose(got, a[::-1, ::-1] @ b[::-1, ::-1], rtol=1e-12, atol=1e-12)
+    # non-finite values stay where the arithmetic puts them
+    a = rng.standard_normal((64, 33))
+    b = rng.standard_normal((33, 64))
+    a[3, 32] = np.inf
+    b[32, 63] = np.nan
+    got = logical(hip.matmul(pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]))
+    with np.errstate(invalid="ignore"):
+        want = a @ b
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+
+
 def test_matmul_f32_few_blocks_cut_along_k(hip, oracle):
     """One f32 product with few output blocks and a long K (a weight gradient) is cut along K; the
     partial sums are added in a fixed order: within the matmul tolerance, and the same bits every call."""
