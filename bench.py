@@ -278,9 +278,26 @@ def next_ops(hip, W, linalg=False):
     cols = hip.unfold(img, *geo)
     timed("fold back to [8,64,128,128] (col2im, 9 taps per output)", lambda: hip.fold(cols, [128, 128], *geo), nin + ncols)
     del img, cols
+    # matmul beside config 4's shapes: float64, and the products a convolution makes of its windows
+    def mm(name, a, b, flops, peak, iters=10):
+        timed(name, lambda: hip.matmul(a, b), 0, iters=iters)
+        tf = flops / (out[-1]["ms"] * 1e-3) / 1e12
+        out[-1] = {"op": name + f" ({hip.last_path()})", "ms": out[-1]["ms"], "TFLOP/s": round(tf, 2),
+                   "frac_mfma": round(tf / peak, 4), "bound": "mfma"}
+    f64 = lambda shape: W.dev(rng.standard_normal(shape), dt.float64)
+    mm("matmul f64 2048^3", f64((2048, 2048)), f64((2048, 2048)), 2.0 * 2048 ** 3, 78.6, iters=5)
+    mm("matmul f64 512^3", f64((512, 512)), f64((512, 512)), 2.0 * 512 ** 3, 78.6)
+    f32 = lambda shape: W.dev(rng.standard_normal(shape).astype(np.float32), dt.float32)
+    mm("matmul f32 1024^3", f32((1024, 1024)), f32((1024, 1024)), 2.0 * 1024 ** 3, 157.3)
+    mm("matmul f32 [64,576] x [32,576,3136] (3x3 windows of [32,64,56,56])",
+       hip.expand(f32((1, 64, 576)), (32, 64, 576)), f32((32, 576, 3136)), 2.0 * 32 * 64 * 576 * 3136, 157.3)
+    mm("matmul f32 [256,2048] x [2048,256] (weight gradient, cut along K)", f32((256, 2048)), f32((2048, 256)),
+       2.0 * 256 * 2048 * 256, 157.3)
     # fused attention and the row kernels at GPT-2-small's shapes (bf16, batch 8, seq 1024)
     bf = lambda shape: W.dev((rng.standard_normal(shape).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16),
                              dt.bfloat16)
+    mm("matmul bf16 [256,2304] x [32,2304,196] (3x3 windows of [32,256,14,14]; rows of 196 via a padded copy)",
+       hip.expand(bf((1, 256, 2304)), (32, 256, 2304)), bf((32, 2304, 196)), 2.0 * 32 * 256 * 2304 * 196, 2500.0)
     b, h, sq, hd = 8, 12, 1024, 64
     q, k, v = (hip.permute(hip.reshape(bf((b, sq, h * hd)), (b, sq, h, hd)), (0, 2, 1, 3)) for _ in range(3))
     timed("attention [8,12,1024,64] bf16, causal, head-split views (attention_fused)",
