@@ -331,6 +331,35 @@ def test_matmul_padded_copies(hip, oracle, d):
     assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
 
 
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16, dt.float64], ids=lambda d: d.name)
+def test_matmul_seeded_shape_sweep(hip, oracle, d):
+    """Eighty seeded shapes per dtype across the dispatch's thresholds (block shapes, the cut along
+    K, padded copies, the general kernel): extents drawn around multiples of the tile sizes, every
+    orientation, with and without a batch, against the float64 product of the stored values."""
+    rng = np.random.default_rng(4200 + d.tag)
+    T = lambda B, t: B.permute(t, tuple(range(len(t.shape) - 2)) + (len(t.shape) - 1, len(t.shape) - 2))  # noqa: E731
+    seen = set()
+    for case in range(80):
+        def extent(bases):
+            return max(1, int(rng.choice(bases)) + int(rng.integers(-9, 10)) * int(rng.integers(0, 4) == 0))
+        m = extent([8, 64, 128, 200, 256, 512, 1024, 2048])
+        n = extent([8, 64, 128, 196, 256, 768, 1536, 2048])
+        k = extent([32, 64, 128, 256, 576, 2048])
+        batch = () if rng.integers(0, 2) else (int(rng.integers(1, 5)),)
+        if m * n * k * int(np.prod(batch, dtype=np.int64)) > 1e9:
+            k = max(32, k // 8)
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        share_b = bool(batch) and bool(rng.integers(0, 2))  # one B for the whole batch
+        a = encode(rng.standard_normal(batch + (m, k)), d, oracle)
+        b = encode(rng.standard_normal((() if share_b else batch) + (k, n)), d, oracle)
+        ha, _ = pair(np.ascontiguousarray(np.swapaxes(a, -1, -2)) if ta else a, d, hip, oracle, T if ta else None)
+        hb, _ = pair(np.ascontiguousarray(np.swapaxes(b, -1, -2)) if tb else b, d, hip, oracle, T if tb else None)
+        check(hip, oracle, d, ha, hb, a, b, f"case {case}: {batch} {m}x{k}x{n} ta={ta} tb={tb} shared B={share_b}")
+        seen.add(hip.last_path())
+    # the sweep is only worth its time if it crosses the dispatch: at least three kernels per dtype
+    assert len(seen) >= 3, seen
+
+
 def test_matmul_f64_matrix_kernel(hip, oracle):
     """float64 on the f64 matrix instruction: the three block shapes, every orientation, ragged M / N / K,
     batches with a broadcast operand, operands with no unit stride; products of doubles summed in
