@@ -77,6 +77,54 @@ def test_replays_match_eager_results_between_other_work(hip, oracle):
     assert hip.memory_stats()["in_use"] == before
 
 
+def test_matmul_forms_with_temporaries_replay(hip, oracle):
+    """The matmul forms that take a pooled block inside the call (the f32 cut along K with its
+    partial sums, the padded copies of ragged operands) and the float64 kernel, recorded once:
+    every replay gives the bits of the eager call on the inputs of the moment."""
+    rng = np.random.default_rng(77)
+
+    def make(seed):
+        r = np.random.default_rng(seed)
+        return (r.standard_normal((256, 2048)).astype(np.float32), r.standard_normal((2048, 256)).astype(np.float32),
+                encode(r.standard_normal((1, 256, 576)), dt.bfloat16, oracle),
+                encode(r.standard_normal((8, 576, 196)), dt.bfloat16, oracle),
+                r.standard_normal((300, 100)), r.standard_normal((100, 200)))
+
+    def dev(x, d):
+        return hip.reshape(hip.from_host(x, d), x.shape)
+
+    kinds = (dt.float32, dt.float32, dt.bfloat16, dt.bfloat16, dt.float64, dt.float64)
+    ts = [dev(x, d) for x, d in zip(make(0), kinds)]
+
+    def run():
+        outs = [hip.matmul(ts[0], ts[1])]
+        paths = [hip.last_path()]
+        outs.append(hip.matmul(hip.expand(ts[2], (8, 256, 576)), ts[3]))
+        paths.append(hip.last_path())
+        outs.append(hip.matmul(ts[4], ts[5]))
+        paths.append(hip.last_path())
+        return outs, paths
+
+    _, paths = run()  # warm
+    assert paths == ["gemm_tile_64x64_splitk", "gemm_tile_padded", "gemm_f64_32x32"], paths
+    with capture(hip) as cap:
+        outs, _ = run()
+    g = cap.graph
+    try:
+        for seed in (1, 2, 3):
+            for t, x, d in zip(ts, make(seed), kinds):
+                hip.assign(t, dev(x, d))
+            junk = hip.matmul(dev(rng.standard_normal((128, 1024)).astype(np.float32), dt.float32),
+                              dev(rng.standard_normal((1024, 64)).astype(np.float32), dt.float32))  # takes and frees a block
+            g.launch()
+            eager, _ = run()
+            for o, e, name in zip(outs, eager, paths):
+                same_bits(logical(o), logical(e), f"replay {seed}: {name}")
+            del junk, eager
+    finally:
+        g.destroy()
+
+
 def test_uploads_are_replayed_and_host_reads_are_refused(hip):
     x = hip.from_host(np.arange(1000, dtype=np.int32), dt.int32)
     with capture(hip) as cap:
