@@ -288,7 +288,9 @@ __device__ __forceinline__ void tile_of_block(const Args &a, uint32_t bid, uint3
   tn = in_strip / gsz;
 }
 
-template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI = false>
+// OUT32: the f32 sums are stored as they are (C is float, `ldc` and the batch strides in floats):
+// the partial sums of a product cut along K, added up by a second kernel.
+template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI = false, bool OUT32 = false>
 __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH::WAVES_PER_SIMD))) void kernel(Args a) {
   constexpr int THREADS = SH::THREADS, BM = SH::BM, BN = SH::BN, TM = SH::TM, TN = SH::TN;
   constexpr int NVA = SH::NVA, NVB = SH::NVB, BK = Geo<EL>::BK;
@@ -453,6 +455,23 @@ __global__ __launch_bounds__(SH::THREADS) __attribute__((amdgpu_waves_per_eu(SH:
     if constexpr (EL::F32) return x;
     else return EL::BF16 ? bf16_to_f32(x) : f16_to_f32(x);
   };
+  if constexpr (OUT32 && !EL::F32) {
+    float *Cf = (float *)a.C + co;
+#pragma unroll
+    for (int t = 0; t < TM; t++)
+#pragma unroll
+      for (int u = 0; u < TN; u++) {
+        const int cl = wn + u * 32 + r32;
+        if (EDGE && cl >= edge_n) continue;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          const int rl = wm + t * 32 + (e >> 2) * 8 + kg * 4 + (e & 3);
+          if (EDGE && rl >= edge_m) continue;
+          Cf[(m0 + rl) * a.ldc + n0 + cl] = acc[t][u][e];
+        }
+      }
+    return;
+  }
   if constexpr (!EL::F32) {
     // 16-bit outputs go through LDS: in accumulator order a lane would store
     // (and, with a residual, load) two bytes at a time. Each wave parks its

@@ -1004,9 +1004,9 @@ static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // The LDS-tiled family of gemm_tile.hpp: K a multiple of one slab (64 two-byte or
 // 32 four-byte elements), 16-byte aligned rows, unit-stride C. Returns -1 when the call does not qualify.
-template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI>
+template <class EL, bool A_KC, bool B_KC, class SH, bool EDGE, bool EPI, bool OUT32 = false>
 static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
-  auto kern = gemm_tile::kernel<EL, A_KC, B_KC, SH, EDGE, EPI>;
+  auto kern = gemm_tile::kernel<EL, A_KC, B_KC, SH, EDGE, EPI, OUT32>;
   constexpr size_t LDS = SH::template lds_bytes<EL>();
   // once per process and kernel (contexts have separate mutexes): allow > 64 KiB of dynamic LDS
   static std::once_flag once;
@@ -1026,11 +1026,11 @@ static int launch_tile(nxh_context *ctx, gemm_tile::Args &g, const char *path) {
   NXH_HIP("matmul", hipGetLastError());
   return NXH_OK;
 }
-template <class EL, class SH, bool EPI>
+template <class EL, class SH, bool EPI, bool OUT32 = false>
 static int launch_tile_oriented(nxh_context *ctx, gemm_tile::Args &g, bool a_kc, bool b_kc, const char *path) {
   const bool edge = g.M % SH::BM != 0 || g.N % SH::BN != 0;
 #define NXH_TILE(AK, BK_)                                                                  \
-  (edge ? launch_tile<EL, AK, BK_, SH, true, EPI>(ctx, g, path) : launch_tile<EL, AK, BK_, SH, false, EPI>(ctx, g, path))
+  (edge ? launch_tile<EL, AK, BK_, SH, true, EPI, OUT32>(ctx, g, path) : launch_tile<EL, AK, BK_, SH, false, EPI, OUT32>(ctx, g, path))
   if (a_kc) return b_kc ? NXH_TILE(true, true) : NXH_TILE(true, false);
   return b_kc ? NXH_TILE(false, true) : NXH_TILE(false, false);
 #undef NXH_TILE
@@ -1223,16 +1223,30 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   }
   if (g.gelu && (a.M % 128 || a.N % 128)) return -1;
   if (pick == 192) pick = 128;
-  if constexpr (EL::F32 && !EPI) {
-    // One f32 product whose blocks leave half of the units idle and whose K is long (a
+  if constexpr (!EPI) {
+    // One product (no batch) whose blocks leave half of the units idle and whose K is long (a
     // weight gradient: [768, 8192] x [8192, 768]): K is cut into `split` equal runs of whole slabs,
-    // walked as a batch dim that writes [split][M][N] partial sums, which a second kernel adds in
-    // run order (a fixed order: the same bits on every call).
+    // walked as a batch dim that writes [split][M][N] f32 partial sums, which a second kernel adds
+    // in run order (a fixed order: the same bits on every call) and rounds to the dtype once.
     if (nbatch == 1 && a.batch.n == 0 && (pick == 1264 || pick == 6464)) {
+      constexpr int DT = EL::F32 ? NXH_F32 : EL::BF16 ? NXH_BF16 : NXH_F16;
       const int64_t blocks = pick == 6464 ? tiles(64, 64) : tiles(128, 64);
       const int64_t slabs = a.K / BK;
-      int64_t split = std::min<int64_t>(cus / blocks, slabs / 4);
-      while (split > 1 && slabs % split) split--;
+      // Worth it when the slabs a block no longer walks (about 0.3 us each for a 16-bit block that
+      // has its unit to itself, 0.7 us for f32) outweigh the second launch and the partial sums'
+      // trip through memory (bf16 [1000,8192] x [8192,1000]: 57 -> 39 us with two runs; [1024,1024]^2
+      // would go from 9.5 to 15 us and stays whole).
+      int64_t split = 1;
+      double best_gain = 0.0;
+      for (int64_t sp = std::min<int64_t>(cus / blocks, slabs / 4); sp >= 2; sp--) {
+        if (slabs % sp) continue;
+        const double saved = (double)slabs * (1.0 - 1.0 / (double)sp) * (EL::F32 ? 0.7 : 0.3);
+        const double cost = 4.0 + (double)sp * (double)a.M * (double)a.N * 8.0 / 4e6;
+        if (saved - 1.2 * cost > best_gain) {
+          best_gain = saved - 1.2 * cost;
+          split = sp;
+        }
+      }
       if (split >= 2) {
         void *part = nullptr;
         int rc = nxh_alloc_locked(ctx, (size_t)split * a.M * a.N * sizeof(float), &part);
@@ -1247,11 +1261,15 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
         gs.bc[0] = a.M * a.N;
         gs.C = part;
         gs.ldc = a.N;
-        rc = pick == 6464 ? launch_tile_oriented<EL, gemm_tile::Shape64x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_64x64_splitk")
-                          : launch_tile_oriented<EL, gemm_tile::Shape128x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
+        if constexpr (EL::F32) {
+          rc = pick == 6464 ? launch_tile_oriented<EL, gemm_tile::Shape64x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_64x64_splitk")
+                            : launch_tile_oriented<EL, gemm_tile::Shape128x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
+        } else {
+          rc = launch_tile_oriented<EL, gemm_tile::Shape128x64, false, true>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
+        }
         if (rc == NXH_OK) {
           const int64_t total = a.M * a.N;
-          hipLaunchKernelGGL((skinny_finish_kernel<NXH_F32>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0,
+          hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0,
                              ctx->stream, (const float *)part, g.C, a.M, a.N, (int)split, g.ldc, (int64_t)1);
           hipError_t e = hipGetLastError();
           if (e != hipSuccess) rc = nxh_hip_fail("matmul", e);

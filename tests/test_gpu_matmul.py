@@ -247,8 +247,6 @@ def test_matmul_big_tile_kernel(hip, oracle, d):
                 check(hip, oracle, d, ha, hb, a, b, f"tile {m}x{k}x{n} ta={ta} tb={tb}")
                 # whole 256-tiles of 16-bit operands take the direct-to-LDS form
                 want_path = "gemm_dl_256x256" if (path, m % 256, n % 256) == ("gemm_tile_256x256", 0, 0) and d is not dt.float32 else path
-                if d is dt.float32 and k >= 256 and want_path == small:
-                    want_path += "_splitk"
                 assert hip.last_path() == want_path, (m, k, n, ta, tb, hip.last_path())
     # odd M and N: only K-contiguous operands (A row-major, B given as its transpose) qualify
     a = encode(rng.standard_normal((203, 128)), d, oracle)
@@ -409,15 +407,18 @@ def test_matmul_f64_matrix_kernel(hip, oracle):
     assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
 
 
-def test_matmul_f32_few_blocks_cut_along_k(hip, oracle):
-    """One f32 product with few output blocks and a long K (a weight gradient) is cut along K; the
-    partial sums are added in a fixed order: within the matmul tolerance, and the same bits every call."""
-    d = dt.float32
-    rng = np.random.default_rng(1460)
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_few_blocks_cut_along_k(hip, oracle, d):
+    """One product with few output blocks and a long K (a weight gradient) is cut along K; the f32
+    partial sums are added in a fixed order and rounded once: within the matmul tolerance, and the
+    same bits every call."""
+    rng = np.random.default_rng(1460 + d.tag)
     T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
-    for (m, k, n, path) in [(128, 4096, 64, "gemm_tile_64x64_splitk"), (256, 2048, 256, "gemm_tile_64x64_splitk"),
-                            (200, 1024, 72, "gemm_tile_64x64_splitk"), (768, 8192, 768, "gemm_tile_64x64"),
-                            (64, 96, 64, "gemm_tile_64x64")]:
+    f32 = d is dt.float32
+    cut = "gemm_tile_64x64_splitk" if f32 else "gemm_tile_128x64_splitk"
+    for (m, k, n, path) in [(128, 4096, 64, cut), (256, 2048, 256, cut), (200, 1024, 72, cut if f32 else "gemm_tile_128x64"),
+                            (768, 8192, 768, "gemm_tile_64x64" if f32 else cut),
+                            (64, 128, 64, "gemm_tile_64x64" if f32 else "gemm_tile_128x64")]:
         a = encode(rng.standard_normal((m, k)), d, oracle)
         b = encode(rng.standard_normal((k, n)), d, oracle)
         for ta in (False, True):
@@ -428,16 +429,20 @@ def test_matmul_f32_few_blocks_cut_along_k(hip, oracle):
                 assert hip.last_path() == path, (m, k, n, ta, tb, hip.last_path())
                 first = logical(hip.matmul(ha, hb))
                 same_bits(logical(hip.matmul(ha, hb)), first, "same bits on every call")
+                if not f32:  # one rounding of the f32 sum: within one unit of the f64 product rounded
+                    got, want = decode(first, d, oracle), ref_f64(a, b, d, oracle)
+                    ulp = 2.0 ** (-8 if d is dt.bfloat16 else -11)
+                    assert np.all(np.abs(got - want) <= ulp * 2 * np.abs(want) + np.sqrt(k) * 4e-6), (m, k, n, ta, tb)
     # into a strided output: a column slice of a wider result
     a = encode(rng.standard_normal((128, 2048)), d, oracle)
     b = encode(rng.standard_normal((2048, 64)), d, oracle)
     ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
     dense = logical(hip.matmul(ha, hb))
-    wide = hip.reshape(hip.from_host(np.zeros(128 * 80, np.float32), d), (128, 80))
+    wide = hip.reshape(hip.from_host(np.zeros(128 * 80, dense.dtype), d), (128, 80))
     import ctypes as C
     view = hip.shrink(wide, [(0, 128), (8, 72)])
     hip._check(hip._lib.nxh_matmul(hip._h, C.byref(view._desc()), C.byref(ha._desc()), C.byref(hb._desc())))
-    assert hip.last_path() == "gemm_tile_64x64_splitk"
+    assert hip.last_path() == cut
     w = logical(wide)
     same_bits(np.ascontiguousarray(w[:, 8:72]), dense, "strided output")
     assert not w[:, :8].any() and not w[:, 72:].any()
