@@ -691,8 +691,9 @@ static int launch_any(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
 
 // ── gemm_f64: float64 on the f64 matrix instruction ─────────────────────────
 // v_mfma_f64_16x16x4: lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16]; register v of
-// lane l of the result is D[4 v + l / 16][l % 16]. A block is 32T x 32T outputs (T = 4, 2 or 1),
-// four waves as 2 x 2, T x T result tiles per wave, K-slabs of BK: global -> registers (the
+// lane l of the result is D[4 v + l / 16][l % 16]. A block is WM x WN waves of TM x TN result
+// tiles each (128 x 128 as 2 x 2 waves of 4 x 4 tiles or 4 x 2 waves of 2 x 4; 64 x 64 as 4 x 2 of
+// 1 x 2; 32 x 32 as 2 x 2 of 1 x 1), K-slabs of BK: global -> registers (the
 // next slab, while this one is multiplied) -> K-contiguous LDS tiles [row][BK + 2] (the pad puts
 // the 16 rows and 2 k-columns a half-wave reads on distinct banks). Operands are read
 // element by element with bounds checks (zeros outside), lanes running along whichever of the
@@ -701,47 +702,51 @@ static int launch_any(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
 // reads with room to spare; several blocks per unit hide the slab barrier.
 typedef __attribute__((ext_vector_type(4))) double f64x4;
 __device__ double gemm_f64_zero[2] = {0.0, 0.0};  // (not const: a load through it stays a global load)
-template <int T, int BK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f64_kernel(GemmArgs a) {
-  constexpr int BMN = 32 * T, LDP = BK + 2, NL = BMN * BK / 256;
-  __shared__ double sA[BMN * LDP];
-  __shared__ double sB[BMN * LDP];
+template <int WM, int WN, int TM, int TN, int BK>
+__global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(2))) void gemm_f64_kernel(GemmArgs a) {
+  constexpr int BM = 16 * TM * WM, BN = 16 * TN * WN, THREADS = 64 * WM * WN, LDP = BK + 2;
+  constexpr int NLA = BM * BK / THREADS, NLB = BN * BK / THREADS;
+  static_assert(NLA >= 1 && NLB >= 1 && NLA * THREADS == BM * BK && NLB * THREADS == BN * BK, "slab loads");
+  static_assert(THREADS % BK == 0 && THREADS % BM == 0 && THREADS % BN == 0, "lanes along k or along rows");
+  __shared__ double sA[BM * LDP];
+  __shared__ double sB[BN * LDP];
   int64_t ao, bo, co;
   batch_decode(a.batch, a.batch0 + blockIdx.z, ao, bo, co);
   const double *A = (const double *)a.A + ao;
   const double *B = (const double *)a.B + bo;
-  const int64_t m0 = (int64_t)blockIdx.y * BMN, n0 = (int64_t)blockIdx.x * BMN;
+  const int64_t m0 = (int64_t)blockIdx.y * BM, n0 = (int64_t)blockIdx.x * BN;
   const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wm = (wave >> 1) * (16 * T), wn = (wave & 1) * (16 * T);
+  const int wm = (wave / WN) * (16 * TM), wn = (wave % WN) * (16 * TN);
   const int r16 = lane & 15, kq = lane >> 4;
 
-  // Element e = thread + 256 i of an operand's slab: lanes run along k (kc) or along the row
-  // index; element e + 256 then lies a fixed number of rows or k-values further on, one uniform
+  // Element e = thread + THREADS i of an operand's slab: lanes run along k (kc) or along the row
+  // index; element e + THREADS then lies a fixed number of rows or k-values further on, one uniform
   // pointer step. No branch around a load and nothing to do to its result (the wait counters
   // stay exact, so a slab's stores wait only for their own loads): an element outside the
   // operand is read from a zero in memory instead.
   struct Lane {
     const double *p;  // this lane's element of slab 0
-    int64_t step;     // to element e + 256
+    int64_t step;     // to element e + THREADS
     int row, k, drow, dk;
   };
-  auto lane_of = [&](const double *P, bool kc, int64_t rs, int64_t ks) {
+  auto lane_of = [&](const double *P, bool kc, int64_t rs, int64_t ks, int rows) {
     Lane l;
-    l.row = kc ? threadIdx.x / BK : threadIdx.x % BMN;
-    l.k = kc ? threadIdx.x % BK : threadIdx.x / BMN;
-    l.drow = kc ? 256 / BK : 0;
-    l.dk = kc ? 0 : 256 / BMN;
+    l.row = kc ? threadIdx.x / BK : threadIdx.x % rows;
+    l.k = kc ? threadIdx.x % BK : threadIdx.x / rows;
+    l.drow = kc ? THREADS / BK : 0;
+    l.dk = kc ? 0 : THREADS / rows;
     l.p = P + l.row * rs + l.k * ks;
     l.step = l.drow * rs + l.dk * ks;
     return l;
   };
-  const Lane la = lane_of(A + m0 * a.ars, a_kc, a.ars, a.acs);
-  const Lane lb = lane_of(B + n0 * a.bcs, b_kc, a.bcs, a.brs);  // B by rows = n
+  const Lane la = lane_of(A + m0 * a.ars, a_kc, a.ars, a.acs, BM);
+  const Lane lb = lane_of(B + n0 * a.bcs, b_kc, a.bcs, a.brs, BN);  // B by rows = n
   const int64_t a_left = a.M - m0, b_left = a.N - n0;
-  auto load = [&](double(&r)[NL], const Lane &l, int64_t ks, int64_t rows_left, int64_t k0) {
+  auto load = [&](auto &r, const Lane &l, int64_t ks, int64_t rows_left, int rows, int64_t k0) {
+    constexpr int NL = sizeof(r) / sizeof(double);
     const double *p = l.p + k0 * ks;
-    if (rows_left >= BMN && k0 + BK <= a.K) {  // (uniform) a whole slab: nothing to check
+    if (rows_left >= rows && k0 + BK <= a.K) {  // (uniform) a whole slab: nothing to check
 #pragma unroll
       for (int i = 0; i < NL; i++) r[i] = p[i * l.step];
       return;
@@ -753,32 +758,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
       p += l.step;
     }
   };
-  auto store = [&](const double(&r)[NL], const Lane &l, double *s) {
+  auto store = [&](const auto &r, const Lane &l, double *s) {
+    constexpr int NL = sizeof(r) / sizeof(double);
 #pragma unroll
     for (int i = 0; i < NL; i++) s[(l.row + i * l.drow) * LDP + l.k + i * l.dk] = r[i];
   };
 
-  f64x4 acc[T][T];
+  f64x4 acc[TM][TN];
 #pragma unroll
-  for (int t = 0; t < T; t++)
+  for (int t = 0; t < TM; t++)
 #pragma unroll
-    for (int u = 0; u < T; u++) acc[t][u] = f64x4{0.0, 0.0, 0.0, 0.0};
+    for (int u = 0; u < TN; u++) acc[t][u] = f64x4{0.0, 0.0, 0.0, 0.0};
   const int64_t nk = (a.K + BK - 1) / BK;
   // one slab: registers -> LDS, the loads of slab kt + 1 into the registers just freed, multiply
-  auto slab = [&](int64_t kt, double(&ra)[NL], double(&rb)[NL]) {
+  auto slab = [&](int64_t kt, double(&ra)[NLA], double(&rb)[NLB]) {
     store(ra, la, sA);
     store(rb, lb, sB);
     __syncthreads();
-    load(ra, la, a.acs, a_left, (kt + 1) * BK);  // (past K: zeros nobody uses)
-    load(rb, lb, a.brs, b_left, (kt + 1) * BK);
+    load(ra, la, a.acs, a_left, BM, (kt + 1) * BK);  // (past K: zeros nobody uses)
+    load(rb, lb, a.brs, b_left, BN, (kt + 1) * BK);
     // the fragments of k-step ks + 1 are read behind the first instructions of k-step ks
-    double fa[2][T], fb[2][T];
-    auto frags = [&](int ks, double(&fa_)[T], double(&fb_)[T]) {
+    double fa[2][TM], fb[2][TN];
+    auto frags = [&](int ks, double(&fa_)[TM], double(&fb_)[TN]) {
 #pragma unroll
-      for (int t = 0; t < T; t++) {
-        fa_[t] = sA[(wm + t * 16 + r16) * LDP + ks * 4 + kq];
-        fb_[t] = sB[(wn + t * 16 + r16) * LDP + ks * 4 + kq];
-      }
+      for (int t = 0; t < TM; t++) fa_[t] = sA[(wm + t * 16 + r16) * LDP + ks * 4 + kq];
+#pragma unroll
+      for (int u = 0; u < TN; u++) fb_[u] = sB[(wn + u * 16 + r16) * LDP + ks * 4 + kq];
     };
     frags(0, fa[0], fb[0]);
 #pragma unroll
@@ -786,34 +791,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
       const int cur = ks & 1;
       if (ks + 1 < BK / 4) frags(ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
 #pragma unroll
-      for (int t = 0; t < T; t++)
+      for (int t = 0; t < TM; t++)
 #pragma unroll
-        for (int u = 0; u < T; u++)
+        for (int u = 0; u < TN; u++)
           acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[cur][t], fb[cur][u], acc[t][u], 0, 0, 0);
       // behind each matrix instruction (64 cycles): an LDS read, and the address arithmetic and
       // issue of one or two of the next slab's loads
 #pragma unroll
-      for (int x = 0; x < T * T; x++) {
+      for (int x = 0; x < TM * TN; x++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // matrix instruction
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
         __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
-        __builtin_amdgcn_sched_group_barrier(0x020, T == 4 ? 1 : 2, 0);  // global loads
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global load
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
   };
-  double ra0[NL], rb0[NL];
+  double ra0[NLA], rb0[NLB];
   if (nk > 0) {
-    load(ra0, la, a.acs, a_left, 0);
-    load(rb0, lb, a.brs, b_left, 0);
+    load(ra0, la, a.acs, a_left, BM, 0);
+    load(rb0, lb, a.brs, b_left, BN, 0);
   }
   for (int64_t kt = 0; kt < nk; kt++) slab(kt, ra0, rb0);
   double *C = (double *)a.C + co;
 #pragma unroll
-  for (int t = 0; t < T; t++)
+  for (int t = 0; t < TM; t++)
 #pragma unroll
-    for (int u = 0; u < T; u++) {
+    for (int u = 0; u < TN; u++) {
       const int64_t col = n0 + wn + u * 16 + r16;
 #pragma unroll
       for (int v = 0; v < 4; v++) {
@@ -841,9 +846,13 @@ static int launch_f64(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
   for (uint32_t b0 = 0; b0 < nbatch; b0 += 65535) {
     a.batch0 = b0;
     const dim3 grid(gx, gy, std::min<uint32_t>(65535, nbatch - b0));
-    if (bmn == 128) hipLaunchKernelGGL((gemm_f64_kernel<4, 16>), grid, dim3(256), 0, ctx->stream, a);
-    else if (bmn == 64) hipLaunchKernelGGL((gemm_f64_kernel<2, 32>), grid, dim3(256), 0, ctx->stream, a);
-    else hipLaunchKernelGGL((gemm_f64_kernel<1, 32>), grid, dim3(256), 0, ctx->stream, a);
+    // eight waves (two per SIMD from the one block) where a unit holds a single block: a wave's
+    // waits are then covered by its neighbour's matrix instructions (2048^3: 372 -> 342 us)
+    const bool one_round = (int64_t)gx * gy * nbatch <= cus;
+    if (bmn == 128 && one_round) hipLaunchKernelGGL((gemm_f64_kernel<4, 2, 2, 4, 16>), grid, dim3(512), 0, ctx->stream, a);
+    else if (bmn == 128) hipLaunchKernelGGL((gemm_f64_kernel<2, 2, 4, 4, 16>), grid, dim3(256), 0, ctx->stream, a);
+    else if (bmn == 64) hipLaunchKernelGGL((gemm_f64_kernel<4, 2, 1, 2, 32>), grid, dim3(512), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((gemm_f64_kernel<2, 2, 1, 1, 32>), grid, dim3(256), 0, ctx->stream, a);
     NXH_HIP("matmul", hipGetLastError());
   }
   return NXH_OK;
