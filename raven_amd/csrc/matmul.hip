@@ -1346,10 +1346,34 @@ __global__ __launch_bounds__(256) void gemm_repack_kernel(RepackArgs a) {
   const S *src = (const S *)a.src + so + r * a.srs;
   union {
     U4 v4;
+    uint32_t w[4];
     S s[VE];
   } o;
   o.v4 = U4{0, 0, 0, 0};
   if (r < a.rows) {
+    if constexpr (sizeof(S) == 2) {
+      if (a.scs == 1) {
+        // 16-bit elements of a contiguous row: whole 4-byte words from the word-aligned address
+        // at or below the first element, shifted by one element where the row starts on an odd
+        // one (eight 2-byte loads per lane held this copy at half the memory rate). A word is
+        // read only if its first element belongs to the row; elements past the row's end are
+        // cleared afterwards.
+        const uintptr_t first = (uintptr_t)(src + c0);
+        const uint32_t *wp = (const uint32_t *)(first & ~(uintptr_t)3);
+        const int odd = (int)((first >> 1) & 1);
+        const int64_t left = a.cols - c0 + odd;  // elements from wp's first to the row's end
+        uint32_t w[5];
+#pragma unroll
+        for (int j = 0; j < 5; j++) w[j] = (2 * j < left && (j < 4 || odd)) ? wp[j] : 0u;
+#pragma unroll
+        for (int j = 0; j < 4; j++) o.w[j] = odd ? __builtin_amdgcn_alignbit(w[j + 1], w[j], 16) : w[j];
+#pragma unroll
+        for (int j = 0; j < VE; j++)
+          if (c0 + j >= a.cols) o.s[j] = (S)0;
+        ((U4 *)a.dst)[v] = o.v4;
+        return;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < VE; j++)
       if (c0 + j < a.cols) o.s[j] = src[(c0 + j) * a.scs];
