@@ -1233,14 +1233,59 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   if (g.gelu && (a.M % 128 || a.N % 128)) return -1;
   if (pick == 192) pick = 128;
   if constexpr (!EPI) {
-    // One product (no batch) whose blocks leave half of the units idle and whose K is long (a
-    // weight gradient: [768, 8192] x [8192, 768]): K is cut into `split` equal runs of whole slabs,
-    // walked as a batch dim that writes [split][M][N] f32 partial sums, which a second kernel adds
-    // in run order (a fixed order: the same bits on every call) and rounds to the dtype once.
-    if (nbatch == 1 && a.batch.n == 0 && (pick == 1264 || pick == 6464)) {
+    // One product (no batch) cut along K: `split` equal runs of whole slabs are walked as a batch
+    // dim that writes [split][M][N] f32 partial sums (the 16-bit kernels in their f32-output
+    // form), which a second kernel adds in run order (a fixed order: the same bits on every
+    // call) and rounds to the dtype once. shape: 0 = 64 x 64 (f32), 1 = 128 x 64, 2 = 128 x 128 (16-bit).
+    auto cut_along_k = [&](int64_t split, int shape) -> int {
       constexpr int DT = EL::F32 ? NXH_F32 : EL::BF16 ? NXH_BF16 : NXH_F16;
+      void *part = nullptr;
+      int rc = nxh_alloc_locked(ctx, (size_t)split * a.M * a.N * sizeof(float), &part);
+      if (rc) return rc;
+      gemm_tile::Args gs = g;
+      gs.K = a.K / split;
+      gs.nbatch = (uint32_t)split;
+      gs.nbd = 1;
+      gs.bshape[0] = (uint32_t)split;
+      gs.ba[0] = gs.K * (a_kc ? 1 : g.lda);
+      gs.bb[0] = gs.K * (b_kc ? 1 : g.ldb);
+      gs.bc[0] = a.M * a.N;
+      gs.C = part;
+      gs.ldc = a.N;
+      if constexpr (EL::F32) {
+        rc = shape == 0 ? launch_tile_oriented<EL, gemm_tile::Shape64x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_64x64_splitk")
+                        : launch_tile_oriented<EL, gemm_tile::Shape128x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
+      } else {
+        rc = shape == 2 ? launch_tile_oriented<EL, gemm_tile::Shape128x128, false, true>(ctx, gs, a_kc, b_kc, "gemm_tile_128x128_splitk")
+                        : launch_tile_oriented<EL, gemm_tile::Shape128x64, false, true>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
+      }
+      if (rc == NXH_OK) {
+        const int64_t total = a.M * a.N;
+        hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0, ctx->stream,
+                           (const float *)part, g.C, a.M, a.N, (int)split, g.ldc, (int64_t)1);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = nxh_hip_fail("matmul", e);
+      }
+      nxh_free_locked(ctx, part);
+      return rc;
+    };
+    const int64_t slabs = a.K / BK;
+    // A 16-bit weight matrix of 16 MiB or more streamed once past at most 128 rows (a decode step
+    // of 17 to 128 sequences): memory-bound on B. 128-column blocks keep 256-byte row segments and
+    // two slabs of 16 KiB in flight each ([32,4096] x [4096,32000], 250 such blocks, streams B
+    // at 6 TB/s); with fewer column blocks than units K is cut until the blocks fill the chip.
+    if constexpr (!EL::F32) {
+      if (nbatch == 1 && a.batch.n == 0 && a.M <= 128 && !forced_tile() &&
+          (double)a.K * (double)a.N * 2.0 >= (double)(16 << 20) && tiles(128, 128) < cus) {
+        int64_t split = std::min<int64_t>(cus / tiles(128, 128), slabs / 8);
+        while (split > 1 && slabs % split) split--;
+        if (split >= 2) return cut_along_k(split, 2);
+      }
+    }
+    // A product whose blocks leave half of the units idle and whose K is long (a weight gradient:
+    // [768, 8192] x [8192, 768]).
+    if (nbatch == 1 && a.batch.n == 0 && (pick == 1264 || pick == 6464)) {
       const int64_t blocks = pick == 6464 ? tiles(64, 64) : tiles(128, 64);
-      const int64_t slabs = a.K / BK;
       // Worth it when the slabs a block no longer walks (about 0.3 us each for a 16-bit block that
       // has its unit to itself, 0.7 us for f32) outweigh the second launch and the partial sums'
       // trip through memory (bf16 [1000,8192] x [8192,1000]: 57 -> 39 us with two runs; [1024,1024]^2
@@ -1256,36 +1301,7 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
           split = sp;
         }
       }
-      if (split >= 2) {
-        void *part = nullptr;
-        int rc = nxh_alloc_locked(ctx, (size_t)split * a.M * a.N * sizeof(float), &part);
-        if (rc) return rc;
-        gemm_tile::Args gs = g;
-        gs.K = a.K / split;
-        gs.nbatch = (uint32_t)split;
-        gs.nbd = 1;
-        gs.bshape[0] = (uint32_t)split;
-        gs.ba[0] = gs.K * (a_kc ? 1 : g.lda);
-        gs.bb[0] = gs.K * (b_kc ? 1 : g.ldb);
-        gs.bc[0] = a.M * a.N;
-        gs.C = part;
-        gs.ldc = a.N;
-        if constexpr (EL::F32) {
-          rc = pick == 6464 ? launch_tile_oriented<EL, gemm_tile::Shape64x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_64x64_splitk")
-                            : launch_tile_oriented<EL, gemm_tile::Shape128x64, false>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
-        } else {
-          rc = launch_tile_oriented<EL, gemm_tile::Shape128x64, false, true>(ctx, gs, a_kc, b_kc, "gemm_tile_128x64_splitk");
-        }
-        if (rc == NXH_OK) {
-          const int64_t total = a.M * a.N;
-          hipLaunchKernelGGL((skinny_finish_kernel<DT>), dim3((unsigned)((total + 1023) / 1024)), dim3(256), 0,
-                             ctx->stream, (const float *)part, g.C, a.M, a.N, (int)split, g.ldc, (int64_t)1);
-          hipError_t e = hipGetLastError();
-          if (e != hipSuccess) rc = nxh_hip_fail("matmul", e);
-        }
-        nxh_free_locked(ctx, part);
-        return rc;
-      }
+      if (split >= 2) return cut_along_k(split, pick == 6464 ? 0 : 1);
     }
   }
   if constexpr (EL::F32) {
@@ -1475,8 +1491,17 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
   if (nbatch == 1 && a.M <= 16 && a.bcs == 1 && a.N >= 1024 && a.K >= 256 && a.batch.n == 0) {
     constexpr int VN = 16 / (int)sizeof(S);  // one 16-byte load per lane and row of B
     if (a.brs % VN == 0 && ((uintptr_t)a.B % (sizeof(S) * VN)) == 0) {
-      if constexpr (sizeof(S) == 2)
+      if constexpr (sizeof(S) == 2) {
+        // fewer 64-column strips than units: the 128-column blocks cut along K (try_tile) stream
+        // B faster than the strips with K split across blocks ([16,4096] x [4096,8192]: 24.5 us there)
+        const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+        if (a.M >= 8 && a.N < (int64_t)64 * cus && (double)a.K * (double)a.N * 2.0 >= (double)(16 << 20)) {
+          using EL = std::conditional_t<MM::DT == NXH_BF16, gemm_tile::ElBF16, gemm_tile::ElF16>;
+          const int rc = try_tile<EL>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
+          if (rc != -1) return rc;
+        }
         if (a.N % 8 == 0) return launch_skinny_mfma<MM::DT>(ctx, a);
+      }
       return launch_skinny<MM::DT, VN>(ctx, a);
     }
   }

@@ -449,6 +449,33 @@ def test_matmul_few_blocks_cut_along_k(hip, oracle, d):
 
 
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_streamed_weights_cut_along_k(hip, oracle, d):
+    """A decode step of 8 to 128 sequences against a weight matrix of 16 MiB or more with fewer
+    128-column blocks than compute units: 128 x 128 blocks cut along K, f32 partial sums added in a
+    fixed order. Both layouts of the weights ([K, N] and the transposed view of [N, K])."""
+    rng = np.random.default_rng(1480 + d.tag)
+    T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
+    for (m, k, n) in [(32, 4096, 4096), (8, 2048, 8192), (100, 4096, 2176)]:
+        a = encode(rng.standard_normal((m, k)), d, oracle)
+        b = encode(rng.standard_normal((k, n)) * 0.1, d, oracle)
+        want = ref_f64(a, b, d, oracle)
+        ha = pair(a, d, hip, oracle)[0]
+        for tb in (False, True):
+            hb = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle, T if tb else None)[0]
+            first = logical(hip.matmul(ha, hb))
+            assert hip.last_path() == "gemm_tile_128x128_splitk", (m, k, n, tb, hip.last_path())
+            got = decode(first, d, oracle)
+            ulp = 2.0 ** (-8 if d is dt.bfloat16 else -11)
+            assert np.all(np.abs(got - want) <= ulp * 2 * np.abs(want) + np.sqrt(k) * 4e-6), (m, k, n, tb)
+            same_bits(logical(hip.matmul(ha, hb)), first, "same bits on every call")
+    # below 16 MiB of weights the strips keep the call
+    a = encode(rng.standard_normal((8, 1024)), d, oracle)
+    b = encode(rng.standard_normal((1024, 4096)), d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "small weights")
+    assert hip.last_path().startswith("gemm_skinny"), hip.last_path()
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
 def test_matmul_direct_to_lds_kernel(hip, oracle, d):
     """The large-product form (operands straight from global memory into swizzled LDS
     tiles, 16x16x32 MFMA): every operand orientation, one to seven K-slabs, batches
