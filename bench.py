@@ -246,7 +246,7 @@ def next_ops(hip, W, linalg=False):
     n = 1 << 24
     ctr = W.dev(np.arange(2 * n, dtype=np.int64).astype(np.int32).reshape(n, 2), dt.int32)
     key = hip.expand(W.dev(np.array([[1234, -99]], np.int32), dt.int32), (n, 2))
-    timed("threefry 2^24 vectors (one key)", lambda: hip.threefry(key, ctr), 2 * n * 8)
+    timed("threefry 2^24 vectors (one key; threefry_dense)", lambda: hip.threefry(key, ctr), 2 * n * 8)
     vocab, dim, ntok = 50257, 768, 8192
     ids = W.dev(rng.integers(0, vocab, (ntok, 1)).astype(np.int32), dt.int32)
     idx = hip.expand(ids, (ntok, dim))

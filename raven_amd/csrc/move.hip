@@ -548,6 +548,48 @@ __global__ __launch_bounds__(256) void threefry_kernel(ThreefryArgs a) {
   a.out[ob + a.out_last] = (int32_t)x1;
 }
 
+// The dense form: counters and results are contiguous (vector, word) pairs, the keys one pair
+// for all vectors or dense too. A lane takes two neighbouring vectors with one 16-byte load and
+// one 16-byte store (two independent chains of rounds) and no division; a lane per vector with
+// 4-byte accesses and a 64-bit division left the call at half the memory rate.
+__device__ __forceinline__ void threefry_block(uint32_t k0, uint32_t k1, uint32_t &x0, uint32_t &x1) {
+  const uint32_t ks[3] = {k0, k1, 0x1BD11BDAu ^ k0 ^ k1};
+  x0 += k0;
+  x1 += k1;
+  constexpr int rots[8] = {13, 15, 26, 6, 17, 29, 16, 24};
+#pragma unroll
+  for (int r = 0; r < 20; r++) {
+    x0 += x1;
+    x1 = rotl32(x1, rots[r % 8]);
+    x1 ^= x0;
+    if ((r + 1) % 4 == 0) {
+      const int s = (r + 1) / 4;
+      x0 += ks[s % 3];
+      x1 += ks[(s + 1) % 3] + (uint32_t)s;
+    }
+  }
+}
+__global__ __launch_bounds__(256) void threefry_dense_kernel(const int32_t *key, int64_t key_step, int64_t key_last,
+                                                             const int32_t *ctr, int32_t *out, int64_t vectors) {
+  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+  const int64_t v = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;
+  if (v >= vectors) return;
+  const uint32_t ka0 = (uint32_t)key[v * key_step], ka1 = (uint32_t)key[v * key_step + key_last];
+  if (v + 1 < vectors) {
+    const uint32_t kb0 = (uint32_t)key[(v + 1) * key_step], kb1 = (uint32_t)key[(v + 1) * key_step + key_last];
+    const u32x4 x = *reinterpret_cast<const u32x4 *>(ctr + 2 * v);
+    uint32_t a0 = x[0], a1 = x[1], b0 = x[2], b1 = x[3];
+    threefry_block(ka0, ka1, a0, a1);
+    threefry_block(kb0, kb1, b0, b1);
+    *reinterpret_cast<u32x4 *>(out + 2 * v) = u32x4{a0, a1, b0, b1};
+  } else {
+    uint32_t x0 = (uint32_t)ctr[2 * v], x1 = (uint32_t)ctr[2 * v + 1];
+    threefry_block(ka0, ka1, x0, x1);
+    out[2 * v] = (int32_t)x0;
+    out[2 * v + 1] = (int32_t)x1;
+  }
+}
+
 NXH_EXPORT int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *key,
                             const nxh_tensor *counter) {
   NXH_DEFER_TOUCH(ctx, 1, out, key, counter);
@@ -585,6 +627,19 @@ NXH_EXPORT int nxh_threefry(nxh_context *ctx, const nxh_tensor *out, const nxh_t
   a.out_last = out->strides[last];
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
+  // dense: every prefix dim composes with the next on all three operands, pairs are contiguous
+  bool dense = last >= 1 && a.ctr_last == 1 && a.out_last == 1 && a.cstride[last - 1] == 2 && a.ostride[last - 1] == 2 &&
+               ((uintptr_t)a.ctr % 16) == 0 && ((uintptr_t)a.out % 16) == 0;
+  for (int d = last - 2; dense && d >= 0; d--)
+    dense = a.cstride[d] == a.cstride[d + 1] * a.shape[d + 1] && a.ostride[d] == a.ostride[d + 1] * a.shape[d + 1] &&
+            a.kstride[d] == a.kstride[d + 1] * a.shape[d + 1];
+  if (dense) {
+    nxh_set_path("threefry_dense");
+    hipLaunchKernelGGL(threefry_dense_kernel, dim3((unsigned)((a.vectors + 511) / 512)), dim3(256), 0, ctx->stream, a.key,
+                       a.kstride[last - 1], a.key_last, a.ctr, a.out, a.vectors);
+    NXH_HIP(op, hipGetLastError());
+    return NXH_OK;
+  }
   nxh_set_path("threefry");
   hipLaunchKernelGGL(threefry_kernel, dim3((unsigned)((a.vectors + 255) / 256)), dim3(256), 0, ctx->stream, a);
   NXH_HIP(op, hipGetLastError());

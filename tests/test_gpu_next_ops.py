@@ -27,11 +27,19 @@ def test_threefry_known_answers_and_oracle(hip, oracle):
         k, c = np.array(case["key"], np.int32), np.array(case["counter"], np.int32)
         assert logical(hip.threefry(mk(hip, k, dt.int32), mk(hip, c, dt.int32))).tolist() == case["out"]
     rng = np.random.default_rng(50)
-    for shape in ((2,), (1000, 2), (7, 33, 2)):
+    # (dense counters and results take two vectors per lane; odd counts end on a single one)
+    for shape, path in (((2,), "threefry"), ((1000, 2), "threefry_dense"), ((7, 33, 2), "threefry_dense"),
+                        ((100001, 2), "threefry_dense")):
         key = rng.integers(-2**31, 2**31, shape).astype(np.int32)
         ctr = rng.integers(-2**31, 2**31, shape).astype(np.int32)
         same_bits(logical(hip.threefry(mk(hip, key, dt.int32), mk(hip, ctr, dt.int32))),
                   logical(oracle.threefry(mk(oracle, key, dt.int32), mk(oracle, ctr, dt.int32))))
+        assert hip.last_path() == path, (shape, hip.last_path())
+    # counters that are a strided view (every other vector) keep the general kernel
+    wide = rng.integers(-2**31, 2**31, (64, 2, 2)).astype(np.int32)
+    key = rng.integers(-2**31, 2**31, (64, 2)).astype(np.int32)
+    hc, oc = (B.reshape(B.shrink(mk(B, wide, dt.int32), [(0, 64), (0, 1), (0, 2)]), (64, 2)) for B in (hip, oracle))
+    same_bits(logical(hip.threefry(mk(hip, key, dt.int32), hc)), logical(oracle.threefry(mk(oracle, key, dt.int32), oc)))
     assert hip.last_path() == "threefry"
     # strided key (word pair along a non-unit stride), broadcast key over counters
     key = rng.integers(-2**31, 2**31, (2, 9)).astype(np.int32)
