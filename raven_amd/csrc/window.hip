@@ -364,9 +364,28 @@ int unfold_launch_v(nxh_context *ctx, const char *op, const WindowArgs &a, int k
 // output allows it: that dim's window count a multiple of 4, windows
 // contiguous, every row of the output starting on a 4-element boundary.
 // `aligned_rows`: the input side of the aligned form (see unfold_kernel) holds.
+// `pair_ok`: the same for pairs of windows (a 14 x 14 image has 196-element rows of windows,
+// whole vectors, but 14 windows per image row: pairs never straddle an image row, fours do).
 template <class E>
-int unfold_launch(nxh_context *ctx, const char *op, WindowArgs &a, int kt, bool vector_ok, bool aligned_rows) {
+int unfold_launch(nxh_context *ctx, const char *op, WindowArgs &a, int kt, bool vector_ok, bool aligned_rows,
+                  bool pair_ok) {
   constexpr int VW = sizeof(E) <= 4 ? 4 : 1;
+  auto in_units_of = [&](int vw) {
+    a.L /= vw;
+    a.win[kt - 1] /= vw;
+    int64_t rest = 256;
+    for (int s = kt - 1; s >= 0; s--) {  // 256 units further, in the new radix
+      a.step[s] = rest % a.win[s];
+      rest /= a.win[s];
+    }
+  };
+  if constexpr (sizeof(E) <= 8) {
+    if (pair_ok && a.win[kt - 1] % 2 == 0 && !(VW > 1 && vector_ok && a.win[kt - 1] % VW == 0)) {
+      in_units_of(2);
+      nxh_set_path("unfold_pairs");
+      return unfold_launch_v<E, 2>(ctx, op, a, kt);
+    }
+  }
   if constexpr (VW > 1) {
     if (vector_ok && a.win[kt - 1] % VW == 0) {
       a.L /= VW;
@@ -484,6 +503,9 @@ NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
     if (a.lshape[d] > 1 && a.l_out[d] % 4 != 0) vector_ok = false;
   // the input side of the aligned form: unit stride along the last window dim, whose rows
   // are whole 4-element vectors, every other step of the input a multiple of 4 elements
+  bool pair_ok = a.win_stride == 1 && a.tap_stride % 2 == 0 && ((uintptr_t)a.out % (uintptr_t)(2 * es)) == 0;
+  for (int d = 0; d < a.ld; d++)
+    if (a.lshape[d] > 1 && a.l_out[d] % 2 != 0) pair_ok = false;
   bool aligned_rows = a.sp_stride[kt - 1] == 1 && a.extent[kt - 1] % 4 == 0 && ((uintptr_t)a.in % (uintptr_t)(4 * es)) == 0;
   for (int d = 0; d < kt - 1; d++)
     if (a.extent[d] > 1 && a.sp_stride[d] % 4 != 0) aligned_rows = false;
@@ -493,11 +515,11 @@ NXH_EXPORT int nxh_unfold(nxh_context *ctx, const nxh_tensor *out, const nxh_ten
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path("unfold");
   switch (es) {
-    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
-    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
-    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
-    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt, vector_ok, aligned_rows); break;
-    default: rc = unfold_launch<G16w>(ctx, op, a, kt, vector_ok, false); break;
+    case 1: rc = unfold_launch<uint8_t>(ctx, op, a, kt, vector_ok, aligned_rows, pair_ok); break;
+    case 2: rc = unfold_launch<uint16_t>(ctx, op, a, kt, vector_ok, aligned_rows, pair_ok); break;
+    case 4: rc = unfold_launch<uint32_t>(ctx, op, a, kt, vector_ok, aligned_rows, pair_ok); break;
+    case 8: rc = unfold_launch<uint64_t>(ctx, op, a, kt, vector_ok, aligned_rows, pair_ok); break;
+    default: rc = unfold_launch<G16w>(ctx, op, a, kt, vector_ok, false, false); break;
   }
   if (rc) return rc;
   NXH_HIP(op, hipGetLastError());

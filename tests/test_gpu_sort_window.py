@@ -186,7 +186,7 @@ def test_window_reference_vectors(hip):
         got = hip.unfold(mk(hip, np.array(c["x"]), dt.float64), c["kernel"], c["stride"], c["dilation"],
                          [tuple(p) for p in c["padding"]])
         assert logical(got).tolist() == c["out"], c["name"]
-        assert hip.last_path() == "unfold"
+        assert hip.last_path() in ("unfold", "unfold_pairs")
     c = W["fold_inverts_unfold"]
     x = np.array(c["x"])
     u = hip.unfold(mk(hip, x, dt.float64), c["kernel"], c["stride"], [1], [(0, 0)])
@@ -248,6 +248,22 @@ def test_unfold_and_fold_match_oracle(hip, oracle, d):
     hp_, op_ = (B.permute(t, (1, 0, 2, 3)) for B, t in ((hip, hip.reshape(hu, (2, 6, 3, 9))), (oracle, oracle.reshape(ou, (2, 6, 3, 9)))))
     same_bits(logical(hip.fold(hp_, [9], [3], [1], [1], [(1, 1)])), logical(oracle.fold(op_, [9], [3], [1], [1], [(1, 1)])),
               "fold permuted")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.uint8], ids=lambda d: d.name)
+def test_unfold_pairs_of_windows(hip, oracle, d):
+    """Window counts per image row that are even but no multiple of four (14 x 14 and 6 x 6 images
+    under a "same" 3 x 3 kernel, a strided 5 x 5): two windows per store."""
+    rng = np.random.default_rng(540 + d.tag)
+    for shape, ks, st, dl, pd in [((2, 3, 14, 14), [3, 3], [1, 1], [1, 1], [(1, 1), (1, 1)]),
+                                  ((3, 2, 6, 6), [3, 3], [1, 1], [1, 1], [(1, 1), (1, 1)]),
+                                  ((2, 2, 13, 19), [5, 5], [2, 2], [1, 1], [(2, 2), (2, 2)]),
+                                  ((4, 30), [3], [1], [2], [(2, 2)])]:
+        x = encode(rng.standard_normal(shape), d, oracle) if d.is_float else rng.integers(0, 100, shape).astype(d.np_storage)
+        h, o = pair(x, d, hip, oracle)
+        hu, ou = hip.unfold(h, ks, st, dl, pd), oracle.unfold(o, ks, st, dl, pd)
+        assert hip.last_path() == "unfold_pairs", (shape, hip.last_path())
+        same_bits(logical(hu), logical(ou), f"unfold {d.name} {shape}")
 
 
 def test_unfold_matmul_is_a_convolution(hip, oracle):
