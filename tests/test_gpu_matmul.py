@@ -396,6 +396,9 @@ def test_matmul_f64_matrix_kernel(hip, oracle):
     fl = lambda B, t: B.flip(t, (True, True))  # noqa: E731
     got = logical(hip.matmul(pair(a, d, hip, oracle, fl)[0], pair(b, d, hip, oracle, fl)[0]))
     assert hip.last_path() == "gemm_f64_32x32" and np.allclose(got, a[::-1, ::-1] @ b[::-1, ::-1], rtol=1e-12, atol=1e-12)
+    # k == 0 stores zeros
+    z = logical(hip.matmul(hip.buffer(d, (70, 0)), hip.buffer(d, (0, 40))))
+    assert z.shape == (70, 40) and not z.any()
     # non-finite values stay where the arithmetic puts them
     a = rng.standard_normal((64, 33))
     b = rng.standard_normal((33, 64))
