@@ -445,6 +445,25 @@ enum {
 };
 int nxh_deferred_stats(nxh_context *ctx, uint64_t *stats, int count);
 
+/* ── memory-side cache policy ────────────────────────────────────────────── */
+
+/* No counterpart in the reference (a CPU's caches need no help from a backend).
+   The MI355X keeps the last 256 MB read or written in a cache in front of HBM.
+   While the tensors of the recent calls add up to more than that, the
+   elementwise kernels write a result that was never read back while cached the
+   last few times its block was written with non-temporal stores, and read an
+   operand whose block was not read again in time with non-temporal loads, so
+   that what the next call reads stays cached. The decision is per call, from a
+   two-bit history per block of 8 MiB or more and the order of the calls; it
+   changes when data reaches HBM, never a result. mode: bit 0 allows streaming
+   loads, bit 1 streaming stores; 3 is the default, 0 turns the policy off (the
+   environment variable NXH_CACHE_HINTS sets the initial value). Bit 2 makes
+   every access stream that a kernel can stream, whatever the history and the
+   size: for tests of those code paths. */
+int nxh_set_cache_policy(nxh_context *ctx, int mode);
+/* Calls so far whose inputs / whose result streamed past the cache. */
+int nxh_cache_policy_stats(nxh_context *ctx, uint64_t *calls_streaming_in, uint64_t *calls_streaming_out);
+
 /* ── recorded sequences ──────────────────────────────────────────────────── */
 
 /* The reference backend has no counterpart: its eager calls cost a C stub

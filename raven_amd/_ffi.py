@@ -112,6 +112,8 @@ SIGNATURES = {
     "nxh_attention": (C.c_int, [_CTX, _T, _T, _T, _T, C.c_void_p, _T, C.c_void_p, C.c_int]),
     "nxh_set_deferred": (C.c_int, [_CTX, C.c_int]),
     "nxh_deferred_stats": (C.c_int, [_CTX, _P(C.c_uint64), C.c_int]),
+    "nxh_set_cache_policy": (C.c_int, [_CTX, C.c_int]),
+    "nxh_cache_policy_stats": (C.c_int, [_CTX, _P(C.c_uint64), _P(C.c_uint64)]),
     "nxh_capture_begin": (C.c_int, [_CTX]),
     "nxh_capture_end": (C.c_int, [_CTX, _P(C.c_void_p)]),
     "nxh_graph_launch": (C.c_int, [_CTX, C.c_void_p]),

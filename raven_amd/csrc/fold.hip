@@ -462,6 +462,7 @@ static int reduce_entry(nxh_context *ctx, int op, const nxh_tensor *out, const n
   }
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(name, hipSetDevice(ctx->device));
+  if (!fixed_scratch) fold_note_access(ctx, x, &sq, g.n_out, g.R);  // (nxh_reduce_noalloc has noted it)
   return fn(ctx, name, x, &sq, g);
 }
 

@@ -41,6 +41,17 @@ static int map_run(nxh_context *ctx, const char *op, map_launch_fn fn, int dt_fo
   if (p.total == 0) return NXH_OK;  // empty tensors are no-ops
   std::lock_guard<std::mutex> g(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
+  // which operands stream past the memory-side cache: distinct bytes per operand
+  const void *base[MAP_MAXOP];
+  uint64_t bytes[MAP_MAXOP];
+  for (int k = 0; k < nop; k++) {
+    int64_t n = 1;
+    for (int d = 0; d < p.ndim; d++)
+      if (p.stride[k][d] != 0) n *= p.shape[d];
+    base[k] = ops[k]->data;
+    bytes[k] = (uint64_t)n * (uint64_t)esize[k];
+  }
+  p.stream = nxh_cache_hints(ctx, nop, base, bytes);
   return fn(ctx, op, p);
 }
 

@@ -20,6 +20,7 @@
 #include <type_traits>
 
 #include "nxh_common.hpp"
+#include "stream_access.hpp"
 
 constexpr int MAP_MAXOP = 4;
 constexpr int MAP_MAXD = 8;
@@ -37,6 +38,7 @@ struct MapPlan {
   int64_t stride[MAP_MAXOP][NXH_MAX_NDIM];  // element strides
   char *base[MAP_MAXOP];                    // byte address of logical element 0
   int esize[MAP_MAXOP];
+  uint32_t stream = 0;  // NXH_STREAM_OUT / NXH_STREAM_IN: accesses that go past the memory-side cache
 };
 
 // Builds the coalesced plan. Returns NXH_OK or a status (aliased output).
@@ -133,10 +135,15 @@ __device__ __forceinline__ typename F::Out map_apply(typename F::In0 a, typename
   else return F::apply(a, b, c);
 }
 
-// Loads V elements of operand type T starting at element index e; `bc` selects a
-// broadcast of the single element at e.
+// Loads V elements of operand type T starting at element index e.
+template <bool STREAM, class T, int V>
+__device__ __forceinline__ Vec<T, V> load_vec(const T *p, int64_t e) {
+  if constexpr (STREAM) return load_stream(reinterpret_cast<const Vec<T, V> *>(p + e));
+  else return *reinterpret_cast<const Vec<T, V> *>(p + e);
+}
+// The same, or a broadcast of the single element at e.
 template <class T, int V>
-__device__ __forceinline__ Vec<T, V> load_vec(const T *p, int64_t e, bool bc) {
+__device__ __forceinline__ Vec<T, V> load_vec_or_splat(const T *p, int64_t e, bool bc) {
   Vec<T, V> r;
   if (bc) {
     T x = p[e];
@@ -156,8 +163,29 @@ struct ContigArgs {
   const typename F::In1 *in1;
   const typename F::In2 *in2;
   int64_t n;       // elements
-  uint32_t bcast;  // bit k set: input k is a broadcast scalar
+  uint32_t bcast;   // bit k set: input k is a broadcast scalar
+  uint32_t stream;  // NXH_STREAM_OUT / NXH_STREAM_IN
 };
+
+// The loads of one lane: UNR vectors of every input that is not a broadcast scalar, issued
+// back to back. Nothing here uses a loaded value, so no load waits for another.
+template <bool STREAM, class F, int V, int UNR>
+__device__ __forceinline__ void contig_fetch(const ContigArgs<F> &a, int64_t base, int64_t nvec,
+                                             Vec<typename F::In0, V> (&x0)[UNR], Vec<typename F::In1, V> (&x1)[UNR],
+                                             Vec<typename F::In2, V> (&x2)[UNR]) {
+  const bool b0 = a.bcast & 1u, b1 = a.bcast & 2u, b2 = a.bcast & 4u;
+#pragma unroll
+  for (int j = 0; j < UNR; j++) {
+    const int64_t u = base + (int64_t)j * MAP_THREADS;
+    if (u < nvec) {
+      if (!b0) x0[j] = load_vec<STREAM, typename F::In0, V>(a.in0, u * V);
+      if constexpr (F::NIN > 1)
+        if (!b1) x1[j] = load_vec<STREAM, typename F::In1, V>(a.in1, u * V);
+      if constexpr (F::NIN > 2)
+        if (!b2) x2[j] = load_vec<STREAM, typename F::In2, V>(a.in2, u * V);
+    }
+  }
+}
 
 template <class F, int V, int UNR>
 __global__ __launch_bounds__(MAP_THREADS) void map_contig_kernel(ContigArgs<F> a) {
@@ -165,26 +193,48 @@ __global__ __launch_bounds__(MAP_THREADS) void map_contig_kernel(ContigArgs<F> a
   const int64_t nvec = a.n / V;
   const int64_t base = (int64_t)blockIdx.x * (MAP_THREADS * UNR) + threadIdx.x;
   const bool b0 = a.bcast & 1u, b1 = a.bcast & 2u, b2 = a.bcast & 4u;
+  // a broadcast scalar is read once, in front of the vector loads, and chosen per element
+  // afterwards: filling a vector with it between the loads would make every later load
+  // wait for the earlier ones
+  typename MT::In0 s0{};
+  typename MT::In1 s1{};
+  typename MT::In2 s2{};
+  if (b0) s0 = a.in0[0];
+  if constexpr (F::NIN > 1)
+    if (b1) s1 = a.in1[0];
+  if constexpr (F::NIN > 2)
+    if (b2) s2 = a.in2[0];
   Vec<typename MT::In0, V> x0[UNR];
   Vec<typename MT::In1, V> x1[UNR];
   Vec<typename MT::In2, V> x2[UNR];
+  if (a.stream & NXH_STREAM_IN) contig_fetch<true, F, V, UNR>(a, base, nvec, x0, x1, x2);
+  else contig_fetch<false, F, V, UNR>(a, base, nvec, x0, x1, x2);
+  wait_for_loads();
+  Vec<typename MT::Out, V> r[UNR];
 #pragma unroll
-  for (int j = 0; j < UNR; j++) {
-    int64_t u = base + (int64_t)j * MAP_THREADS;
-    if (u < nvec) {
-      x0[j] = load_vec<typename MT::In0, V>(a.in0, b0 ? 0 : u * V, b0);
-      if constexpr (F::NIN > 1) x1[j] = load_vec<typename MT::In1, V>(a.in1, b1 ? 0 : u * V, b1);
-      if constexpr (F::NIN > 2) x2[j] = load_vec<typename MT::In2, V>(a.in2, b2 ? 0 : u * V, b2);
+  for (int j = 0; j < UNR; j++)
+    if (base + (int64_t)j * MAP_THREADS < nvec) {
+#pragma unroll
+      for (int i = 0; i < V; i++) {
+        typename MT::In0 v0 = b0 ? s0 : x0[j].v[i];
+        typename MT::In1 v1{};
+        typename MT::In2 v2{};
+        if constexpr (F::NIN > 1) v1 = b1 ? s1 : x1[j].v[i];
+        if constexpr (F::NIN > 2) v2 = b2 ? s2 : x2[j].v[i];
+        r[j].v[i] = map_apply<F>(v0, v1, v2);
+      }
     }
-  }
+  if (a.stream & NXH_STREAM_OUT) {
 #pragma unroll
-  for (int j = 0; j < UNR; j++) {
-    int64_t u = base + (int64_t)j * MAP_THREADS;
-    if (u < nvec) {
-      Vec<typename MT::Out, V> r;
+    for (int j = 0; j < UNR; j++) {
+      const int64_t u = base + (int64_t)j * MAP_THREADS;
+      if (u < nvec) store_stream(reinterpret_cast<Vec<typename MT::Out, V> *>(a.out + u * V), r[j]);
+    }
+  } else {
 #pragma unroll
-      for (int i = 0; i < V; i++) r.v[i] = map_apply<F>(x0[j].v[i], x1[j].v[i], x2[j].v[i]);
-      *reinterpret_cast<Vec<typename MT::Out, V> *>(a.out + u * V) = r;
+    for (int j = 0; j < UNR; j++) {
+      const int64_t u = base + (int64_t)j * MAP_THREADS;
+      if (u < nvec) *reinterpret_cast<Vec<typename MT::Out, V> *>(a.out + u * V) = r[j];
     }
   }
   // ragged tail: fewer than V elements, one lane each
@@ -232,13 +282,13 @@ __global__ __launch_bounds__(MAP_THREADS) void map_generic_kernel(GenericArgs<F>
         for (int k = 0; k <= F::NIN; k++) off[k] += (int64_t)c * a.stride[k][d];
       }
       oo[j] = off[0];
-      x0[j] = load_vec<typename MT::In0, V>((const typename MT::In0 *)a.base[1], off[1],
+      x0[j] = load_vec_or_splat<typename MT::In0, V>((const typename MT::In0 *)a.base[1], off[1],
                                             V > 1 && (a.inner_bcast & 2u));
       if constexpr (F::NIN > 1)
-        x1[j] = load_vec<typename MT::In1, V>((const typename MT::In1 *)a.base[2], off[2],
+        x1[j] = load_vec_or_splat<typename MT::In1, V>((const typename MT::In1 *)a.base[2], off[2],
                                               V > 1 && (a.inner_bcast & 4u));
       if constexpr (F::NIN > 2)
-        x2[j] = load_vec<typename MT::In2, V>((const typename MT::In2 *)a.base[3], off[3],
+        x2[j] = load_vec_or_splat<typename MT::In2, V>((const typename MT::In2 *)a.base[3], off[3],
                                               V > 1 && (a.inner_bcast & 8u));
     }
   }
@@ -260,7 +310,7 @@ __global__ __launch_bounds__(MAP_THREADS) void map_generic_kernel(GenericArgs<F>
 // block. A block of 256 lanes owns a TILE x TILE patch; every lane moves V
 // consecutive elements per access (16 bytes of the widest operand type), so a
 // wave touches whole 256-byte rows on both sides of the turn.
-enum { TILE_ROW = 0, TILE_TURN = 1, TILE_BX = 2, TILE_ANY = 3 };
+enum { TILE_ROW = 0, TILE_TURN = 1, TILE_BX = 2 };
 
 template <class F>
 struct TiledArgs {
@@ -271,18 +321,18 @@ struct TiledArgs {
   int64_t bstride[MAP_MAXOP][MAP_MAXD];
   int64_t sx[MAP_MAXOP], sy[MAP_MAXOP];  // element strides along x / y
   // per input: TILE_ROW unit stride along x, TILE_TURN unit stride along y (read
-  // along y, turned through LDS), TILE_BX broadcast along x, TILE_ANY strided
+  // along y, turned through LDS), TILE_BX broadcast along x
   uint32_t mode[MAP_MAXOP];
   uint32_t any_turn;
+  uint32_t stream;  // NXH_STREAM_OUT / NXH_STREAM_IN (the vector accesses of ROW / TURN operands)
 };
 
 // Tile geometry. The patch is TX (along x) by TY (along y) elements. Everything that is
-// stored, and every input that is not turned, moves in the OUTPUT arrangement: VX
+// stored, and every input with a unit stride along x, moves in the OUTPUT arrangement: VX
 // consecutive x per lane, GXO lanes across a row, RYO rows per pass of the block, NYO
 // passes. A turned input is fetched in its own arrangement: VY consecutive y per lane, GYT
-// lanes along y, RXT columns per pass, NXT passes. VX and VY differ when the output is
-// narrower than the turned input (a compare of 4-byte operands stores 16 one-byte results
-// per lane, so that a wave still writes whole 128-byte rows).
+// lanes along y, RXT columns per pass, NXT passes. The kernel uses VX = VY, which makes
+// NYO = NXT.
 template <int TX, int TY, int VX, int VY>
 struct TileGeom {
   static constexpr int GXO = TX / VX, RYO = MAP_THREADS / GXO, NYO = TY / RYO;
@@ -292,92 +342,89 @@ struct TileGeom {
   static_assert(GYT * VY == TY && GYT * RXT == MAP_THREADS && NXT * RXT == TX && NXT >= 1, "fetch arrangement");
 };
 
-// Issues this lane's global loads of an input that arrives in the output arrangement
-// (VX consecutive x for NYO different y).
-template <class T, class TG, int VX>
-__device__ __forceinline__ void tile_fetch_out(Vec<T, VX> (&r)[TG::NYO], const T *p, int64_t sx, int64_t sy,
-                                               uint32_t x0, uint32_t y0, uint32_t nx, uint32_t ny, uint32_t mode) {
-  const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
-  const uint32_t x = x0 + g * VX;
-  const T *s = p + (int64_t)(y0 + q) * sy + (int64_t)x * sx;
-  const int64_t step = (int64_t)TG::RYO * sy;
-  if (mode == TILE_ROW) {
-#pragma unroll
-    for (int i = 0; i < TG::NYO; i++) {
-      if (x < nx && y0 + q + i * TG::RYO < ny) r[i] = *reinterpret_cast<const Vec<T, VX> *>(s);
-      s += step;
-    }
-  } else if (mode == TILE_BX) {
-#pragma unroll
-    for (int i = 0; i < TG::NYO; i++) {
-      if (x < nx && y0 + q + i * TG::RYO < ny) {
-        const T v = *s;
-#pragma unroll
-        for (int j = 0; j < VX; j++) r[i].v[j] = v;
-      }
-      s += step;
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < TG::NYO; i++) {
-      if (x < nx && y0 + q + i * TG::RYO < ny) {
-#pragma unroll
-        for (int j = 0; j < VX; j++) r[i].v[j] = s[(int64_t)j * sx];
-      }
-      s += step;
-    }
-  }
-}
-// A turned input is fetched along y (VY consecutive y for NXT different x).
-template <class T, class TG, int VY>
-__device__ __forceinline__ void tile_fetch_turn(Vec<T, VY> (&r)[TG::NXT], const T *p, int64_t sx, uint32_t x0,
-                                                uint32_t y0, uint32_t nx, uint32_t ny) {
-  const uint32_t g = threadIdx.x % TG::GYT, q = threadIdx.x / TG::GYT;
-  const uint32_t y = y0 + g * VY;
-  const T *s = p + (int64_t)y + (int64_t)(x0 + q) * sx;
-  const int64_t step = (int64_t)TG::RXT * sx;
-#pragma unroll
-  for (int i = 0; i < TG::NXT; i++) {
-    if (x0 + q + i * TG::RXT < nx && y < ny) r[i] = *reinterpret_cast<const Vec<T, VY> *>(s);
-    s += step;
-  }
-}
-
-// The turn: lds is [y][x] with a one-element pad, written from the fetch arrangement,
-// read in the output arrangement, one element per access.
-template <class T, class TG, int VY>
-__device__ __forceinline__ void tile_put(const Vec<T, VY> (&r)[TG::NXT], T *lds) {
-  const uint32_t g = threadIdx.x % TG::GYT, q = threadIdx.x / TG::GYT;
-#pragma unroll
-  for (int i = 0; i < TG::NXT; i++)
-#pragma unroll
-    for (int j = 0; j < VY; j++) lds[(g * VY + j) * TG::PITCH + q + i * TG::RXT] = r[i].v[j];
-}
-template <class T, class TG, int VX>
-__device__ __forceinline__ void tile_get(Vec<T, VX> (&r)[TG::NYO], const T *lds) {
-  const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
-#pragma unroll
-  for (int i = 0; i < TG::NYO; i++)
-#pragma unroll
-    for (int j = 0; j < VX; j++) r[i].v[j] = lds[(q + i * TG::RYO) * TG::PITCH + g * VX + j];
-}
-
-// One input of the tile: fetched in whichever arrangement its mode asks for.
-template <class T, class TG, int VX, int VY>
+// One input of the tile and this lane's share of it, in two steps. address() works out
+// where the lane's NYO accesses go; fetch() only issues them. The kernel runs address() for
+// every operand before the first fetch(), so that no vector instruction stands between the
+// loads: the compiler reuses registers across the kernel's mutually exclusive paths and, at
+// any instruction that writes a register some other path loads into, waits for all loads.
+// An operand with a unit stride along x (ROW) or along y (TURN) is fetched as V-element
+// vectors along that dim by one piece of code: the two arrangements differ only in which
+// coordinate the lane's vector runs along, a choice that is uniform over the launch. A
+// turned operand then goes through LDS to reach the output arrangement; an operand
+// broadcast along x keeps one value per row in b and is chosen per element where the
+// results are formed.
+template <class T, class TG, int V>
 struct TileOperand {
-  Vec<T, VX> r[TG::NYO];
-  Vec<T, VY> t[TG::NXT];
-  __device__ __forceinline__ void fetch(const T *p, int64_t sx, int64_t sy, uint32_t x0, uint32_t y0, uint32_t nx,
-                                        uint32_t ny, uint32_t mode) {
-    if (mode == TILE_TURN) tile_fetch_turn<T, TG, VY>(t, p, sx, x0, y0, nx, ny);
-    else tile_fetch_out<T, TG, VX>(r, p, sx, sy, x0, y0, nx, ny, mode);
+  static_assert(TG::NYO == TG::NXT, "both arrangements hold the same number of vectors per lane");
+  Vec<T, V> r[TG::NYO];
+  T b[TG::NYO];
+  const NXH_GLOBAL char *at[TG::NYO];
+  bool ok[TG::NYO];
+  __device__ __forceinline__ void address(const T *p, int64_t sx, int64_t sy, uint32_t x0, uint32_t y0, uint32_t nx,
+                                          uint32_t ny, uint32_t mode) {
+    const bool turn = mode == TILE_TURN;
+    // along: the coordinate the vector runs along (x, or y when turned); across: the other
+    const uint32_t G = turn ? TG::GYT : TG::GXO, R = turn ? TG::RXT : TG::RYO;
+    const uint32_t g = threadIdx.x % G, q = threadIdx.x / G;
+    const uint32_t along = (turn ? y0 : x0) + g * V, n_along = turn ? ny : nx;
+    const uint32_t across = (turn ? x0 : y0) + q, n_across = turn ? nx : ny;
+    const int64_t pitch = turn ? sx : sy;
+    const T *s = p + (int64_t)(mode == TILE_BX ? 0u : along) + (int64_t)across * pitch;
+    const int64_t step = (int64_t)R * pitch;
+#pragma unroll
+    for (int i = 0; i < TG::NYO; i++) {
+      at[i] = (const NXH_GLOBAL char *)s;
+      ok[i] = along < n_along && across + i * R < n_across;
+      s += step;
+    }
   }
+  // keeps the addresses computed where address() stands
+  __device__ __forceinline__ void pin() {
+#pragma unroll
+    for (int i = 0; i < TG::NYO; i++) asm volatile("" : "+v"(at[i]));
+  }
+  template <bool STREAM>
+  __device__ __forceinline__ void fetch(uint32_t mode) {
+    if (mode == TILE_BX) {
+#pragma unroll
+      for (int i = 0; i < TG::NYO; i++)
+        if (ok[i]) b[i] = load_global<false, T>(at[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < TG::NYO; i++)
+        if (ok[i]) r[i] = load_global<STREAM, Vec<T, V>>(at[i]);
+    }
+  }
+  // The turn: lds is [y][x] with a one-element pad, written from the fetch arrangement,
+  // read in the output arrangement, one element per access.
+  __device__ __forceinline__ void put(T *lds) const {
+    const uint32_t g = threadIdx.x % TG::GYT, q = threadIdx.x / TG::GYT;
+#pragma unroll
+    for (int i = 0; i < TG::NXT; i++)
+#pragma unroll
+      for (int j = 0; j < V; j++) lds[(g * V + j) * TG::PITCH + q + i * TG::RXT] = r[i].v[j];
+  }
+  __device__ __forceinline__ void get(const T *lds) {
+    const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
+#pragma unroll
+    for (int i = 0; i < TG::NYO; i++)
+#pragma unroll
+      for (int j = 0; j < V; j++) r[i].v[j] = lds[(q + i * TG::RYO) * TG::PITCH + g * V + j];
+  }
+  __device__ __forceinline__ T value(int i, int j, bool bx) const { return bx ? b[i] : r[i].v[j]; }
 };
 
-template <class F, int TX, int TY, int VX, int VY>
+template <bool STREAM, class F, class R0, class R1, class R2>
+__device__ __forceinline__ void tile_fetch_all(const TiledArgs<F> &a, R0 &r0, R1 &r1, R2 &r2) {
+  r0.template fetch<STREAM>(a.mode[1]);
+  if constexpr (F::NIN > 1) r1.template fetch<STREAM>(a.mode[2]);
+  if constexpr (F::NIN > 2) r2.template fetch<STREAM>(a.mode[3]);
+}
+
+template <class F, int TX, int TY, int VX>
 __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) {
   using MT = MapTypes<F>;
-  using TG = TileGeom<TX, TY, VX, VY>;
+  using TG = TileGeom<TX, TY, VX, VX>;
   using I0 = typename MT::In0;
   using I1 = typename MT::In1;
   using I2 = typename MT::In2;
@@ -402,38 +449,62 @@ __global__ __launch_bounds__(MAP_THREADS) void map_tiled_kernel(TiledArgs<F> a) 
     for (int k = 0; k <= F::NIN; k++) off[k] += (int64_t)c * a.bstride[k][d];
   }
   const uint32_t x0 = tx * TX, y0 = ty * TY;
-  TileOperand<I0, TG, VX, VY> r0;
-  TileOperand<I1, TG, VX, VY> r1;
-  TileOperand<I2, TG, VX, VY> r2;
-  r0.fetch((const I0 *)a.base[1] + off[1], a.sx[1], a.sy[1], x0, y0, a.nx, a.ny, a.mode[1]);
-  if constexpr (F::NIN > 1) r1.fetch((const I1 *)a.base[2] + off[2], a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.mode[2]);
-  if constexpr (F::NIN > 2) r2.fetch((const I2 *)a.base[3] + off[3], a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.mode[3]);
+  TileOperand<I0, TG, VX> r0;
+  TileOperand<I1, TG, VX> r1;
+  TileOperand<I2, TG, VX> r2;
+  r0.address((const I0 *)a.base[1] + off[1], a.sx[1], a.sy[1], x0, y0, a.nx, a.ny, a.mode[1]);
+  if constexpr (F::NIN > 1) r1.address((const I1 *)a.base[2] + off[2], a.sx[2], a.sy[2], x0, y0, a.nx, a.ny, a.mode[2]);
+  if constexpr (F::NIN > 2) r2.address((const I2 *)a.base[3] + off[3], a.sx[3], a.sy[3], x0, y0, a.nx, a.ny, a.mode[3]);
+  r0.pin();
+  if constexpr (F::NIN > 1) r1.pin();
+  if constexpr (F::NIN > 2) r2.pin();
+  asm volatile("" ::: "memory");
+  if (a.stream & NXH_STREAM_IN) tile_fetch_all<true, F>(a, r0, r1, r2);
+  else tile_fetch_all<false, F>(a, r0, r1, r2);
+  wait_for_loads();
   if (a.any_turn) {
-    if (a.mode[1] == TILE_TURN) tile_put<I0, TG, VY>(r0.t, l0);
+    if (a.mode[1] == TILE_TURN) r0.put(l0);
     if constexpr (F::NIN > 1)
-      if (a.mode[2] == TILE_TURN) tile_put<I1, TG, VY>(r1.t, l1);
+      if (a.mode[2] == TILE_TURN) r1.put(l1);
     if constexpr (F::NIN > 2)
-      if (a.mode[3] == TILE_TURN) tile_put<I2, TG, VY>(r2.t, l2);
+      if (a.mode[3] == TILE_TURN) r2.put(l2);
     __syncthreads();
-    if (a.mode[1] == TILE_TURN) tile_get<I0, TG, VX>(r0.r, l0);
+    if (a.mode[1] == TILE_TURN) r0.get(l0);
     if constexpr (F::NIN > 1)
-      if (a.mode[2] == TILE_TURN) tile_get<I1, TG, VX>(r1.r, l1);
+      if (a.mode[2] == TILE_TURN) r1.get(l1);
     if constexpr (F::NIN > 2)
-      if (a.mode[3] == TILE_TURN) tile_get<I2, TG, VX>(r2.r, l2);
+      if (a.mode[3] == TILE_TURN) r2.get(l2);
   }
   const uint32_t g = threadIdx.x % TG::GXO, q = threadIdx.x / TG::GXO;
   const uint32_t x = x0 + g * VX;
   O *o = (O *)a.base[0] + off[0] + (int64_t)(y0 + q) * a.sy[0] + x;
   const int64_t step = (int64_t)TG::RYO * a.sy[0];
+  const bool bx0 = a.mode[1] == TILE_BX, bx1 = a.mode[2] == TILE_BX, bx2 = a.mode[3] == TILE_BX;
+  Vec<O, VX> v[TG::NYO];
 #pragma unroll
-  for (int i = 0; i < TG::NYO; i++) {
+  for (int i = 0; i < TG::NYO; i++)
     if (x < a.nx && y0 + q + i * TG::RYO < a.ny) {
-      Vec<O, VX> v;
 #pragma unroll
-      for (int j = 0; j < VX; j++) v.v[j] = map_apply<F>(r0.r[i].v[j], r1.r[i].v[j], r2.r[i].v[j]);
-      *reinterpret_cast<Vec<O, VX> *>(o) = v;
+      for (int j = 0; j < VX; j++) {
+        I1 v1{};
+        I2 v2{};
+        if constexpr (F::NIN > 1) v1 = r1.value(i, j, bx1);
+        if constexpr (F::NIN > 2) v2 = r2.value(i, j, bx2);
+        v[i].v[j] = map_apply<F>(r0.value(i, j, bx0), v1, v2);
+      }
     }
-    o += step;
+  if (a.stream & NXH_STREAM_OUT) {
+#pragma unroll
+    for (int i = 0; i < TG::NYO; i++) {
+      if (x < a.nx && y0 + q + i * TG::RYO < a.ny) store_stream(reinterpret_cast<Vec<O, VX> *>(o), v[i]);
+      o += step;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TG::NYO; i++) {
+      if (x < a.nx && y0 + q + i * TG::RYO < a.ny) *reinterpret_cast<Vec<O, VX> *>(o) = v[i];
+      o += step;
+    }
   }
 }
 
@@ -522,6 +593,7 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       a.in2 = (const typename MT::In2 *)(p.nop > 3 ? p.base[3] : nullptr);
       a.n = p.total;
       a.bcast = bc;
+      a.stream = p.stream;
       nxh_set_path("map_contig");
       if (wide) {
         const int64_t nvec = (p.total + VW - 1) / VW, per_block = MAP_THREADS * UW;
@@ -560,17 +632,20 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       constexpr int TY = MT::smax == 4 ? 32 : (MT::smax < 4 ? 64 : 32);
       TiledArgs<F> a;
       a.any_turn = 0;
+      a.stream = p.stream;
+      bool every_mode = true;
       // 16-byte lanes need every vector of every operand aligned and whole
       bool vec = V > 1 && p.shape[last] % V == 0 && p.shape[ydim] % V == 0;
       for (int k = 0; k < MAP_MAXOP; k++) {
         a.base[k] = k < p.nop ? p.base[k] : nullptr;
         a.sx[k] = k < p.nop ? p.stride[k][last] : 0;
         a.sy[k] = k < p.nop ? p.stride[k][ydim] : 0;
-        a.mode[k] = TILE_ANY;
+        a.mode[k] = TILE_ROW;
         if (k >= p.nop) continue;
         if (a.sx[k] == 1) a.mode[k] = TILE_ROW;
         else if (a.sx[k] == 0) a.mode[k] = TILE_BX;
         else if (a.sy[k] == 1) a.mode[k] = TILE_TURN, a.any_turn = 1;
+        else every_mode = false;  // strided along both: the per-lane index kernel takes it
         if (a.mode[k] == TILE_ROW || a.mode[k] == TILE_TURN) {
           if (!aligned_to(p.base[k], (size_t)esz[k] * V)) vec = false;
           for (int d = 0; d < p.ndim; d++)
@@ -592,13 +667,13 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
         nb *= p.shape[d];
       }
       int64_t blocks = nb * a.tiles_x * a.tiles_y;
-      if (blocks < ((int64_t)1 << 31)) {
+      if (blocks < ((int64_t)1 << 31) && every_mode) {
         nxh_set_path("map_tiled");
         if (vec)
-          hipLaunchKernelGGL((map_tiled_kernel<F, TX, TY, V, V>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+          hipLaunchKernelGGL((map_tiled_kernel<F, TX, TY, V>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
                              ctx->stream, a);
         else
-          hipLaunchKernelGGL((map_tiled_kernel<F, TX, TY, 1, 1>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
+          hipLaunchKernelGGL((map_tiled_kernel<F, TX, TY, 1>), dim3((uint32_t)blocks), dim3(MAP_THREADS), 0,
                              ctx->stream, a);
         NXH_HIP(op, hipGetLastError());
         return NXH_OK;

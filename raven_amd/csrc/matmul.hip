@@ -1692,6 +1692,10 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
 
 NXH_EXPORT int nxh_matmul(nxh_context *ctx, const nxh_tensor *C, const nxh_tensor *A, const nxh_tensor *B) {
   NXH_DEFER_RECORD(ctx, NXH_D_MATMUL, 0, C, 2, nullptr, 0, nullptr, A, B);
+  if (ctx) {
+    const nxh_tensor *touched[] = {C, A, B};
+    nxh_cache_touch(ctx, touched, 3, 1);
+  }
   return matmul_entry(ctx, "matmul", C, A, B, nullptr, nullptr);
 }
 
@@ -1731,6 +1735,7 @@ NXH_EXPORT int nxh_linear_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, con
 int nxh_linear_group(nxh_context *ctx, int n, const nxh_tensor *const *outs, const nxh_tensor *x,
                      const nxh_tensor *const *ws, const nxh_tensor *const *biases) {
   if (n < 2 || n > 3) return nxh_fail(NXH_FAILURE, "linear", "a group has two or three members");
+  nxh_cache_opaque(ctx);  // several outputs and weights, not named one by one to the cache policy
   auto same_layout = [](const nxh_tensor *a, const nxh_tensor *b) {
     if (!a || !b || a->dtype != b->dtype || a->ndim != b->ndim) return false;
     for (int d = 0; d < a->ndim; d++)

@@ -17,6 +17,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/nxhip.h"
@@ -61,6 +62,30 @@ struct nxh_context {
   // this device's copy of the library's static workspace (runtime.hip), for the
   // entry point that may not allocate; shared by every context of the device
   unsigned char *static_ws = nullptr;
+  // Reuse predictor for the 256 MB memory-side cache (runtime.hip, nxh_cache_hints): per
+  // block of 8 MiB or more, where the stream of cache-allocating traffic stood at its
+  // last access, what that access was, and two 2-bit counters: was the block read again
+  // while it could still be cached, after a write and after a read.
+  struct BlockUse {
+    uint64_t pos = 0;
+    uint8_t kind = 0;          // 0 never seen, 1 read, 2 written
+    uint8_t after_write = 2;   // >= 2: keep what is written here in the cache
+    uint8_t after_read = 2;    // >= 2: keep what is read from here in the cache
+    uint64_t opaque = 0;       // opaque_calls at that access
+  };
+  std::unordered_map<const void *, BlockUse> block_use;
+  uint64_t cache_pos = 0;  // bytes of cache-allocating traffic issued so far
+  // the last large-operand accesses (block, bytes): their distinct blocks are the working set
+  static constexpr int RECENT = 32;
+  const void *recent_block[RECENT] = {};
+  uint64_t recent_bytes[RECENT] = {};
+  int recent_next = 0;
+  int cache_hints = 3;     // bit 0: streaming loads allowed, bit 1: streaming stores (NXH_CACHE_HINTS)
+  uint64_t streamed_in = 0, streamed_out = 0;  // calls whose inputs / result streamed
+  // calls so far that may have read or written any block without saying which (transforms,
+  // factorisations, sorts, graph replays, host copies): no block counts as "not touched
+  // again" across one of them
+  uint64_t opaque_calls = 0;
 };
 
 // Size of the static per-device workspace behind nxh_reduce_noalloc.
@@ -90,6 +115,19 @@ int nxh_hip_fail(const char *op, hipError_t e);
 // allocator (runtime.hip)
 int nxh_alloc_locked(nxh_context *ctx, size_t bytes, void **out);
 void nxh_free_locked(nxh_context *ctx, void *p);
+// Cache hints of one launch (runtime.hip). Operand 0 is written, the others are read;
+// `base` are the tensors' data pointers (block bases), `bytes` the distinct bytes the launch
+// touches of each. Returns NXH_STREAM_OUT if what is written should go past the memory-side
+// cache (non-temporal stores) and NXH_STREAM_IN if what is read should (non-temporal loads of
+// every large input). Caller holds ctx->mu.
+enum { NXH_STREAM_OUT = 1u, NXH_STREAM_IN = 2u };
+uint32_t nxh_cache_hints(nxh_context *ctx, int nop, const void *const *base, const uint64_t *bytes,
+                         uint32_t allow = NXH_STREAM_OUT | NXH_STREAM_IN);
+// The same bookkeeping for an entry point whose kernels take no hints: the first n_out
+// tensors are written, the others read (NULL entries are skipped). Takes ctx->mu.
+void nxh_cache_touch(nxh_context *ctx, const nxh_tensor *const *tensors, int n, int n_out);
+// An entry point that may touch blocks it does not name. Takes ctx->mu.
+void nxh_cache_opaque(nxh_context *ctx);
 // the out-of-bounds flag of gather / scatter, read back (or left for the replay) (runtime.hip)
 int nxh_collect_index_fault(nxh_context *ctx, const char *op);
 // Before an eager gather / scatter is launched: a fault that a replayed graph left in
@@ -120,12 +158,15 @@ enum { NXH_D_UNARY, NXH_D_BINARY, NXH_D_COMPARE, NXH_D_WHERE, NXH_D_CAST, NXH_D_
   do {                                                           \
     if ((ctx) && nxh_defer_active(ctx))                          \
       if (int drc__ = nxh_defer_barrier(ctx, ##__VA_ARGS__)) return drc__; \
+    if (ctx) nxh_cache_opaque(ctx);                              \
   } while (0)
 #define NXH_DEFER_TOUCH(ctx, n_out, ...)                                                                      \
   do {                                                                                                        \
-    if ((ctx) && nxh_defer_active(ctx)) {                                                                     \
+    if (ctx) {                                                                                                \
       const nxh_tensor *dts__[] = {__VA_ARGS__};                                                              \
-      if (int drc__ = nxh_defer_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out)) return drc__;  \
+      if (nxh_defer_active(ctx))                                                                              \
+        if (int drc__ = nxh_defer_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out)) return drc__; \
+      nxh_cache_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out);                                \
     }                                                                                                         \
   } while (0)
 #define NXH_DEFER_QUIET(ctx)                                     \

@@ -186,6 +186,16 @@ class Backend:
         self._check(self._lib.nxh_deferred_stats(self._h, v, len(self.DEFER_STATS)))
         return dict(zip(self.DEFER_STATS, (int(x) for x in v)))
 
+    def set_cache_policy(self, mode: int):
+        """Bit 0 allows streaming (non-temporal) loads, bit 1 streaming stores, of blocks whose
+        history says they are not touched again while cached; 0 turns the policy off."""
+        self._check(self._lib.nxh_set_cache_policy(self._h, int(mode)))
+
+    def cache_policy_stats(self):
+        a, b = C.c_uint64(), C.c_uint64()
+        self._check(self._lib.nxh_cache_policy_stats(self._h, C.byref(a), C.byref(b)))
+        return {"streaming_in": a.value, "streaming_out": b.value}
+
     def memory_stats(self):
         v = [C.c_uint64() for _ in range(4)]
         self._check(self._lib.nxh_memory_stats(self._h, *[C.byref(x) for x in v]))

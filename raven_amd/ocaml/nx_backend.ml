@@ -433,6 +433,11 @@ external set_deferred : context -> bool -> unit = "caml_nx_hip_set_deferred"
    softmax_rows, layer_norm_rows, gelu_tanh, attention and linear *)
 external deferred_stats : context -> int array = "caml_nx_hip_deferred_stats"
 
+(* bit 0 allows streaming loads, bit 1 streaming stores, of blocks whose history
+   says they are not touched again while the memory-side cache still holds them *)
+external set_cache_policy : context -> int -> unit = "caml_nx_hip_set_cache_policy"
+external cache_policy_stats : context -> int * int = "caml_nx_hip_cache_policy_stats"
+
 (* nx_effect.ml:376 returns its argument: the reference has one memory. Here a
    tensor of another context of the same GPU is copied by the target context's
    stream once the source stream has drained, and the target is drained before

@@ -38,6 +38,7 @@
   X(triangular_solve) X(qr) X(eigh) X(svd) X(eig) X(device_info)              \
   X(memory_stats) X(trim) X(reduce_noalloc) X(softmax_rows) X(layer_norm_rows) \
   X(gelu_tanh) X(attention) X(linear) X(linear_gelu_tanh) X(set_deferred) X(deferred_stats)        \
+  X(set_cache_policy) X(cache_policy_stats)                                    \
   X(capture_begin) X(capture_end) X(graph_launch) X(graph_destroy)             \
   X(timer_start) X(timer_stop) X(last_path)
 static struct {
@@ -731,6 +732,24 @@ CAMLprim value caml_nx_hip_deferred_stats(value vctx) {
   check(Ctx_val(vctx), L.deferred_stats(Ctx_val(vctx), s, NXH_DEFER_STAT_COUNT));
   v = caml_alloc_tuple(NXH_DEFER_STAT_COUNT);
   for (int i = 0; i < NXH_DEFER_STAT_COUNT; i++) Store_field(v, i, Val_long((long)s[i]));
+  CAMLreturn(v);
+}
+
+/* bit 0: streaming loads, bit 1: streaming stores of blocks that are not touched again while cached */
+CAMLprim value caml_nx_hip_set_cache_policy(value vctx, value vmode) {
+  CAMLparam2(vctx, vmode);
+  check(Ctx_val(vctx), L.set_cache_policy(Ctx_val(vctx), Int_val(vmode)));
+  CAMLreturn(Val_unit);
+}
+/* (calls whose inputs streamed, calls whose result streamed) */
+CAMLprim value caml_nx_hip_cache_policy_stats(value vctx) {
+  CAMLparam1(vctx);
+  CAMLlocal1(v);
+  uint64_t in = 0, out = 0;
+  check(Ctx_val(vctx), L.cache_policy_stats(Ctx_val(vctx), &in, &out));
+  v = caml_alloc_tuple(2);
+  Store_field(v, 0, Val_long((long)in));
+  Store_field(v, 1, Val_long((long)out));
   CAMLreturn(v);
 }
 
