@@ -627,7 +627,8 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       // with a permuted operand: 64 x 64 patches of 4-byte elements ran the config-2 step in
       // 172 us, 64 x 32 in 162 us (more blocks per compute unit, shorter dependent chains
       // through the barrier), 32 x 32 in 177 us, 128 x 64 with 16-byte stores of one-byte
-      // results in 173 us.
+      // results in 173 us; 128 x 32 patches for the one-byte results of a compare (whole
+      // 128-byte rows per store) ran that call four times slower.
       constexpr int TX = MT::smax <= 4 ? 64 : 32;
       constexpr int TY = MT::smax == 4 ? 32 : (MT::smax < 4 ? 64 : 32);
       TiledArgs<F> a;
