@@ -8,8 +8,8 @@
 // nxh_set_deferred(ctx, 1) the primitive entry points (unary, binary, compare,
 // where, cast, reduce, matmul, one-element fill) only RECORD their call. The
 // record is executed, in issue order, as soon as anything else is asked of the
-// context (any other entry point, a host read, a synchronisation) or when it
-// reaches 512 entries. At that moment a run of entries that spells one of the
+// context (any other entry point, a host read, a synchronisation), at a recorded copy
+// once it holds 48 entries, or when it reaches 2048 entries. At that moment a run of entries that spells one of the
 // five sequences is replaced by the fused call (nxh_softmax_rows,
 // nxh_layer_norm_rows, nxh_gelu_tanh, nxh_attention, nxh_linear), provided that
 // every recorded reader of its intermediate results is inside the run. An
@@ -60,6 +60,7 @@ struct DEntry {
   std::vector<unsigned char> payload;  // D_UPLOAD: the host bytes
   bool alive = true;             // the output block has not been freed
   bool done = false;             // issued, or inside a fused run that was issued
+  bool skipped = false;          // done without having been written (a causal mask that every reader took as a flag)
   DEntry *fused_into = nullptr;
   std::vector<DEntry *> readers;
   int64_t causal = 0;  // n: the result is the n x n mask [i][j] = (j <= i)
@@ -129,7 +130,7 @@ bool c_contiguous(const nxh_tensor &t) {
 }
 // The whole result of `e`, as it was written: offset 0, its shape, C-contiguous.
 bool identity_of(const nxh_tensor &v, const DEntry *e) {
-  return v.offset == 0 && same_shape(v, e->out) && c_contiguous(v);
+  return v.offset == 0 && v.dtype == e->out.dtype && same_shape(v, e->out) && c_contiguous(v);
 }
 // A keepdims result [..., 1] expanded along the last axis to `shape`.
 bool row_broadcast(const nxh_tensor &v, const nxh_tensor &shape) {
@@ -180,6 +181,7 @@ bool same_operand(const Opnd &a, const Opnd &b) { return a.prod == b.prod && sam
 DEntry *producer_of(const Opnd &o, int kind, int op = -1, bool identity = true) {
   DEntry *e = o.prod;
   if (!e || e->kind != kind || (op >= 0 && e->op != op) || e->fused_into || e->done) return nullptr;
+  if (o.t->dtype != e->out.dtype) return nullptr;  // a view that reinterprets the bytes is not that result
   if (identity && !identity_of(*o.t, e)) return nullptr;
   return e;
 }
@@ -957,7 +959,7 @@ int flush_locked(nxh_context *ctx, Window *w) {
         flagged = flagged && it != plans.end() && it->second.stat == NXH_DEFER_ATTENTION && it->second.causal_flag;
       }
       if (flagged) {
-        e->done = true;
+        e->done = e->skipped = true;
         continue;
       }
     }
@@ -1017,6 +1019,26 @@ int flush_locked(nxh_context *ctx, Window *w) {
       for (DEntry *m : run) kept[m] = pr.get();
       w->postponed.push_back(std::move(pr));
     }
+  // A scalar fill, an upload or a flagged causal mask that several runs read rides along with
+  // none of them and, with its handle gone, was not written above. A member that stays behind
+  // would read that block when it is issued as recorded later: it is written now, while the
+  // entry that says how still exists (the block is pinned by the member, so it is still there).
+  if (!kept.empty()) {
+    tls_in_flush = true;
+    for (auto &up : entries) {
+      DEntry *e = up.get();
+      if (!kept.count(e)) continue;
+      for (int i = 0; i < 3 && !rc; i++)
+        for (DEntry *src : {e->prod[i], e->upl[i]}) {
+          if (!src || kept.count(src) || (src->done && !src->skipped) || rc) continue;
+          if (src->kind != D_FULL && src->kind != D_UPLOAD && !(src->kind == D_COMPARE && src->causal)) continue;
+          src->done = src->skipped = false;
+          rc = issue(ctx, src);
+          w->stats[NXH_DEFER_ISSUED]++;
+        }
+    }
+    tls_in_flush = false;
+  }
   for (auto &up : entries) {
     DEntry *e = up.get();
     auto k = kept.find(e);
@@ -1229,13 +1251,24 @@ int nxh_defer_uploaded(nxh_context *ctx, void *dst, const void *src, size_t byte
   if (!w) return NXH_OK;
   std::lock_guard<std::mutex> g(w->mu);
   int rc = NXH_OK;
-  const bool pinned = w->pinned.count(dst) != 0;
+  // the ABI takes any device address: what the window knows is kept per block, so an upload
+  // into the middle of one counts as a write of that block
+  void *block = dst;
+  {
+    std::lock_guard<std::mutex> a(ctx->mu);
+    auto it = ctx->live.upper_bound(dst);
+    if (it != ctx->live.begin()) {
+      --it;
+      if ((const char *)dst < (const char *)it->first + std::max<size_t>(it->second, 1)) block = it->first;
+    }
+  }
+  const bool pinned = w->pinned.count(block) != 0;
   if (pinned) {
     rc = flush_locked(ctx, w);
-    if (!rc) rc = settle_write(ctx, w, dst);
+    if (!rc) rc = settle_write(ctx, w, block);
   }
-  w->known.erase(dst);
-  if (rc || !w->on || bytes == 0 || bytes > UPLOAD_LIMIT) return rc;
+  w->known.erase(block);
+  if (rc || !w->on || bytes == 0 || bytes > UPLOAD_LIMIT || block != dst) return rc;
   if (bytes % 4 == 0) {
     Known &k = w->known[dst];
     k.dtype = NXH_I32;

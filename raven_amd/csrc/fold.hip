@@ -468,7 +468,12 @@ static int reduce_entry(nxh_context *ctx, int op, const nxh_tensor *out, const n
 
 NXH_EXPORT int nxh_reduce(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x,
                           const int32_t *axes, int n_axes) {
-  NXH_DEFER_RECORD(ctx, NXH_D_REDUCE, op, out, 1, axes, n_axes, nullptr, x);
+  // what the eager call rejects at once is not recorded (the record would otherwise read a null axis list)
+  const bool recordable = ctx && out && x && (unsigned)op < NXH_REDUCE_COUNT && n_axes >= 0 && n_axes <= NXH_MAX_NDIM &&
+                          (n_axes == 0 || axes) && (unsigned)out->ndim <= NXH_MAX_NDIM && (unsigned)x->ndim <= NXH_MAX_NDIM &&
+                          (unsigned)out->dtype < NXH_DTYPE_COUNT && (unsigned)x->dtype < NXH_DTYPE_COUNT;
+  if (recordable) NXH_DEFER_RECORD(ctx, NXH_D_REDUCE, op, out, 1, axes, n_axes, nullptr, x);
+  else NXH_DEFER_QUIET(ctx);
   return reduce_entry(ctx, op, out, x, axes, n_axes, false);
 }
 

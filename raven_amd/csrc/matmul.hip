@@ -1495,7 +1495,12 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
         // fewer 64-column strips than units: the 128-column blocks cut along K (try_tile) stream
         // B faster than the strips with K split across blocks ([16,4096] x [4096,8192]: 24.5 us there)
         const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
-        if (a.M >= 8 && a.N < (int64_t)64 * cus && (double)a.K * (double)a.N * 2.0 >= (double)(16 << 20)) {
+        // (only when the cut will be taken: try_tile's own rule, 128-column blocks and runs of
+        // at least eight 64-wide slabs of K; a whole-K tile kernel on 8-16 rows would lose to the strips)
+        const int64_t col_blocks = (a.N + 127) / 128, slabs = a.K / 64;
+        int64_t split = a.K % 64 ? 0 : std::min<int64_t>(cus / std::max<int64_t>(col_blocks, 1), slabs / 8);
+        while (split > 1 && slabs % split) split--;
+        if (a.M >= 8 && split >= 2 && a.N < (int64_t)64 * cus && (double)a.K * (double)a.N * 2.0 >= (double)(16 << 20)) {
           using EL = std::conditional_t<MM::DT == NXH_BF16, gemm_tile::ElBF16, gemm_tile::ElF16>;
           const int rc = try_tile<EL>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
           if (rc != -1) return rc;

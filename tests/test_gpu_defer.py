@@ -446,3 +446,46 @@ def test_attention_writes_the_merged_heads_directly(hip, oracle):
     assert (st["attention"], st["issued"], st["fallbacks"]) == (1, 0, 0), st   # the copy was not issued
     assert hip.last_path() == "attention_fused"
     same_bits(got, direct, "attention into the merged layout against attention followed by the copy")
+
+
+def test_a_freed_scalar_shared_by_two_runs_is_written_for_a_member_that_stays_behind(hip, oracle):
+    """One scalar tensor read by two GELU runs rides along with neither; its handle is dropped
+    before the record executes, so it is not filled there. An interior result of one run is
+    still held: when it is read afterwards, its entry is issued as recorded and multiplies by
+    that scalar, which must have been written by then."""
+    rng = np.random.default_rng(77)
+    nx = Nx(hip)
+    d = dt.float32
+    xs = [tensor(hip, rng.standard_normal((48, 96)).astype(np.float32), d) for _ in range(2)]
+
+    def gelu_with(x, c3, keep):
+        # fn.ml:31-38 with the 0.044715 scalar handed in, so that two runs can share one tensor
+        x3 = nx.mul(x, nx.mul(x, x))
+        t = nx.mul(x3, c3)
+        keep.append(t)
+        inner = nx.mul_s(nx.add(x, t), math.sqrt(2.0 / math.pi))
+        return nx.mul_s(nx.mul(x, nx.add_s(nx.tanh(inner), 1.0)), 0.5)
+
+    kept_e = []
+    c3 = nx.scalar(d, 0.044715)
+    eager = [logical(gelu_with(x, c3, kept_e)) for x in xs]
+    eager_t = logical(kept_e[0])
+    del c3, kept_e
+    # the small blocks the allocator hands out next hold another value: a scalar that is
+    # recorded but never filled does not equal 0.044715 by accident
+    poison = [hip.full(d, (), 123.0) for _ in range(16)]
+    hip.synchronize()
+    del poison
+    with deferred(hip) as win:
+        kept = []
+        c3 = nx.scalar(d, 0.044715)
+        outs = [gelu_with(x, c3, kept) for x in xs]
+        held = kept[0]  # an interior of the first run stays referenced
+        del kept, c3     # the shared scalar's handle goes before anything executes
+        got = [logical(o) for o in outs]
+        s = win.delta()
+        assert s["gelu_tanh"] == 2 and s["postponed"] >= 1, s
+        got_t = logical(held)  # issued as recorded now: x3 * c3
+    for g, e in zip(got, eager):
+        same_bits(g, e, "gelu with a shared scalar")
+    same_bits(got_t, eager_t, "the held interior result, computed from the shared scalar")

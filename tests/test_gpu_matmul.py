@@ -476,6 +476,12 @@ def test_matmul_streamed_weights_cut_along_k(hip, oracle, d):
     b = encode(rng.standard_normal((1024, 4096)), d, oracle)
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "small weights")
     assert hip.last_path().startswith("gemm_skinny"), hip.last_path()
+    # a short K leaves nothing to cut (576 = nine slabs): 16 rows stay on the strips instead of
+    # filling one eighth of a whole-K 128-row tile
+    a = encode(rng.standard_normal((16, 576)), d, oracle)
+    b = encode(rng.standard_normal((576, 16000)) * 0.1, d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, "short K")
+    assert hip.last_path().startswith("gemm_skinny_mfma"), hip.last_path()
 
 
 @pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
