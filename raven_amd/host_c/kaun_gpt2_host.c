@@ -17,10 +17,11 @@
      kaun_gpt2_host LIB [--vocab V --positions P --embd D --layers L --heads H --inner I]
                         [--batch B --seq S] [--dtype bf16|f32] [--iters N]
                         [--time eager,deferred,late,replay]
-                        [--params FILE --ids FILE --logits FILE --mode eager|deferred|late]
+                        [--params FILE --ids FILE --logits FILE [--logits-bytes N] --mode eager|deferred|late]
    Without --params the weights are seeded noise of standard deviation 0.02 generated here;
    with it, FILE holds every leaf's storage bytes in the order of `leaves` below, --ids the
-   int32 token ids, and the logits of one forward in --mode are written to --logits (this is
+   int32 token ids, and the logits of one forward in --mode (their first --logits-bytes bytes,
+   when given) are written to --logits (this is
    how the test compares this host with the Python mirror, bit for bit).
    Prints one JSON line. */
 
@@ -345,6 +346,7 @@ int main(int argc, char **argv) {
     return 2;
   }
   const char *params_path = NULL, *ids_path = NULL, *logits_path = NULL, *mode = "deferred", *which = "eager,deferred,late,replay";
+  size_t logits_bytes = 0; /* 0: all of them; else only this many leading bytes go to the file */
   int iters = 5;
   for (int i = 2; i + 1 < argc; i += 2) {
     const char *k = argv[i], *v = argv[i + 1];
@@ -361,6 +363,7 @@ int main(int argc, char **argv) {
     else if (!strcmp(k, "--params")) params_path = v;
     else if (!strcmp(k, "--ids")) ids_path = v;
     else if (!strcmp(k, "--logits")) logits_path = v;
+    else if (!strcmp(k, "--logits-bytes")) logits_bytes = (size_t)atoll(v);
     else if (!strcmp(k, "--mode")) mode = v;
     else if (!strcmp(k, "--time")) which = v;
     else {
@@ -411,7 +414,8 @@ int main(int argc, char **argv) {
     uint64_t s2[NXH_DEFER_STAT_COUNT];
     must(L.deferred_stats(ctx, s2, NXH_DEFER_STAT_COUNT), "deferred_stats");
     FILE *f = fopen(logits_path, "wb");
-    if (!f || fwrite(host, 1, bytes, f) != bytes) {
+    const size_t written = logits_bytes && logits_bytes < bytes ? logits_bytes : bytes;
+    if (!f || fwrite(host, 1, written, f) != written) {
       fprintf(stderr, "logits: cannot write %s\n", logits_path);
       return 2;
     }

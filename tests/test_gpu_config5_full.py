@@ -10,14 +10,21 @@ the full GPU forward, within the reference contract's bfloat16 tolerance
 (rel = abs = 6e-2, backend_contract.ml:179-188), with the top-1 agreement
 reported. The three GPU routes (eager, one call per primitive; through the
 deferred-evaluation window; the windowed forward recorded and replayed as a
-graph) are compared with each other over all 8192 positions."""
+graph) are compared with each other over all 8192 positions, and so is the route
+a binding gets: the library's own deferred mode (nxh_set_deferred), eagerly
+issued and recorded into a graph, bit for bit against the Python window over the
+same fused entry points. The compiled host (raven_amd/host_c) runs the same
+forward from C at the same shape; its logits for batch row 0's first K
+positions are held to the same oracle head."""
 
 import math
+import subprocess
 
 import numpy as np
 import pytest
 
 from helpers import TOL, close, encode, logical
+from raven_amd import _ffi, build
 from raven_amd import dtype as dt
 from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
 from raven_amd.nx_frontend import Nx
@@ -138,6 +145,37 @@ def test_gpt2_small_forward_at_the_stated_shape(hip, oracle):
 
     assert np.array_equal(replays[0], windowed), "replay 1 differs from the windowed forward"
     assert np.array_equal(replays[1], windowed), "replay 2 differs from the windowed forward"
+
+    # what a binding gets: the library's own deferred mode, issued eagerly and recorded into a graph
+    model, params, t_ids = forward(hip, warm=False)
+    hip.set_deferred(True)
+    try:
+        before = hip.deferred_stats()
+        deferred = logical(model.logits(params, t_ids))
+        after = hip.deferred_stats()
+        s = {k: after[k] - before[k] for k in after}
+        assert (s["attention"], s["layer_norm_rows"], s["linear_gelu"], s["linear"], s["fallbacks"]) == (L, 2 * L + 1, L, 5 * L, 0), s
+        hip.synchronize()
+        hip.capture_begin()
+        try:
+            out = model.logits(params, t_ids)
+        finally:
+            graph = hip.capture_end()
+        hip.set_deferred(False)
+        hip.assign(out, hip.expand(hip.full(dt.bfloat16, (), 0.0), out.shape))
+        graph.launch()
+        hip.synchronize()
+        deferred_replay = logical(out)
+        del out
+        graph.destroy()
+    finally:
+        hip.set_deferred(False)
+    del model, params, t_ids
+    hip.trim()
+    assert np.array_equal(deferred_replay, deferred), "the library's deferred forward: replay differs from the issued one"
+    agree = compare_logits(deferred, windowed, "library deferred mode vs the Python window, all 8192 positions")
+    assert agree >= 0.999
+    assert np.array_equal(deferred, windowed), "the library's deferred mode and the Python window run the same fused calls"
     agree = compare_logits(windowed, eager, "window vs eager, all 8192 positions")
     assert agree >= 0.95
 
@@ -147,6 +185,48 @@ def test_gpt2_small_forward_at_the_stated_shape(hip, oracle):
     o_ids = onx.create(dt.int32, (1, K), ids[:1, :K])
     want = logical(Gpt2(onx, cfg).logits(oparams, o_ids))
     assert want.shape == (1, K, cfg.vocab_size)
-    for name, got in (("eager", eager), ("window", windowed), ("replay", replays[1])):
+    for name, got in (("eager", eager), ("window", windowed), ("replay", replays[1]), ("library deferred mode", deferred)):
         agree = compare_logits(got[:1, :K], want, f"{name} vs oracle, batch row 0, first {K} positions")
         assert agree >= 0.90, (name, agree)
+
+
+def test_the_compiled_host_at_the_stated_shape(hip, oracle, tmp_path):
+    """kaun_gpt2_host issues the 12-layer forward at batch 8 x seq 1024 from C with the library's
+    deferred mode on; logits[0, :K, :] go to a file and are held to the oracle's head, and are
+    bit for bit what the Python mirror gets from the same library calls."""
+    from test_gpu_c_host import leaves_in_file_order
+
+    assert build.GPT2_HOST_BIN.exists(), "run __graft_entry__.build() first"
+    cfg = Config.small()
+    hp = host_params(cfg, seed=16)
+    ids = np.random.default_rng(17).integers(0, cfg.vocab_size, (BATCH, SEQ)).astype(np.int32)
+    enc = lambda a, d: encode(a, d, oracle)  # noqa: E731
+    with open(tmp_path / "params.bin", "wb") as f:
+        for a in leaves_in_file_order(hp):
+            f.write(np.ascontiguousarray(enc(a, dt.bfloat16)).tobytes())
+    ids.tofile(tmp_path / "ids.bin")
+    out = tmp_path / "head.bin"
+    cmd = [str(build.GPT2_HOST_BIN), str(_ffi.LIB_PATH), "--batch", str(BATCH), "--seq", str(SEQ), "--dtype", "bf16",
+           "--params", str(tmp_path / "params.bin"), "--ids", str(tmp_path / "ids.bin"), "--logits", str(out),
+           "--logits-bytes", str(K * cfg.vocab_size * 2), "--mode", "deferred"]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.fromfile(out, dtype=np.uint16).reshape(1, K, cfg.vocab_size)
+    # the Python mirror through the same library mode
+    nx = Nx(hip)
+    params = upload(nx, hp, dt.bfloat16, enc)
+    t_ids = nx.create(dt.int32, ids.shape, ids)
+    hip.set_deferred(True)
+    try:
+        mirror = logical(hip.contiguous(hip.shrink(Gpt2(nx, cfg).logits(params, t_ids), [(0, 1), (0, K), (0, cfg.vocab_size)])))
+    finally:
+        hip.set_deferred(False)
+    del params, t_ids
+    hip.trim()
+    assert np.array_equal(got, mirror), "compiled host against the Python mirror, deferred mode"
+    onx = Nx(oracle)
+    oparams = upload(onx, hp, dt.bfloat16, enc)
+    o_ids = onx.create(dt.int32, (1, K), ids[:1, :K])
+    want = logical(Gpt2(onx, cfg).logits(oparams, o_ids))
+    agree = compare_logits(got, want, f"compiled host (deferred mode) vs oracle, batch row 0, first {K} positions")
+    assert agree >= 0.90
