@@ -9,7 +9,7 @@
 
 #include "nxh_common.hpp"
 
-constexpr int FOLD_MAXD = 12;
+constexpr int FOLD_MAXD = NXH_MAX_NDIM;  // any view the ABI can describe: kept and reduced dims together never exceed it
 constexpr int FOLD_THREADS = 256;
 
 static inline bool aligned_to16(const void *p) { return ((uintptr_t)p & 15) == 0; }

@@ -1,4 +1,5 @@
-"""A deferred-evaluation window in front of a backend.
+"""A deferred-evaluation window in front of a backend: the host-side twin of the library's
+own deferred mode (nxh_set_deferred), kept as its cross-check. No binding uses it.
 
 The frontend lowers softmax, layer norm and GELU to a dozen primitives each
 (packages/nx/lib/core/frontend.ml:4242-4252, packages/kaun/lib/layer_norm.ml:43-68,
@@ -33,8 +34,8 @@ from typing import List, Optional, Sequence
 
 import numpy as np
 
-from . import dtype as dt
-from .view import View, c_contiguous_strides, numel
+from raven_amd import dtype as dt
+from raven_amd.view import View, c_contiguous_strides, numel
 
 FUSED_FLOATS = ("float16", "bfloat16", "float32", "float64")
 ISLAND = ("float16", "bfloat16")  # dtypes whose layer-norm statistics run in float32

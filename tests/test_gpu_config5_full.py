@@ -28,7 +28,7 @@ from raven_amd import _ffi, build
 from raven_amd import dtype as dt
 from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
 from raven_amd.nx_frontend import Nx
-from raven_amd.nx_window import Window
+from nx_window import Window
 
 pytestmark = pytest.mark.gpu
 

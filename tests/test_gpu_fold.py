@@ -171,3 +171,38 @@ def test_sum_invariants_and_identities(hip, oracle):
     assert int(logical(hip.argmax(t, 0))) == 0 and int(logical(hip.argmin(t, 0))) == 0
     t, _ = pair(np.array([5, 0x80000000, 3], np.uint32), dt.uint32, hip, oracle)
     assert int(logical(hip.argmax(t, 0))) == 1  # backend_contract.ml:2810-2816
+
+
+def test_views_of_high_rank_with_nothing_to_merge(hip, oracle):
+    """Sixteen dims of size 2, every other one flipped, so that no two neighbours compose
+    (the reference reduces any view up to rank 32: nx_c.h:45, nx_c_engine.c:1052-1170). Reduced
+    over every other axis (eight kept, eight reduced), over the odd ones only (twelve kept),
+    and over all but one; argmax along one axis; a scan along one."""
+    nd = 16
+    rng = np.random.default_rng(1600)
+    x = rng.integers(-1000, 1000, (2,) * nd).astype(np.int32)
+    flips = tuple(i % 2 == 0 for i in range(nd))
+    h, o = pair(x, dt.int32, hip, oracle, lambda B, t: B.flip(t, flips))
+    want_np = x[tuple(slice(None, None, -1) if f else slice(None) for f in flips)]
+    for axes in ([a for a in range(nd) if a % 2 == 0], [1, 5, 9, 13], list(range(1, nd)), list(range(nd - 1))):
+        got = logical(hip.reduce("sum", axes, h))
+        same_bits(got, logical(oracle.reduce("sum", axes, o)), f"sum over {axes}")
+        same_bits(got, want_np.sum(axis=tuple(axes), dtype=np.int32), f"sum over {axes} against numpy")
+        same_bits(logical(hip.reduce("max", axes, h)), logical(oracle.reduce("max", axes, o)), f"max over {axes}")
+    for axis in (0, 7, nd - 1):
+        same_bits(logical(hip.argmax(h, axis)), logical(oracle.argmax(o, axis)), f"argmax along {axis}")
+    for axis in (0, 5, nd - 1):
+        same_bits(logical(hip.associative_scan(axis, "sum", h)), logical(oracle.associative_scan(axis, "sum", o)),
+                  f"cumsum along {axis}")
+    xf = rng.standard_normal((2,) * nd).astype(np.float32)
+    hf, of = pair(xf, dt.float32, hip, oracle, lambda B, t: B.flip(t, flips))
+    got = logical(hip.reduce("sum", [a for a in range(nd) if a % 2], hf))
+    want = logical(oracle.reduce("sum", [a for a in range(nd) if a % 2], of))
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-4)
+    # rank 32 itself: thirty-two dims of size 2 would be 16 GiB of int32; sizes 2 and 1 interleaved
+    shape = tuple(2 if i % 2 == 0 else 1 for i in range(32))
+    y = rng.integers(-50, 50, shape).astype(np.int32)
+    flips32 = tuple(i % 4 == 0 for i in range(32))
+    h32, o32 = pair(y, dt.int32, hip, oracle, lambda B, t: B.flip(t, flips32))
+    axes = [a for a in range(32) if a % 4 == 2]
+    same_bits(logical(hip.reduce("sum", axes, h32)), logical(oracle.reduce("sum", axes, o32)), "rank 32")

@@ -186,7 +186,7 @@ def test_captured_gpt2_forward_replays_the_windowed_forward(hip, oracle, d):
     the captured input tensor and each replay equals the eager windowed result."""
     from raven_amd.kaun_gpt2 import Config, Gpt2, host_params, upload
     from raven_amd.nx_frontend import Nx
-    from raven_amd.nx_window import Window
+    from nx_window import Window
 
     cfg = Config(vocab_size=1031, n_positions=128, n_embd=256, n_layer=2, n_head=4, n_inner=1024)
     hp = host_params(cfg, seed=16, stddev=0.05)

@@ -17,7 +17,7 @@ from oracle.nx_oracle import logical as ological
 from raven_amd import dtype as dt
 from raven_amd.kaun_gpt2 import Config, Gpt2, LayerNorm, host_params, upload
 from raven_amd.nx_frontend import Nx
-from raven_amd.nx_window import Window
+from nx_window import Window
 
 TINY = Config(vocab_size=97, n_positions=16, n_embd=128, n_layer=2, n_head=4, n_inner=256)  # head dim 32
 
