@@ -212,6 +212,7 @@ class Workloads:
             ops.append(self.mk(f"cfg4 {nm} skinny [8,4096]x[4096,16384]", self.lib.nxh_matmul,
                                [out, sa, sb], flops=2 * 8 * 4096 * 16384,
                                nbytes=(8 * 4096 + 4096 * 16384 + 8 * 16384) * es))
+        self.config4_ops = ops
         return ops
 
 
@@ -358,6 +359,158 @@ def next_ops(hip, W, linalg=False):
     la("cholesky [1,512,512] f32", lambda: hip.cholesky(big_spd))
     la("eigh [1,512,512] f32 (Jacobi)", lambda: hip.eigh(big_spd), iters=1)
     return out
+
+
+class Telemetry:
+    """Board power (hwmon power1_input, microwatts) and shader clock (the current line of
+    pp_dpm_sclk) sampled from sysfs every 10 ms while a loop runs. Means over the samples taken
+    after the first fifth of the loop (the clock needs a moment to settle)."""
+
+    def __init__(self):
+        import glob
+
+        self.power = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") + [None])[0]
+        self.sclk = (glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk") + [None])[0]
+        self.samples, self._stop, self._thread = [], False, None
+
+    def _read(self):
+        w = mhz = None
+        try:
+            if self.power:
+                w = int(open(self.power).read()) / 1e6
+            if self.sclk:
+                for line in open(self.sclk).read().splitlines():
+                    if line.rstrip().endswith("*"):
+                        mhz = float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        except (OSError, ValueError, IndexError):
+            pass
+        return time.perf_counter(), w, mhz
+
+    def __enter__(self):
+        import threading
+
+        def loop():
+            while not self._stop:
+                self.samples.append(self._read())
+                time.sleep(0.01)
+
+        self._thread = threading.Thread(target=loop, daemon=True)
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        self._thread.join()
+        return False
+
+    def means(self):
+        s = self.samples[len(self.samples) // 5:]
+        ws, fs = [w for _, w, _ in s if w is not None], [f for _, _, f in s if f is not None]
+        return (round(sum(ws) / len(ws), 1) if ws else None, round(sum(fs) / len(fs)) if fs else None, len(s))
+
+
+def study_row(what, data, ms, fl, tel):
+    w, mhz, k = tel.means()
+    return {"kernel": what, "operands": data, "ms": round(ms, 4), "TFLOP/s": round(fl / (ms * 1e-3) / 1e12, 1),
+            "frac_of_2500": round(fl / (ms * 1e-3) / 1e12 / 2500.0, 4), "board_W": w, "sclk_MHz": mhz, "samples": k}
+
+
+def gemm_study_vendor(seconds):
+    """The rows of gemm_study that the vendor library fills (hipBLASLt behind torch.bmm)."""
+    import torch
+
+    nb, n = 16, 4096
+    flops = 2.0 * nb * n ** 3
+    rows = []
+    for data in ("N(0, 0.02)", "zeros"):
+        if data == "zeros":
+            a = torch.zeros(nb, n, n, device="cuda", dtype=torch.bfloat16)
+            b = torch.zeros(nb, n, n, device="cuda", dtype=torch.bfloat16)
+        else:
+            g = torch.Generator(device="cuda").manual_seed(12)
+            a = (torch.randn(nb, n, n, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+            b = (torch.randn(nb, n, n, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+        c = torch.empty(nb, n, n, device="cuda", dtype=torch.bfloat16)
+        for _ in range(5):
+            torch.bmm(a, b, out=c)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        iters = max(5, int(seconds / 1.8e-3))
+        with Telemetry() as tel:
+            e0.record()
+            for _ in range(iters):
+                torch.bmm(a, b, out=c)
+            e1.record()
+            torch.cuda.synchronize()
+        rows.append(study_row("vendor: torch.bmm (hipBLASLt)", data, e0.elapsed_time(e1) / iters, flops, tel))
+        del a, b, c
+    return rows
+
+
+def gemm_study(hip, seconds, vendor=True):
+    """Config 4's batched bf16 product on all-zero and on N(0, 0.02) operands, by this library and
+    by the vendor library (hipBLASLt behind torch.bmm), beside an MFMA-only loop on the same two
+    kinds of data: time, TFLOP/s, board power and shader clock of each. The board holds its power
+    limit by lowering the clock, so what a GEMM reaches depends on the bits that toggle."""
+    nb, n = 16, 4096
+    flops = 2.0 * nb * n ** 3
+    rows = []
+
+    def record(what, data, ms, fl, tel):
+        rows.append(study_row(what, data, ms, fl, tel))
+
+    W = Workloads(hip)
+    W.config4()
+    keep, cb = W.cfg4["bf16"]
+    desc = [d for ts, ds in W.keep for t, d in zip(ts, ds) if t is cb or (tuple(t.shape) == (nb, n, n) and t.dtype is dt.bfloat16)]
+    normal = [op for op in W.config4_ops if "16,4096" in op.name][0]
+    zero = [hip.full(dt.bfloat16, (nb, n, n), 0.0) for _ in range(2)]
+    zc = hip.buffer(dt.bfloat16, (nb, n, n))
+    zeros = W.mk("cfg4 bf16 matmul, zeros", W.lib.nxh_matmul, [zc, zero[0], zero[1]], flops=flops)
+    for data, op in (("N(0, 0.02)", normal), ("zeros", zeros)):
+        ms1 = time_ops(hip, [op], 5, 3)
+        iters = max(5, int(seconds / (ms1 * 1e-3)))
+        with Telemetry() as tel:
+            ms = time_ops(hip, [op], iters, 0)
+        record(f"libnxhip nxh_matmul ({hip.last_path()})", data, ms, flops, tel)
+    del zero, zc, zeros, normal, desc
+    W.keep.clear()
+    W.cfg4 = None
+    hip.trim()
+
+    # the vendor library runs in a process of its own: torch carries its own HIP runtime, and two of
+    # them in one process do not both find the device
+    import subprocess
+
+    if vendor:
+        r = subprocess.run([sys.executable, str(Path(__file__).resolve()), "--gemm-study-vendor", "--study-seconds", str(seconds)],
+                           capture_output=True, text=True, timeout=600)
+        if r.returncode == 0:
+            rows.extend(json.loads(r.stdout.strip().splitlines()[-1]))
+        else:
+            rows.append({"kernel": "vendor: torch.bmm (hipBLASLt)", "error": r.stderr.strip()[-200:]})
+
+    probe = ROOT / "bench_mfma_probe.so"
+    if probe.exists():
+        lib = C.CDLL(str(probe))
+        lib.mfma_probe_run.restype = C.c_double
+        lib.mfma_probe_run.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
+        blocks = 4 * hip.device_info()["compute_units"]
+        out = hip.buffer(dt.float32, (blocks * 512,))
+        rng = np.random.default_rng(13)
+        for data in ("N(0, 0.02)", "zeros"):
+            host = np.zeros(16384, np.uint16) if data == "zeros" else bf16_bits((rng.standard_normal(16384) * 0.02).astype(np.float32))
+            words = hip.from_host(host.view(np.int32), dt.int32)
+            hip.synchronize()
+            ms = C.c_float()
+            iters = 2000
+            fl = lib.mfma_probe_run(words.buffer.ptr, out.buffer.ptr, blocks, iters, 2, C.byref(ms))
+            reps = max(2, int(seconds / max(ms.value * 1e-3, 1e-6)))
+            with Telemetry() as tel:
+                fl = lib.mfma_probe_run(words.buffer.ptr, out.buffer.ptr, blocks, iters, reps, C.byref(ms))
+            if fl:
+                rows.append(study_row("MFMA-only loop (v_mfma_f32_16x16x32_bf16, operands in registers)", data, ms.value, fl, tel))
+    return rows
 
 
 def time_ops(hip, ops, iters, warmup):
@@ -774,6 +927,14 @@ def main():
     ap.add_argument("--only-next", action="store_true",
                     help="time the operations beside the hot path only (pad ... fft), the linear-algebra family included")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 forward leg only and print its record")
+    ap.add_argument("--gemm-study", action="store_true",
+                    help="config 4's bf16 product on zeros and on N(0, 0.02) data, this library / the vendor library / an "
+                         "MFMA-only loop: time, board power and shader clock of each")
+    ap.add_argument("--gemm-study-vendor", action="store_true",
+                    help="the vendor rows of --gemm-study alone (torch.bmm, in this process)")
+    ap.add_argument("--study-skip-vendor", action="store_true",
+                    help="--gemm-study without the vendor rows (for counter runs: run --gemm-study-vendor as a command of its own)")
+    ap.add_argument("--study-seconds", type=float, default=1.5, help="length of each timed loop of --gemm-study")
     ap.add_argument("--cpu-configs", action="store_true",
                     help="time the CPU oracle on bounded samples of configurations 1, 3, 4, 5 and print the records")
     args = ap.parse_args()
@@ -783,6 +944,9 @@ def main():
 
     if args.cpu_configs:
         print(json.dumps({"cpu_configs": cpu_configs()}))
+        return
+    if args.gemm_study_vendor:
+        print(json.dumps(gemm_study_vendor(args.study_seconds)))
         return
     hip = Backend()
     info = hip.device_info()
@@ -794,6 +958,9 @@ def main():
         return
     if args.only_next:
         print(json.dumps({"ops": next_ops(hip, Workloads(hip), linalg=True)}))
+        return
+    if args.gemm_study:
+        print(json.dumps({"gemm_study": gemm_study(hip, args.study_seconds, vendor=not args.study_skip_vendor)}))
         return
     if args.only_config:
         # one configuration's operations, each timed alone (for profiling runs)

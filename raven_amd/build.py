@@ -103,5 +103,19 @@ def build_gpt2_host() -> Path:
     return GPT2_HOST_BIN
 
 
+MFMA_PROBE_SRC = CSRC.parent.parent / "bench_mfma_probe.hip"
+MFMA_PROBE_LIB = MFMA_PROBE_SRC.with_suffix(".so")
+
+
+def build_mfma_probe() -> Path:
+    """The MFMA-only loop bench.py --gemm-study times beside the GEMMs (not part of libnxhip)."""
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", str(MFMA_PROBE_SRC), "-o", str(MFMA_PROBE_LIB)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {MFMA_PROBE_SRC.name}:\n{r.stderr}")
+    return MFMA_PROBE_LIB
+
+
 if __name__ == "__main__":
     print(build_all(force="--force" in sys.argv))

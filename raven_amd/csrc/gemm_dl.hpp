@@ -7,7 +7,8 @@
 //                                        3072 whole multiples of that
 // Same contract as gemm_tile.hpp (f32 accumulation, one rounding per output element,
 // batched with broadcastable batch dims, the fused linear's epilogue and grouped launch),
-// for whole tiles only: M and N multiples of the block, K a multiple of 64. What differs
+// for whole tiles only: M and N multiples of the block, K a multiple of 64 (the host runs a
+// ragged last column block as a launch of its own). What differs
 // from gemm_tile:
 //   * No register staging. A slab (64 k-values of every row of both operands) is
 //     requested with global_load_lds_dwordx4: each of the 64 lanes of a load delivers
@@ -305,11 +306,15 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
       }
     }
   } else {
+    // C's rows need not be 16-byte aligned here (a row pitch of 50257 elements, GPT-2's tied
+    // head): the hardware takes a 16-byte store at any element boundary, and a lane's eight
+    // neighbours in one store beat eight 2-byte stores by a wide margin
+    typedef V16 V16_any __attribute__((aligned(2)));
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
       const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
       const V16 v = *reinterpret_cast<const V16 *>(patch + row * PITCH + col);
-      *reinterpret_cast<V16 *>(ctile + (int64_t)row * a.ldc + col) = v;
+      *reinterpret_cast<V16_any *>(ctile + (int64_t)row * a.ldc + col) = v;
     }
   }
 }

@@ -1104,6 +1104,28 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   if (a.K % BK || a.K < BK || a.M < VE || a.N < VE) return -1;
   if (a.ccs != 1 || a.batch.n > 4 || !al_a || !al_b) return -1;
   const bool a_kc = a.acs == 1, b_kc = a.brs == 1;
+  // A wide 16-bit product whose N is no whole number of 256-column blocks (GPT-2's tied head,
+  // [8192,768] x [768,50257]): the whole blocks take the direct-to-LDS kernel, which has no
+  // ragged form, and the last columns a launch of their own. Every output element is still
+  // one k-ordered f32 sum rounded once, so the split changes no bit of the result.
+  if constexpr (!EL::F32 && !EPI) {
+    const int64_t n0 = a.N / 256 * 256;
+    if (a.N % 256 && n0 >= 8 * 256 && a.M % 256 == 0 && a.M >= 1024 && !forced_tile() && a.n_ld == a.N) {
+      GemmArgs left = a, right = a;
+      left.N = left.n_ld = n0;
+      right.N = right.n_ld = a.N - n0;
+      right.B = (const char *)a.B + n0 * a.bcs * (int64_t)sizeof(typename EL::S);
+      right.C = (char *)a.C + n0 * (int64_t)sizeof(typename EL::S);
+      int rc = try_tile<EL, false>(ctx, left, nbatch, al_a, al_b, nullptr);
+      if (rc == NXH_OK) {
+        const char *path = nxh_last_path(ctx);
+        // (the right part's B starts n0 columns in: 16-byte aligned, since n0 is a multiple of 256)
+        rc = try_tile<EL, false>(ctx, right, nbatch, al_a, al_b, nullptr);
+        nxh_set_path(path);
+      }
+      if (rc != -1) return rc;  // (-1: the whole product takes the ordinary path below; what the left part wrote is rewritten)
+    }
+  }
   gemm_tile::Args g{};
   g.A = a.A;
   g.B = a.B;
@@ -1202,10 +1224,11 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   // epilogue touches must be 16-byte aligned).
   if constexpr (!EL::F32) {
     const int forced = forced_tile();
-    bool dl_ok = (pick == 256 || pick == 128 || pick == 192) && forced != 257 && forced != 128 && al16(g.C) &&
-                 g.ldc % 8 == 0 && g.lda < ((int64_t)1 << 22) && g.ldb < ((int64_t)1 << 22);
+    // (without an epilogue C's rows may start at any element: the stores are unaligned-capable)
+    bool dl_ok = (pick == 256 || pick == 128 || pick == 192) && forced != 257 && forced != 128 &&
+                 (!EPI || (al16(g.C) && g.ldc % 8 == 0)) && g.lda < ((int64_t)1 << 22) && g.ldb < ((int64_t)1 << 22);
     for (int i = 0; i < a.batch.n; i++)
-      if (g.bc[i] % 8 || (EPI && g.R && g.br[i] % 8)) dl_ok = false;
+      if (EPI && (g.bc[i] % 8 || (g.R && g.br[i] % 8))) dl_ok = false;
     if (EPI && ((g.bias && !al16(g.bias)) || (g.R && (!al16(g.R) || g.ldr % 8)))) dl_ok = false;
     if (dl_ok) {
       // (the f16 conversions make the large shape's epilogue spill: f16 linears keep to the others)

@@ -627,3 +627,30 @@ def test_linear_epilogue_equals_the_sequence(hip, oracle, d):
         hip.linear(hip.full(d, (64, 64), 1.0), hip.full(d, (64, 64), 1.0), hip.full(d, (32,), 1.0))
     with pytest.raises(RuntimeError):
         hip.linear(hip.full(dt.int32, (64, 64), 1), hip.full(dt.int32, (64, 64), 1), hip.full(dt.int32, (64,), 1))
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matmul_wide_product_with_a_ragged_last_column_block(hip, oracle, d):
+    """N = 16 x 256 + 81 (the shape class of GPT-2's tied head, [8192,768] x [768,50257]): the whole
+    256-column blocks go through the direct-to-LDS kernel, whose stores take C's odd row pitch as
+    it is, the last 81 columns through a launch of their own. Both layouts of B; every element is
+    one k-ordered f32 sum rounded once, so the bits equal the unsplit kernels' bits on each side."""
+    rng = np.random.default_rng(1700 + d.tag)
+    T = lambda B, t: B.permute(t, (1, 0))  # noqa: E731
+    m, k, n = 4096, 192, 16 * 256 + 81
+    a = encode(rng.standard_normal((m, k)), d, oracle)
+    b = encode(rng.standard_normal((k, n)), d, oracle)
+    want = ref_f64(a, b, d, oracle)
+    ha = pair(a, d, hip, oracle)[0]
+    for tb in (False, True):
+        if not tb and n % 8:
+            continue  # rows of an N-contiguous B must be whole 16-byte vectors for the tiled kernels
+        hb = pair(np.ascontiguousarray(b.T) if tb else b, d, hip, oracle, T if tb else None)[0]
+        got_bits = logical(hip.matmul(ha, hb))
+        assert hip.last_path() == "gemm_dl_256x256", hip.last_path()
+        got = decode(got_bits, d, oracle)
+        ulp = 2.0 ** (-8 if d is dt.bfloat16 else -11)
+        assert np.all(np.abs(got - want) <= ulp * 2 * np.abs(want) + np.sqrt(k) * 2e-6), float(np.abs(got - want).max())
+        # the left part against the same columns computed alone (aligned C, no split)
+        left = hip.matmul(ha, hip.shrink(hb, [(0, k), (0, 16 * 256)]))
+        same_bits(got_bits[:, :16 * 256], logical(left), "whole blocks: the same bits as the product of those columns alone")
