@@ -113,14 +113,17 @@ struct SoftmaxArgs {
   int64_t mask_last;  // 0 or 1
   double scale, masked;  // exact images of the encoded scalars
 };
-template <int DTX, int DTO, int V, int RW>
+// EP: elements a lane holds at most (a row of up to 64 * RW * EP elements). The short forms
+// exist for their register count: 87 registers for EP = 32 leave five waves per SIMD, and
+// a launch of 2048 blocks then runs as two rounds of blocks instead of one.
+template <int DTX, int DTO, int V, int RW, int EP = EPL>
 __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
   using TX = Tr<DTX>;
   using TO = Tr<DTO>;
   using C = typename TX::C;
   using SX = typename TX::S;
   using SO = typename TO::S;
-  constexpr int NV = EPL / V, T = 64 * RW;
+  constexpr int NV = EP / V, T = 64 * RW;
   __shared__ C lds[4];
   const int tid = RW == 1 ? (threadIdx.x & 63) : threadIdx.x;
   const int64_t row = RW == 1 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
@@ -212,12 +215,12 @@ struct LayerNormArgs {
   const char *gamma, *beta;  // null: that step is left out
   double eps, count;         // exact images of the float scalars the chain would have filled
 };
-template <int DT, int V, int RW>
+template <int DT, int V, int RW, int EP = EPL>
 __global__ __launch_bounds__(256) void layer_norm_rows_kernel(LayerNormArgs a) {
   using TX = Tr<DT>;
   using C = typename TX::C;  // float for the 16-bit dtypes: their float32 island
   using S = typename TX::S;
-  constexpr int NV = EPL / V, T = 64 * RW;
+  constexpr int NV = EP / V, T = 64 * RW;
   __shared__ C lds[4];
   const int tid = RW == 1 ? (threadIdx.x & 63) : threadIdx.x;
   const int64_t row = RW == 1 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
@@ -234,6 +237,17 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(LayerNormArgs a) {
   for (int v = 0; v < NV; v++) {
     const int c = v * T + tid;
     if (c < nvec) raw[v] = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+  }
+  // gamma and beta do not depend on the row: their loads go out with the row's, ahead of the
+  // two reductions, instead of starting a second trip to memory after them
+  Pk<S, V> gv[NV], bv[NV];
+#pragma unroll
+  for (int v = 0; v < NV; v++) {
+    const int c = v * T + tid;
+    if (c < nvec) {
+      if (gamma) gv[v] = *reinterpret_cast<const Pk<S, V> *>(gamma + (int64_t)c * V);
+      if (beta) bv[v] = *reinterpret_cast<const Pk<S, V> *>(beta + (int64_t)c * V);
+    }
   }
   const C count = (C)a.count, eps = (C)a.eps;
   C s = 0;
@@ -261,14 +275,12 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(LayerNormArgs a) {
   for (int v = 0; v < NV; v++) {
     const int c = v * T + tid;
     if (c < nvec) {
-      Pk<S, V> o, gv, bv;
-      if (gamma) gv = *reinterpret_cast<const Pk<S, V> *>(gamma + (int64_t)c * V);
-      if (beta) bv = *reinterpret_cast<const Pk<S, V> *>(beta + (int64_t)c * V);
+      Pk<S, V> o;
 #pragma unroll
       for (int j = 0; j < V; j++) {
         C y = rnd<DT>(t[v][j] / r);  // leaves the float32 island here
-        if (gamma) y = rnd<DT>(y * TX::ld(gv.v[j]));
-        if (beta) y = rnd<DT>(y + TX::ld(bv.v[j]));
+        if (gamma) y = rnd<DT>(y * TX::ld(gv[v].v[j]));
+        if (beta) y = rnd<DT>(y + TX::ld(bv[v].v[j]));
         o.v[j] = TX::st(y);
       }
       *reinterpret_cast<Pk<S, V> *>(out + (int64_t)c * V) = o;
@@ -396,23 +408,40 @@ int out_rows_ok(const char *op, const nxh_tensor *out) {
   return NXH_OK;
 }
 
+// Elements per lane of the vector forms: the smallest of 8 / 16 / 32 that holds the row.
+inline int lane_share(int n, bool wave) {
+  const int need = (n + (wave ? 64 : 256) - 1) / (wave ? 64 : 256);
+  return need <= 8 ? 8 : need <= 16 ? 16 : 32;
+}
 template <int DTX, int DTO>
 void softmax_launch(nxh_context *ctx, const SoftmaxArgs &a, bool vec) {
   const bool wave = a.g.n <= 64 * EPL;
   const dim3 grid((unsigned)(wave ? (a.g.rows + 3) / 4 : a.g.rows));
-  if (wave && vec) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 1>), grid, dim3(256), 0, ctx->stream, a);
-  else if (wave) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 1, 1>), grid, dim3(256), 0, ctx->stream, a);
-  else if (vec) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 4>), grid, dim3(256), 0, ctx->stream, a);
-  else hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
+  const int ep = lane_share(a.g.n, wave);
+  if (wave && vec) {
+    if (ep == 8) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 1, 8>), grid, dim3(256), 0, ctx->stream, a);
+    else if (ep == 16) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 1, 16>), grid, dim3(256), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 1>), grid, dim3(256), 0, ctx->stream, a);
+  } else if (wave) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 1, 1>), grid, dim3(256), 0, ctx->stream, a);
+  else if (vec) {
+    if (ep == 16) hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 4, 16>), grid, dim3(256), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 4, 4>), grid, dim3(256), 0, ctx->stream, a);
+  } else hipLaunchKernelGGL((softmax_rows_kernel<DTX, DTO, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
 }
 template <int DT>
 void layer_norm_launch(nxh_context *ctx, const LayerNormArgs &a, bool vec) {
   const bool wave = a.g.n <= 64 * EPL;
   const dim3 grid((unsigned)(wave ? (a.g.rows + 3) / 4 : a.g.rows));
-  if (wave && vec) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 1>), grid, dim3(256), 0, ctx->stream, a);
-  else if (wave) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 1, 1>), grid, dim3(256), 0, ctx->stream, a);
-  else if (vec) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 4>), grid, dim3(256), 0, ctx->stream, a);
-  else hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
+  const int ep = lane_share(a.g.n, wave);
+  if (wave && vec) {
+    if (ep == 8) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 1, 8>), grid, dim3(256), 0, ctx->stream, a);
+    else if (ep == 16) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 1, 16>), grid, dim3(256), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 1>), grid, dim3(256), 0, ctx->stream, a);
+  } else if (wave) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 1, 1>), grid, dim3(256), 0, ctx->stream, a);
+  else if (vec) {
+    if (ep == 16) hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 4, 16>), grid, dim3(256), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 4, 4>), grid, dim3(256), 0, ctx->stream, a);
+  } else hipLaunchKernelGGL((layer_norm_rows_kernel<DT, 1, 4>), grid, dim3(256), 0, ctx->stream, a);
 }
 template <int DT>
 void gelu_launch(nxh_context *ctx, const GeluArgs &a, bool vec) {
