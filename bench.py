@@ -243,7 +243,7 @@ def next_ops(hip, W, linalg=False):
     timed("cat 4 x [1024,4096] f32 along axis 1", lambda: hip.cat(parts, 1), 2 * 4 * 1024 * 4096 * 4)
     y = W.dev(rng.standard_normal((4096, 8192)).astype(np.float32), dt.float32)
     timed("cumsum [4096,8192] f32 axis 1 (scan_rows)", lambda: hip.associative_scan(1, "sum", y), 2 * 4096 * 8192 * 4)
-    timed("cumsum [4096,8192] f32 axis 0 (scan_chunks: 3 passes over the data)", lambda: hip.associative_scan(0, "sum", y), 2 * 4096 * 8192 * 4)
+    timed("cumsum [4096,8192] f32 axis 0 (scan_cols: one pass, carries handed down between blocks)", lambda: hip.associative_scan(0, "sum", y), 2 * 4096 * 8192 * 4)
     n = 1 << 24
     ctr = W.dev(np.arange(2 * n, dtype=np.int64).astype(np.int32).reshape(n, 2), dt.int32)
     key = hip.expand(W.dev(np.array([[1234, -99]], np.int32), dt.int32), (n, 2))

@@ -86,6 +86,12 @@ struct nxh_context {
   // factorisations, sorts, graph replays, host copies): no block counts as "not touched
   // again" across one of them
   uint64_t opaque_calls = 0;
+  // State of the single-pass column scan (scan.hip, scan_cols): a device block holding one
+  // 64-bit (flag, value) word per column and row chunk; flags carry the launch's epoch, so the words are cleared once, when the block is
+  // made, and never between launches. Freed with the context.
+  unsigned char *scan_state = nullptr;
+  size_t scan_state_bytes = 0;
+  uint32_t scan_epoch = 0;
 };
 
 // Size of the static per-device workspace behind nxh_reduce_noalloc.
@@ -167,6 +173,14 @@ enum { NXH_D_UNARY, NXH_D_BINARY, NXH_D_COMPARE, NXH_D_WHERE, NXH_D_CAST, NXH_D_
       if (nxh_defer_active(ctx))                                                                              \
         if (int drc__ = nxh_defer_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out)) return drc__; \
       nxh_cache_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out);                                \
+    }                                                                                                         \
+  } while (0)
+// As TOUCH, for entry points that ask nxh_cache_hints themselves (once their arguments are checked).
+#define NXH_DEFER_SETTLE(ctx, n_out, ...)                                                                     \
+  do {                                                                                                        \
+    if ((ctx) && nxh_defer_active(ctx)) {                                                                     \
+      const nxh_tensor *dts__[] = {__VA_ARGS__};                                                              \
+      if (int drc__ = nxh_defer_touch(ctx, dts__, (int)(sizeof dts__ / sizeof *dts__), n_out)) return drc__; \
     }                                                                                                         \
   } while (0)
 #define NXH_DEFER_QUIET(ctx)                                     \

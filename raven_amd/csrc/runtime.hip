@@ -117,6 +117,7 @@ NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   for (auto &kv : ctx->live) (void)hipFree(kv.first);
   for (auto &kv : ctx->device_tables) (void)hipFree(kv.second);
   if (ctx->fault_flag) (void)hipFree(ctx->fault_flag);
+  if (ctx->scan_state) (void)hipFree(ctx->scan_state);
   if (ctx->fault_flag_host) (void)hipHostFree(ctx->fault_flag_host);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
   for (hipEvent_t ev : ctx->stage_done)

@@ -17,11 +17,15 @@
 //               to fill the chip the axis is cut into chunks (scan_chunks):
 //               chunk totals, an exclusive scan of the totals per line, then
 //               every chunk is scanned from its carry-in.
+//   scan_cols   the case of scan_chunks that matters most, rows of a matrix with
+//               unit-stride columns (cumsum along axis 0) in dtypes of at most four
+//               bytes: one pass, the carries handed down between blocks (below).
 // Float sums and products are reassociated by scan_rows (tolerance-level
 // differences, inside the reference contract's 6x arithmetic tolerance for
 // scans); integer results are exact.
 
 #include "fold_common.hpp"
+#include "stream_access.hpp"
 
 struct ScanArgs {
   const void *in;
@@ -198,9 +202,246 @@ __global__ __launch_bounds__(FOLD_THREADS) void scan_rows_kernel(ScanArgs a, int
   if (PHASE == 0 && lane == 0) *slot = carry;
 }
 
+// ── scan_cols: the axis is the row dim of a [rows][columns] view with unit-stride columns ──
+// One pass over the data. A block owns SC_ROWS rows of a strip of SC_COLS columns: every wave
+// holds SC_RW rows x 4 columns per lane in registers, scans them down the rows, the waves'
+// totals meet in LDS. What a block needs from the rows above it travels through `status`, one
+// 64-bit (flag, value) word per column and row chunk, written and read with relaxed
+// device-scope atomics (a word is complete by itself, so nothing has to be ordered around it):
+// a block first publishes its own total (flag AGG), then walks the chunks above it from the
+// nearest one up, adding totals until it meets one that already carries everything above it
+// (flag PRE), and publishes that form of its own word; the words of up to SC_WIN chunks are
+// requested together, so the way up costs one trip to memory per window, not per chunk. Block b
+// is chunk b / nstrips of strip b % nstrips: the blocks a block waits for have smaller ids, were
+// handed to the compute units before it, and publish their AGG word before they wait for
+// anything. (An earlier form took its id from a ticket counter instead, which made that order
+// a certainty, and paid for it with one more trip to memory in front of every block's first
+// load: 55 against 49 us.) The wait is bounded all the same: past `spin_limit` polls that found
+// nothing new a lane gives up on the words and adds the rows above it from the input itself.
+// Flags carry the launch's epoch, so words of earlier launches read as "not there yet" and the
+// block of words is never cleared between launches. Results that nothing reads back while
+// they could still be cached are stored past the memory-side cache (the host's per-call
+// decision, runtime.hip): the input then stays cached from one call to the next, which is worth
+// more here than anything else ([4096,8192] f32: 63 -> 49 us; the three-pass form gains nothing
+// from it).
+constexpr int SC_RW = 16, SC_V = 4, SC_COLS = 64 * SC_V;
+constexpr int SC_WIN = 16;  // chunks whose words a lane requests together on its way up
+struct ScanColsArgs {
+  const void *in;
+  void *out;
+  int64_t len, W, in_step, out_step;  // rows, columns, row pitches in elements
+  uint32_t nstrips, epoch, spin_limit;
+  uint32_t stream_out;  // the results go past the memory-side cache (decided per call on the host)
+  uint64_t *status;     // [chunks][nstrips * SC_COLS]
+};
+// The 32 bits of a running value that travel in a word: a float as it is; an integer as its
+// storage form (sums and products are modular and maxima stay inside the storage range, so the
+// storage bits determine every later result).
+template <class TR>
+__device__ __forceinline__ uint32_t sc_pack(typename TR::C c) {
+  using S = typename TR::S;
+  if constexpr (std::is_same<typename TR::C, float>::value) {
+    return __builtin_bit_cast(uint32_t, c);
+  } else {
+    return (uint32_t)(typename std::make_unsigned<S>::type)TR::st(c);
+  }
+}
+template <class TR>
+__device__ __forceinline__ typename TR::C sc_unpack(uint32_t u) {
+  using S = typename TR::S;
+  if constexpr (std::is_same<typename TR::C, float>::value) {
+    return __builtin_bit_cast(float, u);
+  } else {
+    return TR::ld((S)(typename std::make_unsigned<S>::type)u);
+  }
+}
+template <int DT>
+constexpr bool scan_cols_ok() {
+  using TR = Tr<DT>;
+  return sizeof(typename TR::S) <= 4 &&
+         ((TR::cat == CAT_FLOAT && std::is_same<typename TR::C, float>::value) || TR::cat == CAT_SINT || TR::cat == CAT_UINT);
+}
+
+template <int DT, class CB, bool VEC, int SC_WAVES>
+__global__ __launch_bounds__(64 * SC_WAVES) void scan_cols_kernel(ScanColsArgs a) {
+  constexpr int SC_ROWS = SC_RW * SC_WAVES;
+  static_assert(64 * SC_WAVES >= SC_COLS, "a lane per column in the hand-over");
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  // what a lane keeps per element between the two halves of the kernel: the running value
+  // itself for floats, its storage form for integers (half the registers, same information)
+  using K = typename std::conditional<std::is_same<C, float>::value, float, S>::type;
+  __shared__ C tot[SC_WAVES][SC_COLS];
+  __shared__ C pre[SC_COLS];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const uint32_t t = blockIdx.x;
+  const uint32_t strip = t % a.nstrips, chunk = t / a.nstrips;
+  const int c0 = lane * SC_V;
+  const int64_t col = (int64_t)strip * SC_COLS + c0;
+  const int64_t row0 = (int64_t)chunk * SC_ROWS + w * SC_RW;
+  const int ncol = (int)(a.W - col >= SC_V ? SC_V : (a.W - col > 0 ? a.W - col : 0));
+  const int nrow = (int)(a.len - row0 >= SC_RW ? SC_RW : (a.len - row0 > 0 ? a.len - row0 : 0));
+  const S *p = (const S *)a.in + row0 * a.in_step + col;
+  S *q = (S *)a.out + row0 * a.out_step + col;
+  FVec<S, SC_V> x[SC_RW];
+#pragma unroll
+  for (int r = 0; r < SC_RW; r++) {
+    if (r < nrow) {
+      if (VEC && ncol == SC_V) {
+        x[r] = *reinterpret_cast<const FVec<S, SC_V> *>(p + r * a.in_step);
+      } else {
+#pragma unroll
+        for (int j = 0; j < SC_V; j++)
+          if (j < ncol) x[r].v[j] = p[r * a.in_step + j];
+      }
+    }
+  }
+  K v[SC_RW][SC_V];
+  C run[SC_V];
+#pragma unroll
+  for (int j = 0; j < SC_V; j++) run[j] = CB::init();
+#pragma unroll
+  for (int r = 0; r < SC_RW; r++)
+#pragma unroll
+    for (int j = 0; j < SC_V; j++) {
+      if (r < nrow && j < ncol) run[j] = CB::apply(run[j], TR::ld(x[r].v[j]));
+      if constexpr (std::is_same<C, float>::value) v[r][j] = run[j];
+      else v[r][j] = TR::st(run[j]);
+    }
+#pragma unroll
+  for (int j = 0; j < SC_V; j++) tot[w][c0 + j] = run[j];
+  __syncthreads();
+  if (threadIdx.x < SC_COLS) {
+    // The block's first SC_COLS lanes take one column of the strip each through the hand-over.
+    const int cme = threadIdx.x;
+    C agg = tot[0][cme];
+#pragma unroll
+    for (int i = 1; i < SC_WAVES; i++) agg = CB::apply(agg, tot[i][cme]);
+    C ex = CB::init();
+    const uint64_t pitch = (uint64_t)a.nstrips * SC_COLS;
+    uint64_t *mine = a.status + (uint64_t)chunk * pitch + (uint64_t)strip * SC_COLS + cme;
+    const uint32_t f_agg = a.epoch * 2 + 1, f_pre = a.epoch * 2 + 2;
+    if (chunk > 0) {
+      __hip_atomic_store(mine, ((uint64_t)f_agg << 32) | sc_pack<TR>(agg), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // Walk up SC_WIN chunks at a time (their words are requested together: one trip to memory
+      // per window, not per chunk) and take them nearest first while they are there.
+      bool have = false, done = false, gave_up = false;
+      uint32_t polls = 0;
+      int64_t c = (int64_t)chunk - 1;
+      while (c >= 0 && !done) {
+        const int n = c + 1 < SC_WIN ? (int)(c + 1) : SC_WIN;
+        uint64_t word[SC_WIN];
+#pragma unroll
+        for (int k = 0; k < SC_WIN; k++)
+          if (k < n) word[k] = __hip_atomic_load(mine - (uint64_t)(chunk - c + k) * pitch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int took = 0;
+#pragma unroll
+        for (int k = 0; k < SC_WIN; k++) {
+          if (k >= n || done || took != k) continue;
+          const uint32_t f = (uint32_t)(word[k] >> 32);
+          if (f != f_agg && f != f_pre) continue;
+          const C val = sc_unpack<TR>((uint32_t)word[k]);
+          ex = have ? CB::apply(val, ex) : val;  // the earlier rows on the left
+          have = true;
+          done = f == f_pre;
+          took = k + 1;
+        }
+        c -= took;
+        if (took == 0) {
+          if (polls++ >= a.spin_limit) {
+            gave_up = true;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(2);
+        }
+      }
+      if (gave_up) {  // the rows above, from the input itself
+        const int64_t mycol = (int64_t)strip * SC_COLS + cme;
+        ex = CB::init();
+        if (mycol < a.W) {
+          const S *top = (const S *)a.in + mycol;
+          const int64_t above = (int64_t)chunk * SC_ROWS;
+          for (int64_t r = 0; r < above; r++) ex = CB::apply(ex, TR::ld(top[r * a.in_step]));
+        }
+      }
+    }
+    const C incl = chunk > 0 ? CB::apply(ex, agg) : agg;
+    __hip_atomic_store(mine, ((uint64_t)f_pre << 32) | sc_pack<TR>(incl), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    pre[cme] = ex;
+  }
+  __syncthreads();
+  // what lies above this wave's rows: the chunks above (pre) and the block's earlier waves
+  C base[SC_V];
+  const bool has_base = chunk > 0 || w > 0;
+#pragma unroll
+  for (int j = 0; j < SC_V; j++) {
+    C b = CB::init();
+    bool hb = false;
+    if (chunk > 0) {
+      b = pre[c0 + j];
+      hb = true;
+    }
+    for (int i = 0; i < w; i++) {
+      b = hb ? CB::apply(b, tot[i][c0 + j]) : tot[i][c0 + j];
+      hb = true;
+    }
+    base[j] = b;
+  }
+#pragma unroll
+  for (int r = 0; r < SC_RW; r++) {
+    if (r < nrow) {
+      FVec<S, SC_V> y;
+#pragma unroll
+      for (int j = 0; j < SC_V; j++) {
+        C val;
+        if constexpr (std::is_same<C, float>::value) val = v[r][j];
+        else val = TR::ld(v[r][j]);
+        y.v[j] = TR::st(has_base ? CB::apply(base[j], val) : val);
+      }
+      if (VEC && ncol == SC_V) {
+        if (a.stream_out) store_stream(reinterpret_cast<FVec<S, SC_V> *>(q + r * a.out_step), y);
+        else *reinterpret_cast<FVec<S, SC_V> *>(q + r * a.out_step) = y;
+      } else {
+#pragma unroll
+        for (int j = 0; j < SC_V; j++)
+          if (j < ncol) q[r * a.out_step + j] = y.v[j];
+      }
+    }
+  }
+}
+
+// The device words of scan_cols, owned by the context: made (and cleared) on first use and when
+// a launch needs more of them, cleared again only when the epoch counter runs out.
+static int scan_cols_state(nxh_context *ctx, const char *op, size_t need) {
+  if (need > ctx->scan_state_bytes) {
+    if (ctx->scan_state) NXH_HIP(op, hipFree(ctx->scan_state));  // (waits for the device)
+    ctx->scan_state = nullptr;
+    ctx->scan_state_bytes = 0;
+    const size_t bytes = std::max<size_t>(need, (size_t)8 << 20);
+    void *p = nullptr;
+    NXH_HIP(op, hipMalloc(&p, bytes));
+    ctx->scan_state = (unsigned char *)p;
+    ctx->scan_state_bytes = bytes;
+    ctx->scan_epoch = 0x7fffffffu;  // forces the clearing below
+  }
+  if (ctx->scan_epoch >= 0x7ffffff0u) {
+    NXH_HIP(op, hipMemsetAsync(ctx->scan_state, 0, ctx->scan_state_bytes, ctx->stream));
+    ctx->scan_epoch = 0;
+  }
+  return NXH_OK;
+}
+static uint32_t scan_spin_limit() {
+  static const uint32_t v = [] {
+    const char *e = getenv("NXH_SCAN_SPIN");  // 0: every block takes the fallback (tests)
+    return e ? (uint32_t)strtoul(e, nullptr, 10) : (uint32_t)(1u << 16);
+  }();
+  return v;
+}
+
 template <int OP, int DT>
 static int scan_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, const nxh_tensor *out,
-                       const Geom &g, int64_t out_axis_stride) {
+                       const Geom &g, int64_t out_axis_stride, uint32_t stream) {
   using TR = Tr<DT>;
   using S = typename TR::S;
   using CB = Combine<OP, typename TR::C, TR::cat>;
@@ -250,6 +491,50 @@ static int scan_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
     const int cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
     // too few lines for one lane each to fill the chip: cut the axis into chunks
     int64_t chunks = std::min<int64_t>(((int64_t)cus * 1024 + g.n_out - 1) / g.n_out, a.len / 16);
+    if constexpr (scan_cols_ok<DT>()) {
+      // columns with unit stride on both sides, too few of them for a lane each: one pass with
+      // the carries handed down between blocks (not while a graph is captured: a replay would
+      // meet its own epoch in the words)
+      // 256, 128 or 64 rows per block: the tallest that still leaves two chunks. (Measured on
+      // [4096,8192] f32: 16 waves 48.8 us, 8 waves 51.2; with 4 waves the chain of chunks is 64 long.)
+      const int waves = a.len >= 512 ? 16 : a.len >= 256 ? 8 : 4;
+      const int64_t rows_per_block = (int64_t)SC_RW * waves;
+      const int64_t nstrips = (g.n_out + SC_COLS - 1) / SC_COLS, nchunks = (a.len + rows_per_block - 1) / rows_per_block;
+      const size_t need = (size_t)nstrips * SC_COLS * (size_t)nchunks * sizeof(uint64_t);
+      if (chunks >= 2 && g.nk == 1 && g.kin[0] == 1 && g.kout[0] == 1 && !ctx->capture && nchunks >= 2 &&
+          in->data != out->data &&  // (a lane that gives up its wait reads input rows other blocks have long finished)
+          nstrips * nchunks < ((int64_t)1 << 30) && need <= ((size_t)64 << 20)) {
+        int rc = scan_cols_state(ctx, op, need);
+        if (rc) return rc;
+        ScanColsArgs c;
+        c.in = a.in;
+        c.out = a.out;
+        c.len = a.len;
+        c.W = g.n_out;
+        c.in_step = a.in_step;
+        c.out_step = a.out_step;
+        c.nstrips = (uint32_t)nstrips;
+        c.epoch = ++ctx->scan_epoch;
+        c.spin_limit = scan_spin_limit();
+        c.stream_out = (stream & NXH_STREAM_OUT) != 0;
+        c.status = (uint64_t *)ctx->scan_state;
+        const uint32_t nblocks = (uint32_t)(nstrips * nchunks);
+        const uintptr_t al = (uintptr_t)(SC_V * sizeof(S)) - 1;
+        const bool vec = !(((uintptr_t)a.in | (uintptr_t)a.out) & al) && a.in_step % SC_V == 0 && a.out_step % SC_V == 0;
+        nxh_set_path("scan_cols");
+#define NXH_SCAN_COLS(WAVES)                                                                                         \
+  do {                                                                                                               \
+    if (vec) hipLaunchKernelGGL((scan_cols_kernel<DT, CB, true, WAVES>), dim3(nblocks), dim3(64 * WAVES), 0, ctx->stream, c); \
+    else hipLaunchKernelGGL((scan_cols_kernel<DT, CB, false, WAVES>), dim3(nblocks), dim3(64 * WAVES), 0, ctx->stream, c);    \
+  } while (0)
+        if (waves == 4) NXH_SCAN_COLS(4);
+        else if (waves == 8) NXH_SCAN_COLS(8);
+        else NXH_SCAN_COLS(16);
+#undef NXH_SCAN_COLS
+        NXH_HIP(op, hipGetLastError());
+        return NXH_OK;
+      }
+    }
     if (chunks >= 2 && chunks <= 65535) {
       using C = typename TR::C;
       int64_t chunk = (a.len + chunks - 1) / chunks;
@@ -273,7 +558,7 @@ static int scan_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
   return NXH_OK;
 }
 
-typedef int (*scan_fn)(nxh_context *, const char *, const nxh_tensor *, const nxh_tensor *, const Geom &, int64_t);
+typedef int (*scan_fn)(nxh_context *, const char *, const nxh_tensor *, const nxh_tensor *, const Geom &, int64_t, uint32_t);
 template <int OP>
 struct ScanRow {
   scan_fn fn[NXH_DTYPE_COUNT] = {};
@@ -289,7 +574,7 @@ struct ScanRow {
 };
 
 NXH_EXPORT int nxh_scan(nxh_context *ctx, int op, const nxh_tensor *out, const nxh_tensor *x, int axis) {
-  NXH_DEFER_BARRIER(ctx, out);
+  NXH_DEFER_SETTLE(ctx, 1, out, x);
   static const char *const names[NXH_REDUCE_COUNT] = {"cumsum", "cumprod", "cummax", "cummin"};
   if ((unsigned)op >= NXH_REDUCE_COUNT) return nxh_fail(NXH_INVALID_ARGUMENT, "scan", "unknown op");
   const char *name = names[op];
@@ -334,5 +619,16 @@ NXH_EXPORT int nxh_scan(nxh_context *ctx, int op, const nxh_tensor *out, const n
   }
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(name, hipSetDevice(ctx->device));
-  return fn(ctx, name, x, out, g, out->strides[axis]);
+  // whether the results go past the memory-side cache (only the single-pass column form asks)
+  const void *base[2] = {out->data, x->data};
+  uint64_t bytes[2] = {0, 0};
+  for (int k = 0; k < 2; k++) {
+    const nxh_tensor *t = k ? x : out;
+    uint64_t n = 1;
+    for (int d = 0; d < t->ndim; d++)
+      if (t->strides[d] != 0) n *= (uint64_t)t->shape[d];
+    bytes[k] = n * (uint64_t)nxh_elem_size(dt);
+  }
+  const uint32_t stream = nxh_cache_hints(ctx, 2, base, bytes, NXH_STREAM_OUT);
+  return fn(ctx, name, x, out, g, out->strides[axis], stream);
 }

@@ -161,7 +161,7 @@ def test_scan_matches_oracle(hip, oracle, d):
                         assert np.allclose(g, w, rtol=1e-4, atol=1e-4), what
                     else:
                         same_bits(g, w, what)
-    assert hip.last_path() in ("scan_rows", "scan_lines", "scan_chunks", "scan_rows_chunks")
+    assert hip.last_path() in ("scan_rows", "scan_lines", "scan_chunks", "scan_rows_chunks", "scan_cols")
 
 
 def test_scan_paths_nan_and_reference_vector(hip, oracle):
@@ -192,6 +192,9 @@ def test_scan_paths_nan_and_reference_vector(hip, oracle):
     assert hip.last_path() == "scan_rows_chunks"
     hw, ow = pair(np.ascontiguousarray(w.T), dt.int32, hip, oracle)
     same_bits(logical(hip.associative_scan(0, "max", hw)), logical(oracle.associative_scan(0, "max", ow)))
+    assert hip.last_path() == "scan_cols"
+    hw64, ow64 = pair(np.ascontiguousarray(w.T).astype(np.int64), dt.int64, hip, oracle)
+    same_bits(logical(hip.associative_scan(0, "max", hw64)), logical(oracle.associative_scan(0, "max", ow64)))
     assert hip.last_path() == "scan_chunks"
     f = rng.standard_normal((2, 50000)).astype(np.float32)
     f[1, 12345] = np.nan

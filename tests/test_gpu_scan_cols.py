@@ -1,0 +1,221 @@
+"""The single-pass column scan (cumsum / cumprod / cummax / cummin down the rows of a
+[rows][columns] view whose columns have unit stride): blocks hand their carries down through
+(flag, value) words instead of a second and third pass. Against the CPU oracle — integers,
+maxima and minima bit for bit, float sums and products within the reference contract's scan
+tolerance (6 x arithmetic) — over ragged shapes, row pitches, misaligned starts, every dtype the
+form takes and the ones it leaves to the older kernels; launches of different sizes in a row
+(the words are never cleared between launches); the bounded wait forced to give up at once
+from the host (every block then adds the rows above it from the input), in a process of its
+own; and inside a captured graph, where the form is not taken."""
+
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from helpers import TOL, close, encode, logical, pair, same_bits
+from raven_amd import dtype as dt
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+TAKEN = [dt.float32, dt.bfloat16, dt.float16, dt.int8, dt.uint8, dt.int16, dt.uint16, dt.int32, dt.uint32]
+NOT_TAKEN = [dt.float64, dt.int64, dt.uint64, dt.complex64]
+
+
+def data(rng, d, shape, oracle):
+    if d.is_float:
+        return encode(rng.uniform(0.5, 1.5, shape) * rng.choice([-1.0, 1.0], shape), d, oracle)
+    if d.is_complex:
+        return (rng.uniform(0.7, 1.2, shape) + 1j * rng.uniform(-0.5, 0.5, shape)).astype(np.complex64)
+    info = np.iinfo(d.np_storage)
+    return rng.integers(max(info.min, -3), min(info.max, 3), shape, endpoint=True).astype(d.np_storage)
+
+
+def check(hip, oracle, h, o, d, n, what, path="scan_cols"):
+    for op in ("sum", "prod", "max", "min"):
+        if d.is_complex and op in ("max", "min"):
+            continue
+        g, w = logical(hip.associative_scan(0, op, h)), logical(oracle.associative_scan(0, op, o))
+        if path:
+            assert hip.last_path() == path, (what, op, hip.last_path())
+        if d.is_complex:
+            assert np.allclose(g, w, rtol=1e-4, atol=1e-4), (what, op)
+        elif d.is_float and op in ("sum", "prod"):
+            tol = TOL[d.name][0] * 6
+            close(g, w, d, oracle, tol, tol * (n if op == "sum" else 1.0), f"{what} {op}")
+        else:
+            same_bits(g, w, f"{what} {op}")
+
+
+@pytest.mark.parametrize("d", TAKEN, ids=lambda d: d.name)
+def test_column_scan_matches_oracle(hip, oracle, d):
+    rng = np.random.default_rng(900 + d.tag)
+    # (rows, columns): one strip / several, whole and ragged chunks of 64 rows, whole and ragged strips of 256 columns
+    for rows, cols in ((130, 3), (1000, 300), (64 * 5, 256 * 2), (4097, 520), (129, 1028)):
+        x = data(rng, d, (rows, cols), oracle)
+        h, o = pair(x, d, hip, oracle)
+        check(hip, oracle, h, o, d, rows, f"[{rows},{cols}]")
+
+
+def test_row_pitches_misaligned_starts_and_strided_outputs(hip, oracle):
+    rng = np.random.default_rng(910)
+    for d in (dt.float32, dt.int16, dt.uint8):
+        x = data(rng, d, (700, 530), oracle)
+        # a window of a wider matrix: row pitch 530, first column 3 (no aligned vectors), 500 columns
+        h, o = pair(x, d, hip, oracle, lambda B, t: B.shrink(t, [(5, 655), (3, 503)]))
+        check(hip, oracle, h, o, d, 650, f"window {d.name}")
+        # aligned window: first column 8, 512 columns, pitch 530 (even but no multiple of 4 for 4-byte vectors)
+        h, o = pair(x, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 700), (8, 520)]))
+        check(hip, oracle, h, o, d, 700, f"aligned window {d.name}")
+        # rows taken backwards (negative row pitch)
+        h, o = pair(x, d, hip, oracle, lambda B, t: B.flip(t, (True, False)))
+        check(hip, oracle, h, o, d, 700, f"flipped rows {d.name}")
+
+
+@pytest.mark.parametrize("d", NOT_TAKEN, ids=lambda d: d.name)
+def test_wide_and_complex_dtypes_keep_the_three_pass_form(hip, oracle, d):
+    rng = np.random.default_rng(920 + d.tag)
+    x = data(rng, d, (3000, 40), oracle)
+    h, o = pair(x, d, hip, oracle)
+    check(hip, oracle, h, o, d, 3000, d.name, path="scan_chunks")
+
+
+def test_nan_inf_and_wrap(hip, oracle):
+    rng = np.random.default_rng(930)
+    x = rng.standard_normal((2000, 70)).astype(np.float32)
+    x[0, 1] = np.nan      # first row: NaN from the top
+    x[700, 2] = np.nan    # inside a later chunk
+    x[63, 3] = np.inf     # last row of the first chunk
+    x[64, 4] = -np.inf    # first row of the second
+    x[1999, 5] = np.nan
+    h, o = pair(x, dt.float32, hip, oracle)
+    for op in ("max", "min"):
+        same_bits(logical(hip.associative_scan(0, op, h)), logical(oracle.associative_scan(0, op, o)), op)
+        assert hip.last_path() == "scan_cols"
+    got = logical(hip.associative_scan(0, "sum", h))
+    want = logical(oracle.associative_scan(0, "sum", o))
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+    # modular sums and products of int32 / uint8 pass through the 32-bit words unchanged
+    y = np.full((1500, 9), 2**30 + 12345, np.int32)
+    hy, oy = pair(y, dt.int32, hip, oracle)
+    same_bits(logical(hip.associative_scan(0, "sum", hy)), logical(oracle.associative_scan(0, "sum", oy)))
+    z = np.full((600, 9), 3, np.int32)
+    hz, oz = pair(z, dt.int32, hip, oracle)
+    same_bits(logical(hip.associative_scan(0, "prod", hz)), logical(oracle.associative_scan(0, "prod", oz)))
+    b = rng.integers(0, 256, (900, 33)).astype(np.uint8)
+    hb, ob = pair(b, dt.uint8, hip, oracle)
+    for op in ("sum", "prod", "max", "min"):
+        same_bits(logical(hip.associative_scan(0, op, hb)), logical(oracle.associative_scan(0, op, ob)), op)
+    # int32 extremes as running maxima / minima (what the identity must never overwrite)
+    e = rng.integers(-2**31, 2**31, (1000, 17)).astype(np.int32)
+    he, oe = pair(e, dt.int32, hip, oracle)
+    for op in ("max", "min"):
+        same_bits(logical(hip.associative_scan(0, op, he)), logical(oracle.associative_scan(0, op, oe)), op)
+
+
+def test_launches_of_different_sizes_in_a_row(hip, oracle):
+    """The (flag, value) words stay as the last launch left them: a smaller launch after a
+    larger one, the same size twice, a larger one again (the block of words grows)."""
+    rng = np.random.default_rng(940)
+    for rows, cols in ((4096, 1024), (200, 40), (200, 40), (4096, 1024), (64 * 300, 300), (130, 2000), (20000, 2100)):
+        x = rng.integers(-1000, 1000, (rows, cols)).astype(np.int32)
+        h = hip.reshape(hip.from_host(x, dt.int32), (rows, cols))
+        got = logical(hip.associative_scan(0, "sum", h))
+        assert hip.last_path() == "scan_cols"
+        assert np.array_equal(got, np.cumsum(x.astype(np.int64), 0).astype(np.int32)), (rows, cols)
+        gm = logical(hip.associative_scan(0, "max", h))
+        assert np.array_equal(gm, np.maximum.accumulate(x, 0)), (rows, cols)
+
+
+def test_at_the_benchmarked_shape(hip):
+    """[4096, 8192] f32 down the rows: against numpy's float64 cumsum within the scan tolerance."""
+    rng = np.random.default_rng(950)
+    x = rng.standard_normal((4096, 8192)).astype(np.float32)
+    h = hip.reshape(hip.from_host(x, dt.float32), x.shape)
+    got = logical(hip.associative_scan(0, "sum", h))
+    assert hip.last_path() == "scan_cols"
+    want = np.cumsum(x.astype(np.float64), 0)
+    assert np.max(np.abs(got - want)) <= 6e-5 * 4096
+    assert np.array_equal(got[0], x[0])
+
+
+CHILD = """
+import sys
+sys.path.insert(0, {root!r}); sys.path.insert(0, {tests!r})
+import numpy as np
+from raven_amd import dtype as dt
+from raven_amd.nx_backend import Backend, logical
+hip = Backend()
+rng = np.random.default_rng(960)
+for rows, cols, d, npd in ((1000, 300, dt.int32, np.int32), (513, 70, dt.float32, np.float32), (300, 5, dt.uint8, np.uint8)):
+    x = rng.integers(0, 5, (rows, cols)).astype(npd)
+    h = hip.reshape(hip.from_host(x, d), (rows, cols))
+    out = hip.associative_scan(0, "sum", h)
+    assert hip.last_path() == "scan_cols", hip.last_path()
+    got = logical(out)
+    want = np.cumsum(x.astype(np.int64), 0).astype(npd)
+    assert np.array_equal(got, want), (rows, cols)
+hip.synchronize()
+print("ok")
+"""
+
+
+def test_the_wait_gives_up_and_every_block_adds_the_rows_above_itself():
+    """NXH_SCAN_SPIN=0: the first poll that does not find its word ends the wait; the lane then
+    folds the input rows above its chunk. Every kernel still ends by itself, and the results
+    are those of the ordinary run (integers, and floats that are small integers: exact)."""
+    env = dict(os.environ, NXH_SCAN_SPIN="0")
+    r = subprocess.run([sys.executable, "-c", CHILD.format(root=str(ROOT), tests=str(ROOT / "tests"))], env=env,
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-2000:], r.stderr[-4000:])
+
+
+def test_inside_a_captured_graph_the_older_form_runs(hip):
+    rng = np.random.default_rng(970)
+    x = rng.integers(-50, 50, (3000, 40)).astype(np.int32)
+    h = hip.reshape(hip.from_host(x, dt.int32), x.shape)
+    warm = logical(hip.associative_scan(0, "sum", h))
+    assert hip.last_path() == "scan_cols"
+    hip.capture_begin()
+    try:
+        out = hip.associative_scan(0, "sum", h)
+        path = hip.last_path()
+    finally:
+        graph = hip.capture_end()
+    assert path == "scan_chunks"
+    for _ in range(3):
+        graph.launch()
+        hip.synchronize()
+        assert np.array_equal(logical(out), warm)
+        # eager single-pass launches between the replays
+        assert np.array_equal(logical(hip.associative_scan(0, "sum", h)), warm)
+    graph.destroy()
+
+
+def test_a_loop_of_large_scans_streams_its_results_by_itself(hip):
+    """[4096, 8192] f32 in and out (256 MiB together, the size of the memory-side cache): after a
+    few calls whose results nothing reads, the results are stored past the cache; what they
+    hold does not change."""
+    rng = np.random.default_rng(980)
+    x = rng.integers(-3, 4, (4096, 8192)).astype(np.float32)  # small integers: float sums are exact
+    h = hip.reshape(hip.from_host(x, dt.float32), x.shape)
+    want = np.cumsum(x.astype(np.float64), 0).astype(np.float32)
+    hip.trim()
+    hip.set_cache_policy(3)
+    before = hip.cache_policy_stats()
+    for _ in range(6):
+        out = hip.associative_scan(0, "sum", h)
+        assert hip.last_path() == "scan_cols"
+        del out
+    after = hip.cache_policy_stats()
+    assert after["streaming_out"] > before["streaming_out"], (before, after)
+    assert np.array_equal(logical(hip.associative_scan(0, "sum", h)), want)
+    hip.set_cache_policy(0)
+    try:
+        assert np.array_equal(logical(hip.associative_scan(0, "sum", h)), want)
+    finally:
+        hip.set_cache_policy(3)
