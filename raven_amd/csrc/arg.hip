@@ -26,6 +26,18 @@ struct ArgCmp {
       else return v > b;
     }
   }
+  static constexpr Cat category = cat;
+  // strictly better, no NaN rule (a NaN on either side: false)
+  __device__ __forceinline__ static bool better(C v, C b) {
+    if constexpr (IS_MIN) return v < b;
+    else return v > b;
+  }
+  // the value nothing is worse than
+  __device__ __forceinline__ static C worst() {
+    if constexpr (cat == CAT_FLOAT) return IS_MIN ? (C)__builtin_inff() : (C)(-__builtin_inff());
+    else if constexpr (std::is_signed<C>::value) return IS_MIN ? (C)INT64_MAX : (C)INT64_MIN;
+    else return IS_MIN ? (C)UINT64_MAX : (C)0;
+  }
   // merge two (value, index) candidates; index < 0 means "none yet". Written as
   // selects on one predicate: an if-statement form of this function compiled
   // (hipcc 7.2, gfx950, several candidates per lane) to code that never took
@@ -162,9 +174,47 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
   const T *p = (const T *)a.in + in_off + l;
   C bv[V];
   I bi[V];
+  int64_t r = r0 + rg;
+  if constexpr (!HAS_IDX && (CMP::category == CAT_FLOAT || CMP::category == CAT_SINT || CMP::category == CAT_UINT)) {
+    // The first pass over plain values, three instructions per element: the running best
+    // starts at the worst value there is with the lane's first row as its index, so "strictly
+    // better" alone decides (equal values keep the earlier row). A NaN never compares better
+    // and is only noted; a lane that met one (rare) walks its rows again by the full rule below.
+    const I first = r < r1 ? (I)r : (I)-1;
+#pragma unroll
+    for (int k = 0; k < V; k++) bv[k] = CMP::worst(), bi[k] = first;
+    bool odd = false;
+    for (; r + (U - 1) * RG < r1; r += U * RG) {
+      FVec<T, V> x[U];
+#pragma unroll
+      for (int j = 0; j < U; j++) x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j * RG) * a.r_stride);
+#pragma unroll
+      for (int j = 0; j < U; j++)
+#pragma unroll
+        for (int k = 0; k < V; k++) {
+          const C v = IN::ld(x[j].v[k]);
+          const bool take = CMP::better(v, bv[k]);
+          bv[k] = take ? v : bv[k];
+          bi[k] = take ? (I)(r + j * RG) : bi[k];
+          if constexpr (CMP::category == CAT_FLOAT) odd |= v != v;
+        }
+    }
+    for (; r < r1; r += RG) {
+      FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
+#pragma unroll
+      for (int k = 0; k < V; k++) {
+        const C v = IN::ld(x.v[k]);
+        const bool take = CMP::better(v, bv[k]);
+        bv[k] = take ? v : bv[k];
+        bi[k] = take ? (I)r : bi[k];
+        if constexpr (CMP::category == CAT_FLOAT) odd |= v != v;
+      }
+    }
+    if (!odd) goto combine;
+    r = r0 + rg;
+  }
 #pragma unroll
   for (int k = 0; k < V; k++) bv[k] = C{}, bi[k] = -1;
-  int64_t r = r0 + rg;
   for (; r + (U - 1) * RG < r1; r += U * RG) {
     FVec<T, V> x[U];
     int32_t xi[U];
@@ -189,6 +239,7 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
       else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x.v[k]), (I)r);
     }
   }
+combine:
   if constexpr (RG > 1) {
     if (rg > 0) {
 #pragma unroll

@@ -628,7 +628,11 @@ static int map_launch_one(nxh_context *ctx, const char *op, const MapPlan &p) {
       // 172 us, 64 x 32 in 162 us (more blocks per compute unit, shorter dependent chains
       // through the barrier), 32 x 32 in 177 us, 128 x 64 with 16-byte stores of one-byte
       // results in 173 us; 128 x 32 patches for the one-byte results of a compare (whole
-      // 128-byte rows per store) ran that call four times slower.
+      // 128-byte rows per store) ran that call four times slower (15.8 -> 60.8 us; the cast of
+      // a permuted int32 to int8 14.7 -> 46.6). The same compare on contiguous operands takes
+      // 12.7-15.5 us, a permuted add with four-byte results 20.8 against 28.4 x 2/3 for a
+      // contiguous one: the turn through LDS costs every tiled call about a tenth, and the
+      // calls with narrow results show it most because they move the fewest bytes per element.
       constexpr int TX = MT::smax <= 4 ? 64 : 32;
       constexpr int TY = MT::smax == 4 ? 32 : (MT::smax < 4 ? 64 : 32);
       TiledArgs<F> a;

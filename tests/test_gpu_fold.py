@@ -135,6 +135,29 @@ def test_long_rows_columns_and_full_reductions(hip, oracle):
     same_bits(logical(hip.argmax(h, 0)), logical(oracle.argmax(o, 0)))
     assert hip.last_path() == "arg_col_split"
     same_bits(logical(hip.reduce("sum", [0, 1], h)), logical(oracle.reduce("sum", [0, 1], o)))
+    # column form on floats: NaNs (first one wins), whole columns of -inf / +inf / NaN, a NaN in the
+    # last row, ties with the worst value: the three-instruction inner loop and the full rule behind it
+    f = np.round(rng.uniform(-5, 5, (5000, 300))).astype(np.float32)
+    f[4000, 3] = np.nan
+    f[17, 3] = np.nan
+    f[:, 7] = -np.inf
+    f[:, 8] = np.inf
+    f[:, 9] = np.nan
+    f[4999, 10] = np.nan
+    f[0, 11] = -np.inf
+    f[2500:, 12] = -np.inf
+    f[1234, 13] = np.inf
+    for d in (dt.float32, dt.float64, dt.bfloat16):
+        h, o = pair(encode(f, d, oracle), d, hip, oracle)
+        for fn in ("argmax", "argmin"):
+            same_bits(logical(getattr(hip, fn)(h, 0)), logical(getattr(oracle, fn)(o, 0)), f"{fn} {d.name}")
+            assert hip.last_path() == "arg_col_split"
+    u = rng.integers(0, 3, (5000, 300)).astype(np.uint8)
+    u[:, 5] = 0
+    u[:, 6] = 255
+    h, o = pair(u, dt.uint8, hip, oracle)
+    for fn in ("argmax", "argmin"):
+        same_bits(logical(getattr(hip, fn)(h, 0)), logical(getattr(oracle, fn)(o, 0)), fn)
     z = np.round(rng.uniform(-5, 5, (4097, 513))).astype(np.float32)  # ties across chunk boundaries
     h, o = pair(z, dt.float32, hip, oracle)
     for axis in (0, 1):
