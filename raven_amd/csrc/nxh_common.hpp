@@ -89,6 +89,10 @@ struct nxh_context {
   // State of the single-pass column scan (scan.hip, scan_cols): a device block holding one
   // 64-bit (flag, value) word per column and row chunk; flags carry the launch's epoch, so the words are cleared once, when the block is
   // made, and never between launches. Freed with the context.
+  // results of the tanh GELU for all 65 536 inputs of bf16 [0] and f16 [1] (rowfuse.hip), and the
+  // four constants each table was made with
+  void *gelu_lut[2] = {nullptr, nullptr};
+  double gelu_lut_c[2][4] = {};
   unsigned char *scan_state = nullptr;
   size_t scan_state_bytes = 0;
   uint32_t scan_epoch = 0;

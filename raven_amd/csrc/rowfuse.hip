@@ -295,6 +295,25 @@ struct GeluArgs {
   int64_t n;
   double c[4];
 };
+// One element through the nine primitives of the sequence, each result rounded to the dtype.
+template <int DT>
+__device__ __forceinline__ typename Tr<DT>::S gelu_one(typename Tr<DT>::S in, typename Tr<DT>::C c0, typename Tr<DT>::C c1,
+                                                       typename Tr<DT>::C c2, typename Tr<DT>::C c3) {
+  using TX = Tr<DT>;
+  using C = typename TX::C;
+  const C v = TX::ld(in);
+  const C x2 = rnd<DT>(v * v);
+  const C x3 = rnd<DT>(v * x2);
+  const C p = rnd<DT>(x3 * c0);
+  const C q = rnd<DT>(v + p);
+  const C inner = rnd<DT>(q * c1);
+  C th;
+  if constexpr (DT == NXH_BF16 || DT == NXH_F16) th = rnd<DT>(tanh_for_16bit(inner));  // as the tanh primitive of these dtypes
+  else th = rnd<DT>(m_tanh(inner));
+  const C u = rnd<DT>(th + c2);
+  const C w = rnd<DT>(v * u);
+  return TX::st(w * c3);
+}
 template <int DT, int V>
 __global__ __launch_bounds__(256) void gelu_tanh_kernel(GeluArgs a) {
   using TX = Tr<DT>;
@@ -311,25 +330,56 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(GeluArgs a) {
     for (int j = 0; j < V; j++) in.v[j] = i + j < a.n ? x[i + j] : S{};
   const C c0 = (C)a.c[0], c1 = (C)a.c[1], c2 = (C)a.c[2], c3 = (C)a.c[3];
 #pragma unroll
-  for (int j = 0; j < V; j++) {
-    const C v = TX::ld(in.v[j]);
-    const C x2 = rnd<DT>(v * v);
-    const C x3 = rnd<DT>(v * x2);
-    const C p = rnd<DT>(x3 * c0);
-    const C q = rnd<DT>(v + p);
-    const C inner = rnd<DT>(q * c1);
-    C th;
-    if constexpr (DT == NXH_BF16 || DT == NXH_F16) th = rnd<DT>(tanh_for_16bit(inner));  // as the tanh primitive of these dtypes
-    else th = rnd<DT>(m_tanh(inner));
-    const C u = rnd<DT>(th + c2);
-    const C w = rnd<DT>(v * u);
-    o.v[j] = TX::st(w * c3);
-  }
+  for (int j = 0; j < V; j++) o.v[j] = gelu_one<DT>(in.v[j], c0, c1, c2, c3);
   if (V > 1 && i + V <= a.n) *reinterpret_cast<Pk<S, V> *>(out + i) = o;
   else
 #pragma unroll
     for (int j = 0; j < V; j++)
       if (i + j < a.n) out[i + j] = o.v[j];
+}
+
+// The same function by table. A 16-bit dtype has 65 536 inputs: their results, computed once by
+// gelu_one (so every entry holds the bits the arithmetic gives), are 128 KiB, which a block of
+// sixteen waves keeps in LDS; an element then costs one LDS read instead of some forty vector
+// instructions, and a large tensor goes through at the rate of memory ([8192,3072] bf16, 100 MB
+// of traffic: 32.2 us of arithmetic, 17.3 us by table). One block per compute unit walks its
+// share of the tensor, two 16-byte vectors per lane and turn, the next turn's requested before
+// this turn's are looked up.
+template <int DT>
+__global__ __launch_bounds__(256) void gelu_table_kernel(uint16_t *table, GeluArgs a) {
+  using C = typename Tr<DT>::C;
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  table[i] = gelu_one<DT>((uint16_t)i, (C)a.c[0], (C)a.c[1], (C)a.c[2], (C)a.c[3]);
+}
+constexpr int LUT_THREADS = 1024, LUT_BYTES = 65536 * 2;
+__global__ __launch_bounds__(LUT_THREADS) void gelu_lut_kernel(const uint16_t *table, const uint4 *x, uint4 *out, int64_t nvec,
+                                                               int64_t per_block) {
+  extern __shared__ uint16_t lut[];
+  for (int i = threadIdx.x; i < LUT_BYTES / 16; i += LUT_THREADS) reinterpret_cast<uint4 *>(lut)[i] = reinterpret_cast<const uint4 *>(table)[i];
+  __syncthreads();
+  const int64_t v0 = (int64_t)blockIdx.x * per_block, v1 = v0 + per_block < nvec ? v0 + per_block : nvec;
+  auto through = [&](uint32_t w) -> uint32_t { return (uint32_t)lut[w & 0xffffu] | ((uint32_t)lut[w >> 16] << 16); };
+  // the vectors of the next turn are requested before this turn's are looked up
+  constexpr int U = 2;
+  uint4 cur[U], nxt[U];
+  int64_t v = v0 + threadIdx.x;
+#pragma unroll
+  for (int u = 0; u < U; u++)
+    if (v + u * LUT_THREADS < v1) cur[u] = x[v + u * LUT_THREADS];
+  for (; v < v1; v += U * LUT_THREADS) {
+    const int64_t vn = v + U * LUT_THREADS;
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (vn + u * LUT_THREADS < v1) nxt[u] = x[vn + u * LUT_THREADS];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (v + u * LUT_THREADS < v1) {
+        const uint4 p = cur[u];
+        out[v + u * LUT_THREADS] = uint4{through(p.x), through(p.y), through(p.z), through(p.w)};
+      }
+#pragma unroll
+    for (int u = 0; u < U; u++) cur[u] = nxt[u];
+  }
 }
 
 // ── host side ───────────────────────────────────────────────────────────────
@@ -581,6 +631,42 @@ NXH_EXPORT int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_
   const bool vec = ((uintptr_t)a.x % 16) == 0 && ((uintptr_t)a.out % 16) == 0;
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
+  // 16-bit dtypes, four million elements or more, whole aligned vectors: by table (the table of a
+  // dtype is made on first use and again when the constants differ; not while a graph is being
+  // captured unless it already exists, since a capture cannot allocate it)
+  if ((dx == NXH_BF16 || dx == NXH_F16) && vec && n % 8 == 0 && n >= ((int64_t)1 << 22)) {
+    const int slot = dx == NXH_BF16 ? 0 : 1;
+    bool have = ctx->gelu_lut[slot] != nullptr;
+    if (!have && !ctx->capture) {
+      void *t = nullptr;
+      NXH_HIP(op, hipMalloc(&t, LUT_BYTES));
+      ctx->gelu_lut[slot] = t;
+      ctx->gelu_lut_c[slot][0] = std::nan("");
+      have = true;
+    }
+    if (have) {
+      if (memcmp(ctx->gelu_lut_c[slot], a.c, sizeof a.c) != 0) {
+        if (dx == NXH_BF16) hipLaunchKernelGGL((gelu_table_kernel<NXH_BF16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
+        else hipLaunchKernelGGL((gelu_table_kernel<NXH_F16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
+        NXH_HIP(op, hipGetLastError());
+        if (!ctx->capture) memcpy(ctx->gelu_lut_c[slot], a.c, sizeof a.c);  // (a captured fill runs at replay, not now)
+      }
+      static std::once_flag once;
+      static hipError_t attr_status = hipSuccess;
+      std::call_once(once, [] {
+        attr_status = hipFuncSetAttribute((const void *)gelu_lut_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LUT_BYTES);
+      });
+      NXH_HIP(op, attr_status);
+      const int64_t nvec = n / 8;
+      const int blocks = ctx->compute_units > 0 ? ctx->compute_units : 256;
+      const int64_t per_block = (nvec + blocks - 1) / blocks;
+      nxh_set_path("gelu_tanh_table");
+      hipLaunchKernelGGL(gelu_lut_kernel, dim3(blocks), dim3(LUT_THREADS), LUT_BYTES, ctx->stream,
+                         (const uint16_t *)ctx->gelu_lut[slot], (const uint4 *)a.x, (uint4 *)a.out, nvec, per_block);
+      NXH_HIP(op, hipGetLastError());
+      return NXH_OK;
+    }
+  }
   nxh_set_path("gelu_tanh");
   if (dx == NXH_F32) gelu_launch<NXH_F32>(ctx, a, vec);
   else if (dx == NXH_BF16) gelu_launch<NXH_BF16>(ctx, a, vec);

@@ -118,6 +118,8 @@ NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   for (auto &kv : ctx->device_tables) (void)hipFree(kv.second);
   if (ctx->fault_flag) (void)hipFree(ctx->fault_flag);
   if (ctx->scan_state) (void)hipFree(ctx->scan_state);
+  for (void *t : ctx->gelu_lut)
+    if (t) (void)hipFree(t);
   if (ctx->fault_flag_host) (void)hipHostFree(ctx->fault_flag_host);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
   for (hipEvent_t ev : ctx->stage_done)

@@ -126,6 +126,7 @@ class Backend:
 
     def __init__(self):
         self._lib = _ffi.load()
+        self._gelu_constants = {}
         h = C.c_void_p()
         rc = self._lib.nxh_context_create(C.byref(h))
         self._h = h.value
@@ -573,7 +574,10 @@ class Backend:
         if isinstance(constants, np.ndarray):
             enc = np.ascontiguousarray(constants.reshape(4))
         else:
-            enc = np.concatenate([encode_scalar(x.dtype, c) for c in constants])
+            key = (x.dtype.tag, tuple(constants))
+            enc = self._gelu_constants.get(key)
+            if enc is None:  # (encoding four scalars costs more host time than the kernel takes)
+                enc = self._gelu_constants[key] = np.concatenate([encode_scalar(x.dtype, c) for c in constants])
         o, a = out._desc(), x._desc()
         self._check(self._lib.nxh_gelu_tanh(self._h, C.byref(o), C.byref(a), enc.ctypes.data))
         return out

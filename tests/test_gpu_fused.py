@@ -178,3 +178,38 @@ def test_gelu_tanh_equals_the_sequence(hip, oracle, d):
         close(got, want_cpu, d, oracle, TOL[d.name][1], TOL[d.name][1], f"{d.name} {shape} vs oracle sequence")
     with pytest.raises(RuntimeError, match="contiguous"):
         hip.gelu_tanh(hip.permute(hip.full(d, (3, 4), 1.0), (1, 0)))
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_gelu_tanh_by_table_holds_the_arithmetic_bits_of_every_input(hip, d):
+    """Four million elements or more of a 16-bit dtype go through a table of all 65 536 results:
+    every entry must hold the bits the arithmetic kernel gives (NaN payloads included), for the
+    default constants and for others (the table is made again), and in a captured graph."""
+    rng = np.random.default_rng(310 + d.tag)
+    pats = np.arange(65536, dtype=np.uint16)
+    idx = rng.integers(0, 65536, 1 << 22).astype(np.int64)
+    idx[:65536] = pats  # every input at least once
+    small = hip.reshape(hip.from_host(pats, d), (65536,))
+    big = hip.reshape(hip.from_host(pats[idx], d), (2048, 2048))
+    for consts in ((0.044715, 0.7978845608028654, 1.0, 0.5), (0.05, 0.75, 1.0, 0.5), (0.044715, 0.7978845608028654, 1.0, 0.5)):
+        want = logical(hip.gelu_tanh(small, consts))
+        assert hip.last_path() == "gelu_tanh"
+        got = logical(hip.gelu_tanh(big, consts))
+        assert hip.last_path() == "gelu_tanh_table"
+        assert np.array_equal(got.reshape(-1).view(np.uint16), want.view(np.uint16)[idx]), consts
+    # a shape the table form leaves alone: not whole vectors
+    odd = hip.reshape(hip.from_host(np.concatenate([pats[idx], pats[:3]]), d), ((1 << 22) + 3,))
+    hip.gelu_tanh(odd)
+    assert hip.last_path() == "gelu_tanh"
+    hip.capture_begin()
+    try:
+        out = hip.gelu_tanh(big)
+        path = hip.last_path()
+    finally:
+        graph = hip.capture_end()
+    assert path == "gelu_tanh_table"
+    for _ in range(2):
+        graph.launch()
+        hip.synchronize()
+        assert np.array_equal(logical(out).reshape(-1).view(np.uint16), want.view(np.uint16)[idx])
+    graph.destroy()
