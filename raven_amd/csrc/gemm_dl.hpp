@@ -263,6 +263,16 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   // (gemm_tile.hpp: each step rounded to the dtype).
   S *C = (S *)a.C + co;
   auto narrow = [](float x) -> S { return EL::BF16 ? f32_to_bf16(x) : f32_to_f16(x); };
+  // The GELU table (bfloat16, when the host passes one and the idle stage memory behind the
+  // patches holds it): each lane requests at most one 16-byte piece now, and the pieces are
+  // put into LDS behind the barrier, while the patches are written.
+  constexpr bool LUT_ROOM = EPI && EL::BF16 && SH::PATCH_BYTES + 8192 <= SH::LDS_BYTES;
+  const bool use_lut = LUT_ROOM && a.gelu && a.gelu_lut != nullptr;
+  uint16_t *lut = reinterpret_cast<uint16_t *>(smem_raw + SH::PATCH_BYTES);
+  V16 lut_piece = {0, 0, 0, 0};
+  const bool lut_mine = use_lut && threadIdx.x < a.lut_n * 2 / 8;
+  if constexpr (LUT_ROOM)
+    if (lut_mine) lut_piece = reinterpret_cast<const V16 *>(a.gelu_lut)[threadIdx.x];
   wait_loads_and_meet<0>();  // every wave has read its last fragments; no load is in flight
   constexpr int PITCH = SH::PATCH_PITCH;
   S *patch = reinterpret_cast<S *>(smem_raw) + wave * (SH::WM * PITCH);
@@ -272,6 +282,12 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
     for (int j = 0; j < FB; j++)
 #pragma unroll
       for (int e = 0; e < 4; e++) patch[(i * 16 + g16 * 4 + e) * PITCH + j * 16 + q16] = narrow(acc[i][j][e]);
+  if constexpr (LUT_ROOM) {
+    if (use_lut) {  // (uniform over the block)
+      if (lut_mine) reinterpret_cast<V16 *>(lut)[threadIdx.x] = lut_piece;
+      __syncthreads();
+    }
+  }
   // the patch is read back by lanes of the same wave only: LDS serves a wave in order
   constexpr int CPR = SH::WN / 8;             // 16-byte pieces per patch row
   constexpr int NIT = SH::WM * CPR / 64;      // pieces per lane
@@ -300,7 +316,29 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
         for (int w = 0; w < 4; w++) {
           if (btile) q[w] = epi_add2<EL>(q[w], bq[i][w]);
           if (rtile) q[w] = epi_add2<EL>(q[w], rq[i][w]);
-          else if (a.gelu) q[w] = epi_gelu2<EL>(q[w], a.gc[0], a.gc[1], a.gc[2], a.gc[3]);
+        }
+        if (!rtile && a.gelu) {
+          bool by_table = false;
+          if constexpr (LUT_ROOM) {
+            // a register with an input of magnitude bits >= 0x7f00 (the last finite binade,
+            // infinities, NaN) sends the whole piece through the arithmetic
+            uint32_t top = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              const uint32_t lo16 = q[w] & 0x7fffu, hi16 = (q[w] >> 16) & 0x7fffu;
+              top = top > lo16 ? top : lo16;
+              top = top > hi16 ? top : hi16;
+            }
+            by_table = use_lut && top < 0x7f00u;
+            if (by_table) {
+#pragma unroll
+              for (int w = 0; w < 4; w++) q[w] = epi_gelu_lut2(q[w], lut, a.lut_lo, a.lut_n, a.gc[3]);
+            }
+          }
+          if (!by_table) {
+#pragma unroll
+            for (int w = 0; w < 4; w++) q[w] = epi_gelu2<EL>(q[w], a.gc[0], a.gc[1], a.gc[2], a.gc[3]);
+          }
         }
         *reinterpret_cast<V16 *>(ctile + (int64_t)row * a.ldc + col) = q;
       }

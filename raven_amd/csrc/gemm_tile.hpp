@@ -132,6 +132,12 @@ struct Args {
   // (c0..c3 = 0.044715, sqrt(2/pi), 1, 0.5 as the dtype holds them).
   int gelu;
   float gc[4];
+  // bfloat16, direct-to-LDS kernels with room for it: the GELU by table. 2 * lut_n results
+  // for the inputs with magnitude bits [lut_lo, lut_lo + lut_n) of either sign; below that
+  // range the result is narrow(x * c3), above it x or -0, as the host has verified for every
+  // input; infinities, NaN and the last finite binade take the arithmetic.
+  const void *gelu_lut;
+  uint32_t lut_lo, lut_n;
   // EPI kernels: up to three products that share A and differ in (B, bias, C) of one shape and
   // layout, as one launch (the q / k / v linears of an attention layer): tile column tn of
   // the launch belongs to member tn / gtn. Offsets of members 1 and 2 from member 0, in elements.
@@ -193,6 +199,30 @@ __device__ __forceinline__ uint32_t epi_gelu2(uint32_t x, float c0, float c1, fl
   epi_rnd2<EL>(a0, a1);
   a0 = a0 * c3, a1 = a1 * c3;
   return epi_narrow2<EL>(a0, a1);
+}
+
+// The same function for two bfloat16 neighbours through the LDS copy of the table
+// (Args::gelu_lut). The caller has sent registers holding an input of the last finite
+// binade, an infinity or a NaN (magnitude bits >= 0x7f00) to epi_gelu2 instead.
+__device__ __forceinline__ uint32_t epi_gelu_lut2(uint32_t x, const uint16_t *lut, uint32_t lo, uint32_t n, float c3) {
+  float v0, v1;
+  v0 = __builtin_bit_cast(float, x << 16);
+  v1 = __builtin_bit_cast(float, x & 0xffff0000u);
+  const uint32_t small = f32x2_to_bf16x2(v0 * c3, v1 * c3);
+  uint32_t out = 0;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const uint32_t e = h ? x >> 16 : x & 0xffffu;
+    const uint32_t m = e & 0x7fffu, neg = e >> 15;
+    const uint32_t idx = m - lo;  // (wraps below the range)
+    const uint32_t at = (idx < n ? idx : n - 1) + neg * n;
+    const uint32_t t = lut[at];
+    const uint32_t big = neg ? 0x8000u : e;
+    const uint32_t sm = h ? small >> 16 : small & 0xffffu;
+    const uint32_t r = m < lo ? sm : (idx < n ? t : big);
+    out |= r << (16 * h);
+  }
+  return out;
 }
 
 // One k-step of one 32x32 tile: a, b hold this lane's VE k-values of its row.

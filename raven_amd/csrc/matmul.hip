@@ -1173,6 +1173,15 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
         if (g.bc[i] % 8) return -1;
       g.gelu = 1;
       for (int i = 0; i < 4; i++) g.gc[i] = (float)epi->gelu[i];
+      if constexpr (EL::BF16) {
+        const void *lut = nullptr;
+        uint32_t lo = 0, n = 0;
+        if (nxh_gelu_epilogue_table(ctx, epi->gelu, &lut, &lo, &n)) {
+          g.gelu_lut = lut;
+          g.lut_lo = lo;
+          g.lut_n = n;
+        }
+      }
     }
   }
   // tiles of one member: a grouped launch picks the block shape its members would pick alone,

@@ -93,10 +93,25 @@ struct nxh_context {
   // four constants each table was made with
   void *gelu_lut[2] = {nullptr, nullptr};
   double gelu_lut_c[2][4] = {};
+  // The part of the bfloat16 table the fused linear's GELU epilogue keeps in LDS (rowfuse.hip,
+  // nxh_gelu_epilogue_table): entries [lo, lo + n) of either sign, n*2 values on the device;
+  // state 0 not made yet, 1 usable, -1 these constants have no usable form.
+  struct GeluEpilogueTable {
+    int state = 0;
+    double c[4] = {};
+    uint32_t lo = 0, n = 0;
+    void *dev = nullptr;
+  } gelu_epi;
   unsigned char *scan_state = nullptr;
   size_t scan_state_bytes = 0;
   uint32_t scan_epoch = 0;
 };
+
+// bfloat16 only. On success *table is a device array of 2 * *n results (the non-negative
+// inputs with magnitude bits [lo, lo + n), then the negative ones) of the tanh GELU with the
+// constants c; 0 when there is none (being made would need to wait for the stream, which a
+// capture forbids, or the constants do not fit the scheme). Called with ctx->mu held.
+int nxh_gelu_epilogue_table(nxh_context *ctx, const double *c, const void **table, uint32_t *lo, uint32_t *n);
 
 // Size of the static per-device workspace behind nxh_reduce_noalloc.
 constexpr size_t NXH_STATIC_WS_BYTES = (size_t)NXH_STATIC_WORKSPACE_BYTES;

@@ -21,6 +21,8 @@
 // primitives).
 
 #include <cmath>
+#include <cstring>
+#include <vector>
 
 #include "fold_common.hpp"
 #include "softmax_math.hpp"
@@ -602,6 +604,108 @@ NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, cons
   return NXH_OK;
 }
 
+// The table of a 16-bit dtype's 65 536 results (slot 0 bfloat16, 1 float16) for the constants c,
+// made on first use and again when the constants differ. *have is false when there is none and
+// none can be made now (a capture cannot allocate it).
+static int gelu_full_table(nxh_context *ctx, const char *op, int slot, const double *c, bool *have) {
+  *have = ctx->gelu_lut[slot] != nullptr;
+  if (!*have && !ctx->capture) {
+    void *t = nullptr;
+    NXH_HIP(op, hipMalloc(&t, LUT_BYTES));
+    ctx->gelu_lut[slot] = t;
+    ctx->gelu_lut_c[slot][0] = std::nan("");
+    *have = true;
+  }
+  if (*have && memcmp(ctx->gelu_lut_c[slot], c, 4 * sizeof(double)) != 0) {
+    GeluArgs a{};
+    for (int i = 0; i < 4; i++) a.c[i] = c[i];
+    if (slot == 0) hipLaunchKernelGGL((gelu_table_kernel<NXH_BF16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
+    else hipLaunchKernelGGL((gelu_table_kernel<NXH_F16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
+    NXH_HIP(op, hipGetLastError());
+    if (!ctx->capture) memcpy(ctx->gelu_lut_c[slot], c, 4 * sizeof(double));  // (a captured fill runs at replay, not now)
+  }
+  return NXH_OK;
+}
+
+// narrow(x * c3) for every bfloat16 x, computed where the epilogue computes it
+__global__ __launch_bounds__(256) void gelu_small_kernel(uint16_t *out, float c3) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  out[i] = f32_to_bf16(bf16_to_f32((uint16_t)i) * c3);
+}
+
+int nxh_gelu_epilogue_table(nxh_context *ctx, const double *c, const void **table, uint32_t *lo, uint32_t *n) {
+  const char *op = "linear_gelu_tanh";
+  auto &e = ctx->gelu_epi;
+  auto give = [&]() -> int {
+    if (e.state <= 0) return 0;
+    *table = e.dev;
+    *lo = e.lo;
+    *n = e.n;
+    return 1;
+  };
+  if (e.state != 0 && memcmp(e.c, c, sizeof e.c) == 0) return give();
+  if (ctx->capture) return 0;  // making it waits for the stream
+  // The whole table and the closed form of its low end, read back once. The part kept in LDS is
+  // [lo, hi): below lo every result must equal narrow(x * c3), from hi to the last finite binade
+  // x itself (positive) or -0 (negative); both bounds fall on binades (multiples of 128).
+  bool have = false;
+  if (gelu_full_table(ctx, op, 0, c, &have) != NXH_OK || !have) return 0;
+  void *small_dev = nullptr;
+  if (hipMalloc(&small_dev, LUT_BYTES) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  hipLaunchKernelGGL(gelu_small_kernel, dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)small_dev, (float)c[3]);
+  std::vector<uint16_t> full(65536), small(65536);
+  hipError_t err = hipMemcpyAsync(full.data(), ctx->gelu_lut[0], LUT_BYTES, hipMemcpyDeviceToHost, ctx->stream);
+  if (err == hipSuccess) err = hipMemcpyAsync(small.data(), small_dev, LUT_BYTES, hipMemcpyDeviceToHost, ctx->stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(ctx->stream);
+  (void)hipFree(small_dev);
+  memcpy(e.c, c, sizeof e.c);
+  e.state = -1;
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  constexpr uint32_t TOP = 0x7f00u, MAXN = 2048;
+  uint32_t low = 0, high = TOP;
+  while (low < TOP) {  // extend [0, low) binade by binade
+    bool ok = true;
+    for (uint32_t m = low; m < low + 128 && ok; m++) ok = full[m] == small[m] && full[0x8000u | m] == small[0x8000u | m];
+    if (!ok) break;
+    low += 128;
+  }
+  while (high > 0) {  // extend [high, TOP) downwards
+    bool ok = true;
+    for (uint32_t m = high - 128; m < high && ok; m++) ok = full[m] == m && full[0x8000u | m] == 0x8000u;
+    if (!ok) break;
+    high -= 128;
+  }
+  if (low >= high) low = high >= 128 ? high - 128 : 0;  // (the two forms overlap: keep one binade)
+  if (high <= low || high - low > MAXN) return 0;
+  const uint32_t cnt = high - low;
+  std::vector<uint16_t> compact(2 * cnt);
+  for (uint32_t i = 0; i < cnt; i++) {
+    compact[i] = full[low + i];
+    compact[cnt + i] = full[0x8000u | (low + i)];
+  }
+  if (!e.dev && hipMalloc(&e.dev, 2 * MAXN * sizeof(uint16_t)) != hipSuccess) {
+    (void)hipGetLastError();
+    e.dev = nullptr;
+    return 0;
+  }
+  err = hipMemcpyAsync(e.dev, compact.data(), compact.size() * sizeof(uint16_t), hipMemcpyHostToDevice, ctx->stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(ctx->stream);  // (the host copy dies with this call)
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  e.lo = low;
+  e.n = cnt;
+  e.state = 1;
+  return give();
+}
+
 NXH_EXPORT int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *constants) {
   NXH_DEFER_TOUCH(ctx, 1, out, x);
   const char *op = "gelu_tanh";
@@ -636,21 +740,9 @@ NXH_EXPORT int nxh_gelu_tanh(nxh_context *ctx, const nxh_tensor *out, const nxh_
   // captured unless it already exists, since a capture cannot allocate it)
   if ((dx == NXH_BF16 || dx == NXH_F16) && vec && n % 8 == 0 && n >= ((int64_t)1 << 22)) {
     const int slot = dx == NXH_BF16 ? 0 : 1;
-    bool have = ctx->gelu_lut[slot] != nullptr;
-    if (!have && !ctx->capture) {
-      void *t = nullptr;
-      NXH_HIP(op, hipMalloc(&t, LUT_BYTES));
-      ctx->gelu_lut[slot] = t;
-      ctx->gelu_lut_c[slot][0] = std::nan("");
-      have = true;
-    }
+    bool have = false;
+    if (int trc = gelu_full_table(ctx, op, slot, a.c, &have)) return trc;
     if (have) {
-      if (memcmp(ctx->gelu_lut_c[slot], a.c, sizeof a.c) != 0) {
-        if (dx == NXH_BF16) hipLaunchKernelGGL((gelu_table_kernel<NXH_BF16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
-        else hipLaunchKernelGGL((gelu_table_kernel<NXH_F16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
-        NXH_HIP(op, hipGetLastError());
-        if (!ctx->capture) memcpy(ctx->gelu_lut_c[slot], a.c, sizeof a.c);  // (a captured fill runs at replay, not now)
-      }
       static std::once_flag once;
       static hipError_t attr_status = hipSuccess;
       std::call_once(once, [] {

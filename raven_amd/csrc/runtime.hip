@@ -120,6 +120,7 @@ NXH_EXPORT void nxh_context_destroy(nxh_context *ctx) {
   if (ctx->scan_state) (void)hipFree(ctx->scan_state);
   for (void *t : ctx->gelu_lut)
     if (t) (void)hipFree(t);
+  if (ctx->gelu_epi.dev) (void)hipFree(ctx->gelu_epi.dev);
   if (ctx->fault_flag_host) (void)hipHostFree(ctx->fault_flag_host);
   if (ctx->stage) (void)hipHostFree(ctx->stage);
   for (hipEvent_t ev : ctx->stage_done)

@@ -313,6 +313,11 @@ static timing time_replays(const params *p, nxh_tensor ids, int iters) {
   must(L.set_deferred(ctx, 1), "set_deferred");
   nxh_graph *graph = NULL;
   uint64_t s0[NXH_DEFER_STAT_COUNT], s1[NXH_DEFER_STAT_COUNT];
+  /* once outside a capture first: what the library makes on first use (tables, workspaces)
+     cannot be made while a capture is open */
+  val warm = logits(p, ids);
+  must(L.synchronize(ctx), "synchronize");
+  drop(warm);
   must(L.deferred_stats(ctx, s0, NXH_DEFER_STAT_COUNT), "deferred_stats");
   must(L.capture_begin(ctx), "capture_begin");
   val out = logits(p, ids);

@@ -654,3 +654,34 @@ def test_matmul_wide_product_with_a_ragged_last_column_block(hip, oracle, d):
         # the left part against the same columns computed alone (aligned C, no split)
         left = hip.matmul(ha, hip.shrink(hb, [(0, k), (0, 16 * 256)]))
         same_bits(got_bits[:, :16 * 256], logical(left), "whole blocks: the same bits as the product of those columns alone")
+
+
+def test_linear_gelu_by_table_for_every_bfloat16_input(hip):
+    """The bfloat16 linear + GELU epilogue looks its results up in a table held in LDS. A zero
+    product plus a bias that runs through all 65 536 bit patterns (NaNs with their payloads,
+    infinities, subnormals, the last finite binade included) must give, in every row, the bits
+    of the arithmetic GELU kernel on that bias; the same for other constants (another table)
+    and inside a captured graph."""
+    n = 342 * 192  # whole 128 x 192 blocks, >= 65 536
+    pats = np.arange(n, dtype=np.uint32).astype(np.uint16)  # (wraps: the first 128 patterns twice)
+    x = hip.reshape(hip.from_host(np.zeros(128 * 64, np.uint16), dt.bfloat16), (128, 64))
+    w = hip.reshape(hip.from_host(np.zeros(64 * n, np.uint16), dt.bfloat16), (64, n))
+    b = hip.reshape(hip.from_host(pats, dt.bfloat16), (n,))
+    pre = hip.linear(x, w, b)  # 0 + bias: the bias itself, -0 turned into +0
+    row = hip.shrink(pre, [(0, 1), (0, n)])
+    for consts in ((0.044715, 0.7978845608028654, 1.0, 0.5), (0.05, 0.75, 1.0, 0.5)):
+        want = logical(hip.gelu_tanh(hip.contiguous(row), consts)).view(np.uint16)
+        assert hip.last_path() == "gelu_tanh"  # the arithmetic kernel (a small tensor)
+        got = logical(hip.linear_gelu_tanh(x, w, b, consts)).view(np.uint16)
+        assert hip.last_path() == "linear_dl_128x192", hip.last_path()
+        assert np.array_equal(got, np.broadcast_to(want, got.shape)), consts
+    hip.capture_begin()
+    try:
+        out = hip.linear_gelu_tanh(x, w, b, (0.05, 0.75, 1.0, 0.5))
+    finally:
+        graph = hip.capture_end()
+    for _ in range(2):
+        graph.launch()
+        hip.synchronize()
+        assert np.array_equal(logical(out).view(np.uint16), np.broadcast_to(want, got.shape))
+    graph.destroy()
