@@ -130,3 +130,44 @@ def test_a_working_set_that_fits_streams_nothing(hip):
 def test_mode_is_validated(hip):
     with pytest.raises(ValueError):
         hip.set_cache_policy(8)
+
+
+def test_forced_streaming_in_unfold_fold_and_the_column_scan(streaming, oracle):
+    """The other kernels that take the policy's decision: unfold's stores and the one-pass column
+    scan's stores (fold is in the loop as unfold's inverse). Forced to stream, their results are the oracle's."""
+    hip = streaming
+    rng = np.random.default_rng(720)
+    for d in (dt.float32, dt.int16, dt.uint8, dt.float64):
+        x = rng.integers(-50, 50, (2, 3, 16, 20)).astype(d.np_storage)
+        (hx, ox) = pair(x, d, hip, oracle)
+        args = ((3, 3), (1, 1), (1, 1), ((1, 1), (1, 1)))
+        hu, ou = hip.unfold(hx, *args), oracle.unfold(ox, *args)
+        same_bits(logical(hu), logical(ou), f"unfold {d.name}")
+        same_bits(logical(hip.fold(hu, (16, 20), *args)), logical(oracle.fold(ou, (16, 20), *args)), f"fold {d.name}")
+        args = ((3, 2), (2, 1), (1, 2), ((0, 1), (2, 0)))
+        hu, ou = hip.unfold(hx, *args), oracle.unfold(ox, *args)
+        same_bits(logical(hu), logical(ou), f"unfold strided {d.name}")
+    y = rng.integers(-9, 9, (700, 260)).astype(np.int32)
+    hy, oy = pair(y, dt.int32, hip, oracle)
+    same_bits(logical(hip.associative_scan(0, "sum", hy)), logical(oracle.associative_scan(0, "sum", oy)), "column scan")
+    assert hip.last_path() == "scan_cols"
+
+
+def test_a_loop_of_large_unfolds_streams_by_itself(hip):
+    """[8,64,128,128] f32 unfolded 3 x 3 (302 MB of windows nothing reads back): after a few calls
+    the windows are written past the cache; the interior taps still equal the shifted input."""
+    rng = np.random.default_rng(730)
+    x = rng.standard_normal((8, 64, 128, 128)).astype(np.float32)
+    hx = hip.reshape(hip.from_host(x, dt.float32), x.shape)
+    hip.trim()
+    hip.set_cache_policy(3)
+    before = hip.cache_policy_stats()
+    for _ in range(5):
+        u = hip.unfold(hx, (3, 3), (1, 1), (1, 1), ((1, 1), (1, 1)))
+        last = u
+    after = hip.cache_policy_stats()
+    assert after["streaming_out"] > before["streaming_out"], (before, after)
+    got = logical(last).reshape(8, 64, 9, 128, 128)
+    assert np.array_equal(got[:, :, 4], x)                       # the centre tap
+    assert np.array_equal(got[:, :, 0, 1:, 1:], x[:, :, :-1, :-1])  # the top-left tap
+    assert np.all(got[:, :, 0, 0, :] == 0)                       # its padding row
