@@ -352,7 +352,11 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
     for (int i = 0; i < NIT; i++) {
       const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
       const V16 v = *reinterpret_cast<const V16 *>(patch + row * PITCH + col);
-      *reinterpret_cast<V16_any *>(ctile + (int64_t)row * a.ldc + col) = v;
+      V16_any *dst = reinterpret_cast<V16_any *>(ctile + (int64_t)row * a.ldc + col);
+      // (streaming only ever with aligned rows, decided on the host; written as an instruction because
+      // the optimiser merges two stores that differ only in the hint)
+      if (a.stream_c) asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 0" : : "v"(dst), "v"(v) : "memory");
+      else *dst = v;
     }
   }
 }

@@ -138,6 +138,8 @@ struct Args {
   // input; infinities, NaN and the last finite binade take the arithmetic.
   const void *gelu_lut;
   uint32_t lut_lo, lut_n;
+  // direct-to-LDS kernels without an epilogue: C is stored past the memory-side cache
+  int stream_c;
   // EPI kernels: up to three products that share A and differ in (B, bias, C) of one shape and
   // layout, as one launch (the q / k / v linears of an attention layer): tile column tn of
   // the launch belongs to member tn / gtn. Offsets of members 1 and 2 from member 0, in elements.

@@ -1231,6 +1231,13 @@ static int try_tile(nxh_context *ctx, const GemmArgs &a, uint32_t nbatch, bool a
   // Whole tiles of 16-bit operands go straight into LDS (gemm_dl.hpp; load offsets are 32-bit:
   // 256 rows of a k-contiguous operand must stay below 4 GiB, and every row segment the
   // epilogue touches must be 16-byte aligned).
+  // A 16-bit product larger than the memory-side cache, rows of C whole 16-byte pieces: the
+  // direct-to-LDS kernels store C past the cache, which then keeps the operand panels that the
+  // other row and column blocks read again (bf16 [16,4096,4096]^2: 1 199-1 202 -> 1 205-1 224
+  // TFLOP/s). Not for rows at odd offsets (GPT-2's tied head, pitch 50 257): partial lines
+  // written past the cache cost that product 0.34 of its 0.72 ms.
+  if constexpr (!EPI && !EL::F32)
+    g.stream_c = (ctx->cache_hints & 2) && al16(g.C) && g.ldc % 8 == 0 && (uint64_t)nbatch * a.M * a.N * 2 > ((uint64_t)256 << 20);
   if constexpr (!EL::F32) {
     const int forced = forced_tile();
     // (without an epilogue C's rows may start at any element: the stores are unaligned-capable)
