@@ -605,8 +605,8 @@ NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, cons
 }
 
 // The table of a 16-bit dtype's 65 536 results (slot 0 bfloat16, 1 float16) for the constants c,
-// made on first use and again when the constants differ. *have is false when there is none and
-// none can be made now (a capture cannot allocate it).
+// made on first use and again when the constants differ. *have is false when there is none for
+// these constants and none can be made now (a capture can neither allocate nor refill it).
 static int gelu_full_table(nxh_context *ctx, const char *op, int slot, const double *c, bool *have) {
   *have = ctx->gelu_lut[slot] != nullptr;
   if (!*have && !ctx->capture) {
@@ -617,12 +617,16 @@ static int gelu_full_table(nxh_context *ctx, const char *op, int slot, const dou
     *have = true;
   }
   if (*have && memcmp(ctx->gelu_lut_c[slot], c, 4 * sizeof(double)) != 0) {
+    if (ctx->capture) {  // a captured refill would run at every replay, behind the back of this record
+      *have = false;
+      return NXH_OK;
+    }
     GeluArgs a{};
     for (int i = 0; i < 4; i++) a.c[i] = c[i];
     if (slot == 0) hipLaunchKernelGGL((gelu_table_kernel<NXH_BF16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
     else hipLaunchKernelGGL((gelu_table_kernel<NXH_F16>), dim3(256), dim3(256), 0, ctx->stream, (uint16_t *)ctx->gelu_lut[slot], a);
     NXH_HIP(op, hipGetLastError());
-    if (!ctx->capture) memcpy(ctx->gelu_lut_c[slot], c, 4 * sizeof(double));  // (a captured fill runs at replay, not now)
+    memcpy(ctx->gelu_lut_c[slot], c, 4 * sizeof(double));
   }
   return NXH_OK;
 }

@@ -213,3 +213,23 @@ def test_gelu_tanh_by_table_holds_the_arithmetic_bits_of_every_input(hip, d):
         hip.synchronize()
         assert np.array_equal(logical(out).reshape(-1).view(np.uint16), want.view(np.uint16)[idx])
     graph.destroy()
+    # other constants inside a capture: the table cannot be refilled there, the arithmetic runs;
+    # the table of the constants used last outside stays what it was
+    other = (0.03, 0.7, 1.0, 0.5)
+    want_other = logical(hip.gelu_tanh(small, other))
+    hip.gelu_tanh(big)  # (the table holds the default constants again)
+    assert hip.last_path() == "gelu_tanh_table"
+    hip.capture_begin()
+    try:
+        out = hip.gelu_tanh(big, other)
+        path = hip.last_path()
+    finally:
+        graph = hip.capture_end()
+    assert path == "gelu_tanh"
+    graph.launch()
+    hip.synchronize()
+    assert np.array_equal(logical(out).reshape(-1).view(np.uint16), want_other.view(np.uint16)[idx])
+    got = logical(hip.gelu_tanh(big))
+    assert hip.last_path() == "gelu_tanh_table"
+    assert np.array_equal(got.reshape(-1).view(np.uint16), want.view(np.uint16)[idx])
+    graph.destroy()
