@@ -219,3 +219,23 @@ def test_a_loop_of_large_scans_streams_its_results_by_itself(hip):
         assert np.array_equal(logical(hip.associative_scan(0, "sum", h)), want)
     finally:
         hip.set_cache_policy(3)
+
+
+def test_random_shapes_views_and_ops(hip, oracle):
+    """Sixty random cases: shape, dtype, operation, and the matrix as a window of a larger one."""
+    rng = np.random.default_rng(990)
+    dts = [dt.float32, dt.bfloat16, dt.float16, dt.int8, dt.uint8, dt.int16, dt.uint16, dt.int32, dt.uint32]
+    for case in range(60):
+        d = dts[int(rng.integers(len(dts)))]
+        rows, cols = int(rng.integers(64, 3000)), int(rng.integers(1, 700))
+        top, left, right = int(rng.integers(0, 3)), int(rng.integers(0, 5)), int(rng.integers(0, 5))
+        x = data(rng, d, (rows + top, cols + left + right), oracle)
+        h, o = pair(x, d, hip, oracle, lambda B, t: B.shrink(t, [(top, top + rows), (left, left + cols)]))
+        op = ("sum", "prod", "max", "min")[int(rng.integers(4))]
+        g, w = logical(hip.associative_scan(0, op, h)), logical(oracle.associative_scan(0, op, o))
+        what = f"case {case}: {d.name} {op} [{rows},{cols}] window at ({top},{left}) of width {cols + left + right}"
+        if d.is_float and op in ("sum", "prod"):
+            tol = TOL[d.name][0] * 6
+            close(g, w, d, oracle, tol, tol * (rows if op == "sum" else 1.0), what)
+        else:
+            same_bits(g, w, what)
