@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Nx eager hot path on one MI355X.
 
-A "step" is one pass of BASELINE.json's config 2 (broadcast / strided
+A "step" is one pass of the benchmark's configuration 2 (broadcast / strided
 elementwise) over synthetic input already resident in HBM:
 
   f32:   a[64,512,512] viewed through permute(0,2,1); b[1,512,1] expanded

@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterArgs a, int64_
       bad |= index < 0 || index >= a.axis_len;
       t[k] = (int)index;
     }
-    // also separates this round's LDS writes from the last round's reads
+    // also separates this pass's LDS writes from the last pass's reads
     if (__syncthreads_or(bad)) {
       if (threadIdx.x == 0) atomicOr(a.fault, 1);
       return;

@@ -1,7 +1,7 @@
 """The memory-side cache policy (nxh_set_cache_policy): which accesses of the elementwise
 kernels go past the cache is a per-call decision that may change when bytes reach HBM and
 never what they are. Checked three ways: every map operation of the layout matrix with
-every access forced to stream (mode 7) against the CPU oracle, bit for bit; BASELINE
+every access forced to stream (mode 7) against the CPU oracle, bit for bit; benchmark
 config 2's step repeated until the policy streams by itself, against the oracle and
 against the same step with the policy off; and that a working set that fits the cache
 streams nothing."""

@@ -1,4 +1,4 @@
-"""Parity at BASELINE.json's configurations, full size, through the C ABI.
+"""Parity at the benchmark's five configurations, full size, through the C ABI.
 
 Configs 1-3 are compared with the CPU oracle directly (it finishes them in
 seconds). Config 4's big GEMMs are compared with an f64 product on sampled
