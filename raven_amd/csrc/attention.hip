@@ -19,7 +19,9 @@
 // which is the correctly rounded quotient in all but rare cases. Both sit far
 // below the 16-bit rounding that follows them.
 //
-// Layout of the work: a block of two wave64s owns one 64-query tile of one
+// Layout of the work (the two-wave kernel; the default for a positive scale and a -inf fill is
+// its four-wave variant further down, which also splits every key tile between two waves): a
+// block of two wave64s owns one 64-query tile of one
 // (batch, head), each wave 32 queries; the grid hands out the late tiles of all
 // heads first, which under a causal mask are the long ones (pairing tile t with
 // tile T-1-t in one block balanced the blocks but left three waves per two SIMDs:
@@ -420,6 +422,215 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
   }
 }
 
+// The one-pass form with the scale in the exponent (AttArgs::raw), four waves per 64-query
+// tile instead of two. What bounds the two-wave kernel under a causal mask is not throughput but
+// the chain of its longest tiles: a wave walks up to sixteen key tiles one after the other and
+// each step is a string of dependent latencies (LDS tile, score MFMAs, maximum, exponentials,
+// the exchange with lane ^ 32, the MFMAs with V); at batch 2 the kernel takes as long as at
+// batch 8. Here waves 2p and 2p + 1 share the 32 queries of pair p and split every key tile
+// between them, keys 0..31 and 32..63: half the scores, exponentials and V products per step
+// and wave. Each wave keeps its own running reference, row sum and output; at the end the odd
+// wave hands its three to the even one through LDS and they are merged against the larger
+// reference, O = O_a 2^((m_a - m) c) + O_b 2^((m_b - m) c) and the same for the row sum, before
+// the one division. Rounding points are those of the two-wave form; only the f32 sums of the
+// output and of the row sum are added in another order.
+template <class EL, int DHEAD>
+__global__ __launch_bounds__(256) void attention_split_kernel(AttArgs a) {
+  using S = uint16_t;
+  constexpr int KSTEPS = DHEAD / 16, OT = DHEAD / 32, PK = DHEAD + 8, PV = DHEAD + 16, VPR = DHEAD / 8;
+  __shared__ __attribute__((aligned(16))) S Ks[KEYS * PK];
+  __shared__ __attribute__((aligned(16))) S Vs[KEYS * PV];
+  __shared__ float mrg[2][OT * 16 + 2][64];
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c32 = lane & 31, g = lane >> 5;
+  const int qh = wave >> 1, kh = wave & 1;
+  const int64_t bid = blockIdx.x;
+  const int tile = a.qtiles - 1 - (int)(bid / a.batches);  // late (long) tiles first
+  int64_t batch = bid % a.batches;
+  int64_t qo = 0, ko = 0, vo = 0, oo = 0, mo = 0;
+  for (int d = a.nouter - 1; d >= 0; d--) {
+    const int64_t c = batch % a.oshape[d];
+    batch /= a.oshape[d];
+    qo += c * a.q.outer[d];
+    ko += c * a.k.outer[d];
+    vo += c * a.v.outer[d];
+    oo += c * a.out.outer[d];
+    mo += c * a.mask.outer[d];
+  }
+  const S *Q = reinterpret_cast<const S *>(a.q.base) + qo;
+  const S *K = reinterpret_cast<const S *>(a.k.base) + ko;
+  const S *V = reinterpret_cast<const S *>(a.v.base) + vo;
+  S *O = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
+  const uint8_t *M = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
+
+  const int qw = tile * 64 + qh * 32;          // first query of the pair
+  const int qi = qw + c32;                     // this lane's query
+  const int qrow = qi < a.sq ? qi : a.sq - 1;  // clamp: rows past the end are never stored
+  V16 qf[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; s++)
+    qf[s] = *reinterpret_cast<const V16 *>(Q + (int64_t)qrow * a.q.row + s * 16 + g * 8);
+  const int qend = (tile + 1) * 64;
+  const int klimit = a.causal ? (qend < a.sk ? qend : a.sk) : a.sk;
+  const int ktiles = (klimit + KEYS - 1) / KEYS;
+
+  float m_run = -__builtin_inff(), l_run = 0.0f;
+  f32x16 oacc[OT];
+#pragma unroll
+  for (int t = 0; t < OT; t++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) oacc[t][e] = 0.0f;
+
+  // t[e]: the unscaled score of key j0 + (e/4)*8 + g*4 + e%4 against query qi, -inf where masked
+  auto scores = [&](int j0, float (&t)[16], bool inner) {
+    f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    const S *kr = Ks + (j0 % KEYS + c32) * PK + g * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++) {
+      const V16 kf = *reinterpret_cast<const V16 *>(kr + s * 16);
+      gemm_tile::mfma_step<EL>(acc, kf, qf[s]);
+    }
+    if (inner) {
+#pragma unroll
+      for (int e = 0; e < 16; e++) t[e] = acc[e];
+      return;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+      const int j = j0 + (e >> 2) * 8 + g * 4 + (e & 3);
+      bool keep = true;
+      if (a.causal) keep = j <= qi;
+      else if (a.has_mask) keep = M[(int64_t)qrow * a.mask.row + (int64_t)(j < a.sk ? j : a.sk - 1) * a.mask_col] != 0;
+      t[e] = keep && j < a.sk ? acc[e] : -__builtin_inff();  // (the fill of this form is -inf)
+    }
+  };
+
+  constexpr int NV = KEYS * VPR / 256;
+  static_assert(NV >= 1 && NV * 256 == KEYS * VPR, "whole vectors per lane");
+  V16 kpre[NV], vpre[NV];
+  auto prefetch = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int v = threadIdx.x + i * 256;
+      const int r = v / VPR, c = (v % VPR) * 8;
+      int key = kt * KEYS + r;
+      key = key < a.sk ? key : a.sk - 1;
+      kpre[i] = *reinterpret_cast<const V16 *>(K + (int64_t)key * a.k.row + c);
+      vpre[i] = *reinterpret_cast<const V16 *>(V + (int64_t)key * a.v.row + c);
+    }
+  };
+  prefetch(0);
+  for (int kt = 0; kt < ktiles; kt++) {
+    __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int v = threadIdx.x + i * 256;
+      const int r = v / VPR, c = (v % VPR) * 8;
+      *reinterpret_cast<V16 *>(Ks + r * PK + c) = kpre[i];
+      *reinterpret_cast<V16 *>(Vs + r * PV + c) = vpre[i];
+    }
+    __syncthreads();
+    if (kt + 1 < ktiles) prefetch(kt + 1);
+    const int j0 = kt * KEYS + kh * 32;
+    // nothing of this wave's half of the tile is visible to its queries
+    if (j0 >= a.sk || (a.causal && j0 > qw + 31)) continue;
+    float t[16];
+    scores(j0, t, j0 + 32 <= a.sk && !a.has_mask && (!a.causal || j0 + 31 <= qw));
+    float tm = t[0];
+#pragma unroll
+    for (int e = 1; e < 16; e++) tm = __builtin_fmaxf(tm, t[e]);
+    tm = __builtin_fmaxf(tm, xor32(tm));  // this query's maximum over the half tile, both lane halves agree
+    // the reference follows the maximum lazily, as in the two-wave kernel
+    const bool first = m_run == -__builtin_inff();
+    const bool grow = tm > m_run && (first || __builtin_fmaf(tm, a.c2, -m_run * a.c2) > 8.0f);
+    const float m_new = grow ? tm : m_run;
+    const float m_ref = m_new == -__builtin_inff() ? 0.0f : m_new;
+    const float mc = -m_ref * a.c2;
+    const float alpha = grow ? __builtin_amdgcn_exp2f(__builtin_fmaf(m_run, a.c2, mc)) : 1.0f;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) oacc[ot][e] = oacc[ot][e] * alpha;
+    }
+    uint32_t pk[8];
+    float sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+      const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(t[e], a.c2, mc));
+      const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(t[e + 1], a.c2, mc));
+      sum = sum + p0 + p1;
+      pk[e >> 1] = narrow2<EL>(p0, p1);
+    }
+    // O^T += V^T P^T for this wave's 32 keys (the B operand wants keys g*8 + 0..7 per k-step: the
+    // accumulator gave g*4 + 0..3 and 8 + g*4 + 0..3, so one half is swapped with lane ^ 32)
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      const uint32_t a0 = pk[ks * 4 + 0], a1 = pk[ks * 4 + 1];
+      const uint32_t b0 = pk[ks * 4 + 2], b1 = pk[ks * 4 + 3];
+      const uint32_t s0 = g == 0 ? b0 : a0, s1 = g == 0 ? b1 : a1;
+      const uint32_t r0 = (uint32_t)__shfl_xor((int)s0, 32, 64), r1 = (uint32_t)__shfl_xor((int)s1, 32, 64);
+      const V16 pf = g == 0 ? V16{a0, a1, r0, r1} : V16{r0, r1, b0, b1};
+#pragma unroll
+      for (int ot = 0; ot < OT; ot++) {
+        const int kk = kh * 32 + ks * 16 + g * 8 + ((lane & 15) >> 2);
+        const int rr = ot * 32 + ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
+        const S *src = Vs + kk * PV + rr;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)src);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(src + 4 * PV));
+        typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        gemm_tile::mfma_step<EL>(oacc[ot], V16{l2[0], l2[1], h2[0], h2[1]}, pf);
+      }
+    }
+    l_run = __builtin_fmaf(l_run, alpha, sum);
+    m_run = m_new;
+  }
+  // the odd wave of a pair hands over, the even one merges, divides and stores
+  if (kh == 1) {
+#pragma unroll
+    for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) mrg[qh][ot * 16 + e][lane] = oacc[ot][e];
+    mrg[qh][OT * 16][lane] = m_run;
+    mrg[qh][OT * 16 + 1][lane] = l_run;
+  }
+  __syncthreads();
+  if (kh == 1) return;
+  {
+    const float m_b = mrg[qh][OT * 16][lane], l_b = mrg[qh][OT * 16 + 1][lane];
+    const float m = __builtin_fmaxf(m_run, m_b);
+    const float m_ref = m == -__builtin_inff() ? 0.0f : m;
+    // (a wave that saw nothing has reference -inf, sum 0 and output 0: its factor is 2^-inf = 0)
+    const float s_a = __builtin_amdgcn_exp2f((m_run - m_ref) * a.c2), s_b = __builtin_amdgcn_exp2f((m_b - m_ref) * a.c2);
+    l_run = l_run * s_a + l_b * s_b;
+#pragma unroll
+    for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) oacc[ot][e] = oacc[ot][e] * s_a + mrg[qh][ot * 16 + e][lane] * s_b;
+  }
+  const float l_total = l_run + xor32(l_run);
+#pragma unroll
+  for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) oacc[ot][e] = oacc[ot][e] / l_total;
+  if (qi < a.sq) {
+    S *orow = O + (int64_t)qi * a.out.row;
+#pragma unroll
+    for (int ot = 0; ot < OT; ot++)
+#pragma unroll
+      for (int e = 0; e < 16; e += 4) {
+        const int d = ot * 32 + (e >> 2) * 8 + g * 4;
+        uint2 w;
+        w.x = narrow2<EL>(oacc[ot][e], oacc[ot][e + 1]);
+        w.y = narrow2<EL>(oacc[ot][e + 2], oacc[ot][e + 3]);
+        *reinterpret_cast<uint2 *>(orow + d) = w;
+      }
+  }
+}
+
 // NXH_ATTENTION=twopass selects the form that rounds each probability after the division by
 // the full row sum, as the primitive sequence does; the default walks the keys once.
 bool two_pass_wanted() {
@@ -432,6 +643,18 @@ int attention_launch(nxh_context *ctx, const char *op, const AttArgs &a, int hd)
   const int64_t blocks = a.batches * a.qtiles;
   if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many elements for one launch");
   const dim3 grid((unsigned)blocks), block(128);
+  if constexpr (ONLINE) {
+    if (a.raw) {  // the four-wave form ([b,12,1024,64] causal, b = 1 / 2 / 4 / 8 / 16: 19.9 / 20.9 / 23.4 / 37.3 / 74.0 us
+                  // against 29.2 / 30.4 / 32.4 / 42.5 / 80.8 us with two waves per tile)
+      switch (hd) {
+        case 32: hipLaunchKernelGGL((attention_split_kernel<EL, 32>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 64: hipLaunchKernelGGL((attention_split_kernel<EL, 64>), grid, dim3(256), 0, ctx->stream, a); break;
+        case 128: hipLaunchKernelGGL((attention_split_kernel<EL, 128>), grid, dim3(256), 0, ctx->stream, a); break;
+        default: return nxh_fail(NXH_FAILURE, op, "head dimension must be 32, 64 or 128");
+      }
+      return NXH_OK;
+    }
+  }
   switch (hd) {
     case 32: hipLaunchKernelGGL((attention_kernel<EL, 32, ONLINE>), grid, block, 0, ctx->stream, a); break;
     case 64: hipLaunchKernelGGL((attention_kernel<EL, 64, ONLINE>), grid, block, 0, ctx->stream, a); break;
