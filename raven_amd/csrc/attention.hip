@@ -434,6 +434,8 @@ __global__ __launch_bounds__(128) void attention_kernel(AttArgs a) {
 // reference, O = O_a 2^((m_a - m) c) + O_b 2^((m_b - m) c) and the same for the row sum, before
 // the one division. Rounding points are those of the two-wave form; only the f32 sums of the
 // output and of the row sum are added in another order.
+// (Asking the compiler for four waves per SIMD at head dim 64, 128 registers instead of the 136
+// it takes, changed nothing at batch 8 or 16: the kernel is bound by what it issues.)
 template <class EL, int DHEAD>
 __global__ __launch_bounds__(256) void attention_split_kernel(AttArgs a) {
   using S = uint16_t;
@@ -510,7 +512,28 @@ __global__ __launch_bounds__(256) void attention_split_kernel(AttArgs a) {
   constexpr int NV = KEYS * VPR / 256;
   static_assert(NV >= 1 && NV * 256 == KEYS * VPR, "whole vectors per lane");
   V16 kpre[NV], vpre[NV];
+  // this lane's vectors inside a key tile as element offsets from the tile's first row: a whole
+  // tile then costs one uniform base per operand and no address arithmetic per load
+  uint32_t koff[NV], voff[NV];
+  const bool short_offsets = (int64_t)KEYS * a.k.row < ((int64_t)1 << 31) && (int64_t)KEYS * a.v.row < ((int64_t)1 << 31) &&
+                             a.k.row >= 0 && a.v.row >= 0;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int v = threadIdx.x + i * 256;
+    const int r = v / VPR, c = (v % VPR) * 8;
+    koff[i] = (uint32_t)(r * a.k.row + c);
+    voff[i] = (uint32_t)(r * a.v.row + c);
+  }
   auto prefetch = [&](int kt) {
+    if (short_offsets && (kt + 1) * KEYS <= a.sk) {  // uniform: every key of the tile exists
+      const S *kb = K + (int64_t)kt * KEYS * a.k.row, *vb = V + (int64_t)kt * KEYS * a.v.row;
+#pragma unroll
+      for (int i = 0; i < NV; i++) {
+        kpre[i] = *reinterpret_cast<const V16 *>(kb + koff[i]);
+        vpre[i] = *reinterpret_cast<const V16 *>(vb + voff[i]);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int v = threadIdx.x + i * 256;
