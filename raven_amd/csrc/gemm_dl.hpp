@@ -273,7 +273,29 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
   const bool lut_mine = use_lut && threadIdx.x < a.lut_n * 2 / 8;
   if constexpr (LUT_ROOM)
     if (lut_mine) lut_piece = reinterpret_cast<const V16 *>(a.gelu_lut)[threadIdx.x];
-  wait_loads_and_meet<0>();  // every wave has read its last fragments; no load is in flight
+  // The epilogue's first bias and residual pieces are requested here already: their trip to
+  // memory then runs under the barrier and the patch writes instead of behind them. (The slab
+  // loads have all been waited for by now, so the barrier below need not wait for memory.)
+  constexpr int CPR = SH::WN / 8;             // 16-byte pieces per patch row
+  constexpr int NIT = SH::WM * CPR / 64;      // pieces per lane
+  static_assert(NIT * 64 == SH::WM * CPR, "whole passes");
+  constexpr int G = NIT <= 8 ? NIT : 4;       // pieces in flight per lane
+  static_assert(NIT % G == 0, "whole groups");
+  const S *btile = nullptr, *rtile = nullptr;
+  V16 bq0[G], rq0[G];
+  if constexpr (EPI) {
+    btile = a.bias ? (const S *)a.bias + n0 + wn : nullptr;
+    rtile = a.R ? (const S *)a.R + ro + (m0 + wm) * a.ldr + n0 + wn : nullptr;
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+      const int ch = i * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
+      if (btile) bq0[i] = *reinterpret_cast<const V16 *>(btile + col);
+      if (rtile) rq0[i] = *reinterpret_cast<const V16 *>(rtile + (int64_t)row * a.ldr + col);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave has read its last fragments
+  } else {
+    wait_loads_and_meet<0>();  // every wave has read its last fragments; no load is in flight
+  }
   constexpr int PITCH = SH::PATCH_PITCH;
   S *patch = reinterpret_cast<S *>(smem_raw) + wave * (SH::WM * PITCH);
 #pragma unroll
@@ -289,21 +311,19 @@ __global__ __launch_bounds__(SH::THREADS) void kernel(Args a) {
     }
   }
   // the patch is read back by lanes of the same wave only: LDS serves a wave in order
-  constexpr int CPR = SH::WN / 8;             // 16-byte pieces per patch row
-  constexpr int NIT = SH::WM * CPR / 64;      // pieces per lane
-  static_assert(NIT * 64 == SH::WM * CPR, "whole passes");
   S *ctile = C + (m0 + wm) * a.ldc + n0 + wn;
   if constexpr (EPI) {
     // the bias and residual pieces of a group are requested before the first one is used
-    const S *btile = a.bias ? (const S *)a.bias + n0 + wn : nullptr;
-    const S *rtile = a.R ? (const S *)a.R + ro + (m0 + wm) * a.ldr + n0 + wn : nullptr;
-    constexpr int G = NIT <= 8 ? NIT : 4;  // pieces in flight per lane
-    static_assert(NIT % G == 0, "whole groups");
 #pragma unroll
     for (int i0 = 0; i0 < NIT; i0 += G) {
       V16 bq[G], rq[G];
 #pragma unroll
       for (int i = 0; i < G; i++) {
+        if (i0 == 0) {  // (requested in front of the barrier above)
+          bq[i] = bq0[i];
+          rq[i] = rq0[i];
+          continue;
+        }
         const int ch = (i0 + i) * 64 + lane, row = ch / CPR, col = (ch % CPR) * 8;
         if (btile) bq[i] = *reinterpret_cast<const V16 *>(btile + col);
         if (rtile) rq[i] = *reinterpret_cast<const V16 *>(rtile + (int64_t)row * a.ldr + col);
