@@ -294,6 +294,16 @@ def next_ops(hip, W, linalg=False):
        hip.expand(f32((1, 64, 576)), (32, 64, 576)), f32((32, 576, 3136)), 2.0 * 32 * 64 * 576 * 3136, 157.3)
     mm("matmul f32 [256,2048] x [2048,256] (weight gradient, cut along K)", f32((256, 2048)), f32((2048, 256)),
        2.0 * 256 * 2048 * 256, 157.3)
+    # the dtypes without a matrix instruction: register-blocked on the vector unit (no matrix peak applies)
+    def mmv(name, a, b, ops):
+        timed(name, lambda: hip.matmul(a, b), 0, iters=5)
+        out[-1] = {"op": name + f" ({hip.last_path()})", "ms": out[-1]["ms"],
+                   "Top/s": round(ops / (out[-1]["ms"] * 1e-3) / 1e12, 2), "bound": "valu"}
+    ints = lambda shape, d: W.dev(rng.integers(-100, 100, shape).astype(d.np_storage), d)
+    mmv("matmul int32 2048^3", ints((2048, 2048), dt.int32), ints((2048, 2048), dt.int32), 2.0 * 2048 ** 3)
+    mmv("matmul int64 2048^3", ints((2048, 2048), dt.int64), ints((2048, 2048), dt.int64), 2.0 * 2048 ** 3)
+    c64 = lambda shape: W.dev((rng.standard_normal(shape) + 1j * rng.standard_normal(shape)).astype(np.complex64), dt.complex64)
+    mmv("matmul complex64 2048^3 (8 flops per term)", c64((2048, 2048)), c64((2048, 2048)), 8.0 * 2048 ** 3)
     # fused attention and the row kernels at GPT-2-small's shapes (bf16, batch 8, seq 1024)
     bf = lambda shape: W.dev((rng.standard_normal(shape).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16),
                              dt.bfloat16)

@@ -20,7 +20,8 @@
 //               the chip and the f32 partials are summed by a second pass. f32
 //               runs lane-per-column FMAs, bf16 / f16 run v_mfma_f32_16x16x32
 //               behind a wave-private transposing LDS tile.
-//   gemm_any    every other dtype / layout: one lane per output element.
+//   gemm_block  (gemm_block.hip) integers, float8, complex: register-blocked through LDS.
+//   gemm_any    what is left (thin products of those dtypes): one lane per output element.
 // Summation order differs from the reference's k-sequential loop, so float
 // results agree within the reference's GEMM tolerances; integer results are
 // exact (modular arithmetic is order-free).
@@ -28,40 +29,10 @@
 #include <algorithm>
 #include <cstdlib>
 
+#include "gemm_args.hpp"
 #include "gemm_tile.hpp"
 #include "gemm_dl.hpp"
 #include "nxh_common.hpp"
-
-constexpr int MM_MAXB = 8;  // batch dims decoded on the device
-
-struct BatchDims {
-  int n;
-  uint32_t shape[MM_MAXB];
-  int64_t a[MM_MAXB], b[MM_MAXB], c[MM_MAXB];
-};
-__device__ __forceinline__ void batch_decode(const BatchDims &d, uint32_t idx, int64_t &ao, int64_t &bo,
-                                             int64_t &co) {
-  ao = bo = co = 0;
-  for (int i = d.n - 1; i >= 0; i--) {
-    uint32_t q = idx / d.shape[i], c = idx - q * d.shape[i];
-    idx = q;
-    ao += (int64_t)c * d.a[i];
-    bo += (int64_t)c * d.b[i];
-    co += (int64_t)c * d.c[i];
-  }
-}
-
-struct GemmArgs {
-  const void *A, *B;
-  void *C;
-  int64_t M, N, K;
-  int64_t ars, acs, brs, bcs, crs, ccs;  // element strides: row, col
-  BatchDims batch;
-  uint32_t batch0;   // first batch index of this launch
-  int a_vec, b_vec;  // 16-byte loads allowed (alignment + stride multiple)
-  // tiled kernels only: extents that may be loaded along M / N (a padded copy's row length)
-  int64_t m_ld, n_ld;
-};
 
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -1714,8 +1685,11 @@ static int matmul_entry(nxh_context *ctx, const char *op, const nxh_tensor *C, c
     case NXH_BF16: return run_mfma_dtype<MMbf16>(ctx, g, (uint32_t)nbatch, al_a, al_b);
     case NXH_F16: return run_mfma_dtype<MMf16>(ctx, g, (uint32_t)nbatch, al_a, al_b);
     case NXH_F32: return run_mfma_dtype<MMf32>(ctx, g, (uint32_t)nbatch, al_a, al_b);
-#define NXH_CASE(DT) \
-  case DT: return launch_any<DT>(ctx, g, (uint32_t)nbatch);
+#define NXH_CASE(DT)                                         \
+  case DT: {                                                 \
+    const int rc = nxh_gemm_block(ctx, DT, g, (uint32_t)nbatch); \
+    return rc != -1 ? rc : launch_any<DT>(ctx, g, (uint32_t)nbatch); \
+  }
     case NXH_F64: return launch_f64(ctx, g, (uint32_t)nbatch);
       NXH_CASE(NXH_F8E4M3)
       NXH_CASE(NXH_F8E5M2)
