@@ -306,11 +306,17 @@ __global__ __launch_bounds__(256) void scatter_kernel(ScatterArgs a) {
 // at a time when their targets are pairwise distinct. Outputs of different
 // blocks are disjoint and each lane sees its column's updates in the serial
 // order, so the result is the reference's.
-template <int DT, bool ADD>
+// With V > 1 a lane owns V adjacent columns, moved as one 16-byte vector (the columns of `out`
+// and `updates` are then contiguous and every row starts on a 16-byte boundary: checked on the
+// host); a.columns counts lanes.
+template <int DT, bool ADD, int V>
 __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterArgs a, int64_t range_rows) {
   using TR = Tr<DT>;
-  using S = typename TR::S;
+  using E = typename TR::S;
   using C = typename TR::C;
+  struct alignas(V > 1 ? 16 : alignof(E)) S {
+    E v[V];
+  };
   constexpr int SCAN = 8, SPAN = 256 * SCAN, B = 8;
   __shared__ int s_cnt[4 * SCAN];
   __shared__ int s_pos[SPAN], s_tgt[SPAN];
@@ -318,21 +324,33 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterArgs a, int64_
   int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const bool live = col < a.columns;
   if (!live) col = a.columns - 1;  // idle lanes still take part in ballots and barriers
-  int64_t rem = col, oo = 0, uo = 0;
-  for (int d = a.ncol_dims - 1; d >= 0; d--) {
-    const int64_t c = rem % a.cshape[d];
-    rem /= a.cshape[d];
-    oo += c * a.c_ostride[d];
-    uo += c * a.c_ustride[d];
+  int64_t oo = 0, uo = 0;
+  if constexpr (V > 1) {
+    oo = uo = col * V;
+  } else {
+    int64_t rem = col;
+    for (int d = a.ncol_dims - 1; d >= 0; d--) {
+      const int64_t c = rem % a.cshape[d];
+      rem /= a.cshape[d];
+      oo += c * a.c_ostride[d];
+      uo += c * a.c_ustride[d];
+    }
   }
-  S *out = reinterpret_cast<S *>(a.out) + oo;
-  const S *upd = reinterpret_cast<const S *>(a.upd) + uo;
+  // (the strides along the axis are multiples of V when V > 1, so S-sized steps stay whole)
+  S *out = reinterpret_cast<S *>(reinterpret_cast<E *>(a.out) + oo);
+  const S *upd = reinterpret_cast<const S *>(reinterpret_cast<const E *>(a.upd) + uo);
+  const int64_t a_os = a.a_ostride / V, a_us = a.a_ustride / V;
   const int64_t lo = (int64_t)blockIdx.y * range_rows, hi = lo + range_rows;
   auto combine = [](S cur, S u) -> S {
     if constexpr (ADD) {
-      const C x = TR::ld(cur), y = TR::ld(u);
-      if constexpr (TR::cat == CAT_SINT) return TR::st((C)((uint64_t)x + (uint64_t)y));
-      else return TR::st((C)(x + y));
+      S r;
+#pragma unroll
+      for (int e = 0; e < V; e++) {
+        const C x = TR::ld(cur.v[e]), y = TR::ld(u.v[e]);
+        if constexpr (TR::cat == CAT_SINT) r.v[e] = TR::st((C)((uint64_t)x + (uint64_t)y));
+        else r.v[e] = TR::st((C)(x + y));
+      }
+      return r;
     } else {
       return u;
     }
@@ -383,7 +401,7 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterArgs a, int64_
 #pragma unroll
       for (int j = 0; j < B; j++) {
         tg[j] = s_tgt[m + j];
-        u[j] = upd[(base + s_pos[m + j]) * a.a_ustride];
+        u[j] = upd[(base + s_pos[m + j]) * a_us];
       }
       bool distinct = true;
 #pragma unroll
@@ -394,32 +412,41 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterArgs a, int64_
         S cur[B];
         if constexpr (ADD) {
 #pragma unroll
-          for (int j = 0; j < B; j++) cur[j] = out[(int64_t)tg[j] * a.a_ostride];
+          for (int j = 0; j < B; j++) cur[j] = out[(int64_t)tg[j] * a_os];
         }
 #pragma unroll
-        for (int j = 0; j < B; j++) out[(int64_t)tg[j] * a.a_ostride] = combine(cur[j], u[j]);
+        for (int j = 0; j < B; j++) out[(int64_t)tg[j] * a_os] = combine(cur[j], u[j]);
       } else {
         for (int j = 0; j < B; j++) {
-          S *o = out + (int64_t)tg[j] * a.a_ostride;
+          S *o = out + (int64_t)tg[j] * a_os;
           *o = combine(*o, u[j]);
         }
       }
     }
     for (; m < total; m++) {
-      S *o = out + (int64_t)s_tgt[m] * a.a_ostride;
-      *o = combine(*o, upd[(base + s_pos[m]) * a.a_ustride]);
+      S *o = out + (int64_t)s_tgt[m] * a_os;
+      *o = combine(*o, upd[(base + s_pos[m]) * a_us]);
     }
   }
 }
-typedef void (*scatter_launch_fn)(nxh_context *, const ScatterArgs &, bool, int64_t);
-// range_rows > 0 selects the kernel that also splits the targets into ranges.
+typedef void (*scatter_launch_fn)(nxh_context *, const ScatterArgs &, bool, int64_t, bool);
+// range_rows > 0 selects the kernel that also splits the targets into ranges; `vec` its form
+// with 16 bytes of columns per lane (a.columns then counts lanes).
 template <int DT>
-static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add, int64_t range_rows) {
+static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add, int64_t range_rows, bool vec) {
   const unsigned col_blocks = (unsigned)((a.columns + 255) / 256);
   if (range_rows > 0) {
     const dim3 grid(col_blocks, (unsigned)((a.axis_len + range_rows - 1) / range_rows));
-    if (add) hipLaunchKernelGGL((scatter_rows_kernel<DT, true>), grid, dim3(256), 0, ctx->stream, a, range_rows);
-    else hipLaunchKernelGGL((scatter_rows_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, a, range_rows);
+    constexpr int V = 16 / (int)sizeof(typename Tr<DT>::S);
+    if constexpr (V > 1) {
+      if (vec) {
+        if (add) hipLaunchKernelGGL((scatter_rows_kernel<DT, true, V>), grid, dim3(256), 0, ctx->stream, a, range_rows);
+        else hipLaunchKernelGGL((scatter_rows_kernel<DT, false, V>), grid, dim3(256), 0, ctx->stream, a, range_rows);
+        return;
+      }
+    }
+    if (add) hipLaunchKernelGGL((scatter_rows_kernel<DT, true, 1>), grid, dim3(256), 0, ctx->stream, a, range_rows);
+    else hipLaunchKernelGGL((scatter_rows_kernel<DT, false, 1>), grid, dim3(256), 0, ctx->stream, a, range_rows);
     return;
   }
   const dim3 grid(col_blocks);
@@ -492,8 +519,18 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
   bool uniform_index = a.axis_len <= 0x7fffffffLL;
   for (int d = 0; d < a.ncol_dims; d++)
     if (a.cshape[d] > 1 && a.c_istride[d] != 0) uniform_index = false;
+  // 16 bytes of columns per lane: the off-axis dims of `out` and `updates` are one contiguous
+  // run, a whole number of vectors long, and every row of both starts on a 16-byte boundary
+  // (embedding gradient [8192, 768] f32 into [50257, 768]: 38 -> 33 us)
+  bool vec = uniform_index && es < 16 && a.columns % (16 / es) == 0 && a.a_ostride % (16 / es) == 0 &&
+             a.a_ustride % (16 / es) == 0 && ((uintptr_t)a.out | (uintptr_t)a.upd) % 16 == 0;
+  for (int64_t d = a.ncol_dims - 1, run = 1; d >= 0 && vec; d--) {
+    if (a.cshape[d] > 1 && (a.c_ostride[d] != run || a.c_ustride[d] != run)) vec = false;
+    run *= a.cshape[d];
+  }
   int64_t range_rows = 0;
-  const int64_t col_blocks = (a.columns + 255) / 256;
+  const int64_t lanes = vec ? a.columns / (16 / es) : a.columns;
+  const int64_t col_blocks = (lanes + 255) / 256;
   const int64_t want_blocks = (int64_t)ctx->compute_units * 3;  // measured best on the embedding-gradient shape
   if (uniform_index && a.n_idx >= 256 && col_blocks * 4 <= want_blocks) {
     int64_t ranges = want_blocks / col_blocks;
@@ -501,8 +538,10 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
     if (ranges > 65535) ranges = 65535;
     if (ranges >= 2) range_rows = (a.axis_len + ranges - 1) / ranges;
   }
-  nxh_set_path(range_rows > 0 ? "scatter_rows" : "scatter_columns");
-  table[dt](ctx, a, mode == 1, range_rows);
+  vec = vec && range_rows > 0;
+  if (vec) a.columns = lanes;
+  nxh_set_path(vec ? "scatter_rows_16B" : range_rows > 0 ? "scatter_rows" : "scatter_columns");
+  table[dt](ctx, a, mode == 1, range_rows, vec);
   NXH_HIP(op, hipGetLastError());
   return nxh_collect_index_fault(ctx, op);
 }

@@ -291,9 +291,12 @@ def test_scatter_one_index_per_position_matches_oracle(hip, oracle, d):
     take the kernel that also splits the targets over blocks; sums of inexact
     floats with heavy duplication pin the order of accumulation."""
     rng = np.random.default_rng(90 + d.tag)
-    for axis, tshape, n in ((0, (301, 70), 2000), (1, (33, 517), 1111), (0, (9, 5), 700)):
+    for axis, tshape, n in ((0, (301, 70), 2000), (1, (33, 517), 1111), (0, (9, 5), 700), (0, (301, 72), 2500),
+                            (0, (57, 6, 8), 900)):
         ishape = list(tshape)
         ishape[axis] = n
+        # 16 bytes of columns per lane where the rows are whole vectors
+        vec = axis == 0 and int(np.prod(tshape[1:])) % (16 // d.itemsize) == 0
         ids = rng.integers(-tshape[axis], tshape[axis], n).astype(np.int32)
         if d.is_float:
             t = encode(rng.standard_normal(tshape), d, oracle)
@@ -303,12 +306,19 @@ def test_scatter_one_index_per_position_matches_oracle(hip, oracle, d):
             upd = rng.integers(-30000, 30000, ishape).astype(d.np_storage)
         ht, ot = pair(t, d, hip, oracle)
         hu, ou = pair(upd, d, hip, oracle)
-        line = [1, 1]
+        line = [1] * len(tshape)
         line[axis] = n
         hi, oi = (B.expand(B.reshape(B.from_host(ids, dt.int32), tuple(line)), tuple(ishape)) for B in (hip, oracle))
         for mode in ("set", "add"):
             same_bits(logical(hip.scatter(mode, False, ht, hi, hu, axis)),
                       logical(oracle.scatter(mode, False, ot, oi, ou, axis)), f"{mode} axis {axis} {tshape}")
+            assert hip.last_path() == ("scatter_rows_16B" if vec else "scatter_rows"), (tshape, hip.last_path())
+        if vec and len(tshape) == 2:
+            # updates whose rows start off a 16-byte boundary: one element per lane again
+            wide = np.concatenate([upd[:, :1], upd], axis=1)
+            hw, ow = pair(wide, d, hip, oracle, lambda B, t_: B.shrink(t_, [(0, n), (1, tshape[1] + 1)]))
+            same_bits(logical(hip.scatter("add", False, ht, hi, hw, axis)),
+                      logical(oracle.scatter("add", False, ot, oi, ow, axis)), "unaligned updates")
             assert hip.last_path() == "scatter_rows"
     bad = ids.copy()
     bad[n // 2] = tshape[axis]
