@@ -13,7 +13,8 @@
 // fold: (leading..., prod(kernel), L) -> (leading..., output...). One lane per
 // OUTPUT element sums the taps that land on it, in ascending tap order and in
 // the dtype's compute type, as nx_c_move.c:745-787 does: no atomics, no zeroing
-// pass, and float results equal the reference's bit for bit.
+// pass, and float results equal the reference's bit for bit. With window stride 1 and rows of
+// whole 16-byte vectors a lane owns a vector of adjacent outputs (fold_vec_kernel).
 //
 // Limits: at most 6 window dims and 8 leading dims (the reference allows 32 in
 // total); beyond that the call fails with Failure.
@@ -277,6 +278,124 @@ __global__ __launch_bounds__(256) void fold_kernel(WindowArgs a) {
   reinterpret_cast<S *>(a.out)[oo] = TR::st(acc);
 }
 
+// The same sums with V adjacent outputs of the last dim per lane (V x sizeof(S) = 16 bytes), for
+// window stride 1 everywhere, a unit-stride last output dim whose extent is a multiple of V and
+// a plain row-major windowed tensor of `in_elems` elements. The V outputs share everything about
+// a tap but their position in the last window dim, so a tap is one (unaligned) 16-byte load at
+// the first output's window and V selects; the address and validity arithmetic, which bounded
+// the one-output-per-lane form, is done once per V outputs. A vector that straddles the row's
+// ends is loaded whole and its outside elements are not added; it lies inside the tensor except
+// at the tensor's very first and last elements, where the elements are fetched one by one.
+// Every output still adds its taps in ascending order.
+template <int DT, int KT, int V>
+__global__ __launch_bounds__(256) void fold_vec_kernel(WindowArgs a, int32_t in_elems) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  using I = int32_t;
+  struct __attribute__((packed, aligned(alignof(S)))) VecU {
+    S v[V];
+  };
+  struct alignas(16) VecA {
+    S v[V];
+  };
+  const int64_t it64 = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (it64 >= a.total / V) return;
+  I ol = (I)it64;
+  I oc[KT];  // position in the padded frame (of the lane's first output, in the last dim)
+  I oo = 0, il = 0;
+  {
+    const I ev = (I)a.extent[KT - 1] / V, c = (ol % ev) * V;
+    ol /= ev;
+    oc[KT - 1] = c + (I)a.before[KT - 1];
+    oo += c;
+  }
+#pragma unroll
+  for (int d = KT - 2; d >= 0; d--) {
+    const I c = ol % (I)a.extent[d];
+    ol /= (I)a.extent[d];
+    oc[d] = c + (I)a.before[d];
+    oo += c * (I)a.sp_stride[d];
+  }
+  for (int d = a.ld - 1; d >= 0; d--) {
+    const I c = ol % (I)a.lshape[d];
+    ol /= (I)a.lshape[d];
+    oo += c * (I)a.l_out[d];
+    il += c * (I)a.l_in[d];
+  }
+  const S *in = reinterpret_cast<const S *>(a.in);
+  C acc[V];
+#pragma unroll
+  for (int e = 0; e < V; e++) {
+    if constexpr (TR::cat == CAT_COMPLEX) acc[e] = C{0, 0};
+    else acc[e] = (C)0;
+  }
+  auto add = [](C x, C v) -> C {
+    if constexpr (TR::cat == CAT_SINT) return (C)((uint64_t)x + (uint64_t)v);
+    else return (C)(x + v);
+  };
+  constexpr int TB = 9;
+  const I win_last = (I)a.win[KT - 1];
+  I kc[KT];
+#pragma unroll
+  for (int d = 0; d < KT; d++) kc[d] = 0;
+  const I taps = (I)a.kernel_prod;
+  for (I kf0 = 0; kf0 < taps; kf0 += TB) {
+    bool whole[TB], piecewise[TB];  // loaded as one vector / element by element (the tensor's two ends)
+    I at[TB], first[TB];            // offset of the first output's window; its coordinate in the last window dim
+#pragma unroll
+    for (int j = 0; j < TB; j++) {
+      bool valid = kf0 + j < taps;
+      I wf = 0;
+#pragma unroll
+      for (int d = 0; d < KT; d++) {
+        const I num = oc[d] - kc[d] * (I)a.dilation[d];
+        if (d == KT - 1) {
+          first[j] = num;
+          valid = valid && num > -V && num < win_last;  // some output of the V has a window here
+        } else {
+          valid = valid && num >= 0 && num < (I)a.win[d];
+        }
+        wf += num * (I)a.win_cp[d];
+      }
+      const I off = il + (kf0 + j) * (I)a.tap_stride + wf;
+      const bool inside = off >= 0 && off + V <= in_elems;
+      whole[j] = valid && inside;
+      piecewise[j] = valid && !inside;
+      at[j] = off;
+      bool carry = true;
+#pragma unroll
+      for (int d = KT - 1; d >= 0; d--) {
+        if (carry) {
+          kc[d]++;
+          carry = kc[d] >= (I)a.kernel[d];
+          if (carry) kc[d] = 0;
+        }
+      }
+    }
+    VecU raw[TB];
+#pragma unroll
+    for (int j = 0; j < TB; j++) raw[j] = *reinterpret_cast<const VecU *>(in + (whole[j] ? at[j] : 0));
+#pragma unroll
+    for (int j = 0; j < TB; j++) {
+#pragma unroll
+      for (int e = 0; e < V; e++) {
+        const bool ok = whole[j] && (uint32_t)(first[j] + e) < (uint32_t)win_last;
+        const C sum = add(acc[e], TR::ld(raw[j].v[e]));
+        acc[e] = ok ? sum : acc[e];
+      }
+      if (piecewise[j]) {
+        for (int e = 0; e < V; e++)
+          if ((uint32_t)(first[j] + e) < (uint32_t)win_last) acc[e] = add(acc[e], TR::ld(in[at[j] + e]));
+      }
+    }
+  }
+  VecA res;
+#pragma unroll
+  for (int e = 0; e < V; e++) res.v[e] = TR::st(acc[e]);
+  *reinterpret_cast<VecA *>(reinterpret_cast<S *>(a.out) + oo) = res;
+}
+
 struct G16w {
   uint64_t lo, hi;
 };
@@ -307,13 +426,35 @@ bool spans_fit_int32(const WindowArgs &a, int64_t windows) {
 }
 int rank_class(int K) { return K <= 3 ? K : WIN_MAXK; }
 
-typedef void (*fold_launch_fn)(nxh_context *, const WindowArgs &, int);
+typedef void (*fold_launch_fn)(nxh_context *, const WindowArgs &, int, bool);
+// `plain_in`: the windowed tensor is row-major without gaps (its offsets then lie in [0, rows x L)).
 template <int DT>
-void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt) {
+void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt, bool plain_in) {
   const dim3 grid((unsigned)((a.total + 255) / 256)), block(256);
   const bool narrow = fits_int32(a) && spans_fit_int32(a, a.L);  // 32-bit index arithmetic, offsets included
   bool unit = true;
   for (int d = 0; d < WIN_MAXK; d++) unit = unit && a.stride[d] == 1;
+  // 16 bytes of adjacent outputs per lane
+  constexpr int V = 16 / (int)sizeof(typename Tr<DT>::S);
+  if constexpr (V == 2 || V == 4 || V == 8) {
+    const int last = (kt <= 3 ? kt : WIN_MAXK) - 1;
+    bool vec = narrow && unit && plain_in && a.rows * a.L >= V && a.extent[last] % V == 0 && a.sp_stride[last] == 1 &&
+               (uintptr_t)a.out % 16 == 0;
+    for (int d = 0; d < last; d++) vec = vec && (a.extent[d] == 1 || a.sp_stride[d] % V == 0);
+    for (int d = 0; d < a.ld; d++) vec = vec && (a.lshape[d] == 1 || a.l_out[d] % V == 0);
+    if (vec) {
+      nxh_set_path("fold_16B");
+      const dim3 vgrid((unsigned)((a.total / V + 255) / 256));
+      const int32_t in_elems = (int32_t)(a.rows * a.L);
+      switch (kt) {
+        case 1: hipLaunchKernelGGL((fold_vec_kernel<DT, 1, V>), vgrid, block, 0, ctx->stream, a, in_elems); break;
+        case 2: hipLaunchKernelGGL((fold_vec_kernel<DT, 2, V>), vgrid, block, 0, ctx->stream, a, in_elems); break;
+        case 3: hipLaunchKernelGGL((fold_vec_kernel<DT, 3, V>), vgrid, block, 0, ctx->stream, a, in_elems); break;
+        default: hipLaunchKernelGGL((fold_vec_kernel<DT, WIN_MAXK, V>), vgrid, block, 0, ctx->stream, a, in_elems); break;
+      }
+      return;
+    }
+  }
 #define NXH_FOLD_CASE(KT)                                                                                        \
   case KT:                                                                                                       \
     if (narrow && unit) hipLaunchKernelGGL((fold_kernel<DT, int32_t, KT, true>), grid, block, 0, ctx->stream, a); \
@@ -595,7 +736,12 @@ NXH_EXPORT int nxh_fold(nxh_context *ctx, const nxh_tensor *out, const nxh_tenso
   nxh_set_path("fold");
   a.stream_out = 0;
   (void)window_cache_hints(ctx, out, x, 0);  // (the accounting only)
-  table.fn[dt](ctx, a, kt);
+  bool plain_in = a.win_stride == 1 && a.tap_stride == a.L;
+  for (int64_t d = a.ld - 1, run = a.kernel_prod * a.L; d >= 0; d--) {
+    if (a.lshape[d] > 1 && a.l_in[d] != run) plain_in = false;
+    run *= a.lshape[d];
+  }
+  table.fn[dt](ctx, a, kt, plain_in);
   NXH_HIP(op, hipGetLastError());
   return NXH_OK;
 }

@@ -191,7 +191,7 @@ def test_window_reference_vectors(hip):
     x = np.array(c["x"])
     u = hip.unfold(mk(hip, x, dt.float64), c["kernel"], c["stride"], [1], [(0, 0)])
     assert np.array_equal(logical(hip.fold(u, [x.shape[1]], c["kernel"], c["stride"], [1], [(0, 0)])), x)
-    assert hip.last_path() == "fold"
+    assert hip.last_path() in ("fold", "fold_16B")
     for leading, length, k, s in W["fold_overlap"]:
         x = ((np.arange(leading * length) % 13) + 1).astype(np.float64).reshape(leading, length)
         u = hip.unfold(mk(hip, x, dt.float64), [k], [s], [1], [(0, 0)])
@@ -248,6 +248,48 @@ def test_unfold_and_fold_match_oracle(hip, oracle, d):
     hp_, op_ = (B.permute(t, (1, 0, 2, 3)) for B, t in ((hip, hip.reshape(hu, (2, 6, 3, 9))), (oracle, oracle.reshape(ou, (2, 6, 3, 9)))))
     same_bits(logical(hip.fold(hp_, [9], [3], [1], [1], [(1, 1)])), logical(oracle.fold(op_, [9], [3], [1], [1], [(1, 1)])),
               "fold permuted")
+
+
+UNIT_STRIDE = [
+    # (output shape, kernel, dilation, padding): window stride 1, last extent a multiple of 8
+    ((2, 3, 8, 16), [3, 3], [1, 1], [(1, 1), (1, 1)]),
+    ((2, 2, 5, 24), [2, 5], [2, 3], [(0, 2), (7, 5)]),       # padding wider than a vector
+    ((3, 40), [7], [1], [(3, 3)]),
+    ((1, 64), [64], [1], [(0, 0)]),                          # one window
+    ((2, 8), [3], [4], [(4, 4)]),                            # most taps miss
+    ((2, 3, 4, 8), [2, 2, 3], [1, 1, 2], [(0, 0), (1, 0), (2, 2)]),
+    ((1, 2, 3, 2, 2, 2, 16), [1, 2, 1, 2, 2, 3], [1] * 6, [(0, 0), (1, 0), (0, 0), (0, 1), (1, 1), (1, 1)]),
+]
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.int16, dt.int32, dt.uint64], ids=lambda d: d.name)
+def test_fold_with_a_vector_of_outputs_per_lane(hip, oracle, d):
+    """Window stride 1 and rows of whole 16-byte vectors: a lane sums its taps for a vector of
+    adjacent outputs. Inexact float data pins the order of each output's additions
+    (nx_c_move.c:745-787)."""
+    rng = np.random.default_rng(540 + d.tag)
+    for shape, ks, dl, pd in UNIT_STRIDE:
+        k = len(ks)
+        st = [1] * k
+        cols_shape = tuple(oracle.unfold(oracle.buffer(d, shape), ks, st, dl, pd).shape)
+        if d.is_float:
+            c = encode(rng.standard_normal(cols_shape) * 3, d, oracle)
+        else:
+            c = rng.integers(0, 1000, cols_shape).astype(d.np_storage)
+        hc, oc = pair(c, d, hip, oracle)
+        got = logical(hip.fold(hc, shape[-k:], ks, st, dl, pd))
+        assert hip.last_path() == "fold_16B", (shape, hip.last_path())
+        same_bits(got, logical(oracle.fold(oc, shape[-k:], ks, st, dl, pd)), f"fold {d.name} {shape}")
+    # a windowed tensor with gaps (a slice along the windows) takes one output per lane again
+    shape, ks, dl, pd = UNIT_STRIDE[0]
+    cols_shape = tuple(oracle.unfold(oracle.buffer(d, shape), ks, [1, 1], dl, pd).shape)
+    wide = cols_shape[:-1] + (cols_shape[-1] + 3,)
+    c = encode(rng.standard_normal(wide), d, oracle) if d.is_float else rng.integers(0, 1000, wide).astype(d.np_storage)
+    cut = [(0, n) for n in cols_shape[:-1]] + [(2, cols_shape[-1] + 2)]
+    hc, oc = pair(c, d, hip, oracle, lambda B, t: B.shrink(t, cut))
+    got = logical(hip.fold(hc, shape[-2:], ks, [1, 1], dl, pd))
+    assert hip.last_path() == "fold"
+    same_bits(got, logical(oracle.fold(oc, shape[-2:], ks, [1, 1], dl, pd)), "fold of a slice")
 
 
 @pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.uint8], ids=lambda d: d.name)
