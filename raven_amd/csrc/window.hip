@@ -438,8 +438,9 @@ void fold_launch(nxh_context *ctx, const WindowArgs &a, int kt, bool plain_in) {
   constexpr int V = 16 / (int)sizeof(typename Tr<DT>::S);
   if constexpr (V == 2 || V == 4 || V == 8) {
     const int last = (kt <= 3 ? kt : WIN_MAXK) - 1;
-    bool vec = narrow && unit && plain_in && a.rows * a.L >= V && a.extent[last] % V == 0 && a.sp_stride[last] == 1 &&
-               (uintptr_t)a.out % 16 == 0;
+    // (offsets of the windowed tensor, plus a vector, stay below 2^31)
+    bool vec = narrow && unit && plain_in && a.rows * a.L >= V && a.rows * a.L < ((int64_t)1 << 31) - 16 &&
+               a.extent[last] % V == 0 && a.sp_stride[last] == 1 && (uintptr_t)a.out % 16 == 0;
     for (int d = 0; d < last; d++) vec = vec && (a.extent[d] == 1 || a.sp_stride[d] % V == 0);
     for (int d = 0; d < a.ld; d++) vec = vec && (a.lshape[d] == 1 || a.l_out[d] % V == 0);
     if (vec) {
