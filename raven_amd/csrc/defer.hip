@@ -1184,6 +1184,9 @@ int nxh_defer_record(nxh_context *ctx, int kind, int op, const nxh_tensor *out, 
   if (ok && kind == D_FULL) ok = numel(*out) == 1 && !nxh_is_packed(out->dtype);
   if (!ok) {
     int rc = flush_locked(ctx, w);
+    // the flush itself may have postponed the run that writes one of this call's operands
+    for (int k = 0; !rc && k < nin; k++)
+      if (ins[k]) rc = settle_read(ctx, w, ins[k]->data);
     if (out) {
       if (!rc) rc = settle_write(ctx, w, out->data);
       w->known.erase(out->data);

@@ -410,7 +410,11 @@ int main(int argc, char **argv) {
     val out = logits(&p, ids.t);
     const size_t bytes = (size_t)numel(&out.t) * elem_size(cfg.dtype);
     void *host = malloc(bytes);
-    must(L.memcpy_d2h(ctx, host, out.block, bytes), "to_host");
+    /* the head's result is a view of a block with padded rows (matmul in nx_host.h): gathered first */
+    const int nd = out.t.ndim, pitched = out.t.strides[nd - 2] != out.t.shape[nd - 1];
+    val dense = pitched ? contiguous(out.t) : out;
+    must(L.memcpy_d2h(ctx, host, dense.block, bytes), "to_host");
+    if (pitched) drop(dense);
     must(L.deferred_stats(ctx, s1, NXH_DEFER_STAT_COUNT), "deferred_stats");
     drop(out);
     nxhost_collect();

@@ -207,6 +207,17 @@ static val matmul(nxh_tensor a, nxh_tensor b) { /* frontend.ml:2346-2352, equal 
   int64_t shape[NXH_MAX_NDIM];
   memcpy(shape, a.shape, sizeof shape);
   shape[a.ndim - 1] = b.shape[b.ndim - 1];
+  /* A long row that is no whole number of 128-byte lines (GPT-2's 50257 logits per token): the
+     block's row pitch is rounded up to whole lines and the result is the [.., n] view of it, as
+     the Python mirror's matmul does. The reference allocates C-contiguous (nx_backend.ml:485-500). */
+  const int64_t n = shape[a.ndim - 1], line = 128 / (int64_t)elem_size(a.dtype);
+  if (n >= 4096 && n % line) {
+    shape[a.ndim - 1] = (n + line - 1) / line * line;
+    val o = fresh(a.dtype, a.ndim, shape);
+    o.t.shape[a.ndim - 1] = n;
+    must(L.matmul(ctx, &o.t, &a, &b), "matmul");
+    return o;
+  }
   val o = fresh(a.dtype, a.ndim, shape);
   must(L.matmul(ctx, &o.t, &a, &b), "matmul");
   return o;

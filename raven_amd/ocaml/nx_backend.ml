@@ -228,7 +228,20 @@ let matmul x y =
   let batch = Array.init (nd - 2) (fun i ->
       let ai = i - (nd - xnd) and bi = i - (nd - ynd) in
       Int.max (if ai >= 0 then xs.(ai) else 1) (if bi >= 0 then ys.(bi) else 1)) in
-  let out = create_tensor x.context x.dtype (Array.append batch [| xs.(xnd - 2); ys.(ynd - 1) |]) in
+  let shape = Array.append batch [| xs.(xnd - 2); ys.(ynd - 1) |] in
+  (* A long row that is no whole number of 128-byte lines (GPT-2's 50257 logits per token) gets a
+     row pitch rounded up to whole lines; the result is the [..; n] view of that block, so every
+     row of the GEMM's output starts on a line. The C backend allocates C-contiguous
+     (nx_backend.ml:485-500 there). *)
+  let n = shape.(nd - 1) in
+  let line = 128 / Int.max 1 (nbytes x.dtype 1) in
+  let out =
+    if n < 4096 || n mod line = 0 || Array.exists (fun d -> d = 0) shape then create_tensor x.context x.dtype shape
+    else begin
+      let padded = Array.copy shape in
+      padded.(nd - 1) <- (n + line - 1) / line * line;
+      shrink (create_tensor x.context x.dtype padded) (Array.map (fun d -> (0, d)) shape)
+    end in
   caml_matmul out x y; out
 
 (* nx_backend.ml:309-319 of the C backend *)

@@ -376,6 +376,8 @@ class Window:
             r = self.B.compare(e.op, ins[0], ins[1])
         elif e.kind == "matmul":
             r = self.B.matmul(ins[0], ins[1])
+            if r.view != View.create(e.shape):  # rows with a padded pitch: the record promised a plain block
+                r = self.B.contiguous(r)
         else:
             r = self.B.reduce(e.op, e.axes, ins[0])
         self.stats["issued"] += 1

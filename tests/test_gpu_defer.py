@@ -143,6 +143,28 @@ def test_postponed_entries_run_before_whatever_reads_them(hip, oracle, reader):
     del out
 
 
+def test_a_call_that_runs_at_once_reads_what_its_own_flush_postponed(hip, oracle):
+    """A recordable primitive whose result cannot be recorded (a matmul result with padded rows
+    is no plain block) executes the record and runs at once. Its operand here is the interior of a
+    fused run, which that very flush postpones because the caller still holds it: it has to be
+    written before the call reads it."""
+    rng = np.random.default_rng(37)
+    nx = Nx(hip)
+    x = tensor(hip, rng.standard_normal((20, 64)).astype(np.float32), dt.float32)
+    w = tensor(hip, rng.standard_normal((64, 4099)).astype(np.float32), dt.float32)
+    want = logical(hip.matmul(nx.exp(nx.sub(x, nx.max(x, [-1], keepdims=True))), w))
+    with deferred(hip) as win:
+        e = nx.exp(nx.sub(x, nx.max(x, [-1], keepdims=True)))
+        p = nx.div(e, nx.sum(e, [-1], keepdims=True))
+        out = hip.matmul(e, w)
+        assert tuple(out.strides) == (4128, 1)  # 4099 float32 per row, in whole 128-byte lines
+        s = win.delta()
+        assert (s["softmax_rows"], s["materialised"]) == (1, 4), s
+        got = logical(out)
+    same_bits(got, want, "matmul over the interior of a run that its own flush postponed")
+    del p
+
+
 def test_postponed_entries_run_before_their_operand_is_overwritten(hip, oracle):
     rng = np.random.default_rng(36)
     nx = Nx(hip)

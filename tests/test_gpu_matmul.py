@@ -685,3 +685,30 @@ def test_linear_gelu_by_table_for_every_bfloat16_input(hip):
         hip.synchronize()
         assert np.array_equal(logical(out).view(np.uint16), np.broadcast_to(want, got.shape))
     graph.destroy()
+
+
+@pytest.mark.parametrize("d", [dt.bfloat16, dt.float32, dt.int32], ids=lambda d: d.name)
+def test_long_ragged_rows_get_whole_memory_lines(hip, oracle, d):
+    """The binding gives a matmul result whose rows are long and no whole number of 128-byte
+    lines a padded row pitch and returns the [..., n] view of it (the reference allocates
+    C-contiguous, nx_backend.ml:485-500; GPT-2's tied head writes 50257 logits per token). The
+    view has the product's values, reshapes where its dims merge, and feeds further calls."""
+    rng = np.random.default_rng(1700 + d.tag)
+    line = 128 // d.itemsize
+    for (batch, m, k, n) in (((), 64, 64, 4099), ((2, 3), 16, 32, 4100), ((), 8, 128, 50257)):
+        a = encode(rng.integers(-4, 5, batch + (m, k)).astype(np.float64), d, oracle)
+        b = encode(rng.integers(-4, 5, (k, n)).astype(np.float64), d, oracle)
+        (ha, oa), (hb, ob) = pair(a, d, hip, oracle), pair(b, d, hip, oracle)
+        got = hip.matmul(ha, hb)
+        pitch = (n + line - 1) // line * line
+        assert tuple(got.shape) == batch + (m, n) and tuple(got.strides)[-2:] == (pitch, 1), (got.shape, got.strides)
+        want = logical(oracle.matmul(oa, ob))
+        same_bits(logical(got), want, f"{d.name} {batch} {m}x{k}x{n}")  # small integers: every sum is exact
+        flat = hip.reshape(got, (int(np.prod(batch, dtype=np.int64)) * m, n))  # the leading dims merge: still a view
+        same_bits(logical(flat), want.reshape(-1, n))
+        same_bits(logical(hip.contiguous(got)), want)
+        same_bits(logical(hip.reduce("max", [len(batch) + 1], got)), logical(oracle.reduce("max", [len(batch) + 1], oracle.matmul(oa, ob))))
+    # whole lines, or short rows: the plain block
+    for n in (4096, 4160, 1000):
+        got = hip.matmul(hip.full(d, (4, 8), 1), hip.full(d, (8, n), 1))
+        assert tuple(got.strides) == (n, 1)
