@@ -241,6 +241,11 @@ def next_ops(hip, W, linalg=False):
     parts = [W.dev(rng.standard_normal((1024, 4096)).astype(np.float32), dt.float32) for _ in range(4)]
     timed("cat 4 x [1024,4096] f32 along axis 0", lambda: hip.cat(parts, 0), 2 * 4 * 1024 * 4096 * 4)
     timed("cat 4 x [1024,4096] f32 along axis 1", lambda: hip.cat(parts, 1), 2 * 4 * 1024 * 4096 * 4)
+    # a result larger than the memory-side cache that nothing reads back: written past the cache
+    big = [W.dev(rng.standard_normal((2048, 8192)).astype(np.float32), dt.float32) for _ in range(4)]
+    timed("cat 4 x [2048,8192] f32 along axis 0 (256 MiB result, streamed by the cache policy)", lambda: hip.cat(big, 0),
+          2 * 4 * 2048 * 8192 * 4, iters=10)
+    del big
     y = W.dev(rng.standard_normal((4096, 8192)).astype(np.float32), dt.float32)
     timed("cumsum [4096,8192] f32 axis 1 (scan_rows)", lambda: hip.associative_scan(1, "sum", y), 2 * 4096 * 8192 * 4)
     timed("cumsum [4096,8192] f32 axis 0 (scan_cols: one pass, carries handed down between blocks)", lambda: hip.associative_scan(0, "sum", y), 2 * 4096 * 8192 * 4)

@@ -31,6 +31,7 @@
 // (key, counter) vector; normative bit for bit.
 
 #include "nxh_common.hpp"
+#include "stream_access.hpp"
 
 struct alignas(16) G16 {
   uint64_t lo, hi;
@@ -706,6 +707,7 @@ struct PadArgs {
   int64_t ostride[PAD_MAXD], istride[PAD_MAXD];  // elements (outer dims)
   int64_t before[PAD_MAXD], ishape[PAD_MAXD];
   unsigned char fill[16];
+  uint32_t stream_out;  // the stores go past the memory-side cache (decided per call, runtime.hip nxh_cache_hints)
 };
 template <class E, int VP>
 __global__ __launch_bounds__(256) void pad_kernel(PadArgs a) {
@@ -746,7 +748,9 @@ __global__ __launch_bounds__(256) void pad_kernel(PadArgs a) {
   } pk;
 #pragma unroll
   for (int j = 0; j < VP; j++) pk.v[j] = v[j];
-  *reinterpret_cast<Pack *>(reinterpret_cast<E *>(a.out) + oo) = pk;
+  Pack *dst = reinterpret_cast<Pack *>(reinterpret_cast<E *>(a.out) + oo);
+  if (a.stream_out) store_stream(dst, pk);
+  else *dst = pk;
 }
 template <class E>
 static void pad_launch(nxh_context *ctx, const PadArgs &a, int vp) {
@@ -790,6 +794,14 @@ static int pad_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP("pad", hipSetDevice(ctx->device));
   nxh_set_path("pad_fused");
+  {
+    uint64_t in_elems = 1;
+    for (int d = 0; d < nd; d++)
+      if (x->strides[d] != 0) in_elems *= (uint64_t)x->shape[d];
+    const void *base[2] = {out->data, x->data};
+    const uint64_t bytes[2] = {(uint64_t)total * (uint64_t)es, in_elems * (uint64_t)es};
+    a.stream_out = nxh_cache_hints(ctx, 2, base, bytes, NXH_STREAM_OUT) & NXH_STREAM_OUT;
+  }
   switch (es) {
     case 1: pad_launch<uint8_t>(ctx, a, vp); break;
     case 2: pad_launch<uint16_t>(ctx, a, vp); break;
@@ -803,7 +815,7 @@ static int pad_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *
 
 NXH_EXPORT int nxh_pad(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *fill_value,
                        const int64_t *pad_before) {
-  NXH_DEFER_TOUCH(ctx, 1, out, x);
+  NXH_DEFER_SETTLE(ctx, 1, out, x);  // (the fused kernel asks the cache policy itself; fills and copies do their own accounting)
   const char *op = "pad";
   if (!ctx || !out || !x || !fill_value || (out->ndim > 0 && !pad_before))
     return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
@@ -858,6 +870,7 @@ struct CatArgs {
   int64_t ostride[PAD_MAXD];
   int64_t istride[CAT_MAXM][PAD_MAXD];
   int64_t start[CAT_MAXM + 1];  // first axis coordinate of each member, and the end
+  uint32_t stream_out;          // as in PadArgs
 };
 template <class E, int VP>
 __global__ __launch_bounds__(256) void cat_kernel(CatArgs a) {
@@ -896,7 +909,9 @@ __global__ __launch_bounds__(256) void cat_kernel(CatArgs a) {
       pk.v[j] = reinterpret_cast<const E *>(a.in[m])[io];
     }
   }
-  *reinterpret_cast<Pack *>(reinterpret_cast<E *>(a.out) + oo) = pk;
+  Pack *dst = reinterpret_cast<Pack *>(reinterpret_cast<E *>(a.out) + oo);
+  if (a.stream_out) store_stream(dst, pk);
+  else *dst = pk;
 }
 template <class E>
 static void cat_launch(nxh_context *ctx, const CatArgs &a, int vp) {
@@ -955,6 +970,18 @@ static int cat_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP("cat", hipSetDevice(ctx->device));
   nxh_set_path("cat_fused");
+  {
+    const void *base[CAT_MAXM + 1] = {out->data};
+    uint64_t bytes[CAT_MAXM + 1] = {(uint64_t)total * (uint64_t)es};
+    for (int m = 0; m < n; m++) {
+      uint64_t e = 1;
+      for (int d = 0; d < nd; d++)
+        if (inputs[m]->strides[d] != 0) e *= (uint64_t)inputs[m]->shape[d];
+      base[m + 1] = inputs[m]->data;
+      bytes[m + 1] = e * (uint64_t)es;
+    }
+    a.stream_out = nxh_cache_hints(ctx, n + 1, base, bytes, NXH_STREAM_OUT) & NXH_STREAM_OUT;
+  }
   switch (es) {
     case 1: cat_launch<uint8_t>(ctx, a, vp); break;
     case 2: cat_launch<uint16_t>(ctx, a, vp); break;
@@ -968,7 +995,8 @@ static int cat_fused(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *
 
 NXH_EXPORT int nxh_cat(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *const *inputs, int n_inputs,
                        int axis) {
-  NXH_DEFER_BARRIER(ctx, out);
+  if (ctx && nxh_defer_active(ctx))
+    if (int drc = nxh_defer_barrier(ctx, out)) return drc;
   const char *op = "cat";
   if (!ctx || !out || (n_inputs > 0 && !inputs)) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -989,8 +1017,9 @@ NXH_EXPORT int nxh_cat(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor
   if (nxh_is_packed(out->dtype)) return nxh_fail(NXH_FAILURE, op, NXH_ERR_PACKED);
   for (int d = 0; d < out->ndim; d++)
     if (out->shape[d] > 1 && out->strides[d] == 0) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_OUT_ALIASED);
-  rc = cat_fused(ctx, out, inputs, n_inputs, axis);
+  rc = cat_fused(ctx, out, inputs, n_inputs, axis);  // (asks the cache policy with its operands' names)
   if (rc != -1) return rc;
+  nxh_cache_opaque(ctx);
   pos = 0;
   for (int m = 0; m < n_inputs; m++) {
     const nxh_tensor *in = inputs[m];

@@ -171,3 +171,44 @@ def test_a_loop_of_large_unfolds_streams_by_itself(hip):
     assert np.array_equal(got[:, :, 4], x)                       # the centre tap
     assert np.array_equal(got[:, :, 0, 1:, 1:], x[:, :, :-1, :-1])  # the top-left tap
     assert np.all(got[:, :, 0, 0, :] == 0)                       # its padding row
+
+
+def test_forced_streaming_in_pad_and_cat(streaming, oracle):
+    """pad and cat as one kernel take the policy's decision for their stores: forced to stream,
+    vectors and single elements alike, the results are the oracle's."""
+    hip = streaming
+    rng = np.random.default_rng(740)
+    for d in (dt.float32, dt.int16, dt.uint8, dt.float64, dt.complex128):
+        for shape, padding in (((6, 40), ((1, 2), (4, 4))), ((3, 5, 7), ((0, 1), (2, 0), (3, 1)))):
+            x = rng.integers(0, 100, shape).astype(d.np_storage)
+            hx, ox = pair(x, d, hip, oracle)
+            fill = np.array([7]).astype(d.np_storage)
+            same_bits(logical(hip.pad(hx, padding, fill)), logical(oracle.pad(ox, padding, fill)), f"pad {d.name} {shape}")
+            assert hip.last_path() == "pad_fused"
+        parts = [rng.integers(0, 100, (4, n, 8)).astype(d.np_storage) for n in (3, 8, 1)]
+        hs, os_ = zip(*(pair(p_, d, hip, oracle) for p_ in parts))
+        for axis in (0, 1, 2):
+            members = parts if axis == 1 else parts[:1] * 3
+            hm, om = (hs, os_) if axis == 1 else (hs[:1] * 3, os_[:1] * 3)
+            same_bits(logical(hip.cat(list(hm), axis)), logical(oracle.cat(list(om), axis)), f"cat {d.name} axis {axis}")
+            assert hip.last_path() == "cat_fused"
+            assert logical(hip.cat(list(hm), axis)).shape[axis] == sum(m.shape[axis] for m in members)
+
+
+def test_a_loop_of_large_cats_streams_by_itself(hip):
+    """4 x 64 MiB joined into 256 MiB that nothing reads back: after a few calls the result is
+    written past the cache; its values stay the members'."""
+    rng = np.random.default_rng(750)
+    parts = [rng.integers(-1000, 1000, (2048, 8192)).astype(np.int32) for _ in range(4)]
+    hs = [hip.reshape(hip.from_host(p_, dt.int32), p_.shape) for p_ in parts]
+    hip.trim()
+    hip.set_cache_policy(3)
+    before = hip.cache_policy_stats()
+    for _ in range(5):
+        last = hip.cat(hs, 0)
+    after = hip.cache_policy_stats()
+    assert hip.last_path() == "cat_fused"
+    assert after["streaming_out"] > before["streaming_out"], (before, after)
+    got = logical(last)
+    for i, p_ in enumerate(parts):
+        assert np.array_equal(got[2048 * i:2048 * (i + 1)], p_)
