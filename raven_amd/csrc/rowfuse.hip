@@ -26,6 +26,7 @@
 
 #include "fold_common.hpp"
 #include "softmax_math.hpp"
+#include "stream_access.hpp"
 #include "map_ops.hpp"
 
 namespace {
@@ -114,6 +115,9 @@ struct SoftmaxArgs {
   int has_scale, has_mask;
   int64_t mask_last;  // 0 or 1
   double scale, masked;  // exact images of the encoded scalars
+  // NXH_STREAM_IN / _OUT: the scores are read, the probabilities written past the memory-side
+  // cache (decided per call on the host, runtime.hip nxh_cache_hints)
+  uint32_t stream;
 };
 // EP: elements a lane holds at most (a row of up to 64 * RW * EP elements). The short forms
 // exist for their register count: 87 registers for EP = 32 leave five waves per SIMD, and
@@ -143,7 +147,8 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
   for (int v = 0; v < NV; v++) {
     const int c = v * T + tid;
     if (c < nvec) {
-      raw[v] = *reinterpret_cast<const Pk<SX, V> *>(x + (int64_t)c * V);
+      const Pk<SX, V> *src = reinterpret_cast<const Pk<SX, V> *>(x + (int64_t)c * V);
+      raw[v] = (a.stream & NXH_STREAM_IN) ? load_stream(src) : *src;
       if (a.has_mask) {
         if (a.mask_last) mk[v] = *reinterpret_cast<const Pk<uint8_t, V> *>(mask + (int64_t)c * V);
         else
@@ -205,7 +210,9 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(SoftmaxArgs a) {
         else y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t[v][j], s));
         o.v[j] = TO::st((typename TO::C)y);
       }
-      *reinterpret_cast<Pk<SO, V> *>(out + (int64_t)c * V) = o;
+      Pk<SO, V> *dst = reinterpret_cast<Pk<SO, V> *>(out + (int64_t)c * V);
+      if (a.stream & NXH_STREAM_OUT) store_stream(dst, o);
+      else *dst = o;
     }
   }
 }
@@ -506,7 +513,7 @@ void gelu_launch(nxh_context *ctx, const GeluArgs &a, bool vec) {
 
 NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x, const void *scale,
                                 const nxh_tensor *mask, const void *masked_value) {
-  NXH_DEFER_TOUCH(ctx, 1, out, x, mask);
+  NXH_DEFER_SETTLE(ctx, 1, out, x, mask);  // (the cache policy is asked below, once the call is known to launch)
   const char *op = "softmax_rows";
   if (!ctx || !out || !x || (mask && !masked_value)) return nxh_fail(NXH_INVALID_ARGUMENT, op, "null argument");
   int rc = nxh_check_tensor(op, out);
@@ -543,6 +550,21 @@ NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const n
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path("softmax_rows");
+  {
+    const nxh_tensor *ts[3] = {out, x, mask};
+    const void *base[3];
+    uint64_t bytes[3];
+    int nop = 0;
+    for (int k = 0; k < 3; k++) {
+      if (!ts[k]) continue;
+      uint64_t n = 1;
+      for (int d = 0; d < ts[k]->ndim; d++)
+        if (ts[k]->strides[d] != 0) n *= (uint64_t)ts[k]->shape[d];
+      base[nop] = ts[k]->data;
+      bytes[nop++] = n * (uint64_t)nxh_elem_size(ts[k]->dtype);
+    }
+    a.stream = nxh_cache_hints(ctx, nop, base, bytes);
+  }
   if (dx == NXH_F32 && dout == NXH_F32) softmax_launch<NXH_F32, NXH_F32>(ctx, a, vec);
   else if (dx == NXH_F32 && dout == NXH_BF16) softmax_launch<NXH_F32, NXH_BF16>(ctx, a, vec);
   else if (dx == NXH_F32) softmax_launch<NXH_F32, NXH_F16>(ctx, a, vec);

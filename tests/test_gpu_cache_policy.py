@@ -212,3 +212,37 @@ def test_a_loop_of_large_cats_streams_by_itself(hip):
     got = logical(last)
     for i, p_ in enumerate(parts):
         assert np.array_equal(got[2048 * i:2048 * (i + 1)], p_)
+
+
+def test_forced_streaming_in_softmax_rows(streaming, oracle):
+    """The fused softmax reads its scores and writes its probabilities past the cache when the
+    policy says so: forced, the result is what the kernel gives with plain accesses."""
+    hip = streaming
+    rng = np.random.default_rng(760)
+    for shape, out_d in (((7, 300), dt.float32), ((3, 5, 1024), dt.bfloat16), ((9, 70), dt.float32)):
+        x = rng.standard_normal(shape).astype(np.float32) * 3
+        hx = hip.reshape(hip.from_host(x, dt.float32), shape)
+        got = logical(hip.softmax_rows(hx, 0.125, None, None, out_d))
+        hip.set_cache_policy(0)
+        want = logical(hip.softmax_rows(hx, 0.125, None, None, out_d))
+        hip.set_cache_policy(7)
+        same_bits(got, want, f"softmax {shape} -> {out_d.name}")
+    e = np.exp(x * 0.125 - (x * 0.125).max(-1, keepdims=True))
+    assert np.allclose(got, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-7)
+
+
+def test_a_loop_of_large_softmaxes_streams_by_itself(hip):
+    """[24576,4096] float32 scores (402 MB) to bfloat16 probabilities nobody reads back."""
+    rng = np.random.default_rng(770)
+    x = rng.standard_normal((24576, 4096)).astype(np.float32)
+    hx = hip.reshape(hip.from_host(x, dt.float32), x.shape)
+    hip.trim()
+    hip.set_cache_policy(3)
+    before = hip.cache_policy_stats()
+    for _ in range(5):
+        last = hip.softmax_rows(hx, None, None, None, dt.bfloat16)
+    after = hip.cache_policy_stats()
+    assert after["streaming_out"] > before["streaming_out"] or after["streaming_in"] > before["streaming_in"], (before, after)
+    got = (logical(last)[:64].astype(np.uint32) << 16).view(np.float32)
+    e = np.exp(x[:64] - x[:64].max(-1, keepdims=True))
+    assert np.allclose(got, e / e.sum(-1, keepdims=True), rtol=2 ** -7, atol=1e-7)
