@@ -275,7 +275,9 @@ int nxh_fold(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *x,
    They have no binding of their own in the reference: a caller that sees the
    sequence (a deferred-evaluation window in the binding) substitutes the call.
    Floating dtypes f16/bf16/f32/f64; rows (the last axis) contiguous and at most
-   8192 long, otherwise Failure and the caller issues the primitives. */
+   2^24 long (a row of up to 8192 elements is held in registers, a longer one
+   is walked three times), otherwise Failure and the caller issues the
+   primitives. */
 
 /* frontend.ml:4242-4252 softmax over the last axis: max, sub, exp, sum, div.
    With `scale` (one storage element of x's dtype, host memory) x is first

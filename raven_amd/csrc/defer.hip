@@ -48,7 +48,7 @@ constexpr size_t LIMIT = 2048;
 // this many entries it is executed there, so that the device works while the host records on.
 constexpr size_t COPY_FLUSH = 48;
 constexpr size_t UPLOAD_LIMIT = 65536;  // bytes of a host upload that may wait in the record
-constexpr int64_t MAX_ROW = 8192;
+constexpr int64_t MAX_ROW = (int64_t)1 << 24;  // the longest row the fused row kernels take
 
 struct DEntry {
   int kind = 0, op = 0, nin = 0, n_axes = 0;

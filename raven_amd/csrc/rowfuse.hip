@@ -17,8 +17,9 @@
 // which a row's sum is added up.
 //
 // Rows live in registers: one wave64 per row up to 2048 elements, one block of
-// four waves up to 8192; longer rows are rejected (the caller then issues the
-// primitives).
+// four waves up to 8192. A longer row (a softmax over 50 257 logits) is walked
+// three times by its block — the statistics first, then the results — out of
+// the caches the first walk filled (softmax_long_kernel, layer_norm_long_kernel).
 
 #include <cmath>
 #include <cstring>
@@ -32,7 +33,10 @@
 namespace {
 
 constexpr int ROW_MAXD = 8;
-constexpr int EPL = 32;  // elements per lane at most
+constexpr int EPL = 32;  // elements per lane at most (rows held in registers)
+constexpr int ROW_REGS = 64 * 4 * EPL;  // the longest row a block holds in registers
+constexpr int LONG_THREADS = 1024, LONG_WAVES = LONG_THREADS / 64;  // a block of the long-row kernels
+constexpr int64_t ROW_MAX = (int64_t)1 << 24;  // the longest row at all (float32 counts it exactly)
 
 struct RowGeom {
   int64_t rows;
@@ -297,6 +301,148 @@ __global__ __launch_bounds__(256) void layer_norm_rows_kernel(LayerNormArgs a) {
   }
 }
 
+// ── rows longer than a block holds in registers ─────────────────────────────
+// A block of sixteen waves per row, as many blocks as the chip has units (each takes every
+// gridDim.x-th row): the rows in flight then fit the caches, and the second and third walk do not
+// go back to memory (one block of four waves per row, all rows at once: 380 us for [2048, 50257]
+// float32, the working set of 2048 rows being larger than the memory-side cache). Three walks: the maximum, the sum of the exponentials, the
+// quotients (softmax); the sum, the sum of squared differences, the results (layer norm). Every
+// elementwise step is the expression of the short kernels, so a result differs from theirs (and
+// from the primitives') only through the order of a row's sum; the second and third walk find
+// the row in the caches.
+template <int DTX, int DTO, int V>
+__global__ __launch_bounds__(LONG_THREADS) void softmax_long_kernel(SoftmaxArgs a) {
+  using TX = Tr<DTX>;
+  using TO = Tr<DTO>;
+  using C = typename TX::C;
+  using SX = typename TX::S;
+  using SO = typename TO::S;
+  __shared__ C lds[LONG_WAVES];
+  for (int64_t row = blockIdx.x; row < a.g.rows; row += gridDim.x) {
+  int64_t oo, mo;
+  const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.mask, oo, mo);
+  const SX *x = reinterpret_cast<const SX *>(a.x.base) + xo;
+  SO *out = reinterpret_cast<SO *>(const_cast<char *>(a.out.base)) + oo;
+  const uint8_t *mask = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
+  const int nvec = a.g.n / V;
+  const C scale = (C)a.scale, masked = (C)a.masked;
+  constexpr bool SHORT = DTX == NXH_F32 && (DTO == NXH_BF16 || DTO == NXH_F16);
+  // the scaled, masked scores of vector c
+  auto scores = [&](int c, C(&e)[V]) {
+    const Pk<SX, V> raw = *reinterpret_cast<const Pk<SX, V> *>(x + (int64_t)c * V);
+    Pk<uint8_t, V> mk;
+    if (a.has_mask) {
+      if (a.mask_last) mk = *reinterpret_cast<const Pk<uint8_t, V> *>(mask + (int64_t)c * V);
+      else
+#pragma unroll
+        for (int j = 0; j < V; j++) mk.v[j] = mask[0];
+    }
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+      C v = TX::ld(raw.v[j]);
+      if (a.has_scale) v = rnd<DTX>(OpMul::eval<CAT_FLOAT, C>(v, scale));
+      if (a.has_mask) v = mk.v[j] != 0 ? v : masked;
+      e[j] = v;
+    }
+  };
+  C m = Combine<NXH_RMAX, C, CAT_FLOAT>::init();
+#pragma unroll 8
+  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
+    C e[V];
+    scores(c, e);
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+      if constexpr (SHORT) m = __builtin_fmaxf(m, e[j]);
+      else m = Combine<NXH_RMAX, C, CAT_FLOAT>::apply(m, e[j]);
+    }
+  }
+  m = row_combine<NXH_RMAX, C, LONG_WAVES>(m, lds);
+  auto exponential = [&](C v) -> C {
+    const C d = rnd<DTX>(OpSub::eval<CAT_FLOAT, C>(v, m));
+    if constexpr (SHORT) return exp_nonpositive(d);
+    else return rnd<DTX>(OpExp::eval<CAT_FLOAT, C>(d));
+  };
+  C s = 0;
+#pragma unroll 8
+  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
+    C e[V];
+    scores(c, e);
+#pragma unroll
+    for (int j = 0; j < V; j++) s = s + exponential(e[j]);
+  }
+  s = rnd<DTX>(row_combine<NXH_SUM, C, LONG_WAVES>(s, lds));
+  C s_recip = 0;
+  if constexpr (SHORT) s_recip = 1.0f / s;
+#pragma unroll 8
+  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
+    C e[V];
+    scores(c, e);
+    Pk<SO, V> o;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+      const C t = exponential(e[j]);
+      C y;
+      if constexpr (SHORT) y = div_by_reciprocal(t, s, s_recip);
+      else y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t, s));
+      o.v[j] = TO::st((typename TO::C)y);
+    }
+    *reinterpret_cast<Pk<SO, V> *>(out + (int64_t)c * V) = o;
+  }
+  }
+}
+
+template <int DT, int V>
+__global__ __launch_bounds__(LONG_THREADS) void layer_norm_long_kernel(LayerNormArgs a) {
+  using TX = Tr<DT>;
+  using C = typename TX::C;
+  using S = typename TX::S;
+  __shared__ C lds[LONG_WAVES];
+  for (int64_t row = blockIdx.x; row < a.g.rows; row += gridDim.x) {
+  int64_t oo, uo;
+  const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.unused, oo, uo);
+  const S *x = reinterpret_cast<const S *>(a.x.base) + xo;
+  S *out = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
+  const S *gamma = reinterpret_cast<const S *>(a.gamma), *beta = reinterpret_cast<const S *>(a.beta);
+  const int nvec = a.g.n / V;
+  const C count = (C)a.count, eps = (C)a.eps;
+  C s = 0;
+#pragma unroll 8
+  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
+    const Pk<S, V> raw = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+#pragma unroll
+    for (int j = 0; j < V; j++) s = s + TX::ld(raw.v[j]);
+  }
+  const C mu = row_combine<NXH_SUM, C, LONG_WAVES>(s, lds) / count;
+  s = 0;
+#pragma unroll 8
+  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
+    const Pk<S, V> raw = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+      const C t = TX::ld(raw.v[j]) - mu;
+      s = s + t * t;
+    }
+  }
+  const C var = row_combine<NXH_SUM, C, LONG_WAVES>(s, lds) / count;
+  const C r = m_sqrt(var + eps);
+#pragma unroll 8
+  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
+    const Pk<S, V> raw = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+    Pk<S, V> gv, bv, o;
+    if (gamma) gv = *reinterpret_cast<const Pk<S, V> *>(gamma + (int64_t)c * V);
+    if (beta) bv = *reinterpret_cast<const Pk<S, V> *>(beta + (int64_t)c * V);
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+      C y = rnd<DT>((TX::ld(raw.v[j]) - mu) / r);  // leaves the float32 island here
+      if (gamma) y = rnd<DT>(y * TX::ld(gv.v[j]));
+      if (beta) y = rnd<DT>(y + TX::ld(bv.v[j]));
+      o.v[j] = TX::st(y);
+    }
+    *reinterpret_cast<Pk<S, V> *>(out + (int64_t)c * V) = o;
+  }
+  }
+}
+
 // ── gelu (tanh form) ────────────────────────────────────────────────────────
 struct GeluArgs {
   const char *x;
@@ -413,7 +559,7 @@ double decode_scalar(int dt, const void *p) {
 int row_geometry(const char *op, const nxh_tensor *x, RowGeom &g) {
   if (x->ndim < 1) return nxh_fail(NXH_INVALID_ARGUMENT, op, "input must not be a scalar");
   if (x->ndim - 1 > ROW_MAXD) return nxh_fail(NXH_FAILURE, op, "more than 8 outer dimensions");
-  if (x->shape[x->ndim - 1] > 64 * 4 * EPL) return nxh_fail(NXH_FAILURE, op, "rows longer than 8192 elements");
+  if (x->shape[x->ndim - 1] > ROW_MAX) return nxh_fail(NXH_FAILURE, op, "rows longer than 2^24 elements");
   g.n = (int)x->shape[x->ndim - 1];
   g.nouter = x->ndim - 1;
   g.rows = 1;
@@ -474,6 +620,12 @@ inline int lane_share(int n, bool wave) {
 }
 template <int DTX, int DTO>
 void softmax_launch(nxh_context *ctx, const SoftmaxArgs &a, bool vec) {
+  if (a.g.n > ROW_REGS) {
+    const dim3 grid((unsigned)std::min<int64_t>(a.g.rows, ctx->compute_units > 0 ? ctx->compute_units : 256));
+    if (vec) hipLaunchKernelGGL((softmax_long_kernel<DTX, DTO, 4>), grid, dim3(LONG_THREADS), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((softmax_long_kernel<DTX, DTO, 1>), grid, dim3(LONG_THREADS), 0, ctx->stream, a);
+    return;
+  }
   const bool wave = a.g.n <= 64 * EPL;
   const dim3 grid((unsigned)(wave ? (a.g.rows + 3) / 4 : a.g.rows));
   const int ep = lane_share(a.g.n, wave);
@@ -489,6 +641,12 @@ void softmax_launch(nxh_context *ctx, const SoftmaxArgs &a, bool vec) {
 }
 template <int DT>
 void layer_norm_launch(nxh_context *ctx, const LayerNormArgs &a, bool vec) {
+  if (a.g.n > ROW_REGS) {
+    const dim3 grid((unsigned)std::min<int64_t>(a.g.rows, ctx->compute_units > 0 ? ctx->compute_units : 256));
+    if (vec) hipLaunchKernelGGL((layer_norm_long_kernel<DT, 4>), grid, dim3(LONG_THREADS), 0, ctx->stream, a);
+    else hipLaunchKernelGGL((layer_norm_long_kernel<DT, 1>), grid, dim3(LONG_THREADS), 0, ctx->stream, a);
+    return;
+  }
   const bool wave = a.g.n <= 64 * EPL;
   const dim3 grid((unsigned)(wave ? (a.g.rows + 3) / 4 : a.g.rows));
   const int ep = lane_share(a.g.n, wave);
@@ -549,7 +707,7 @@ NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const n
                    (!mask || a.mask_last == 0 || rows_vector_ok(mask, 4));
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
-  nxh_set_path("softmax_rows");
+  nxh_set_path(a.g.n > ROW_REGS ? "softmax_rows_long" : "softmax_rows");
   {
     const nxh_tensor *ts[3] = {out, x, mask};
     const void *base[3];
@@ -617,7 +775,7 @@ NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, cons
                    (!gamma || ((uintptr_t)a.gamma % (es * 4)) == 0) && (!beta || ((uintptr_t)a.beta % (es * 4)) == 0);
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
-  nxh_set_path("layer_norm_rows");
+  nxh_set_path(a.g.n > ROW_REGS ? "layer_norm_rows_long" : "layer_norm_rows");
   if (dx == NXH_F32) layer_norm_launch<NXH_F32>(ctx, a, vec);
   else if (dx == NXH_BF16) layer_norm_launch<NXH_BF16>(ctx, a, vec);
   else if (dx == NXH_F16) layer_norm_launch<NXH_F16>(ctx, a, vec);

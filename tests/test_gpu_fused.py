@@ -41,7 +41,7 @@ def softmax_sequence(B, x, scale, mask, out_dtype):
 
 
 @pytest.mark.parametrize("d", FLOATS, ids=lambda d: d.name)
-@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (5, 770), (3, 2050), (2, 4100), (1, 8192), (4, 1)],
+@pytest.mark.parametrize("shape", [(2, 3, 64, 64), (5, 770), (3, 2050), (2, 4100), (1, 8192), (4, 1), (3, 8196), (2, 50257)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_softmax_rows_matches_the_sequence(hip, oracle, d, shape):
     rng = np.random.default_rng(sum(shape) + d.tag)
@@ -57,7 +57,7 @@ def test_softmax_rows_matches_the_sequence(hip, oracle, d, shape):
             hm, om = (B.expand(B.reshape(B.from_host(tri, dt.bool_), (1,) * (len(shape) - 2) + tri.shape), shape)
                       for B in (hip, oracle))
         got = hip.softmax_rows(hx, scale, hm, float("-inf") if masked else None, cast)
-        assert hip.last_path() == "softmax_rows"
+        assert hip.last_path() == ("softmax_rows_long" if shape[-1] > 8192 else "softmax_rows")
         od = cast or d
         want_cpu = logical(softmax_sequence(oracle, ox, scale, om, cast))
         want_gpu = logical(softmax_sequence(hip, hx, scale, hm, cast))
@@ -96,8 +96,9 @@ def test_softmax_rows_special_values_and_errors(hip, oracle):
     want = logical(nx.softmax(nx.where(om, nx.mul_s(ox, 2.0), nx.scalar_like(ox, -1e4))))
     assert np.array_equal(np.isnan(got), np.isnan(want))
     assert np.allclose(got[~np.isnan(got)], want[~np.isnan(want)], rtol=1e-6)
-    with pytest.raises(RuntimeError, match="8192"):
-        hip.softmax_rows(hip.full(dt.float32, (2, 8200), 0.0))
+    # a row that no block holds in registers: walked three times, same result
+    long_ = logical(hip.softmax_rows(hip.full(dt.float32, (2, 8200), 0.0)))
+    assert hip.last_path() == "softmax_rows_long" and np.array_equal(long_, np.full((2, 8200), np.float32(1) / np.float32(8200)))
     with pytest.raises(RuntimeError, match="contiguous"):
         hip.softmax_rows(hip.permute(hx, (1, 0)))
     with pytest.raises(RuntimeError):
@@ -112,7 +113,7 @@ def test_softmax_rows_special_values_and_errors(hip, oracle):
 
 
 @pytest.mark.parametrize("d", FLOATS, ids=lambda d: d.name)
-@pytest.mark.parametrize("shape", [(4, 33, 768), (7, 770), (3, 4100), (5, 1)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(4, 33, 768), (7, 770), (3, 4100), (5, 1), (3, 8196), (2, 50257)], ids=lambda s: "x".join(map(str, s)))
 def test_layer_norm_rows_matches_the_sequence(hip, oracle, d, shape):
     rng = np.random.default_rng(sum(shape) + 7 * d.tag)
     n = shape[-1]
@@ -124,14 +125,16 @@ def test_layer_norm_rows_matches_the_sequence(hip, oracle, d, shape):
     hb, ob = pair(beta, d, hip, oracle)
     eps = 1e-5
     got = hip.layer_norm_rows(hx, hg, hb, eps)
-    assert hip.last_path() == "layer_norm_rows"
+    assert hip.last_path() == ("layer_norm_rows_long" if n > 8192 else "layer_norm_rows")
     cfg = Config()
     want_cpu = logical(Gpt2(Nx(oracle), cfg).layer_norm(LayerNorm(og, ob), ox, eps))
     want_gpu = logical(Gpt2(Nx(hip), cfg).layer_norm(LayerNorm(hg, hb), hx, eps))
     what = f"{d.name} {shape}"
     # the mean and variance carry the sum-order difference into every element:
     # a few ulp of float32 in the statistics, at most one rounding step of d
-    close(logical(got), want_gpu, d, oracle, 2 * ULP[d.name] + 1e-5, 1e-5, what + " vs GPU sequence")
+    # (where y * gamma and beta nearly cancel, the one rounding step is one of y * gamma's size)
+    step = ULP[d.name] * float(np.abs(decode(beta, d, oracle)).max())
+    close(logical(got), want_gpu, d, oracle, 2 * ULP[d.name] + 1e-5, 1e-5 + step, what + " vs GPU sequence")
     close(logical(got), want_cpu, d, oracle, TOL[d.name][0], TOL[d.name][0], what + " vs oracle sequence")
     if d in (dt.bfloat16, dt.float16) and n > 1:
         frac = np.mean(logical(got) == want_gpu)
@@ -152,8 +155,9 @@ def test_layer_norm_rows_errors(hip):
         hip.layer_norm_rows(x, None, None, -1.0)
     with pytest.raises(RuntimeError):
         hip.layer_norm_rows(x, hip.full(dt.float64, (8,), 1.0), None, 1e-5)
-    with pytest.raises(RuntimeError, match="8192"):
-        hip.layer_norm_rows(hip.full(dt.float32, (1, 9000), 1.0), None, None, 1e-5)
+    assert np.array_equal(logical(hip.layer_norm_rows(hip.full(dt.float32, (1, 9000), 1.0), None, None, 1e-5)),
+                          np.zeros((1, 9000), np.float32))
+    assert hip.last_path() == "layer_norm_rows_long"
     # a constant row has zero variance: 0 / sqrt(eps) = 0
     assert np.array_equal(logical(hip.layer_norm_rows(x, None, None, 1e-5)), np.zeros((4, 8), np.float32))
 

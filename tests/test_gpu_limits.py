@@ -1,5 +1,5 @@
 """The limits this backend has and the reference does not (sort axis 2^30, transform length
-2^26 / 2^25, eigh / svd 4096 rows, eig 2048, fused rows 8192): each one refused with its
+2^26 / 2^25, eigh / svd 4096 rows, eig 2048): each one refused with its
 message one step beyond it, before anything is launched, and the cheap ones exercised
 exactly at it. Results at the limit are checked through closed forms (a shifted impulse's
 spectrum, the counts of a sorted byte array), not against the oracle, whose run times at
@@ -69,11 +69,11 @@ def test_factorisations_refuse_what_they_cannot_hold(hip):
     hip.trim()
 
 
-@pytest.mark.parametrize("row", [8192, 8193])
-def test_fused_rows_at_and_beyond_8192(hip, row):
-    """softmax over rows of 8192 elements is one fused kernel; one element more and the recorded
-    primitives are issued as they were recorded. Both equal the eager sequence's row sums and
-    agree with it within the sum's reassociation."""
+@pytest.mark.parametrize("row", [8192, 8193, 50257])
+def test_fused_rows_at_and_beyond_what_a_block_holds(hip, row):
+    """softmax over rows of 8192 elements is one fused kernel with the row in registers; a longer
+    row is still one fused kernel, which walks it three times. Both agree with the eager sequence
+    within the sum's reassociation."""
     rng = np.random.default_rng(row)
     nx = Nx(hip)
     x = hip.reshape(hip.from_host(rng.standard_normal((24, row)).astype(np.float32), dt.float32), (24, row))
@@ -86,9 +86,6 @@ def test_fused_rows_at_and_beyond_8192(hip, row):
     finally:
         hip.set_deferred(False)
     s = {k: after[k] - before[k] for k in after}
-    if row <= 8192:
-        assert s["softmax_rows"] == 1 and s["issued"] == 0, s
-        assert np.allclose(got, eager, rtol=2e-6, atol=1e-9)
-    else:
-        assert s["softmax_rows"] == 0 and s["issued"] == 5, s
-        same_bits(got, eager, "issued as recorded: the eager bits")
+    assert s["softmax_rows"] == 1 and s["issued"] == 0, s
+    assert np.allclose(got, eager, rtol=4e-6, atol=1e-9)
+    assert np.allclose(got.sum(-1), 1.0, atol=1e-5)
