@@ -133,6 +133,7 @@ class Workloads:
         ]
         ops[5].name = "cfg2 i32 cmplt(broadcast b, permuted a)"
         self.cfg2_out = {"v": v, "w": w, "m": m}
+        self.cfg2_in = {"a": a, "ai": ai}
         return ops
 
     # -- config 1: the CPU-runnable chain --------------------------------------
@@ -928,6 +929,40 @@ def check_config5(work, heads):
     return ok, out
 
 
+def host_buffer_step(hip, steps, warmup):
+    """The headline step as a caller with host buffers sees it: per step the two 64 MiB operands go up
+    (nxh_memcpy_h2d from pageable numpy arrays, staged through the library's pinned slots), the seven
+    calls run, and the f16, bool and int32 results come back (nxh_memcpy_d2h). GB/s over the same
+    algorithmic bytes as the headline, so the two figures compare directly."""
+    W = Workloads(hip)
+    ops = W.config2()
+    step_bytes = sum(o.nbytes for o in ops)
+    lib, h = hip._lib, hip._h
+    ups = [(t.buffer.ptr, np.ascontiguousarray(hip.to_host(t))) for t in W.cfg2_in.values()]
+    downs = [(t.buffer.ptr, np.empty(t.buffer.nbytes, np.uint8)) for t in W.cfg2_out.values()]
+    moved = sum(x.nbytes for _, x in ups) + sum(x.nbytes for _, x in downs)
+
+    def step():
+        for ptr, host in ups:
+            hip._check(lib.nxh_memcpy_h2d(h, ptr, host.ctypes.data, host.nbytes))
+        for op in ops:
+            op()
+        for ptr, host in downs:
+            hip._check(lib.nxh_memcpy_d2h(h, host.ctypes.data, ptr, host.nbytes))
+
+    for _ in range(warmup):
+        step()
+    hip.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    hip.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {"ms_per_step": round(ms, 3), "GBs_over_algorithmic_bytes": round(step_bytes / ms / 1e6, 1),
+            "bytes_over_pcie_per_step": moved, "pcie_GBs": round(moved / ms / 1e6, 1),
+            "algorithmic_bytes_per_step": step_bytes, "steps": steps}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -950,6 +985,9 @@ def main():
     ap.add_argument("--study-skip-vendor", action="store_true",
                     help="--gemm-study without the vendor rows (for counter runs: run --gemm-study-vendor as a command of its own)")
     ap.add_argument("--study-seconds", type=float, default=1.5, help="length of each timed loop of --gemm-study")
+    ap.add_argument("--host-buffers", action="store_true",
+                    help="the headline step with its two large operands uploaded from host memory and its three "
+                         "results read back inside the timed region (the PCIe-inclusive rate; never the headline)")
     ap.add_argument("--cpu-configs", action="store_true",
                     help="time the CPU oracle on bounded samples of configurations 1, 3, 4, 5 and print the records")
     args = ap.parse_args()
@@ -976,6 +1014,9 @@ def main():
         return
     if args.gemm_study:
         print(json.dumps({"gemm_study": gemm_study(hip, args.study_seconds, vendor=not args.study_skip_vendor)}))
+        return
+    if args.host_buffers:
+        print(json.dumps({"host_buffers": host_buffer_step(hip, args.steps, args.warmup)}))
         return
     if args.only_config:
         # one configuration's operations, each timed alone (for profiling runs)

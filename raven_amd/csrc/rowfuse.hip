@@ -23,6 +23,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 #include "fold_common.hpp"
@@ -319,75 +320,89 @@ __global__ __launch_bounds__(LONG_THREADS) void softmax_long_kernel(SoftmaxArgs 
   using SO = typename TO::S;
   __shared__ C lds[LONG_WAVES];
   for (int64_t row = blockIdx.x; row < a.g.rows; row += gridDim.x) {
-  int64_t oo, mo;
-  const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.mask, oo, mo);
-  const SX *x = reinterpret_cast<const SX *>(a.x.base) + xo;
-  SO *out = reinterpret_cast<SO *>(const_cast<char *>(a.out.base)) + oo;
-  const uint8_t *mask = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
-  const int nvec = a.g.n / V;
-  const C scale = (C)a.scale, masked = (C)a.masked;
-  constexpr bool SHORT = DTX == NXH_F32 && (DTO == NXH_BF16 || DTO == NXH_F16);
-  // the scaled, masked scores of vector c
-  auto scores = [&](int c, C(&e)[V]) {
-    const Pk<SX, V> raw = *reinterpret_cast<const Pk<SX, V> *>(x + (int64_t)c * V);
-    Pk<uint8_t, V> mk;
-    if (a.has_mask) {
-      if (a.mask_last) mk = *reinterpret_cast<const Pk<uint8_t, V> *>(mask + (int64_t)c * V);
-      else
+    int64_t oo, mo;
+    const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.mask, oo, mo);
+    const SX *x = reinterpret_cast<const SX *>(a.x.base) + xo;
+    SO *out = reinterpret_cast<SO *>(const_cast<char *>(a.out.base)) + oo;
+    const uint8_t *mask = reinterpret_cast<const uint8_t *>(a.mask.base) + mo;
+    // A row that starts off a vector boundary, or ends off one: `head` single elements, whole
+    // vectors, then the rest as single elements (the host has checked that out and mask are
+    // off their boundaries by as much as x). The single elements go one to a lane.
+    const int off = V > 1 ? (V - (int)(((uintptr_t)x / sizeof(SX)) % V)) % V : 0;
+    const int head = off < a.g.n ? off : a.g.n;
+    const int nvec = (a.g.n - head) / V;
+    const int nedge = a.g.n - nvec * V;
+    const C scale = (C)a.scale, masked = (C)a.masked;
+    constexpr bool SHORT = DTX == NXH_F32 && (DTO == NXH_BF16 || DTO == NXH_F16);
+    // the scaled, masked scores of the W elements from i on
+    auto scores = [&](int64_t i, auto w, C *e) {
+      constexpr int W = decltype(w)::value;
+      const Pk<SX, W> raw = *reinterpret_cast<const Pk<SX, W> *>(x + i);
+      Pk<uint8_t, W> mk;
+      if (a.has_mask) {
+        if (a.mask_last) mk = *reinterpret_cast<const Pk<uint8_t, W> *>(mask + i);
+        else
 #pragma unroll
-        for (int j = 0; j < V; j++) mk.v[j] = mask[0];
-    }
+          for (int j = 0; j < W; j++) mk.v[j] = mask[0];
+      }
 #pragma unroll
-    for (int j = 0; j < V; j++) {
-      C v = TX::ld(raw.v[j]);
-      if (a.has_scale) v = rnd<DTX>(OpMul::eval<CAT_FLOAT, C>(v, scale));
-      if (a.has_mask) v = mk.v[j] != 0 ? v : masked;
-      e[j] = v;
-    }
-  };
-  C m = Combine<NXH_RMAX, C, CAT_FLOAT>::init();
+      for (int j = 0; j < W; j++) {
+        C v = TX::ld(raw.v[j]);
+        if (a.has_scale) v = rnd<DTX>(OpMul::eval<CAT_FLOAT, C>(v, scale));
+        if (a.has_mask) v = mk.v[j] != 0 ? v : masked;
+        e[j] = v;
+      }
+    };
+    // body(i, W): once for every vector of the row and once for every single element
+    auto walk = [&](auto &&body) {
 #pragma unroll 8
-  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
-    C e[V];
-    scores(c, e);
+      for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) body(head + (int64_t)c * V, std::integral_constant<int, V>{});
+      if (V > 1 && (int)threadIdx.x < nedge)
+        body((int)threadIdx.x < head ? (int64_t)threadIdx.x : (int64_t)nvec * V + threadIdx.x, std::integral_constant<int, 1>{});
+    };
+    C m = Combine<NXH_RMAX, C, CAT_FLOAT>::init();
+    walk([&](int64_t i, auto w) {
+      constexpr int W = decltype(w)::value;
+      C e[W];
+      scores(i, w, e);
 #pragma unroll
-    for (int j = 0; j < V; j++) {
-      if constexpr (SHORT) m = __builtin_fmaxf(m, e[j]);
-      else m = Combine<NXH_RMAX, C, CAT_FLOAT>::apply(m, e[j]);
-    }
-  }
-  m = row_combine<NXH_RMAX, C, LONG_WAVES>(m, lds);
-  auto exponential = [&](C v) -> C {
-    const C d = rnd<DTX>(OpSub::eval<CAT_FLOAT, C>(v, m));
-    if constexpr (SHORT) return exp_nonpositive(d);
-    else return rnd<DTX>(OpExp::eval<CAT_FLOAT, C>(d));
-  };
-  C s = 0;
-#pragma unroll 8
-  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
-    C e[V];
-    scores(c, e);
+      for (int j = 0; j < W; j++) {
+        if constexpr (SHORT) m = __builtin_fmaxf(m, e[j]);
+        else m = Combine<NXH_RMAX, C, CAT_FLOAT>::apply(m, e[j]);
+      }
+    });
+    m = row_combine<NXH_RMAX, C, LONG_WAVES>(m, lds);
+    auto exponential = [&](C v) -> C {
+      const C d = rnd<DTX>(OpSub::eval<CAT_FLOAT, C>(v, m));
+      if constexpr (SHORT) return exp_nonpositive(d);
+      else return rnd<DTX>(OpExp::eval<CAT_FLOAT, C>(d));
+    };
+    C s = 0;
+    walk([&](int64_t i, auto w) {
+      constexpr int W = decltype(w)::value;
+      C e[W];
+      scores(i, w, e);
 #pragma unroll
-    for (int j = 0; j < V; j++) s = s + exponential(e[j]);
-  }
-  s = rnd<DTX>(row_combine<NXH_SUM, C, LONG_WAVES>(s, lds));
-  C s_recip = 0;
-  if constexpr (SHORT) s_recip = 1.0f / s;
-#pragma unroll 8
-  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
-    C e[V];
-    scores(c, e);
-    Pk<SO, V> o;
+      for (int j = 0; j < W; j++) s = s + exponential(e[j]);
+    });
+    s = rnd<DTX>(row_combine<NXH_SUM, C, LONG_WAVES>(s, lds));
+    C s_recip = 0;
+    if constexpr (SHORT) s_recip = 1.0f / s;
+    walk([&](int64_t i, auto w) {
+      constexpr int W = decltype(w)::value;
+      C e[W];
+      scores(i, w, e);
+      Pk<SO, W> o;
 #pragma unroll
-    for (int j = 0; j < V; j++) {
-      const C t = exponential(e[j]);
-      C y;
-      if constexpr (SHORT) y = div_by_reciprocal(t, s, s_recip);
-      else y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t, s));
-      o.v[j] = TO::st((typename TO::C)y);
-    }
-    *reinterpret_cast<Pk<SO, V> *>(out + (int64_t)c * V) = o;
-  }
+      for (int j = 0; j < W; j++) {
+        const C t = exponential(e[j]);
+        C y;
+        if constexpr (SHORT) y = div_by_reciprocal(t, s, s_recip);
+        else y = rnd<DTX>(OpFdiv::eval<CAT_FLOAT, C>(t, s));
+        o.v[j] = TO::st((typename TO::C)y);
+      }
+      *reinterpret_cast<Pk<SO, W> *>(out + i) = o;
+    });
   }
 }
 
@@ -398,48 +413,71 @@ __global__ __launch_bounds__(LONG_THREADS) void layer_norm_long_kernel(LayerNorm
   using S = typename TX::S;
   __shared__ C lds[LONG_WAVES];
   for (int64_t row = blockIdx.x; row < a.g.rows; row += gridDim.x) {
-  int64_t oo, uo;
-  const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.unused, oo, uo);
-  const S *x = reinterpret_cast<const S *>(a.x.base) + xo;
-  S *out = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
-  const S *gamma = reinterpret_cast<const S *>(a.gamma), *beta = reinterpret_cast<const S *>(a.beta);
-  const int nvec = a.g.n / V;
-  const C count = (C)a.count, eps = (C)a.eps;
-  C s = 0;
+    int64_t oo, uo;
+    const int64_t xo = row_offsets(a.g, row, a.x, a.out, a.unused, oo, uo);
+    const S *x = reinterpret_cast<const S *>(a.x.base) + xo;
+    S *out = reinterpret_cast<S *>(const_cast<char *>(a.out.base)) + oo;
+    const S *gamma = reinterpret_cast<const S *>(a.gamma), *beta = reinterpret_cast<const S *>(a.beta);
+    // head, vectors, rest: as in softmax_long_kernel; gamma and beta, which every row shares, are
+    // read by vectors only from a row that is off its boundary by as much as they are
+    const int off = V > 1 ? (V - (int)(((uintptr_t)x / sizeof(S)) % V)) % V : 0;
+    const int head = off < a.g.n ? off : a.g.n;
+    const int nvec = (a.g.n - head) / V;
+    const int nedge = a.g.n - nvec * V;
+    const bool gvec = !gamma || ((uintptr_t)(gamma + head) / sizeof(S)) % V == 0;
+    const bool bvec = !beta || ((uintptr_t)(beta + head) / sizeof(S)) % V == 0;
+    const C count = (C)a.count, eps = (C)a.eps;
+    auto walk = [&](auto &&body) {
 #pragma unroll 8
-  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
-    const Pk<S, V> raw = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+      for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) body(head + (int64_t)c * V, std::integral_constant<int, V>{});
+      if (V > 1 && (int)threadIdx.x < nedge)
+        body((int)threadIdx.x < head ? (int64_t)threadIdx.x : (int64_t)nvec * V + threadIdx.x, std::integral_constant<int, 1>{});
+    };
+    C s = 0;
+    walk([&](int64_t i, auto w) {
+      constexpr int W = decltype(w)::value;
+      const Pk<S, W> raw = *reinterpret_cast<const Pk<S, W> *>(x + i);
 #pragma unroll
-    for (int j = 0; j < V; j++) s = s + TX::ld(raw.v[j]);
-  }
-  const C mu = row_combine<NXH_SUM, C, LONG_WAVES>(s, lds) / count;
-  s = 0;
-#pragma unroll 8
-  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
-    const Pk<S, V> raw = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
+      for (int j = 0; j < W; j++) s = s + TX::ld(raw.v[j]);
+    });
+    const C mu = row_combine<NXH_SUM, C, LONG_WAVES>(s, lds) / count;
+    s = 0;
+    walk([&](int64_t i, auto w) {
+      constexpr int W = decltype(w)::value;
+      const Pk<S, W> raw = *reinterpret_cast<const Pk<S, W> *>(x + i);
 #pragma unroll
-    for (int j = 0; j < V; j++) {
-      const C t = TX::ld(raw.v[j]) - mu;
-      s = s + t * t;
-    }
-  }
-  const C var = row_combine<NXH_SUM, C, LONG_WAVES>(s, lds) / count;
-  const C r = m_sqrt(var + eps);
-#pragma unroll 8
-  for (int c = threadIdx.x; c < nvec; c += LONG_THREADS) {
-    const Pk<S, V> raw = *reinterpret_cast<const Pk<S, V> *>(x + (int64_t)c * V);
-    Pk<S, V> gv, bv, o;
-    if (gamma) gv = *reinterpret_cast<const Pk<S, V> *>(gamma + (int64_t)c * V);
-    if (beta) bv = *reinterpret_cast<const Pk<S, V> *>(beta + (int64_t)c * V);
+      for (int j = 0; j < W; j++) {
+        const C t = TX::ld(raw.v[j]) - mu;
+        s = s + t * t;
+      }
+    });
+    const C var = row_combine<NXH_SUM, C, LONG_WAVES>(s, lds) / count;
+    const C r = m_sqrt(var + eps);
+    walk([&](int64_t i, auto w) {
+      constexpr int W = decltype(w)::value;
+      const Pk<S, W> raw = *reinterpret_cast<const Pk<S, W> *>(x + i);
+      Pk<S, W> gv, bv, o;
+      if (gamma) {
+        if (W == 1 || gvec) gv = *reinterpret_cast<const Pk<S, W> *>(gamma + i);
+        else
 #pragma unroll
-    for (int j = 0; j < V; j++) {
-      C y = rnd<DT>((TX::ld(raw.v[j]) - mu) / r);  // leaves the float32 island here
-      if (gamma) y = rnd<DT>(y * TX::ld(gv.v[j]));
-      if (beta) y = rnd<DT>(y + TX::ld(bv.v[j]));
-      o.v[j] = TX::st(y);
-    }
-    *reinterpret_cast<Pk<S, V> *>(out + (int64_t)c * V) = o;
-  }
+          for (int j = 0; j < W; j++) gv.v[j] = gamma[i + j];
+      }
+      if (beta) {
+        if (W == 1 || bvec) bv = *reinterpret_cast<const Pk<S, W> *>(beta + i);
+        else
+#pragma unroll
+          for (int j = 0; j < W; j++) bv.v[j] = beta[i + j];
+      }
+#pragma unroll
+      for (int j = 0; j < W; j++) {
+        C y = rnd<DT>((TX::ld(raw.v[j]) - mu) / r);  // leaves the float32 island here
+        if (gamma) y = rnd<DT>(y * TX::ld(gv.v[j]));
+        if (beta) y = rnd<DT>(y + TX::ld(bv.v[j]));
+        o.v[j] = TX::st(y);
+      }
+      *reinterpret_cast<Pk<S, W> *>(out + i) = o;
+    });
   }
 }
 
@@ -601,6 +639,17 @@ bool rows_vector_ok(const nxh_tensor *t, int v) {
     if (t->shape[d] > 1 && t->strides[d] % v != 0) return false;
   return true;
 }
+// Rows of a and b are off their V-element boundaries by the same amount, row by row: the
+// long-row kernels then peel the same head and tail from both.
+bool rows_congruent(const nxh_tensor *a, const nxh_tensor *b, int v) {
+  const uintptr_t ea = (uintptr_t)a->data / nxh_elem_size(a->dtype) + (uintptr_t)a->offset;
+  const uintptr_t eb = (uintptr_t)b->data / nxh_elem_size(b->dtype) + (uintptr_t)b->offset;
+  if ((uintptr_t)a->data % nxh_elem_size(a->dtype) || (uintptr_t)b->data % nxh_elem_size(b->dtype)) return false;
+  if (ea % v != eb % v) return false;
+  for (int d = 0; d < a->ndim - 1; d++)
+    if (a->shape[d] > 1 && ((a->strides[d] - b->strides[d]) % v) != 0) return false;
+  return true;
+}
 int same_shape(const char *op, const nxh_tensor *a, const nxh_tensor *b) {
   if (a->ndim != b->ndim) return nxh_fail(NXH_INVALID_ARGUMENT, op, NXH_ERR_SHAPE);
   for (int d = 0; d < a->ndim; d++)
@@ -703,8 +752,10 @@ NXH_EXPORT int nxh_softmax_rows(nxh_context *ctx, const nxh_tensor *out, const n
   a.mask_last = mask ? mask->strides[nd - 1] : 0;
   a.scale = scale ? decode_scalar(dx, scale) : 1.0;
   a.masked = mask ? decode_scalar(dx, masked_value) : 0.0;
-  const bool vec = a.g.n % 4 == 0 && rows_vector_ok(x, 4) && rows_vector_ok(out, 4) &&
-                   (!mask || a.mask_last == 0 || rows_vector_ok(mask, 4));
+  const bool vec = a.g.n > ROW_REGS
+                       ? rows_congruent(x, out, 4) && (!mask || a.mask_last == 0 || rows_congruent(x, mask, 4))
+                       : a.g.n % 4 == 0 && rows_vector_ok(x, 4) && rows_vector_ok(out, 4) &&
+                             (!mask || a.mask_last == 0 || rows_vector_ok(mask, 4));
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path(a.g.n > ROW_REGS ? "softmax_rows_long" : "softmax_rows");
@@ -771,8 +822,10 @@ NXH_EXPORT int nxh_layer_norm_rows(nxh_context *ctx, const nxh_tensor *out, cons
   // filled into the statistics dtype (float32 for 16-bit inputs)
   a.eps = dx == NXH_F64 ? eps : (double)(float)eps;
   a.count = dx == NXH_F64 ? (double)a.g.n : (double)(float)a.g.n;
-  const bool vec = a.g.n % 4 == 0 && rows_vector_ok(x, 4) && rows_vector_ok(out, 4) &&
-                   (!gamma || ((uintptr_t)a.gamma % (es * 4)) == 0) && (!beta || ((uintptr_t)a.beta % (es * 4)) == 0);
+  const bool vec = a.g.n > ROW_REGS
+                       ? rows_congruent(x, out, 4)
+                       : a.g.n % 4 == 0 && rows_vector_ok(x, 4) && rows_vector_ok(out, 4) &&
+                             (!gamma || ((uintptr_t)a.gamma % (es * 4)) == 0) && (!beta || ((uintptr_t)a.beta % (es * 4)) == 0);
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   nxh_set_path(a.g.n > ROW_REGS ? "layer_norm_rows_long" : "layer_norm_rows");
