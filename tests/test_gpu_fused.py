@@ -68,6 +68,32 @@ def test_softmax_rows_matches_the_sequence(hip, oracle, d, shape):
         assert np.all(np.abs(rows - 1) <= 8 * shape[-1] ** 0.5 * ULP[od.name] + 1e-6)
 
 
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16], ids=lambda d: d.name)
+@pytest.mark.parametrize("start, width", [(0, 8201), (1, 8199), (2, 8205), (3, 9000), (1, 8193), (4, 8203), (0, 9011)])
+def test_long_rows_off_their_vector_boundaries(hip, oracle, d, start, width):
+    """Rows of a window [3, start:start+width] of a [3, 9011] matrix start off a 4-element boundary by
+    a different amount each (9011 is odd). Where the fresh result's rows are off by the same amounts
+    (start = 4, width = 8203: both row pitches are 3 modulo 4) the long-row kernels move vectors and
+    take head and tail one element to a lane; the other windows move single elements. Both must
+    agree with the result on a contiguous copy of the window within the reassociation of a row's
+    sum."""
+    rng = np.random.default_rng(start * 10007 + width + d.tag)
+    wide = encode(rng.standard_normal((3, 9011)) * 2, d, oracle)
+    gamma = encode(rng.standard_normal(width) * 0.5 + 1, d, oracle)
+    beta = encode(rng.standard_normal(width) * 0.1, d, oracle)
+    hw = hip.reshape(hip.from_host(wide, d), (3, 9011))
+    view = hip.shrink(hw, [(0, 3), (start, start + width)])
+    flat = hip.reshape(hip.from_host(np.ascontiguousarray(wide[:, start:start + width]), d), (3, width))
+    got, want = hip.softmax_rows(view), hip.softmax_rows(flat)
+    assert hip.last_path() == "softmax_rows_long"
+    within_ulps(logical(got), logical(want), d, oracle, 4 if d.itemsize == 2 else 16, f"softmax {d.name} {start}+{width}")
+    hg, hb = hip.from_host(gamma, d), hip.from_host(beta, d)
+    got, want = hip.layer_norm_rows(view, hg, hb, 1e-5), hip.layer_norm_rows(flat, hg, hb, 1e-5)
+    assert hip.last_path() == "layer_norm_rows_long"
+    step = ULP[d.name] * float(np.abs(decode(beta, d, oracle)).max())
+    close(logical(got), logical(want), d, oracle, 2 * ULP[d.name] + 1e-5, 1e-5 + step, f"layer norm {d.name} {start}+{width}")
+
+
 def test_softmax_rows_special_values_and_errors(hip, oracle):
     x = np.zeros((6, 8), np.float32)
     x[0] = np.arange(8)
