@@ -262,7 +262,14 @@ constexpr bool scan_cols_ok() {
          ((TR::cat == CAT_FLOAT && std::is_same<typename TR::C, float>::value) || TR::cat == CAT_SINT || TR::cat == CAT_UINT);
 }
 
-template <int DT, class CB, bool VEC, int SC_WAVES>
+// ORDERED (float sums and products, whose result depends on how the additions are nested): the
+// way up takes a fixed shape instead of whatever is there first. Every SC_WIN-th chunk is an
+// anchor; only anchors publish the PRE form; a lane takes the AGG words of the chunks down to
+// the nearest anchor below it and that anchor's PRE word, for which it waits. The value a chunk
+// starts from is then P(anchor) + (a + (b + ...)) over the chunks in between, the same nesting
+// on every run. The other operations are exact and associative, any mix of words gives the
+// same bits, and they keep taking what is there.
+template <int DT, class CB, bool VEC, int SC_WAVES, bool ORDERED>
 __global__ __launch_bounds__(64 * SC_WAVES) void scan_cols_kernel(ScanColsArgs a) {
   constexpr int SC_ROWS = SC_RW * SC_WAVES;
   static_assert(64 * SC_WAVES >= SC_COLS, "a lane per column in the hand-over");
@@ -340,11 +347,12 @@ __global__ __launch_bounds__(64 * SC_WAVES) void scan_cols_kernel(ScanColsArgs a
         for (int k = 0; k < SC_WIN; k++) {
           if (k >= n || done || took != k) continue;
           const uint32_t f = (uint32_t)(word[k] >> 32);
-          if (f != f_agg && f != f_pre) continue;
+          const bool anchor = ((c - k) % SC_WIN) == 0;
+          if (ORDERED ? f != (anchor ? f_pre : f_agg) : (f != f_agg && f != f_pre)) continue;
           const C val = sc_unpack<TR>((uint32_t)word[k]);
           ex = have ? CB::apply(val, ex) : val;  // the earlier rows on the left
           have = true;
-          done = f == f_pre;
+          done = ORDERED ? anchor : f == f_pre;
           took = k + 1;
         }
         c -= took;
@@ -367,7 +375,8 @@ __global__ __launch_bounds__(64 * SC_WAVES) void scan_cols_kernel(ScanColsArgs a
       }
     }
     const C incl = chunk > 0 ? CB::apply(ex, agg) : agg;
-    __hip_atomic_store(mine, ((uint64_t)f_pre << 32) | sc_pack<TR>(incl), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!ORDERED || chunk % SC_WIN == 0)
+      __hip_atomic_store(mine, ((uint64_t)f_pre << 32) | sc_pack<TR>(incl), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     pre[cme] = ex;
   }
   __syncthreads();
@@ -522,10 +531,11 @@ static int scan_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
         const uintptr_t al = (uintptr_t)(SC_V * sizeof(S)) - 1;
         const bool vec = !(((uintptr_t)a.in | (uintptr_t)a.out) & al) && a.in_step % SC_V == 0 && a.out_step % SC_V == 0;
         nxh_set_path("scan_cols");
+        constexpr bool ORD = TR::cat == CAT_FLOAT && (OP == NXH_SUM || OP == NXH_PROD);
 #define NXH_SCAN_COLS(WAVES)                                                                                         \
   do {                                                                                                               \
-    if (vec) hipLaunchKernelGGL((scan_cols_kernel<DT, CB, true, WAVES>), dim3(nblocks), dim3(64 * WAVES), 0, ctx->stream, c); \
-    else hipLaunchKernelGGL((scan_cols_kernel<DT, CB, false, WAVES>), dim3(nblocks), dim3(64 * WAVES), 0, ctx->stream, c);    \
+    if (vec) hipLaunchKernelGGL((scan_cols_kernel<DT, CB, true, WAVES, ORD>), dim3(nblocks), dim3(64 * WAVES), 0, ctx->stream, c); \
+    else hipLaunchKernelGGL((scan_cols_kernel<DT, CB, false, WAVES, ORD>), dim3(nblocks), dim3(64 * WAVES), 0, ctx->stream, c);    \
   } while (0)
         if (waves == 4) NXH_SCAN_COLS(4);
         else if (waves == 8) NXH_SCAN_COLS(8);

@@ -239,3 +239,59 @@ def test_random_shapes_views_and_ops(hip, oracle):
             close(g, w, d, oracle, tol, tol * (rows if op == "sum" else 1.0), what)
         else:
             same_bits(g, w, what)
+
+
+def nested_as_the_kernel_nests(x):
+    """float32 cumsum down the rows with every addition in the order the single-pass kernel fixes for
+    float sums: sixteen rows per wave added one after the other, the waves' totals left to right,
+    and across blocks the totals of the chunks above nested from the nearest one up, ending at the
+    nearest sixteenth chunk's published prefix."""
+    f = np.float32
+    rows = x.shape[0]
+    waves = 16 if rows >= 512 else 8 if rows >= 256 else 4
+    per_block, out = 16 * waves, np.empty_like(x)
+    aggs, prefix = [], {}
+    for k in range((rows + per_block - 1) // per_block):
+        blk = x[k * per_block:(k + 1) * per_block]
+        tots, runs = [], []
+        for w in range(waves):
+            run, seg = np.zeros(x.shape[1], f), []
+            for row in blk[w * 16:(w + 1) * 16]:
+                run = (run + row).astype(f)
+                seg.append(run)
+            tots.append(run)
+            runs.append(seg)
+        agg = tots[0]
+        for t in tots[1:]:
+            agg = (agg + t).astype(f)
+        ex = None
+        if k > 0:
+            anchor = (k - 1) - (k - 1) % 16
+            for c in range(k - 1, anchor - 1, -1):
+                val = prefix[c] if c == anchor else aggs[c]
+                ex = val if ex is None else (val + ex).astype(f)
+        if k % 16 == 0:
+            prefix[k] = (ex + agg).astype(f) if k > 0 else agg
+        aggs.append(agg)
+        for w in range(waves):
+            base = ex
+            for t in tots[:w]:
+                base = t if base is None else (base + t).astype(f)
+            for r, run in enumerate(runs[w]):
+                out[k * per_block + w * 16 + r] = run if base is None else (base + run).astype(f)
+    return out
+
+
+@pytest.mark.parametrize("rows, cols", [(8967, 260), (4096, 512), (700, 300)])
+def test_float_sums_nest_the_same_way_on_every_run(hip, rows, cols):
+    """A float sum's bits depend on how the additions are nested, and blocks finish in a different
+    order from run to run: the kernel nests the chunks above a block in one fixed way, so the
+    result equals that nesting evaluated on the host, bit for bit and on every one of ten runs."""
+    rng = np.random.default_rng(rows)
+    x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    h = hip.reshape(hip.from_host(x, dt.float32), (rows, cols))
+    want = nested_as_the_kernel_nests(x)
+    for run in range(10):
+        got = logical(hip.associative_scan(0, "sum", h))
+        assert hip.last_path() == "scan_cols"
+        same_bits(got, want, f"[{rows},{cols}] run {run}")
