@@ -93,6 +93,9 @@ struct nxh_context {
   // four constants each table was made with
   void *gelu_lut[2] = {nullptr, nullptr};
   double gelu_lut_c[2][4] = {};
+  // a recorded graph reads the table: it keeps its constants from then on (other constants take the arithmetic)
+  bool gelu_lut_recorded[2] = {false, false};
+  int graphs_alive = 0;  // recorded graphs not yet destroyed (the one being captured included)
   // The part of the bfloat16 table the fused linear's GELU epilogue keeps in LDS (rowfuse.hip,
   // nxh_gelu_epilogue_table): entries [lo, lo + n) of either sign, n*2 values on the device;
   // state 0 not made yet, 1 usable, -1 these constants have no usable form.
@@ -101,6 +104,7 @@ struct nxh_context {
     double c[4] = {};
     uint32_t lo = 0, n = 0;
     void *dev = nullptr;
+    bool recorded = false;  // a recorded graph reads dev: its contents stay
   } gelu_epi;
   unsigned char *scan_state = nullptr;
   size_t scan_state_bytes = 0;

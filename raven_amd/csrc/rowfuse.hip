@@ -850,7 +850,9 @@ static int gelu_full_table(nxh_context *ctx, const char *op, int slot, const dou
     *have = true;
   }
   if (*have && memcmp(ctx->gelu_lut_c[slot], c, 4 * sizeof(double)) != 0) {
-    if (ctx->capture) {  // a captured refill would run at every replay, behind the back of this record
+    // a captured refill would run at every replay, behind the back of this record; a refill
+    // outside a capture would change what an earlier record's launches read at their next replay
+    if (ctx->capture || ctx->gelu_lut_recorded[slot]) {
       *have = false;
       return NXH_OK;
     }
@@ -861,6 +863,7 @@ static int gelu_full_table(nxh_context *ctx, const char *op, int slot, const dou
     NXH_HIP(op, hipGetLastError());
     memcpy(ctx->gelu_lut_c[slot], c, 4 * sizeof(double));
   }
+  if (*have && ctx->capture) ctx->gelu_lut_recorded[slot] = true;
   return NXH_OK;
 }
 
@@ -875,6 +878,7 @@ int nxh_gelu_epilogue_table(nxh_context *ctx, const double *c, const void **tabl
   auto &e = ctx->gelu_epi;
   auto give = [&]() -> int {
     if (e.state <= 0) return 0;
+    if (ctx->capture) e.recorded = true;
     *table = e.dev;
     *lo = e.lo;
     *n = e.n;
@@ -882,6 +886,7 @@ int nxh_gelu_epilogue_table(nxh_context *ctx, const double *c, const void **tabl
   };
   if (e.state != 0 && memcmp(e.c, c, sizeof e.c) == 0) return give();
   if (ctx->capture) return 0;  // making it waits for the stream
+  if (e.recorded) return 0;    // a recorded graph reads the table made for other constants
   // The whole table and the closed form of its low end, read back once. The part kept in LDS is
   // [lo, hi): below lo every result must equal narrow(x * c3), from hi to the last finite binade
   // x itself (positive) or -0 (negative); both bounds fall on binades (multiples of 128).

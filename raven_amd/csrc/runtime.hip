@@ -543,6 +543,11 @@ static void graph_release(nxh_context *ctx, nxh_graph *gr) {
   for (auto it = ctx->graph_blocks.begin(); it != ctx->graph_blocks.end();)
     it = it->second == gr ? ctx->graph_blocks.erase(it) : std::next(it);
   delete gr;
+  if (--ctx->graphs_alive <= 0) {  // no record reads the GELU tables any more: they may take other constants
+    ctx->graphs_alive = 0;
+    ctx->gelu_lut_recorded[0] = ctx->gelu_lut_recorded[1] = false;
+    ctx->gelu_epi.recorded = false;
+  }
 }
 
 NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
@@ -554,9 +559,11 @@ NXH_EXPORT int nxh_capture_begin(nxh_context *ctx) {
   NXH_HIP("capture_begin", hipSetDevice(ctx->device));
   NXH_HIP("capture_begin", hipStreamSynchronize(ctx->stream));
   nxh_graph *gr = new nxh_graph();
+  ctx->graphs_alive++;
   hipError_t e = hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed);
   if (e != hipSuccess) {
     delete gr;
+    ctx->graphs_alive--;
     return nxh_hip_fail("capture_begin", e);
   }
   ctx->capture = gr;

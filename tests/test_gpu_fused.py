@@ -263,3 +263,52 @@ def test_gelu_tanh_by_table_holds_the_arithmetic_bits_of_every_input(hip, d):
     assert hip.last_path() == "gelu_tanh_table"
     assert np.array_equal(got.reshape(-1).view(np.uint16), want.view(np.uint16)[idx])
     graph.destroy()
+
+
+def test_a_recorded_gelu_keeps_its_table_when_other_constants_come_later(hip):
+    """A recorded graph reads the table that was there when it was captured. A later eager call with
+    other constants must not refill that table (it takes the arithmetic while the graph lives): the
+    graph's next replay still gives the results of its own constants. Once the graph is destroyed
+    the table takes the other constants again. The same for the table of the linear + GELU epilogue."""
+    d = dt.bfloat16
+    rng = np.random.default_rng(77)
+    pats = np.arange(65536, dtype=np.uint16)
+    idx = rng.integers(0, 65536, 1 << 22).astype(np.int64)
+    small = hip.reshape(hip.from_host(pats, d), (65536,))
+    big = hip.reshape(hip.from_host(pats[idx], d), (2048, 2048))
+    mine, other = (0.044715, 0.7978845608028654, 1.0, 0.5), (0.06, 0.7, 1.0, 0.5)
+    want = {c: logical(hip.gelu_tanh(small, c)).view(np.uint16)[idx] for c in (mine, other)}
+    n = 4 * 192
+    x = hip.reshape(hip.from_host(np.zeros(128 * 64, np.uint16), d), (128, 64))
+    w = hip.reshape(hip.from_host(np.zeros(64 * n, np.uint16), d), (64, n))
+    b = hip.reshape(hip.from_host(pats[idx[:n]], d), (n,))
+    want_lin = {c: logical(hip.gelu_tanh(hip.contiguous(hip.shrink(hip.linear(x, w, b), [(0, 1), (0, n)])), c)).view(np.uint16)
+                for c in (mine, other)}
+    hip.gelu_tanh(big, mine)  # the tables exist, made for `mine`
+    hip.linear_gelu_tanh(x, w, b, mine)
+    hip.capture_begin()
+    try:
+        out = hip.gelu_tanh(big, mine)
+        path = hip.last_path()
+        lin = hip.linear_gelu_tanh(x, w, b, mine)
+    finally:
+        graph = hip.capture_end()
+    assert path == "gelu_tanh_table"
+    try:
+        got = logical(hip.gelu_tanh(big, other))
+        assert hip.last_path() == "gelu_tanh"  # not by table: the graph's table stays
+        assert np.array_equal(got.reshape(-1).view(np.uint16), want[other])
+        got = logical(hip.linear_gelu_tanh(x, w, b, other)).view(np.uint16)
+        assert np.array_equal(got, np.broadcast_to(want_lin[other], got.shape))
+        for _ in range(2):
+            graph.launch()
+            hip.synchronize()
+            assert np.array_equal(logical(out).reshape(-1).view(np.uint16), want[mine])
+            assert np.array_equal(logical(lin).view(np.uint16), np.broadcast_to(want_lin[mine], got.shape))
+    finally:
+        graph.destroy()
+    got = logical(hip.gelu_tanh(big, other))
+    assert hip.last_path() == "gelu_tanh_table"
+    assert np.array_equal(got.reshape(-1).view(np.uint16), want[other])
+    got = logical(hip.linear_gelu_tanh(x, w, b, other)).view(np.uint16)
+    assert np.array_equal(got, np.broadcast_to(want_lin[other], got.shape))
