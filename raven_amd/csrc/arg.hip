@@ -199,16 +199,22 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
           if constexpr (CMP::category == CAT_FLOAT) odd |= v != v;
         }
     }
-    for (; r < r1; r += RG) {
-      FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
+    if (r < r1) {  // the rest, fewer than U rows of this group: requested together, taken in row order
+      FVec<T, V> x[U - 1];
 #pragma unroll
-      for (int k = 0; k < V; k++) {
-        const C v = IN::ld(x.v[k]);
-        const bool take = CMP::better(v, bv[k]);
-        bv[k] = take ? v : bv[k];
-        bi[k] = take ? (I)r : bi[k];
-        if constexpr (CMP::category == CAT_FLOAT) odd |= v != v;
-      }
+      for (int j = 0; j < U - 1; j++)
+        if (r + j * RG < r1) x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j * RG) * a.r_stride);
+#pragma unroll
+      for (int j = 0; j < U - 1; j++)
+        if (r + j * RG < r1)
+#pragma unroll
+          for (int k = 0; k < V; k++) {
+            const C v = IN::ld(x[j].v[k]);
+            const bool take = CMP::better(v, bv[k]);
+            bv[k] = take ? v : bv[k];
+            bi[k] = take ? (I)(r + j * RG) : bi[k];
+            if constexpr (CMP::category == CAT_FLOAT) odd |= v != v;
+          }
     }
     if (!odd) goto combine;
     r = r0 + rg;
@@ -231,13 +237,23 @@ __global__ __launch_bounds__(FOLD_THREADS) void arg_col_kernel(ArgArgs a) {
         else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x[j].v[k]), (I)(r + j * RG));
       }
   }
-  for (; r < r1; r += RG) {
-    FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
+  if (r < r1) {  // the rest of this group, requested together
+    FVec<T, V> x[U - 1];
+    int32_t xi[U - 1];
 #pragma unroll
-    for (int k = 0; k < V; k++) {
-      if (HAS_IDX) CMP::merge(bv[k], bi[k], IN::ld(x.v[k]), (I)a.in_idx[in_off + l + r * a.r_stride]);
-      else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x.v[k]), (I)r);
-    }
+    for (int j = 0; j < U - 1; j++)
+      if (r + j * RG < r1) {
+        x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j * RG) * a.r_stride);
+        if (HAS_IDX) xi[j] = a.in_idx[in_off + l + (r + j * RG) * a.r_stride];
+      }
+#pragma unroll
+    for (int j = 0; j < U - 1; j++)
+      if (r + j * RG < r1)
+#pragma unroll
+        for (int k = 0; k < V; k++) {
+          if (HAS_IDX) CMP::merge(bv[k], bi[k], IN::ld(x[j].v[k]), (I)xi[j]);
+          else arg_take<CMP, C>(bv[k], bi[k], IN::ld(x[j].v[k]), (I)(r + j * RG));
+        }
   }
 combine:
   if constexpr (RG > 1) {
@@ -349,11 +365,15 @@ static int arg_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, co
         b.r_stride = g.n_out;
         b.chunk = nsplit;
         b.nsplit = 1;
+        // 48 partial rows or more: sixteen row groups, a lane's four (value, index) pairs in
+        // flight at once (the second pass is all latency)
+        const bool rg16b = nsplit >= 48;
         const bool rg4b = nsplit >= 16;
-        const int64_t lanes2 = rg4b ? FOLD_THREADS / 4 : FOLD_THREADS;
+        const int64_t lanes2 = rg16b ? FOLD_THREADS / 16 : rg4b ? FOLD_THREADS / 4 : FOLD_THREADS;
         b.lane_blocks = (uint32_t)((L + lanes2 - 1) / lanes2);
         dim3 grid2((unsigned)(b.lane_blocks * n_outer), 1);
-        if (rg4b) hipLaunchKernelGGL((arg_col_kernel<InC<C>, CMP, 1, 4, true>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+        if (rg16b) hipLaunchKernelGGL((arg_col_kernel<InC<C>, CMP, 1, 16, true>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+        else if (rg4b) hipLaunchKernelGGL((arg_col_kernel<InC<C>, CMP, 1, 4, true>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
         else hipLaunchKernelGGL((arg_col_kernel<InC<C>, CMP, 1, 1, true>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
         NXH_HIP(op, hipGetLastError());
       }

@@ -111,12 +111,11 @@ struct ColArgs {
 // of the block's chunk with 8 loads in flight, and the RG partial results meet
 // in LDS. RG > 1 keeps the number of partial rows a split leaves for the
 // second pass small while the grid still fills the chip.
-template <class IN, class CB, class OUT, int V, int RG>
+template <class IN, class CB, class OUT, int V, int RG, int U = 8>
 __global__ __launch_bounds__(FOLD_THREADS) void fold_col_kernel(ColArgs a) {
   using T = typename IN::T;
   using C = typename IN::C;
   constexpr int LANES = FOLD_THREADS / RG;
-  constexpr int U = 8;
   __shared__ C lds[RG > 1 ? (RG - 1) * LANES * V : 1];
   // blocks walk the input from its end (see fold_row_kernel)
   const uint32_t bx = gridDim.x - 1 - blockIdx.x;
@@ -144,10 +143,16 @@ __global__ __launch_bounds__(FOLD_THREADS) void fold_col_kernel(ColArgs a) {
 #pragma unroll
       for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x[j].v[k]));
   }
-  for (; r < r1; r += RG) {
-    FVec<T, V> x = *reinterpret_cast<const FVec<T, V> *>(p + r * a.r_stride);
+  if (r < r1) {  // the rest, fewer than U rows of this group: requested together, added in row order
+    FVec<T, V> x[U - 1];
 #pragma unroll
-    for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x.v[k]));
+    for (int j = 0; j < U - 1; j++)
+      if (r + j * RG < r1) x[j] = *reinterpret_cast<const FVec<T, V> *>(p + (r + j * RG) * a.r_stride);
+#pragma unroll
+    for (int j = 0; j < U - 1; j++)
+      if (r + j * RG < r1)
+#pragma unroll
+        for (int k = 0; k < V; k++) acc[k] = CB::apply(acc[k], IN::ld(x[j].v[k]));
   }
   if constexpr (RG > 1) {
     if (rg > 0) {
@@ -341,11 +346,18 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
           b.nsplit = 1;
           const bool vec2 = L % VC == 0;
           const int v2 = vec2 ? VC : 1;
+          // 48 partial rows or more: sixteen row groups of four loads each, so that a lane's whole
+          // share is in flight at once and four times as many blocks carry the launch (the second
+          // pass is all latency: [64][8192] f32 partials, 2 MiB)
+          const bool rg16b = nsplit >= 48;
           const bool rg4b = nsplit >= 16;
-          const int64_t lanes2 = rg4b ? FOLD_THREADS / 4 : FOLD_THREADS;
+          const int64_t lanes2 = rg16b ? FOLD_THREADS / 16 : rg4b ? FOLD_THREADS / 4 : FOLD_THREADS;
           b.lane_blocks = (uint32_t)((L + lanes2 * v2 - 1) / (lanes2 * v2));
           dim3 grid2((unsigned)(b.lane_blocks * n_outer), 1);
-          if (rg4b) {
+          if (rg16b) {
+            if (vec2) hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, VC, 16, 4>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+            else hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, 1, 16, 4>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+          } else if (rg4b) {
             if (vec2) hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, VC, 4>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
             else hipLaunchKernelGGL((fold_col_kernel<InC<C>, CB, OutS<DT>, 1, 4>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
           } else {
