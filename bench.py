@@ -267,9 +267,9 @@ def next_ops(hip, W, linalg=False):
     # sort moves each element once in and once out; the network in between is
     # compare-exchange work, so the rate is quoted in keys per second too
     rows = W.dev(rng.standard_normal((16384, 1024)).astype(np.float32), dt.float32)
-    timed("sort [16384,1024] f32 axis 1 (sort_lds)", lambda: hip.sort(rows, 1, False), 2 * 16384 * 1024 * 4)
+    timed("sort [16384,1024] f32 axis 1 (sort_registers)", lambda: hip.sort(rows, 1, False), 2 * 16384 * 1024 * 4)
     out[-1]["Mkeys/s"] = round(16384 * 1024 / out[-1]["ms"] / 1e3, 1)
-    timed("argsort [16384,1024] f32 axis 1, descending (sort_lds)", lambda: hip.argsort(rows, 1, True),
+    timed("argsort [16384,1024] f32 axis 1, descending (sort_registers)", lambda: hip.argsort(rows, 1, True),
           2 * 16384 * 1024 * 4)
     out[-1]["Mkeys/s"] = round(16384 * 1024 / out[-1]["ms"] / 1e3, 1)
     one = W.dev(rng.standard_normal(1 << 24).astype(np.float32), dt.float32)

@@ -87,10 +87,14 @@ def test_sort_and_argsort_match_oracle(hip, oracle, d):
 
 
 def path_for(n):
-    return "sort_lds" if n <= 4096 else "sort_radix"  # packed dtypes; (key, index) pairs take sort_global
+    # packed dtypes ((key, index) pairs take sort_lds / sort_global): slices that pad to 128 .. 2048
+    # elements are sorted in registers, shorter ones and 4096 in LDS, longer ones by radix
+    if 64 < n <= 2048:
+        return "sort_registers"
+    return "sort_lds" if n <= 4096 else "sort_radix"
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 1000, 4096, 4097, 12000, 16383, 16384, 16385, 20000, 70001])
+@pytest.mark.parametrize("n", [1, 2, 3, 64, 65, 128, 129, 300, 512, 1000, 1024, 1025, 2048, 2049, 4096, 4097, 12000, 16383, 16384, 16385, 20000, 70001])
 def test_sort_lengths_across_both_paths(hip, oracle, n):
     rng = np.random.default_rng(n)
     x = rng.integers(-1000, 1000, (3, n)).astype(np.float32)
@@ -347,3 +351,33 @@ def test_window_large_and_errors(hip):
         hip.fold(u, [100, 128], [3, 3], [1, 1], [1, 1], [(1, 1), (1, 1)])   # windows do not match the geometry
     with pytest.raises(RuntimeError, match="packed"):
         hip.unfold(hip.buffer(dt.int4, (2, 8)), [2], [1], [1], [(0, 0)])
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16, dt.float8_e4m3, dt.int8, dt.uint8, dt.int16,
+                               dt.uint16, dt.int32, dt.uint32, dt.bool_], ids=lambda d: d.name)
+def test_slices_sorted_in_registers(hip, oracle, d):
+    """Slices that pad to 128 .. 2048 elements (every dtype whose key packs into one word) run the
+    whole network in registers: ragged and whole lengths for each of the five sizes, along the
+    contiguous axis (vector loads and stores where a lane's eight elements are whole and aligned,
+    single elements where the slice is a window of a wider row) and along a strided one, both
+    directions, sort and argsort, ties and NaNs included, bit for bit against the oracle."""
+    rng = np.random.default_rng(4800 + d.tag)
+    for n in (100, 128, 250, 512, 700, 1024, 1500, 2048):
+        wide = values_for(d, (5, n + 3), rng, oracle)
+        if d.is_float:
+            flat = wide.reshape(-1)
+            flat[rng.integers(0, flat.size, 6)] = encode(np.array([np.nan]), d, oracle)[0]
+        cases = (("rows", np.ascontiguousarray(wide[:, :n]), None, 1),
+                 ("window", wide, lambda B, t, n=n: B.shrink(t, [(0, 5), (1, n + 1)]), 1),
+                 ("columns", np.ascontiguousarray(wide[:, :n].T), None, 0))
+        for lname, x, build, axis in cases:
+            h, o = pair(x, d, hip, oracle, build)
+            for desc in (False, True):
+                what = f"{d.name} n={n} {lname} desc={desc}"
+                got, want = logical(hip.sort(h, axis, desc)), logical(oracle.sort(o, axis, desc))
+                assert hip.last_path() == "sort_registers", (what, hip.last_path())
+                if d.is_float:
+                    same_bits_nan_any(got, want, d, oracle, "sort " + what)
+                else:
+                    same_bits(got, want, "sort " + what)
+                same_bits(logical(hip.argsort(h, axis, desc)), logical(oracle.argsort(o, axis, desc)), "argsort " + what)
