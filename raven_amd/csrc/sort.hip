@@ -397,9 +397,30 @@ __global__ __launch_bounds__(256) void psort_lds_kernel(SortArgs a, int spb) {
 // only distances of 512 and more (the last one or three steps of the largest slices) go through
 // LDS. No barrier and no LDS traffic in any other step, and the slice's offsets are worked out
 // once per lane: [16384,1024] f32 along axis 1, 398 us with the network in LDS.
+// The word of the lane m places away (lane ^ m). Distances 1, 2 and 8 are data-parallel moves
+// inside the vector unit (the pairs of a quad swapped, a row of sixteen turned by eight); the others
+// go through the cross-lane network of the LDS, which this kernel keeps busier than anything
+// else (eight clocks a 32-bit move: with every distance there, [16384,1024] f32 took 168 us).
 __device__ __forceinline__ uint64_t lane_xor64(uint64_t x, int m) {
-  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)x, m, 64), hi = (uint32_t)__shfl_xor((int)(uint32_t)(x >> 32), m, 64);
-  return ((uint64_t)hi << 32) | lo;
+  int lo = (int)(uint32_t)x, hi = (int)(uint32_t)(x >> 32);
+  switch (m) {
+    case 1:  // quad_perm:[1,0,3,2]
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0xB1, 0xF, 0xF, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0xB1, 0xF, 0xF, false);
+      break;
+    case 2:  // quad_perm:[2,3,0,1]
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x4E, 0xF, 0xF, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x4E, 0xF, 0xF, false);
+      break;
+    case 8:  // row_ror:8
+      lo = __builtin_amdgcn_update_dpp(0, lo, 0x128, 0xF, 0xF, false);
+      hi = __builtin_amdgcn_update_dpp(0, hi, 0x128, 0xF, 0xF, false);
+      break;
+    default:
+      lo = __shfl_xor(lo, m, 64);
+      hi = __shfl_xor(hi, m, 64);
+  }
+  return ((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo;
 }
 
 template <int DT, int MODE, int LOGNP>
@@ -439,15 +460,18 @@ __global__ __launch_bounds__(256) void psort_reg_kernel(SortArgs a) {
 #pragma unroll
         for (int r = 0; r < E; r++) {
           if (r & j) continue;
-          const bool up = ((i0 + r) & kk) == 0;
+          // ascending run: the pair changes places when the second is smaller; descending: when
+          // the first is (one comparison, the direction folded into its lane mask; equal words
+          // are padding and may go either way)
+          const bool down = ((i0 + r) & kk) != 0;
           const uint64_t x = e[r], y = e[r | j];
-          const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
-          e[r] = up ? lo : hi;
-          e[r | j] = up ? hi : lo;
+          const bool change = (y < x) != down;
+          e[r] = change ? y : x;
+          e[r | j] = change ? x : y;
         }
       } else {
         const int m = j / E;  // the partner lane's distance
-        const bool keep_min = ((i0 & kk) == 0) == ((t & m) == 0);
+        const bool keep_max = ((i0 & kk) == 0) != ((t & m) == 0);
         if (m >= 64) {
           if constexpr (CROSS_WAVE) {
             __syncthreads();
@@ -457,14 +481,14 @@ __global__ __launch_bounds__(256) void psort_reg_kernel(SortArgs a) {
 #pragma unroll
             for (int r = 0; r < E; r++) {
               const uint64_t y = xch[r * 256 + (threadIdx.x ^ m)];
-              e[r] = keep_min ? (e[r] < y ? e[r] : y) : (e[r] < y ? y : e[r]);
+              e[r] = ((y < e[r]) != keep_max) ? y : e[r];
             }
           }
         } else {
 #pragma unroll
           for (int r = 0; r < E; r++) {
             const uint64_t y = lane_xor64(e[r], m);
-            e[r] = keep_min ? (e[r] < y ? e[r] : y) : (e[r] < y ? y : e[r]);
+            e[r] = ((y < e[r]) != keep_max) ? y : e[r];
           }
         }
       }
