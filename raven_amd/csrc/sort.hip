@@ -17,8 +17,10 @@
 // Algorithm: bitonic sorting network, the slice padded to a power of two with
 // elements that sort last. Elements are (key, index) pairs for 64-bit and
 // complex keys and one packed 64-bit word otherwise (see "packed keys").
-//   sort_lds     slices of up to 4096 elements (2048 for 16-byte keys): whole
-//                network in LDS, several short slices per block;
+//   sort_registers  packed slices of up to 4096 elements: the whole network in
+//                registers, eight or sixteen elements a lane;
+//   sort_lds     (key, index) slices of up to 4096 elements (2048 for 16-byte keys):
+//                whole network in LDS, several short slices per block;
 //   sort_global  longer slices of (key, index) pairs: staged in scratch memory;
 //                chunks are sorted in LDS, then each merge level runs its
 //                long-distance exchanges as passes over global memory and
@@ -300,54 +302,6 @@ struct Packed {
   }
 };
 constexpr uint64_t PACKED_PAD = ~(uint64_t)0;
-constexpr int PNL = 4096;  // packed elements per LDS chunk (32 KB)
-
-__device__ __forceinline__ void packed_step(uint64_t *w, int count, int j, int64_t kk, int64_t base, int64_t mask) {
-  for (int p = threadIdx.x; p < count / 2; p += 256) {
-    const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1));
-    const int l = i | j;
-    const bool up = (((base + i) & mask) & kk) == 0;
-    const uint64_t x = w[i], y = w[l];
-    const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
-    w[i] = up ? lo : hi;
-    w[l] = up ? hi : lo;
-  }
-  __syncthreads();
-}
-
-// The last log2(4) steps of every merge level stay inside aligned groups of
-// four elements: one lane takes a group through both of them in registers.
-__device__ __forceinline__ void packed_tail4(uint64_t *w, int count, int64_t kk, int64_t base, int64_t mask) {
-  for (int q = threadIdx.x; q < count / 4; q += 256) {
-    const int i = q * 4;
-    const bool up = (((base + i) & mask) & kk) == 0;
-    uint64_t e0 = w[i], e1 = w[i + 1], e2 = w[i + 2], e3 = w[i + 3];
-    auto cx = [&](uint64_t &x, uint64_t &y) {
-      const uint64_t lo = x < y ? x : y, hi = x < y ? y : x;
-      x = up ? lo : hi;
-      y = up ? hi : lo;
-    };
-    cx(e0, e2);
-    cx(e1, e3);
-    cx(e0, e1);
-    cx(e2, e3);
-    w[i] = e0;
-    w[i + 1] = e1;
-    w[i + 2] = e2;
-    w[i + 3] = e3;
-  }
-  __syncthreads();
-}
-
-// All steps j of level kk from `jtop` down to 1 inside LDS.
-__device__ __forceinline__ void packed_level(uint64_t *w, int count, int64_t kk, int jtop, int64_t base, int64_t mask) {
-  int j = jtop;
-  for (; j >= 4; j >>= 1) packed_step(w, count, j, kk, base, mask);
-  if (jtop >= 2 && count >= 4) packed_tail4(w, count, kk, base, mask);
-  else
-    for (; j >= 1; j >>= 1) packed_step(w, count, j, kk, base, mask);
-}
-
 template <int DT, int MODE>
 __device__ __forceinline__ void packed_store(const SortArgs &a, int64_t oo, int64_t io, int64_t i, uint64_t word) {
   using TR = Tr<DT>;
@@ -359,43 +313,12 @@ __device__ __forceinline__ void packed_store(const SortArgs &a, int64_t oo, int6
         TR::st(TR::ld(reinterpret_cast<const S *>(a.in)[io + (int64_t)src * a.in_axis]));
 }
 
-template <int DT, int MODE>
-__global__ __launch_bounds__(256) void psort_lds_kernel(SortArgs a, int spb) {
-  using TR = Tr<DT>;
-  using S = typename TR::S;
-  __shared__ uint64_t w[PNL];
-  const int np = (int)a.n_pad, count = spb * np;
-  const int64_t first = (int64_t)blockIdx.x * spb;
-  for (int e = threadIdx.x; e < count; e += 256) {
-    const int64_t s = first + e / np;
-    const int i = e % np;
-    uint64_t word = PACKED_PAD;
-    if (s < a.slices && i < a.n) {
-      int64_t io, oo;
-      slice_offsets(a, s, io, oo);
-      word = Packed<DT>::template pack<MODE>(TR::ld(reinterpret_cast<const S *>(a.in)[io + i * a.in_axis]), (uint32_t)i);
-    }
-    w[e] = word;
-  }
-  __syncthreads();
-  for (int kk = 2; kk <= np; kk <<= 1) packed_level(w, count, kk, kk >> 1, 0, np - 1);
-  for (int e = threadIdx.x; e < count; e += 256) {
-    const int64_t s = first + e / np;
-    const int i = e % np;
-    if (s < a.slices && i < a.n) {
-      int64_t io, oo;
-      slice_offsets(a, s, io, oo);
-      packed_store<DT, MODE>(a, oo, io, i, w[e]);
-    }
-  }
-}
-
-// Slices of 128 to 2048 padded elements: the whole network in registers. A lane holds eight
-// consecutive elements of its slice, NP / 8 lanes a slice, 2048 / NP slices a block. Exchanges at
-// distances 1, 2, 4 stay inside the lane; distances 8 .. 256 meet the lane 1 .. 32 places away
-// through the cross-lane network, the lane keeping the smaller or the larger word of each pair;
-// only distances of 512 and more (the last one or three steps of the largest slices) go through
-// LDS. No barrier and no LDS traffic in any other step, and the slice's offsets are worked out
+// Slices of up to 4096 padded elements: the whole network in registers. A lane holds E = 8
+// consecutive elements of its slice (16 for slices of 4096), NP / E lanes a slice, 256 E / NP
+// slices a block; slices shorter than 64 are padded to 64. Exchanges at distances below E stay
+// inside the lane; distances E .. 32 E meet the lane 1 .. 32 places away through the cross-lane
+// network, the lane keeping the smaller or the larger word of each pair; only distances of 64 E
+// and more (the last one or three steps of the largest slices) go through LDS. No barrier and no LDS traffic in any other step, and the slice's offsets are worked out
 // once per lane: [16384,1024] f32 along axis 1, 398 us with the network in LDS.
 // The word of the lane m places away (lane ^ m). Distances 1, 2 and 8 are data-parallel moves
 // inside the vector unit (the pairs of a quad swapped, a row of sixteen turned by eight); the others
@@ -427,7 +350,7 @@ template <int DT, int MODE, int LOGNP>
 __global__ __launch_bounds__(256) void psort_reg_kernel(SortArgs a) {
   using TR = Tr<DT>;
   using S = typename TR::S;
-  constexpr int NP = 1 << LOGNP, E = 8, TPS = NP / E, SPB = 256 / TPS;
+  constexpr int NP = 1 << LOGNP, E = LOGNP >= 12 ? 16 : 8, TPS = NP / E, SPB = 256 / TPS;
   static_assert(TPS >= 1 && TPS <= 256, "a slice is held by one block");
   constexpr bool CROSS_WAVE = TPS > 64;
   __shared__ uint64_t xch[CROSS_WAVE ? 256 * E : 1];
@@ -842,27 +765,21 @@ int radix_run(nxh_context *ctx, const char *op, SortArgs &a) {
 
 template <int DT, int MODE>
 int psort_run(nxh_context *ctx, const char *op, SortArgs &a) {
-  if (a.n_pad >= 128 && a.n_pad <= 2048) {
-    const int64_t spb = 2048 / a.n_pad, blocks = (a.slices + spb - 1) / spb;
+  if (a.n_pad <= 4096) {
+    const int64_t np = std::max<int64_t>(a.n_pad, 64);
+    const int64_t spb = np == 4096 ? 1 : 2048 / np, blocks = (a.slices + spb - 1) / spb;
     if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many slices for one launch");
     nxh_set_path("sort_registers");
-    switch (a.n_pad) {
-      case 128: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 7>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a); break;
-      case 256: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 8>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a); break;
-      case 512: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 9>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a); break;
-      case 1024: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 10>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a); break;
-      default: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 11>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a); break;
+    const dim3 grid((unsigned)blocks), block(256);
+    switch (np) {
+      case 64: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 6>), grid, block, 0, ctx->stream, a); break;
+      case 128: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 7>), grid, block, 0, ctx->stream, a); break;
+      case 256: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 8>), grid, block, 0, ctx->stream, a); break;
+      case 512: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 9>), grid, block, 0, ctx->stream, a); break;
+      case 1024: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 10>), grid, block, 0, ctx->stream, a); break;
+      case 2048: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 11>), grid, block, 0, ctx->stream, a); break;
+      default: hipLaunchKernelGGL((psort_reg_kernel<DT, MODE, 12>), grid, block, 0, ctx->stream, a); break;
     }
-    NXH_HIP(op, hipGetLastError());
-    return NXH_OK;
-  }
-  if (a.n_pad <= PNL) {
-    int spb = (int)std::max<int64_t>(1, 1024 / a.n_pad);
-    if (spb > a.slices) spb = (int)a.slices;
-    const int64_t blocks = (a.slices + spb - 1) / spb;
-    if (blocks > 0x7fffffffLL) return nxh_fail(NXH_FAILURE, op, "too many slices for one launch");
-    nxh_set_path("sort_lds");
-    hipLaunchKernelGGL((psort_lds_kernel<DT, MODE>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, a, spb);
     NXH_HIP(op, hipGetLastError());
     return NXH_OK;
   }

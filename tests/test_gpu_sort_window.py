@@ -83,15 +83,14 @@ def test_sort_and_argsort_match_oracle(hip, oracle, d):
                 else:
                     same_bits(got, want, "sort " + what)
                 same_bits(logical(hip.argsort(h, axis, desc)), logical(oracle.argsort(o, axis, desc)), "argsort " + what)
-    assert hip.last_path() == "sort_lds"
+    pairs = d in (dt.float64, dt.uint64, dt.int64, dt.complex64, dt.complex128)
+    assert hip.last_path() == ("sort_lds" if pairs else "sort_registers")
 
 
 def path_for(n):
-    # packed dtypes ((key, index) pairs take sort_lds / sort_global): slices that pad to 128 .. 2048
-    # elements are sorted in registers, shorter ones and 4096 in LDS, longer ones by radix
-    if 64 < n <= 2048:
-        return "sort_registers"
-    return "sort_lds" if n <= 4096 else "sort_radix"
+    # packed dtypes ((key, index) pairs take sort_lds / sort_global): slices that pad to 4096 elements
+    # or fewer are sorted in registers, longer ones by radix
+    return "sort_registers" if n <= 4096 else "sort_radix"
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 64, 65, 128, 129, 300, 512, 1000, 1024, 1025, 2048, 2049, 4096, 4097, 12000, 16383, 16384, 16385, 20000, 70001])
@@ -356,13 +355,13 @@ def test_window_large_and_errors(hip):
 @pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16, dt.float8_e4m3, dt.int8, dt.uint8, dt.int16,
                                dt.uint16, dt.int32, dt.uint32, dt.bool_], ids=lambda d: d.name)
 def test_slices_sorted_in_registers(hip, oracle, d):
-    """Slices that pad to 128 .. 2048 elements (every dtype whose key packs into one word) run the
-    whole network in registers: ragged and whole lengths for each of the five sizes, along the
+    """Slices of up to 4096 elements (every dtype whose key packs into one word) run the
+    whole network in registers: ragged and whole lengths for each of the seven sizes, along the
     contiguous axis (vector loads and stores where a lane's eight elements are whole and aligned,
     single elements where the slice is a window of a wider row) and along a strided one, both
     directions, sort and argsort, ties and NaNs included, bit for bit against the oracle."""
     rng = np.random.default_rng(4800 + d.tag)
-    for n in (100, 128, 250, 512, 700, 1024, 1500, 2048):
+    for n in (5, 33, 64, 100, 128, 250, 512, 700, 1024, 1500, 2048, 3000, 4096):
         wide = values_for(d, (5, n + 3), rng, oracle)
         if d.is_float:
             flat = wide.reshape(-1)
