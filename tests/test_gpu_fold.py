@@ -229,3 +229,41 @@ def test_views_of_high_rank_with_nothing_to_merge(hip, oracle):
     h32, o32 = pair(y, dt.int32, hip, oracle, lambda B, t: B.flip(t, flips32))
     axes = [a for a in range(32) if a % 4 == 2]
     same_bits(logical(hip.reduce("sum", axes, h32)), logical(oracle.reduce("sum", axes, o32)), "rank 32")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.int32, dt.int8, dt.float64], ids=lambda d: d.name)
+def test_two_reduced_dims_that_do_not_merge(hip, oracle, d):
+    """Sums, maxima and minima over two axes with a kept axis between them (the batch and the
+    positions of [N, C, H, W] with the channels kept; axes 0 and 2 of a rank-3 tensor): the
+    unit-stride or the longer reduced dim is walked, every index of the other is a partial result
+    that the second pass folds. Both forms (a reduced dim with unit stride; a kept dim with unit
+    stride), ragged extents, a window of a wider tensor, against the oracle."""
+    rng = np.random.default_rng(1300 + d.tag)
+    cases = [
+        ("NCHW, channels kept", (9, 20, 13, 11), None, [0, 2, 3], "fold_row_outer"),
+        ("axes 0 and 2", (33, 50, 130), None, [0, 2], "fold_row_outer"),
+        ("axes 0 and 2, short rows", (70, 6, 9), None, [0, 2], "fold_row_outer"),
+        ("window of a wider tensor", (12, 22, 70), lambda B, t: B.shrink(t, [(1, 11), (2, 20), (3, 67)]), [0, 2], "fold_row_outer"),
+        ("unit stride kept: axes 0 and 2 of rank 4", (7, 30, 12, 64), None, [0, 2], "fold_col_outer"),
+        ("unit stride kept, the earlier dim longer", (40, 3, 9, 48), None, [0, 2], "fold_col_outer"),
+        ("channels last, batch and one position axis", (10, 9, 8, 32), None, [0, 2], "fold_col_outer"),
+    ]
+    for what, shape, build, axes, path in cases:
+        if d.is_float:
+            x = encode(rng.uniform(-2, 2, shape), d, oracle)
+        else:
+            info = np.iinfo(d.np_storage)
+            x = rng.integers(max(info.min, -100), min(info.max, 100), shape, endpoint=True).astype(d.np_storage)
+        h, o = pair(x, d, hip, oracle, build)
+        k = int(np.prod([h.shape[a] for a in axes]))
+        for op in ("sum", "max", "min"):
+            g, w = logical(hip.reduce(op, axes, h)), logical(oracle.reduce(op, axes, o))
+            assert hip.last_path() == path, (what, op, hip.last_path())
+            if d.is_float and op == "sum":
+                close(g, w, d, oracle, TOL[d.name][0], TOL[d.name][0] * 2.0 * k, f"{what} {op}")
+            else:
+                same_bits(g, w, f"{what} {op}")
+    # sums of ones count the reduced elements exactly
+    ones = hip.contiguous(hip.full(dt.float32, (64, 48, 512), 1.0))
+    same_bits(logical(hip.reduce("sum", [0, 2], ones)), np.full((48,), 64.0 * 512.0, np.float32), "sum of ones")
+    assert hip.last_path() == "fold_row_outer"
