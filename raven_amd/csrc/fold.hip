@@ -182,6 +182,53 @@ __global__ __launch_bounds__(FOLD_THREADS) void fold_col_kernel(ColArgs a) {
   }
 }
 
+// ── fold_narrow ─────────────────────────────────────────────────────────────
+// A contiguous [rows][L] matrix with fewer than 16 columns, reduced down its rows (class counts,
+// the bias gradient of a small output layer): too narrow for fold_col's column lanes. The matrix
+// is read as the flat run it is: the block's first (256 / L) * L lanes step through it that many
+// elements at a time, so a lane always meets the same column and neighbouring lanes neighbouring
+// addresses; the lanes of a column then meet in LDS. Blocks take runs of rows and leave partial
+// results [block][L], which one more block of the same kernel folds.
+struct NarrowArgs {
+  const void *in;
+  void *out;
+  int64_t R, rows_per_block;
+  int L, final_;
+};
+template <class IN, class CB, class OUT>
+__global__ __launch_bounds__(FOLD_THREADS) void fold_narrow_kernel(NarrowArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  __shared__ C lds[FOLD_THREADS];
+  const int per_pass = FOLD_THREADS / a.L, active = per_pass * a.L;
+  const int t = threadIdx.x;
+  const int64_t r_begin = (int64_t)blockIdx.x * a.rows_per_block;
+  const int64_t rows = (r_begin + a.rows_per_block < a.R ? r_begin + a.rows_per_block : a.R) - r_begin;
+  C acc = CB::init();
+  if (t < active) {
+    const T *q = (const T *)a.in + r_begin * a.L + t;
+    const int row0 = t / a.L;
+    const int64_t mine = rows > row0 ? (rows - row0 + per_pass - 1) / per_pass : 0;  // this lane's elements
+    int64_t i = 0;
+    for (; i + 8 <= mine; i += 8) {
+      T x[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) x[j] = q[(i + j) * active];
+#pragma unroll
+      for (int j = 0; j < 8; j++) acc = CB::apply(acc, IN::ld(x[j]));
+    }
+    for (; i < mine; i++) acc = CB::apply(acc, IN::ld(q[i * active]));
+  }
+  lds[t] = acc;
+  __syncthreads();
+  if (t < a.L) {
+    C r = lds[t];
+    for (int i = 1; i < per_pass; i++) r = CB::apply(r, lds[t + i * a.L]);
+    if (a.final_) ((typename OUT::T *)a.out)[t] = OUT::st(r);
+    else ((C *)a.out)[(int64_t)blockIdx.x * a.L + t] = r;
+  }
+}
+
 // ── fold_any ────────────────────────────────────────────────────────────────
 struct AnyArgs {
   const void *in;
@@ -250,7 +297,7 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
   const int row_dim = g.nr == 1 ? 0 : (g.nr == 2 ? (g.rin[1] == 1 ? 1 : (g.rin[0] == 1 ? 0 : -1)) : -1);
   const bool row_two = g.nr == 2 && row_dim >= 0;
   if (row_dim >= 0 && g.rin[row_dim] == 1 && g.n_out <= 0x7fffffffLL * 4 &&
-      (row_two ? g.rshape[row_dim] >= 8 && outer_fits(g.rshape[1 - row_dim]) : g.R >= 64)) {
+      (row_two ? g.rshape[row_dim] >= 8 && outer_fits(g.rshape[1 - row_dim]) : g.R >= 32)) {
     RowArgs a;
     if (dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout)) {
       const int64_t run = g.rshape[row_dim], outer = row_two ? g.rshape[1 - row_dim] : 1;
@@ -301,6 +348,42 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
         b.nsplit = 1;
         dim3 grid2((unsigned)((g.n_out + 3) / 4), 1);
         hipLaunchKernelGGL((fold_row_kernel<InC<C>, CB, OutS<DT>, 64, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
+        NXH_HIP(op, hipGetLastError());
+      }
+      return NXH_OK;
+    }
+  }
+
+  // ---- fold_narrow: a contiguous [rows][L] matrix, L < 16, reduced down its rows ----
+  if (g.nr == 1 && g.nk == 1 && g.kin[0] == 1 && g.kout[0] == 1 && g.kshape[0] < 16 && g.rin[0] == g.kshape[0] &&
+      g.R >= 512) {
+    NarrowArgs a;
+    a.L = (int)g.kshape[0];
+    a.R = g.R;
+    const int64_t nblocks = std::min<int64_t>((int64_t)cus * 8, (g.R + 1023) / 1024);
+    a.rows_per_block = (g.R + nblocks - 1) / nblocks;
+    const int64_t used = (g.R + a.rows_per_block - 1) / a.rows_per_block;
+    const size_t bytes = (size_t)used * a.L * sizeof(C);
+    if (!g.fixed_scratch || bytes <= NXH_STATIC_WS_BYTES) {
+      a.in = ibase;
+      a.final_ = used == 1;
+      a.out = obase;
+      if (used > 1) {
+        int rc = scratch.get(0, bytes);
+        if (rc) return rc;
+        a.out = scratch.p[0];
+      }
+      nxh_set_path("fold_narrow");
+      hipLaunchKernelGGL((fold_narrow_kernel<InS<DT>, CB, OutS<DT>>), dim3((unsigned)used), dim3(FOLD_THREADS), 0, ctx->stream, a);
+      NXH_HIP(op, hipGetLastError());
+      if (used > 1) {
+        NarrowArgs b = a;
+        b.in = scratch.p[0];
+        b.out = obase;
+        b.R = used;
+        b.rows_per_block = used;
+        b.final_ = 1;
+        hipLaunchKernelGGL((fold_narrow_kernel<InC<C>, CB, OutS<DT>>), dim3(1), dim3(FOLD_THREADS), 0, ctx->stream, b);
         NXH_HIP(op, hipGetLastError());
       }
       return NXH_OK;

@@ -267,3 +267,56 @@ def test_two_reduced_dims_that_do_not_merge(hip, oracle, d):
     ones = hip.contiguous(hip.full(dt.float32, (64, 48, 512), 1.0))
     same_bits(logical(hip.reduce("sum", [0, 2], ones)), np.full((48,), 64.0 * 512.0, np.float32), "sum of ones")
     assert hip.last_path() == "fold_row_outer"
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.int32, dt.int8, dt.uint8, dt.complex64],
+                         ids=lambda d: d.name)
+def test_tall_narrow_matrices_reduced_down_their_rows(hip, oracle, d):
+    """[rows, L] with fewer than 16 columns, reduced over the rows (class counts, the bias gradient of a
+    small layer): read as one flat run, a lane always on the same column. One block and many,
+    ragged last blocks, every L from 2 to 15 among the cases."""
+    rng = np.random.default_rng(1400 + d.tag)
+    for rows, L in ((512, 2), (700, 15), (5000, 10), (100001, 3), (40000, 7), (3000, 13)):
+        if d.is_complex:
+            x = (rng.uniform(-1, 1, (rows, L)) + 1j * rng.uniform(-1, 1, (rows, L))).astype(np.complex64)
+        elif d.is_float:
+            x = encode(rng.uniform(-2, 2, (rows, L)), d, oracle)
+        else:
+            info = np.iinfo(d.np_storage)
+            x = rng.integers(max(info.min, -100), min(info.max, 100), (rows, L), endpoint=True).astype(d.np_storage)
+        h, o = pair(x, d, hip, oracle)
+        for op in ("sum", "max", "min"):
+            if d.is_complex and op != "sum":
+                continue
+            g, w = logical(hip.reduce(op, [0], h)), logical(oracle.reduce(op, [0], o))
+            assert hip.last_path() == "fold_narrow", (rows, L, op, hip.last_path())
+            if d.is_complex:
+                assert np.allclose(g, w, rtol=1e-4, atol=1e-4 * rows), (rows, L)
+            elif d.is_float and op == "sum":
+                close(g, w, d, oracle, TOL[d.name][0], TOL[d.name][0] * 2.0 * rows, f"[{rows},{L}] {op}")
+            else:
+                same_bits(g, w, f"[{rows},{L}] {op}")
+    ones = hip.contiguous(hip.full(dt.float32, (1 << 20, 10), 1.0))
+    same_bits(logical(hip.reduce("sum", [0], ones)), np.full((10,), float(1 << 20), np.float32), "sum of ones")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.int32, dt.uint8], ids=lambda d: d.name)
+def test_argreduce_of_many_short_rows(hip, oracle, d):
+    """argmax / argmin along rows of fewer than 32 elements, 65 536 rows or more: a lane per row.
+    Ties (the first index wins) and NaNs (the first NaN wins) included, bit for bit."""
+    rng = np.random.default_rng(1500 + d.tag)
+    for rows, n in ((70000, 10), (65536 + 7, 31), (100000, 2)):
+        if d.is_float:
+            v = rng.integers(-5, 6, (rows, n)).astype(np.float64)  # many ties
+            v[rng.random(v.shape) < 0.01] = np.nan
+            x = encode(v, d, oracle)
+        else:
+            info = np.iinfo(d.np_storage)
+            x = rng.integers(max(info.min, -5), min(info.max, 5), (rows, n), endpoint=True).astype(d.np_storage)
+        h, o = pair(x, d, hip, oracle)
+        same_bits(logical(hip.argmax(h, 1)), logical(oracle.argmax(o, 1)), f"argmax [{rows},{n}]")
+        assert hip.last_path() == "arg_row_lane", hip.last_path()
+        same_bits(logical(hip.argmin(h, 1)), logical(oracle.argmin(o, 1)), f"argmin [{rows},{n}]")
+        # the same rows as columns of the transposed matrix (strided axis)
+        ht, ot = pair(np.ascontiguousarray(x.T), d, hip, oracle)
+        same_bits(logical(hip.argmax(ht, 0)), logical(oracle.argmax(ot, 0)), f"argmax axis 0 [{n},{rows}]")
