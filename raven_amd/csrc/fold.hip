@@ -297,7 +297,7 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
   const int row_dim = g.nr == 1 ? 0 : (g.nr == 2 ? (g.rin[1] == 1 ? 1 : (g.rin[0] == 1 ? 0 : -1)) : -1);
   const bool row_two = g.nr == 2 && row_dim >= 0;
   if (row_dim >= 0 && g.rin[row_dim] == 1 && g.n_out <= 0x7fffffffLL * 4 &&
-      (row_two ? g.rshape[row_dim] >= 8 && outer_fits(g.rshape[1 - row_dim]) : g.R >= 32)) {
+      (row_two ? g.rshape[row_dim] >= 8 && outer_fits(g.rshape[1 - row_dim]) : g.R >= 64)) {
     RowArgs a;
     if (dims_fill(&a.kept, g.nk, g.kshape, g.kin, g.kout)) {
       const int64_t run = g.rshape[row_dim], outer = row_two ? g.rshape[1 - row_dim] : 1;

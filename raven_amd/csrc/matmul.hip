@@ -15,6 +15,8 @@
 //               K-slab while the current one is multiplied. Either operand may
 //               be K-contiguous or M/N-contiguous in memory; the turn happens
 //               on the way into LDS.
+//   gemm_rowdot n <= 4 with A's rows along K (matrix x vector): a wave per row of A,
+//               16-byte pieces, float32 sums met through the cross-lane network.
 //   gemm_skinny m <= 16 (decode-like GEMV): HBM-bound on B, which is streamed
 //               once; K is split across blocks only as far as it takes to fill
 //               the chip and the f32 partials are summed by a second pass. f32
@@ -1492,11 +1494,102 @@ static int try_tile_repacked(nxh_context *ctx, const GemmArgs &a0, uint32_t nbat
   return rc;
 }
 
+// ── gemm_rowdot: a matrix whose rows run along K, times one to four columns ──
+// (matrix x vector: C[m][n] = sum over k of A[m][k] B[k][n], N <= 4.) A wave per row of A: its
+// lanes take the row in 16-byte pieces, four in flight, multiply by the matching pieces of the
+// columns (a few KB, served by the caches), add in float32 and meet through the cross-lane
+// network. A is read once at the rate of a reduction over its rows; the tiled kernels spent a whole
+// 128-column block on the one column ([4096,4096] x [4096,1] f32: 444 us).
+template <int DT, int NC>
+__global__ __launch_bounds__(256) void gemm_rowdot_kernel(GemmArgs a) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  constexpr int V = 16 / (int)sizeof(S);
+  struct alignas(16) Piece {
+    S v[V];
+  };
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t m = (int64_t)blockIdx.x * 4 + wave;
+  if (m >= a.M) return;
+  int64_t ao, bo, co;
+  batch_decode(a.batch, a.batch0 + blockIdx.y, ao, bo, co);
+  const S *A = (const S *)a.A + ao + m * a.ars;
+  const S *B = (const S *)a.B + bo;
+  float acc[NC];
+#pragma unroll
+  for (int n = 0; n < NC; n++) acc[n] = 0.0f;
+  const int64_t nv = a.a_vec ? a.K / V : 0;
+  const bool b_pieces = NC == 1 && a.b_vec;  // the one column is a contiguous, aligned run
+  auto piece = [&](int64_t i, const Piece &x) {
+    if (b_pieces) {
+      const Piece y = *reinterpret_cast<const Piece *>(B + i * V);
+#pragma unroll
+      for (int j = 0; j < V; j++) acc[0] = acc[0] + (float)TR::ld(x.v[j]) * (float)TR::ld(y.v[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; j++) {
+        const float av = (float)TR::ld(x.v[j]);
+        const S *b = B + (i * V + j) * a.brs;
+#pragma unroll
+        for (int n = 0; n < NC; n++)
+          if (n < a.N) acc[n] = acc[n] + av * (float)TR::ld(b[n * a.bcs]);
+      }
+    }
+  };
+  int64_t i = lane;
+  for (; i + 192 < nv; i += 256) {
+    Piece x[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) x[u] = *reinterpret_cast<const Piece *>(A + (i + 64 * u) * V);
+#pragma unroll
+    for (int u = 0; u < 4; u++) piece(i + 64 * u, x[u]);
+  }
+  for (; i < nv; i += 64) piece(i, *reinterpret_cast<const Piece *>(A + i * V));
+  for (int64_t k = nv * V + lane; k < a.K; k += 64) {
+    const float av = (float)TR::ld(A[k]);
+#pragma unroll
+    for (int n = 0; n < NC; n++)
+      if (n < a.N) acc[n] = acc[n] + av * (float)TR::ld(B[k * a.brs + n * a.bcs]);
+  }
+#pragma unroll
+  for (int n = 0; n < NC; n++)
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) acc[n] = acc[n] + __shfl_down(acc[n], d, 64);
+  if (lane == 0) {
+    S *C = (S *)a.C + co + m * a.crs;
+#pragma unroll
+    for (int n = 0; n < NC; n++)
+      if (n < a.N) C[n * a.ccs] = TR::st((typename TR::C)acc[n]);
+  }
+}
+
+template <int DT>
+static int launch_rowdot(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool batch_aligned_a, bool batch_aligned_b) {
+  using S = typename Tr<DT>::S;
+  constexpr int V = 16 / (int)sizeof(S);
+  a.a_vec = al16(a.A) && batch_aligned_a && a.ars % V == 0;
+  a.b_vec = a.N == 1 && a.brs == 1 && al16(a.B) && batch_aligned_b;
+  nxh_set_path("gemm_rowdot");
+  const dim3 block(256);
+  for (uint32_t b0 = 0; b0 < nbatch; b0 += 65535) {
+    a.batch0 = b0;
+    const dim3 grid((unsigned)((a.M + 3) / 4), std::min<uint32_t>(65535, nbatch - b0));
+    if (a.N == 1) hipLaunchKernelGGL((gemm_rowdot_kernel<DT, 1>), grid, block, 0, ctx->stream, a);
+    else if (a.N == 2) hipLaunchKernelGGL((gemm_rowdot_kernel<DT, 2>), grid, block, 0, ctx->stream, a);
+    else hipLaunchKernelGGL((gemm_rowdot_kernel<DT, 4>), grid, block, 0, ctx->stream, a);
+    NXH_HIP("matmul", hipGetLastError());
+  }
+  return NXH_OK;
+}
+
 template <class MM>
 static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool batch_aligned_a,
                           bool batch_aligned_b) {
   using S = typename MM::S;
   constexpr int VL = MM::VL;
+  // matrix x vector (up to four columns), the matrix's rows along K: a wave per row
+  if (a.N <= 4 && a.acs == 1 && a.K >= 64 && (double)a.M * (double)nbatch >= 256.0 && a.M <= 0x7fffffffLL)
+    return launch_rowdot<MM::DT>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);
   // decode-like shape: one batch, few rows, B row-major: stream B once
   if (nbatch == 1 && a.M <= 16 && a.bcs == 1 && a.N >= 1024 && a.K >= 256 && a.batch.n == 0) {
     constexpr int VN = 16 / (int)sizeof(S);  // one 16-byte load per lane and row of B

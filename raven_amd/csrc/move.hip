@@ -72,14 +72,20 @@ struct GatherAnyArgs {
   int64_t dstride[NXH_MAX_NDIM], istride[NXH_MAX_NDIM], ostride[NXH_MAX_NDIM];
   int *fault;
 };
-template <class E>
+// N: the type the element number is unravelled in (uint32_t when the output holds fewer than 2^32
+// elements). With random indices the reads, not the arithmetic, are what costs: [8192,8192] f32 along
+// axis 1 takes 448 us with either type, every lane of a wave on a cache line of its own.
+template <class E, class N>
 __global__ __launch_bounds__(256) void gather_any_kernel(GatherAnyArgs a) {
   const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (it >= a.total) return;
-  int64_t rem = it, io = 0, oo = 0, doff = 0;
+  N rem = (N)it;
+  int64_t io = 0, oo = 0, doff = 0;
   for (int d = a.ndim - 1; d >= 0; d--) {
-    const int64_t c = rem % a.shape[d];
-    rem /= a.shape[d];
+    const N extent = (N)a.shape[d];
+    const N q = rem / extent;
+    const int64_t c = (int64_t)(rem - q * extent);
+    rem = q;
     io += c * a.istride[d];
     oo += c * a.ostride[d];
     if (d != a.axis) doff += c * a.dstride[d];
@@ -107,7 +113,9 @@ static bool contiguous_off0(const nxh_tensor *a) {
 
 template <class E>
 static void launch_any_e(nxh_context *ctx, const GatherAnyArgs &a) {
-  hipLaunchKernelGGL((gather_any_kernel<E>), dim3((unsigned)((a.total + 255) / 256)), dim3(256), 0, ctx->stream, a);
+  const dim3 grid((unsigned)((a.total + 255) / 256));
+  if (a.total <= 0xffffffffLL) hipLaunchKernelGGL((gather_any_kernel<E, uint32_t>), grid, dim3(256), 0, ctx->stream, a);
+  else hipLaunchKernelGGL((gather_any_kernel<E, int64_t>), grid, dim3(256), 0, ctx->stream, a);
 }
 
 NXH_EXPORT int nxh_gather(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *data,

@@ -712,3 +712,30 @@ def test_long_ragged_rows_get_whole_memory_lines(hip, oracle, d):
     for n in (4096, 4160, 1000):
         got = hip.matmul(hip.full(d, (4, 8), 1), hip.full(d, (8, n), 1))
         assert tuple(got.strides) == (n, 1)
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_matrix_times_vector(hip, oracle, d):
+    """A matrix whose rows run along K times one to four columns takes a wave per row
+    (gemm_rowdot): whole and ragged K, rows that are no whole vectors (element loads), a window of a
+    wider matrix, two to four columns of a strided B, a batch with a shared vector, against the
+    float64 product of the stored values."""
+    rng = np.random.default_rng(5200 + d.tag)
+    for m, k, n in ((4096, 4096, 1), (300, 1000, 1), (257, 67, 1), (512, 2051, 2), (1000, 768, 3), (256, 4096, 4)):
+        a = encode(rng.standard_normal((m, k)), d, oracle)
+        b = encode(rng.standard_normal((k, n)), d, oracle)
+        ha, hb = pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0]
+        check(hip, oracle, d, ha, hb, a, b, f"{m}x{k}x{n}")
+        assert hip.last_path() == "gemm_rowdot", hip.last_path()
+    # a window of a wider matrix (row pitch 1003, first column 1: no aligned pieces) and B as a column of a wider one
+    wide = encode(rng.standard_normal((700, 1003)), d, oracle)
+    bw = encode(rng.standard_normal((1000, 5)), d, oracle)
+    ha = pair(wide, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 700), (1, 1001)]))[0]
+    hb = pair(bw, d, hip, oracle, lambda B, t: B.shrink(t, [(0, 1000), (2, 3)]))[0]
+    check(hip, oracle, d, ha, hb, wide[:, 1:1001], bw[:, 2:3], "windows")
+    assert hip.last_path() == "gemm_rowdot", hip.last_path()
+    # a batch of matrices, one vector for all
+    a = encode(rng.standard_normal((6, 128, 320)), d, oracle)
+    v = encode(rng.standard_normal((320, 1)), d, oracle)
+    check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(v, d, hip, oracle)[0], a, v, "batch, shared vector")
+    assert hip.last_path() == "gemm_rowdot", hip.last_path()
