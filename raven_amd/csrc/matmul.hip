@@ -15,6 +15,7 @@
 //               K-slab while the current one is multiplied. Either operand may
 //               be K-contiguous or M/N-contiguous in memory; the turn happens
 //               on the way into LDS.
+//   gemm_tiny   batches of products of a few elements each: a lane per output.
 //   gemm_rowdot n <= 4 with A's rows along K (matrix x vector): a wave per row of A,
 //               16-byte pieces, float32 sums met through the cross-lane network.
 //   gemm_skinny m <= 16 (decode-like GEMV): HBM-bound on B, which is streamed
@@ -1494,6 +1495,41 @@ static int try_tile_repacked(nxh_context *ctx, const GemmArgs &a0, uint32_t nbat
   return rc;
 }
 
+// ── gemm_tiny: many products of matrices of a few elements each ─────────────
+// ([65536, 4, 4] x [65536, 4, 4]: transforms, small covariance blocks.) One lane per output over
+// the whole batch, so a wave holds the outputs of several products and neighbouring lanes share
+// their operands' cache lines; a tiled block per product left all but a few of its lanes on
+// padding (that shape: 798 us).
+template <int DT>
+__global__ __launch_bounds__(256) void gemm_tiny_kernel(GemmArgs a, uint32_t total) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  const uint32_t o = blockIdx.x * 256u + threadIdx.x;
+  if (o >= total) return;
+  const uint32_t per = (uint32_t)(a.M * a.N);
+  const uint32_t b = o / per, r = o - b * per;
+  const uint32_t m = r / (uint32_t)a.N, n = r - m * (uint32_t)a.N;
+  int64_t ao, bo, co;
+  batch_decode(a.batch, a.batch0 + b, ao, bo, co);
+  const S *A = (const S *)a.A + ao + (int64_t)m * a.ars;
+  const S *B = (const S *)a.B + bo + (int64_t)n * a.bcs;
+  float acc = 0.0f;
+  for (int64_t k = 0; k < a.K; k++) acc = acc + (float)TR::ld(A[k * a.acs]) * (float)TR::ld(B[k * a.brs]);
+  ((S *)a.C)[co + (int64_t)m * a.crs + (int64_t)n * a.ccs] = TR::st((typename TR::C)acc);
+}
+template <int DT>
+static int launch_tiny(nxh_context *ctx, GemmArgs &a, uint32_t nbatch) {
+  nxh_set_path("gemm_tiny");
+  const uint32_t per = (uint32_t)(a.M * a.N), step = 0x7fffff00u / per;  // products per launch
+  for (uint32_t b0 = 0; b0 < nbatch; b0 += step) {
+    a.batch0 = b0;
+    const uint32_t total = std::min<uint32_t>(step, nbatch - b0) * per;
+    hipLaunchKernelGGL((gemm_tiny_kernel<DT>), dim3((total + 255) / 256), dim3(256), 0, ctx->stream, a, total);
+    NXH_HIP("matmul", hipGetLastError());
+  }
+  return NXH_OK;
+}
+
 // ── gemm_rowdot: a matrix whose rows run along K, times one to four columns ──
 // (matrix x vector: C[m][n] = sum over k of A[m][k] B[k][n], N <= 4.) A wave per row of A: its
 // lanes take the row in 16-byte pieces, four in flight, multiply by the matching pieces of the
@@ -1587,6 +1623,8 @@ static int run_mfma_dtype(nxh_context *ctx, GemmArgs &a, uint32_t nbatch, bool b
                           bool batch_aligned_b) {
   using S = typename MM::S;
   constexpr int VL = MM::VL;
+  // many products of a few elements each: a lane per output over the whole batch
+  if (a.M * a.N <= 256 && a.K <= 64 && nbatch >= 256) return launch_tiny<MM::DT>(ctx, a, nbatch);
   // matrix x vector (up to four columns), the matrix's rows along K: a wave per row
   if (a.N <= 4 && a.acs == 1 && a.K >= 64 && (double)a.M * (double)nbatch >= 256.0 && a.M <= 0x7fffffffLL)
     return launch_rowdot<MM::DT>(ctx, a, nbatch, batch_aligned_a, batch_aligned_b);

@@ -739,3 +739,23 @@ def test_matrix_times_vector(hip, oracle, d):
     v = encode(rng.standard_normal((320, 1)), d, oracle)
     check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(v, d, hip, oracle)[0], a, v, "batch, shared vector")
     assert hip.last_path() == "gemm_rowdot", hip.last_path()
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float16], ids=lambda d: d.name)
+def test_many_products_of_tiny_matrices(hip, oracle, d):
+    """Batches of matrices of a few elements each take a lane per output over the whole batch
+    (gemm_tiny): square and ragged shapes, a shared right operand, a batch of two dims, transposed
+    operands, against the float64 product of the stored values."""
+    rng = np.random.default_rng(5300 + d.tag)
+    T = lambda B, t: B.permute(t, tuple(range(len(t.shape) - 2)) + (len(t.shape) - 1, len(t.shape) - 2))  # noqa: E731
+    for batch, m, k, n in (((5000,), 4, 4, 4), ((300,), 3, 7, 5), ((16, 40), 2, 3, 2), ((1000,), 16, 16, 16), ((257,), 1, 64, 9)):
+        a = encode(rng.standard_normal(batch + (m, k)), d, oracle)
+        b = encode(rng.standard_normal(batch + (k, n)), d, oracle)
+        check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(b, d, hip, oracle)[0], a, b, f"{batch} {m}x{k}x{n}")
+        assert hip.last_path() == "gemm_tiny", hip.last_path()
+        shared = encode(rng.standard_normal((k, n)), d, oracle)
+        check(hip, oracle, d, pair(a, d, hip, oracle)[0], pair(shared, d, hip, oracle)[0], a, shared, "shared B")
+        assert hip.last_path() == "gemm_tiny", hip.last_path()
+        at = np.ascontiguousarray(np.swapaxes(a, -1, -2))
+        check(hip, oracle, d, pair(at, d, hip, oracle, T)[0], pair(b, d, hip, oracle)[0], a, b, "transposed A")
+        assert hip.last_path() == "gemm_tiny", hip.last_path()
