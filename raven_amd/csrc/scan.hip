@@ -112,6 +112,28 @@ __global__ __launch_bounds__(FOLD_THREADS) void scan_carry_kernel(C *carry, uint
   }
 }
 
+// The same for few lines and many chunks (one long vector cut into thousands of chunks): a block
+// per line, a lane per run of consecutive chunks; the lanes' totals meet in LDS. One lane per line
+// walked the 4096 chunks of a 2^24-element vector one after the other: 0.3 of that scan's 0.44 ms.
+template <class C, class CB>
+__global__ __launch_bounds__(FOLD_THREADS) void scan_carry_block_kernel(C *carry, uint64_t n_lines, int chunks) {
+  __shared__ C tot[FOLD_THREADS];
+  const uint64_t line = blockIdx.x;
+  const int per = (chunks + FOLD_THREADS - 1) / FOLD_THREADS;
+  const int c0 = (int)threadIdx.x * per, c1 = c0 + per < chunks ? c0 + per : chunks;
+  C s = CB::init();
+  for (int c = c0; c < c1; c++) s = CB::apply(s, carry[(uint64_t)c * n_lines + line]);
+  tot[threadIdx.x] = s;
+  __syncthreads();
+  C run = CB::init();
+  for (int i = 0; i < (int)threadIdx.x; i++) run = CB::apply(run, tot[i]);
+  for (int c = c0; c < c1; c++) {
+    const C t = carry[(uint64_t)c * n_lines + line];
+    carry[(uint64_t)c * n_lines + line] = run;
+    run = CB::apply(run, t);
+  }
+}
+
 template <class T>
 __device__ __forceinline__ T shfl_up_any(T v, int delta) {
   constexpr int W = (sizeof(T) + 3) / 4;
@@ -485,8 +507,12 @@ static int scan_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
       nxh_set_path("scan_rows_chunks");
       if (vec) hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, true, 0>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
       else hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, false, 0>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
-      hipLaunchKernelGGL((scan_carry_kernel<C, CB>), dim3((unsigned)((g.n_out + FOLD_THREADS - 1) / FOLD_THREADS)),
-                         dim3(FOLD_THREADS), 0, ctx->stream, (C *)scratch.p[0], (uint64_t)g.n_out, (int)chunks);
+      if (g.n_out < 64 && chunks >= 64)
+        hipLaunchKernelGGL((scan_carry_block_kernel<C, CB>), dim3((unsigned)g.n_out), dim3(FOLD_THREADS), 0, ctx->stream,
+                           (C *)scratch.p[0], (uint64_t)g.n_out, (int)chunks);
+      else
+        hipLaunchKernelGGL((scan_carry_kernel<C, CB>), dim3((unsigned)((g.n_out + FOLD_THREADS - 1) / FOLD_THREADS)),
+                           dim3(FOLD_THREADS), 0, ctx->stream, (C *)scratch.p[0], (uint64_t)g.n_out, (int)chunks);
       if (vec) hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, true, 2>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
       else hipLaunchKernelGGL((scan_rows_kernel<DT, CB, V, false, 2>), grid, dim3(FOLD_THREADS), 0, ctx->stream, a, chunk, scratch.p[0]);
     } else {

@@ -295,3 +295,23 @@ def test_float_sums_nest_the_same_way_on_every_run(hip, rows, cols):
         got = logical(hip.associative_scan(0, "sum", h))
         assert hip.last_path() == "scan_cols"
         same_bits(got, want, f"[{rows},{cols}] run {run}")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.int32, dt.bfloat16], ids=lambda d: d.name)
+def test_one_long_vector_is_cut_into_chunks_whose_carries_are_scanned_in_parallel(hip, oracle, d):
+    """cumsum / cummax / cummin of one vector of a million elements (and of three such lines): the
+    vector is cut into thousands of chunks, and their carries are scanned by a block per line, a
+    lane per run of chunks. Integers and extremes bit for bit, float sums within the scan tolerance."""
+    rng = np.random.default_rng(960 + d.tag)
+    for shape, axis in (((1 << 20) + 13,), 0), ((3, 300001), 1):
+        x = data(rng, d, shape, oracle)
+        h, o = pair(x, d, hip, oracle)
+        n = shape[axis]
+        for op in ("sum", "max", "min"):
+            g, w = logical(hip.associative_scan(axis, op, h)), logical(oracle.associative_scan(axis, op, o))
+            assert hip.last_path() == "scan_rows_chunks", hip.last_path()
+            if d.is_float and op == "sum":
+                tol = TOL[d.name][0] * 6
+                close(g, w, d, oracle, tol, tol * n, f"{shape} {op}")
+            else:
+                same_bits(g, w, f"{shape} {op}")
