@@ -463,6 +463,130 @@ static void scatter_launch(nxh_context *ctx, const ScatterArgs &a, bool add, int
   else hipLaunchKernelGGL((scatter_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, a);
 }
 
+// ── scatter of one column (a vector's scatter: histograms, bin counts) ──────
+// With a single column the kernels above have one lane per block to apply the updates with, and
+// every block reads the whole index list (2^20 updates into 1000 bins: 2.1 ms). Here the updates
+// are put in target order by a stable argsort of the (normalised) indices, and the first lane of
+// every target's run applies the run in its order, which is index order: the serial result, no
+// atomics. A lane's work is its target's number of updates.
+__global__ __launch_bounds__(256) void scatter_keys_kernel(const int32_t *idx, int64_t stride, int64_t n, int64_t axis_len,
+                                                           int32_t *key, int *fault) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  int64_t v = idx[i * stride];
+  if (v < 0) v += axis_len;
+  if (v < 0 || v >= axis_len) {
+    atomicOr(fault, 1);
+    v = -1;  // sorts first, applied by nobody
+  }
+  key[i] = (int32_t)v;
+}
+template <int DT, bool ADD>
+__global__ __launch_bounds__(256) void scatter_sorted_kernel(const int32_t *key, const int32_t *perm, int64_t n, char *out_c,
+                                                             int64_t os, const char *upd_c, int64_t us) {
+  using TR = Tr<DT>;
+  using S = typename TR::S;
+  using C = typename TR::C;
+  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (p >= n) return;
+  const int32_t k = key[perm[p]];
+  if (k < 0 || (p > 0 && key[perm[p - 1]] == k)) return;  // out of range, or not the first of its target
+  S *o = reinterpret_cast<S *>(out_c) + (int64_t)k * os;
+  const S *upd = reinterpret_cast<const S *>(upd_c);
+  S acc = *o;
+  auto apply = [&](S u) {
+    if constexpr (ADD) {
+      const C x = TR::ld(acc), y = TR::ld(u);
+      if constexpr (TR::cat == CAT_SINT) acc = TR::st((C)((uint64_t)x + (uint64_t)y));
+      else acc = TR::st((C)(x + y));
+    } else {
+      acc = u;
+    }
+  };
+  // eight positions at a time: their indices, targets and updates are fetched together, only the
+  // additions wait for one another (a run of a thousand updates is a thousand dependent trips to
+  // memory otherwise)
+  constexpr int B = 8;
+  int64_t q = p;
+  bool more = true;
+  while (more && q + B <= n) {
+    int32_t i[B], t[B];
+    S u[B];
+#pragma unroll
+    for (int j = 0; j < B; j++) i[j] = perm[q + j];
+#pragma unroll
+    for (int j = 0; j < B; j++) t[j] = key[i[j]];
+#pragma unroll
+    for (int j = 0; j < B; j++) u[j] = upd[(int64_t)i[j] * us];
+#pragma unroll
+    for (int j = 0; j < B; j++) {
+      more = more && t[j] == k;
+      if (more) apply(u[j]);
+    }
+    q += B;
+  }
+  for (; more && q < n; q++) {
+    const int32_t i = perm[q];
+    if (key[i] != k) break;
+    apply(upd[(int64_t)i * us]);
+  }
+  *o = acc;
+}
+typedef void (*scatter_sorted_fn)(nxh_context *, const int32_t *, const int32_t *, const ScatterArgs &, bool);
+template <int DT>
+static void scatter_sorted_launch(nxh_context *ctx, const int32_t *key, const int32_t *perm, const ScatterArgs &a, bool add) {
+  const dim3 grid((unsigned)((a.n_idx + 255) / 256));
+  if (add) hipLaunchKernelGGL((scatter_sorted_kernel<DT, true>), grid, dim3(256), 0, ctx->stream, key, perm, a.n_idx, a.out,
+                              a.a_ostride, a.upd, a.a_ustride);
+  else hipLaunchKernelGGL((scatter_sorted_kernel<DT, false>), grid, dim3(256), 0, ctx->stream, key, perm, a.n_idx, a.out,
+                          a.a_ostride, a.upd, a.a_ustride);
+}
+static int scatter_sorted(nxh_context *ctx, const char *op, const ScatterArgs &a, int dt, bool add) {
+  struct Table {
+    scatter_sorted_fn fn[NXH_DTYPE_COUNT] = {};
+    Table() {
+#define NXH_SC(DT) fn[DT] = &scatter_sorted_launch<DT>;
+      NXH_FOR_COMPUTE_DTYPES(NXH_SC)
+#undef NXH_SC
+    }
+  };
+  static const Table table;
+  if (!table.fn[dt]) return -1;
+  void *key = nullptr, *perm = nullptr;
+  const size_t bytes = (size_t)a.n_idx * sizeof(int32_t);
+  int rc = nxh_alloc(ctx, bytes, &key);
+  if (!rc) rc = nxh_alloc(ctx, bytes, &perm);
+  if (!rc) {
+    std::lock_guard<std::mutex> guard(ctx->mu);
+    rc = nxh_settle_replay_faults(ctx, op);
+    if (!rc) {
+      hipLaunchKernelGGL(scatter_keys_kernel, dim3((unsigned)((a.n_idx + 255) / 256)), dim3(256), 0, ctx->stream, a.idx,
+                         a.a_istride, a.n_idx, a.axis_len, (int32_t *)key, a.fault);
+      if (hipGetLastError() != hipSuccess) rc = nxh_fail(NXH_FAILURE, op, "launch failed");
+    }
+  }
+  if (!rc) {
+    nxh_tensor kt{}, pt{};
+    kt.data = key;
+    pt.data = perm;
+    kt.dtype = pt.dtype = NXH_I32;
+    kt.ndim = pt.ndim = 1;
+    kt.shape[0] = pt.shape[0] = a.n_idx;
+    kt.strides[0] = pt.strides[0] = 1;
+    rc = nxh_argsort(ctx, &pt, &kt, 0, 0);  // stable: equal targets stay in index order
+  }
+  if (!rc) {
+    std::lock_guard<std::mutex> guard(ctx->mu);
+    nxh_set_path("scatter_sorted");
+    table.fn[dt](ctx, (const int32_t *)key, (const int32_t *)perm, a, add);
+    if (hipGetLastError() != hipSuccess) rc = nxh_fail(NXH_FAILURE, op, "launch failed");
+    else rc = nxh_collect_index_fault(ctx, op);
+  }
+  if (key) (void)nxh_free(ctx, key);
+  if (perm) (void)nxh_free(ctx, perm);
+  return rc;
+}
+
 NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_tensor *indices,
                            const nxh_tensor *updates, int axis, int mode) {
   NXH_DEFER_TOUCH(ctx, 1, out, indices, updates);
@@ -519,6 +643,10 @@ NXH_EXPORT int nxh_scatter(nxh_context *ctx, const nxh_tensor *out, const nxh_te
   static const Table table_;
   const scatter_launch_fn *table = table_.fn;
   if (!table[dt]) return nxh_fail(NXH_FAILURE, op, NXH_ERR_UNSUPPORTED);
+  if (a.columns == 1 && a.n_idx >= 4096 && a.n_idx <= 0x3fffffffLL && a.axis_len <= 0x7fffffffLL && !ctx->capture) {
+    const int src = scatter_sorted(ctx, op, a, dt, mode == 1);
+    if (src != -1) return src;
+  }
   std::lock_guard<std::mutex> guard(ctx->mu);
   NXH_HIP(op, hipSetDevice(ctx->device));
   if (int frc = nxh_settle_replay_faults(ctx, op)) return frc;

@@ -339,3 +339,39 @@ def test_scatter_add_large_is_a_histogram(hip):
     out = logical(hip.scatter("add", False, hip.full(dt.int32, (vocab, dim), 0), idx, upd, 0))
     hist = np.bincount(ids, minlength=vocab).astype(np.int32)
     assert np.array_equal(out, np.repeat(hist[:, None], dim, 1))
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.int32, dt.uint8], ids=lambda d: d.name)
+def test_scatter_of_one_column_applies_every_target_in_index_order(hip, oracle, d):
+    """A vector's scatter (histograms, bin counts): the updates are sorted by target and each
+    target's run is applied by one lane in index order. Inexact float sums with thousands of
+    updates per bin pin that order bit for bit; negative indices, bins nobody hits, a strided
+    index list, "set" keeping the last update, and the out-of-bounds report."""
+    rng = np.random.default_rng(120 + d.tag)
+    for bins, n in ((1000, 100000), (7, 5000), (70000, 4096)):
+        ids = rng.integers(-bins, bins, n).astype(np.int32)
+        ids[ids == bins // 2] = 0  # a bin nobody hits
+        if d.is_float:
+            t = encode(rng.standard_normal(bins), d, oracle)
+            upd = encode(rng.standard_normal(n) * 3, d, oracle)
+        else:
+            info = np.iinfo(d.np_storage)
+            t = rng.integers(info.min, info.max, bins, endpoint=True).astype(d.np_storage)
+            upd = rng.integers(info.min, info.max, n, endpoint=True).astype(d.np_storage)
+        (ht, ot), (hu, ou), (hi, oi) = pair(t, d, hip, oracle), pair(upd, d, hip, oracle), pair(ids, dt.int32, hip, oracle)
+        for mode in ("set", "add"):
+            same_bits(logical(hip.scatter(mode, False, ht, hi, hu, 0)), logical(oracle.scatter(mode, False, ot, oi, ou, 0)),
+                      f"{mode} {bins} bins, {n} updates")
+            assert hip.last_path() == "scatter_sorted", hip.last_path()
+        # every other entry of a longer index list
+        wide = np.stack([ids, rng.integers(0, bins, n).astype(np.int32)], axis=1)
+        hw, ow = pair(wide, dt.int32, hip, oracle, lambda B, t: B.reshape(B.shrink(t, [(0, n), (0, 1)]), (n,)))
+        same_bits(logical(hip.scatter("add", False, ht, hw, hu, 0)), logical(oracle.scatter("add", False, ot, ow, ou, 0)),
+                  "strided index list")
+        assert hip.last_path() == "scatter_sorted", hip.last_path()
+    bad = ids.copy()
+    bad[n // 2] = 70000
+    with pytest.raises(RuntimeError, match="out of bounds"):
+        hip.scatter("add", False, ht, pair(bad, dt.int32, hip, oracle)[0], hu, 0)
+    same_bits(logical(hip.scatter("add", False, ht, hi, hu, 0)), logical(oracle.scatter("add", False, ot, oi, ou, 0)),
+              "usable after a reported fault")
