@@ -190,10 +190,14 @@ def test_scan_paths_nan_and_reference_vector(hip, oracle):
     hw, ow = pair(w, dt.int32, hip, oracle)
     same_bits(logical(hip.associative_scan(1, "sum", hw)), logical(oracle.associative_scan(1, "sum", ow)))
     assert hip.last_path() == "scan_rows_chunks"
-    hw, ow = pair(np.ascontiguousarray(w.T), dt.int32, hip, oracle)
+    hw, ow = pair(np.ascontiguousarray(w.T), dt.int32, hip, oracle)  # three columns: the flat form
+    same_bits(logical(hip.associative_scan(0, "max", hw)), logical(oracle.associative_scan(0, "max", ow)))
+    assert hip.last_path() == "scan_narrow"
+    w20 = rng.integers(-9, 9, (70001, 20)).astype(np.int32)
+    hw, ow = pair(w20, dt.int32, hip, oracle)
     same_bits(logical(hip.associative_scan(0, "max", hw)), logical(oracle.associative_scan(0, "max", ow)))
     assert hip.last_path() == "scan_cols"
-    hw64, ow64 = pair(np.ascontiguousarray(w.T).astype(np.int64), dt.int64, hip, oracle)
+    hw64, ow64 = pair(w20.astype(np.int64), dt.int64, hip, oracle)
     same_bits(logical(hip.associative_scan(0, "max", hw64)), logical(oracle.associative_scan(0, "max", ow64)))
     assert hip.last_path() == "scan_chunks"
     f = rng.standard_normal((2, 50000)).astype(np.float32)

@@ -315,3 +315,14 @@ def test_one_long_vector_is_cut_into_chunks_whose_carries_are_scanned_in_paralle
                 close(g, w, d, oracle, tol, tol * n, f"{shape} {op}")
             else:
                 same_bits(g, w, f"{shape} {op}")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.float64, dt.int32, dt.uint8, dt.complex64], ids=lambda d: d.name)
+def test_tall_matrices_of_a_few_columns_scanned_down_their_rows(hip, oracle, d):
+    """[rows, L] with fewer than 16 columns (running totals of a table of a few series): read as one
+    flat run, 256 / L rows a pass. One block and many, ragged last passes and blocks, in place."""
+    rng = np.random.default_rng(970 + d.tag)
+    for rows, L in ((1024, 2), (5000, 10), (100001, 3), (40000, 15), (1500, 7)):
+        x = data(rng, d, (rows, L), oracle)
+        h, o = pair(x, d, hip, oracle)
+        check(hip, oracle, h, o, d, rows, f"[{rows},{L}]", path="scan_narrow")
