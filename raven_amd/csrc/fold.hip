@@ -229,6 +229,48 @@ __global__ __launch_bounds__(FOLD_THREADS) void fold_narrow_kernel(NarrowArgs a)
   }
 }
 
+// ── fold_short_rows ─────────────────────────────────────────────────────────
+// Many contiguous rows of 2 .. 32 elements each (the classes of a batch of logits), reduced along
+// the row: too short for a wave per row. A block brings 256 rows into LDS with neighbouring lanes
+// on neighbouring addresses (row pitch odd, so that the lanes' walks along their rows meet
+// different banks), then a lane folds its own row in row order.
+struct ShortRowsArgs {
+  const void *in;
+  void *out;
+  int64_t rows;
+  int R;
+};
+template <class IN, class CB, class OUT>
+__global__ __launch_bounds__(FOLD_THREADS) void fold_short_rows_kernel(ShortRowsArgs a) {
+  using T = typename IN::T;
+  using C = typename IN::C;
+  static_assert(sizeof(T) <= 4, "the tile is sized for storage types of up to four bytes");
+  __shared__ T tile[FOLD_THREADS * 33];
+  const int R = a.R, pitch = R | 1;
+  const int64_t row_base = (int64_t)blockIdx.x * FOLD_THREADS;
+  const int64_t left = a.rows - row_base;
+  const int nrows = (int)(left < FOLD_THREADS ? left : FOLD_THREADS);
+  const int count = nrows * R;
+  const T *src = (const T *)a.in + row_base * R;
+  int row = (int)threadIdx.x / R, col = (int)threadIdx.x - row * R;
+  const int drow = FOLD_THREADS / R, dcol = FOLD_THREADS - drow * R;
+  for (int i = threadIdx.x; i < count; i += FOLD_THREADS) {
+    tile[row * pitch + col] = src[i];
+    row += drow;
+    col += dcol;
+    if (col >= R) {
+      col -= R;
+      row++;
+    }
+  }
+  __syncthreads();
+  if ((int)threadIdx.x >= nrows) return;
+  const T *mine = tile + threadIdx.x * pitch;
+  C acc = CB::init();
+  for (int j = 0; j < R; j++) acc = CB::apply(acc, IN::ld(mine[j]));
+  ((typename OUT::T *)a.out)[row_base + threadIdx.x] = OUT::st(acc);
+}
+
 // ── fold_any ────────────────────────────────────────────────────────────────
 struct AnyArgs {
   const void *in;
@@ -350,6 +392,23 @@ static int fold_launch(nxh_context *ctx, const char *op, const nxh_tensor *in, c
         hipLaunchKernelGGL((fold_row_kernel<InC<C>, CB, OutS<DT>, 64, 1>), grid2, dim3(FOLD_THREADS), 0, ctx->stream, b);
         NXH_HIP(op, hipGetLastError());
       }
+      return NXH_OK;
+    }
+  }
+
+  // ---- fold_short_rows: many contiguous rows of 2 .. 32 elements, reduced along the row ----
+  if constexpr (sizeof(S) <= 4) {
+    if (g.nr == 1 && g.nk == 1 && g.rin[0] == 1 && g.R >= 2 && g.R <= 32 && g.kin[0] == g.R && g.kout[0] == 1 &&
+        g.n_out >= 4096 && g.n_out <= 0x7fffffffLL * 128) {
+      ShortRowsArgs a;
+      a.in = ibase;
+      a.out = obase;
+      a.rows = g.n_out;
+      a.R = (int)g.R;
+      nxh_set_path("fold_short_rows");
+      hipLaunchKernelGGL((fold_short_rows_kernel<InS<DT>, CB, OutS<DT>>), dim3((unsigned)((g.n_out + FOLD_THREADS - 1) / FOLD_THREADS)),
+                         dim3(FOLD_THREADS), 0, ctx->stream, a);
+      NXH_HIP(op, hipGetLastError());
       return NXH_OK;
     }
   }

@@ -320,3 +320,33 @@ def test_argreduce_of_many_short_rows(hip, oracle, d):
         # the same rows as columns of the transposed matrix (strided axis)
         ht, ot = pair(np.ascontiguousarray(x.T), d, hip, oracle)
         same_bits(logical(hip.argmax(ht, 0)), logical(oracle.argmax(ot, 0)), f"argmax axis 0 [{n},{rows}]")
+
+
+@pytest.mark.parametrize("d", [dt.float32, dt.bfloat16, dt.int32, dt.int8, dt.uint8, dt.bool_], ids=lambda d: d.name)
+def test_many_short_rows_reduced_along_the_row(hip, oracle, d):
+    """[rows, R] with R from 2 to 32 and thousands of rows (the classes of a batch of logits): a block
+    brings 256 rows into LDS and a lane folds its own. Every R at the bank-conflict corners (2, 16,
+    31, 32), a ragged last block, NaNs in float rows."""
+    rng = np.random.default_rng(1600 + d.tag)
+    for rows, R in ((4096, 2), (5000, 10), (70001, 3), (4100, 16), (9000, 31), (8192, 32)):
+        if d.is_float:
+            v = rng.uniform(-2, 2, (rows, R))
+            v.reshape(-1)[rng.integers(0, v.size, 7)] = np.nan
+            x = encode(v, d, oracle)
+        elif d is dt.bool_:
+            x = rng.integers(0, 2, (rows, R)).astype(np.uint8)
+        else:
+            info = np.iinfo(d.np_storage)
+            x = rng.integers(max(info.min, -100), min(info.max, 100), (rows, R), endpoint=True).astype(d.np_storage)
+        h, o = pair(x, d, hip, oracle)
+        for op in (("max", "min") if d is dt.bool_ else ("sum", "max", "min", "prod")):
+            g, w = logical(hip.reduce(op, [1], h)), logical(oracle.reduce(op, [1], o))
+            assert hip.last_path() == "fold_short_rows", (rows, R, op, hip.last_path())
+            if d.is_float and op in ("sum", "prod"):
+                gv, wv = decode(g, d, oracle), decode(w, d, oracle)
+                assert np.array_equal(np.isnan(gv), np.isnan(wv)), (rows, R, op)
+                ok = ~np.isnan(wv)
+                lim = TOL[d.name][0] * R * (np.abs(wv[ok]) + 2.0 ** R if op == "prod" else np.abs(wv[ok]) + 2.0 * R)
+                assert np.all(np.abs(gv[ok] - wv[ok]) <= lim), (rows, R, op)
+            else:
+                same_bits(g, w, f"[{rows},{R}] {op}")
