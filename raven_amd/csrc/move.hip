@@ -552,6 +552,10 @@ static int scatter_sorted(nxh_context *ctx, const char *op, const ScatterArgs &a
   };
   static const Table table;
   if (!table.fn[dt]) return -1;
+  // several calls in a row: no capture may begin between them (it would record the later launches
+  // with blocks that are freed below)
+  std::lock_guard<std::mutex> whole_call(ctx->call_mu);
+  if (ctx->capture) return -1;
   void *key = nullptr, *perm = nullptr;
   const size_t bytes = (size_t)a.n_idx * sizeof(int32_t);
   int rc = nxh_alloc(ctx, bytes, &key);
