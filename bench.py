@@ -53,7 +53,7 @@ METRIC = "Nx op GB/s (elementwise/reduce) + GEMM TFLOP/s, as % of MI355X rooflin
 # [64,512,512]), from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of
 # `bench.py --only-step --no-cpu --pmc-calibration`: 32 799 KiB fetched x 1.9991 (a plain
 # 64 MiB copy reads 32 782 KiB on the same counter) + 65 536 KiB written x 1.0000.
-DOMINANT_KERNEL_HBM_TRAFFIC = 134252356
+DOMINANT_KERNEL_HBM_TRAFFIC = 134252296
 
 
 class Op:
